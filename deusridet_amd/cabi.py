@@ -1,0 +1,104 @@
+"""ctypes binding of the C ABI declared in include/drk_kv.h.
+
+Loads deusridet_amd/lib/libdrk_kv.so.  If the library is missing this module
+raises ImportError: nothing here computes anything on its own.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdrk_kv.so")
+
+F16, BF16, INT8, FP8_E4M3 = 0, 1, 2, 3
+OK, ERR_INVALID, ERR_HIP, ERR_UNSUPPORTED, ERR_WORKSPACE = 0, -1, -2, -3, -4
+
+
+class DrkError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"drk error {code}: {text}")
+        self.code = code
+
+
+class Layout(C.Structure):
+    """drk_kv_layout"""
+    _fields_ = [(n, C.c_int32) for n in (
+        "num_layers", "num_kv_heads", "num_q_heads", "head_dim", "block_size",
+        "max_phys_blocks", "dtype", "reserved")]
+
+
+def layout(L, KVH, QH, D, bs, NB, dtype):
+    return Layout(L, KVH, QH, D, bs, NB, dtype, 0)
+
+
+_vp, _i32, _sz, _f32 = C.c_void_p, C.c_int32, C.c_size_t, C.c_float
+_LP = C.POINTER(Layout)
+
+# name -> (restype, argtypes); mirrors include/drk_kv.h one to one
+SIGNATURES = {
+    "drk_abi_version": (_i32, []),
+    "drk_last_error": (C.c_char_p, []),
+    "drk_strerror": (C.c_char_p, [_i32]),
+    "drk_device_count": (_i32, [C.POINTER(_i32)]),
+    "drk_kv_layout_check": (_i32, [_LP]),
+    "drk_kv_elem_bytes": (_sz, [_LP]),
+    "drk_kv_plane_bytes": (_sz, [_LP]),
+    "drk_kv_block_stride_bytes": (_sz, [_LP]),
+    "drk_kv_layer_stride_bytes": (_sz, [_LP]),
+    "drk_kv_pool_bytes": (_sz, [_LP]),
+    "drk_kv_k_offset": (_sz, [_LP, _i32, _i32]),
+    "drk_kv_v_offset": (_sz, [_LP, _i32, _i32]),
+    "drk_kv_max_blocks_for_budget": (_i32, [_LP, _sz]),
+    "drk_dev_malloc": (_i32, [C.POINTER(_vp), _sz]),
+    "drk_dev_free": (_i32, [_vp]),
+    "drk_dev_memset_async": (_i32, [_vp, _i32, _sz, _vp]),
+    "drk_memcpy_h2d_async": (_i32, [_vp, _vp, _sz, _vp]),
+    "drk_memcpy_d2h": (_i32, [_vp, _vp, _sz, _vp]),
+    "drk_stream_create": (_i32, [C.POINTER(_vp)]),
+    "drk_stream_destroy": (_i32, [_vp]),
+    "drk_stream_synchronize": (_i32, [_vp]),
+    "drk_kv_append_token": (_i32, [_LP, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp]),
+    "drk_kv_append_batch": (_i32, [_LP, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp]),
+    "drk_kv_append_branches": (_i32, [_LP, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _i32, _vp]),
+    "drk_kv_extract": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "drk_kv_inject": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "drk_kv_copy_blocks": (_i32, [_LP, _vp, _vp, _i32, _vp]),
+    "drk_decode_workspace_bytes": (_sz, [_LP, _i32, _i32]),
+    "drk_decode_workspace_bytes_for_split": (_sz, [_LP, _i32, _i32, _i32]),
+    "drk_decode_default_split": (_i32, [_LP, _i32, _i32]),
+    "drk_debug_force_portable_decode": (None, [_i32]),
+    "drk_paged_decode_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
+    "drk_paged_decode_attention_branches": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32,
+                                                   _f32, _i32, _i32, _vp, _sz, _vp]),
+    "drk_prefill_workspace_bytes": (_sz, [_LP, _i32, _i32]),
+    "drk_paged_prefill_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
+    "drk_importance_update": (_i32, [_vp, _vp, _i32, _f32, _vp]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library (raises ImportError when it has not been built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `make -C deusridet_amd/csrc`")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def check(code):
+    if code != OK:
+        raise DrkError(code, lib().drk_last_error().decode())
+    return code
+
+
+def call(name, *args):
+    """Call an int-returning entry point and raise DrkError on failure."""
+    return check(getattr(lib(), name)(*args))

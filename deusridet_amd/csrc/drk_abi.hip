@@ -1,0 +1,158 @@
+// drk_abi.hip -- library plumbing of libdrk_kv.so: error text, layout
+// arithmetic (host only) and the device-memory calls the host classes need.
+#include "drk_common.hpp"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+namespace drk {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int make_lay(const drk_kv_layout *g, Lay *a)
+{
+    if (!g) return fail(DRK_ERR_INVALID, "layout is NULL");
+    if (g->num_layers < 1 || g->num_kv_heads < 1 || g->num_q_heads < 1 || g->head_dim < 1 ||
+        g->block_size < 1 || g->max_phys_blocks < 1)
+        return fail(DRK_ERR_INVALID, "layout: every dimension must be >= 1");
+    if (g->dtype < DRK_F16 || g->dtype > DRK_FP8_E4M3)
+        return fail(DRK_ERR_INVALID, "layout: unknown dtype %d", g->dtype);
+    if (g->reserved != 0) return fail(DRK_ERR_INVALID, "layout: reserved must be 0");
+    if (g->num_q_heads % g->num_kv_heads)
+        return fail(DRK_ERR_INVALID, "layout: num_q_heads %d not a multiple of num_kv_heads %d",
+                    g->num_q_heads, g->num_kv_heads);
+    if (g->head_dim % 8)
+        return fail(DRK_ERR_UNSUPPORTED, "layout: head_dim %d must be a multiple of 8", g->head_dim);
+    a->L = g->num_layers; a->KVH = g->num_kv_heads; a->QH = g->num_q_heads; a->D = g->head_dim;
+    a->bs = g->block_size; a->NB = g->max_phys_blocks; a->dtype = g->dtype;
+    a->E = (g->dtype == DRK_F16 || g->dtype == DRK_BF16) ? 2 : 1;
+    size_t row = (size_t)a->D * a->E;
+    size_t head = row * a->bs;
+    size_t plane = head * a->KVH;
+    size_t sp = g->dtype == DRK_INT8 ? (size_t)a->KVH * a->bs * 2 : 0;
+    size_t bstride = 2 * plane + 2 * sp;
+    if (bstride > 0x7fffffffu)
+        return fail(DRK_ERR_UNSUPPORTED, "layout: one (layer, block) exceeds 2 GiB");
+    a->row_bytes = (unsigned)row; a->head_stride = (unsigned)head; a->kv_plane = (unsigned)plane;
+    a->scale_plane = (unsigned)sp; a->block_stride = (unsigned)bstride;
+    a->layer_stride = (size_t)a->NB * bstride;
+    return DRK_OK;
+}
+
+} // namespace drk
+
+using drk::Lay;
+using drk::fail;
+
+extern "C" {
+
+int drk_abi_version(void) { return 1; }
+const char *drk_last_error(void) { return drk::g_err; }
+const char *drk_strerror(int code)
+{
+    switch (code) {
+    case DRK_OK: return "ok";
+    case DRK_ERR_INVALID: return "invalid argument";
+    case DRK_ERR_HIP: return "HIP runtime error";
+    case DRK_ERR_UNSUPPORTED: return "unsupported geometry";
+    case DRK_ERR_WORKSPACE: return "workspace missing or too small";
+    default: return "unknown error";
+    }
+}
+
+int drk_device_count(int *count)
+{
+    if (!count) return fail(DRK_ERR_INVALID, "count is NULL");
+    *count = 0;
+    DRK_HIP(hipGetDeviceCount(count));
+    return DRK_OK;
+}
+
+int drk_kv_layout_check(const drk_kv_layout *g) { Lay a; return drk::make_lay(g, &a); }
+
+#define LAY_OR_ZERO(g) Lay a; if (drk::make_lay(g, &a) != DRK_OK) return 0
+size_t drk_kv_elem_bytes(const drk_kv_layout *g) { LAY_OR_ZERO(g); return a.E; }
+size_t drk_kv_plane_bytes(const drk_kv_layout *g) { LAY_OR_ZERO(g); return a.kv_plane; }
+size_t drk_kv_block_stride_bytes(const drk_kv_layout *g) { LAY_OR_ZERO(g); return a.block_stride; }
+size_t drk_kv_layer_stride_bytes(const drk_kv_layout *g) { LAY_OR_ZERO(g); return a.layer_stride; }
+size_t drk_kv_pool_bytes(const drk_kv_layout *g) { LAY_OR_ZERO(g); return (size_t)a.L * a.layer_stride; }
+size_t drk_kv_k_offset(const drk_kv_layout *g, int layer, int block)
+{
+    LAY_OR_ZERO(g);
+    return drk::lay_block_base(a, layer, block);
+}
+size_t drk_kv_v_offset(const drk_kv_layout *g, int layer, int block)
+{
+    LAY_OR_ZERO(g);
+    return drk::lay_block_base(a, layer, block) + a.kv_plane;
+}
+int drk_kv_max_blocks_for_budget(const drk_kv_layout *g, size_t budget_bytes)
+{
+    // max_phys_blocks is the unknown here: validate with a stand-in of 1
+    if (!g) return 0;
+    drk_kv_layout t = *g;
+    t.max_phys_blocks = 1;
+    Lay a;
+    if (drk::make_lay(&t, &a) != DRK_OK) return 0;
+    size_t per_block = (size_t)a.L * a.block_stride;
+    size_t n = budget_bytes / per_block;
+    return n > 0x7fffffff ? 0x7fffffff : (int)n;
+}
+
+int drk_dev_malloc(void **d_ptr, size_t bytes)
+{
+    if (!d_ptr) return fail(DRK_ERR_INVALID, "d_ptr is NULL");
+    *d_ptr = nullptr;
+    DRK_HIP(hipMalloc(d_ptr, bytes));
+    return DRK_OK;
+}
+int drk_dev_free(void *d_ptr)
+{
+    if (d_ptr) DRK_HIP(hipFree(d_ptr));
+    return DRK_OK;
+}
+int drk_dev_memset_async(void *d_ptr, int byte, size_t bytes, void *stream)
+{
+    DRK_HIP(hipMemsetAsync(d_ptr, byte, bytes, (hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_memcpy_h2d_async(void *d_dst, const void *h_src, size_t bytes, void *stream)
+{
+    DRK_HIP(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream)
+{
+    DRK_HIP(hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    DRK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_stream_create(void **stream)
+{
+    if (!stream) return fail(DRK_ERR_INVALID, "stream is NULL");
+    hipStream_t s;
+    DRK_HIP(hipStreamCreate(&s));
+    *stream = (void *)s;
+    return DRK_OK;
+}
+int drk_stream_destroy(void *stream)
+{
+    if (stream) DRK_HIP(hipStreamDestroy((hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_stream_synchronize(void *stream)
+{
+    DRK_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return DRK_OK;
+}
+
+} // extern "C"

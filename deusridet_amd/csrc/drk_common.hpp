@@ -1,0 +1,87 @@
+// drk_common.hpp -- shared between the translation units of libdrk_kv.so:
+// error reporting, the device-side view of the pool layout, element helpers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "drk_kv.h"
+
+namespace drk {
+
+// ---- error reporting ----------------------------------------------------
+int fail(int code, const char *fmt, ...);
+#define DRK_HIP(call)                                                          \
+    do {                                                                       \
+        hipError_t e__ = (call);                                               \
+        if (e__ != hipSuccess)                                                 \
+            return drk::fail(DRK_ERR_HIP, "%s: %s", #call, hipGetErrorString(e__)); \
+    } while (0)
+// kernel launches report through hipGetLastError
+#define DRK_LAUNCH_CHECK(name)                                                 \
+    do {                                                                       \
+        hipError_t e__ = hipGetLastError();                                    \
+        if (e__ != hipSuccess)                                                 \
+            return drk::fail(DRK_ERR_HIP, "launch %s: %s", name, hipGetErrorString(e__)); \
+    } while (0)
+
+// ---- layout, precomputed in bytes ---------------------------------------
+// Contract: see the comment above drk_kv_layout in drk_kv.h.
+struct Lay {
+    int L, KVH, QH, D, bs, NB, dtype, E;
+    unsigned row_bytes;          // D*E
+    unsigned head_stride;        // bs*D*E: one head's rows inside a K or V plane
+    unsigned kv_plane;           // KVH*bs*D*E
+    unsigned scale_plane;        // INT8: KVH*bs*2, else 0
+    unsigned block_stride;       // 2*kv_plane + 2*scale_plane
+    size_t layer_stride;         // NB*block_stride
+};
+
+int make_lay(const drk_kv_layout *g, Lay *out);   // validates, returns DRK_*
+
+__host__ __device__ inline size_t lay_block_base(const Lay &a, int layer, int blk)
+{
+    return (size_t)layer * a.layer_stride + (size_t)blk * a.block_stride;
+}
+
+inline int ilog2_exact(unsigned v)                 // -1 when v is not a power of two
+{
+    if (v == 0 || (v & (v - 1))) return -1;
+    int s = 0;
+    while ((1u << s) != v) s++;
+    return s;
+}
+
+// ---- element helpers (device) -------------------------------------------
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ float f16_bits_to_f(uint16_t h)
+{
+    return __half2float(__ushort_as_half(h));
+}
+__device__ __forceinline__ float elem16_to_f(uint16_t x, int dtype)
+{
+    return dtype == DRK_BF16 ? __uint_as_float((uint32_t)x << 16) : f16_bits_to_f(x);
+}
+// round-to-nearest-even fp32 -> bf16 bits
+__device__ __forceinline__ uint16_t f_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if (f != f) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint16_t f_to_elem16(float f, int dtype)
+{
+    return dtype == DRK_BF16 ? f_to_bf16_bits(f) : __half_as_ushort(__float2half_rn(f));
+}
+
+// unsigned divide with a power-of-two fast path chosen on the host
+__device__ __forceinline__ unsigned udiv(unsigned x, unsigned d, int shift)
+{
+    return shift >= 0 ? (x >> shift) : (x / d);
+}
+
+} // namespace drk

@@ -1,0 +1,400 @@
+// drk_pages.hip -- data movement between token-major buffers and pages:
+// append (with int8 / fp8 quantisation on the way in), extract, inject,
+// copy-on-write block copies, importance-score update.
+//
+// All of it is HBM-bound byte work.  Every thread moves 16-byte chunks; the
+// chunk index inside a workgroup enumerates [token][head][chunk], which is the
+// order of the token-major side, so that side is read or written as one
+// contiguous run per workgroup and the paged side as whole head rows.
+#include "drk_common.hpp"
+
+namespace drk {
+
+constexpr int kThreads = 256;
+constexpr int kTokensPerGroup = 16;   // tokens one workgroup moves per (layer, K|V)
+
+__device__ __forceinline__ size_t row_off(const Lay &a, int layer, int blk, int kv, int h, int p)
+{
+    return lay_block_base(a, layer, blk) + (size_t)kv * a.kv_plane + (size_t)h * a.head_stride +
+           (size_t)p * a.row_bytes;
+}
+__device__ __forceinline__ size_t scale_off(const Lay &a, int layer, int blk, int kv, int h, int p)
+{
+    return lay_block_base(a, layer, blk) + 2 * (size_t)a.kv_plane + (size_t)kv * a.scale_plane +
+           ((size_t)h * a.bs + p) * 2;
+}
+
+struct Div {            // divisor with a power-of-two fast path
+    unsigned d;
+    int shift;
+};
+static Div mk_div(unsigned d) { return Div{d, ilog2_exact(d)}; }
+__device__ __forceinline__ unsigned dv(unsigned x, Div v) { return udiv(x, v.d, v.shift); }
+
+// ------------------------------------------------------------------------
+// extract / inject
+// grid = (token groups, num_layers*2); flat side [layer][K|V][token][head][dim]
+// ------------------------------------------------------------------------
+template <bool EXTRACT>
+__global__ __launch_bounds__(kThreads) void flat_copy_kernel(
+    Lay a, uint8_t *__restrict__ pool, uint8_t *__restrict__ flat, uint8_t *__restrict__ flat_scales,
+    const int32_t *__restrict__ table, int start_token, int num_tokens, Div tok_div, Div row_div,
+    Div bs_div)
+{
+    const int tg = blockIdx.x;
+    const int layer = blockIdx.y >> 1, kv = blockIdx.y & 1;
+    const int t0 = tg * kTokensPerGroup;
+    const int ntok = min(kTokensPerGroup, num_tokens - t0);
+    const unsigned rc = row_div.d;                       // 16-byte chunks per row
+    const unsigned items = (unsigned)ntok * tok_div.d;   // tok_div.d = KVH*rc
+    uint8_t *fbase = flat + ((size_t)(layer * 2 + kv) * num_tokens + t0) * a.KVH * a.row_bytes;
+
+    constexpr int U = 4;
+    for (unsigned base = threadIdx.x; base < items; base += kThreads * U) {
+        uint4 val[U];
+        size_t poff[U];
+        bool live[U], hole[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            unsigned ci = base + u * kThreads;
+            live[u] = ci < items;
+            hole[u] = true;
+            poff[u] = 0;
+            val[u] = make_uint4(0, 0, 0, 0);
+            if (live[u]) {
+                unsigned t = dv(ci, tok_div), r = ci - t * tok_div.d;
+                unsigned h = dv(r, row_div), c = r - h * rc;
+                unsigned gt = (unsigned)(start_token + t0) + t;
+                unsigned lb = dv(gt, bs_div);
+                int blk = table[lb];
+                if (blk >= 0 && blk < a.NB) {
+                    hole[u] = false;
+                    poff[u] = row_off(a, layer, blk, kv, h, gt - lb * bs_div.d) + (size_t)c * 16;
+                }
+                if (EXTRACT) { if (!hole[u]) val[u] = *(const uint4 *)(pool + poff[u]); }
+                else val[u] = *(const uint4 *)(fbase + (size_t)ci * 16);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            unsigned ci = base + u * kThreads;
+            if (!live[u]) continue;
+            if (EXTRACT) *(uint4 *)(fbase + (size_t)ci * 16) = val[u];          // hole => zeros
+            else if (!hole[u]) *(uint4 *)(pool + poff[u]) = val[u];              // hole => skip
+        }
+    }
+
+    if (a.dtype == DRK_INT8 && flat_scales) {
+        uint8_t *sbase = flat_scales + ((size_t)(layer * 2 + kv) * num_tokens + t0) * a.KVH * 2;
+        for (unsigned i = threadIdx.x; i < (unsigned)ntok * a.KVH; i += kThreads) {
+            unsigned t = i / a.KVH, h = i - t * a.KVH;
+            unsigned gt = (unsigned)(start_token + t0) + t;
+            unsigned lb = dv(gt, bs_div);
+            int blk = table[lb];
+            bool ok = blk >= 0 && blk < a.NB;
+            size_t so = ok ? scale_off(a, layer, blk, kv, h, gt - lb * bs_div.d) : 0;
+            if (EXTRACT) *(uint16_t *)(sbase + (size_t)i * 2) = ok ? *(const uint16_t *)(pool + so) : (uint16_t)0;
+            else if (ok) *(uint16_t *)(pool + so) = *(const uint16_t *)(sbase + (size_t)i * 2);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------
+// append
+// grid = (token groups, layer_count, 2); source [layer][token][head][dim] of
+// 16-bit elements, one 16-byte chunk (8 elements) per thread.
+// "token" i is position pos_start+i of one table (batch mode, d_pos == NULL) or
+// the single new token of branch i at d_pos[i] with table row i (branch mode).
+// QMODE 0: copy.  1: int8 codes + fp16 scale per row.  2: fp8 e4m3 codes.
+// ------------------------------------------------------------------------
+__device__ __forceinline__ void unpack8(const uint4 &v, int src_dtype, float *x)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        x[2 * i] = elem16_to_f((uint16_t)(w[i] & 0xffffu), src_dtype);
+        x[2 * i + 1] = elem16_to_f((uint16_t)(w[i] >> 16), src_dtype);
+    }
+}
+
+// E4M3FN code of x: round-half-even, |x| >= 448 and +-inf saturate to +-448,
+// NaN stays NaN.  The clamp runs before the hardware conversion so that the
+// conversion never sees an out-of-range input.
+__device__ __forceinline__ uint32_t fp8_pair(float x0, float x1)
+{
+    x0 = (x0 != x0) ? x0 : fminf(fmaxf(x0, -448.0f), 448.0f);
+    x1 = (x1 != x1) ? x1 : fminf(fmaxf(x1, -448.0f), 448.0f);
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(x0, x1, 0, false) & 0xffffu;
+#else
+    (void)x0; (void)x1;
+    return 0;
+#endif
+}
+
+template <int QMODE>
+__global__ __launch_bounds__(kThreads) void append_kernel(
+    Lay a, uint8_t *__restrict__ pool, const int32_t *__restrict__ tables, int table_stride,
+    const int32_t *__restrict__ d_pos, int pos_start, int ntokens, int layer0,
+    const uint8_t *__restrict__ src_k, const uint8_t *__restrict__ src_v, int src_dtype, Div tok_div,
+    Div row_div, Div bs_div)
+{
+    const int tg = blockIdx.x, li = blockIdx.y, kv = blockIdx.z;
+    const int layer = layer0 + li;
+    const int t0 = tg * kTokensPerGroup;
+    const int ntok = min(kTokensPerGroup, ntokens - t0);
+    const unsigned rc = row_div.d;                       // D/8 chunks per source row
+    const unsigned items = (unsigned)ntok * tok_div.d;   // tok_div.d = KVH*rc
+    const size_t src_row = (size_t)a.D * 2;
+    const uint8_t *sbase = (kv ? src_v : src_k) + ((size_t)li * ntokens + t0) * a.KVH * src_row;
+    const unsigned rounds = (items + kThreads - 1) / kThreads;
+
+    for (unsigned rnd = 0; rnd < rounds; rnd++) {
+        unsigned ci = rnd * kThreads + threadIdx.x;
+        bool live = ci < items;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        size_t poff = 0, soff = 0;
+        unsigned c = 0;
+        bool hole = true;
+        if (live) {
+            unsigned t = dv(ci, tok_div), r = ci - t * tok_div.d;
+            unsigned h = dv(r, row_div);
+            c = r - h * rc;
+            int ti = t0 + (int)t;
+            int pos = d_pos ? d_pos[ti] : pos_start + ti;
+            const int32_t *tab = tables + (size_t)(d_pos ? ti : 0) * table_stride;
+            if (pos >= 0) {
+                unsigned lb = dv((unsigned)pos, bs_div);
+                int blk = tab[lb];
+                if (blk >= 0 && blk < a.NB) {
+                    hole = false;
+                    int p = pos - lb * bs_div.d;
+                    poff = row_off(a, layer, blk, kv, h, p);
+                    if (QMODE == 1) soff = scale_off(a, layer, blk, kv, h, p);
+                }
+            }
+            val = *(const uint4 *)(sbase + (size_t)ci * 16);
+        }
+        if (QMODE == 0) {
+            if (live && !hole) *(uint4 *)(pool + poff + (size_t)c * 16) = val;
+        } else {
+            float x[8];
+            unpack8(val, src_dtype, x);
+            if (QMODE == 1) {
+                // row absmax over the rc lanes that hold this row (rc is a power
+                // of two <= 64 and rows never straddle a wave)
+                float amax = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(x[i]));
+                for (unsigned off = rc >> 1; off > 0; off >>= 1)
+                    amax = fmaxf(amax, __shfl_xor(amax, (int)off));
+                float s32 = __fdiv_rn(amax, 127.0f);
+                uint16_t sh = __half_as_ushort(__float2half_rn(s32));
+                if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
+                float sf = f16_bits_to_f(sh);
+                float rcp = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
+                uint32_t lo = 0, hi = 0;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float r = rintf(__fmul_rn(x[i], rcp));
+                    r = fminf(fmaxf(r, -127.0f), 127.0f);
+                    uint32_t b = (uint32_t)((int)r) & 0xffu;
+                    if (i < 4) lo |= b << (8 * i); else hi |= b << (8 * (i - 4));
+                }
+                if (live && !hole) {
+                    *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
+                    if (c == 0) *(uint16_t *)(pool + soff) = sh;
+                }
+            } else {
+                uint32_t lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
+                uint32_t hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
+                if (live && !hole) *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------
+// copy-on-write: every layer of block src -> block dst
+// grid = (chunk groups, L, pairs)
+// ------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void copy_blocks_kernel(Lay a, uint8_t *__restrict__ pool,
+                                                               const int32_t *__restrict__ pairs)
+{
+    const int layer = blockIdx.y;
+    const int src = pairs[2 * blockIdx.z], dst = pairs[2 * blockIdx.z + 1];
+    if (src < 0 || dst < 0 || src >= a.NB || dst >= a.NB || src == dst) return;
+    const uint4 *s = (const uint4 *)(pool + lay_block_base(a, layer, src));
+    uint4 *d = (uint4 *)(pool + lay_block_base(a, layer, dst));
+    const unsigned n = a.block_stride / 16;
+    constexpr int U = 4;
+    for (unsigned base = blockIdx.x * kThreads * U + threadIdx.x; base < n; base += gridDim.x * kThreads * U) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            unsigned i = base + u * kThreads;
+            if (i < n) v[u] = s[i];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            unsigned i = base + u * kThreads;
+            if (i < n) d[i] = v[u];
+        }
+    }
+}
+
+// importance_update_kernel, importance_scorer.cu:27-36
+__global__ void importance_update_kernel(float *__restrict__ scores, const float *__restrict__ new_scores,
+                                         int n, float decay)
+{
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < n) scores[b] = __fadd_rn(__fmul_rn(scores[b], decay), new_scores[b]);
+}
+
+static int check_src_dtype(int d)
+{
+    if (d != DRK_F16 && d != DRK_BF16) return fail(DRK_ERR_INVALID, "src_dtype must be F16 or BF16");
+    return DRK_OK;
+}
+
+static int launch_append(const drk_kv_layout *g, void *pool, const int32_t *tables, int table_stride,
+                         const int32_t *d_pos, int pos_start, int ntokens, int layer, int layer_count,
+                         const void *src_k, const void *src_v, int src_dtype, void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if ((rc = check_src_dtype(src_dtype))) return rc;
+    if (!pool || !tables || !src_k || !src_v) return fail(DRK_ERR_INVALID, "append: NULL pointer");
+    if (layer < 0 || layer_count < 1 || layer + layer_count > a.L)
+        return fail(DRK_ERR_INVALID, "append: layers [%d,%d) outside [0,%d)", layer, layer + layer_count, a.L);
+    if (layer_count > 65535) return fail(DRK_ERR_INVALID, "append: layer_count > 65535");
+    if (ntokens < 0 || pos_start < 0) return fail(DRK_ERR_INVALID, "append: negative token count or position");
+    if (ntokens == 0) return DRK_OK;
+    if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && src_dtype != a.dtype)
+        return fail(DRK_ERR_INVALID, "append: src_dtype %d differs from the pool's %d", src_dtype, a.dtype);
+    unsigned rowc = a.D / 8;
+    if (a.dtype == DRK_INT8 || a.dtype == DRK_FP8_E4M3) {
+        if (ilog2_exact(rowc) < 0 || rowc > 64)
+            return fail(DRK_ERR_UNSUPPORTED, "append: quantising pools need head_dim in {8..512} power of two, got %d", a.D);
+    }
+    Div tok_div = mk_div((unsigned)a.KVH * rowc), row_div = mk_div(rowc), bs_div = mk_div((unsigned)a.bs);
+    dim3 grid((ntokens + kTokensPerGroup - 1) / kTokensPerGroup, layer_count, 2);
+    hipStream_t s = (hipStream_t)stream;
+#define GO(Q)                                                                                       \
+    hipLaunchKernelGGL(append_kernel<Q>, grid, dim3(kThreads), 0, s, a, (uint8_t *)pool, tables,    \
+                       table_stride, d_pos, pos_start, ntokens, layer, (const uint8_t *)src_k,      \
+                       (const uint8_t *)src_v, src_dtype, tok_div, row_div, bs_div)
+    if (a.dtype == DRK_INT8) GO(1);
+    else if (a.dtype == DRK_FP8_E4M3) GO(2);
+    else GO(0);
+#undef GO
+    DRK_LAUNCH_CHECK("append_kernel");
+    return DRK_OK;
+}
+
+static int launch_flat(bool extract, const drk_kv_layout *g, void *pool, void *flat, void *flat_scales,
+                       const int32_t *table, int start_token, int num_tokens, int num_layers, void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (!pool || !flat || !table) return fail(DRK_ERR_INVALID, "extract/inject: NULL pointer");
+    if (num_layers < 0 || num_layers > a.L) return fail(DRK_ERR_INVALID, "extract/inject: num_layers %d outside [0,%d]", num_layers, a.L);
+    if (start_token < 0 || num_tokens < 0) return fail(DRK_ERR_INVALID, "extract/inject: negative token range");
+    if (num_tokens == 0 || num_layers == 0) return DRK_OK;
+    if (a.row_bytes % 16) return fail(DRK_ERR_UNSUPPORTED, "extract/inject: row of %u bytes is not a multiple of 16", a.row_bytes);
+    if (num_layers * 2 > 65535) return fail(DRK_ERR_INVALID, "extract/inject: too many layers");
+    unsigned rowc = a.row_bytes / 16;
+    Div tok_div = mk_div((unsigned)a.KVH * rowc), row_div = mk_div(rowc), bs_div = mk_div((unsigned)a.bs);
+    dim3 grid((num_tokens + kTokensPerGroup - 1) / kTokensPerGroup, num_layers * 2);
+    hipStream_t s = (hipStream_t)stream;
+    if (extract)
+        hipLaunchKernelGGL(flat_copy_kernel<true>, grid, dim3(kThreads), 0, s, a, (uint8_t *)pool, (uint8_t *)flat,
+                           (uint8_t *)flat_scales, table, start_token, num_tokens, tok_div, row_div, bs_div);
+    else
+        hipLaunchKernelGGL(flat_copy_kernel<false>, grid, dim3(kThreads), 0, s, a, (uint8_t *)pool, (uint8_t *)flat,
+                           (uint8_t *)flat_scales, table, start_token, num_tokens, tok_div, row_div, bs_div);
+    DRK_LAUNCH_CHECK("flat_copy_kernel");
+    return DRK_OK;
+}
+
+} // namespace drk
+
+using namespace drk;
+
+extern "C" {
+
+int drk_kv_append_token(const drk_kv_layout *g, void *pool, const int32_t *d_block_table, int layer,
+                        const int32_t *d_pos, const void *src_k, const void *src_v, int src_dtype,
+                        void *stream)
+{
+    if (!d_pos) return fail(DRK_ERR_INVALID, "append_token: d_pos is NULL");
+    return launch_append(g, pool, d_block_table, 0, d_pos, 0, 1, layer, 1, src_k, src_v, src_dtype, stream);
+}
+
+int drk_kv_append_batch(const drk_kv_layout *g, void *pool, const int32_t *d_block_table, int layer,
+                        int layer_count, int pos_start, int M, const void *src_k, const void *src_v,
+                        int src_dtype, void *stream)
+{
+    return launch_append(g, pool, d_block_table, 0, nullptr, pos_start, M, layer, layer_count, src_k, src_v,
+                         src_dtype, stream);
+}
+
+int drk_kv_append_branches(const drk_kv_layout *g, void *pool, const int32_t *d_tables, int table_stride,
+                           const int32_t *d_pos, int B, int layer, int layer_count, const void *src_k,
+                           const void *src_v, int src_dtype, void *stream)
+{
+    if (!d_pos) return fail(DRK_ERR_INVALID, "append_branches: d_pos is NULL");
+    if (table_stride < 0) return fail(DRK_ERR_INVALID, "append_branches: negative table_stride");
+    return launch_append(g, pool, d_tables, table_stride, d_pos, 0, B, layer, layer_count, src_k, src_v,
+                         src_dtype, stream);
+}
+
+int drk_kv_extract(const drk_kv_layout *g, void *d_dst, void *d_dst_scales, const void *pool,
+                   const int32_t *d_block_table, int start_token, int num_tokens, int num_layers,
+                   void *stream)
+{
+    return launch_flat(true, g, (void *)pool, d_dst, d_dst_scales, d_block_table, start_token, num_tokens,
+                       num_layers, stream);
+}
+
+int drk_kv_inject(const drk_kv_layout *g, void *pool, const void *d_src, const void *d_src_scales,
+                  const int32_t *d_block_table, int start_token, int num_tokens, int num_layers,
+                  void *stream)
+{
+    return launch_flat(false, g, pool, (void *)d_src, (void *)d_src_scales, d_block_table, start_token,
+                       num_tokens, num_layers, stream);
+}
+
+int drk_kv_copy_blocks(const drk_kv_layout *g, void *pool, const int32_t *d_pairs, int n, void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (!pool || (!d_pairs && n > 0)) return fail(DRK_ERR_INVALID, "copy_blocks: NULL pointer");
+    if (n < 0) return fail(DRK_ERR_INVALID, "copy_blocks: negative pair count");
+    if (a.block_stride % 16) return fail(DRK_ERR_UNSUPPORTED, "copy_blocks: block of %u bytes is not a multiple of 16", a.block_stride);
+    if (a.L > 65535) return fail(DRK_ERR_INVALID, "copy_blocks: too many layers");
+    unsigned chunks = a.block_stride / 16;
+    unsigned gx = (chunks + kThreads * 4 - 1) / (kThreads * 4);
+    for (int done = 0; done < n; done += 65535) {
+        int cnt = n - done < 65535 ? n - done : 65535;
+        hipLaunchKernelGGL(copy_blocks_kernel, dim3(gx, a.L, cnt), dim3(kThreads), 0, (hipStream_t)stream, a,
+                           (uint8_t *)pool, d_pairs + 2 * (size_t)done);
+        DRK_LAUNCH_CHECK("copy_blocks_kernel");
+    }
+    return DRK_OK;
+}
+
+int drk_importance_update(float *d_scores, const float *d_new_scores, int n, float decay, void *stream)
+{
+    if (n <= 0) return DRK_OK;
+    if (!d_scores || !d_new_scores) return fail(DRK_ERR_INVALID, "importance_update: NULL pointer");
+    hipLaunchKernelGGL(importance_update_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       d_scores, d_new_scores, n, decay);
+    DRK_LAUNCH_CHECK("importance_update_kernel");
+    return DRK_OK;
+}
+
+} // extern "C"

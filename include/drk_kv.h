@@ -1,0 +1,185 @@
+/*
+ * drk_kv.h -- C ABI of the MI355X (gfx950) paged-KV hot path.
+ *
+ * This is the only layer that touches HIP.  The C++ host interface that mirrors
+ * DeusRidet's Memoria/Machina classes (deusridet_amd/memoria/, machina/) is
+ * written against these entry points and nothing else; any other language binds
+ * the same symbols (cgo, JNI, ctypes ...).
+ *
+ * Conventions
+ *   - every call returns DRK_OK (0) or a negative DRK_ERR_* code; the text of the
+ *     last error on the calling thread is at drk_last_error();
+ *   - pointers named d_* / pool / q / out / src_* / workspace are DEVICE pointers;
+ *     h_* are host pointers;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     every launch is asynchronous on it, nothing here synchronises unless it
+ *     says so, and no kernel entry point allocates or frees memory;
+ *   - geometry travels in a drk_kv_layout (the reference spreads it over
+ *     PagedKVConfig constexprs, block_pool.h:34-52, and ModelConfig statics,
+ *     model.h:39-42, 73);
+ *   - citations are file:line in the DeusRidet tree.
+ */
+#ifndef DRK_KV_H
+#define DRK_KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DRK_OK               0
+#define DRK_ERR_INVALID     -1   /* bad argument / shape the kernels do not take */
+#define DRK_ERR_HIP         -2   /* a HIP runtime call failed                     */
+#define DRK_ERR_UNSUPPORTED -3   /* geometry outside the compiled set             */
+#define DRK_ERR_WORKSPACE   -4   /* workspace missing or too small                */
+
+/* storage type of the pool / element type of Q, out and append sources */
+enum { DRK_F16 = 0, DRK_BF16 = 1, DRK_INT8 = 2, DRK_FP8_E4M3 = 3 };
+
+/*
+ * Pool layout (bytes), the contract shared by every kernel and by the host
+ * classes (block_pool.cpp:23-39, 81-95; paged_attention.cu:36-64;
+ * cache_kernels.cu:71-84):
+ *   E            = 2 (F16, BF16) or 1 (INT8, FP8_E4M3)
+ *   kv_plane     = num_kv_heads * block_size * head_dim * E
+ *   scale_plane  = INT8 ? num_kv_heads * block_size * 2 : 0      (fp16 scales)
+ *   block_stride = 2*kv_plane + 2*scale_plane
+ *   layer_stride = max_phys_blocks * block_stride
+ *   K(l,b,h,p,d) = l*layer_stride + b*block_stride + ((h*block_size+p)*head_dim+d)*E
+ *   V(l,b,h,p,d) = K(l,b,h,p,d) + kv_plane
+ *   Kscale(l,b,h,p) = l*layer_stride + b*block_stride + 2*kv_plane + (h*block_size+p)*2
+ *   Vscale(l,b,h,p) = Kscale(l,b,h,p) + scale_plane
+ */
+typedef struct drk_kv_layout {
+    int32_t num_layers;       /* ModelConfig::NUM_FA_LAYERS  (model.h:73)        */
+    int32_t num_kv_heads;     /* ModelConfig::NUM_KV_HEADS   (model.h:40)        */
+    int32_t num_q_heads;      /* ModelConfig::NUM_ATTN_HEADS (model.h:39)        */
+    int32_t head_dim;         /* ModelConfig::HEAD_DIM       (model.h:41)        */
+    int32_t block_size;       /* tokens per block (block_pool.h:35, runtime)     */
+    int32_t max_phys_blocks;  /* BlockPool::max_blocks()     (block_pool.h:80)   */
+    int32_t dtype;            /* DRK_*: storage type of the pool                 */
+    int32_t reserved;         /* must be 0                                       */
+} drk_kv_layout;
+
+/* ---- library ---------------------------------------------------------- */
+int         drk_abi_version(void);
+const char *drk_last_error(void);
+const char *drk_strerror(int code);
+int         drk_device_count(int *count);
+
+/* ---- layout arithmetic (host only, no GPU needed) --------------------- */
+/* block_pool.cpp:23-39: strides; block_pool.cpp:28-32: budget -> max_blocks */
+int drk_kv_layout_check(const drk_kv_layout *g);
+size_t drk_kv_elem_bytes(const drk_kv_layout *g);
+size_t drk_kv_plane_bytes(const drk_kv_layout *g);
+size_t drk_kv_block_stride_bytes(const drk_kv_layout *g);
+size_t drk_kv_layer_stride_bytes(const drk_kv_layout *g);
+size_t drk_kv_pool_bytes(const drk_kv_layout *g);
+/* BlockPool::k_offset / v_offset, block_pool.cpp:89-95 */
+size_t drk_kv_k_offset(const drk_kv_layout *g, int layer, int block);
+size_t drk_kv_v_offset(const drk_kv_layout *g, int layer, int block);
+int    drk_kv_max_blocks_for_budget(const drk_kv_layout *g, size_t budget_bytes);
+
+/* ---- device memory plumbing for the host classes ---------------------- */
+/* cudaMalloc/cudaMemset/cudaFree in BlockPool::init/destroy
+ * (block_pool.cpp:42-49, 97-101) and CacheManager::init (cache_manager.cpp:46-53);
+ * cudaMemcpyAsync in CacheManager::sync_block_table (cache_manager.cpp:108-112). */
+int drk_dev_malloc(void **d_ptr, size_t bytes);
+int drk_dev_free(void *d_ptr);
+int drk_dev_memset_async(void *d_ptr, int byte, size_t bytes, void *stream);
+int drk_memcpy_h2d_async(void *d_dst, const void *h_src, size_t bytes, void *stream);
+int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream); /* syncs */
+int drk_stream_create(void **stream);
+int drk_stream_destroy(void *stream);
+int drk_stream_synchronize(void *stream);
+
+/* ---- append into pages ------------------------------------------------ */
+/* paged_kv_cache_write, paged_attention.cu:73-115: one token at *d_pos.
+ * src_k/src_v [num_kv_heads, head_dim] of src_dtype (F16/BF16); an INT8/FP8 pool
+ * quantises on the way in (round-half-even). */
+int drk_kv_append_token(const drk_kv_layout *g, void *pool, const int32_t *d_block_table,
+                        int layer, const int32_t *d_pos, const void *src_k,
+                        const void *src_v, int src_dtype, void *stream);
+/* paged_kv_cache_write_batch, paged_attention.cu:123-167: M consecutive tokens
+ * from src [M, num_kv_heads, head_dim].  layer_count > 1 appends the same
+ * positions for layers layer..layer+layer_count-1 in one launch from
+ * src [layer_count, M, num_kv_heads, head_dim]. */
+int drk_kv_append_batch(const drk_kv_layout *g, void *pool, const int32_t *d_block_table,
+                        int layer, int layer_count, int pos_start, int M,
+                        const void *src_k, const void *src_v, int src_dtype, void *stream);
+/* One token for each of B branches in one launch (no reference counterpart; the
+ * reference has one sequence).  d_tables [B, table_stride], d_pos [B],
+ * src [layer_count, B, num_kv_heads, head_dim]. */
+int drk_kv_append_branches(const drk_kv_layout *g, void *pool, const int32_t *d_tables,
+                           int table_stride, const int32_t *d_pos, int B, int layer,
+                           int layer_count, const void *src_k, const void *src_v,
+                           int src_dtype, void *stream);
+
+/* ---- gather / scatter ------------------------------------------------- */
+/* invoke_extract_kv_from_pages, cache_kernels.cu:30-87, 147-166:
+ * dst [num_layers][2][num_tokens][num_kv_heads][head_dim] in the pool's storage
+ * type; INT8 pools also fill d_dst_scales [num_layers][2][num_tokens][num_kv_heads]
+ * fp16 when it is not NULL.  A hole (table entry < 0) is zero-filled. */
+int drk_kv_extract(const drk_kv_layout *g, void *d_dst, void *d_dst_scales, const void *pool,
+                   const int32_t *d_block_table, int start_token, int num_tokens,
+                   int num_layers, void *stream);
+/* invoke_inject_kv_to_pages, cache_kernels.cu:93-141, 168-187; a hole is skipped. */
+int drk_kv_inject(const drk_kv_layout *g, void *pool, const void *d_src, const void *d_src_scales,
+                  const int32_t *d_block_table, int start_token, int num_tokens,
+                  int num_layers, void *stream);
+/* Copy-on-write: copy every layer of physical block src to dst for n pairs
+ * (no reference counterpart; intent docs/en/architecture/02-memoria.md:25-26).
+ * d_pairs [n][2] = (src, dst). */
+int drk_kv_copy_blocks(const drk_kv_layout *g, void *pool, const int32_t *d_pairs, int n,
+                       void *stream);
+
+/* ---- paged GQA decode attention --------------------------------------- */
+/* Bytes of workspace the split-K decode needs for B branches of at most
+ * max_seq_len tokens. */
+size_t drk_decode_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len);
+/* Same for an explicit split_tokens: B*num_q_heads*ceil(max_seq_len/split)*(head_dim+2)*4. */
+size_t drk_decode_workspace_bytes_for_split(const drk_kv_layout *g, int B, int max_seq_len,
+                                            int split_tokens);
+/* The split (tokens per workgroup, a multiple of 64) the library picks when
+ * split_tokens == 0. */
+int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len);
+/* Diagnostic: route every decode / prefill through the portable kernel (any
+ * geometry, any storage type) instead of the tiled one, so that tests can
+ * check the two against each other.  Process-wide, not thread-safe. */
+void drk_debug_force_portable_decode(int on);
+/* paged_gqa_decode_attention, paged_attention.cu:179-282: one sequence.
+ * q/out [num_q_heads, head_dim] of io_dtype (F16/BF16). */
+int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void *pool,
+                               const int32_t *d_block_table, void *out, int layer,
+                               int seq_len, float scale, int io_dtype, void *workspace,
+                               size_t workspace_bytes, void *stream);
+/* B branches in one launch: d_tables [B, table_stride], d_seq_lens [B] (device),
+ * q/out [B, num_q_heads, head_dim]; max_seq_len >= every d_seq_lens[b] sizes the
+ * grid.  split_tokens = 0 lets the library choose. */
+int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, const void *pool,
+                                        const int32_t *d_tables, int table_stride,
+                                        const int32_t *d_seq_lens, int B, int max_seq_len,
+                                        void *out, int layer, float scale, int io_dtype,
+                                        int split_tokens, void *workspace,
+                                        size_t workspace_bytes, void *stream);
+
+/* ---- paged causal prefill attention ------------------------------------ */
+/* paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630:
+ * q/out [M, num_q_heads, head_dim]; row t attends to tokens 0..pos_start+t. */
+size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M);
+int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
+                                const int32_t *d_block_table, void *out, int layer,
+                                int pos_start, int M, float scale, int io_dtype,
+                                void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- importance scores -------------------------------------------------- */
+/* importance_update_kernel, importance_scorer.cu:27-36, 67-73 */
+int drk_importance_update(float *d_scores, const float *d_new_scores, int n, float decay,
+                          void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DRK_KV_H */
