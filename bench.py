@@ -1,0 +1,252 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-KV hot path on one MI355X.
+
+Workload (BASELINE config 2): 36 layers, 32 Q / 8 KV heads x 128, bf16 KV in
+16-token pages shuffled across a 40 GB pool, 8 decode branches at 32k context.
+One step = for every layer: append one token per branch, then paged GQA decode
+attention over all branches.  Prints ONE JSON line (see README / DESIGN).
+
+Torch is used for device memory, streams and events only; every kernel is
+reached through the C ABI in include/drk_kv.h.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--layers", type=int, default=36)
+    ap.add_argument("--branches", type=int, default=8)
+    ap.add_argument("--ctx", type=int, default=32768, help="context length of every branch at the last timed step")
+    ap.add_argument("--ctx-mode", choices=["fixed", "uniform"], default="fixed",
+                    help="fixed: every branch at --ctx (the 70%% target point); uniform: U{1024..ctx}")
+    ap.add_argument("--pool-gb", type=float, default=40.0)
+    ap.add_argument("--split", type=int, default=0, help="tokens per split-K workgroup (0 = library default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="context per branch for the CPU sample (0 = auto)")
+    ap.add_argument("--bulk-append-tokens", type=int, default=2048)
+    ap.add_argument("--seed", type=int, default=2)
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (sharding across GPUs is "
+              "described in DESIGN.md, not implemented)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from deusridet_amd import cabi
+    from tests import util as U
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    lib = cabi.lib()
+    torch.cuda.set_device(0)
+    rng = np.random.default_rng(args.seed)
+
+    L, KVH, QH, D, bs = args.layers, 8, 32, 128, 16
+    B, W, K = args.branches, args.warmup, args.steps
+    probe = cabi.layout(L, KVH, QH, D, bs, 1, cabi.BF16)
+    NB = lib.drk_kv_max_blocks_for_budget(C.byref(probe), int(args.pool_gb * 1e9))
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    pool_bytes = lib.drk_kv_pool_bytes(C.byref(g))
+
+    # context lengths at the START of the run; every step appends one token
+    if args.ctx_mode == "fixed":
+        final = np.full(B, args.ctx, dtype=np.int64)
+    else:
+        final = rng.integers(1024, args.ctx + 1, size=B)
+    start = np.maximum(final - (W + K), 1).astype(np.int32)
+    nblk = [(int(s) + W + K + bs - 1) // bs for s in start]
+    assert sum(nblk) <= NB, f"pool of {NB} blocks too small for {sum(nblk)}"
+    stride = max(nblk) + 1
+    perm = rng.permutation(NB).astype(np.int32)           # physical blocks shuffled over the whole pool
+    tables = np.full((B, stride), -1, dtype=np.int32)
+    o = 0
+    for b in range(B):
+        tables[b, :nblk[b]] = perm[o:o + nblk[b]]
+        o += nblk[b]
+
+    stream = torch.cuda.current_stream()
+    sp = C.c_void_p(stream.cuda_stream)
+    pool = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    pool.zero_()
+    dtab = torch.from_numpy(tables).cuda()
+
+    # fill the pages through the append path itself, N(0,1)*0.5 -> bf16
+    chunk = 2048
+    t_fill = time.time()
+    for b in range(B):
+        n = int(start[b])
+        for p0 in range(0, n, chunk):
+            m = min(chunk, n - p0)
+            k = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+            v = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(dtab[b].data_ptr()), 0, L, p0, m,
+                      U.p(k), U.p(v), cabi.BF16, sp)
+            del k, v
+    torch.cuda.synchronize()
+    t_fill = time.time() - t_fill
+
+    scale = 1.0 / np.sqrt(D)
+    q = (torch.randn(L, B, QH, D, device="cuda") * 0.5).to(torch.bfloat16)
+    newk = (torch.randn(L, B, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+    newv = (torch.randn(L, B, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+    out = torch.zeros(L, B, QH, D, device="cuda", dtype=torch.bfloat16)
+    max_ctx = int(final.max())
+    split = args.split or lib.drk_decode_default_split(C.byref(g), B, max_ctx)
+    wsb = lib.drk_decode_workspace_bytes_for_split(C.byref(g), B, max_ctx, split)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    # device arrays of positions / lengths for every step, prepared up front so the
+    # timed loop does no host->device traffic
+    pos_steps = torch.from_numpy(np.stack([start + s for s in range(W + K)]).astype(np.int32)).cuda()
+    len_steps = pos_steps + 1                                 # write-then-attend: the new token is visible
+    qrow, krow = B * QH * D * 2, B * KVH * D * 2
+
+    def step(s):
+        dpos = C.c_void_p(pos_steps[s].data_ptr())
+        dlen = C.c_void_p(len_steps[s].data_ptr())
+        for l in range(L):
+            cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), stride, dpos, B, l, 1,
+                      C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, sp)
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow),
+                      U.p(pool), U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
+                      float(scale), cabi.BF16, split, U.p(ws), wsb, sp)
+
+    for s in range(W):
+        step(s)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for s in range(W, W + K):
+        step(s)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    total_ms = e0.elapsed_time(e1)
+    ms_per_step = total_ms / K
+
+    ctx_sum_steps = [int((start + s + 1).sum()) for s in range(W, W + K)]       # tokens attended per layer
+    kv_bytes_per_token = 2 * KVH * D * 2                                          # K + V, all kv heads, bf16
+    attn_bytes = sum(ctx_sum_steps) * kv_bytes_per_token * L
+    value_gbps = attn_bytes / (total_ms * 1e-3) / 1e9
+
+    # ---- dominant kernel alone: the split-K partial kernel of one layer -------
+    lib.drk_debug_time_decode_kernel(1)
+    ker_ms = []
+    last = W + K - 1
+    dlen = C.c_void_p(len_steps[last].data_ptr())
+    for it in range(max(K, 10)):
+        l = it % L
+        cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
+                  U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
+                  cabi.BF16, split, U.p(ws), wsb, sp)
+        ms = C.c_float(0)
+        cabi.call("drk_debug_last_decode_kernel_ms", C.byref(ms))
+        ker_ms.append(ms.value)
+    lib.drk_debug_time_decode_kernel(0)
+    ker_ms = ker_ms[2:]
+    ker_avg_ms = float(np.mean(ker_ms))
+    launch_bytes = int((start + last + 1).sum()) * kv_bytes_per_token               # one layer, one launch
+    achieved = launch_bytes / (ker_avg_ms * 1e-3) / 1e9
+
+    # ---- bulk append bandwidth (read source + write pages), all layers in one launch
+    m = args.bulk_append_tokens
+    scratch_tab = torch.from_numpy(perm[o:o + (m + bs - 1) // bs].copy()).cuda() if o + (m + bs - 1) // bs <= NB else None
+    append_gbps = None
+    if scratch_tab is not None:
+        k = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+        v = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+        for _ in range(3):
+            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(scratch_tab), 0, L, 0, m, U.p(k), U.p(v),
+                      cabi.BF16, sp)
+        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a0.record(stream)
+        reps = 10
+        for _ in range(reps):
+            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(scratch_tab), 0, L, 0, m, U.p(k), U.p(v),
+                      cabi.BF16, sp)
+        a1.record(stream)
+        torch.cuda.synchronize()
+        ab = 2 * (2 * L * m * KVH * D * 2)                                          # K,V read + written
+        append_gbps = ab * reps / (a0.elapsed_time(a1) * 1e-3) / 1e9
+
+    # ---- CPU baseline: the oracle's restatement of the reference loop, OpenMP ----
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import binding as orc
+        cores = min(os.cpu_count() or 1, 16)
+        n_cpu = args.cpu_sample_tokens or 4096
+        og = orc.layout(1, KVH, QH, D, bs, B * (n_cpu // bs + 1), orc.BF16)
+        hp = orc.new_pool(og)
+        nb1 = n_cpu // bs + 1
+        htab = np.arange(B * nb1, dtype=np.int32).reshape(B, nb1)
+        crng = np.random.default_rng(7)
+        for b in range(B):
+            kk = U.normal_bits(crng, (n_cpu, KVH, D), cabi.BF16, 0.5)
+            vv = U.normal_bits(crng, (n_cpu, KVH, D), cabi.BF16, 0.5)
+            orc.append_batch(og, hp, htab[b], 0, 0, kk, vv, orc.BF16)
+        hq = U.normal_bits(crng, (B, QH, D), cabi.BF16, 0.5)
+        lens = np.full(B, n_cpu, dtype=np.int32)
+        t0 = time.time()
+        reps = 0
+        while time.time() - t0 < 10.0:
+            orc.decode_branches(og, hq, hp, htab, lens, 0, float(scale), orc.BF16, threads=cores)
+            reps += 1
+        dt = time.time() - t0
+        cpu_bytes = reps * B * n_cpu * kv_bytes_per_token
+        cpu = {"value": cpu_bytes / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+               "sample": f"{reps} x (1 layer, {B} branches x {n_cpu} tokens) of the same decode attention, "
+                         f"oracle's reference-order loop, OpenMP over (branch, q head)"}
+
+    tokens_per_s = B * K / (total_ms * 1e-3)
+    line = {
+        "metric": "paged_decode_attention_GBps",
+        "value": round(value_gbps, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"config 2: {L} layers, 32 Q / 8 KV heads x 128, bf16 KV, 16-token pages shuffled over a "
+                        f"{args.pool_gb:g} GB pool ({NB} blocks), {B} branches, ctx {args.ctx_mode} "
+                        f"{int(final.min())}..{int(final.max())}; step = per layer: append 1 token/branch + paged decode attention",
+            "branches": B, "layers": L, "ctx_final": [int(x) for x in final], "split_tokens": int(split),
+        },
+        "hbm_frac_step": round(value_gbps / HBM_PEAK_GBPS, 4),
+        "us_per_step": round(ms_per_step * 1e3, 1),
+        "tokens_per_s": round(tokens_per_s, 1),
+        "bulk_append_GBps": None if append_gbps is None else round(append_gbps, 1),
+        "bulk_append_hbm_frac": None if append_gbps is None else round(append_gbps / HBM_PEAK_GBPS, 4),
+        "fill_seconds": round(t_fill, 2),
+        "roofline": {
+            "kernel": "decode_tiled_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None, "avg_launch_us": round(ker_avg_ms * 1e3, 2), "bytes_per_launch": launch_bytes,
+        },
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -29,6 +29,9 @@
 namespace drk {
 
 static int g_force_portable = 0;
+static int g_time_kernel = 0;                 // diagnostic: bracket the partial kernel with events
+static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
+static int g_lds_pad = 0;                     // diagnostic: extra dynamic LDS per workgroup (caps occupancy)
 
 constexpr int kTile = 64;            // tokens per tile
 constexpr int kKRow = 272;           // LDS bytes per staged K row: 256 + 16 pad
@@ -447,9 +450,12 @@ __global__ void decode_merge_kernel(const float *__restrict__ part_o, const floa
 // ------------------------------------------------------------------------
 static int choose_split(const Lay &a, int B, int max_seq_len)
 {
-    // largest run (multiple of the tile) that still yields >= 8 workgroups per CU
-    const long want = 2048;
-    int split = 2048;
+    // Longest run (a multiple of the tile, at most 4096 tokens) that still yields
+    // two workgroups per CU of a 256-CU part: measured on MI355X, long runs win
+    // because the per-workgroup prologue (table -> first K/V tile) and epilogue are
+    // paid once, and a grid that is resident in a single round has no tail.
+    const long want = 512;
+    int split = 4096;
     while (split > kTile) {
         long wgs = (long)B * a.KVH * ((max_seq_len + split - 1) / split);
         if (wgs >= want) break;
@@ -499,6 +505,10 @@ static int launch_decode(const drk_kv_layout *g, const void *q, const void *pool
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(S, a.KVH, B);
 
+    if (g_time_kernel) {
+        if (!g_ev0) { DRK_HIP(hipEventCreate(&g_ev0)); DRK_HIP(hipEventCreate(&g_ev1)); }
+        DRK_HIP(hipEventRecord(g_ev0, st));
+    }
     const bool tiled = !g_force_portable && a.D == 128 && a.E == 2 && G == 4 && (a.bs % 16) == 0;
     if (tiled) {
         TiledArgs A;
@@ -510,8 +520,8 @@ static int launch_decode(const drk_kv_layout *g, const void *q, const void *pool
         A.bs_shift = ilog2_exact((unsigned)a.bs);
         A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
         A.scale_log2e = sl2;
-        if (a.dtype == DRK_BF16) hipLaunchKernelGGL(decode_tiled_kernel<DRK_BF16>, grid, dim3(256), 0, st, A);
-        else hipLaunchKernelGGL(decode_tiled_kernel<DRK_F16>, grid, dim3(256), 0, st, A);
+        if (a.dtype == DRK_BF16) hipLaunchKernelGGL(decode_tiled_kernel<DRK_BF16>, grid, dim3(256), g_lds_pad, st, A);
+        else hipLaunchKernelGGL(decode_tiled_kernel<DRK_F16>, grid, dim3(256), g_lds_pad, st, A);
         DRK_LAUNCH_CHECK("decode_tiled_kernel");
     } else {
         if ((a.dtype == DRK_INT8 || a.dtype == DRK_FP8_E4M3) && a.D / 64 > 8)
@@ -539,6 +549,7 @@ static int launch_decode(const drk_kv_layout *g, const void *q, const void *pool
 #undef GO
         DRK_LAUNCH_CHECK("decode_portable_kernel");
     }
+    if (g_time_kernel) DRK_HIP(hipEventRecord(g_ev1, st));
     hipLaunchKernelGGL(decode_merge_kernel, dim3(a.QH, B), dim3(a.D), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                        d_seq_lens, seq_len_host, causal_base, split, S, a.D, a.QH, io_dtype);
     DRK_LAUNCH_CHECK("decode_merge_kernel");
@@ -573,6 +584,18 @@ int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len)
 }
 
 void drk_debug_force_portable_decode(int on) { g_force_portable = on ? 1 : 0; }
+
+void drk_debug_time_decode_kernel(int on) { g_time_kernel = on ? 1 : 0; }
+void drk_debug_set_decode_lds_pad(int bytes) { g_lds_pad = bytes > 0 ? bytes : 0; }
+
+int drk_debug_last_decode_kernel_ms(float *ms)
+{
+    if (!ms) return fail(DRK_ERR_INVALID, "ms is NULL");
+    if (!g_ev0) return fail(DRK_ERR_INVALID, "no timed decode launch yet");
+    DRK_HIP(hipEventSynchronize(g_ev1));
+    DRK_HIP(hipEventElapsedTime(ms, g_ev0, g_ev1));
+    return DRK_OK;
+}
 
 int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void *pool,
                                const int32_t *d_block_table, void *out, int layer, int seq_len, float scale,

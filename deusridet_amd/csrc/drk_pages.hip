@@ -243,12 +243,14 @@ __global__ __launch_bounds__(kThreads) void copy_blocks_kernel(Lay a, uint8_t *_
     }
 }
 
-// importance_update_kernel, importance_scorer.cu:27-36
+// importance_update_kernel, importance_scorer.cu:27-36: score*decay + new.  The
+// reference is built by nvcc, which contracts that expression into one fused
+// multiply-add; the fused form is written out here so the rounding is fixed.
 __global__ void importance_update_kernel(float *__restrict__ scores, const float *__restrict__ new_scores,
                                          int n, float decay)
 {
     int b = blockIdx.x * blockDim.x + threadIdx.x;
-    if (b < n) scores[b] = __fadd_rn(__fmul_rn(scores[b], decay), new_scores[b]);
+    if (b < n) scores[b] = __builtin_fmaf(scores[b], decay, new_scores[b]);
 }
 
 static int check_src_dtype(int d)

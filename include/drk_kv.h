@@ -69,6 +69,12 @@ const char *drk_last_error(void);
 const char *drk_strerror(int code);
 int         drk_device_count(int *count);
 
+/* Measurement aid (precedent tools/probe_bw.cu:74-97): sustained GB/s of a plain
+ * 128-bit streaming read of `bytes` of device memory on the default stream,
+ * 5 warm-up + `iters` timed passes; d_sink is 4 bytes of device memory.
+ * Synchronises. */
+int drk_probe_read_bandwidth(const void *d_ptr, size_t bytes, int iters, void *d_sink, float *gbps);
+
 /* ---- layout arithmetic (host only, no GPU needed) --------------------- */
 /* block_pool.cpp:23-39: strides; block_pool.cpp:28-32: budget -> max_blocks */
 int drk_kv_layout_check(const drk_kv_layout *g);
@@ -149,6 +155,14 @@ int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len);
  * geometry, any storage type) instead of the tiled one, so that tests can
  * check the two against each other.  Process-wide, not thread-safe. */
 void drk_debug_force_portable_decode(int on);
+/* Diagnostic for benchmarks: while on, every decode launch records a HIP event
+ * on its stream right before and right after the split-K partial kernel (the
+ * merge kernel is outside the pair); drk_debug_last_decode_kernel_ms waits for
+ * the last pair and returns the elapsed milliseconds.  Process-wide. */
+void drk_debug_time_decode_kernel(int on);
+/* Diagnostic: extra dynamic LDS bytes per decode workgroup (lowers occupancy). */
+void drk_debug_set_decode_lds_pad(int bytes);
+int  drk_debug_last_decode_kernel_ms(float *ms);
 /* paged_gqa_decode_attention, paged_attention.cu:179-282: one sequence.
  * q/out [num_q_heads, head_dim] of io_dtype (F16/BF16). */
 int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void *pool,

@@ -565,9 +565,11 @@ void orc_decode_branches(const orc_layout *g, const uint16_t *Q, const void *poo
 /* importance scorer -- importance_scorer.cu:27-36 (update), 75-87 (argmin)  */
 /* ======================================================================== */
 
+/* nvcc's default (-fmad=true) contracts score*decay + new into one fused
+ * multiply-add, so the restatement uses fmaf: one rounding. */
 void orc_importance_update(float *scores, const float *new_scores, int n, float decay)
 {
-    for (int b = 0; b < n; b++) scores[b] = scores[b] * decay + new_scores[b];
+    for (int b = 0; b < n; b++) scores[b] = fmaf(scores[b], decay, new_scores[b]);
 }
 
 int orc_least_important(const float *scores, const int *ids, int n)

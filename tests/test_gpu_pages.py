@@ -61,8 +61,8 @@ def test_config1_append_and_gather(dev):
     assert np.array_equal(U.host(dpool, np.uint8), opool)
     # gathered K/V, bit exact, against the oracle and against the source itself
     flat = U.dev_zeros(2 * 512 * 4 * 128 * 2)
-    cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(dpool), U.p(U.dev_i32(table)), 0, 512, 1,
-              U.stream_ptr())
+    dtab = U.dev_i32(table)
+    cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(dpool), U.p(dtab), 0, 512, 1, U.stream_ptr())
     U.sync()
     got = U.host(flat, np.uint16, (1, 2, 512, 4, 128))
     want, _ = orc.extract(og, opool, table, 0, 512, 1)
@@ -139,8 +139,9 @@ def test_quantising_append_bit_exact(dev, dtype, src_dtype):
     for l in range(L):
         orc.append_batch(og, opool, table, l, 3, kb[l], vb[l], src_dtype)
     dpool = U.dev_zeros(orc.pool_bytes(og))
-    cabi.call("drk_kv_append_batch", C.byref(g), U.p(dpool), U.p(U.dev_i32(table)), 0, L, 3, M,
-              U.p(U.dev_bytes(kb)), U.p(U.dev_bytes(vb)), src_dtype, U.stream_ptr())
+    dtab, dk, dv = U.dev_i32(table), U.dev_bytes(kb), U.dev_bytes(vb)      # keep the buffers alive
+    cabi.call("drk_kv_append_batch", C.byref(g), U.p(dpool), U.p(dtab), 0, L, 3, M, U.p(dk), U.p(dv), src_dtype,
+              U.stream_ptr())
     U.sync()
     got = U.host(dpool, np.uint8)
     bad = np.nonzero(got != opool)[0]
@@ -166,9 +167,9 @@ def test_fp8_codes_exhaustive(dev, src_dtype):
     opool = orc.new_pool(og)
     orc.append_batch(og, opool, table, 0, 0, src, src, src_dtype)
     dpool = U.dev_zeros(orc.pool_bytes(og))
-    d = U.dev_bytes(src)
-    cabi.call("drk_kv_append_batch", C.byref(g), U.p(dpool), U.p(U.dev_i32(table)), 0, 1, 0, M, U.p(d), U.p(d),
-              src_dtype, U.stream_ptr())
+    d, dtab = U.dev_bytes(src), U.dev_i32(table)
+    cabi.call("drk_kv_append_batch", C.byref(g), U.p(dpool), U.p(dtab), 0, 1, 0, M, U.p(d), U.p(d), src_dtype,
+              U.stream_ptr())
     U.sync()
     assert np.array_equal(U.host(dpool, np.uint8), opool)
 
@@ -197,8 +198,8 @@ def test_extract_inject_roundtrip_and_holes(dev, geom, dtype):
     dpool = U.dev_zeros(orc.pool_bytes(og))
     dtab = U.dev_i32(table)
     dsc = U.dev_bytes(scales) if scales is not None else None
-    cabi.call("drk_kv_inject", C.byref(g), U.p(dpool), U.p(U.dev_bytes(flat)), U.p(dsc), U.p(dtab), start, T, L,
-              U.stream_ptr())
+    dflat = U.dev_bytes(flat)
+    cabi.call("drk_kv_inject", C.byref(g), U.p(dpool), U.p(dflat), U.p(dsc), U.p(dtab), start, T, L, U.stream_ptr())
     U.sync()
     assert np.array_equal(U.host(dpool, np.uint8), opool)
     out = U.dev_bytes(np.full(flat.size, 0xAB, dtype=np.uint8))
@@ -227,7 +228,8 @@ def test_copy_blocks(dev, dtype):
     for s, d in pairs:
         if s >= 0 and d >= 0 and s != d:
             orc.copy_block(og, opool, int(s), int(d))
-    cabi.call("drk_kv_copy_blocks", C.byref(g), U.p(dpool), U.p(U.dev_i32(pairs)), len(pairs), U.stream_ptr())
+    dpairs = U.dev_i32(pairs)
+    cabi.call("drk_kv_copy_blocks", C.byref(g), U.p(dpool), U.p(dpairs), len(pairs), U.stream_ptr())
     U.sync()
     assert np.array_equal(U.host(dpool, np.uint8), opool)
 
