@@ -1,0 +1,181 @@
+"""ctypes binding of the C shim over the C++ host classes (include/drk_host.h,
+deusridet_amd/lib/libdeusridet_memoria.so).  Method names follow the C++
+classes, which follow the reference's (src/memoria/cache_manager.h:52-169,
+block_pool.h:58-123, importance_scorer.h:25-67, machina/paged_attention.h:27-73).
+Raises ImportError when the library has not been built."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import cabi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdeusridet_memoria.so")
+
+_vp, _i32, _sz, _f32 = C.c_void_p, C.c_int32, C.c_size_t, C.c_float
+_ip = C.POINTER(C.c_int32)
+
+SIGNATURES = {
+    "drkh_set_attention_geometry": (_i32, [_i32] * 6),
+    "drkh_scorer_create": (_vp, []), "drkh_scorer_destroy": (None, [_vp]),
+    "drkh_scorer_init": (_i32, [_vp, _i32, _f32]), "drkh_scorer_init_detached": (_i32, [_vp, _i32, _f32]),
+    "drkh_scorer_update": (None, [_vp, _vp, _i32]), "drkh_scorer_least_important": (_i32, [_vp, _vp, _i32]),
+    "drkh_scorer_score": (_f32, [_vp, _i32]), "drkh_scorer_sync_to_host": (None, [_vp]),
+    "drkh_scorer_load_host_scores": (None, [_vp, _vp, _i32]),
+    "drkh_cm_create": (_vp, []), "drkh_cm_destroy": (None, [_vp]),
+    "drkh_cm_init": (_i32, [_vp, _sz, _i32, _vp, _i32]),
+    "drkh_cm_init_detached": (_i32, [_vp, _i32, _i32, _vp, _i32]),
+    "drkh_cm_ensure_blocks_for": (_i32, [_vp, _i32, _i32]),
+    "drkh_cm_ensure_blocks_for_range": (_i32, [_vp, _i32, _i32, _i32]),
+    "drkh_cm_sync_block_table": (None, [_vp, _vp]),
+    "drkh_cm_d_block_table": (_vp, [_vp, _i32]), "drkh_cm_h_block_table": (_ip, [_vp, _i32]),
+    "drkh_cm_table_stride": (_i32, [_vp]),
+    "drkh_cm_seq_len": (_i32, [_vp, _i32]), "drkh_cm_set_seq_len": (None, [_vp, _i32, _i32]),
+    "drkh_cm_num_logical_blocks": (_i32, [_vp, _i32]),
+    "drkh_cm_fork_branch": (_i32, [_vp, _i32, _i32]), "drkh_cm_release_branch": (None, [_vp, _i32]),
+    "drkh_cm_touch_block": (None, [_vp, _i32, _i32]), "drkh_cm_block_location": (_i32, [_vp, _i32, _i32]),
+    "drkh_cm_evict_blocks": (_i32, [_vp, _i32]), "drkh_cm_ensure_free_blocks": (_i32, [_vp, _i32]),
+    "drkh_cm_gpu_blocks_used": (_i32, [_vp]), "drkh_cm_free_blocks": (_i32, [_vp]),
+    "drkh_cm_lru_snapshot": (_i32, [_vp, _vp, _vp, _i32]),
+    "drkh_cm_take_pending_copies": (_i32, [_vp, _vp, _vp, _i32]),
+    "drkh_pool_alloc_block": (_i32, [_vp]), "drkh_pool_free_block": (None, [_vp, _i32]),
+    "drkh_pool_free_count": (_i32, [_vp]), "drkh_pool_max_blocks": (_i32, [_vp]),
+    "drkh_pool_block_size": (_i32, [_vp]), "drkh_pool_refcount": (_i32, [_vp, _i32]),
+    "drkh_pool_ptr": (_vp, [_vp]), "drkh_pool_k_offset": (_sz, [_vp, _i32, _i32]),
+    "drkh_pool_v_offset": (_sz, [_vp, _i32, _i32]), "drkh_pool_total_bytes": (_sz, [_vp]),
+    "drkh_pool_free_stack": (_i32, [_vp, _vp, _i32]),
+    "drkh_paged_kv_cache_write": (None, [_vp, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp]),
+    "drkh_paged_kv_cache_write_batch": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "drkh_paged_kv_cache_write_branches": (None, [_vp, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _vp]),
+    "drkh_paged_gqa_decode_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp]),
+    "drkh_paged_gqa_decode_attention_branches": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _i32,
+                                                        _i32, _f32, _vp]),
+    "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
+    "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32]),
+    "drkh_invoke_extract_kv_from_pages": (None, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "drkh_invoke_inject_kv_to_pages": (None, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+}
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        cabi.lib()
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is missing: run __graft_entry__.build() or make -C deusridet_amd/host")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def set_attention_geometry(num_fa_layers, num_attn_heads, num_kv_heads, head_dim, kv_dtype=cabi.F16, io_dtype=-1):
+    return bool(lib().drkh_set_attention_geometry(num_fa_layers, num_attn_heads, num_kv_heads, head_dim, kv_dtype,
+                                                  io_dtype))
+
+
+class ImportanceScorer:
+    def __init__(self):
+        self._h = lib().drkh_scorer_create()
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().drkh_scorer_destroy(self._h)
+            self._h = None
+
+    def init(self, max_blocks, decay=0.95): return bool(lib().drkh_scorer_init(self._h, max_blocks, decay))
+    def init_detached(self, max_blocks, decay=0.95): return bool(lib().drkh_scorer_init_detached(self._h, max_blocks, decay))
+    def update(self, d_scores_ptr, n): lib().drkh_scorer_update(self._h, d_scores_ptr, n)
+    def score(self, b): return lib().drkh_scorer_score(self._h, b)
+    def sync_to_host(self): lib().drkh_scorer_sync_to_host(self._h)
+
+    def least_important(self, ids):
+        a = np.ascontiguousarray(ids, dtype=np.int32)
+        return lib().drkh_scorer_least_important(self._h, _p(a), a.shape[0])
+
+    def load_host_scores(self, scores):
+        a = np.ascontiguousarray(scores, dtype=np.float32)
+        lib().drkh_scorer_load_host_scores(self._h, _p(a), a.shape[0])
+
+
+class CacheManager:
+    GPU, INVALID, SSD = 0, -1, -2
+
+    def __init__(self):
+        self._h = lib().drkh_cm_create()
+        self._scorer = None
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().drkh_cm_destroy(self._h)
+            self._h = None
+
+    def init(self, kv_budget_bytes, block_size=256, scorer=None, max_branches=1):
+        self._scorer = scorer
+        return bool(lib().drkh_cm_init(self._h, int(kv_budget_bytes), block_size, scorer._h if scorer else None,
+                                       max_branches))
+
+    def init_detached(self, max_blocks, block_size, scorer=None, max_branches=1):
+        self._scorer = scorer
+        return bool(lib().drkh_cm_init_detached(self._h, max_blocks, block_size, scorer._h if scorer else None,
+                                                max_branches))
+
+    def ensure_blocks_for(self, branch, pos): return bool(lib().drkh_cm_ensure_blocks_for(self._h, branch, pos))
+    def ensure_blocks_for_range(self, branch, pos, M): return bool(lib().drkh_cm_ensure_blocks_for_range(self._h, branch, pos, M))
+    def sync_block_table(self, stream=None): lib().drkh_cm_sync_block_table(self._h, stream)
+    def d_block_table(self, branch=0): return lib().drkh_cm_d_block_table(self._h, branch)
+    def table_stride(self): return lib().drkh_cm_table_stride(self._h)
+    def seq_len(self, branch=0): return lib().drkh_cm_seq_len(self._h, branch)
+    def set_seq_len(self, branch, n): lib().drkh_cm_set_seq_len(self._h, branch, n)
+    def num_logical_blocks(self, branch=0): return lib().drkh_cm_num_logical_blocks(self._h, branch)
+    def fork_branch(self, parent, pos): return lib().drkh_cm_fork_branch(self._h, parent, pos)
+    def release_branch(self, branch): lib().drkh_cm_release_branch(self._h, branch)
+    def touch_block(self, branch, logical): lib().drkh_cm_touch_block(self._h, branch, logical)
+    def block_location(self, branch, logical): return lib().drkh_cm_block_location(self._h, branch, logical)
+    def evict_blocks(self, n): return lib().drkh_cm_evict_blocks(self._h, n)
+    def ensure_free_blocks(self, n): return bool(lib().drkh_cm_ensure_free_blocks(self._h, n))
+    def gpu_blocks_used(self): return lib().drkh_cm_gpu_blocks_used(self._h)
+    def free_blocks(self): return lib().drkh_cm_free_blocks(self._h)
+
+    def h_block_table(self, branch=0):
+        p = lib().drkh_cm_h_block_table(self._h, branch)
+        return np.ctypeslib.as_array(p, shape=(self.table_stride(),)).copy()
+
+    def lru_snapshot(self):
+        cap = self.pool_max_blocks() * 64 + 16
+        bo, lo = np.empty(cap, dtype=np.int32), np.empty(cap, dtype=np.int32)
+        n = lib().drkh_cm_lru_snapshot(self._h, _p(bo), _p(lo), cap)
+        return list(zip(bo[:n].tolist(), lo[:n].tolist()))
+
+    def take_pending_copies(self):
+        cap = 65536
+        so, dn = np.empty(cap, dtype=np.int32), np.empty(cap, dtype=np.int32)
+        n = lib().drkh_cm_take_pending_copies(self._h, _p(so), _p(dn), cap)
+        return list(zip(so[:n].tolist(), dn[:n].tolist()))
+
+    # BlockPool
+    def pool_alloc_block(self): return lib().drkh_pool_alloc_block(self._h)
+    def pool_free_block(self, i): lib().drkh_pool_free_block(self._h, i)
+    def pool_free_count(self): return lib().drkh_pool_free_count(self._h)
+    def pool_max_blocks(self): return lib().drkh_pool_max_blocks(self._h)
+    def pool_block_size(self): return lib().drkh_pool_block_size(self._h)
+    def pool_refcount(self, i): return lib().drkh_pool_refcount(self._h, i)
+    def pool_ptr(self): return lib().drkh_pool_ptr(self._h)
+    def pool_k_offset(self, layer, block): return lib().drkh_pool_k_offset(self._h, layer, block)
+    def pool_v_offset(self, layer, block): return lib().drkh_pool_v_offset(self._h, layer, block)
+    def pool_total_bytes(self): return lib().drkh_pool_total_bytes(self._h)
+
+    def pool_free_stack(self):
+        cap = self.pool_max_blocks()
+        out = np.empty(max(cap, 1), dtype=np.int32)
+        n = lib().drkh_pool_free_stack(self._h, _p(out), cap)
+        return out[:n].copy()

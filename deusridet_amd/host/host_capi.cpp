@@ -1,0 +1,166 @@
+// host_capi.cpp -- the C shim declared in include/drk_host.h: one-line forwarders
+// to the C++ host classes.
+#include "drk_host.h"
+
+#include "../machina/paged_attention.h"
+#include "../memoria/cache_kernels.h"
+#include "../memoria/cache_manager.h"
+
+#include <algorithm>
+
+using namespace deusridet;
+
+#define CM(p) (static_cast<CacheManager *>(p))
+#define SC(p) (static_cast<ImportanceScorer *>(p))
+#define H(p) (reinterpret_cast<__half *>(p))
+#define CH(p) (reinterpret_cast<const __half *>(p))
+#define ST(p) (static_cast<hipStream_t>(p))
+
+extern "C" {
+
+int drkh_set_attention_geometry(int num_fa_layers, int num_attn_heads, int num_kv_heads, int head_dim, int kv_dtype,
+                                int io_dtype)
+{
+    return ModelConfig::set_attention_geometry(num_fa_layers, num_attn_heads, num_kv_heads, head_dim, kv_dtype,
+                                               io_dtype) ? 1 : 0;
+}
+
+void *drkh_scorer_create(void) { return new ImportanceScorer(); }
+void drkh_scorer_destroy(void *s) { delete SC(s); }
+int drkh_scorer_init(void *s, int max_blocks, float decay) { return SC(s)->init(max_blocks, decay) ? 1 : 0; }
+int drkh_scorer_init_detached(void *s, int max_blocks, float decay) { return SC(s)->init_detached(max_blocks, decay) ? 1 : 0; }
+void drkh_scorer_update(void *s, const float *d, int n) { SC(s)->update(d, n); }
+int drkh_scorer_least_important(void *s, const int *ids, int n) { return SC(s)->least_important(ids, n); }
+float drkh_scorer_score(void *s, int b) { return SC(s)->score(b); }
+void drkh_scorer_sync_to_host(void *s) { SC(s)->sync_to_host(); }
+void drkh_scorer_load_host_scores(void *s, const float *scores, int n) { SC(s)->load_host_scores(scores, n); }
+
+void *drkh_cm_create(void) { return new CacheManager(); }
+void drkh_cm_destroy(void *cm) { delete CM(cm); }
+int drkh_cm_init(void *cm, size_t budget, int block_size, void *scorer, int max_branches)
+{
+    return CM(cm)->init(budget, "", block_size, nullptr, SC(scorer), max_branches) ? 1 : 0;
+}
+int drkh_cm_init_detached(void *cm, int max_blocks, int block_size, void *scorer, int max_branches)
+{
+    return CM(cm)->init_detached(max_blocks, block_size, SC(scorer), max_branches) ? 1 : 0;
+}
+int drkh_cm_ensure_blocks_for(void *cm, int branch, int pos) { return CM(cm)->ensure_blocks_for(branch, pos) ? 1 : 0; }
+int drkh_cm_ensure_blocks_for_range(void *cm, int branch, int pos_start, int M)
+{
+    return CM(cm)->ensure_blocks_for_range(branch, pos_start, M) ? 1 : 0;
+}
+void drkh_cm_sync_block_table(void *cm, void *stream) { CM(cm)->sync_block_table(ST(stream)); }
+const int32_t *drkh_cm_d_block_table(void *cm, int branch) { return CM(cm)->d_block_table(branch); }
+const int32_t *drkh_cm_h_block_table(void *cm, int branch) { return CM(cm)->h_block_table(branch); }
+int drkh_cm_table_stride(void *cm) { return CM(cm)->table_stride(); }
+int drkh_cm_seq_len(void *cm, int branch) { return CM(cm)->seq_len(branch); }
+void drkh_cm_set_seq_len(void *cm, int branch, int len) { CM(cm)->set_seq_len(branch, len); }
+int drkh_cm_num_logical_blocks(void *cm, int branch) { return CM(cm)->num_logical_blocks(branch); }
+int drkh_cm_fork_branch(void *cm, int parent, int pos) { return CM(cm)->fork_branch(parent, pos); }
+void drkh_cm_release_branch(void *cm, int branch) { CM(cm)->release_branch(branch); }
+void drkh_cm_touch_block(void *cm, int branch, int logical) { CM(cm)->touch_block(branch, logical); }
+int drkh_cm_block_location(void *cm, int branch, int logical) { return (int)CM(cm)->block_location(branch, logical); }
+int drkh_cm_evict_blocks(void *cm, int n) { return CM(cm)->evict_blocks(n); }
+int drkh_cm_ensure_free_blocks(void *cm, int n_free) { return CM(cm)->ensure_free_blocks(n_free) ? 1 : 0; }
+int drkh_cm_gpu_blocks_used(void *cm) { return CM(cm)->gpu_blocks_used(); }
+int drkh_cm_free_blocks(void *cm) { return CM(cm)->free_blocks(); }
+
+int drkh_cm_lru_snapshot(void *cm, int32_t *bo, int32_t *lo, int cap)
+{
+    auto v = CM(cm)->lru_snapshot();
+    int n = std::min<int>(cap, (int)v.size());
+    for (int i = 0; i < n; i++) { bo[i] = v[i].first; lo[i] = v[i].second; }
+    return (int)v.size();
+}
+int drkh_cm_take_pending_copies(void *cm, int32_t *so, int32_t *dn, int cap)
+{
+    auto v = CM(cm)->take_pending_copies();
+    int n = std::min<int>(cap, (int)v.size());
+    for (int i = 0; i < n; i++) { so[i] = v[i].first; dn[i] = v[i].second; }
+    return (int)v.size();
+}
+
+int drkh_pool_alloc_block(void *cm) { return CM(cm)->block_pool().alloc_block(); }
+void drkh_pool_free_block(void *cm, int id) { CM(cm)->block_pool().free_block(id); }
+int drkh_pool_free_count(void *cm) { return CM(cm)->block_pool().free_count(); }
+int drkh_pool_max_blocks(void *cm) { return CM(cm)->block_pool().max_blocks(); }
+int drkh_pool_block_size(void *cm) { return CM(cm)->block_pool().block_size(); }
+int drkh_pool_refcount(void *cm, int id) { return CM(cm)->block_pool().refcount(id); }
+void *drkh_pool_ptr(void *cm) { return CM(cm)->block_pool().pool_raw(); }
+size_t drkh_pool_k_offset(void *cm, int layer, int block) { return CM(cm)->block_pool().k_offset(layer, block); }
+size_t drkh_pool_v_offset(void *cm, int layer, int block) { return CM(cm)->block_pool().v_offset(layer, block); }
+size_t drkh_pool_total_bytes(void *cm) { return CM(cm)->block_pool().total_bytes(); }
+int drkh_pool_free_stack(void *cm, int32_t *out, int cap)
+{
+    auto v = CM(cm)->block_pool().free_stack_snapshot();
+    int n = std::min<int>(cap, (int)v.size());
+    for (int i = 0; i < n; i++) out[i] = v[i];
+    return (int)v.size();
+}
+
+void drkh_paged_kv_cache_write(const void *src_k, const void *src_v, void *kv_pool, const int32_t *d_block_table,
+                               int fa_layer_idx, const int32_t *d_pos, int max_phys_blocks, int block_size,
+                               void *stream)
+{
+    paged_kv_cache_write(CH(src_k), CH(src_v), H(kv_pool), d_block_table, fa_layer_idx, d_pos, max_phys_blocks,
+                         block_size, ST(stream));
+}
+void drkh_paged_kv_cache_write_batch(const void *src_k, const void *src_v, void *kv_pool,
+                                     const int32_t *d_block_table, int fa_layer_idx, int pos_start, int M,
+                                     int max_phys_blocks, int block_size, void *stream)
+{
+    paged_kv_cache_write_batch(CH(src_k), CH(src_v), H(kv_pool), d_block_table, fa_layer_idx, pos_start, M,
+                               max_phys_blocks, block_size, ST(stream));
+}
+void drkh_paged_kv_cache_write_branches(const void *src_k, const void *src_v, void *kv_pool,
+                                        const int32_t *d_tables, int table_stride, const int32_t *d_pos, int B,
+                                        int fa_layer_idx, int max_phys_blocks, int block_size, void *stream)
+{
+    paged_kv_cache_write_branches(CH(src_k), CH(src_v), H(kv_pool), d_tables, table_stride, d_pos, B, fa_layer_idx,
+                                  max_phys_blocks, block_size, ST(stream));
+}
+void drkh_paged_gqa_decode_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
+                                     int fa_layer_idx, int seq_len, int max_phys_blocks, int block_size,
+                                     float scale, void *stream)
+{
+    paged_gqa_decode_attention(CH(Q), H(kv_pool), d_block_table, H(out), fa_layer_idx, seq_len, max_phys_blocks,
+                               block_size, scale, ST(stream));
+}
+void drkh_paged_gqa_decode_attention_branches(const void *Q, void *kv_pool, const int32_t *d_tables,
+                                              int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len,
+                                              void *out, int fa_layer_idx, int max_phys_blocks, int block_size,
+                                              float scale, void *stream)
+{
+    paged_gqa_decode_attention_branches(CH(Q), H(kv_pool), d_tables, table_stride, d_seq_lens, B, max_seq_len,
+                                        H(out), fa_layer_idx, max_phys_blocks, block_size, scale, ST(stream));
+}
+void drkh_paged_prefill_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
+                                  int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
+                                  float scale, void *stream)
+{
+    paged_prefill_attention(CH(Q), H(kv_pool), d_block_table, H(out), fa_layer_idx, pos_start, M, max_phys_blocks,
+                            block_size, scale, ST(stream));
+}
+int drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size)
+{
+    return paged_attention_reserve_workspace(max_branches, max_seq_len, max_prefill_rows, block_size) ? 1 : 0;
+}
+void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,
+                                       int num_tokens, int num_layers, int num_kv_heads, int head_dim,
+                                       int block_size, int max_phys_blocks, void *stream)
+{
+    invoke_extract_kv_from_pages_typed(dst, nullptr, kv_pool, block_table, start_token, num_tokens, num_layers,
+                                       num_kv_heads, head_dim, block_size, max_phys_blocks, ModelConfig::KV_DTYPE,
+                                       ST(stream));
+}
+void drkh_invoke_inject_kv_to_pages(void *kv_pool, const void *src, const int32_t *block_table, int start_token,
+                                    int num_tokens, int num_layers, int num_kv_heads, int head_dim, int block_size,
+                                    int max_phys_blocks, void *stream)
+{
+    invoke_inject_kv_to_pages_typed(kv_pool, src, nullptr, block_table, start_token, num_tokens, num_layers,
+                                    num_kv_heads, head_dim, block_size, max_phys_blocks, ModelConfig::KV_DTYPE,
+                                    ST(stream));
+}
+
+} // extern "C"

@@ -1,0 +1,31 @@
+// model.h -- the part of the reference's ModelConfig that the paged-KV path
+// reads (src/machina/model.h:30-73): runtime statics for the attention geometry.
+// The reference fills them from a model's config.json (src/machina/model.cpp:
+// 127-221); here set_attention_geometry() does it, because this build ships the
+// KV-cache path only, not the model loader.
+#pragma once
+
+#include "drk_kv.h"
+
+namespace deusridet {
+
+struct ModelConfig {
+    static int NUM_ATTN_HEADS;   // model.h:39
+    static int NUM_KV_HEADS;     // model.h:40
+    static int HEAD_DIM;         // model.h:41
+    static int NUM_KV_GROUPS;    // model.h:42, ATTN_HEADS / KV_HEADS
+    static int NUM_FA_LAYERS;    // model.h:73
+    // Not in the reference (its cache is fp16 only): storage type of the pool and
+    // element type of Q / out / append sources, DRK_* from drk_kv.h.
+    static int KV_DTYPE;         // DRK_F16 (default), DRK_BF16, DRK_INT8, DRK_FP8_E4M3
+    static int IO_DTYPE;         // DRK_F16 (default) or DRK_BF16
+
+    // Returns false (and changes nothing) when the numbers are inconsistent.
+    static bool set_attention_geometry(int num_fa_layers, int num_attn_heads, int num_kv_heads, int head_dim,
+                                       int kv_dtype = DRK_F16, int io_dtype = -1);
+
+    // The C-ABI layout for a pool of max_phys_blocks blocks of block_size tokens.
+    static drk_kv_layout layout(int max_phys_blocks, int block_size);
+};
+
+} // namespace deusridet

@@ -1,0 +1,66 @@
+// paged_attention.h -- paged KV-cache write and paged GQA attention.  The first
+// three functions have the reference's names, parameter order and meaning
+// (src/machina/paged_attention.h:27-73) with HIP vocabulary types; head counts
+// and head_dim come from ModelConfig's runtime statics exactly as in the
+// reference's launchers (paged_attention.cu:110-114, 276-281).  Element types:
+// ModelConfig::KV_DTYPE for the pool, ModelConfig::IO_DTYPE for Q / out / sources
+// (both fp16 by default, as in the reference); the `__half*` in the signatures
+// is then just "16-bit element".
+//
+// Launchers return void, are asynchronous on `stream`, and log a failure
+// (the reference's launchers check nothing).  Order of use is write-then-attend:
+// the token written at `pos` is visible to its own query, seq_len = pos + 1
+// (paged_attention.cu:359-368, stream.cpp:319-334).
+//
+// The two full-layer wrappers of the reference (full_attention_forward_paged*,
+// paged_attention.h:75-106) run projections, norms and RoPE around these calls;
+// they belong to the model code and keep calling the functions below.
+#pragma once
+
+#include "model.h"
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime_api.h>
+
+namespace deusridet {
+
+// ---- the reference's entry points --------------------------------------------
+void paged_kv_cache_write(const __half* src_k, const __half* src_v, __half* kv_pool, const int* d_block_table,
+                          int fa_layer_idx, const int* d_pos, int max_phys_blocks, int block_size,
+                          hipStream_t stream = 0);
+
+void paged_kv_cache_write_batch(const __half* src_k, const __half* src_v, __half* kv_pool, const int* d_block_table,
+                                int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
+                                hipStream_t stream = 0);
+
+void paged_gqa_decode_attention(const __half* Q, __half* kv_pool, const int* d_block_table, __half* out,
+                                int fa_layer_idx, int seq_len, int max_phys_blocks, int block_size, float scale,
+                                hipStream_t stream = 0);
+
+// The attention step of the reference's prefill wrapper (static kernel launched at
+// paged_attention.cu:621-630): Q/out [M, NUM_ATTN_HEADS, HEAD_DIM], row t sees
+// tokens 0 .. pos_start + t.
+void paged_prefill_attention(const __half* Q, __half* kv_pool, const int* d_block_table, __half* out,
+                             int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
+                             float scale, hipStream_t stream = 0);
+
+// ---- several decode branches in one launch (not in the reference) ------------
+// d_tables [B, table_stride] (CacheManager::d_block_tables()), d_pos / d_seq_lens
+// [B] on the device, src [B, NUM_KV_HEADS, HEAD_DIM], Q/out [B, NUM_ATTN_HEADS,
+// HEAD_DIM]; max_seq_len bounds every d_seq_lens[b].
+void paged_kv_cache_write_branches(const __half* src_k, const __half* src_v, __half* kv_pool, const int* d_tables,
+                                   int table_stride, const int* d_pos, int B, int fa_layer_idx,
+                                   int max_phys_blocks, int block_size, hipStream_t stream = 0);
+
+void paged_gqa_decode_attention_branches(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                         const int* d_seq_lens, int B, int max_seq_len, __half* out,
+                                         int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                         hipStream_t stream = 0);
+
+// The attention calls keep split-K partials in a device workspace that this
+// library owns and grows on demand (device allocation = implicit sync).  Call
+// this once up front with the largest shapes to keep the steady state free of
+// allocations, e.g. before capturing a HIP graph.  false on allocation failure.
+bool paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
+void paged_attention_release_workspace();
+
+} // namespace deusridet

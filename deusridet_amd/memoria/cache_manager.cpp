@@ -1,0 +1,428 @@
+// cache_manager.cpp -- see cache_manager.h.  Host bookkeeping only; the device is
+// reached through the C ABI (table upload, copy-on-write block copies).
+#include "cache_manager.h"
+#include "../communis/log.h"
+
+#include <algorithm>
+#include <unordered_set>
+
+namespace deusridet {
+
+CacheManager::~CacheManager() { destroy(); }
+
+bool CacheManager::setup_tables(int max_branches)
+{
+    if (max_branches < 1) max_branches = 1;
+    max_branches_ = max_branches;
+    // twice the physical blocks of logical space (cache_manager.cpp:37-39)
+    max_logical_blocks_ = pool_.max_blocks() * 2;
+    size_t cells = (size_t)max_branches_ * max_logical_blocks_;
+    h_tables_.assign(cells, -1);
+    location_.assign(cells, BlockLocation::INVALID);
+    stamp_.assign(cells, 0);
+    next_stamp_ = 1;
+    evictable_.clear();
+    refs_.assign(pool_.max_blocks(), {});
+    seq_len_.assign(max_branches_, 0);
+    alive_.assign(max_branches_, 0);
+    alive_[0] = 1;
+    dirty_lo_.assign(max_branches_, max_logical_blocks_);
+    dirty_hi_.assign(max_branches_, 0);
+    pending_copies_.clear();
+    return true;
+}
+
+bool CacheManager::init(size_t kv_budget_bytes, const std::string& cache_dir, int block_size,
+                        KVSwapper* swapper, ImportanceScorer* scorer, int max_branches)
+{
+    destroy();
+    block_size_ = block_size;
+    scorer_ = scorer;
+    detached_ = false;
+    if (swapper || !cache_dir.empty())
+        LOG_WARN("Memoria", "CacheManager: the SSD tier is not part of this build; cache_dir/swapper ignored, "
+                            "evicted blocks are discarded");
+    if (!pool_.init(kv_budget_bytes, block_size)) return false;
+    setup_tables(max_branches);
+
+    size_t table_bytes = (size_t)max_branches_ * max_logical_blocks_ * sizeof(int);
+    void* p = nullptr;
+    if (drk_dev_malloc(&p, table_bytes) != DRK_OK) {
+        LOG_ERROR("Memoria", "CacheManager: d_block_table alloc failed: %s", drk_last_error());
+        destroy();
+        return false;
+    }
+    d_tables_ = static_cast<int*>(p);
+    pairs_capacity_ = 1024;
+    if (drk_dev_malloc(&p, (size_t)pairs_capacity_ * 2 * sizeof(int)) != DRK_OK) {
+        LOG_ERROR("Memoria", "CacheManager: copy staging alloc failed: %s", drk_last_error());
+        destroy();
+        return false;
+    }
+    d_pairs_ = static_cast<int*>(p);
+    // -1 everywhere (cache_manager.cpp:53)
+    if (drk_dev_memset_async(d_tables_, 0xFF, table_bytes, nullptr) != DRK_OK ||
+        drk_stream_synchronize(nullptr) != DRK_OK) {
+        LOG_ERROR("Memoria", "CacheManager: table init failed: %s", drk_last_error());
+        destroy();
+        return false;
+    }
+    LOG_INFO("Memoria", "CacheManager: %d phys blocks, %d max logical, %d branches, SSD=disabled",
+             pool_.max_blocks(), max_logical_blocks_, max_branches_);
+    return true;
+}
+
+bool CacheManager::init_detached(int max_blocks, int block_size, ImportanceScorer* scorer, int max_branches)
+{
+    destroy();
+    block_size_ = block_size;
+    scorer_ = scorer;
+    detached_ = true;
+    if (!pool_.init_detached(max_blocks, block_size)) return false;
+    return setup_tables(max_branches);
+}
+
+void CacheManager::mark_dirty(int branch, int logical)
+{
+    dirty_lo_[branch] = std::min(dirty_lo_[branch], logical);
+    dirty_hi_[branch] = std::max(dirty_hi_[branch], logical + 1);
+}
+
+// The cell takes a reference on `phys` that alloc_block()/retain() has already
+// counted in the pool.
+void CacheManager::attach_nolock(int c, int phys, bool fresh_stamp)
+{
+    h_tables_[c] = phys;
+    location_[c] = BlockLocation::GPU;
+    if (fresh_stamp || stamp_[c] == 0) stamp_[c] = next_stamp_++;
+    std::vector<int>& r = refs_[phys];
+    if (r.size() == 1) evictable_.erase({stamp_[r[0]], r[0]});   // the sole owner is now sharing
+    r.push_back(c);
+    if (r.size() == 1) evictable_.insert({stamp_[c], c});
+}
+
+// The cell gives up its reference; the block is freed when it was the last.
+void CacheManager::detach_nolock(int c)
+{
+    int phys = h_tables_[c];
+    std::vector<int>& r = refs_[phys];
+    if (r.size() == 1) evictable_.erase({stamp_[c], c});
+    r.erase(std::remove(r.begin(), r.end(), c), r.end());
+    pool_.release(phys);
+    if (r.size() == 1) evictable_.insert({stamp_[r[0]], r[0]});
+    h_tables_[c] = -1;
+}
+
+bool CacheManager::pick_victim_nolock(int& cell_out)
+{
+    if (evictable_.empty()) return false;
+    if (!scorer_) {                               // oldest first (cache_manager.cpp:203-204)
+        cell_out = evictable_.begin()->second;
+        return true;
+    }
+    // least important; the first minimum in LRU order wins (cache_manager.cpp:188-201,
+    // importance_scorer.cu:75-87)
+    bool have = false;
+    float best = 0.0f;
+    for (const auto& e : evictable_) {
+        float s = scorer_->score(e.second % max_logical_blocks_);
+        if (!have || s < best) {
+            have = true;
+            best = s;
+            cell_out = e.second;
+        }
+    }
+    return have;
+}
+
+int CacheManager::evict_nolock(int n)
+{
+    int evicted = 0;
+    while (evicted < n) {
+        int c;
+        if (!pick_victim_nolock(c)) break;
+        int branch = c / max_logical_blocks_, logical = c % max_logical_blocks_;
+        detach_nolock(c);                         // frees the block: it had one reference
+        location_[c] = BlockLocation::INVALID;
+        stamp_[c] = 0;
+        mark_dirty(branch, logical);
+        evicted++;
+    }
+    if (evicted > 0)
+        LOG_INFO("Memoria", "Evicted %d blocks (SSD=no), %d free now", evicted, pool_.free_count());
+    return evicted;
+}
+
+bool CacheManager::ensure_free_nolock(int n_free)
+{
+    while (pool_.free_count() < n_free) {
+        if (evict_nolock(1) == 0) return false;
+    }
+    return true;
+}
+
+int CacheManager::alloc_phys_nolock()
+{
+    int phys = pool_.alloc_block();
+    if (phys < 0) {                               // cache_manager.cpp:311-319
+        if (!ensure_free_nolock(1)) {
+            LOG_ERROR("Memoria", "Cannot allocate a block: pool exhausted, eviction failed");
+            return -1;
+        }
+        phys = pool_.alloc_block();
+    }
+    return phys;
+}
+
+bool CacheManager::ensure_nolock(int branch, int pos)
+{
+    if (branch < 0 || branch >= max_branches_ || !alive_[branch] || pos < 0) return false;
+    int logical = pos / block_size_;
+    if (logical >= max_logical_blocks_) {
+        LOG_ERROR("Memoria", "Position %d exceeds max logical blocks (%d)", pos, max_logical_blocks_);
+        return false;
+    }
+    int c = (int)cell(branch, logical);
+    if (location_[c] == BlockLocation::GPU) {
+        int phys = h_tables_[c];
+        if (pool_.refcount(phys) > 1) {
+            // copy-on-write: the write must not be seen by the other tables
+            int fresh = alloc_phys_nolock();
+            if (fresh < 0) return false;
+            pending_copies_.push_back({phys, fresh});
+            detach_nolock(c);                     // the old block keeps its other references
+            attach_nolock(c, fresh, false);       // same place in the LRU order
+            mark_dirty(branch, logical);
+        }
+        return true;
+    }
+    int phys = alloc_phys_nolock();
+    if (phys < 0) return false;
+    attach_nolock(c, phys, true);                 // cache_manager.cpp:321-323
+    mark_dirty(branch, logical);
+    return true;
+}
+
+bool CacheManager::ensure_blocks_for(int pos) { return ensure_blocks_for(0, pos); }
+bool CacheManager::ensure_blocks_for_range(int pos_start, int M) { return ensure_blocks_for_range(0, pos_start, M); }
+
+bool CacheManager::ensure_blocks_for(int branch, int pos)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    return ensure_nolock(branch, pos);
+}
+
+bool CacheManager::ensure_blocks_for_range(int branch, int pos_start, int M)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (M <= 0) return true;
+    int first = pos_start / block_size_, last = (pos_start + M - 1) / block_size_;
+    for (int b = first; b <= last; b++)
+        if (!ensure_nolock(branch, b * block_size_)) return false;
+    return true;
+}
+
+const int* CacheManager::d_block_table(int branch) const
+{
+    if (!d_tables_ || branch < 0 || branch >= max_branches_) return nullptr;
+    return d_tables_ + cell(branch, 0);
+}
+
+const int* CacheManager::h_block_table(int branch) const
+{
+    if (branch < 0 || branch >= max_branches_) return nullptr;
+    return h_tables_.data() + cell(branch, 0);
+}
+
+// Copies whose source is written by an earlier queued copy (or whose target is
+// touched by one) must not share a launch: the queue is cut into launches at
+// such dependencies and the launches are stream-ordered.
+void CacheManager::flush_copies(hipStream_t stream)
+{
+    size_t i = 0;
+    const drk_kv_layout& g = pool_.layout();
+    while (i < pending_copies_.size()) {
+        std::unordered_set<int> written, read;
+        std::vector<int> flat;
+        while (i < pending_copies_.size() && (int)flat.size() / 2 < pairs_capacity_) {
+            int s = pending_copies_[i].first, d = pending_copies_[i].second;
+            if (written.count(s) || written.count(d) || read.count(d)) break;
+            written.insert(d);
+            read.insert(s);
+            flat.push_back(s);
+            flat.push_back(d);
+            i++;
+        }
+        int n = (int)flat.size() / 2;
+        if (n == 0) break;
+        if (drk_memcpy_h2d_async(d_pairs_, flat.data(), flat.size() * sizeof(int), stream) != DRK_OK ||
+            drk_kv_copy_blocks(&g, pool_.pool_raw(), d_pairs_, n, stream) != DRK_OK)
+            LOG_ERROR("Memoria", "copy-on-write copy failed: %s", drk_last_error());
+    }
+    pending_copies_.clear();
+}
+
+void CacheManager::sync_block_table(hipStream_t stream)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (!detached_ && d_tables_) {
+        flush_copies(stream);
+        for (int b = 0; b < max_branches_; b++) {
+            if (dirty_hi_[b] <= dirty_lo_[b]) continue;
+            size_t off = cell(b, dirty_lo_[b]);
+            size_t bytes = (size_t)(dirty_hi_[b] - dirty_lo_[b]) * sizeof(int);
+            if (drk_memcpy_h2d_async(d_tables_ + off, h_tables_.data() + off, bytes, stream) != DRK_OK)
+                LOG_ERROR("Memoria", "block table upload failed: %s", drk_last_error());
+        }
+    }
+    for (int b = 0; b < max_branches_; b++) {
+        dirty_lo_[b] = max_logical_blocks_;
+        dirty_hi_[b] = 0;
+    }
+}
+
+int CacheManager::seq_len(int branch) const
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    return (branch >= 0 && branch < max_branches_) ? seq_len_[branch] : 0;
+}
+
+void CacheManager::set_seq_len(int branch, int len)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (branch >= 0 && branch < max_branches_) seq_len_[branch] = len;
+}
+
+int CacheManager::num_logical_blocks(int branch) const
+{
+    return (seq_len(branch) + block_size_ - 1) / block_size_;
+}
+
+int CacheManager::fork_branch(int parent, int pos)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (parent < 0 || parent >= max_branches_ || !alive_[parent] || pos < 0) return -1;
+    int id = -1;
+    for (int i = 0; i < max_branches_; i++)
+        if (!alive_[i]) { id = i; break; }
+    if (id < 0) return -1;
+    int nshared = (pos + block_size_ - 1) / block_size_;
+    if (nshared > max_logical_blocks_) return -1;
+    alive_[id] = 1;
+    seq_len_[id] = pos;
+    for (int l = 0; l < nshared; l++) {
+        int pc = (int)cell(parent, l), cc = (int)cell(id, l);
+        if (location_[pc] != BlockLocation::GPU) continue;   // a hole in the parent stays a hole
+        int phys = h_tables_[pc];
+        pool_.retain(phys);
+        attach_nolock(cc, phys, true);
+        mark_dirty(id, l);
+    }
+    return id;
+}
+
+void CacheManager::release_branch(int branch)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (branch < 0 || branch >= max_branches_ || !alive_[branch]) return;
+    for (int l = 0; l < max_logical_blocks_; l++) {
+        int c = (int)cell(branch, l);
+        if (location_[c] != BlockLocation::GPU) continue;
+        detach_nolock(c);
+        location_[c] = BlockLocation::INVALID;
+        stamp_[c] = 0;
+        mark_dirty(branch, l);
+    }
+    seq_len_[branch] = 0;
+    if (branch != 0) alive_[branch] = 0;
+}
+
+bool CacheManager::branch_alive(int branch) const
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    return branch >= 0 && branch < max_branches_ && alive_[branch];
+}
+
+void CacheManager::touch_block(int branch, int logical_idx)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (branch < 0 || branch >= max_branches_ || logical_idx < 0 || logical_idx >= max_logical_blocks_) return;
+    int c = (int)cell(branch, logical_idx);
+    if (location_[c] != BlockLocation::GPU) return;
+    bool sole = refs_[h_tables_[c]].size() == 1;
+    if (sole) evictable_.erase({stamp_[c], c});
+    stamp_[c] = next_stamp_++;
+    if (sole) evictable_.insert({stamp_[c], c});
+}
+
+BlockLocation CacheManager::block_location(int branch, int logical_idx) const
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (branch < 0 || branch >= max_branches_ || logical_idx < 0 || logical_idx >= max_logical_blocks_)
+        return BlockLocation::INVALID;
+    return location_[cell(branch, logical_idx)];
+}
+
+int CacheManager::evict_blocks(int n)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    return evict_nolock(n);
+}
+
+bool CacheManager::ensure_free_blocks(int n_free)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    return ensure_free_nolock(n_free);
+}
+
+void CacheManager::prefetch_block(int) {}
+
+int CacheManager::gpu_blocks_used() const { return pool_.max_blocks() - pool_.free_count(); }
+
+std::vector<std::pair<int, int>> CacheManager::lru_snapshot() const
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    std::vector<std::pair<uint64_t, int>> order;
+    for (size_t c = 0; c < stamp_.size(); c++)
+        if (stamp_[c]) order.push_back({stamp_[c], (int)c});
+    std::sort(order.begin(), order.end());
+    std::vector<std::pair<int, int>> out;
+    out.reserve(order.size());
+    for (const auto& e : order) out.push_back({e.second / max_logical_blocks_, e.second % max_logical_blocks_});
+    return out;
+}
+
+std::vector<std::pair<int, int>> CacheManager::take_pending_copies()
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    std::vector<std::pair<int, int>> out;
+    out.swap(pending_copies_);
+    return out;
+}
+
+void CacheManager::destroy()
+{
+    if (d_tables_) {
+        drk_dev_free(d_tables_);
+        d_tables_ = nullptr;
+    }
+    if (d_pairs_) {
+        drk_dev_free(d_pairs_);
+        d_pairs_ = nullptr;
+    }
+    pool_.destroy();
+    h_tables_.clear();
+    location_.clear();
+    stamp_.clear();
+    evictable_.clear();
+    refs_.clear();
+    seq_len_.clear();
+    alive_.clear();
+    dirty_lo_.clear();
+    dirty_hi_.clear();
+    pending_copies_.clear();
+    max_logical_blocks_ = 0;
+    max_branches_ = 0;
+}
+
+} // namespace deusridet

@@ -1,0 +1,51 @@
+// importance_scorer.h -- per-block importance with exponential decay:
+// score = score*decay + new.  Same interface as the reference's
+// ImportanceScorer (src/memoria/importance_scorer.h:25-67).
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+#include <vector>
+
+namespace deusridet {
+
+class ImportanceScorer {
+public:
+    ImportanceScorer() = default;
+    ~ImportanceScorer();
+    ImportanceScorer(const ImportanceScorer&) = delete;
+    ImportanceScorer& operator=(const ImportanceScorer&) = delete;
+
+    // Device scores for max_blocks logical blocks, zeroed; own stream
+    // (importance_scorer.cu:46-65).
+    bool init(int max_blocks, float decay = 0.95f);
+    // Host mirror only, no device memory: least_important()/score() work on what
+    // load_host_scores() put there.  For tests and planning without a GPU.
+    bool init_detached(int max_blocks, float decay = 0.95f);
+
+    // scores[b] = scores[b]*decay + d_block_scores[b] for b < num_blocks, on the
+    // scorer's stream, asynchronous (importance_scorer.cu:67-73).
+    void update(const float* d_block_scores, int num_blocks);
+
+    // First minimum over the given logical block ids in list order, from the host
+    // mirror (importance_scorer.cu:75-87).  -1 when n <= 0.
+    int least_important(const int* gpu_resident, int n) const;
+    float score(int logical_block) const;
+    // Waits for the scorer's stream and copies the scores to the host mirror
+    // (importance_scorer.cu:94-99).
+    void sync_to_host();
+    // Replace the host mirror (restoring a snapshot; no arithmetic).
+    void load_host_scores(const float* scores, int n);
+
+    void destroy();
+    hipStream_t stream() const { return scorer_stream_; }
+    int max_blocks() const { return max_blocks_; }
+
+private:
+    float* d_scores_ = nullptr;
+    std::vector<float> h_scores_;
+    int max_blocks_ = 0;
+    float decay_ = 0.95f;
+    hipStream_t scorer_stream_ = nullptr;
+};
+
+} // namespace deusridet

@@ -1,0 +1,104 @@
+/*
+ * drk_host.h -- C shim over the C++ host classes (deusridet::CacheManager,
+ * BlockPool, ImportanceScorer, ModelConfig and the paged_attention.h
+ * functions), exported by libdeusridet_memoria.so for language bindings: the
+ * Python tests and the benchmark drive the host classes through it.  C++ callers
+ * include the class headers directly.  Every function forwards to the method of
+ * the same name; see the headers under deusridet_amd/memoria and machina/paged_attention.h for
+ * the semantics and the reference citations.
+ */
+#ifndef DRK_HOST_H
+#define DRK_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ModelConfig::set_attention_geometry (src/machina/model.h:39-42, 73) */
+int drkh_set_attention_geometry(int num_fa_layers, int num_attn_heads, int num_kv_heads, int head_dim,
+                                int kv_dtype, int io_dtype);
+
+/* ImportanceScorer (src/memoria/importance_scorer.h:25-67) */
+void *drkh_scorer_create(void);
+void  drkh_scorer_destroy(void *s);
+int   drkh_scorer_init(void *s, int max_blocks, float decay);
+int   drkh_scorer_init_detached(void *s, int max_blocks, float decay);
+void  drkh_scorer_update(void *s, const float *d_block_scores, int num_blocks);
+int   drkh_scorer_least_important(void *s, const int *ids, int n);
+float drkh_scorer_score(void *s, int logical_block);
+void  drkh_scorer_sync_to_host(void *s);
+void  drkh_scorer_load_host_scores(void *s, const float *scores, int n);
+
+/* CacheManager (src/memoria/cache_manager.h:52-169) and its BlockPool
+ * (src/memoria/block_pool.h:58-123) */
+void *drkh_cm_create(void);
+void  drkh_cm_destroy(void *cm);
+int   drkh_cm_init(void *cm, size_t kv_budget_bytes, int block_size, void *scorer, int max_branches);
+int   drkh_cm_init_detached(void *cm, int max_blocks, int block_size, void *scorer, int max_branches);
+int   drkh_cm_ensure_blocks_for(void *cm, int branch, int pos);
+int   drkh_cm_ensure_blocks_for_range(void *cm, int branch, int pos_start, int M);
+void  drkh_cm_sync_block_table(void *cm, void *stream);
+const int32_t *drkh_cm_d_block_table(void *cm, int branch);
+const int32_t *drkh_cm_h_block_table(void *cm, int branch);
+int   drkh_cm_table_stride(void *cm);
+int   drkh_cm_seq_len(void *cm, int branch);
+void  drkh_cm_set_seq_len(void *cm, int branch, int len);
+int   drkh_cm_num_logical_blocks(void *cm, int branch);
+int   drkh_cm_fork_branch(void *cm, int parent, int pos);
+void  drkh_cm_release_branch(void *cm, int branch);
+void  drkh_cm_touch_block(void *cm, int branch, int logical);
+int   drkh_cm_block_location(void *cm, int branch, int logical);
+int   drkh_cm_evict_blocks(void *cm, int n);
+int   drkh_cm_ensure_free_blocks(void *cm, int n_free);
+int   drkh_cm_gpu_blocks_used(void *cm);
+int   drkh_cm_free_blocks(void *cm);
+int   drkh_cm_lru_snapshot(void *cm, int32_t *branch_out, int32_t *logical_out, int cap);
+int   drkh_cm_take_pending_copies(void *cm, int32_t *src_out, int32_t *dst_out, int cap);
+/* BlockPool through the manager */
+int    drkh_pool_alloc_block(void *cm);
+void   drkh_pool_free_block(void *cm, int id);
+int    drkh_pool_free_count(void *cm);
+int    drkh_pool_max_blocks(void *cm);
+int    drkh_pool_block_size(void *cm);
+int    drkh_pool_refcount(void *cm, int id);
+void  *drkh_pool_ptr(void *cm);
+size_t drkh_pool_k_offset(void *cm, int layer, int block);
+size_t drkh_pool_v_offset(void *cm, int layer, int block);
+size_t drkh_pool_total_bytes(void *cm);
+int    drkh_pool_free_stack(void *cm, int32_t *out, int cap);
+
+/* src/machina/paged_attention.h:27-73 and src/memoria/cache_kernels.h:44-74 */
+void drkh_paged_kv_cache_write(const void *src_k, const void *src_v, void *kv_pool, const int32_t *d_block_table,
+                               int fa_layer_idx, const int32_t *d_pos, int max_phys_blocks, int block_size,
+                               void *stream);
+void drkh_paged_kv_cache_write_batch(const void *src_k, const void *src_v, void *kv_pool,
+                                     const int32_t *d_block_table, int fa_layer_idx, int pos_start, int M,
+                                     int max_phys_blocks, int block_size, void *stream);
+void drkh_paged_kv_cache_write_branches(const void *src_k, const void *src_v, void *kv_pool,
+                                        const int32_t *d_tables, int table_stride, const int32_t *d_pos, int B,
+                                        int fa_layer_idx, int max_phys_blocks, int block_size, void *stream);
+void drkh_paged_gqa_decode_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
+                                     int fa_layer_idx, int seq_len, int max_phys_blocks, int block_size,
+                                     float scale, void *stream);
+void drkh_paged_gqa_decode_attention_branches(const void *Q, void *kv_pool, const int32_t *d_tables,
+                                              int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len,
+                                              void *out, int fa_layer_idx, int max_phys_blocks, int block_size,
+                                              float scale, void *stream);
+void drkh_paged_prefill_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
+                                  int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
+                                  float scale, void *stream);
+int  drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
+void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,
+                                       int num_tokens, int num_layers, int num_kv_heads, int head_dim,
+                                       int block_size, int max_phys_blocks, void *stream);
+void drkh_invoke_inject_kv_to_pages(void *kv_pool, const void *src, const int32_t *block_table, int start_token,
+                                    int num_tokens, int num_layers, int num_kv_heads, int head_dim, int block_size,
+                                    int max_phys_blocks, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,213 @@
+"""GPU: the C++ host classes (CacheManager / BlockPool / ImportanceScorer) and the
+reference-named launchers of machina/paged_attention.h, driven in the caller's
+order (src/conscientia/stream.cpp:151-156, 297-305, 319-334: ensure blocks ->
+sync table -> write K/V -> attend with seq_len = pos + 1)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from deusridet_amd import cabi, host
+from oracle import binding as orc
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def d2h(ptr, nbytes):
+    out = np.empty(nbytes, dtype=np.uint8)
+    cabi.call("drk_memcpy_d2h", out.ctypes.data_as(C.c_void_p), C.c_void_p(ptr), nbytes, U.stream_ptr())
+    return out
+
+
+def test_config1_through_the_reference_interface(dev):
+    L, KVH, QH, D, bs, T = 1, 4, 16, 128, 16, 512
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.F16)
+    cm = host.CacheManager()
+    block_bytes = L * 2 * KVH * bs * D * 2
+    assert cm.init(256 * block_bytes, bs)
+    NB = cm.pool_max_blocks()
+    assert NB == 256 and cm.pool_total_bytes() == 256 * block_bytes and cm.free_blocks() == 256
+    assert not d2h(cm.pool_ptr(), 4096).any()                     # zero-filled (block_pool.cpp:49)
+    rng = np.random.default_rng(1)
+    # a shuffled table: allocate all, free in random order, then let the sequence allocate
+    ids = [cm.pool_alloc_block() for _ in range(NB)]
+    for i in rng.permutation(NB):
+        cm.pool_free_block(int(ids[i]))
+    assert cm.ensure_blocks_for_range(0, 0, T)
+    table = cm.h_block_table(0)
+    assert sorted(table[:T // bs].tolist()) != table[:T // bs].tolist() and (table[T // bs:] == -1).all()
+    cm.sync_block_table(U.stream_ptr())
+    k, v, q = (U.normal_bits(rng, s, cabi.F16) for s in ((T, KVH, D), (T, KVH, D), (QH, D)))
+    dk, dv, dq = U.dev_bytes(k), U.dev_bytes(v), U.dev_bytes(q)
+    L_ = host.lib()
+    L_.drkh_paged_kv_cache_write_batch(U.p(dk), U.p(dv), cm.pool_ptr(), cm.d_block_table(0), 0, 0, T, NB, bs,
+                                       U.stream_ptr())
+    cm.set_seq_len(0, T)
+    assert cm.num_logical_blocks(0) == T // bs
+    out = U.dev_zeros(QH * D * 2)
+    scale = 1 / np.sqrt(D)
+    L_.drkh_paged_gqa_decode_attention(U.p(dq), cm.pool_ptr(), cm.d_block_table(0), U.p(out), 0, T, NB, bs,
+                                       float(scale), U.stream_ptr())
+    flat = U.dev_zeros(2 * T * KVH * D * 2)
+    L_.drkh_invoke_extract_kv_from_pages(U.p(flat), cm.pool_ptr(), cm.d_block_table(0), 0, T, 1, KVH, D, bs, NB,
+                                         U.stream_ptr())
+    U.sync()
+    og = orc.layout(L, KVH, QH, D, bs, NB, orc.F16)
+    opool = orc.new_pool(og)
+    orc.append_batch(og, opool, table, 0, 0, k, v, orc.F16)
+    assert np.array_equal(d2h(cm.pool_ptr(), cm.pool_total_bytes()), opool)
+    got_flat = U.host(flat, np.uint16, (1, 2, T, KVH, D))
+    assert np.array_equal(got_flat[0, 0], k) and np.array_equal(got_flat[0, 1], v)
+    want = orc.decode_f64(og, q, opool, table, 0, T, scale, orc.F16)
+    ok, ma, _ = U.rel_abs_ok(U.from_bits(U.host(out, np.uint16, (QH, D)), cabi.F16), want)
+    assert ok, ma
+
+
+def test_decode_loop_protocol_with_eviction(dev):
+    """One sequence decoding token by token in a pool that is too small: old pages
+    are evicted (FIFO), the table keeps -1 holes, attention skips them."""
+    L, KVH, QH, D, bs = 2, 4, 16, 128, 16
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    cm = host.CacheManager()
+    NBw = 6
+    assert cm.init(NBw * L * 2 * KVH * bs * D * 2, bs)
+    NB = cm.pool_max_blocks()
+    og = orc.layout(L, KVH, QH, D, bs, NB, orc.BF16)
+    opool = orc.new_pool(og)
+    oc = orc.CacheManager(NB, bs)
+    rng = np.random.default_rng(12)
+    steps = 8 * bs + 3
+    lib = host.lib()
+    dpos = U.dev_i32(np.zeros(1, dtype=np.int32))
+    scale = 1 / np.sqrt(D)
+    for pos in range(steps):
+        assert cm.ensure_blocks_for(0, pos) and oc.ensure(0, pos)
+        cm.sync_block_table(U.stream_ptr())
+        dpos.fill_(pos)
+        k, v = U.normal_bits(rng, (L, KVH, D), cabi.BF16), U.normal_bits(rng, (L, KVH, D), cabi.BF16)
+        dk, dv = U.dev_bytes(k), U.dev_bytes(v)
+        for l in range(L):
+            lib.drkh_paged_kv_cache_write(C.c_void_p(dk.data_ptr() + l * KVH * D * 2),
+                                          C.c_void_p(dv.data_ptr() + l * KVH * D * 2), cm.pool_ptr(),
+                                          cm.d_block_table(0), l, U.p(dpos), NB, bs, U.stream_ptr())
+            orc.append_token(og, opool, oc.table(0), l, pos, k[l], v[l], orc.BF16)
+        cm.set_seq_len(0, pos + 1)
+        if pos % 23 == 0 or pos == steps - 1:
+            q = U.normal_bits(rng, (QH, D), cabi.BF16)
+            dq, out = U.dev_bytes(q), U.dev_zeros(QH * D * 2)
+            lib.drkh_paged_gqa_decode_attention(U.p(dq), cm.pool_ptr(), cm.d_block_table(0), U.p(out), L - 1,
+                                                pos + 1, NB, bs, float(scale), U.stream_ptr())
+            U.sync()
+            want = orc.decode_f64(og, q, opool, oc.table(0), L - 1, pos + 1, scale, orc.BF16)
+            ok, ma, _ = U.rel_abs_ok(U.from_bits(U.host(out, np.uint16, (QH, D)), cabi.BF16), want)
+            assert ok, (pos, ma)
+        U.sync()
+    assert np.array_equal(cm.h_block_table(0), oc.table(0))
+    assert (cm.h_block_table(0)[:3] == -1).all() and cm.gpu_blocks_used() == NB
+    assert np.array_equal(d2h(cm.pool_ptr(), cm.pool_total_bytes()), opool)
+    dtab = d2h(cm.d_block_table(0), cm.table_stride() * 4).view(np.int32)
+    assert np.array_equal(dtab, cm.h_block_table(0))              # device mirror follows the host table
+
+
+def test_shared_prefix_branches_copy_on_write(dev):
+    """BASELINE config 3 in small: a persistent prefix shared by several branches
+    that fork at block boundaries and inside a block, append privately, get evicted
+    and released; every branch's gathered K/V and attention output must equal a
+    model in which the branch owns a private copy."""
+    L, KVH, QH, D, bs, branches = 2, 8, 32, 128, 16, 6
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    cm = host.CacheManager()
+    assert cm.init(64 * L * 2 * KVH * bs * D * 2, bs, None, branches)
+    NB = cm.pool_max_blocks()
+    stride = cm.table_stride()
+    og = orc.layout(L, KVH, QH, D, bs, NB, orc.BF16)
+    rng = np.random.default_rng(33)
+    lib = host.lib()
+    model = {0: []}                                        # branch -> list of (k, v) [L, KVH, D]
+
+    def append(bs_list):
+        """one token for each listed branch, one launch per layer"""
+        for b in bs_list:
+            assert cm.ensure_blocks_for(b, len(model[b]))
+        cm.sync_block_table(U.stream_ptr())               # issues the COW copies, uploads tables
+        B = len(bs_list)
+        k, v = U.normal_bits(rng, (L, B, KVH, D), cabi.BF16), U.normal_bits(rng, (L, B, KVH, D), cabi.BF16)
+        pos = np.array([len(model[b]) for b in bs_list], dtype=np.int32)
+        tabs = np.stack([cm.h_block_table(b) for b in bs_list])
+        dk, dv, dpos, dtabs = U.dev_bytes(k), U.dev_bytes(v), U.dev_i32(pos), U.dev_i32(tabs)
+        for l in range(L):
+            lib.drkh_paged_kv_cache_write_branches(C.c_void_p(dk.data_ptr() + l * B * KVH * D * 2),
+                                                   C.c_void_p(dv.data_ptr() + l * B * KVH * D * 2), cm.pool_ptr(),
+                                                   U.p(dtabs), stride, U.p(dpos), B, l, NB, bs, U.stream_ptr())
+        U.sync()
+        for i, b in enumerate(bs_list):
+            model[b].append((k[:, i].copy(), v[:, i].copy()))
+            cm.set_seq_len(b, len(model[b]))
+
+    for _ in range(5 * bs + 7):                            # the persistent prefix on branch 0
+        append([0])
+    kids = []
+    for fork_pos in (5 * bs, 3 * bs, 5 * bs + 7, 2 * bs + 1):     # block boundaries and mid-block
+        nb = cm.fork_branch(0, fork_pos)
+        assert nb > 0
+        model[nb] = list(model[0][:fork_pos])
+        kids.append(nb)
+    assert cm.pool_refcount(int(cm.h_block_table(0)[0])) == 5
+    used_before = cm.gpu_blocks_used()
+    for _ in range(2 * bs + 3):
+        append(kids + [0])
+    assert cm.gpu_blocks_used() > used_before
+    cm.release_branch(kids[1])
+    del model[kids[1]]
+    assert cm.evict_blocks(3) == 3                          # private pages of someone, oldest first
+    for _ in range(5):
+        append([kids[0], kids[2]])
+
+    pool_host = d2h(cm.pool_ptr(), cm.pool_total_bytes())
+    scale = 1 / np.sqrt(D)
+    alive = sorted(model)
+    for b in alive:
+        tab, n = cm.h_block_table(b), len(model[b])
+        flat, _ = orc.extract(og, pool_host, tab, 0, n, L)
+        for t in range(n):
+            if tab[t // bs] < 0:
+                assert not flat[:, :, t].any()
+            else:
+                k, v = model[b][t]
+                assert np.array_equal(flat[:, 0, t], k) and np.array_equal(flat[:, 1, t], v), (b, t)
+    # all branches attend in one launch; the oracle runs on the private-copy model
+    B = len(alive)
+    q = U.normal_bits(rng, (B, QH, D), cabi.BF16)
+    lens = np.array([len(model[b]) for b in alive], dtype=np.int32)
+    tabs = np.stack([cm.h_block_table(b) for b in alive])
+    dq, dl, dt, out = U.dev_bytes(q), U.dev_i32(lens), U.dev_i32(tabs), U.dev_zeros(B * QH * D * 2)
+    lib.drkh_paged_gqa_decode_attention_branches(U.p(dq), cm.pool_ptr(), U.p(dt), stride, U.p(dl), B,
+                                                 int(lens.max()), U.p(out), 1, NB, bs, float(scale), U.stream_ptr())
+    U.sync()
+    got = U.from_bits(U.host(out, np.uint16, (B, QH, D)), cabi.BF16)
+    for i, b in enumerate(alive):
+        n = len(model[b])
+        pg = orc.layout(L, KVH, QH, D, bs, (n + bs - 1) // bs, orc.BF16)
+        ppool = orc.new_pool(pg)
+        ptab = np.arange((n + bs - 1) // bs, dtype=np.int32)
+        ptab[cm.h_block_table(b)[:len(ptab)] < 0] = -1     # evicted pages are holes in the model too
+        kk = np.stack([m[0][1] for m in model[b]])
+        vv = np.stack([m[1][1] for m in model[b]])
+        orc.append_batch(pg, ppool, ptab, 1, 0, kk, vv, orc.BF16)
+        want = orc.decode_f64(pg, q[i], ppool, ptab, 1, n, scale, orc.BF16)
+        ok, ma, _ = U.rel_abs_ok(got[i], want)
+        assert ok, (b, ma)
+
+
+def test_importance_scorer_on_device(dev):
+    sc = host.ImportanceScorer()
+    assert sc.init(64, 0.5)
+    new = np.arange(64, dtype=np.float32)
+    dn = U.dev_bytes(new)
+    for _ in range(3):
+        sc.update(U.p(dn), 64)
+    sc.sync_to_host()
+    want = new * (1 + 0.5 + 0.25)
+    assert [sc.score(i) for i in range(64)] == want.tolist()
+    assert sc.least_important([9, 3, 7]) == 3
