@@ -145,23 +145,38 @@ def main():
     value_gbps = attn_bytes / (total_ms * 1e-3) / 1e9
 
     # ---- dominant kernel alone: the split-K partial kernel of one layer -------
-    lib.drk_debug_time_decode_kernel(1)
-    ker_ms = []
+    # timed back to back (queue busy) with one event pair per launch around the
+    # partial kernel only; the merge kernel sits between the pairs
     last = W + K - 1
     dlen = C.c_void_p(len_steps[last].data_ptr())
-    for it in range(max(K, 10)):
-        l = it % L
-        cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
-                  U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
-                  cabi.BF16, split, U.p(ws), wsb, sp)
-        ms = C.c_float(0)
-        cabi.call("drk_debug_last_decode_kernel_ms", C.byref(ms))
-        ker_ms.append(ms.value)
+    n_timed = max(2 * L, 40)
+
+    def attn_only(n):
+        for it in range(n):
+            l = it % L
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
+                      U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
+                      cabi.BF16, split, U.p(ws), wsb, sp)
+
+    attn_only(8)
+    lib.drk_debug_time_decode_kernel(1)
+    attn_only(n_timed)
+    buf = (C.c_float * 256)()
+    cnt = C.c_int32(0)
+    cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
     lib.drk_debug_time_decode_kernel(0)
-    ker_ms = ker_ms[2:]
-    ker_avg_ms = float(np.mean(ker_ms))
+    ker_ms = np.array(buf[:cnt.value])
+    ker_avg_ms = float(ker_ms.mean())
     launch_bytes = int((start + last + 1).sum()) * kv_bytes_per_token               # one layer, one launch
     achieved = launch_bytes / (ker_avg_ms * 1e-3) / 1e9
+
+    # ---- achievable ceiling on this box: plain 128-bit streaming read of the pool
+    probe_bytes = min(pool_bytes, 32 << 30)
+    sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    gb = C.c_float(0)
+    torch.cuda.synchronize()
+    cabi.call("drk_probe_read_bandwidth", U.p(pool), probe_bytes, 5, U.p(sink), C.byref(gb))
+    read_probe_gbps = float(gb.value)
 
     # ---- bulk append bandwidth (read source + write pages), all layers in one launch
     m = args.bulk_append_tokens
@@ -237,6 +252,7 @@ def main():
         "tokens_per_s": round(tokens_per_s, 1),
         "bulk_append_GBps": None if append_gbps is None else round(append_gbps, 1),
         "bulk_append_hbm_frac": None if append_gbps is None else round(append_gbps / HBM_PEAK_GBPS, 4),
+        "hbm_read_probe_GBps": round(read_probe_gbps, 1),
         "fill_seconds": round(t_fill, 2),
         "roofline": {
             "kernel": "decode_tiled_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),

@@ -30,7 +30,10 @@ namespace drk {
 
 static int g_force_portable = 0;
 static int g_time_kernel = 0;                 // diagnostic: bracket the partial kernel with events
-static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
+constexpr int kMaxTimed = 256;                // event pairs kept per timing session
+static hipEvent_t g_ev[2 * kMaxTimed];
+static bool g_ev_made = false;
+static int g_ev_count = 0;
 static int g_lds_pad = 0;                     // diagnostic: extra dynamic LDS per workgroup (caps occupancy)
 
 constexpr int kTile = 64;            // tokens per tile
@@ -505,9 +508,13 @@ static int launch_decode(const drk_kv_layout *g, const void *q, const void *pool
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(S, a.KVH, B);
 
-    if (g_time_kernel) {
-        if (!g_ev0) { DRK_HIP(hipEventCreate(&g_ev0)); DRK_HIP(hipEventCreate(&g_ev1)); }
-        DRK_HIP(hipEventRecord(g_ev0, st));
+    const bool timed = g_time_kernel && g_ev_count < kMaxTimed;
+    if (timed) {
+        if (!g_ev_made) {
+            for (int i = 0; i < 2 * kMaxTimed; i++) DRK_HIP(hipEventCreate(&g_ev[i]));
+            g_ev_made = true;
+        }
+        DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count], st));
     }
     const bool tiled = !g_force_portable && a.D == 128 && a.E == 2 && G == 4 && (a.bs % 16) == 0;
     if (tiled) {
@@ -549,7 +556,7 @@ static int launch_decode(const drk_kv_layout *g, const void *q, const void *pool
 #undef GO
         DRK_LAUNCH_CHECK("decode_portable_kernel");
     }
-    if (g_time_kernel) DRK_HIP(hipEventRecord(g_ev1, st));
+    if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
     hipLaunchKernelGGL(decode_merge_kernel, dim3(a.QH, B), dim3(a.D), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                        d_seq_lens, seq_len_host, causal_base, split, S, a.D, a.QH, io_dtype);
     DRK_LAUNCH_CHECK("decode_merge_kernel");
@@ -585,15 +592,22 @@ int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len)
 
 void drk_debug_force_portable_decode(int on) { g_force_portable = on ? 1 : 0; }
 
-void drk_debug_time_decode_kernel(int on) { g_time_kernel = on ? 1 : 0; }
+void drk_debug_time_decode_kernel(int on)
+{
+    g_time_kernel = on ? 1 : 0;
+    if (on) g_ev_count = 0;
+}
 void drk_debug_set_decode_lds_pad(int bytes) { g_lds_pad = bytes > 0 ? bytes : 0; }
 
-int drk_debug_last_decode_kernel_ms(float *ms)
+int drk_debug_decode_kernel_times(float *ms, int cap, int *count)
 {
-    if (!ms) return fail(DRK_ERR_INVALID, "ms is NULL");
-    if (!g_ev0) return fail(DRK_ERR_INVALID, "no timed decode launch yet");
-    DRK_HIP(hipEventSynchronize(g_ev1));
-    DRK_HIP(hipEventElapsedTime(ms, g_ev0, g_ev1));
+    if (!ms || !count || cap < 0) return fail(DRK_ERR_INVALID, "decode_kernel_times: bad argument");
+    int n = g_ev_count < cap ? g_ev_count : cap;
+    for (int i = 0; i < n; i++) {
+        DRK_HIP(hipEventSynchronize(g_ev[2 * i + 1]));
+        DRK_HIP(hipEventElapsedTime(&ms[i], g_ev[2 * i], g_ev[2 * i + 1]));
+    }
+    *count = n;
     return DRK_OK;
 }
 

@@ -155,14 +155,17 @@ int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len);
  * geometry, any storage type) instead of the tiled one, so that tests can
  * check the two against each other.  Process-wide, not thread-safe. */
 void drk_debug_force_portable_decode(int on);
-/* Diagnostic for benchmarks: while on, every decode launch records a HIP event
- * on its stream right before and right after the split-K partial kernel (the
- * merge kernel is outside the pair); drk_debug_last_decode_kernel_ms waits for
- * the last pair and returns the elapsed milliseconds.  Process-wide. */
+/* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
+ * session; switching it on starts a new session) records a HIP event on its
+ * stream right before and right after the split-K partial kernel; the merge
+ * kernel is outside the pair.  drk_debug_decode_kernel_times waits for the pairs
+ * recorded so far and returns their elapsed milliseconds.  Launch back to back
+ * (no host sync in between) so that the queue stays busy and the pairs bracket
+ * the kernel tightly.  Process-wide. */
 void drk_debug_time_decode_kernel(int on);
+int  drk_debug_decode_kernel_times(float *ms, int cap, int *count);
 /* Diagnostic: extra dynamic LDS bytes per decode workgroup (lowers occupancy). */
 void drk_debug_set_decode_lds_pad(int bytes);
-int  drk_debug_last_decode_kernel_ms(float *ms);
 /* paged_gqa_decode_attention, paged_attention.cu:179-282: one sequence.
  * q/out [num_q_heads, head_dim] of io_dtype (F16/BF16). */
 int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void *pool,
