@@ -22,6 +22,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the decode kernel from two `rocprofv3 --pmc` runs of this
+# script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), scaled by what the same
+# counters read for a plain 32 GiB read (x2.0) and a bulk append of known size
+# (x1.0).  Keyed by the algorithmic bytes of the launch it was measured on.
+MEASURED_TRAFFIC_BYTES = {1073741824: (524893 * 2 + 1152) * 1024}
 
 
 def parse():
@@ -257,7 +262,7 @@ def main():
         "roofline": {
             "kernel": "decode_tiled_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None, "avg_launch_us": round(ker_avg_ms * 1e3, 2), "bytes_per_launch": launch_bytes,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(launch_bytes), "avg_launch_us": round(ker_avg_ms * 1e3, 2), "bytes_per_launch": launch_bytes,
         },
         "cpu_baseline": cpu,
     }
