@@ -54,6 +54,13 @@ inline int ilog2_exact(unsigned v)                 // -1 when v is not a power o
     return s;
 }
 
+// ---- shared between the decode and prefill translation units ---------------
+extern int g_force_portable;
+int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
+                  int table_stride, const int32_t *d_seq_lens, int seq_len_host, int causal_base, int B,
+                  int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
 // ---- element helpers (device) -------------------------------------------
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }

@@ -28,7 +28,7 @@
 
 namespace drk {
 
-static int g_force_portable = 0;
+int g_force_portable = 0;                    // diagnostic, shared with the prefill unit
 static int g_time_kernel = 0;                 // diagnostic: bracket the partial kernel with events
 constexpr int kMaxTimed = 256;                // event pairs kept per timing session
 static hipEvent_t g_ev[2 * kMaxTimed];
@@ -474,7 +474,7 @@ static size_t workspace_need(const Lay &a, int B, int max_seq_len, int split)
     return (size_t)B * a.QH * S * (a.D + 2) * sizeof(float);
 }
 
-static int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
+int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                          int table_stride, const int32_t *d_seq_lens, int seq_len_host, int causal_base,
                          int B, int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
                          void *workspace, size_t workspace_bytes, void *stream)
@@ -629,25 +629,6 @@ int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, c
     if (!d_seq_lens) return fail(DRK_ERR_INVALID, "decode: d_seq_lens is NULL");
     return launch_decode(g, q, pool, d_tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
                          io_dtype, split_tokens, workspace, workspace_bytes, stream);
-}
-
-size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
-{
-    return drk_decode_workspace_bytes(g, M, pos_start + M);
-}
-
-// Row t of the chunk is a decode over tokens 0..pos_start+t (the reference
-// kernel is exactly that loop, paged_attention.cu:481, 506-549): each row runs
-// as one "branch" of the decode kernels with a causal length.
-int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
-                                const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
-                                float scale, int io_dtype, void *workspace, size_t workspace_bytes,
-                                void *stream)
-{
-    if (pos_start < 0 || M < 0) return fail(DRK_ERR_INVALID, "prefill: negative pos_start or M");
-    if (M == 0) return DRK_OK;
-    return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
-                         io_dtype, 0, workspace, workspace_bytes, stream);
 }
 
 } // extern "C"

@@ -1,0 +1,350 @@
+// drk_prefill.hip -- paged causal prefill attention on the gfx950 matrix cores.
+//
+// Replaces paged_prefill_attention_kernel (paged_attention.cu:465-554), which runs
+// the token-at-a-time decode loop once per (query head, query token): O(M*L)
+// serial dot products, no tensor cores.  Here the one dense contraction of the
+// path, QK^T and PV of a chunk against all pages before it, runs on
+// v_mfma_f32_32x32x16_{bf16,f16}.
+//
+// Formulation: everything is kept transposed so that one lane owns one query row.
+//   S^T[token][row] = K[token][:] . Q[row][:]      A = K tile (LDS), B = Q (registers)
+//   O^T[d][row]    += V^T[d][token] . P^T[token][row]   A = V tile read transposed
+//                                                       (ds_read_b64_tr_b16), B = P
+// The C layout of the first product (lane l: column l%32 = query row, 16 tokens)
+// is, after exp2 and packing to 16 bit, exactly the B layout of the second, so P
+// never moves between lanes, and the online-softmax rescale of O^T is a per-lane
+// scalar multiply.  "Row" = (query token, query head of the group): the 4 query
+// heads that share a KV head are stacked into the row dimension, so K/V tiles are
+// read once for all of them.
+//
+// Workgroup = 4 waves = 128 rows = 32 query tokens x 4 heads of one KV head; it
+// walks the KV tiles (64 tokens) from token 0 to its causal limit.  K/V tiles are
+// gathered from 16-token page row runs with 128-bit loads (next tile in flight
+// while the current one is multiplied) and staged in LDS with a 272-byte pitch.
+#include "drk_common.hpp"
+
+#include <math.h>
+
+namespace drk {
+
+constexpr int kPfBN = 64;         // KV tokens per tile
+constexpr int kPfPitch = 272;     // LDS bytes per staged row (256 + 16)
+constexpr int kPfRows = 128;      // rows per workgroup (32 query tokens x 4 heads)
+constexpr float kLog2eP = 1.4426950408889634f;
+
+typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 pf_f16x8 __attribute__((ext_vector_type(8)));
+typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
+typedef short pf_v4s __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ pf_f32x16 mfma32(const uint4 &a, const uint4 &b, pf_f32x16 c)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (DT == DRK_BF16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, a), __builtin_bit_cast(pf_bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_f16x8, a), __builtin_bit_cast(pf_f16x8, b), c, 0, 0, 0);
+#else
+    (void)a; (void)b;
+    return c;
+#endif
+}
+
+// two fp32 -> one dword of two 16-bit values, round to nearest even
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi)
+{
+    if constexpr (DT == DRK_BF16) {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        b2 v = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    } else {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+}
+
+// LDS transpose read: the 16 lanes of a group pass 16 addresses of 4 consecutive
+// 16-bit elements; lane i receives, for k = 0..3, element (i % 4) at the address
+// given by lane (i / 4 + 4 * k) of its group.
+__device__ __forceinline__ uint2 lds_read_tr16(const uint8_t *p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    pf_v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_v4s __attribute__((address_space(3))) *)p);
+    return __builtin_bit_cast(uint2, r);
+#else
+    (void)p;
+    return make_uint2(0, 0);
+#endif
+}
+
+struct PrefillArgs {
+    const uint8_t *pool_layer;    // pool + layer * layer_stride
+    const int32_t *table;
+    const uint8_t *q;
+    uint8_t *out;
+    int pos_start, M, QH, NB, bs, bs_shift;
+    unsigned head_stride, kv_plane, block_stride;
+    float scale_log2e;
+};
+
+struct PfGroup {
+    uint4 r0, r1, r2, r3;
+};
+
+__device__ __forceinline__ PfGroup pf_load_group(const uint8_t *__restrict__ base, bool valid, size_t off, int lane)
+{
+    PfGroup g;
+    g.r0 = g.r1 = g.r2 = g.r3 = make_uint4(0, 0, 0, 0);
+    if (valid) {
+        const uint8_t *p = base + off + (size_t)lane * 16;
+        g.r0 = *(const uint4 *)(p);
+        g.r1 = *(const uint4 *)(p + 1024);
+        g.r2 = *(const uint4 *)(p + 2048);
+        g.r3 = *(const uint4 *)(p + 3072);
+    }
+    return g;
+}
+
+__device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, int w, int lane)
+{
+    uint8_t *dst = lds + (w * 16 + (lane >> 4)) * kPfPitch + (lane & 15) * 16;
+    *(uint4 *)(dst) = g.r0;
+    *(uint4 *)(dst + 4 * kPfPitch) = g.r1;
+    *(uint4 *)(dst + 8 * kPfPitch) = g.r2;
+    *(uint4 *)(dst + 12 * kPfPitch) = g.r3;
+}
+
+// grid = (ceil(M/32), KVH); block = 256
+template <int DT>
+__global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
+{
+    __shared__ __align__(16) uint8_t k_lds[kPfBN * kPfPitch];
+    __shared__ __align__(16) uint8_t v_lds[kPfBN * kPfPitch];
+    __shared__ int valid_lds[4];
+
+    const int qt = blockIdx.x, kvh = blockIdx.y;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, g = lane >> 5;
+
+    // this lane's query row: token tq of the chunk, head hq of the group
+    const int tq = qt * 32 + w * 8 + (n >> 2);
+    const int head = kvh * 4 + (n & 3);
+    const bool row_live = tq < A.M;
+    const int vis = A.pos_start + tq + 1;                       // tokens [0, vis) are visible to the row
+    const int lim_wg = A.pos_start + min((qt + 1) * 32, A.M);   // exclusive limit over the workgroup
+    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+    const int first_masked_tile = (A.pos_start + qt * 32 + 1) / kPfBN;   // tiles below are fully visible
+
+    // Q as the B operand of S^T: 8 k-steps of 16 dims; lane holds dims ks*16 + g*8 .. +8
+    uint4 qf[8];
+    {
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * 256 + g * 16;
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) qf[ks] = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+    }
+
+    const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+    auto lookup = [&](int tile, bool &valid) -> size_t {
+        int tg = tile * kPfBN + w * 16;
+        valid = false;
+        if (tg >= lim_wg) return 0;
+        int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
+        int blk = A.table[lb];
+        if (blk < 0 || blk >= A.NB) return 0;
+        valid = true;
+        return (size_t)blk * A.block_stride + (size_t)(tg - lb * A.bs) * 256;
+    };
+
+    pf_f32x16 o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    bool cur_valid, nxt_valid = false;
+    size_t off = lookup(0, cur_valid);
+    PfGroup kreg = pf_load_group(kbase, cur_valid, off, lane);
+    PfGroup vreg = pf_load_group(kbase + A.kv_plane, cur_valid, off, lane);
+
+    for (int it = 0; it < ntiles; it++) {
+        const int tile_t = it * kPfBN;
+        // ---- stage the tile; rows at or past the workgroup's limit may hold anything ----
+        if (tile_t + kPfBN > lim_wg) {
+            const int lim = lim_wg - tile_t - w * 16 - (lane >> 4);   // rows r0, r0+4, ... of this lane
+            const uint4 z = make_uint4(0, 0, 0, 0);
+            if (0 >= lim) { vreg.r0 = z; kreg.r0 = z; }
+            if (4 >= lim) { vreg.r1 = z; kreg.r1 = z; }
+            if (8 >= lim) { vreg.r2 = z; kreg.r2 = z; }
+            if (12 >= lim) { vreg.r3 = z; kreg.r3 = z; }
+        }
+        pf_store_group(k_lds, kreg, w, lane);
+        pf_store_group(v_lds, vreg, w, lane);
+        if (lane == 0) valid_lds[w] = cur_valid ? 1 : 0;
+        if (it + 1 < ntiles) {
+            off = lookup(it + 1, nxt_valid);
+            kreg = pf_load_group(kbase, nxt_valid, off, lane);
+            vreg = pf_load_group(kbase + A.kv_plane, nxt_valid, off, lane);
+        }
+        __syncthreads();
+
+        // ---- S^T = K Q^T : two 32-token tiles x 32 rows, 8 k-steps of 16 dims ----
+        pf_f32x16 s[2];
+#pragma unroll
+        for (int i = 0; i < 16; i++) { s[0][i] = 0.0f; s[1][i] = 0.0f; }
+        {
+            const uint8_t *ka = k_lds + n * kPfPitch + g * 16;
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                const uint4 a0 = *(const uint4 *)(ka + ks * 32);
+                const uint4 a1 = *(const uint4 *)(ka + 32 * kPfPitch + ks * 32);
+                s[0] = mfma32<DT>(a0, qf[ks], s[0]);
+                s[1] = mfma32<DT>(a1, qf[ks], s[1]);
+            }
+        }
+
+        // ---- tile softmax for this lane's row; register i of tile tt is token
+        //      tile_t + tt*32 + 8*(i/4) + 4*g + i%4 ----
+        const bool all_groups_valid = (valid_lds[0] & valid_lds[1] & valid_lds[2] & valid_lds[3]) != 0;
+        const bool need_mask = it >= first_masked_tile || !all_groups_valid;
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                float v = s[tt][i] * A.scale_log2e;
+                if (need_mask) {
+                    const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    const bool ok = (tile_t + tl) < vis && valid_lds[tl >> 4] != 0;
+                    v = ok ? v : -INFINITY;
+                }
+                s[tt][i] = v;
+                tmax = fmaxf(tmax, v);
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));               // the row's other 32 tokens
+        const float m_new = fmaxf(m_run, tmax);
+        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        float psum = 0.0f;
+        uint4 pb[2][2];                                          // [token tile][k-half]: B operand of PV
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            float p[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                p[i] = __builtin_amdgcn_exp2f(s[tt][i] - m_use);
+                psum += p[i];
+            }
+            pb[tt][0] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+            pb[tt][1] = make_uint4(pack2<DT>(p[8], p[9]), pack2<DT>(p[10], p[11]), pack2<DT>(p[12], p[13]), pack2<DT>(p[14], p[15]));
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (!__all(alpha == 1.0f)) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+        }
+
+        // ---- O^T += V^T P^T : k-slot j of MFMA (tt, mh) is token tt*32 + 16*mh + 8*(j/4) + 4*g + j%4 ----
+        {
+            const int j16 = lane & 15;
+            const int dsub = 16 * ((lane >> 4) & 1) + 4 * (j16 & 3);           // d offset inside a 32-d tile
+            const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPfPitch + dsub * 2;
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int mh = 0; mh < 2; mh++) {
+                    const uint8_t *vt = vb + (tt * 32 + 16 * mh) * kPfPitch;
+#pragma unroll
+                    for (int dt = 0; dt < 4; dt++) {
+                        const uint2 lo = lds_read_tr16(vt + dt * 64);
+                        const uint2 hi = lds_read_tr16(vt + 8 * kPfPitch + dt * 64);
+                        o[dt] = mfma32<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pb[tt][mh], o[dt]);
+                    }
+                }
+        }
+        cur_valid = nxt_valid;
+        __syncthreads();
+    }
+
+    // ---- normalise and write: register i of tile dt is d = dt*32 + 8*(i/4) + 4*g + i%4 ----
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (row_live && l_tot > 0.0f) {
+        const float inv = 1.0f / l_tot;
+        uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * 256;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; b4++) {
+                const int d0 = dt * 32 + 8 * b4 + 4 * g;
+                uint2 v = make_uint2(pack2<DT>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
+                                     pack2<DT>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv));
+                *(uint2 *)(orow + d0 * 2) = v;
+            }
+    }
+}
+
+} // namespace drk
+
+using namespace drk;
+
+extern "C" {
+
+size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
+{
+    Lay a;
+    if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
+    const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0;
+    if (mfma) return 0;
+    return drk_decode_workspace_bytes(g, M, pos_start + M);
+}
+
+// paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630.
+// head_dim 128, 16-bit K/V, 4 query heads per KV head: the MFMA kernel above (no
+// workspace).  Any other geometry or storage type: row t of the chunk runs as one
+// causal "branch" of the decode kernels -- the reference's algorithm verbatim
+// (paged_attention.cu:481, 506-549) -- and needs the workspace.
+int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
+                                const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
+                                float scale, int io_dtype, void *workspace, size_t workspace_bytes,
+                                void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (pos_start < 0 || M < 0) return fail(DRK_ERR_INVALID, "prefill: negative pos_start or M");
+    if (M == 0) return DRK_OK;
+    if (!q || !pool || !d_block_table || !out) return fail(DRK_ERR_INVALID, "prefill: NULL pointer");
+    if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "prefill: io_dtype must be F16 or BF16");
+    if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
+        return fail(DRK_ERR_INVALID, "prefill: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
+    if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
+
+    const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0;
+    if (!mfma)
+        return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
+                             io_dtype, 0, workspace, workspace_bytes, stream);
+    if (a.KVH > 65535) return fail(DRK_ERR_INVALID, "prefill: more than 65535 kv heads");
+    PrefillArgs A;
+    A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
+    A.table = d_block_table;
+    A.q = (const uint8_t *)q;
+    A.out = (uint8_t *)out;
+    A.pos_start = pos_start; A.M = M; A.QH = a.QH; A.NB = a.NB; A.bs = a.bs;
+    A.bs_shift = ilog2_exact((unsigned)a.bs);
+    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
+    A.scale_log2e = scale * kLog2eP;
+    dim3 grid((M + 31) / 32, a.KVH);
+    if (a.dtype == DRK_BF16) hipLaunchKernelGGL(prefill_mfma_kernel<DRK_BF16>, grid, dim3(256), 0, (hipStream_t)stream, A);
+    else hipLaunchKernelGGL(prefill_mfma_kernel<DRK_F16>, grid, dim3(256), 0, (hipStream_t)stream, A);
+    DRK_LAUNCH_CHECK("prefill_mfma_kernel");
+    return DRK_OK;
+}
+
+} // extern "C"

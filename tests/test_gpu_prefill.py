@@ -1,0 +1,136 @@
+"""GPU parity: chunked causal prefill over pages (paged_attention.cu:465-554) --
+the MFMA kernel and the row-wise path against the fp64 oracle, tolerance
+|err| <= 2e-2 + 1e-2*|want|."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from deusridet_amd import cabi
+from oracle import binding as orc
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def run_prefill(g, dq, dpool, dtab, layer, pos_start, M, scale, dtype, QH, D):
+    lib = cabi.lib()
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    ws = U.dev_zeros(max(wsb, 16))
+    out = U.dev_bytes(np.full(M * QH * D * 2, 0x7B, dtype=np.uint8))
+    cabi.call("drk_paged_prefill_attention", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), layer, pos_start, M,
+              float(scale), dtype, U.p(ws), wsb, U.stream_ptr())
+    U.sync()
+    return U.host(out, np.uint16, (M, QH, D))
+
+
+def build(geom, dtype, total, seed, holes=(), mul=1.0):
+    L, KVH, QH, D, bs, NB = geom
+    g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
+    rng = np.random.default_rng(seed)
+    nblk = (total + bs - 1) // bs
+    table = U.shuffled_table(rng, NB, nblk, nblk + 2)
+    opool = orc.new_pool(og)
+    k = U.normal_bits(rng, (total, KVH, D), dtype, mul)
+    v = U.normal_bits(rng, (total, KVH, D), dtype, mul)
+    orc.append_batch(og, opool, table, L - 1, 0, k, v, dtype)
+    for h in holes:
+        table[h] = -1
+    return g, og, rng, table, opool
+
+
+@pytest.fixture(params=["mfma", "rowwise"])
+def path(request):
+    cabi.lib().drk_debug_force_portable_decode(1 if request.param == "rowwise" else 0)
+    yield request.param
+    cabi.lib().drk_debug_force_portable_decode(0)
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
+@pytest.mark.parametrize("pos_start,M", [(0, 1), (0, 32), (0, 200), (37, 45), (64, 64), (100, 129), (509, 77), (1000, 256)])
+def test_prefill_matches_oracle(dev, path, dtype, pos_start, M):
+    geom = (2, 4, 16, 128, 16, 100)
+    g, og, rng, table, opool = build(geom, dtype, pos_start + M, seed=pos_start * 7 + M)
+    QH, D = geom[2], geom[3]
+    q = U.normal_bits(rng, (M, QH, D), dtype)
+    scale = 1 / np.sqrt(D)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    got = U.from_bits(run_prefill(g, dq, dpool, dtab, 1, pos_start, M, scale, dtype, QH, D), dtype)
+    want = orc.prefill_f64(og, q, opool, table, 1, pos_start, scale, dtype)
+    ok, ma, _ = U.rel_abs_ok(got, want)
+    assert ok, ma
+
+
+def test_first_row_of_first_chunk_is_v0_bitwise(dev, path):
+    geom = (1, 4, 16, 128, 16, 16)
+    g, og, rng, table, opool = build(geom, cabi.BF16, 40, seed=3)
+    q = U.normal_bits(rng, (40, 16, 128), cabi.BF16)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    got = run_prefill(g, dq, dpool, dtab, 0, 0, 40, 0.1, cabi.BF16, 16, 128)
+    flat, _ = orc.extract(og, opool, table, 0, 1, 1)
+    assert np.array_equal(got[0], np.repeat(flat[0, 1, 0], 4, axis=0))
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
+def test_chunked_prefill_config5_small(dev, dtype):
+    """BASELINE config 5 in small: chunks appended into 16-token pages, causal
+    attention over all prior pages plus the chunk, 32 Q / 8 KV heads x 128; every
+    chunk's rows must equal decode attention at that row's length."""
+    L, KVH, QH, D, bs, NB = 1, 8, 32, 128, 16, 80
+    g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
+    rng = np.random.default_rng(55)
+    chunk, nchunks = 160, 6
+    total = chunk * nchunks
+    table = U.shuffled_table(rng, NB, (total + bs - 1) // bs)
+    dpool = U.dev_zeros(orc.pool_bytes(og))
+    dtab = U.dev_i32(table)
+    opool = orc.new_pool(og)
+    scale = 1 / np.sqrt(D)
+    for c in range(nchunks):
+        k = U.normal_bits(rng, (chunk, KVH, D), dtype)
+        v = U.normal_bits(rng, (chunk, KVH, D), dtype)
+        q = U.normal_bits(rng, (chunk, QH, D), dtype)
+        dk, dv, dq = U.dev_bytes(k), U.dev_bytes(v), U.dev_bytes(q)
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(dpool), U.p(dtab), 0, 1, c * chunk, chunk, U.p(dk), U.p(dv),
+                  dtype, U.stream_ptr())
+        orc.append_batch(og, opool, table, 0, c * chunk, k, v, dtype)
+        got = U.from_bits(run_prefill(g, dq, dpool, dtab, 0, c * chunk, chunk, scale, dtype, QH, D), dtype)
+        rows = [0, 1, 31, 32, 77, chunk - 1]
+        for t in rows:
+            want = orc.decode_f64(og, q[t], opool, table, 0, c * chunk + t + 1, scale, dtype)
+            ok, ma, _ = U.rel_abs_ok(got[t], want)
+            assert ok, (c, t, ma)
+    assert np.array_equal(U.host(dpool, np.uint8), opool)
+
+
+def test_prefill_with_holes_and_stale_rows(dev, path):
+    geom = (1, 4, 16, 128, 16, 64)
+    pos_start, M = 130, 70
+    g, og, rng, table, opool = build(geom, cabi.BF16, pos_start + M, seed=9, holes=(1, 5))
+    # NaN patterns in the slots of the last page past the end
+    flat = np.full((1, 2, 8, 4, 128), 0x7FC0, dtype=np.uint16)
+    orc.inject(og, opool, flat, None, table, pos_start + M, 8, 1)
+    q = U.normal_bits(rng, (M, 16, 128), cabi.BF16)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    scale = 1 / np.sqrt(128)
+    got = U.from_bits(run_prefill(g, dq, dpool, dtab, 0, pos_start, M, scale, cabi.BF16, 16, 128), cabi.BF16)
+    want = orc.prefill_f64(og, q, opool, table, 0, pos_start, scale, cabi.BF16)
+    ok, ma, _ = U.rel_abs_ok(got, want)
+    assert ok, ma
+
+
+def test_mfma_and_rowwise_paths_agree(dev):
+    geom = (1, 8, 32, 128, 16, 120)
+    pos_start, M = 1024, 512
+    g, og, rng, table, opool = build(geom, cabi.BF16, pos_start + M, seed=21, mul=0.7)
+    q = U.normal_bits(rng, (M, 32, 128), cabi.BF16, 0.7)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    scale = 1 / np.sqrt(128)
+    a = U.from_bits(run_prefill(g, dq, dpool, dtab, 0, pos_start, M, scale, cabi.BF16, 32, 128), cabi.BF16)
+    cabi.lib().drk_debug_force_portable_decode(1)
+    try:
+        b = U.from_bits(run_prefill(g, dq, dpool, dtab, 0, pos_start, M, scale, cabi.BF16, 32, 128), cabi.BF16)
+    finally:
+        cabi.lib().drk_debug_force_portable_decode(0)
+    ok, ma, _ = U.rel_abs_ok(a, b)
+    assert ok, ma
