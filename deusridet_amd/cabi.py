@@ -66,6 +66,8 @@ SIGNATURES = {
     "drk_decode_workspace_bytes_for_split": (_sz, [_LP, _i32, _i32, _i32]),
     "drk_decode_default_split": (_i32, [_LP, _i32, _i32]),
     "drk_debug_force_portable_decode": (None, [_i32]),
+    "drk_debug_set_decode_kernel": (None, [_i32]),
+    "drk_debug_set_stream_workgroups": (None, [_i32]),
     "drk_debug_time_decode_kernel": (None, [_i32]),
     "drk_debug_set_decode_lds_pad": (None, [_i32]),
     "drk_probe_read_bandwidth": (_i32, [_vp, _sz, _i32, _vp, C.POINTER(C.c_float)]),

@@ -61,6 +61,14 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
                   int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
                   void *workspace, size_t workspace_bytes, void *stream);
 
+// persistent stream-K decode (drk_decode_stream.hip)
+extern int g_stream_wgs;
+bool stream_decode_supported(const Lay &a, int B);
+size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens);
+int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
+                         const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
+                         float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st);
+
 // ---- element helpers (device) -------------------------------------------
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }

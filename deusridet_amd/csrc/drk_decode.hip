@@ -29,6 +29,7 @@
 namespace drk {
 
 int g_force_portable = 0;                    // diagnostic, shared with the prefill unit
+static int g_decode_kernel = 0;               // diagnostic: 0 auto, 2 fixed-split tiled kernel, 3 stream kernel
 static int g_time_kernel = 0;                 // diagnostic: bracket the partial kernel with events
 constexpr int kMaxTimed = 256;                // event pairs kept per timing session
 static hipEvent_t g_ev[2 * kMaxTimed];
@@ -496,7 +497,8 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     if (split_tokens < 0 || (split_tokens % kTile)) return fail(DRK_ERR_INVALID, "decode: split_tokens must be a multiple of %d", kTile);
     const int split = split_tokens ? split_tokens : choose_split(a, B, max_seq_len);
     const int S = (max_seq_len + split - 1) / split;
-    const size_t need = workspace_need(a, B, max_seq_len, split);
+    const bool use_stream = !g_force_portable && g_decode_kernel != 2 && causal_base < 0 && stream_decode_supported(a, B);
+    const size_t need = use_stream ? stream_workspace_need(a, B, max_seq_len, split_tokens) : workspace_need(a, B, max_seq_len, split);
     if (!workspace || workspace_bytes < need)
         return fail(DRK_ERR_WORKSPACE, "decode: workspace of %zu bytes, need %zu", workspace_bytes, need);
     if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode: workspace must be 16-byte aligned");
@@ -517,7 +519,11 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
         DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count], st));
     }
     const bool tiled = !g_force_portable && a.D == 128 && a.E == 2 && G == 4 && (a.bs % 16) == 0;
-    if (tiled) {
+    if (use_stream) {
+        rc = launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, seq_len_host, B, max_seq_len, out, layer,
+                                  scale, io_dtype, split_tokens, workspace, false, st);
+        if (rc) return rc;
+    } else if (tiled) {
         TiledArgs A;
         A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
         A.tables = tables; A.seq_lens = d_seq_lens; A.q = (const uint8_t *)q;
@@ -557,6 +563,9 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
         DRK_LAUNCH_CHECK("decode_portable_kernel");
     }
     if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
+    if (use_stream)
+        return launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, seq_len_host, B, max_seq_len, out, layer,
+                                    scale, io_dtype, split_tokens, workspace, true, st);
     hipLaunchKernelGGL(decode_merge_kernel, dim3(a.QH, B), dim3(a.D), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                        d_seq_lens, seq_len_host, causal_base, split, S, a.D, a.QH, io_dtype);
     DRK_LAUNCH_CHECK("decode_merge_kernel");
@@ -573,14 +582,24 @@ size_t drk_decode_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len
 {
     Lay a;
     if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0) return 0;
-    return workspace_need(a, B, max_seq_len, choose_split(a, B, max_seq_len));
+    size_t need = workspace_need(a, B, max_seq_len, choose_split(a, B, max_seq_len));
+    if (stream_decode_supported(a, B)) {
+        size_t s2 = stream_workspace_need(a, B, max_seq_len, 0);
+        if (s2 > need) need = s2;
+    }
+    return need;
 }
 
 size_t drk_decode_workspace_bytes_for_split(const drk_kv_layout *g, int B, int max_seq_len, int split_tokens)
 {
     Lay a;
     if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0 || split_tokens <= 0) return 0;
-    return workspace_need(a, B, max_seq_len, split_tokens);
+    size_t need = workspace_need(a, B, max_seq_len, split_tokens);
+    if (stream_decode_supported(a, B)) {
+        size_t s2 = stream_workspace_need(a, B, max_seq_len, split_tokens);
+        if (s2 > need) need = s2;
+    }
+    return need;
 }
 
 int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len)
@@ -591,6 +610,8 @@ int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len)
 }
 
 void drk_debug_force_portable_decode(int on) { g_force_portable = on ? 1 : 0; }
+void drk_debug_set_decode_kernel(int which) { g_decode_kernel = which; }
+void drk_debug_set_stream_workgroups(int n) { g_stream_wgs = n > 0 ? n : 512; }
 
 void drk_debug_time_decode_kernel(int on)
 {

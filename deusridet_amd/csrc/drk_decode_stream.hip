@@ -1,0 +1,612 @@
+// drk_decode_stream.hip -- the production paged GQA decode kernel: persistent,
+// stream-K style, for head_dim 128 with 4 query heads per KV head and fp16, bf16,
+// int8 (+fp16 scale per token and head) or fp8-e4m3 pages.
+//
+// The unit of work is one 64-token tile of one (branch, kv head).  Units are
+// numbered branch-major, then kv head, then tile; workgroup g owns the run
+// [g*U, (g+1)*U).  Every workgroup therefore streams the same number of tiles
+// whatever the branch lengths are, the whole grid is resident in one round, and a
+// run that crosses from one (branch, kv head) to the next keeps its load pipeline
+// full: the next unit's K/V (and the next segment's Q) are already in flight when
+// the current segment's partial result is written.  A (branch, kv head) is cut
+// into at most ceil(tiles/U)+1 pieces; each piece leaves (o[128], m, l) per query
+// head in the workspace and stream_merge_kernel folds them.
+//
+// Per tile (the same three phases as decode_tiled_kernel in drk_decode.hip):
+//   A  each wave stores the 16-token page row run it loaded one tile earlier into
+//      LDS (K only; 272-byte pitch), converting int8 / fp8 codes to fp16 on the
+//      way, and issues the 128-bit loads of the next unit's K;
+//   B  wave w = query head w: lane = token, Q in 64 SGPRs, v_dot2 over the row in
+//      LDS, no cross-lane reduction for the dot; tile softmax by wave reductions;
+//      p (times the V scale for int8) to LDS;
+//   C  wave w multiplies its own 16 tokens of V, straight from the global loads,
+//      into 4 heads x 8 dims of fp32 per lane; then issues the next unit's V loads.
+#include "drk_common.hpp"
+
+#include <math.h>
+
+namespace drk {
+
+int g_stream_wgs = 512;              // workgroups of the persistent grid (2 per CU of a 256-CU part)
+
+constexpr int kSTile = 64;
+constexpr int kSRow = 272;
+constexpr float kSLog2e = 1.4426950408889634f;
+
+typedef __bf16 s_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 s_f16x2 __attribute__((ext_vector_type(2)));
+
+template <int DT> struct KvTraits;
+template <> struct KvTraits<DRK_F16>      { static constexpr bool q8 = false; static constexpr int dot = DRK_F16; };
+template <> struct KvTraits<DRK_BF16>     { static constexpr bool q8 = false; static constexpr int dot = DRK_BF16; };
+template <> struct KvTraits<DRK_INT8>     { static constexpr bool q8 = true;  static constexpr int dot = DRK_F16; };
+template <> struct KvTraits<DRK_FP8_E4M3> { static constexpr bool q8 = true;  static constexpr int dot = DRK_F16; };
+
+template <int DOT>
+__device__ __forceinline__ float s_dot2(uint32_t k, uint32_t q, float acc)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (DOT == DRK_BF16)
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(s_bf16x2, k), __builtin_bit_cast(s_bf16x2, q), acc, false);
+    else
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(s_f16x2, k), __builtin_bit_cast(s_f16x2, q), acc, false);
+#else
+    (void)k; (void)q;
+    return acc;
+#endif
+}
+
+__device__ __forceinline__ float s_exp2(float x)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_exp2f(x);
+#else
+    return exp2f(x);
+#endif
+}
+
+__device__ __forceinline__ float s_wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+__device__ __forceinline__ float s_wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// four int8 codes -> two dwords of packed fp16, exact: (code ^ 0x80) | 0x6400 is the
+// fp16 number 1024 + code + 128
+__device__ __forceinline__ void int8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t x = w ^ 0x80808080u;
+    const uint32_t a = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);   // bytes x0,64,x1,64
+    const uint32_t b = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);   // bytes x2,64,x3,64
+    const s_f16x2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s_f16x2, a) - bias);
+    hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s_f16x2, b) - bias);
+#else
+    (void)w; lo = hi = 0;
+#endif
+}
+
+// four fp8-e4m3 codes -> two dwords of packed fp16 (exact: e4m3 fits in fp16)
+__device__ __forceinline__ void fp8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    const f2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a[0], a[1]));
+    hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(b[0], b[1]));
+#else
+    (void)w; lo = hi = 0;
+#endif
+}
+
+struct StreamArgs {
+    const uint8_t *pool_layer;      // pool + layer * layer_stride
+    const int32_t *tables;
+    const int32_t *seq_lens;        // [B] on the device, or NULL: one sequence of seq_len_host
+    const uint8_t *q;
+    float *part_o, *part_m, *part_l;
+    int table_stride, seq_len_host, B, KVH, QH, NB, bs, bs_shift, io_dtype;
+    int unit_tiles;                 // tiles per workgroup, or 0: ceil(total / gridDim.x)
+    int Pmax;                       // partial slots per (branch, q head)
+    unsigned head_stride, kv_plane, block_stride, scale_plane, row_bytes;
+    float scale_log2e;
+};
+
+constexpr int kMaxUnits = 256;       // units one workgroup may own (descriptor table in LDS)
+
+struct UnitDesc {                    // one 64-token tile of one (branch, kv head)
+    int tile_lim;                    // tokens of the tile that exist: seq_len - tile*64 (may exceed 64)
+    int flags;                       // bit 0: first tile of a segment of this workgroup, bit 1: last
+    int bq;                          // branch*QH + kvh*4: first query row of the group (Q, partial slots)
+    int piece;                       // partial slot of the segment inside its (branch, q head)
+};
+
+// one wave's 16-token group of a tile, as loaded from the pool
+template <int DT> struct KRegs { uint4 r0, r1, r2, r3; };
+template <> struct KRegs<DRK_INT8> { uint4 r0, r1; };
+template <> struct KRegs<DRK_FP8_E4M3> { uint4 r0, r1; };
+template <int DT> struct VRegs { uint4 r0, r1, r2, r3; };
+template <> struct VRegs<DRK_INT8> { uint2 r0, r1, r2, r3; };
+template <> struct VRegs<DRK_FP8_E4M3> { uint2 r0, r1, r2, r3; };
+
+template <int DT>
+__device__ __forceinline__ KRegs<DT> load_k(const uint8_t *__restrict__ p, bool valid, int lane)
+{
+    KRegs<DT> k;
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    if constexpr (KvTraits<DT>::q8) {
+        k.r0 = k.r1 = z;
+        if (valid) {
+            p += (size_t)lane * 16;
+            k.r0 = *(const uint4 *)(p);
+            k.r1 = *(const uint4 *)(p + 1024);
+        }
+    } else {
+        k.r0 = k.r1 = k.r2 = k.r3 = z;
+        if (valid) {
+            p += (size_t)lane * 16;
+            k.r0 = *(const uint4 *)(p);
+            k.r1 = *(const uint4 *)(p + 1024);
+            k.r2 = *(const uint4 *)(p + 2048);
+            k.r3 = *(const uint4 *)(p + 3072);
+        }
+    }
+    return k;
+}
+
+template <int DT>
+__device__ __forceinline__ VRegs<DT> load_v(const uint8_t *__restrict__ p, bool valid, int lane)
+{
+    VRegs<DT> v;
+    if constexpr (KvTraits<DT>::q8) {
+        const uint2 z = make_uint2(0, 0);
+        v.r0 = v.r1 = v.r2 = v.r3 = z;
+        if (valid) {
+            p += (size_t)lane * 8;
+            v.r0 = *(const uint2 *)(p);
+            v.r1 = *(const uint2 *)(p + 512);
+            v.r2 = *(const uint2 *)(p + 1024);
+            v.r3 = *(const uint2 *)(p + 1536);
+        }
+    } else {
+        const uint4 z = make_uint4(0, 0, 0, 0);
+        v.r0 = v.r1 = v.r2 = v.r3 = z;
+        if (valid) {
+            p += (size_t)lane * 16;
+            v.r0 = *(const uint4 *)(p);
+            v.r1 = *(const uint4 *)(p + 1024);
+            v.r2 = *(const uint4 *)(p + 2048);
+            v.r3 = *(const uint4 *)(p + 3072);
+        }
+    }
+    return v;
+}
+
+// stage the wave's 16 K rows as 16-bit values: rows w*16 .. w*16+15 of the tile
+template <int DT>
+__device__ __forceinline__ void stage_k(uint8_t *tile_lds, const KRegs<DT> &k, int w, int lane)
+{
+    if constexpr (KvTraits<DT>::q8) {
+        // a loaded register holds 16 codes of row (lane>>3) + 8*j, dims (lane&7)*16 ..
+        uint8_t *dst = tile_lds + (w * 16 + (lane >> 3)) * kSRow + (lane & 7) * 32;
+        const uint4 regs[2] = {k.r0, k.r1};
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            uint32_t h[8];
+            if constexpr (DT == DRK_INT8) {
+                int8x4_to_f16x4(regs[j].x, h[0], h[1]);
+                int8x4_to_f16x4(regs[j].y, h[2], h[3]);
+                int8x4_to_f16x4(regs[j].z, h[4], h[5]);
+                int8x4_to_f16x4(regs[j].w, h[6], h[7]);
+            } else {
+                fp8x4_to_f16x4(regs[j].x, h[0], h[1]);
+                fp8x4_to_f16x4(regs[j].y, h[2], h[3]);
+                fp8x4_to_f16x4(regs[j].z, h[4], h[5]);
+                fp8x4_to_f16x4(regs[j].w, h[6], h[7]);
+            }
+            *(uint4 *)(dst + j * 8 * kSRow) = make_uint4(h[0], h[1], h[2], h[3]);
+            *(uint4 *)(dst + j * 8 * kSRow + 16) = make_uint4(h[4], h[5], h[6], h[7]);
+        }
+    } else {
+        uint8_t *dst = tile_lds + (w * 16 + (lane >> 4)) * kSRow + (lane & 15) * 16;
+        *(uint4 *)(dst) = k.r0;
+        *(uint4 *)(dst + 4 * kSRow) = k.r1;
+        *(uint4 *)(dst + 8 * kSRow) = k.r2;
+        *(uint4 *)(dst + 12 * kSRow) = k.r3;
+    }
+}
+
+// o[h][e] += pp[h] * V[row][dims of this lane], 8 dims per lane
+template <int DT, typename VR>
+__device__ __forceinline__ void pv_row(float (&o)[4][8], float (&psum)[4], const VR &vv, const float4 pp)
+{
+    float x[8];
+    if constexpr (DT == DRK_INT8) {
+        const uint32_t a = vv.x ^ 0x80808080u, b = vv.y ^ 0x80808080u;        // code + 128, 0..255
+        x[0] = (float)(a & 0xffu); x[1] = (float)((a >> 8) & 0xffu); x[2] = (float)((a >> 16) & 0xffu); x[3] = (float)(a >> 24);
+        x[4] = (float)(b & 0xffu); x[5] = (float)((b >> 8) & 0xffu); x[6] = (float)((b >> 16) & 0xffu); x[7] = (float)(b >> 24);
+        psum[0] += pp.x; psum[1] += pp.y; psum[2] += pp.z; psum[3] += pp.w;   // the +128 is taken out at the end
+    } else if constexpr (DT == DRK_FP8_E4M3) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        const f2 a0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.x, false), a1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.x, true);
+        const f2 b0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.y, false), b1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.y, true);
+        x[0] = a0[0]; x[1] = a0[1]; x[2] = a1[0]; x[3] = a1[1];
+        x[4] = b0[0]; x[5] = b0[1]; x[6] = b1[0]; x[7] = b1[1];
+#endif
+    } else {
+        const uint32_t wds[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if constexpr (DT == DRK_BF16) { x[2 * i] = bf16_lo(wds[i]); x[2 * i + 1] = bf16_hi(wds[i]); }
+            else { x[2 * i] = f16_bits_to_f((uint16_t)(wds[i] & 0xffffu)); x[2 * i + 1] = f16_bits_to_f((uint16_t)(wds[i] >> 16)); }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        o[0][e] = fmaf(pp.x, x[e], o[0][e]);
+        o[1][e] = fmaf(pp.y, x[e], o[1][e]);
+        o[2][e] = fmaf(pp.z, x[e], o[2][e]);
+        o[3][e] = fmaf(pp.w, x[e], o[3][e]);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void decode_stream_kernel(StreamArgs A)
+{
+    constexpr bool Q8 = KvTraits<DT>::q8;
+    constexpr int DOT = KvTraits<DT>::dot;
+    constexpr uint32_t kNone = 0xffffffffu;
+    __shared__ __align__(16) uint8_t k_lds[2][kSTile * kSRow];
+    __shared__ __align__(16) float p_lds[2][kSTile * 4];
+    __shared__ __align__(16) float alpha_lds[2][4];
+    __shared__ __align__(16) float kscale_lds[2][kSTile];
+    __shared__ __align__(16) float vscale_lds[2][kSTile];
+    __shared__ __align__(16) UnitDesc udesc[kMaxUnits];
+    __shared__ __align__(16) uint2 gdesc[kMaxUnits][4];       // per 16-token group: K byte offset (kNone: skip), scale offset
+    __shared__ int s_incl[64], s_len[64];
+
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int lrow = lane >> 4, lchunk = lane & 15;
+
+    // ---- the workgroup's run of units and one descriptor per unit ---------------------
+    const int len_i = lane < A.B ? (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host) : 0;
+    const int nt_i = len_i > 0 ? (len_i + kSTile - 1) / kSTile : 0;
+    int incl = nt_i;                                           // inclusive prefix of tiles over branches
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int t = __shfl_up(incl, off);
+        if (lane >= off) incl += t;
+    }
+    const int T = __builtin_amdgcn_readlane(incl, 63) * A.KVH;
+    if (T == 0) return;
+    const int U = A.unit_tiles > 0 ? A.unit_tiles : (T + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int u0 = (int)blockIdx.x * U;
+    if (u0 >= T) return;
+    const int nunits = min(U, T - u0);
+    if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nunits * 4; i += 256) {
+        const int ui = i >> 2, grp = i & 3, u = u0 + ui;
+        int lo = 0, hi = A.B - 1;                              // first branch whose cumulative units exceed u
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (A.KVH * s_incl[mid] > u) hi = mid; else lo = mid + 1;
+        }
+        const int b = lo;
+        const int excl = b ? s_incl[b - 1] : 0, nt = s_incl[b] - excl, len = s_len[b];
+        const int rem = u - A.KVH * excl, kvh = rem / nt, tile = rem - kvh * nt;
+        const int tg = tile * kSTile + grp * 16;
+        uint2 gd = make_uint2(kNone, 0u);
+        if (tg < len) {
+            const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
+            const int blk = A.tables[(size_t)b * A.table_stride + lb];
+            if (blk >= 0 && blk < A.NB) {
+                const unsigned pp = (unsigned)(tg - lb * A.bs);
+                const unsigned base = (unsigned)blk * A.block_stride;
+                gd.x = base + (unsigned)kvh * A.head_stride + pp * A.row_bytes;
+                gd.y = base + 2u * A.kv_plane + ((unsigned)kvh * A.bs + pp) * 2u;
+            }
+        }
+        gdesc[ui][grp] = gd;
+        if (grp == 0) {
+            UnitDesc d;
+            d.tile_lim = len - tile * kSTile;
+            d.flags = ((ui == 0 || tile == 0) ? 1 : 0) | ((ui == nunits - 1 || tile + 1 == nt) ? 2 : 0);
+            d.bq = b * A.QH + kvh * 4;
+            d.piece = (int)blockIdx.x - (A.KVH * excl + kvh * nt) / U;
+            udesc[ui] = d;
+        }
+    }
+    __syncthreads();
+
+    auto load_scales = [&](uint2 gd) -> uint32_t {
+        // lanes 0-15: K scale of token lane, lanes 16-31: V scale of token lane-16
+        if (DT != DRK_INT8 || gd.x == kNone || lane >= 32) return 0u;
+        return *(const uint16_t *)(A.pool_layer + gd.y + (lane & 15) * 2 + (lane >= 16 ? A.scale_plane : 0u));
+    };
+    auto load_q = [&](int bq) -> uint32_t {
+        // one packed pair of query head (bq + w) per lane; quantised pages multiply in fp16
+        uint32_t v = ((const uint32_t *)(A.q + (size_t)(bq + w) * 256))[lane];
+#if defined(__HIP_DEVICE_COMPILE__)
+        if (Q8 && A.io_dtype == DRK_BF16)
+            v = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v), bf16_hi(v)));
+#endif
+        return v;
+    };
+
+    float o[4][8], psum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int hh = 0; hh < 4; hh++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[hh][e] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+    uint32_t qs[64];
+
+    uint2 gd = gdesc[0][w];
+    KRegs<DT> kreg = load_k<DT>(A.pool_layer + gd.x, gd.x != kNone, lane);
+    VRegs<DT> vreg = load_v<DT>(A.pool_layer + gd.x + A.kv_plane, gd.x != kNone, lane);
+    uint32_t sreg = load_scales(gd);
+    uint32_t qv = load_q(udesc[0].bq);
+
+    for (int it = 0; it < nunits; it++) {
+        const int buf = it & 1;
+        const UnitDesc ud = udesc[it];
+        const int flags = __builtin_amdgcn_readfirstlane(ud.flags);
+        const int tile_lim = __builtin_amdgcn_readfirstlane(ud.tile_lim);
+        const bool has_next = it + 1 < nunits;
+        if (flags & 1) {                          // Q of the segment's head into scalar registers
+#pragma unroll
+            for (int i = 0; i < 64; i++) qs[i] = __builtin_amdgcn_readlane(qv, i);
+        }
+
+        // ---- A: stage K (and scales), start the next unit's K loads -------------------
+        stage_k<DT>(&k_lds[buf][0], kreg, w, lane);
+        if (DT == DRK_INT8 && lane < 32) {
+            const float sc = f16_bits_to_f((uint16_t)sreg);
+            if (lane < 16) kscale_lds[buf][w * 16 + lane] = sc;
+            else vscale_lds[buf][w * 16 + lane - 16] = sc;
+        }
+        if (has_next) {
+            gd = gdesc[it + 1][w];
+            kreg = load_k<DT>(A.pool_layer + gd.x, gd.x != kNone, lane);
+            sreg = load_scales(gd);
+            if (flags & 2) qv = load_q(udesc[it + 1].bq);
+        }
+        __syncthreads();
+
+        // ---- B: scores of head w for the tile's 64 tokens, tile softmax -----------------
+        {
+            const uint8_t *krow = &k_lds[buf][lane * kSRow];
+            float acc = 0.0f;
+            uint4 ka[4], kb[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) ka[c] = *(const uint4 *)(krow + c * 16);
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                if (g4 < 3) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) kb[c] = *(const uint4 *)(krow + ((g4 + 1) * 4 + c) * 16);
+                }
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const int qi = (g4 * 4 + c) * 4;
+                    acc = s_dot2<DOT>(ka[c].x, qs[qi + 0], acc);
+                    acc = s_dot2<DOT>(ka[c].y, qs[qi + 1], acc);
+                    acc = s_dot2<DOT>(ka[c].z, qs[qi + 2], acc);
+                    acc = s_dot2<DOT>(ka[c].w, qs[qi + 3], acc);
+                }
+                asm volatile("" : "+v"(acc) :: "memory");   // at most two groups of LDS reads in flight
+#pragma unroll
+                for (int c = 0; c < 4; c++) ka[c] = kb[c];
+            }
+            const bool live = lane < tile_lim && gdesc[it][lane >> 4].x != kNone;
+            float sc = acc * A.scale_log2e;
+            if (DT == DRK_INT8) sc *= kscale_lds[buf][lane];
+            sc = live ? sc : -INFINITY;
+            const float m_new = fmaxf(m_run, s_wave_max(sc));
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float p = s_exp2(sc - m_use);
+            const float alpha = s_exp2(m_run - m_use);
+            l_run = l_run * alpha + s_wave_sum(p);
+            m_run = m_new;
+            float pw = p;
+            if (DT == DRK_INT8) pw = live ? p * vscale_lds[buf][lane] : 0.0f;   // a stale scale may be anything
+            p_lds[buf][lane * 4 + w] = pw;
+            if (lane == 0) alpha_lds[buf][w] = alpha;
+        }
+        __syncthreads();
+
+        // ---- C: o += P V over this wave's 16 tokens, all 4 heads ----------------------
+        {
+            const float4 al = *(const float4 *)&alpha_lds[buf][0];
+            if (al.x != 1.0f || al.y != 1.0f || al.z != 1.0f || al.w != 1.0f) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    o[0][e] *= al.x; o[1][e] *= al.y; o[2][e] *= al.z; o[3][e] *= al.w;
+                }
+                psum[0] *= al.x; psum[1] *= al.y; psum[2] *= al.z; psum[3] *= al.w;
+            }
+            const int r0 = w * 16 + lrow;
+            if (DT != DRK_INT8 && tile_lim < kSTile) {        // rows past the end may hold anything
+                if (r0 >= tile_lim) vreg.r0 = {};
+                if (r0 + 4 >= tile_lim) vreg.r1 = {};
+                if (r0 + 8 >= tile_lim) vreg.r2 = {};
+                if (r0 + 12 >= tile_lim) vreg.r3 = {};
+            }
+            const float *pl = &p_lds[buf][r0 * 4];
+            pv_row<DT>(o, psum, vreg.r0, *(const float4 *)(pl));
+            pv_row<DT>(o, psum, vreg.r1, *(const float4 *)(pl + 16));
+            pv_row<DT>(o, psum, vreg.r2, *(const float4 *)(pl + 32));
+            pv_row<DT>(o, psum, vreg.r3, *(const float4 *)(pl + 48));
+        }
+        if (has_next) vreg = load_v<DT>(A.pool_layer + gd.x + A.kv_plane, gd.x != kNone, lane);
+
+        // ---- the segment's last tile: leave (o, m, l) for the merge ----------------------
+        if (flags & 2) {
+#pragma unroll
+            for (int hh = 0; hh < 4; hh++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    float v = o[hh][e];
+                    if (DT == DRK_INT8) v -= 128.0f * psum[hh];
+                    v += __shfl_xor(v, 16);
+                    v += __shfl_xor(v, 32);
+                    o[hh][e] = v;
+                }
+            float *o_lds = (float *)&k_lds[0][0];        // [wave][head][128] fp32 = 8 KiB; K reads are done
+            __syncthreads();
+            if (lrow == 0) {
+#pragma unroll
+                for (int hh = 0; hh < 4; hh++) {
+                    float *dst = o_lds + (w * 4 + hh) * 128 + lchunk * 8;
+                    *(float4 *)dst = make_float4(o[hh][0], o[hh][1], o[hh][2], o[hh][3]);
+                    *(float4 *)(dst + 4) = make_float4(o[hh][4], o[hh][5], o[hh][6], o[hh][7]);
+                }
+            }
+            __syncthreads();
+            {
+                const int d = lane * 2;
+                float2 acc = make_float2(0.0f, 0.0f);
+#pragma unroll
+                for (int ww = 0; ww < 4; ww++) {
+                    const float2 v = *(const float2 *)(o_lds + (ww * 4 + w) * 128 + d);
+                    acc.x += v.x;
+                    acc.y += v.y;
+                }
+                const size_t pi = (size_t)(ud.bq + w) * A.Pmax + ud.piece;
+                *(float2 *)(A.part_o + pi * 128 + d) = acc;
+                if (lane == 0) {
+                    A.part_m[pi] = m_run;
+                    A.part_l[pi] = l_run;
+                }
+            }
+            __syncthreads();                             // o_lds is free again before the next tile is staged
+#pragma unroll
+            for (int hh = 0; hh < 4; hh++) {
+                psum[hh] = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[hh][e] = 0.0f;
+            }
+            m_run = -INFINITY;
+            l_run = 0.0f;
+        }
+    }
+}
+
+// grid (QH, B), block 128: fold the pieces of (branch, q head); out is written only
+// when some token took part (paged_attention.cu:266)
+__global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_m,
+                                                           const float *__restrict__ part_l, uint16_t *__restrict__ out,
+                                                           const int32_t *__restrict__ seq_lens, int seq_len_host, int B,
+                                                           int KVH, int QH, int unit_tiles, int grid_wgs, int Pmax,
+                                                           int io_dtype)
+{
+    const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    int excl = 0, total = 0, nt_b = 0;
+    for (int i = 0; i < B; i++) {
+        const int len = seq_lens ? seq_lens[i] : seq_len_host;
+        const int nt = len > 0 ? (len + kSTile - 1) / kSTile : 0;
+        if (i < b) excl += nt;
+        if (i == b) nt_b = nt;
+        total += nt;
+    }
+    if (nt_b == 0) return;
+    const int T = total * KVH;
+    const int U = unit_tiles > 0 ? unit_tiles : (T + grid_wgs - 1) / grid_wgs;
+    const int kvh = h / (QH / KVH);
+    const int first = KVH * excl + kvh * nt_b, last = first + nt_b - 1;
+    const int npieces = last / U - first / U + 1;
+    const size_t base = ((size_t)b * QH + h) * Pmax;
+    float M = -INFINITY;
+    for (int s = 0; s < npieces; s++)
+        if (part_l[base + s] > 0.0f) M = fmaxf(M, part_m[base + s]);
+    float acc = 0.0f, L = 0.0f;
+    for (int s = 0; s < npieces; s++) {
+        const float pl = part_l[base + s];
+        if (!(pl > 0.0f)) continue;
+        const float wgt = s_exp2(part_m[base + s] - M);
+        acc = fmaf(part_o[(base + s) * 128 + d], wgt, acc);
+        L = fmaf(pl, wgt, L);
+    }
+    if (L > 0.0f) out[((size_t)b * QH + h) * 128 + d] = f_to_elem16(acc / L, io_dtype);
+}
+
+bool stream_decode_supported(const Lay &a, int B)
+{
+    // offsets inside a layer are kept in 32 bits by the unit descriptors
+    return a.D == 128 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && B >= 1 && B <= 64 &&
+           a.layer_stride <= 0xffff0000ull;
+}
+
+static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens, int *grid, int *unit_tiles, int *Pmax)
+{
+    const long t_upper = (long)a.KVH * B * ((max_seq_len + kSTile - 1) / kSTile);
+    if (split_tokens > 0) {
+        const int U = split_tokens / kSTile;
+        *unit_tiles = U;
+        *grid = (int)((t_upper + U - 1) / U);
+        *Pmax = ((max_seq_len + kSTile - 1) / kSTile + U - 1) / U + 2;
+    } else {
+        long G = t_upper < g_stream_wgs ? t_upper : g_stream_wgs;
+        if ((t_upper + G - 1) / G > kMaxUnits) G = (t_upper + kMaxUnits - 1) / kMaxUnits;   // descriptor table size
+        *unit_tiles = 0;
+        *grid = (int)G;
+        *Pmax = (int)((G + a.KVH - 1) / a.KVH) + 2;
+    }
+}
+
+size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens)
+{
+    int grid, U, Pmax;
+    stream_shape(a, B, max_seq_len, split_tokens, &grid, &U, &Pmax);
+    return (size_t)B * a.QH * Pmax * (a.D + 2) * sizeof(float);
+}
+
+// launches the partial kernel; *merge_fn_args are filled for the caller to launch the merge
+int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
+                         const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
+                         float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st)
+{
+    int grid, U, Pmax;
+    stream_shape(a, B, max_seq_len, split_tokens, &grid, &U, &Pmax);
+    float *part_o = (float *)workspace;
+    float *part_m = part_o + (size_t)B * a.QH * Pmax * a.D;
+    float *part_l = part_m + (size_t)B * a.QH * Pmax;
+    if (!merge_only) {
+        StreamArgs A;
+        A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
+        A.tables = tables; A.seq_lens = d_seq_lens; A.q = (const uint8_t *)q;
+        A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
+        A.table_stride = table_stride; A.seq_len_host = seq_len_host; A.B = B; A.KVH = a.KVH; A.QH = a.QH;
+        A.NB = a.NB; A.bs = a.bs; A.bs_shift = ilog2_exact((unsigned)a.bs); A.io_dtype = io_dtype;
+        A.unit_tiles = U; A.Pmax = Pmax;
+        A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
+        A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
+        A.scale_log2e = scale * kSLog2e;
+        switch (a.dtype) {
+        case DRK_F16: hipLaunchKernelGGL(decode_stream_kernel<DRK_F16>, dim3(grid), dim3(256), 0, st, A); break;
+        case DRK_BF16: hipLaunchKernelGGL(decode_stream_kernel<DRK_BF16>, dim3(grid), dim3(256), 0, st, A); break;
+        case DRK_INT8: hipLaunchKernelGGL(decode_stream_kernel<DRK_INT8>, dim3(grid), dim3(256), 0, st, A); break;
+        default: hipLaunchKernelGGL(decode_stream_kernel<DRK_FP8_E4M3>, dim3(grid), dim3(256), 0, st, A); break;
+        }
+        DRK_LAUNCH_CHECK("decode_stream_kernel");
+    } else {
+        hipLaunchKernelGGL(stream_merge_kernel, dim3(a.QH, B), dim3(128), 0, st, part_o, part_m, part_l, (uint16_t *)out,
+                           d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype);
+        DRK_LAUNCH_CHECK("stream_merge_kernel");
+    }
+    return DRK_OK;
+}
+
+} // namespace drk

@@ -155,6 +155,12 @@ int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len);
  * geometry, any storage type) instead of the tiled one, so that tests can
  * check the two against each other.  Process-wide, not thread-safe. */
 void drk_debug_force_portable_decode(int on);
+/* Diagnostic: which kernel produces the decode partials when the geometry allows
+ * a choice: 0 = automatic (the persistent stream kernel), 2 = the fixed-split
+ * tiled kernel (16-bit pages only), 3 = same as 0.  Process-wide. */
+void drk_debug_set_decode_kernel(int which);
+/* Diagnostic: workgroups of the persistent decode grid (default 512). */
+void drk_debug_set_stream_workgroups(int n);
 /* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
  * session; switching it on starts a new session) records a HIP event on its
  * stream right before and right after the split-K partial kernel; the merge

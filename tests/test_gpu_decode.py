@@ -20,7 +20,7 @@ REL, ABS = 1e-2, 2e-2
 class Case:
     """A filled pool on host (oracle) and device, B branches with disjoint pages."""
 
-    def __init__(self, geom, dtype, seq_lens, seed, mul=1.0, io_dtype=None, holes=()):
+    def __init__(self, geom, dtype, seq_lens, seed, mul=1.0, io_dtype=None, holes=(), outliers=False, stale=0):
         L, KVH, QH, D, bs, NB = geom
         self.geom, self.dtype = geom, dtype
         self.io = io_dtype if io_dtype is not None else (dtype if dtype in (cabi.F16, cabi.BF16) else cabi.BF16)
@@ -40,14 +40,18 @@ class Case:
             o += nblk[b]
         self.opool = orc.new_pool(self.og)
         # stale garbage everywhere first: positions past seq_len must not matter
-        self.opool[:] = 0
+        self.opool[:] = stale
         self.layer = L - 1
         for b in range(B):
             n = int(seq_lens[b])
             if n == 0:
                 continue
-            k = U.normal_bits(rng, (n, KVH, D), self.io, mul)
-            v = U.normal_bits(rng, (n, KVH, D), self.io, mul)
+            kf = rng.standard_normal((n, KVH, D)).astype(np.float32) * np.float32(mul)
+            vf = rng.standard_normal((n, KVH, D)).astype(np.float32) * np.float32(mul)
+            if outliers:
+                kf = np.where(rng.random(kf.shape) < 0.01, kf * 20, kf)
+                vf = np.where(rng.random(vf.shape) < 0.01, vf * 20, vf)
+            k, v = U.to_bits(kf, self.io), U.to_bits(vf, self.io)
             orc.append_batch(self.og, self.opool, self.tables[b], self.layer, 0, k, v, self.io)
         for (b, lb) in holes:
             self.tables[b, lb] = -1
@@ -99,11 +103,13 @@ def _check(case, got):
     return max_abs
 
 
-@pytest.fixture(params=["tiled", "portable"])
+@pytest.fixture(params=["stream", "tiled", "portable"])
 def kernel(request):
     cabi.lib().drk_debug_force_portable_decode(1 if request.param == "portable" else 0)
+    cabi.lib().drk_debug_set_decode_kernel(2 if request.param == "tiled" else 0)
     yield request.param
     cabi.lib().drk_debug_force_portable_decode(0)
+    cabi.lib().drk_debug_set_decode_kernel(0)
 
 
 def test_config1_decode(dev, kernel):
@@ -237,10 +243,19 @@ def test_other_geometries(dev, geom, dtype):
 
 @pytest.mark.parametrize("dtype", [cabi.INT8, cabi.FP8_E4M3])
 @pytest.mark.parametrize("io", [cabi.F16, cabi.BF16])
-def test_quantised_pools(dev, dtype, io):
-    """Dequantisation inside attention: the fp64 oracle runs on the same codes."""
-    case = Case((1, 8, 32, 128, 16, 200), dtype, [1500, 260], seed=71, io_dtype=io)
-    _check(case, case.run_branches())
+@pytest.mark.parametrize("portable", [0, 1])
+def test_quantised_pools(dev, dtype, io, portable):
+    """Dequantisation inside attention: the fp64 oracle runs on the same codes
+    (BASELINE config 4 in small: K/V with 1 % outliers x20, ragged lengths, a hole,
+    stale bytes after the end)."""
+    cabi.lib().drk_debug_force_portable_decode(portable)
+    try:
+        case = Case((1, 8, 32, 128, 16, 400), dtype, [1500, 260, 64, 1, 2047], seed=71, io_dtype=io, outliers=True,
+                    holes=[(0, 7)], stale=0xFF)
+        _check(case, case.run_branches())
+        _check(case, case.run_branches(split=128))
+    finally:
+        cabi.lib().drk_debug_force_portable_decode(0)
 
 
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
