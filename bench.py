@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), scaled by what the same
 # counters read for a plain 32 GiB read (x2.0) and a bulk append of known size
 # (x1.0).  Keyed by the algorithmic bytes of the launch it was measured on.
-MEASURED_TRAFFIC_BYTES = {1073741824: (524893 * 2 + 1152) * 1024}
+MEASURED_TRAFFIC_BYTES = {1073741824: int((524643.0 * 2 + 1154.8) * 1024)}
 
 
 def parse():
@@ -45,6 +45,10 @@ def parse():
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="context per branch for the CPU sample (0 = auto)")
     ap.add_argument("--bulk-append-tokens", type=int, default=2048)
     ap.add_argument("--seed", type=int, default=2)
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5],
+                    help="BASELINE config: 2 (default, the headline) | 3 shared prefix + COW + eviction | "
+                         "4 int8/fp8 pages at 128k | 5 chunked MFMA prefill interleaved with decode")
+    ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8", help="config 4 storage type")
     return ap.parse_args()
 
 
@@ -59,6 +63,10 @@ def main():
     from tests import util as U
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.config != 2:
+        import bench_extra
+        print(json.dumps(bench_extra.run(args)))
+        return
     lib = cabi.lib()
     torch.cuda.set_device(0)
     rng = np.random.default_rng(args.seed)
@@ -260,7 +268,7 @@ def main():
         "hbm_read_probe_GBps": round(read_probe_gbps, 1),
         "fill_seconds": round(t_fill, 2),
         "roofline": {
-            "kernel": "decode_tiled_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
+            "kernel": "decode_stream_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(launch_bytes), "avg_launch_us": round(ker_avg_ms * 1e3, 2), "bytes_per_launch": launch_bytes,
         },

@@ -1,0 +1,350 @@
+"""bench.py --config 3|4|5: the other BASELINE configurations, same JSON shape.
+
+Not the headline line (that is config 2, bench.py's default); these runs put
+measured numbers beside the parity tests of the same shapes.  Torch is plumbing
+for memory, streams and events; kernels go through the C ABI, block tables of
+config 3 through the C++ CacheManager.
+"""
+import ctypes as C
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def _common(args):
+    import torch
+    from deusridet_amd import cabi
+    from tests import util as U
+    lib = cabi.lib()
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream()
+    return torch, cabi, U, lib, stream, C.c_void_p(stream.cuda_stream)
+
+
+def _timed_decode(lib, cabi, call, n):
+    """average duration of the partial kernel over n back-to-back launches"""
+    call(6)
+    lib.drk_debug_time_decode_kernel(1)
+    call(n)
+    buf = (C.c_float * 256)()
+    cnt = C.c_int32(0)
+    cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
+    lib.drk_debug_time_decode_kernel(0)
+    return float(np.mean(buf[:cnt.value]))
+
+
+def config4(args):
+    """4 branches x 128k tokens, 8 KV heads x 128, int8 (+fp16 scale per token and
+    head) or fp8-e4m3 pages quantised on append, dequantised inside attention."""
+    torch, cabi, U, lib, stream, sp = _common(args)
+    dt = cabi.INT8 if args.kv_dtype == "int8" else cabi.FP8_E4M3
+    L, KVH, QH, D, bs, B, ctx = args.layers, 8, 32, 128, 16, 4, 131072
+    W, K = args.warmup, args.steps
+    probe = cabi.layout(L, KVH, QH, D, bs, 1, dt)
+    NB = lib.drk_kv_max_blocks_for_budget(C.byref(probe), int(args.pool_gb * 1e9))
+    g = cabi.layout(L, KVH, QH, D, bs, NB, dt)
+    rng = np.random.default_rng(4)
+    start = ctx - (W + K)
+    nblk = ctx // bs + 1
+    assert B * nblk <= NB, "pool too small"
+    perm = rng.permutation(NB).astype(np.int32)
+    tables = np.stack([perm[b * nblk:(b + 1) * nblk] for b in range(B)])
+    pool = torch.zeros(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    dtab = torch.from_numpy(tables).cuda()
+    # fill through the quantising append: N(0,1) with 1 % outliers x20; time it as the bulk append figure
+    chunk = 2048
+    a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    append_ms, append_tokens = 0.0, 0
+    for b in range(B):
+        for p0 in range(0, start, chunk):
+            m = min(chunk, start - p0)
+            k = torch.randn(L, m, KVH, D, device="cuda")
+            k = torch.where(torch.rand_like(k) < 0.01, k * 20, k).to(torch.bfloat16)
+            v = torch.randn(L, m, KVH, D, device="cuda")
+            v = torch.where(torch.rand_like(v) < 0.01, v * 20, v).to(torch.bfloat16)
+            a0.record(stream)
+            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(dtab[b].data_ptr()), 0, L, p0, m,
+                      U.p(k), U.p(v), cabi.BF16, sp)
+            a1.record(stream)
+            torch.cuda.synchronize()
+            if m == chunk and p0 > 0:
+                append_ms += a0.elapsed_time(a1)
+                append_tokens += m
+    code_bytes = 2 * KVH * D + (2 * KVH * 2 if dt == cabi.INT8 else 0)      # per token and layer
+    append_gbps = append_tokens * L * (2 * KVH * D * 2 + code_bytes) / (append_ms * 1e-3) / 1e9
+    scale = 1.0 / np.sqrt(D)
+    q = torch.randn(L, B, QH, D, device="cuda").to(torch.bfloat16)
+    nk = torch.randn(L, B, KVH, D, device="cuda").to(torch.bfloat16)
+    nv = torch.randn(L, B, KVH, D, device="cuda").to(torch.bfloat16)
+    out = torch.zeros(L, B, QH, D, device="cuda", dtype=torch.bfloat16)
+    wsb = lib.drk_decode_workspace_bytes(C.byref(g), B, ctx)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    pos_steps = torch.from_numpy(np.stack([np.full(B, start + s, dtype=np.int32) for s in range(W + K)])).cuda()
+    len_steps = pos_steps + 1
+    qrow, krow = B * QH * D * 2, B * KVH * D * 2
+
+    def attn(l, dlen):
+        cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
+                  U.p(dtab), nblk, dlen, B, ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.BF16, 0,
+                  U.p(ws), wsb, sp)
+
+    def step(s):
+        dpos, dlen = C.c_void_p(pos_steps[s].data_ptr()), C.c_void_p(len_steps[s].data_ptr())
+        for l in range(L):
+            cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), nblk, dpos, B, l, 1,
+                      C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
+            attn(l, dlen)
+
+    for s in range(W):
+        step(s)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for s in range(W, W + K):
+        step(s)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    total_ms = e0.elapsed_time(e1)
+    toks = sum(B * (start + s + 1) for s in range(W, W + K))
+    value = toks * code_bytes * L / (total_ms * 1e-3) / 1e9
+    dlen = C.c_void_p(len_steps[W + K - 1].data_ptr())
+    ker_ms = _timed_decode(lib, cabi, lambda n: [attn(i % L, dlen) for i in range(n)], 60)
+    launch_bytes = B * ctx * code_bytes
+    ach = launch_bytes / (ker_ms * 1e-3) / 1e9
+    return {
+        "metric": "paged_decode_attention_GBps", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": round(total_ms / K, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8" if dt == cabi.INT8 else "fp8", "data": "synthetic",
+        "config": {"workload": f"config 4: {L} layers, 32 Q / 8 KV heads x 128, {args.kv_dtype} pages "
+                               f"({code_bytes} B per token and layer), 4 branches x 131072 tokens, K/V N(0,1) with 1 % x20 "
+                               f"outliers quantised on append; step = per layer: append 1 token/branch + decode attention",
+                   "branches": B, "layers": L, "ctx_final": [ctx] * B},
+        "tokens_per_s": round(B * K / (total_ms * 1e-3), 1), "us_per_step": round(total_ms / K * 1e3, 1),
+        "quantising_append_GBps": round(append_gbps, 1),
+        "quantising_append_hbm_frac": round(append_gbps / HBM_PEAK_GBPS, 4),
+        "roofline": {"kernel": f"decode_stream_kernel<{args.kv_dtype}>", "bound": "hbm", "achieved": round(ach, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "avg_launch_us": round(ker_ms * 1e3, 2), "bytes_per_launch": launch_bytes},
+        "cpu_baseline": None,
+    }
+
+
+def config3(args):
+    """One persistent 64k-token prefix shared by 16 branches (copy-on-write forks,
+    refcounts), 0-4k private tokens each, eviction down to 25 % free."""
+    torch, cabi, U, lib, stream, sp = _common(args)
+    from deusridet_amd import host
+    L, KVH, QH, D, bs, NBR = args.layers, 8, 32, 128, 16, 16
+    W, K = args.warmup, args.steps
+    prefix = 65536
+    rng = np.random.default_rng(3)
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    cm = host.CacheManager()
+    assert cm.init(int(args.pool_gb * 1e9), bs, None, NBR + 1), "CacheManager.init failed"
+    NB, stride = cm.pool_max_blocks(), cm.table_stride()
+    hl = host.lib()
+    pool_ptr = C.c_void_p(cm.pool_ptr())
+    chunk = 2048
+
+    def bulk(branch, p0, m):
+        assert cm.ensure_blocks_for_range(branch, p0, m)
+        cm.sync_block_table(sp)
+        k = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+        v = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+        g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+        cabi.call("drk_kv_append_batch", C.byref(g), pool_ptr, C.c_void_p(cm.d_block_table(branch)), 0, L, p0, m,
+                  U.p(k), U.p(v), cabi.BF16, sp)
+        torch.cuda.synchronize()
+        cm.set_seq_len(branch, p0 + m)
+
+    for p0 in range(0, prefix, chunk):
+        bulk(0, p0, chunk)
+    t0 = time.perf_counter()
+    forks = []
+    for i in range(NBR):
+        # block boundaries, except every fourth fork lands inside a block (forces a copy-on-write)
+        fp = prefix if i % 4 else prefix - int(rng.integers(1, bs))
+        forks.append(cm.fork_branch(0, fp))
+    fork_ns = (time.perf_counter() - t0) / NBR * 1e9
+    assert min(forks) > 0
+    private = rng.integers(0, 4097, size=NBR)
+    for b, n in zip(forks, private):
+        base = cm.seq_len(b)
+        for p0 in range(0, int(n), chunk):
+            bulk(b, base + p0, min(chunk, int(n) - p0))
+    lens0 = np.array([cm.seq_len(b) for b in forks], dtype=np.int32)
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    B = NBR
+    scale = 1.0 / np.sqrt(D)
+    q = (torch.randn(L, B, QH, D, device="cuda") * 0.5).to(torch.bfloat16)
+    nk = (torch.randn(L, B, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+    nv = (torch.randn(L, B, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+    out = torch.zeros(L, B, QH, D, device="cuda", dtype=torch.bfloat16)
+    max_ctx = int(lens0.max()) + W + K + 1
+    wsb = lib.drk_decode_workspace_bytes(C.byref(g), B, max_ctx)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    dpos = torch.zeros(B, dtype=torch.int32, device="cuda")
+    dlen = torch.zeros(B, dtype=torch.int32, device="cuda")
+    # the forked branches' rows are consecutive in the device table: branch ids forks[0]..forks[-1]
+    assert forks == list(range(forks[0], forks[0] + B))
+    dtabs = C.c_void_p(cm.d_block_table(forks[0]))
+    qrow, krow = B * QH * D * 2, B * KVH * D * 2
+    ensure_ns, evicted, evict_ns = [], 0, 0.0
+
+    def step(s, lens):
+        nonlocal evicted, evict_ns
+        t = time.perf_counter()
+        for i, b in enumerate(forks):
+            assert cm.ensure_blocks_for(b, int(lens[i]))
+        ensure_ns.append((time.perf_counter() - t) / B * 1e9)
+        if s == W + K // 2:                                   # pressure: free 25 % of the pool, oldest private pages first
+            t = time.perf_counter()
+            before = cm.free_blocks()
+            cm.ensure_free_blocks(NB // 4)
+            evicted += cm.free_blocks() - before
+            evict_ns += (time.perf_counter() - t) * 1e9
+        cm.sync_block_table(sp)                               # COW copies, then table deltas
+        dpos.copy_(torch.from_numpy(lens))
+        dlen.copy_(torch.from_numpy(lens + 1))
+        for l in range(L):
+            cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, U.p(dpos), B, l, 1,
+                      C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr,
+                      dtabs, stride, U.p(dlen), B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
+                      cabi.BF16, 0, U.p(ws), wsb, sp)
+        for i, b in enumerate(forks):
+            cm.set_seq_len(b, int(lens[i]) + 1)
+
+    lens = lens0.copy()
+    for s in range(W):
+        step(s, lens); lens += 1
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    logical = 0
+    for s in range(W, W + K):
+        step(s, lens); lens += 1
+        logical += int(lens.sum())
+    e1.record(stream)
+    torch.cuda.synchronize()
+    total_ms = e0.elapsed_time(e1)
+    per_tok = 2 * KVH * D * 2
+    unique_tokens = cm.gpu_blocks_used() * bs
+    value = logical * per_tok * L / (total_ms * 1e-3) / 1e9
+    dl = U.p(dlen)
+    ker_ms = _timed_decode(lib, cabi, lambda n: [cabi.call(
+        "drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + (i % L) * qrow), pool_ptr, dtabs,
+        stride, dl, B, max_ctx, C.c_void_p(out.data_ptr() + (i % L) * qrow), i % L, float(scale), cabi.BF16, 0, U.p(ws),
+        wsb, sp) for i in range(n)], 60)
+    launch_logical = int(lens.sum()) * per_tok
+    ach = launch_logical / (ker_ms * 1e-3) / 1e9
+    return {
+        "metric": "paged_decode_attention_GBps", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": round(total_ms / K, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config 3: {L} layers, 8 KV heads x 128 bf16, 65536-token prefix shared by 16 copy-on-write "
+                               f"branches (+0..4096 private tokens), eviction to 25 % free once in the timed region; "
+                               f"value counts LOGICAL bytes (every branch's whole context), the prefix is re-read per branch",
+                   "branches": B, "layers": L, "ctx_final": [int(x) for x in lens]},
+        "logical_GB_per_layer_step": round(launch_logical / 1e9, 3),
+        "unique_GB_per_layer": round(unique_tokens * per_tok / 1e9, 3),
+        "us_per_step": round(total_ms / K * 1e3, 1), "tokens_per_s": round(B * K / (total_ms * 1e-3), 1),
+        "host_ns": {"fork_branch": round(fork_ns), "ensure_blocks_for": round(float(np.mean(ensure_ns))),
+                    "evict_per_block": round(evict_ns / max(evicted, 1)), "blocks_evicted": int(evicted)},
+        "roofline": {"kernel": "decode_stream_kernel<bf16>", "bound": "hbm", "achieved": round(ach, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "avg_launch_us": round(ker_ms * 1e3, 2), "bytes_per_launch": launch_logical,
+                     "note": "logical bytes: shared prefix pages are requested once per branch and partly served by "
+                             "L2 / Infinity Cache, so this figure can exceed what HBM alone delivers"},
+        "cpu_baseline": None,
+    }
+
+
+def config5(args):
+    """Chunked prefill to 32k in 2048-token chunks (append into pages, then causal
+    MFMA attention over all prior pages plus the chunk) with 4 decode branches at
+    8k interleaved on the same pool."""
+    torch, cabi, U, lib, stream, sp = _common(args)
+    L, KVH, QH, D, bs = min(args.layers, 4), 8, 32, 128, 16
+    chunk, total, DB, dctx = 2048, 32768, 4, 8192
+    NB = (total + DB * (dctx + 64)) // bs + 64
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    rng = np.random.default_rng(5)
+    perm = rng.permutation(NB).astype(np.int32)
+    nb_seq, nb_dec = total // bs, dctx // bs + 4
+    tab_seq = torch.from_numpy(perm[:nb_seq].copy()).cuda()
+    tab_dec = torch.from_numpy(np.stack([perm[nb_seq + b * nb_dec: nb_seq + (b + 1) * nb_dec] for b in range(DB)])).cuda()
+    pool = torch.zeros(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    for b in range(DB):
+        for p0 in range(0, dctx, chunk):
+            k = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+            v = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(tab_dec[b].data_ptr()), 0, L, p0, chunk,
+                      U.p(k), U.p(v), cabi.BF16, sp)
+            torch.cuda.synchronize()
+    qd = torch.randn(L, DB, QH, D, device="cuda").to(torch.bfloat16)
+    od = torch.zeros_like(qd)
+    nk = torch.randn(L, DB, KVH, D, device="cuda").to(torch.bfloat16)
+    nv = torch.randn(L, DB, KVH, D, device="cuda").to(torch.bfloat16)
+    wsb = lib.drk_decode_workspace_bytes(C.byref(g), DB, dctx + 64)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    dpos = torch.full((DB,), dctx, dtype=torch.int32, device="cuda")
+    dlen = dpos + 1
+    qrow, krow = DB * QH * D * 2, DB * KVH * D * 2
+    pf_ms, pf_flops, ap_ms, dec_ms = 0.0, 0.0, 0.0, []
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    passes = max(1, args.steps // 16) + 1                        # first pass warms up
+    for ps in range(passes):
+        for c in range(total // chunk):
+            k = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+            v = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+            q = torch.randn(L, chunk, QH, D, device="cuda").to(torch.bfloat16)
+            o = torch.empty_like(q)
+            ev[0].record(stream)
+            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(tab_seq), 0, L, c * chunk, chunk, U.p(k), U.p(v),
+                      cabi.BF16, sp)
+            ev[1].record(stream)
+            for l in range(L):
+                cabi.call("drk_paged_prefill_attention", C.byref(g), C.c_void_p(q.data_ptr() + l * chunk * QH * D * 2),
+                          U.p(pool), U.p(tab_seq), C.c_void_p(o.data_ptr() + l * chunk * QH * D * 2), l, c * chunk, chunk,
+                          float(scale), cabi.BF16, None, 0, sp)
+            ev[2].record(stream)
+            for l in range(L):                                   # one interleaved decode step of the 4 branches
+                cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(tab_dec), nb_dec, U.p(dpos), DB, l, 1,
+                          C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
+                cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(qd.data_ptr() + l * qrow),
+                          U.p(pool), U.p(tab_dec), nb_dec, U.p(dlen), DB, dctx + 64, C.c_void_p(od.data_ptr() + l * qrow),
+                          l, float(scale), cabi.BF16, 0, U.p(ws), wsb, sp)
+            ev[3].record(stream)
+            torch.cuda.synchronize()
+            if ps > 0:
+                ap_ms += ev[0].elapsed_time(ev[1])
+                pf_ms += ev[1].elapsed_time(ev[2])
+                pf_flops += L * 4.0 * chunk * (c * chunk + (chunk + 1) / 2.0) * D * QH
+                dec_ms.append(ev[2].elapsed_time(ev[3]))
+    tfl = pf_flops / (pf_ms * 1e-3) / 1e12
+    nchunks = (passes - 1) * (total // chunk)
+    ap_gbps = nchunks * L * chunk * 2 * (2 * KVH * D * 2) / (ap_ms * 1e-3) / 1e9
+    return {
+        "metric": "chunked_prefill_attention_TFLOPs", "value": round(tfl, 1), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": nchunks, "warmup": total // chunk, "ms_per_step": round(pf_ms / nchunks / L, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config 5: one sequence prefilled to 32768 in 2048-token chunks, 32 Q / 8 KV heads x 128 "
+                               f"bf16, 16-token pages, {L} layers; per chunk: append, causal attention over all pages so far "
+                               f"(MFMA), then one decode step of 4 branches at 8192 on the same pool; a step here is one "
+                               f"(chunk, layer) attention launch", "layers": L},
+        "chunk_append_GBps": round(ap_gbps, 1),
+        "interleaved_decode_us_per_layer": round(float(np.mean(dec_ms)) / L * 1e3, 1),
+        "roofline": {"kernel": "prefill_mfma_kernel<bf16>", "bound": "mfma", "achieved": round(tfl, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": None},
+        "cpu_baseline": None,
+    }
+
+
+def run(args):
+    return {3: config3, 4: config4, 5: config5}[args.config](args)

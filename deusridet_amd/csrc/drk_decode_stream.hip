@@ -65,17 +65,41 @@ __device__ __forceinline__ float s_exp2(float x)
 #endif
 }
 
+// Wave-wide reductions: four DPP steps reduce inside each row of 16 lanes
+// (quad swaps, then half-row and row mirrors), four v_readlane fold the rows.
+template <int CTRL>
+__device__ __forceinline__ float s_dpp(float v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+#else
+    return v;
+#endif
+}
+__device__ __forceinline__ float s_lane(float v, int l)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+#else
+    (void)l;
+    return v;
+#endif
+}
 __device__ __forceinline__ float s_wave_max(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
+    v = fmaxf(v, s_dpp<0xB1>(v));      // quad_perm [1,0,3,2]
+    v = fmaxf(v, s_dpp<0x4E>(v));      // quad_perm [2,3,0,1]
+    v = fmaxf(v, s_dpp<0x141>(v));     // row_half_mirror
+    v = fmaxf(v, s_dpp<0x140>(v));     // row_mirror
+    return fmaxf(fmaxf(s_lane(v, 0), s_lane(v, 16)), fmaxf(s_lane(v, 32), s_lane(v, 48)));
 }
 __device__ __forceinline__ float s_wave_sum(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+    v += s_dpp<0xB1>(v);
+    v += s_dpp<0x4E>(v);
+    v += s_dpp<0x141>(v);
+    v += s_dpp<0x140>(v);
+    return (s_lane(v, 0) + s_lane(v, 16)) + (s_lane(v, 32) + s_lane(v, 48));
 }
 
 // four int8 codes -> two dwords of packed fp16, exact: (code ^ 0x80) | 0x6400 is the
