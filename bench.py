@@ -49,6 +49,7 @@ def parse():
                     help="BASELINE config: 2 (default, the headline) | 3 shared prefix + COW + eviction | "
                          "4 int8/fp8 pages at 128k | 5 chunked MFMA prefill interleaved with decode")
     ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8", help="config 4 storage type")
+    ap.add_argument("--no-cascade", action="store_true", help="config 3: read the shared prefix once per branch")
     return ap.parse_args()
 
 

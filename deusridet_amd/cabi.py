@@ -75,6 +75,9 @@ SIGNATURES = {
     "drk_paged_decode_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
     "drk_paged_decode_attention_branches": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32,
                                                    _f32, _i32, _i32, _vp, _sz, _vp]),
+    "drk_decode_shared_workspace_bytes": (_sz, [_LP, _i32, _i32, _i32]),
+    "drk_paged_decode_attention_shared": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _i32, _f32,
+                                                 _i32, _vp, _sz, _vp]),
     "drk_prefill_workspace_bytes": (_sz, [_LP, _i32, _i32]),
     "drk_paged_prefill_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
     "drk_importance_update": (_i32, [_vp, _vp, _i32, _f32, _vp]),

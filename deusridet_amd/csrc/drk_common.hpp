@@ -67,7 +67,14 @@ bool stream_decode_supported(const Lay &a, int B);
 size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens);
 int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
-                         float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st);
+                         float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
+                         int start_tile = 0, const float *pre_o = nullptr, const float *pre_m = nullptr,
+                         const float *pre_l = nullptr, int pre_splits = 0);
+// shared-prefix pass on the matrix cores (drk_prefill.hip)
+void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
+int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
+                         const int32_t *d_seq_lens, int B, int shared, int layer, float scale, float *part_o,
+                         float *part_m, float *part_l, hipStream_t st);
 
 // ---- element helpers (device) -------------------------------------------
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }

@@ -572,6 +572,67 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     return DRK_OK;
 }
 
+// Shared-prefix decode: tokens [0, shared) live in the same physical pages for all
+// B branches, so their K/V are streamed once for all B*QH query rows (matrix-core
+// pass), the private tails go through the stream kernel, one merge folds both.
+static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size_t *stream_part)
+{
+    int ct, ns;
+    shared_prefix_shape(shared, &ct, &ns);
+    size_t sp = stream_workspace_need(a, B, max_seq_len, 0);
+    sp = (sp + 255) & ~(size_t)255;
+    if (stream_part) *stream_part = sp;
+    return sp + (size_t)B * a.QH * ns * (a.D + 2) * sizeof(float);
+}
+
+static bool shared_path_ok(const Lay &a, int B, int shared)
+{
+    return !g_force_portable && stream_decode_supported(a, B) && a.E == 2 && shared >= kTile;
+}
+
+int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
+                         int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, int shared_tokens,
+                         void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
+                         void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
+    if (!shared_path_ok(a, B, shared) || shared > max_seq_len)
+        return launch_decode(g, q, pool, tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
+                             io_dtype, 0, workspace, workspace_bytes, stream);
+    if (!q || !pool || !tables || !out || !d_seq_lens) return fail(DRK_ERR_INVALID, "decode: NULL pointer");
+    if (io_dtype != a.dtype) return fail(DRK_ERR_INVALID, "decode: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
+    if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "decode: layer %d outside [0,%d)", layer, a.L);
+    size_t sp;
+    const size_t need = shared_need(a, B, max_seq_len, shared, &sp);
+    if (!workspace || workspace_bytes < need)
+        return fail(DRK_ERR_WORKSPACE, "decode: workspace of %zu bytes, need %zu", workspace_bytes, need);
+    if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode: workspace must be 16-byte aligned");
+    int ct, ns;
+    shared_prefix_shape(shared, &ct, &ns);
+    float *pre_o = (float *)((uint8_t *)workspace + sp);
+    float *pre_m = pre_o + (size_t)B * a.QH * ns * a.D;
+    float *pre_l = pre_m + (size_t)B * a.QH * ns;
+    hipStream_t st = (hipStream_t)stream;
+    const bool timed = g_time_kernel && g_ev_count < kMaxTimed;
+    if (timed) {
+        if (!g_ev_made) {
+            for (int i = 0; i < 2 * kMaxTimed; i++) DRK_HIP(hipEventCreate(&g_ev[i]));
+            g_ev_made = true;
+        }
+        DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count], st));
+    }
+    // branch 0's table addresses the shared pages (identical in every row by the caller's promise)
+    if ((rc = launch_shared_prefix(a, q, pool, tables, d_seq_lens, B, shared, layer, scale, pre_o, pre_m, pre_l, st))) return rc;
+    if ((rc = launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
+                                   io_dtype, 0, workspace, false, st, shared / kTile))) return rc;
+    if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
+    return launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
+                                io_dtype, 0, workspace, true, st, shared / kTile, pre_o, pre_m, pre_l, ns);
+}
+
 } // namespace drk
 
 using namespace drk;
@@ -639,6 +700,31 @@ int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void
     if (seq_len < 0) return fail(DRK_ERR_INVALID, "decode: negative seq_len");
     return launch_decode(g, q, pool, d_block_table, 0, nullptr, seq_len, -1, 1, seq_len, out, layer, scale, io_dtype,
                          0, workspace, workspace_bytes, stream);
+}
+
+size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len, int shared_tokens)
+{
+    Lay a;
+    if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0) return 0;
+    size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);
+    const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
+    if (stream_decode_supported(a, B) && a.E == 2 && shared >= kTile) {
+        size_t s2 = shared_need(a, B, max_seq_len, shared, nullptr);
+        if (s2 > need) need = s2;
+    }
+    return need;
+}
+
+int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, const void *pool,
+                                      const int32_t *d_tables, int table_stride, const int32_t *d_seq_lens, int B,
+                                      int max_seq_len, int shared_tokens, void *out, int layer, float scale,
+                                      int io_dtype, void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!d_seq_lens) return fail(DRK_ERR_INVALID, "decode: d_seq_lens is NULL");
+    if (B < 0 || max_seq_len < 0 || table_stride < 0 || shared_tokens < 0) return fail(DRK_ERR_INVALID, "decode: negative size");
+    if (B == 0 || max_seq_len == 0) return DRK_OK;
+    return launch_decode_shared(g, q, pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, shared_tokens, out,
+                                layer, scale, io_dtype, workspace, workspace_bytes, stream);
 }
 
 int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, const void *pool,

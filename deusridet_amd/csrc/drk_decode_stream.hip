@@ -141,6 +141,7 @@ struct StreamArgs {
     int table_stride, seq_len_host, B, KVH, QH, NB, bs, bs_shift, io_dtype;
     int unit_tiles;                 // tiles per workgroup, or 0: ceil(total / gridDim.x)
     int Pmax;                       // partial slots per (branch, q head)
+    int start_tile;                 // tiles [0, start_tile) of every branch are handled elsewhere (shared prefix)
     unsigned head_stride, kv_plane, block_stride, scale_plane, row_bytes;
     float scale_log2e;
 };
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
     // ---- the workgroup's run of units and one descriptor per unit ---------------------
     const int len_i = lane < A.B ? (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host) : 0;
-    const int nt_i = len_i > 0 ? (len_i + kSTile - 1) / kSTile : 0;
+    const int nt_i = len_i > 0 ? max((len_i + kSTile - 1) / kSTile - A.start_tile, 0) : 0;
     int incl = nt_i;                                           // inclusive prefix of tiles over branches
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -329,7 +330,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         }
         const int b = lo;
         const int excl = b ? s_incl[b - 1] : 0, nt = s_incl[b] - excl, len = s_len[b];
-        const int rem = u - A.KVH * excl, kvh = rem / nt, tile = rem - kvh * nt;
+        const int rem = u - A.KVH * excl, kvh = rem / nt, trel = rem - kvh * nt;
+        const int tile = trel + A.start_tile;                  // absolute tile of the branch
         const int tg = tile * kSTile + grp * 16;
         uint2 gd = make_uint2(kNone, 0u);
         if (tg < len) {
@@ -346,7 +348,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         if (grp == 0) {
             UnitDesc d;
             d.tile_lim = len - tile * kSTile;
-            d.flags = ((ui == 0 || tile == 0) ? 1 : 0) | ((ui == nunits - 1 || tile + 1 == nt) ? 2 : 0);
+            d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0);
             d.bq = b * A.QH + kvh * 4;
             d.piece = (int)blockIdx.x - (A.KVH * excl + kvh * nt) / U;
             udesc[ui] = d;
@@ -528,39 +530,54 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
 }
 
-// grid (QH, B), block 128: fold the pieces of (branch, q head); out is written only
-// when some token took part (paged_attention.cu:266)
+// grid (QH, B), block 128: fold the pieces of (branch, q head) -- the stream kernel's
+// and, in shared-prefix mode, the prefix pass's; out is written only when some
+// token took part (paged_attention.cu:266)
 __global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_m,
                                                            const float *__restrict__ part_l, uint16_t *__restrict__ out,
                                                            const int32_t *__restrict__ seq_lens, int seq_len_host, int B,
                                                            int KVH, int QH, int unit_tiles, int grid_wgs, int Pmax,
-                                                           int io_dtype)
+                                                           int io_dtype, int start_tile, const float *__restrict__ pre_o,
+                                                           const float *__restrict__ pre_m, const float *__restrict__ pre_l,
+                                                           int pre_splits)
 {
     const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
     int excl = 0, total = 0, nt_b = 0;
     for (int i = 0; i < B; i++) {
         const int len = seq_lens ? seq_lens[i] : seq_len_host;
-        const int nt = len > 0 ? (len + kSTile - 1) / kSTile : 0;
+        const int nt = len > 0 ? max((len + kSTile - 1) / kSTile - start_tile, 0) : 0;
         if (i < b) excl += nt;
         if (i == b) nt_b = nt;
         total += nt;
     }
-    if (nt_b == 0) return;
-    const int T = total * KVH;
-    const int U = unit_tiles > 0 ? unit_tiles : (T + grid_wgs - 1) / grid_wgs;
-    const int kvh = h / (QH / KVH);
-    const int first = KVH * excl + kvh * nt_b, last = first + nt_b - 1;
-    const int npieces = last / U - first / U + 1;
+    int npieces = 0;
+    if (nt_b > 0) {
+        const int T = total * KVH;
+        const int U = unit_tiles > 0 ? unit_tiles : (T + grid_wgs - 1) / grid_wgs;
+        const int kvh = h / (QH / KVH);
+        const int first = KVH * excl + kvh * nt_b, last = first + nt_b - 1;
+        npieces = last / U - first / U + 1;
+    }
     const size_t base = ((size_t)b * QH + h) * Pmax;
+    const size_t pbase = ((size_t)b * QH + h) * pre_splits;
     float M = -INFINITY;
     for (int s = 0; s < npieces; s++)
         if (part_l[base + s] > 0.0f) M = fmaxf(M, part_m[base + s]);
+    for (int s = 0; s < pre_splits; s++)
+        if (pre_l[pbase + s] > 0.0f) M = fmaxf(M, pre_m[pbase + s]);
     float acc = 0.0f, L = 0.0f;
     for (int s = 0; s < npieces; s++) {
         const float pl = part_l[base + s];
         if (!(pl > 0.0f)) continue;
         const float wgt = s_exp2(part_m[base + s] - M);
         acc = fmaf(part_o[(base + s) * 128 + d], wgt, acc);
+        L = fmaf(pl, wgt, L);
+    }
+    for (int s = 0; s < pre_splits; s++) {
+        const float pl = pre_l[pbase + s];
+        if (!(pl > 0.0f)) continue;
+        const float wgt = s_exp2(pre_m[pbase + s] - M);
+        acc = fmaf(pre_o[(pbase + s) * 128 + d], wgt, acc);
         L = fmaf(pl, wgt, L);
     }
     if (L > 0.0f) out[((size_t)b * QH + h) * 128 + d] = f_to_elem16(acc / L, io_dtype);
@@ -600,7 +617,8 @@ size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tok
 // launches the partial kernel; *merge_fn_args are filled for the caller to launch the merge
 int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
-                         float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st)
+                         float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
+                         int start_tile, const float *pre_o, const float *pre_m, const float *pre_l, int pre_splits)
 {
     int grid, U, Pmax;
     stream_shape(a, B, max_seq_len, split_tokens, &grid, &U, &Pmax);
@@ -614,7 +632,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
         A.table_stride = table_stride; A.seq_len_host = seq_len_host; A.B = B; A.KVH = a.KVH; A.QH = a.QH;
         A.NB = a.NB; A.bs = a.bs; A.bs_shift = ilog2_exact((unsigned)a.bs); A.io_dtype = io_dtype;
-        A.unit_tiles = U; A.Pmax = Pmax;
+        A.unit_tiles = U; A.Pmax = Pmax; A.start_tile = start_tile;
         A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
         A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
         A.scale_log2e = scale * kSLog2e;
@@ -627,7 +645,8 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         DRK_LAUNCH_CHECK("decode_stream_kernel");
     } else {
         hipLaunchKernelGGL(stream_merge_kernel, dim3(a.QH, B), dim3(128), 0, st, part_o, part_m, part_l, (uint16_t *)out,
-                           d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype);
+                           d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
+                           pre_l, pre_splits);
         DRK_LAUNCH_CHECK("stream_merge_kernel");
     }
     return DRK_OK;

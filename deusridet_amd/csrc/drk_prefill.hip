@@ -88,6 +88,10 @@ struct PrefillArgs {
     int pos_start, M, QH, NB, bs, bs_shift;
     unsigned head_stride, kv_plane, block_stride;
     float scale_log2e;
+    // shared-prefix mode: row "token" = branch; every row sees tokens [0, min(len, shared))
+    const int32_t *seq_lens;      // [M] on the device
+    int shared, chunk_tiles, nsplits;
+    float *part_o, *part_m, *part_l;
 };
 
 struct PfGroup {
@@ -117,8 +121,12 @@ __device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, i
     *(uint4 *)(dst + 12 * kPfPitch) = g.r3;
 }
 
-// grid = (ceil(M/32), KVH); block = 256
-template <int DT>
+// grid = (ceil(M/32), KVH[, splits]); block = 256.
+// SHARED = false: causal prefill of a chunk, normalised output.
+// SHARED = true:  the M rows are decode branches that share the pages of tokens
+//                 [0, shared); workgroup z handles tokens [z, z+1) * chunk_tiles * 64 of
+//                 them, no causal mask, and leaves (o, m, l) per (branch, q head, z).
+template <int DT, bool SHARED>
 __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
 {
     __shared__ __align__(16) uint8_t k_lds[kPfBN * kPfPitch];
@@ -134,10 +142,18 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
     const int tq = qt * 32 + w * 8 + (n >> 2);
     const int head = kvh * 4 + (n & 3);
     const bool row_live = tq < A.M;
-    const int vis = A.pos_start + tq + 1;                       // tokens [0, vis) are visible to the row
-    const int lim_wg = A.pos_start + min((qt + 1) * 32, A.M);   // exclusive limit over the workgroup
+    int vis, lim_wg, t_begin = 0, first_masked_tile = 0;
+    if (SHARED) {
+        const int len = row_live ? A.seq_lens[tq] : 0;
+        vis = min(len, A.shared);                               // tokens [0, vis) are visible to the row
+        t_begin = (int)blockIdx.z * A.chunk_tiles;
+        lim_wg = min(A.shared, (t_begin + A.chunk_tiles) * kPfBN);
+    } else {
+        vis = A.pos_start + tq + 1;
+        lim_wg = A.pos_start + min((qt + 1) * 32, A.M);         // exclusive limit over the workgroup
+        first_masked_tile = (A.pos_start + qt * 32 + 1) / kPfBN;   // tiles below are fully visible
+    }
     const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
-    const int first_masked_tile = (A.pos_start + qt * 32 + 1) / kPfBN;   // tiles below are fully visible
 
     // Q as the B operand of S^T: 8 k-steps of 16 dims; lane holds dims ks*16 + g*8 .. +8
     uint4 qf[8];
@@ -167,11 +183,11 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
     float m_run = -INFINITY, l_run = 0.0f;
 
     bool cur_valid, nxt_valid = false;
-    size_t off = lookup(0, cur_valid);
+    size_t off = lookup(t_begin, cur_valid);
     PfGroup kreg = pf_load_group(kbase, cur_valid, off, lane);
     PfGroup vreg = pf_load_group(kbase + A.kv_plane, cur_valid, off, lane);
 
-    for (int it = 0; it < ntiles; it++) {
+    for (int it = t_begin; it < ntiles; it++) {
         const int tile_t = it * kPfBN;
         // ---- stage the tile; rows at or past the workgroup's limit may hold anything ----
         if (tile_t + kPfBN > lim_wg) {
@@ -210,7 +226,8 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
         // ---- tile softmax for this lane's row; register i of tile tt is token
         //      tile_t + tt*32 + 8*(i/4) + 4*g + i%4 ----
         const bool all_groups_valid = (valid_lds[0] & valid_lds[1] & valid_lds[2] & valid_lds[3]) != 0;
-        const bool need_mask = it >= first_masked_tile || !all_groups_valid;
+        const bool need_mask = !all_groups_valid ||
+                               (SHARED ? (__any(tile_t + kPfBN > vis) != 0) : (it >= first_masked_tile));
         float tmax = -INFINITY;
 #pragma unroll
         for (int tt = 0; tt < 2; tt++)
@@ -273,9 +290,24 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
         __syncthreads();
     }
 
-    // ---- normalise and write: register i of tile dt is d = dt*32 + 8*(i/4) + 4*g + i%4 ----
+    // ---- register i of tile dt is d = dt*32 + 8*(i/4) + 4*g + i%4 ----
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if (row_live && l_tot > 0.0f) {
+    if (SHARED) {
+        if (row_live) {                      // unnormalised partial; an empty range leaves (0, -inf, 0)
+            const size_t pi = ((size_t)tq * A.QH + head) * A.nsplits + blockIdx.z;
+            float *orow = A.part_o + pi * 128;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int b4 = 0; b4 < 4; b4++)
+                    *(float4 *)(orow + dt * 32 + 8 * b4 + 4 * g) =
+                        make_float4(o[dt][4 * b4], o[dt][4 * b4 + 1], o[dt][4 * b4 + 2], o[dt][4 * b4 + 3]);
+            if (g == 0) {
+                A.part_m[pi] = m_run;
+                A.part_l[pi] = l_tot;
+            }
+        }
+    } else if (row_live && l_tot > 0.0f) {
         const float inv = 1.0f / l_tot;
         uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * 256;
 #pragma unroll
@@ -288,6 +320,43 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
                 *(uint2 *)(orow + d0 * 2) = v;
             }
     }
+}
+
+// ---- shared-prefix ("cascade") decode: host side of the prefix pass -------------------
+// One launch covers tokens [0, shared) for all B branches; the private tails go
+// through the stream kernel with start_tile = shared / 64.
+void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits)
+{
+    const int tiles = shared / kPfBN;
+    int ns = tiles < 32 ? tiles : 32;                     // 8 kv heads x 32 splits = one workgroup per CU
+    if (ns < 1) ns = 1;
+    *chunk_tiles = (tiles + ns - 1) / ns;
+    if (*chunk_tiles < 1) *chunk_tiles = 1;
+    *nsplits = (tiles + *chunk_tiles - 1) / *chunk_tiles;
+    if (*nsplits < 1) *nsplits = 1;
+}
+
+int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
+                         const int32_t *d_seq_lens, int B, int shared, int layer, float scale, float *part_o,
+                         float *part_m, float *part_l, hipStream_t st)
+{
+    PrefillArgs A;
+    A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
+    A.table = table0;
+    A.q = (const uint8_t *)q;
+    A.out = nullptr;
+    A.pos_start = 0; A.M = B; A.QH = a.QH; A.NB = a.NB; A.bs = a.bs;
+    A.bs_shift = ilog2_exact((unsigned)a.bs);
+    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
+    A.scale_log2e = scale * kLog2eP;
+    A.seq_lens = d_seq_lens; A.shared = shared;
+    shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
+    A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
+    dim3 grid((B + 31) / 32, a.KVH, A.nsplits);
+    if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, true>), grid, dim3(256), 0, st, A);
+    else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, true>), grid, dim3(256), 0, st, A);
+    DRK_LAUNCH_CHECK("prefill_mfma_kernel<shared>");
+    return DRK_OK;
 }
 
 } // namespace drk
@@ -341,8 +410,9 @@ int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const voi
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
     A.scale_log2e = scale * kLog2eP;
     dim3 grid((M + 31) / 32, a.KVH);
-    if (a.dtype == DRK_BF16) hipLaunchKernelGGL(prefill_mfma_kernel<DRK_BF16>, grid, dim3(256), 0, (hipStream_t)stream, A);
-    else hipLaunchKernelGGL(prefill_mfma_kernel<DRK_F16>, grid, dim3(256), 0, (hipStream_t)stream, A);
+    A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
+    if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
+    else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
     DRK_LAUNCH_CHECK("prefill_mfma_kernel");
     return DRK_OK;
 }

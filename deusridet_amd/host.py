@@ -34,7 +34,8 @@ SIGNATURES = {
     "drkh_cm_seq_len": (_i32, [_vp, _i32]), "drkh_cm_set_seq_len": (None, [_vp, _i32, _i32]),
     "drkh_cm_num_logical_blocks": (_i32, [_vp, _i32]),
     "drkh_cm_fork_branch": (_i32, [_vp, _i32, _i32]), "drkh_cm_release_branch": (None, [_vp, _i32]),
-    "drkh_cm_touch_block": (None, [_vp, _i32, _i32]), "drkh_cm_block_location": (_i32, [_vp, _i32, _i32]),
+    "drkh_cm_touch_block": (None, [_vp, _i32, _i32]),
+    "drkh_cm_common_prefix_tokens": (_i32, [_vp, _vp, _i32]), "drkh_cm_block_location": (_i32, [_vp, _i32, _i32]),
     "drkh_cm_evict_blocks": (_i32, [_vp, _i32]), "drkh_cm_ensure_free_blocks": (_i32, [_vp, _i32]),
     "drkh_cm_gpu_blocks_used": (_i32, [_vp]), "drkh_cm_free_blocks": (_i32, [_vp]),
     "drkh_cm_lru_snapshot": (_i32, [_vp, _vp, _vp, _i32]),
@@ -51,6 +52,8 @@ SIGNATURES = {
     "drkh_paged_gqa_decode_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_paged_gqa_decode_attention_branches": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _i32,
                                                         _i32, _f32, _vp]),
+    "drkh_paged_gqa_decode_attention_shared": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _i32, _i32, _i32,
+                                                      _f32, _vp]),
     "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32]),
     "drkh_invoke_extract_kv_from_pages": (None, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
@@ -140,6 +143,11 @@ class CacheManager:
     def fork_branch(self, parent, pos): return lib().drkh_cm_fork_branch(self._h, parent, pos)
     def release_branch(self, branch): lib().drkh_cm_release_branch(self._h, branch)
     def touch_block(self, branch, logical): lib().drkh_cm_touch_block(self._h, branch, logical)
+
+    def common_prefix_tokens(self, branches):
+        a = np.ascontiguousarray(branches, dtype=np.int32)
+        return lib().drkh_cm_common_prefix_tokens(self._h, _p(a), a.shape[0])
+
     def block_location(self, branch, logical): return lib().drkh_cm_block_location(self._h, branch, logical)
     def evict_blocks(self, n): return lib().drkh_cm_evict_blocks(self._h, n)
     def ensure_free_blocks(self, n): return bool(lib().drkh_cm_ensure_free_blocks(self._h, n))

@@ -112,6 +112,22 @@ void paged_gqa_decode_attention_branches(const __half* Q, __half* kv_pool, const
         LOG_ERROR("Machina", "paged_gqa_decode_attention_branches: %s", drk_last_error());
 }
 
+void paged_gqa_decode_attention_shared(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                       const int* d_seq_lens, int B, int max_seq_len, int shared_tokens,
+                                       __half* out, int fa_layer_idx, int max_phys_blocks, int block_size,
+                                       float scale, hipStream_t stream)
+{
+    if (B <= 0 || max_seq_len <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    size_t need = drk_decode_shared_workspace_bytes(&g, B, max_seq_len, shared_tokens);
+    void* ws = workspace(need);
+    if (!ws) return;
+    if (drk_paged_decode_attention_shared(&g, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len,
+                                          shared_tokens, out, fa_layer_idx, scale, ModelConfig::IO_DTYPE, ws,
+                                          g_ws_bytes, stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_gqa_decode_attention_shared: %s", drk_last_error());
+}
+
 void paged_prefill_attention(const __half* Q, __half* kv_pool, const int* d_block_table, __half* out,
                              int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
                              float scale, hipStream_t stream)

@@ -56,6 +56,14 @@ void paged_gqa_decode_attention_branches(const __half* Q, __half* kv_pool, const
                                          int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
                                          hipStream_t stream = 0);
 
+// Same, for branches whose first shared_tokens tokens live in the same physical
+// pages (CacheManager::common_prefix_tokens): those pages are read from HBM once
+// for all branches.
+void paged_gqa_decode_attention_shared(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                       const int* d_seq_lens, int B, int max_seq_len, int shared_tokens,
+                                       __half* out, int fa_layer_idx, int max_phys_blocks, int block_size,
+                                       float scale, hipStream_t stream = 0);
+
 // The attention calls keep split-K partials in a device workspace that this
 // library owns and grows on demand (device allocation = implicit sync).  Call
 // this once up front with the largest shapes to keep the steady state free of

@@ -337,6 +337,28 @@ void CacheManager::release_branch(int branch)
     if (branch != 0) alive_[branch] = 0;
 }
 
+int CacheManager::common_prefix_tokens(const int* branches, int n) const
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (!branches || n <= 0) return 0;
+    int min_len = 0x7fffffff;
+    for (int i = 0; i < n; i++) {
+        int b = branches[i];
+        if (b < 0 || b >= max_branches_ || !alive_[b]) return 0;
+        min_len = std::min(min_len, seq_len_[b]);
+    }
+    int limit = std::min(min_len / block_size_, max_logical_blocks_);
+    int blocks = 0;
+    for (; blocks < limit; blocks++) {
+        int phys = h_tables_[cell(branches[0], blocks)];
+        if (phys < 0) break;
+        bool same = true;
+        for (int i = 1; i < n && same; i++) same = h_tables_[cell(branches[i], blocks)] == phys;
+        if (!same) break;
+    }
+    return blocks * block_size_;
+}
+
 bool CacheManager::branch_alive(int branch) const
 {
     std::lock_guard<std::mutex> lock(mu_);

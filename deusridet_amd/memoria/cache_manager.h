@@ -89,6 +89,10 @@ public:
     void release_branch(int branch);
     bool branch_alive(int branch) const;
     int  max_branches() const { return max_branches_; }
+    // Tokens [0, n) whose pages are the same physical blocks in every listed branch
+    // (whole blocks only, capped by the shortest seq_len): what
+    // paged_gqa_decode_attention_shared() may stream once for all of them.
+    int  common_prefix_tokens(const int* branches, int n) const;
     // Recency update: move the entry to the back of the LRU order.
     void touch_block(int branch, int logical_idx);
     int  refcount(int phys_block) const { return pool_.refcount(phys_block); }

@@ -50,6 +50,7 @@ int   drkh_cm_num_logical_blocks(void *cm, int branch);
 int   drkh_cm_fork_branch(void *cm, int parent, int pos);
 void  drkh_cm_release_branch(void *cm, int branch);
 void  drkh_cm_touch_block(void *cm, int branch, int logical);
+int   drkh_cm_common_prefix_tokens(void *cm, const int32_t *branches, int n);
 int   drkh_cm_block_location(void *cm, int branch, int logical);
 int   drkh_cm_evict_blocks(void *cm, int n);
 int   drkh_cm_ensure_free_blocks(void *cm, int n_free);
@@ -87,6 +88,10 @@ void drkh_paged_gqa_decode_attention_branches(const void *Q, void *kv_pool, cons
                                               int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len,
                                               void *out, int fa_layer_idx, int max_phys_blocks, int block_size,
                                               float scale, void *stream);
+void drkh_paged_gqa_decode_attention_shared(const void *Q, void *kv_pool, const int32_t *d_tables, int table_stride,
+                                            const int32_t *d_seq_lens, int B, int max_seq_len, int shared_tokens,
+                                            void *out, int fa_layer_idx, int max_phys_blocks, int block_size,
+                                            float scale, void *stream);
 void drkh_paged_prefill_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
                                   int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
                                   float scale, void *stream);

@@ -188,6 +188,24 @@ int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, c
                                         int split_tokens, void *workspace,
                                         size_t workspace_bytes, void *stream);
 
+/* Branches that share a prefix (no reference counterpart; intent
+ * docs/en/architecture/03-cogitatio.md:3-5, 18-22: decode branches over one
+ * persistent Conscientia prefix).  The caller promises that the pages holding
+ * tokens [0, shared_tokens) are the same physical blocks in all B table rows and
+ * that every d_seq_lens[b] >= shared_tokens (CacheManager::common_prefix_tokens
+ * computes it).  Those pages are then streamed from HBM once for all B branches
+ * instead of once per branch.  shared_tokens is rounded down to a multiple of 64;
+ * 0, or a geometry / storage type the shared pass does not take, gives exactly
+ * drk_paged_decode_attention_branches.  Results equal the per-branch call up to
+ * summation order. */
+size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len, int shared_tokens);
+int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, const void *pool,
+                                      const int32_t *d_tables, int table_stride,
+                                      const int32_t *d_seq_lens, int B, int max_seq_len,
+                                      int shared_tokens, void *out, int layer, float scale,
+                                      int io_dtype, void *workspace, size_t workspace_bytes,
+                                      void *stream);
+
 /* ---- paged causal prefill attention ------------------------------------ */
 /* paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630:
  * q/out [M, num_q_heads, head_dim]; row t attends to tokens 0..pos_start+t (the

@@ -287,3 +287,61 @@ def test_workspace_too_small_is_refused(dev):
     rc = cabi.lib().drk_paged_decode_attention(C.byref(case.g), U.p(case.dq), U.p(case.dpool), U.p(case.dtab[0]),
                                                U.p(out), 0, 100, 0.1, cabi.F16, U.p(ws), 64, None)
     assert rc == cabi.ERR_WORKSPACE
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
+@pytest.mark.parametrize("shared,extra", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17]), (960 + 16, [5, 300]),
+                                          (64, [0]), (4096, list(range(0, 400, 10)))])
+def test_shared_prefix_decode(dev, dtype, shared, extra):
+    """Branches whose leading pages are the same physical blocks (BASELINE config 3
+    in small): the shared pass + private tails must agree with the fp64 oracle run
+    per branch, and with the plain per-branch call."""
+    L, KVH, QH, D, bs = 1, 8, 32, 128, 16
+    B = len(extra)
+    lens = np.array([shared + e for e in extra], dtype=np.int32)
+    n_shared_blk = shared // bs
+    priv_blk = [(int(l) + bs - 1) // bs - n_shared_blk for l in lens]
+    NB = n_shared_blk + sum(priv_blk) + 8
+    g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
+    rng = np.random.default_rng(shared + B)
+    perm = rng.permutation(NB).astype(np.int32)
+    stride = n_shared_blk + max(priv_blk) + 2
+    tables = np.full((B, stride), -1, dtype=np.int32)
+    o = n_shared_blk
+    for b in range(B):
+        tables[b, :n_shared_blk] = perm[:n_shared_blk]
+        tables[b, n_shared_blk:n_shared_blk + priv_blk[b]] = perm[o:o + priv_blk[b]]
+        o += priv_blk[b]
+    opool = orc.new_pool(og)
+    k = U.normal_bits(rng, (shared, KVH, D), dtype, 0.7)
+    v = U.normal_bits(rng, (shared, KVH, D), dtype, 0.7)
+    orc.append_batch(og, opool, tables[0], 0, 0, k, v, dtype)
+    for b in range(B):
+        n = int(lens[b]) - n_shared_blk * bs
+        if n > 0:
+            # a branch's private part starts at the first non-shared block boundary
+            kk = U.normal_bits(rng, (n, KVH, D), dtype, 0.7)
+            vv = U.normal_bits(rng, (n, KVH, D), dtype, 0.7)
+            orc.append_batch(og, opool, tables[b], 0, n_shared_blk * bs, kk, vv, dtype)
+    q = U.normal_bits(rng, (B, QH, D), dtype, 0.7)
+    scale = 1 / np.sqrt(D)
+    dq, dpool, dtab, dl = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(tables), U.dev_i32(lens)
+    lib = cabi.lib()
+    mx = int(lens.max())
+    shared_arg = n_shared_blk * bs
+    wsb = lib.drk_decode_shared_workspace_bytes(C.byref(g), B, mx, shared_arg)
+    ws = U.dev_zeros(wsb)
+    out = U.dev_bytes(np.full(B * QH * D * 2, 0x7B, dtype=np.uint8))
+    cabi.call("drk_paged_decode_attention_shared", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dl), B, mx,
+              shared_arg, U.p(out), 0, float(scale), dtype, U.p(ws), wsb, U.stream_ptr())
+    out2 = U.dev_zeros(B * QH * D * 2)
+    cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dl), B, mx,
+              U.p(out2), 0, float(scale), dtype, 0, U.p(ws), wsb, U.stream_ptr())
+    U.sync()
+    got = U.from_bits(U.host(out, np.uint16, (B, QH, D)), dtype)
+    plain = U.from_bits(U.host(out2, np.uint16, (B, QH, D)), dtype)
+    want = np.stack([orc.decode_f64(og, q[b], opool, tables[b], 0, int(lens[b]), scale, dtype) for b in range(B)])
+    ok, ma, _ = U.rel_abs_ok(got, want, REL, ABS)
+    assert ok, ma
+    ok, ma, _ = U.rel_abs_ok(got, plain, REL, ABS)
+    assert ok, ma
