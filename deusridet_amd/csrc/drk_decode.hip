@@ -587,7 +587,7 @@ static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size
 
 static bool shared_path_ok(const Lay &a, int B, int shared)
 {
-    return !g_force_portable && stream_decode_supported(a, B) && a.E == 2 && shared >= kTile;
+    return !g_force_portable && stream_decode_supported(a, B) && a.E == 2 && shared >= kTile;   // the caller checks scale > 0
 }
 
 int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
@@ -599,7 +599,7 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
     int rc = make_lay(g, &a);
     if (rc) return rc;
     const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
-    if (!shared_path_ok(a, B, shared) || shared > max_seq_len)
+    if (!shared_path_ok(a, B, shared) || shared > max_seq_len || !(scale > 0.0f))
         return launch_decode(g, q, pool, tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
                              io_dtype, 0, workspace, workspace_bytes, stream);
     if (!q || !pool || !tables || !out || !d_seq_lens) return fail(DRK_ERR_INVALID, "decode: NULL pointer");

@@ -127,7 +127,7 @@ __device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, i
 //                 [0, shared); workgroup z handles tokens [z, z+1) * chunk_tiles * 64 of
 //                 them, no causal mask, and leaves (o, m, l) per (branch, q head, z).
 template <int DT, bool SHARED>
-__global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
+__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
 {
     __shared__ __align__(16) uint8_t k_lds[kPfBN * kPfPitch];
     __shared__ __align__(16) uint8_t v_lds[kPfBN * kPfPitch];
@@ -228,22 +228,23 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
         const bool all_groups_valid = (valid_lds[0] & valid_lds[1] & valid_lds[2] & valid_lds[3]) != 0;
         const bool need_mask = !all_groups_valid ||
                                (SHARED ? (__any(tile_t + kPfBN > vis) != 0) : (it >= first_masked_tile));
+        // raw scores stay in s; the scale (> 0) is folded into the exponent's fma
         float tmax = -INFINITY;
 #pragma unroll
         for (int tt = 0; tt < 2; tt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                float v = s[tt][i] * A.scale_log2e;
+                float v = s[tt][i];
                 if (need_mask) {
                     const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
                     const bool ok = (tile_t + tl) < vis && valid_lds[tl >> 4] != 0;
                     v = ok ? v : -INFINITY;
+                    s[tt][i] = v;
                 }
-                s[tt][i] = v;
                 tmax = fmaxf(tmax, v);
             }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32));               // the row's other 32 tokens
-        const float m_new = fmaxf(m_run, tmax);
+        const float m_new = fmaxf(m_run, tmax * A.scale_log2e);
         const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
         float psum = 0.0f;
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(PrefillArgs A)
             float p[16];
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                p[i] = __builtin_amdgcn_exp2f(s[tt][i] - m_use);
+                p[i] = __builtin_amdgcn_exp2f(fmaf(s[tt][i], A.scale_log2e, -m_use));
                 psum += p[i];
             }
             pb[tt][0] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
@@ -395,7 +396,7 @@ int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const voi
         return fail(DRK_ERR_INVALID, "prefill: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
 
-    const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0;
+    const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && scale > 0.0f;
     if (!mfma)
         return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
                              io_dtype, 0, workspace, workspace_bytes, stream);
