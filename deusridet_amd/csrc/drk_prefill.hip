@@ -85,7 +85,7 @@ struct PrefillArgs {
     const int32_t *table;
     const uint8_t *q;
     uint8_t *out;
-    int pos_start, M, QH, NB, bs, bs_shift;
+    int pos_start, M, QH, KVH, NB, bs, bs_shift;
     unsigned head_stride, kv_plane, block_stride;
     float scale_log2e;
     // shared-prefix mode: row "token" = branch; every row sees tokens [0, min(len, shared))
@@ -121,7 +121,7 @@ __device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, i
     *(uint4 *)(dst + 12 * kPfPitch) = g.r3;
 }
 
-// grid = (ceil(M/32), KVH[, splits]); block = 256.
+// grid = (ceil(M/32) * KVH, 1[, splits]); block = 256.
 // SHARED = false: causal prefill of a chunk, normalised output.
 // SHARED = true:  the M rows are decode branches that share the pages of tokens
 //                 [0, shared); workgroup z handles tokens [z, z+1) * chunk_tiles * 64 of
@@ -133,7 +133,9 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
     __shared__ __align__(16) uint8_t v_lds[kPfBN * kPfPitch];
     __shared__ int valid_lds[4];
 
-    const int qt = blockIdx.x, kvh = blockIdx.y;
+    // Workgroups are dealt to the 8 XCDs round-robin by linear id; kv head = id % KVH
+    // keeps one kv head's pages in one XCD's L2 (8 kv heads on 8 XCDs).
+    const int kvh = (int)blockIdx.x % A.KVH, qt = (int)blockIdx.x / A.KVH;
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
@@ -346,14 +348,14 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.table = table0;
     A.q = (const uint8_t *)q;
     A.out = nullptr;
-    A.pos_start = 0; A.M = B; A.QH = a.QH; A.NB = a.NB; A.bs = a.bs;
+    A.pos_start = 0; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs;
     A.bs_shift = ilog2_exact((unsigned)a.bs);
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
     A.scale_log2e = scale * kLog2eP;
     A.seq_lens = d_seq_lens; A.shared = shared;
     shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
     A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
-    dim3 grid((B + 31) / 32, a.KVH, A.nsplits);
+    dim3 grid(((B + 31) / 32) * a.KVH, 1, A.nsplits);
     if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, true>), grid, dim3(256), 0, st, A);
     else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, true>), grid, dim3(256), 0, st, A);
     DRK_LAUNCH_CHECK("prefill_mfma_kernel<shared>");
@@ -406,11 +408,11 @@ int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const voi
     A.table = d_block_table;
     A.q = (const uint8_t *)q;
     A.out = (uint8_t *)out;
-    A.pos_start = pos_start; A.M = M; A.QH = a.QH; A.NB = a.NB; A.bs = a.bs;
+    A.pos_start = pos_start; A.M = M; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs;
     A.bs_shift = ilog2_exact((unsigned)a.bs);
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
     A.scale_log2e = scale * kLog2eP;
-    dim3 grid((M + 31) / 32, a.KVH);
+    dim3 grid(((M + 31) / 32) * a.KVH);
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
     else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
