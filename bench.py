@@ -213,6 +213,29 @@ def main():
         ab = 2 * (2 * L * m * KVH * D * 2)                                          # K,V read + written
         append_gbps = ab * reps / (a0.elapsed_time(a1) * 1e-3) / 1e9
 
+    # ---- bulk gather (extract) and scatter (inject) of the same tokens, all layers, read + write
+    gather_gbps = scatter_gbps = None
+    if scratch_tab is not None:
+        flat = torch.empty(L * 2 * m * KVH * D * 2, dtype=torch.uint8, device="cuda")
+        for name in ("drk_kv_extract", "drk_kv_inject"):
+            def go():
+                if name == "drk_kv_extract":
+                    cabi.call(name, C.byref(g), U.p(flat), None, U.p(pool), U.p(scratch_tab), 0, m, L, sp)
+                else:
+                    cabi.call(name, C.byref(g), U.p(pool), U.p(flat), None, U.p(scratch_tab), 0, m, L, sp)
+            for _ in range(3):
+                go()
+            a0.record(stream)
+            for _ in range(reps):
+                go()
+            a1.record(stream)
+            torch.cuda.synchronize()
+            gbps = 2 * flat.numel() * reps / (a0.elapsed_time(a1) * 1e-3) / 1e9
+            if name == "drk_kv_extract":
+                gather_gbps = gbps
+            else:
+                scatter_gbps = gbps
+
     # ---- CPU baseline: the oracle's restatement of the reference loop, OpenMP ----
     cpu = None
     if not args.no_cpu_baseline:
@@ -266,6 +289,8 @@ def main():
         "tokens_per_s": round(tokens_per_s, 1),
         "bulk_append_GBps": None if append_gbps is None else round(append_gbps, 1),
         "bulk_append_hbm_frac": None if append_gbps is None else round(append_gbps / HBM_PEAK_GBPS, 4),
+        "bulk_gather_GBps": None if gather_gbps is None else round(gather_gbps, 1),
+        "bulk_scatter_GBps": None if scatter_gbps is None else round(scatter_gbps, 1),
         "hbm_read_probe_GBps": round(read_probe_gbps, 1),
         "fill_seconds": round(t_fill, 2),
         "roofline": {

@@ -1,0 +1,192 @@
+"""GPU: BASELINE's full sizes, checked through size-independent properties (the
+CPU oracle would take minutes here): round trips, equality of independent
+kernels, invariance under physical placement, closed-form attention results."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from deusridet_amd import cabi
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def test_config2_full_size_properties(dev):
+    """8 branches x 32k tokens, 32Q/8KV x128 bf16, pages shuffled over a 16 954-block
+    pool (one layer of it resident here: the layer stride is the full 1.1 GB)."""
+    torch = _torch()
+    L, KVH, QH, D, bs, B, ctx = 2, 8, 32, 128, 16, 8, 32768
+    NB = 16954
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    lib = cabi.lib()
+    rng = np.random.default_rng(2)
+    perm = rng.permutation(NB).astype(np.int32)
+    nblk = ctx // bs
+    tables = np.stack([perm[b * nblk:(b + 1) * nblk] for b in range(B)])
+    pool = torch.zeros(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    dtab = torch.from_numpy(tables).cuda()
+    sp = U.stream_ptr()
+    layer = 1
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    srcs = []
+    for b in range(B):
+        k = (torch.randn(ctx, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        v = (torch.randn(ctx, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(dtab[b].data_ptr()), layer, 1, 0, ctx,
+                  U.p(k), U.p(v), cabi.BF16, sp)
+        srcs.append((k, v))
+    # 1. append then gather returns the source bit for bit (every branch, every token)
+    flat = torch.empty(2 * 2 * ctx * KVH * D * 2, dtype=torch.uint8, device="cuda")
+    for b in range(B):
+        cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(pool), C.c_void_p(dtab[b].data_ptr()), 0, ctx, 2, sp)
+        f = flat.view(torch.bfloat16).view(2, 2, ctx, KVH, D)
+        assert torch.equal(f[1, 0], srcs[b][0]) and torch.equal(f[1, 1], srcs[b][1])
+        assert not f[0].any()                                  # layer 0 was never written
+    # 2. three independent kernels agree on the attention output
+    q = (torch.randn(B, QH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+    lens = torch.full((B,), ctx, dtype=torch.int32, device="cuda")
+    scale = 1 / np.sqrt(D)
+    outs = {}
+    for name, portable, which, split in (("stream", 0, 0, 0), ("tiled", 0, 2, 1024), ("portable", 1, 0, 2048)):
+        lib.drk_debug_force_portable_decode(portable)
+        lib.drk_debug_set_decode_kernel(which)
+        wsb = max(lib.drk_decode_workspace_bytes(C.byref(g), B, ctx),
+                  lib.drk_decode_workspace_bytes_for_split(C.byref(g), B, ctx, split) if split else 0)
+        ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+        out = torch.zeros(B, QH, D, dtype=torch.bfloat16, device="cuda")
+        try:
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(q), U.p(pool), U.p(dtab), nblk, U.p(lens), B,
+                      ctx, U.p(out), layer, float(scale), cabi.BF16, split, U.p(ws), wsb, sp)
+            U.sync()
+        finally:
+            lib.drk_debug_force_portable_decode(0)
+            lib.drk_debug_set_decode_kernel(0)
+        outs[name] = out.float().cpu().numpy()
+    for name in ("tiled", "portable"):
+        ok, ma, _ = U.rel_abs_ok(outs[name], outs["stream"])
+        assert ok, (name, ma)
+    # 3. torch's own fp32 attention on the gathered K/V of two branches
+    for b in (0, B - 1):
+        k, v = srcs[b][0].float(), srcs[b][1].float()                     # [ctx, KVH, D]
+        qq = q[b].float().view(KVH, 4, D)
+        s = torch.einsum("hgd,thd->hgt", qq, k) * scale
+        want = torch.einsum("hgt,thd->hgd", torch.softmax(s, dim=-1), v).reshape(QH, D).cpu().numpy()
+        ok, ma, _ = U.rel_abs_ok(outs["stream"][b], want)
+        assert ok, (b, ma)
+    # 4. moving every page to another physical block changes no bit of the output
+    perm2 = np.roll(perm, 4321)
+    tables2 = np.stack([perm2[b * nblk:(b + 1) * nblk] for b in range(B)])
+    dtab2 = torch.from_numpy(tables2).cuda()
+    pool2 = torch.zeros_like(pool)
+    for b in range(B):
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool2), C.c_void_p(dtab2[b].data_ptr()), layer, 1, 0, ctx,
+                  U.p(srcs[b][0]), U.p(srcs[b][1]), cabi.BF16, sp)
+    wsb = lib.drk_decode_workspace_bytes(C.byref(g), B, ctx)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    o1 = torch.zeros(B, QH, D, dtype=torch.bfloat16, device="cuda")
+    o2 = torch.zeros_like(o1)
+    for pl, tb, oo in ((pool, dtab, o1), (pool2, dtab2, o2)):
+        cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(q), U.p(pl), U.p(tb), nblk, U.p(lens), B, ctx,
+                  U.p(oo), layer, float(scale), cabi.BF16, 0, U.p(ws), wsb, sp)
+    U.sync()
+    assert torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize("dtype,tdt", [(cabi.INT8, "int8"), (cabi.FP8_E4M3, "fp8")])
+def test_config4_full_length_quantised(dev, dtype, tdt):
+    """One branch of 131 072 tokens with 1 % x20 outliers, quantised on append;
+    attention must match torch fp32 attention on the DEQUANTISED pages, and the
+    stream kernel must match the portable one."""
+    torch = _torch()
+    L, KVH, QH, D, bs, ctx = 1, 8, 32, 128, 16, 131072
+    NB = ctx // bs + 4
+    g = cabi.layout(L, KVH, QH, D, bs, NB, dtype)
+    lib = cabi.lib()
+    rng = np.random.default_rng(4)
+    table = torch.from_numpy(rng.permutation(NB).astype(np.int32)).cuda()
+    pool = torch.zeros(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    sp = U.stream_ptr()
+    chunk = 16384
+    for p0 in range(0, ctx, chunk):
+        k = torch.randn(chunk, KVH, D, device="cuda", generator=gen)
+        k = torch.where(torch.rand(k.shape, device="cuda", generator=gen) < 0.01, k * 20, k).to(torch.bfloat16)
+        v = torch.randn(chunk, KVH, D, device="cuda", generator=gen)
+        v = torch.where(torch.rand(v.shape, device="cuda", generator=gen) < 0.01, v * 20, v).to(torch.bfloat16)
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(table), 0, 1, p0, chunk, U.p(k), U.p(v), cabi.BF16, sp)
+        U.sync()
+    # dequantise what is stored (gather codes and scales through the C ABI)
+    codes = torch.empty(2 * ctx * KVH * D, dtype=torch.uint8, device="cuda")
+    scales = torch.empty(2 * ctx * KVH, dtype=torch.float16, device="cuda") if dtype == cabi.INT8 else None
+    cabi.call("drk_kv_extract", C.byref(g), U.p(codes), U.p(scales), U.p(pool), U.p(table), 0, ctx, 1, sp)
+    U.sync()
+    if dtype == cabi.INT8:
+        deq = codes.view(torch.int8).view(2, ctx, KVH, D).float() * scales.view(2, ctx, KVH, 1).float()
+    else:
+        deq = codes.view(torch.float8_e4m3fn).view(2, ctx, KVH, D).float()
+    q = torch.randn(1, QH, D, device="cuda", generator=gen).to(torch.bfloat16)
+    scale = 1 / np.sqrt(D)
+    s = torch.einsum("hgd,thd->hgt", q[0].float().view(KVH, 4, D), deq[0]) * scale
+    want = torch.einsum("hgt,thd->hgd", torch.softmax(s, dim=-1), deq[1]).reshape(QH, D).cpu().numpy()
+    lens = torch.full((1,), ctx, dtype=torch.int32, device="cuda")
+    res = {}
+    for portable in (0, 1):
+        lib.drk_debug_force_portable_decode(portable)
+        try:
+            wsb = lib.drk_decode_workspace_bytes(C.byref(g), 1, ctx)
+            ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+            out = torch.zeros(1, QH, D, dtype=torch.bfloat16, device="cuda")
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(q), U.p(pool), U.p(table), NB, U.p(lens), 1,
+                      ctx, U.p(out), 0, float(scale), cabi.BF16, 0, U.p(ws), wsb, sp)
+            U.sync()
+        finally:
+            lib.drk_debug_force_portable_decode(0)
+        res[portable] = out[0].float().cpu().numpy()
+    for portable in (0, 1):
+        ok, ma, _ = U.rel_abs_ok(res[portable], want)
+        assert ok, (portable, ma)
+
+
+def test_config5_full_chunk_prefill_rows(dev):
+    """A 2 048-token chunk at position 30 720 (the last chunk of config 5): sampled
+    rows of the MFMA prefill must equal decode attention at that row's length."""
+    torch = _torch()
+    L, KVH, QH, D, bs = 1, 8, 32, 128, 16
+    total, M = 32768, 2048
+    pos_start = total - M
+    NB = total // bs
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    lib = cabi.lib()
+    rng = np.random.default_rng(5)
+    table = torch.from_numpy(rng.permutation(NB).astype(np.int32)).cuda()
+    pool = torch.zeros(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(13)
+    sp = U.stream_ptr()
+    for p0 in range(0, total, 8192):
+        k = torch.randn(8192, KVH, D, device="cuda", generator=gen).to(torch.bfloat16)
+        v = torch.randn(8192, KVH, D, device="cuda", generator=gen).to(torch.bfloat16)
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(table), 0, 1, p0, 8192, U.p(k), U.p(v), cabi.BF16, sp)
+        U.sync()
+    q = torch.randn(M, QH, D, device="cuda", generator=gen).to(torch.bfloat16)
+    out = torch.zeros_like(q)
+    scale = 1 / np.sqrt(D)
+    cabi.call("drk_paged_prefill_attention", C.byref(g), U.p(q), U.p(pool), U.p(table), U.p(out), 0, pos_start, M,
+              float(scale), cabi.BF16, None, 0, sp)
+    rows = [0, 1, 31, 32, 1000, 2047]
+    lens = torch.tensor([pos_start + t + 1 for t in rows], dtype=torch.int32, device="cuda")
+    tabs = table.repeat(len(rows), 1).contiguous()
+    qd = q[rows].contiguous()
+    od = torch.zeros_like(qd)
+    wsb = lib.drk_decode_workspace_bytes(C.byref(g), len(rows), total)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(qd), U.p(pool), U.p(tabs), NB, U.p(lens), len(rows),
+              total, U.p(od), 0, float(scale), cabi.BF16, 0, U.p(ws), wsb, sp)
+    U.sync()
+    ok, ma, _ = U.rel_abs_ok(out[rows].float().cpu().numpy(), od.float().cpu().numpy())
+    assert ok, ma
