@@ -49,6 +49,8 @@ def parse():
                     help="BASELINE config: 2 (default, the headline) | 3 shared prefix + COW + eviction | "
                          "4 int8/fp8 pages at 128k | 5 chunked MFMA prefill interleaved with decode")
     ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8", help="config 4 storage type")
+    ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "
+                                                            "replaying one captured HIP graph per step")
     ap.add_argument("--no-cascade", action="store_true", help="config 3: read the shared prefix once per branch")
     return ap.parse_args()
 
@@ -141,15 +143,53 @@ def main():
                       U.p(pool), U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
                       float(scale), cabi.BF16, split, U.p(ws), wsb, sp)
 
-    for s in range(W):
-        step(s)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for s in range(W, W + K):
-        step(s)
-    e1.record(stream)
-    torch.cuda.synchronize()
+    use_graph = not args.no_graph
+    if use_graph:
+        # one step captured once: positions / lengths live in device buffers that the
+        # graph itself advances, so a replay is the whole step with no host work
+        pos_cur, len_cur = pos_steps[0].clone(), len_steps[0].clone()
+
+        def graph_step():
+            dpos, dlen = C.c_void_p(pos_cur.data_ptr()), C.c_void_p(len_cur.data_ptr())
+            gsp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            for l in range(L):
+                cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), stride, dpos, B, l, 1,
+                          C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, gsp)
+                cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow),
+                          U.p(pool), U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
+                          float(scale), cabi.BF16, split, U.p(ws), wsb, gsp)
+            pos_cur.add_(1)
+            len_cur.add_(1)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        with torch.cuda.stream(side):
+            graph_step()                                   # step 0, eager, on the capture stream
+        stream.wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            graph_step()                                   # step 1 (captured; runs on first replay)
+        for s in range(1, W):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for s in range(W, W + K):
+            graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        assert int(pos_cur[0]) == int(start[0]) + W + K, "graph replays did not advance the positions"
+    else:
+        for s in range(W):
+            step(s)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for s in range(W, W + K):
+            step(s)
+        e1.record(stream)
+        torch.cuda.synchronize()
     total_ms = e0.elapsed_time(e1)
     ms_per_step = total_ms / K
 
@@ -282,7 +322,8 @@ def main():
             "workload": f"config 2: {L} layers, 32 Q / 8 KV heads x 128, bf16 KV, 16-token pages shuffled over a "
                         f"{args.pool_gb:g} GB pool ({NB} blocks), {B} branches, ctx {args.ctx_mode} "
                         f"{int(final.min())}..{int(final.max())}; step = per layer: append 1 token/branch + paged decode attention",
-            "branches": B, "layers": L, "ctx_final": [int(x) for x in final], "split_tokens": int(split),
+            "branches": B, "layers": L, "ctx_final": [int(x) for x in final],
+            "launch": "one captured HIP graph per step" if use_graph else "host launches",
         },
         "hbm_frac_step": round(value_gbps / HBM_PEAK_GBPS, 4),
         "us_per_step": round(ms_per_step * 1e3, 1),
