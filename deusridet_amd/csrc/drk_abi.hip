@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4 *__restrict
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     for (; i + 3 * stride < nvec; i += 4 * stride) {
-        uint4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], d = p[i + 3 * stride];
+        uint4 a = ld_stream128(p + i), b = ld_stream128(p + i + stride), c = ld_stream128(p + i + 2 * stride), d = ld_stream128(p + i + 3 * stride);
         acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
     }
     for (; i < nvec; i += stride) { uint4 a = p[i]; acc ^= a.x ^ a.y ^ a.z ^ a.w; }

@@ -107,10 +107,10 @@ __device__ __forceinline__ Group4 load_group(const uint8_t *__restrict__ base, b
     g.r0 = g.r1 = g.r2 = g.r3 = make_uint4(0, 0, 0, 0);
     if (valid) {
         const uint8_t *p = base + off + (size_t)lane * 16;
-        g.r0 = *(const uint4 *)(p);
-        g.r1 = *(const uint4 *)(p + 1024);
-        g.r2 = *(const uint4 *)(p + 2048);
-        g.r3 = *(const uint4 *)(p + 3072);
+        g.r0 = ld_stream128(p);
+        g.r1 = ld_stream128(p + 1024);
+        g.r2 = ld_stream128(p + 2048);
+        g.r3 = ld_stream128(p + 3072);
     }
     return g;
 }

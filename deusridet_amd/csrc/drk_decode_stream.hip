@@ -172,17 +172,17 @@ __device__ __forceinline__ KRegs<DT> load_k(const uint8_t *__restrict__ p, bool 
         k.r0 = k.r1 = z;
         if (valid) {
             p += (size_t)lane * 16;
-            k.r0 = *(const uint4 *)(p);
-            k.r1 = *(const uint4 *)(p + 1024);
+            k.r0 = ld_stream128(p);
+            k.r1 = ld_stream128(p + 1024);
         }
     } else {
         k.r0 = k.r1 = k.r2 = k.r3 = z;
         if (valid) {
             p += (size_t)lane * 16;
-            k.r0 = *(const uint4 *)(p);
-            k.r1 = *(const uint4 *)(p + 1024);
-            k.r2 = *(const uint4 *)(p + 2048);
-            k.r3 = *(const uint4 *)(p + 3072);
+            k.r0 = ld_stream128(p);
+            k.r1 = ld_stream128(p + 1024);
+            k.r2 = ld_stream128(p + 2048);
+            k.r3 = ld_stream128(p + 3072);
         }
     }
     return k;
@@ -197,20 +197,20 @@ __device__ __forceinline__ VRegs<DT> load_v(const uint8_t *__restrict__ p, bool 
         v.r0 = v.r1 = v.r2 = v.r3 = z;
         if (valid) {
             p += (size_t)lane * 8;
-            v.r0 = *(const uint2 *)(p);
-            v.r1 = *(const uint2 *)(p + 512);
-            v.r2 = *(const uint2 *)(p + 1024);
-            v.r3 = *(const uint2 *)(p + 1536);
+            v.r0 = ld_stream64(p);
+            v.r1 = ld_stream64(p + 512);
+            v.r2 = ld_stream64(p + 1024);
+            v.r3 = ld_stream64(p + 1536);
         }
     } else {
         const uint4 z = make_uint4(0, 0, 0, 0);
         v.r0 = v.r1 = v.r2 = v.r3 = z;
         if (valid) {
             p += (size_t)lane * 16;
-            v.r0 = *(const uint4 *)(p);
-            v.r1 = *(const uint4 *)(p + 1024);
-            v.r2 = *(const uint4 *)(p + 2048);
-            v.r3 = *(const uint4 *)(p + 3072);
+            v.r0 = ld_stream128(p);
+            v.r1 = ld_stream128(p + 1024);
+            v.r2 = ld_stream128(p + 2048);
+            v.r3 = ld_stream128(p + 3072);
         }
     }
     return v;
@@ -560,26 +560,40 @@ __global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restri
     }
     const size_t base = ((size_t)b * QH + h) * Pmax;
     const size_t pbase = ((size_t)b * QH + h) * pre_splits;
+    // Pieces 0..npieces-1 are the stream kernel's, the rest the prefix pass's.  Lane s of
+    // each wave owns piece s (+64, ...): every (m, l) is fetched by one round of loads
+    // instead of a chain of dependent ones, and the o rows are loaded unconditionally,
+    // four at a time, with the weight deciding whether they count.
+    const int n_all = npieces + pre_splits, lane = d & 63;
     float M = -INFINITY;
-    for (int s = 0; s < npieces; s++)
-        if (part_l[base + s] > 0.0f) M = fmaxf(M, part_m[base + s]);
-    for (int s = 0; s < pre_splits; s++)
-        if (pre_l[pbase + s] > 0.0f) M = fmaxf(M, pre_m[pbase + s]);
+    for (int s = lane; s < n_all; s += 64) {
+        const float pl = s < npieces ? part_l[base + s] : pre_l[pbase + (s - npieces)];
+        const float pm = s < npieces ? part_m[base + s] : pre_m[pbase + (s - npieces)];
+        if (pl > 0.0f) M = fmaxf(M, pm);
+    }
+    M = s_wave_max(M);
     float acc = 0.0f, L = 0.0f;
-    for (int s = 0; s < npieces; s++) {
-        const float pl = part_l[base + s];
-        if (!(pl > 0.0f)) continue;
-        const float wgt = s_exp2(part_m[base + s] - M);
-        acc = fmaf(part_o[(base + s) * 128 + d], wgt, acc);
-        L = fmaf(pl, wgt, L);
+    for (int c0 = 0; c0 < n_all; c0 += 64) {
+        const int s = c0 + lane, cnt = min(64, n_all - c0);
+        float w = 0.0f;
+        if (s < n_all) {
+            const float pl = s < npieces ? part_l[base + s] : pre_l[pbase + (s - npieces)];
+            const float pm = s < npieces ? part_m[base + s] : pre_m[pbase + (s - npieces)];
+            if (pl > 0.0f) { w = s_exp2(pm - M); L = fmaf(pl, w, L); }
+        }
+        for (int j = 0; j < cnt; j += 4) {
+            float o[4], wj[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int jj = min(j + u, cnt - 1), sj = c0 + jj;
+                wj[u] = j + u < cnt ? s_lane(w, jj) : 0.0f;
+                o[u] = sj < npieces ? part_o[(base + sj) * 128 + d] : pre_o[(pbase + (sj - npieces)) * 128 + d];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) acc += wj[u] != 0.0f ? o[u] * wj[u] : 0.0f;
+        }
     }
-    for (int s = 0; s < pre_splits; s++) {
-        const float pl = pre_l[pbase + s];
-        if (!(pl > 0.0f)) continue;
-        const float wgt = s_exp2(pre_m[pbase + s] - M);
-        acc = fmaf(pre_o[(pbase + s) * 128 + d], wgt, acc);
-        L = fmaf(pl, wgt, L);
-    }
+    L = s_wave_sum(L);
     if (L > 0.0f) out[((size_t)b * QH + h) * 128 + d] = f_to_elem16(acc / L, io_dtype);
 }
 

@@ -71,16 +71,16 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(
                     hole[u] = false;
                     poff[u] = row_off(a, layer, blk, kv, h, gt - lb * bs_div.d) + (size_t)c * 16;
                 }
-                if (EXTRACT) { if (!hole[u]) val[u] = *(const uint4 *)(pool + poff[u]); }
-                else val[u] = *(const uint4 *)(fbase + (size_t)ci * 16);
+                if (EXTRACT) { if (!hole[u]) val[u] = ld_stream128(pool + poff[u]); }
+                else val[u] = ld_stream128(fbase + (size_t)ci * 16);
             }
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
             unsigned ci = base + u * kThreads;
             if (!live[u]) continue;
-            if (EXTRACT) *(uint4 *)(fbase + (size_t)ci * 16) = val[u];          // hole => zeros
-            else if (!hole[u]) *(uint4 *)(pool + poff[u]) = val[u];              // hole => skip
+            if (EXTRACT) st_stream128(fbase + (size_t)ci * 16, val[u]);         // hole => zeros
+            else if (!hole[u]) st_stream128(pool + poff[u], val[u]);            // hole => skip
         }
     }
 
@@ -173,10 +173,10 @@ __global__ __launch_bounds__(kThreads) void append_kernel(
                     if (QMODE == 1) soff = scale_off(a, layer, blk, kv, h, p);
                 }
             }
-            val = *(const uint4 *)(sbase + (size_t)ci * 16);
+            val = ld_stream128(sbase + (size_t)ci * 16);
         }
         if (QMODE == 0) {
-            if (live && !hole) *(uint4 *)(pool + poff + (size_t)c * 16) = val;
+            if (live && !hole) st_stream128(pool + poff + (size_t)c * 16, val);
         } else {
             float x[8];
             unpack8(val, src_dtype, x);

@@ -98,16 +98,24 @@ struct PfGroup {
     uint4 r0, r1, r2, r3;
 };
 
+template <bool ONCE>
 __device__ __forceinline__ PfGroup pf_load_group(const uint8_t *__restrict__ base, bool valid, size_t off, int lane)
 {
     PfGroup g;
     g.r0 = g.r1 = g.r2 = g.r3 = make_uint4(0, 0, 0, 0);
     if (valid) {
         const uint8_t *p = base + off + (size_t)lane * 16;
-        g.r0 = *(const uint4 *)(p);
-        g.r1 = *(const uint4 *)(p + 1024);
-        g.r2 = *(const uint4 *)(p + 2048);
-        g.r3 = *(const uint4 *)(p + 3072);
+        if constexpr (ONCE) {       // every page is read by one workgroup only: stream it
+            g.r0 = ld_stream128(p);
+            g.r1 = ld_stream128(p + 1024);
+            g.r2 = ld_stream128(p + 2048);
+            g.r3 = ld_stream128(p + 3072);
+        } else {                    // 64 row tiles of a chunk share each page through the L2
+            g.r0 = *(const uint4 *)(p);
+            g.r1 = *(const uint4 *)(p + 1024);
+            g.r2 = *(const uint4 *)(p + 2048);
+            g.r3 = *(const uint4 *)(p + 3072);
+        }
     }
     return g;
 }
@@ -186,8 +194,8 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
 
     bool cur_valid, nxt_valid = false;
     size_t off = lookup(t_begin, cur_valid);
-    PfGroup kreg = pf_load_group(kbase, cur_valid, off, lane);
-    PfGroup vreg = pf_load_group(kbase + A.kv_plane, cur_valid, off, lane);
+    PfGroup kreg = pf_load_group<SHARED>(kbase, cur_valid, off, lane);
+    PfGroup vreg = pf_load_group<SHARED>(kbase + A.kv_plane, cur_valid, off, lane);
 
     for (int it = t_begin; it < ntiles; it++) {
         const int tile_t = it * kPfBN;
@@ -205,8 +213,8 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         if (lane == 0) valid_lds[w] = cur_valid ? 1 : 0;
         if (it + 1 < ntiles) {
             off = lookup(it + 1, nxt_valid);
-            kreg = pf_load_group(kbase, nxt_valid, off, lane);
-            vreg = pf_load_group(kbase + A.kv_plane, nxt_valid, off, lane);
+            kreg = pf_load_group<SHARED>(kbase, nxt_valid, off, lane);
+            vreg = pf_load_group<SHARED>(kbase + A.kv_plane, nxt_valid, off, lane);
         }
         __syncthreads();
 
