@@ -5,6 +5,7 @@ raises ImportError: nothing here computes anything on its own.
 """
 import ctypes as C
 import os
+import sys
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libdrk_kv.so")
@@ -68,6 +69,7 @@ SIGNATURES = {
     "drk_debug_force_portable_decode": (None, [_i32]),
     "drk_debug_set_decode_kernel": (None, [_i32]),
     "drk_debug_set_stream_workgroups": (None, [_i32]),
+    "drk_debug_set_shared_splits": (None, [_i32]),
     "drk_debug_time_decode_kernel": (None, [_i32]),
     "drk_debug_set_decode_lds_pad": (None, [_i32]),
     "drk_probe_read_bandwidth": (_i32, [_vp, _sz, _i32, _vp, C.POINTER(C.c_float)]),
@@ -94,6 +96,16 @@ def lib():
             raise ImportError(
                 f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
                 "or `make -C deusridet_amd/csrc`")
+        # A process must hold ONE HIP runtime.  PyTorch-ROCm ships its own libamdhip64;
+        # when this library is loaded first it binds /opt/rocm's copy instead, torch then
+        # brings a second one, and HIP calls of the later-initialised copy fail with
+        # "no ROCm-capable device is detected".  Loading torch first makes both share
+        # torch's copy; a process without torch simply uses /opt/rocm's.
+        if "torch" not in sys.modules:
+            try:
+                import torch  # noqa: F401
+            except ImportError:
+                pass
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(L, name)

@@ -48,17 +48,23 @@ int make_lay(const drk_kv_layout *g, Lay *a)
     return DRK_OK;
 }
 
+// Each workgroup streams whole 64 KiB chunks, round-robin over the grid: the pattern
+// (of those tried: grid-stride, chunked, permuted 4 KiB granules; plain and streaming
+// loads) that sustains the most on MI355X.
+constexpr size_t kProbeChunkVec = 65536 / 16;
 __global__ __launch_bounds__(256) void read_probe_kernel(const uint4 *__restrict__ p, size_t nvec,
                                                         unsigned *__restrict__ sink)
 {
     unsigned acc = 0;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for (; i + 3 * stride < nvec; i += 4 * stride) {
-        uint4 a = ld_stream128(p + i), b = ld_stream128(p + i + stride), c = ld_stream128(p + i + 2 * stride), d = ld_stream128(p + i + 3 * stride);
-        acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    const size_t nchunks = nvec / kProbeChunkVec;
+    for (size_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+        const uint4 *q = p + c * kProbeChunkVec;
+        for (unsigned i = threadIdx.x; i < kProbeChunkVec; i += 4 * 256) {
+            uint4 a = ld_stream128(q + i), b = ld_stream128(q + i + 256), cc = ld_stream128(q + i + 512),
+                  d = ld_stream128(q + i + 768);
+            acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ cc.x ^ cc.y ^ cc.z ^ cc.w ^ d.x ^ d.y ^ d.z ^ d.w;
+        }
     }
-    for (; i < nvec; i += stride) { uint4 a = p[i]; acc ^= a.x ^ a.y ^ a.z ^ a.w; }
     if (acc == 0x9e3779b9u) *sink = acc;      // practically never: keeps the loads alive
 }
 
@@ -177,11 +183,11 @@ int drk_probe_read_bandwidth(const void *d_ptr, size_t bytes, int iters, void *d
 {
     if (!d_ptr || !d_sink || !gbps || bytes < (1u << 20) || iters < 1)
         return fail(DRK_ERR_INVALID, "probe: bad argument");
-    size_t nvec = bytes / 16;
+    size_t nvec = bytes / 16 / drk::kProbeChunkVec * drk::kProbeChunkVec;     // whole 64 KiB chunks
     hipEvent_t e0, e1;
     DRK_HIP(hipEventCreate(&e0));
     DRK_HIP(hipEventCreate(&e1));
-    dim3 grid(256 * 8), block(256);
+    dim3 grid(256 * 4), block(256);
     for (int i = 0; i < 5; i++)
         hipLaunchKernelGGL(drk::read_probe_kernel, grid, block, 0, 0, (const uint4 *)d_ptr, nvec, (unsigned *)d_sink);
     DRK_HIP(hipEventRecord(e0, 0));

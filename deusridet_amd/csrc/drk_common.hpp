@@ -63,6 +63,7 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
 
 // persistent stream-K decode (drk_decode_stream.hip)
 extern int g_stream_wgs;
+extern int g_shared_splits;
 bool stream_decode_supported(const Lay &a, int B);
 size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens);
 int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,

@@ -27,7 +27,11 @@
 
 namespace drk {
 
-int g_stream_wgs = 512;              // workgroups of the persistent grid (2 per CU of a 256-CU part)
+// Workgroups of the persistent grid on a 256-CU part; 0 = by storage type: 2 per CU
+// for 16-bit pages (bandwidth-bound: fewer, longer runs stream best), 3 per CU for
+// 8-bit pages (the dequantising waves need the extra latency hiding).
+int g_stream_wgs = 0;
+static inline int stream_wgs(const Lay &a) { return g_stream_wgs > 0 ? g_stream_wgs : (a.E == 1 ? 768 : 512); }
 
 constexpr int kSTile = 64;
 constexpr int kSRow = 272;
@@ -102,34 +106,44 @@ __device__ __forceinline__ float s_wave_sum(float v)
     return (s_lane(v, 0) + s_lane(v, 16)) + (s_lane(v, 32) + s_lane(v, 48));
 }
 
-// four int8 codes -> two dwords of packed fp16, exact: (code ^ 0x80) | 0x6400 is the
-// fp16 number 1024 + code + 128
-__device__ __forceinline__ void int8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+__device__ __forceinline__ uint32_t s_perm(uint32_t hi, uint32_t lo, uint32_t sel)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t x = w ^ 0x80808080u;
-    const uint32_t a = __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u);   // bytes x0,64,x1,64
-    const uint32_t b = __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u);   // bytes x2,64,x3,64
-    const s_f16x2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-    lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s_f16x2, a) - bias);
-    hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(s_f16x2, b) - bias);
+    return __builtin_amdgcn_perm(hi, lo, sel);      // result byte i = byte sel[i] of {lo: 0-3, hi: 4-7}
 #else
-    (void)w; lo = hi = 0;
+    (void)hi; (void)sel;
+    return lo;
 #endif
 }
 
-// four fp8-e4m3 codes -> two dwords of packed fp16 (exact: e4m3 fits in fp16)
-__device__ __forceinline__ void fp8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+// int8 codes travel as fp16 1152 + code: byte (code ^ 0x80) under the exponent byte 0x64
+// is exactly that number, so a code costs one byte permute and the constant is taken
+// out once per dot product (1152 * sum of the other operand) instead of once per value.
+constexpr float kI8Bias = 1152.0f;
+constexpr uint32_t kF16Ones = 0x3C003C00u;
+
+// four int8 codes -> two dwords of packed fp16 (1152 + code)
+__device__ __forceinline__ void int8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+{
+    const uint32_t x = w ^ 0x80808080u;
+    lo = s_perm(0x64646464u, x, 0x04010400u);   // bytes x0,64,x1,64
+    hi = s_perm(0x64646464u, x, 0x04030402u);   // bytes x2,64,x3,64
+}
+
+// two fp8-e4m3 codes (the low or the high half of w) -> packed fp16 (exact: e4m3 fits in fp16)
+template <bool HIGH>
+__device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t w)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
-    typedef float f2 __attribute__((ext_vector_type(2)));
-    const f2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
-    const f2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
-    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a[0], a[1]));
-    hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(b[0], b[1]));
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, HIGH));
 #else
-    (void)w; lo = hi = 0;
+    return w;
 #endif
+}
+__device__ __forceinline__ void fp8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+{
+    lo = fp8x2_to_f16x2<false>(w);
+    hi = fp8x2_to_f16x2<true>(w);
 }
 
 struct StreamArgs {
@@ -163,55 +177,44 @@ template <int DT> struct VRegs { uint4 r0, r1, r2, r3; };
 template <> struct VRegs<DRK_INT8> { uint2 r0, r1, r2, r3; };
 template <> struct VRegs<DRK_FP8_E4M3> { uint2 r0, r1, r2, r3; };
 
+// The 16-token run of one kv head at byte offset `off` of the layer (kNone: the run has no
+// page).  A missing run is loaded from offset 0 -- always mapped -- instead of being
+// predicated off: its K only feeds scores that are masked anyway, and its V is cleared
+// by the consumer where a stale bit pattern could matter.
 template <int DT>
-__device__ __forceinline__ KRegs<DT> load_k(const uint8_t *__restrict__ p, bool valid, int lane)
+__device__ __forceinline__ KRegs<DT> load_k(const uint8_t *__restrict__ layer, uint32_t off, int lane)
 {
     KRegs<DT> k;
-    const uint4 z = make_uint4(0, 0, 0, 0);
+    const uint8_t *p = layer + (off == 0xffffffffu ? 0u : off) + (size_t)lane * 16;
     if constexpr (KvTraits<DT>::q8) {
-        k.r0 = k.r1 = z;
-        if (valid) {
-            p += (size_t)lane * 16;
-            k.r0 = ld_stream128(p);
-            k.r1 = ld_stream128(p + 1024);
-        }
+        k.r0 = ld_stream128(p);
+        k.r1 = ld_stream128(p + 1024);
     } else {
-        k.r0 = k.r1 = k.r2 = k.r3 = z;
-        if (valid) {
-            p += (size_t)lane * 16;
-            k.r0 = ld_stream128(p);
-            k.r1 = ld_stream128(p + 1024);
-            k.r2 = ld_stream128(p + 2048);
-            k.r3 = ld_stream128(p + 3072);
-        }
+        k.r0 = ld_stream128(p);
+        k.r1 = ld_stream128(p + 1024);
+        k.r2 = ld_stream128(p + 2048);
+        k.r3 = ld_stream128(p + 3072);
     }
     return k;
 }
 
 template <int DT>
-__device__ __forceinline__ VRegs<DT> load_v(const uint8_t *__restrict__ p, bool valid, int lane)
+__device__ __forceinline__ VRegs<DT> load_v(const uint8_t *__restrict__ layer, uint32_t off, uint32_t kv_plane, int lane)
 {
     VRegs<DT> v;
+    const uint8_t *p = layer + (off == 0xffffffffu ? 0u : off) + kv_plane;
     if constexpr (KvTraits<DT>::q8) {
-        const uint2 z = make_uint2(0, 0);
-        v.r0 = v.r1 = v.r2 = v.r3 = z;
-        if (valid) {
-            p += (size_t)lane * 8;
-            v.r0 = ld_stream64(p);
-            v.r1 = ld_stream64(p + 512);
-            v.r2 = ld_stream64(p + 1024);
-            v.r3 = ld_stream64(p + 1536);
-        }
+        p += (size_t)lane * 8;
+        v.r0 = ld_stream64(p);
+        v.r1 = ld_stream64(p + 512);
+        v.r2 = ld_stream64(p + 1024);
+        v.r3 = ld_stream64(p + 1536);
     } else {
-        const uint4 z = make_uint4(0, 0, 0, 0);
-        v.r0 = v.r1 = v.r2 = v.r3 = z;
-        if (valid) {
-            p += (size_t)lane * 16;
-            v.r0 = ld_stream128(p);
-            v.r1 = ld_stream128(p + 1024);
-            v.r2 = ld_stream128(p + 2048);
-            v.r3 = ld_stream128(p + 3072);
-        }
+        p += (size_t)lane * 16;
+        v.r0 = ld_stream128(p);
+        v.r1 = ld_stream128(p + 1024);
+        v.r2 = ld_stream128(p + 2048);
+        v.r3 = ld_stream128(p + 3072);
     }
     return v;
 }
@@ -250,38 +253,46 @@ __device__ __forceinline__ void stage_k(uint8_t *tile_lds, const KRegs<DT> &k, i
     }
 }
 
-// o[h][e] += pp[h] * V[row][dims of this lane], 8 dims per lane
+// o[h][e] += p[a][h] * V[a][e] + p[b][h] * V[b][e] for two token rows a, b and the 8 dims of
+// this lane: one v_dot2 per (head, dim) over the token pair.  pp holds, per head, the packed
+// 16-bit weights (p[a], p[b]); the rows' values are paired up by byte permutes.
 template <int DT, typename VR>
-__device__ __forceinline__ void pv_row(float (&o)[4][8], float (&psum)[4], const VR &vv, const float4 pp)
+__device__ __forceinline__ void pv_pair(float (&o)[4][8], float (&psum)[4], const VR &va, const VR &vb, const uint4 pp)
 {
-    float x[8];
-    if constexpr (DT == DRK_INT8) {
-        const uint32_t a = vv.x ^ 0x80808080u, b = vv.y ^ 0x80808080u;        // code + 128, 0..255
-        x[0] = (float)(a & 0xffu); x[1] = (float)((a >> 8) & 0xffu); x[2] = (float)((a >> 16) & 0xffu); x[3] = (float)(a >> 24);
-        x[4] = (float)(b & 0xffu); x[5] = (float)((b >> 8) & 0xffu); x[6] = (float)((b >> 16) & 0xffu); x[7] = (float)(b >> 24);
-        psum[0] += pp.x; psum[1] += pp.y; psum[2] += pp.z; psum[3] += pp.w;   // the +128 is taken out at the end
-    } else if constexpr (DT == DRK_FP8_E4M3) {
-#if defined(__HIP_DEVICE_COMPILE__)
-        typedef float f2 __attribute__((ext_vector_type(2)));
-        const f2 a0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.x, false), a1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.x, true);
-        const f2 b0 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.y, false), b1 = __builtin_amdgcn_cvt_pk_f32_fp8((int)vv.y, true);
-        x[0] = a0[0]; x[1] = a0[1]; x[2] = a1[0]; x[3] = a1[1];
-        x[4] = b0[0]; x[5] = b0[1]; x[6] = b1[0]; x[7] = b1[1];
-#endif
+    constexpr int DOT = KvTraits<DT>::dot;
+    uint32_t pr[8];
+    if constexpr (KvTraits<DT>::q8) {
+        const uint32_t i0 = s_perm(vb.x, va.x, 0x05010400u), i1 = s_perm(vb.x, va.x, 0x07030602u);   // a0 b0 a1 b1 | a2 b2 a3 b3
+        const uint32_t i2 = s_perm(vb.y, va.y, 0x05010400u), i3 = s_perm(vb.y, va.y, 0x07030602u);
+        if constexpr (DT == DRK_INT8) {
+            int8x4_to_f16x4(i0, pr[0], pr[1]);
+            int8x4_to_f16x4(i1, pr[2], pr[3]);
+            int8x4_to_f16x4(i2, pr[4], pr[5]);
+            int8x4_to_f16x4(i3, pr[6], pr[7]);
+            psum[0] = s_dot2<DOT>(pp.x, kF16Ones, psum[0]);          // the +1152 is taken out at the end
+            psum[1] = s_dot2<DOT>(pp.y, kF16Ones, psum[1]);
+            psum[2] = s_dot2<DOT>(pp.z, kF16Ones, psum[2]);
+            psum[3] = s_dot2<DOT>(pp.w, kF16Ones, psum[3]);
+        } else {
+            fp8x4_to_f16x4(i0, pr[0], pr[1]);
+            fp8x4_to_f16x4(i1, pr[2], pr[3]);
+            fp8x4_to_f16x4(i2, pr[4], pr[5]);
+            fp8x4_to_f16x4(i3, pr[6], pr[7]);
+        }
     } else {
-        const uint32_t wds[4] = {vv.x, vv.y, vv.z, vv.w};
+        const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            if constexpr (DT == DRK_BF16) { x[2 * i] = bf16_lo(wds[i]); x[2 * i + 1] = bf16_hi(wds[i]); }
-            else { x[2 * i] = f16_bits_to_f((uint16_t)(wds[i] & 0xffffu)); x[2 * i + 1] = f16_bits_to_f((uint16_t)(wds[i] >> 16)); }
+            pr[2 * i] = s_perm(wb[i], wa[i], 0x05040100u);
+            pr[2 * i + 1] = s_perm(wb[i], wa[i], 0x07060302u);
         }
     }
 #pragma unroll
     for (int e = 0; e < 8; e++) {
-        o[0][e] = fmaf(pp.x, x[e], o[0][e]);
-        o[1][e] = fmaf(pp.y, x[e], o[1][e]);
-        o[2][e] = fmaf(pp.z, x[e], o[2][e]);
-        o[3][e] = fmaf(pp.w, x[e], o[3][e]);
+        o[0][e] = s_dot2<DOT>(pr[e], pp.x, o[0][e]);
+        o[1][e] = s_dot2<DOT>(pr[e], pp.y, o[1][e]);
+        o[2][e] = s_dot2<DOT>(pr[e], pp.z, o[2][e]);
+        o[3][e] = s_dot2<DOT>(pr[e], pp.w, o[3][e]);
     }
 }
 
@@ -292,7 +303,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     constexpr int DOT = KvTraits<DT>::dot;
     constexpr uint32_t kNone = 0xffffffffu;
     __shared__ __align__(16) uint8_t k_lds[2][kSTile * kSRow];
-    __shared__ __align__(16) float p_lds[2][kSTile * 4];
+    __shared__ __align__(16) uint16_t p_lds[2][kSTile * 4];   // [pair of rows][head][row of the pair], 16-bit weights
     __shared__ __align__(16) float alpha_lds[2][4];
     __shared__ __align__(16) float kscale_lds[2][kSTile];
     __shared__ __align__(16) float vscale_lds[2][kSTile];
@@ -376,12 +387,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     for (int hh = 0; hh < 4; hh++)
 #pragma unroll
         for (int e = 0; e < 8; e++) o[hh][e] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f, qbias = 0.0f;
     uint32_t qs[64];
 
     uint2 gd = gdesc[0][w];
-    KRegs<DT> kreg = load_k<DT>(A.pool_layer + gd.x, gd.x != kNone, lane);
-    VRegs<DT> vreg = load_v<DT>(A.pool_layer + gd.x + A.kv_plane, gd.x != kNone, lane);
+    KRegs<DT> kreg = load_k<DT>(A.pool_layer, gd.x, lane);
+    VRegs<DT> vreg = load_v<DT>(A.pool_layer, gd.x, A.kv_plane, lane);
+    bool vhole = gd.x == kNone;                               // the run vreg was loaded for has no page
     uint32_t sreg = load_scales(gd);
     uint32_t qv = load_q(udesc[0].bq);
 
@@ -394,6 +406,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         if (flags & 1) {                          // Q of the segment's head into scalar registers
 #pragma unroll
             for (int i = 0; i < 64; i++) qs[i] = __builtin_amdgcn_readlane(qv, i);
+            if (DT == DRK_INT8) {                 // sum of the head's (fp16) query values, for the code offset
+                float sq = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 64; i++) sq = s_dot2<DOT>(qs[i], kF16Ones, sq);
+                qbias = kI8Bias * sq;
+            }
         }
 
         // ---- A: stage K (and scales), start the next unit's K loads -------------------
@@ -405,7 +423,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         }
         if (has_next) {
             gd = gdesc[it + 1][w];
-            kreg = load_k<DT>(A.pool_layer + gd.x, gd.x != kNone, lane);
+            kreg = load_k<DT>(A.pool_layer, gd.x, lane);
             sreg = load_scales(gd);
             if (flags & 2) qv = load_q(udesc[it + 1].bq);
         }
@@ -437,8 +455,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                 for (int c = 0; c < 4; c++) ka[c] = kb[c];
             }
             const bool live = lane < tile_lim && gdesc[it][lane >> 4].x != kNone;
+            if (DT == DRK_INT8) acc = (acc - qbias) * kscale_lds[buf][lane];
             float sc = acc * A.scale_log2e;
-            if (DT == DRK_INT8) sc *= kscale_lds[buf][lane];
             sc = live ? sc : -INFINITY;
             const float m_new = fmaxf(m_run, s_wave_max(sc));
             const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
@@ -448,7 +466,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             m_run = m_new;
             float pw = p;
             if (DT == DRK_INT8) pw = live ? p * vscale_lds[buf][lane] : 0.0f;   // a stale scale may be anything
-            p_lds[buf][lane * 4 + w] = pw;
+            {
+                // rows r, r+4 of a wave's 16 form a pair, and so do r+8, r+12: phase C holds exactly these
+                uint16_t pb;
+                if constexpr (DOT == DRK_BF16) pb = __builtin_bit_cast(uint16_t, (__bf16)pw);
+                else pb = __builtin_bit_cast(uint16_t, (_Float16)pw);
+                const int r = lane & 15, pidx = ((lane >> 4) * 4 + (r & 3)) * 2 + (r >> 3);
+                p_lds[buf][(pidx * 4 + w) * 2 + ((r >> 2) & 1)] = pb;
+            }
             if (lane == 0) alpha_lds[buf][w] = alpha;
         }
         __syncthreads();
@@ -464,19 +489,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                 psum[0] *= al.x; psum[1] *= al.y; psum[2] *= al.z; psum[3] *= al.w;
             }
             const int r0 = w * 16 + lrow;
-            if (DT != DRK_INT8 && tile_lim < kSTile) {        // rows past the end may hold anything
-                if (r0 >= tile_lim) vreg.r0 = {};
-                if (r0 + 4 >= tile_lim) vreg.r1 = {};
-                if (r0 + 8 >= tile_lim) vreg.r2 = {};
-                if (r0 + 12 >= tile_lim) vreg.r3 = {};
+            if (DT != DRK_INT8 && (tile_lim < kSTile || vhole)) {   // rows without a token may hold anything (NaN)
+                if (vhole || r0 >= tile_lim) vreg.r0 = {};
+                if (vhole || r0 + 4 >= tile_lim) vreg.r1 = {};
+                if (vhole || r0 + 8 >= tile_lim) vreg.r2 = {};
+                if (vhole || r0 + 12 >= tile_lim) vreg.r3 = {};
             }
-            const float *pl = &p_lds[buf][r0 * 4];
-            pv_row<DT>(o, psum, vreg.r0, *(const float4 *)(pl));
-            pv_row<DT>(o, psum, vreg.r1, *(const float4 *)(pl + 16));
-            pv_row<DT>(o, psum, vreg.r2, *(const float4 *)(pl + 32));
-            pv_row<DT>(o, psum, vreg.r3, *(const float4 *)(pl + 48));
+            const uint4 *pl = (const uint4 *)&p_lds[buf][(w * 4 + lrow) * 16];
+            pv_pair<DT>(o, psum, vreg.r0, vreg.r1, pl[0]);
+            pv_pair<DT>(o, psum, vreg.r2, vreg.r3, pl[1]);
         }
-        if (has_next) vreg = load_v<DT>(A.pool_layer + gd.x + A.kv_plane, gd.x != kNone, lane);
+        if (has_next) {
+            vreg = load_v<DT>(A.pool_layer, gd.x, A.kv_plane, lane);
+            vhole = gd.x == kNone;
+        }
 
         // ---- the segment's last tile: leave (o, m, l) for the merge ----------------------
         if (flags & 2) {
@@ -485,7 +511,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     float v = o[hh][e];
-                    if (DT == DRK_INT8) v -= 128.0f * psum[hh];
+                    if (DT == DRK_INT8) v -= kI8Bias * psum[hh];
                     v += __shfl_xor(v, 16);
                     v += __shfl_xor(v, 32);
                     o[hh][e] = v;
@@ -613,7 +639,7 @@ static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens,
         *grid = (int)((t_upper + U - 1) / U);
         *Pmax = ((max_seq_len + kSTile - 1) / kSTile + U - 1) / U + 2;
     } else {
-        long G = t_upper < g_stream_wgs ? t_upper : g_stream_wgs;
+        long G = t_upper < stream_wgs(a) ? t_upper : stream_wgs(a);
         if ((t_upper + G - 1) / G > kMaxUnits) G = (t_upper + kMaxUnits - 1) / kMaxUnits;   // descriptor table size
         *unit_tiles = 0;
         *grid = (int)G;

@@ -336,10 +336,12 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
 // ---- shared-prefix ("cascade") decode: host side of the prefix pass -------------------
 // One launch covers tokens [0, shared) for all B branches; the private tails go
 // through the stream kernel with start_tile = shared / 64.
+int g_shared_splits = 64;              // context splits of the prefix pass: 8 kv heads x 64 = two workgroups per CU
+
 void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits)
 {
     const int tiles = shared / kPfBN;
-    int ns = tiles < 32 ? tiles : 32;                     // 8 kv heads x 32 splits = one workgroup per CU
+    int ns = tiles < g_shared_splits ? tiles : g_shared_splits;
     if (ns < 1) ns = 1;
     *chunk_tiles = (tiles + ns - 1) / ns;
     if (*chunk_tiles < 1) *chunk_tiles = 1;

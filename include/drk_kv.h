@@ -159,8 +159,12 @@ void drk_debug_force_portable_decode(int on);
  * a choice: 0 = automatic (the persistent stream kernel), 2 = the fixed-split
  * tiled kernel (16-bit pages only), 3 = same as 0.  Process-wide. */
 void drk_debug_set_decode_kernel(int which);
-/* Diagnostic: workgroups of the persistent decode grid (default 512). */
+/* Diagnostic: workgroups of the persistent decode grid; 0 restores the default (512 for 16-bit pages,
+ * 768 for 8-bit pages). */
 void drk_debug_set_stream_workgroups(int n);
+/* Diagnostic: context splits of the shared-prefix pass (default 64, at most 256; 0 restores the
+ * default).  Changes drk_decode_shared_workspace_bytes. */
+void drk_debug_set_shared_splits(int n);
 /* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
  * session; switching it on starts a new session) records a HIP event on its
  * stream right before and right after the split-K partial kernel; the merge
