@@ -556,10 +556,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
 }
 
-// grid (QH, B), block 128: fold the pieces of (branch, q head) -- the stream kernel's
+// grid (QH, B), block 256: fold the pieces of (branch, q head) -- the stream kernel's
 // and, in shared-prefix mode, the prefix pass's; out is written only when some
-// token took part (paged_attention.cu:266)
-__global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_m,
+// token took part (paged_attention.cu:266).  Lane s of every wave owns the (m, l) of
+// piece s (+64, ...), so they arrive in one round of loads; wave w then folds the o
+// rows of pieces w, w+4, ... for two dims per lane, eight rows in flight, and the four
+// waves' sums meet in LDS.
+__global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_m,
                                                            const float *__restrict__ part_l, uint16_t *__restrict__ out,
                                                            const int32_t *__restrict__ seq_lens, int seq_len_host, int B,
                                                            int KVH, int QH, int unit_tiles, int grid_wgs, int Pmax,
@@ -567,7 +570,8 @@ __global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restri
                                                            const float *__restrict__ pre_m, const float *__restrict__ pre_l,
                                                            int pre_splits)
 {
-    const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    __shared__ float2 red[4][64];
+    const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * 2;
     int excl = 0, total = 0, nt_b = 0;
     for (int i = 0; i < B; i++) {
         const int len = seq_lens ? seq_lens[i] : seq_len_host;
@@ -586,11 +590,7 @@ __global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restri
     }
     const size_t base = ((size_t)b * QH + h) * Pmax;
     const size_t pbase = ((size_t)b * QH + h) * pre_splits;
-    // Pieces 0..npieces-1 are the stream kernel's, the rest the prefix pass's.  Lane s of
-    // each wave owns piece s (+64, ...): every (m, l) is fetched by one round of loads
-    // instead of a chain of dependent ones, and the o rows are loaded unconditionally,
-    // four at a time, with the weight deciding whether they count.
-    const int n_all = npieces + pre_splits, lane = d & 63;
+    const int n_all = npieces + pre_splits;                  // pieces 0..npieces-1: stream kernel; then the prefix pass
     float M = -INFINITY;
     for (int s = lane; s < n_all; s += 64) {
         const float pl = s < npieces ? part_l[base + s] : pre_l[pbase + (s - npieces)];
@@ -598,7 +598,8 @@ __global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restri
         if (pl > 0.0f) M = fmaxf(M, pm);
     }
     M = s_wave_max(M);
-    float acc = 0.0f, L = 0.0f;
+    float2 acc = make_float2(0.0f, 0.0f);
+    float L = 0.0f;
     for (int c0 = 0; c0 < n_all; c0 += 64) {
         const int s = c0 + lane, cnt = min(64, n_all - c0);
         float w = 0.0f;
@@ -607,20 +608,28 @@ __global__ __launch_bounds__(128) void stream_merge_kernel(const float *__restri
             const float pm = s < npieces ? part_m[base + s] : pre_m[pbase + (s - npieces)];
             if (pl > 0.0f) { w = s_exp2(pm - M); L = fmaf(pl, w, L); }
         }
-        for (int j = 0; j < cnt; j += 4) {
-            float o[4], wj[4];
+        for (int j = wv; j < cnt; j += 32) {
+            float2 o[8];
+            float wj[8];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int jj = min(j + u, cnt - 1), sj = c0 + jj;
-                wj[u] = j + u < cnt ? s_lane(w, jj) : 0.0f;
-                o[u] = sj < npieces ? part_o[(base + sj) * 128 + d] : pre_o[(pbase + (sj - npieces)) * 128 + d];
+            for (int u = 0; u < 8; u++) {
+                const int jj = min(j + 4 * u, cnt - 1), sj = c0 + jj;
+                wj[u] = j + 4 * u < cnt ? s_lane(w, jj) : 0.0f;
+                o[u] = *(const float2 *)(sj < npieces ? part_o + (base + sj) * 128 + d : pre_o + (pbase + (sj - npieces)) * 128 + d);
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) acc += wj[u] != 0.0f ? o[u] * wj[u] : 0.0f;
+            for (int u = 0; u < 8; u++)
+                if (wj[u] != 0.0f) { acc.x = fmaf(o[u].x, wj[u], acc.x); acc.y = fmaf(o[u].y, wj[u], acc.y); }   // a piece without tokens may hold anything
         }
     }
     L = s_wave_sum(L);
-    if (L > 0.0f) out[((size_t)b * QH + h) * 128 + d] = f_to_elem16(acc / L, io_dtype);
+    red[wv][lane] = acc;
+    __syncthreads();
+    if (wv == 0 && L > 0.0f) {
+        const float2 a1 = red[1][lane], a2 = red[2][lane], a3 = red[3][lane];
+        const float x = ((acc.x + a1.x) + (a2.x + a3.x)) / L, y = ((acc.y + a1.y) + (a2.y + a3.y)) / L;
+        *(uint32_t *)(out + ((size_t)b * QH + h) * 128 + d) = (uint32_t)f_to_elem16(x, io_dtype) | ((uint32_t)f_to_elem16(y, io_dtype) << 16);
+    }
 }
 
 bool stream_decode_supported(const Lay &a, int B)
@@ -684,7 +693,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         }
         DRK_LAUNCH_CHECK("decode_stream_kernel");
     } else {
-        hipLaunchKernelGGL(stream_merge_kernel, dim3(a.QH, B), dim3(128), 0, st, part_o, part_m, part_l, (uint16_t *)out,
+        hipLaunchKernelGGL(stream_merge_kernel, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                            d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
                            pre_l, pre_splits);
         DRK_LAUNCH_CHECK("stream_merge_kernel");
