@@ -149,66 +149,78 @@ __global__ __launch_bounds__(kThreads) void append_kernel(
     const uint8_t *sbase = (kv ? src_v : src_k) + ((size_t)li * ntokens + t0) * a.KVH * src_row;
     const unsigned rounds = (items + kThreads - 1) / kThreads;
 
-    for (unsigned rnd = 0; rnd < rounds; rnd++) {
-        unsigned ci = rnd * kThreads + threadIdx.x;
-        bool live = ci < items;
-        uint4 val = make_uint4(0, 0, 0, 0);
-        size_t poff = 0, soff = 0;
-        unsigned c = 0;
-        bool hole = true;
-        if (live) {
-            unsigned t = dv(ci, tok_div), r = ci - t * tok_div.d;
-            unsigned h = dv(r, row_div);
-            c = r - h * rc;
-            int ti = t0 + (int)t;
-            int pos = d_pos ? d_pos[ti] : pos_start + ti;
-            const int32_t *tab = tables + (size_t)(d_pos ? ti : 0) * table_stride;
-            if (pos >= 0) {
-                unsigned lb = dv((unsigned)pos, bs_div);
-                int blk = tab[lb];
-                if (blk >= 0 && blk < a.NB) {
-                    hole = false;
-                    int p = pos - lb * bs_div.d;
-                    poff = row_off(a, layer, blk, kv, h, p);
-                    if (QMODE == 1) soff = scale_off(a, layer, blk, kv, h, p);
+    // U rounds at a time: all their source loads are issued before the first is consumed
+    constexpr int U = QMODE == 0 ? 2 : 4;
+    for (unsigned rnd0 = 0; rnd0 < rounds; rnd0 += U) {
+        uint4 val[U];
+        size_t poff[U], soff[U];
+        unsigned cc[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const unsigned ci = (rnd0 + u) * kThreads + threadIdx.x;
+            val[u] = make_uint4(0, 0, 0, 0);
+            poff[u] = soff[u] = 0;
+            cc[u] = 0;
+            ok[u] = false;
+            if (ci < items) {
+                unsigned t = dv(ci, tok_div), r = ci - t * tok_div.d;
+                unsigned h = dv(r, row_div);
+                cc[u] = r - h * rc;
+                int ti = t0 + (int)t;
+                int pos = d_pos ? d_pos[ti] : pos_start + ti;
+                const int32_t *tab = tables + (size_t)(d_pos ? ti : 0) * table_stride;
+                if (pos >= 0) {
+                    unsigned lb = dv((unsigned)pos, bs_div);
+                    int blk = tab[lb];
+                    if (blk >= 0 && blk < a.NB) {
+                        ok[u] = true;
+                        int p = pos - lb * bs_div.d;
+                        poff[u] = row_off(a, layer, blk, kv, h, p);
+                        if (QMODE == 1) soff[u] = scale_off(a, layer, blk, kv, h, p);
+                    }
                 }
+                val[u] = ld_stream128(sbase + (size_t)ci * 16);
             }
-            val = ld_stream128(sbase + (size_t)ci * 16);
         }
-        if (QMODE == 0) {
-            if (live && !hole) st_stream128(pool + poff + (size_t)c * 16, val);
-        } else {
-            float x[8];
-            unpack8(val, src_dtype, x);
-            if (QMODE == 1) {
-                // row absmax over the rc lanes that hold this row (rc is a power
-                // of two <= 64 and rows never straddle a wave)
-                float amax = 0.0f;
 #pragma unroll
-                for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(x[i]));
-                for (unsigned off = rc >> 1; off > 0; off >>= 1)
-                    amax = fmaxf(amax, __shfl_xor(amax, (int)off));
-                float s32 = __fdiv_rn(amax, 127.0f);
-                uint16_t sh = __half_as_ushort(__float2half_rn(s32));
-                if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
-                float sf = f16_bits_to_f(sh);
-                float rcp = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
-                uint32_t lo = 0, hi = 0;
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    float r = rintf(__fmul_rn(x[i], rcp));
-                    r = fminf(fmaxf(r, -127.0f), 127.0f);
-                    uint32_t b = (uint32_t)((int)r) & 0xffu;
-                    if (i < 4) lo |= b << (8 * i); else hi |= b << (8 * (i - 4));
-                }
-                if (live && !hole) {
-                    *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
-                    if (c == 0) *(uint16_t *)(pool + soff) = sh;
-                }
+        for (int u = 0; u < U; u++) {
+            const unsigned c = cc[u];
+            if (QMODE == 0) {
+                if (ok[u]) st_stream128(pool + poff[u] + (size_t)c * 16, val[u]);
             } else {
-                uint32_t lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
-                uint32_t hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
-                if (live && !hole) *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
+                float x[8];
+                unpack8(val[u], src_dtype, x);
+                if (QMODE == 1) {
+                    // row absmax over the rc lanes that hold this row (rc is a power
+                    // of two <= 64 and rows never straddle a wave)
+                    float amax = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(x[i]));
+                    for (unsigned off = rc >> 1; off > 0; off >>= 1)
+                        amax = fmaxf(amax, __shfl_xor(amax, (int)off));
+                    float s32 = __fdiv_rn(amax, 127.0f);
+                    uint16_t sh = __half_as_ushort(__float2half_rn(s32));
+                    if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
+                    float sf = f16_bits_to_f(sh);
+                    float rcp = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
+                    uint32_t lo = 0, hi = 0;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        float r = rintf(__fmul_rn(x[i], rcp));
+                        r = fminf(fmaxf(r, -127.0f), 127.0f);
+                        uint32_t b = (uint32_t)((int)r) & 0xffu;
+                        if (i < 4) lo |= b << (8 * i); else hi |= b << (8 * (i - 4));
+                    }
+                    if (ok[u]) {
+                        *(uint2 *)(pool + poff[u] + (size_t)c * 8) = make_uint2(lo, hi);
+                        if (c == 0) *(uint16_t *)(pool + soff[u]) = sh;
+                    }
+                } else {
+                    uint32_t lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
+                    uint32_t hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
+                    if (ok[u]) *(uint2 *)(pool + poff[u] + (size_t)c * 8) = make_uint2(lo, hi);
+                }
             }
         }
     }
