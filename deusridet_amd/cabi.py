@@ -82,6 +82,17 @@ SIGNATURES = {
                                                  _i32, _vp, _sz, _vp]),
     "drk_prefill_workspace_bytes": (_sz, [_LP, _i32, _i32]),
     "drk_paged_prefill_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
+    "drk_rope_table_fill": (_i32, [_vp, _i32, _i32, _f32, _vp]),
+    "drk_head_norm": (_i32, [_vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp]),
+    "drk_apply_rope": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _i32, _f32, _vp, _i32, _i32, _vp]),
+    "drk_split_q_gate": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _vp]),
+    "drk_sigmoid_gate": (_i32, [_vp, _vp, _vp, _sz, _i32, _sz, _i32, _vp]),
+    "drk_qk_norm_rope_append": (_i32, [_LP, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _f32,
+                                       _i32, _f32, _vp, _i32, _vp, _i32, _vp]),
+    "drk_paged_decode_attention_gated": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _f32, _i32,
+                                                _vp, _sz, _vp, _sz, _vp]),
+    "drk_paged_prefill_attention_gated": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz,
+                                                 _vp, _sz, _vp]),
     "drk_importance_update": (_i32, [_vp, _vp, _i32, _f32, _vp]),
 }
 

@@ -1,0 +1,96 @@
+// drk_codec.hpp -- what the append-side kernels share: byte offsets of page rows and
+// scales, the int8 / fp8 codecs, and the store of one 16-byte source chunk into a page.
+#pragma once
+#include "drk_common.hpp"
+
+namespace drk {
+
+__device__ __forceinline__ size_t row_off(const Lay &a, int layer, int blk, int kv, int h, int p)
+{
+    return lay_block_base(a, layer, blk) + (size_t)kv * a.kv_plane + (size_t)h * a.head_stride +
+           (size_t)p * a.row_bytes;
+}
+__device__ __forceinline__ size_t scale_off(const Lay &a, int layer, int blk, int kv, int h, int p)
+{
+    return lay_block_base(a, layer, blk) + 2 * (size_t)a.kv_plane + (size_t)kv * a.scale_plane +
+           ((size_t)h * a.bs + p) * 2;
+}
+
+struct Div {            // divisor with a power-of-two fast path
+    unsigned d;
+    int shift;
+};
+static inline Div mk_div(unsigned d) { return Div{d, ilog2_exact(d)}; }
+__device__ __forceinline__ unsigned dv(unsigned x, Div v) { return udiv(x, v.d, v.shift); }
+
+__device__ __forceinline__ void unpack8(const uint4 &v, int src_dtype, float *x)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        x[2 * i] = elem16_to_f((uint16_t)(w[i] & 0xffffu), src_dtype);
+        x[2 * i + 1] = elem16_to_f((uint16_t)(w[i] >> 16), src_dtype);
+    }
+}
+
+// E4M3FN code of x: round-half-even, |x| >= 448 and +-inf saturate to +-448,
+// NaN stays NaN.  The clamp runs before the hardware conversion so that the
+// conversion never sees an out-of-range input.
+__device__ __forceinline__ uint32_t fp8_pair(float x0, float x1)
+{
+    x0 = (x0 != x0) ? x0 : fminf(fmaxf(x0, -448.0f), 448.0f);
+    x1 = (x1 != x1) ? x1 : fminf(fmaxf(x1, -448.0f), 448.0f);
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(x0, x1, 0, false) & 0xffffu;
+#else
+    (void)x0; (void)x1;
+    return 0;
+#endif
+}
+
+// Store one source chunk (8 elements of type src_dtype, `val`) into the page row at byte
+// offset poff as chunk c of its row.  rc = chunks per row; the rc lanes that hold one row
+// are consecutive lanes of one wave (rc is a power of two <= 64), and every lane of the
+// wave must call this (the int8 row maximum is a lane exchange); ok = this lane stores.
+// QMODE 0: copy.  1: int8 codes + fp16 scale per row (soff).  2: fp8 e4m3 codes.
+template <int QMODE>
+__device__ __forceinline__ void store_page_chunk(uint8_t *__restrict__ pool, size_t poff, size_t soff, unsigned c,
+                                                 unsigned rc, const uint4 &val, int src_dtype, bool ok)
+{
+    if (QMODE == 0) {
+        if (ok) st_stream128(pool + poff + (size_t)c * 16, val);
+    } else {
+        float x[8];
+        unpack8(val, src_dtype, x);
+        if (QMODE == 1) {
+            float amax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(x[i]));
+            for (unsigned off = rc >> 1; off > 0; off >>= 1)
+                amax = fmaxf(amax, __shfl_xor(amax, (int)off));
+            float s32 = __fdiv_rn(amax, 127.0f);
+            uint16_t sh = __half_as_ushort(__float2half_rn(s32));
+            if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
+            float sf = f16_bits_to_f(sh);
+            float rcp = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float r = rintf(__fmul_rn(x[i], rcp));
+                r = fminf(fmaxf(r, -127.0f), 127.0f);
+                uint32_t b = (uint32_t)((int)r) & 0xffu;
+                if (i < 4) lo |= b << (8 * i); else hi |= b << (8 * (i - 4));
+            }
+            if (ok) {
+                *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
+                if (c == 0) *(uint16_t *)(pool + soff) = sh;
+            }
+        } else {
+            uint32_t lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
+            uint32_t hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
+            if (ok) *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
+        }
+    }
+}
+
+} // namespace drk

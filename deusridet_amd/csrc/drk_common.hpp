@@ -59,7 +59,11 @@ extern int g_force_portable;
 int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                   int table_stride, const int32_t *d_seq_lens, int seq_len_host, int causal_base, int B,
                   int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
-                  void *workspace, size_t workspace_bytes, void *stream);
+                  void *workspace, size_t workspace_bytes, void *stream, const void *gate = nullptr,
+                  size_t gate_stride = 0);
+// out[row][d] *= sigmoid(gate[row * gate_stride + d]), rows of D elements (drk_layer.hip)
+int launch_sigmoid_gate(const void *x, const void *gate, void *out, size_t rows, int D, size_t gate_stride_elems,
+                        int dtype, hipStream_t st);
 
 // persistent stream-K decode (drk_decode_stream.hip)
 extern int g_stream_wgs;
@@ -70,7 +74,8 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
                          float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
                          int start_tile = 0, const float *pre_o = nullptr, const float *pre_m = nullptr,
-                         const float *pre_l = nullptr, int pre_splits = 0);
+                         const float *pre_l = nullptr, int pre_splits = 0, const void *gate = nullptr,
+                         size_t gate_stride = 0);
 // shared-prefix pass on the matrix cores (drk_prefill.hip)
 void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
@@ -120,6 +125,23 @@ __device__ __forceinline__ uint16_t f_to_bf16_bits(float f)
 __device__ __forceinline__ uint16_t f_to_elem16(float f, int dtype)
 {
     return dtype == DRK_BF16 ? f_to_bf16_bits(f) : __half_as_ushort(__float2half_rn(f));
+}
+
+// Correctly rounded fp32 square root: the fp32 device routine is the hardware
+// approximation (about one unit in the last place); the fp64 one is exact to the last
+// bit, and rounding it to fp32 is the correctly rounded fp32 result (53 >= 2*24 + 2).
+__device__ __forceinline__ float sqrt_rn(float x) { return (float)sqrt((double)x); }
+
+// sigmoid_gate_kernel, layer.cu:406-431: v / (1 + exp(-g)), every operation rounded once
+__device__ __forceinline__ float sigmoid_gate_value(float v, float g)
+{
+    return __fdiv_rn(v, __fadd_rn(1.0f, expf(-g)));
+}
+// the attention epilogue with the gate folded in: the 16-bit attention output times
+// sigmoid(gate), rounded to 16 bits again -- the two roundings the separate kernels make
+__device__ __forceinline__ uint16_t gated_elem16(uint16_t x16, uint16_t g16, int dtype)
+{
+    return f_to_elem16(sigmoid_gate_value(elem16_to_f(x16, dtype), elem16_to_f(g16, dtype)), dtype);
 }
 
 // unsigned divide with a power-of-two fast path chosen on the host

@@ -478,12 +478,14 @@ static size_t workspace_need(const Lay &a, int B, int max_seq_len, int split)
 int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                          int table_stride, const int32_t *d_seq_lens, int seq_len_host, int causal_base,
                          int B, int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
-                         void *workspace, size_t workspace_bytes, void *stream)
+                         void *workspace, size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
 {
     Lay a;
     int rc = make_lay(g, &a);
     if (rc) return rc;
     if (!q || !pool || !tables || !out) return fail(DRK_ERR_INVALID, "decode: NULL pointer");
+    if (gate && (gate_stride < (size_t)a.D || (gate_stride % 8) || ((uintptr_t)gate % 16)))
+        return fail(DRK_ERR_INVALID, "decode: gate rows must be 16-byte aligned and at least head_dim apart");
     if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode: io_dtype must be F16 or BF16");
     if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
         return fail(DRK_ERR_INVALID, "decode: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
@@ -565,10 +567,12 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
     if (use_stream)
         return launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, seq_len_host, B, max_seq_len, out, layer,
-                                    scale, io_dtype, split_tokens, workspace, true, st);
+                                    scale, io_dtype, split_tokens, workspace, true, st, 0, nullptr, nullptr, nullptr, 0,
+                                    gate, gate_stride);
     hipLaunchKernelGGL(decode_merge_kernel, dim3(a.QH, B), dim3(a.D), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                        d_seq_lens, seq_len_host, causal_base, split, S, a.D, a.QH, io_dtype);
     DRK_LAUNCH_CHECK("decode_merge_kernel");
+    if (gate) return launch_sigmoid_gate(out, gate, out, (size_t)B * a.QH, a.D, gate_stride, io_dtype, st);
     return DRK_OK;
 }
 
@@ -737,6 +741,20 @@ int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, c
     if (!d_seq_lens) return fail(DRK_ERR_INVALID, "decode: d_seq_lens is NULL");
     return launch_decode(g, q, pool, d_tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
                          io_dtype, split_tokens, workspace, workspace_bytes, stream);
+}
+
+// steps 6 + 7 of full_attention_forward_paged (paged_attention.cu:362-370) in one call:
+// out = attention * sigmoid(gate); gate rows [B * num_q_heads] are gate_stride elements apart
+int drk_paged_decode_attention_gated(const drk_kv_layout *g, const void *q, const void *pool,
+                                     const int32_t *d_tables, int table_stride, const int32_t *d_seq_lens,
+                                     int B, int max_seq_len, void *out, int layer, float scale, int io_dtype,
+                                     const void *gate, size_t gate_stride, void *workspace,
+                                     size_t workspace_bytes, void *stream)
+{
+    if (!d_seq_lens) return fail(DRK_ERR_INVALID, "decode: d_seq_lens is NULL");
+    if (!gate) return fail(DRK_ERR_INVALID, "decode: gate is NULL");
+    return launch_decode(g, q, pool, d_tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
+                         io_dtype, 0, workspace, workspace_bytes, stream, gate, gate_stride);
 }
 
 } // extern "C"

@@ -568,7 +568,8 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
                                                            int KVH, int QH, int unit_tiles, int grid_wgs, int Pmax,
                                                            int io_dtype, int start_tile, const float *__restrict__ pre_o,
                                                            const float *__restrict__ pre_m, const float *__restrict__ pre_l,
-                                                           int pre_splits)
+                                                           int pre_splits, const uint16_t *__restrict__ gate,
+                                                           size_t gate_stride)
 {
     __shared__ float2 red[4][64];
     const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * 2;
@@ -625,10 +626,25 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
     L = s_wave_sum(L);
     red[wv][lane] = acc;
     __syncthreads();
-    if (wv == 0 && L > 0.0f) {
-        const float2 a1 = red[1][lane], a2 = red[2][lane], a3 = red[3][lane];
-        const float x = ((acc.x + a1.x) + (a2.x + a3.x)) / L, y = ((acc.y + a1.y) + (a2.y + a3.y)) / L;
-        *(uint32_t *)(out + ((size_t)b * QH + h) * 128 + d) = (uint32_t)f_to_elem16(x, io_dtype) | ((uint32_t)f_to_elem16(y, io_dtype) << 16);
+    if (wv == 0) {
+        // with a gate the row is always rewritten: the reference gates whatever the attention
+        // kernel left in out, also when no token took part (paged_attention.cu:266, 368-370)
+        uint32_t *dst = (uint32_t *)(out + ((size_t)b * QH + h) * 128 + d);
+        uint32_t packed;
+        if (L > 0.0f) {
+            const float2 a1 = red[1][lane], a2 = red[2][lane], a3 = red[3][lane];
+            const float x = ((acc.x + a1.x) + (a2.x + a3.x)) / L, y = ((acc.y + a1.y) + (a2.y + a3.y)) / L;
+            packed = (uint32_t)f_to_elem16(x, io_dtype) | ((uint32_t)f_to_elem16(y, io_dtype) << 16);
+        } else {
+            if (!gate) return;
+            packed = *dst;
+        }
+        if (gate) {
+            const uint32_t g2 = *(const uint32_t *)(gate + ((size_t)b * QH + h) * gate_stride + d);
+            packed = (uint32_t)gated_elem16((uint16_t)(packed & 0xffffu), (uint16_t)(g2 & 0xffffu), io_dtype) |
+                     ((uint32_t)gated_elem16((uint16_t)(packed >> 16), (uint16_t)(g2 >> 16), io_dtype) << 16);
+        }
+        *dst = packed;
     }
 }
 
@@ -667,7 +683,8 @@ size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tok
 int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
                          float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
-                         int start_tile, const float *pre_o, const float *pre_m, const float *pre_l, int pre_splits)
+                         int start_tile, const float *pre_o, const float *pre_m, const float *pre_l, int pre_splits,
+                         const void *gate, size_t gate_stride)
 {
     int grid, U, Pmax;
     stream_shape(a, B, max_seq_len, split_tokens, &grid, &U, &Pmax);
@@ -695,7 +712,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
     } else {
         hipLaunchKernelGGL(stream_merge_kernel, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                            d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
-                           pre_l, pre_splits);
+                           pre_l, pre_splits, (const uint16_t *)gate, gate_stride);
         DRK_LAUNCH_CHECK("stream_merge_kernel");
     }
     return DRK_OK;

@@ -92,6 +92,9 @@ struct PrefillArgs {
     const int32_t *seq_lens;      // [M] on the device
     int shared, chunk_tiles, nsplits;
     float *part_o, *part_m, *part_l;
+    // optional epilogue: out *= sigmoid(gate), gate rows gate_stride elements apart
+    const uint16_t *gate;
+    size_t gate_stride;
 };
 
 struct PfGroup {
@@ -318,16 +321,29 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
                 A.part_l[pi] = l_tot;
             }
         }
-    } else if (row_live && l_tot > 0.0f) {
-        const float inv = 1.0f / l_tot;
+    } else if (row_live && (l_tot > 0.0f || A.gate)) {
+        // with a gate the row is always rewritten: the reference gates whatever the attention
+        // kernel left in out, also when no token took part (paged_attention.cu:551, 633-634)
+        const bool have = l_tot > 0.0f;
+        const float inv = have ? 1.0f / l_tot : 0.0f;
         uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * 256;
+        const uint16_t *grow = A.gate ? A.gate + ((size_t)tq * A.QH + head) * A.gate_stride : nullptr;
+        constexpr int IO = DT;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int b4 = 0; b4 < 4; b4++) {
                 const int d0 = dt * 32 + 8 * b4 + 4 * g;
-                uint2 v = make_uint2(pack2<DT>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
-                                     pack2<DT>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv));
+                uint2 v = have ? make_uint2(pack2<DT>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
+                                            pack2<DT>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv))
+                               : *(const uint2 *)(orow + d0 * 2);
+                if (grow) {
+                    const uint2 gv = *(const uint2 *)(grow + d0);
+                    v.x = (uint32_t)gated_elem16((uint16_t)(v.x & 0xffffu), (uint16_t)(gv.x & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.x >> 16), (uint16_t)(gv.x >> 16), IO) << 16);
+                    v.y = (uint32_t)gated_elem16((uint16_t)(v.y & 0xffffu), (uint16_t)(gv.y & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.y >> 16), (uint16_t)(gv.y >> 16), IO) << 16);
+                }
                 *(uint2 *)(orow + d0 * 2) = v;
             }
     }
@@ -365,6 +381,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.seq_lens = d_seq_lens; A.shared = shared;
     shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
     A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
+    A.gate = nullptr; A.gate_stride = 0;
     dim3 grid(((B + 31) / 32) * a.KVH, 1, A.nsplits);
     if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, true>), grid, dim3(256), 0, st, A);
     else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, true>), grid, dim3(256), 0, st, A);
@@ -392,10 +409,9 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 // workspace).  Any other geometry or storage type: row t of the chunk runs as one
 // causal "branch" of the decode kernels -- the reference's algorithm verbatim
 // (paged_attention.cu:481, 506-549) -- and needs the workspace.
-int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
-                                const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
-                                float scale, int io_dtype, void *workspace, size_t workspace_bytes,
-                                void *stream)
+static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
+                        void *out, int layer, int pos_start, int M, float scale, int io_dtype, void *workspace,
+                        size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
 {
     Lay a;
     int rc = make_lay(g, &a);
@@ -411,8 +427,10 @@ int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const voi
     const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && scale > 0.0f;
     if (!mfma)
         return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
-                             io_dtype, 0, workspace, workspace_bytes, stream);
+                             io_dtype, 0, workspace, workspace_bytes, stream, gate, gate_stride);
     if (a.KVH > 65535) return fail(DRK_ERR_INVALID, "prefill: more than 65535 kv heads");
+    if (gate && (gate_stride < (size_t)a.D || (gate_stride % 8) || ((uintptr_t)gate % 16)))
+        return fail(DRK_ERR_INVALID, "prefill: gate rows must be 16-byte aligned and at least head_dim apart");
     PrefillArgs A;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
     A.table = d_block_table;
@@ -424,10 +442,31 @@ int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const voi
     A.scale_log2e = scale * kLog2eP;
     dim3 grid(((M + 31) / 32) * a.KVH);
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
+    A.gate = (const uint16_t *)gate; A.gate_stride = gate_stride;
     if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
     else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
     DRK_LAUNCH_CHECK("prefill_mfma_kernel");
     return DRK_OK;
+}
+
+int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
+                                const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
+                                float scale, int io_dtype, void *workspace, size_t workspace_bytes,
+                                void *stream)
+{
+    return prefill_impl(g, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
+                        workspace_bytes, stream, nullptr, 0);
+}
+
+// steps 8 + 9 of full_attention_forward_paged_prefill (paged_attention.cu:621-634) in one launch
+int drk_paged_prefill_attention_gated(const drk_kv_layout *g, const void *q, const void *pool,
+                                      const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
+                                      float scale, int io_dtype, const void *gate, size_t gate_stride,
+                                      void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!gate) return fail(DRK_ERR_INVALID, "prefill: gate is NULL");
+    return prefill_impl(g, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
+                        workspace_bytes, stream, gate, gate_stride);
 }
 
 } // extern "C"

@@ -56,6 +56,17 @@ SIGNATURES = {
                                                       _f32, _vp]),
     "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32]),
+    "drkh_set_rope": (_i32, [_i32, _f32, _f32]),
+    "drkh_sigmoid_gate": (None, [_vp, _vp, _vp, _i32, _vp]),
+    "drkh_apply_rope": (None, [_vp, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _vp]),
+    "drkh_head_norm": (None, [_vp, _vp, _vp, _i32, _i32, _f32, _vp]),
+    "drkh_paged_qk_norm_rope_write_batch": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
+                                                   _vp, _i32, _vp]),
+    "drkh_paged_qk_norm_rope_write_branches": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32,
+                                                      _i32, _vp, _i32, _vp]),
+    "drkh_paged_gqa_decode_attention_gated_branches": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _vp, _i32,
+                                                              _i32, _i32, _f32, _vp]),
+    "drkh_paged_prefill_attention_gated": (None, [_vp, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_invoke_extract_kv_from_pages": (None, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     "drkh_invoke_inject_kv_to_pages": (None, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
 }

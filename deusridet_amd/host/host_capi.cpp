@@ -3,6 +3,7 @@
 #include "drk_host.h"
 
 #include "../machina/paged_attention.h"
+#include "../machina/layer.h"
 #include "../memoria/cache_kernels.h"
 #include "../memoria/cache_manager.h"
 
@@ -151,6 +152,58 @@ void drkh_paged_prefill_attention(const void *Q, void *kv_pool, const int32_t *d
 {
     paged_prefill_attention(CH(Q), H(kv_pool), d_block_table, H(out), fa_layer_idx, pos_start, M, max_phys_blocks,
                             block_size, scale, ST(stream));
+}
+int drkh_set_rope(int rotary_dim, float theta, float rms_eps) { return ModelConfig::set_rope(rotary_dim, theta, rms_eps) ? 1 : 0; }
+void drkh_sigmoid_gate(const void *x, const void *gate, void *out, int n, void *stream)
+{
+    sigmoid_gate(CH(x), CH(gate), H(out), n, (hipStream_t)stream);
+}
+void drkh_apply_rope(void *q, void *k, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
+                     const int32_t *d_pos, float theta, void *stream)
+{
+    apply_rope(H(q), H(k), num_heads, num_kv_heads, head_dim, rotary_dim, d_pos, theta, (hipStream_t)stream);
+}
+void drkh_head_norm(const void *x, const void *weight, void *out, int num_heads, int head_dim, float eps,
+                    void *stream)
+{
+    head_norm(CH(x), CH(weight), H(out), num_heads, head_dim, eps, (hipStream_t)stream);
+}
+void drkh_paged_qk_norm_rope_write_batch(const void *qg, const void *k, const void *v, const void *q_norm,
+                                         const void *k_norm, void *q_out, void *kv_pool,
+                                         const int32_t *d_block_table, int fa_layer_idx, int pos_start, int M,
+                                         int max_phys_blocks, int block_size, const float *d_rope_table,
+                                         int table_positions, void *stream)
+{
+    paged_qk_norm_rope_write_batch(CH(qg), CH(k), CH(v), CH(q_norm), CH(k_norm), H(q_out), H(kv_pool), d_block_table,
+                                   fa_layer_idx, pos_start, M, max_phys_blocks, block_size, d_rope_table,
+                                   table_positions, (hipStream_t)stream);
+}
+void drkh_paged_qk_norm_rope_write_branches(const void *qg, const void *k, const void *v, const void *q_norm,
+                                            const void *k_norm, void *q_out, void *kv_pool, const int32_t *d_tables,
+                                            int table_stride, const int32_t *d_pos, int B, int fa_layer_idx,
+                                            int max_phys_blocks, int block_size, const float *d_rope_table,
+                                            int table_positions, void *stream)
+{
+    paged_qk_norm_rope_write_branches(CH(qg), CH(k), CH(v), CH(q_norm), CH(k_norm), H(q_out), H(kv_pool), d_tables,
+                                      table_stride, d_pos, B, fa_layer_idx, max_phys_blocks, block_size, d_rope_table,
+                                      table_positions, (hipStream_t)stream);
+}
+void drkh_paged_gqa_decode_attention_gated_branches(const void *Q, void *kv_pool, const int32_t *d_tables,
+                                                    int table_stride, const int32_t *d_seq_lens, int B,
+                                                    int max_seq_len, const void *gate, int gate_stride, void *out,
+                                                    int fa_layer_idx, int max_phys_blocks, int block_size,
+                                                    float scale, void *stream)
+{
+    paged_gqa_decode_attention_gated_branches(CH(Q), H(kv_pool), d_tables, table_stride, d_seq_lens, B, max_seq_len,
+                                              CH(gate), gate_stride, H(out), fa_layer_idx, max_phys_blocks,
+                                              block_size, scale, (hipStream_t)stream);
+}
+void drkh_paged_prefill_attention_gated(const void *Q, void *kv_pool, const int32_t *d_block_table, const void *gate,
+                                        int gate_stride, void *out, int fa_layer_idx, int pos_start, int M,
+                                        int max_phys_blocks, int block_size, float scale, void *stream)
+{
+    paged_prefill_attention_gated(CH(Q), H(kv_pool), d_block_table, CH(gate), gate_stride, H(out), fa_layer_idx,
+                                  pos_start, M, max_phys_blocks, block_size, scale, (hipStream_t)stream);
 }
 int drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size)
 {

@@ -15,6 +15,9 @@ struct ModelConfig {
     static int HEAD_DIM;         // model.h:41
     static int NUM_KV_GROUPS;    // model.h:42, ATTN_HEADS / KV_HEADS
     static int NUM_FA_LAYERS;    // model.h:73
+    static float RMS_EPS;        // model.h:36 (default 1e-6)
+    static float ROPE_THETA;     // model.h:49 (default 1e7)
+    static int ROTARY_DIM;       // model.h:51, HEAD_DIM * partial_rotary_factor (default HEAD_DIM / 4)
     // Not in the reference (its cache is fp16 only): storage type of the pool and
     // element type of Q / out / append sources, DRK_* from drk_kv.h.
     static int KV_DTYPE;         // DRK_F16 (default), DRK_BF16, DRK_INT8, DRK_FP8_E4M3
@@ -23,6 +26,9 @@ struct ModelConfig {
     // Returns false (and changes nothing) when the numbers are inconsistent.
     static bool set_attention_geometry(int num_fa_layers, int num_attn_heads, int num_kv_heads, int head_dim,
                                        int kv_dtype = DRK_F16, int io_dtype = -1);
+
+    // rotary_dim must be 16 * 2^k and at most HEAD_DIM; false (nothing changed) otherwise.
+    static bool set_rope(int rotary_dim, float theta, float rms_eps);
 
     // The C-ABI layout for a pool of max_phys_blocks blocks of block_size tokens.
     static drk_kv_layout layout(int max_phys_blocks, int block_size);

@@ -142,4 +142,77 @@ void paged_prefill_attention(const __half* Q, __half* kv_pool, const int* d_bloc
         LOG_ERROR("Machina", "paged_prefill_attention: %s", drk_last_error());
 }
 
+namespace {
+void fused_write(const char* who, const __half* qg, const __half* k, const __half* v, const __half* q_norm,
+                 const __half* k_norm, __half* q_out, __half* kv_pool, const int* d_tables, int table_stride,
+                 const int* d_pos, int pos_start, int T, int fa_layer_idx, int max_phys_blocks, int block_size,
+                 const float* d_rope_table, int table_positions, hipStream_t stream)
+{
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    if (drk_qk_norm_rope_append(&g, kv_pool, d_tables, table_stride, d_pos, pos_start, T, fa_layer_idx, qg, k, v, q_norm,
+                                k_norm, ModelConfig::RMS_EPS, ModelConfig::ROTARY_DIM, ModelConfig::ROPE_THETA,
+                                d_rope_table, table_positions, q_out, ModelConfig::IO_DTYPE, stream) != DRK_OK)
+        LOG_ERROR("Machina", "%s: %s", who, drk_last_error());
+}
+} // namespace
+
+void paged_qk_norm_rope_write(const __half* qg, const __half* k, const __half* v, const __half* q_norm,
+                              const __half* k_norm, __half* q_out, __half* kv_pool, const int* d_block_table,
+                              int fa_layer_idx, const int* d_pos, int max_phys_blocks, int block_size,
+                              const float* d_rope_table, int table_positions, hipStream_t stream)
+{
+    fused_write("paged_qk_norm_rope_write", qg, k, v, q_norm, k_norm, q_out, kv_pool, d_block_table, 0, d_pos, 0, 1,
+                fa_layer_idx, max_phys_blocks, block_size, d_rope_table, table_positions, stream);
+}
+
+void paged_qk_norm_rope_write_batch(const __half* qg, const __half* k, const __half* v, const __half* q_norm,
+                                    const __half* k_norm, __half* q_out, __half* kv_pool, const int* d_block_table,
+                                    int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
+                                    const float* d_rope_table, int table_positions, hipStream_t stream)
+{
+    fused_write("paged_qk_norm_rope_write_batch", qg, k, v, q_norm, k_norm, q_out, kv_pool, d_block_table, 0, nullptr,
+                pos_start, M, fa_layer_idx, max_phys_blocks, block_size, d_rope_table, table_positions, stream);
+}
+
+void paged_qk_norm_rope_write_branches(const __half* qg, const __half* k, const __half* v, const __half* q_norm,
+                                       const __half* k_norm, __half* q_out, __half* kv_pool, const int* d_tables,
+                                       int table_stride, const int* d_pos, int B, int fa_layer_idx,
+                                       int max_phys_blocks, int block_size, const float* d_rope_table,
+                                       int table_positions, hipStream_t stream)
+{
+    fused_write("paged_qk_norm_rope_write_branches", qg, k, v, q_norm, k_norm, q_out, kv_pool, d_tables, table_stride,
+                d_pos, 0, B, fa_layer_idx, max_phys_blocks, block_size, d_rope_table, table_positions, stream);
+}
+
+void paged_gqa_decode_attention_gated_branches(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                               const int* d_seq_lens, int B, int max_seq_len, const __half* gate,
+                                               int gate_stride, __half* out, int fa_layer_idx, int max_phys_blocks,
+                                               int block_size, float scale, hipStream_t stream)
+{
+    if (B <= 0 || max_seq_len <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    size_t need = drk_decode_workspace_bytes(&g, B, max_seq_len);
+    void* ws = workspace(need);
+    if (!ws) return;
+    if (drk_paged_decode_attention_gated(&g, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, out,
+                                         fa_layer_idx, scale, ModelConfig::IO_DTYPE, gate, (size_t)gate_stride, ws,
+                                         g_ws_bytes, stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_gqa_decode_attention_gated_branches: %s", drk_last_error());
+}
+
+void paged_prefill_attention_gated(const __half* Q, __half* kv_pool, const int* d_block_table, const __half* gate,
+                                   int gate_stride, __half* out, int fa_layer_idx, int pos_start, int M,
+                                   int max_phys_blocks, int block_size, float scale, hipStream_t stream)
+{
+    if (M <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    size_t need = drk_prefill_workspace_bytes(&g, pos_start, M);
+    void* ws = workspace(need);
+    if (!ws) return;
+    if (drk_paged_prefill_attention_gated(&g, Q, kv_pool, d_block_table, out, fa_layer_idx, pos_start, M, scale,
+                                          ModelConfig::IO_DTYPE, gate, (size_t)gate_stride, ws, g_ws_bytes,
+                                          stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_prefill_attention_gated: %s", drk_last_error());
+}
+
 } // namespace deusridet

@@ -64,6 +64,39 @@ void paged_gqa_decode_attention_shared(const __half* Q, __half* kv_pool, const i
                                        __half* out, int fa_layer_idx, int max_phys_blocks, int block_size,
                                        float scale, hipStream_t stream = 0);
 
+// ---- fused layer steps (not in the reference as single functions) ---------------
+// Steps 1b-5 of full_attention_forward_paged (paged_attention.cu:331-360) in one launch:
+// qg is the interleaved Q|gate projection [T, NUM_ATTN_HEADS, 2*HEAD_DIM], k / v the K and
+// V projections [T, NUM_KV_HEADS, HEAD_DIM]; q_out [T, NUM_ATTN_HEADS, HEAD_DIM] receives
+// rope(norm(q)); rope(norm(k)) and v go into the pages.  RMS_EPS, ROTARY_DIM and ROPE_THETA
+// come from ModelConfig.  d_rope_table (float [table_positions][ROTARY_DIM/2][2], see
+// drk_rope_table_fill) may be null.  The gate halves stay in qg: pass qg + HEAD_DIM with
+// stride 2*HEAD_DIM to the gated attention calls below.
+void paged_qk_norm_rope_write(const __half* qg, const __half* k, const __half* v, const __half* q_norm,
+                              const __half* k_norm, __half* q_out, __half* kv_pool, const int* d_block_table,
+                              int fa_layer_idx, const int* d_pos, int max_phys_blocks, int block_size,
+                              const float* d_rope_table = nullptr, int table_positions = 0, hipStream_t stream = 0);
+void paged_qk_norm_rope_write_batch(const __half* qg, const __half* k, const __half* v, const __half* q_norm,
+                                    const __half* k_norm, __half* q_out, __half* kv_pool, const int* d_block_table,
+                                    int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
+                                    const float* d_rope_table = nullptr, int table_positions = 0,
+                                    hipStream_t stream = 0);
+void paged_qk_norm_rope_write_branches(const __half* qg, const __half* k, const __half* v, const __half* q_norm,
+                                       const __half* k_norm, __half* q_out, __half* kv_pool, const int* d_tables,
+                                       int table_stride, const int* d_pos, int B, int fa_layer_idx,
+                                       int max_phys_blocks, int block_size, const float* d_rope_table = nullptr,
+                                       int table_positions = 0, hipStream_t stream = 0);
+
+// Attention with the sigmoid gate (paged_attention.cu:368-370, 633-634) folded into the
+// epilogue; gate rows are gate_stride elements apart.
+void paged_gqa_decode_attention_gated_branches(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                               const int* d_seq_lens, int B, int max_seq_len, const __half* gate,
+                                               int gate_stride, __half* out, int fa_layer_idx, int max_phys_blocks,
+                                               int block_size, float scale, hipStream_t stream = 0);
+void paged_prefill_attention_gated(const __half* Q, __half* kv_pool, const int* d_block_table, const __half* gate,
+                                   int gate_stride, __half* out, int fa_layer_idx, int pos_start, int M,
+                                   int max_phys_blocks, int block_size, float scale, hipStream_t stream = 0);
+
 // The attention calls keep split-K partials in a device workspace that this
 // library owns and grows on demand (device allocation = implicit sync).  Call
 // this once up front with the largest shapes to keep the steady state free of

@@ -10,6 +10,9 @@ int ModelConfig::NUM_KV_HEADS = 4;
 int ModelConfig::HEAD_DIM = 256;
 int ModelConfig::NUM_KV_GROUPS = 6;
 int ModelConfig::NUM_FA_LAYERS = 16;
+float ModelConfig::RMS_EPS = 1e-6f;
+float ModelConfig::ROPE_THETA = 1.0e7f;
+int ModelConfig::ROTARY_DIM = 64;
 int ModelConfig::KV_DTYPE = DRK_F16;
 int ModelConfig::IO_DTYPE = DRK_F16;
 
@@ -29,6 +32,20 @@ bool ModelConfig::set_attention_geometry(int num_fa_layers, int num_attn_heads, 
     NUM_KV_GROUPS = num_attn_heads / num_kv_heads;
     KV_DTYPE = kv_dtype;
     IO_DTYPE = io_dtype;
+    return true;
+}
+
+bool ModelConfig::set_rope(int rotary_dim, float theta, float rms_eps)
+{
+    const int q = rotary_dim / 16;
+    if (rotary_dim < 16 || rotary_dim > HEAD_DIM || (rotary_dim % 16) || (q & (q - 1)) || !(theta > 0.0f) || !(rms_eps >= 0.0f)) {
+        LOG_ERROR("Machina", "ModelConfig: rotary_dim %d / theta %g / eps %g not usable with head_dim %d", rotary_dim,
+                  (double)theta, (double)rms_eps, HEAD_DIM);
+        return false;
+    }
+    ROTARY_DIM = rotary_dim;
+    ROPE_THETA = theta;
+    RMS_EPS = rms_eps;
     return true;
 }
 

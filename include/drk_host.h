@@ -95,6 +95,31 @@ void drkh_paged_gqa_decode_attention_shared(const void *Q, void *kv_pool, const 
 void drkh_paged_prefill_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
                                   int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
                                   float scale, void *stream);
+/* src/machina/layer.h:77-79, 124-140 and the fused forms in machina/paged_attention.h */
+int  drkh_set_rope(int rotary_dim, float theta, float rms_eps);
+void drkh_sigmoid_gate(const void *x, const void *gate, void *out, int n, void *stream);
+void drkh_apply_rope(void *q, void *k, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
+                     const int32_t *d_pos, float theta, void *stream);
+void drkh_head_norm(const void *x, const void *weight, void *out, int num_heads, int head_dim, float eps,
+                    void *stream);
+void drkh_paged_qk_norm_rope_write_batch(const void *qg, const void *k, const void *v, const void *q_norm,
+                                         const void *k_norm, void *q_out, void *kv_pool,
+                                         const int32_t *d_block_table, int fa_layer_idx, int pos_start, int M,
+                                         int max_phys_blocks, int block_size, const float *d_rope_table,
+                                         int table_positions, void *stream);
+void drkh_paged_qk_norm_rope_write_branches(const void *qg, const void *k, const void *v, const void *q_norm,
+                                            const void *k_norm, void *q_out, void *kv_pool, const int32_t *d_tables,
+                                            int table_stride, const int32_t *d_pos, int B, int fa_layer_idx,
+                                            int max_phys_blocks, int block_size, const float *d_rope_table,
+                                            int table_positions, void *stream);
+void drkh_paged_gqa_decode_attention_gated_branches(const void *Q, void *kv_pool, const int32_t *d_tables,
+                                                    int table_stride, const int32_t *d_seq_lens, int B,
+                                                    int max_seq_len, const void *gate, int gate_stride, void *out,
+                                                    int fa_layer_idx, int max_phys_blocks, int block_size,
+                                                    float scale, void *stream);
+void drkh_paged_prefill_attention_gated(const void *Q, void *kv_pool, const int32_t *d_block_table, const void *gate,
+                                        int gate_stride, void *out, int fa_layer_idx, int pos_start, int M,
+                                        int max_phys_blocks, int block_size, float scale, void *stream);
 int  drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
 void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,
                                        int num_tokens, int num_layers, int num_kv_heads, int head_dim,

@@ -223,6 +223,69 @@ int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const voi
                                 int pos_start, int M, float scale, int io_dtype,
                                 void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- the layer steps either side of the page kernels --------------------- */
+/* full_attention_forward_paged / _paged_prefill, paged_attention.cu:314-376, 563-638:
+ * split of the interleaved Q|gate projection, per-head RMSNorm, partial half-half
+ * RoPE, [page write, attention], sigmoid gate.  All tensors hold 16-bit elements of
+ * type dtype (DRK_F16 / DRK_BF16); head_dim is a power of two in [8, 512];
+ * rotary_dim = 16 * 2^k <= head_dim.  Rows are heads of head_dim elements.
+ *
+ * A rope table is float [table_positions][rotary_dim/2][2] = (cos, sin) of
+ * pos * theta^(-2 pair / rotary_dim), formed in fp32 as rope_kernel does
+ * (layer_attention.cu:42-48).  Entry points that take one use it for positions inside
+ * it and evaluate the same expressions in the kernel for any other (or when it is NULL). */
+int drk_rope_table_fill(float *d_table, int n_pos, int rotary_dim, float theta, void *stream);
+/* head_norm, layer_attention.cu:86-135: out = (x * rsqrt(mean(x^2) + eps)) * weight per row */
+int drk_head_norm(const void *x, const void *weight, void *out, int num_rows, int head_dim,
+                  float eps, int dtype, void *stream);
+/* apply_rope, layer_attention.cu:32-79 (T = 1, position *d_pos) and
+ * paged_rope_batch_kernel, paged_attention.cu:412-451 (T tokens at pos_start + t): in place
+ * on q [T, num_q_heads, head_dim] and k [T, num_kv_heads, head_dim].  d_pos != NULL: one
+ * position per token (decode branches), read on the device. */
+int drk_apply_rope(void *q, void *k, int T, int num_q_heads, int num_kv_heads, int head_dim,
+                   int rotary_dim, const int32_t *d_pos, int pos_start, float theta,
+                   const float *d_rope_table, int table_positions, int dtype, void *stream);
+/* paged_split_q_gate[_batch_kernel], paged_attention.cu:288-298, 386-404:
+ * qg [T, num_heads, 2 * head_dim] -> q, gate [T, num_heads, head_dim] */
+int drk_split_q_gate(const void *qg, void *q, void *gate, int T, int num_heads, int head_dim,
+                     void *stream);
+/* sigmoid_gate, layer.cu:406-439: out = x * sigmoid(gate); x, out [num_rows, head_dim]
+ * (may alias), gate rows gate_stride elements apart (head_dim when gate is its own tensor,
+ * 2 * head_dim when it still sits in the Q|gate projection: pass qg + head_dim) */
+int drk_sigmoid_gate(const void *x, const void *gate, void *out, size_t num_rows, int head_dim,
+                     size_t gate_stride, int dtype, void *stream);
+/* Steps 1b-5 of full_attention_forward_paged (paged_attention.cu:331-360; batch form
+ * 589-619) in ONE launch, no reference counterpart as a single function: reads the raw
+ * projections qg [T, QH, 2*D], k, v [T, KVH, D] and the norm weights [D]; writes
+ * q_out [T, QH, D] = rope(norm(q)); appends rope(norm(k)) and v into the pages of layer
+ * `layer` (quantising for int8 / fp8 pools exactly as drk_kv_append_* does).  The gate
+ * halves of qg are left where they are (see drk_sigmoid_gate / the _gated attention
+ * calls).  d_pos != NULL: token t is the new token of branch t at d_pos[t] with table row
+ * t (as drk_kv_append_branches); NULL: positions pos_start + t of one table (as
+ * drk_kv_append_batch).  Equals split + head_norm x2 + apply_rope + append bit for bit. */
+int drk_qk_norm_rope_append(const drk_kv_layout *g, void *pool, const int32_t *d_tables,
+                            int table_stride, const int32_t *d_pos, int pos_start, int T, int layer,
+                            const void *qg, const void *k, const void *v, const void *q_norm_w,
+                            const void *k_norm_w, float eps, int rotary_dim, float theta,
+                            const float *d_rope_table, int table_positions, void *q_out,
+                            int src_dtype, void *stream);
+/* Attention with the sigmoid gate folded into the epilogue (steps 6+7 / 8+9 of the
+ * wrappers above): out = f16(f16(attention) * sigmoid(gate)), the same two roundings the
+ * separate kernels make.  gate rows [B or M][num_q_heads] are gate_stride elements apart
+ * and 16-byte aligned.  As in the reference, a row no token took part in is gated too
+ * (out must then hold defined values). */
+int drk_paged_decode_attention_gated(const drk_kv_layout *g, const void *q, const void *pool,
+                                     const int32_t *d_tables, int table_stride,
+                                     const int32_t *d_seq_lens, int B, int max_seq_len, void *out,
+                                     int layer, float scale, int io_dtype, const void *gate,
+                                     size_t gate_stride, void *workspace, size_t workspace_bytes,
+                                     void *stream);
+int drk_paged_prefill_attention_gated(const drk_kv_layout *g, const void *q, const void *pool,
+                                      const int32_t *d_block_table, void *out, int layer,
+                                      int pos_start, int M, float scale, int io_dtype,
+                                      const void *gate, size_t gate_stride, void *workspace,
+                                      size_t workspace_bytes, void *stream);
+
 /* ---- importance scores -------------------------------------------------- */
 /* importance_update_kernel, importance_scorer.cu:27-36, 67-73 */
 int drk_importance_update(float *d_scores, const float *d_new_scores, int n, float decay,

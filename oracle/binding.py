@@ -52,6 +52,11 @@ def lib():
         "orc_extract": (None, [P, vp, vp, vp, vp, i32, i32, i32]),
         "orc_inject": (None, [P, vp, vp, vp, vp, i32, i32, i32]),
         "orc_copy_block": (None, [P, vp, i32, i32]),
+        "orc_split_q_gate": (None, [vp, vp, vp, i32, i32, i32]),
+        "orc_head_norm": (None, [vp, vp, vp, i32, i32, f32, i32]),
+        "orc_rope_table": (None, [vp, i32, i32, f32]),
+        "orc_apply_rope": (None, [vp, i32, i32, i32, i32, vp, vp, i32]),
+        "orc_sigmoid_gate": (None, [vp, vp, vp, sz, i32]),
         "orc_quant_row_int8": (None, [vp, i32, i32, vp, vp]),
         "orc_quant_row_fp8": (None, [vp, i32, i32, vp]),
         "orc_decode_ref_order": (i32, [P, vp, vp, vp, vp, i32, i32, f32, i32]),
@@ -183,6 +188,48 @@ def quant_row_fp8(x, src_dtype):
     codes = np.empty(x.shape[0], dtype=np.uint8)
     lib().orc_quant_row_fp8(ptr(x), x.shape[0], src_dtype, ptr(codes))
     return codes
+
+
+def split_q_gate(qg, T, H, D):
+    """qg uint16 [T][H][2D] -> (q, gate), each [T][H][D]"""
+    qg = np.ascontiguousarray(qg, dtype=np.uint16)
+    q = np.empty((T, H, D), np.uint16)
+    gate = np.empty((T, H, D), np.uint16)
+    lib().orc_split_q_gate(ptr(qg), ptr(q), ptr(gate), T, H, D)
+    return q, gate
+
+
+def head_norm(x, w, eps, dtype):
+    """x uint16 [rows][D], w uint16 [D]"""
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    w = np.ascontiguousarray(w, dtype=np.uint16)
+    D = x.shape[-1]
+    out = np.empty_like(x)
+    lib().orc_head_norm(ptr(x), ptr(w), ptr(out), x.size // D, D, float(eps), dtype)
+    return out
+
+
+def rope_table(n_pos, rotary_dim, theta):
+    t = np.empty((n_pos, rotary_dim // 2, 2), np.float32)
+    lib().orc_rope_table(ptr(t), n_pos, rotary_dim, float(theta))
+    return t
+
+
+def apply_rope(x, pos, table, rotary_dim, dtype):
+    """x uint16 [T][H][D] (a rotated copy is returned), pos int32 [T]"""
+    x = np.array(x, dtype=np.uint16, order="C", copy=True)
+    pos = np.ascontiguousarray(pos, dtype=np.int32)
+    T, H, D = x.shape
+    lib().orc_apply_rope(ptr(x), T, H, D, rotary_dim, ptr(pos), ptr(table), dtype)
+    return x
+
+
+def sigmoid_gate(x, gate, dtype):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    gate = np.ascontiguousarray(gate, dtype=np.uint16)
+    out = np.empty_like(x)
+    lib().orc_sigmoid_gate(ptr(x), ptr(gate), ptr(out), x.size, dtype)
+    return out
 
 
 class CacheManager:

@@ -16,7 +16,11 @@
  *   - int8 codec: numpy restatement (np.rint is round-half-even) + enumerated ties;
  *   - fp8 codec: torch.float8_e4m3fn casts for |x|<=448, saturation by spec;
  *   - branches / refcount / COW: model-based check against a naive simulator in
- *     which every branch owns a private copy of its K/V.
+ *     which every branch owns a private copy of its K/V;
+ *   - head norm / RoPE / gate: fp64 numpy closed forms (x / sqrt(mean(x^2) + eps) * w,
+ *     plane rotation by pos * theta^(-2i/rd), x * logistic(g)) to one unit in the
+ *     last place of the 16-bit type, rotation by position 0 == identity, rotations
+ *     keep each pair's length.
  * Parity of the *reference decode kernel's exact fp16 output bits* (it is built
  * with --use_fast_math) is unpinned: the tolerance in the tests is against fp64.
  */
@@ -558,6 +562,97 @@ void orc_decode_branches(const orc_layout *g, const uint16_t *Q, const void *poo
             for (int d = 0; d < D; d++)
                 out[((size_t)b * g->QH + h) * D + d] = f_to_elem(o[d] / l, io_dtype);
         free(q);
+    }
+}
+
+/* ======================================================================== */
+/* layer steps either side of the kernels                                   */
+/* ======================================================================== */
+
+/* paged_split_q_gate, paged_attention.cu:288-298 (batch form 386-404) */
+void orc_split_q_gate(const uint16_t *qg, uint16_t *q, uint16_t *gate, int T, int H, int D)
+{
+    for (int t = 0; t < T; t++)
+        for (int h = 0; h < H; h++)
+            for (int d = 0; d < D; d++) {
+                q[((size_t)t * H + h) * D + d] = qg[((size_t)t * H + h) * 2 * D + d];
+                gate[((size_t)t * H + h) * D + d] = qg[((size_t)t * H + h) * 2 * D + D + d];
+            }
+}
+
+/* head_norm_kernel, layer_attention.cu:86-127: sum of squares in fp32,
+ * inv_rms = rsqrt(ss / D + eps), out = fp16((x * inv_rms) * w).
+ * The reference's summation order is a property of its 128/256-thread launch and
+ * rsqrtf is an approximation under --use_fast_math; the order fixed here is the
+ * one the HIP kernels use so that both sides agree to the bit: D/8 partial sums
+ * of 8 consecutive elements each (fused multiply-adds), folded by an xor
+ * butterfly with strides D/16, ..., 2, 1; then 1 / sqrt(.) correctly rounded. */
+void orc_head_norm(const uint16_t *x, const uint16_t *w, uint16_t *out, int rows, int D, float eps, int dtype)
+{
+    const int nl = D / 8;
+    float part[64];
+    for (int r = 0; r < rows; r++) {
+        const uint16_t *xr = x + (size_t)r * D;
+        for (int l = 0; l < nl; l++) {
+            float s = 0.0f;
+            for (int i = 0; i < 8; i++) {
+                const float v = elem_to_f(xr[l * 8 + i], dtype);
+                s = fmaf(v, v, s);
+            }
+            part[l] = s;
+        }
+        for (int off = nl >> 1; off > 0; off >>= 1) {
+            float nxt[64];
+            for (int l = 0; l < nl; l++) nxt[l] = part[l] + part[l ^ off];
+            memcpy(part, nxt, sizeof(float) * (size_t)nl);
+        }
+        const float inv_rms = 1.0f / sqrtf(part[0] / (float)D + eps);
+        for (int d = 0; d < D; d++) {
+            const float v = elem_to_f(xr[d], dtype) * inv_rms;
+            out[(size_t)r * D + d] = f_to_elem(v * elem_to_f(w[d], dtype), dtype);
+        }
+    }
+}
+
+/* rope_kernel, layer_attention.cu:42-48: freq = 1 / powf(theta, 2 pair / rd),
+ * angle = pos * freq, all in fp32 */
+void orc_rope_table(float *table, int n_pos, int rotary_dim, float theta)
+{
+    const int np = rotary_dim / 2;
+    for (int pos = 0; pos < n_pos; pos++)
+        for (int pair = 0; pair < np; pair++) {
+            const float freq = 1.0f / powf(theta, (2.0f * (float)pair) / (float)rotary_dim);
+            const float angle = (float)pos * freq;
+            table[((size_t)pos * np + pair) * 2] = cosf(angle);
+            table[((size_t)pos * np + pair) * 2 + 1] = sinf(angle);
+        }
+}
+
+/* rope_kernel, layer_attention.cu:50-69 (half-half pairing (i, i + rd/2));
+ * nvcc contracts x0*c - x1*s and x1*c + x0*s into one product and one fused
+ * multiply-add each; the form fixed here rounds the second product first. */
+void orc_apply_rope(uint16_t *x, int T, int H, int D, int rotary_dim, const int32_t *pos, const float *table,
+                    int dtype)
+{
+    const int np = rotary_dim / 2;
+    for (int t = 0; t < T; t++)
+        for (int h = 0; h < H; h++) {
+            uint16_t *row = x + ((size_t)t * H + h) * D;
+            for (int pair = 0; pair < np; pair++) {
+                const float c = table[((size_t)pos[t] * np + pair) * 2], s = table[((size_t)pos[t] * np + pair) * 2 + 1];
+                const float x0 = elem_to_f(row[pair], dtype), x1 = elem_to_f(row[pair + np], dtype);
+                row[pair] = f_to_elem(fmaf(x0, c, -(x1 * s)), dtype);
+                row[pair + np] = f_to_elem(fmaf(x1, c, x0 * s), dtype);
+            }
+        }
+}
+
+/* sigmoid_gate_kernel, layer.cu:406-431: v / (1 + exp(-g)) */
+void orc_sigmoid_gate(const uint16_t *x, const uint16_t *gate, uint16_t *out, size_t n, int dtype)
+{
+    for (size_t i = 0; i < n; i++) {
+        const float v = elem_to_f(x[i], dtype), g = elem_to_f(gate[i], dtype);
+        out[i] = f_to_elem(v / (1.0f + expf(-g)), dtype);
     }
 }
 

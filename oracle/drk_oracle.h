@@ -109,6 +109,26 @@ void orc_importance_update(float *scores, const float *new_scores, int n,
                            float decay);
 int  orc_least_important(const float *scores, const int *ids, int n);
 
+/* ---- the layer steps either side of the kernels --------------------------
+ * (full_attention_forward_paged, paged_attention.cu:314-376: split Q|gate,
+ * per-head RMSNorm, partial RoPE, [write, attend], sigmoid gate).  16-bit
+ * elements of type dtype (ORC_F16 / ORC_BF16). */
+/* paged_attention.cu:288-298, 386-404: qg [T][H][2D] -> q, gate [T][H][D] */
+void orc_split_q_gate(const uint16_t *qg, uint16_t *q, uint16_t *gate, int T,
+                      int H, int D);
+/* layer_attention.cu:86-135: rows of D elements, one weight vector [D] */
+void orc_head_norm(const uint16_t *x, const uint16_t *w, uint16_t *out,
+                   int rows, int D, float eps, int dtype);
+/* layer_attention.cu:32-55: table[pos][pair] = (cos, sin) of pos * theta^(-2 pair / rd) */
+void orc_rope_table(float *table, int n_pos, int rotary_dim, float theta);
+/* layer_attention.cu:57-79 / paged_attention.cu:412-451: rotate pairs
+ * (i, i + rd/2) of every head of token t at position pos[t], in place */
+void orc_apply_rope(uint16_t *x, int T, int H, int D, int rotary_dim,
+                    const int32_t *pos, const float *table, int dtype);
+/* layer.cu:406-431: out = x * sigmoid(gate) */
+void orc_sigmoid_gate(const uint16_t *x, const uint16_t *gate, uint16_t *out,
+                      size_t n, int dtype);
+
 /* ---- host bookkeeping: pool + cache manager ------------------------------ */
 typedef struct orc_cm orc_cm;
 orc_cm *orc_cm_create(int NB, int bs, int max_branches);

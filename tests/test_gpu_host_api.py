@@ -211,3 +211,68 @@ def test_importance_scorer_on_device(dev):
     want = new * (1 + 0.5 + 0.25)
     assert [sc.score(i) for i in range(64)] == want.tolist()
     assert sc.least_important([9, 3, 7]) == 3
+
+
+@pytest.mark.parametrize("geom", [(24, 4, 256, 64, cabi.F16), (32, 8, 128, 32, cabi.BF16)])
+def test_layer_steps_in_the_wrappers_order_fused_and_separate(dev, geom):
+    """full_attention_forward_paged's steps 1b-7 (paged_attention.cu:331-370) for 3 decode branches:
+    once as the reference's separate calls (split, head_norm x2, apply_rope, write, attend,
+    sigmoid_gate; layer.h:77-79, 124-140), once as the two fused launches.  Same bits."""
+    QH, KVH, D, rd, dt = geom
+    L, bs, B = 2, 16, 3
+    assert host.set_attention_geometry(L, QH, KVH, D, dt)
+    assert host.lib().drkh_set_rope(rd, 1.0e7, 1e-6)
+    assert not host.lib().drkh_set_rope(48, 1.0e7, 1e-6)             # 48 / 16 is no power of two: refused, nothing changes
+    L_ = host.lib()
+    rng = np.random.default_rng(90)
+    outs = []
+    for fused in (False, True):
+        cm = host.CacheManager()
+        assert cm.init(64 * L * 2 * KVH * bs * D * 2, bs, None, B)
+        NB = cm.pool_max_blocks()
+        ctx = [40, 17, 33]
+        rs = np.random.default_rng(91)                                # the same inputs in both passes
+        # prior context: plain appends into three independent branches (forks at position 0 share nothing)
+        assert [cm.fork_branch(0, 0) for _ in range(B - 1)] == [1, 2]
+        for b in range(B):
+            assert cm.ensure_blocks_for_range(b, 0, ctx[b] + 1)
+        cm.sync_block_table(U.stream_ptr())
+        keep = []
+        for b in range(B):
+            k0, v0 = U.normal_bits(rs, (ctx[b], KVH, D), dt, 0.5), U.normal_bits(rs, (ctx[b], KVH, D), dt, 0.5)
+            dk0, dv0 = U.dev_bytes(k0), U.dev_bytes(v0)
+            keep += [dk0, dv0]
+            L_.drkh_paged_kv_cache_write_batch(U.p(dk0), U.p(dv0), cm.pool_ptr(), cm.d_block_table(b), 1, 0, ctx[b], NB, bs,
+                                               U.stream_ptr())
+        qg = U.normal_bits(rs, (B, QH, 2 * D), dt, 1.5)
+        k, v = U.normal_bits(rs, (B, KVH, D), dt), U.normal_bits(rs, (B, KVH, D), dt)
+        qw, kw = U.normal_bits(rs, (D,), dt), U.normal_bits(rs, (D,), dt)
+        dqg, dk, dv, dqw, dkw = (U.dev_bytes(a) for a in (qg, k, v, qw, kw))
+        dpos, dlens = U.dev_i32(np.array(ctx)), U.dev_i32(np.array(ctx) + 1)
+        dq, dgate, out = U.dev_zeros(B * QH * D * 2), U.dev_zeros(B * QH * D * 2), U.dev_zeros(B * QH * D * 2)
+        scale, st = float(1 / np.sqrt(D)), U.stream_ptr()
+        if fused:
+            L_.drkh_paged_qk_norm_rope_write_branches(U.p(dqg), U.p(dk), U.p(dv), U.p(dqw), U.p(dkw), U.p(dq), cm.pool_ptr(),
+                                                      cm.d_block_table(0), cm.table_stride(), U.p(dpos), B, 1, NB, bs, None, 0, st)
+            L_.drkh_paged_gqa_decode_attention_gated_branches(U.p(dq), cm.pool_ptr(), cm.d_block_table(0), cm.table_stride(),
+                                                              U.p(dlens), B, max(ctx) + 1, C.c_void_p(dqg.data_ptr() + D * 2), 2 * D,
+                                                              U.p(out), 1, NB, bs, scale, st)
+        else:
+            cabi.call("drk_split_q_gate", U.p(dqg), U.p(dq), U.p(dgate), B, QH, D, st)
+            L_.drkh_head_norm(U.p(dq), U.p(dqw), U.p(dq), B * QH, D, 1e-6, st)
+            L_.drkh_head_norm(U.p(dk), U.p(dkw), U.p(dk), B * KVH, D, 1e-6, st)
+            for b in range(B):                                        # one token per call, as the reference does
+                L_.drkh_apply_rope(C.c_void_p(dq.data_ptr() + b * QH * D * 2), C.c_void_p(dk.data_ptr() + b * KVH * D * 2), QH, KVH, D,
+                                   rd, C.c_void_p(dpos.data_ptr() + 4 * b), 1.0e7, st)
+            L_.drkh_paged_kv_cache_write_branches(U.p(dk), U.p(dv), cm.pool_ptr(), cm.d_block_table(0), cm.table_stride(), U.p(dpos),
+                                                  B, 1, NB, bs, st)
+            L_.drkh_paged_gqa_decode_attention_branches(U.p(dq), cm.pool_ptr(), cm.d_block_table(0), cm.table_stride(), U.p(dlens), B,
+                                                        max(ctx) + 1, U.p(out), 1, NB, bs, scale, st)
+            L_.drkh_sigmoid_gate(U.p(out), U.p(dgate), U.p(out), B * QH * D, st)
+        U.sync()
+        outs.append((U.host(out, np.uint16).copy(), d2h(cm.pool_ptr(), cm.pool_total_bytes()), U.host(dq, np.uint16).copy()))
+        del cm
+    assert np.array_equal(outs[0][2], outs[1][2])          # Q after norm + rope
+    assert np.array_equal(outs[0][1], outs[1][1])          # every byte of the pool
+    assert np.array_equal(outs[0][0], outs[1][0])          # gated attention output
+    assert outs[0][0].any()

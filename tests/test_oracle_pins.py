@@ -356,3 +356,89 @@ def test_importance_update_closed_form():
     sc = np.array([9, 1.0, 1.0, 5, 3, 0, 0, 1.0], dtype=np.float32)
     assert lib.orc_least_important(orc.ptr(sc), orc.ptr(ids), 4) == 2      # first minimum in list order
     assert lib.orc_least_important(orc.ptr(sc), orc.ptr(ids), 0) == -1
+
+
+# ---- layer steps either side of the kernels: split, head norm, RoPE, gate ----
+
+def test_split_q_gate_is_the_reshape():
+    rng = np.random.default_rng(50)
+    T, H, D = 3, 5, 16
+    qg = rng.integers(0, 65536, size=(T, H, 2 * D)).astype(np.uint16)
+    q, gate = orc.split_q_gate(qg, T, H, D)
+    r = qg.reshape(T, H, 2, D)
+    assert np.array_equal(q, r[:, :, 0]) and np.array_equal(gate, r[:, :, 1])
+
+
+@pytest.mark.parametrize("dtype", [orc.F16, orc.BF16])
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_head_norm_matches_fp64_closed_form(dtype, D):
+    rng = np.random.default_rng(51 + D)
+    rows, eps = 37, 1e-6
+    x = U.normal_bits(rng, (rows, D), dtype, 2.0)
+    w = U.normal_bits(rng, (D,), dtype, 1.0)
+    got = orc.head_norm(x, w, eps, dtype)
+    xf = U.from_bits(x, dtype).astype(np.float64)
+    wf = U.from_bits(w, dtype).astype(np.float64)
+    want = xf / np.sqrt((xf * xf).mean(axis=1, keepdims=True) + eps) * wf
+    # two fp32 roundings sit between the exact value and the 16-bit result: one ulp
+    assert U.ulp_distance(got, U.to_bits(want.astype(np.float32), dtype)).max() <= 1
+    # a dropped 1/D, a misplaced eps or a missing weight are far outside that
+    assert np.abs(U.from_bits(got, dtype) - want).max() < 0.02 * np.abs(want).max()
+    # a zero row stays zero; a constant row with unit weights becomes +-1
+    z = orc.head_norm(np.zeros((1, D), np.uint16), w, eps, dtype)
+    assert not U.from_bits(z, dtype).any()
+    c = orc.head_norm(U.to_bits(np.full((1, D), -3.0, np.float32), dtype), U.to_bits(np.ones(D, np.float32), dtype), eps, dtype)
+    assert np.array_equal(U.from_bits(c, dtype), np.full((1, D), -1.0, np.float32))
+
+
+def test_rope_table_matches_fp64_angles():
+    rd, theta, n = 64, 1.0e7, 4096
+    t = orc.rope_table(n, rd, theta)
+    pos = np.arange(n, dtype=np.float64)[:, None]
+    freq = theta ** (-2.0 * np.arange(rd // 2) / rd)
+    ang = pos * freq[None, :]
+    # the angle is formed in fp32 (as in the reference): its rounding error grows with pos
+    tol = 2e-7 * np.maximum(1.0, ang) + 1e-6
+    assert (np.abs(t[:, :, 0] - np.cos(ang)) <= tol).all()
+    assert (np.abs(t[:, :, 1] - np.sin(ang)) <= tol).all()
+    assert np.array_equal(t[0, :, 0], np.ones(rd // 2, np.float32)) and not t[0, :, 1].any()
+
+
+@pytest.mark.parametrize("dtype", [orc.F16, orc.BF16])
+def test_rope_is_a_rotation_of_half_half_pairs(dtype):
+    rng = np.random.default_rng(53)
+    T, H, D, rd, theta = 9, 3, 128, 32, 10000.0
+    tab = orc.rope_table(600, rd, theta)
+    x = U.normal_bits(rng, (T, H, D), dtype)
+    pos = rng.integers(0, 600, size=T).astype(np.int32)
+    pos[0] = 0
+    got = orc.apply_rope(x, pos, tab, rd, dtype)
+    assert np.array_equal(got[0], x[0])                      # position 0: identity, to the bit
+    assert np.array_equal(got[:, :, rd:], x[:, :, rd:])      # dims past rotary_dim are not touched
+    xf = U.from_bits(x, dtype).astype(np.float64)
+    np_ = rd // 2
+    c = tab[pos][:, None, :, 0].astype(np.float64)
+    s = tab[pos][:, None, :, 1].astype(np.float64)
+    want = xf.copy()
+    want[:, :, :np_] = xf[:, :, :np_] * c - xf[:, :, np_:rd] * s
+    want[:, :, np_:rd] = xf[:, :, np_:rd] * c + xf[:, :, :np_] * s
+    assert U.ulp_distance(got, U.to_bits(want.astype(np.float32), dtype)).max() <= 1
+    # direction: (1, 0) at angle a goes to (cos a, sin a)
+    e = np.zeros((1, 1, D), np.float32)
+    e[0, 0, 0] = 1.0
+    r = U.from_bits(orc.apply_rope(U.to_bits(e, dtype), np.array([7], np.int32), tab, rd, dtype), dtype)
+    assert abs(r[0, 0, 0] - tab[7, 0, 0]) < 4e-3 and abs(r[0, 0, np_] - tab[7, 0, 1]) < 4e-3
+    assert np.sign(r[0, 0, np_]) == np.sign(tab[7, 0, 1])
+
+
+@pytest.mark.parametrize("dtype", [orc.F16, orc.BF16])
+def test_sigmoid_gate_matches_fp64_logistic(dtype):
+    rng = np.random.default_rng(54)
+    x = U.normal_bits(rng, (4096,), dtype, 2.0)
+    g = U.normal_bits(rng, (4096,), dtype, 3.0)
+    got = orc.sigmoid_gate(x, g, dtype)
+    xf, gf = U.from_bits(x, dtype).astype(np.float64), U.from_bits(g, dtype).astype(np.float64)
+    want = xf / (1.0 + np.exp(-gf))
+    assert U.ulp_distance(got, U.to_bits(want.astype(np.float32), dtype)).max() <= 1
+    half = orc.sigmoid_gate(x, np.zeros_like(g), dtype)      # gate 0: exactly x / 2
+    assert np.array_equal(U.from_bits(half, dtype), U.from_bits(x, dtype) / 2)

@@ -95,3 +95,13 @@ def rel_abs_ok(got, want, rel=1e-2, abs_=2e-2):
     err = np.abs(got - want)
     lim = abs_ + rel * np.abs(want)
     return bool(np.all(err <= lim)), float(err.max()), float((err / np.maximum(np.abs(want), 1e-30)).max())
+
+
+def ulp_distance(a_bits, b_bits):
+    """Distance in units in the last place between two arrays of 16-bit float bit
+    patterns (fp16 or bf16: both are sign-magnitude, so the patterns order like
+    the values once negative ones are mirrored)."""
+    def key(b):
+        b = np.ascontiguousarray(b, dtype=np.uint16).astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
+    return np.abs(key(a_bits) - key(b_bits))
