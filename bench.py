@@ -276,6 +276,78 @@ def main():
             else:
                 scatter_gbps = gbps
 
+    # ---- the whole attention block of a layer, raw projections in, gated output out:
+    # the reference's sequence of separate launches (split, head_norm x2, rope, page write,
+    # attention, sigmoid gate: paged_attention.cu:331-370) against the two fused launches
+    layer_steps = None
+    if use_graph:
+        rd, theta, eps = D // 4, 1.0e7, 1e-6
+        qg = (torch.randn(L, B, QH, 2 * D, device="cuda") * 0.5).to(torch.bfloat16)
+        qw = torch.randn(D, device="cuda").to(torch.bfloat16)
+        kw = torch.randn(D, device="cuda").to(torch.bfloat16)
+        qsep, gsep = torch.empty_like(q), torch.empty_like(q)
+        ktmp = torch.empty_like(newk)
+        npos = max_ctx + 1
+        rtab = torch.empty(npos * (rd // 2) * 2, dtype=torch.float32, device="cuda")
+        cabi.call("drk_rope_table_fill", U.p(rtab), npos, rd, theta, sp)
+        dpos_l, dlen_l = C.c_void_p(pos_steps[last].data_ptr()), C.c_void_p(len_steps[last].data_ptr())
+        qgrow = B * QH * 2 * D * 2
+        wsb_g = lib.drk_decode_workspace_bytes(C.byref(g), B, max_ctx)
+        ws_g = torch.empty(wsb_g, dtype=torch.uint8, device="cuda")
+
+        def separate(gsp):
+            for l in range(L):
+                qp, gp, op = (C.c_void_p(t.data_ptr() + l * qrow) for t in (qsep, gsep, out))
+                kp = C.c_void_p(ktmp.data_ptr() + l * krow)
+                cabi.call("drk_split_q_gate", C.c_void_p(qg.data_ptr() + l * qgrow), qp, gp, B, QH, D, gsp)
+                cabi.call("drk_head_norm", qp, U.p(qw), qp, B * QH, D, eps, cabi.BF16, gsp)
+                cabi.call("drk_head_norm", C.c_void_p(newk.data_ptr() + l * krow), U.p(kw), kp, B * KVH, D, eps, cabi.BF16, gsp)
+                cabi.call("drk_apply_rope", qp, kp, B, QH, KVH, D, rd, dpos_l, 0, theta, U.p(rtab), npos, cabi.BF16, gsp)
+                cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), stride, dpos_l, B, l, 1, kp,
+                          C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, gsp)
+                cabi.call("drk_paged_decode_attention_branches", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen_l, B,
+                          max_ctx, op, l, float(scale), cabi.BF16, split, U.p(ws), wsb, gsp)
+                cabi.call("drk_sigmoid_gate", op, gp, op, B * QH, D, D, cabi.BF16, gsp)
+
+        def fused(gsp):
+            for l in range(L):
+                qp, op = (C.c_void_p(t.data_ptr() + l * qrow) for t in (qsep, out))
+                qgp = qg.data_ptr() + l * qgrow
+                cabi.call("drk_qk_norm_rope_append", C.byref(g), U.p(pool), U.p(dtab), stride, dpos_l, 0, B, l,
+                          C.c_void_p(qgp), C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow),
+                          U.p(qw), U.p(kw), eps, rd, theta, U.p(rtab), npos, qp, cabi.BF16, gsp)
+                cabi.call("drk_paged_decode_attention_gated", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen_l, B, max_ctx,
+                          op, l, float(scale), cabi.BF16, C.c_void_p(qgp + D * 2), 2 * D, U.p(ws_g), wsb_g, gsp)
+
+        res = {}
+        for name, fn in (("separate", separate), ("fused", fused)):
+            sd = torch.cuda.Stream()
+            sd.wait_stream(stream)
+            with torch.cuda.stream(sd):
+                fn(C.c_void_p(sd.cuda_stream))
+            stream.wait_stream(sd)
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=sd):
+                fn(C.c_void_p(torch.cuda.current_stream().cuda_stream))
+            gr.replay()
+            torch.cuda.synchronize()
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record(stream)
+            for _ in range(5):
+                gr.replay()
+            a1.record(stream)
+            torch.cuda.synchronize()
+            res[name] = a0.elapsed_time(a1) / 5 * 1e3
+            res[name + "_out"] = out.clone()
+        layer_steps = {
+            "what": "per layer: Q|gate split, head RMSNorm of Q and K, partial RoPE (rotary_dim %d), page write, "
+                    "decode attention, sigmoid gate; one captured graph per step" % rd,
+            "separate_us_per_step": round(res["separate"], 1), "separate_launches_per_layer": 8,
+            "fused_us_per_step": round(res["fused"], 1), "fused_launches_per_layer": 3,
+            "same_output_bits": bool(torch.equal(res["separate_out"], res["fused_out"])),
+        }
+
     # ---- CPU baseline: the oracle's restatement of the reference loop, OpenMP ----
     cpu = None
     if not args.no_cpu_baseline:
@@ -334,6 +406,7 @@ def main():
         "bulk_scatter_GBps": None if scatter_gbps is None else round(scatter_gbps, 1),
         "hbm_read_probe_GBps": round(read_probe_gbps, 1),
         "fill_seconds": round(t_fill, 2),
+        "layer_steps": layer_steps,
         "roofline": {
             "kernel": "decode_stream_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
