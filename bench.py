@@ -348,6 +348,36 @@ def main():
             "same_output_bits": bool(torch.equal(res["separate_out"], res["fused_out"])),
         }
 
+    # ---- decode attention that also reports the attention mass per block (importance scores)
+    mass_wsb = lib.drk_decode_mass_workspace_bytes(C.byref(g), B, max_ctx)
+    attention_mass = None
+    if mass_wsb:
+        mws = torch.empty(mass_wsb, dtype=torch.uint8, device="cuda")
+        mstride = (max_ctx + bs - 1) // bs
+        mass = torch.zeros(B * mstride, dtype=torch.float32, device="cuda")
+        tm = {}
+        for name in ("plain", "with_mass"):
+            def go(n):
+                for it in range(n):
+                    l = it % L
+                    qp, op = C.c_void_p(q.data_ptr() + l * qrow), C.c_void_p(out.data_ptr() + l * qrow)
+                    if name == "plain":
+                        cabi.call("drk_paged_decode_attention_branches", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen, B,
+                                  max_ctx, op, l, float(scale), cabi.BF16, 0, U.p(mws), mass_wsb, sp)
+                    else:
+                        cabi.call("drk_paged_decode_attention_mass", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen, B,
+                                  max_ctx, op, l, float(scale), cabi.BF16, U.p(mass), mstride, 1 if l else 0, U.p(mws),
+                                  mass_wsb, sp)
+            go(4)
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record(stream)
+            go(2 * L)
+            a1.record(stream)
+            torch.cuda.synchronize()
+            tm[name] = a0.elapsed_time(a1) / (2 * L) * 1e3
+        attention_mass = {"plain_us_per_layer": round(tm["plain"], 2), "with_mass_us_per_layer": round(tm["with_mass"], 2),
+                          "mass_sum_branch0": round(float(mass[:mstride].sum()), 2), "expected_sum": L * QH}
+
     # ---- CPU baseline: the oracle's restatement of the reference loop, OpenMP ----
     cpu = None
     if not args.no_cpu_baseline:
@@ -407,6 +437,7 @@ def main():
         "hbm_read_probe_GBps": round(read_probe_gbps, 1),
         "fill_seconds": round(t_fill, 2),
         "layer_steps": layer_steps,
+        "attention_mass": attention_mass,
         "roofline": {
             "kernel": "decode_stream_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),

@@ -75,7 +75,10 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
                          float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
                          int start_tile = 0, const float *pre_o = nullptr, const float *pre_m = nullptr,
                          const float *pre_l = nullptr, int pre_splits = 0, const void *gate = nullptr,
-                         size_t gate_stride = 0);
+                         size_t gate_stride = 0, float *lse_groups = nullptr, float *lse_rows = nullptr,
+                         int lse_stride = 0);
+int launch_block_mass(const float *lse_groups, const float *lse_rows, const int32_t *d_seq_lens, int B, int QH,
+                      int lse_stride, int bs, float *mass, int mass_stride, int accumulate, hipStream_t st);
 // shared-prefix pass on the matrix cores (drk_prefill.hip)
 void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,

@@ -743,6 +743,69 @@ int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, c
                          io_dtype, split_tokens, workspace, workspace_bytes, stream);
 }
 
+// ---- attention mass per block (importance scoring) -----------------------------------
+static size_t mass_extra(const Lay &a, int B, int max_seq_len, int *lse_stride)
+{
+    const int ls = 4 * ((max_seq_len + kTile - 1) / kTile);
+    if (lse_stride) *lse_stride = ls;
+    return ((size_t)B * a.QH * ls + (size_t)B * a.QH) * sizeof(float);
+}
+
+size_t drk_decode_mass_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len)
+{
+    Lay a;
+    if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0 || !stream_decode_supported(a, B)) return 0;
+    size_t sp = stream_workspace_need(a, B, max_seq_len, 0);
+    sp = (sp + 255) & ~(size_t)255;
+    return sp + mass_extra(a, B, max_seq_len, nullptr);
+}
+
+// Decode attention that also reports, per (branch, logical block), the attention mass the
+// block received: sum over its tokens and all query heads of the softmax probability --
+// the "new importance values from attention" ImportanceScorer::update takes
+// (importance_scorer.h:37-41; docs/en/architecture/02-memoria.md:40-44).
+int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_tables,
+                                    int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, void *out,
+                                    int layer, float scale, int io_dtype, float *d_block_mass, int mass_stride,
+                                    int accumulate, void *workspace, size_t workspace_bytes, void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (!q || !pool || !d_tables || !out || !d_seq_lens || !d_block_mass) return fail(DRK_ERR_INVALID, "decode_mass: NULL pointer");
+    if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode_mass: io_dtype must be F16 or BF16");
+    if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
+        return fail(DRK_ERR_INVALID, "decode_mass: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
+    if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "decode_mass: layer %d outside [0,%d)", layer, a.L);
+    if (B < 0 || max_seq_len < 0 || table_stride < 0 || mass_stride < 0) return fail(DRK_ERR_INVALID, "decode_mass: negative size");
+    if (B == 0 || max_seq_len == 0) return DRK_OK;
+    if (B > 65535) return fail(DRK_ERR_INVALID, "decode_mass: more than 65535 branches");
+    if (g_force_portable || !stream_decode_supported(a, B))
+        return fail(DRK_ERR_UNSUPPORTED, "decode_mass: needs head_dim 128, 4 query heads per kv head, block_size %% 16 == 0, at most 64 branches");
+    if (mass_stride < (max_seq_len + a.bs - 1) / a.bs)
+        return fail(DRK_ERR_INVALID, "decode_mass: mass_stride %d is less than the %d blocks of max_seq_len", mass_stride,
+                    (max_seq_len + a.bs - 1) / a.bs);
+    int ls;
+    size_t sp = stream_workspace_need(a, B, max_seq_len, 0);
+    sp = (sp + 255) & ~(size_t)255;
+    const size_t need = sp + mass_extra(a, B, max_seq_len, &ls);
+    if (!workspace || workspace_bytes < need)
+        return fail(DRK_ERR_WORKSPACE, "decode_mass: workspace of %zu bytes, need %zu", workspace_bytes, need);
+    if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode_mass: workspace must be 16-byte aligned");
+    float *lse_groups = (float *)((uint8_t *)workspace + sp);
+    float *lse_rows = lse_groups + (size_t)B * a.QH * ls;
+    hipStream_t st = (hipStream_t)stream;
+    if ((rc = launch_decode_stream(a, q, pool, d_tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
+                                   io_dtype, 0, workspace, false, st, 0, nullptr, nullptr, nullptr, 0, nullptr, 0,
+                                   lse_groups, lse_rows, ls)))
+        return rc;
+    if ((rc = launch_decode_stream(a, q, pool, d_tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
+                                   io_dtype, 0, workspace, true, st, 0, nullptr, nullptr, nullptr, 0, nullptr, 0,
+                                   lse_groups, lse_rows, ls)))
+        return rc;
+    return launch_block_mass(lse_groups, lse_rows, d_seq_lens, B, a.QH, ls, a.bs, d_block_mass, mass_stride, accumulate, st);
+}
+
 // steps 6 + 7 of full_attention_forward_paged (paged_attention.cu:362-370) in one call:
 // out = attention * sigmoid(gate); gate rows [B * num_q_heads] are gate_stride elements apart
 int drk_paged_decode_attention_gated(const drk_kv_layout *g, const void *q, const void *pool,

@@ -158,13 +158,17 @@ struct StreamArgs {
     int start_tile;                 // tiles [0, start_tile) of every branch are handled elsewhere (shared prefix)
     unsigned head_stride, kv_plane, block_stride, scale_plane, row_bytes;
     float scale_log2e;
+    // optional: log2-sum-exp of every 16-token group's scaled scores, [B*QH][lse_stride]
+    // (what the attention-mass pass needs; -inf for a group without a visible token)
+    float *lse_groups;
+    int lse_stride;
 };
 
 constexpr int kMaxUnits = 256;       // units one workgroup may own (descriptor table in LDS)
 
 struct UnitDesc {                    // one 64-token tile of one (branch, kv head)
     int tile_lim;                    // tokens of the tile that exist: seq_len - tile*64 (may exceed 64)
-    int flags;                       // bit 0: first tile of a segment of this workgroup, bit 1: last
+    int flags;                       // bit 0: first tile of a segment of this workgroup, bit 1: last; bits 2..: tile index
     int bq;                          // branch*QH + kvh*4: first query row of the group (Q, partial slots)
     int piece;                       // partial slot of the segment inside its (branch, q head)
 };
@@ -359,7 +363,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         if (grp == 0) {
             UnitDesc d;
             d.tile_lim = len - tile * kSTile;
-            d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0);
+            d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0) | (tile << 2);
             d.bq = b * A.QH + kvh * 4;
             d.piece = (int)blockIdx.x - (A.KVH * excl + kvh * nt) / U;
             udesc[ui] = d;
@@ -462,7 +466,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
             const float p = s_exp2(sc - m_use);
             const float alpha = s_exp2(m_run - m_use);
-            l_run = l_run * alpha + s_wave_sum(p);
+            // sum of p: the DPP steps leave each row of 16 lanes (= one 16-token group) with its own sum
+            float rs = p;
+            rs += s_dpp<0xB1>(rs);
+            rs += s_dpp<0x4E>(rs);
+            rs += s_dpp<0x141>(rs);
+            rs += s_dpp<0x140>(rs);
+            l_run = l_run * alpha + ((s_lane(rs, 0) + s_lane(rs, 16)) + (s_lane(rs, 32) + s_lane(rs, 48)));
+            if (A.lse_groups && (lane & 15) == 0) {
+                const int gi = (flags >> 2) * 4 + (lane >> 4);
+                if (gi < A.lse_stride)
+                    A.lse_groups[(size_t)(ud.bq + w) * A.lse_stride + gi] = rs > 0.0f ? m_use + __builtin_log2f(rs) : -INFINITY;
+            }
             m_run = m_new;
             float pw = p;
             if (DT == DRK_INT8) pw = live ? p * vscale_lds[buf][lane] : 0.0f;   // a stale scale may be anything
@@ -569,7 +584,7 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
                                                            int io_dtype, int start_tile, const float *__restrict__ pre_o,
                                                            const float *__restrict__ pre_m, const float *__restrict__ pre_l,
                                                            int pre_splits, const uint16_t *__restrict__ gate,
-                                                           size_t gate_stride)
+                                                           size_t gate_stride, float *__restrict__ lse_rows)
 {
     __shared__ float2 red[4][64];
     const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * 2;
@@ -624,6 +639,7 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
         }
     }
     L = s_wave_sum(L);
+    if (lse_rows && threadIdx.x == 0) lse_rows[(size_t)b * QH + h] = L > 0.0f ? M + __builtin_log2f(L) : -INFINITY;
     red[wv][lane] = acc;
     __syncthreads();
     if (wv == 0) {
@@ -646,6 +662,44 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
         }
         *dst = packed;
     }
+}
+
+// Attention mass per (branch, logical block): sum over the block's tokens and all query heads of
+// the softmax probability, from the per-group and per-row log-sum-exps the two kernels above
+// left.  One thread per (branch, block); consecutive threads read consecutive groups.
+__global__ __launch_bounds__(256) void block_mass_kernel(const float *__restrict__ lse_groups, const float *__restrict__ lse_rows,
+                                                         const int32_t *__restrict__ seq_lens, int B, int QH, int lse_stride,
+                                                         int bs, float *__restrict__ mass, int mass_stride, int accumulate)
+{
+    const int lb = (int)(blockIdx.x * 256 + threadIdx.x), b = blockIdx.y;
+    if (lb >= mass_stride) return;
+    const int len = seq_lens[b];
+    const int nblk = len > 0 ? (len + bs - 1) / bs : 0;
+    float *dst = mass + (size_t)b * mass_stride + lb;
+    if (lb >= nblk) {
+        if (!accumulate) *dst = 0.0f;
+        return;
+    }
+    const int g0 = lb * (bs / 16), g1 = min(g0 + bs / 16, lse_stride);
+    float m = 0.0f;
+    for (int h = 0; h < QH; h++) {
+        const float row = lse_rows[(size_t)b * QH + h];
+        const float *grp = lse_groups + ((size_t)b * QH + h) * lse_stride;
+        for (int gi = g0; gi < g1; gi++) {
+            const float v = grp[gi];
+            if (v > -INFINITY && row > -INFINITY) m += s_exp2(v - row);
+        }
+    }
+    *dst = accumulate ? *dst + m : m;
+}
+
+int launch_block_mass(const float *lse_groups, const float *lse_rows, const int32_t *d_seq_lens, int B, int QH,
+                      int lse_stride, int bs, float *mass, int mass_stride, int accumulate, hipStream_t st)
+{
+    hipLaunchKernelGGL(block_mass_kernel, dim3((mass_stride + 255) / 256, B), dim3(256), 0, st, lse_groups, lse_rows,
+                       d_seq_lens, B, QH, lse_stride, bs, mass, mass_stride, accumulate);
+    DRK_LAUNCH_CHECK("block_mass_kernel");
+    return DRK_OK;
 }
 
 bool stream_decode_supported(const Lay &a, int B)
@@ -684,7 +738,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
                          float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
                          int start_tile, const float *pre_o, const float *pre_m, const float *pre_l, int pre_splits,
-                         const void *gate, size_t gate_stride)
+                         const void *gate, size_t gate_stride, float *lse_groups, float *lse_rows, int lse_stride)
 {
     int grid, U, Pmax;
     stream_shape(a, B, max_seq_len, split_tokens, &grid, &U, &Pmax);
@@ -702,6 +756,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
         A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
         A.scale_log2e = scale * kSLog2e;
+        A.lse_groups = lse_groups; A.lse_stride = lse_stride;
         switch (a.dtype) {
         case DRK_F16: hipLaunchKernelGGL(decode_stream_kernel<DRK_F16>, dim3(grid), dim3(256), 0, st, A); break;
         case DRK_BF16: hipLaunchKernelGGL(decode_stream_kernel<DRK_BF16>, dim3(grid), dim3(256), 0, st, A); break;
@@ -712,7 +767,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
     } else {
         hipLaunchKernelGGL(stream_merge_kernel, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                            d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
-                           pre_l, pre_splits, (const uint16_t *)gate, gate_stride);
+                           pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows);
         DRK_LAUNCH_CHECK("stream_merge_kernel");
     }
     return DRK_OK;

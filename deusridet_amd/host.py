@@ -56,6 +56,10 @@ SIGNATURES = {
                                                       _f32, _vp]),
     "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32]),
+    "drkh_scorer_d_new_scores": (_vp, [_vp]),
+    "drkh_scorer_apply_new_scores": (None, [_vp, _vp]),
+    "drkh_paged_gqa_decode_attention_branches_scored": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32,
+                                                               _f32, _vp, _i32, _vp]),
     "drkh_set_rope": (_i32, [_i32, _f32, _f32]),
     "drkh_sigmoid_gate": (None, [_vp, _vp, _vp, _i32, _vp]),
     "drkh_apply_rope": (None, [_vp, _vp, _i32, _i32, _i32, _i32, _vp, _f32, _vp]),
@@ -111,6 +115,8 @@ class ImportanceScorer:
     def update(self, d_scores_ptr, n): lib().drkh_scorer_update(self._h, d_scores_ptr, n)
     def score(self, b): return lib().drkh_scorer_score(self._h, b)
     def sync_to_host(self): lib().drkh_scorer_sync_to_host(self._h)
+    def d_new_scores(self): return lib().drkh_scorer_d_new_scores(self._h)
+    def apply_new_scores(self, stream=None): lib().drkh_scorer_apply_new_scores(self._h, stream)
 
     def least_important(self, ids):
         a = np.ascontiguousarray(ids, dtype=np.int32)

@@ -205,6 +205,18 @@ void drkh_paged_prefill_attention_gated(const void *Q, void *kv_pool, const int3
     paged_prefill_attention_gated(CH(Q), H(kv_pool), d_block_table, CH(gate), gate_stride, H(out), fa_layer_idx,
                                   pos_start, M, max_phys_blocks, block_size, scale, (hipStream_t)stream);
 }
+void *drkh_scorer_d_new_scores(void *s) { return SC(s)->d_new_scores(); }
+void drkh_scorer_apply_new_scores(void *s, void *stream) { SC(s)->apply_new_scores((hipStream_t)stream); }
+void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_pool, const int32_t *d_tables,
+                                                     int table_stride, const int32_t *d_seq_lens, int B,
+                                                     int max_seq_len, void *out, int fa_layer_idx,
+                                                     int max_phys_blocks, int block_size, float scale,
+                                                     float *d_block_mass, int accumulate, void *stream)
+{
+    paged_gqa_decode_attention_branches_scored(CH(Q), H(kv_pool), d_tables, table_stride, d_seq_lens, B, max_seq_len,
+                                               H(out), fa_layer_idx, max_phys_blocks, block_size, scale, d_block_mass,
+                                               accumulate != 0, (hipStream_t)stream);
+}
 int drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size)
 {
     return paged_attention_reserve_workspace(max_branches, max_seq_len, max_prefill_rows, block_size) ? 1 : 0;

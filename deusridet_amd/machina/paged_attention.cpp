@@ -200,6 +200,26 @@ void paged_gqa_decode_attention_gated_branches(const __half* Q, __half* kv_pool,
         LOG_ERROR("Machina", "paged_gqa_decode_attention_gated_branches: %s", drk_last_error());
 }
 
+void paged_gqa_decode_attention_branches_scored(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                                const int* d_seq_lens, int B, int max_seq_len, __half* out,
+                                                int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                                float* d_block_mass, bool accumulate, hipStream_t stream)
+{
+    if (B <= 0 || max_seq_len <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    size_t need = drk_decode_mass_workspace_bytes(&g, B, max_seq_len);
+    if (need == 0) {
+        LOG_ERROR("Machina", "paged_gqa_decode_attention_branches_scored: geometry not supported by the scored kernel");
+        return;
+    }
+    void* ws = workspace(need);
+    if (!ws) return;
+    if (drk_paged_decode_attention_mass(&g, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, out,
+                                        fa_layer_idx, scale, ModelConfig::IO_DTYPE, d_block_mass, table_stride,
+                                        accumulate ? 1 : 0, ws, g_ws_bytes, stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_gqa_decode_attention_branches_scored: %s", drk_last_error());
+}
+
 void paged_prefill_attention_gated(const __half* Q, __half* kv_pool, const int* d_block_table, const __half* gate,
                                    int gate_stride, __half* out, int fa_layer_idx, int pos_start, int M,
                                    int max_phys_blocks, int block_size, float scale, hipStream_t stream)

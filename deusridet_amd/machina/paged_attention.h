@@ -97,6 +97,15 @@ void paged_prefill_attention_gated(const __half* Q, __half* kv_pool, const int* 
                                    int gate_stride, __half* out, int fa_layer_idx, int pos_start, int M,
                                    int max_phys_blocks, int block_size, float scale, hipStream_t stream = 0);
 
+// Decode attention that also reports the attention mass each block received (sum of the
+// softmax probabilities of its tokens over all query heads) into d_block_mass
+// [B, table_stride] -- ImportanceScorer::d_new_scores() for a CacheManager's tables.
+// accumulate = false on the first full-attention layer of a step, true on the others.
+void paged_gqa_decode_attention_branches_scored(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                                const int* d_seq_lens, int B, int max_seq_len, __half* out,
+                                                int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                                float* d_block_mass, bool accumulate, hipStream_t stream = 0);
+
 // The attention calls keep split-K partials in a device workspace that this
 // library owns and grows on demand (device allocation = implicit sync).  Call
 // this once up front with the largest shapes to keep the steady state free of

@@ -125,7 +125,7 @@ bool CacheManager::pick_victim_nolock(int& cell_out)
     bool have = false;
     float best = 0.0f;
     for (const auto& e : evictable_) {
-        float s = scorer_->score(e.second % max_logical_blocks_);
+        float s = scorer_->score(e.second);       // by table cell; branch 0: the logical block index
         if (!have || s < best) {
             have = true;
             best = s;

@@ -54,6 +54,32 @@ void ImportanceScorer::update(const float* d_block_scores, int num_blocks)
         LOG_ERROR("Memoria", "ImportanceScorer: update: %s", drk_last_error());
 }
 
+float* ImportanceScorer::d_new_scores()
+{
+    if (!d_scores_) return nullptr;
+    if (!d_new_) {
+        void* p = nullptr;
+        size_t bytes = (size_t)max_blocks_ * sizeof(float);
+        if (drk_dev_malloc(&p, bytes) != DRK_OK) {
+            LOG_ERROR("Memoria", "ImportanceScorer: alloc of the new-score buffer failed: %s", drk_last_error());
+            return nullptr;
+        }
+        d_new_ = static_cast<float*>(p);
+        drk_dev_memset_async(d_new_, 0, bytes, nullptr);
+        drk_stream_synchronize(nullptr);
+    }
+    return d_new_;
+}
+
+void ImportanceScorer::apply_new_scores(hipStream_t stream)
+{
+    if (!d_scores_ || !d_new_) return;
+    if (drk_importance_update(d_scores_, d_new_, max_blocks_, decay_, stream) != DRK_OK)
+        LOG_ERROR("Memoria", "ImportanceScorer: apply_new_scores: %s", drk_last_error());
+    last_apply_stream_ = stream;
+    applied_ = true;
+}
+
 int ImportanceScorer::least_important(const int* gpu_resident, int n) const
 {
     if (n <= 0) return -1;
@@ -78,6 +104,10 @@ float ImportanceScorer::score(int logical_block) const
 void ImportanceScorer::sync_to_host()
 {
     if (!d_scores_) return;
+    if (applied_) {
+        drk_stream_synchronize(last_apply_stream_);
+        applied_ = false;
+    }
     if (drk_memcpy_d2h(h_scores_.data(), d_scores_, (size_t)max_blocks_ * sizeof(float), scorer_stream_) != DRK_OK)
         LOG_ERROR("Memoria", "ImportanceScorer: sync_to_host: %s", drk_last_error());
 }
@@ -95,6 +125,11 @@ void ImportanceScorer::destroy()
         drk_dev_free(d_scores_);
         d_scores_ = nullptr;
     }
+    if (d_new_) {
+        drk_dev_free(d_new_);
+        d_new_ = nullptr;
+    }
+    applied_ = false;
     if (scorer_stream_) {
         drk_stream_destroy(scorer_stream_);
         scorer_stream_ = nullptr;

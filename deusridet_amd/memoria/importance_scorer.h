@@ -26,6 +26,16 @@ public:
     // scorer's stream, asynchronous (importance_scorer.cu:67-73).
     void update(const float* d_block_scores, int num_blocks);
 
+    // Not in the reference (its scorer is never fed): a device buffer [max_blocks] for the
+    // attention masses of one step, zeroed at init().  The scored attention call of
+    // machina/paged_attention.h writes (first layer of a step) or accumulates (other layers)
+    // into it; apply_new_scores() then folds it in with update()'s formula, on `stream` -- the
+    // stream the attention ran on, so no cross-stream wait is needed.  sync_to_host() waits for
+    // that stream too.  With a CacheManager of several branches the index is the table cell
+    // branch * table_stride + logical block, so max_blocks must cover max_branches * table_stride.
+    float* d_new_scores();
+    void apply_new_scores(hipStream_t stream);
+
     // First minimum over the given logical block ids in list order, from the host
     // mirror (importance_scorer.cu:75-87).  -1 when n <= 0.
     int least_important(const int* gpu_resident, int n) const;
@@ -42,6 +52,9 @@ public:
 
 private:
     float* d_scores_ = nullptr;
+    float* d_new_ = nullptr;
+    hipStream_t last_apply_stream_ = nullptr;
+    bool applied_ = false;
     std::vector<float> h_scores_;
     int max_blocks_ = 0;
     float decay_ = 0.95f;

@@ -120,6 +120,13 @@ void drkh_paged_gqa_decode_attention_gated_branches(const void *Q, void *kv_pool
 void drkh_paged_prefill_attention_gated(const void *Q, void *kv_pool, const int32_t *d_block_table, const void *gate,
                                         int gate_stride, void *out, int fa_layer_idx, int pos_start, int M,
                                         int max_phys_blocks, int block_size, float scale, void *stream);
+void *drkh_scorer_d_new_scores(void *s);
+void drkh_scorer_apply_new_scores(void *s, void *stream);
+void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_pool, const int32_t *d_tables,
+                                                     int table_stride, const int32_t *d_seq_lens, int B,
+                                                     int max_seq_len, void *out, int fa_layer_idx,
+                                                     int max_phys_blocks, int block_size, float scale,
+                                                     float *d_block_mass, int accumulate, void *stream);
 int  drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
 void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,
                                        int num_tokens, int num_layers, int num_kv_heads, int head_dim,

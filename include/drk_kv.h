@@ -287,6 +287,23 @@ int drk_paged_prefill_attention_gated(const drk_kv_layout *g, const void *q, con
                                       size_t workspace_bytes, void *stream);
 
 /* ---- importance scores -------------------------------------------------- */
+/* Decode attention (as drk_paged_decode_attention_branches) that also reports the attention
+ * mass every block received: d_block_mass[b * mass_stride + lb] = sum over the tokens of
+ * logical block lb of branch b and over all query heads of the softmax probability (so a
+ * branch's blocks sum to num_q_heads).  This is the per-block "new importance value from
+ * attention" that ImportanceScorer::update consumes (importance_scorer.h:37-41; the
+ * reference never computes it: its scorer is unwired).  accumulate != 0 adds to what
+ * d_block_mass holds (sum over the layers of a step); 0 overwrites, and zeroes the entries
+ * of blocks past a branch's length.  mass_stride >= ceil(max_seq_len / block_size); with
+ * mass_stride = CacheManager::table_stride() the array is indexed like the block tables.
+ * Geometry: head_dim 128, 4 query heads per kv head, block_size % 16 == 0, B <= 64. */
+size_t drk_decode_mass_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len);
+int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const void *pool,
+                                    const int32_t *d_tables, int table_stride,
+                                    const int32_t *d_seq_lens, int B, int max_seq_len, void *out,
+                                    int layer, float scale, int io_dtype, float *d_block_mass,
+                                    int mass_stride, int accumulate, void *workspace,
+                                    size_t workspace_bytes, void *stream);
 /* importance_update_kernel, importance_scorer.cu:27-36, 67-73 */
 int drk_importance_update(float *d_scores, const float *d_new_scores, int n, float decay,
                           void *stream);

@@ -52,6 +52,7 @@ def lib():
         "orc_extract": (None, [P, vp, vp, vp, vp, i32, i32, i32]),
         "orc_inject": (None, [P, vp, vp, vp, vp, i32, i32, i32]),
         "orc_copy_block": (None, [P, vp, i32, i32]),
+        "orc_block_attention_mass": (None, [P, vp, vp, vp, i32, vp, i32, i32, f64, i32, vp, i32]),
         "orc_split_q_gate": (None, [vp, vp, vp, i32, i32, i32]),
         "orc_head_norm": (None, [vp, vp, vp, i32, i32, f32, i32]),
         "orc_rope_table": (None, [vp, i32, i32, f32]),
@@ -188,6 +189,18 @@ def quant_row_fp8(x, src_dtype):
     codes = np.empty(x.shape[0], dtype=np.uint8)
     lib().orc_quant_row_fp8(ptr(x), x.shape[0], src_dtype, ptr(codes))
     return codes
+
+
+def block_attention_mass(g, q, pool, tables, seq_lens, layer, scale, io_dtype, mass_stride):
+    """fp64 attention mass per (branch, logical block): [B][mass_stride]"""
+    tables = np.ascontiguousarray(tables, dtype=np.int32)
+    seq_lens = np.ascontiguousarray(seq_lens, dtype=np.int32)
+    q = np.ascontiguousarray(q, dtype=np.uint16)
+    B = seq_lens.shape[0]
+    mass = np.zeros((B, mass_stride), np.float64)
+    lib().orc_block_attention_mass(C.byref(g), ptr(q), ptr(pool), ptr(tables), tables.shape[1], ptr(seq_lens), B, layer,
+                                   float(scale), io_dtype, ptr(mass), mass_stride)
+    return mass
 
 
 def split_q_gate(qg, T, H, D):

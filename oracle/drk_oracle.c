@@ -565,6 +565,44 @@ void orc_decode_branches(const orc_layout *g, const uint16_t *Q, const void *poo
     }
 }
 
+/* Attention mass per (branch, logical block): sum over the block's tokens and over all
+ * query heads of the softmax probability, in fp64 (builder-specified; it is the "new
+ * importance value from attention" of importance_scorer.h:37-41, which the reference
+ * never computes).  mass [B][mass_stride], entries past a branch's blocks are set to 0. */
+void orc_block_attention_mass(const orc_layout *g, const uint16_t *Q, const void *pool,
+                              const int32_t *tables, int table_stride, const int32_t *seq_lens,
+                              int B, int layer, double scale, int io_dtype, double *mass,
+                              int mass_stride)
+{
+    int D = g->D, groups = g->QH / g->KVH;
+    float *row = (float *)malloc(sizeof(float) * D);
+    for (int b = 0; b < B; b++) {
+        const int32_t *table = tables + (size_t)b * table_stride;
+        int n = seq_lens[b];
+        double *s = (double *)malloc(sizeof(double) * (n > 0 ? n : 1));
+        for (int lb = 0; lb < mass_stride; lb++) mass[(size_t)b * mass_stride + lb] = 0.0;
+        for (int h = 0; h < g->QH; h++) {
+            const uint16_t *Qh = Q + ((size_t)b * g->QH + h) * D;
+            double mx = -INFINITY, denom = 0.0;
+            for (int t = 0; t < n; t++) {
+                int blk = table[t / g->bs];
+                if (blk < 0) { s[t] = -INFINITY; continue; }
+                load_row(g, (const uint8_t *)pool, layer, blk, h / groups, t % g->bs, 0, row);
+                double acc = 0.0;
+                for (int d = 0; d < D; d++) acc += (double)elem_to_f(Qh[d], io_dtype) * (double)row[d];
+                s[t] = acc * scale;
+                if (s[t] > mx) mx = s[t];
+            }
+            for (int t = 0; t < n; t++) if (s[t] != -INFINITY) denom += exp(s[t] - mx);
+            if (!(denom > 0.0)) continue;
+            for (int t = 0; t < n; t++)
+                if (s[t] != -INFINITY) mass[(size_t)b * mass_stride + t / g->bs] += exp(s[t] - mx) / denom;
+        }
+        free(s);
+    }
+    free(row);
+}
+
 /* ======================================================================== */
 /* layer steps either side of the kernels                                   */
 /* ======================================================================== */
@@ -692,7 +730,8 @@ struct orc_cm {
     int32_t *seq_len; int8_t *alive;
     /* lru_order_ deque (cache_manager.h:139): front = oldest */
     int32_t *lru_b, *lru_l; int lru_n;
-    /* optional scores indexed by logical block (cache_manager.cpp:188-201) */
+    /* optional scores indexed by table cell = branch * max_logical + logical block; for branch 0,
+     * the reference's one sequence, that is its logical block index (cache_manager.cpp:188-201) */
     float *scores; int nscores;
     /* queued COW copies */
     int32_t *cp_src, *cp_dst; int cp_n, cp_cap;
@@ -782,8 +821,9 @@ static int pick_victim(orc_cm *c, int *vb, int *vl)
         int phys = c->table[CELL(c, b, l)];
         if (c->loc[CELL(c, b, l)] != 0 || phys < 0 || c->refcount[phys] != 1) continue;
         if (!c->scores) { best = i; break; }              /* lru_order_.front() */
-        float s = l < c->nscores ? c->scores[l] : 0.0f;
-        float sb = best < 0 ? 0.0f : (c->lru_l[best] < c->nscores ? c->scores[c->lru_l[best]] : 0.0f);
+        int cell = CELL(c, b, l), cbest = best < 0 ? 0 : CELL(c, c->lru_b[best], c->lru_l[best]);
+        float s = cell < c->nscores ? c->scores[cell] : 0.0f;
+        float sb = best < 0 ? 0.0f : (cbest < c->nscores ? c->scores[cbest] : 0.0f);
         if (best < 0 || s < sb) best = i;                 /* first minimum */
     }
     if (best < 0) return 0;

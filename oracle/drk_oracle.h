@@ -104,6 +104,12 @@ void orc_decode_branches(const orc_layout *g, const uint16_t *Q, const void *poo
                          const int32_t *seq_lens, int B, uint16_t *out, int layer,
                          float scale, int io_dtype, int threads);
 
+/* attention mass per (branch, logical block), fp64; builder-specified, see drk_oracle.c */
+void orc_block_attention_mass(const orc_layout *g, const uint16_t *Q, const void *pool,
+                              const int32_t *tables, int table_stride,
+                              const int32_t *seq_lens, int B, int layer, double scale,
+                              int io_dtype, double *mass, int mass_stride);
+
 /* ---- importance scorer (importance_scorer.cu:27-36, 75-87) --------------- */
 void orc_importance_update(float *scores, const float *new_scores, int n,
                            float decay);

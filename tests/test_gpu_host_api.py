@@ -276,3 +276,74 @@ def test_layer_steps_in_the_wrappers_order_fused_and_separate(dev, geom):
     assert np.array_equal(outs[0][1], outs[1][1])          # every byte of the pool
     assert np.array_equal(outs[0][0], outs[1][0])          # gated attention output
     assert outs[0][0].any()
+
+
+def test_eviction_guided_by_measured_attention_mass(dev):
+    """The loop the reference describes but never wires (docs/en/architecture/02-memoria.md:40-44,
+    importance_scorer.h:7-14): attention reports the weight each block received, summed over the
+    full-attention layers; the scorer folds it in; the next eviction takes the least attended
+    block of any branch."""
+    L, QH, KVH, D, bs, B = 2, 32, 8, 128, 16, 2
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    cm, sc = host.CacheManager(), host.ImportanceScorer()
+    NBLK = 40
+    assert cm.init(NBLK * L * 2 * KVH * bs * D * 2, bs, sc, B)
+    stride = cm.table_stride()
+    assert sc.init(B * stride, 0.5)
+    NB = cm.pool_max_blocks()
+    assert cm.fork_branch(0, 0) == 1
+    ctx = [10 * bs, 7 * bs]                         # whole blocks: a short last block would trivially weigh least
+    rng = np.random.default_rng(92)
+    q = rng.standard_normal((L, B, QH, D)).astype(np.float32) * 0.5
+    og = orc.layout(L, KVH, QH, D, bs, NB, orc.BF16)
+    keep = []
+    for b in range(B):
+        assert cm.ensure_blocks_for_range(b, 0, ctx[b])
+    cm.sync_block_table(U.stream_ptr())
+    L_ = host.lib()
+    cold = (1, 4)                                   # branch 1, logical block 4: keys opposed to every query of its group
+    kv_host = []
+    for b in range(B):
+        k = rng.standard_normal((L, ctx[b], KVH, D)).astype(np.float32) * 0.5
+        if b == cold[0]:
+            for l in range(L):
+                for h in range(KVH):
+                    k[l, cold[1] * bs:(cold[1] + 1) * bs, h] = -2.0 * q[l, b, 4 * h:4 * h + 4].mean(axis=0)
+        v = rng.standard_normal((L, ctx[b], KVH, D)).astype(np.float32) * 0.5
+        kb, vb = U.to_bits(k, cabi.BF16), U.to_bits(v, cabi.BF16)
+        kv_host.append((kb, vb))
+        for l in range(L):
+            dk, dv = U.dev_bytes(kb[l]), U.dev_bytes(vb[l])
+            keep += [dk, dv]
+            L_.drkh_paged_kv_cache_write_batch(U.p(dk), U.p(dv), cm.pool_ptr(), cm.d_block_table(b), l, 0, ctx[b], NB, bs,
+                                               U.stream_ptr())
+    qb = U.to_bits(q, cabi.BF16)
+    dq, dlens, out = U.dev_bytes(qb), U.dev_i32(np.array(ctx)), U.dev_zeros(L * B * QH * D * 2)
+    scale = float(1 / np.sqrt(D))
+    for l in range(L):
+        L_.drkh_paged_gqa_decode_attention_branches_scored(
+            C.c_void_p(dq.data_ptr() + l * B * QH * D * 2), cm.pool_ptr(), cm.d_block_table(0), stride, U.p(dlens), B, max(ctx),
+            C.c_void_p(out.data_ptr() + l * B * QH * D * 2), l, NB, bs, scale, sc.d_new_scores(), 1 if l > 0 else 0,
+            U.stream_ptr())
+    sc.apply_new_scores(U.stream_ptr())
+    sc.sync_to_host()
+    # the oracle's masses on the same pool contents
+    tables = np.stack([cm.h_block_table(b) for b in range(B)])
+    opool = orc.new_pool(og)
+    for b in range(B):
+        for l in range(L):
+            orc.append_batch(og, opool, tables[b], l, 0, kv_host[b][0][l], kv_host[b][1][l], orc.BF16)
+    want = sum(orc.block_attention_mass(og, qb[l], opool, tables, np.array(ctx, np.int32), l, scale, orc.BF16, stride)
+               for l in range(L))
+    got = np.array([[sc.score(b * stride + lb) for lb in range(stride)] for b in range(B)])
+    assert np.all(np.abs(got - want) <= 4e-3 + 2e-3 * np.abs(want)), float(np.abs(got - want).max())
+    assert np.allclose(got.sum(axis=1), L * QH, atol=5e-2)
+    live = [(b, lb) for b in range(B) for lb in range((ctx[b] + bs - 1) // bs)]
+    assert min(live, key=lambda c: want[c]) == cold and want[cold] < 0.5 * sorted(want[c] for c in live)[1]
+    # the next eviction takes exactly that block
+    before = tables.copy()
+    assert cm.evict_blocks(1) == 1
+    after = np.stack([cm.h_block_table(b) for b in range(B)])
+    changed = np.argwhere(before != after)
+    assert changed.tolist() == [list(cold)] and after[cold] == -1
+    assert cm.block_location(*cold) == host.CacheManager.INVALID

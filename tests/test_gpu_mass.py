@@ -1,0 +1,100 @@
+"""GPU parity of the attention-mass output of the decode path (the per-block importance
+values ImportanceScorer::update consumes, importance_scorer.h:37-41) against the fp64
+oracle.  Floating point: |err| <= 2e-3 + 2e-3 * |want| on masses that range over
+[0, num_q_heads]; the attention output itself must keep the bits of the plain call."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from deusridet_amd import cabi
+from oracle import binding as orc
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(dtype, bs, seed, B=4, ctx=900, holes=True):
+    L, KVH, QH, D = 2, 8, 32, 128
+    nblk = (ctx + bs - 1) // bs
+    NB = B * nblk + 2
+    g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
+    io = dtype if dtype in (cabi.F16, cabi.BF16) else cabi.BF16
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(1, ctx + 1, size=B).astype(np.int32)
+    lens[0] = ctx
+    if B > 2:
+        lens[2] = 0
+    perm = rng.permutation(NB).astype(np.int32)
+    stride = nblk + 3
+    tables = np.full((B, stride), -1, np.int32)
+    tables[:, :nblk] = perm[:B * nblk].reshape(B, nblk)
+    opool = orc.new_pool(og)
+    for b in range(B):
+        n = int(lens[b])
+        if n:
+            # a few sharp keys so that the mass is far from uniform
+            kf = rng.standard_normal((n, KVH, D)).astype(np.float32) * 0.5
+            kf[rng.integers(0, n, size=max(1, n // 50))] *= 4.0
+            orc.append_batch(og, opool, tables[b], 1, 0, U.to_bits(kf, io), U.normal_bits(rng, (n, KVH, D), io, 0.5), io)
+    if holes:
+        tables[0, 1] = -1
+    q = U.normal_bits(rng, (B, QH, D), io, 0.7)
+    return g, og, io, lens, tables, stride, opool, q, (B, QH, D, ctx)
+
+
+def _run(g, io, lens, tables, stride, opool, q, shape, mass0=None, accumulate=0):
+    B, QH, D, ctx = shape
+    lib = cabi.lib()
+    dpool, dq, dtab, dlens = U.dev_bytes(opool), U.dev_bytes(q), U.dev_i32(tables), U.dev_i32(lens)
+    wsb = lib.drk_decode_mass_workspace_bytes(C.byref(g), B, ctx)
+    assert wsb > lib.drk_decode_workspace_bytes(C.byref(g), B, ctx) - 4096
+    ws = U.dev_zeros(wsb)
+    out, out_plain = U.dev_zeros(B * QH * D * 2), U.dev_zeros(B * QH * D * 2)
+    mass = U.dev_bytes(mass0 if mass0 is not None else np.full((B, stride), 7.0, np.float32))
+    scale = 1.0 / np.sqrt(D)
+    cabi.call("drk_paged_decode_attention_mass", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dlens), B, ctx,
+              U.p(out), 1, scale, io, U.p(mass), stride, accumulate, U.p(ws), wsb, U.stream_ptr())
+    cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dlens), B, ctx,
+              U.p(out_plain), 1, scale, io, 0, U.p(ws), wsb, U.stream_ptr())
+    U.sync()
+    assert np.array_equal(U.host(out, np.uint16), U.host(out_plain, np.uint16))
+    return U.host(mass, np.float32, (B, stride)).copy()
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
+@pytest.mark.parametrize("bs", [16, 64])
+def test_block_mass_matches_fp64(dev, dtype, bs):
+    g, og, io, lens, tables, stride, opool, q, shape = _case(dtype, bs, seed=100 + bs)
+    got = _run(g, io, lens, tables, stride, opool, q, shape)
+    want = orc.block_attention_mass(og, q, opool, tables, lens, 1, 1.0 / np.sqrt(shape[2]), io, stride)
+    assert np.all(np.abs(got - want) <= 2e-3 + 2e-3 * np.abs(want)), float(np.abs(got - want).max())
+    QH = shape[1]
+    sums = got.sum(axis=1)
+    assert np.allclose(sums[lens > 0], QH, atol=2e-2) and sums[2] == 0.0          # an empty branch: all zero
+    assert got[0, 1] == 0.0                                                        # the hole
+    nblk = (lens + bs - 1) // bs
+    for b in range(len(lens)):
+        assert not got[b, nblk[b]:].any()                                          # overwritten with zeros past the length
+
+
+def test_block_mass_accumulates_over_layers(dev):
+    g, og, io, lens, tables, stride, opool, q, shape = _case(cabi.BF16, 16, seed=7, holes=False)
+    base = np.random.default_rng(3).random((shape[0], stride)).astype(np.float32)
+    once = _run(g, io, lens, tables, stride, opool, q, shape)
+    acc = _run(g, io, lens, tables, stride, opool, q, shape, mass0=base, accumulate=1)
+    assert np.allclose(acc, base + once, rtol=0, atol=1e-5)
+
+
+def test_block_mass_argument_errors(dev):
+    g, og, io, lens, tables, stride, opool, q, shape = _case(cabi.BF16, 16, seed=8, B=2, ctx=100, holes=False)
+    B, QH, D, ctx = shape
+    x = U.dev_zeros(1 << 16)
+    with pytest.raises(cabi.DrkError):       # mass rows shorter than the blocks of max_seq_len
+        cabi.call("drk_paged_decode_attention_mass", C.byref(g), U.p(x), U.p(x), U.p(x), stride, U.p(x), B, ctx, U.p(x), 0,
+                  0.1, io, U.p(x), 3, 0, U.p(x), 1 << 16, U.stream_ptr())
+    g2 = cabi.layout(1, 4, 24, 256, 16, 8, cabi.F16)       # a geometry the tiled kernels do not take
+    assert cabi.lib().drk_decode_mass_workspace_bytes(C.byref(g2), 1, 100) == 0
+    with pytest.raises(cabi.DrkError):
+        cabi.call("drk_paged_decode_attention_mass", C.byref(g2), U.p(x), U.p(x), U.p(x), 8, U.p(x), 1, 100, U.p(x), 0,
+                  0.1, cabi.F16, U.p(x), 8, 0, U.p(x), 1 << 16, U.stream_ptr())

@@ -149,9 +149,10 @@ def test_random_trace_matches_oracle(seed):
     sc = None
     cm_scorer = None
     if use_scores:
-        scores = rng.random(2 * NB).astype(np.float32).round(1)        # ties on purpose
+        # one score per table cell (branch, logical block); ties on purpose
+        scores = rng.random(branches * 2 * NB).astype(np.float32).round(1)
         cm_scorer = host.ImportanceScorer()
-        assert cm_scorer.init_detached(2 * NB)
+        assert cm_scorer.init_detached(branches * 2 * NB)
         cm_scorer.load_host_scores(scores)
         sc = scores
     cm = make(NB, bs, branches, cm_scorer)

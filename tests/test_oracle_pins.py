@@ -442,3 +442,48 @@ def test_sigmoid_gate_matches_fp64_logistic(dtype):
     assert U.ulp_distance(got, U.to_bits(want.astype(np.float32), dtype)).max() <= 1
     half = orc.sigmoid_gate(x, np.zeros_like(g), dtype)      # gate 0: exactly x / 2
     assert np.array_equal(U.from_bits(half, dtype), U.from_bits(x, dtype) / 2)
+
+
+def test_block_attention_mass_closed_forms():
+    """Sum over a branch's blocks = number of query heads; equal keys spread the mass by token
+    count; one dominant key collects it; a hole collects nothing."""
+    L, KVH, QH, D, bs, NB = 1, 2, 8, 64, 16, 12
+    g = orc.layout(L, KVH, QH, D, bs, NB, orc.BF16)
+    rng = np.random.default_rng(55)
+    n = 3 * bs + 5
+    tables = np.array([[4, 9, 1, 7, -1], [2, 3, -1, 5, -1]], np.int32)
+    lens = np.array([n, n], np.int32)
+    pool = orc.new_pool(g)
+    k = U.normal_bits(rng, (n, KVH, D), orc.BF16)
+    v = U.normal_bits(rng, (n, KVH, D), orc.BF16)
+    for b in range(2):
+        orc.append_batch(g, pool, tables[b], 0, 0, k, v, orc.BF16)      # branch 1 has a hole at block 2
+    q = U.normal_bits(rng, (2, QH, D), orc.BF16)
+    m = orc.block_attention_mass(g, q, pool, tables, lens, 0, 0.125, orc.BF16, 5)
+    assert np.allclose(m.sum(axis=1), QH, rtol=0, atol=1e-9)
+    assert m[1, 2] == 0.0 and (m[:, 4] == 0.0).all() and (m[0, :4] > 0).all()
+    # independent numpy softmax for branch 0
+    kf = U.from_bits(k, orc.BF16).astype(np.float64)
+    qf = U.from_bits(q[0], orc.BF16).astype(np.float64)
+    want = np.zeros(5)
+    for h in range(QH):
+        s = kf[:, h // (QH // KVH)] @ qf[h] * 0.125
+        p = np.exp(s - s.max())
+        p /= p.sum()
+        for t in range(n):
+            want[t // bs] += p[t]
+    assert np.allclose(m[0], want, rtol=1e-12, atol=1e-12)
+    # equal keys: every token weighs 1/n
+    pool2 = orc.new_pool(g)
+    kc = np.broadcast_to(k[:1], k.shape).copy()
+    orc.append_batch(g, pool2, tables[0], 0, 0, kc, v, orc.BF16)
+    m2 = orc.block_attention_mass(g, q[:1], pool2, tables[:1], lens[:1], 0, 0.125, orc.BF16, 5)
+    assert np.allclose(m2[0, :4], QH * np.array([bs, bs, bs, 5]) / n, atol=1e-9)
+    # one dominant key (token 20, block 1) under a large scale
+    kd = U.to_bits(np.zeros((n, KVH, D), np.float32), orc.BF16)
+    kd[20] = U.to_bits(np.ones((KVH, D), np.float32), orc.BF16)
+    qd = U.to_bits(np.ones((1, QH, D), np.float32), orc.BF16)
+    pool3 = orc.new_pool(g)
+    orc.append_batch(g, pool3, tables[0], 0, 0, kd, v, orc.BF16)
+    m3 = orc.block_attention_mass(g, qd, pool3, tables[:1], lens[:1], 0, 1.0, orc.BF16, 5)
+    assert abs(m3[0, 1] - QH) < 1e-9
