@@ -378,6 +378,28 @@ def main():
         attention_mass = {"plain_us_per_layer": round(tm["plain"], 2), "with_mass_us_per_layer": round(tm["with_mass"], 2),
                           "mass_sum_branch0": round(float(mass[:mstride].sum()), 2), "expected_sum": L * QH}
 
+    # ---- overflow tier: one block (all layers) per strided 2-D copy to / from pinned host memory
+    overflow = None
+    blk_bytes = lib.drk_kv_block_total_bytes(C.byref(g))
+    hp = C.c_void_p()
+    nswap = 64
+    if cabi.lib().drk_host_malloc(C.byref(hp), blk_bytes * 4) == 0:
+        res = {}
+        for name in ("drk_kv_block_to_host", "drk_kv_block_from_host"):
+            def go(n):
+                for i in range(n):
+                    cabi.call(name, C.byref(g), U.p(pool), int(perm[i % NB]), C.c_void_p(hp.value + (i % 4) * blk_bytes), sp)
+            go(4)
+            torch.cuda.synchronize()
+            t0 = time.time()
+            go(nswap)
+            torch.cuda.synchronize()
+            res[name] = blk_bytes * nswap / (time.time() - t0) / 1e9
+        cabi.call("drk_host_free", hp)
+        overflow = {"block_MiB": round(blk_bytes / 2**20, 2), "to_host_GBps": round(res["drk_kv_block_to_host"], 1),
+                    "from_host_GBps": round(res["drk_kv_block_from_host"], 1),
+                    "what": "%d blocks of %d layers each way, one strided copy per block, pinned host memory" % (nswap, L)}
+
     # ---- CPU baseline: the oracle's restatement of the reference loop, OpenMP ----
     cpu = None
     if not args.no_cpu_baseline:
@@ -438,6 +460,7 @@ def main():
         "fill_seconds": round(t_fill, 2),
         "layer_steps": layer_steps,
         "attention_mass": attention_mass,
+        "overflow_tier": overflow,
         "roofline": {
             "kernel": "decode_stream_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),

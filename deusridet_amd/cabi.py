@@ -54,6 +54,12 @@ SIGNATURES = {
     "drk_dev_memset_async": (_i32, [_vp, _i32, _sz, _vp]),
     "drk_memcpy_h2d_async": (_i32, [_vp, _vp, _sz, _vp]),
     "drk_memcpy_d2h": (_i32, [_vp, _vp, _sz, _vp]),
+    "drk_device_synchronize": (_i32, []),
+    "drk_host_malloc": (_i32, [C.POINTER(_vp), _sz]),
+    "drk_host_free": (_i32, [_vp]),
+    "drk_kv_block_total_bytes": (_sz, [_LP]),
+    "drk_kv_block_to_host": (_i32, [_LP, _vp, _i32, _vp, _vp]),
+    "drk_kv_block_from_host": (_i32, [_LP, _vp, _i32, _vp, _vp]),
     "drk_stream_create": (_i32, [C.POINTER(_vp)]),
     "drk_stream_destroy": (_i32, [_vp]),
     "drk_stream_synchronize": (_i32, [_vp]),

@@ -156,6 +156,62 @@ int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream)
     DRK_HIP(hipStreamSynchronize((hipStream_t)stream));
     return DRK_OK;
 }
+int drk_device_synchronize(void)
+{
+    DRK_HIP(hipDeviceSynchronize());
+    return DRK_OK;
+}
+
+// pinned host memory for staging (allocated pinned; existing memory is never registered)
+int drk_host_malloc(void **h_ptr, size_t bytes)
+{
+    if (!h_ptr) return fail(DRK_ERR_INVALID, "h_ptr is NULL");
+    *h_ptr = nullptr;
+    DRK_HIP(hipHostMalloc(h_ptr, bytes, hipHostMallocDefault));
+    return DRK_OK;
+}
+int drk_host_free(void *h_ptr)
+{
+    if (h_ptr) DRK_HIP(hipHostFree(h_ptr));
+    return DRK_OK;
+}
+
+size_t drk_kv_block_total_bytes(const drk_kv_layout *g)
+{
+    Lay a;
+    if (drk::make_lay(g, &a) != DRK_OK) return 0;
+    return (size_t)a.L * a.block_stride;
+}
+
+// One physical block, all layers, between the pool and a contiguous host image
+// [layer][K plane | V plane | K scales | V scales] -- the order KVSwapper::swap_out writes
+// its .kv files in (kv_swapper.cpp:183-198).  The block's layers lie layer_stride apart in
+// the pool: one strided 2-D copy instead of the reference's 2 x layers separate copies.
+static int block_copy(const drk_kv_layout *g, void *pool, int blk, void *host, bool to_host, void *stream)
+{
+    Lay a;
+    int rc = drk::make_lay(g, &a);
+    if (rc) return rc;
+    if (!pool || !host) return fail(DRK_ERR_INVALID, "block copy: NULL pointer");
+    if (blk < 0 || blk >= a.NB) return fail(DRK_ERR_INVALID, "block copy: block %d outside [0,%d)", blk, a.NB);
+    uint8_t *dev = (uint8_t *)pool + (size_t)blk * a.block_stride;
+    if (to_host)
+        DRK_HIP(hipMemcpy2DAsync(host, a.block_stride, dev, a.layer_stride, a.block_stride, (size_t)a.L,
+                                 hipMemcpyDeviceToHost, (hipStream_t)stream));
+    else
+        DRK_HIP(hipMemcpy2DAsync(dev, a.layer_stride, host, a.block_stride, a.block_stride, (size_t)a.L,
+                                 hipMemcpyHostToDevice, (hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_kv_block_to_host(const drk_kv_layout *g, const void *pool, int blk, void *h_dst, void *stream)
+{
+    return block_copy(g, (void *)pool, blk, h_dst, true, stream);
+}
+int drk_kv_block_from_host(const drk_kv_layout *g, void *pool, int blk, const void *h_src, void *stream)
+{
+    return block_copy(g, pool, blk, (void *)h_src, false, stream);
+}
+
 int drk_stream_create(void **stream)
 {
     if (!stream) return fail(DRK_ERR_INVALID, "stream is NULL");

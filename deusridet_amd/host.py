@@ -25,6 +25,19 @@ SIGNATURES = {
     "drkh_scorer_load_host_scores": (None, [_vp, _vp, _i32]),
     "drkh_cm_create": (_vp, []), "drkh_cm_destroy": (None, [_vp]),
     "drkh_cm_init": (_i32, [_vp, _sz, _i32, _vp, _i32]),
+    "drkh_cm_init_ssd": (_i32, [_vp, _sz, C.c_char_p, _i32, _vp, _vp, _i32]),
+    "drkh_cm_ssd_blocks_used": (_i32, [_vp]),
+    "drkh_cm_prefetch_block": (None, [_vp, _i32, _i32]),
+    "drkh_swapper_create": (_vp, []),
+    "drkh_swapper_destroy": (None, [_vp]),
+    "drkh_swapper_init": (_i32, [_vp, _vp, C.c_char_p, _i32]),
+    "drkh_swapper_shutdown": (None, [_vp]),
+    "drkh_swapper_drain": (None, [_vp]),
+    "drkh_swapper_pending": (_i32, [_vp]),
+    "drkh_swapper_prefetch": (None, [_vp, _i32, C.c_char_p]),
+    "drkh_swapper_is_prefetched": (_i32, [_vp, _i32]),
+    "drkh_swapper_block_bytes": (_sz, [_vp]),
+    "drkh_swapper_swap": (_i32, [_vp, _i32, _i32, _i32, C.c_char_p]),
     "drkh_cm_init_detached": (_i32, [_vp, _i32, _i32, _vp, _i32]),
     "drkh_cm_ensure_blocks_for": (_i32, [_vp, _i32, _i32]),
     "drkh_cm_ensure_blocks_for_range": (_i32, [_vp, _i32, _i32, _i32]),
@@ -127,6 +140,30 @@ class ImportanceScorer:
         lib().drkh_scorer_load_host_scores(self._h, _p(a), a.shape[0])
 
 
+class KVSwapper:
+    """src/memoria/kv_swapper.h:50-114; init() takes the CacheManager whose pool it serves."""
+
+    def __init__(self):
+        self._h = lib().drkh_swapper_create()
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().drkh_swapper_destroy(self._h)
+            self._h = None
+
+    def init(self, cm, ssd_dir, staging_blocks=2):
+        return bool(lib().drkh_swapper_init(self._h, cm._h, str(ssd_dir).encode(), staging_blocks))
+
+    def shutdown(self): lib().drkh_swapper_shutdown(self._h)
+    def drain(self): lib().drkh_swapper_drain(self._h)
+    def pending(self): return lib().drkh_swapper_pending(self._h)
+    def prefetch(self, idx, path): lib().drkh_swapper_prefetch(self._h, idx, str(path).encode())
+    def is_prefetched(self, idx): return bool(lib().drkh_swapper_is_prefetched(self._h, idx))
+    def block_bytes(self): return lib().drkh_swapper_block_bytes(self._h)
+    def swap_out(self, idx, phys, path): return bool(lib().drkh_swapper_swap(self._h, 0, idx, phys, str(path).encode()))
+    def swap_in(self, idx, phys, path): return bool(lib().drkh_swapper_swap(self._h, 1, idx, phys, str(path).encode()))
+
+
 class CacheManager:
     GPU, INVALID, SSD = 0, -1, -2
 
@@ -143,6 +180,14 @@ class CacheManager:
         self._scorer = scorer
         return bool(lib().drkh_cm_init(self._h, int(kv_budget_bytes), block_size, scorer._h if scorer else None,
                                        max_branches))
+
+    def init_ssd(self, kv_budget_bytes, cache_dir, block_size, swapper, scorer=None, max_branches=1):
+        self._scorer, self._swapper = scorer, swapper
+        return bool(lib().drkh_cm_init_ssd(self._h, int(kv_budget_bytes), str(cache_dir).encode(), block_size,
+                                           swapper._h if swapper else None, scorer._h if scorer else None, max_branches))
+
+    def ssd_blocks_used(self): return lib().drkh_cm_ssd_blocks_used(self._h)
+    def prefetch_block(self, branch, logical): lib().drkh_cm_prefetch_block(self._h, branch, logical)
 
     def init_detached(self, max_blocks, block_size, scorer=None, max_branches=1):
         self._scorer = scorer

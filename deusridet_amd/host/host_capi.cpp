@@ -4,6 +4,7 @@
 
 #include "../machina/paged_attention.h"
 #include "../machina/layer.h"
+#include "../memoria/kv_swapper.h"
 #include "../memoria/cache_kernels.h"
 #include "../memoria/cache_manager.h"
 
@@ -13,6 +14,7 @@ using namespace deusridet;
 
 #define CM(p) (static_cast<CacheManager *>(p))
 #define SC(p) (static_cast<ImportanceScorer *>(p))
+#define SW(p) (static_cast<KVSwapper *>(p))
 #define H(p) (reinterpret_cast<__half *>(p))
 #define CH(p) (reinterpret_cast<const __half *>(p))
 #define ST(p) (static_cast<hipStream_t>(p))
@@ -41,6 +43,38 @@ void drkh_cm_destroy(void *cm) { delete CM(cm); }
 int drkh_cm_init(void *cm, size_t budget, int block_size, void *scorer, int max_branches)
 {
     return CM(cm)->init(budget, "", block_size, nullptr, SC(scorer), max_branches) ? 1 : 0;
+}
+int drkh_cm_init_ssd(void *cm, size_t budget, const char *cache_dir, int block_size, void *swapper, void *scorer,
+                     int max_branches)
+{
+    return CM(cm)->init(budget, cache_dir ? cache_dir : "", block_size, SW(swapper), SC(scorer), max_branches) ? 1 : 0;
+}
+int drkh_cm_ssd_blocks_used(void *cm) { return CM(cm)->ssd_blocks_used(); }
+void drkh_cm_prefetch_block(void *cm, int branch, int logical_idx) { CM(cm)->prefetch_block(branch, logical_idx); }
+void *drkh_swapper_create(void) { return new KVSwapper(); }
+void drkh_swapper_destroy(void *sw) { delete SW(sw); }
+int drkh_swapper_init(void *sw, void *cm, const char *ssd_dir, int staging_blocks)
+{
+    return SW(sw)->init(CM(cm)->block_pool(), ssd_dir ? ssd_dir : "", staging_blocks) ? 1 : 0;
+}
+void drkh_swapper_shutdown(void *sw) { SW(sw)->shutdown(); }
+void drkh_swapper_drain(void *sw) { SW(sw)->drain(); }
+int drkh_swapper_pending(void *sw) { return SW(sw)->pending(); }
+void drkh_swapper_prefetch(void *sw, int logical_block_idx, const char *path) { SW(sw)->prefetch(logical_block_idx, path ? path : ""); }
+int drkh_swapper_is_prefetched(void *sw, int logical_block_idx) { return SW(sw)->is_prefetched(logical_block_idx) ? 1 : 0; }
+size_t drkh_swapper_block_bytes(void *sw) { return SW(sw)->block_bytes(); }
+int drkh_swapper_swap(void *sw, int direction, int logical_block_idx, int physical_block_id, const char *path)
+{
+    bool success = false;
+    SwapRequest req;
+    req.direction = direction == 0 ? SwapDirection::GPU_TO_SSD : SwapDirection::SSD_TO_GPU;
+    req.logical_block_idx = logical_block_idx;
+    req.physical_block_id = physical_block_id;
+    req.ssd_path = path ? path : "";
+    req.callback = [&success](bool ok) { success = ok; };
+    SW(sw)->submit(std::move(req));
+    SW(sw)->drain();
+    return success ? 1 : 0;
 }
 int drkh_cm_init_detached(void *cm, int max_blocks, int block_size, void *scorer, int max_branches)
 {

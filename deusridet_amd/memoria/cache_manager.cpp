@@ -1,7 +1,11 @@
 // cache_manager.cpp -- see cache_manager.h.  Host bookkeeping only; the device is
 // reached through the C ABI (table upload, copy-on-write block copies).
 #include "cache_manager.h"
+#include "kv_swapper.h"
 #include "../communis/log.h"
+
+#include <sys/stat.h>
+#include <unistd.h>
 
 #include <algorithm>
 #include <unordered_set>
@@ -23,6 +27,7 @@ bool CacheManager::setup_tables(int max_branches)
     next_stamp_ = 1;
     evictable_.clear();
     refs_.assign(pool_.max_blocks(), {});
+    ssd_paths_.assign(cells, std::string());
     seq_len_.assign(max_branches_, 0);
     alive_.assign(max_branches_, 0);
     alive_[0] = 1;
@@ -39,11 +44,19 @@ bool CacheManager::init(size_t kv_budget_bytes, const std::string& cache_dir, in
     block_size_ = block_size;
     scorer_ = scorer;
     detached_ = false;
-    if (swapper || !cache_dir.empty())
-        LOG_WARN("Memoria", "CacheManager: the SSD tier is not part of this build; cache_dir/swapper ignored, "
-                            "evicted blocks are discarded");
+    swapper_ = swapper;
+    cache_dir_ = cache_dir;
     if (!pool_.init(kv_budget_bytes, block_size)) return false;
     setup_tables(max_branches);
+    // cache_manager.cpp:55-65: create the directory; without one the tier stays off
+    if (!cache_dir_.empty()) {
+        struct stat st;
+        if (stat(cache_dir_.c_str(), &st) != 0 && mkdir(cache_dir_.c_str(), 0755) != 0) {
+            LOG_WARN("Memoria", "Cannot create SSD cache dir: %s", cache_dir_.c_str());
+            cache_dir_.clear();
+        }
+    }
+    ssd_enabled_ = !cache_dir_.empty();
 
     size_t table_bytes = (size_t)max_branches_ * max_logical_blocks_ * sizeof(int);
     void* p = nullptr;
@@ -67,8 +80,8 @@ bool CacheManager::init(size_t kv_budget_bytes, const std::string& cache_dir, in
         destroy();
         return false;
     }
-    LOG_INFO("Memoria", "CacheManager: %d phys blocks, %d max logical, %d branches, SSD=disabled",
-             pool_.max_blocks(), max_logical_blocks_, max_branches_);
+    LOG_INFO("Memoria", "CacheManager: %d phys blocks, %d max logical, %d branches, SSD=%s", pool_.max_blocks(),
+             max_logical_blocks_, max_branches_, ssd_enabled_ ? cache_dir_.c_str() : "disabled");
     return true;
 }
 
@@ -77,6 +90,9 @@ bool CacheManager::init_detached(int max_blocks, int block_size, ImportanceScore
     destroy();
     block_size_ = block_size;
     scorer_ = scorer;
+    swapper_ = nullptr;
+    cache_dir_.clear();
+    ssd_enabled_ = false;
     detached_ = true;
     if (!pool_.init_detached(max_blocks, block_size)) return false;
     return setup_tables(max_branches);
@@ -142,14 +158,20 @@ int CacheManager::evict_nolock(int n)
         int c;
         if (!pick_victim_nolock(c)) break;
         int branch = c / max_logical_blocks_, logical = c % max_logical_blocks_;
+        BlockLocation where = BlockLocation::INVALID;
+        if (ssd_enabled_ && swapper_ && swapper_->ready()) {          // cache_manager.cpp:132-141
+            if (swap_to_ssd_nolock(c)) where = BlockLocation::SSD;
+            else LOG_WARN("Memoria", "SSD swap-out failed for block %d of branch %d, discarding", logical, branch);
+        }
         detach_nolock(c);                         // frees the block: it had one reference
-        location_[c] = BlockLocation::INVALID;
+        location_[c] = where;
         stamp_[c] = 0;
         mark_dirty(branch, logical);
         evicted++;
     }
     if (evicted > 0)
-        LOG_INFO("Memoria", "Evicted %d blocks (SSD=no), %d free now", evicted, pool_.free_count());
+        LOG_INFO("Memoria", "Evicted %d blocks (SSD=%s), %d free now", evicted,
+                 (ssd_enabled_ && swapper_ && swapper_->ready()) ? "yes" : "no", pool_.free_count());
     return evicted;
 }
 
@@ -196,10 +218,64 @@ bool CacheManager::ensure_nolock(int branch, int pos)
         }
         return true;
     }
+    if (location_[c] == BlockLocation::SSD) return swap_from_ssd_nolock(c);   // cache_manager.cpp:88-90
     int phys = alloc_phys_nolock();
     if (phys < 0) return false;
     attach_nolock(c, phys, true);                 // cache_manager.cpp:321-323
     mark_dirty(branch, logical);
+    return true;
+}
+
+// cache_manager.cpp:207-213; branch 0 keeps the reference's file names
+std::string CacheManager::ssd_path_for(int c) const
+{
+    int branch = c / max_logical_blocks_, logical = c % max_logical_blocks_;
+    std::string name = branch == 0 ? "block_" + std::to_string(logical) : "b" + std::to_string(branch) + "_block_" + std::to_string(logical);
+    return cache_dir_ + "/" + name + ".kv";
+}
+
+// cache_manager.cpp:215-243: synchronous on the eviction path; the caller frees the block
+bool CacheManager::swap_to_ssd_nolock(int c)
+{
+    int phys = h_tables_[c];
+    if (phys < 0) return false;
+    std::string path = ssd_path_for(c);
+    bool success = false;
+    SwapRequest req;
+    req.direction = SwapDirection::GPU_TO_SSD;
+    req.logical_block_idx = c;
+    req.physical_block_id = phys;
+    req.ssd_path = path;
+    req.callback = [&success](bool ok) { success = ok; };
+    swapper_->drop_prefetch(c);                   // a stale prefetched image must not outlive the new file
+    swapper_->submit(std::move(req));
+    swapper_->drain();
+    if (success) ssd_paths_[c] = path;
+    return success;
+}
+
+// cache_manager.cpp:245-292.  The fresh block comes from the ordinary allocation path (which
+// may evict, and swap out, another block first: requests are executed one after the other).
+bool CacheManager::swap_from_ssd_nolock(int c)
+{
+    if (!swapper_ || !swapper_->ready()) return false;
+    int phys = alloc_phys_nolock();
+    if (phys < 0) return false;
+    bool success = false;
+    SwapRequest req;
+    req.direction = SwapDirection::SSD_TO_GPU;
+    req.logical_block_idx = c;
+    req.physical_block_id = phys;
+    req.ssd_path = ssd_paths_[c];
+    req.callback = [&success](bool ok) { success = ok; };
+    swapper_->submit(std::move(req));
+    swapper_->drain();
+    if (!success) {
+        pool_.free_block(phys);
+        return false;
+    }
+    attach_nolock(c, phys, true);                 // back of the LRU order (cache_manager.cpp:290)
+    mark_dirty(c / max_logical_blocks_, c % max_logical_blocks_);
     return true;
 }
 
@@ -327,6 +403,13 @@ void CacheManager::release_branch(int branch)
     if (branch < 0 || branch >= max_branches_ || !alive_[branch]) return;
     for (int l = 0; l < max_logical_blocks_; l++) {
         int c = (int)cell(branch, l);
+        if (location_[c] == BlockLocation::SSD) {             // forget the swapped-out copy
+            if (swapper_) swapper_->drop_prefetch(c);
+            unlink(ssd_paths_[c].c_str());
+            ssd_paths_[c].clear();
+            location_[c] = BlockLocation::INVALID;
+            continue;
+        }
         if (location_[c] != BlockLocation::GPU) continue;
         detach_nolock(c);
         location_[c] = BlockLocation::INVALID;
@@ -397,7 +480,23 @@ bool CacheManager::ensure_free_blocks(int n_free)
     return ensure_free_nolock(n_free);
 }
 
-void CacheManager::prefetch_block(int) {}
+void CacheManager::prefetch_block(int branch, int logical_idx)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (branch < 0 || branch >= max_branches_ || logical_idx < 0 || logical_idx >= max_logical_blocks_) return;
+    int c = (int)cell(branch, logical_idx);
+    if (location_[c] != BlockLocation::SSD || !swapper_ || !swapper_->ready()) return;
+    swapper_->prefetch(c, ssd_paths_[c]);         // fire and forget (cache_manager.cpp:171-178)
+}
+
+int CacheManager::ssd_blocks_used() const
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    int n = 0;
+    for (BlockLocation loc : location_)
+        if (loc == BlockLocation::SSD) n++;
+    return n;
+}
 
 int CacheManager::gpu_blocks_used() const { return pool_.max_blocks() - pool_.free_count(); }
 

@@ -18,9 +18,14 @@
 //   - sync_block_table() uploads only the table ranges that changed (the
 //     reference re-sends the whole table every step, cache_manager.cpp:108-112).
 //
-// The SSD tier (KVSwapper) is not part of this build: a non-null swapper is
-// refused, blocks are discarded on eviction (the reference's path without a
-// swapper, cache_manager.cpp:143-147).
+// Overflow tier: with a cache_dir and a KVSwapper (initialised by the caller on
+// block_pool() after init(), as the reference's two-step set-up implies), an
+// evicted block is written to <cache_dir>/block_<logical>.kv (branch 0; other
+// branches: b<branch>_block_<logical>.kv) and its entry becomes SSD;
+// ensure_blocks_for() on such an entry brings it back into a fresh physical block
+// (cache_manager.cpp:118-156, 207-292).  Without them blocks are discarded
+// (cache_manager.cpp:143-147).  Only unshared blocks are ever evicted, so a block
+// on SSD belongs to exactly one table entry; fork_branch() treats it as a hole.
 #pragma once
 
 #include "block_pool.h"
@@ -34,7 +39,7 @@
 
 namespace deusridet {
 
-class KVSwapper;   // SSD tier: declared for signature compatibility only
+class KVSwapper;
 
 enum class BlockLocation : int8_t {   // cache_manager.h:42-46
     GPU = 0,
@@ -101,13 +106,14 @@ public:
     // ---- eviction -------------------------------------------------------------
     int  evict_blocks(int n);                  // cache_manager.cpp:118-156
     bool ensure_free_blocks(int n_free);       // cache_manager.cpp:158-164
-    void prefetch_block(int logical_idx);      // SSD tier absent: no-op (cache_manager.cpp:166-179)
+    void prefetch_block(int logical_idx) { prefetch_block(0, logical_idx); }   // cache_manager.cpp:166-179
+    void prefetch_block(int branch, int logical_idx);
 
     BlockPool& block_pool() { return pool_; }
     const BlockPool& block_pool() const { return pool_; }
 
     int gpu_blocks_used() const;               // cache_manager.cpp:294-296
-    int ssd_blocks_used() const { return 0; }
+    int ssd_blocks_used() const;               // cache_manager.cpp:298-304
     int free_blocks() const { return pool_.free_count(); }
 
     // LRU order, oldest first, as (branch, logical) pairs (tests, state dumps).
@@ -120,6 +126,10 @@ public:
 private:
     BlockPool pool_;
     ImportanceScorer* scorer_ = nullptr;       // not owned (cache_manager.h:129-130)
+    KVSwapper* swapper_ = nullptr;             // not owned
+    std::string cache_dir_;
+    bool ssd_enabled_ = false;
+    std::vector<std::string> ssd_paths_;       // per cell, set while the block is on SSD
     int max_logical_blocks_ = 0;
     int max_branches_ = 0;
     int block_size_ = PagedKVConfig::BLOCK_SIZE;
@@ -151,6 +161,9 @@ private:
     int  evict_nolock(int n);
     bool ensure_free_nolock(int n_free);
     bool pick_victim_nolock(int& cell_out);
+    std::string ssd_path_for(int cell_idx) const;
+    bool swap_to_ssd_nolock(int cell_idx);
+    bool swap_from_ssd_nolock(int cell_idx);
     void attach_nolock(int cell_idx, int phys, bool fresh_stamp);
     void detach_nolock(int cell_idx);
     void flush_copies(hipStream_t stream);

@@ -37,6 +37,24 @@ void  drkh_scorer_load_host_scores(void *s, const float *scores, int n);
 void *drkh_cm_create(void);
 void  drkh_cm_destroy(void *cm);
 int   drkh_cm_init(void *cm, size_t kv_budget_bytes, int block_size, void *scorer, int max_branches);
+/* with the overflow tier: cache_dir and a KVSwapper (src/memoria/cache_manager.h:60-64); the swapper is
+ * initialised afterwards on the manager's pool with drkh_swapper_init */
+int   drkh_cm_init_ssd(void *cm, size_t kv_budget_bytes, const char *cache_dir, int block_size, void *swapper,
+                       void *scorer, int max_branches);
+int   drkh_cm_ssd_blocks_used(void *cm);
+void  drkh_cm_prefetch_block(void *cm, int branch, int logical_idx);
+/* src/memoria/kv_swapper.h:50-114 */
+void *drkh_swapper_create(void);
+void  drkh_swapper_destroy(void *sw);
+int   drkh_swapper_init(void *sw, void *cm, const char *ssd_dir, int staging_blocks);
+void  drkh_swapper_shutdown(void *sw);
+void  drkh_swapper_drain(void *sw);
+int   drkh_swapper_pending(void *sw);
+void  drkh_swapper_prefetch(void *sw, int logical_block_idx, const char *path);
+int   drkh_swapper_is_prefetched(void *sw, int logical_block_idx);
+size_t drkh_swapper_block_bytes(void *sw);
+/* one synchronous request through the queue: direction 0 = GPU -> file, 1 = file -> GPU; returns success */
+int   drkh_swapper_swap(void *sw, int direction, int logical_block_idx, int physical_block_id, const char *path);
 int   drkh_cm_init_detached(void *cm, int max_blocks, int block_size, void *scorer, int max_branches);
 int   drkh_cm_ensure_blocks_for(void *cm, int branch, int pos);
 int   drkh_cm_ensure_blocks_for_range(void *cm, int branch, int pos_start, int M);

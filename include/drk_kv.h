@@ -97,6 +97,18 @@ int drk_dev_free(void *d_ptr);
 int drk_dev_memset_async(void *d_ptr, int byte, size_t bytes, void *stream);
 int drk_memcpy_h2d_async(void *d_dst, const void *h_src, size_t bytes, void *stream);
 int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream); /* syncs */
+/* Waits for all work on every stream of the current device. */
+int drk_device_synchronize(void);
+/* Pinned host memory (allocated pinned, for staging buffers). */
+int drk_host_malloc(void **h_ptr, size_t bytes);
+int drk_host_free(void *h_ptr);
+/* One physical block, all layers, to / from a contiguous host image of
+ * drk_kv_block_total_bytes(): [layer][K plane | V plane (| K scales | V scales)], the
+ * order KVSwapper writes its .kv files in (kv_swapper.cpp:183-198, 268-283).
+ * Asynchronous on `stream`; the host side should be pinned. */
+size_t drk_kv_block_total_bytes(const drk_kv_layout *g);
+int drk_kv_block_to_host(const drk_kv_layout *g, const void *pool, int blk, void *h_dst, void *stream);
+int drk_kv_block_from_host(const drk_kv_layout *g, void *pool, int blk, const void *h_src, void *stream);
 int drk_stream_create(void **stream);
 int drk_stream_destroy(void *stream);
 int drk_stream_synchronize(void *stream);

@@ -52,6 +52,8 @@ def lib():
         "orc_extract": (None, [P, vp, vp, vp, vp, i32, i32, i32]),
         "orc_inject": (None, [P, vp, vp, vp, vp, i32, i32, i32]),
         "orc_copy_block": (None, [P, vp, i32, i32]),
+        "orc_block_image": (None, [P, vp, i32, vp]),
+        "orc_block_from_image": (None, [P, vp, i32, vp]),
         "orc_block_attention_mass": (None, [P, vp, vp, vp, i32, vp, i32, i32, f64, i32, vp, i32]),
         "orc_split_q_gate": (None, [vp, vp, vp, i32, i32, i32]),
         "orc_head_norm": (None, [vp, vp, vp, i32, i32, f32, i32]),
@@ -134,6 +136,18 @@ def inject(g, pool, src, src_scales, table, start, n, num_layers):
 
 def copy_block(g, pool, src, dst):
     lib().orc_copy_block(C.byref(g), ptr(pool), src, dst)
+
+
+def block_image(g, pool, blk):
+    """bytes of the .kv file image of physical block blk (all layers)"""
+    out = np.empty(g.L * lib().orc_block_stride_bytes(C.byref(g)), np.uint8)
+    lib().orc_block_image(C.byref(g), ptr(pool), blk, ptr(out))
+    return out
+
+
+def block_from_image(g, pool, blk, image):
+    image = np.ascontiguousarray(image, dtype=np.uint8)
+    lib().orc_block_from_image(C.byref(g), ptr(pool), blk, ptr(image))
 
 
 def decode_ref_order(g, q, pool, table, layer, seq_len, scale, io_dtype, out=None):

@@ -178,6 +178,24 @@ int orc_max_blocks_for_budget(const orc_layout *g, size_t budget_bytes)
     return (int)(budget_bytes / per_block);
 }
 
+/* The consolidated image of one physical block that KVSwapper::swap_out writes to its
+ * .kv file (kv_swapper.cpp:183-198): for every layer the block's K plane, then its V
+ * plane (then, for int8 pools, the two scale planes) -- i.e. the block's bytes of each
+ * layer, layers in order. */
+void orc_block_image(const orc_layout *g, const void *pool, int blk, void *out)
+{
+    size_t bs = orc_block_stride_bytes(g), ls = orc_layer_stride_bytes(g);
+    for (int l = 0; l < g->L; l++)
+        memcpy((uint8_t *)out + (size_t)l * bs, (const uint8_t *)pool + (size_t)l * ls + (size_t)blk * bs, bs);
+}
+
+void orc_block_from_image(const orc_layout *g, void *pool, int blk, const void *image)
+{
+    size_t bs = orc_block_stride_bytes(g), ls = orc_layer_stride_bytes(g);
+    for (int l = 0; l < g->L; l++)
+        memcpy((uint8_t *)pool + (size_t)l * ls + (size_t)blk * bs, (const uint8_t *)image + (size_t)l * bs, bs);
+}
+
 /* ======================================================================== */
 /* codecs                                                                   */
 /* ======================================================================== */

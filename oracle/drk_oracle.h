@@ -69,6 +69,9 @@ void orc_inject(const orc_layout *g, void *pool, const void *src,
                 const void *src_scales, const int32_t *table, int start_token,
                 int num_tokens, int num_layers);
 void orc_copy_block(const orc_layout *g, void *pool, int src_blk, int dst_blk);
+/* the .kv file image of one block, all layers (kv_swapper.cpp:183-198, 268-283) */
+void orc_block_image(const orc_layout *g, const void *pool, int blk, void *out);
+void orc_block_from_image(const orc_layout *g, void *pool, int blk, const void *image);
 
 /* ---- codecs (builder-specified; precedent layer_int8_dual.cu:239-293) ---- */
 /* one row of D elements -> D int8 codes + one fp16 scale */

@@ -487,3 +487,28 @@ def test_block_attention_mass_closed_forms():
     orc.append_batch(g, pool3, tables[0], 0, 0, kd, v, orc.BF16)
     m3 = orc.block_attention_mass(g, qd, pool3, tables[:1], lens[:1], 0, 1.0, orc.BF16, 5)
     assert abs(m3[0, 1] - QH) < 1e-9
+
+
+@pytest.mark.parametrize("dtype", [orc.F16, orc.INT8])
+def test_block_image_is_k_then_v_per_layer(dtype):
+    """kv_swapper.cpp:183-198: for each layer the K plane of the block, then the V plane."""
+    L, KVH, QH, D, bs, NB = 3, 2, 4, 16, 4, 5
+    g = orc.layout(L, KVH, QH, D, bs, NB, dtype)
+    lib = orc.lib()
+    rng = np.random.default_rng(56)
+    pool = rng.integers(0, 256, size=orc.pool_bytes(g)).astype(np.uint8)
+    blk = 3
+    img = orc.block_image(g, pool, blk)
+    plane = lib.orc_kv_plane_bytes(C.byref(g))
+    bstride = lib.orc_block_stride_bytes(C.byref(g))
+    assert img.size == L * bstride
+    for l in range(L):
+        k0, v0 = lib.orc_k_off(C.byref(g), l, blk, 0, 0, 0), lib.orc_v_off(C.byref(g), l, blk, 0, 0, 0)
+        assert np.array_equal(img[l * bstride:l * bstride + plane], pool[k0:k0 + plane])
+        assert np.array_equal(img[l * bstride + plane:l * bstride + 2 * plane], pool[v0:v0 + plane])
+        if dtype == orc.INT8:
+            s0 = lib.orc_kscale_off(C.byref(g), l, blk, 0, 0)
+            assert np.array_equal(img[l * bstride + 2 * plane:(l + 1) * bstride], pool[s0:s0 + bstride - 2 * plane])
+    pool2 = np.zeros_like(pool)
+    orc.block_from_image(g, pool2, 1, img)
+    assert np.array_equal(orc.block_image(g, pool2, 1), img) and pool2.sum() == img.astype(np.int64).sum()
