@@ -28,7 +28,14 @@
 namespace drk {
 
 constexpr int kPfBN = 64;         // KV tokens per tile
-constexpr int kPfPitch = 272;     // LDS bytes per staged row (256 + 16)
+// LDS bytes per staged row.  The LDS has 32 four-byte banks.  K rows are read whole-row
+// (lane = token, 16 bytes per lane, 8 lanes per clock): consecutive rows must start 4 banks
+// apart -> 256 + 16.  V rows are read transposed (16 lanes per clock touch 4 consecutive
+// rows, 4 x 8 bytes each): consecutive rows must start 8 banks apart -> 256 + 32; with the
+// K pitch every other row pair collides (measured: half of the LDS-active cycles were
+// bank-conflict cycles).
+constexpr int kPfPitch = 272;
+constexpr int kPfPitchV = 288;
 constexpr int kPfRows = 128;      // rows per workgroup (32 query tokens x 4 heads)
 constexpr float kLog2eP = 1.4426950408889634f;
 
@@ -66,6 +73,32 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi)
     }
 }
 
+// acc + the eight 16-bit values packed in v
+template <int DT>
+__device__ __forceinline__ float pf_sum2(const uint4 &v, float acc)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (DT == DRK_BF16) {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        const b2 one = {(__bf16)1.0f, (__bf16)1.0f};
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, v.x), one, acc, false);
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, v.y), one, acc, false);
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, v.z), one, acc, false);
+        acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, v.w), one, acc, false);
+    } else {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.x), one, acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.y), one, acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.z), one, acc, false);
+        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, v.w), one, acc, false);
+    }
+#else
+    (void)v;
+#endif
+    return acc;
+}
+
 // LDS transpose read: the 16 lanes of a group pass 16 addresses of 4 consecutive
 // 16-bit elements; lane i receives, for k = 0..3, element (i % 4) at the address
 // given by lane (i / 4 + 4 * k) of its group.
@@ -97,6 +130,21 @@ struct PrefillArgs {
     size_t gate_stride;
 };
 
+// scheduling hints: order instruction groups inside one basic block
+template <int MASK, int N>
+__device__ __forceinline__ void pf_sched_group()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
+#endif
+}
+__device__ __forceinline__ void pf_sched_barrier()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+}
+
 struct PfGroup {
     uint4 r0, r1, r2, r3;
 };
@@ -123,13 +171,14 @@ __device__ __forceinline__ PfGroup pf_load_group(const uint8_t *__restrict__ bas
     return g;
 }
 
+template <int PITCH>
 __device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, int w, int lane)
 {
-    uint8_t *dst = lds + (w * 16 + (lane >> 4)) * kPfPitch + (lane & 15) * 16;
+    uint8_t *dst = lds + (w * 16 + (lane >> 4)) * PITCH + (lane & 15) * 16;
     *(uint4 *)(dst) = g.r0;
-    *(uint4 *)(dst + 4 * kPfPitch) = g.r1;
-    *(uint4 *)(dst + 8 * kPfPitch) = g.r2;
-    *(uint4 *)(dst + 12 * kPfPitch) = g.r3;
+    *(uint4 *)(dst + 4 * PITCH) = g.r1;
+    *(uint4 *)(dst + 8 * PITCH) = g.r2;
+    *(uint4 *)(dst + 12 * PITCH) = g.r3;
 }
 
 // grid = (ceil(M/32) * KVH, 1[, splits]); block = 256.
@@ -140,9 +189,12 @@ __device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, i
 template <int DT, bool SHARED>
 __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
 {
-    __shared__ __align__(16) uint8_t k_lds[kPfBN * kPfPitch];
-    __shared__ __align__(16) uint8_t v_lds[kPfBN * kPfPitch];
-    __shared__ int valid_lds[4];
+    // Two buffers per operand.  The loop is software-pipelined by one tile: while the softmax of
+    // tile i runs on the vector ALU, the matrix cores already compute the scores of tile i+1, so
+    // K is staged one tile further ahead than V.  One barrier per tile.
+    __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPfPitch];
+    __shared__ __align__(16) uint8_t v_lds2[2][kPfBN * kPfPitchV];
+    __shared__ int valid_lds4[4][4];                       // page present, per (tile & 3, 16-token group)
 
     // Workgroups are dealt to the 8 XCDs round-robin by linear id; kv head = id % KVH
     // keeps one kv head's pages in one XCD's L2 (8 kv heads on 8 XCDs).
@@ -195,67 +247,107 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;
 
-    bool cur_valid, nxt_valid = false;
-    size_t off = lookup(t_begin, cur_valid);
-    PfGroup kreg = pf_load_group<SHARED>(kbase, cur_valid, off, lane);
-    PfGroup vreg = pf_load_group<SHARED>(kbase + A.kv_plane, cur_valid, off, lane);
-
-    for (int it = t_begin; it < ntiles; it++) {
-        const int tile_t = it * kPfBN;
-        // ---- stage the tile; rows at or past the workgroup's limit may hold anything ----
-        if (tile_t + kPfBN > lim_wg) {
-            const int lim = lim_wg - tile_t - w * 16 - (lane >> 4);   // rows r0, r0+4, ... of this lane
+    // registers -> LDS; rows at or past the workgroup's limit may hold anything and are cleared
+    bool kreg_valid = false;
+    PfGroup kreg, vreg;
+    auto clear_tail = [&](PfGroup &r, int tile) {
+        const int tile_t0 = tile * kPfBN;
+        if (tile_t0 + kPfBN > lim_wg) {
+            const int lim = lim_wg - tile_t0 - w * 16 - (lane >> 4);   // rows r0, r0+4, ... of this lane
             const uint4 z = make_uint4(0, 0, 0, 0);
-            if (0 >= lim) { vreg.r0 = z; kreg.r0 = z; }
-            if (4 >= lim) { vreg.r1 = z; kreg.r1 = z; }
-            if (8 >= lim) { vreg.r2 = z; kreg.r2 = z; }
-            if (12 >= lim) { vreg.r3 = z; kreg.r3 = z; }
+            if (0 >= lim) r.r0 = z;
+            if (4 >= lim) r.r1 = z;
+            if (8 >= lim) r.r2 = z;
+            if (12 >= lim) r.r3 = z;
         }
-        pf_store_group(k_lds, kreg, w, lane);
-        pf_store_group(v_lds, vreg, w, lane);
-        if (lane == 0) valid_lds[w] = cur_valid ? 1 : 0;
+    };
+    auto fetch_k = [&](int tile) {
+        const size_t off = lookup(tile, kreg_valid);
+        kreg = pf_load_group<SHARED>(kbase, kreg_valid, off, lane);
+    };
+    auto fetch_v = [&](int tile) {
+        bool ok;
+        const size_t off = lookup(tile, ok);
+        vreg = pf_load_group<SHARED>(kbase + A.kv_plane, ok, off, lane);
+    };
+    auto stage_k = [&](int tile) {
+        clear_tail(kreg, tile);
+        pf_store_group<kPfPitch>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane);
+        if (lane == 0) valid_lds4[tile & 3][w] = kreg_valid ? 1 : 0;
+    };
+    auto stage_v = [&](int tile) {
+        clear_tail(vreg, tile);
+        pf_store_group<kPfPitchV>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane);
+    };
+    // S^T = K Q^T : two 32-token tiles x 32 rows, 8 k-steps of 16 dims
+    auto qk = [&](int tile, pf_f32x16 (&s)[2]) {
+        const uint8_t *ka = &k_lds2[(tile - t_begin) & 1][0] + n * kPfPitch + g * 16;
+        const pf_f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};     // constant C operand of the first k-step
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            const uint4 a0 = *(const uint4 *)(ka + ks * 32);
+            const uint4 a1 = *(const uint4 *)(ka + 32 * kPfPitch + ks * 32);
+            s[0] = mfma32<DT>(a0, qf[ks], ks == 0 ? zero : s[0]);
+            s[1] = mfma32<DT>(a1, qf[ks], ks == 0 ? zero : s[1]);
+        }
+    };
+
+    pf_f32x16 s_even[2], s_odd[2];          // scores of the tiles at even / odd distance from t_begin
+    pf_f32x16 (&s)[2] = s_even;
+    if (t_begin < ntiles) {
+        fetch_k(t_begin);
+        fetch_v(t_begin);
+        stage_k(t_begin);
+        stage_v(t_begin);
+        if (t_begin + 1 < ntiles) {
+            fetch_k(t_begin + 1);
+            fetch_v(t_begin + 1);
+        }
+    }
+    __syncthreads();
+    if (t_begin < ntiles) {
+        qk(t_begin, s);
+        if (t_begin + 1 < ntiles) {
+            stage_k(t_begin + 1);
+            if (t_begin + 2 < ntiles) fetch_k(t_begin + 2);
+        }
+    }
+    __syncthreads();
+
+    auto tile_step = [&](int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
+        // here: s = scores of tile it; K(it+1) and V(it) are in LDS; kreg holds K(it+2), vreg V(it+1)
+        const int tile_t = it * kPfBN;
+        const uint8_t *v_lds = &v_lds2[(it - t_begin) & 1][0];
+        const int *valid_lds = &valid_lds4[it & 3][0];
+        if (it + 2 < ntiles) {
+            stage_k(it + 2);                       // into the buffer K(it) was read from one iteration ago
+            if (it + 3 < ntiles) fetch_k(it + 3);
+        }
         if (it + 1 < ntiles) {
-            off = lookup(it + 1, nxt_valid);
-            kreg = pf_load_group<SHARED>(kbase, nxt_valid, off, lane);
-            vreg = pf_load_group<SHARED>(kbase + A.kv_plane, nxt_valid, off, lane);
+            stage_v(it + 1);                       // into the buffer V(it-1) was read from
+            if (it + 2 < ntiles) fetch_v(it + 2);
         }
-        __syncthreads();
-
-        // ---- S^T = K Q^T : two 32-token tiles x 32 rows, 8 k-steps of 16 dims ----
-        pf_f32x16 s[2];
-#pragma unroll
-        for (int i = 0; i < 16; i++) { s[0][i] = 0.0f; s[1][i] = 0.0f; }
-        {
-            const uint8_t *ka = k_lds + n * kPfPitch + g * 16;
-#pragma unroll
-            for (int ks = 0; ks < 8; ks++) {
-                const uint4 a0 = *(const uint4 *)(ka + ks * 32);
-                const uint4 a1 = *(const uint4 *)(ka + 32 * kPfPitch + ks * 32);
-                s[0] = mfma32<DT>(a0, qf[ks], s[0]);
-                s[1] = mfma32<DT>(a1, qf[ks], s[1]);
-            }
-        }
-
         // ---- tile softmax for this lane's row; register i of tile tt is token
         //      tile_t + tt*32 + 8*(i/4) + 4*g + i%4 ----
         const bool all_groups_valid = (valid_lds[0] & valid_lds[1] & valid_lds[2] & valid_lds[3]) != 0;
         const bool need_mask = !all_groups_valid ||
                                (SHARED ? (__any(tile_t + kPfBN > vis) != 0) : (it >= first_masked_tile));
         // raw scores stay in s; the scale (> 0) is folded into the exponent's fma
+        if (need_mask) {                                         // one uniform branch around all 32 selects
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    const bool ok = (tile_t + tl) < vis && valid_lds[tl >> 4] != 0;
+                    s[tt][i] = ok ? s[tt][i] : -INFINITY;
+                }
+        }
         float tmax = -INFINITY;
 #pragma unroll
         for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float v = s[tt][i];
-                if (need_mask) {
-                    const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-                    const bool ok = (tile_t + tl) < vis && valid_lds[tl >> 4] != 0;
-                    v = ok ? v : -INFINITY;
-                    s[tt][i] = v;
-                }
-                tmax = fmaxf(tmax, v);
-            }
+            for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[tt][i]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32));               // the row's other 32 tokens
         const float m_new = fmaxf(m_run, tmax * A.scale_log2e);
         const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
@@ -266,12 +358,12 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         for (int tt = 0; tt < 2; tt++) {
             float p[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                p[i] = __builtin_amdgcn_exp2f(fmaf(s[tt][i], A.scale_log2e, -m_use));
-                psum += p[i];
-            }
+            for (int i = 0; i < 16; i++) p[i] = __builtin_amdgcn_exp2f(fmaf(s[tt][i], A.scale_log2e, -m_use));
             pb[tt][0] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
             pb[tt][1] = make_uint4(pack2<DT>(p[8], p[9]), pack2<DT>(p[10], p[11]), pack2<DT>(p[12], p[13]), pack2<DT>(p[14], p[15]));
+            // the row sum is taken over the rounded weights, the ones PV multiplies: one dot2 per pair
+            psum = pf_sum2<DT>(pb[tt][0], psum);
+            psum = pf_sum2<DT>(pb[tt][1], psum);
         }
         l_run = l_run * alpha + psum;
         m_run = m_new;
@@ -282,26 +374,35 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
                 for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
         }
 
+        // The next tile's scores, in the same basic block as the exponentials and the PV product so
+        // that matrix and vector instructions alternate.  Unconditional: past the last tile it
+        // multiplies whatever the other K buffer holds and the result is dropped.
+        qk(it + 1, s_next);
+
         // ---- O^T += V^T P^T : k-slot j of MFMA (tt, mh) is token tt*32 + 16*mh + 8*(j/4) + 4*g + j%4 ----
         {
             const int j16 = lane & 15;
             const int dsub = 16 * ((lane >> 4) & 1) + 4 * (j16 & 3);           // d offset inside a 32-d tile
-            const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPfPitch + dsub * 2;
+            const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPfPitchV + dsub * 2;
 #pragma unroll
             for (int tt = 0; tt < 2; tt++)
 #pragma unroll
                 for (int mh = 0; mh < 2; mh++) {
-                    const uint8_t *vt = vb + (tt * 32 + 16 * mh) * kPfPitch;
+                    const uint8_t *vt = vb + (tt * 32 + 16 * mh) * kPfPitchV;
 #pragma unroll
                     for (int dt = 0; dt < 4; dt++) {
                         const uint2 lo = lds_read_tr16(vt + dt * 64);
-                        const uint2 hi = lds_read_tr16(vt + 8 * kPfPitch + dt * 64);
+                        const uint2 hi = lds_read_tr16(vt + 8 * kPfPitchV + dt * 64);
                         o[dt] = mfma32<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pb[tt][mh], o[dt]);
                     }
                 }
         }
-        cur_valid = nxt_valid;
         __syncthreads();
+    };
+    // two tiles per trip, the two score register sets swapping roles (no copies)
+    for (int it = t_begin; it < ntiles; it += 2) {
+        tile_step(it, s_even, s_odd);
+        if (it + 1 < ntiles) tile_step(it + 1, s_odd, s_even);
     }
 
     // ---- register i of tile dt is d = dt*32 + 8*(i/4) + 4*g + i%4 ----
