@@ -424,9 +424,17 @@ def main():
             reps += 1
         dt = time.time() - t0
         cpu_bytes = reps * B * n_cpu * kv_bytes_per_token
+        # the same loop on one thread, a shorter sample
+        t1 = time.time()
+        reps1 = 0
+        while time.time() - t1 < 4.0:
+            orc.decode_branches(og, hq, hp, htab, lens, 0, float(scale), orc.BF16, threads=1)
+            reps1 += 1
+        dt1 = time.time() - t1
         cpu = {"value": cpu_bytes / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": f"{reps} x (1 layer, {B} branches x {n_cpu} tokens) of the same decode attention, "
-                         f"oracle's reference-order loop, OpenMP over (branch, q head)"}
+                         f"oracle's reference-order loop, OpenMP over (branch, q head)",
+               "single_thread_value": reps1 * B * n_cpu * kv_bytes_per_token / dt1 / 1e9}
 
     tokens_per_s = B * K / (total_ms * 1e-3)
     line = {
