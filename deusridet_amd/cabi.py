@@ -54,6 +54,11 @@ SIGNATURES = {
     "drk_dev_memset_async": (_i32, [_vp, _i32, _sz, _vp]),
     "drk_memcpy_h2d_async": (_i32, [_vp, _vp, _sz, _vp]),
     "drk_memcpy_d2h": (_i32, [_vp, _vp, _sz, _vp]),
+    "drk_positions_advance": (_i32, [_vp, _vp, _i32, _i32, _vp]),
+    "drk_graph_begin_capture": (_i32, [_vp]),
+    "drk_graph_end_capture": (_i32, [_vp, C.POINTER(_vp)]),
+    "drk_graph_launch": (_i32, [_vp, _vp]),
+    "drk_graph_destroy": (_i32, [_vp]),
     "drk_device_synchronize": (_i32, []),
     "drk_host_malloc": (_i32, [C.POINTER(_vp), _sz]),
     "drk_host_free": (_i32, [_vp]),

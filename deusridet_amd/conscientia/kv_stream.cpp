@@ -1,0 +1,261 @@
+// kv_stream.cpp -- see kv_stream.h.
+#include "kv_stream.h"
+#include "../communis/log.h"
+#include "drk_kv.h"
+
+#include <cmath>
+
+namespace deusridet {
+
+KvStream::~KvStream() { destroy(); }
+
+bool KvStream::init(CacheManager& cm, int max_context_len, ImportanceScorer* scorer, const float* d_rope_table,
+                    int table_positions)
+{
+    destroy();
+    cm_ = &cm;
+    scorer_ = scorer;
+    d_rope_table_ = d_rope_table;
+    table_positions_ = table_positions;
+    max_context_len_ = max_context_len;
+    current_pos_ = cm.seq_len(0);
+    void* p = nullptr;
+    size_t bytes = (size_t)cm.max_branches() * sizeof(int);
+    if (drk_dev_malloc(&p, bytes) != DRK_OK) {
+        LOG_ERROR("Conscientia", "KvStream: position buffer: %s", drk_last_error());
+        return false;
+    }
+    d_pos_ = static_cast<int*>(p);
+    if (drk_dev_malloc(&p, bytes) != DRK_OK) {
+        LOG_ERROR("Conscientia", "KvStream: length buffer: %s", drk_last_error());
+        destroy();
+        return false;
+    }
+    d_len_ = static_cast<int*>(p);
+    // every attention call below finds its split-K workspace ready: nothing allocates later
+    if (!paged_attention_reserve_workspace(cm.max_branches(), max_context_len, 0, cm.block_pool().block_size())) {
+        destroy();
+        return false;
+    }
+    return true;
+}
+
+void KvStream::destroy()
+{
+    if (graph_) {
+        drk_graph_destroy(graph_);
+        graph_ = nullptr;
+    }
+    if (cm_) close_branches();
+    if (d_pos_) drk_dev_free(d_pos_);
+    if (d_len_) drk_dev_free(d_len_);
+    d_pos_ = d_len_ = nullptr;
+    cm_ = nullptr;
+    scorer_ = nullptr;
+    positions_on_device_ = false;
+}
+
+// ---- perception (stream.cpp:145-238) -----------------------------------------------------------
+
+bool KvStream::begin_prefill(int M, hipStream_t stream)
+{
+    if (!cm_ || M <= 0) return M == 0;
+    if (!branches_.empty()) {
+        LOG_ERROR("Conscientia", "KvStream: prefill while decode branches are open");
+        return false;
+    }
+    if (current_pos_ + M > max_context_len_) {
+        LOG_ERROR("Conscientia", "KvStream: context of %d tokens exceeds max_context_len %d", current_pos_ + M, max_context_len_);
+        return false;
+    }
+    if (!cm_->ensure_blocks_for_range(0, current_pos_, M)) {              // stream.cpp:151-155
+        LOG_ERROR("Conscientia", "Block allocation failed for pos=%d M=%d", current_pos_, M);
+        return false;
+    }
+    cm_->sync_block_table(stream);                                        // stream.cpp:156
+    return true;
+}
+
+void KvStream::prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipStream_t stream)
+{
+    const BlockPool& pool = cm_->block_pool();
+    const int hd = ModelConfig::HEAD_DIM;
+    // steps 4-9 of full_attention_forward_paged_prefill (paged_attention.cu:589-634) in two launches
+    paged_qk_norm_rope_write_batch(io.qg, io.k, io.v, io.q_norm, io.k_norm, io.q_scratch, pool.pool_ptr(),
+                                   cm_->d_block_table(0), fa_layer_idx, current_pos_, M, pool.max_blocks(),
+                                   pool.block_size(), d_rope_table_, table_positions_, stream);
+    paged_prefill_attention_gated(io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), io.qg + hd, 2 * hd, io.attn_out,
+                                  fa_layer_idx, current_pos_, M, pool.max_blocks(), pool.block_size(),
+                                  1.0f / std::sqrt((float)hd), stream);
+}
+
+void KvStream::end_prefill(int M)
+{
+    current_pos_ += M;                                                    // stream.cpp:238-239
+    cm_->set_seq_len(0, current_pos_);
+}
+
+// ---- decode branches ------------------------------------------------------------------------------
+
+int KvStream::open_branches(int n)
+{
+    if (!cm_ || !branches_.empty()) return 0;
+    for (int i = 0; i < n; i++) {
+        int id = cm_->fork_branch(0, current_pos_);
+        if (id < 0) break;
+        // launches address the branches' table rows as one [B, stride] array: ids must be consecutive
+        if (!branches_.empty() && id != branches_.back() + 1) {
+            cm_->release_branch(id);
+            break;
+        }
+        branches_.push_back(id);
+        pos_.push_back(current_pos_);
+    }
+    positions_on_device_ = false;
+    shared_tokens_ = branches_.empty() ? 0 : cm_->common_prefix_tokens(branches_.data(), (int)branches_.size());
+    return (int)branches_.size();
+}
+
+void KvStream::close_branches()
+{
+    for (int id : branches_) cm_->release_branch(id);
+    branches_.clear();
+    pos_.clear();
+    positions_on_device_ = false;
+    shared_tokens_ = 0;
+    if (graph_) {                        // a captured step is tied to the branch set it was recorded for
+        drk_graph_destroy(graph_);
+        graph_ = nullptr;
+    }
+}
+
+bool KvStream::host_begin(hipStream_t stream)
+{
+    const int B = (int)branches_.size();
+    if (B == 0) return false;
+    for (int i = 0; i < B; i++) {
+        if (pos_[i] + 1 > max_context_len_) {
+            LOG_ERROR("Conscientia", "KvStream: branch %d reached max_context_len %d", branches_[i], max_context_len_);
+            return false;
+        }
+        if (!cm_->ensure_blocks_for(branches_[i], pos_[i])) {             // stream.cpp:297-301
+            LOG_ERROR("Conscientia", "Block allocation failed at pos=%d (branch %d)", pos_[i], branches_[i]);
+            return false;
+        }
+    }
+    cm_->sync_block_table(stream);                                        // stream.cpp:302
+    if (!positions_on_device_) {                                          // stream.cpp:304-305, once per branch set
+        std::vector<int> len(B);
+        for (int i = 0; i < B; i++) len[i] = pos_[i] + 1;
+        if (drk_memcpy_h2d_async(d_pos_, pos_.data(), (size_t)B * sizeof(int), stream) != DRK_OK ||
+            drk_memcpy_h2d_async(d_len_, len.data(), (size_t)B * sizeof(int), stream) != DRK_OK ||
+            drk_stream_synchronize(stream) != DRK_OK) {                   // the host vectors go out of scope
+            LOG_ERROR("Conscientia", "KvStream: position upload: %s", drk_last_error());
+            return false;
+        }
+        positions_on_device_ = true;
+    }
+    return true;
+}
+
+void KvStream::host_end()
+{
+    for (size_t i = 0; i < branches_.size(); i++) {
+        pos_[i]++;                                                        // stream.cpp:371-372
+        cm_->set_seq_len(branches_[i], pos_[i]);
+    }
+}
+
+bool KvStream::begin_decode_step(hipStream_t stream)
+{
+    first_layer_of_step_ = -1;
+    return host_begin(stream);
+}
+
+void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t stream)
+{
+    const int B = (int)branches_.size();
+    if (B == 0) return;
+    const BlockPool& pool = cm_->block_pool();
+    const int hd = ModelConfig::HEAD_DIM, stride = cm_->table_stride();
+    const int* tables = cm_->d_block_table(branches_[0]);
+    const float scale = 1.0f / std::sqrt((float)hd);
+    int max_len = 0;
+    for (int p : pos_) max_len = p + 1 > max_len ? p + 1 : max_len;
+    // a captured step is replayed while the branches grow: size the launch for the whole context
+    if (max_context_len_ > max_len) max_len = max_context_len_;
+    paged_qk_norm_rope_write_branches(io.qg, io.k, io.v, io.q_norm, io.k_norm, io.q_scratch, pool.pool_ptr(), tables, stride,
+                                      d_pos_, B, fa_layer_idx, pool.max_blocks(), pool.block_size(), d_rope_table_,
+                                      table_positions_, stream);
+    const __half* gate = io.qg + hd;
+    if (scorer_ && scorer_->d_new_scores()) {
+        if (first_layer_of_step_ < 0) first_layer_of_step_ = fa_layer_idx;
+        float* mass = scorer_->d_new_scores() + (size_t)branches_[0] * stride;
+        paged_gqa_decode_attention_branches_scored(io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
+                                                   io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(), scale,
+                                                   mass, fa_layer_idx != first_layer_of_step_, stream);
+        if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
+                             ModelConfig::IO_DTYPE, stream) != DRK_OK)
+            LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
+    } else if (B >= 4 && shared_tokens_ >= 4096) {
+        // the branches' common prefix is streamed once for all of them
+        paged_gqa_decode_attention_shared(io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, shared_tokens_,
+                                          io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(), scale, stream);
+        if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
+                             ModelConfig::IO_DTYPE, stream) != DRK_OK)
+            LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
+    } else {
+        paged_gqa_decode_attention_gated_branches(io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, gate,
+                                                  2 * hd, io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(),
+                                                  scale, stream);
+    }
+}
+
+void KvStream::end_decode_step(hipStream_t stream)
+{
+    const int B = (int)branches_.size();
+    if (B == 0) return;
+    if (scorer_ && first_layer_of_step_ >= 0) scorer_->apply_new_scores(stream);
+    if (drk_positions_advance(d_pos_, d_len_, B, 1, stream) != DRK_OK)
+        LOG_ERROR("Conscientia", "positions_advance: %s", drk_last_error());
+    host_end();
+}
+
+bool KvStream::capture_decode_step(const std::function<void(hipStream_t)>& layers, hipStream_t stream)
+{
+    if (branches_.empty()) return false;
+    if (graph_) {
+        drk_graph_destroy(graph_);
+        graph_ = nullptr;
+    }
+    // host part first: the capture must not contain table uploads or the position upload
+    first_layer_of_step_ = -1;
+    if (!host_begin(stream)) return false;
+    if (drk_graph_begin_capture(stream) != DRK_OK) {
+        LOG_ERROR("Conscientia", "KvStream: begin capture: %s", drk_last_error());
+        return false;
+    }
+    layers(stream);
+    if (scorer_ && first_layer_of_step_ >= 0) scorer_->apply_new_scores(stream);
+    drk_positions_advance(d_pos_, d_len_, (int)branches_.size(), 1, stream);
+    if (drk_graph_end_capture(stream, &graph_) != DRK_OK) {
+        LOG_ERROR("Conscientia", "KvStream: end capture: %s", drk_last_error());
+        graph_ = nullptr;
+        return false;
+    }
+    return true;                          // nothing ran yet: the first replay_decode_step() is this step
+}
+
+bool KvStream::replay_decode_step(hipStream_t stream)
+{
+    if (!graph_) return false;
+    if (!host_begin(stream)) return false;
+    if (drk_graph_launch(graph_, stream) != DRK_OK) {
+        LOG_ERROR("Conscientia", "KvStream: graph launch: %s", drk_last_error());
+        return false;
+    }
+    host_end();
+    return true;
+}
+
+} // namespace deusridet

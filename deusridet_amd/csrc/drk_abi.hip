@@ -68,6 +68,17 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4 *__restrict
     if (acc == 0x9e3779b9u) *sink = acc;      // practically never: keeps the loads alive
 }
 
+// positions and lengths of the decode branches move on by `delta` inside the stream (so that a
+// captured step advances them itself)
+__global__ void advance_i32_kernel(int32_t *__restrict__ a, int32_t *__restrict__ b, int n, int delta)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        if (a) a[i] += delta;
+        if (b) b[i] += delta;
+    }
+}
+
 } // namespace drk
 
 using drk::Lay;
@@ -159,6 +170,46 @@ int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream)
 int drk_device_synchronize(void)
 {
     DRK_HIP(hipDeviceSynchronize());
+    return DRK_OK;
+}
+
+int drk_positions_advance(int32_t *d_pos, int32_t *d_seq_lens, int n, int delta, void *stream)
+{
+    if (n < 0 || (!d_pos && !d_seq_lens)) return fail(DRK_ERR_INVALID, "positions_advance: bad argument");
+    if (n == 0) return DRK_OK;
+    hipLaunchKernelGGL(drk::advance_i32_kernel, dim3((n + 63) / 64), dim3(64), 0, (hipStream_t)stream, d_pos, d_seq_lens, n, delta);
+    DRK_LAUNCH_CHECK("advance_i32_kernel");
+    return DRK_OK;
+}
+
+// stream capture of a launch sequence into an executable graph
+int drk_graph_begin_capture(void *stream)
+{
+    DRK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+    return DRK_OK;
+}
+int drk_graph_end_capture(void *stream, void **graph_exec)
+{
+    if (!graph_exec) return fail(DRK_ERR_INVALID, "graph_exec is NULL");
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    DRK_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    hipGraphDestroy(graph);
+    if (e != hipSuccess) return fail(DRK_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    *graph_exec = (void *)exec;
+    return DRK_OK;
+}
+int drk_graph_launch(void *graph_exec, void *stream)
+{
+    if (!graph_exec) return fail(DRK_ERR_INVALID, "graph_exec is NULL");
+    DRK_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_graph_destroy(void *graph_exec)
+{
+    if (graph_exec) DRK_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
     return DRK_OK;
 }
 

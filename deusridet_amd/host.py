@@ -69,6 +69,23 @@ SIGNATURES = {
                                                       _f32, _vp]),
     "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32]),
+    "drkh_kvs_create": (_vp, []),
+    "drkh_kvs_destroy": (None, [_vp]),
+    "drkh_kvs_init": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32]),
+    "drkh_kvs_begin_prefill": (_i32, [_vp, _i32, _vp]),
+    "drkh_kvs_prefill_layer": (None, [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp]),
+    "drkh_kvs_end_prefill": (None, [_vp, _i32]),
+    "drkh_kvs_current_pos": (_i32, [_vp]),
+    "drkh_kvs_open_branches": (_i32, [_vp, _i32]),
+    "drkh_kvs_close_branches": (None, [_vp]),
+    "drkh_kvs_num_branches": (_i32, [_vp]),
+    "drkh_kvs_branch_id": (_i32, [_vp, _i32]),
+    "drkh_kvs_branch_pos": (_i32, [_vp, _i32]),
+    "drkh_kvs_begin_decode_step": (_i32, [_vp, _vp]),
+    "drkh_kvs_decode_layer": (None, [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "drkh_kvs_end_decode_step": (None, [_vp, _vp]),
+    "drkh_kvs_capture_decode_step": (_i32, [_vp, _vp, _vp, _vp]),
+    "drkh_kvs_replay_decode_step": (_i32, [_vp, _vp]),
     "drkh_scorer_d_new_scores": (_vp, [_vp]),
     "drkh_scorer_apply_new_scores": (None, [_vp, _vp]),
     "drkh_paged_gqa_decode_attention_branches_scored": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32,
@@ -114,14 +131,19 @@ def set_attention_geometry(num_fa_layers, num_attn_heads, num_kv_heads, head_dim
                                                   io_dtype))
 
 
+def _destroy(obj, fn):
+    """Free a native handle once; at interpreter shutdown the module may already be torn down."""
+    h, obj._h = getattr(obj, "_h", None), None
+    if h and lib is not None:
+        getattr(lib(), fn)(h)
+
+
 class ImportanceScorer:
     def __init__(self):
         self._h = lib().drkh_scorer_create()
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            lib().drkh_scorer_destroy(self._h)
-            self._h = None
+        _destroy(self, "drkh_scorer_destroy")
 
     def init(self, max_blocks, decay=0.95): return bool(lib().drkh_scorer_init(self._h, max_blocks, decay))
     def init_detached(self, max_blocks, decay=0.95): return bool(lib().drkh_scorer_init_detached(self._h, max_blocks, decay))
@@ -140,6 +162,44 @@ class ImportanceScorer:
         lib().drkh_scorer_load_host_scores(self._h, _p(a), a.shape[0])
 
 
+LAYERS_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_void_p)
+
+
+class KvStream:
+    """conscientia/kv_stream.h; io = (qg, k, v, q_norm, k_norm, q_scratch, attn_out) device pointers."""
+
+    def __init__(self):
+        self._h = lib().drkh_kvs_create()
+
+    def __del__(self):
+        _destroy(self, "drkh_kvs_destroy")
+
+    def init(self, cm, max_context_len, scorer=None, rope_table=None, table_positions=0):
+        self._cm, self._scorer = cm, scorer
+        return bool(lib().drkh_kvs_init(self._h, cm._h, max_context_len, scorer._h if scorer else None, rope_table,
+                                        table_positions))
+
+    def begin_prefill(self, M, stream=None): return bool(lib().drkh_kvs_begin_prefill(self._h, M, stream))
+    def prefill_layer(self, layer, io, M, stream=None): lib().drkh_kvs_prefill_layer(self._h, layer, *io, M, stream)
+    def end_prefill(self, M): lib().drkh_kvs_end_prefill(self._h, M)
+    def current_pos(self): return lib().drkh_kvs_current_pos(self._h)
+    def open_branches(self, n): return lib().drkh_kvs_open_branches(self._h, n)
+    def close_branches(self): lib().drkh_kvs_close_branches(self._h)
+    def num_branches(self): return lib().drkh_kvs_num_branches(self._h)
+    def branch_id(self, i): return lib().drkh_kvs_branch_id(self._h, i)
+    def branch_pos(self, i): return lib().drkh_kvs_branch_pos(self._h, i)
+    def begin_decode_step(self, stream=None): return bool(lib().drkh_kvs_begin_decode_step(self._h, stream))
+    def decode_layer(self, layer, io, stream=None): lib().drkh_kvs_decode_layer(self._h, layer, *io, stream)
+    def end_decode_step(self, stream=None): lib().drkh_kvs_end_decode_step(self._h, stream)
+
+    def capture_decode_step(self, layers, stream=None):
+        """layers(stream_ptr) enqueues one step (decode_layer per full-attention layer)."""
+        cb = LAYERS_FN(lambda s, _u: layers(C.c_void_p(s)))
+        return bool(lib().drkh_kvs_capture_decode_step(self._h, C.cast(cb, C.c_void_p), None, stream))
+
+    def replay_decode_step(self, stream=None): return bool(lib().drkh_kvs_replay_decode_step(self._h, stream))
+
+
 class KVSwapper:
     """src/memoria/kv_swapper.h:50-114; init() takes the CacheManager whose pool it serves."""
 
@@ -147,9 +207,7 @@ class KVSwapper:
         self._h = lib().drkh_swapper_create()
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            lib().drkh_swapper_destroy(self._h)
-            self._h = None
+        _destroy(self, "drkh_swapper_destroy")
 
     def init(self, cm, ssd_dir, staging_blocks=2):
         return bool(lib().drkh_swapper_init(self._h, cm._h, str(ssd_dir).encode(), staging_blocks))
@@ -172,9 +230,7 @@ class CacheManager:
         self._scorer = None
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            lib().drkh_cm_destroy(self._h)
-            self._h = None
+        _destroy(self, "drkh_cm_destroy")
 
     def init(self, kv_budget_bytes, block_size=256, scorer=None, max_branches=1):
         self._scorer = scorer

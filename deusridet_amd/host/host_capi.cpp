@@ -5,6 +5,7 @@
 #include "../machina/paged_attention.h"
 #include "../machina/layer.h"
 #include "../memoria/kv_swapper.h"
+#include "../conscientia/kv_stream.h"
 #include "../memoria/cache_kernels.h"
 #include "../memoria/cache_manager.h"
 
@@ -15,6 +16,7 @@ using namespace deusridet;
 #define CM(p) (static_cast<CacheManager *>(p))
 #define SC(p) (static_cast<ImportanceScorer *>(p))
 #define SW(p) (static_cast<KVSwapper *>(p))
+#define KS(p) (static_cast<KvStream *>(p))
 #define H(p) (reinterpret_cast<__half *>(p))
 #define CH(p) (reinterpret_cast<const __half *>(p))
 #define ST(p) (static_cast<hipStream_t>(p))
@@ -239,6 +241,42 @@ void drkh_paged_prefill_attention_gated(const void *Q, void *kv_pool, const int3
     paged_prefill_attention_gated(CH(Q), H(kv_pool), d_block_table, CH(gate), gate_stride, H(out), fa_layer_idx,
                                   pos_start, M, max_phys_blocks, block_size, scale, (hipStream_t)stream);
 }
+static KvLayerIO make_io(const void *qg, const void *k, const void *v, const void *q_norm, const void *k_norm,
+                         void *q_scratch, void *attn_out)
+{
+    return KvLayerIO{CH(qg), CH(k), CH(v), CH(q_norm), CH(k_norm), H(q_scratch), H(attn_out)};
+}
+void *drkh_kvs_create(void) { return new KvStream(); }
+void drkh_kvs_destroy(void *ks) { delete KS(ks); }
+int drkh_kvs_init(void *ks, void *cm, int max_context_len, void *scorer, const float *d_rope_table, int table_positions)
+{
+    return KS(ks)->init(*CM(cm), max_context_len, SC(scorer), d_rope_table, table_positions) ? 1 : 0;
+}
+int drkh_kvs_begin_prefill(void *ks, int M, void *stream) { return KS(ks)->begin_prefill(M, (hipStream_t)stream) ? 1 : 0; }
+void drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
+                            const void *k_norm, void *q_scratch, void *attn_out, int M, void *stream)
+{
+    KS(ks)->prefill_layer(fa_layer_idx, make_io(qg, k, v, q_norm, k_norm, q_scratch, attn_out), M, (hipStream_t)stream);
+}
+void drkh_kvs_end_prefill(void *ks, int M) { KS(ks)->end_prefill(M); }
+int drkh_kvs_current_pos(void *ks) { return KS(ks)->current_pos(); }
+int drkh_kvs_open_branches(void *ks, int n) { return KS(ks)->open_branches(n); }
+void drkh_kvs_close_branches(void *ks) { KS(ks)->close_branches(); }
+int drkh_kvs_num_branches(void *ks) { return KS(ks)->num_branches(); }
+int drkh_kvs_branch_id(void *ks, int i) { return KS(ks)->branch_id(i); }
+int drkh_kvs_branch_pos(void *ks, int i) { return KS(ks)->branch_pos(i); }
+int drkh_kvs_begin_decode_step(void *ks, void *stream) { return KS(ks)->begin_decode_step((hipStream_t)stream) ? 1 : 0; }
+void drkh_kvs_decode_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
+                           const void *k_norm, void *q_scratch, void *attn_out, void *stream)
+{
+    KS(ks)->decode_layer(fa_layer_idx, make_io(qg, k, v, q_norm, k_norm, q_scratch, attn_out), (hipStream_t)stream);
+}
+void drkh_kvs_end_decode_step(void *ks, void *stream) { KS(ks)->end_decode_step((hipStream_t)stream); }
+int drkh_kvs_capture_decode_step(void *ks, void (*layers)(void *stream, void *user), void *user, void *stream)
+{
+    return KS(ks)->capture_decode_step([&](hipStream_t s) { layers((void *)s, user); }, (hipStream_t)stream) ? 1 : 0;
+}
+int drkh_kvs_replay_decode_step(void *ks, void *stream) { return KS(ks)->replay_decode_step((hipStream_t)stream) ? 1 : 0; }
 void *drkh_scorer_d_new_scores(void *s) { return SC(s)->d_new_scores(); }
 void drkh_scorer_apply_new_scores(void *s, void *stream) { SC(s)->apply_new_scores((hipStream_t)stream); }
 void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_pool, const int32_t *d_tables,

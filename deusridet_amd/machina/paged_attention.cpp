@@ -37,7 +37,13 @@ void* workspace(size_t need)
 bool paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size)
 {
     drk_kv_layout g = ModelConfig::layout(1, block_size);
-    size_t need = drk_decode_workspace_bytes(&g, max_branches > 0 ? max_branches : 1, max_seq_len);
+    const int B = max_branches > 0 ? max_branches : 1;
+    size_t need = drk_decode_workspace_bytes(&g, B, max_seq_len);
+    // the shared-prefix and the scored variants keep more partials than the plain call
+    size_t s = drk_decode_shared_workspace_bytes(&g, B, max_seq_len, max_seq_len);
+    if (s > need) need = s;
+    s = drk_decode_mass_workspace_bytes(&g, B, max_seq_len);
+    if (s > need) need = s;
     if (max_prefill_rows > 0) {
         size_t p = drk_decode_workspace_bytes(&g, max_prefill_rows, max_seq_len);
         if (p > need) need = p;

@@ -138,6 +138,27 @@ void drkh_paged_gqa_decode_attention_gated_branches(const void *Q, void *kv_pool
 void drkh_paged_prefill_attention_gated(const void *Q, void *kv_pool, const int32_t *d_block_table, const void *gate,
                                         int gate_stride, void *out, int fa_layer_idx, int pos_start, int M,
                                         int max_phys_blocks, int block_size, float scale, void *stream);
+/* conscientia/kv_stream.h: the KV side of ConscientiStream (src/conscientia/stream.cpp:145-401) */
+void *drkh_kvs_create(void);
+void  drkh_kvs_destroy(void *ks);
+int   drkh_kvs_init(void *ks, void *cm, int max_context_len, void *scorer, const float *d_rope_table, int table_positions);
+int   drkh_kvs_begin_prefill(void *ks, int M, void *stream);
+void  drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
+                             const void *k_norm, void *q_scratch, void *attn_out, int M, void *stream);
+void  drkh_kvs_end_prefill(void *ks, int M);
+int   drkh_kvs_current_pos(void *ks);
+int   drkh_kvs_open_branches(void *ks, int n);
+void  drkh_kvs_close_branches(void *ks);
+int   drkh_kvs_num_branches(void *ks);
+int   drkh_kvs_branch_id(void *ks, int i);
+int   drkh_kvs_branch_pos(void *ks, int i);
+int   drkh_kvs_begin_decode_step(void *ks, void *stream);
+void  drkh_kvs_decode_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
+                            const void *k_norm, void *q_scratch, void *attn_out, void *stream);
+void  drkh_kvs_end_decode_step(void *ks, void *stream);
+/* layers(stream, user) enqueues one step's work (drkh_kvs_decode_layer per full-attention layer) */
+int   drkh_kvs_capture_decode_step(void *ks, void (*layers)(void *stream, void *user), void *user, void *stream);
+int   drkh_kvs_replay_decode_step(void *ks, void *stream);
 void *drkh_scorer_d_new_scores(void *s);
 void drkh_scorer_apply_new_scores(void *s, void *stream);
 void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_pool, const int32_t *d_tables,

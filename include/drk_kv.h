@@ -97,6 +97,16 @@ int drk_dev_free(void *d_ptr);
 int drk_dev_memset_async(void *d_ptr, int byte, size_t bytes, void *stream);
 int drk_memcpy_h2d_async(void *d_dst, const void *h_src, size_t bytes, void *stream);
 int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream); /* syncs */
+/* d_pos[i] += delta and d_seq_lens[i] += delta for i < n (either may be NULL), in the stream:
+ * lets a captured decode step move its own positions on. */
+int drk_positions_advance(int32_t *d_pos, int32_t *d_seq_lens, int n, int delta, void *stream);
+/* Capture what is enqueued on `stream` between begin and end into an executable graph
+ * (thread-local capture mode), launch it, destroy it.  None of the append / attention entry
+ * points allocates, memsets or synchronises, so a whole decode step can be captured. */
+int drk_graph_begin_capture(void *stream);
+int drk_graph_end_capture(void *stream, void **graph_exec);
+int drk_graph_launch(void *graph_exec, void *stream);
+int drk_graph_destroy(void *graph_exec);
 /* Waits for all work on every stream of the current device. */
 int drk_device_synchronize(void);
 /* Pinned host memory (allocated pinned, for staging buffers). */

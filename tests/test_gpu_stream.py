@@ -1,0 +1,207 @@
+"""GPU: the KV side of the consciousness stream (conscientia/kv_stream.h, after
+src/conscientia/stream.cpp:145-401): chunked perception into branch 0, decode branches forked
+copy-on-write from it, one fused launch pair per layer, and a captured step replayed.
+
+Checked against the oracle's composition of the reference's separate steps (split, head norm,
+RoPE, page write, attention, gate): the pool bit for bit, the attention output within the
+attention tolerance; and the replayed graph against the eager session bit for bit."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from deusridet_amd import cabi, host
+from oracle import binding as orc
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+L, QH, KVH, D, BS, RD = 2, 32, 8, 128, 16, 32
+EPS, THETA = 1e-6, 1.0e7
+DT = cabi.BF16
+NPOS = 512
+
+
+def d2h(ptr, nbytes):
+    out = np.empty(nbytes, dtype=np.uint8)
+    cabi.call("drk_memcpy_d2h", out.ctypes.data_as(C.c_void_p), C.c_void_p(ptr), nbytes, U.stream_ptr())
+    return out
+
+
+class Session:
+    """One cache manager + stream driver + the device buffers a model would own."""
+
+    def __init__(self, nbranch, scorer=False):
+        import torch
+        assert host.set_attention_geometry(L, QH, KVH, D, DT)
+        assert host.lib().drkh_set_rope(RD, THETA, EPS)
+        self.cm = host.CacheManager()
+        self.sc = host.ImportanceScorer() if scorer else None
+        assert self.cm.init(48 * L * 2 * KVH * BS * D * 2, BS, self.sc, 1 + nbranch)
+        if scorer:
+            assert self.sc.init((1 + nbranch) * self.cm.table_stride(), 0.5)
+        self.tab = orc.rope_table(NPOS, RD, THETA)
+        self.dtab = torch.from_numpy(self.tab).cuda()
+        self.ks = host.KvStream()
+        assert self.ks.init(self.cm, NPOS, self.sc, U.p(self.dtab), NPOS)
+        T = 64
+        self.qw, self.kw = None, None
+        self.bufs = dict(qg=U.dev_zeros(T * QH * 2 * D * 2), k=U.dev_zeros(T * KVH * D * 2), v=U.dev_zeros(T * KVH * D * 2),
+                         q=U.dev_zeros(T * QH * D * 2), out=U.dev_zeros(T * QH * D * 2))
+        self.NB = self.cm.pool_max_blocks()
+
+    def set_weights(self, qw, kw):
+        self.dqw, self.dkw = U.dev_bytes(qw), U.dev_bytes(kw)
+
+    def load(self, qg, k, v):
+        import torch
+        for name, a in (("qg", qg), ("k", k), ("v", v)):
+            t = torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1))
+            self.bufs[name][:t.numel()].copy_(t)
+
+    def io(self):
+        b = self.bufs
+        return (U.p(b["qg"]), U.p(b["k"]), U.p(b["v"]), U.p(self.dqw), U.p(self.dkw), U.p(b["q"]), U.p(b["out"]))
+
+    def out(self, T):
+        U.sync()
+        return U.host(self.bufs["out"], np.uint16)[:T * QH * D].reshape(T, QH, D).copy()
+
+    def pool(self):
+        return d2h(self.cm.pool_ptr(), self.cm.pool_total_bytes())
+
+
+def oracle_layer(og, opool, table_rows, pos, layer, qg, k, v, qw, kw, tab, prefill_start=None):
+    """The reference's sequence for T tokens; table_rows[t] is the table token t writes through."""
+    T = qg.shape[0]
+    q0, gate = orc.split_q_gate(qg, T, QH, D)
+    qr = orc.apply_rope(orc.head_norm(q0, qw, EPS, DT).reshape(T, QH, D), pos, tab, RD, DT)
+    kr = orc.apply_rope(orc.head_norm(k, kw, EPS, DT).reshape(T, KVH, D), pos, tab, RD, DT)
+    for t in range(T):
+        orc.append_token(og, opool, table_rows[t], layer, int(pos[t]), kr[t], v[t], DT)
+    want = np.empty((T, QH, D), np.float64)
+    for t in range(T):
+        want[t] = orc.decode_f64(og, qr[t], opool, table_rows[t], layer, int(pos[t]) + 1, 1 / np.sqrt(D), DT)
+    g = U.from_bits(gate, DT).astype(np.float64)
+    return want / (1.0 + np.exp(-g))
+
+
+def run_session(nbranch, steps, mode, seed=120, scorer=False):
+    """mode 'eager' or 'graph'.  Returns (prefill outs, per-step decode outs, final pool, session)."""
+    s = Session(nbranch, scorer)
+    rng = np.random.default_rng(seed)
+    qw, kw = U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT)
+    s.set_weights(qw, kw)
+    st = U.stream_ptr()
+    og = orc.layout(L, KVH, QH, D, BS, s.NB, DT)
+    opool = orc.new_pool(og)
+    record = dict(prefill=[], decode=[], inputs=[])
+    # ---- perception: 100 tokens in chunks of 64 + 36 ----
+    for M in (64, 36):
+        pos0 = s.ks.current_pos()
+        assert s.ks.begin_prefill(M, st)
+        table0 = s.cm.h_block_table(0).copy()
+        for layer in range(L):
+            qg, k, v = (U.normal_bits(rng, sh, DT, m) for sh, m in (((M, QH, 2 * D), 1.0), ((M, KVH, D), 0.7), ((M, KVH, D), 0.5)))
+            s.load(qg, k, v)
+            s.ks.prefill_layer(layer, s.io(), M, st)
+            got = s.out(M)
+            pos = (pos0 + np.arange(M)).astype(np.int32)
+            want = oracle_layer(og, opool, [table0] * M, pos, layer, qg, k, v, qw, kw, s.tab)
+            ok, mx, _ = U.rel_abs_ok(U.from_bits(got, DT), want)
+            assert ok, (M, layer, mx)
+            record["prefill"].append(got)
+        s.ks.end_prefill(M)
+    assert s.ks.current_pos() == 100 and s.cm.seq_len(0) == 100
+    assert np.array_equal(s.pool(), opool)
+    # ---- decode branches ----
+    assert s.ks.open_branches(nbranch) == nbranch
+    ids = [s.ks.branch_id(i) for i in range(nbranch)]
+    assert ids == list(range(1, nbranch + 1)) and all(s.ks.branch_pos(i) == 100 for i in range(nbranch))
+    step_inputs = [[tuple(U.normal_bits(rng, sh, DT, m) for sh, m in (((nbranch, QH, 2 * D), 1.0), ((nbranch, KVH, D), 0.7),
+                                                                       ((nbranch, KVH, D), 0.5))) for _ in range(L)]
+                   for _ in range(steps)]
+    if mode == "graph":
+        # the model's buffers are fixed; one set per layer so that a replay reads this step's inputs
+        import torch
+        lay_bufs = [dict(qg=U.dev_zeros(nbranch * QH * 2 * D * 2), k=U.dev_zeros(nbranch * KVH * D * 2), v=U.dev_zeros(nbranch * KVH * D * 2),
+                         q=U.dev_zeros(nbranch * QH * D * 2), out=U.dev_zeros(nbranch * QH * D * 2)) for _ in range(L)]
+
+        def layers(stream):
+            for layer in range(L):
+                b = lay_bufs[layer]
+                s.ks.decode_layer(layer, (U.p(b["qg"]), U.p(b["k"]), U.p(b["v"]), U.p(s.dqw), U.p(s.dkw), U.p(b["q"]), U.p(b["out"])), stream)
+
+        side = torch.cuda.Stream()
+        sp = C.c_void_p(side.cuda_stream)
+        assert s.ks.capture_decode_step(layers, sp)
+    for step in range(steps):
+        if mode == "eager":
+            assert s.ks.begin_decode_step(st)
+            tables = [s.cm.h_block_table(b).copy() for b in ids]
+            outs = []
+            for layer in range(L):
+                qg, k, v = step_inputs[step][layer]
+                s.load(qg, k, v)
+                s.ks.decode_layer(layer, s.io(), st)
+                got = s.out(nbranch)
+                pos = np.full(nbranch, 100 + step, np.int32)
+                if step == 0 and layer == 0:                         # first write into the shared tail block: copy-on-write
+                    for b in range(nbranch):
+                        for src_blk, dst_blk in [(s.cm.h_block_table(0)[6], tables[b][6])]:
+                            assert src_blk != dst_blk
+                            orc.copy_block(og, opool, int(src_blk), int(dst_blk))
+                want = oracle_layer(og, opool, tables, pos, layer, qg, k, v, qw, kw, s.tab)
+                ok, mx, _ = U.rel_abs_ok(U.from_bits(got, DT), want)
+                assert ok, (step, layer, mx)
+                outs.append(got)
+            s.ks.end_decode_step(st)
+            record["decode"].append(outs)
+        else:
+            import torch
+            for layer in range(L):
+                qg, k, v = step_inputs[step][layer]
+                for name, a in (("qg", qg), ("k", k), ("v", v)):
+                    lay_bufs[layer][name].copy_(torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)))
+            torch.cuda.synchronize()
+            assert s.ks.replay_decode_step(sp)
+            side.synchronize()
+            record["decode"].append([U.host(lay_bufs[layer]["out"], np.uint16).reshape(nbranch, QH, D).copy() for layer in range(L)])
+        assert [s.ks.branch_pos(i) for i in range(nbranch)] == [101 + step] * nbranch
+        assert [s.cm.seq_len(b) for b in ids] == [101 + step] * nbranch
+    final_pool = s.pool()
+    if mode == "eager":
+        assert np.array_equal(final_pool, opool)                      # every byte, all branches, all layers
+    return record, final_pool, s
+
+
+def test_stream_session_matches_the_oracle_and_its_graph_replay(dev):
+    rec_e, pool_e, s_e = run_session(3, 5, "eager")
+    # the prefix blocks are shared: 6 whole blocks of branch 0 are referenced by all four tables
+    shared = s_e.cm.h_block_table(0)[:6]
+    for b in (1, 2, 3):
+        assert np.array_equal(s_e.cm.h_block_table(b)[:6], shared) and s_e.cm.h_block_table(b)[6] != s_e.cm.h_block_table(0)[6]
+    s_e.ks.close_branches()
+    assert s_e.cm.gpu_blocks_used() == 7                               # only the stream's own blocks stay
+    del s_e
+    rec_g, pool_g, s_g = run_session(3, 5, "graph")
+    for step in range(5):
+        for layer in range(L):
+            assert np.array_equal(rec_g["decode"][step][layer], rec_e["decode"][step][layer]), (step, layer)
+    assert np.array_equal(pool_g, pool_e)
+    s_g.ks.close_branches()
+
+
+def test_stream_session_feeds_the_scorer(dev):
+    """With a scorer attached every decode step leaves the attention mass of the step in the
+    scores (score = score * decay + mass, summed over the layers): a branch's blocks sum to
+    L * QH per step."""
+    rec, pool, s = run_session(2, 3, "eager", seed=121, scorer=True)
+    s.sc.sync_to_host()
+    stride = s.cm.table_stride()
+    for b in (1, 2):
+        tot = sum(s.sc.score(b * stride + lb) for lb in range(8))
+        want = L * QH * (1 + 0.5 + 0.25)                               # three steps, decay 0.5
+        assert abs(tot - want) < 0.05 * want, (b, tot, want)
+    assert sum(s.sc.score(lb) for lb in range(8)) == 0.0              # branch 0 took no decode step
+    s.ks.close_branches()
