@@ -45,9 +45,10 @@ def parse():
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="context per branch for the CPU sample (0 = auto)")
     ap.add_argument("--bulk-append-tokens", type=int, default=2048)
     ap.add_argument("--seed", type=int, default=2)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5],
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6],
                     help="BASELINE config: 2 (default, the headline) | 3 shared prefix + COW + eviction | "
-                         "4 int8/fp8 pages at 128k | 5 chunked MFMA prefill interleaved with decode")
+                         "4 int8/fp8 pages at 128k | 5 chunked MFMA prefill interleaved with decode | "
+                         "6 config 3's shape through the stream driver (whole layer path, captured step)")
     ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8", help="config 4 storage type")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "
                                                             "replaying one captured HIP graph per step")

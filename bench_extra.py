@@ -360,5 +360,107 @@ def config5(args):
     }
 
 
+def config6(args):
+    """The caller protocol at config 3's shape: one perception stream takes a 64k-token prefix in
+    2048-token chunks through the whole layer path (fused split + norm + RoPE + page write, then
+    MFMA prefill attention with the gate), 16 decode branches fork from it copy-on-write and step
+    together -- from the host layer by layer, and as one captured step replayed."""
+    torch, cabi, U, lib, _, _ = _common(args)
+    from deusridet_amd import host
+    stream = torch.cuda.Stream()                     # the default stream cannot be captured
+    sp = C.c_void_p(stream.cuda_stream)
+    L, KVH, QH, D, bs, NBR = args.layers, 8, 32, 128, 16, 16
+    W, K = args.warmup, args.steps
+    prefix, chunk, RD, THETA = 65536, 2048, 32, 1.0e7
+    max_ctx = prefix + 2 * (W + K) + 64
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    assert host.lib().drkh_set_rope(RD, THETA, 1e-6)
+    cm = host.CacheManager()
+    blocks = prefix // bs + NBR * ((2 * (W + K)) // bs + 3) + 64
+    assert cm.init(blocks * L * 2 * KVH * bs * D * 2, bs, None, NBR + 1), "CacheManager.init failed"
+    table = torch.empty(max_ctx * RD, dtype=torch.float32, device="cuda")
+    cabi.call("drk_rope_table_fill", U.p(table), max_ctx, RD, THETA, sp)
+    ks = host.KvStream()
+    assert ks.init(cm, max_ctx, None, U.p(table), max_ctx)
+    bf = torch.bfloat16
+    qw = (1 + 0.1 * torch.randn(D, device="cuda")).to(bf)
+    kw = (1 + 0.1 * torch.randn(D, device="cuda")).to(bf)
+    # ---- perception ----
+    qg = (torch.randn(chunk, QH, 2 * D, device="cuda")).to(bf)
+    k = (torch.randn(chunk, KVH, D, device="cuda") * 0.7).to(bf)
+    v = (torch.randn(chunk, KVH, D, device="cuda") * 0.5).to(bf)
+    qs, ao = torch.empty(chunk, QH, D, device="cuda", dtype=bf), torch.empty(chunk, QH, D, device="cuda", dtype=bf)
+    io = (U.p(qg), U.p(k), U.p(v), U.p(qw), U.p(kw), U.p(qs), U.p(ao))
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for p0 in range(0, prefix, chunk):
+        assert ks.begin_prefill(chunk, sp)
+        for l in range(L):
+            ks.prefill_layer(l, io, chunk, sp)
+        ks.end_prefill(chunk)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    prefill_ms = e0.elapsed_time(e1)
+    prefill_flops = 4.0 * QH * D * L * sum((p0 + (chunk + 1) / 2.0) * chunk for p0 in range(0, prefix, chunk))
+    # ---- decode branches ----
+    assert ks.open_branches(NBR) == NBR and ks.shared_tokens() == prefix
+    B = NBR
+    lay = [dict(qg=torch.randn(B, QH, 2 * D, device="cuda").to(bf), k=(torch.randn(B, KVH, D, device="cuda") * 0.7).to(bf),
+                v=(torch.randn(B, KVH, D, device="cuda") * 0.5).to(bf), q=torch.empty(B, QH, D, device="cuda", dtype=bf),
+                out=torch.empty(B, QH, D, device="cuda", dtype=bf)) for _ in range(L)]
+
+    torch.cuda.synchronize()
+
+    def layers(st):
+        for l in range(L):
+            b = lay[l]
+            ks.decode_layer(l, (U.p(b["qg"]), U.p(b["k"]), U.p(b["v"]), U.p(qw), U.p(kw), U.p(b["q"]), U.p(b["out"])), st)
+
+    per_tok = 2 * KVH * D * 2
+
+    def timed(step_fn):
+        for _ in range(W):
+            step_fn()
+        torch.cuda.synchronize()
+        host_s, logical = 0.0, 0
+        e0.record(stream)
+        for _ in range(K):
+            t = time.perf_counter()
+            step_fn()
+            host_s += time.perf_counter() - t
+            logical += sum(ks.branch_pos(i) for i in range(B))
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / K, host_s / K * 1e3, logical
+
+    def eager():
+        assert ks.begin_decode_step(sp)
+        layers(sp)
+        ks.end_decode_step(sp)
+
+    eager_ms, eager_host_ms, _ = timed(eager)
+    assert ks.capture_decode_step(layers, sp)
+    graph_ms, graph_host_ms, logical = timed(lambda: ks.replay_decode_step(sp) or (_ for _ in ()).throw(RuntimeError("replay failed")))
+    value = logical * per_tok * L / (graph_ms * K * 1e-3) / 1e9
+    launch_unique = (prefix + sum(ks.branch_pos(i) - prefix for i in range(B))) * per_tok
+    ks.close_branches()
+    return {
+        "metric": "paged_decode_attention_GBps", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": round(graph_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config 3's shape through the stream driver: {L} layers, 32 Q / 8 KV heads x 128 bf16, a "
+                               f"{prefix}-token prefix taken in {chunk}-token chunks (whole layer path), then {B} copy-on-write "
+                               f"branches decoding together, one captured step replayed; value counts LOGICAL bytes",
+                   "branches": B, "layers": L, "shared_tokens": prefix},
+        "decode_step_ms": {"graph_replay": round(graph_ms, 4), "host_launched": round(eager_ms, 4),
+                           "host_time_graph_replay": round(graph_host_ms, 4), "host_time_host_launched": round(eager_host_ms, 4)},
+        "unique_GBps": round(launch_unique * L / (graph_ms * 1e-3) / 1e9, 1),
+        "prefill": {"tokens_per_s": round(prefix / (prefill_ms * 1e-3), 1), "ms": round(prefill_ms, 1),
+                    "attention_TFLOPs_over_whole_path_time": round(prefill_flops / (prefill_ms * 1e-3) / 1e12, 1)},
+        "roofline": None, "cpu_baseline": None,
+    }
+
+
 def run(args):
-    return {3: config3, 4: config4, 5: config5}[args.config](args)
+    return {3: config3, 4: config4, 5: config5, 6: config6}[args.config](args)

@@ -197,7 +197,7 @@ void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t s
         if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
                              ModelConfig::IO_DTYPE, stream) != DRK_OK)
             LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
-    } else if (B >= 4 && shared_tokens_ >= 4096) {
+    } else if (B >= shared_min_branches_ && shared_tokens_ >= shared_min_tokens_) {
         // the branches' common prefix is streamed once for all of them
         paged_gqa_decode_attention_shared(io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, shared_tokens_,
                                           io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(), scale, stream);

@@ -65,6 +65,11 @@ public:
     int  num_branches() const { return (int)branches_.size(); }
     int  branch_id(int i) const { return branches_[i]; }
     int  branch_pos(int i) const { return pos_[i]; }
+    // The prefix (whole blocks) all open branches share.  With at least min_branches open and
+    // at least min_tokens shared, decode streams that prefix once for all branches instead of
+    // once per branch.  Defaults: 4 branches, 4096 tokens.
+    int  shared_tokens() const { return shared_tokens_; }
+    void set_shared_prefix_policy(int min_branches, int min_tokens) { shared_min_branches_ = min_branches; shared_min_tokens_ = min_tokens; }
 
     // One decode step = begin, decode_layer for every full-attention layer, end.
     // begin: blocks for the token each branch is about to write, table sync (this also issues the
@@ -97,6 +102,8 @@ private:
     int* d_len_ = nullptr;
     bool positions_on_device_ = false;
     int shared_tokens_ = 0;          // prefix the open branches share (whole blocks)
+    int shared_min_branches_ = 4;
+    int shared_min_tokens_ = 4096;
     void* graph_ = nullptr;
     int first_layer_of_step_ = -1;   // the layer whose scored call overwrites instead of accumulating
 

@@ -185,6 +185,7 @@ int drk_positions_advance(int32_t *d_pos, int32_t *d_seq_lens, int n, int delta,
 // stream capture of a launch sequence into an executable graph
 int drk_graph_begin_capture(void *stream)
 {
+    if (!stream) return fail(DRK_ERR_INVALID, "graph capture needs a stream of its own: the default (NULL) stream cannot be captured");
     DRK_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
     return DRK_OK;
 }

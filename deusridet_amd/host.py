@@ -81,6 +81,8 @@ SIGNATURES = {
     "drkh_kvs_num_branches": (_i32, [_vp]),
     "drkh_kvs_branch_id": (_i32, [_vp, _i32]),
     "drkh_kvs_branch_pos": (_i32, [_vp, _i32]),
+    "drkh_kvs_shared_tokens": (_i32, [_vp]),
+    "drkh_kvs_set_shared_prefix_policy": (None, [_vp, _i32, _i32]),
     "drkh_kvs_begin_decode_step": (_i32, [_vp, _vp]),
     "drkh_kvs_decode_layer": (None, [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "drkh_kvs_end_decode_step": (None, [_vp, _vp]),
@@ -184,6 +186,8 @@ class KvStream:
     def end_prefill(self, M): lib().drkh_kvs_end_prefill(self._h, M)
     def current_pos(self): return lib().drkh_kvs_current_pos(self._h)
     def open_branches(self, n): return lib().drkh_kvs_open_branches(self._h, n)
+    def shared_tokens(self): return lib().drkh_kvs_shared_tokens(self._h)
+    def set_shared_prefix_policy(self, min_branches, min_tokens): lib().drkh_kvs_set_shared_prefix_policy(self._h, min_branches, min_tokens)
     def close_branches(self): lib().drkh_kvs_close_branches(self._h)
     def num_branches(self): return lib().drkh_kvs_num_branches(self._h)
     def branch_id(self, i): return lib().drkh_kvs_branch_id(self._h, i)

@@ -152,6 +152,8 @@ void  drkh_kvs_close_branches(void *ks);
 int   drkh_kvs_num_branches(void *ks);
 int   drkh_kvs_branch_id(void *ks, int i);
 int   drkh_kvs_branch_pos(void *ks, int i);
+int   drkh_kvs_shared_tokens(void *ks);
+void  drkh_kvs_set_shared_prefix_policy(void *ks, int min_branches, int min_tokens);
 int   drkh_kvs_begin_decode_step(void *ks, void *stream);
 void  drkh_kvs_decode_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
                             const void *k_norm, void *q_scratch, void *attn_out, void *stream);

@@ -101,7 +101,7 @@ int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream); 
  * lets a captured decode step move its own positions on. */
 int drk_positions_advance(int32_t *d_pos, int32_t *d_seq_lens, int n, int delta, void *stream);
 /* Capture what is enqueued on `stream` between begin and end into an executable graph
- * (thread-local capture mode), launch it, destroy it.  None of the append / attention entry
+ * (thread-local capture mode; a stream of its own, not the NULL stream), launch it, destroy it.  None of the append / attention entry
  * points allocates, memsets or synchronises, so a whole decode step can be captured. */
 int drk_graph_begin_capture(void *stream);
 int drk_graph_end_capture(void *stream, void **graph_exec);

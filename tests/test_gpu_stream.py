@@ -86,9 +86,11 @@ def oracle_layer(og, opool, table_rows, pos, layer, qg, k, v, qw, kw, tab, prefi
     return want / (1.0 + np.exp(-g))
 
 
-def run_session(nbranch, steps, mode, seed=120, scorer=False):
+def run_session(nbranch, steps, mode, seed=120, scorer=False, shared_policy=None):
     """mode 'eager' or 'graph'.  Returns (prefill outs, per-step decode outs, final pool, session)."""
     s = Session(nbranch, scorer)
+    if shared_policy:
+        s.ks.set_shared_prefix_policy(*shared_policy)
     rng = np.random.default_rng(seed)
     qw, kw = U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT)
     s.set_weights(qw, kw)
@@ -116,6 +118,7 @@ def run_session(nbranch, steps, mode, seed=120, scorer=False):
     assert np.array_equal(s.pool(), opool)
     # ---- decode branches ----
     assert s.ks.open_branches(nbranch) == nbranch
+    assert s.ks.shared_tokens() == 96                                  # six whole blocks of the 100-token prefix
     ids = [s.ks.branch_id(i) for i in range(nbranch)]
     assert ids == list(range(1, nbranch + 1)) and all(s.ks.branch_pos(i) == 100 for i in range(nbranch))
     step_inputs = [[tuple(U.normal_bits(rng, sh, DT, m) for sh, m in (((nbranch, QH, 2 * D), 1.0), ((nbranch, KVH, D), 0.7),
@@ -190,6 +193,29 @@ def test_stream_session_matches_the_oracle_and_its_graph_replay(dev):
             assert np.array_equal(rec_g["decode"][step][layer], rec_e["decode"][step][layer]), (step, layer)
     assert np.array_equal(pool_g, pool_e)
     s_g.ks.close_branches()
+
+
+def test_stream_session_with_the_prefix_streamed_once(dev):
+    """Same session, but the decode attention reads the branches' common prefix once for all of
+    them (here from 64 shared tokens on; the default asks for 4096): still the oracle's results
+    within the attention tolerance (checked inside run_session), the same pool bytes as the
+    per-branch path, and the captured step replays to the eager bits."""
+    rec_e, pool_e, s_e = run_session(4, 4, "eager", seed=122, shared_policy=(2, 64))
+    s_e.ks.close_branches()
+    del s_e
+    rec_g, pool_g, s_g = run_session(4, 4, "graph", seed=122, shared_policy=(2, 64))
+    for step in range(4):
+        for layer in range(L):
+            assert np.array_equal(rec_g["decode"][step][layer], rec_e["decode"][step][layer]), (step, layer)
+    assert np.array_equal(pool_g, pool_e)
+    s_g.ks.close_branches()
+    del s_g
+    rec_p, pool_p, s_p = run_session(4, 4, "eager", seed=122)           # per-branch path, same inputs
+    assert np.array_equal(pool_p, pool_e)
+    diff = max(np.abs(U.from_bits(rec_p["decode"][st][l], DT).astype(np.float64) - U.from_bits(rec_e["decode"][st][l], DT)).max()
+               for st in range(4) for l in range(L))
+    assert 0 < diff < 2e-2                                             # another summation order, not another result
+    s_p.ks.close_branches()
 
 
 def test_stream_session_feeds_the_scorer(dev):
