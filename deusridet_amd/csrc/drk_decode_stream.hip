@@ -181,15 +181,15 @@ template <int DT> struct VRegs { uint4 r0, r1, r2, r3; };
 template <> struct VRegs<DRK_INT8> { uint2 r0, r1, r2, r3; };
 template <> struct VRegs<DRK_FP8_E4M3> { uint2 r0, r1, r2, r3; };
 
-// The 16-token run of one kv head at byte offset `off` of the layer (kNone: the run has no
-// page).  A missing run is loaded from offset 0 -- always mapped -- instead of being
+// The 16-token run of one kv head at offset `off` of the layer, in units of 16 bytes (kNone:
+// the run has no page).  A missing run is loaded from offset 0 -- always mapped -- instead of being
 // predicated off: its K only feeds scores that are masked anyway, and its V is cleared
 // by the consumer where a stale bit pattern could matter.
 template <int DT>
 __device__ __forceinline__ KRegs<DT> load_k(const uint8_t *__restrict__ layer, uint32_t off, int lane)
 {
     KRegs<DT> k;
-    const uint8_t *p = layer + (off == 0xffffffffu ? 0u : off) + (size_t)lane * 16;
+    const uint8_t *p = layer + ((size_t)(off == 0xffffffffu ? 0u : off) << 4) + (size_t)lane * 16;
     if constexpr (KvTraits<DT>::q8) {
         k.r0 = ld_stream128(p);
         k.r1 = ld_stream128(p + 1024);
@@ -206,7 +206,7 @@ template <int DT>
 __device__ __forceinline__ VRegs<DT> load_v(const uint8_t *__restrict__ layer, uint32_t off, uint32_t kv_plane, int lane)
 {
     VRegs<DT> v;
-    const uint8_t *p = layer + (off == 0xffffffffu ? 0u : off) + kv_plane;
+    const uint8_t *p = layer + ((size_t)(off == 0xffffffffu ? 0u : off) << 4) + kv_plane;
     if constexpr (KvTraits<DT>::q8) {
         p += (size_t)lane * 8;
         v.r0 = ld_stream64(p);
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     __shared__ __align__(16) float kscale_lds[2][kSTile];
     __shared__ __align__(16) float vscale_lds[2][kSTile];
     __shared__ __align__(16) UnitDesc udesc[kMaxUnits];
-    __shared__ __align__(16) uint2 gdesc[kMaxUnits][4];       // per 16-token group: K byte offset (kNone: skip), scale offset
+    __shared__ __align__(16) uint2 gdesc[kMaxUnits][4];       // per 16-token group: K offset (kNone: skip), scale offset; 16-byte units
     __shared__ int s_incl[64], s_len[64];
 
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -353,10 +353,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
             const int blk = A.tables[(size_t)b * A.table_stride + lb];
             if (blk >= 0 && blk < A.NB) {
+                // every term is a multiple of 16 bytes (pp is a multiple of 16, plane sizes of 16 * 16)
                 const unsigned pp = (unsigned)(tg - lb * A.bs);
-                const unsigned base = (unsigned)blk * A.block_stride;
-                gd.x = base + (unsigned)kvh * A.head_stride + pp * A.row_bytes;
-                gd.y = base + 2u * A.kv_plane + ((unsigned)kvh * A.bs + pp) * 2u;
+                const size_t base = (size_t)blk * A.block_stride;
+                gd.x = (unsigned)((base + (size_t)kvh * A.head_stride + (size_t)pp * A.row_bytes) >> 4);
+                gd.y = (unsigned)((base + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + pp) * 2) >> 4);
             }
         }
         gdesc[ui][grp] = gd;
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     auto load_scales = [&](uint2 gd) -> uint32_t {
         // lanes 0-15: K scale of token lane, lanes 16-31: V scale of token lane-16
         if (DT != DRK_INT8 || gd.x == kNone || lane >= 32) return 0u;
-        return *(const uint16_t *)(A.pool_layer + gd.y + (lane & 15) * 2 + (lane >= 16 ? A.scale_plane : 0u));
+        return *(const uint16_t *)(A.pool_layer + ((size_t)gd.y << 4) + (lane & 15) * 2 + (lane >= 16 ? A.scale_plane : 0u));
     };
     auto load_q = [&](int bq) -> uint32_t {
         // one packed pair of query head (bq + w) per lane; quantised pages multiply in fp16
@@ -394,19 +395,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     float m_run = -INFINITY, l_run = 0.0f, qbias = 0.0f;
     uint32_t qs[64];
 
-    uint2 gd = gdesc[0][w];
-    KRegs<DT> kreg = load_k<DT>(A.pool_layer, gd.x, lane);
-    VRegs<DT> vreg = load_v<DT>(A.pool_layer, gd.x, A.kv_plane, lane);
-    bool vhole = gd.x == kNone;                               // the run vreg was loaded for has no page
-    uint32_t sreg = load_scales(gd);
+    // Loads run PF tiles ahead of their use: one for 16-bit pages; two for 8-bit pages, whose
+    // tiles are half the bytes, so that as much is in flight per workgroup.
+    constexpr int PF = Q8 ? 2 : 1;
+    uint2 gd0 = gdesc[0][w];
+    KRegs<DT> kreg0 = load_k<DT>(A.pool_layer, gd0.x, lane);
+    VRegs<DT> vreg0 = load_v<DT>(A.pool_layer, gd0.x, A.kv_plane, lane);
+    bool vhole0 = gd0.x == kNone;                             // the run vreg was loaded for has no page
+    uint32_t sreg0 = load_scales(gd0);
+    uint2 gd1 = make_uint2(kNone, 0u);
+    KRegs<DT> kreg1 = {};
+    VRegs<DT> vreg1 = {};
+    bool vhole1 = true;
+    uint32_t sreg1 = 0u;
+    if (PF == 2 && nunits > 1) {
+        gd1 = gdesc[1][w];
+        kreg1 = load_k<DT>(A.pool_layer, gd1.x, lane);
+        vreg1 = load_v<DT>(A.pool_layer, gd1.x, A.kv_plane, lane);
+        vhole1 = gd1.x == kNone;
+        sreg1 = load_scales(gd1);
+    }
     uint32_t qv = load_q(udesc[0].bq);
 
-    for (int it = 0; it < nunits; it++) {
+    auto tile_step = [&](const int it, KRegs<DT> &kreg, VRegs<DT> &vreg, uint32_t &sreg, bool &vhole, uint2 &gd) {
         const int buf = it & 1;
         const UnitDesc ud = udesc[it];
         const int flags = __builtin_amdgcn_readfirstlane(ud.flags);
         const int tile_lim = __builtin_amdgcn_readfirstlane(ud.tile_lim);
-        const bool has_next = it + 1 < nunits;
+        const bool has_next = it + PF < nunits;
         if (flags & 1) {                          // Q of the segment's head into scalar registers
 #pragma unroll
             for (int i = 0; i < 64; i++) qs[i] = __builtin_amdgcn_readlane(qv, i);
@@ -426,11 +442,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             else vscale_lds[buf][w * 16 + lane - 16] = sc;
         }
         if (has_next) {
-            gd = gdesc[it + 1][w];
+            gd = gdesc[it + PF][w];
             kreg = load_k<DT>(A.pool_layer, gd.x, lane);
             sreg = load_scales(gd);
-            if (flags & 2) qv = load_q(udesc[it + 1].bq);
         }
+        if ((flags & 2) && it + 1 < nunits) qv = load_q(udesc[it + 1].bq);
         __syncthreads();
 
         // ---- B: scores of head w for the tile's 64 tokens, tile softmax -----------------
@@ -568,6 +584,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             m_run = -INFINITY;
             l_run = 0.0f;
         }
+    };
+
+    if constexpr (PF == 1) {
+        for (int it = 0; it < nunits; it++) tile_step(it, kreg0, vreg0, sreg0, vhole0, gd0);
+    } else {
+        for (int it = 0; it < nunits; it += 2) {
+            tile_step(it, kreg0, vreg0, sreg0, vhole0, gd0);
+            if (it + 1 < nunits) tile_step(it + 1, kreg1, vreg1, sreg1, vhole1, gd1);
+        }
     }
 }
 
@@ -704,9 +729,10 @@ int launch_block_mass(const float *lse_groups, const float *lse_rows, const int3
 
 bool stream_decode_supported(const Lay &a, int B)
 {
-    // offsets inside a layer are kept in 32 bits by the unit descriptors
+    // offsets inside a layer are kept in 32 bits, in units of 16 bytes, by the unit descriptors:
+    // a layer of the pool may hold up to 64 GiB
     return a.D == 128 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && B >= 1 && B <= 64 &&
-           a.layer_stride <= 0xffff0000ull;
+           a.layer_stride <= (0xffff0000ull << 4);
 }
 
 static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens, int *grid, int *unit_tiles, int *Pmax)

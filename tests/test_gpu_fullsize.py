@@ -190,3 +190,80 @@ def test_config5_full_chunk_prefill_rows(dev):
     U.sync()
     ok, ma, _ = U.rel_abs_ok(out[rows].float().cpu().numpy(), od.float().cpu().numpy())
     assert ok, ma
+
+
+@pytest.mark.parametrize("dtype", [cabi.BF16, cabi.INT8])
+def test_pages_beyond_4GiB_of_a_layer(dev, dtype):
+    """A pool whose single layer holds more than 4 GiB (a 288 GB part at 36 layers has 7 GiB per
+    layer): pages at the top of it must be appended, gathered and attended exactly like the same
+    tokens in a small pool -- same bits from the same production kernel, which must really be the
+    tiled one (the portable kernel agrees within the attention tolerance only)."""
+    torch = _torch()
+    L, KVH, QH, D, bs = 1, 8, 32, 128, 16
+    lib = cabi.lib()
+    probe = cabi.layout(L, KVH, QH, D, bs, 1, dtype)
+    per_block = lib.drk_kv_pool_bytes(C.byref(probe))
+    NB_big = int(5.2 * 2 ** 30) // per_block
+    lens_h = np.array([1500, 333], dtype=np.int32)
+    nblk = [(int(n) + bs - 1) // bs for n in lens_h]
+    stride = max(nblk) + 1
+    NB_small = sum(nblk) + 3
+    rng = np.random.default_rng(44)
+    sp = U.stream_ptr()
+    gen = torch.Generator(device="cuda").manual_seed(44)
+    q = torch.randn(2, QH, D, device="cuda", generator=gen).to(torch.bfloat16)
+    kv = [(torch.randn(int(n), KVH, D, device="cuda", generator=gen).to(torch.bfloat16),
+           torch.randn(int(n), KVH, D, device="cuda", generator=gen).to(torch.bfloat16)) for n in lens_h]
+    lens = torch.from_numpy(lens_h).cuda()
+    outs, flats = {}, {}
+    for name, NB in (("small", NB_small), ("big", NB_big)):
+        g = cabi.layout(L, KVH, QH, D, bs, NB, dtype)
+        assert lib.drk_kv_pool_bytes(C.byref(g)) > (4 << 30) or name == "small"
+        ids = rng.permutation(NB_small) if name == "small" else NB - 1 - 5 * rng.permutation(NB_small)   # the top of the layer
+        tab = np.full((2, stride), -1, dtype=np.int32)
+        o = 0
+        for b in range(2):
+            tab[b, :nblk[b]] = ids[o:o + nblk[b]]
+            o += nblk[b]
+        dtab = torch.from_numpy(tab).cuda()
+        pool = torch.empty(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+        for b in range(2):
+            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(dtab.data_ptr() + b * stride * 4), 0, 1, 0,
+                      int(lens_h[b]), U.p(kv[b][0]), U.p(kv[b][1]), cabi.BF16, sp)
+        E = 1 if dtype == cabi.INT8 else 2
+        n0 = int(lens_h[0])
+        flat = torch.empty(2 * n0 * KVH * D * E, dtype=torch.uint8, device="cuda")
+        scales = torch.empty(2 * n0 * KVH, dtype=torch.float16, device="cuda") if dtype == cabi.INT8 else None
+        cabi.call("drk_kv_extract", C.byref(g), U.p(flat), U.p(scales), U.p(pool), U.p(dtab), 0, n0, 1, sp)
+        wsb = lib.drk_decode_workspace_bytes(C.byref(g), 2, int(lens_h.max()))
+        ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+        out = torch.zeros(2, QH, D, dtype=torch.bfloat16, device="cuda")
+        cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(q), U.p(pool), U.p(dtab), stride, U.p(lens), 2,
+                  int(lens_h.max()), U.p(out), 0, float(1 / np.sqrt(D)), cabi.BF16, 0, U.p(ws), wsb, sp)
+        U.sync()
+        outs[name] = out.view(torch.int16).cpu().numpy()
+        flats[name] = (flat.cpu().numpy(), scales.view(torch.int16).cpu().numpy() if scales is not None else None)
+        if name == "big":
+            lib.drk_debug_force_portable_decode(1)
+            try:
+                out2 = torch.zeros(2, QH, D, dtype=torch.bfloat16, device="cuda")
+                wsb2 = lib.drk_decode_workspace_bytes(C.byref(g), 2, int(lens_h.max()))
+                ws2 = torch.empty(wsb2, dtype=torch.uint8, device="cuda")
+                cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(q), U.p(pool), U.p(dtab), stride, U.p(lens), 2,
+                          int(lens_h.max()), U.p(out2), 0, float(1 / np.sqrt(D)), cabi.BF16, 0, U.p(ws2), wsb2, sp)
+                U.sync()
+            finally:
+                lib.drk_debug_force_portable_decode(0)
+            portable = out2.float().cpu().numpy()
+        del pool
+    assert np.array_equal(flats["big"][0], flats["small"][0])
+    if dtype == cabi.INT8:
+        assert np.array_equal(flats["big"][1], flats["small"][1])
+    else:
+        k0 = kv[0][0].view(torch.int16).cpu().numpy().reshape(-1)
+        assert np.array_equal(flats["big"][0].view(np.int16)[:k0.size], k0)               # 16-bit pages: pure copies
+    assert np.array_equal(outs["big"], outs["small"])
+    got = torch.from_numpy(outs["big"]).view(torch.bfloat16).float().numpy()
+    assert not np.array_equal(got, portable)                         # a different kernel produced the bits ...
+    ok, ma, _ = U.rel_abs_ok(got, portable.astype(np.float64))
+    assert ok, ma                                                     # ... of the same result
