@@ -197,7 +197,7 @@ int drk_graph_end_capture(void *stream, void **graph_exec)
     DRK_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    hipGraphDestroy(graph);
+    (void)hipGraphDestroy(graph);
     if (e != hipSuccess) return fail(DRK_ERR_HIP, "hipGraphInstantiate: %s", hipGetErrorString(e));
     *graph_exec = (void *)exec;
     return DRK_OK;

@@ -12,15 +12,21 @@
 // into at most ceil(tiles/U)+1 pieces; each piece leaves (o[128], m, l) per query
 // head in the workspace and stream_merge_kernel folds them.
 //
-// Per tile (the same three phases as decode_tiled_kernel in drk_decode.hip):
-//   A  each wave stores the 16-token page row run it loaded one tile earlier into
-//      LDS (K only; 272-byte pitch), converting int8 / fp8 codes to fp16 on the
-//      way, and issues the 128-bit loads of the next unit's K;
-//   B  wave w = query head w: lane = token, Q in 64 SGPRs, v_dot2 over the row in
-//      LDS, no cross-lane reduction for the dot; tile softmax by wave reductions;
-//      p (times the V scale for int8) to LDS;
-//   C  wave w multiplies its own 16 tokens of V, straight from the global loads,
-//      into 4 heads x 8 dims of fp32 per lane; then issues the next unit's V loads.
+// Inside the tile loop a wave never waits for another.  Wave w owns tokens [16w, 16w+16)
+// of every tile with a softmax state of its own (running maximum and sum per query head,
+// 4 heads x 128 dims of output), and both products run on the matrix cores with the four
+// query heads padded to a 16-wide operand:
+//   S[token][head] = K[16 tokens x 128 dims] Q^T                    4 x v_mfma_f32_16x16x32
+//   O[head][dim]  += P[heads x 16 tokens] V[16 tokens x 128 dims]   8 x v_mfma_f32_16x16x16
+// The accumulator layout of the first product (lane = head + 16 g, registers = tokens
+// 4g..4g+3) is exactly the A-operand layout of the second, so the probabilities never
+// leave their lane.  K goes through a wave-private LDS region (272-byte pitch) only to
+// change lanes -- 16-byte chunks as loaded become one token row per lane -- and int8 /
+// fp8 codes become fp16 on the way; V is loaded with tokens 4g..4g+3 of 8 dims in each
+// lane and paired up by byte permutes (which is also where its codes become fp16).  The
+// padding costs nothing that matters: the matrix cores are idle otherwise, and the vector
+// ALU work per tile is a third of what the same products cost as v_dot2.  The four waves'
+// states meet once per segment, through LDS, in the usual (o, m, l) algebra.
 #include "drk_common.hpp"
 
 #include <math.h>
@@ -28,10 +34,10 @@
 namespace drk {
 
 // Workgroups of the persistent grid on a 256-CU part; 0 = by storage type: 2 per CU
-// for 16-bit pages (bandwidth-bound: fewer, longer runs stream best), 3 per CU for
-// 8-bit pages (the dequantising waves need the extra latency hiding).
+// for 16-bit pages (bandwidth-bound: fewer, longer runs stream best), 4 per CU -- all
+// that fit -- for 8-bit pages, whose tiles are half the bytes.
 int g_stream_wgs = 0;
-static inline int stream_wgs(const Lay &a) { return g_stream_wgs > 0 ? g_stream_wgs : (a.E == 1 ? 768 : 512); }
+static inline int stream_wgs(const Lay &a) { return g_stream_wgs > 0 ? g_stream_wgs : (a.E == 1 ? 1024 : 512); }
 
 constexpr int kSTile = 64;
 constexpr int kSRow = 272;
@@ -177,9 +183,6 @@ struct UnitDesc {                    // one 64-token tile of one (branch, kv hea
 template <int DT> struct KRegs { uint4 r0, r1, r2, r3; };
 template <> struct KRegs<DRK_INT8> { uint4 r0, r1; };
 template <> struct KRegs<DRK_FP8_E4M3> { uint4 r0, r1; };
-template <int DT> struct VRegs { uint4 r0, r1, r2, r3; };
-template <> struct VRegs<DRK_INT8> { uint2 r0, r1, r2, r3; };
-template <> struct VRegs<DRK_FP8_E4M3> { uint2 r0, r1, r2, r3; };
 
 // The 16-token run of one kv head at offset `off` of the layer, in units of 16 bytes (kNone:
 // the run has no page).  A missing run is loaded from offset 0 -- always mapped -- instead of being
@@ -200,27 +203,6 @@ __device__ __forceinline__ KRegs<DT> load_k(const uint8_t *__restrict__ layer, u
         k.r3 = ld_stream128(p + 3072);
     }
     return k;
-}
-
-template <int DT>
-__device__ __forceinline__ VRegs<DT> load_v(const uint8_t *__restrict__ layer, uint32_t off, uint32_t kv_plane, int lane)
-{
-    VRegs<DT> v;
-    const uint8_t *p = layer + ((size_t)(off == 0xffffffffu ? 0u : off) << 4) + kv_plane;
-    if constexpr (KvTraits<DT>::q8) {
-        p += (size_t)lane * 8;
-        v.r0 = ld_stream64(p);
-        v.r1 = ld_stream64(p + 512);
-        v.r2 = ld_stream64(p + 1024);
-        v.r3 = ld_stream64(p + 1536);
-    } else {
-        p += (size_t)lane * 16;
-        v.r0 = ld_stream128(p);
-        v.r1 = ld_stream128(p + 1024);
-        v.r2 = ld_stream128(p + 2048);
-        v.r3 = ld_stream128(p + 3072);
-    }
-    return v;
 }
 
 // stage the wave's 16 K rows as 16-bit values: rows w*16 .. w*16+15 of the tile
@@ -257,72 +239,122 @@ __device__ __forceinline__ void stage_k(uint8_t *tile_lds, const KRegs<DT> &k, i
     }
 }
 
-// o[h][e] += p[a][h] * V[a][e] + p[b][h] * V[b][e] for two token rows a, b and the 8 dims of
-// this lane: one v_dot2 per (head, dim) over the token pair.  pp holds, per head, the packed
-// 16-bit weights (p[a], p[b]); the rows' values are paired up by byte permutes.
-template <int DT, typename VR>
-__device__ __forceinline__ void pv_pair(float (&o)[4][8], float (&psum)[4], const VR &va, const VR &vb, const uint4 pp)
+typedef _Float16 w_f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 w_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 w_f16x4 __attribute__((ext_vector_type(4)));
+typedef short w_s16x4 __attribute__((ext_vector_type(4)));
+typedef float w_f32x4 __attribute__((ext_vector_type(4)));
+
+template <int DOT>
+__device__ __forceinline__ w_f32x4 w_mfma_qk(const uint4 &a, const uint4 &b, w_f32x4 c)
 {
-    constexpr int DOT = KvTraits<DT>::dot;
-    uint32_t pr[8];
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (DOT == DRK_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(w_bf16x8, a), __builtin_bit_cast(w_bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(w_f16x8, a), __builtin_bit_cast(w_f16x8, b), c, 0, 0, 0);
+#else
+    (void)a; (void)b;
+    return c;
+#endif
+}
+template <int DOT>
+__device__ __forceinline__ w_f32x4 w_mfma_pv(const uint2 &a, const uint2 &b, w_f32x4 c)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (DOT == DRK_BF16)
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(w_s16x4, a), __builtin_bit_cast(w_s16x4, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(w_f16x4, a), __builtin_bit_cast(w_f16x4, b), c, 0, 0, 0);
+#else
+    (void)a; (void)b;
+    return c;
+#endif
+}
+
+// V of one 16-token group as the second product wants it: lane (g = lane/16, c = lane%16)
+// holds rows 4g..4g+3, dims 8c..8c+7
+template <int DT> struct VRegsW { uint4 r[4]; };
+template <> struct VRegsW<DRK_INT8> { uint2 r[4]; };
+template <> struct VRegsW<DRK_FP8_E4M3> { uint2 r[4]; };
+
+template <int DT>
+__device__ __forceinline__ VRegsW<DT> load_v_w(const uint8_t *__restrict__ layer, uint32_t off, uint32_t kv_plane, int lane)
+{
+    VRegsW<DT> v;
+    const uint8_t *p = layer + ((size_t)(off == 0xffffffffu ? 0u : off) << 4) + kv_plane;
     if constexpr (KvTraits<DT>::q8) {
-        const uint32_t i0 = s_perm(vb.x, va.x, 0x05010400u), i1 = s_perm(vb.x, va.x, 0x07030602u);   // a0 b0 a1 b1 | a2 b2 a3 b3
-        const uint32_t i2 = s_perm(vb.y, va.y, 0x05010400u), i3 = s_perm(vb.y, va.y, 0x07030602u);
-        if constexpr (DT == DRK_INT8) {
-            int8x4_to_f16x4(i0, pr[0], pr[1]);
-            int8x4_to_f16x4(i1, pr[2], pr[3]);
-            int8x4_to_f16x4(i2, pr[4], pr[5]);
-            int8x4_to_f16x4(i3, pr[6], pr[7]);
-            psum[0] = s_dot2<DOT>(pp.x, kF16Ones, psum[0]);          // the +1152 is taken out at the end
-            psum[1] = s_dot2<DOT>(pp.y, kF16Ones, psum[1]);
-            psum[2] = s_dot2<DOT>(pp.z, kF16Ones, psum[2]);
-            psum[3] = s_dot2<DOT>(pp.w, kF16Ones, psum[3]);
-        } else {
-            fp8x4_to_f16x4(i0, pr[0], pr[1]);
-            fp8x4_to_f16x4(i1, pr[2], pr[3]);
-            fp8x4_to_f16x4(i2, pr[4], pr[5]);
-            fp8x4_to_f16x4(i3, pr[6], pr[7]);
+        p += (size_t)(lane >> 4) * 512 + (lane & 15) * 8;
+#pragma unroll
+        for (int j = 0; j < 4; j++) v.r[j] = ld_stream64(p + j * 128);
+    } else {
+        p += (size_t)(lane >> 4) * 1024 + (lane & 15) * 16;
+#pragma unroll
+        for (int j = 0; j < 4; j++) v.r[j] = ld_stream128(p + j * 256);
+    }
+    return v;
+}
+
+// B operands of the second product: vb[e] = V[4g..4g+3][8c+e] as four 16-bit values
+template <int DT>
+__device__ __forceinline__ void v_operands(const VRegsW<DT> &v, uint2 (&vb)[8])
+{
+    if constexpr (KvTraits<DT>::q8) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {                     // low / high dword of the 8 codes: dims 4h..4h+3
+            const uint32_t a0 = h ? v.r[0].y : v.r[0].x, a1 = h ? v.r[1].y : v.r[1].x;
+            const uint32_t a2 = h ? v.r[2].y : v.r[2].x, a3 = h ? v.r[3].y : v.r[3].x;
+            const uint32_t i01a = s_perm(a1, a0, 0x05010400u), i01b = s_perm(a1, a0, 0x07030602u);   // t0 t1 pairs of dims 0,1 | 2,3
+            const uint32_t i23a = s_perm(a3, a2, 0x05010400u), i23b = s_perm(a3, a2, 0x07030602u);   // t2 t3
+            uint32_t lo[4], hi[4];
+            if constexpr (DT == DRK_INT8) {
+                int8x4_to_f16x4(i01a, lo[0], lo[1]);
+                int8x4_to_f16x4(i01b, lo[2], lo[3]);
+                int8x4_to_f16x4(i23a, hi[0], hi[1]);
+                int8x4_to_f16x4(i23b, hi[2], hi[3]);
+            } else {
+                fp8x4_to_f16x4(i01a, lo[0], lo[1]);
+                fp8x4_to_f16x4(i01b, lo[2], lo[3]);
+                fp8x4_to_f16x4(i23a, hi[0], hi[1]);
+                fp8x4_to_f16x4(i23b, hi[2], hi[3]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) vb[4 * h + e] = make_uint2(lo[e], hi[e]);
         }
     } else {
-        const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
+        const uint32_t w0[4] = {v.r[0].x, v.r[0].y, v.r[0].z, v.r[0].w}, w1[4] = {v.r[1].x, v.r[1].y, v.r[1].z, v.r[1].w};
+        const uint32_t w2[4] = {v.r[2].x, v.r[2].y, v.r[2].z, v.r[2].w}, w3[4] = {v.r[3].x, v.r[3].y, v.r[3].z, v.r[3].w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            pr[2 * i] = s_perm(wb[i], wa[i], 0x05040100u);
-            pr[2 * i + 1] = s_perm(wb[i], wa[i], 0x07060302u);
+            vb[2 * i] = make_uint2(s_perm(w1[i], w0[i], 0x05040100u), s_perm(w3[i], w2[i], 0x05040100u));
+            vb[2 * i + 1] = make_uint2(s_perm(w1[i], w0[i], 0x07060302u), s_perm(w3[i], w2[i], 0x07060302u));
         }
-    }
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-        o[0][e] = s_dot2<DOT>(pr[e], pp.x, o[0][e]);
-        o[1][e] = s_dot2<DOT>(pr[e], pp.y, o[1][e]);
-        o[2][e] = s_dot2<DOT>(pr[e], pp.z, o[2][e]);
-        o[3][e] = s_dot2<DOT>(pr[e], pp.w, o[3][e]);
     }
 }
 
+constexpr int kWaveLds = 16 * kSRow;       // one wave's K rows
+
 template <int DT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void decode_stream_kernel(StreamArgs A)
+__global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
 {
-    constexpr bool Q8 = KvTraits<DT>::q8;
+    [[maybe_unused]] constexpr bool Q8 = KvTraits<DT>::q8;
     constexpr int DOT = KvTraits<DT>::dot;
     constexpr uint32_t kNone = 0xffffffffu;
-    __shared__ __align__(16) uint8_t k_lds[2][kSTile * kSRow];
-    __shared__ __align__(16) uint16_t p_lds[2][kSTile * 4];   // [pair of rows][head][row of the pair], 16-bit weights
-    __shared__ __align__(16) float alpha_lds[2][4];
-    __shared__ __align__(16) float kscale_lds[2][kSTile];
-    __shared__ __align__(16) float vscale_lds[2][kSTile];
+    __shared__ __align__(16) uint8_t k_lds[4][kWaveLds];
+    __shared__ __align__(16) float o_lds[4][4][128];          // [wave][head][dim], segment ends only
+    __shared__ float mw_lds[4][4], lw_lds[4][4];
     __shared__ __align__(16) UnitDesc udesc[kMaxUnits];
-    __shared__ __align__(16) uint2 gdesc[kMaxUnits][4];       // per 16-token group: K offset (kNone: skip), scale offset; 16-byte units
+    __shared__ __align__(16) uint2 gdesc[kMaxUnits][4];
     __shared__ int s_incl[64], s_len[64];
 
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
-    const int lrow = lane >> 4, lchunk = lane & 15;
+    const int g = lane >> 4, c = lane & 15;
 
     // ---- the workgroup's run of units and one descriptor per unit ---------------------
     const int len_i = lane < A.B ? (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host) : 0;
     const int nt_i = len_i > 0 ? max((len_i + kSTile - 1) / kSTile - A.start_tile, 0) : 0;
-    int incl = nt_i;                                           // inclusive prefix of tiles over branches
+    int incl = nt_i;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
         const int t = __shfl_up(incl, off);
@@ -338,7 +370,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     __syncthreads();
     for (int i = threadIdx.x; i < nunits * 4; i += 256) {
         const int ui = i >> 2, grp = i & 3, u = u0 + ui;
-        int lo = 0, hi = A.B - 1;                              // first branch whose cumulative units exceed u
+        int lo = 0, hi = A.B - 1;
         while (lo < hi) {
             const int mid = (lo + hi) >> 1;
             if (A.KVH * s_incl[mid] > u) hi = mid; else lo = mid + 1;
@@ -346,14 +378,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         const int b = lo;
         const int excl = b ? s_incl[b - 1] : 0, nt = s_incl[b] - excl, len = s_len[b];
         const int rem = u - A.KVH * excl, kvh = rem / nt, trel = rem - kvh * nt;
-        const int tile = trel + A.start_tile;                  // absolute tile of the branch
+        const int tile = trel + A.start_tile;
         const int tg = tile * kSTile + grp * 16;
         uint2 gd = make_uint2(kNone, 0u);
         if (tg < len) {
             const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
             const int blk = A.tables[(size_t)b * A.table_stride + lb];
             if (blk >= 0 && blk < A.NB) {
-                // every term is a multiple of 16 bytes (pp is a multiple of 16, plane sizes of 16 * 16)
                 const unsigned pp = (unsigned)(tg - lb * A.bs);
                 const size_t base = (size_t)blk * A.block_stride;
                 gd.x = (unsigned)((base + (size_t)kvh * A.head_stride + (size_t)pp * A.row_bytes) >> 4);
@@ -372,189 +403,193 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
     __syncthreads();
 
-    auto load_scales = [&](uint2 gd) -> uint32_t {
-        // lanes 0-15: K scale of token lane, lanes 16-31: V scale of token lane-16
-        if (DT != DRK_INT8 || gd.x == kNone || lane >= 32) return 0u;
-        return *(const uint16_t *)(A.pool_layer + ((size_t)gd.y << 4) + (lane & 15) * 2 + (lane >= 16 ? A.scale_plane : 0u));
-    };
-    auto load_q = [&](int bq) -> uint32_t {
-        // one packed pair of query head (bq + w) per lane; quantised pages multiply in fp16
-        uint32_t v = ((const uint32_t *)(A.q + (size_t)(bq + w) * 256))[lane];
-#if defined(__HIP_DEVICE_COMPILE__)
-        if (Q8 && A.io_dtype == DRK_BF16)
-            v = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v), bf16_hi(v)));
-#endif
-        return v;
+    uint8_t *const klds = &k_lds[w][0];
+    // the 4 K scales and the 4 V scales of tokens 4g..4g+3 (int8 pages)
+    auto load_scales_w = [&](uint2 gd, uint2 &ks, uint2 &vs) {
+        if (DT != DRK_INT8) return;
+        const uint8_t *p = A.pool_layer + ((size_t)(gd.x == kNone ? 0u : gd.y) << 4) + g * 8;
+        ks = *(const uint2 *)p;
+        vs = *(const uint2 *)(p + A.scale_plane);
     };
 
-    float o[4][8], psum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    w_f32x4 o[8];
 #pragma unroll
-    for (int hh = 0; hh < 4; hh++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[hh][e] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f, qbias = 0.0f;
-    uint32_t qs[64];
+    for (int e = 0; e < 8; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -INFINITY, l_lane = 0.0f, ps_lane = 0.0f, qbias = 0.0f;
+    uint4 qop[4];
 
-    // Loads run PF tiles ahead of their use: one for 16-bit pages; two for 8-bit pages, whose
-    // tiles are half the bytes, so that as much is in flight per workgroup.
-    constexpr int PF = Q8 ? 2 : 1;
-    uint2 gd0 = gdesc[0][w];
+    uint2 gd0 = gdesc[0][w], ks0 = {}, vs0 = {};
     KRegs<DT> kreg0 = load_k<DT>(A.pool_layer, gd0.x, lane);
-    VRegs<DT> vreg0 = load_v<DT>(A.pool_layer, gd0.x, A.kv_plane, lane);
-    bool vhole0 = gd0.x == kNone;                             // the run vreg was loaded for has no page
-    uint32_t sreg0 = load_scales(gd0);
-    uint2 gd1 = make_uint2(kNone, 0u);
-    KRegs<DT> kreg1 = {};
-    VRegs<DT> vreg1 = {};
-    bool vhole1 = true;
-    uint32_t sreg1 = 0u;
-    if (PF == 2 && nunits > 1) {
-        gd1 = gdesc[1][w];
-        kreg1 = load_k<DT>(A.pool_layer, gd1.x, lane);
-        vreg1 = load_v<DT>(A.pool_layer, gd1.x, A.kv_plane, lane);
-        vhole1 = gd1.x == kNone;
-        sreg1 = load_scales(gd1);
-    }
-    uint32_t qv = load_q(udesc[0].bq);
+    VRegsW<DT> vreg0 = load_v_w<DT>(A.pool_layer, gd0.x, A.kv_plane, lane);
+    load_scales_w(gd0, ks0, vs0);
 
-    auto tile_step = [&](const int it, KRegs<DT> &kreg, VRegs<DT> &vreg, uint32_t &sreg, bool &vhole, uint2 &gd) {
-        const int buf = it & 1;
+    auto tile_step = [&](const int it, KRegs<DT> &kreg, VRegsW<DT> &vreg, uint2 &ksr, uint2 &vsr, uint2 &gd) {
         const UnitDesc ud = udesc[it];
         const int flags = __builtin_amdgcn_readfirstlane(ud.flags);
         const int tile_lim = __builtin_amdgcn_readfirstlane(ud.tile_lim);
-        const bool has_next = it + PF < nunits;
-        if (flags & 1) {                          // Q of the segment's head into scalar registers
+        const bool hole = __builtin_amdgcn_readfirstlane((int)gd.x) == (int)kNone;   // the group this step's registers were loaded for
+        const bool has_next = it + 1 < nunits;
+        if (flags & 1) {
+            // Q^T as the B operand: lane (head c, dims 32 kk + 8 g ..) -- heads 4..15 are padding
+            float sq = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 64; i++) qs[i] = __builtin_amdgcn_readlane(qv, i);
-            if (DT == DRK_INT8) {                 // sum of the head's (fp16) query values, for the code offset
-                float sq = 0.0f;
-#pragma unroll
-                for (int i = 0; i < 64; i++) sq = s_dot2<DOT>(qs[i], kF16Ones, sq);
+            for (int kk = 0; kk < 4; kk++) {
+                uint4 v = make_uint4(0u, 0u, 0u, 0u);
+                if (c < 4) v = *(const uint4 *)(A.q + (size_t)(ud.bq + c) * 256 + kk * 64 + g * 16);
+#if defined(__HIP_DEVICE_COMPILE__)
+                if (Q8 && A.io_dtype == DRK_BF16) {          // quantised pages multiply in fp16
+                    v.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.x), bf16_hi(v.x)));
+                    v.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.y), bf16_hi(v.y)));
+                    v.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.z), bf16_hi(v.z)));
+                    v.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.w), bf16_hi(v.w)));
+                }
+#endif
+                qop[kk] = v;
+                if (DT == DRK_INT8) {
+                    sq = s_dot2<DOT>(v.x, kF16Ones, sq);
+                    sq = s_dot2<DOT>(v.y, kF16Ones, sq);
+                    sq = s_dot2<DOT>(v.z, kF16Ones, sq);
+                    sq = s_dot2<DOT>(v.w, kF16Ones, sq);
+                }
+            }
+            if (DT == DRK_INT8) {                            // sum of the head's query values, for the code offset
+                sq += __shfl_xor(sq, 16);
+                sq += __shfl_xor(sq, 32);
                 qbias = kI8Bias * sq;
             }
         }
 
-        // ---- A: stage K (and scales), start the next unit's K loads -------------------
-        stage_k<DT>(&k_lds[buf][0], kreg, w, lane);
-        if (DT == DRK_INT8 && lane < 32) {
-            const float sc = f16_bits_to_f((uint16_t)sreg);
-            if (lane < 16) kscale_lds[buf][w * 16 + lane] = sc;
-            else vscale_lds[buf][w * 16 + lane - 16] = sc;
+        // ---- K: registers -> the wave's LDS rows -> one token row per lane; next K loads ----
+        stage_k<DT>(klds, kreg, 0, lane);
+        float ks[4] = {1.0f, 1.0f, 1.0f, 1.0f}, vs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+        if (DT == DRK_INT8) {
+            ks[0] = f16_bits_to_f((uint16_t)(ksr.x & 0xffffu)); ks[1] = f16_bits_to_f((uint16_t)(ksr.x >> 16));
+            ks[2] = f16_bits_to_f((uint16_t)(ksr.y & 0xffffu)); ks[3] = f16_bits_to_f((uint16_t)(ksr.y >> 16));
+            vs[0] = f16_bits_to_f((uint16_t)(vsr.x & 0xffffu)); vs[1] = f16_bits_to_f((uint16_t)(vsr.x >> 16));
+            vs[2] = f16_bits_to_f((uint16_t)(vsr.y & 0xffffu)); vs[3] = f16_bits_to_f((uint16_t)(vsr.y >> 16));
         }
         if (has_next) {
-            gd = gdesc[it + PF][w];
+            gd = gdesc[it + 1][w];
             kreg = load_k<DT>(A.pool_layer, gd.x, lane);
-            sreg = load_scales(gd);
+            load_scales_w(gd, ksr, vsr);
         }
-        if ((flags & 2) && it + 1 < nunits) qv = load_q(udesc[it + 1].bq);
-        __syncthreads();
-
-        // ---- B: scores of head w for the tile's 64 tokens, tile softmax -----------------
+        w_f32x4 sacc = {0.0f, 0.0f, 0.0f, 0.0f};
         {
-            const uint8_t *krow = &k_lds[buf][lane * kSRow];
-            float acc = 0.0f;
-            uint4 ka[4], kb[4];
+            const uint8_t *arow = klds + c * kSRow + g * 16;
+            uint4 ka[4];
 #pragma unroll
-            for (int c = 0; c < 4; c++) ka[c] = *(const uint4 *)(krow + c * 16);
+            for (int kk = 0; kk < 4; kk++) ka[kk] = *(const uint4 *)(arow + kk * 64);
 #pragma unroll
-            for (int g4 = 0; g4 < 4; g4++) {
-                if (g4 < 3) {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) kb[c] = *(const uint4 *)(krow + ((g4 + 1) * 4 + c) * 16);
-                }
-#pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    const int qi = (g4 * 4 + c) * 4;
-                    acc = s_dot2<DOT>(ka[c].x, qs[qi + 0], acc);
-                    acc = s_dot2<DOT>(ka[c].y, qs[qi + 1], acc);
-                    acc = s_dot2<DOT>(ka[c].z, qs[qi + 2], acc);
-                    acc = s_dot2<DOT>(ka[c].w, qs[qi + 3], acc);
-                }
-                asm volatile("" : "+v"(acc) :: "memory");   // at most two groups of LDS reads in flight
-#pragma unroll
-                for (int c = 0; c < 4; c++) ka[c] = kb[c];
-            }
-            const bool live = lane < tile_lim && gdesc[it][lane >> 4].x != kNone;
-            if (DT == DRK_INT8) acc = (acc - qbias) * kscale_lds[buf][lane];
-            float sc = acc * A.scale_log2e;
-            sc = live ? sc : -INFINITY;
-            const float m_new = fmaxf(m_run, s_wave_max(sc));
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-            const float p = s_exp2(sc - m_use);
-            const float alpha = s_exp2(m_run - m_use);
-            // sum of p: the DPP steps leave each row of 16 lanes (= one 16-token group) with its own sum
-            float rs = p;
-            rs += s_dpp<0xB1>(rs);
-            rs += s_dpp<0x4E>(rs);
-            rs += s_dpp<0x141>(rs);
-            rs += s_dpp<0x140>(rs);
-            l_run = l_run * alpha + ((s_lane(rs, 0) + s_lane(rs, 16)) + (s_lane(rs, 32) + s_lane(rs, 48)));
-            if (A.lse_groups && (lane & 15) == 0) {
-                const int gi = (flags >> 2) * 4 + (lane >> 4);
-                if (gi < A.lse_stride)
-                    A.lse_groups[(size_t)(ud.bq + w) * A.lse_stride + gi] = rs > 0.0f ? m_use + __builtin_log2f(rs) : -INFINITY;
-            }
-            m_run = m_new;
-            float pw = p;
-            if (DT == DRK_INT8) pw = live ? p * vscale_lds[buf][lane] : 0.0f;   // a stale scale may be anything
-            {
-                // rows r, r+4 of a wave's 16 form a pair, and so do r+8, r+12: phase C holds exactly these
-                uint16_t pb;
-                if constexpr (DOT == DRK_BF16) pb = __builtin_bit_cast(uint16_t, (__bf16)pw);
-                else pb = __builtin_bit_cast(uint16_t, (_Float16)pw);
-                const int r = lane & 15, pidx = ((lane >> 4) * 4 + (r & 3)) * 2 + (r >> 3);
-                p_lds[buf][(pidx * 4 + w) * 2 + ((r >> 2) & 1)] = pb;
-            }
-            if (lane == 0) alpha_lds[buf][w] = alpha;
+            for (int kk = 0; kk < 4; kk++) sacc = w_mfma_qk<DOT>(ka[kk], qop[kk], sacc);
         }
-        __syncthreads();
 
-        // ---- C: o += P V over this wave's 16 tokens, all 4 heads ----------------------
+        // ---- softmax of head c over this wave's tokens 4g..4g+3 (+ the other three lane groups) ----
+        const int t0 = w * 16 + g * 4;
+        float sc[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float x = sacc[j];
+            if (DT == DRK_INT8) x = (x - qbias) * ks[j];
+            x *= A.scale_log2e;
+            sc[j] = (!hole && t0 + j < tile_lim) ? x : -INFINITY;
+        }
+        float mloc = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = s_exp2(m_run - m_use);
+        m_run = m_new;
+        float p[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) p[j] = s_exp2(sc[j] - m_use);
+        const float rs = (p[0] + p[1]) + (p[2] + p[3]);
+        l_lane = fmaf(l_lane, alpha, rs);
+        if (A.lse_groups) {
+            float rt = rs;
+            rt += __shfl_xor(rt, 16);
+            rt += __shfl_xor(rt, 32);
+            const int gi = (flags >> 2) * 4 + w;
+            if (lane < 4 && gi < A.lse_stride)
+                A.lse_groups[(size_t)(ud.bq + lane) * A.lse_stride + gi] = rt > 0.0f ? m_use + __builtin_log2f(rt) : -INFINITY;
+        }
+        uint2 pa;                                             // A operand of the second product: P[head c][tokens 4g..4g+3]
         {
-            const float4 al = *(const float4 *)&alpha_lds[buf][0];
-            if (al.x != 1.0f || al.y != 1.0f || al.z != 1.0f || al.w != 1.0f) {
+            float pw[4];
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    o[0][e] *= al.x; o[1][e] *= al.y; o[2][e] *= al.z; o[3][e] *= al.w;
-                }
-                psum[0] *= al.x; psum[1] *= al.y; psum[2] *= al.z; psum[3] *= al.w;
+            for (int j = 0; j < 4; j++) pw[j] = (DT == DRK_INT8) ? ((!hole && t0 + j < tile_lim) ? p[j] * vs[j] : 0.0f) : p[j];
+            if constexpr (DOT == DRK_BF16) {
+                pa.x = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[1]) << 16);
+                pa.y = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[3]) << 16);
+            } else {
+                pa.x = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[1]) << 16);
+                pa.y = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[3]) << 16);
             }
-            const int r0 = w * 16 + lrow;
-            if (DT != DRK_INT8 && (tile_lim < kSTile || vhole)) {   // rows without a token may hold anything (NaN)
-                if (vhole || r0 >= tile_lim) vreg.r0 = {};
-                if (vhole || r0 + 4 >= tile_lim) vreg.r1 = {};
-                if (vhole || r0 + 8 >= tile_lim) vreg.r2 = {};
-                if (vhole || r0 + 12 >= tile_lim) vreg.r3 = {};
+            if (DT == DRK_INT8) {                             // sum of the weights as the product sees them, for the code offset
+                float t = s_dot2<DOT>(pa.x, kF16Ones, 0.0f);
+                t = s_dot2<DOT>(pa.y, kF16Ones, t);
+                ps_lane = fmaf(ps_lane, alpha, t);
             }
-            const uint4 *pl = (const uint4 *)&p_lds[buf][(w * 4 + lrow) * 16];
-            pv_pair<DT>(o, psum, vreg.r0, vreg.r1, pl[0]);
-            pv_pair<DT>(o, psum, vreg.r2, vreg.r3, pl[1]);
-        }
-        if (has_next) {
-            vreg = load_v<DT>(A.pool_layer, gd.x, A.kv_plane, lane);
-            vhole = gd.x == kNone;
         }
 
-        // ---- the segment's last tile: leave (o, m, l) for the merge ----------------------
+        // ---- O: rescale (the accumulators hold head j in register j, lanes 0..15), then P V ----
+        {
+            const float a0 = s_lane(alpha, 0), a1 = s_lane(alpha, 1), a2 = s_lane(alpha, 2), a3 = s_lane(alpha, 3);
+            if (a0 != 1.0f || a1 != 1.0f || a2 != 1.0f || a3 != 1.0f) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) { o[e][0] *= a0; o[e][1] *= a1; o[e][2] *= a2; o[e][3] *= a3; }
+            }
+            if (DT != DRK_INT8 && (hole || w * 16 + 16 > tile_lim)) {    // rows without a token may hold anything (NaN)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (hole || t0 + j >= tile_lim) vreg.r[j] = {};
+            }
+            uint2 vb[8];
+            v_operands<DT>(vreg, vb);
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = w_mfma_pv<DOT>(pa, vb[e], o[e]);
+        }
+        if (has_next) vreg = load_v_w<DT>(A.pool_layer, gd.x, A.kv_plane, lane);
+
+        // ---- the segment's last tile: fold the four waves, leave (o, m, l) for the merge ----
         if (flags & 2) {
-#pragma unroll
-            for (int hh = 0; hh < 4; hh++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    float v = o[hh][e];
-                    if (DT == DRK_INT8) v -= kI8Bias * psum[hh];
-                    v += __shfl_xor(v, 16);
-                    v += __shfl_xor(v, 32);
-                    o[hh][e] = v;
-                }
-            float *o_lds = (float *)&k_lds[0][0];        // [wave][head][128] fp32 = 8 KiB; K reads are done
+            float lw = l_lane, pw = ps_lane;
+            lw += __shfl_xor(lw, 16);
+            lw += __shfl_xor(lw, 32);
+            if (DT == DRK_INT8) {
+                pw += __shfl_xor(pw, 16);
+                pw += __shfl_xor(pw, 32);
+            }
+            if (lane < 4) { mw_lds[w][lane] = m_run; lw_lds[w][lane] = lw; }
             __syncthreads();
-            if (lrow == 0) {
+            float f_own[4], M_all = -INFINITY, L_all = 0.0f;         // f_own[j]: this wave's weight for head j
 #pragma unroll
-                for (int hh = 0; hh < 4; hh++) {
-                    float *dst = o_lds + (w * 4 + hh) * 128 + lchunk * 8;
-                    *(float4 *)dst = make_float4(o[hh][0], o[hh][1], o[hh][2], o[hh][3]);
-                    *(float4 *)(dst + 4) = make_float4(o[hh][4], o[hh][5], o[hh][6], o[hh][7]);
+            for (int j = 0; j < 4; j++) {
+                const float M = fmaxf(fmaxf(mw_lds[0][j], mw_lds[1][j]), fmaxf(mw_lds[2][j], mw_lds[3][j]));
+                const float mo = mw_lds[w][j];
+                f_own[j] = mo == -INFINITY ? 0.0f : s_exp2(mo - M);
+                if (j == w) {
+                    M_all = M;
+#pragma unroll
+                    for (int ww = 0; ww < 4; ww++) {
+                        const float mm = mw_lds[ww][j];
+                        if (mm != -INFINITY) L_all = fmaf(lw_lds[ww][j], s_exp2(mm - M), L_all);
+                    }
+                }
+            }
+            float bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (DT == DRK_INT8) {
+                bias[0] = kI8Bias * s_lane(pw, 0); bias[1] = kI8Bias * s_lane(pw, 1);
+                bias[2] = kI8Bias * s_lane(pw, 2); bias[3] = kI8Bias * s_lane(pw, 3);
+            }
+            if (lane < 16) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float *dst = &o_lds[w][j][c * 8];
+                    *(float4 *)dst = make_float4((o[0][j] - bias[j]) * f_own[j], (o[1][j] - bias[j]) * f_own[j],
+                                                 (o[2][j] - bias[j]) * f_own[j], (o[3][j] - bias[j]) * f_own[j]);
+                    *(float4 *)(dst + 4) = make_float4((o[4][j] - bias[j]) * f_own[j], (o[5][j] - bias[j]) * f_own[j],
+                                                       (o[6][j] - bias[j]) * f_own[j], (o[7][j] - bias[j]) * f_own[j]);
                 }
             }
             __syncthreads();
@@ -563,37 +598,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                 float2 acc = make_float2(0.0f, 0.0f);
 #pragma unroll
                 for (int ww = 0; ww < 4; ww++) {
-                    const float2 v = *(const float2 *)(o_lds + (ww * 4 + w) * 128 + d);
+                    const float2 v = *(const float2 *)&o_lds[ww][w][d];
                     acc.x += v.x;
                     acc.y += v.y;
                 }
                 const size_t pi = (size_t)(ud.bq + w) * A.Pmax + ud.piece;
                 *(float2 *)(A.part_o + pi * 128 + d) = acc;
                 if (lane == 0) {
-                    A.part_m[pi] = m_run;
-                    A.part_l[pi] = l_run;
+                    A.part_m[pi] = M_all;
+                    A.part_l[pi] = L_all;
                 }
             }
-            __syncthreads();                             // o_lds is free again before the next tile is staged
 #pragma unroll
-            for (int hh = 0; hh < 4; hh++) {
-                psum[hh] = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 8; e++) o[hh][e] = 0.0f;
-            }
+            for (int e = 0; e < 8; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             m_run = -INFINITY;
-            l_run = 0.0f;
+            l_lane = 0.0f;
+            ps_lane = 0.0f;
         }
     };
 
-    if constexpr (PF == 1) {
-        for (int it = 0; it < nunits; it++) tile_step(it, kreg0, vreg0, sreg0, vhole0, gd0);
-    } else {
-        for (int it = 0; it < nunits; it += 2) {
-            tile_step(it, kreg0, vreg0, sreg0, vhole0, gd0);
-            if (it + 1 < nunits) tile_step(it + 1, kreg1, vreg1, sreg1, vhole1, gd1);
-        }
-    }
+    for (int it = 0; it < nunits; it++) tile_step(it, kreg0, vreg0, ks0, vs0, gd0);
 }
 
 // grid (QH, B), block 256: fold the pieces of (branch, q head) -- the stream kernel's

@@ -36,7 +36,6 @@ constexpr int kPfBN = 64;         // KV tokens per tile
 // bank-conflict cycles).
 constexpr int kPfPitch = 272;
 constexpr int kPfPitchV = 288;
-constexpr int kPfRows = 128;      // rows per workgroup (32 query tokens x 4 heads)
 constexpr float kLog2eP = 1.4426950408889634f;
 
 typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
