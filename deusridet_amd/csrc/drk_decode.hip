@@ -6,7 +6,9 @@
 // byte is fetched from HBM once (the reference launches one block per query head
 // and re-reads the kv head's pages QH/KVH times, paged_attention.cu:179-282).
 //
-// Two kernels produce the partials:
+// The production kernel is decode_stream_kernel (drk_decode_stream.hip: head_dim 128 or
+// 256, up to 16 query heads per kv head, every storage type).  Two more kernels produce
+// partials here, for everything else and as cross-checks:
 //   decode_tiled_kernel    head_dim 128, 16-bit K/V, 4 query heads per kv head:
 //                          64-token K tiles staged in LDS (row-padded so that
 //                          lane = token reads are bank-conflict free), Q held in
@@ -591,7 +593,9 @@ static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size
 
 static bool shared_path_ok(const Lay &a, int B, int shared)
 {
-    return !g_force_portable && stream_decode_supported(a, B) && a.E == 2 && shared >= kTile;   // the caller checks scale > 0
+    // the prefix pass is the MFMA prefill kernel: head_dim 128, 4 query heads per kv head, 16-bit pages
+    return !g_force_portable && stream_decode_supported(a, B) && a.D == 128 && a.QH / a.KVH == 4 && a.E == 2 &&
+           shared >= kTile;   // the caller checks scale > 0
 }
 
 int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
@@ -713,7 +717,7 @@ size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_
     if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0) return 0;
     size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);
     const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
-    if (stream_decode_supported(a, B) && a.E == 2 && shared >= kTile) {
+    if (stream_decode_supported(a, B) && a.D == 128 && a.QH / a.KVH == 4 && a.E == 2 && shared >= kTile) {
         size_t s2 = shared_need(a, B, max_seq_len, shared, nullptr);
         if (s2 > need) need = s2;
     }
@@ -781,7 +785,7 @@ int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const
     if (B == 0 || max_seq_len == 0) return DRK_OK;
     if (B > 65535) return fail(DRK_ERR_INVALID, "decode_mass: more than 65535 branches");
     if (g_force_portable || !stream_decode_supported(a, B))
-        return fail(DRK_ERR_UNSUPPORTED, "decode_mass: needs head_dim 128, 4 query heads per kv head, block_size %% 16 == 0, at most 64 branches");
+        return fail(DRK_ERR_UNSUPPORTED, "decode_mass: needs head_dim 128 or 256, at most 16 query heads per kv head, block_size %% 16 == 0, at most 64 branches");
     if (mass_stride < (max_seq_len + a.bs - 1) / a.bs)
         return fail(DRK_ERR_INVALID, "decode_mass: mass_stride %d is less than the %d blocks of max_seq_len", mass_stride,
                     (max_seq_len + a.bs - 1) / a.bs);

@@ -1,6 +1,6 @@
 // drk_decode_stream.hip -- the production paged GQA decode kernel: persistent,
-// stream-K style, for head_dim 128 with 4 query heads per KV head and fp16, bf16,
-// int8 (+fp16 scale per token and head) or fp8-e4m3 pages.
+// stream-K style, for head_dim 128 or 256 with 1..16 query heads per KV head and fp16,
+// bf16, int8 (+fp16 scale per token and head) or fp8-e4m3 pages.
 //
 // The unit of work is one 64-token tile of one (branch, kv head).  Units are
 // numbered branch-major, then kv head, then tile; workgroup g owns the run
@@ -9,18 +9,18 @@
 // run that crosses from one (branch, kv head) to the next keeps its load pipeline
 // full: the next unit's K/V (and the next segment's Q) are already in flight when
 // the current segment's partial result is written.  A (branch, kv head) is cut
-// into at most ceil(tiles/U)+1 pieces; each piece leaves (o[128], m, l) per query
+// into at most ceil(tiles/U)+1 pieces; each piece leaves (o[D], m, l) per query
 // head in the workspace and stream_merge_kernel folds them.
 //
 // Inside the tile loop a wave never waits for another.  Wave w owns tokens [16w, 16w+16)
 // of every tile with a softmax state of its own (running maximum and sum per query head,
-// 4 heads x 128 dims of output), and both products run on the matrix cores with the four
-// query heads padded to a 16-wide operand:
-//   S[token][head] = K[16 tokens x 128 dims] Q^T                    4 x v_mfma_f32_16x16x32
-//   O[head][dim]  += P[heads x 16 tokens] V[16 tokens x 128 dims]   8 x v_mfma_f32_16x16x16
+// heads x head_dim of output), and both products run on the matrix cores with the query
+// heads of the group padded to a 16-wide operand (for head_dim D):
+//   S[token][head] = K[16 tokens x D dims] Q^T                  D/32 x v_mfma_f32_16x16x32
+//   O[head][dim]  += P[heads x 16 tokens] V[16 tokens x D dims]   D/16 x v_mfma_f32_16x16x16
 // The accumulator layout of the first product (lane = head + 16 g, registers = tokens
 // 4g..4g+3) is exactly the A-operand layout of the second, so the probabilities never
-// leave their lane.  K goes through a wave-private LDS region (272-byte pitch) only to
+// leave their lane.  K goes through a wave-private LDS region (pitch 2 D + 16 bytes) only to
 // change lanes -- 16-byte chunks as loaded become one token row per lane -- and int8 /
 // fp8 codes become fp16 on the way; V is loaded with tokens 4g..4g+3 of 8 dims in each
 // lane and paired up by byte permutes (which is also where its codes become fp16).  The
@@ -34,13 +34,12 @@
 namespace drk {
 
 // Workgroups of the persistent grid on a 256-CU part; 0 = by storage type: 2 per CU
-// for 16-bit pages (bandwidth-bound: fewer, longer runs stream best), 4 per CU -- all
-// that fit -- for 8-bit pages, whose tiles are half the bytes.
+// for 16-bit pages (bandwidth-bound: fewer, longer runs stream best) and for head_dim
+// 256 (all that fit), 4 per CU for 8-bit pages of head_dim 128, whose tiles are half the bytes.
 int g_stream_wgs = 0;
-static inline int stream_wgs(const Lay &a) { return g_stream_wgs > 0 ? g_stream_wgs : (a.E == 1 ? 1024 : 512); }
+static inline int stream_wgs(const Lay &a) { return g_stream_wgs > 0 ? g_stream_wgs : (a.E == 1 && a.D == 128 ? 1024 : 512); }
 
 constexpr int kSTile = 64;
-constexpr int kSRow = 272;
 constexpr float kSLog2e = 1.4426950408889634f;
 
 typedef __bf16 s_bf16x2 __attribute__((ext_vector_type(2)));
@@ -175,67 +174,66 @@ constexpr int kMaxUnits = 256;       // units one workgroup may own (descriptor 
 struct UnitDesc {                    // one 64-token tile of one (branch, kv head)
     int tile_lim;                    // tokens of the tile that exist: seq_len - tile*64 (may exceed 64)
     int flags;                       // bit 0: first tile of a segment of this workgroup, bit 1: last; bits 2..: tile index
-    int bq;                          // branch*QH + kvh*4: first query row of the group (Q, partial slots)
+    int bq;                          // branch*QH + kvh*(QH/KVH): first query row of the group (Q, partial slots)
     int piece;                       // partial slot of the segment inside its (branch, q head)
 };
 
-// one wave's 16-token group of a tile, as loaded from the pool
-template <int DT> struct KRegs { uint4 r0, r1, r2, r3; };
-template <> struct KRegs<DRK_INT8> { uint4 r0, r1; };
-template <> struct KRegs<DRK_FP8_E4M3> { uint4 r0, r1; };
+// Geometry of one instantiation: head_dim D (128 or 256) and the storage type.
+template <int DT, int D> struct StreamGeo {
+    static constexpr bool q8 = KvTraits<DT>::q8;
+    static constexpr int RB = D * (q8 ? 1 : 2);        // bytes of one token row of one kv head in the pool
+    static constexpr int NK = RB / 64;                 // 128-bit loads per lane for a 16-token K run
+    static constexpr int PITCH = D * 2 + 16;           // LDS pitch of a staged (16-bit) K row: 272 / 528
+    static constexpr int NQK = D / 32;                 // v_mfma_f32_16x16x32 per tile and wave
+    static constexpr int NCH = D / 128;                // 8-dim chunks a lane holds of each of its V rows
+    static constexpr int NPV = D / 16;                 // v_mfma_f32_16x16x16 per tile and wave
+};
+
+// one wave's 16-token group of a tile, as loaded from the pool: 16 x RB contiguous bytes
+template <int DT, int D> struct KRegs { uint4 r[StreamGeo<DT, D>::NK]; };
 
 // The 16-token run of one kv head at offset `off` of the layer, in units of 16 bytes (kNone:
 // the run has no page).  A missing run is loaded from offset 0 -- always mapped -- instead of being
 // predicated off: its K only feeds scores that are masked anyway, and its V is cleared
 // by the consumer where a stale bit pattern could matter.
-template <int DT>
-__device__ __forceinline__ KRegs<DT> load_k(const uint8_t *__restrict__ layer, uint32_t off, int lane)
+template <int DT, int D>
+__device__ __forceinline__ KRegs<DT, D> load_k(const uint8_t *__restrict__ layer, uint32_t off, int lane)
 {
-    KRegs<DT> k;
+    KRegs<DT, D> k;
     const uint8_t *p = layer + ((size_t)(off == 0xffffffffu ? 0u : off) << 4) + (size_t)lane * 16;
-    if constexpr (KvTraits<DT>::q8) {
-        k.r0 = ld_stream128(p);
-        k.r1 = ld_stream128(p + 1024);
-    } else {
-        k.r0 = ld_stream128(p);
-        k.r1 = ld_stream128(p + 1024);
-        k.r2 = ld_stream128(p + 2048);
-        k.r3 = ld_stream128(p + 3072);
-    }
+#pragma unroll
+    for (int j = 0; j < StreamGeo<DT, D>::NK; j++) k.r[j] = ld_stream128(p + 1024 * j);
     return k;
 }
 
-// stage the wave's 16 K rows as 16-bit values: rows w*16 .. w*16+15 of the tile
-template <int DT>
-__device__ __forceinline__ void stage_k(uint8_t *tile_lds, const KRegs<DT> &k, int w, int lane)
+// stage the wave's 16 K rows as 16-bit values, one row per PITCH bytes
+template <int DT, int D>
+__device__ __forceinline__ void stage_k(uint8_t *lds, const KRegs<DT, D> &k, int lane)
 {
-    if constexpr (KvTraits<DT>::q8) {
-        // a loaded register holds 16 codes of row (lane>>3) + 8*j, dims (lane&7)*16 ..
-        uint8_t *dst = tile_lds + (w * 16 + (lane >> 3)) * kSRow + (lane & 7) * 32;
-        const uint4 regs[2] = {k.r0, k.r1};
+    using G = StreamGeo<DT, D>;
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < G::NK; j++) {
+        const int bp = lane * 16 + 1024 * j;                 // byte position inside the run
+        const int row = bp / G::RB, col = bp % G::RB;
+        if constexpr (G::q8) {
             uint32_t h[8];
             if constexpr (DT == DRK_INT8) {
-                int8x4_to_f16x4(regs[j].x, h[0], h[1]);
-                int8x4_to_f16x4(regs[j].y, h[2], h[3]);
-                int8x4_to_f16x4(regs[j].z, h[4], h[5]);
-                int8x4_to_f16x4(regs[j].w, h[6], h[7]);
+                int8x4_to_f16x4(k.r[j].x, h[0], h[1]);
+                int8x4_to_f16x4(k.r[j].y, h[2], h[3]);
+                int8x4_to_f16x4(k.r[j].z, h[4], h[5]);
+                int8x4_to_f16x4(k.r[j].w, h[6], h[7]);
             } else {
-                fp8x4_to_f16x4(regs[j].x, h[0], h[1]);
-                fp8x4_to_f16x4(regs[j].y, h[2], h[3]);
-                fp8x4_to_f16x4(regs[j].z, h[4], h[5]);
-                fp8x4_to_f16x4(regs[j].w, h[6], h[7]);
+                fp8x4_to_f16x4(k.r[j].x, h[0], h[1]);
+                fp8x4_to_f16x4(k.r[j].y, h[2], h[3]);
+                fp8x4_to_f16x4(k.r[j].z, h[4], h[5]);
+                fp8x4_to_f16x4(k.r[j].w, h[6], h[7]);
             }
-            *(uint4 *)(dst + j * 8 * kSRow) = make_uint4(h[0], h[1], h[2], h[3]);
-            *(uint4 *)(dst + j * 8 * kSRow + 16) = make_uint4(h[4], h[5], h[6], h[7]);
+            uint8_t *dst = lds + row * G::PITCH + col * 2;
+            *(uint4 *)(dst) = make_uint4(h[0], h[1], h[2], h[3]);
+            *(uint4 *)(dst + 16) = make_uint4(h[4], h[5], h[6], h[7]);
+        } else {
+            *(uint4 *)(lds + row * G::PITCH + col) = k.r[j];
         }
-    } else {
-        uint8_t *dst = tile_lds + (w * 16 + (lane >> 4)) * kSRow + (lane & 15) * 16;
-        *(uint4 *)(dst) = k.r0;
-        *(uint4 *)(dst + 4 * kSRow) = k.r1;
-        *(uint4 *)(dst + 8 * kSRow) = k.r2;
-        *(uint4 *)(dst + 12 * kSRow) = k.r3;
     }
 }
 
@@ -273,76 +271,75 @@ __device__ __forceinline__ w_f32x4 w_mfma_pv(const uint2 &a, const uint2 &b, w_f
 }
 
 // V of one 16-token group as the second product wants it: lane (g = lane/16, c = lane%16)
-// holds rows 4g..4g+3, dims 8c..8c+7
-template <int DT> struct VRegsW { uint4 r[4]; };
-template <> struct VRegsW<DRK_INT8> { uint2 r[4]; };
-template <> struct VRegsW<DRK_FP8_E4M3> { uint2 r[4]; };
+// holds rows 4g..4g+3, dims 128 ch + 8c .. + 7 for each chunk ch
+template <int DT, int D, bool Q8 = KvTraits<DT>::q8> struct VRegs { uint4 r[4][StreamGeo<DT, D>::NCH]; };
+template <int DT, int D> struct VRegs<DT, D, true> { uint2 r[4][StreamGeo<DT, D>::NCH]; };
 
-template <int DT>
-__device__ __forceinline__ VRegsW<DT> load_v_w(const uint8_t *__restrict__ layer, uint32_t off, uint32_t kv_plane, int lane)
+template <int DT, int D>
+__device__ __forceinline__ VRegs<DT, D> load_v(const uint8_t *__restrict__ layer, uint32_t off, uint32_t kv_plane, int lane)
 {
-    VRegsW<DT> v;
-    const uint8_t *p = layer + ((size_t)(off == 0xffffffffu ? 0u : off) << 4) + kv_plane;
-    if constexpr (KvTraits<DT>::q8) {
-        p += (size_t)(lane >> 4) * 512 + (lane & 15) * 8;
+    using G = StreamGeo<DT, D>;
+    VRegs<DT, D> v;
+    const uint8_t *p = layer + ((size_t)(off == 0xffffffffu ? 0u : off) << 4) + kv_plane + (size_t)(lane >> 4) * (4 * G::RB);
 #pragma unroll
-        for (int j = 0; j < 4; j++) v.r[j] = ld_stream64(p + j * 128);
-    } else {
-        p += (size_t)(lane >> 4) * 1024 + (lane & 15) * 16;
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) v.r[j] = ld_stream128(p + j * 256);
-    }
+        for (int ch = 0; ch < G::NCH; ch++) {
+            if constexpr (G::q8) v.r[j][ch] = ld_stream64(p + j * G::RB + ch * 128 + (lane & 15) * 8);
+            else v.r[j][ch] = ld_stream128(p + j * G::RB + ch * 256 + (lane & 15) * 16);
+        }
     return v;
 }
 
-// B operands of the second product: vb[e] = V[4g..4g+3][8c+e] as four 16-bit values
+// B operands of the second product for one chunk: vb[e] = V[4g..4g+3][128 ch + 8c + e] as four 16-bit values
 template <int DT>
-__device__ __forceinline__ void v_operands(const VRegsW<DT> &v, uint2 (&vb)[8])
+__device__ __forceinline__ void v_operands(const uint2 &r0, const uint2 &r1, const uint2 &r2, const uint2 &r3, uint2 (&vb)[8])
 {
-    if constexpr (KvTraits<DT>::q8) {
 #pragma unroll
-        for (int h = 0; h < 2; h++) {                     // low / high dword of the 8 codes: dims 4h..4h+3
-            const uint32_t a0 = h ? v.r[0].y : v.r[0].x, a1 = h ? v.r[1].y : v.r[1].x;
-            const uint32_t a2 = h ? v.r[2].y : v.r[2].x, a3 = h ? v.r[3].y : v.r[3].x;
-            const uint32_t i01a = s_perm(a1, a0, 0x05010400u), i01b = s_perm(a1, a0, 0x07030602u);   // t0 t1 pairs of dims 0,1 | 2,3
-            const uint32_t i23a = s_perm(a3, a2, 0x05010400u), i23b = s_perm(a3, a2, 0x07030602u);   // t2 t3
-            uint32_t lo[4], hi[4];
-            if constexpr (DT == DRK_INT8) {
-                int8x4_to_f16x4(i01a, lo[0], lo[1]);
-                int8x4_to_f16x4(i01b, lo[2], lo[3]);
-                int8x4_to_f16x4(i23a, hi[0], hi[1]);
-                int8x4_to_f16x4(i23b, hi[2], hi[3]);
-            } else {
-                fp8x4_to_f16x4(i01a, lo[0], lo[1]);
-                fp8x4_to_f16x4(i01b, lo[2], lo[3]);
-                fp8x4_to_f16x4(i23a, hi[0], hi[1]);
-                fp8x4_to_f16x4(i23b, hi[2], hi[3]);
-            }
-#pragma unroll
-            for (int e = 0; e < 4; e++) vb[4 * h + e] = make_uint2(lo[e], hi[e]);
+    for (int h = 0; h < 2; h++) {                         // low / high dword of the 8 codes: dims 4h..4h+3
+        const uint32_t a0 = h ? r0.y : r0.x, a1 = h ? r1.y : r1.x, a2 = h ? r2.y : r2.x, a3 = h ? r3.y : r3.x;
+        const uint32_t i01a = s_perm(a1, a0, 0x05010400u), i01b = s_perm(a1, a0, 0x07030602u);   // t0 t1 pairs of dims 0,1 | 2,3
+        const uint32_t i23a = s_perm(a3, a2, 0x05010400u), i23b = s_perm(a3, a2, 0x07030602u);   // t2 t3
+        uint32_t lo[4], hi[4];
+        if constexpr (DT == DRK_INT8) {
+            int8x4_to_f16x4(i01a, lo[0], lo[1]);
+            int8x4_to_f16x4(i01b, lo[2], lo[3]);
+            int8x4_to_f16x4(i23a, hi[0], hi[1]);
+            int8x4_to_f16x4(i23b, hi[2], hi[3]);
+        } else {
+            fp8x4_to_f16x4(i01a, lo[0], lo[1]);
+            fp8x4_to_f16x4(i01b, lo[2], lo[3]);
+            fp8x4_to_f16x4(i23a, hi[0], hi[1]);
+            fp8x4_to_f16x4(i23b, hi[2], hi[3]);
         }
-    } else {
-        const uint32_t w0[4] = {v.r[0].x, v.r[0].y, v.r[0].z, v.r[0].w}, w1[4] = {v.r[1].x, v.r[1].y, v.r[1].z, v.r[1].w};
-        const uint32_t w2[4] = {v.r[2].x, v.r[2].y, v.r[2].z, v.r[2].w}, w3[4] = {v.r[3].x, v.r[3].y, v.r[3].z, v.r[3].w};
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            vb[2 * i] = make_uint2(s_perm(w1[i], w0[i], 0x05040100u), s_perm(w3[i], w2[i], 0x05040100u));
-            vb[2 * i + 1] = make_uint2(s_perm(w1[i], w0[i], 0x07060302u), s_perm(w3[i], w2[i], 0x07060302u));
-        }
+        for (int e = 0; e < 4; e++) vb[4 * h + e] = make_uint2(lo[e], hi[e]);
+    }
+}
+template <int DT>
+__device__ __forceinline__ void v_operands(const uint4 &r0, const uint4 &r1, const uint4 &r2, const uint4 &r3, uint2 (&vb)[8])
+{
+    const uint32_t w0[4] = {r0.x, r0.y, r0.z, r0.w}, w1[4] = {r1.x, r1.y, r1.z, r1.w};
+    const uint32_t w2[4] = {r2.x, r2.y, r2.z, r2.w}, w3[4] = {r3.x, r3.y, r3.z, r3.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        vb[2 * i] = make_uint2(s_perm(w1[i], w0[i], 0x05040100u), s_perm(w3[i], w2[i], 0x05040100u));
+        vb[2 * i + 1] = make_uint2(s_perm(w1[i], w0[i], 0x07060302u), s_perm(w3[i], w2[i], 0x07060302u));
     }
 }
 
-constexpr int kWaveLds = 16 * kSRow;       // one wave's K rows
-
-template <int DT>
-__global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
+// G4: at most 4 query heads per kv head -- they all live in lane group 0 of the accumulators, so
+// per-head factors are wave-uniform (v_readlane) and a segment ends in one round.
+template <int DT, int D, bool G4>
+__global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(StreamArgs A)
 {
-    [[maybe_unused]] constexpr bool Q8 = KvTraits<DT>::q8;
+    using Geo = StreamGeo<DT, D>;
+    [[maybe_unused]] constexpr bool Q8 = Geo::q8;
     constexpr int DOT = KvTraits<DT>::dot;
     constexpr uint32_t kNone = 0xffffffffu;
-    __shared__ __align__(16) uint8_t k_lds[4][kWaveLds];
-    __shared__ __align__(16) float o_lds[4][4][128];          // [wave][head][dim], segment ends only
-    __shared__ float mw_lds[4][4], lw_lds[4][4];
+    __shared__ __align__(16) uint8_t k_lds[4][16 * Geo::PITCH];
+    __shared__ __align__(16) float o_lds[4][4][D];            // [wave][head of the round][dim], segment ends only
+    __shared__ float mw_lds[4][16], lw_lds[4][16];
     __shared__ __align__(16) UnitDesc udesc[kMaxUnits];
     __shared__ __align__(16) uint2 gdesc[kMaxUnits][4];
     __shared__ int s_incl[64], s_len[64];
@@ -350,6 +347,7 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int g = lane >> 4, c = lane & 15;
+    const int GQ = A.QH / A.KVH;                               // query heads per kv head, 1..16
 
     // ---- the workgroup's run of units and one descriptor per unit ---------------------
     const int len_i = lane < A.B ? (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host) : 0;
@@ -370,7 +368,7 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
     __syncthreads();
     for (int i = threadIdx.x; i < nunits * 4; i += 256) {
         const int ui = i >> 2, grp = i & 3, u = u0 + ui;
-        int lo = 0, hi = A.B - 1;
+        int lo = 0, hi = A.B - 1;                              // first branch whose cumulative units exceed u
         while (lo < hi) {
             const int mid = (lo + hi) >> 1;
             if (A.KVH * s_incl[mid] > u) hi = mid; else lo = mid + 1;
@@ -378,13 +376,14 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
         const int b = lo;
         const int excl = b ? s_incl[b - 1] : 0, nt = s_incl[b] - excl, len = s_len[b];
         const int rem = u - A.KVH * excl, kvh = rem / nt, trel = rem - kvh * nt;
-        const int tile = trel + A.start_tile;
+        const int tile = trel + A.start_tile;                  // absolute tile of the branch
         const int tg = tile * kSTile + grp * 16;
         uint2 gd = make_uint2(kNone, 0u);
         if (tg < len) {
             const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
             const int blk = A.tables[(size_t)b * A.table_stride + lb];
             if (blk >= 0 && blk < A.NB) {
+                // every term is a multiple of 16 bytes (pp is a multiple of 16, plane sizes of 16 * 16)
                 const unsigned pp = (unsigned)(tg - lb * A.bs);
                 const size_t base = (size_t)blk * A.block_stride;
                 gd.x = (unsigned)((base + (size_t)kvh * A.head_stride + (size_t)pp * A.row_bytes) >> 4);
@@ -396,7 +395,7 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
             UnitDesc d;
             d.tile_lim = len - tile * kSTile;
             d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0) | (tile << 2);
-            d.bq = b * A.QH + kvh * 4;
+            d.bq = b * A.QH + kvh * GQ;
             d.piece = (int)blockIdx.x - (A.KVH * excl + kvh * nt) / U;
             udesc[ui] = d;
         }
@@ -405,37 +404,38 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
 
     uint8_t *const klds = &k_lds[w][0];
     // the 4 K scales and the 4 V scales of tokens 4g..4g+3 (int8 pages)
-    auto load_scales_w = [&](uint2 gd, uint2 &ks, uint2 &vs) {
+    auto load_scales = [&](uint2 gd, uint2 &ks, uint2 &vs) {
         if (DT != DRK_INT8) return;
         const uint8_t *p = A.pool_layer + ((size_t)(gd.x == kNone ? 0u : gd.y) << 4) + g * 8;
         ks = *(const uint2 *)p;
         vs = *(const uint2 *)(p + A.scale_plane);
     };
 
-    w_f32x4 o[8];
+    w_f32x4 o[Geo::NPV];
 #pragma unroll
-    for (int e = 0; e < 8; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int e = 0; e < Geo::NPV; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     float m_run = -INFINITY, l_lane = 0.0f, ps_lane = 0.0f, qbias = 0.0f;
-    uint4 qop[4];
+    uint4 qop[Geo::NQK];
 
-    uint2 gd0 = gdesc[0][w], ks0 = {}, vs0 = {};
-    KRegs<DT> kreg0 = load_k<DT>(A.pool_layer, gd0.x, lane);
-    VRegsW<DT> vreg0 = load_v_w<DT>(A.pool_layer, gd0.x, A.kv_plane, lane);
-    load_scales_w(gd0, ks0, vs0);
+    uint2 gd = gdesc[0][w], ksr = {}, vsr = {};
+    KRegs<DT, D> kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
+    VRegs<DT, D> vreg = load_v<DT, D>(A.pool_layer, gd.x, A.kv_plane, lane);
+    load_scales(gd, ksr, vsr);
 
-    auto tile_step = [&](const int it, KRegs<DT> &kreg, VRegsW<DT> &vreg, uint2 &ksr, uint2 &vsr, uint2 &gd) {
+    for (int it = 0; it < nunits; it++) {
         const UnitDesc ud = udesc[it];
         const int flags = __builtin_amdgcn_readfirstlane(ud.flags);
         const int tile_lim = __builtin_amdgcn_readfirstlane(ud.tile_lim);
-        const bool hole = __builtin_amdgcn_readfirstlane((int)gd.x) == (int)kNone;   // the group this step's registers were loaded for
+        const bool hole = __builtin_amdgcn_readfirstlane((int)gd.x) == (int)kNone;   // the group the registers were loaded for
+        const int lim = hole ? 0 : tile_lim;                    // tokens of the tile this wave may look at
         const bool has_next = it + 1 < nunits;
         if (flags & 1) {
-            // Q^T as the B operand: lane (head c, dims 32 kk + 8 g ..) -- heads 4..15 are padding
+            // Q^T as the B operand: lane (head c, dims 32 kk + 8 g ..) -- heads GQ..15 are padding
             float sq = 0.0f;
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
+            for (int kk = 0; kk < Geo::NQK; kk++) {
                 uint4 v = make_uint4(0u, 0u, 0u, 0u);
-                if (c < 4) v = *(const uint4 *)(A.q + (size_t)(ud.bq + c) * 256 + kk * 64 + g * 16);
+                if (c < GQ) v = *(const uint4 *)(A.q + (size_t)(ud.bq + c) * (D * 2) + kk * 64 + g * 16);
 #if defined(__HIP_DEVICE_COMPILE__)
                 if (Q8 && A.io_dtype == DRK_BF16) {          // quantised pages multiply in fp16
                     v.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.x), bf16_hi(v.x)));
@@ -460,7 +460,7 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
         }
 
         // ---- K: registers -> the wave's LDS rows -> one token row per lane; next K loads ----
-        stage_k<DT>(klds, kreg, 0, lane);
+        stage_k<DT, D>(klds, kreg, lane);
         float ks[4] = {1.0f, 1.0f, 1.0f, 1.0f}, vs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
         if (DT == DRK_INT8) {
             ks[0] = f16_bits_to_f((uint16_t)(ksr.x & 0xffffu)); ks[1] = f16_bits_to_f((uint16_t)(ksr.x >> 16));
@@ -470,17 +470,20 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
         }
         if (has_next) {
             gd = gdesc[it + 1][w];
-            kreg = load_k<DT>(A.pool_layer, gd.x, lane);
-            load_scales_w(gd, ksr, vsr);
+            kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
+            load_scales(gd, ksr, vsr);
         }
         w_f32x4 sacc = {0.0f, 0.0f, 0.0f, 0.0f};
         {
-            const uint8_t *arow = klds + c * kSRow + g * 16;
-            uint4 ka[4];
+            const uint8_t *arow = klds + c * Geo::PITCH + g * 16;
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++) ka[kk] = *(const uint4 *)(arow + kk * 64);
+            for (int k0 = 0; k0 < Geo::NQK; k0 += 4) {
+                uint4 ka[4];
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++) sacc = w_mfma_qk<DOT>(ka[kk], qop[kk], sacc);
+                for (int kk = 0; kk < 4; kk++) ka[kk] = *(const uint4 *)(arow + (k0 + kk) * 64);
+#pragma unroll
+                for (int kk = 0; kk < 4; kk++) sacc = w_mfma_qk<DOT>(ka[kk], qop[k0 + kk], sacc);
+            }
         }
 
         // ---- softmax of head c over this wave's tokens 4g..4g+3 (+ the other three lane groups) ----
@@ -491,7 +494,7 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
             float x = sacc[j];
             if (DT == DRK_INT8) x = (x - qbias) * ks[j];
             x *= A.scale_log2e;
-            sc[j] = (!hole && t0 + j < tile_lim) ? x : -INFINITY;
+            sc[j] = t0 + j < lim ? x : -INFINITY;
         }
         float mloc = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
@@ -510,14 +513,14 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
             rt += __shfl_xor(rt, 16);
             rt += __shfl_xor(rt, 32);
             const int gi = (flags >> 2) * 4 + w;
-            if (lane < 4 && gi < A.lse_stride)
+            if (lane < GQ && gi < A.lse_stride)
                 A.lse_groups[(size_t)(ud.bq + lane) * A.lse_stride + gi] = rt > 0.0f ? m_use + __builtin_log2f(rt) : -INFINITY;
         }
         uint2 pa;                                             // A operand of the second product: P[head c][tokens 4g..4g+3]
         {
             float pw[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) pw[j] = (DT == DRK_INT8) ? ((!hole && t0 + j < tile_lim) ? p[j] * vs[j] : 0.0f) : p[j];
+            for (int j = 0; j < 4; j++) pw[j] = (DT == DRK_INT8) ? (t0 + j < lim ? p[j] * vs[j] : 0.0f) : p[j];
             if constexpr (DOT == DRK_BF16) {
                 pa.x = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[1]) << 16);
                 pa.y = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[3]) << 16);
@@ -532,24 +535,37 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
             }
         }
 
-        // ---- O: rescale (the accumulators hold head j in register j, lanes 0..15), then P V ----
+        // ---- O: rescale (register j of lane group g holds head 4g + j), then P V ----------------
         {
-            const float a0 = s_lane(alpha, 0), a1 = s_lane(alpha, 1), a2 = s_lane(alpha, 2), a3 = s_lane(alpha, 3);
-            if (a0 != 1.0f || a1 != 1.0f || a2 != 1.0f || a3 != 1.0f) {
+            if constexpr (G4) {
+                const float a0 = s_lane(alpha, 0), a1 = s_lane(alpha, 1), a2 = s_lane(alpha, 2), a3 = s_lane(alpha, 3);
+                if (a0 != 1.0f || a1 != 1.0f || a2 != 1.0f || a3 != 1.0f) {
 #pragma unroll
-                for (int e = 0; e < 8; e++) { o[e][0] *= a0; o[e][1] *= a1; o[e][2] *= a2; o[e][3] *= a3; }
+                    for (int e = 0; e < Geo::NPV; e++) { o[e][0] *= a0; o[e][1] *= a1; o[e][2] *= a2; o[e][3] *= a3; }
+                }
+            } else if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+                const float a0 = __shfl(alpha, 4 * g), a1 = __shfl(alpha, 4 * g + 1);
+                const float a2 = __shfl(alpha, 4 * g + 2), a3 = __shfl(alpha, 4 * g + 3);
+#pragma unroll
+                for (int e = 0; e < Geo::NPV; e++) { o[e][0] *= a0; o[e][1] *= a1; o[e][2] *= a2; o[e][3] *= a3; }
             }
-            if (DT != DRK_INT8 && (hole || w * 16 + 16 > tile_lim)) {    // rows without a token may hold anything (NaN)
+            if (DT != DRK_INT8 && w * 16 + 16 > lim) {               // rows without a token may hold anything (NaN)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    if (hole || t0 + j >= tile_lim) vreg.r[j] = {};
-            }
-            uint2 vb[8];
-            v_operands<DT>(vreg, vb);
+                    if (t0 + j >= lim) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = w_mfma_pv<DOT>(pa, vb[e], o[e]);
+                        for (int ch = 0; ch < Geo::NCH; ch++) vreg.r[j][ch] = {};
+                    }
+            }
+#pragma unroll
+            for (int ch = 0; ch < Geo::NCH; ch++) {
+                uint2 vb[8];
+                v_operands<DT>(vreg.r[0][ch], vreg.r[1][ch], vreg.r[2][ch], vreg.r[3][ch], vb);
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[ch * 8 + e] = w_mfma_pv<DOT>(pa, vb[e], o[ch * 8 + e]);
+            }
         }
-        if (has_next) vreg = load_v_w<DT>(A.pool_layer, gd.x, A.kv_plane, lane);
+        if (has_next) vreg = load_v<DT, D>(A.pool_layer, gd.x, A.kv_plane, lane);
 
         // ---- the segment's last tile: fold the four waves, leave (o, m, l) for the merge ----
         if (flags & 2) {
@@ -560,64 +576,71 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
                 pw += __shfl_xor(pw, 16);
                 pw += __shfl_xor(pw, 32);
             }
-            if (lane < 4) { mw_lds[w][lane] = m_run; lw_lds[w][lane] = lw; }
+            if (lane < 16) { mw_lds[w][lane] = m_run; lw_lds[w][lane] = lw; }   // padded heads too: defined values
             __syncthreads();
-            float f_own[4], M_all = -INFINITY, L_all = 0.0f;         // f_own[j]: this wave's weight for head j
+            float f_own[4], bias[4];                                 // this wave's weight / code offset for head 4g + j
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float M = fmaxf(fmaxf(mw_lds[0][j], mw_lds[1][j]), fmaxf(mw_lds[2][j], mw_lds[3][j]));
-                const float mo = mw_lds[w][j];
+                const int h = G4 ? j : 4 * g + j;
+                const float M = fmaxf(fmaxf(mw_lds[0][h], mw_lds[1][h]), fmaxf(mw_lds[2][h], mw_lds[3][h]));
+                const float mo = mw_lds[w][h];
                 f_own[j] = mo == -INFINITY ? 0.0f : s_exp2(mo - M);
-                if (j == w) {
-                    M_all = M;
+                if constexpr (G4) bias[j] = DT == DRK_INT8 ? kI8Bias * s_lane(pw, j) : 0.0f;
+                else bias[j] = DT == DRK_INT8 ? kI8Bias * __shfl(pw, h) : 0.0f;
+            }
+            const int rounds = G4 ? 1 : (GQ + 3) >> 2;               // 4 heads per round: head 4r + w is stored by wave w
+            for (int r = 0; r < rounds; r++) {
+                if (r > 0) __syncthreads();                          // the previous round's sums have been read
+                if (g == r) {
 #pragma unroll
-                    for (int ww = 0; ww < 4; ww++) {
-                        const float mm = mw_lds[ww][j];
-                        if (mm != -INFINITY) L_all = fmaf(lw_lds[ww][j], s_exp2(mm - M), L_all);
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int ch = 0; ch < Geo::NCH; ch++) {
+                            float *dst = &o_lds[w][j][ch * 128 + c * 8];
+                            const w_f32x4 *oc = &o[ch * 8];
+                            *(float4 *)dst = make_float4((oc[0][j] - bias[j]) * f_own[j], (oc[1][j] - bias[j]) * f_own[j],
+                                                         (oc[2][j] - bias[j]) * f_own[j], (oc[3][j] - bias[j]) * f_own[j]);
+                            *(float4 *)(dst + 4) = make_float4((oc[4][j] - bias[j]) * f_own[j], (oc[5][j] - bias[j]) * f_own[j],
+                                                               (oc[6][j] - bias[j]) * f_own[j], (oc[7][j] - bias[j]) * f_own[j]);
+                        }
+                }
+                // (m, l) of head 4r + w over the four waves; read here, before the barrier, because a wave
+                // that is through with this segment may overwrite its slots for the next one
+                const int h = 4 * r + w;
+                const float M = fmaxf(fmaxf(mw_lds[0][h], mw_lds[1][h]), fmaxf(mw_lds[2][h], mw_lds[3][h]));
+                float L = 0.0f;
+#pragma unroll
+                for (int ww = 0; ww < 4; ww++) {
+                    const float mm = mw_lds[ww][h];
+                    if (mm != -INFINITY) L = fmaf(lw_lds[ww][h], s_exp2(mm - M), L);
+                }
+                __syncthreads();
+                if (h < GQ) {
+                    constexpr int VEC = D / 64;
+                    const int d = lane * VEC;
+                    float acc[VEC];
+#pragma unroll
+                    for (int x = 0; x < VEC; x++) acc[x] = 0.0f;
+#pragma unroll
+                    for (int ww = 0; ww < 4; ww++)
+#pragma unroll
+                        for (int x = 0; x < VEC; x++) acc[x] += o_lds[ww][w][d + x];
+                    const size_t pi = (size_t)(ud.bq + h) * A.Pmax + ud.piece;
+#pragma unroll
+                    for (int x = 0; x < VEC; x++) A.part_o[pi * D + d + x] = acc[x];
+                    if (lane == 0) {
+                        A.part_m[pi] = M;
+                        A.part_l[pi] = L;
                     }
                 }
             }
-            float bias[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (DT == DRK_INT8) {
-                bias[0] = kI8Bias * s_lane(pw, 0); bias[1] = kI8Bias * s_lane(pw, 1);
-                bias[2] = kI8Bias * s_lane(pw, 2); bias[3] = kI8Bias * s_lane(pw, 3);
-            }
-            if (lane < 16) {
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    float *dst = &o_lds[w][j][c * 8];
-                    *(float4 *)dst = make_float4((o[0][j] - bias[j]) * f_own[j], (o[1][j] - bias[j]) * f_own[j],
-                                                 (o[2][j] - bias[j]) * f_own[j], (o[3][j] - bias[j]) * f_own[j]);
-                    *(float4 *)(dst + 4) = make_float4((o[4][j] - bias[j]) * f_own[j], (o[5][j] - bias[j]) * f_own[j],
-                                                       (o[6][j] - bias[j]) * f_own[j], (o[7][j] - bias[j]) * f_own[j]);
-                }
-            }
-            __syncthreads();
-            {
-                const int d = lane * 2;
-                float2 acc = make_float2(0.0f, 0.0f);
-#pragma unroll
-                for (int ww = 0; ww < 4; ww++) {
-                    const float2 v = *(const float2 *)&o_lds[ww][w][d];
-                    acc.x += v.x;
-                    acc.y += v.y;
-                }
-                const size_t pi = (size_t)(ud.bq + w) * A.Pmax + ud.piece;
-                *(float2 *)(A.part_o + pi * 128 + d) = acc;
-                if (lane == 0) {
-                    A.part_m[pi] = M_all;
-                    A.part_l[pi] = L_all;
-                }
-            }
-#pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int e = 0; e < Geo::NPV; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             m_run = -INFINITY;
             l_lane = 0.0f;
             ps_lane = 0.0f;
         }
-    };
-
-    for (int it = 0; it < nunits; it++) tile_step(it, kreg0, vreg0, ks0, vs0, gd0);
+    }
 }
 
 // grid (QH, B), block 256: fold the pieces of (branch, q head) -- the stream kernel's
@@ -626,6 +649,7 @@ __global__ __launch_bounds__(256, 4) void decode_stream_kernel(StreamArgs A)
 // piece s (+64, ...), so they arrive in one round of loads; wave w then folds the o
 // rows of pieces w, w+4, ... for two dims per lane, eight rows in flight, and the four
 // waves' sums meet in LDS.
+template <int D>
 __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_m,
                                                            const float *__restrict__ part_l, uint16_t *__restrict__ out,
                                                            const int32_t *__restrict__ seq_lens, int seq_len_host, int B,
@@ -635,8 +659,10 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
                                                            int pre_splits, const uint16_t *__restrict__ gate,
                                                            size_t gate_stride, float *__restrict__ lse_rows)
 {
-    __shared__ float2 red[4][64];
-    const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * 2;
+    constexpr int VEC = D / 64;                                  // dims per lane: 2 or 4
+    typedef float fvec __attribute__((ext_vector_type(VEC)));
+    __shared__ fvec red[4][64];
+    const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * VEC;
     int excl = 0, total = 0, nt_b = 0;
     for (int i = 0; i < B; i++) {
         const int len = seq_lens ? seq_lens[i] : seq_len_host;
@@ -663,7 +689,7 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
         if (pl > 0.0f) M = fmaxf(M, pm);
     }
     M = s_wave_max(M);
-    float2 acc = make_float2(0.0f, 0.0f);
+    fvec acc = {};
     float L = 0.0f;
     for (int c0 = 0; c0 < n_all; c0 += 64) {
         const int s = c0 + lane, cnt = min(64, n_all - c0);
@@ -674,17 +700,20 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
             if (pl > 0.0f) { w = s_exp2(pm - M); L = fmaf(pl, w, L); }
         }
         for (int j = wv; j < cnt; j += 32) {
-            float2 o[8];
+            fvec o[8];
             float wj[8];
 #pragma unroll
             for (int u = 0; u < 8; u++) {
                 const int jj = min(j + 4 * u, cnt - 1), sj = c0 + jj;
                 wj[u] = j + 4 * u < cnt ? s_lane(w, jj) : 0.0f;
-                o[u] = *(const float2 *)(sj < npieces ? part_o + (base + sj) * 128 + d : pre_o + (pbase + (sj - npieces)) * 128 + d);
+                o[u] = *(const fvec *)(sj < npieces ? part_o + (base + sj) * D + d : pre_o + (pbase + (sj - npieces)) * D + d);
             }
 #pragma unroll
             for (int u = 0; u < 8; u++)
-                if (wj[u] != 0.0f) { acc.x = fmaf(o[u].x, wj[u], acc.x); acc.y = fmaf(o[u].y, wj[u], acc.y); }   // a piece without tokens may hold anything
+                if (wj[u] != 0.0f) {                                  // a piece without tokens may hold anything
+#pragma unroll
+                    for (int x = 0; x < VEC; x++) acc[x] = fmaf(o[u][x], wj[u], acc[x]);
+                }
         }
     }
     L = s_wave_sum(L);
@@ -694,22 +723,27 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
     if (wv == 0) {
         // with a gate the row is always rewritten: the reference gates whatever the attention
         // kernel left in out, also when no token took part (paged_attention.cu:266, 368-370)
-        uint32_t *dst = (uint32_t *)(out + ((size_t)b * QH + h) * 128 + d);
-        uint32_t packed;
+        uint16_t *dst = out + ((size_t)b * QH + h) * D + d;
+        uint16_t vals[VEC];
         if (L > 0.0f) {
-            const float2 a1 = red[1][lane], a2 = red[2][lane], a3 = red[3][lane];
-            const float x = ((acc.x + a1.x) + (a2.x + a3.x)) / L, y = ((acc.y + a1.y) + (a2.y + a3.y)) / L;
-            packed = (uint32_t)f_to_elem16(x, io_dtype) | ((uint32_t)f_to_elem16(y, io_dtype) << 16);
+            const fvec a1 = red[1][lane], a2 = red[2][lane], a3 = red[3][lane];
+#pragma unroll
+            for (int x = 0; x < VEC; x++) vals[x] = f_to_elem16(((acc[x] + a1[x]) + (a2[x] + a3[x])) / L, io_dtype);
         } else {
             if (!gate) return;
-            packed = *dst;
+#pragma unroll
+            for (int x = 0; x < VEC; x++) vals[x] = dst[x];
         }
         if (gate) {
-            const uint32_t g2 = *(const uint32_t *)(gate + ((size_t)b * QH + h) * gate_stride + d);
-            packed = (uint32_t)gated_elem16((uint16_t)(packed & 0xffffu), (uint16_t)(g2 & 0xffffu), io_dtype) |
-                     ((uint32_t)gated_elem16((uint16_t)(packed >> 16), (uint16_t)(g2 >> 16), io_dtype) << 16);
+            const uint16_t *gp = gate + ((size_t)b * QH + h) * gate_stride + d;
+#pragma unroll
+            for (int x = 0; x < VEC; x++) vals[x] = gated_elem16(vals[x], gp[x], io_dtype);
         }
-        *dst = packed;
+        if constexpr (VEC == 2) {
+            *(uint32_t *)dst = (uint32_t)vals[0] | ((uint32_t)vals[1] << 16);
+        } else {
+            *(uint2 *)dst = make_uint2((uint32_t)vals[0] | ((uint32_t)vals[1] << 16), (uint32_t)vals[2] | ((uint32_t)vals[3] << 16));
+        }
     }
 }
 
@@ -729,7 +763,8 @@ __global__ __launch_bounds__(256) void block_mass_kernel(const float *__restrict
         if (!accumulate) *dst = 0.0f;
         return;
     }
-    const int g0 = lb * (bs / 16), g1 = min(g0 + bs / 16, lse_stride);
+    // only the groups of tiles that exist were written by this launch (a block may span several tiles)
+    const int g0 = lb * (bs / 16), g1 = min(min(g0 + bs / 16, lse_stride), ((len + kSTile - 1) / kSTile) * 4);
     float m = 0.0f;
     for (int h = 0; h < QH; h++) {
         const float row = lse_rows[(size_t)b * QH + h];
@@ -755,8 +790,8 @@ bool stream_decode_supported(const Lay &a, int B)
 {
     // offsets inside a layer are kept in 32 bits, in units of 16 bytes, by the unit descriptors:
     // a layer of the pool may hold up to 64 GiB
-    return a.D == 128 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && B >= 1 && B <= 64 &&
-           a.layer_stride <= (0xffff0000ull << 4);
+    return (a.D == 128 || a.D == 256) && a.KVH > 0 && a.QH % a.KVH == 0 && a.QH / a.KVH <= 16 && (a.bs % 16) == 0 &&
+           B >= 1 && B <= 64 && a.layer_stride <= (0xffff0000ull << 4);
 }
 
 static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens, int *grid, int *unit_tiles, int *Pmax)
@@ -807,17 +842,31 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
         A.scale_log2e = scale * kSLog2e;
         A.lse_groups = lse_groups; A.lse_stride = lse_stride;
+#define DRK_STREAM_LAUNCH(DT)                                                                                           \
+    do {                                                                                                                \
+        const bool g4 = a.QH / a.KVH <= 4;                                                                              \
+        if (a.D == 128 && g4) hipLaunchKernelGGL((decode_stream_kernel<DT, 128, true>), dim3(grid), dim3(256), 0, st, A);   \
+        else if (a.D == 128) hipLaunchKernelGGL((decode_stream_kernel<DT, 128, false>), dim3(grid), dim3(256), 0, st, A);   \
+        else if (g4) hipLaunchKernelGGL((decode_stream_kernel<DT, 256, true>), dim3(grid), dim3(256), 0, st, A);            \
+        else hipLaunchKernelGGL((decode_stream_kernel<DT, 256, false>), dim3(grid), dim3(256), 0, st, A);                   \
+    } while (0)
         switch (a.dtype) {
-        case DRK_F16: hipLaunchKernelGGL(decode_stream_kernel<DRK_F16>, dim3(grid), dim3(256), 0, st, A); break;
-        case DRK_BF16: hipLaunchKernelGGL(decode_stream_kernel<DRK_BF16>, dim3(grid), dim3(256), 0, st, A); break;
-        case DRK_INT8: hipLaunchKernelGGL(decode_stream_kernel<DRK_INT8>, dim3(grid), dim3(256), 0, st, A); break;
-        default: hipLaunchKernelGGL(decode_stream_kernel<DRK_FP8_E4M3>, dim3(grid), dim3(256), 0, st, A); break;
+        case DRK_F16: DRK_STREAM_LAUNCH(DRK_F16); break;
+        case DRK_BF16: DRK_STREAM_LAUNCH(DRK_BF16); break;
+        case DRK_INT8: DRK_STREAM_LAUNCH(DRK_INT8); break;
+        default: DRK_STREAM_LAUNCH(DRK_FP8_E4M3); break;
         }
+#undef DRK_STREAM_LAUNCH
         DRK_LAUNCH_CHECK("decode_stream_kernel");
     } else {
-        hipLaunchKernelGGL(stream_merge_kernel, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
-                           d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
-                           pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows);
+        if (a.D == 128)
+            hipLaunchKernelGGL(stream_merge_kernel<128>, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
+                               d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
+                               pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows);
+        else
+            hipLaunchKernelGGL(stream_merge_kernel<256>, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
+                               d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
+                               pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows);
         DRK_LAUNCH_CHECK("stream_merge_kernel");
     }
     return DRK_OK;

@@ -164,8 +164,11 @@ int drk_kv_copy_blocks(const drk_kv_layout *g, void *pool, const int32_t *d_pair
                        void *stream);
 
 /* ---- paged GQA decode attention --------------------------------------- */
-/* Bytes of workspace the split-K decode needs for B branches of at most
- * max_seq_len tokens. */
+/* Kernels: head_dim 128 or 256 with 1..16 query heads per kv head, block_size % 16 == 0 and at
+ * most 64 branches per call run on the persistent tiled kernel (every storage type; the
+ * reference's own 24 Q / 4 KV x 256, block 256 included); any other geometry (head_dim a
+ * multiple of 64 up to 512, group size <= 16) on a portable one.
+ * Bytes of workspace the split-K decode needs for B branches of at most max_seq_len tokens: */
 size_t drk_decode_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len);
 /* Same for an explicit split_tokens: B*num_q_heads*ceil(max_seq_len/split)*(head_dim+2)*4. */
 size_t drk_decode_workspace_bytes_for_split(const drk_kv_layout *g, int B, int max_seq_len,
@@ -181,8 +184,8 @@ void drk_debug_force_portable_decode(int on);
  * a choice: 0 = automatic (the persistent stream kernel), 2 = the fixed-split
  * tiled kernel (16-bit pages only), 3 = same as 0.  Process-wide. */
 void drk_debug_set_decode_kernel(int which);
-/* Diagnostic: workgroups of the persistent decode grid; 0 restores the default (512 for 16-bit pages,
- * 768 for 8-bit pages). */
+/* Diagnostic: workgroups of the persistent decode grid; 0 restores the default (512; 1024 for
+ * 8-bit pages of head_dim 128). */
 void drk_debug_set_stream_workgroups(int n);
 /* Diagnostic: context splits of the shared-prefix pass (default 64, at most 256; 0 restores the
  * default).  Changes drk_decode_shared_workspace_bytes. */
@@ -318,7 +321,8 @@ int drk_paged_prefill_attention_gated(const drk_kv_layout *g, const void *q, con
  * d_block_mass holds (sum over the layers of a step); 0 overwrites, and zeroes the entries
  * of blocks past a branch's length.  mass_stride >= ceil(max_seq_len / block_size); with
  * mass_stride = CacheManager::table_stride() the array is indexed like the block tables.
- * Geometry: head_dim 128, 4 query heads per kv head, block_size % 16 == 0, B <= 64. */
+ * Geometry: head_dim 128 or 256, at most 16 query heads per kv head, block_size % 16 == 0,
+ * B <= 64. */
 size_t drk_decode_mass_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len);
 int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const void *pool,
                                     const int32_t *d_tables, int table_stride,

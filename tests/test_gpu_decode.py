@@ -241,6 +241,28 @@ def test_other_geometries(dev, geom, dtype):
     _check(case, case.run_branches())
 
 
+@pytest.mark.parametrize("geom", [(1, 2, 32, 128, 16, 120), (1, 2, 24, 128, 16, 120), (1, 4, 12, 128, 32, 60), (1, 2, 10, 256, 16, 120),
+                                  (1, 2, 8, 256, 32, 60), (1, 1, 16, 256, 16, 120), (1, 3, 3, 256, 16, 120)])
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
+def test_stream_kernel_group_sizes_and_head_dims(dev, geom, dtype):
+    """The tiled kernel takes head_dim 128 and 256 with 1..16 query heads per kv head (here 16, 12,
+    3, 5, 4, 16, 1), every storage type: ragged branches, a hole, stale bytes past the end, against
+    the fp64 oracle; and its bits are not the portable kernel's (it really is the one that ran)."""
+    case = Case(geom, dtype, [900, 130, 64, 1, 333], seed=62, mul=0.7, holes=[(0, 3)], stale=0xFF, outliers=dtype in (cabi.INT8, cabi.FP8_E4M3))
+    got = case.run_branches()
+    _check(case, got)
+    _check(case, case.run_branches(split=128))
+    cabi.lib().drk_debug_force_portable_decode(1)
+    try:
+        other = case.run_branches()
+    finally:
+        cabi.lib().drk_debug_force_portable_decode(0)
+    _check(case, other)
+    assert not np.array_equal(got, other)
+    for b in (0, 3):
+        assert np.array_equal(case.run_single(b), got[b])               # one sequence per call: same bits
+
+
 @pytest.mark.parametrize("dtype", [cabi.INT8, cabi.FP8_E4M3])
 @pytest.mark.parametrize("io", [cabi.F16, cabi.BF16])
 @pytest.mark.parametrize("portable", [0, 1])

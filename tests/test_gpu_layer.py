@@ -222,8 +222,9 @@ def test_fused_equals_the_librarys_own_separate_kernels(dev, dtype):
     assert np.array_equal(U.host(gate_b, np.uint16, (T, QH, D)), c["gate"])
 
 
-def _decode_inputs(dtype, seed, B=5, ctx=700):
-    L, KVH, QH, D, bs = 1, 8, 32, 128, 16
+def _decode_inputs(dtype, seed, B=5, ctx=700, heads=(8, 32, 128)):
+    L, bs = 1, 16
+    KVH, QH, D = heads
     nblk = (ctx + bs - 1) // bs
     NB = B * nblk + 3
     g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
@@ -244,9 +245,10 @@ def _decode_inputs(dtype, seed, B=5, ctx=700):
 
 
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8])
-@pytest.mark.parametrize("kernel", ["stream", "portable"])
-def test_gated_decode_equals_decode_then_gate(dev, dtype, kernel):
-    g, og, io, lens, tables, opool, q, qg, (B, QH, D, ctx) = _decode_inputs(dtype, 80)
+@pytest.mark.parametrize("kernel,heads", [("stream", (8, 32, 128)), ("portable", (8, 32, 128)),
+                                          ("stream", (4, 24, 256)), ("stream", (2, 32, 128))])   # the last two: the reference's model; 16 heads per kv head
+def test_gated_decode_equals_decode_then_gate(dev, dtype, kernel, heads):
+    g, og, io, lens, tables, opool, q, qg, (B, QH, D, ctx) = _decode_inputs(dtype, 80, heads=heads)
     lib = cabi.lib()
     lib.drk_debug_force_portable_decode(1 if kernel == "portable" else 0)
     try:

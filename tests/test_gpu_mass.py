@@ -14,8 +14,9 @@ from tests import util as U
 pytestmark = pytest.mark.gpu
 
 
-def _case(dtype, bs, seed, B=4, ctx=900, holes=True):
-    L, KVH, QH, D = 2, 8, 32, 128
+def _case(dtype, bs, seed, B=4, ctx=900, holes=True, heads=(8, 32, 128)):
+    L = 2
+    KVH, QH, D = heads
     nblk = (ctx + bs - 1) // bs
     NB = B * nblk + 2
     g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
@@ -78,6 +79,16 @@ def test_block_mass_matches_fp64(dev, dtype, bs):
         assert not got[b, nblk[b]:].any()                                          # overwritten with zeros past the length
 
 
+@pytest.mark.parametrize("heads", [(4, 24, 256), (2, 32, 128)])
+def test_block_mass_other_head_shapes(dev, heads):
+    """The reference's own model (24 Q / 4 KV heads x 256, block 256) and 16 query heads per kv head."""
+    g, og, io, lens, tables, stride, opool, q, shape = _case(cabi.F16, 256, seed=9, B=3, ctx=1500, holes=False, heads=heads)
+    got = _run(g, io, lens, tables, stride, opool, q, shape)
+    want = orc.block_attention_mass(og, q, opool, tables, lens, 1, 1.0 / np.sqrt(shape[2]), io, stride)
+    assert np.all(np.abs(got - want) <= 2e-3 + 2e-3 * np.abs(want)), float(np.abs(got - want).max())
+    assert np.allclose(got.sum(axis=1)[lens > 0], shape[1], atol=2e-2)
+
+
 def test_block_mass_accumulates_over_layers(dev):
     g, og, io, lens, tables, stride, opool, q, shape = _case(cabi.BF16, 16, seed=7, holes=False)
     base = np.random.default_rng(3).random((shape[0], stride)).astype(np.float32)
@@ -93,7 +104,7 @@ def test_block_mass_argument_errors(dev):
     with pytest.raises(cabi.DrkError):       # mass rows shorter than the blocks of max_seq_len
         cabi.call("drk_paged_decode_attention_mass", C.byref(g), U.p(x), U.p(x), U.p(x), stride, U.p(x), B, ctx, U.p(x), 0,
                   0.1, io, U.p(x), 3, 0, U.p(x), 1 << 16, U.stream_ptr())
-    g2 = cabi.layout(1, 4, 24, 256, 16, 8, cabi.F16)       # a geometry the tiled kernels do not take
+    g2 = cabi.layout(1, 4, 24, 64, 16, 8, cabi.F16)        # a geometry the tiled kernels do not take (head_dim 64)
     assert cabi.lib().drk_decode_mass_workspace_bytes(C.byref(g2), 1, 100) == 0
     with pytest.raises(cabi.DrkError):
         cabi.call("drk_paged_decode_attention_mass", C.byref(g2), U.p(x), U.p(x), U.p(x), 8, U.p(x), 1, 100, U.p(x), 0,
