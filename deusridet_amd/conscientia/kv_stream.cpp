@@ -60,10 +60,9 @@ void KvStream::destroy()
 bool KvStream::begin_prefill(int M, hipStream_t stream)
 {
     if (!cm_ || M <= 0) return M == 0;
-    if (!branches_.empty()) {
-        LOG_ERROR("Conscientia", "KvStream: prefill while decode branches are open");
-        return false;
-    }
+    // Decode branches may be open (time division: perception goes on while they think).  They
+    // keep the pages they forked from; the stream's first write into a block it still shares
+    // with them makes a private copy, as a branch's would.
     if (current_pos_ + M > max_context_len_) {
         LOG_ERROR("Conscientia", "KvStream: context of %d tokens exceeds max_context_len %d", current_pos_ + M, max_context_len_);
         return false;
@@ -100,7 +99,19 @@ void KvStream::end_prefill(int M)
 int KvStream::open_branches(int n)
 {
     if (!cm_ || !branches_.empty()) return 0;
-    for (int i = 0; i < n; i++) {
+    return set_branch_count(n);
+}
+
+int KvStream::set_branch_count(int n)
+{
+    if (!cm_ || n < 0) return (int)branches_.size();
+    if (n == (int)branches_.size()) return n;
+    while ((int)branches_.size() > n) {                       // close the youngest
+        cm_->release_branch(branches_.back());
+        branches_.pop_back();
+        pos_.pop_back();
+    }
+    while ((int)branches_.size() < n) {                       // fork more, at the stream's position of now
         int id = cm_->fork_branch(0, current_pos_);
         if (id < 0) break;
         // launches address the branches' table rows as one [B, stride] array: ids must be consecutive
@@ -113,6 +124,10 @@ int KvStream::open_branches(int n)
     }
     positions_on_device_ = false;
     shared_tokens_ = branches_.empty() ? 0 : cm_->common_prefix_tokens(branches_.data(), (int)branches_.size());
+    if (graph_) {                        // a captured step is tied to the branch set it was recorded for
+        drk_graph_destroy(graph_);
+        graph_ = nullptr;
+    }
     return (int)branches_.size();
 }
 

@@ -52,6 +52,8 @@ public:
     void destroy();
 
     // ---- perception: the persistent stream, branch 0 -------------------------------------
+    // May run between the decode steps of open branches (time division): the branches keep the
+    // pages they forked from, the stream copies a block it still shares before it writes into it.
     bool begin_prefill(int M, hipStream_t stream);
     void prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipStream_t stream);
     void end_prefill(int M);
@@ -61,6 +63,10 @@ public:
     // Fork n branches from the stream at current_pos (copy-on-write: they share every block of
     // the prefix).  Returns how many were opened (fewer when the manager runs out of ids).
     int  open_branches(int n);
+    // Change the number of open branches (the scheduler's 1 / 2 / 4 by wakefulness state,
+    // scheduler.h:53-56): the youngest are closed, new ones fork at the stream's current position.
+    // Returns the number open afterwards.  A captured step is dropped.
+    int  set_branch_count(int n);
     void close_branches();
     int  num_branches() const { return (int)branches_.size(); }
     int  branch_id(int i) const { return branches_[i]; }

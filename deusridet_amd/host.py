@@ -77,6 +77,7 @@ SIGNATURES = {
     "drkh_kvs_end_prefill": (None, [_vp, _i32]),
     "drkh_kvs_current_pos": (_i32, [_vp]),
     "drkh_kvs_open_branches": (_i32, [_vp, _i32]),
+    "drkh_kvs_set_branch_count": (_i32, [_vp, _i32]),
     "drkh_kvs_close_branches": (None, [_vp]),
     "drkh_kvs_num_branches": (_i32, [_vp]),
     "drkh_kvs_branch_id": (_i32, [_vp, _i32]),
@@ -186,6 +187,7 @@ class KvStream:
     def end_prefill(self, M): lib().drkh_kvs_end_prefill(self._h, M)
     def current_pos(self): return lib().drkh_kvs_current_pos(self._h)
     def open_branches(self, n): return lib().drkh_kvs_open_branches(self._h, n)
+    def set_branch_count(self, n): return lib().drkh_kvs_set_branch_count(self._h, n)
     def shared_tokens(self): return lib().drkh_kvs_shared_tokens(self._h)
     def set_shared_prefix_policy(self, min_branches, min_tokens): lib().drkh_kvs_set_shared_prefix_policy(self._h, min_branches, min_tokens)
     def close_branches(self): lib().drkh_kvs_close_branches(self._h)

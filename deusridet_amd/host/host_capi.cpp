@@ -261,6 +261,7 @@ void drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const vo
 void drkh_kvs_end_prefill(void *ks, int M) { KS(ks)->end_prefill(M); }
 int drkh_kvs_current_pos(void *ks) { return KS(ks)->current_pos(); }
 int drkh_kvs_open_branches(void *ks, int n) { return KS(ks)->open_branches(n); }
+int drkh_kvs_set_branch_count(void *ks, int n) { return KS(ks)->set_branch_count(n); }
 void drkh_kvs_close_branches(void *ks) { KS(ks)->close_branches(); }
 int drkh_kvs_num_branches(void *ks) { return KS(ks)->num_branches(); }
 int drkh_kvs_branch_id(void *ks, int i) { return KS(ks)->branch_id(i); }

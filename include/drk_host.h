@@ -148,6 +148,7 @@ void  drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const v
 void  drkh_kvs_end_prefill(void *ks, int M);
 int   drkh_kvs_current_pos(void *ks);
 int   drkh_kvs_open_branches(void *ks, int n);
+int   drkh_kvs_set_branch_count(void *ks, int n);
 void  drkh_kvs_close_branches(void *ks);
 int   drkh_kvs_num_branches(void *ks);
 int   drkh_kvs_branch_id(void *ks, int i);

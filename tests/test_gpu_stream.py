@@ -231,3 +231,94 @@ def test_stream_session_feeds_the_scorer(dev):
         assert abs(tot - want) < 0.05 * want, (b, tot, want)
     assert sum(s.sc.score(lb) for lb in range(8)) == 0.0              # branch 0 took no decode step
     s.ks.close_branches()
+
+
+def test_time_division_perception_between_decode_steps_and_a_changing_branch_count(dev):
+    """The scheduler's regime (scheduler.h:8-24, 53-56): perception goes on while branches think, and
+    the number of branches follows the wakefulness state.  The stream writes into a block it still
+    shares with its branches (copy-on-write on the stream's side), two more branches fork later at
+    another position, the youngest are closed again.  Every step against the oracle; the pool bit
+    for bit at the end."""
+    s = Session(4)
+    rng = np.random.default_rng(123)
+    qw, kw = U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT)
+    s.set_weights(qw, kw)
+    st = U.stream_ptr()
+    og = orc.layout(L, KVH, QH, D, BS, s.NB, DT)
+    opool = orc.new_pool(og)
+    tables = {0: s.cm.h_block_table(0).copy()}
+
+    def follow_tables(ids):
+        """copy-on-write in the oracle: a table cell that moved to another block took the old block's bytes along"""
+        for b in ids:
+            new = s.cm.h_block_table(b).copy()
+            old = tables.get(b)
+            if old is not None:
+                for lb in np.nonzero((old >= 0) & (new >= 0) & (old != new))[0]:
+                    orc.copy_block(og, opool, int(old[lb]), int(new[lb]))
+            tables[b] = new
+
+    def perceive(M):
+        pos0 = s.ks.current_pos()
+        assert s.ks.begin_prefill(M, st)
+        follow_tables([0])
+        for layer in range(L):
+            qg, k, v = (U.normal_bits(rng, sh, DT, m) for sh, m in (((M, QH, 2 * D), 1.0), ((M, KVH, D), 0.7), ((M, KVH, D), 0.5)))
+            s.load(qg, k, v)
+            s.ks.prefill_layer(layer, s.io(), M, st)
+            got = s.out(M)
+            pos = (pos0 + np.arange(M)).astype(np.int32)
+            want = oracle_layer(og, opool, [tables[0]] * M, pos, layer, qg, k, v, qw, kw, s.tab)
+            ok, mx, _ = U.rel_abs_ok(U.from_bits(got, DT), want)
+            assert ok, ("prefill", M, layer, mx)
+        s.ks.end_prefill(M)
+
+    def think():
+        n = s.ks.num_branches()
+        ids = [s.ks.branch_id(i) for i in range(n)]
+        pos = np.array([s.ks.branch_pos(i) for i in range(n)], np.int32)
+        assert s.ks.begin_decode_step(st)
+        follow_tables(ids)
+        for layer in range(L):
+            qg, k, v = (U.normal_bits(rng, sh, DT, m) for sh, m in (((n, QH, 2 * D), 1.0), ((n, KVH, D), 0.7), ((n, KVH, D), 0.5)))
+            s.load(qg, k, v)
+            s.ks.decode_layer(layer, s.io(), st)
+            got = s.out(n)
+            want = oracle_layer(og, opool, [tables[b] for b in ids], pos, layer, qg, k, v, qw, kw, s.tab)
+            ok, mx, _ = U.rel_abs_ok(U.from_bits(got, DT), want)
+            assert ok, ("decode", n, layer, mx)
+        s.ks.end_decode_step(st)
+        assert [s.ks.branch_pos(i) for i in range(n)] == (pos + 1).tolist()
+
+    def fork_tables():
+        for i in range(s.ks.num_branches()):
+            b = s.ks.branch_id(i)
+            if b not in tables:
+                tables[b] = s.cm.h_block_table(b).copy()
+
+    perceive(64)
+    perceive(36)
+    assert s.ks.set_branch_count(2) == 2                      # DAYDREAM: two branches at 100
+    fork_tables()
+    shared_tail = int(tables[0][6])
+    perceive(12)                                              # ACTIVE again: the stream writes tokens 100..111 into block 6,
+    assert int(tables[0][6]) != shared_tail                   # which its branches still share: the stream takes a copy
+    assert [int(tables[b][6]) for b in (1, 2)] == [shared_tail] * 2
+    think(); think()
+    perceive(16)
+    assert s.ks.current_pos() == 128
+    think()
+    assert s.ks.set_branch_count(4) == 4                      # DREAMING: two more, forked at 128
+    fork_tables()
+    assert [s.ks.branch_pos(i) for i in range(4)] == [103, 103, 128, 128]
+    assert s.ks.shared_tokens() == 96
+    think(); think()
+    assert s.ks.set_branch_count(1) == 1 and s.ks.branch_id(0) == 1
+    for b in (2, 3, 4):
+        tables.pop(b)
+    think()
+    perceive(16)
+    think()
+    assert np.array_equal(s.pool(), opool)
+    s.ks.close_branches()
+    assert s.cm.gpu_blocks_used() == 9                        # 144 tokens of the stream
