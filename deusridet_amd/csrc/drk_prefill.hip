@@ -501,14 +501,16 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
     const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0;
     if (mfma) return 0;
+    if (!g_force_portable && stream_decode_supported(a, 1)) return prefill_stream_workspace_need(a, pos_start, M);
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
 // paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630.
 // head_dim 128, 16-bit K/V, 4 query heads per KV head: the MFMA kernel above (no
-// workspace).  Any other geometry or storage type: row t of the chunk runs as one
-// causal "branch" of the decode kernels -- the reference's algorithm verbatim
-// (paged_attention.cu:481, 506-549) -- and needs the workspace.
+// workspace).  8-bit pages, head_dim 256 or another group size (<= 16): blocks of query
+// tokens through the tiled decode kernel in its causal mode (drk_decode_stream.hip).  Anything
+// else: row t of the chunk runs as one causal "branch" of the portable decode kernel -- the
+// reference's algorithm verbatim (paged_attention.cu:481, 506-549).  Both need the workspace.
 static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
                         void *out, int layer, int pos_start, int M, float scale, int io_dtype, void *workspace,
                         size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
@@ -525,6 +527,11 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
 
     const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && scale > 0.0f;
+    if (!mfma && !g_force_portable && scale > 0.0f && stream_decode_supported(a, 1)) {
+        if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "prefill: workspace must be 16-byte aligned");
+        return launch_prefill_stream(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
+                                     workspace_bytes, (hipStream_t)stream, gate, gate_stride);
+    }
     if (!mfma)
         return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
                              io_dtype, 0, workspace, workspace_bytes, stream, gate, gate_stride);

@@ -134,3 +134,65 @@ def test_mfma_and_rowwise_paths_agree(dev):
         cabi.lib().drk_debug_force_portable_decode(0)
     ok, ma, _ = U.rel_abs_ok(a, b)
     assert ok, ma
+
+
+def build_io(geom, dtype, io, total, seed, holes=(), mul=1.0):
+    """like build(), for a pool whose storage type differs from the type K/V arrive in"""
+    L, KVH, QH, D, bs, NB = geom
+    g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
+    rng = np.random.default_rng(seed)
+    nblk = (total + bs - 1) // bs
+    table = U.shuffled_table(rng, NB, nblk, nblk + 2)
+    opool = orc.new_pool(og)
+    opool[:] = 0xFF                                               # stale bytes everywhere first
+    k = U.normal_bits(rng, (total, KVH, D), io, mul)
+    v = U.normal_bits(rng, (total, KVH, D), io, mul)
+    orc.append_batch(og, opool, table, L - 1, 0, k, v, io)
+    for h in holes:
+        table[h] = -1
+    return g, og, rng, table, opool
+
+
+@pytest.mark.parametrize("geom,dtype", [((1, 8, 32, 128, 16, 100), cabi.INT8), ((1, 8, 32, 128, 16, 100), cabi.FP8_E4M3),
+                                        ((2, 4, 24, 256, 256, 8), cabi.F16), ((1, 2, 32, 128, 16, 100), cabi.BF16),
+                                        ((1, 4, 4, 128, 16, 100), cabi.BF16), ((1, 2, 6, 256, 16, 100), cabi.INT8),
+                                        ((1, 2, 10, 128, 32, 60), cabi.F16)])
+@pytest.mark.parametrize("pos_start,M", [(0, 1), (0, 70), (37, 45), (509, 77), (1000, 300)])
+def test_prefill_other_shapes_through_the_tiled_decode_kernel(dev, geom, dtype, pos_start, M):
+    """8-bit pages, head_dim 256, group sizes 4, 6, 16, 1, 3, 5: blocks of query tokens fill the padded
+    columns of the tiled decode kernel (4, 2, 1, 16, 5, 3 tokens per block; M is not a multiple of the
+    block, so the first block is partial), a hole in the table, stale bytes behind the end.  Against
+    the fp64 oracle, and the gated form against plain + gate."""
+    io = dtype if dtype in (cabi.F16, cabi.BF16) else cabi.BF16
+    L, KVH, QH, D, bs, NB = geom
+    holes = (1,) if pos_start + M > 3 * bs else ()
+    g, og, rng, table, opool = build_io(geom, dtype, io, pos_start + M, seed=pos_start * 5 + M + D, holes=holes, mul=0.7)
+    q = U.normal_bits(rng, (M, QH, D), io, 0.7)
+    qg = U.normal_bits(rng, (M, QH, 2 * D), io, 2.0)
+    scale = 1 / np.sqrt(D)
+    dq, dpool, dtab, dqg = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table), U.dev_bytes(qg)
+    raw = run_prefill(g, dq, dpool, dtab, L - 1, pos_start, M, scale, io, QH, D)
+    want = orc.prefill_f64(og, q, opool, table, L - 1, pos_start, scale, io)
+    ok, ma, _ = U.rel_abs_ok(U.from_bits(raw, io), want)
+    assert ok, ma
+    lib = cabi.lib()
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    assert wsb < 64 << 20
+    ws = U.dev_zeros(max(wsb, 16))
+    out = U.dev_zeros(M * QH * D * 2)
+    gptr = C.c_void_p(dqg.data_ptr() + D * 2)
+    cabi.call("drk_paged_prefill_attention_gated", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), L - 1, pos_start, M,
+              float(scale), io, gptr, 2 * D, U.p(ws), wsb, U.stream_ptr())
+    U.sync()
+    gated = orc.sigmoid_gate(raw, np.ascontiguousarray(qg[:, :, D:]), io)
+    assert U.ulp_distance(U.host(out, np.uint16, (M, QH, D)), gated).max() <= 1
+    # and it is not the row-wise path that produced the bits
+    lib.drk_debug_force_portable_decode(1)
+    try:
+        other = run_prefill(g, dq, dpool, dtab, L - 1, pos_start, M, scale, io, QH, D)
+    finally:
+        lib.drk_debug_force_portable_decode(0)
+    ok, ma, _ = U.rel_abs_ok(U.from_bits(other, io), want)
+    assert ok, ma
+    if M > 1:
+        assert not np.array_equal(other, raw)
