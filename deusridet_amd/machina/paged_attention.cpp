@@ -45,7 +45,9 @@ bool paged_attention_reserve_workspace(int max_branches, int max_seq_len, int ma
     s = drk_decode_mass_workspace_bytes(&g, B, max_seq_len);
     if (s > need) need = s;
     if (max_prefill_rows > 0) {
-        size_t p = drk_decode_workspace_bytes(&g, max_prefill_rows, max_seq_len);
+        // the last chunk of the longest context needs the most (0 for the MFMA prefill kernel)
+        const int rows = max_prefill_rows < max_seq_len ? max_prefill_rows : max_seq_len;
+        size_t p = drk_prefill_workspace_bytes(&g, max_seq_len - rows, rows);
         if (p > need) need = p;
     }
     return need == 0 || workspace(need) != nullptr;

@@ -20,6 +20,18 @@ L, QH, KVH, D, BS, RD = 2, 32, 8, 128, 16, 32
 EPS, THETA = 1e-6, 1.0e7
 DT = cabi.BF16
 NPOS = 512
+POOL_BLOCKS = 48
+
+
+@pytest.fixture
+def reference_model_shape():
+    """24 Q / 4 KV heads x 256, 256-token blocks, 64 rotary dims, fp16: the reference's own model
+    (model.h:39-42, block_pool.h:34-38) instead of the 8B-class shape of the other tests."""
+    global QH, KVH, D, BS, RD, DT, POOL_BLOCKS
+    saved = (QH, KVH, D, BS, RD, DT, POOL_BLOCKS)
+    QH, KVH, D, BS, RD, DT, POOL_BLOCKS = 24, 4, 256, 256, 64, cabi.F16, 10
+    yield
+    QH, KVH, D, BS, RD, DT, POOL_BLOCKS = saved
 
 
 def d2h(ptr, nbytes):
@@ -37,7 +49,7 @@ class Session:
         assert host.lib().drkh_set_rope(RD, THETA, EPS)
         self.cm = host.CacheManager()
         self.sc = host.ImportanceScorer() if scorer else None
-        assert self.cm.init(48 * L * 2 * KVH * BS * D * 2, BS, self.sc, 1 + nbranch)
+        assert self.cm.init(POOL_BLOCKS * L * 2 * KVH * BS * D * 2, BS, self.sc, 1 + nbranch)
         if scorer:
             assert self.sc.init((1 + nbranch) * self.cm.table_stride(), 0.5)
         self.tab = orc.rope_table(NPOS, RD, THETA)
@@ -118,7 +130,7 @@ def run_session(nbranch, steps, mode, seed=120, scorer=False, shared_policy=None
     assert np.array_equal(s.pool(), opool)
     # ---- decode branches ----
     assert s.ks.open_branches(nbranch) == nbranch
-    assert s.ks.shared_tokens() == 96                                  # six whole blocks of the 100-token prefix
+    assert s.ks.shared_tokens() == 100 // BS * BS                      # the whole blocks of the 100-token prefix
     ids = [s.ks.branch_id(i) for i in range(nbranch)]
     assert ids == list(range(1, nbranch + 1)) and all(s.ks.branch_pos(i) == 100 for i in range(nbranch))
     step_inputs = [[tuple(U.normal_bits(rng, sh, DT, m) for sh, m in (((nbranch, QH, 2 * D), 1.0), ((nbranch, KVH, D), 0.7),
@@ -150,8 +162,9 @@ def run_session(nbranch, steps, mode, seed=120, scorer=False, shared_policy=None
                 got = s.out(nbranch)
                 pos = np.full(nbranch, 100 + step, np.int32)
                 if step == 0 and layer == 0:                         # first write into the shared tail block: copy-on-write
+                    tail = 100 // BS
                     for b in range(nbranch):
-                        for src_blk, dst_blk in [(s.cm.h_block_table(0)[6], tables[b][6])]:
+                        for src_blk, dst_blk in [(s.cm.h_block_table(0)[tail], tables[b][tail])]:
                             assert src_blk != dst_blk
                             orc.copy_block(og, opool, int(src_blk), int(dst_blk))
                 want = oracle_layer(og, opool, tables, pos, layer, qg, k, v, qw, kw, s.tab)
@@ -189,6 +202,22 @@ def test_stream_session_matches_the_oracle_and_its_graph_replay(dev):
     del s_e
     rec_g, pool_g, s_g = run_session(3, 5, "graph")
     for step in range(5):
+        for layer in range(L):
+            assert np.array_equal(rec_g["decode"][step][layer], rec_e["decode"][step][layer]), (step, layer)
+    assert np.array_equal(pool_g, pool_e)
+    s_g.ks.close_branches()
+
+
+def test_stream_session_at_the_reference_models_shape(dev, reference_model_shape):
+    """The whole KV path at 24 Q / 4 KV heads x 256 with 256-token blocks: fused norm + RoPE + page write
+    at head_dim 256, prefill through the tiled kernel's causal mode (2 tokens x 6 heads per block), decode
+    with 6 heads per kv head, copy-on-write of a 256-token block, and the captured step."""
+    rec_e, pool_e, s_e = run_session(2, 3, "eager", seed=124)
+    s_e.ks.close_branches()
+    assert s_e.cm.gpu_blocks_used() == 1
+    del s_e
+    rec_g, pool_g, s_g = run_session(2, 3, "graph", seed=124)
+    for step in range(3):
         for layer in range(L):
             assert np.array_equal(rec_g["decode"][step][layer], rec_e["decode"][step][layer]), (step, layer)
     assert np.array_equal(pool_g, pool_e)
