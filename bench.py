@@ -49,7 +49,8 @@ def parse():
                     help="BASELINE config: 2 (default, the headline) | 3 shared prefix + COW + eviction | "
                          "4 int8/fp8 pages at 128k | 5 chunked MFMA prefill interleaved with decode | "
                          "6 config 3's shape through the stream driver (whole layer path, captured step)")
-    ap.add_argument("--kv-dtype", choices=["int8", "fp8"], default="int8", help="config 4 storage type")
+    ap.add_argument("--kv-dtype", choices=["bf16", "int8", "fp8"], default=None,
+                    help="storage type of the pages: config 4 int8 (default) | fp8; config 5 bf16 (default) | int8 | fp8")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "
                                                             "replaying one captured HIP graph per step")
     ap.add_argument("--no-cascade", action="store_true", help="config 3: read the shared prefix once per branch")

@@ -40,7 +40,8 @@ def config4(args):
     """4 branches x 128k tokens, 8 KV heads x 128, int8 (+fp16 scale per token and
     head) or fp8-e4m3 pages quantised on append, dequantised inside attention."""
     torch, cabi, U, lib, stream, sp = _common(args)
-    dt = cabi.INT8 if args.kv_dtype == "int8" else cabi.FP8_E4M3
+    kv_name = args.kv_dtype if args.kv_dtype in ("int8", "fp8") else "int8"
+    dt = cabi.INT8 if kv_name == "int8" else cabi.FP8_E4M3
     L, KVH, QH, D, bs, B, ctx = args.layers, 8, 32, 128, 16, 4, 131072
     W, K = args.warmup, args.steps
     probe = cabi.layout(L, KVH, QH, D, bs, 1, dt)
@@ -118,14 +119,14 @@ def config4(args):
         "metric": "paged_decode_attention_GBps", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K,
         "warmup": W, "ms_per_step": round(total_ms / K, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8" if dt == cabi.INT8 else "fp8", "data": "synthetic",
-        "config": {"workload": f"config 4: {L} layers, 32 Q / 8 KV heads x 128, {args.kv_dtype} pages "
+        "config": {"workload": f"config 4: {L} layers, 32 Q / 8 KV heads x 128, {kv_name} pages "
                                f"({code_bytes} B per token and layer), 4 branches x 131072 tokens, K/V N(0,1) with 1 % x20 "
                                f"outliers quantised on append; step = per layer: append 1 token/branch + decode attention",
                    "branches": B, "layers": L, "ctx_final": [ctx] * B},
         "tokens_per_s": round(B * K / (total_ms * 1e-3), 1), "us_per_step": round(total_ms / K * 1e3, 1),
         "quantising_append_GBps": round(append_gbps, 1),
         "quantising_append_hbm_frac": round(append_gbps / HBM_PEAK_GBPS, 4),
-        "roofline": {"kernel": f"decode_stream_kernel<{args.kv_dtype}>", "bound": "hbm", "achieved": round(ach, 1),
+        "roofline": {"kernel": f"decode_stream_kernel<{kv_name}>", "bound": "hbm", "achieved": round(ach, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
                      "avg_launch_us": round(ker_ms * 1e3, 2), "bytes_per_launch": launch_bytes},
         "cpu_baseline": None,
@@ -285,7 +286,8 @@ def config5(args):
     L, KVH, QH, D, bs = min(args.layers, 4), 8, 32, 128, 16
     chunk, total, DB, dctx = 2048, 32768, 4, 8192
     NB = (total + DB * (dctx + 64)) // bs + 64
-    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    kv_name = args.kv_dtype or "bf16"
+    g = cabi.layout(L, KVH, QH, D, bs, NB, {"bf16": cabi.BF16, "int8": cabi.INT8, "fp8": cabi.FP8_E4M3}[kv_name])
     rng = np.random.default_rng(5)
     perm = rng.permutation(NB).astype(np.int32)
     nb_seq, nb_dec = total // bs, dctx // bs + 4
@@ -346,14 +348,15 @@ def config5(args):
     return {
         "metric": "chunked_prefill_attention_TFLOPs", "value": round(tfl, 1), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": nchunks, "warmup": total // chunk, "ms_per_step": round(pf_ms / nchunks / L, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if kv_name == "bf16" else "f16",
+        "data": "synthetic",
         "config": {"workload": f"config 5: one sequence prefilled to 32768 in 2048-token chunks, 32 Q / 8 KV heads x 128 "
-                               f"bf16, 16-token pages, {L} layers; per chunk: append, causal attention over all pages so far "
+                               f"bf16 in, {kv_name} 16-token pages, {L} layers; per chunk: append, causal attention over all pages so far "
                                f"(MFMA), then one decode step of 4 branches at 8192 on the same pool; a step here is one "
                                f"(chunk, layer) attention launch", "layers": L},
         "chunk_append_GBps": round(ap_gbps, 1),
         "interleaved_decode_us_per_layer": round(float(np.mean(dec_ms)) / L * 1e3, 1),
-        "roofline": {"kernel": "prefill_mfma_kernel<bf16>", "bound": "mfma", "achieved": round(tfl, 1),
+        "roofline": {"kernel": f"prefill_mfma_kernel<{kv_name}>", "bound": "mfma", "achieved": round(tfl, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": None},
         "cpu_baseline": None,

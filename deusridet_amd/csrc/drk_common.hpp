@@ -151,6 +151,47 @@ __device__ __forceinline__ uint16_t gated_elem16(uint16_t x16, uint16_t g16, int
     return f_to_elem16(sigmoid_gate_value(elem16_to_f(x16, dtype), elem16_to_f(g16, dtype)), dtype);
 }
 
+// ---- 8-bit page codes -> fp16, shared by the decode and prefill kernels ----
+__device__ __forceinline__ uint32_t s_perm(uint32_t hi, uint32_t lo, uint32_t sel)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_perm(hi, lo, sel);      // result byte i = byte sel[i] of {lo: 0-3, hi: 4-7}
+#else
+    (void)hi; (void)sel;
+    return lo;
+#endif
+}
+
+// int8 codes travel as fp16 1152 + code: byte (code ^ 0x80) under the exponent byte 0x64
+// is exactly that number, so a code costs one byte permute and the constant is taken
+// out once per dot product (1152 * sum of the other operand) instead of once per value.
+constexpr float kI8Bias = 1152.0f;
+constexpr uint32_t kF16Ones = 0x3C003C00u;
+
+// four int8 codes -> two dwords of packed fp16 (1152 + code)
+__device__ __forceinline__ void int8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+{
+    const uint32_t x = w ^ 0x80808080u;
+    lo = s_perm(0x64646464u, x, 0x04010400u);   // bytes x0,64,x1,64
+    hi = s_perm(0x64646464u, x, 0x04030402u);   // bytes x2,64,x3,64
+}
+
+// two fp8-e4m3 codes (the low or the high half of w) -> packed fp16 (exact: e4m3 fits in fp16)
+template <bool HIGH>
+__device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t w)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, HIGH));
+#else
+    return w;
+#endif
+}
+__device__ __forceinline__ void fp8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)
+{
+    lo = fp8x2_to_f16x2<false>(w);
+    hi = fp8x2_to_f16x2<true>(w);
+}
+
 // unsigned divide with a power-of-two fast path chosen on the host
 __device__ __forceinline__ unsigned udiv(unsigned x, unsigned d, int shift)
 {

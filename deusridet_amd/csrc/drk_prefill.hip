@@ -118,7 +118,7 @@ struct PrefillArgs {
     const uint8_t *q;
     uint8_t *out;
     int pos_start, M, QH, KVH, NB, bs, bs_shift;
-    unsigned head_stride, kv_plane, block_stride;
+    unsigned head_stride, kv_plane, block_stride, scale_plane;
     float scale_log2e;
     // shared-prefix mode: row "token" = branch; every row sees tokens [0, min(len, shared))
     const int32_t *seq_lens;      // [M] on the device
@@ -148,7 +148,8 @@ struct PfGroup {
     uint4 r0, r1, r2, r3;
 };
 
-template <bool ONCE>
+// one wave's 16-token group of a tile: 16 rows of 256 bytes (16-bit pages) or 128 bytes (8-bit)
+template <bool ONCE, bool Q8>
 __device__ __forceinline__ PfGroup pf_load_group(const uint8_t *__restrict__ base, bool valid, size_t off, int lane)
 {
     PfGroup g;
@@ -158,13 +159,17 @@ __device__ __forceinline__ PfGroup pf_load_group(const uint8_t *__restrict__ bas
         if constexpr (ONCE) {       // every page is read by one workgroup only: stream it
             g.r0 = ld_stream128(p);
             g.r1 = ld_stream128(p + 1024);
-            g.r2 = ld_stream128(p + 2048);
-            g.r3 = ld_stream128(p + 3072);
+            if constexpr (!Q8) {
+                g.r2 = ld_stream128(p + 2048);
+                g.r3 = ld_stream128(p + 3072);
+            }
         } else {                    // 64 row tiles of a chunk share each page through the L2
             g.r0 = *(const uint4 *)(p);
             g.r1 = *(const uint4 *)(p + 1024);
-            g.r2 = *(const uint4 *)(p + 2048);
-            g.r3 = *(const uint4 *)(p + 3072);
+            if constexpr (!Q8) {
+                g.r2 = *(const uint4 *)(p + 2048);
+                g.r3 = *(const uint4 *)(p + 3072);
+            }
         }
     }
     return g;
@@ -180,14 +185,60 @@ __device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, i
     *(uint4 *)(dst + 12 * PITCH) = g.r3;
 }
 
+// 8-bit pages: a lane holds 16 codes of row (lane / 8) + 8 j, dims (lane % 8) * 16 ..; they are
+// stored as the fp16 values code * scale (int8; sc = the two rows' fp16 scales, low / high half)
+// or as the fp8 values themselves.  Rows at or past `lim` may hold anything -- codes and scales --
+// and are stored as zeros.
+template <int PITCH, int KV>
+__device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup &g, int w, int lane, uint32_t sc, int lim)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const uint4 regs[2] = {g.r0, g.r1};
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int row = (lane >> 3) + 8 * j;
+        uint32_t h[8];
+        if constexpr (KV == DRK_INT8) {
+            int8x4_to_f16x4(regs[j].x, h[0], h[1]);
+            int8x4_to_f16x4(regs[j].y, h[2], h[3]);
+            int8x4_to_f16x4(regs[j].z, h[4], h[5]);
+            int8x4_to_f16x4(regs[j].w, h[6], h[7]);
+            const uint32_t s16 = j ? (sc >> 16) : (sc & 0xffffu);
+            const h2 scale = __builtin_bit_cast(h2, s16 | (s16 << 16));
+            const h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+#pragma unroll
+            for (int i = 0; i < 8; i++) {                     // (1152 + code) - 1152 is exact; one rounding in the product
+                const h2 v = (__builtin_bit_cast(h2, h[i]) - bias) * scale;
+                h[i] = __builtin_bit_cast(uint32_t, v);
+            }
+        } else {
+            fp8x4_to_f16x4(regs[j].x, h[0], h[1]);
+            fp8x4_to_f16x4(regs[j].y, h[2], h[3]);
+            fp8x4_to_f16x4(regs[j].z, h[4], h[5]);
+            fp8x4_to_f16x4(regs[j].w, h[6], h[7]);
+        }
+        if (row >= lim) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) h[i] = 0u;
+        }
+        uint8_t *dst = lds + (w * 16 + row) * PITCH + (lane & 7) * 32;
+        *(uint4 *)(dst) = make_uint4(h[0], h[1], h[2], h[3]);
+        *(uint4 *)(dst + 16) = make_uint4(h[4], h[5], h[6], h[7]);
+    }
+}
+
 // grid = (ceil(M/32) * KVH, 1[, splits]); block = 256.
 // SHARED = false: causal prefill of a chunk, normalised output.
 // SHARED = true:  the M rows are decode branches that share the pages of tokens
 //                 [0, shared); workgroup z handles tokens [z, z+1) * chunk_tiles * 64 of
 //                 them, no causal mask, and leaves (o, m, l) per (branch, q head, z).
-template <int DT, bool SHARED>
+// DT: the type the matrix cores multiply in; KV: the pages' storage type (DT, or int8 / fp8 with
+// DT = fp16: the codes are dequantised on their way into LDS); IO: the type of q and out.
+template <int DT, bool SHARED, int KV = DT, int IO = DT>
 __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
 {
+    constexpr bool Q8 = KV == DRK_INT8 || KV == DRK_FP8_E4M3;
+    constexpr int RB = Q8 ? 128 : 256;                      // bytes of one token row of one kv head
     // Two buffers per operand.  The loop is software-pipelined by one tile: while the softmax of
     // tile i runs on the vector ALU, the matrix cores already compute the scores of tile i+1, so
     // K is staged one tile further ahead than V.  One barrier per tile.
@@ -224,19 +275,34 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
     {
         const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * 256 + g * 16;
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) qf[ks] = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+        for (int ks = 0; ks < 8; ks++) {
+            uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+#if defined(__HIP_DEVICE_COMPILE__)
+            if constexpr (IO == DRK_BF16 && DT == DRK_F16) {      // 8-bit pages multiply in fp16
+                v.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.x), bf16_hi(v.x)));
+                v.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.y), bf16_hi(v.y)));
+                v.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.z), bf16_hi(v.z)));
+                v.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.w), bf16_hi(v.w)));
+            }
+#endif
+            qf[ks] = v;
+        }
     }
 
     const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
-    auto lookup = [&](int tile, bool &valid) -> size_t {
+    // byte offset of the wave's 16-token row run of `tile` (soff: of its 16 fp16 K scales, int8 pages)
+    auto lookup = [&](int tile, bool &valid, size_t &soff) -> size_t {
         int tg = tile * kPfBN + w * 16;
         valid = false;
+        soff = 0;
         if (tg >= lim_wg) return 0;
         int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
         int blk = A.table[lb];
         if (blk < 0 || blk >= A.NB) return 0;
         valid = true;
-        return (size_t)blk * A.block_stride + (size_t)(tg - lb * A.bs) * 256;
+        const size_t base = (size_t)blk * A.block_stride;
+        soff = base + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + (tg - lb * A.bs)) * 2;
+        return base + (size_t)(tg - lb * A.bs) * RB;
     };
 
     pf_f32x16 o[4];
@@ -249,6 +315,7 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
     // registers -> LDS; rows at or past the workgroup's limit may hold anything and are cleared
     bool kreg_valid = false;
     PfGroup kreg, vreg;
+    uint32_t ksc = 0u, vsc = 0u;               // int8 pages: the fp16 scales of this lane's two rows
     auto clear_tail = [&](PfGroup &r, int tile) {
         const int tile_t0 = tile * kPfBN;
         if (tile_t0 + kPfBN > lim_wg) {
@@ -260,23 +327,40 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
             if (12 >= lim) r.r3 = z;
         }
     };
+    auto load_scales = [&](bool valid, size_t soff) -> uint32_t {
+        if (KV != DRK_INT8 || !valid) return 0u;               // no page: zero codes times zero
+        const uint8_t *p = A.pool_layer + soff + (lane >> 3) * 2;
+        return (uint32_t)*(const uint16_t *)p | ((uint32_t)*(const uint16_t *)(p + 16) << 16);
+    };
     auto fetch_k = [&](int tile) {
-        const size_t off = lookup(tile, kreg_valid);
-        kreg = pf_load_group<SHARED>(kbase, kreg_valid, off, lane);
+        size_t soff;
+        const size_t off = lookup(tile, kreg_valid, soff);
+        kreg = pf_load_group<SHARED, Q8>(kbase, kreg_valid, off, lane);
+        ksc = load_scales(kreg_valid, soff);
     };
     auto fetch_v = [&](int tile) {
         bool ok;
-        const size_t off = lookup(tile, ok);
-        vreg = pf_load_group<SHARED>(kbase + A.kv_plane, ok, off, lane);
+        size_t soff;
+        const size_t off = lookup(tile, ok, soff);
+        vreg = pf_load_group<SHARED, Q8>(kbase + A.kv_plane, ok, off, lane);
+        vsc = load_scales(ok, soff + A.scale_plane);
     };
     auto stage_k = [&](int tile) {
-        clear_tail(kreg, tile);
-        pf_store_group<kPfPitch>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane);
+        if constexpr (Q8) {
+            pf_store_group_q8<kPfPitch, KV>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane, ksc, lim_wg - tile * kPfBN - w * 16);
+        } else {
+            clear_tail(kreg, tile);
+            pf_store_group<kPfPitch>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane);
+        }
         if (lane == 0) valid_lds4[tile & 3][w] = kreg_valid ? 1 : 0;
     };
     auto stage_v = [&](int tile) {
-        clear_tail(vreg, tile);
-        pf_store_group<kPfPitchV>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane);
+        if constexpr (Q8) {
+            pf_store_group_q8<kPfPitchV, KV>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane, vsc, lim_wg - tile * kPfBN - w * 16);
+        } else {
+            clear_tail(vreg, tile);
+            pf_store_group<kPfPitchV>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane);
+        }
     };
     // S^T = K Q^T : two 32-token tiles x 32 rows, 8 k-steps of 16 dims
     auto qk = [&](int tile, pf_f32x16 (&s)[2]) {
@@ -428,14 +512,13 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         const float inv = have ? 1.0f / l_tot : 0.0f;
         uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * 256;
         const uint16_t *grow = A.gate ? A.gate + ((size_t)tq * A.QH + head) * A.gate_stride : nullptr;
-        constexpr int IO = DT;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int b4 = 0; b4 < 4; b4++) {
                 const int d0 = dt * 32 + 8 * b4 + 4 * g;
-                uint2 v = have ? make_uint2(pack2<DT>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
-                                            pack2<DT>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv))
+                uint2 v = have ? make_uint2(pack2<IO>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
+                                            pack2<IO>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv))
                                : *(const uint2 *)(orow + d0 * 2);
                 if (grow) {
                     const uint2 gv = *(const uint2 *)(grow + d0);
@@ -476,7 +559,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.out = nullptr;
     A.pos_start = 0; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs;
     A.bs_shift = ilog2_exact((unsigned)a.bs);
-    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
+    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
     A.scale_log2e = scale * kLog2eP;
     A.seq_lens = d_seq_lens; A.shared = shared;
     shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
@@ -499,15 +582,15 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 {
     Lay a;
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
-    const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0;
+    const bool mfma = !g_force_portable && a.D == 128 && a.QH / a.KVH == 4 && (a.bs % 16) == 0;
     if (mfma) return 0;
     if (!g_force_portable && stream_decode_supported(a, 1)) return prefill_stream_workspace_need(a, pos_start, M);
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
 // paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630.
-// head_dim 128, 16-bit K/V, 4 query heads per KV head: the MFMA kernel above (no
-// workspace).  8-bit pages, head_dim 256 or another group size (<= 16): blocks of query
+// head_dim 128, 4 query heads per KV head: the MFMA kernel above (no workspace; 8-bit
+// pages are dequantised on their way into LDS).  head_dim 256 or another group size (<= 16): blocks of query
 // tokens through the tiled decode kernel in its causal mode (drk_decode_stream.hip).  Anything
 // else: row t of the chunk runs as one causal "branch" of the portable decode kernel -- the
 // reference's algorithm verbatim (paged_attention.cu:481, 506-549).  Both need the workspace.
@@ -526,7 +609,7 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         return fail(DRK_ERR_INVALID, "prefill: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
 
-    const bool mfma = !g_force_portable && a.D == 128 && a.E == 2 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && scale > 0.0f;
+    const bool mfma = !g_force_portable && a.D == 128 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && scale > 0.0f;
     if (!mfma && !g_force_portable && scale > 0.0f && stream_decode_supported(a, 1)) {
         if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "prefill: workspace must be 16-byte aligned");
         return launch_prefill_stream(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
@@ -545,13 +628,22 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     A.out = (uint8_t *)out;
     A.pos_start = pos_start; A.M = M; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs;
     A.bs_shift = ilog2_exact((unsigned)a.bs);
-    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
+    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
     A.scale_log2e = scale * kLog2eP;
     dim3 grid(((M + 31) / 32) * a.KVH);
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = (const uint16_t *)gate; A.gate_stride = gate_stride;
-    if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
-    else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false>), grid, dim3(256), 0, (hipStream_t)stream, A);
+    hipStream_t st = (hipStream_t)stream;
+    if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, st, A);
+    else if (a.dtype == DRK_F16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false>), grid, dim3(256), 0, st, A);
+    else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16)
+        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_INT8, DRK_BF16>), grid, dim3(256), 0, st, A);
+    else if (a.dtype == DRK_INT8)
+        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_INT8, DRK_F16>), grid, dim3(256), 0, st, A);
+    else if (io_dtype == DRK_BF16)
+        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_FP8_E4M3, DRK_BF16>), grid, dim3(256), 0, st, A);
+    else
+        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_FP8_E4M3, DRK_F16>), grid, dim3(256), 0, st, A);
     DRK_LAUNCH_CHECK("prefill_mfma_kernel");
     return DRK_OK;
 }
