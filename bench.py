@@ -45,10 +45,11 @@ def parse():
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="context per branch for the CPU sample (0 = auto)")
     ap.add_argument("--bulk-append-tokens", type=int, default=2048)
     ap.add_argument("--seed", type=int, default=2)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6],
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5, 6, 7],
                     help="BASELINE config: 2 (default, the headline) | 3 shared prefix + COW + eviction | "
                          "4 int8/fp8 pages at 128k | 5 chunked MFMA prefill interleaved with decode | "
-                         "6 config 3's shape through the stream driver (whole layer path, captured step)")
+                         "6 config 3's shape through the stream driver (whole layer path, captured step) | "
+                         "7 config 2's workload at the reference's own model shape (24 Q / 4 KV x 256, block 256)")
     ap.add_argument("--kv-dtype", choices=["bf16", "int8", "fp8"], default=None,
                     help="storage type of the pages: config 4 int8 (default) | fp8; config 5 bf16 (default) | int8 | fp8")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "

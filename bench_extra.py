@@ -465,5 +465,86 @@ def config6(args):
     }
 
 
+def config7(args):
+    """The reference's own model shape (24 Q / 4 KV heads x 256, 256-token blocks, fp16, 16 full-attention
+    layers; model.h:39-42, block_pool.h:34-38) on config 2's workload: 8 branches x 32k tokens; step = per
+    layer the fused split + norm + RoPE + page write, then decode attention with the gate."""
+    torch, cabi, U, lib, stream, sp = _common(args)
+    L, KVH, QH, D, bs, B, ctx, RD = min(args.layers, 16), 4, 24, 256, 256, 8, 32768, 64
+    W, K = args.warmup, args.steps
+    nblk = ctx // bs + 1
+    NB = B * nblk + 8
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.F16)
+    rng = np.random.default_rng(7)
+    perm = rng.permutation(NB).astype(np.int32)
+    tables = np.stack([perm[b * nblk:(b + 1) * nblk] for b in range(B)])
+    dtab = torch.from_numpy(tables).cuda()
+    pool = torch.empty(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    pool.view(torch.float16).normal_(0, 0.5)
+    start = ctx - (W + K)
+    pos_steps = torch.from_numpy(np.stack([np.full(B, start + s, dtype=np.int32) for s in range(W + K)])).cuda()
+    len_steps = pos_steps + 1
+    h = torch.float16
+    qg = (torch.randn(L, B, QH, 2 * D, device="cuda") * 0.5).to(h)
+    k = (torch.randn(L, B, KVH, D, device="cuda") * 0.5).to(h)
+    v = (torch.randn(L, B, KVH, D, device="cuda") * 0.5).to(h)
+    qn = (1 + 0.1 * torch.randn(D, device="cuda")).to(h)
+    kn = (1 + 0.1 * torch.randn(D, device="cuda")).to(h)
+    qs = torch.empty(L, B, QH, D, device="cuda", dtype=h)
+    out = torch.empty(L, B, QH, D, device="cuda", dtype=h)
+    table = torch.empty(ctx * RD, dtype=torch.float32, device="cuda")
+    cabi.call("drk_rope_table_fill", U.p(table), ctx, RD, 1.0e7, sp)
+    wsb = lib.drk_decode_workspace_bytes(C.byref(g), B, ctx)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    qgrow, krow, qrow = B * QH * 2 * D * 2, B * KVH * D * 2, B * QH * D * 2
+
+    def attn(l, dlen):
+        cabi.call("drk_paged_decode_attention_gated", C.byref(g), C.c_void_p(qs.data_ptr() + l * qrow), U.p(pool), U.p(dtab),
+                  nblk, dlen, B, ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.F16,
+                  C.c_void_p(qg.data_ptr() + l * qgrow + D * 2), 2 * D, U.p(ws), wsb, sp)
+
+    def step(s):
+        dpos, dlen = C.c_void_p(pos_steps[s].data_ptr()), C.c_void_p(len_steps[s].data_ptr())
+        for l in range(L):
+            cabi.call("drk_qk_norm_rope_append", C.byref(g), U.p(pool), U.p(dtab), nblk, dpos, 0, B, l,
+                      C.c_void_p(qg.data_ptr() + l * qgrow), C.c_void_p(k.data_ptr() + l * krow),
+                      C.c_void_p(v.data_ptr() + l * krow), U.p(qn), U.p(kn), 1e-6, RD, 1.0e7, U.p(table), ctx,
+                      C.c_void_p(qs.data_ptr() + l * qrow), cabi.F16, sp)
+            attn(l, dlen)
+
+    for s in range(W):
+        step(s)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for s in range(W, W + K):
+        step(s)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    total_ms = e0.elapsed_time(e1)
+    per_tok = 2 * KVH * D * 2
+    toks = sum(B * (start + s + 1) for s in range(W, W + K))
+    value = toks * per_tok * L / (total_ms * 1e-3) / 1e9
+    dlen = C.c_void_p(len_steps[W + K - 1].data_ptr())
+    ker_ms = _timed_decode(lib, cabi, lambda n: [attn(i % L, dlen) for i in range(n)], 60)
+    launch_bytes = B * ctx * per_tok
+    ach = launch_bytes / (ker_ms * 1e-3) / 1e9
+    return {
+        "metric": "paged_decode_attention_GBps", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": round(total_ms / K, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"the reference's model shape: {L} full-attention layers, 24 Q / 4 KV heads x 256, fp16, 256-token "
+                               f"blocks, 64 rotary dims, 8 branches x 32768 tokens; step = per layer: fused split + head norm + "
+                               f"RoPE + page write, decode attention with the sigmoid gate; kernels launched from the host",
+                   "branches": B, "layers": L, "ctx_final": [ctx] * B},
+        "tokens_per_s": round(B * K / (total_ms * 1e-3), 1), "us_per_step": round(total_ms / K * 1e3, 1),
+        "roofline": {"kernel": "decode_stream_kernel<f16, 256>", "bound": "hbm", "achieved": round(ach, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "avg_launch_us": round(ker_ms * 1e3, 2), "bytes_per_launch": launch_bytes},
+        "cpu_baseline": None,
+    }
+
+
 def run(args):
-    return {3: config3, 4: config4, 5: config5, 6: config6}[args.config](args)
+    return {3: config3, 4: config4, 5: config5, 6: config6, 7: config7}[args.config](args)
