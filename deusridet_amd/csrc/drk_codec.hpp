@@ -48,6 +48,25 @@ __device__ __forceinline__ uint32_t fp8_pair(float x0, float x1)
 #endif
 }
 
+// maximum over each aligned group of 16 lanes, by DPP (quad swaps, half-row and row mirrors)
+template <int CTRL>
+__device__ __forceinline__ float codec_dpp(float v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+#else
+    return v;
+#endif
+}
+__device__ __forceinline__ float row16_max(float v)
+{
+    v = fmaxf(v, codec_dpp<0xB1>(v));
+    v = fmaxf(v, codec_dpp<0x4E>(v));
+    v = fmaxf(v, codec_dpp<0x141>(v));
+    v = fmaxf(v, codec_dpp<0x140>(v));
+    return v;
+}
+
 // Store one source chunk (8 elements of type src_dtype, `val`) into the page row at byte
 // offset poff as chunk c of its row.  rc = chunks per row; the rc lanes that hold one row
 // are consecutive lanes of one wave (rc is a power of two <= 64), and every lane of the
@@ -66,8 +85,12 @@ __device__ __forceinline__ void store_page_chunk(uint8_t *__restrict__ pool, siz
             float amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; i++) amax = fmaxf(amax, fabsf(x[i]));
-            for (unsigned off = rc >> 1; off > 0; off >>= 1)
-                amax = fmaxf(amax, __shfl_xor(amax, (int)off));
+            if (rc == 16) {                                   // head_dim 128: one row = one DPP row of 16 lanes
+                amax = row16_max(amax);
+            } else {
+                for (unsigned off = rc >> 1; off > 0; off >>= 1)
+                    amax = fmaxf(amax, __shfl_xor(amax, (int)off));
+            }
             float s32 = __fdiv_rn(amax, 127.0f);
             uint16_t sh = __half_as_ushort(__float2half_rn(s32));
             if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
@@ -82,13 +105,13 @@ __device__ __forceinline__ void store_page_chunk(uint8_t *__restrict__ pool, siz
                 if (i < 4) lo |= b << (8 * i); else hi |= b << (8 * (i - 4));
             }
             if (ok) {
-                *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
+                st_stream64(pool + poff + (size_t)c * 8, make_uint2(lo, hi));
                 if (c == 0) *(uint16_t *)(pool + soff) = sh;
             }
         } else {
             uint32_t lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
             uint32_t hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
-            if (ok) *(uint2 *)(pool + poff + (size_t)c * 8) = make_uint2(lo, hi);
+            if (ok) st_stream64(pool + poff + (size_t)c * 8, make_uint2(lo, hi));
         }
     }
 }

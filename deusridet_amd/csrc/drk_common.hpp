@@ -110,6 +110,11 @@ __device__ __forceinline__ void st_stream128(void *p, uint4 v)
     drk_u32x4 w = {v.x, v.y, v.z, v.w};
     __builtin_nontemporal_store(w, (drk_u32x4 *)p);
 }
+__device__ __forceinline__ void st_stream64(void *p, uint2 v)
+{
+    drk_u32x2 w = {v.x, v.y};
+    __builtin_nontemporal_store(w, (drk_u32x2 *)p);
+}
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
