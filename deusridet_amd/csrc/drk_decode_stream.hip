@@ -726,38 +726,46 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
 
 // Attention mass per (branch, logical block): sum over the block's tokens and all query heads of
 // the softmax probability, from the per-group and per-row log-sum-exps the two kernels above
-// left.  One thread per (branch, block); consecutive threads read consecutive groups.
+// left.  A workgroup takes 64 blocks of one branch; wave w sums the heads w, w+4, ... (consecutive
+// lanes read consecutive groups), the four sums meet in LDS.
 __global__ __launch_bounds__(256) void block_mass_kernel(const float *__restrict__ lse_groups, const float *__restrict__ lse_rows,
                                                          const int32_t *__restrict__ seq_lens, int B, int QH, int lse_stride,
                                                          int bs, float *__restrict__ mass, int mass_stride, int accumulate)
 {
-    const int lb = (int)(blockIdx.x * 256 + threadIdx.x), b = blockIdx.y;
-    if (lb >= mass_stride) return;
+    __shared__ float part[4][64];
+    const int x = threadIdx.x & 63, hq = threadIdx.x >> 6;
+    const int lb = (int)blockIdx.x * 64 + x, b = blockIdx.y;
     const int len = seq_lens[b];
     const int nblk = len > 0 ? (len + bs - 1) / bs : 0;
+    float m = 0.0f;
+    if (lb < nblk) {
+        // only the groups of tiles that exist were written by this launch (a block may span several tiles)
+        const int g0 = lb * (bs / 16), g1 = min(min(g0 + bs / 16, lse_stride), ((len + kSTile - 1) / kSTile) * 4);
+        for (int h = hq; h < QH; h += 4) {
+            const float row = lse_rows[(size_t)b * QH + h];
+            const float *grp = lse_groups + ((size_t)b * QH + h) * lse_stride;
+            for (int gi = g0; gi < g1; gi++) {
+                const float v = grp[gi];
+                if (v > -INFINITY && row > -INFINITY) m += s_exp2(v - row);
+            }
+        }
+    }
+    part[hq][x] = m;
+    __syncthreads();
+    if (hq != 0 || lb >= mass_stride) return;
     float *dst = mass + (size_t)b * mass_stride + lb;
     if (lb >= nblk) {
         if (!accumulate) *dst = 0.0f;
         return;
     }
-    // only the groups of tiles that exist were written by this launch (a block may span several tiles)
-    const int g0 = lb * (bs / 16), g1 = min(min(g0 + bs / 16, lse_stride), ((len + kSTile - 1) / kSTile) * 4);
-    float m = 0.0f;
-    for (int h = 0; h < QH; h++) {
-        const float row = lse_rows[(size_t)b * QH + h];
-        const float *grp = lse_groups + ((size_t)b * QH + h) * lse_stride;
-        for (int gi = g0; gi < g1; gi++) {
-            const float v = grp[gi];
-            if (v > -INFINITY && row > -INFINITY) m += s_exp2(v - row);
-        }
-    }
+    m = (part[0][x] + part[1][x]) + (part[2][x] + part[3][x]);
     *dst = accumulate ? *dst + m : m;
 }
 
 int launch_block_mass(const float *lse_groups, const float *lse_rows, const int32_t *d_seq_lens, int B, int QH,
                       int lse_stride, int bs, float *mass, int mass_stride, int accumulate, hipStream_t st)
 {
-    hipLaunchKernelGGL(block_mass_kernel, dim3((mass_stride + 255) / 256, B), dim3(256), 0, st, lse_groups, lse_rows,
+    hipLaunchKernelGGL(block_mass_kernel, dim3((mass_stride + 63) / 64, B), dim3(256), 0, st, lse_groups, lse_rows,
                        d_seq_lens, B, QH, lse_stride, bs, mass, mass_stride, accumulate);
     DRK_LAUNCH_CHECK("block_mass_kernel");
     return DRK_OK;
