@@ -19,19 +19,28 @@ pytestmark = pytest.mark.gpu
 L, QH, KVH, D, BS, RD = 2, 32, 8, 128, 16, 32
 EPS, THETA = 1e-6, 1.0e7
 DT = cabi.BF16
+KVDT = cabi.BF16          # storage type of the pages (DT: what the model hands over and gets back)
 NPOS = 512
 POOL_BLOCKS = 48
+
+
+@pytest.fixture(params=[cabi.INT8, cabi.FP8_E4M3])
+def eight_bit_pages(request):
+    global KVDT
+    KVDT = request.param
+    yield
+    KVDT = cabi.BF16
 
 
 @pytest.fixture
 def reference_model_shape():
     """24 Q / 4 KV heads x 256, 256-token blocks, 64 rotary dims, fp16: the reference's own model
     (model.h:39-42, block_pool.h:34-38) instead of the 8B-class shape of the other tests."""
-    global QH, KVH, D, BS, RD, DT, POOL_BLOCKS
-    saved = (QH, KVH, D, BS, RD, DT, POOL_BLOCKS)
-    QH, KVH, D, BS, RD, DT, POOL_BLOCKS = 24, 4, 256, 256, 64, cabi.F16, 10
+    global QH, KVH, D, BS, RD, DT, KVDT, POOL_BLOCKS
+    saved = (QH, KVH, D, BS, RD, DT, KVDT, POOL_BLOCKS)
+    QH, KVH, D, BS, RD, DT, KVDT, POOL_BLOCKS = 24, 4, 256, 256, 64, cabi.F16, cabi.F16, 10
     yield
-    QH, KVH, D, BS, RD, DT, POOL_BLOCKS = saved
+    QH, KVH, D, BS, RD, DT, KVDT, POOL_BLOCKS = saved
 
 
 def d2h(ptr, nbytes):
@@ -45,7 +54,7 @@ class Session:
 
     def __init__(self, nbranch, scorer=False):
         import torch
-        assert host.set_attention_geometry(L, QH, KVH, D, DT)
+        assert host.set_attention_geometry(L, QH, KVH, D, KVDT, DT)
         assert host.lib().drkh_set_rope(RD, THETA, EPS)
         self.cm = host.CacheManager()
         self.sc = host.ImportanceScorer() if scorer else None
@@ -107,7 +116,7 @@ def run_session(nbranch, steps, mode, seed=120, scorer=False, shared_policy=None
     qw, kw = U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT)
     s.set_weights(qw, kw)
     st = U.stream_ptr()
-    og = orc.layout(L, KVH, QH, D, BS, s.NB, DT)
+    og = orc.layout(L, KVH, QH, D, BS, s.NB, KVDT)
     opool = orc.new_pool(og)
     record = dict(prefill=[], decode=[], inputs=[])
     # ---- perception: 100 tokens in chunks of 64 + 36 ----
@@ -224,6 +233,21 @@ def test_stream_session_at_the_reference_models_shape(dev, reference_model_shape
     s_g.ks.close_branches()
 
 
+def test_stream_session_with_8bit_pages(dev, eight_bit_pages):
+    """int8 (+ fp16 scales) and fp8 pages under the same session: K and V are quantised by the fused
+    norm + RoPE + page write (codes and scales bit for bit the oracle's), prefill and decode dequantise
+    inside attention, the copy-on-write copies carry the scales along, and the captured step replays."""
+    rec_e, pool_e, s_e = run_session(3, 3, "eager", seed=125)
+    s_e.ks.close_branches()
+    del s_e
+    rec_g, pool_g, s_g = run_session(3, 3, "graph", seed=125)
+    for step in range(3):
+        for layer in range(L):
+            assert np.array_equal(rec_g["decode"][step][layer], rec_e["decode"][step][layer]), (step, layer)
+    assert np.array_equal(pool_g, pool_e)
+    s_g.ks.close_branches()
+
+
 def test_stream_session_with_the_prefix_streamed_once(dev):
     """Same session, but the decode attention reads the branches' common prefix once for all of
     them (here from 64 shared tokens on; the default asks for 4096): still the oracle's results
@@ -273,7 +297,7 @@ def test_time_division_perception_between_decode_steps_and_a_changing_branch_cou
     qw, kw = U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT)
     s.set_weights(qw, kw)
     st = U.stream_ptr()
-    og = orc.layout(L, KVH, QH, D, BS, s.NB, DT)
+    og = orc.layout(L, KVH, QH, D, BS, s.NB, KVDT)
     opool = orc.new_pool(og)
     tables = {0: s.cm.h_block_table(0).copy()}
 
