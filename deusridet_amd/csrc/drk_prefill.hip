@@ -118,6 +118,7 @@ struct PrefillArgs {
     const uint8_t *q;
     uint8_t *out;
     int pos_start, M, QH, KVH, NB, bs, bs_shift;
+    int tpw;                      // query tokens per workgroup: 128 / (QH / KVH)
     unsigned head_stride, kv_plane, block_stride, scale_plane;
     float scale_log2e;
     // shared-prefix mode: row "token" = branch; every row sees tokens [0, min(len, shared))
@@ -227,7 +228,7 @@ __device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup &g
     }
 }
 
-// grid = (ceil(M/32) * KVH, 1[, splits]); block = 256.
+// grid = (ceil(M/TPW) * KVH, 1[, splits]), TPW = 128 / (QH/KVH) query tokens per workgroup; block = 256.
 // SHARED = false: causal prefill of a chunk, normalised output.
 // SHARED = true:  the M rows are decode branches that share the pages of tokens
 //                 [0, shared); workgroup z handles tokens [z, z+1) * chunk_tiles * 64 of
@@ -253,10 +254,13 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
 
-    // this lane's query row: token tq of the chunk, head hq of the group
-    const int tq = qt * 32 + w * 8 + (n >> 2);
-    const int head = kvh * 4 + (n & 3);
-    const bool row_live = tq < A.M;
+    // this lane's query row: row r of the workgroup's 128 = token r / G of its TPW = 128 / G query
+    // tokens, head r % G of the kv head's G query heads (the last 128 - TPW * G rows are idle)
+    const int G = A.QH / A.KVH, TPW = A.tpw;
+    const int r = w * 32 + n, rt = r / G;
+    const int tq = qt * TPW + rt;
+    const int head = kvh * G + (r - rt * G);
+    const bool row_live = rt < TPW && tq < A.M;
     int vis, lim_wg, t_begin = 0, first_masked_tile = 0;
     if (SHARED) {
         const int len = row_live ? A.seq_lens[tq] : 0;
@@ -265,8 +269,8 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         lim_wg = min(A.shared, (t_begin + A.chunk_tiles) * kPfBN);
     } else {
         vis = A.pos_start + tq + 1;
-        lim_wg = A.pos_start + min((qt + 1) * 32, A.M);         // exclusive limit over the workgroup
-        first_masked_tile = (A.pos_start + qt * 32 + 1) / kPfBN;   // tiles below are fully visible
+        lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);        // exclusive limit over the workgroup
+        first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;  // tiles below are fully visible
     }
     const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
 
@@ -557,7 +561,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.table = table0;
     A.q = (const uint8_t *)q;
     A.out = nullptr;
-    A.pos_start = 0; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs;
+    A.pos_start = 0; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs; A.tpw = 32;
     A.bs_shift = ilog2_exact((unsigned)a.bs);
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
     A.scale_log2e = scale * kLog2eP;
@@ -582,15 +586,15 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 {
     Lay a;
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
-    const bool mfma = !g_force_portable && a.D == 128 && a.QH / a.KVH == 4 && (a.bs % 16) == 0;
+    const bool mfma = !g_force_portable && a.D == 128 && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 && (a.bs % 16) == 0;
     if (mfma) return 0;
     if (!g_force_portable && stream_decode_supported(a, 1)) return prefill_stream_workspace_need(a, pos_start, M);
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
 // paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630.
-// head_dim 128, 4 query heads per KV head: the MFMA kernel above (no workspace; 8-bit
-// pages are dequantised on their way into LDS).  head_dim 256 or another group size (<= 16): blocks of query
+// head_dim 128: the MFMA kernel above (no workspace; any group size; 8-bit pages are
+// dequantised on their way into LDS).  head_dim 256 (group size <= 16): blocks of query
 // tokens through the tiled decode kernel in its causal mode (drk_decode_stream.hip).  Anything
 // else: row t of the chunk runs as one causal "branch" of the portable decode kernel -- the
 // reference's algorithm verbatim (paged_attention.cu:481, 506-549).  Both need the workspace.
@@ -609,7 +613,8 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         return fail(DRK_ERR_INVALID, "prefill: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
 
-    const bool mfma = !g_force_portable && a.D == 128 && a.QH / a.KVH == 4 && (a.bs % 16) == 0 && scale > 0.0f;
+    const bool mfma = !g_force_portable && a.D == 128 && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 && (a.bs % 16) == 0 &&
+                      scale > 0.0f;
     if (!mfma && !g_force_portable && scale > 0.0f && stream_decode_supported(a, 1)) {
         if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "prefill: workspace must be 16-byte aligned");
         return launch_prefill_stream(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
@@ -627,10 +632,11 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     A.q = (const uint8_t *)q;
     A.out = (uint8_t *)out;
     A.pos_start = pos_start; A.M = M; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs;
+    A.tpw = 128 / (a.QH / a.KVH);
     A.bs_shift = ilog2_exact((unsigned)a.bs);
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
     A.scale_log2e = scale * kLog2eP;
-    dim3 grid(((M + 31) / 32) * a.KVH);
+    dim3 grid(((M + A.tpw - 1) / A.tpw) * a.KVH);
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = (const uint16_t *)gate; A.gate_stride = gate_stride;
     hipStream_t st = (hipStream_t)stream;
