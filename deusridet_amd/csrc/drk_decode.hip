@@ -593,9 +593,8 @@ static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size
 
 static bool shared_path_ok(const Lay &a, int B, int shared)
 {
-    // the prefix pass is the MFMA prefill kernel: head_dim 128, 4 query heads per kv head, 16-bit pages
-    return !g_force_portable && stream_decode_supported(a, B) && a.D == 128 && a.QH / a.KVH == 4 && a.E == 2 &&
-           shared >= kTile;   // the caller checks scale > 0
+    // the prefix pass is the MFMA prefill kernel in its shared mode: head_dim 128, 16-bit pages
+    return !g_force_portable && stream_decode_supported(a, B) && a.D == 128 && a.E == 2 && shared >= kTile;   // the caller checks scale > 0
 }
 
 int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
@@ -717,7 +716,7 @@ size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_
     if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0) return 0;
     size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);
     const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
-    if (stream_decode_supported(a, B) && a.D == 128 && a.QH / a.KVH == 4 && a.E == 2 && shared >= kTile) {
+    if (stream_decode_supported(a, B) && a.D == 128 && a.E == 2 && shared >= kTile) {
         size_t s2 = shared_need(a, B, max_seq_len, shared, nullptr);
         if (s2 > need) need = s2;
     }

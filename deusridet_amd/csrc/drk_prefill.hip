@@ -561,7 +561,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.table = table0;
     A.q = (const uint8_t *)q;
     A.out = nullptr;
-    A.pos_start = 0; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs; A.tpw = 32;
+    A.pos_start = 0; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs; A.tpw = 128 / (a.QH / a.KVH);
     A.bs_shift = ilog2_exact((unsigned)a.bs);
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
     A.scale_log2e = scale * kLog2eP;
@@ -569,7 +569,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
     A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
     A.gate = nullptr; A.gate_stride = 0;
-    dim3 grid(((B + 31) / 32) * a.KVH, 1, A.nsplits);
+    dim3 grid(((B + A.tpw - 1) / A.tpw) * a.KVH, 1, A.nsplits);
     if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, true>), grid, dim3(256), 0, st, A);
     else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, true>), grid, dim3(256), 0, st, A);
     DRK_LAUNCH_CHECK("prefill_mfma_kernel<shared>");

@@ -312,13 +312,15 @@ def test_workspace_too_small_is_refused(dev):
 
 
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
-@pytest.mark.parametrize("shared,extra", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17]), (960 + 16, [5, 300]),
-                                          (64, [0]), (4096, list(range(0, 400, 10)))])
-def test_shared_prefix_decode(dev, dtype, shared, extra):
+@pytest.mark.parametrize("shared,extra,heads", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17], (8, 32)), (960 + 16, [5, 300], (8, 32)),
+                                                (64, [0], (8, 32)), (4096, list(range(0, 400, 10)), (8, 32)),
+                                                (1024, [3, 200, 64, 700, 1], (2, 16)), (512, [9, 100, 33], (4, 24))])
+def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
     """Branches whose leading pages are the same physical blocks (BASELINE config 3
     in small): the shared pass + private tails must agree with the fp64 oracle run
-    per branch, and with the plain per-branch call."""
-    L, KVH, QH, D, bs = 1, 8, 32, 128, 16
+    per branch, and with the plain per-branch call.  Also with 8 and 6 query heads per kv head."""
+    L, D, bs = 1, 128, 16
+    KVH, QH = heads
     B = len(extra)
     lens = np.array([shared + e for e in extra], dtype=np.int32)
     n_shared_blk = shared // bs
