@@ -227,6 +227,30 @@ def main():
     launch_bytes = int((start + last + 1).sum()) * kv_bytes_per_token               # one layer, one launch
     achieved = launch_bytes / (ker_avg_ms * 1e-3) / 1e9
 
+    # ---- the same kernel on config 2's context distribution, U{1024..32768} per branch (same pool and
+    # tables; only the lengths change), when the headline run is the fixed 32k point
+    ragged = None
+    if args.ctx_mode == "fixed":
+        rl = np.random.default_rng(args.seed + 1).integers(1024, min(args.ctx, max_ctx) + 1, size=B).astype(np.int32)
+        rlen = torch.from_numpy(rl).cuda()
+
+        def ragged_only(n):
+            for it in range(n):
+                l = it % L
+                cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
+                          U.p(dtab), stride, U.p(rlen), B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
+                          cabi.BF16, split, U.p(ws), wsb, sp)
+
+        ragged_only(8)
+        lib.drk_debug_time_decode_kernel(1)
+        ragged_only(n_timed)
+        cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
+        lib.drk_debug_time_decode_kernel(0)
+        r_ms = float(np.mean(buf[:cnt.value]))
+        r_bytes = int(rl.sum()) * kv_bytes_per_token
+        ragged = {"ctx": [int(x) for x in rl], "kernel_us": round(r_ms * 1e3, 2), "bytes_per_launch": r_bytes,
+                  "GBps": round(r_bytes / (r_ms * 1e-3) / 1e9, 1), "hbm_frac": round(r_bytes / (r_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
     # ---- achievable ceiling on this box: plain 128-bit streaming read of the pool
     probe_bytes = min(pool_bytes, 32 << 30)
     sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
@@ -468,6 +492,7 @@ def main():
         "bulk_gather_GBps": None if gather_gbps is None else round(gather_gbps, 1),
         "bulk_scatter_GBps": None if scatter_gbps is None else round(scatter_gbps, 1),
         "hbm_read_probe_GBps": round(read_probe_gbps, 1),
+        "ragged_ctx_decode": ragged,
         "fill_seconds": round(t_fill, 2),
         "layer_steps": layer_steps,
         "attention_mass": attention_mass,
