@@ -33,9 +33,7 @@ constexpr int kPfBN = 64;         // KV tokens per tile
 // apart -> 256 + 16.  V rows are read transposed (16 lanes per clock touch 4 consecutive
 // rows, 4 x 8 bytes each): consecutive rows must start 8 banks apart -> 256 + 32; with the
 // K pitch every other row pair collides (measured: half of the LDS-active cycles were
-// bank-conflict cycles).
-constexpr int kPfPitch = 272;
-constexpr int kPfPitchV = 288;
+// bank-conflict cycles).  For head_dim D: 2 D + 16 and 2 D + 32.
 constexpr float kLog2eP = 1.4426950408889634f;
 
 typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
@@ -145,66 +143,66 @@ __device__ __forceinline__ void pf_sched_barrier()
 #endif
 }
 
+// one wave's 16-token group of a tile: 16 rows of RB bytes = NL 128-bit loads per lane
+template <int RB>
 struct PfGroup {
-    uint4 r0, r1, r2, r3;
+    static constexpr int NL = RB / 64;
+    uint4 r[NL];
 };
 
-// one wave's 16-token group of a tile: 16 rows of 256 bytes (16-bit pages) or 128 bytes (8-bit)
-template <bool ONCE, bool Q8>
-__device__ __forceinline__ PfGroup pf_load_group(const uint8_t *__restrict__ base, bool valid, size_t off, int lane)
+template <bool ONCE, int RB>
+__device__ __forceinline__ PfGroup<RB> pf_load_group(const uint8_t *__restrict__ base, bool valid, size_t off, int lane)
 {
-    PfGroup g;
-    g.r0 = g.r1 = g.r2 = g.r3 = make_uint4(0, 0, 0, 0);
+    PfGroup<RB> g;
+#pragma unroll
+    for (int j = 0; j < PfGroup<RB>::NL; j++) g.r[j] = make_uint4(0, 0, 0, 0);
     if (valid) {
         const uint8_t *p = base + off + (size_t)lane * 16;
-        if constexpr (ONCE) {       // every page is read by one workgroup only: stream it
-            g.r0 = ld_stream128(p);
-            g.r1 = ld_stream128(p + 1024);
-            if constexpr (!Q8) {
-                g.r2 = ld_stream128(p + 2048);
-                g.r3 = ld_stream128(p + 3072);
-            }
-        } else {                    // 64 row tiles of a chunk share each page through the L2
-            g.r0 = *(const uint4 *)(p);
-            g.r1 = *(const uint4 *)(p + 1024);
-            if constexpr (!Q8) {
-                g.r2 = *(const uint4 *)(p + 2048);
-                g.r3 = *(const uint4 *)(p + 3072);
-            }
+#pragma unroll
+        for (int j = 0; j < PfGroup<RB>::NL; j++) {
+            if constexpr (ONCE) g.r[j] = ld_stream128(p + 1024 * j);   // every page is read by one workgroup only: stream it
+            else g.r[j] = *(const uint4 *)(p + 1024 * j);              // the row tiles of a chunk share each page through the L2
         }
     }
     return g;
 }
 
-template <int PITCH>
-__device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup &g, int w, int lane)
+// 16-bit pages: the 16-byte chunk j of a lane belongs to row (lane * 16 + 1024 j) / RB of the group.
+// Rows at or past `lim` may hold anything and are stored as zeros.
+template <int PITCH, int RB>
+__device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup<RB> &g, int w, int lane, int lim)
 {
-    uint8_t *dst = lds + (w * 16 + (lane >> 4)) * PITCH + (lane & 15) * 16;
-    *(uint4 *)(dst) = g.r0;
-    *(uint4 *)(dst + 4 * PITCH) = g.r1;
-    *(uint4 *)(dst + 8 * PITCH) = g.r2;
-    *(uint4 *)(dst + 12 * PITCH) = g.r3;
+    const int bp0 = lane * 16, row0 = bp0 / RB;
+    uint8_t *dst = lds + (w * 16 + row0) * PITCH + bp0 % RB;
+    constexpr int RSTEP = 1024 / RB;                          // rows between a lane's consecutive chunks
+    if (lim >= 16) {                                          // the common case, wave-uniform
+#pragma unroll
+        for (int j = 0; j < PfGroup<RB>::NL; j++) *(uint4 *)(dst + j * RSTEP * PITCH) = g.r[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < PfGroup<RB>::NL; j++)
+            *(uint4 *)(dst + j * RSTEP * PITCH) = row0 + j * RSTEP < lim ? g.r[j] : make_uint4(0, 0, 0, 0);
+    }
 }
 
-// 8-bit pages: a lane holds 16 codes of row (lane / 8) + 8 j, dims (lane % 8) * 16 ..; they are
-// stored as the fp16 values code * scale (int8; sc = the two rows' fp16 scales, low / high half)
-// or as the fp8 values themselves.  Rows at or past `lim` may hold anything -- codes and scales --
-// and are stored as zeros.
-template <int PITCH, int KV>
-__device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup &g, int w, int lane, uint32_t sc, int lim)
+// 8-bit pages: chunk j of a lane holds 16 codes of row (lane * 16 + 1024 j) / RB; they are stored as
+// the fp16 values code * scale (int8; sc[j] = the row's fp16 scale) or as the fp8 values themselves.
+// Rows at or past `lim` may hold anything -- codes and scales -- and are stored as zeros.
+template <int PITCH, int KV, int RB>
+__device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup<RB> &g, int w, int lane,
+                                                  const uint16_t (&sc)[PfGroup<RB>::NL], int lim)
 {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    const uint4 regs[2] = {g.r0, g.r1};
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int row = (lane >> 3) + 8 * j;
+    for (int j = 0; j < PfGroup<RB>::NL; j++) {
+        const int bp = lane * 16 + 1024 * j, row = bp / RB, col = bp % RB;
         uint32_t h[8];
         if constexpr (KV == DRK_INT8) {
-            int8x4_to_f16x4(regs[j].x, h[0], h[1]);
-            int8x4_to_f16x4(regs[j].y, h[2], h[3]);
-            int8x4_to_f16x4(regs[j].z, h[4], h[5]);
-            int8x4_to_f16x4(regs[j].w, h[6], h[7]);
-            const uint32_t s16 = j ? (sc >> 16) : (sc & 0xffffu);
+            int8x4_to_f16x4(g.r[j].x, h[0], h[1]);
+            int8x4_to_f16x4(g.r[j].y, h[2], h[3]);
+            int8x4_to_f16x4(g.r[j].z, h[4], h[5]);
+            int8x4_to_f16x4(g.r[j].w, h[6], h[7]);
+            const uint32_t s16 = sc[j];
             const h2 scale = __builtin_bit_cast(h2, s16 | (s16 << 16));
             const h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
 #pragma unroll
@@ -213,16 +211,16 @@ __device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup &g
                 h[i] = __builtin_bit_cast(uint32_t, v);
             }
         } else {
-            fp8x4_to_f16x4(regs[j].x, h[0], h[1]);
-            fp8x4_to_f16x4(regs[j].y, h[2], h[3]);
-            fp8x4_to_f16x4(regs[j].z, h[4], h[5]);
-            fp8x4_to_f16x4(regs[j].w, h[6], h[7]);
+            fp8x4_to_f16x4(g.r[j].x, h[0], h[1]);
+            fp8x4_to_f16x4(g.r[j].y, h[2], h[3]);
+            fp8x4_to_f16x4(g.r[j].z, h[4], h[5]);
+            fp8x4_to_f16x4(g.r[j].w, h[6], h[7]);
         }
         if (row >= lim) {
 #pragma unroll
             for (int i = 0; i < 8; i++) h[i] = 0u;
         }
-        uint8_t *dst = lds + (w * 16 + row) * PITCH + (lane & 7) * 32;
+        uint8_t *dst = lds + (w * 16 + row) * PITCH + col * 2;
         *(uint4 *)(dst) = make_uint4(h[0], h[1], h[2], h[3]);
         *(uint4 *)(dst + 16) = make_uint4(h[4], h[5], h[6], h[7]);
     }
@@ -235,16 +233,20 @@ __device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup &g
 //                 them, no causal mask, and leaves (o, m, l) per (branch, q head, z).
 // DT: the type the matrix cores multiply in; KV: the pages' storage type (DT, or int8 / fp8 with
 // DT = fp16: the codes are dequantised on their way into LDS); IO: the type of q and out.
-template <int DT, bool SHARED, int KV = DT, int IO = DT>
-__global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
+// D: head_dim, 128 (two workgroups per CU) or 256 (one: twice the LDS and the accumulators).
+template <int DT, bool SHARED, int KV = DT, int IO = DT, int D = 128>
+__global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(PrefillArgs A)
 {
     constexpr bool Q8 = KV == DRK_INT8 || KV == DRK_FP8_E4M3;
-    constexpr int RB = Q8 ? 128 : 256;                      // bytes of one token row of one kv head
+    constexpr int RB = D * (Q8 ? 1 : 2);                    // bytes of one token row of one kv head
+    constexpr int kPitchK = D * 2 + 16, kPitchV = D * 2 + 32;   // LDS row pitches: conflict-free for the two read patterns
+    constexpr int NKS = D / 16;                             // k-steps of the first product
+    constexpr int NDT = D / 32;                             // 32-dim tiles of the second
     // Two buffers per operand.  The loop is software-pipelined by one tile: while the softmax of
     // tile i runs on the vector ALU, the matrix cores already compute the scores of tile i+1, so
     // K is staged one tile further ahead than V.  One barrier per tile.
-    __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPfPitch];
-    __shared__ __align__(16) uint8_t v_lds2[2][kPfBN * kPfPitchV];
+    __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPitchK];
+    __shared__ __align__(16) uint8_t v_lds2[2][kPfBN * kPitchV];
     __shared__ int valid_lds4[4][4];                       // page present, per (tile & 3, 16-token group)
 
     // Workgroups are dealt to the 8 XCDs round-robin by linear id; kv head = id % KVH
@@ -274,12 +276,12 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
     }
     const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
 
-    // Q as the B operand of S^T: 8 k-steps of 16 dims; lane holds dims ks*16 + g*8 .. +8
-    uint4 qf[8];
+    // Q as the B operand of S^T: NKS k-steps of 16 dims; lane holds dims ks*16 + g*8 .. +8
+    uint4 qf[NKS];
     {
-        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * 256 + g * 16;
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
 #if defined(__HIP_DEVICE_COMPILE__)
             if constexpr (IO == DRK_BF16 && DT == DRK_F16) {      // 8-bit pages multiply in fp16
@@ -309,71 +311,59 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         return base + (size_t)(tg - lb * A.bs) * RB;
     };
 
-    pf_f32x16 o[4];
+    pf_f32x16 o[NDT];
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++)
+    for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
     float m_run = -INFINITY, l_run = 0.0f;
 
     // registers -> LDS; rows at or past the workgroup's limit may hold anything and are cleared
     bool kreg_valid = false;
-    PfGroup kreg, vreg;
-    uint32_t ksc = 0u, vsc = 0u;               // int8 pages: the fp16 scales of this lane's two rows
-    auto clear_tail = [&](PfGroup &r, int tile) {
-        const int tile_t0 = tile * kPfBN;
-        if (tile_t0 + kPfBN > lim_wg) {
-            const int lim = lim_wg - tile_t0 - w * 16 - (lane >> 4);   // rows r0, r0+4, ... of this lane
-            const uint4 z = make_uint4(0, 0, 0, 0);
-            if (0 >= lim) r.r0 = z;
-            if (4 >= lim) r.r1 = z;
-            if (8 >= lim) r.r2 = z;
-            if (12 >= lim) r.r3 = z;
+    PfGroup<RB> kreg, vreg;
+    constexpr int NL = PfGroup<RB>::NL;
+    uint16_t ksc[NL], vsc[NL];                 // int8 pages: the fp16 scales of the rows of this lane's chunks
+#pragma unroll
+    for (int j = 0; j < NL; j++) ksc[j] = vsc[j] = 0;
+    auto load_scales = [&](bool valid, size_t soff, uint16_t (&sc)[NL]) {
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            const int row = (lane * 16 + 1024 * j) / RB;
+            sc[j] = (KV == DRK_INT8 && valid) ? *(const uint16_t *)(A.pool_layer + soff + row * 2) : (uint16_t)0;   // no page: zero codes times zero
         }
-    };
-    auto load_scales = [&](bool valid, size_t soff) -> uint32_t {
-        if (KV != DRK_INT8 || !valid) return 0u;               // no page: zero codes times zero
-        const uint8_t *p = A.pool_layer + soff + (lane >> 3) * 2;
-        return (uint32_t)*(const uint16_t *)p | ((uint32_t)*(const uint16_t *)(p + 16) << 16);
     };
     auto fetch_k = [&](int tile) {
         size_t soff;
         const size_t off = lookup(tile, kreg_valid, soff);
-        kreg = pf_load_group<SHARED, Q8>(kbase, kreg_valid, off, lane);
-        ksc = load_scales(kreg_valid, soff);
+        kreg = pf_load_group<SHARED, RB>(kbase, kreg_valid, off, lane);
+        load_scales(kreg_valid, soff, ksc);
     };
     auto fetch_v = [&](int tile) {
         bool ok;
         size_t soff;
         const size_t off = lookup(tile, ok, soff);
-        vreg = pf_load_group<SHARED, Q8>(kbase + A.kv_plane, ok, off, lane);
-        vsc = load_scales(ok, soff + A.scale_plane);
+        vreg = pf_load_group<SHARED, RB>(kbase + A.kv_plane, ok, off, lane);
+        load_scales(ok, soff + A.scale_plane, vsc);
     };
     auto stage_k = [&](int tile) {
-        if constexpr (Q8) {
-            pf_store_group_q8<kPfPitch, KV>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane, ksc, lim_wg - tile * kPfBN - w * 16);
-        } else {
-            clear_tail(kreg, tile);
-            pf_store_group<kPfPitch>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane);
-        }
+        const int lim = lim_wg - tile * kPfBN - w * 16;        // rows of this wave's group that exist
+        if constexpr (Q8) pf_store_group_q8<kPitchK, KV, RB>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane, ksc, lim);
+        else pf_store_group<kPitchK, RB>(&k_lds2[(tile - t_begin) & 1][0], kreg, w, lane, lim);
         if (lane == 0) valid_lds4[tile & 3][w] = kreg_valid ? 1 : 0;
     };
     auto stage_v = [&](int tile) {
-        if constexpr (Q8) {
-            pf_store_group_q8<kPfPitchV, KV>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane, vsc, lim_wg - tile * kPfBN - w * 16);
-        } else {
-            clear_tail(vreg, tile);
-            pf_store_group<kPfPitchV>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane);
-        }
+        const int lim = lim_wg - tile * kPfBN - w * 16;
+        if constexpr (Q8) pf_store_group_q8<kPitchV, KV, RB>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane, vsc, lim);
+        else pf_store_group<kPitchV, RB>(&v_lds2[(tile - t_begin) & 1][0], vreg, w, lane, lim);
     };
-    // S^T = K Q^T : two 32-token tiles x 32 rows, 8 k-steps of 16 dims
+    // S^T = K Q^T : two 32-token tiles x 32 rows, NKS k-steps of 16 dims
     auto qk = [&](int tile, pf_f32x16 (&s)[2]) {
-        const uint8_t *ka = &k_lds2[(tile - t_begin) & 1][0] + n * kPfPitch + g * 16;
+        const uint8_t *ka = &k_lds2[(tile - t_begin) & 1][0] + n * kPitchK + g * 16;
         const pf_f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};     // constant C operand of the first k-step
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
+        for (int ks = 0; ks < NKS; ks++) {
             const uint4 a0 = *(const uint4 *)(ka + ks * 32);
-            const uint4 a1 = *(const uint4 *)(ka + 32 * kPfPitch + ks * 32);
+            const uint4 a1 = *(const uint4 *)(ka + 32 * kPitchK + ks * 32);
             s[0] = mfma32<DT>(a0, qf[ks], ks == 0 ? zero : s[0]);
             s[1] = mfma32<DT>(a1, qf[ks], ks == 0 ? zero : s[1]);
         }
@@ -456,7 +446,7 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         m_run = m_new;
         if (!__all(alpha == 1.0f)) {
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++)
+            for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
         }
@@ -470,16 +460,16 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         {
             const int j16 = lane & 15;
             const int dsub = 16 * ((lane >> 4) & 1) + 4 * (j16 & 3);           // d offset inside a 32-d tile
-            const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPfPitchV + dsub * 2;
+            const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPitchV + dsub * 2;
 #pragma unroll
             for (int tt = 0; tt < 2; tt++)
 #pragma unroll
                 for (int mh = 0; mh < 2; mh++) {
-                    const uint8_t *vt = vb + (tt * 32 + 16 * mh) * kPfPitchV;
+                    const uint8_t *vt = vb + (tt * 32 + 16 * mh) * kPitchV;
 #pragma unroll
-                    for (int dt = 0; dt < 4; dt++) {
+                    for (int dt = 0; dt < NDT; dt++) {
                         const uint2 lo = lds_read_tr16(vt + dt * 64);
-                        const uint2 hi = lds_read_tr16(vt + 8 * kPfPitchV + dt * 64);
+                        const uint2 hi = lds_read_tr16(vt + 8 * kPitchV + dt * 64);
                         o[dt] = mfma32<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pb[tt][mh], o[dt]);
                     }
                 }
@@ -497,9 +487,9 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
     if (SHARED) {
         if (row_live) {                      // unnormalised partial; an empty range leaves (0, -inf, 0)
             const size_t pi = ((size_t)tq * A.QH + head) * A.nsplits + blockIdx.z;
-            float *orow = A.part_o + pi * 128;
+            float *orow = A.part_o + pi * D;
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++)
+            for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
                 for (int b4 = 0; b4 < 4; b4++)
                     *(float4 *)(orow + dt * 32 + 8 * b4 + 4 * g) =
@@ -514,10 +504,10 @@ __global__ __launch_bounds__(256, 2) void prefill_mfma_kernel(PrefillArgs A)
         // kernel left in out, also when no token took part (paged_attention.cu:551, 633-634)
         const bool have = l_tot > 0.0f;
         const float inv = have ? 1.0f / l_tot : 0.0f;
-        uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * 256;
+        uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * (D * 2);
         const uint16_t *grow = A.gate ? A.gate + ((size_t)tq * A.QH + head) * A.gate_stride : nullptr;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
             for (int b4 = 0; b4 < 4; b4++) {
                 const int d0 = dt * 32 + 8 * b4 + 4 * g;
@@ -586,16 +576,18 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 {
     Lay a;
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
-    const bool mfma = !g_force_portable && a.D == 128 && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 && (a.bs % 16) == 0;
+    const bool mfma = !g_force_portable && (a.D == 128 || (a.D == 256 && a.E == 2)) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 &&
+                      (a.bs % 16) == 0;
     if (mfma) return 0;
     if (!g_force_portable && stream_decode_supported(a, 1)) return prefill_stream_workspace_need(a, pos_start, M);
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
 // paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630.
-// head_dim 128: the MFMA kernel above (no workspace; any group size; 8-bit pages are
-// dequantised on their way into LDS).  head_dim 256 (group size <= 16): blocks of query
-// tokens through the tiled decode kernel in its causal mode (drk_decode_stream.hip).  Anything
+// head_dim 128, and 256 with 16-bit pages: the MFMA kernel above (no workspace; any group
+// size; 8-bit pages are dequantised on their way into LDS).  8-bit pages at head_dim 256
+// (group size <= 16): blocks of query tokens through the tiled decode kernel in its causal
+// mode (drk_decode_stream.hip).  Anything
 // else: row t of the chunk runs as one causal "branch" of the portable decode kernel -- the
 // reference's algorithm verbatim (paged_attention.cu:481, 506-549).  Both need the workspace.
 static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
@@ -613,8 +605,8 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         return fail(DRK_ERR_INVALID, "prefill: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
 
-    const bool mfma = !g_force_portable && a.D == 128 && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 && (a.bs % 16) == 0 &&
-                      scale > 0.0f;
+    const bool mfma = !g_force_portable && (a.D == 128 || (a.D == 256 && a.E == 2)) && a.QH % a.KVH == 0 &&
+                      a.QH / a.KVH <= 128 && (a.bs % 16) == 0 && scale > 0.0f;
     if (!mfma && !g_force_portable && scale > 0.0f && stream_decode_supported(a, 1)) {
         if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "prefill: workspace must be 16-byte aligned");
         return launch_prefill_stream(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
@@ -640,7 +632,11 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = (const uint16_t *)gate; A.gate_stride = gate_stride;
     hipStream_t st = (hipStream_t)stream;
-    if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, st, A);
+    if (a.D == 256 && a.dtype == DRK_BF16)
+        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false, DRK_BF16, DRK_BF16, 256>), grid, dim3(256), 0, st, A);
+    else if (a.D == 256)
+        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_F16, DRK_F16, 256>), grid, dim3(256), 0, st, A);
+    else if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, st, A);
     else if (a.dtype == DRK_F16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false>), grid, dim3(256), 0, st, A);
     else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16)
         hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_INT8, DRK_BF16>), grid, dim3(256), 0, st, A);
