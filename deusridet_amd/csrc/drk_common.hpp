@@ -69,10 +69,6 @@ int launch_sigmoid_gate(const void *x, const void *gate, void *out, size_t rows,
 extern int g_stream_wgs;
 extern int g_shared_splits;
 bool stream_decode_supported(const Lay &a, int B);
-size_t prefill_stream_workspace_need(const Lay &a, int pos_start, int M);
-int launch_prefill_stream(const Lay &a, const void *q, const void *pool, const int32_t *table, void *out, int layer,
-                          int pos_start, int M, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
-                          hipStream_t st, const void *gate, size_t gate_stride);
 size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens);
 int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,

@@ -127,13 +127,6 @@ struct StreamArgs {
     // (what the attention-mass pass needs; -inf for a group without a visible token)
     float *lse_groups;
     int lse_stride;
-    // Causal mode (chunked prefill through this kernel), cq_tq > 0: a "branch" is a block of cq_tq
-    // consecutive query tokens of one sequence, whose cq_tq * (QH/KVH) <= 16 (token, head) pairs fill
-    // the padded columns.  Block i sees cq_base + (i+1) * cq_tq tokens, its column of token k
-    // (0-based inside the block) cq_tq - 1 - k fewer; tokens i * cq_tq + k < cq_pad do not exist
-    // (the first block of a chunk may be partial).  q / partial rows are query rows [token][head],
-    // counted from the first existing token.  seq_lens is not read.
-    int cq_tq, cq_base, cq_pad;
 };
 
 constexpr int kMaxUnits = 256;       // units one workgroup may own (descriptor table in LDS)
@@ -142,7 +135,7 @@ struct UnitDesc {                    // one 64-token tile of one (branch, kv hea
     int tile_lim;                    // tokens of the tile that exist: seq_len - tile*64 (may exceed 64)
     int flags;                       // bit 0: first tile of a segment of this workgroup, bit 1: last; bits 2..: tile index
     int bq;                          // branch*QH + kvh*(QH/KVH): first query row of the group (Q, partial slots)
-    int piece;                       // bits 0-15: partial slot of the segment inside its (branch, q head); 16..: branch
+    int piece;                       // partial slot of the segment inside its (branch, q head)
 };
 
 // Geometry of one instantiation: head_dim D (128 or 256) and the storage type.
@@ -315,14 +308,8 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
     const int lane = threadIdx.x & 63;
     const int g = lane >> 4, c = lane & 15;
     const int GQ = A.QH / A.KVH;                               // query heads per kv head, 1..16
-    const int TQ = A.cq_tq > 0 ? A.cq_tq : 1;                  // query tokens per branch (causal mode), else 1
-    const int ncols = TQ * GQ;                                 // columns in use, <= 16
-    const int ctok = c / GQ, chead = c - ctok * GQ;            // this lane's column: token of the block, head of the group
-    const int coff = ctok * A.QH + chead;                      // its query row, relative to the block's first
-    const int cdef = A.cq_tq > 0 ? TQ - 1 - ctok : 0;          // tokens at the end of the block's context it must not see
-
     // ---- the workgroup's run of units and one descriptor per unit ---------------------
-    const int len_i = lane < A.B ? (A.cq_tq > 0 ? A.cq_base + (lane + 1) * TQ : (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host)) : 0;
+    const int len_i = lane < A.B ? (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host) : 0;
     const int nt_i = len_i > 0 ? max((len_i + kSTile - 1) / kSTile - A.start_tile, 0) : 0;
     int incl = nt_i;
 #pragma unroll
@@ -367,8 +354,8 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
             UnitDesc d;
             d.tile_lim = len - tile * kSTile;
             d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0) | (tile << 2);
-            d.bq = (b * TQ - A.cq_pad) * A.QH + kvh * GQ;
-            d.piece = ((int)blockIdx.x - (A.KVH * excl + kvh * nt) / U) | (b << 16);
+            d.bq = b * A.QH + kvh * GQ;
+            d.piece = (int)blockIdx.x - (A.KVH * excl + kvh * nt) / U;
             udesc[ui] = d;
         }
     }
@@ -402,13 +389,12 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
         const int lim = hole ? 0 : tile_lim;                    // tokens of the tile this wave may look at
         const bool has_next = it + 1 < nunits;
         if (flags & 1) {
-            // Q^T as the B operand: lane (column c, dims 32 kk + 8 g ..) -- columns past ncols are padding
-            const bool col_ok = c < ncols && (ud.piece >> 16) * TQ + ctok >= A.cq_pad;
+            // Q^T as the B operand: lane (head c, dims 32 kk + 8 g ..) -- heads GQ..15 are padding
             float sq = 0.0f;
 #pragma unroll
             for (int kk = 0; kk < Geo::NQK; kk++) {
                 uint4 v = make_uint4(0u, 0u, 0u, 0u);
-                if (col_ok) v = *(const uint4 *)(A.q + (size_t)(ud.bq + coff) * (D * 2) + kk * 64 + g * 16);
+                if (c < GQ) v = *(const uint4 *)(A.q + (size_t)(ud.bq + c) * (D * 2) + kk * 64 + g * 16);
 #if defined(__HIP_DEVICE_COMPILE__)
                 if (Q8 && A.io_dtype == DRK_BF16) {          // quantised pages multiply in fp16
                     v.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.x), bf16_hi(v.x)));
@@ -467,7 +453,7 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
             float x = sacc[j];
             if (DT == DRK_INT8) x = (x - qbias) * ks[j];
             x *= A.scale_log2e;
-            sc[j] = t0 + j < lim - cdef ? x : -INFINITY;
+            sc[j] = t0 + j < lim ? x : -INFINITY;
         }
         float mloc = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
         mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
@@ -493,7 +479,7 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
         {
             float pw[4];
 #pragma unroll
-            for (int j = 0; j < 4; j++) pw[j] = (DT == DRK_INT8) ? (t0 + j < lim - cdef ? p[j] * vs[j] : 0.0f) : p[j];
+            for (int j = 0; j < 4; j++) pw[j] = (DT == DRK_INT8) ? (t0 + j < lim ? p[j] * vs[j] : 0.0f) : p[j];
             if constexpr (DOT == DRK_BF16) {
                 pa.x = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[1]) << 16);
                 pa.y = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[3]) << 16);
@@ -561,7 +547,7 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
                 if constexpr (G4) bias[j] = DT == DRK_INT8 ? kI8Bias * s_lane(pw, j) : 0.0f;
                 else bias[j] = DT == DRK_INT8 ? kI8Bias * __shfl(pw, h) : 0.0f;
             }
-            const int rounds = G4 ? 1 : (ncols + 3) >> 2;            // 4 columns per round: column 4r + w is stored by wave w
+            const int rounds = G4 ? 1 : (GQ + 3) >> 2;               // 4 heads per round: head 4r + w is stored by wave w
             for (int r = 0; r < rounds; r++) {
                 if (r > 0) __syncthreads();                          // the previous round's sums have been read
                 if (g == r) {
@@ -588,8 +574,7 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
                     if (mm != -INFINITY) L = fmaf(lw_lds[ww][h], s_exp2(mm - M), L);
                 }
                 __syncthreads();
-                const int htok = h / GQ;
-                if (h < ncols && (ud.piece >> 16) * TQ + htok >= A.cq_pad) {
+                if (h < GQ) {
                     constexpr int VEC = D / 64;
                     const int d = lane * VEC;
                     float acc[VEC];
@@ -599,7 +584,7 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
                     for (int ww = 0; ww < 4; ww++)
 #pragma unroll
                         for (int x = 0; x < VEC; x++) acc[x] += o_lds[ww][w][d + x];
-                    const size_t pi = (size_t)(ud.bq + htok * A.QH + (h - htok * GQ)) * A.Pmax + (ud.piece & 0xffff);
+                    const size_t pi = (size_t)(ud.bq + h) * A.Pmax + ud.piece;
 #pragma unroll
                     for (int x = 0; x < VEC; x++) A.part_o[pi * D + d + x] = acc[x];
                     if (lane == 0) {
@@ -631,21 +616,18 @@ __global__ __launch_bounds__(256) void stream_merge_kernel(const float *__restri
                                                            int io_dtype, int start_tile, const float *__restrict__ pre_o,
                                                            const float *__restrict__ pre_m, const float *__restrict__ pre_l,
                                                            int pre_splits, const uint16_t *__restrict__ gate,
-                                                           size_t gate_stride, float *__restrict__ lse_rows, int cq_tq,
-                                                           int cq_base, int cq_pad)
+                                                           size_t gate_stride, float *__restrict__ lse_rows)
 {
     constexpr int VEC = D / 64;                                  // dims per lane: 2 or 4
     typedef float fvec __attribute__((ext_vector_type(VEC)));
     __shared__ fvec red[4][64];
     const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * VEC;
-    // causal mode: row b is a query token of a chunk, B counts blocks of cq_tq tokens (see StreamArgs)
-    const int blk = cq_tq > 0 ? (b + cq_pad) / cq_tq : b;
     int excl = 0, total = 0, nt_b = 0;
     for (int i = 0; i < B; i++) {
-        const int len = cq_tq > 0 ? cq_base + (i + 1) * cq_tq : (seq_lens ? seq_lens[i] : seq_len_host);
+        const int len = seq_lens ? seq_lens[i] : seq_len_host;
         const int nt = len > 0 ? max((len + kSTile - 1) / kSTile - start_tile, 0) : 0;
-        if (i < blk) excl += nt;
-        if (i == blk) nt_b = nt;
+        if (i < b) excl += nt;
+        if (i == b) nt_b = nt;
         total += nt;
     }
     int npieces = 0;
@@ -827,7 +809,6 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
         A.scale_log2e = scale * kSLog2e;
         A.lse_groups = lse_groups; A.lse_stride = lse_stride;
-        A.cq_tq = 0; A.cq_base = 0; A.cq_pad = 0;
 #define DRK_STREAM_LAUNCH(DT)                                                                                           \
     do {                                                                                                                \
         const bool g4 = a.QH / a.KVH <= 4;                                                                              \
@@ -848,116 +829,12 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         if (a.D == 128)
             hipLaunchKernelGGL(stream_merge_kernel<128>, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                                d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
-                               pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows, 0, 0, 0);
+                               pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows);
         else
             hipLaunchKernelGGL(stream_merge_kernel<256>, dim3(a.QH, B), dim3(256), 0, st, part_o, part_m, part_l, (uint16_t *)out,
                                d_seq_lens, seq_len_host, B, a.KVH, a.QH, U, grid, Pmax, io_dtype, start_tile, pre_o, pre_m,
-                               pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows, 0, 0, 0);
+                               pre_l, pre_splits, (const uint16_t *)gate, gate_stride, lse_rows);
         DRK_LAUNCH_CHECK("stream_merge_kernel");
-    }
-    return DRK_OK;
-}
-
-// ---- chunked causal prefill through the same kernel ------------------------------------------
-// For what the MFMA prefill kernel does not take (8-bit pages, head_dim 256, other group sizes):
-// the chunk's query tokens are cut into blocks of TQ = 16 / (QH/KVH) tokens whose (token, head)
-// pairs fill the 16 padded columns of the two products, 64 blocks per launch; a block streams the
-// context it can see once for all its columns.  The pages are read M / TQ times per kv head
-// instead of once per 32 tokens as in the MFMA kernel -- mostly out of the L2 and the memory-side
-// cache, since consecutive blocks read the same pages -- which is why this is the fallback.
-static void causal_plan(const Lay &a, int B, int TQ, int cq_base, int *grid, int *Pmax)
-{
-    long T = 0;
-    int max_tiles = 0;
-    for (int i = 0; i < B; i++) {
-        const int nt = (cq_base + (i + 1) * TQ + kSTile - 1) / kSTile;
-        T += nt;
-        if (nt > max_tiles) max_tiles = nt;
-    }
-    T *= a.KVH;
-    long G = T < stream_wgs(a) ? T : stream_wgs(a);
-    if (G < 1) G = 1;
-    if ((T + G - 1) / G > kMaxUnits) G = (T + kMaxUnits - 1) / kMaxUnits;
-    const long U = (T + G - 1) / G;
-    *grid = (int)G;
-    *Pmax = (int)((max_tiles + U - 1) / U) + 2;
-}
-
-static inline int causal_tq(const Lay &a) { const int gq = a.QH / a.KVH; return 16 / gq > 0 ? 16 / gq : 1; }
-
-size_t prefill_stream_workspace_need(const Lay &a, int pos_start, int M)
-{
-    if (M <= 0) return 0;
-    const int TQ = causal_tq(a), nb = (M + TQ - 1) / TQ, pad = nb * TQ - M;
-    size_t need = 0;
-    for (int blk0 = 0; blk0 < nb; blk0 += 64) {
-        const int B = nb - blk0 < 64 ? nb - blk0 : 64;
-        int grid, Pmax;
-        causal_plan(a, B, TQ, pos_start + blk0 * TQ - pad, &grid, &Pmax);
-        const size_t rows = (size_t)B * TQ;
-        const size_t n = rows * a.QH * Pmax * (a.D + 2) * sizeof(float);
-        if (n > need) need = n;
-    }
-    return need;
-}
-
-int launch_prefill_stream(const Lay &a, const void *q, const void *pool, const int32_t *table, void *out, int layer,
-                          int pos_start, int M, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
-                          hipStream_t st, const void *gate, size_t gate_stride)
-{
-    if (M <= 0) return DRK_OK;
-    if (workspace_bytes < prefill_stream_workspace_need(a, pos_start, M) || !workspace)
-        return fail(DRK_ERR_WORKSPACE, "prefill: workspace of %zu bytes, need %zu", workspace_bytes,
-                    prefill_stream_workspace_need(a, pos_start, M));
-    const int TQ = causal_tq(a), nb = (M + TQ - 1) / TQ, pad = nb * TQ - M;
-    const size_t row_bytes = (size_t)a.QH * a.D * 2;
-    for (int blk0 = 0; blk0 < nb; blk0 += 64) {
-        const int B = nb - blk0 < 64 ? nb - blk0 : 64;
-        const int pad_l = blk0 == 0 ? pad : 0;
-        const int first_tok = blk0 == 0 ? 0 : blk0 * TQ - pad;          // the launch's first existing query token
-        const int rows = B * TQ - pad_l;
-        int grid, Pmax;
-        const int cq_base = pos_start + blk0 * TQ - pad;
-        causal_plan(a, B, TQ, cq_base, &grid, &Pmax);
-        float *part_o = (float *)workspace;
-        float *part_m = part_o + (size_t)rows * a.QH * Pmax * a.D;
-        float *part_l = part_m + (size_t)rows * a.QH * Pmax;
-        StreamArgs A;
-        A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
-        A.tables = table; A.seq_lens = nullptr; A.q = (const uint8_t *)q + first_tok * row_bytes;
-        A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
-        A.table_stride = 0; A.seq_len_host = 0; A.B = B; A.KVH = a.KVH; A.QH = a.QH;
-        A.NB = a.NB; A.bs = a.bs; A.bs_shift = ilog2_exact((unsigned)a.bs); A.io_dtype = io_dtype;
-        A.unit_tiles = 0; A.Pmax = Pmax; A.start_tile = 0;
-        A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
-        A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
-        A.scale_log2e = scale * kSLog2e;
-        A.lse_groups = nullptr; A.lse_stride = 0;
-        A.cq_tq = TQ; A.cq_base = cq_base; A.cq_pad = pad_l;
-#define DRK_CAUSAL_LAUNCH(DT)                                                                                           \
-    do {                                                                                                                \
-        if (a.D == 128) hipLaunchKernelGGL((decode_stream_kernel<DT, 128, false>), dim3(grid), dim3(256), 0, st, A);    \
-        else hipLaunchKernelGGL((decode_stream_kernel<DT, 256, false>), dim3(grid), dim3(256), 0, st, A);               \
-    } while (0)
-        switch (a.dtype) {
-        case DRK_F16: DRK_CAUSAL_LAUNCH(DRK_F16); break;
-        case DRK_BF16: DRK_CAUSAL_LAUNCH(DRK_BF16); break;
-        case DRK_INT8: DRK_CAUSAL_LAUNCH(DRK_INT8); break;
-        default: DRK_CAUSAL_LAUNCH(DRK_FP8_E4M3); break;
-        }
-#undef DRK_CAUSAL_LAUNCH
-        DRK_LAUNCH_CHECK("decode_stream_kernel (causal)");
-        uint16_t *out_l = (uint16_t *)((uint8_t *)out + first_tok * row_bytes);
-        const uint16_t *gate_l = gate ? (const uint16_t *)gate + (size_t)first_tok * a.QH * gate_stride : nullptr;
-        if (a.D == 128)
-            hipLaunchKernelGGL(stream_merge_kernel<128>, dim3(a.QH, rows), dim3(256), 0, st, part_o, part_m, part_l, out_l,
-                               nullptr, 0, B, a.KVH, a.QH, 0, grid, Pmax, io_dtype, 0, nullptr, nullptr, nullptr, 0, gate_l,
-                               gate_stride, nullptr, TQ, cq_base, pad_l);
-        else
-            hipLaunchKernelGGL(stream_merge_kernel<256>, dim3(a.QH, rows), dim3(256), 0, st, part_o, part_m, part_l, out_l,
-                               nullptr, 0, B, a.KVH, a.QH, 0, grid, Pmax, io_dtype, 0, nullptr, nullptr, nullptr, 0, gate_l,
-                               gate_stride, nullptr, TQ, cq_base, pad_l);
-        DRK_LAUNCH_CHECK("stream_merge_kernel (causal)");
     }
     return DRK_OK;
 }

@@ -576,20 +576,17 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 {
     Lay a;
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
-    const bool mfma = !g_force_portable && (a.D == 128 || (a.D == 256 && a.E == 2)) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 &&
+    const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 &&
                       (a.bs % 16) == 0;
     if (mfma) return 0;
-    if (!g_force_portable && stream_decode_supported(a, 1)) return prefill_stream_workspace_need(a, pos_start, M);
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
 // paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630.
-// head_dim 128, and 256 with 16-bit pages: the MFMA kernel above (no workspace; any group
-// size; 8-bit pages are dequantised on their way into LDS).  8-bit pages at head_dim 256
-// (group size <= 16): blocks of query tokens through the tiled decode kernel in its causal
-// mode (drk_decode_stream.hip).  Anything
-// else: row t of the chunk runs as one causal "branch" of the portable decode kernel -- the
-// reference's algorithm verbatim (paged_attention.cu:481, 506-549).  Both need the workspace.
+// head_dim 128 or 256, block_size a multiple of 16: the MFMA kernel above (no workspace; any
+// group size; 8-bit pages are dequantised on their way into LDS).  Anything else: row t of the
+// chunk runs as one causal "branch" of the portable decode kernel -- the reference's algorithm
+// verbatim (paged_attention.cu:481, 506-549) -- and needs the workspace.
 static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
                         void *out, int layer, int pos_start, int M, float scale, int io_dtype, void *workspace,
                         size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
@@ -605,13 +602,8 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         return fail(DRK_ERR_INVALID, "prefill: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
 
-    const bool mfma = !g_force_portable && (a.D == 128 || (a.D == 256 && a.E == 2)) && a.QH % a.KVH == 0 &&
+    const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 &&
                       a.QH / a.KVH <= 128 && (a.bs % 16) == 0 && scale > 0.0f;
-    if (!mfma && !g_force_portable && scale > 0.0f && stream_decode_supported(a, 1)) {
-        if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "prefill: workspace must be 16-byte aligned");
-        return launch_prefill_stream(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
-                                     workspace_bytes, (hipStream_t)stream, gate, gate_stride);
-    }
     if (!mfma)
         return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
                              io_dtype, 0, workspace, workspace_bytes, stream, gate, gate_stride);
@@ -632,20 +624,18 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = (const uint16_t *)gate; A.gate_stride = gate_stride;
     hipStream_t st = (hipStream_t)stream;
-    if (a.D == 256 && a.dtype == DRK_BF16)
-        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false, DRK_BF16, DRK_BF16, 256>), grid, dim3(256), 0, st, A);
-    else if (a.D == 256)
-        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_F16, DRK_F16, 256>), grid, dim3(256), 0, st, A);
-    else if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, false>), grid, dim3(256), 0, st, A);
-    else if (a.dtype == DRK_F16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false>), grid, dim3(256), 0, st, A);
-    else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16)
-        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_INT8, DRK_BF16>), grid, dim3(256), 0, st, A);
-    else if (a.dtype == DRK_INT8)
-        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_INT8, DRK_F16>), grid, dim3(256), 0, st, A);
-    else if (io_dtype == DRK_BF16)
-        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_FP8_E4M3, DRK_BF16>), grid, dim3(256), 0, st, A);
-    else
-        hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, false, DRK_FP8_E4M3, DRK_F16>), grid, dim3(256), 0, st, A);
+#define DRK_PF_LAUNCH(DT, KV, IO)                                                                                        \
+    do {                                                                                                                \
+        if (a.D == 128) hipLaunchKernelGGL((prefill_mfma_kernel<DT, false, KV, IO, 128>), grid, dim3(256), 0, st, A);   \
+        else hipLaunchKernelGGL((prefill_mfma_kernel<DT, false, KV, IO, 256>), grid, dim3(256), 0, st, A);              \
+    } while (0)
+    if (a.dtype == DRK_BF16) DRK_PF_LAUNCH(DRK_BF16, DRK_BF16, DRK_BF16);
+    else if (a.dtype == DRK_F16) DRK_PF_LAUNCH(DRK_F16, DRK_F16, DRK_F16);
+    else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16) DRK_PF_LAUNCH(DRK_F16, DRK_INT8, DRK_BF16);
+    else if (a.dtype == DRK_INT8) DRK_PF_LAUNCH(DRK_F16, DRK_INT8, DRK_F16);
+    else if (io_dtype == DRK_BF16) DRK_PF_LAUNCH(DRK_F16, DRK_FP8_E4M3, DRK_BF16);
+    else DRK_PF_LAUNCH(DRK_F16, DRK_FP8_E4M3, DRK_F16);
+#undef DRK_PF_LAUNCH
     DRK_LAUNCH_CHECK("prefill_mfma_kernel");
     return DRK_OK;
 }

@@ -239,11 +239,10 @@ int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, con
 /* paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630:
  * q/out [M, num_q_heads, head_dim]; row t attends to tokens 0..pos_start+t (the
  * chunk's own K/V must already be in the pages: write, then attend).
- * head_dim 128 (any storage type) and head_dim 256 with 16-bit pages, any number of query
- * heads per KV head up to 128, run on the MFMA prefill kernel and need no workspace
- * (drk_prefill_workspace_bytes returns 0).  8-bit pages at head_dim 256 (group size <= 16)
- * run in blocks of query tokens through the tiled decode kernel; anything else row by row
- * through the portable one.  Both need the workspace. */
+ * head_dim 128 or 256 with block_size % 16 == 0 (any storage type, any number of query
+ * heads per KV head up to 128) runs on the MFMA prefill kernel and needs no workspace
+ * (drk_prefill_workspace_bytes returns 0); anything else row by row through the portable
+ * decode kernel, which needs the workspace. */
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M);
 int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
                                 const int32_t *d_block_table, void *out, int layer,

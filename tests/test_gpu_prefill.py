@@ -160,12 +160,11 @@ def build_io(geom, dtype, io, total, seed, holes=(), mul=1.0):
                                            ((1, 2, 10, 128, 32, 60), cabi.F16, cabi.F16), ((1, 2, 16, 128, 16, 100), cabi.FP8_E4M3, cabi.F16)])
 @pytest.mark.parametrize("pos_start,M", [(0, 1), (0, 70), (37, 45), (509, 77), (1000, 300)])
 def test_prefill_of_8bit_pages_and_other_head_shapes(dev, geom, dtype, io, pos_start, M):
-    """What the 16-bit MFMA prefill kernel of the headline shape does not cover.  8-bit pages at
-    32 Q / 8 KV x 128: the same kernel, codes dequantised on their way into LDS (int8: code * scale
-    rounded to fp16 once).  head_dim 256 and group sizes 6, 16, 1, 3, 5, 8: blocks of query tokens fill
-    the padded columns of the tiled decode kernel (2, 1, 16, 5, 3, 2 tokens per block; M is not a
-    multiple of the block, so the first block is partial).  A hole in the table, stale bytes behind
-    the end.  Against the fp64 oracle, and the gated form against plain + gate."""
+    """The MFMA prefill kernel away from the headline shape: 8-bit pages (codes dequantised on their
+    way into LDS; int8: code * scale rounded to fp16 once), head_dim 256, and 4, 6, 16, 1, 3, 5, 8 query
+    heads per kv head (a workgroup's 128 rows are 128 / G tokens x G heads).  A hole in the table,
+    stale bytes behind the end.  Against the fp64 oracle, the gated form against plain + gate, and
+    not the bits of the row-wise path."""
     L, KVH, QH, D, bs, NB = geom
     holes = (1,) if pos_start + M > 3 * bs else ()
     g, og, rng, table, opool = build_io(geom, dtype, io, pos_start + M, seed=pos_start * 5 + M + D, holes=holes, mul=0.7)

@@ -219,7 +219,7 @@ def test_stream_session_matches_the_oracle_and_its_graph_replay(dev):
 
 def test_stream_session_at_the_reference_models_shape(dev, reference_model_shape):
     """The whole KV path at 24 Q / 4 KV heads x 256 with 256-token blocks: fused norm + RoPE + page write
-    at head_dim 256, prefill through the tiled kernel's causal mode (2 tokens x 6 heads per block), decode
+    at head_dim 256, MFMA prefill at head_dim 256 with 21 tokens x 6 heads per workgroup, decode
     with 6 heads per kv head, copy-on-write of a 256-token block, and the captured step."""
     rec_e, pool_e, s_e = run_session(2, 3, "eager", seed=124)
     s_e.ks.close_branches()
