@@ -82,8 +82,8 @@ int launch_block_mass(const float *lse_groups, const float *lse_rows, const int3
 // shared-prefix pass on the matrix cores (drk_prefill.hip)
 void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
-                         const int32_t *d_seq_lens, int B, int shared, int layer, float scale, float *part_o,
-                         float *part_m, float *part_l, hipStream_t st);
+                         const int32_t *d_seq_lens, int B, int shared, int layer, float scale, int io_dtype,
+                         float *part_o, float *part_m, float *part_l, hipStream_t st);
 
 // ---- element helpers (device) -------------------------------------------
 // Streaming ("non-temporal") 128- and 64-bit accesses for data that is touched once

@@ -593,8 +593,8 @@ static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size
 
 static bool shared_path_ok(const Lay &a, int B, int shared)
 {
-    // the prefix pass is the MFMA prefill kernel in its shared mode: head_dim 128, 16-bit pages
-    return !g_force_portable && stream_decode_supported(a, B) && a.D == 128 && a.E == 2 && shared >= kTile;   // the caller checks scale > 0
+    // the prefix pass is the MFMA prefill kernel in its shared mode (every shape the stream kernel takes)
+    return !g_force_portable && stream_decode_supported(a, B) && shared >= kTile;   // the caller checks scale > 0
 }
 
 int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
@@ -610,7 +610,9 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
         return launch_decode(g, q, pool, tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
                              io_dtype, 0, workspace, workspace_bytes, stream);
     if (!q || !pool || !tables || !out || !d_seq_lens) return fail(DRK_ERR_INVALID, "decode: NULL pointer");
-    if (io_dtype != a.dtype) return fail(DRK_ERR_INVALID, "decode: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
+    if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode: io_dtype must be F16 or BF16");
+    if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
+        return fail(DRK_ERR_INVALID, "decode: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "decode: layer %d outside [0,%d)", layer, a.L);
     size_t sp;
     const size_t need = shared_need(a, B, max_seq_len, shared, &sp);
@@ -632,7 +634,7 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
         DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count], st));
     }
     // branch 0's table addresses the shared pages (identical in every row by the caller's promise)
-    if ((rc = launch_shared_prefix(a, q, pool, tables, d_seq_lens, B, shared, layer, scale, pre_o, pre_m, pre_l, st))) return rc;
+    if ((rc = launch_shared_prefix(a, q, pool, tables, d_seq_lens, B, shared, layer, scale, io_dtype, pre_o, pre_m, pre_l, st))) return rc;
     if ((rc = launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
                                    io_dtype, 0, workspace, false, st, shared / kTile))) return rc;
     if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
@@ -716,7 +718,7 @@ size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_
     if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0) return 0;
     size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);
     const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
-    if (stream_decode_supported(a, B) && a.D == 128 && a.E == 2 && shared >= kTile) {
+    if (stream_decode_supported(a, B) && shared >= kTile) {
         size_t s2 = shared_need(a, B, max_seq_len, shared, nullptr);
         if (s2 > need) need = s2;
     }

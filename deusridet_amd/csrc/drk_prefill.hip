@@ -543,8 +543,8 @@ void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits)
 }
 
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
-                         const int32_t *d_seq_lens, int B, int shared, int layer, float scale, float *part_o,
-                         float *part_m, float *part_l, hipStream_t st)
+                         const int32_t *d_seq_lens, int B, int shared, int layer, float scale, int io_dtype,
+                         float *part_o, float *part_m, float *part_l, hipStream_t st)
 {
     PrefillArgs A;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
@@ -560,8 +560,18 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
     A.gate = nullptr; A.gate_stride = 0;
     dim3 grid(((B + A.tpw - 1) / A.tpw) * a.KVH, 1, A.nsplits);
-    if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_mfma_kernel<DRK_BF16, true>), grid, dim3(256), 0, st, A);
-    else hipLaunchKernelGGL((prefill_mfma_kernel<DRK_F16, true>), grid, dim3(256), 0, st, A);
+#define DRK_PF_SHARED(DT, KV, IO)                                                                                        \
+    do {                                                                                                                \
+        if (a.D == 128) hipLaunchKernelGGL((prefill_mfma_kernel<DT, true, KV, IO, 128>), grid, dim3(256), 0, st, A);    \
+        else hipLaunchKernelGGL((prefill_mfma_kernel<DT, true, KV, IO, 256>), grid, dim3(256), 0, st, A);               \
+    } while (0)
+    if (a.dtype == DRK_BF16) DRK_PF_SHARED(DRK_BF16, DRK_BF16, DRK_BF16);
+    else if (a.dtype == DRK_F16) DRK_PF_SHARED(DRK_F16, DRK_F16, DRK_F16);
+    else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16) DRK_PF_SHARED(DRK_F16, DRK_INT8, DRK_BF16);
+    else if (a.dtype == DRK_INT8) DRK_PF_SHARED(DRK_F16, DRK_INT8, DRK_F16);
+    else if (io_dtype == DRK_BF16) DRK_PF_SHARED(DRK_F16, DRK_FP8_E4M3, DRK_BF16);
+    else DRK_PF_SHARED(DRK_F16, DRK_FP8_E4M3, DRK_F16);
+#undef DRK_PF_SHARED
     DRK_LAUNCH_CHECK("prefill_mfma_kernel<shared>");
     return DRK_OK;
 }

@@ -224,8 +224,8 @@ int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, c
  * that every d_seq_lens[b] >= shared_tokens (CacheManager::common_prefix_tokens
  * computes it).  Those pages are then streamed from HBM once for all B branches
  * instead of once per branch.  shared_tokens is rounded down to a multiple of 64;
- * 0, or a geometry / storage type the shared pass does not take, gives exactly
- * drk_paged_decode_attention_branches.  Results equal the per-branch call up to
+ * 0, or a geometry the tiled decode kernel does not take, gives exactly
+ * drk_paged_decode_attention_branches (every storage type has the shared pass).  Results equal the per-branch call up to
  * summation order. */
 size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len, int shared_tokens);
 int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, const void *pool,

@@ -311,16 +311,18 @@ def test_workspace_too_small_is_refused(dev):
     assert rc == cabi.ERR_WORKSPACE
 
 
-@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
-@pytest.mark.parametrize("shared,extra,heads", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17], (8, 32)), (960 + 16, [5, 300], (8, 32)),
-                                                (64, [0], (8, 32)), (4096, list(range(0, 400, 10)), (8, 32)),
-                                                (1024, [3, 200, 64, 700, 1], (2, 16)), (512, [9, 100, 33], (4, 24))])
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
+@pytest.mark.parametrize("shared,extra,heads", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17], (8, 32, 128)), (960 + 16, [5, 300], (8, 32, 128)),
+                                                (64, [0], (8, 32, 128)), (4096, list(range(0, 400, 10)), (8, 32, 128)),
+                                                (1024, [3, 200, 64, 700, 1], (2, 16, 128)), (512, [9, 100, 33], (4, 24, 256))])
 def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
     """Branches whose leading pages are the same physical blocks (BASELINE config 3
     in small): the shared pass + private tails must agree with the fp64 oracle run
-    per branch, and with the plain per-branch call.  Also with 8 and 6 query heads per kv head."""
-    L, D, bs = 1, 128, 16
-    KVH, QH = heads
+    per branch, and with the plain per-branch call.  Also with 8 and 6 query heads per kv head,
+    head_dim 256, and 8-bit pages."""
+    L, bs = 1, 16
+    KVH, QH, D = heads
+    io = dtype if dtype in (cabi.F16, cabi.BF16) else cabi.BF16
     B = len(extra)
     lens = np.array([shared + e for e in extra], dtype=np.int32)
     n_shared_blk = shared // bs
@@ -337,17 +339,17 @@ def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
         tables[b, n_shared_blk:n_shared_blk + priv_blk[b]] = perm[o:o + priv_blk[b]]
         o += priv_blk[b]
     opool = orc.new_pool(og)
-    k = U.normal_bits(rng, (shared, KVH, D), dtype, 0.7)
-    v = U.normal_bits(rng, (shared, KVH, D), dtype, 0.7)
-    orc.append_batch(og, opool, tables[0], 0, 0, k, v, dtype)
+    k = U.normal_bits(rng, (shared, KVH, D), io, 0.7)
+    v = U.normal_bits(rng, (shared, KVH, D), io, 0.7)
+    orc.append_batch(og, opool, tables[0], 0, 0, k, v, io)
     for b in range(B):
         n = int(lens[b]) - n_shared_blk * bs
         if n > 0:
             # a branch's private part starts at the first non-shared block boundary
-            kk = U.normal_bits(rng, (n, KVH, D), dtype, 0.7)
-            vv = U.normal_bits(rng, (n, KVH, D), dtype, 0.7)
-            orc.append_batch(og, opool, tables[b], 0, n_shared_blk * bs, kk, vv, dtype)
-    q = U.normal_bits(rng, (B, QH, D), dtype, 0.7)
+            kk = U.normal_bits(rng, (n, KVH, D), io, 0.7)
+            vv = U.normal_bits(rng, (n, KVH, D), io, 0.7)
+            orc.append_batch(og, opool, tables[b], 0, n_shared_blk * bs, kk, vv, io)
+    q = U.normal_bits(rng, (B, QH, D), io, 0.7)
     scale = 1 / np.sqrt(D)
     dq, dpool, dtab, dl = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(tables), U.dev_i32(lens)
     lib = cabi.lib()
@@ -357,14 +359,14 @@ def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
     ws = U.dev_zeros(wsb)
     out = U.dev_bytes(np.full(B * QH * D * 2, 0x7B, dtype=np.uint8))
     cabi.call("drk_paged_decode_attention_shared", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dl), B, mx,
-              shared_arg, U.p(out), 0, float(scale), dtype, U.p(ws), wsb, U.stream_ptr())
+              shared_arg, U.p(out), 0, float(scale), io, U.p(ws), wsb, U.stream_ptr())
     out2 = U.dev_zeros(B * QH * D * 2)
     cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dl), B, mx,
-              U.p(out2), 0, float(scale), dtype, 0, U.p(ws), wsb, U.stream_ptr())
+              U.p(out2), 0, float(scale), io, 0, U.p(ws), wsb, U.stream_ptr())
     U.sync()
-    got = U.from_bits(U.host(out, np.uint16, (B, QH, D)), dtype)
-    plain = U.from_bits(U.host(out2, np.uint16, (B, QH, D)), dtype)
-    want = np.stack([orc.decode_f64(og, q[b], opool, tables[b], 0, int(lens[b]), scale, dtype) for b in range(B)])
+    got = U.from_bits(U.host(out, np.uint16, (B, QH, D)), io)
+    plain = U.from_bits(U.host(out2, np.uint16, (B, QH, D)), io)
+    want = np.stack([orc.decode_f64(og, q[b], opool, tables[b], 0, int(lens[b]), scale, io) for b in range(B)])
     ok, ma, _ = U.rel_abs_ok(got, want, REL, ABS)
     assert ok, ma
     ok, ma, _ = U.rel_abs_ok(got, plain, REL, ABS)
