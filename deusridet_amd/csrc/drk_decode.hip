@@ -499,6 +499,20 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     if (a.D % 64 || a.D > 512) return fail(DRK_ERR_UNSUPPORTED, "decode: head_dim %d (need a multiple of 64, <= 512)", a.D);
     if (G > 16) return fail(DRK_ERR_UNSUPPORTED, "decode: %d query heads per kv head (max 16)", G);
     if (split_tokens < 0 || (split_tokens % kTile)) return fail(DRK_ERR_INVALID, "decode: split_tokens must be a multiple of %d", kTile);
+    // more branches than one launch of the tiled kernel takes: 64 at a time, one after the other
+    // through the same workspace (the launches are ordered by the stream)
+    if (B > 64 && d_seq_lens && !g_force_portable && g_decode_kernel != 2 && causal_base < 0 && stream_decode_supported(a, 64)) {
+        const size_t row = (size_t)a.QH * a.D * 2;
+        for (int b0 = 0; b0 < B; b0 += 64) {
+            const int nb = B - b0 < 64 ? B - b0 : 64;
+            rc = launch_decode(g, (const uint8_t *)q + b0 * row, pool, tables + (size_t)b0 * table_stride, table_stride,
+                               d_seq_lens + b0, 0, -1, nb, max_seq_len, (uint8_t *)out + b0 * row, layer, scale, io_dtype,
+                               split_tokens, workspace, workspace_bytes, stream,
+                               gate ? (const uint8_t *)gate + (size_t)b0 * a.QH * gate_stride * 2 : nullptr, gate_stride);
+            if (rc) return rc;
+        }
+        return DRK_OK;
+    }
     const int split = split_tokens ? split_tokens : choose_split(a, B, max_seq_len);
     const int S = (max_seq_len + split - 1) / split;
     const bool use_stream = !g_force_portable && g_decode_kernel != 2 && causal_base < 0 && stream_decode_supported(a, B);
@@ -653,8 +667,9 @@ size_t drk_decode_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len
     Lay a;
     if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0) return 0;
     size_t need = workspace_need(a, B, max_seq_len, choose_split(a, B, max_seq_len));
-    if (stream_decode_supported(a, B)) {
-        size_t s2 = stream_workspace_need(a, B, max_seq_len, 0);
+    const int bs = B < 64 ? B : 64;                      // the tiled kernel takes 64 branches per launch
+    if (stream_decode_supported(a, bs)) {
+        size_t s2 = stream_workspace_need(a, bs, max_seq_len, 0);
         if (s2 > need) need = s2;
     }
     return need;
@@ -665,8 +680,9 @@ size_t drk_decode_workspace_bytes_for_split(const drk_kv_layout *g, int B, int m
     Lay a;
     if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0 || split_tokens <= 0) return 0;
     size_t need = workspace_need(a, B, max_seq_len, split_tokens);
-    if (stream_decode_supported(a, B)) {
-        size_t s2 = stream_workspace_need(a, B, max_seq_len, split_tokens);
+    const int bs = B < 64 ? B : 64;
+    if (stream_decode_supported(a, bs)) {
+        size_t s2 = stream_workspace_need(a, bs, max_seq_len, split_tokens);
         if (s2 > need) need = s2;
     }
     return need;

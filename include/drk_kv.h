@@ -164,9 +164,9 @@ int drk_kv_copy_blocks(const drk_kv_layout *g, void *pool, const int32_t *d_pair
                        void *stream);
 
 /* ---- paged GQA decode attention --------------------------------------- */
-/* Kernels: head_dim 128 or 256 with 1..16 query heads per kv head, block_size % 16 == 0 and at
- * most 64 branches per call run on the persistent tiled kernel (every storage type; the
- * reference's own 24 Q / 4 KV x 256, block 256 included); any other geometry (head_dim a
+/* Kernels: head_dim 128 or 256 with 1..16 query heads per kv head and block_size % 16 == 0 run
+ * on the persistent tiled kernel (every storage type; the reference's own 24 Q / 4 KV x 256,
+ * block 256 included; 64 branches per launch, more branches take several launches); any other geometry (head_dim a
  * multiple of 64 up to 512, group size <= 16) on a portable one.
  * Bytes of workspace the split-K decode needs for B branches of at most max_seq_len tokens: */
 size_t drk_decode_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len);

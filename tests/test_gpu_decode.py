@@ -371,3 +371,15 @@ def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
     assert ok, ma
     ok, ma, _ = U.rel_abs_ok(got, plain, REL, ABS)
     assert ok, ma
+
+
+def test_more_branches_than_one_launch_takes(dev):
+    """150 branches: the tiled kernel takes 64 per launch, so the call runs three launches through
+    the same workspace; each branch must come out as if it had been called alone."""
+    lens = [int(x) for x in np.random.default_rng(5).integers(1, 300, size=150)]
+    case = Case((1, 8, 32, 128, 16, 150 * 20), cabi.BF16, lens, seed=63, mul=0.7)
+    got = case.run_branches()
+    _check(case, got)
+    for b in (0, 63, 64, 127, 128, 149):                     # another split of the context: equal up to summation order
+        ok, ma, _ = U.rel_abs_ok(U.from_bits(case.run_single(b), case.io), U.from_bits(got[b], case.io).astype(np.float64), REL, ABS)
+        assert ok, (b, ma)
