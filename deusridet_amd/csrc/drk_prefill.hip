@@ -263,6 +263,9 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(Pre
     const int tq = qt * TPW + rt;
     const int head = kvh * G + (r - rt * G);
     const bool row_live = rt < TPW && tq < A.M;
+    // shared mode with few branches: a wave whose 32 rows are all idle only helps to stage the
+    // tiles; its first row decides, the rows of a wave being consecutive
+    const bool wave_live = (w * 32) / G < TPW && qt * TPW + (w * 32) / G < A.M;
     int vis, lim_wg, t_begin = 0, first_masked_tile = 0;
     if (SHARED) {
         const int len = row_live ? A.seq_lens[tq] : 0;
@@ -383,7 +386,7 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(Pre
     }
     __syncthreads();
     if (t_begin < ntiles) {
-        qk(t_begin, s);
+        if (!SHARED || wave_live) qk(t_begin, s);
         if (t_begin + 1 < ntiles) {
             stage_k(t_begin + 1);
             if (t_begin + 2 < ntiles) fetch_k(t_begin + 2);
@@ -404,75 +407,77 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(Pre
             stage_v(it + 1);                       // into the buffer V(it-1) was read from
             if (it + 2 < ntiles) fetch_v(it + 2);
         }
-        // ---- tile softmax for this lane's row; register i of tile tt is token
-        //      tile_t + tt*32 + 8*(i/4) + 4*g + i%4 ----
-        const bool all_groups_valid = (valid_lds[0] & valid_lds[1] & valid_lds[2] & valid_lds[3]) != 0;
-        const bool need_mask = !all_groups_valid ||
-                               (SHARED ? (__any(tile_t + kPfBN > vis) != 0) : (it >= first_masked_tile));
-        // raw scores stay in s; the scale (> 0) is folded into the exponent's fma
-        if (need_mask) {                                         // one uniform branch around all 32 selects
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-                    const bool ok = (tile_t + tl) < vis && valid_lds[tl >> 4] != 0;
-                    s[tt][i] = ok ? s[tt][i] : -INFINITY;
-                }
-        }
-        float tmax = -INFINITY;
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[tt][i]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));               // the row's other 32 tokens
-        const float m_new = fmaxf(m_run, tmax * A.scale_log2e);
-        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-        float psum = 0.0f;
-        uint4 pb[2][2];                                          // [token tile][k-half]: B operand of PV
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++) {
-            float p[16];
-#pragma unroll
-            for (int i = 0; i < 16; i++) p[i] = __builtin_amdgcn_exp2f(fmaf(s[tt][i], A.scale_log2e, -m_use));
-            pb[tt][0] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
-            pb[tt][1] = make_uint4(pack2<DT>(p[8], p[9]), pack2<DT>(p[10], p[11]), pack2<DT>(p[12], p[13]), pack2<DT>(p[14], p[15]));
-            // the row sum is taken over the rounded weights, the ones PV multiplies: one dot2 per pair
-            psum = pf_sum2<DT>(pb[tt][0], psum);
-            psum = pf_sum2<DT>(pb[tt][1], psum);
-        }
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
-        if (!__all(alpha == 1.0f)) {
-#pragma unroll
-            for (int dt = 0; dt < NDT; dt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
-        }
-
-        // The next tile's scores, in the same basic block as the exponentials and the PV product so
-        // that matrix and vector instructions alternate.  Unconditional: past the last tile it
-        // multiplies whatever the other K buffer holds and the result is dropped.
-        qk(it + 1, s_next);
-
-        // ---- O^T += V^T P^T : k-slot j of MFMA (tt, mh) is token tt*32 + 16*mh + 8*(j/4) + 4*g + j%4 ----
-        {
-            const int j16 = lane & 15;
-            const int dsub = 16 * ((lane >> 4) & 1) + 4 * (j16 & 3);           // d offset inside a 32-d tile
-            const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPitchV + dsub * 2;
-#pragma unroll
-            for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-                for (int mh = 0; mh < 2; mh++) {
-                    const uint8_t *vt = vb + (tt * 32 + 16 * mh) * kPitchV;
-#pragma unroll
-                    for (int dt = 0; dt < NDT; dt++) {
-                        const uint2 lo = lds_read_tr16(vt + dt * 64);
-                        const uint2 hi = lds_read_tr16(vt + 8 * kPitchV + dt * 64);
-                        o[dt] = mfma32<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pb[tt][mh], o[dt]);
+        if (!SHARED || wave_live) {                           // (a chunk's rows are all live but for its last workgroup)
+            // ---- tile softmax for this lane's row; register i of tile tt is token
+            //      tile_t + tt*32 + 8*(i/4) + 4*g + i%4 ----
+            const bool all_groups_valid = (valid_lds[0] & valid_lds[1] & valid_lds[2] & valid_lds[3]) != 0;
+            const bool need_mask = !all_groups_valid ||
+                                   (SHARED ? (__any(tile_t + kPfBN > vis) != 0) : (it >= first_masked_tile));
+            // raw scores stay in s; the scale (> 0) is folded into the exponent's fma
+            if (need_mask) {                                         // one uniform branch around all 32 selects
+    #pragma unroll
+                for (int tt = 0; tt < 2; tt++)
+    #pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                        const bool ok = (tile_t + tl) < vis && valid_lds[tl >> 4] != 0;
+                        s[tt][i] = ok ? s[tt][i] : -INFINITY;
                     }
-                }
+            }
+            float tmax = -INFINITY;
+    #pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+    #pragma unroll
+                for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[tt][i]);
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));               // the row's other 32 tokens
+            const float m_new = fmaxf(m_run, tmax * A.scale_log2e);
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+            float psum = 0.0f;
+            uint4 pb[2][2];                                          // [token tile][k-half]: B operand of PV
+    #pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                float p[16];
+    #pragma unroll
+                for (int i = 0; i < 16; i++) p[i] = __builtin_amdgcn_exp2f(fmaf(s[tt][i], A.scale_log2e, -m_use));
+                pb[tt][0] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+                pb[tt][1] = make_uint4(pack2<DT>(p[8], p[9]), pack2<DT>(p[10], p[11]), pack2<DT>(p[12], p[13]), pack2<DT>(p[14], p[15]));
+                // the row sum is taken over the rounded weights, the ones PV multiplies: one dot2 per pair
+                psum = pf_sum2<DT>(pb[tt][0], psum);
+                psum = pf_sum2<DT>(pb[tt][1], psum);
+            }
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            if (!__all(alpha == 1.0f)) {
+    #pragma unroll
+                for (int dt = 0; dt < NDT; dt++)
+    #pragma unroll
+                    for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+            }
+
+            // The next tile's scores, in the same basic block as the exponentials and the PV product so
+            // that matrix and vector instructions alternate.  Unconditional: past the last tile it
+            // multiplies whatever the other K buffer holds and the result is dropped.
+            qk(it + 1, s_next);
+
+            // ---- O^T += V^T P^T : k-slot j of MFMA (tt, mh) is token tt*32 + 16*mh + 8*(j/4) + 4*g + j%4 ----
+            {
+                const int j16 = lane & 15;
+                const int dsub = 16 * ((lane >> 4) & 1) + 4 * (j16 & 3);           // d offset inside a 32-d tile
+                const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPitchV + dsub * 2;
+    #pragma unroll
+                for (int tt = 0; tt < 2; tt++)
+    #pragma unroll
+                    for (int mh = 0; mh < 2; mh++) {
+                        const uint8_t *vt = vb + (tt * 32 + 16 * mh) * kPitchV;
+    #pragma unroll
+                        for (int dt = 0; dt < NDT; dt++) {
+                            const uint2 lo = lds_read_tr16(vt + dt * 64);
+                            const uint2 hi = lds_read_tr16(vt + 8 * kPitchV + dt * 64);
+                            o[dt] = mfma32<DT>(make_uint4(lo.x, lo.y, hi.x, hi.y), pb[tt][mh], o[dt]);
+                        }
+                    }
+            }
         }
         __syncthreads();
     };
