@@ -127,8 +127,9 @@ def main():
     newv = (torch.randn(L, B, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
     out = torch.zeros(L, B, QH, D, device="cuda", dtype=torch.bfloat16)
     max_ctx = int(final.max())
-    split = args.split or lib.drk_decode_default_split(C.byref(g), B, max_ctx)
-    wsb = lib.drk_decode_workspace_bytes_for_split(C.byref(g), B, max_ctx, split)
+    split = args.split          # 0: the library's own choice (persistent workgroups, equal tiles each)
+    wsb = (lib.drk_decode_workspace_bytes_for_split(C.byref(g), B, max_ctx, split) if split
+           else lib.drk_decode_workspace_bytes(C.byref(g), B, max_ctx))
     ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
     # device arrays of positions / lengths for every step, prepared up front so the
     # timed loop does no host->device traffic
