@@ -263,6 +263,39 @@ def test_stream_kernel_group_sizes_and_head_dims(dev, geom, dtype):
         assert np.array_equal(case.run_single(b), got[b])               # one sequence per call: same bits
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_geometries_lengths_and_holes(dev, seed):
+    """A seeded draw over what the tiled kernel takes: head_dim 128 / 256, 1..16 query heads per kv head,
+    blocks of 16..256 tokens, every storage type, 1..9 branches of ragged lengths (some empty), a few
+    holes in the tables, stale bytes in unused rows -- against fp64 on the stored values."""
+    rng = np.random.default_rng(1000 + seed)
+    D = int(rng.choice([128, 256]))
+    KVH = int(rng.choice([1, 2, 4, 8]))
+    G = int(rng.choice([1, 2, 3, 4, 5, 6, 8, 12, 16]))
+    bs = int(rng.choice([16, 32, 48, 64, 256]))
+    dtype = int(rng.choice([cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3]))
+    io = dtype if dtype in (cabi.F16, cabi.BF16) else int(rng.choice([cabi.F16, cabi.BF16]))
+    B = int(rng.integers(1, 10))
+    lens = rng.integers(0, 1400, size=B)
+    lens[rng.integers(0, B)] = int(rng.choice([1, 63, 64, 65, 1023, 1024, 1025]))
+    nblk = sum((int(n) + bs - 1) // bs for n in lens)
+    holes = []
+    for _ in range(int(rng.integers(0, 4))):
+        b = int(rng.integers(0, B))
+        if lens[b] > bs:
+            holes.append((b, int(rng.integers(0, (int(lens[b]) + bs - 1) // bs))))
+    case = Case((2, KVH, KVH * G, D, bs, nblk + 3), dtype, lens, seed=seed, io_dtype=io, holes=holes,
+                outliers=bool(seed & 1), stale=0x7F if dtype in (cabi.F16, cabi.BF16) else 0x3C)
+    got = case.run_branches()
+    for b in range(B):        # a branch with no visible token leaves its rows as they were
+        if lens[b] == 0 or all((b, lb) in holes for lb in range((int(lens[b]) + bs - 1) // bs)):
+            assert np.all(got[b].view(np.uint8) == 0x7B)
+            continue
+        want = orc.decode_f64(case.og, case.q[b], case.opool, case.tables[b], case.layer, int(lens[b]), case.scale, case.io)
+        ok, ma, mr = U.rel_abs_ok(U.from_bits(got[b], case.io), want, REL, ABS)
+        assert ok, f"branch {b}: max abs err {ma:.4g}, max rel err {mr:.4g} ({D=} {KVH=} {G=} {bs=} {dtype=} lens={lens.tolist()} {holes=})"
+
+
 @pytest.mark.parametrize("dtype", [cabi.INT8, cabi.FP8_E4M3])
 @pytest.mark.parametrize("io", [cabi.F16, cabi.BF16])
 @pytest.mark.parametrize("portable", [0, 1])

@@ -197,3 +197,33 @@ def test_prefill_of_8bit_pages_and_other_head_shapes(dev, geom, dtype, io, pos_s
     assert ok, ma
     if M > 1:
         assert not np.array_equal(other, raw)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_prefill_shapes(dev, seed):
+    """A seeded draw over what the MFMA kernel takes: head_dim 128 / 256, 1..16 query heads per kv head
+    (powers of two and not), blocks of 16..256 tokens, every storage type, any chunk position and
+    length, holes, stale bytes -- against fp64 on the stored values."""
+    rng = np.random.default_rng(2000 + seed)
+    D = int(rng.choice([128, 256]))
+    KVH = int(rng.choice([1, 2, 4]))
+    G = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 12, 16]))
+    bs = int(rng.choice([16, 32, 48, 64, 256]))
+    dtype = int(rng.choice([cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3]))
+    io = dtype if dtype in (cabi.F16, cabi.BF16) else int(rng.choice([cabi.F16, cabi.BF16]))
+    pos_start = int(rng.choice([0, 1, 63, 64, 65, int(rng.integers(0, 900))]))
+    M = int(rng.choice([1, 31, 32, 33, 127, 128, 129, int(rng.integers(1, 400))]))
+    total = pos_start + M
+    nblk = (total + bs - 1) // bs
+    holes = tuple(int(h) for h in rng.choice(nblk, size=min(nblk - 1, int(rng.integers(0, 3))), replace=False)) if nblk > 1 else ()
+    geom = (2, KVH, KVH * G, D, bs, nblk + 3)
+    g, og, rng2, table, opool = build_io(geom, dtype, io, total, seed=seed, holes=holes, mul=0.7)
+    q = U.normal_bits(rng2, (M, KVH * G, D), io, 0.7)
+    scale = 1 / np.sqrt(D)
+    got = run_prefill(g, U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table), 1, pos_start, M, scale, io, KVH * G, D)
+    want = orc.prefill_f64(og, q, opool, table, 1, pos_start, scale, io)
+    # a row that sees no token (every page before it is a hole) keeps the bytes the caller left in out
+    seen = np.array([any(table[t // bs] >= 0 for t in range(pos_start + r + 1)) for r in range(M)])
+    assert np.all(got[~seen].view(np.uint8) == 0x7B)
+    ok, ma, _ = U.rel_abs_ok(U.from_bits(got[seen], io), want[seen])
+    assert ok, f"max abs err {ma:.4g} ({D=} {KVH=} {G=} {bs=} {dtype=} {pos_start=} {M=} {holes=})"
