@@ -67,6 +67,26 @@ __device__ __forceinline__ float row16_max(float v)
     return v;
 }
 
+// The 8 codes of chunk c of a row: the even lane of each lane pair takes its neighbour's
+// 8 bytes (chunks of one row sit in consecutive lanes, so both belong to the same row) and
+// stores 16 (fp8 bulk append 4.60 -> 5.02 TB/s against 8-byte stores from every lane);
+// every lane of the wave must call this.
+__device__ __forceinline__ void store_codes(uint8_t *__restrict__ row, unsigned c, unsigned rc, uint32_t lo, uint32_t hi,
+                                            bool ok)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (rc < 2) {                                            // a row of one chunk has no neighbour
+        if (ok) st_stream64(row, make_uint2(lo, hi));
+        return;
+    }
+    const uint32_t lo_n = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)lo, 0xB1, 0xf, 0xf, false);
+    const uint32_t hi_n = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)hi, 0xB1, 0xf, 0xf, false);
+    if (ok && !(c & 1u)) st_stream128(row + (size_t)c * 8, make_uint4(lo, hi, lo_n, hi_n));
+#else
+    (void)row; (void)c; (void)rc; (void)lo; (void)hi; (void)ok;
+#endif
+}
+
 // Store one source chunk (8 elements of type src_dtype, `val`) into the page row at byte
 // offset poff as chunk c of its row.  rc = chunks per row; the rc lanes that hold one row
 // are consecutive lanes of one wave (rc is a power of two <= 64), and every lane of the
@@ -104,14 +124,12 @@ __device__ __forceinline__ void store_page_chunk(uint8_t *__restrict__ pool, siz
                 uint32_t b = (uint32_t)((int)r) & 0xffu;
                 if (i < 4) lo |= b << (8 * i); else hi |= b << (8 * (i - 4));
             }
-            if (ok) {
-                st_stream64(pool + poff + (size_t)c * 8, make_uint2(lo, hi));
-                if (c == 0) *(uint16_t *)(pool + soff) = sh;
-            }
+            store_codes(pool + poff, c, rc, lo, hi, ok);
+            if (ok && c == 0) *(uint16_t *)(pool + soff) = sh;
         } else {
             uint32_t lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
             uint32_t hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
-            if (ok) st_stream64(pool + poff + (size_t)c * 8, make_uint2(lo, hi));
+            store_codes(pool + poff, c, rc, lo, hi, ok);
         }
     }
 }
