@@ -116,14 +116,18 @@ __device__ __forceinline__ void store_page_chunk(uint8_t *__restrict__ pool, siz
             if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
             float sf = f16_bits_to_f(sh);
             float rcp = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
-            uint32_t lo = 0, hi = 0;
+            // code = clamp(rint(x * rcp), -127, 127).  The clamp bounds are integers, so it may run before
+            // the rounding, and adding 1.5 * 2^23 rounds to the nearest integer, ties to even, exactly as
+            // rint does -- and leaves the code's two's-complement byte as the low byte of the sum.
+            uint32_t u[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                float r = rintf(__fmul_rn(x[i], rcp));
+                float r = __fmul_rn(x[i], rcp);
                 r = fminf(fmaxf(r, -127.0f), 127.0f);
-                uint32_t b = (uint32_t)((int)r) & 0xffu;
-                if (i < 4) lo |= b << (8 * i); else hi |= b << (8 * (i - 4));
+                u[i] = __float_as_uint(__fadd_rn(r, 12582912.0f));
             }
+            const uint32_t lo = s_perm(s_perm(u[3], u[2], 0x04000c0cu), s_perm(u[1], u[0], 0x0c0c0400u), 0x07060100u);
+            const uint32_t hi = s_perm(s_perm(u[7], u[6], 0x04000c0cu), s_perm(u[5], u[4], 0x0c0c0400u), 0x07060100u);
             store_codes(pool + poff, c, rc, lo, hi, ok);
             if (ok && c == 0) *(uint16_t *)(pool + soff) = sh;
         } else {

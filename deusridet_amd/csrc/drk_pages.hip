@@ -16,8 +16,8 @@ constexpr int kThreads = 256;
 // Plain copies run best in many short workgroups -- measured on 2 048 tokens x 36 layers, 8 x 128
 // bf16: append 5.14 / 5.39 / 5.57 TB/s at 2 048 / 512 / 256 chunks per workgroup, extract 5.78 /
 // 5.94 / 5.80, inject 5.06 / 5.35 / 5.42 -- the quantising modes with four rounds of loads in
-// flight, int8 twice per workgroup (4.3 TB/s; 4.0-4.2 at 1 024), fp8 once (5.0 TB/s; 4.7 at 2 048).
-int g_copy_chunks = 256, g_flat_chunks = 512, g_quant_chunks = 0;      // 0: 2 048 for int8, 1 024 for fp8
+// flight once per workgroup (1 024 chunks: int8 4.3 TB/s, fp8 5.0; 4.15 and 4.7 at 2 048).
+int g_copy_chunks = 256, g_flat_chunks = 512, g_quant_chunks = 1024;
 static int tokens_per_group(unsigned chunks_per_token, int target_chunks)
 {
     const unsigned target = (unsigned)target_chunks;
@@ -226,9 +226,7 @@ static int launch_append(const drk_kv_layout *g, void *pool, const int32_t *tabl
             return fail(DRK_ERR_UNSUPPORTED, "append: quantising pools need head_dim in {8..512} power of two, got %d", a.D);
     }
     Div tok_div = mk_div((unsigned)a.KVH * rowc), row_div = mk_div(rowc), bs_div = mk_div((unsigned)a.bs);
-    const int tpg = tokens_per_group((unsigned)a.KVH * rowc, a.dtype == DRK_INT8       ? (g_quant_chunks ? g_quant_chunks : 2048)
-                                                             : a.dtype == DRK_FP8_E4M3 ? (g_quant_chunks ? g_quant_chunks : 1024)
-                                                                                       : g_copy_chunks);
+    const int tpg = tokens_per_group((unsigned)a.KVH * rowc, (a.dtype == DRK_INT8 || a.dtype == DRK_FP8_E4M3) ? g_quant_chunks : g_copy_chunks);
     dim3 grid((ntokens + tpg - 1) / tpg, layer_count, 2);
     hipStream_t s = (hipStream_t)stream;
 #define GO(Q)                                                                                       \
@@ -280,7 +278,7 @@ void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chu
 {
     g_copy_chunks = copy_chunks > 0 ? copy_chunks : 256;
     g_flat_chunks = flat_chunks > 0 ? flat_chunks : 512;
-    g_quant_chunks = quant_chunks > 0 ? quant_chunks : 0;
+    g_quant_chunks = quant_chunks > 0 ? quant_chunks : 1024;
 }
 
 int drk_kv_append_token(const drk_kv_layout *g, void *pool, const int32_t *d_block_table, int layer,

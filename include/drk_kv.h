@@ -202,7 +202,7 @@ int  drk_debug_decode_kernel_times(float *ms, int cap, int *count);
 /* Diagnostic: extra dynamic LDS bytes per decode workgroup (lowers occupancy). */
 void drk_debug_set_decode_lds_pad(int bytes);
 /* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
- * extract / inject, and in the quantising append (0 = default: 256, 512, 2048 for int8 / 1024 for fp8). */
+ * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */
 void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chunks);
 /* paged_gqa_decode_attention, paged_attention.cu:179-282: one sequence.
  * q/out [num_q_heads, head_dim] of io_dtype (F16/BF16). */
