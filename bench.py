@@ -26,7 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), scaled by what the same
 # counters read for a plain 32 GiB read (x2.0) and a bulk append of known size
 # (x1.0).  Keyed by the algorithmic bytes of the launch it was measured on.
-MEASURED_TRAFFIC_BYTES = {1073741824: int((524638.0 * 2 + 1340.7) * 1024)}
+MEASURED_TRAFFIC_BYTES = {1073741824: int((524763.5 * 2 + 1850.5) * 1024)}
 
 
 def parse():
@@ -42,6 +42,7 @@ def parse():
     ap.add_argument("--pool-gb", type=float, default=40.0)
     ap.add_argument("--split", type=int, default=0, help="tokens per split-K workgroup (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-ragged", action="store_true", help="skip the ragged-context launches of the decode kernel (profiling: keeps one shape per kernel name)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="context per branch for the CPU sample (0 = auto)")
     ap.add_argument("--bulk-append-tokens", type=int, default=2048)
     ap.add_argument("--seed", type=int, default=2)
@@ -231,7 +232,7 @@ def main():
     # ---- the same kernel on config 2's context distribution, U{1024..32768} per branch (same pool and
     # tables; only the lengths change), when the headline run is the fixed 32k point
     ragged = None
-    if args.ctx_mode == "fixed":
+    if args.ctx_mode == "fixed" and not args.no_ragged:
         rl = np.random.default_rng(args.seed + 1).integers(1024, min(args.ctx, max_ctx) + 1, size=B).astype(np.int32)
         rlen = torch.from_numpy(rl).cuda()
 
