@@ -515,6 +515,8 @@ void orc_prefill_f64(const orc_layout *g, const uint16_t *Q, const void *pool,
                      int M, double scale, int io_dtype)
 {
     size_t row = (size_t)g->QH * g->D;
+    /* rows are independent (each call allocates its own scratch): the threads only shorten the tests */
+#pragma omp parallel for schedule(dynamic, 4)
     for (int t = 0; t < M; t++)
         orc_decode_f64(g, Q + t * row, pool, table, out + t * row, layer,
                        pos_start + t + 1, scale, io_dtype);
