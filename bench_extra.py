@@ -345,6 +345,31 @@ def config5(args):
     tfl = pf_flops / (pf_ms * 1e-3) / 1e12
     nchunks = (passes - 1) * (total // chunk)
     ap_gbps = nchunks * L * chunk * 2 * (2 * KVH * D * 2) / (ap_ms * 1e-3) / 1e9
+    # a short chunk at the end of the same context (a perception frame of a few tokens): the chunk kernel
+    # against the path that splits the context over the chip
+    short = {}
+    for rows in (16, 64):
+        pos = total - rows
+        qs = torch.randn(rows, QH, D, device="cuda").to(torch.bfloat16)
+        os_ = torch.empty_like(qs)
+        us = []
+        for mode in (0, -1):
+            lib.drk_debug_set_prefill_split(mode)
+            wsb_s = lib.drk_prefill_workspace_bytes(C.byref(g), pos, rows)
+            ws_s = torch.empty(max(wsb_s, 256), dtype=torch.uint8, device="cuda")
+
+            def go(n):
+                for i in range(n):
+                    cabi.call("drk_paged_prefill_attention", C.byref(g), U.p(qs), U.p(pool), U.p(tab_seq), U.p(os_), i % L, pos, rows,
+                              float(scale), cabi.BF16, U.p(ws_s), wsb_s, sp)
+            go(3)
+            ev[0].record(stream)
+            go(20)
+            ev[1].record(stream)
+            torch.cuda.synchronize()
+            us.append(ev[0].elapsed_time(ev[1]) / 20 * 1e3)
+        lib.drk_debug_set_prefill_split(-1)
+        short[f"{rows}_rows_at_{pos}"] = {"chunk_kernel_us": round(us[0], 1), "context_split_us": round(us[1], 1)}
     return {
         "metric": "chunked_prefill_attention_TFLOPs", "value": round(tfl, 1), "unit": "TFLOP/s", "n_gpus": 1,
         "steps": nchunks, "warmup": total // chunk, "ms_per_step": round(pf_ms / nchunks / L, 4),
@@ -356,6 +381,7 @@ def config5(args):
                                f"(chunk, layer) attention launch", "layers": L},
         "chunk_append_GBps": round(ap_gbps, 1),
         "interleaved_decode_us_per_layer": round(float(np.mean(dec_ms)) / L * 1e3, 1),
+        "short_chunk_attention": short,
         "roofline": {"kernel": f"prefill_mfma_kernel<{kv_name}>", "bound": "mfma", "achieved": round(tfl, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tfl / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": None},

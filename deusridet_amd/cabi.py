@@ -84,6 +84,7 @@ SIGNATURES = {
     "drk_debug_time_decode_kernel": (None, [_i32]),
     "drk_debug_set_decode_lds_pad": (None, [_i32]),
     "drk_debug_set_append_chunks": (None, [_i32, _i32, _i32]),
+    "drk_debug_set_prefill_split": (None, [_i32]),
     "drk_probe_read_bandwidth": (_i32, [_vp, _sz, _i32, _vp, C.POINTER(C.c_float)]),
     "drk_debug_decode_kernel_times": (_i32, [C.POINTER(C.c_float), _i32, C.POINTER(_i32)]),
     "drk_paged_decode_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),

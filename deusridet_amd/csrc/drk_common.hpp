@@ -69,7 +69,7 @@ int launch_sigmoid_gate(const void *x, const void *gate, void *out, size_t rows,
 extern int g_stream_wgs;
 extern int g_shared_splits;
 bool stream_decode_supported(const Lay &a, int B);
-size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens);
+size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens, int start_tile = 0);
 int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
                          float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
@@ -79,6 +79,12 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
                          int lse_stride = 0);
 int launch_block_mass(const float *lse_groups, const float *lse_rows, const int32_t *d_seq_lens, int B, int QH,
                       int lse_stride, int bs, float *mass, int mass_stride, int accumulate, hipStream_t st);
+// branches over a shared prefix: prefix pass + tails + one merge (drk_decode.hip); table_stride 0 = one table for all
+size_t shared_workspace_need(const Lay &a, int B, int max_seq_len, int shared);
+int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
+                         int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, int shared_tokens,
+                         void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
+                         void *stream, const void *gate = nullptr, size_t gate_stride = 0);
 // shared-prefix pass on the matrix cores (drk_prefill.hip)
 void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,

@@ -599,10 +599,15 @@ static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size
 {
     int ct, ns;
     shared_prefix_shape(shared, &ct, &ns);
-    size_t sp = stream_workspace_need(a, B, max_seq_len, 0);
+    size_t sp = stream_workspace_need(a, B, max_seq_len, 0, shared / kTile);
     sp = (sp + 255) & ~(size_t)255;
     if (stream_part) *stream_part = sp;
     return sp + (size_t)B * a.QH * ns * (a.D + 2) * sizeof(float);
+}
+
+size_t shared_workspace_need(const Lay &a, int B, int max_seq_len, int shared)
+{
+    return shared_need(a, B, max_seq_len, (shared / kTile) * kTile, nullptr);
 }
 
 static bool shared_path_ok(const Lay &a, int B, int shared)
@@ -614,7 +619,7 @@ static bool shared_path_ok(const Lay &a, int B, int shared)
 int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                          int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, int shared_tokens,
                          void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
-                         void *stream)
+                         void *stream, const void *gate, size_t gate_stride)
 {
     Lay a;
     int rc = make_lay(g, &a);
@@ -622,7 +627,7 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
     const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
     if (!shared_path_ok(a, B, shared) || shared > max_seq_len || !(scale > 0.0f))
         return launch_decode(g, q, pool, tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
-                             io_dtype, 0, workspace, workspace_bytes, stream);
+                             io_dtype, 0, workspace, workspace_bytes, stream, gate, gate_stride);
     if (!q || !pool || !tables || !out || !d_seq_lens) return fail(DRK_ERR_INVALID, "decode: NULL pointer");
     if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode: io_dtype must be F16 or BF16");
     if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
@@ -653,7 +658,7 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
                                    io_dtype, 0, workspace, false, st, shared / kTile))) return rc;
     if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
     return launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
-                                io_dtype, 0, workspace, true, st, shared / kTile, pre_o, pre_m, pre_l, ns);
+                                io_dtype, 0, workspace, true, st, shared / kTile, pre_o, pre_m, pre_l, ns, gate, gate_stride);
 }
 
 } // namespace drk

@@ -761,7 +761,8 @@ bool stream_decode_supported(const Lay &a, int B)
            B >= 1 && B <= 64 && a.layer_stride <= (0xffff0000ull << 4);
 }
 
-static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens, int *grid, int *unit_tiles, int *Pmax)
+static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens, int start_tile, int *grid, int *unit_tiles,
+                         int *Pmax)
 {
     const long t_upper = (long)a.KVH * B * ((max_seq_len + kSTile - 1) / kSTile);
     if (split_tokens > 0) {
@@ -775,13 +776,17 @@ static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens,
         *unit_tiles = 0;
         *grid = (int)G;
         *Pmax = (int)((G + a.KVH - 1) / a.KVH) + 2;
+        // a branch's run of n tiles meets at most n + 1 workgroups: short private tails behind a long
+        // shared prefix (start_tile > 0) need far fewer pieces than the grid could give one branch
+        const int tail_tiles = (max_seq_len + kSTile - 1) / kSTile - start_tile;
+        if (start_tile > 0 && tail_tiles + 2 < *Pmax) *Pmax = (tail_tiles > 0 ? tail_tiles : 0) + 2;
     }
 }
 
-size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens)
+size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens, int start_tile)
 {
     int grid, U, Pmax;
-    stream_shape(a, B, max_seq_len, split_tokens, &grid, &U, &Pmax);
+    stream_shape(a, B, max_seq_len, split_tokens, start_tile, &grid, &U, &Pmax);
     return (size_t)B * a.QH * Pmax * (a.D + 2) * sizeof(float);
 }
 
@@ -793,7 +798,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
                          const void *gate, size_t gate_stride, float *lse_groups, float *lse_rows, int lse_stride)
 {
     int grid, U, Pmax;
-    stream_shape(a, B, max_seq_len, split_tokens, &grid, &U, &Pmax);
+    stream_shape(a, B, max_seq_len, split_tokens, start_tile, &grid, &U, &Pmax);
     float *part_o = (float *)workspace;
     float *part_m = part_o + (size_t)B * a.QH * Pmax * a.D;
     float *part_l = part_m + (size_t)B * a.QH * Pmax;

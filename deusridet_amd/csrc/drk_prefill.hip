@@ -581,11 +581,77 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     return DRK_OK;
 }
 
+// ---- short chunks behind a long context ------------------------------------------------
+// The chunk kernel walks the whole context in every workgroup and has ceil(M / 32) x KVH of
+// them: a chunk of a few tokens behind 32k tokens keeps 8 of 256 CUs busy for a millisecond.
+// Such a chunk is the shared-prefix decode over again -- row t is a "branch" of length
+// pos_start + t + 1, all rows read one table -- so it runs through that machinery: the
+// context is split over the whole chip (matrix-core pass over the tokens every row sees, the
+// stream kernel over the last few, one merge), 64 rows per round.
+// When it pays (measured, 32 Q / 8 KV x 128 bf16): the chunk kernel takes 27 us per 1 024 tokens of
+// context whatever the chunk length up to 1 024 rows; a round of 64 rows here takes 50 us + 1.7 us per
+// 1 024 tokens (56 / 70 / 109 / 269 us behind 2k / 8k / 32k / 128k).  16 rows behind 32k: 874 -> 52 us;
+// 64 behind 128k: 3 955 -> 269 us; 256 behind 32k: 871 -> 423 us.
+int g_prefill_split = -1;                      // -1: by that rule; 0: never; n > 0: every chunk of up to n rows (tests)
+constexpr int kSplitRows = 64;                 // rows per round: the stream kernel's branch limit
+constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024;
+
+__global__ void iota_kernel(int32_t *__restrict__ dst, int n, int first)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = first + i;
+}
+
+static bool prefill_split_applies(const Lay &a, int pos_start, int M)
+{
+    if (g_prefill_split == 0 || pos_start < kSplitMinPos || !stream_decode_supported(a, M < kSplitRows ? M : kSplitRows))
+        return false;
+    if (g_prefill_split > 0) return M <= g_prefill_split;
+    const int rounds = (M + kSplitRows - 1) / kSplitRows;
+    return M <= kSplitMaxM && rounds * (50.0f + pos_start / 580.0f) < 0.027f * pos_start;
+}
+
+static size_t prefill_split_need(const Lay &a, int pos_start, int M, size_t *lens_bytes)
+{
+    const size_t lb = ((size_t)M * sizeof(int32_t) + 255) & ~(size_t)255;
+    if (lens_bytes) *lens_bytes = lb;
+    size_t need = 0;
+    for (int r0 = 0; r0 < M; r0 += kSplitRows) {
+        const int B = M - r0 < kSplitRows ? M - r0 : kSplitRows;
+        const size_t n = shared_workspace_need(a, B, pos_start + r0 + B, pos_start + r0 + 1);
+        if (n > need) need = n;
+    }
+    return lb + need;
+}
+
+static int prefill_split(const drk_kv_layout *g, const Lay &a, const void *q, const void *pool, const int32_t *table,
+                         void *out, int layer, int pos_start, int M, float scale, int io_dtype, void *workspace,
+                         size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
+{
+    size_t lb;
+    prefill_split_need(a, pos_start, M, &lb);
+    int32_t *lens = (int32_t *)workspace;
+    hipLaunchKernelGGL(iota_kernel, dim3((M + 255) / 256), dim3(256), 0, (hipStream_t)stream, lens, M, pos_start + 1);
+    DRK_LAUNCH_CHECK("iota_kernel");
+    const size_t row = (size_t)a.QH * a.D * 2;
+    for (int r0 = 0; r0 < M; r0 += kSplitRows) {
+        const int B = M - r0 < kSplitRows ? M - r0 : kSplitRows;
+        const uint16_t *grow = gate ? (const uint16_t *)gate + (size_t)r0 * a.QH * gate_stride : nullptr;
+        const int rc = launch_decode_shared(g, (const uint8_t *)q + r0 * row, pool, table, 0, lens + r0, B, pos_start + r0 + B,
+                                            pos_start + r0 + 1, (uint8_t *)out + r0 * row, layer, scale, io_dtype,
+                                            (uint8_t *)workspace + lb, workspace_bytes - lb, stream, grow, gate_stride);
+        if (rc) return rc;
+    }
+    return DRK_OK;
+}
+
 } // namespace drk
 
 using namespace drk;
 
 extern "C" {
+
+void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
 
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 {
@@ -593,7 +659,7 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
     const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 &&
                       (a.bs % 16) == 0;
-    if (mfma) return 0;
+    if (mfma) return prefill_split_applies(a, pos_start, M) ? prefill_split_need(a, pos_start, M, nullptr) : 0;
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
@@ -625,6 +691,12 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     if (a.KVH > 65535) return fail(DRK_ERR_INVALID, "prefill: more than 65535 kv heads");
     if (gate && (gate_stride < (size_t)a.D || (gate_stride % 8) || ((uintptr_t)gate % 16)))
         return fail(DRK_ERR_INVALID, "prefill: gate rows must be 16-byte aligned and at least head_dim apart");
+    // a short chunk behind a long context: split the context over the chip (needs the workspace
+    // drk_prefill_workspace_bytes reports; without it the chunk kernel below does the work)
+    if (prefill_split_applies(a, pos_start, M) && workspace && ((uintptr_t)workspace % 256) == 0 &&
+        workspace_bytes >= prefill_split_need(a, pos_start, M, nullptr))
+        return prefill_split(g, a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
+                             workspace_bytes, stream, gate, gate_stride);
     PrefillArgs A;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
     A.table = d_block_table;

@@ -49,6 +49,13 @@ bool paged_attention_reserve_workspace(int max_branches, int max_seq_len, int ma
         const int rows = max_prefill_rows < max_seq_len ? max_prefill_rows : max_seq_len;
         size_t p = drk_prefill_workspace_bytes(&g, max_seq_len - rows, rows);
         if (p > need) need = p;
+        // ... and a short chunk behind a long context runs with the context split over the chip, which
+        // keeps partial results: room for any chunk length up to max_prefill_rows
+        for (int m = 64; m <= 256; m *= 2) {
+            const int r = m < rows ? m : rows;
+            p = drk_prefill_workspace_bytes(&g, max_seq_len - r, r);
+            if (p > need) need = p;
+        }
     }
     return need == 0 || workspace(need) != nullptr;
 }

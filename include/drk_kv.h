@@ -201,6 +201,9 @@ void drk_debug_time_decode_kernel(int on);
 int  drk_debug_decode_kernel_times(float *ms, int cap, int *count);
 /* Diagnostic: extra dynamic LDS bytes per decode workgroup (lowers occupancy). */
 void drk_debug_set_decode_lds_pad(int bytes);
+/* Tuning: which prefill chunks run with the context split over the chip (they must stand behind 2 048 tokens
+ * or more): negative = the library's cost rule (default); 0 = none; n = every chunk of up to n rows. */
+void drk_debug_set_prefill_split(int max_rows);
 /* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
  * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */
 void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chunks);
@@ -243,9 +246,14 @@ int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, con
  * q/out [M, num_q_heads, head_dim]; row t attends to tokens 0..pos_start+t (the
  * chunk's own K/V must already be in the pages: write, then attend).
  * head_dim 128 or 256 with block_size % 16 == 0 (any storage type, any number of query
- * heads per KV head up to 128) runs on the MFMA prefill kernel and needs no workspace
- * (drk_prefill_workspace_bytes returns 0); anything else row by row through the portable
- * decode kernel, which needs the workspace. */
+ * heads per KV head up to 128) runs on the MFMA prefill kernel, which needs no workspace.
+ * A short chunk behind a long context (up to 64 rows behind 2 048 tokens, more behind
+ * more; at most 16 query heads per KV head) is spread over the whole chip instead -- the
+ * context split as in drk_paged_decode_attention_shared, rows = the chunk's tokens -- when
+ * the workspace drk_prefill_workspace_bytes reports for it is passed (256-byte aligned);
+ * without that workspace the MFMA kernel does the work, some 10-30 times slower for such a
+ * chunk.  Anything else runs row by row through the portable decode kernel, which needs
+ * the workspace. */
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M);
 int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
                                 const int32_t *d_block_table, void *out, int layer,
