@@ -375,3 +375,45 @@ def test_time_division_perception_between_decode_steps_and_a_changing_branch_cou
     assert np.array_equal(s.pool(), opool)
     s.ks.close_branches()
     assert s.cm.gpu_blocks_used() == 9                        # 144 tokens of the stream
+
+
+def test_perception_frames_behind_a_long_context(dev):
+    """Frames of a few tokens after 2 112 tokens of context: prefill_layer then runs with the context
+    split over the chip (rows = the frame's tokens) instead of the chunk kernel -- same pool bits, same
+    outputs within the attention tolerance."""
+    global NPOS, POOL_BLOCKS
+    saved = (NPOS, POOL_BLOCKS)
+    NPOS, POOL_BLOCKS = 2304, 160
+    try:
+        s = Session(1)
+        rng = np.random.default_rng(7)
+        qw, kw = U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT)
+        s.set_weights(qw, kw)
+        st = U.stream_ptr()
+        og = orc.layout(L, KVH, QH, D, BS, s.NB, KVDT)
+        opool = orc.new_pool(og)
+        g = cabi.layout(L, KVH, QH, D, BS, s.NB, KVDT)
+        for M, check in [(64, False)] * 33 + [(5, True), (17, True), (1, True)]:
+            pos0 = s.ks.current_pos()
+            # from 2 048 tokens on, frames take the split path: it is the one that asks for a workspace
+            assert (cabi.lib().drk_prefill_workspace_bytes(C.byref(g), pos0, M) > 0) == (pos0 >= 2048)
+            assert s.ks.begin_prefill(M, st)
+            table0 = s.cm.h_block_table(0).copy()
+            pos = (pos0 + np.arange(M)).astype(np.int32)
+            for layer in range(L):
+                qg, k, v = (U.normal_bits(rng, sh, DT, m) for sh, m in (((M, QH, 2 * D), 1.0), ((M, KVH, D), 0.7), ((M, KVH, D), 0.5)))
+                s.load(qg, k, v)
+                s.ks.prefill_layer(layer, s.io(), M, st)
+                if check:
+                    got = s.out(M)
+                    want = oracle_layer(og, opool, [table0] * M, pos, layer, qg, k, v, qw, kw, s.tab)
+                    ok, mx, _ = U.rel_abs_ok(U.from_bits(got, DT), want)
+                    assert ok, (M, layer, mx)
+                else:                                                  # the context itself: only the pages are mirrored
+                    kr = orc.apply_rope(orc.head_norm(k, kw, EPS, DT).reshape(M, KVH, D), pos, s.tab, RD, DT)
+                    orc.append_batch(og, opool, table0, layer, pos0, kr, v, DT)
+            s.ks.end_prefill(M)
+        assert s.ks.current_pos() == 33 * 64 + 23
+        assert np.array_equal(s.pool(), opool)
+    finally:
+        NPOS, POOL_BLOCKS = saved
