@@ -80,7 +80,6 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
 int launch_block_mass(const float *lse_groups, const float *lse_rows, const int32_t *d_seq_lens, int B, int QH,
                       int lse_stride, int bs, float *mass, int mass_stride, int accumulate, hipStream_t st);
 // branches over a shared prefix: prefix pass + tails + one merge (drk_decode.hip); table_stride 0 = one table for all
-size_t shared_workspace_need(const Lay &a, int B, int max_seq_len, int shared);
 int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                          int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, int shared_tokens,
                          void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
@@ -89,7 +88,8 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
 void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
                          const int32_t *d_seq_lens, int B, int shared, int layer, float scale, int io_dtype,
-                         float *part_o, float *part_m, float *part_l, hipStream_t st);
+                         float *part_o, float *part_m, float *part_l, hipStream_t st, int chunk_tiles = 0,
+                         int nsplits = 0);
 
 // ---- element helpers (device) -------------------------------------------
 // Streaming ("non-temporal") 128- and 64-bit accesses for data that is touched once

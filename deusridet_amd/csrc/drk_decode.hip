@@ -605,11 +605,6 @@ static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size
     return sp + (size_t)B * a.QH * ns * (a.D + 2) * sizeof(float);
 }
 
-size_t shared_workspace_need(const Lay &a, int B, int max_seq_len, int shared)
-{
-    return shared_need(a, B, max_seq_len, (shared / kTile) * kTile, nullptr);
-}
-
 static bool shared_path_ok(const Lay &a, int B, int shared)
 {
     // the prefix pass is the MFMA prefill kernel in its shared mode (every shape the stream kernel takes)

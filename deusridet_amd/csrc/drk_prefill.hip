@@ -549,7 +549,7 @@ void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits)
 
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
                          const int32_t *d_seq_lens, int B, int shared, int layer, float scale, int io_dtype,
-                         float *part_o, float *part_m, float *part_l, hipStream_t st)
+                         float *part_o, float *part_m, float *part_l, hipStream_t st, int chunk_tiles, int nsplits)
 {
     PrefillArgs A;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
@@ -561,7 +561,8 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
     A.scale_log2e = scale * kLog2eP;
     A.seq_lens = d_seq_lens; A.shared = shared;
-    shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
+    if (nsplits > 0) { A.chunk_tiles = chunk_tiles; A.nsplits = nsplits; }      // the caller's split (shared need not be whole tiles)
+    else shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
     A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
     A.gate = nullptr; A.gate_stride = 0;
     dim3 grid(((B + A.tpw - 1) / A.tpw) * a.KVH, 1, A.nsplits);
@@ -582,19 +583,14 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 }
 
 // ---- short chunks behind a long context ------------------------------------------------
-// The chunk kernel walks the whole context in every workgroup and has ceil(M / 32) x KVH of
+// The chunk kernel walks the whole context in every workgroup and has ceil(M / TPW) x KVH of
 // them: a chunk of a few tokens behind 32k tokens keeps 8 of 256 CUs busy for a millisecond.
-// Such a chunk is the shared-prefix decode over again -- row t is a "branch" of length
-// pos_start + t + 1, all rows read one table -- so it runs through that machinery: the
-// context is split over the whole chip (matrix-core pass over the tokens every row sees, the
-// stream kernel over the last few, one merge), 64 rows per round.
-// When it pays (measured, 32 Q / 8 KV x 128 bf16): the chunk kernel takes 27 us per 1 024 tokens of
-// context whatever the chunk length up to 1 024 rows; a round of 64 rows here takes 50 us + 1.7 us per
-// 1 024 tokens (56 / 70 / 109 / 269 us behind 2k / 8k / 32k / 128k).  16 rows behind 32k: 874 -> 52 us;
-// 64 behind 128k: 3 955 -> 269 us; 256 behind 32k: 871 -> 423 us.
-int g_prefill_split = -1;                      // -1: by that rule; 0: never; n > 0: every chunk of up to n rows (tests)
-constexpr int kSplitRows = 64;                 // rows per round: the stream kernel's branch limit
-constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024;
+// Such a chunk is the shared-prefix pass over again -- row t is a "branch" of length
+// pos_start + t + 1, all rows read one table -- so the kernel runs in that mode over tokens
+// [0, pos_start + M) with the context split over the whole chip, and a small kernel folds each
+// row's pieces (and applies the gate).
+int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
+constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
 
 __global__ void iota_kernel(int32_t *__restrict__ dst, int n, int first)
 {
@@ -602,46 +598,149 @@ __global__ void iota_kernel(int32_t *__restrict__ dst, int n, int first)
     if (i < n) dst[i] = first + i;
 }
 
+// grid = rows (query token x query head), block = 64: lane s owns the (m, l) of piece s (at most 128
+// pieces: two per lane), so the weights come in one round of loads; then the lanes own dims
+// [l VEC, l VEC + VEC) and fold the o rows eight at a time.  Pieces are unnormalised (o, m, l) in the
+// base-2 exponent domain; an empty piece carries l = 0 and may hold anything else.
+__device__ __forceinline__ float pm_lane(float v, int l)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+#else
+    (void)l;
+    return v;
+#endif
+}
+
+template <int D>
+__global__ __launch_bounds__(64) void prefill_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_m,
+                                                           const float *__restrict__ part_l, uint16_t *__restrict__ out,
+                                                           int nsplits, int io_dtype, const uint16_t *__restrict__ gate,
+                                                           size_t gate_stride)
+{
+    constexpr int VEC = D / 64;
+    typedef float fvec __attribute__((ext_vector_type(VEC)));
+    const size_t row = blockIdx.x;
+    const int lane = threadIdx.x, d = lane * VEC;
+    float pm[2], pl[2], w[2];
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const int sidx = lane + 64 * r;
+        pl[r] = sidx < nsplits ? part_l[row * nsplits + sidx] : 0.0f;
+        pm[r] = sidx < nsplits ? part_m[row * nsplits + sidx] : -INFINITY;
+    }
+    float M = fmaxf(pl[0] > 0.0f ? pm[0] : -INFINITY, pl[1] > 0.0f ? pm[1] : -INFINITY);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
+    float L = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        w[r] = pl[r] > 0.0f ? __builtin_amdgcn_exp2f(pm[r] - M) : 0.0f;
+        L = fmaf(pl[r], w[r], L);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off);
+    fvec acc = {};
+    const float *obase = part_o + row * nsplits * D + d;
+    for (int j = 0; j < nsplits; j += 8) {
+        fvec o[8];
+        float wj[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const int sj = min(j + u, nsplits - 1);
+            const float ws = sj < 64 ? pm_lane(w[0], sj) : pm_lane(w[1], sj - 64);
+            wj[u] = j + u < nsplits ? ws : 0.0f;
+            o[u] = *(const fvec *)(obase + (size_t)sj * D);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (wj[u] != 0.0f) {
+#pragma unroll
+                for (int x = 0; x < VEC; x++) acc[x] = fmaf(o[u][x], wj[u], acc[x]);
+            }
+    }
+    // with a gate the row is always rewritten: the reference gates whatever the attention kernel
+    // left in out, also when no token took part (paged_attention.cu:551, 633-634)
+    uint16_t *dst = out + row * D + d;
+    uint16_t vals[VEC];
+    if (L > 0.0f) {
+#pragma unroll
+        for (int x = 0; x < VEC; x++) vals[x] = f_to_elem16(acc[x] / L, io_dtype);
+    } else {
+        if (!gate) return;
+#pragma unroll
+        for (int x = 0; x < VEC; x++) vals[x] = dst[x];
+    }
+    if (gate) {
+        const uint16_t *gp = gate + row * gate_stride + d;
+#pragma unroll
+        for (int x = 0; x < VEC; x++) vals[x] = gated_elem16(vals[x], gp[x], io_dtype);
+    }
+#pragma unroll
+    for (int x = 0; x < VEC; x++) dst[x] = vals[x];
+}
+
+// context splits: two workgroups per CU over the whole grid -- one resident round -- of whole tiles each
+static void prefill_split_shape(const Lay &a, int pos_start, int M, int *chunk_tiles, int *nsplits)
+{
+    const int tpw = 128 / (a.QH / a.KVH);
+    const int per_split = ((M + tpw - 1) / tpw) * a.KVH;
+    const int tiles = (pos_start + M + kPfBN - 1) / kPfBN;
+    int ns = (512 + per_split - 1) / per_split;
+    if (ns > kSplitMaxPieces) ns = kSplitMaxPieces;
+    if (ns > tiles) ns = tiles;
+    if (ns < 1) ns = 1;
+    *chunk_tiles = (tiles + ns - 1) / ns;
+    *nsplits = (tiles + *chunk_tiles - 1) / *chunk_tiles;
+}
+
+// When it pays (measured, 32 Q / 8 KV x 128 bf16): the chunk kernel takes 27 us per 1 024 tokens of
+// context whatever the chunk length up to 1 024 rows (one workgroup per CU at most); the split pass
+// keeps every CU busy.  Rows behind 2k / 32k / 128k tokens, chunk kernel -> split:
+//   16: 59 -> 18, 878 -> 48, 3 992 -> 115 us;  256: 66 -> 37, 868 -> 211, 3 857 -> 799 us;
+//   1 024: 92 -> 98, 928 -> 715, 3 896 -> 2 566 us.
 static bool prefill_split_applies(const Lay &a, int pos_start, int M)
 {
-    if (g_prefill_split == 0 || pos_start < kSplitMinPos || !stream_decode_supported(a, M < kSplitRows ? M : kSplitRows))
-        return false;
+    (void)a;
+    if (g_prefill_split == 0 || pos_start < kSplitMinPos) return false;
     if (g_prefill_split > 0) return M <= g_prefill_split;
-    const int rounds = (M + kSplitRows - 1) / kSplitRows;
-    return M <= kSplitMaxM && rounds * (50.0f + pos_start / 580.0f) < 0.027f * pos_start;
+    return M <= 512 || (M <= kSplitMaxM && pos_start >= 2 * kSplitMinPos);
 }
 
 static size_t prefill_split_need(const Lay &a, int pos_start, int M, size_t *lens_bytes)
 {
     const size_t lb = ((size_t)M * sizeof(int32_t) + 255) & ~(size_t)255;
     if (lens_bytes) *lens_bytes = lb;
-    size_t need = 0;
-    for (int r0 = 0; r0 < M; r0 += kSplitRows) {
-        const int B = M - r0 < kSplitRows ? M - r0 : kSplitRows;
-        const size_t n = shared_workspace_need(a, B, pos_start + r0 + B, pos_start + r0 + 1);
-        if (n > need) need = n;
-    }
-    return lb + need;
+    int ct, ns;
+    prefill_split_shape(a, pos_start, M, &ct, &ns);
+    return lb + (size_t)M * a.QH * ns * (a.D + 2) * sizeof(float);
 }
 
-static int prefill_split(const drk_kv_layout *g, const Lay &a, const void *q, const void *pool, const int32_t *table,
-                         void *out, int layer, int pos_start, int M, float scale, int io_dtype, void *workspace,
-                         size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
+static int prefill_split(const Lay &a, const void *q, const void *pool, const int32_t *table, void *out, int layer,
+                         int pos_start, int M, float scale, int io_dtype, void *workspace, hipStream_t st,
+                         const void *gate, size_t gate_stride)
 {
     size_t lb;
     prefill_split_need(a, pos_start, M, &lb);
     int32_t *lens = (int32_t *)workspace;
-    hipLaunchKernelGGL(iota_kernel, dim3((M + 255) / 256), dim3(256), 0, (hipStream_t)stream, lens, M, pos_start + 1);
+    hipLaunchKernelGGL(iota_kernel, dim3((M + 255) / 256), dim3(256), 0, st, lens, M, pos_start + 1);
     DRK_LAUNCH_CHECK("iota_kernel");
-    const size_t row = (size_t)a.QH * a.D * 2;
-    for (int r0 = 0; r0 < M; r0 += kSplitRows) {
-        const int B = M - r0 < kSplitRows ? M - r0 : kSplitRows;
-        const uint16_t *grow = gate ? (const uint16_t *)gate + (size_t)r0 * a.QH * gate_stride : nullptr;
-        const int rc = launch_decode_shared(g, (const uint8_t *)q + r0 * row, pool, table, 0, lens + r0, B, pos_start + r0 + B,
-                                            pos_start + r0 + 1, (uint8_t *)out + r0 * row, layer, scale, io_dtype,
-                                            (uint8_t *)workspace + lb, workspace_bytes - lb, stream, grow, gate_stride);
-        if (rc) return rc;
-    }
+    int ct, ns;
+    prefill_split_shape(a, pos_start, M, &ct, &ns);
+    float *part_o = (float *)((uint8_t *)workspace + lb);
+    float *part_m = part_o + (size_t)M * a.QH * ns * a.D;
+    float *part_l = part_m + (size_t)M * a.QH * ns;
+    int rc = launch_shared_prefix(a, q, pool, table, lens, M, pos_start + M, layer, scale, io_dtype, part_o, part_m, part_l, st,
+                                  ct, ns);
+    if (rc) return rc;
+    const dim3 grid((unsigned)((size_t)M * a.QH));
+    if (a.D == 128)
+        hipLaunchKernelGGL(prefill_merge_kernel<128>, grid, dim3(64), 0, st, part_o, part_m, part_l, (uint16_t *)out, ns, io_dtype,
+                           (const uint16_t *)gate, gate_stride);
+    else
+        hipLaunchKernelGGL(prefill_merge_kernel<256>, grid, dim3(64), 0, st, part_o, part_m, part_l, (uint16_t *)out, ns, io_dtype,
+                           (const uint16_t *)gate, gate_stride);
+    DRK_LAUNCH_CHECK("prefill_merge_kernel");
     return DRK_OK;
 }
 
@@ -695,8 +794,8 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     // drk_prefill_workspace_bytes reports; without it the chunk kernel below does the work)
     if (prefill_split_applies(a, pos_start, M) && workspace && ((uintptr_t)workspace % 256) == 0 &&
         workspace_bytes >= prefill_split_need(a, pos_start, M, nullptr))
-        return prefill_split(g, a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
-                             workspace_bytes, stream, gate, gate_stride);
+        return prefill_split(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
+                             (hipStream_t)stream, gate, gate_stride);
     PrefillArgs A;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
     A.table = d_block_table;

@@ -247,12 +247,12 @@ int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, con
  * chunk's own K/V must already be in the pages: write, then attend).
  * head_dim 128 or 256 with block_size % 16 == 0 (any storage type, any number of query
  * heads per KV head up to 128) runs on the MFMA prefill kernel, which needs no workspace.
- * A short chunk behind a long context (up to 64 rows behind 2 048 tokens, more behind
- * more; at most 16 query heads per KV head) is spread over the whole chip instead -- the
- * context split as in drk_paged_decode_attention_shared, rows = the chunk's tokens -- when
- * the workspace drk_prefill_workspace_bytes reports for it is passed (256-byte aligned);
- * without that workspace the MFMA kernel does the work, some 10-30 times slower for such a
- * chunk.  Anything else runs row by row through the portable decode kernel, which needs
+ * A chunk of up to 512 rows behind 2 048 tokens or more (1 024 behind 4 096) is spread over
+ * the whole chip instead -- the same kernel with the context split as in
+ * drk_paged_decode_attention_shared, rows = the chunk's tokens, then a merge -- when the
+ * workspace drk_prefill_workspace_bytes reports for it is passed (256-byte aligned, up to
+ * ~35 MB at 32 query heads x 128); without it the unsplit kernel does the work, up to 30
+ * times slower for a chunk of a few tokens behind a long context.  Anything else runs row by row through the portable decode kernel, which needs
  * the workspace. */
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M);
 int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,

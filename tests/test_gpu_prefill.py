@@ -233,9 +233,9 @@ def test_random_prefill_shapes(dev, seed):
                                            ((2, 2, 8, 128, 32, 150), cabi.INT8, cabi.BF16), ((2, 2, 12, 128, 16, 300), cabi.FP8_E4M3, cabi.F16)])
 @pytest.mark.parametrize("pos_start,M", [(2048, 1), (2049, 17), (3000, 64), (4095, 65), (2500, 130), (2048, 256)])
 def test_short_chunks_behind_a_long_context(dev, geom, dtype, io, pos_start, M):
-    """A chunk of up to 256 tokens behind 2 048 or more runs with the context split over the chip (the
-    shared-prefix machinery with rows = query tokens): against the fp64 oracle, against the chunk
-    kernel, the gated form against plain + gate; a hole in the table, stale bytes behind the end."""
+    """A chunk of up to 1 024 tokens behind 2 048 or more runs with the context split over the chip (the
+    kernel's shared-prefix mode with rows = query tokens, then a merge): against the fp64 oracle, against
+    the chunk kernel, the gated form against plain + gate; a hole in the table, stale bytes behind the end."""
     L, KVH, QH, D, bs, NB = geom
     lib = cabi.lib()
     g, og, rng, table, opool = build_io(geom, dtype, io, pos_start + M, seed=pos_start + M + D, holes=(2,), mul=0.7)
@@ -243,15 +243,9 @@ def test_short_chunks_behind_a_long_context(dev, geom, dtype, io, pos_start, M):
     qg = U.normal_bits(rng, (M, QH, 2 * D), io, 2.0)
     scale = 1 / np.sqrt(D)
     dq, dpool, dtab, dqg = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table), U.dev_bytes(qg)
-    # the library's own rule takes a single round of rows at these context lengths
-    assert (lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M) > 0) == (M <= 64)
-    lib.drk_debug_set_prefill_split(4096)                           # ... the test takes every shape through it
-    try:
-        wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
-        assert wsb > 0                                              # room for the partial results
-        raw = run_prefill(g, dq, dpool, dtab, L - 1, pos_start, M, scale, io, QH, D)
-    finally:
-        lib.drk_debug_set_prefill_split(-1)
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    assert wsb > 0                                                  # the split path asks for room for its partial results
+    raw = run_prefill(g, dq, dpool, dtab, L - 1, pos_start, M, scale, io, QH, D)
     got = U.from_bits(raw, io)
     want = orc.prefill_f64(og, q, opool, table, L - 1, pos_start, scale, io)
     ok, ma, _ = U.rel_abs_ok(got, want)
@@ -266,12 +260,8 @@ def test_short_chunks_behind_a_long_context(dev, geom, dtype, io, pos_start, M):
     ws = U.dev_zeros(wsb)
     out = U.dev_zeros(M * QH * D * 2)
     gptr = C.c_void_p(dqg.data_ptr() + D * 2)
-    lib.drk_debug_set_prefill_split(4096)
-    try:
-        cabi.call("drk_paged_prefill_attention_gated", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), L - 1, pos_start, M,
-                  float(scale), io, gptr, 2 * D, U.p(ws), wsb, U.stream_ptr())
-        U.sync()
-    finally:
-        lib.drk_debug_set_prefill_split(-1)
+    cabi.call("drk_paged_prefill_attention_gated", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), L - 1, pos_start, M,
+              float(scale), io, gptr, 2 * D, U.p(ws), wsb, U.stream_ptr())
+    U.sync()
     gated = orc.sigmoid_gate(raw, np.ascontiguousarray(qg[:, :, D:]), io)
     assert U.ulp_distance(U.host(out, np.uint16, (M, QH, D)), gated).max() <= 1
