@@ -42,7 +42,7 @@ def parse():
     ap.add_argument("--pool-gb", type=float, default=40.0)
     ap.add_argument("--split", type=int, default=0, help="tokens per split-K workgroup (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-ragged", action="store_true", help="skip the ragged-context launches of the decode kernel (profiling: keeps one shape per kernel name)")
+    ap.add_argument("--no-ragged", action="store_true", help="skip the side measurements that launch the headline kernel on other shapes (profiling: one shape per kernel name)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="context per branch for the CPU sample (0 = auto)")
     ap.add_argument("--bulk-append-tokens", type=int, default=2048)
     ap.add_argument("--seed", type=int, default=2)

@@ -348,7 +348,7 @@ def config5(args):
     # a short chunk at the end of the same context (a perception frame of a few tokens): the chunk kernel
     # against the path that splits the context over the chip
     short = {}
-    for rows in (16, 64):
+    for rows in (() if getattr(args, "no_ragged", False) else (16, 64)):
         pos = total - rows
         qs = torch.randn(rows, QH, D, device="cuda").to(torch.bfloat16)
         os_ = torch.empty_like(qs)

@@ -89,7 +89,7 @@ void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
                          const int32_t *d_seq_lens, int B, int shared, int layer, float scale, int io_dtype,
                          float *part_o, float *part_m, float *part_l, hipStream_t st, int chunk_tiles = 0,
-                         int nsplits = 0);
+                         int nsplits = 0, int causal_pos_start = 0);
 
 // ---- element helpers (device) -------------------------------------------
 // Streaming ("non-temporal") 128- and 64-bit accesses for data that is touched once

@@ -268,7 +268,8 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(Pre
     const bool wave_live = (w * 32) / G < TPW && qt * TPW + (w * 32) / G < A.M;
     int vis, lim_wg, t_begin = 0, first_masked_tile = 0;
     if (SHARED) {
-        const int len = row_live ? A.seq_lens[tq] : 0;
+        // a row's length: the branch's, or -- the rows being the tokens of a chunk -- pos_start + t + 1
+        const int len = row_live ? (A.seq_lens ? A.seq_lens[tq] : A.pos_start + tq + 1) : 0;
         vis = min(len, A.shared);                               // tokens [0, vis) are visible to the row
         t_begin = (int)blockIdx.z * A.chunk_tiles;
         lim_wg = min(A.shared, (t_begin + A.chunk_tiles) * kPfBN);
@@ -549,14 +550,15 @@ void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits)
 
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
                          const int32_t *d_seq_lens, int B, int shared, int layer, float scale, int io_dtype,
-                         float *part_o, float *part_m, float *part_l, hipStream_t st, int chunk_tiles, int nsplits)
+                         float *part_o, float *part_m, float *part_l, hipStream_t st, int chunk_tiles, int nsplits,
+                         int causal_pos_start)
 {
     PrefillArgs A;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
     A.table = table0;
     A.q = (const uint8_t *)q;
     A.out = nullptr;
-    A.pos_start = 0; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs; A.tpw = 128 / (a.QH / a.KVH);
+    A.pos_start = causal_pos_start; A.M = B; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs; A.tpw = 128 / (a.QH / a.KVH);
     A.bs_shift = ilog2_exact((unsigned)a.bs);
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
     A.scale_log2e = scale * kLog2eP;
@@ -591,12 +593,6 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 // row's pieces (and applies the gate).
 int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
 constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
-
-__global__ void iota_kernel(int32_t *__restrict__ dst, int n, int first)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) dst[i] = first + i;
-}
 
 // grid = rows (query token x query head), block = 64: lane s owns the (m, l) of piece s (at most 128
 // pieces: two per lane), so the weights come in one round of loads; then the lanes own dims
@@ -707,31 +703,24 @@ static bool prefill_split_applies(const Lay &a, int pos_start, int M)
     return M <= 512 || (M <= kSplitMaxM && pos_start >= 2 * kSplitMinPos);
 }
 
-static size_t prefill_split_need(const Lay &a, int pos_start, int M, size_t *lens_bytes)
+static size_t prefill_split_need(const Lay &a, int pos_start, int M)
 {
-    const size_t lb = ((size_t)M * sizeof(int32_t) + 255) & ~(size_t)255;
-    if (lens_bytes) *lens_bytes = lb;
     int ct, ns;
     prefill_split_shape(a, pos_start, M, &ct, &ns);
-    return lb + (size_t)M * a.QH * ns * (a.D + 2) * sizeof(float);
+    return (size_t)M * a.QH * ns * (a.D + 2) * sizeof(float);
 }
 
 static int prefill_split(const Lay &a, const void *q, const void *pool, const int32_t *table, void *out, int layer,
                          int pos_start, int M, float scale, int io_dtype, void *workspace, hipStream_t st,
                          const void *gate, size_t gate_stride)
 {
-    size_t lb;
-    prefill_split_need(a, pos_start, M, &lb);
-    int32_t *lens = (int32_t *)workspace;
-    hipLaunchKernelGGL(iota_kernel, dim3((M + 255) / 256), dim3(256), 0, st, lens, M, pos_start + 1);
-    DRK_LAUNCH_CHECK("iota_kernel");
     int ct, ns;
     prefill_split_shape(a, pos_start, M, &ct, &ns);
-    float *part_o = (float *)((uint8_t *)workspace + lb);
+    float *part_o = (float *)workspace;
     float *part_m = part_o + (size_t)M * a.QH * ns * a.D;
     float *part_l = part_m + (size_t)M * a.QH * ns;
-    int rc = launch_shared_prefix(a, q, pool, table, lens, M, pos_start + M, layer, scale, io_dtype, part_o, part_m, part_l, st,
-                                  ct, ns);
+    int rc = launch_shared_prefix(a, q, pool, table, nullptr, M, pos_start + M, layer, scale, io_dtype, part_o, part_m, part_l, st,
+                                  ct, ns, pos_start);
     if (rc) return rc;
     const dim3 grid((unsigned)((size_t)M * a.QH));
     if (a.D == 128)
@@ -758,7 +747,7 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
     const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 &&
                       (a.bs % 16) == 0;
-    if (mfma) return prefill_split_applies(a, pos_start, M) ? prefill_split_need(a, pos_start, M, nullptr) : 0;
+    if (mfma) return prefill_split_applies(a, pos_start, M) ? prefill_split_need(a, pos_start, M) : 0;
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
@@ -792,8 +781,8 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         return fail(DRK_ERR_INVALID, "prefill: gate rows must be 16-byte aligned and at least head_dim apart");
     // a short chunk behind a long context: split the context over the chip (needs the workspace
     // drk_prefill_workspace_bytes reports; without it the chunk kernel below does the work)
-    if (prefill_split_applies(a, pos_start, M) && workspace && ((uintptr_t)workspace % 256) == 0 &&
-        workspace_bytes >= prefill_split_need(a, pos_start, M, nullptr))
+    if (prefill_split_applies(a, pos_start, M) && workspace && ((uintptr_t)workspace % 16) == 0 &&
+        workspace_bytes >= prefill_split_need(a, pos_start, M))
         return prefill_split(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
                              (hipStream_t)stream, gate, gate_stride);
     PrefillArgs A;

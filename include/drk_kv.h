@@ -250,7 +250,7 @@ int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, con
  * A chunk of up to 512 rows behind 2 048 tokens or more (1 024 behind 4 096) is spread over
  * the whole chip instead -- the same kernel with the context split as in
  * drk_paged_decode_attention_shared, rows = the chunk's tokens, then a merge -- when the
- * workspace drk_prefill_workspace_bytes reports for it is passed (256-byte aligned, up to
+ * workspace drk_prefill_workspace_bytes reports for it is passed (16-byte aligned, up to
  * ~35 MB at 32 query heads x 128); without it the unsplit kernel does the work, up to 30
  * times slower for a chunk of a few tokens behind a long context.  Anything else runs row by row through the portable decode kernel, which needs
  * the workspace. */
