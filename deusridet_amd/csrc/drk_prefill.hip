@@ -251,7 +251,15 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(Pre
 
     // Workgroups are dealt to the 8 XCDs round-robin by linear id; kv head = id % KVH
     // keeps one kv head's pages in one XCD's L2 (8 kv heads on 8 XCDs).
-    const int kvh = (int)blockIdx.x % A.KVH, qt = (int)blockIdx.x / A.KVH;
+    const int kvh = (int)blockIdx.x % A.KVH;
+    int qt = (int)blockIdx.x / A.KVH;
+    if (!SHARED) {
+        // causal chunks: row tile q walks pos_start + 32 (q + 1) tokens.  The second half of the grid is
+        // taken in reverse, so that the two workgroups a CU holds when the grid is one resident round
+        // (dispatch order: all first slots, then all second slots) are a short walk and a long one
+        const int nqt = (int)gridDim.x / A.KVH, half = (nqt + 1) / 2;
+        if (qt >= half) qt = nqt - 1 - (qt - half);
+    }
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
