@@ -69,6 +69,7 @@ SIGNATURES = {
                                                       _f32, _vp]),
     "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32]),
+    "drkh_paged_attention_release_workspace": (None, []),
     "drkh_kvs_create": (_vp, []),
     "drkh_kvs_destroy": (None, [_vp]),
     "drkh_kvs_init": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32]),

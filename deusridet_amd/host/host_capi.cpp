@@ -296,6 +296,7 @@ int drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, in
 {
     return paged_attention_reserve_workspace(max_branches, max_seq_len, max_prefill_rows, block_size) ? 1 : 0;
 }
+void drkh_paged_attention_release_workspace(void) { paged_attention_release_workspace(); }
 void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,
                                        int num_tokens, int num_layers, int num_kv_heads, int head_dim,
                                        int block_size, int max_phys_blocks, void *stream)

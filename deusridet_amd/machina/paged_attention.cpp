@@ -151,9 +151,9 @@ void paged_prefill_attention(const __half* Q, __half* kv_pool, const int* d_bloc
     drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
     size_t need = drk_prefill_workspace_bytes(&g, pos_start, M);
     void* ws = workspace(need);
-    if (!ws) return;
+    if (!ws && need) return;            // need == 0 (the MFMA kernel on a long chunk) and nothing reserved yet: no workspace
     if (drk_paged_prefill_attention(&g, Q, kv_pool, d_block_table, out, fa_layer_idx, pos_start, M, scale,
-                                    ModelConfig::IO_DTYPE, ws, g_ws_bytes, stream) != DRK_OK)
+                                    ModelConfig::IO_DTYPE, ws, ws ? g_ws_bytes : 0, stream) != DRK_OK)
         LOG_ERROR("Machina", "paged_prefill_attention: %s", drk_last_error());
 }
 
@@ -243,9 +243,9 @@ void paged_prefill_attention_gated(const __half* Q, __half* kv_pool, const int* 
     drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
     size_t need = drk_prefill_workspace_bytes(&g, pos_start, M);
     void* ws = workspace(need);
-    if (!ws) return;
+    if (!ws && need) return;
     if (drk_paged_prefill_attention_gated(&g, Q, kv_pool, d_block_table, out, fa_layer_idx, pos_start, M, scale,
-                                          ModelConfig::IO_DTYPE, gate, (size_t)gate_stride, ws, g_ws_bytes,
+                                          ModelConfig::IO_DTYPE, gate, (size_t)gate_stride, ws, ws ? g_ws_bytes : 0,
                                           stream) != DRK_OK)
         LOG_ERROR("Machina", "paged_prefill_attention_gated: %s", drk_last_error());
 }

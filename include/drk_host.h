@@ -170,6 +170,7 @@ void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_poo
                                                      int max_phys_blocks, int block_size, float scale,
                                                      float *d_block_mass, int accumulate, void *stream);
 int  drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
+void drkh_paged_attention_release_workspace(void);
 void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,
                                        int num_tokens, int num_layers, int num_kv_heads, int head_dim,
                                        int block_size, int max_phys_blocks, void *stream);

@@ -347,3 +347,33 @@ def test_eviction_guided_by_measured_attention_mass(dev):
     changed = np.argwhere(before != after)
     assert changed.tolist() == [list(cold)] and after[cold] == -1
     assert cm.block_location(*cold) == host.CacheManager.INVALID
+
+
+def test_prefill_as_the_first_call_without_a_reserved_workspace(dev):
+    """The usual order of a session is prefill first.  A long chunk on the MFMA kernel needs no workspace: the
+    wrapper must launch it also when nothing has been reserved or allocated yet (it once returned silently)."""
+    L, KVH, QH, D, bs, M = 1, 4, 16, 128, 16, 40
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.F16)
+    cm = host.CacheManager()
+    assert cm.init(16 * L * 2 * KVH * bs * D * 2, bs)
+    NB = cm.pool_max_blocks()
+    assert cm.ensure_blocks_for_range(0, 0, M)
+    cm.sync_block_table(U.stream_ptr())
+    rng = np.random.default_rng(5)
+    k, v, q = (U.normal_bits(rng, s, cabi.F16) for s in ((M, KVH, D), (M, KVH, D), (M, QH, D)))
+    dk, dv, dq = U.dev_bytes(k), U.dev_bytes(v), U.dev_bytes(q)
+    L_ = host.lib()
+    L_.drkh_paged_kv_cache_write_batch(U.p(dk), U.p(dv), cm.pool_ptr(), cm.d_block_table(0), 0, 0, M, NB, bs, U.stream_ptr())
+    out = U.dev_bytes(np.full(M * QH * D * 2, 0x7B, np.uint8))
+    U.sync()
+    L_.drkh_paged_attention_release_workspace()
+    scale = 1 / np.sqrt(D)
+    L_.drkh_paged_prefill_attention(U.p(dq), cm.pool_ptr(), cm.d_block_table(0), U.p(out), 0, 0, M, NB, bs, float(scale),
+                                    U.stream_ptr())
+    U.sync()
+    og = orc.layout(L, KVH, QH, D, bs, NB, orc.F16)
+    opool = orc.new_pool(og)
+    orc.append_batch(og, opool, cm.h_block_table(0), 0, 0, k, v, orc.F16)
+    want = orc.prefill_f64(og, q, opool, cm.h_block_table(0), 0, 0, scale, orc.F16)
+    ok, ma, _ = U.rel_abs_ok(U.from_bits(U.host(out, np.uint16, (M, QH, D)), cabi.F16), want)
+    assert ok, ma
