@@ -20,7 +20,10 @@
  *   - head norm / RoPE / gate: fp64 numpy closed forms (x / sqrt(mean(x^2) + eps) * w,
  *     plane rotation by pos * theta^(-2i/rd), x * logistic(g)) to one unit in the
  *     last place of the 16-bit type, rotation by position 0 == identity, rotations
- *     keep each pair's length.
+ *     keep each pair's length;
+ *   - fixtures written without this file (tests/golden: the E4M3FN table with encode
+ *     cases, int8 rows in IEEE arithmetic, a free-stack trace, fp64 attention of the
+ *     512-token fp16 configuration).
  * Parity of the *reference decode kernel's exact fp16 output bits* (it is built
  * with --use_fast_math) is unpinned: the tolerance in the tests is against fp64.
  */
