@@ -595,11 +595,14 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
 // Shared-prefix decode: tokens [0, shared) live in the same physical pages for all
 // B branches, so their K/V are streamed once for all B*QH query rows (matrix-core
 // pass), the private tails go through the stream kernel, one merge folds both.
-static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size_t *stream_part)
+// exact: what a launch with this very prefix length uses (short tails keep few pieces); otherwise
+// an upper bound for any prefix up to `shared`, which is what callers size their workspace by
+static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size_t *stream_part, bool exact)
 {
     int ct, ns;
     shared_prefix_shape(shared, &ct, &ns);
-    size_t sp = stream_workspace_need(a, B, max_seq_len, 0, shared / kTile);
+    if (!exact && ns < g_shared_splits) ns = g_shared_splits;
+    size_t sp = stream_workspace_need(a, B, max_seq_len, 0, exact ? shared / kTile : 0);
     sp = (sp + 255) & ~(size_t)255;
     if (stream_part) *stream_part = sp;
     return sp + (size_t)B * a.QH * ns * (a.D + 2) * sizeof(float);
@@ -629,7 +632,7 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
         return fail(DRK_ERR_INVALID, "decode: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "decode: layer %d outside [0,%d)", layer, a.L);
     size_t sp;
-    const size_t need = shared_need(a, B, max_seq_len, shared, &sp);
+    const size_t need = shared_need(a, B, max_seq_len, shared, &sp, true);
     if (!workspace || workspace_bytes < need)
         return fail(DRK_ERR_WORKSPACE, "decode: workspace of %zu bytes, need %zu", workspace_bytes, need);
     if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode: workspace must be 16-byte aligned");
@@ -735,7 +738,7 @@ size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_
     size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);
     const int shared = shared_tokens > 0 ? (shared_tokens / kTile) * kTile : 0;
     if (stream_decode_supported(a, B) && shared >= kTile) {
-        size_t s2 = shared_need(a, B, max_seq_len, shared, nullptr);
+        size_t s2 = shared_need(a, B, max_seq_len, shared, nullptr, false);
         if (s2 > need) need = s2;
     }
     return need;

@@ -404,6 +404,18 @@ def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
     assert ok, ma
     ok, ma, _ = U.rel_abs_ok(got, plain, REL, ABS)
     assert ok, ma
+    # a workspace sized for the longest prefix the caller may ever pass serves every shorter one
+    # (the pieces the private tails need grow as the prefix shrinks)
+    assert wsb <= lib.drk_decode_shared_workspace_bytes(C.byref(g), B, mx, mx)
+    wsb_max = lib.drk_decode_shared_workspace_bytes(C.byref(g), B, mx, mx)
+    ws_max = U.dev_zeros(wsb_max)
+    if shared_arg >= 128:
+        out3 = U.dev_zeros(B * QH * D * 2)
+        cabi.call("drk_paged_decode_attention_shared", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dl), B, mx,
+                  shared_arg - 64, U.p(out3), 0, float(scale), io, U.p(ws_max), wsb_max, U.stream_ptr())
+        U.sync()
+        ok, ma, _ = U.rel_abs_ok(U.from_bits(U.host(out3, np.uint16, (B, QH, D)), io), want, REL, ABS)
+        assert ok, ma
 
 
 def test_more_branches_than_one_launch_takes(dev):
