@@ -1,0 +1,33 @@
+"""GPU: every workload of bench.py runs to its one JSON line on a reduced number of layers and steps --
+the entry points are used there the way a caller would (workspaces sized once for the largest case, one
+captured graph per step), which is how a change of a size contract shows."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+KEYS = {"metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline",
+        "dtype", "data", "config", "roofline", "cpu_baseline"}
+
+
+@pytest.mark.parametrize("extra", [[], ["--ctx-mode", "uniform"], ["--config", "3"], ["--config", "4"], ["--config", "4", "--kv-dtype", "fp8"],
+                                   ["--config", "5"], ["--config", "5", "--kv-dtype", "int8"], ["--config", "6"], ["--config", "7"]],
+                         ids=lambda e: "-".join(x.strip("-") for x in e) or "default")
+def test_bench_workload_runs(dev, extra):
+    cmd = [sys.executable, os.path.join(ROOT, "bench.py"), "--layers", "2", "--steps", "2", "--warmup", "1", "--no-cpu-baseline"] + extra
+    r = subprocess.run(cmd, cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    j = json.loads(lines[0])
+    assert KEYS <= set(j) and j["n_gpus"] == 1 and j["value"] > 0 and "workload" in j["config"]
+
+
+def test_more_than_one_gpu_is_refused():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], cwd=ROOT, capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "ONE GPU" in (r.stdout + r.stderr)
