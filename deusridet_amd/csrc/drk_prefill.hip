@@ -701,7 +701,7 @@ static void prefill_split_shape(const Lay &a, int pos_start, int M, int *chunk_t
 // When it pays (measured, 32 Q / 8 KV x 128 bf16): the chunk kernel takes 27 us per 1 024 tokens of
 // context whatever the chunk length up to 1 024 rows (one workgroup per CU at most); the split pass
 // keeps every CU busy.  Rows behind 2k / 32k / 128k tokens, chunk kernel -> split:
-//   16: 59 -> 18, 878 -> 48, 3 992 -> 115 us;  256: 66 -> 37, 868 -> 211, 3 857 -> 799 us;
+//   16: 59 -> 18, 878 -> 42, 3 992 -> 115 us;  256: 66 -> 37, 868 -> 211, 3 857 -> 799 us;
 //   1 024: 92 -> 98, 928 -> 715, 3 896 -> 2 566 us.
 static bool prefill_split_applies(const Lay &a, int pos_start, int M)
 {
