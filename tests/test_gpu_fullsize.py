@@ -267,3 +267,103 @@ def test_pages_beyond_4GiB_of_a_layer(dev, dtype):
     assert not np.array_equal(got, portable)                         # a different kernel produced the bits ...
     ok, ma, _ = U.rel_abs_ok(got, portable.astype(np.float64))
     assert ok, ma                                                     # ... of the same result
+
+
+def test_config3_full_size_properties(dev):
+    """BASELINE config 3 at its real sizes on one layer: a 65 536-token prefix (4 096 blocks) shared by 16
+    copy-on-write branches with private tails of up to 4 096 tokens.  Properties that need no oracle at
+    this size: every prefix block carries 17 references and the tables agree on them; the call that
+    streams the prefix once equals the per-branch call; evicting down to 25 % free blocks frees private
+    pages only -- the prefix keeps its references and its bytes (attention over it is unchanged)."""
+    torch = _torch()
+    from deusridet_amd import host
+    L, KVH, QH, D, bs, B, P = 1, 8, 32, 128, 16, 16, 65536
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    cm = host.CacheManager()
+    NBW = P // bs + B * (4096 // bs + 1) + 64
+    assert cm.init(NBW * L * 2 * KVH * bs * D * 2, bs, None, 1 + B)
+    NB, stride = cm.pool_max_blocks(), cm.table_stride()
+    hl = host.lib()
+    st = U.stream_ptr()
+    gen = torch.Generator(device="cuda").manual_seed(3)
+
+    def write(branch, pos0, n):
+        k = (torch.randn(n, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        v = (torch.randn(n, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        hl.drkh_paged_kv_cache_write_batch(U.p(k), U.p(v), cm.pool_ptr(), cm.d_block_table(branch), 0, pos0, n, NB, bs, st)
+        U.sync()
+
+    assert cm.ensure_blocks_for_range(0, 0, P)
+    cm.sync_block_table(st)
+    for p0 in range(0, P, 8192):
+        write(0, p0, 8192)
+    cm.set_seq_len(0, P)
+    rng = np.random.default_rng(3)
+    priv = rng.integers(0, 4097, size=B)
+    priv[0], priv[1] = 0, 4096
+    kids = []
+    for i in range(B):
+        b = cm.fork_branch(0, P)
+        assert b > 0
+        kids.append(b)
+    prefix = cm.h_block_table(0)[:P // bs].copy()
+    assert all(cm.pool_refcount(int(x)) == 1 + B for x in prefix[[0, 1, 2047, 4095]])
+    for i, b in enumerate(kids):
+        n = int(priv[i])
+        if n:
+            assert cm.ensure_blocks_for_range(b, P, n)
+    cm.sync_block_table(st)
+    for i, b in enumerate(kids):
+        if priv[i]:
+            write(b, P, int(priv[i]))
+        cm.set_seq_len(b, P + int(priv[i]))
+        assert np.array_equal(cm.h_block_table(b)[:P // bs], prefix)           # the shared pages, not copies
+    assert cm.common_prefix_tokens(kids) == P
+    lens = (P + priv).astype(np.int32)
+    mx = int(lens.max())
+    tabs = np.stack([cm.h_block_table(b) for b in kids])
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    lib = cabi.lib()
+    pool_ptr = C.c_void_p(cm.pool_ptr()) if not isinstance(cm.pool_ptr(), C.c_void_p) else cm.pool_ptr()
+    q = (torch.randn(B, QH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+    dl, dt = U.dev_i32(lens), U.dev_i32(tabs)
+    wsb = max(lib.drk_decode_shared_workspace_bytes(C.byref(g), B, mx, P), lib.drk_decode_workspace_bytes(C.byref(g), B, mx))
+    ws = U.dev_zeros(wsb)
+    scale = float(1 / np.sqrt(D))
+
+    def attend(shared):
+        out = torch.zeros_like(q)
+        if shared:
+            cabi.call("drk_paged_decode_attention_shared", C.byref(g), U.p(q), pool_ptr, U.p(dt), stride, U.p(dl), B, mx, P, U.p(out),
+                      0, scale, cabi.BF16, U.p(ws), wsb, st)
+        else:
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), U.p(q), pool_ptr, U.p(dt), stride, U.p(dl), B, mx, U.p(out),
+                      0, scale, cabi.BF16, 0, U.p(ws), wsb, st)
+        U.sync()
+        return out.float().cpu().numpy()
+
+    once, per_branch = attend(True), attend(False)
+    ok, ma, _ = U.rel_abs_ok(once, per_branch)
+    assert ok, ma
+    # make room for 500 more blocks: private pages go (oldest first), the prefix stays
+    private_blocks = int(sum((int(n) + bs - 1) // bs for n in priv))
+    assert private_blocks > 600
+    free0 = cm.free_blocks()
+    assert cm.ensure_free_blocks(free0 + 500) and cm.free_blocks() == free0 + 500
+    assert not cm.ensure_free_blocks(NB - P // bs + 1)                          # more than everything unshared: refused ...
+    assert cm.free_blocks() == NB - P // bs                                     # ... after every private page has gone
+    assert all(cm.pool_refcount(int(x)) == 1 + B for x in prefix[[0, 1, 2047, 4095]])
+    for b in kids:
+        assert np.array_equal(cm.h_block_table(b)[:P // bs], prefix)
+        assert (cm.h_block_table(b)[P // bs:] < 0).all()
+    # attention over the prefix alone is what it was: same bytes, same tables
+    cm.sync_block_table(st)
+    dl2 = U.dev_i32(np.full(B, P, np.int32))
+    dt2 = U.dev_i32(np.stack([cm.h_block_table(b) for b in kids]))
+    out_a, out_b = torch.zeros_like(q), torch.zeros_like(q)
+    cabi.call("drk_paged_decode_attention_shared", C.byref(g), U.p(q), pool_ptr, U.p(dt2), stride, U.p(dl2), B, P, P, U.p(out_a), 0,
+              scale, cabi.BF16, U.p(ws), wsb, st)
+    cabi.call("drk_paged_decode_attention_shared", C.byref(g), U.p(q), pool_ptr, U.p(dt), stride, U.p(dl2), B, P, P, U.p(out_b), 0,
+              scale, cabi.BF16, U.p(ws), wsb, st)
+    U.sync()
+    assert torch.equal(out_a, out_b)
