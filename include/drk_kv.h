@@ -232,7 +232,8 @@ int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, c
  * instead of once per branch.  shared_tokens is rounded down to a multiple of 64;
  * 0, or a geometry the tiled decode kernel does not take, gives exactly
  * drk_paged_decode_attention_branches (every storage type has the shared pass).  Results equal the per-branch call up to
- * summation order. */
+ * summation order.  drk_decode_shared_workspace_bytes(g, B, max_seq_len, s) is enough for every call with these B and
+ * max_seq_len and any shared_tokens up to s. */
 size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len, int shared_tokens);
 int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, const void *pool,
                                       const int32_t *d_tables, int table_stride,
