@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libdrk_kv.so")
 
 F16, BF16, INT8, FP8_E4M3 = 0, 1, 2, 3
 OK, ERR_INVALID, ERR_HIP, ERR_UNSUPPORTED, ERR_WORKSPACE = 0, -1, -2, -3, -4
+STATIC_SCRATCH_BYTES = 32 << 20
 
 
 class DrkError(RuntimeError):
@@ -90,6 +91,8 @@ SIGNATURES = {
     "drk_paged_decode_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
     "drk_paged_decode_attention_branches": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32,
                                                    _f32, _i32, _i32, _vp, _sz, _vp]),
+    "drk_paged_decode_attention_branches_static": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32,
+                                                          _f32, _i32, _vp]),
     "drk_decode_shared_workspace_bytes": (_sz, [_LP, _i32, _i32, _i32]),
     "drk_paged_decode_attention_shared": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _i32, _f32,
                                                  _i32, _vp, _sz, _vp]),

@@ -28,6 +28,14 @@
 
 #include <math.h>
 
+#include <mutex>
+
+// Scratch of drk_paged_decode_attention_branches_static: the split-K partials of the one
+// entry point that takes no workspace.  Every GPU the library runs on holds its own copy
+// until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels are given the address that call returned, never the name.
+static __device__ __align__(256) unsigned char scratch[DRK_STATIC_SCRATCH_BYTES];
+
 namespace drk {
 
 int g_force_portable = 0;                    // diagnostic, shared with the prefill unit
@@ -828,6 +836,52 @@ int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const
                                    lse_groups, lse_rows, ls)))
         return rc;
     return launch_block_mass(lse_groups, lse_rows, d_seq_lens, B, a.QH, ls, a.bs, d_block_mass, mass_stride, accumulate, st);
+}
+
+// ---- decode that allocates nothing and takes no workspace ------------------------------
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];        // device address of `scratch` on device i, once looked up
+static std::mutex g_scratch_mu;
+
+// The address of this device's copy of `scratch` (each GPU maps the array at an address of
+// its own), looked up once per device with that device current.
+static int static_scratch(void **ptr)
+{
+    int dev = -1;
+    DRK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(DRK_ERR_INVALID, "decode_static: device %d outside [0,%d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        DRK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(DRK_ERR_HIP, "decode_static: the scratch array has no address on device %d", dev);
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return DRK_OK;
+}
+
+int drk_paged_decode_attention_branches_static(const drk_kv_layout *g, const void *q, const void *pool,
+                                               const int32_t *d_tables, int table_stride,
+                                               const int32_t *d_seq_lens, int B, int max_seq_len, void *out,
+                                               int layer, float scale, int io_dtype, void *stream)
+{
+    if (!d_seq_lens) return fail(DRK_ERR_INVALID, "decode_static: d_seq_lens is NULL");
+    if (B < 0 || max_seq_len < 0) return fail(DRK_ERR_INVALID, "decode_static: negative size");
+    if (B == 0 || max_seq_len == 0) return DRK_OK;
+    const size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);
+    if (need == 0) return fail(DRK_ERR_INVALID, "decode_static: bad layout");
+    if (need > (size_t)DRK_STATIC_SCRATCH_BYTES)
+        return fail(DRK_ERR_WORKSPACE,
+                    "decode_static: %d branches of up to %d tokens need %zu bytes of partials, the static scratch holds %zu; "
+                    "use drk_paged_decode_attention_branches with a workspace",
+                    B, max_seq_len, need, (size_t)DRK_STATIC_SCRATCH_BYTES);
+    void *ptr = nullptr;
+    int rc = static_scratch(&ptr);
+    if (rc) return rc;
+    // nothing in the scratch has to start at zero: the partial kernel writes every slot the merge reads
+    return launch_decode(g, q, pool, d_tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale,
+                         io_dtype, 0, ptr, (size_t)DRK_STATIC_SCRATCH_BYTES, stream);
 }
 
 // steps 6 + 7 of full_attention_forward_paged (paged_attention.cu:362-370) in one call:

@@ -223,6 +223,25 @@ int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, c
                                         int split_tokens, void *workspace,
                                         size_t workspace_bytes, void *stream);
 
+/* The same call for callers that cannot allocate or carry a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  The split-K partials live in a file-scope device array of
+ * DRK_STATIC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends;
+ * the call allocates and frees nothing, picks the split itself, and fails with
+ * DRK_ERR_WORKSPACE when drk_decode_workspace_bytes(g, B, max_seq_len) exceeds that size
+ * (config 2's 8 x 32k needs 8.8 MB; 16 branches x 32 query heads x 128 at 32k, 17.6 MB).
+ * Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams,
+ * two threads) race on the partials -- serialise them, or use the call above with a
+ * workspace per stream.  Nothing in the array needs clearing between calls.  The first call
+ * on each device looks the array's address up (hipGetSymbolAddress): make it outside a
+ * stream capture. */
+#define DRK_STATIC_SCRATCH_BYTES (32u << 20)
+int drk_paged_decode_attention_branches_static(const drk_kv_layout *g, const void *q, const void *pool,
+                                               const int32_t *d_tables, int table_stride,
+                                               const int32_t *d_seq_lens, int B, int max_seq_len,
+                                               void *out, int layer, float scale, int io_dtype,
+                                               void *stream);
+
 /* Branches that share a prefix (no reference counterpart; intent
  * docs/en/architecture/03-cogitatio.md:3-5, 18-22: decode branches over one
  * persistent Conscientia prefix).  The caller promises that the pages holding
