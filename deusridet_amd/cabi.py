@@ -35,7 +35,7 @@ def layout(L, KVH, QH, D, bs, NB, dtype):
 _vp, _i32, _sz, _f32 = C.c_void_p, C.c_int32, C.c_size_t, C.c_float
 _LP = C.POINTER(Layout)
 
-# name -> (restype, argtypes); mirrors include/drk_kv.h one to one
+# name -> (restype, argtypes); mirrors include/drk_kv.h and include/drk_debug.h one to one
 SIGNATURES = {
     "drk_abi_version": (_i32, []),
     "drk_last_error": (C.c_char_p, []),
@@ -54,6 +54,7 @@ SIGNATURES = {
     "drk_dev_free": (_i32, [_vp]),
     "drk_dev_memset_async": (_i32, [_vp, _i32, _sz, _vp]),
     "drk_memcpy_h2d_async": (_i32, [_vp, _vp, _sz, _vp]),
+    "drk_memcpy_d2d_async": (_i32, [_vp, _vp, _sz, _vp]),
     "drk_memcpy_d2h": (_i32, [_vp, _vp, _sz, _vp]),
     "drk_positions_advance": (_i32, [_vp, _vp, _i32, _i32, _vp]),
     "drk_graph_begin_capture": (_i32, [_vp]),
@@ -69,6 +70,12 @@ SIGNATURES = {
     "drk_stream_create": (_i32, [C.POINTER(_vp)]),
     "drk_stream_destroy": (_i32, [_vp]),
     "drk_stream_synchronize": (_i32, [_vp]),
+    "drk_stream_is_capturing": (_i32, [_vp, C.POINTER(_i32)]),
+    "drk_event_create": (_i32, [C.POINTER(_vp)]),
+    "drk_event_destroy": (_i32, [_vp]),
+    "drk_event_record": (_i32, [_vp, _vp]),
+    "drk_event_synchronize": (_i32, [_vp]),
+    "drk_stream_wait_event": (_i32, [_vp, _vp]),
     "drk_kv_append_token": (_i32, [_LP, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp]),
     "drk_kv_append_batch": (_i32, [_LP, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp]),
     "drk_kv_append_branches": (_i32, [_LP, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _i32, _vp]),
@@ -87,6 +94,9 @@ SIGNATURES = {
     "drk_debug_set_append_chunks": (None, [_i32, _i32, _i32]),
     "drk_debug_set_prefill_split": (None, [_i32]),
     "drk_probe_read_bandwidth": (_i32, [_vp, _sz, _i32, _vp, C.POINTER(C.c_float)]),
+    "drk_probe_read_bandwidth_permuted": (_i32, [_vp, _sz, _i32, _i32, _vp, C.POINTER(C.c_float)]),
+    "drk_probe_mfma_rate": (_i32, [_i32, _vp, C.POINTER(C.c_float)]),
+    "drk_prefill_workspace_bytes_max": (_sz, [_LP, _i32, _i32]),
     "drk_debug_decode_kernel_times": (_i32, [C.POINTER(C.c_float), _i32, C.POINTER(_i32)]),
     "drk_paged_decode_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
     "drk_paged_decode_attention_branches": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32,

@@ -10,9 +10,18 @@ namespace deusridet {
 KvStream::~KvStream() { destroy(); }
 
 bool KvStream::init(CacheManager& cm, int max_context_len, ImportanceScorer* scorer, const float* d_rope_table,
-                    int table_positions)
+                    int table_positions, int max_prefill_rows)
 {
     destroy();
+    // the scored attention call writes one row of table_stride() masses per branch into the scorer's
+    // buffer, indexed like the block tables
+    if (scorer && scorer->d_new_scores() &&
+        (long long)scorer->max_blocks() < (long long)cm.max_branches() * cm.table_stride()) {
+        LOG_ERROR("Conscientia", "KvStream: the scorer holds %d blocks, %d branches x %d table entries need %lld",
+                  scorer->max_blocks(), cm.max_branches(), cm.table_stride(), (long long)cm.max_branches() * cm.table_stride());
+        return false;
+    }
+    max_prefill_rows_ = max_prefill_rows;
     cm_ = &cm;
     scorer_ = scorer;
     d_rope_table_ = d_rope_table;
@@ -33,7 +42,9 @@ bool KvStream::init(CacheManager& cm, int max_context_len, ImportanceScorer* sco
     }
     d_len_ = static_cast<int*>(p);
     // every attention call below finds its split-K workspace ready: nothing allocates later
-    if (!paged_attention_reserve_workspace(cm.max_branches(), max_context_len, 0, cm.block_pool().block_size())) {
+    const int bs = cm.block_pool().block_size();
+    if (!ws_decode_.reserve_for(cm.max_branches(), max_context_len, 0, bs) ||
+        !ws_prefill_.reserve_for(1, max_context_len, max_prefill_rows, bs)) {
         destroy();
         return false;
     }
@@ -46,9 +57,15 @@ void KvStream::destroy()
         drk_graph_destroy(graph_);
         graph_ = nullptr;
     }
+    scorer_ = nullptr;                            // borrowed, and possibly gone already: its rows are not cleared here
     if (cm_) close_branches();
     if (d_pos_) drk_dev_free(d_pos_);
     if (d_len_) drk_dev_free(d_len_);
+    if (ws_decode_.ptr() || ws_prefill_.ptr()) {
+        drk_device_synchronize();                 // launches that use the partials may still be running
+        ws_decode_.release();
+        ws_prefill_.release();
+    }
     d_pos_ = d_len_ = nullptr;
     cm_ = nullptr;
     scorer_ = nullptr;
@@ -63,6 +80,10 @@ bool KvStream::begin_prefill(int M, hipStream_t stream)
     // Decode branches may be open (time division: perception goes on while they think).  They
     // keep the pages they forked from; the stream's first write into a block it still shares
     // with them makes a private copy, as a branch's would.
+    if (M > max_prefill_rows_) {
+        LOG_ERROR("Conscientia", "KvStream: chunk of %d tokens exceeds max_prefill_rows %d", M, max_prefill_rows_);
+        return false;
+    }
     if (current_pos_ + M > max_context_len_) {
         LOG_ERROR("Conscientia", "KvStream: context of %d tokens exceeds max_context_len %d", current_pos_ + M, max_context_len_);
         return false;
@@ -83,7 +104,7 @@ void KvStream::prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipSt
     paged_qk_norm_rope_write_batch(io.qg, io.k, io.v, io.q_norm, io.k_norm, io.q_scratch, pool.pool_ptr(),
                                    cm_->d_block_table(0), fa_layer_idx, current_pos_, M, pool.max_blocks(),
                                    pool.block_size(), d_rope_table_, table_positions_, stream);
-    paged_prefill_attention_gated(io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), io.qg + hd, 2 * hd, io.attn_out,
+    paged_prefill_attention_gated(ws_prefill_, io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), io.qg + hd, 2 * hd, io.attn_out,
                                   fa_layer_idx, current_pos_, M, pool.max_blocks(), pool.block_size(),
                                   1.0f / std::sqrt((float)hd), stream);
 }
@@ -107,6 +128,7 @@ int KvStream::set_branch_count(int n)
     if (!cm_ || n < 0) return (int)branches_.size();
     if (n == (int)branches_.size()) return n;
     while ((int)branches_.size() > n) {                       // close the youngest
+        clear_mass_rows(branches_.back(), 1);
         cm_->release_branch(branches_.back());
         branches_.pop_back();
         pos_.pop_back();
@@ -131,8 +153,24 @@ int KvStream::set_branch_count(int n)
     return (int)branches_.size();
 }
 
+// The scorer folds its whole new-score buffer into the scores on every step.  The rows of a branch
+// that leaves the set must not be folded in again and again, nor be inherited by a later branch
+// that gets the same id: they are cleared when the branch closes (in the NULL stream, then
+// waited for: closing a branch is rare and happens between steps).
+void KvStream::clear_mass_rows(int first_branch, int count)
+{
+    if (!scorer_ || !scorer_->d_new_scores() || count <= 0) return;
+    const size_t stride = (size_t)cm_->table_stride();
+    if (drk_device_synchronize() != DRK_OK ||
+        drk_dev_memset_async(scorer_->d_new_scores() + (size_t)first_branch * stride, 0, (size_t)count * stride * sizeof(float),
+                             nullptr) != DRK_OK ||
+        drk_stream_synchronize(nullptr) != DRK_OK)
+        LOG_ERROR("Conscientia", "KvStream: clearing attention masses: %s", drk_last_error());
+}
+
 void KvStream::close_branches()
 {
+    if (!branches_.empty()) clear_mass_rows(branches_.front(), (int)branches_.size());
     for (int id : branches_) cm_->release_branch(id);
     branches_.clear();
     pos_.clear();
@@ -206,7 +244,7 @@ void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t s
     if (scorer_ && scorer_->d_new_scores()) {
         if (first_layer_of_step_ < 0) first_layer_of_step_ = fa_layer_idx;
         float* mass = scorer_->d_new_scores() + (size_t)branches_[0] * stride;
-        paged_gqa_decode_attention_branches_scored(io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
+        paged_gqa_decode_attention_branches_scored(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
                                                    io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(), scale,
                                                    mass, fa_layer_idx != first_layer_of_step_, stream);
         if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
@@ -214,13 +252,13 @@ void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t s
             LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
     } else if (B >= shared_min_branches_ && shared_tokens_ >= shared_min_tokens_) {
         // the branches' common prefix is streamed once for all of them
-        paged_gqa_decode_attention_shared(io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, shared_tokens_,
+        paged_gqa_decode_attention_shared(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, shared_tokens_,
                                           io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(), scale, stream);
         if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
                              ModelConfig::IO_DTYPE, stream) != DRK_OK)
             LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
     } else {
-        paged_gqa_decode_attention_gated_branches(io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, gate,
+        paged_gqa_decode_attention_gated_branches(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, gate,
                                                   2 * hd, io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(),
                                                   scale, stream);
     }

@@ -45,10 +45,16 @@ public:
     KvStream& operator=(const KvStream&) = delete;
 
     // cm must be initialised with max_branches >= 1 + the decode branches ever open at once.
-    // scorer (optional): decode attention reports the attention mass per block into it.
+    // scorer (optional): decode attention reports the attention mass per block into it; it must
+    // cover cm.max_branches() * cm.table_stride() cells (init fails otherwise).
     // d_rope_table (optional): see drk_rope_table_fill.
+    // max_prefill_rows: the longest chunk begin_prefill will be given.
+    // Two workspaces for split-K partials are reserved here, one for perception and one for
+    // decode, sized for max_context_len, every branch and max_prefill_rows: perception and decode
+    // may run on different streams at the same time, and nothing allocates after init -- a
+    // captured step keeps the addresses it was recorded with.
     bool init(CacheManager& cm, int max_context_len, ImportanceScorer* scorer = nullptr,
-              const float* d_rope_table = nullptr, int table_positions = 0);
+              const float* d_rope_table = nullptr, int table_positions = 0, int max_prefill_rows = 2048);
     void destroy();
 
     // ---- perception: the persistent stream, branch 0 -------------------------------------
@@ -111,10 +117,13 @@ private:
     int shared_min_branches_ = 4;
     int shared_min_tokens_ = 4096;
     void* graph_ = nullptr;
+    AttentionWorkspace ws_prefill_, ws_decode_;
+    int max_prefill_rows_ = 0;
     int first_layer_of_step_ = -1;   // the layer whose scored call overwrites instead of accumulating
 
     bool host_begin(hipStream_t stream);
     void host_end();
+    void clear_mass_rows(int first_branch, int count);
 };
 
 } // namespace deusridet

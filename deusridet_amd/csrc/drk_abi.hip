@@ -68,6 +68,53 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4 *__restrict
     if (acc == 0x9e3779b9u) *sink = acc;      // practically never: keeps the loads alive
 }
 
+// The decode kernels' access pattern: aligned granules (4 KiB = one 16-token K or V run of one kv
+// head at head_dim 128, 16-bit) visited in a scattered order.  With the granule count a power of
+// two, i -> (i * odd) mod count is a permutation; four granules are in flight per workgroup.
+__global__ __launch_bounds__(256) void read_probe_permuted_kernel(const uint8_t *__restrict__ p, unsigned ngran_log2,
+                                                                 unsigned gran_vec, unsigned *__restrict__ sink)
+{
+    unsigned acc = 0;
+    const unsigned ngran = 1u << ngran_log2, mask = ngran - 1;
+    const unsigned per = gran_vec / 256;                       // 16-byte loads per thread and granule
+    for (unsigned i = blockIdx.x * 4; i < ngran; i += gridDim.x * 4) {
+#pragma unroll
+        for (unsigned u = 0; u < 4; u++) {
+            const unsigned gi = ((i + u) * 2654435761u) & mask;
+            const uint8_t *q = p + (size_t)gi * gran_vec * 16;
+            for (unsigned j = 0; j < per; j++) {
+                const uint4 a = ld_stream128(q + ((size_t)j * 256 + threadIdx.x) * 16);
+                acc ^= a.x ^ a.y ^ a.z ^ a.w;
+            }
+        }
+    }
+    if (acc == 0x9e3779b9u) *sink = acc;
+}
+
+// Registers-only matrix-core loop: what v_mfma_f32_32x32x16_bf16 sustains on this part with no
+// memory traffic at all (four independent accumulator chains per wave, 8 waves per CU).
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, float *__restrict__ sink)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    probe_bf16x8 a, b;
+    for (int i = 0; i < 8; i++) { a[i] = (__bf16)(float)(threadIdx.x + i); b[i] = (__bf16)(float)(i + 1); }
+    probe_f32x16 c0 = {}, c1 = {}, c2 = {}, c3 = {};
+    for (int it = 0; it < iters; it++) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c3, 0, 0, 0);
+    }
+    float t = 0.0f;
+    for (int i = 0; i < 16; i++) t += c0[i] + c1[i] + c2[i] + c3[i];
+    if (t == 12345.678f) *sink = t;                           // practically never: keeps the chain alive
+#else
+    (void)iters; (void)sink;
+#endif
+}
+
 // positions and lengths of the decode branches move on by `delta` inside the stream (so that a
 // captured step advances them itself)
 __global__ void advance_i32_kernel(int32_t *__restrict__ a, int32_t *__restrict__ b, int n, int delta)
@@ -159,6 +206,11 @@ int drk_dev_memset_async(void *d_ptr, int byte, size_t bytes, void *stream)
 int drk_memcpy_h2d_async(void *d_dst, const void *h_src, size_t bytes, void *stream)
 {
     DRK_HIP(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_memcpy_d2d_async(void *d_dst, const void *d_src, size_t bytes, void *stream)
+{
+    DRK_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
     return DRK_OK;
 }
 int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream)
@@ -282,6 +334,49 @@ int drk_stream_synchronize(void *stream)
     DRK_HIP(hipStreamSynchronize((hipStream_t)stream));
     return DRK_OK;
 }
+int drk_stream_is_capturing(void *stream, int *capturing)
+{
+    if (!capturing) return fail(DRK_ERR_INVALID, "capturing is NULL");
+    *capturing = 0;
+    if (!stream) return DRK_OK;                       // the NULL stream cannot be captured
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    DRK_HIP(hipStreamIsCapturing((hipStream_t)stream, &st));
+    *capturing = st != hipStreamCaptureStatusNone;
+    return DRK_OK;
+}
+
+// events: order one stream behind what another has been given so far, without stalling the device
+int drk_event_create(void **event)
+{
+    if (!event) return fail(DRK_ERR_INVALID, "event is NULL");
+    hipEvent_t e;
+    DRK_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    *event = (void *)e;
+    return DRK_OK;
+}
+int drk_event_destroy(void *event)
+{
+    if (event) DRK_HIP(hipEventDestroy((hipEvent_t)event));
+    return DRK_OK;
+}
+int drk_event_record(void *event, void *stream)
+{
+    if (!event) return fail(DRK_ERR_INVALID, "event is NULL");
+    DRK_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+    return DRK_OK;
+}
+int drk_event_synchronize(void *event)
+{
+    if (!event) return fail(DRK_ERR_INVALID, "event is NULL");
+    DRK_HIP(hipEventSynchronize((hipEvent_t)event));
+    return DRK_OK;
+}
+int drk_stream_wait_event(void *stream, void *event)
+{
+    if (!event) return fail(DRK_ERR_INVALID, "event is NULL");
+    DRK_HIP(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0));
+    return DRK_OK;
+}
 
 // Read-bandwidth probe: streams `bytes` of device memory with 128-bit loads and
 // returns the sustained GB/s over `iters` passes (5 warm-up passes first, the
@@ -308,6 +403,56 @@ int drk_probe_read_bandwidth(const void *d_ptr, size_t bytes, int iters, void *d
     DRK_HIP(hipEventDestroy(e0));
     DRK_HIP(hipEventDestroy(e1));
     *gbps = (float)((double)(nvec * 16) * iters / (ms * 1e-3) / 1e9);
+    return DRK_OK;
+}
+
+int drk_probe_read_bandwidth_permuted(const void *d_ptr, size_t bytes, int granule_bytes, int iters, void *d_sink,
+                                      float *gbps)
+{
+    if (!d_ptr || !d_sink || !gbps || iters < 1 || granule_bytes < 4096 || (granule_bytes % 4096))
+        return fail(DRK_ERR_INVALID, "probe: bad argument (granules are multiples of 4096 bytes)");
+    unsigned lg = 0;
+    while (((size_t)granule_bytes << (lg + 1)) <= bytes && lg < 30) lg++;      // largest power-of-two granule count that fits
+    if (((size_t)granule_bytes << lg) > bytes || lg < 10) return fail(DRK_ERR_INVALID, "probe: at least 1024 granules");
+    const unsigned gran_vec = (unsigned)granule_bytes / 16;
+    hipEvent_t e0, e1;
+    DRK_HIP(hipEventCreate(&e0));
+    DRK_HIP(hipEventCreate(&e1));
+    dim3 grid(256 * 8), block(256);
+    for (int i = 0; i < 3; i++)
+        hipLaunchKernelGGL(drk::read_probe_permuted_kernel, grid, block, 0, 0, (const uint8_t *)d_ptr, lg, gran_vec, (unsigned *)d_sink);
+    DRK_HIP(hipEventRecord(e0, 0));
+    for (int i = 0; i < iters; i++)
+        hipLaunchKernelGGL(drk::read_probe_permuted_kernel, grid, block, 0, 0, (const uint8_t *)d_ptr, lg, gran_vec, (unsigned *)d_sink);
+    DRK_HIP(hipEventRecord(e1, 0));
+    DRK_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    DRK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    DRK_HIP(hipEventDestroy(e0));
+    DRK_HIP(hipEventDestroy(e1));
+    *gbps = (float)((double)((size_t)granule_bytes << lg) * iters / (ms * 1e-3) / 1e9);
+    return DRK_OK;
+}
+
+int drk_probe_mfma_rate(int iters, void *d_sink, float *tflops)
+{
+    if (!d_sink || !tflops || iters < 1) return fail(DRK_ERR_INVALID, "probe: bad argument");
+    const int loop = 4096, wgs = 256 * 2;                      // 8 waves per CU, 4 chains each
+    hipEvent_t e0, e1;
+    DRK_HIP(hipEventCreate(&e0));
+    DRK_HIP(hipEventCreate(&e1));
+    hipLaunchKernelGGL(drk::mfma_probe_kernel, dim3(wgs), dim3(256), 0, 0, loop, (float *)d_sink);
+    DRK_HIP(hipEventRecord(e0, 0));
+    for (int i = 0; i < iters; i++)
+        hipLaunchKernelGGL(drk::mfma_probe_kernel, dim3(wgs), dim3(256), 0, 0, loop, (float *)d_sink);
+    DRK_HIP(hipEventRecord(e1, 0));
+    DRK_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    DRK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    DRK_HIP(hipEventDestroy(e0));
+    DRK_HIP(hipEventDestroy(e1));
+    const double flops = (double)iters * wgs * 4.0 /*waves*/ * loop * 4.0 /*chains*/ * (2.0 * 32 * 32 * 16);
+    *tflops = (float)(flops / (ms * 1e-3) / 1e12);
     return DRK_OK;
 }
 

@@ -8,6 +8,7 @@
 #include <stddef.h>
 
 #include "drk_kv.h"
+#include "drk_debug.h"
 
 namespace drk {
 
@@ -66,6 +67,8 @@ int launch_sigmoid_gate(const void *x, const void *gate, void *out, size_t rows,
                         int dtype, hipStream_t st);
 
 // persistent stream-K decode (drk_decode_stream.hip)
+constexpr int kStreamMaxUnits = 256;                          // 64-token tiles one workgroup may own (descriptor table in LDS)
+constexpr int kStreamMaxSplitTokens = kStreamMaxUnits * 64;   // the longest explicit split: 16 384 tokens
 extern int g_stream_wgs;
 extern int g_shared_splits;
 bool stream_decode_supported(const Lay &a, int B);
@@ -174,6 +177,7 @@ __device__ __forceinline__ uint32_t s_perm(uint32_t hi, uint32_t lo, uint32_t se
 // out once per dot product (1152 * sum of the other operand) instead of once per value.
 constexpr float kI8Bias = 1152.0f;
 constexpr uint32_t kF16Ones = 0x3C003C00u;
+constexpr uint32_t kBf16Ones = 0x3F803F80u;
 
 // four int8 codes -> two dwords of packed fp16 (1152 + code)
 __device__ __forceinline__ void int8x4_to_f16x4(uint32_t w, uint32_t &lo, uint32_t &hi)

@@ -524,6 +524,10 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     const int split = split_tokens ? split_tokens : choose_split(a, B, max_seq_len);
     const int S = (max_seq_len + split - 1) / split;
     const bool use_stream = !g_force_portable && g_decode_kernel != 2 && causal_base < 0 && stream_decode_supported(a, B);
+    // the persistent kernel keeps one descriptor per tile of a workgroup's run in LDS
+    if (use_stream && split_tokens > kStreamMaxSplitTokens)
+        return fail(DRK_ERR_INVALID, "decode: split_tokens %d exceeds %d (the tiled kernel's run length)", split_tokens,
+                    kStreamMaxSplitTokens);
     const size_t need = use_stream ? stream_workspace_need(a, B, max_seq_len, split_tokens) : workspace_need(a, B, max_seq_len, split);
     if (!workspace || workspace_bytes < need)
         return fail(DRK_ERR_WORKSPACE, "decode: workspace of %zu bytes, need %zu", workspace_bytes, need);

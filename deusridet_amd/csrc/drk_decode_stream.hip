@@ -129,7 +129,7 @@ struct StreamArgs {
     int lse_stride;
 };
 
-constexpr int kMaxUnits = 256;       // units one workgroup may own (descriptor table in LDS)
+constexpr int kMaxUnits = kStreamMaxUnits;    // units one workgroup may own (descriptor table in LDS)
 
 struct UnitDesc {                    // one 64-token tile of one (branch, kv head)
     int tile_lim;                    // tokens of the tile that exist: seq_len - tile*64 (may exceed 64)
@@ -322,7 +322,9 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
     const int U = A.unit_tiles > 0 ? A.unit_tiles : (T + (int)gridDim.x - 1) / (int)gridDim.x;
     const int u0 = (int)blockIdx.x * U;
     if (u0 >= T) return;
-    const int nunits = min(U, T - u0);
+    // the host sizes U from max_seq_len; a length on the device beyond that bound must not overrun the
+    // descriptor table (the tiles past it are then left out: the caller broke its promise)
+    const int nunits = min(min(U, T - u0), kMaxUnits);
     if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
     __syncthreads();
     for (int i = threadIdx.x; i < nunits * 4; i += 256) {
@@ -465,16 +467,6 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
         float p[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) p[j] = s_exp2(sc[j] - m_use);
-        const float rs = (p[0] + p[1]) + (p[2] + p[3]);
-        l_lane = fmaf(l_lane, alpha, rs);
-        if (A.lse_groups) {
-            float rt = rs;
-            rt += __shfl_xor(rt, 16);
-            rt += __shfl_xor(rt, 32);
-            const int gi = (flags >> 2) * 4 + w;
-            if (lane < GQ && gi < A.lse_stride)
-                A.lse_groups[(size_t)(ud.bq + lane) * A.lse_stride + gi] = rt > 0.0f ? m_use + __builtin_log2f(rt) : -INFINITY;
-        }
         uint2 pa;                                             // A operand of the second product: P[head c][tokens 4g..4g+3]
         {
             float pw[4];
@@ -492,6 +484,21 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
                 t = s_dot2<DOT>(pa.y, kF16Ones, t);
                 ps_lane = fmaf(ps_lane, alpha, t);
             }
+        }
+        // The row's denominator is the sum of the weights the second product multiplies -- the rounded
+        // ones, as in the prefill kernel -- so that numerator and denominator carry the same rounding.
+        // (int8: the product multiplies p times the V scale, rounded; its sum of plain p stays exact.)
+        float rs;
+        if (DT == DRK_INT8) rs = (p[0] + p[1]) + (p[2] + p[3]);
+        else rs = s_dot2<DOT>(pa.y, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, s_dot2<DOT>(pa.x, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, 0.0f));
+        l_lane = fmaf(l_lane, alpha, rs);
+        if (A.lse_groups) {
+            float rt = rs;
+            rt += __shfl_xor(rt, 16);
+            rt += __shfl_xor(rt, 32);
+            const int gi = (flags >> 2) * 4 + w;
+            if (lane < GQ && gi < A.lse_stride)
+                A.lse_groups[(size_t)(ud.bq + lane) * A.lse_stride + gi] = rt > 0.0f ? m_use + __builtin_log2f(rt) : -INFINITY;
         }
 
         // ---- O: rescale (register j of lane group g holds head 4g + j), then P V ----------------

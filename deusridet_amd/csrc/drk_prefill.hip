@@ -759,6 +759,24 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
+size_t drk_prefill_workspace_bytes_max(const drk_kv_layout *g, int max_seq_len, int max_rows)
+{
+    Lay a;
+    if (make_lay(g, &a) != DRK_OK || max_seq_len <= 0 || max_rows <= 0) return 0;
+    if (max_rows > max_seq_len) max_rows = max_seq_len;
+    const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 &&
+                      (a.bs % 16) == 0;
+    if (!mfma) return drk_decode_workspace_bytes(g, max_rows, max_seq_len);
+    // the pieces per row grow with the context: the chunk that ends at max_seq_len needs the most for its length
+    size_t need = 0;
+    const int top = max_rows < kSplitMaxM ? max_rows : kSplitMaxM;
+    for (int M = 1; M <= top; M++) {
+        const size_t n = drk_prefill_workspace_bytes(g, max_seq_len - M, M);
+        if (n > need) need = n;
+    }
+    return need;
+}
+
 // paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630.
 // head_dim 128 or 256, block_size a multiple of 16: the MFMA kernel above (no workspace; any
 // group size; 8-bit pages are dequantised on their way into LDS).  Anything else: row t of the

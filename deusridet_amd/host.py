@@ -68,11 +68,17 @@ SIGNATURES = {
     "drkh_paged_gqa_decode_attention_shared": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _i32, _i32, _i32,
                                                       _f32, _vp]),
     "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
-    "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32]),
+    "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32, _vp]),
+    "drkh_paged_attention_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
+    "drkh_set_rope_table": (None, [_vp, _i32]),
+    "drkh_full_attention_forward_paged": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
+                                                 C.POINTER(_vp), _vp, _vp]),
+    "drkh_full_attention_forward_paged_prefill": (None, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
+                                                         _i32, C.POINTER(_vp), _vp]),
     "drkh_paged_attention_release_workspace": (None, []),
     "drkh_kvs_create": (_vp, []),
     "drkh_kvs_destroy": (None, [_vp]),
-    "drkh_kvs_init": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32]),
+    "drkh_kvs_init": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _i32]),
     "drkh_kvs_begin_prefill": (_i32, [_vp, _i32, _vp]),
     "drkh_kvs_prefill_layer": (None, [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp]),
     "drkh_kvs_end_prefill": (None, [_vp, _i32]),
@@ -178,10 +184,10 @@ class KvStream:
     def __del__(self):
         _destroy(self, "drkh_kvs_destroy")
 
-    def init(self, cm, max_context_len, scorer=None, rope_table=None, table_positions=0):
+    def init(self, cm, max_context_len, scorer=None, rope_table=None, table_positions=0, max_prefill_rows=2048):
         self._cm, self._scorer = cm, scorer
         return bool(lib().drkh_kvs_init(self._h, cm._h, max_context_len, scorer._h if scorer else None, rope_table,
-                                        table_positions))
+                                        table_positions, max_prefill_rows))
 
     def begin_prefill(self, M, stream=None): return bool(lib().drkh_kvs_begin_prefill(self._h, M, stream))
     def prefill_layer(self, layer, io, M, stream=None): lib().drkh_kvs_prefill_layer(self._h, layer, *io, M, stream)

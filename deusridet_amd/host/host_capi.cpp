@@ -248,9 +248,10 @@ static KvLayerIO make_io(const void *qg, const void *k, const void *v, const voi
 }
 void *drkh_kvs_create(void) { return new KvStream(); }
 void drkh_kvs_destroy(void *ks) { delete KS(ks); }
-int drkh_kvs_init(void *ks, void *cm, int max_context_len, void *scorer, const float *d_rope_table, int table_positions)
+int drkh_kvs_init(void *ks, void *cm, int max_context_len, void *scorer, const float *d_rope_table, int table_positions,
+                  int max_prefill_rows)
 {
-    return KS(ks)->init(*CM(cm), max_context_len, SC(scorer), d_rope_table, table_positions) ? 1 : 0;
+    return KS(ks)->init(*CM(cm), max_context_len, SC(scorer), d_rope_table, table_positions, max_prefill_rows) ? 1 : 0;
 }
 int drkh_kvs_begin_prefill(void *ks, int M, void *stream) { return KS(ks)->begin_prefill(M, (hipStream_t)stream) ? 1 : 0; }
 void drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
@@ -292,9 +293,68 @@ void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_poo
                                                H(out), fa_layer_idx, max_phys_blocks, block_size, scale, d_block_mass,
                                                accumulate != 0, (hipStream_t)stream);
 }
-int drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size)
+int drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size,
+                                           void *stream)
 {
-    return paged_attention_reserve_workspace(max_branches, max_seq_len, max_prefill_rows, block_size) ? 1 : 0;
+    return paged_attention_reserve_workspace(max_branches, max_seq_len, max_prefill_rows, block_size, ST(stream)) ? 1 : 0;
+}
+size_t drkh_paged_attention_workspace_bytes(int max_branches, int max_seq_len, int max_prefill_rows, int block_size)
+{
+    return paged_attention_workspace_bytes(max_branches, max_seq_len, max_prefill_rows, block_size);
+}
+
+// The two layer wrappers with the projections served from buffers: the GEMMs are the model's
+// code, so the shim registers a stand-in that copies M rows of a precomputed projection
+// (Linear::weight points at it) into place, and passes the gated attention output through
+// as the "O projection" (weight NULL).
+static void projection_from_buffer(const __half *x, const Linear &w, __half *y, int M, hipStream_t stream)
+{
+    const void *src = w.weight ? (const void *)w.weight : (const void *)x;
+    drk_memcpy_d2d_async(y, src, (size_t)M * w.out_features * sizeof(__half), stream);
+}
+
+static void wrapper_operands(FullAttentionWeights &attn, InferenceState &st, const void *qg_proj, const void *k_proj,
+                             const void *v_proj, const void *q_norm, const void *k_norm, void *const *state_bufs,
+                             int32_t *d_pos)
+{
+    const int qd = ModelConfig::NUM_ATTN_HEADS * ModelConfig::HEAD_DIM, kd = ModelConfig::NUM_KV_HEADS * ModelConfig::HEAD_DIM;
+    attn.fp16_q.weight = H(const_cast<void *>(qg_proj)); attn.fp16_q.out_features = 2 * qd;
+    attn.fp16_k.weight = H(const_cast<void *>(k_proj));  attn.fp16_k.out_features = kd;
+    attn.fp16_v.weight = H(const_cast<void *>(v_proj));  attn.fp16_v.out_features = kd;
+    attn.fp16_o.weight = nullptr;                        attn.fp16_o.out_features = qd;
+    attn.q_norm = H(const_cast<void *>(q_norm));
+    attn.k_norm = H(const_cast<void *>(k_norm));
+    st.q_buf = H(state_bufs[0]); st.kv_buf = H(state_bufs[1]); st.dn_z = H(state_bufs[2]); st.dn_qkv = H(state_bufs[3]);
+    st.attn_out = H(state_bufs[4]); st.norm_out = H(state_bufs[5]);
+    st.d_pos = d_pos;
+    set_linear_forward(projection_from_buffer);
+}
+
+void drkh_set_rope_table(const float *d_rope_table, int table_positions) { set_rope_table(d_rope_table, table_positions); }
+
+void drkh_full_attention_forward_paged(const void *qg_proj, const void *k_proj, const void *v_proj, const void *q_norm,
+                                       const void *k_norm, void *kv_pool, const int32_t *d_block_table, int fa_layer_idx,
+                                       int pos, int seq_len, int max_phys_blocks, int block_size, void *const *state_bufs,
+                                       int32_t *d_pos, void *stream)
+{
+    FullAttentionWeights attn;
+    InferenceState st;
+    wrapper_operands(attn, st, qg_proj, k_proj, v_proj, q_norm, k_norm, state_bufs, d_pos);
+    full_attention_forward_paged(nullptr, attn, H(kv_pool), d_block_table, fa_layer_idx, pos, seq_len, max_phys_blocks,
+                                 block_size, st, ST(stream));
+}
+
+void drkh_full_attention_forward_paged_prefill(const void *qg_proj, const void *k_proj, const void *v_proj,
+                                               const void *q_norm, const void *k_norm, void *kv_pool,
+                                               const int32_t *d_block_table, int fa_layer_idx, int pos_start, int M,
+                                               int seq_len, int max_phys_blocks, int block_size, void *const *state_bufs,
+                                               void *stream)
+{
+    FullAttentionWeights attn;
+    InferenceState st;
+    wrapper_operands(attn, st, qg_proj, k_proj, v_proj, q_norm, k_norm, state_bufs, nullptr);
+    full_attention_forward_paged_prefill(nullptr, attn, H(kv_pool), d_block_table, fa_layer_idx, pos_start, M, seq_len,
+                                         max_phys_blocks, block_size, st, ST(stream));
 }
 void drkh_paged_attention_release_workspace(void) { paged_attention_release_workspace(); }
 void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,

@@ -6,8 +6,40 @@
 #pragma once
 
 #include "drk_kv.h"
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime_api.h>
 
 namespace deusridet {
+
+// The members of the reference's weight and state structs that the two layer wrappers
+// full_attention_forward_paged[_prefill] read (src/machina/model.h:89-93, 132-146, 232-293);
+// same names, same meaning.  A build inside the reference's tree uses its own model.h instead.
+struct Linear {                      // model.h:89-93
+    __half* weight = nullptr;        // [out_features, in_features] row-major
+    int in_features  = 0;
+    int out_features = 0;
+};
+
+struct FullAttentionWeights {        // model.h:132-146
+    Linear fp16_q;                   // hidden -> NUM_ATTN_HEADS * HEAD_DIM * 2 (Q | gate, interleaved per head)
+    Linear fp16_k;                   // hidden -> NUM_KV_HEADS * HEAD_DIM
+    Linear fp16_v;
+    Linear fp16_o;                   // NUM_ATTN_HEADS * HEAD_DIM -> hidden
+    __half* q_norm = nullptr;        // [HEAD_DIM]
+    __half* k_norm = nullptr;        // [HEAD_DIM]
+};
+
+struct InferenceState {              // model.h:232-293, the buffers this path touches
+    __half* norm_out = nullptr;      // [max_seq, hidden]            O projection lands here
+    __half* attn_out = nullptr;      // [max_seq, NUM_ATTN_HEADS * HEAD_DIM]
+    __half* q_buf    = nullptr;      // [max_seq, NUM_ATTN_HEADS * HEAD_DIM * 2]   Q | gate projection
+    __half* kv_buf   = nullptr;      // [max_seq, NUM_KV_HEADS * HEAD_DIM]         K projection (prefill)
+    __half* mlp_gate = nullptr;      // scratch the reference parks the gate in; not written here
+    __half* dn_qkv   = nullptr;      // [max_seq, >= NUM_ATTN_HEADS * HEAD_DIM]    rope(norm(q))
+    __half* dn_z     = nullptr;      // [max_seq, >= 2 * NUM_KV_HEADS * HEAD_DIM]  K, V projections (decode), V (prefill)
+    int*    d_pos    = nullptr;      // [1] device: current sequence position
+    hipStream_t compute_stream = nullptr;
+};
 
 struct ModelConfig {
     static int NUM_ATTN_HEADS;   // model.h:39

@@ -13,8 +13,19 @@
 // (paged_attention.cu:359-368, stream.cpp:319-334).
 //
 // The two full-layer wrappers of the reference (full_attention_forward_paged*,
-// paged_attention.h:75-106) run projections, norms and RoPE around these calls;
-// they belong to the model code and keep calling the functions below.
+// paged_attention.h:75-106) are at the end of this header: every step but the four
+// projections is this library's; the projections go through a function the model code
+// registers (set_linear_forward).
+//
+// Split-K partials.  The attention calls keep partial results in device memory.  The calls
+// with the reference's signatures take that memory from a workspace this library keeps PER
+// STREAM, so that a prefill on one stream and a decode on another never share partials.
+// Such a workspace grows on demand -- by a new allocation; the old buffer is kept until
+// paged_attention_release_workspace(), so work already enqueued, or a captured graph, never
+// loses the memory it was launched with -- and never while its stream is being captured.
+// Overloads that take an AttentionWorkspace use the caller's buffer instead and never
+// allocate: a decode call that does not fit logs an error and launches nothing, a short
+// prefill chunk that does not fit runs unsplit.
 #pragma once
 
 #include "model.h"
@@ -22,6 +33,34 @@
 #include <hip/hip_runtime_api.h>
 
 namespace deusridet {
+
+// Device memory for split-K partials, owned by the caller: reserved once, never moved.
+class AttentionWorkspace {
+public:
+    AttentionWorkspace() = default;
+    ~AttentionWorkspace();
+    AttentionWorkspace(const AttentionWorkspace&) = delete;
+    AttentionWorkspace& operator=(const AttentionWorkspace&) = delete;
+
+    // Allocates `bytes` (16-byte aligned).  True when the workspace already holds at least
+    // that much; false -- and nothing changes -- when it holds less (it is never reallocated:
+    // launches already enqueued, or a captured graph, may be using it) or the allocation fails.
+    bool reserve(size_t bytes);
+    // Enough for every attention call of up to max_branches branches (and the shared-prefix and
+    // scored variants), contexts up to max_seq_len and prefill chunks of up to max_prefill_rows.
+    bool reserve_for(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
+    // Frees the buffer; the caller makes sure nothing on the device still uses it.
+    void release();
+    void*  ptr() const { return ptr_; }
+    size_t bytes() const { return bytes_; }
+
+private:
+    void* ptr_ = nullptr;
+    size_t bytes_ = 0;
+};
+
+// The size AttentionWorkspace::reserve_for allocates.
+size_t paged_attention_workspace_bytes(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
 
 // ---- the reference's entry points --------------------------------------------
 void paged_kv_cache_write(const __half* src_k, const __half* src_v, __half* kv_pool, const int* d_block_table,
@@ -106,11 +145,71 @@ void paged_gqa_decode_attention_branches_scored(const __half* Q, __half* kv_pool
                                                 int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
                                                 float* d_block_mass, bool accumulate, hipStream_t stream = 0);
 
-// The attention calls keep split-K partials in a device workspace that this
-// library owns and grows on demand (device allocation = implicit sync).  Call
-// this once up front with the largest shapes to keep the steady state free of
-// allocations, e.g. before capturing a HIP graph.  false on allocation failure.
-bool paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
+// ---- the same attention calls on a workspace of the caller's ---------------------
+void paged_gqa_decode_attention(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
+                                __half* out, int fa_layer_idx, int seq_len, int max_phys_blocks, int block_size,
+                                float scale, hipStream_t stream = 0);
+void paged_prefill_attention(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
+                             __half* out, int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
+                             float scale, hipStream_t stream = 0);
+void paged_gqa_decode_attention_branches(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_tables,
+                                         int table_stride, const int* d_seq_lens, int B, int max_seq_len, __half* out,
+                                         int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                         hipStream_t stream = 0);
+void paged_gqa_decode_attention_shared(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_tables,
+                                       int table_stride, const int* d_seq_lens, int B, int max_seq_len,
+                                       int shared_tokens, __half* out, int fa_layer_idx, int max_phys_blocks,
+                                       int block_size, float scale, hipStream_t stream = 0);
+void paged_gqa_decode_attention_gated_branches(AttentionWorkspace& ws, const __half* Q, __half* kv_pool,
+                                               const int* d_tables, int table_stride, const int* d_seq_lens, int B,
+                                               int max_seq_len, const __half* gate, int gate_stride, __half* out,
+                                               int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                               hipStream_t stream = 0);
+void paged_prefill_attention_gated(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
+                                   const __half* gate, int gate_stride, __half* out, int fa_layer_idx, int pos_start,
+                                   int M, int max_phys_blocks, int block_size, float scale, hipStream_t stream = 0);
+void paged_gqa_decode_attention_branches_scored(AttentionWorkspace& ws, const __half* Q, __half* kv_pool,
+                                                const int* d_tables, int table_stride, const int* d_seq_lens, int B,
+                                                int max_seq_len, __half* out, int fa_layer_idx, int max_phys_blocks,
+                                                int block_size, float scale, float* d_block_mass, bool accumulate,
+                                                hipStream_t stream = 0);
+
+// ---- the per-stream workspaces behind the calls that take none ---------------------
+// Reserve the workspace of `stream` up front for the largest shapes, so that the steady
+// state is free of allocations (a device allocation is an implicit synchronisation, and is
+// not allowed while a stream is being captured).  false on allocation failure.
+bool paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size,
+                                       hipStream_t stream = 0);
+// Waits for the device, then frees every per-stream workspace, retired buffers included.
 void paged_attention_release_workspace();
+
+// ---- the reference's two layer wrappers -----------------------------------------------
+// The projections of the wrappers below (fp16_gemv / linear_forward in the reference,
+// paged_attention.cu:326, 340-343, 373, 576-582, 637) are the model's code: y [M, out_features]
+// = x [M, in_features] W^T.  Registered once; without it the wrappers log an error and return.
+using LinearForwardFn = void (*)(const __half* x, const Linear& w, __half* y, int M, hipStream_t stream);
+void set_linear_forward(LinearForwardFn fn);
+// Optional cos/sin table for the wrappers' RoPE step (float [table_positions][ROTARY_DIM/2][2], see
+// drk_rope_table_fill); without one, and for positions beyond it, the kernel evaluates
+// pos * theta^(-2 pair / rotary_dim) and its cos / sin itself, as the reference's kernels do.
+void set_rope_table(const float* d_rope_table, int table_positions);
+
+// full_attention_forward_paged, paged_attention.h:75-86 / paged_attention.cu:314-376: one
+// token at position `pos` (also in *state.d_pos), seq_len = pos + 1.  Q|gate, K and V
+// projections (K, V into state.dn_z), then ONE launch for split + per-head RMSNorm + partial
+// RoPE + page write (rope(norm(q)) lands in state.dn_qkv), attention into state.attn_out,
+// sigmoid gate read in place from state.q_buf, O projection into state.norm_out.
+void full_attention_forward_paged(const __half* x, const FullAttentionWeights& attn, __half* kv_pool,
+                                  const int* d_block_table, int fa_layer_idx, int pos, int seq_len,
+                                  int max_phys_blocks, int block_size, InferenceState& state, hipStream_t stream = 0);
+
+// full_attention_forward_paged_prefill, paged_attention.h:92-104 / paged_attention.cu:563-638:
+// M tokens at pos_start .. pos_start + M - 1; K into state.kv_buf, V into state.dn_z; two
+// launches (fused split/norm/RoPE/write, MFMA prefill attention with the gate in its epilogue)
+// between the projections.
+void full_attention_forward_paged_prefill(const __half* x, const FullAttentionWeights& attn, __half* kv_pool,
+                                          const int* d_block_table, int fa_layer_idx, int pos_start, int M,
+                                          int seq_len, int max_phys_blocks, int block_size, InferenceState& state,
+                                          hipStream_t stream = 0);
 
 } // namespace deusridet

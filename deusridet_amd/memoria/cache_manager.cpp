@@ -27,6 +27,11 @@ bool CacheManager::setup_tables(int max_branches)
     next_stamp_ = 1;
     evictable_.clear();
     refs_.assign(pool_.max_blocks(), {});
+    held_.assign(cells, 0);
+    held_cells_.clear();
+    copy_pin_.assign(pool_.max_blocks(), 0);
+    pending_copies_issued_.clear();
+    deferred_release_.clear();
     ssd_paths_.assign(cells, std::string());
     seq_len_.assign(max_branches_, 0);
     alive_.assign(max_branches_, 0);
@@ -104,6 +109,15 @@ void CacheManager::mark_dirty(int branch, int logical)
     dirty_hi_[branch] = std::max(dirty_hi_[branch], logical + 1);
 }
 
+// A resident cell is a candidate for eviction when its block has no other reference, the cell
+// is not held (see hold_nolock) and no queued copy names the block.
+void CacheManager::candidate_add_nolock(int c)
+{
+    if (!held_[c] && copy_pin_[h_tables_[c]] == 0) evictable_.insert({stamp_[c], c});
+}
+
+void CacheManager::candidate_remove_nolock(int c) { evictable_.erase({stamp_[c], c}); }
+
 // The cell takes a reference on `phys` that alloc_block()/retain() has already
 // counted in the pool.
 void CacheManager::attach_nolock(int c, int phys, bool fresh_stamp)
@@ -112,9 +126,9 @@ void CacheManager::attach_nolock(int c, int phys, bool fresh_stamp)
     location_[c] = BlockLocation::GPU;
     if (fresh_stamp || stamp_[c] == 0) stamp_[c] = next_stamp_++;
     std::vector<int>& r = refs_[phys];
-    if (r.size() == 1) evictable_.erase({stamp_[r[0]], r[0]});   // the sole owner is now sharing
+    if (r.size() == 1) candidate_remove_nolock(r[0]);            // the sole owner is now sharing
     r.push_back(c);
-    if (r.size() == 1) evictable_.insert({stamp_[c], c});
+    if (r.size() == 1) candidate_add_nolock(c);
 }
 
 // The cell gives up its reference; the block is freed when it was the last.
@@ -122,25 +136,77 @@ void CacheManager::detach_nolock(int c)
 {
     int phys = h_tables_[c];
     std::vector<int>& r = refs_[phys];
-    if (r.size() == 1) evictable_.erase({stamp_[c], c});
+    if (r.size() == 1) candidate_remove_nolock(c);
     r.erase(std::remove(r.begin(), r.end(), c), r.end());
-    pool_.release(phys);
-    if (r.size() == 1) evictable_.insert({stamp_[r[0]], r[0]});
+    // a block that a queued copy still reads or writes keeps its last reference until the copy has
+    // been issued: nobody else may be handed the block (and fill it) before that
+    if (r.empty() && copy_pin_[phys] > 0) deferred_release_.push_back(phys);
+    else pool_.release(phys);
+    if (r.size() == 1) candidate_add_nolock(r[0]);
     h_tables_[c] = -1;
 }
 
-bool CacheManager::pick_victim_nolock(int& cell_out)
+// A cell that ensure_blocks_for has just made resident is about to be written by the caller's
+// next launches, and may be the target of a copy that is still queued: until the next
+// sync_block_table (which issues the copies) it must not be picked as a victim by a later
+// allocation of the same step -- the reference never evicts the block it is about to write.
+void CacheManager::hold_nolock(int c)
 {
-    if (evictable_.empty()) return false;
+    if (held_[c]) return;
+    held_[c] = 1;
+    held_cells_.push_back(c);
+    candidate_remove_nolock(c);
+}
+
+// The queued copies have been issued (or handed out): their blocks are ordinary blocks again,
+// and so are the cells of the step.
+void CacheManager::release_holds_nolock()
+{
+    std::vector<int> named;
+    for (const auto& cp : pending_copies_issued_) {
+        copy_pin_[cp.first]--;
+        copy_pin_[cp.second]--;
+        named.push_back(cp.first);
+        named.push_back(cp.second);
+    }
+    pending_copies_issued_.clear();
+    for (int phys : deferred_release_) pool_.release(phys);
+    deferred_release_.clear();
+    for (int c : held_cells_) held_[c] = 0;
+    for (int c : held_cells_)
+        if (location_[c] == BlockLocation::GPU && refs_[h_tables_[c]].size() == 1) candidate_add_nolock(c);
+    held_cells_.clear();
+    for (int phys : named)
+        if (copy_pin_[phys] == 0 && refs_[phys].size() == 1) candidate_add_nolock(refs_[phys][0]);
+}
+
+// for_branch: the branch whose allocation needs room, or -1 for an explicit eviction request.
+bool CacheManager::pick_victim_nolock(int& cell_out, int for_branch)
+{
+    const std::set<std::pair<uint64_t, int>>* from = &evictable_;
+    std::set<std::pair<uint64_t, int>> last_resort;
+    if (evictable_.empty()) {
+        // Nothing but cells of the current step is left.  A branch that outgrows the pool loses its own
+        // oldest blocks, as the reference's single sequence does (cache_manager.cpp:306-319); an explicit
+        // request may take any of them; a block named by a queued copy, and another branch's block of this
+        // step, are never taken.
+        for (int c : held_cells_) {
+            if (location_[c] != BlockLocation::GPU || refs_[h_tables_[c]].size() != 1 || copy_pin_[h_tables_[c]] > 0) continue;
+            if (for_branch >= 0 && c / max_logical_blocks_ != for_branch) continue;
+            last_resort.insert({stamp_[c], c});
+        }
+        if (last_resort.empty()) return false;
+        from = &last_resort;
+    }
     if (!scorer_) {                               // oldest first (cache_manager.cpp:203-204)
-        cell_out = evictable_.begin()->second;
+        cell_out = from->begin()->second;
         return true;
     }
     // least important; the first minimum in LRU order wins (cache_manager.cpp:188-201,
     // importance_scorer.cu:75-87)
     bool have = false;
     float best = 0.0f;
-    for (const auto& e : evictable_) {
+    for (const auto& e : *from) {
         float s = scorer_->score(e.second);       // by table cell; branch 0: the logical block index
         if (!have || s < best) {
             have = true;
@@ -151,23 +217,41 @@ bool CacheManager::pick_victim_nolock(int& cell_out)
     return have;
 }
 
-int CacheManager::evict_nolock(int n)
+int CacheManager::evict_nolock(int n, int for_branch)
 {
     int evicted = 0;
+    const bool to_ssd = ssd_enabled_ && swapper_ && swapper_->ready();
+    // With the overflow tier every victim's swap-out is submitted first and all of them are waited
+    // for once (the swapper pipelines them: one block's copy runs while its neighbour's file is
+    // written).  A freed block cannot be handed out before that: the lock is held until then.
+    std::vector<std::pair<int, char>> outcome;    // (cell, swap-out succeeded); the flags are written by the swapper's thread
+    if (to_ssd) outcome.reserve(std::min((size_t)std::max(n, 0), evictable_.size() + held_cells_.size()));   // never reallocated: the flags are pointed at
     while (evicted < n) {
         int c;
-        if (!pick_victim_nolock(c)) break;
+        if (!pick_victim_nolock(c, for_branch)) break;
         int branch = c / max_logical_blocks_, logical = c % max_logical_blocks_;
-        BlockLocation where = BlockLocation::INVALID;
-        if (ssd_enabled_ && swapper_ && swapper_->ready()) {          // cache_manager.cpp:132-141
-            if (swap_to_ssd_nolock(c)) where = BlockLocation::SSD;
-            else LOG_WARN("Memoria", "SSD swap-out failed for block %d of branch %d, discarding", logical, branch);
+        if (to_ssd) {                                                 // cache_manager.cpp:132-141
+            outcome.push_back({c, 0});
+            submit_swap_out_nolock(c, &outcome.back().second);
         }
         detach_nolock(c);                         // frees the block: it had one reference
-        location_[c] = where;
+        location_[c] = BlockLocation::INVALID;
         stamp_[c] = 0;
         mark_dirty(branch, logical);
         evicted++;
+    }
+    if (to_ssd && !outcome.empty()) {
+        swapper_->drain();
+        for (const auto& o : outcome) {
+            const int c = o.first;
+            if (o.second) {
+                location_[c] = BlockLocation::SSD;
+                ssd_paths_[c] = ssd_path_for(c);
+            } else {
+                LOG_WARN("Memoria", "SSD swap-out failed for block %d of branch %d, discarding", c % max_logical_blocks_,
+                         c / max_logical_blocks_);
+            }
+        }
     }
     if (evicted > 0)
         LOG_INFO("Memoria", "Evicted %d blocks (SSD=%s), %d free now", evicted,
@@ -175,19 +259,19 @@ int CacheManager::evict_nolock(int n)
     return evicted;
 }
 
-bool CacheManager::ensure_free_nolock(int n_free)
+bool CacheManager::ensure_free_nolock(int n_free, int for_branch)
 {
-    while (pool_.free_count() < n_free) {
-        if (evict_nolock(1) == 0) return false;
+    while (pool_.free_count() < n_free) {         // the whole deficit in one batch (one wait for the overflow tier)
+        if (evict_nolock(n_free - pool_.free_count(), for_branch) == 0) return false;
     }
     return true;
 }
 
-int CacheManager::alloc_phys_nolock()
+int CacheManager::alloc_phys_nolock(int for_branch)
 {
     int phys = pool_.alloc_block();
     if (phys < 0) {                               // cache_manager.cpp:311-319
-        if (!ensure_free_nolock(1)) {
+        if (!ensure_free_nolock(1, for_branch)) {
             LOG_ERROR("Memoria", "Cannot allocate a block: pool exhausted, eviction failed");
             return -1;
         }
@@ -207,21 +291,30 @@ bool CacheManager::ensure_nolock(int branch, int pos)
     int c = (int)cell(branch, logical);
     if (location_[c] == BlockLocation::GPU) {
         int phys = h_tables_[c];
+        hold_nolock(c);                           // before any allocation below can look for a victim
         if (pool_.refcount(phys) > 1) {
             // copy-on-write: the write must not be seen by the other tables
-            int fresh = alloc_phys_nolock();
+            int fresh = alloc_phys_nolock(branch);
             if (fresh < 0) return false;
             pending_copies_.push_back({phys, fresh});
+            pending_copies_issued_.push_back({phys, fresh});
+            copy_pin_[phys]++;                    // neither block changes hands before the copy is issued
+            copy_pin_[fresh]++;
             detach_nolock(c);                     // the old block keeps its other references
             attach_nolock(c, fresh, false);       // same place in the LRU order
             mark_dirty(branch, logical);
         }
         return true;
     }
-    if (location_[c] == BlockLocation::SSD) return swap_from_ssd_nolock(c);   // cache_manager.cpp:88-90
-    int phys = alloc_phys_nolock();
+    if (location_[c] == BlockLocation::SSD) {     // cache_manager.cpp:88-90
+        if (!swap_from_ssd_nolock(c)) return false;
+        hold_nolock(c);
+        return true;
+    }
+    int phys = alloc_phys_nolock(branch);
     if (phys < 0) return false;
     attach_nolock(c, phys, true);                 // cache_manager.cpp:321-323
+    hold_nolock(c);
     mark_dirty(branch, logical);
     return true;
 }
@@ -234,24 +327,18 @@ std::string CacheManager::ssd_path_for(int c) const
     return cache_dir_ + "/" + name + ".kv";
 }
 
-// cache_manager.cpp:215-243: synchronous on the eviction path; the caller frees the block
-bool CacheManager::swap_to_ssd_nolock(int c)
+// cache_manager.cpp:215-243: the request is queued; *ok is set by the swapper's thread before the
+// request counts as complete (the caller drains before it reads the flag or lets the block go)
+void CacheManager::submit_swap_out_nolock(int c, char* ok)
 {
-    int phys = h_tables_[c];
-    if (phys < 0) return false;
-    std::string path = ssd_path_for(c);
-    bool success = false;
     SwapRequest req;
     req.direction = SwapDirection::GPU_TO_SSD;
     req.logical_block_idx = c;
-    req.physical_block_id = phys;
-    req.ssd_path = path;
-    req.callback = [&success](bool ok) { success = ok; };
+    req.physical_block_id = h_tables_[c];
+    req.ssd_path = ssd_path_for(c);
+    req.callback = [ok](bool success) { *ok = success ? 1 : 0; };
     swapper_->drop_prefetch(c);                   // a stale prefetched image must not outlive the new file
     swapper_->submit(std::move(req));
-    swapper_->drain();
-    if (success) ssd_paths_[c] = path;
-    return success;
 }
 
 // cache_manager.cpp:245-292.  The fresh block comes from the ordinary allocation path (which
@@ -259,7 +346,7 @@ bool CacheManager::swap_to_ssd_nolock(int c)
 bool CacheManager::swap_from_ssd_nolock(int c)
 {
     if (!swapper_ || !swapper_->ready()) return false;
-    int phys = alloc_phys_nolock();
+    int phys = alloc_phys_nolock(c / max_logical_blocks_);
     if (phys < 0) return false;
     bool success = false;
     SwapRequest req;
@@ -341,6 +428,7 @@ void CacheManager::flush_copies(hipStream_t stream)
 void CacheManager::sync_block_table(hipStream_t stream)
 {
     std::lock_guard<std::mutex> lock(mu_);
+    if (swapper_ && swapper_->ready()) swapper_->add_writer_stream(stream);   // swaps order themselves behind this stream
     if (!detached_ && d_tables_) {
         flush_copies(stream);
         for (int b = 0; b < max_branches_; b++) {
@@ -355,6 +443,7 @@ void CacheManager::sync_block_table(hipStream_t stream)
         dirty_lo_[b] = max_logical_blocks_;
         dirty_hi_[b] = 0;
     }
+    if (!detached_) release_holds_nolock();       // the copies are issued: the step's cells are ordinary cells again
 }
 
 int CacheManager::seq_len(int branch) const
@@ -416,6 +505,12 @@ void CacheManager::release_branch(int branch)
         stamp_[c] = 0;
         mark_dirty(branch, l);
     }
+    // a hold on a cell of this branch has nothing left to protect
+    held_cells_.erase(std::remove_if(held_cells_.begin(), held_cells_.end(), [&](int c) {
+                          if (c / max_logical_blocks_ != branch) return false;
+                          held_[c] = 0;
+                          return true;
+                      }), held_cells_.end());
     seq_len_[branch] = 0;
     if (branch != 0) alive_[branch] = 0;
 }
@@ -455,9 +550,9 @@ void CacheManager::touch_block(int branch, int logical_idx)
     int c = (int)cell(branch, logical_idx);
     if (location_[c] != BlockLocation::GPU) return;
     bool sole = refs_[h_tables_[c]].size() == 1;
-    if (sole) evictable_.erase({stamp_[c], c});
+    if (sole) candidate_remove_nolock(c);
     stamp_[c] = next_stamp_++;
-    if (sole) evictable_.insert({stamp_[c], c});
+    if (sole) candidate_add_nolock(c);
 }
 
 BlockLocation CacheManager::block_location(int branch, int logical_idx) const
@@ -471,13 +566,13 @@ BlockLocation CacheManager::block_location(int branch, int logical_idx) const
 int CacheManager::evict_blocks(int n)
 {
     std::lock_guard<std::mutex> lock(mu_);
-    return evict_nolock(n);
+    return evict_nolock(n, -1);
 }
 
 bool CacheManager::ensure_free_blocks(int n_free)
 {
     std::lock_guard<std::mutex> lock(mu_);
-    return ensure_free_nolock(n_free);
+    return ensure_free_nolock(n_free, -1);
 }
 
 void CacheManager::prefetch_block(int branch, int logical_idx)
@@ -518,6 +613,7 @@ std::vector<std::pair<int, int>> CacheManager::take_pending_copies()
     std::lock_guard<std::mutex> lock(mu_);
     std::vector<std::pair<int, int>> out;
     out.swap(pending_copies_);
+    release_holds_nolock();                       // detached: handing the copies out is this manager's "issued"
     return out;
 }
 
@@ -537,6 +633,11 @@ void CacheManager::destroy()
     stamp_.clear();
     evictable_.clear();
     refs_.clear();
+    held_.clear();
+    held_cells_.clear();
+    copy_pin_.clear();
+    pending_copies_issued_.clear();
+    deferred_release_.clear();
     seq_len_.clear();
     alive_.clear();
     dirty_lo_.clear();

@@ -12,6 +12,9 @@
 //     reference allocates a fresh block, queues a device copy of every layer and
 //     remaps the entry; the copies are issued by sync_block_table(), ahead of the
 //     table upload, on the caller's stream;
+//   - a cell that ensure_blocks_for() has made resident is not a victim until the next
+//     sync_block_table(): a later allocation of the same step never takes the block the
+//     caller is about to write, or the target of a copy that is still queued;
 //   - refcount-aware eviction: an entry whose block is shared is pinned; victims
 //     are taken in LRU order (allocation order, moved to the back by
 //     touch_block()) or by lowest importance when a scorer is attached;
@@ -142,6 +145,11 @@ private:
     uint64_t next_stamp_ = 1;
     std::set<std::pair<uint64_t, int>> evictable_;   // resident cells whose block has one reference
     std::vector<std::vector<int>> refs_;       // physical block -> cells that reference it
+    std::vector<char> held_;                   // cell was ensured since the last sync_block_table: not a victim
+    std::vector<int> held_cells_;
+    std::vector<int> copy_pin_;                // physical block -> queued copies that name it (source or target)
+    std::vector<std::pair<int, int>> pending_copies_issued_;   // the pairs behind copy_pin_, until the holds are released
+    std::vector<int> deferred_release_;        // blocks whose last reference went while a queued copy named them
     std::vector<int> seq_len_;
     std::vector<char> alive_;
     std::vector<int> dirty_lo_, dirty_hi_;     // per branch, [lo, hi) of changed table entries
@@ -157,12 +165,16 @@ private:
     bool setup_tables(int max_branches);
     void mark_dirty(int branch, int logical);
     bool ensure_nolock(int branch, int pos);
-    int  alloc_phys_nolock();
-    int  evict_nolock(int n);
-    bool ensure_free_nolock(int n_free);
-    bool pick_victim_nolock(int& cell_out);
+    int  alloc_phys_nolock(int for_branch);
+    int  evict_nolock(int n, int for_branch);
+    bool ensure_free_nolock(int n_free, int for_branch);
+    bool pick_victim_nolock(int& cell_out, int for_branch);
     std::string ssd_path_for(int cell_idx) const;
-    bool swap_to_ssd_nolock(int cell_idx);
+    void submit_swap_out_nolock(int cell_idx, char* ok);
+    void candidate_add_nolock(int cell_idx);
+    void candidate_remove_nolock(int cell_idx);
+    void hold_nolock(int cell_idx);
+    void release_holds_nolock();
     bool swap_from_ssd_nolock(int cell_idx);
     void attach_nolock(int cell_idx, int phys, bool fresh_stamp);
     void detach_nolock(int cell_idx);

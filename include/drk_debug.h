@@ -1,0 +1,51 @@
+/*
+ * drk_debug.h -- diagnostic and tuning switches of libdrk_kv.so.  They are process-wide,
+ * not thread-safe, and no part of the drop-in surface: tests use them to hold the kernels
+ * against each other, the benchmark to time single kernels and to sweep launch shapes.
+ * A product caller never needs this header.
+ */
+#ifndef DRK_DEBUG_H
+#define DRK_DEBUG_H
+
+#include "drk_kv.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Diagnostic: route every decode / prefill through the portable kernel (any
+ * geometry, any storage type) instead of the tiled one, so that tests can
+ * check the two against each other.  Process-wide, not thread-safe. */
+void drk_debug_force_portable_decode(int on);
+/* Diagnostic: which kernel produces the decode partials when the geometry allows
+ * a choice: 0 = automatic (the persistent stream kernel), 2 = the fixed-split
+ * tiled kernel (16-bit pages only), 3 = same as 0.  Process-wide. */
+void drk_debug_set_decode_kernel(int which);
+/* Diagnostic: workgroups of the persistent decode grid; 0 restores the default (512; 1024 for
+ * 8-bit pages of head_dim 128). */
+void drk_debug_set_stream_workgroups(int n);
+/* Diagnostic: context splits of the shared-prefix pass (default 64, at most 256; 0 restores the
+ * default).  Changes drk_decode_shared_workspace_bytes. */
+void drk_debug_set_shared_splits(int n);
+/* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
+ * session; switching it on starts a new session) records a HIP event on its
+ * stream right before and right after the split-K partial kernel; the merge
+ * kernel is outside the pair.  drk_debug_decode_kernel_times waits for the pairs
+ * recorded so far and returns their elapsed milliseconds.  Launch back to back
+ * (no host sync in between) so that the queue stays busy and the pairs bracket
+ * the kernel tightly.  Process-wide. */
+void drk_debug_time_decode_kernel(int on);
+int  drk_debug_decode_kernel_times(float *ms, int cap, int *count);
+/* Diagnostic: extra dynamic LDS bytes per decode workgroup (lowers occupancy). */
+void drk_debug_set_decode_lds_pad(int bytes);
+/* Tuning: which prefill chunks run with the context split over the chip (they must stand behind 2 048 tokens
+ * or more): negative = the library's cost rule (default); 0 = none; n = every chunk of up to n rows. */
+void drk_debug_set_prefill_split(int max_rows);
+/* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
+ * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */
+void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chunks);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DRK_DEBUG_H */

@@ -141,7 +141,8 @@ void drkh_paged_prefill_attention_gated(const void *Q, void *kv_pool, const int3
 /* conscientia/kv_stream.h: the KV side of ConscientiStream (src/conscientia/stream.cpp:145-401) */
 void *drkh_kvs_create(void);
 void  drkh_kvs_destroy(void *ks);
-int   drkh_kvs_init(void *ks, void *cm, int max_context_len, void *scorer, const float *d_rope_table, int table_positions);
+int   drkh_kvs_init(void *ks, void *cm, int max_context_len, void *scorer, const float *d_rope_table, int table_positions,
+                    int max_prefill_rows);
 int   drkh_kvs_begin_prefill(void *ks, int M, void *stream);
 void  drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
                              const void *k_norm, void *q_scratch, void *attn_out, int M, void *stream);
@@ -169,7 +170,25 @@ void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_poo
                                                      int max_seq_len, void *out, int fa_layer_idx,
                                                      int max_phys_blocks, int block_size, float scale,
                                                      float *d_block_mass, int accumulate, void *stream);
-int  drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
+/* the workspace of `stream` (the calls above keep one per stream) */
+int  drkh_paged_attention_reserve_workspace(int max_branches, int max_seq_len, int max_prefill_rows, int block_size,
+                                            void *stream);
+size_t drkh_paged_attention_workspace_bytes(int max_branches, int max_seq_len, int max_prefill_rows, int block_size);
+/* full_attention_forward_paged / _paged_prefill (src/machina/paged_attention.h:75-106) with the four
+ * projections served from buffers instead of GEMMs (which are the model's code): qg_proj [M, QH, 2 D],
+ * k_proj, v_proj [M, KVH, D] are what the Q|gate, K and V projections would produce; the gated attention
+ * output passes through the "O projection" unchanged.  state_bufs = {q_buf, kv_buf, dn_z, dn_qkv,
+ * attn_out, norm_out} (InferenceState, src/machina/model.h:232-293). */
+void drkh_set_rope_table(const float *d_rope_table, int table_positions);
+void drkh_full_attention_forward_paged(const void *qg_proj, const void *k_proj, const void *v_proj, const void *q_norm,
+                                       const void *k_norm, void *kv_pool, const int32_t *d_block_table, int fa_layer_idx,
+                                       int pos, int seq_len, int max_phys_blocks, int block_size, void *const *state_bufs,
+                                       int32_t *d_pos, void *stream);
+void drkh_full_attention_forward_paged_prefill(const void *qg_proj, const void *k_proj, const void *v_proj,
+                                               const void *q_norm, const void *k_norm, void *kv_pool,
+                                               const int32_t *d_block_table, int fa_layer_idx, int pos_start, int M,
+                                               int seq_len, int max_phys_blocks, int block_size, void *const *state_bufs,
+                                               void *stream);
 void drkh_paged_attention_release_workspace(void);
 void drkh_invoke_extract_kv_from_pages(void *dst, const void *kv_pool, const int32_t *block_table, int start_token,
                                        int num_tokens, int num_layers, int num_kv_heads, int head_dim,

@@ -74,6 +74,16 @@ int         drk_device_count(int *count);
  * 5 warm-up + `iters` timed passes; d_sink is 4 bytes of device memory.
  * Synchronises. */
 int drk_probe_read_bandwidth(const void *d_ptr, size_t bytes, int iters, void *d_sink, float *gbps);
+/* Same, with the decode kernels' access pattern: aligned granules of granule_bytes (a multiple of
+ * 4096; 4096 = one 16-token K or V run of one kv head at head_dim 128, 16-bit) read in a
+ * scattered order over the largest power-of-two number of granules that fits in `bytes`. */
+int drk_probe_read_bandwidth_permuted(const void *d_ptr, size_t bytes, int granule_bytes, int iters,
+                                      void *d_sink, float *gbps);
+/* Measurement aid: dense bf16 TFLOP/s a registers-only v_mfma_f32_32x32x16_bf16 loop sustains
+ * (8 waves per CU, four independent accumulator chains per wave, no memory traffic): the rate
+ * the matrix cores of the part reach on their own.  d_sink is 4 bytes of device memory.
+ * Synchronises. */
+int drk_probe_mfma_rate(int iters, void *d_sink, float *tflops);
 
 /* ---- layout arithmetic (host only, no GPU needed) --------------------- */
 /* block_pool.cpp:23-39: strides; block_pool.cpp:28-32: budget -> max_blocks */
@@ -96,6 +106,7 @@ int drk_dev_malloc(void **d_ptr, size_t bytes);
 int drk_dev_free(void *d_ptr);
 int drk_dev_memset_async(void *d_ptr, int byte, size_t bytes, void *stream);
 int drk_memcpy_h2d_async(void *d_dst, const void *h_src, size_t bytes, void *stream);
+int drk_memcpy_d2d_async(void *d_dst, const void *d_src, size_t bytes, void *stream);
 int drk_memcpy_d2h(void *h_dst, const void *d_src, size_t bytes, void *stream); /* syncs */
 /* d_pos[i] += delta and d_seq_lens[i] += delta for i < n (either may be NULL), in the stream:
  * lets a captured decode step move its own positions on. */
@@ -122,6 +133,17 @@ int drk_kv_block_from_host(const drk_kv_layout *g, void *pool, int blk, const vo
 int drk_stream_create(void **stream);
 int drk_stream_destroy(void *stream);
 int drk_stream_synchronize(void *stream);
+/* *capturing = 1 while `stream` records into a graph (hipStreamIsCapturing); NULL stream: 0. */
+int drk_stream_is_capturing(void *stream, int *capturing);
+/* Events without timing: drk_event_record marks what `stream` has been given so far,
+ * drk_stream_wait_event makes another stream wait for exactly that (cudaEventRecord /
+ * cudaStreamWaitEvent in the reference's vocabulary, model.h:292-293), drk_event_synchronize
+ * blocks the host until it has happened. */
+int drk_event_create(void **event);
+int drk_event_destroy(void *event);
+int drk_event_record(void *event, void *stream);
+int drk_event_synchronize(void *event);
+int drk_stream_wait_event(void *stream, void *event);
 
 /* ---- append into pages ------------------------------------------------ */
 /* paged_kv_cache_write, paged_attention.cu:73-115: one token at *d_pos.
@@ -176,37 +198,6 @@ size_t drk_decode_workspace_bytes_for_split(const drk_kv_layout *g, int B, int m
 /* The split (tokens per workgroup, a multiple of 64) the library picks when
  * split_tokens == 0. */
 int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len);
-/* Diagnostic: route every decode / prefill through the portable kernel (any
- * geometry, any storage type) instead of the tiled one, so that tests can
- * check the two against each other.  Process-wide, not thread-safe. */
-void drk_debug_force_portable_decode(int on);
-/* Diagnostic: which kernel produces the decode partials when the geometry allows
- * a choice: 0 = automatic (the persistent stream kernel), 2 = the fixed-split
- * tiled kernel (16-bit pages only), 3 = same as 0.  Process-wide. */
-void drk_debug_set_decode_kernel(int which);
-/* Diagnostic: workgroups of the persistent decode grid; 0 restores the default (512; 1024 for
- * 8-bit pages of head_dim 128). */
-void drk_debug_set_stream_workgroups(int n);
-/* Diagnostic: context splits of the shared-prefix pass (default 64, at most 256; 0 restores the
- * default).  Changes drk_decode_shared_workspace_bytes. */
-void drk_debug_set_shared_splits(int n);
-/* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
- * session; switching it on starts a new session) records a HIP event on its
- * stream right before and right after the split-K partial kernel; the merge
- * kernel is outside the pair.  drk_debug_decode_kernel_times waits for the pairs
- * recorded so far and returns their elapsed milliseconds.  Launch back to back
- * (no host sync in between) so that the queue stays busy and the pairs bracket
- * the kernel tightly.  Process-wide. */
-void drk_debug_time_decode_kernel(int on);
-int  drk_debug_decode_kernel_times(float *ms, int cap, int *count);
-/* Diagnostic: extra dynamic LDS bytes per decode workgroup (lowers occupancy). */
-void drk_debug_set_decode_lds_pad(int bytes);
-/* Tuning: which prefill chunks run with the context split over the chip (they must stand behind 2 048 tokens
- * or more): negative = the library's cost rule (default); 0 = none; n = every chunk of up to n rows. */
-void drk_debug_set_prefill_split(int max_rows);
-/* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
- * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */
-void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chunks);
 /* paged_gqa_decode_attention, paged_attention.cu:179-282: one sequence.
  * q/out [num_q_heads, head_dim] of io_dtype (F16/BF16). */
 int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void *pool,
@@ -215,7 +206,8 @@ int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void
                                size_t workspace_bytes, void *stream);
 /* B branches in one launch: d_tables [B, table_stride], d_seq_lens [B] (device),
  * q/out [B, num_q_heads, head_dim]; max_seq_len >= every d_seq_lens[b] sizes the
- * grid.  split_tokens = 0 lets the library choose. */
+ * grid.  split_tokens = 0 lets the library choose; otherwise a multiple of 64, at most 16 384 on the tiled
+ * kernel (larger values are refused with DRK_ERR_INVALID). */
 int drk_paged_decode_attention_branches(const drk_kv_layout *g, const void *q, const void *pool,
                                         const int32_t *d_tables, int table_stride,
                                         const int32_t *d_seq_lens, int B, int max_seq_len,
@@ -275,6 +267,9 @@ int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, con
  * times slower for a chunk of a few tokens behind a long context.  Anything else runs row by row through the portable decode kernel, which needs
  * the workspace. */
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M);
+/* The most drk_prefill_workspace_bytes reports for any chunk of up to max_rows rows that
+ * ends at or before max_seq_len tokens: what a caller reserves once, up front. */
+size_t drk_prefill_workspace_bytes_max(const drk_kv_layout *g, int max_seq_len, int max_rows);
 int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
                                 const int32_t *d_block_table, void *out, int layer,
                                 int pos_start, int M, float scale, int io_dtype,

@@ -758,6 +758,12 @@ struct orc_cm {
     float *scores; int nscores;
     /* queued COW copies */
     int32_t *cp_src, *cp_dst; int cp_n, cp_cap;
+    /* builder-specified protection of the current step: a cell that ensure() made resident is held
+     * until the queued copies are drained; a block named by a queued copy is pinned; a pinned block
+     * that loses its last reference is freed only at the drain */
+    int8_t *held;                            /* per cell */
+    int32_t *pin;                            /* per physical block */
+    int32_t *deferred; int deferred_n;
 };
 
 orc_cm *orc_cm_create(int NB, int bs, int max_branches)
@@ -781,6 +787,9 @@ orc_cm *orc_cm_create(int NB, int bs, int max_branches)
     c->cp_cap = 1024;
     c->cp_src = (int32_t *)malloc(sizeof(int32_t) * c->cp_cap);
     c->cp_dst = (int32_t *)malloc(sizeof(int32_t) * c->cp_cap);
+    c->held = (int8_t *)calloc(cells, 1);
+    c->pin = (int32_t *)calloc(NB, sizeof(int32_t));
+    c->deferred = (int32_t *)malloc(sizeof(int32_t) * NB);
     return c;
 }
 
@@ -789,7 +798,7 @@ void orc_cm_destroy(orc_cm *c)
     if (!c) return;
     free(c->free_stack); free(c->refcount); free(c->table); free(c->loc);
     free(c->seq_len); free(c->alive); free(c->lru_b); free(c->lru_l);
-    free(c->scores); free(c->cp_src); free(c->cp_dst); free(c);
+    free(c->scores); free(c->cp_src); free(c->cp_dst); free(c->held); free(c->pin); free(c->deferred); free(c);
 }
 
 /* block_pool.cpp:63-69 */
@@ -817,6 +826,10 @@ int orc_cm_free_stack(const orc_cm *c, int32_t *out, int cap)
 
 static void drop_ref(orc_cm *c, int phys)
 {
+    if (c->refcount[phys] == 1 && c->pin[phys] > 0) {    /* last reference of a block a queued copy names */
+        c->deferred[c->deferred_n++] = phys;
+        return;
+    }
     if (--c->refcount[phys] <= 0) orc_cm_free_block(c, phys);
 }
 
@@ -834,33 +847,42 @@ static void lru_push(orc_cm *c, int b, int l)
 
 #define CELL(c, b, l) ((size_t)(b) * (c)->max_logical + (l))
 
-/* cache_manager.cpp:185-205.  Builder-specified filter: an entry whose
- * physical block is referenced by more than one table is pinned. */
-static int pick_victim(orc_cm *c, int *vb, int *vl)
+/* cache_manager.cpp:185-205.  Builder-specified filters: an entry whose physical block is
+ * referenced by more than one table is pinned, and so is a block a queued copy names.  Cells of
+ * the current step (held) are passed over; only when nothing else is left (second pass) may a
+ * branch's allocation take that branch's own held cells, and an explicit request (for_branch < 0)
+ * any held cell. */
+static int pick_victim(orc_cm *c, int *vb, int *vl, int for_branch)
 {
-    int best = -1;
-    for (int i = 0; i < c->lru_n; i++) {
-        int b = c->lru_b[i], l = c->lru_l[i];
-        int phys = c->table[CELL(c, b, l)];
-        if (c->loc[CELL(c, b, l)] != 0 || phys < 0 || c->refcount[phys] != 1) continue;
-        if (!c->scores) { best = i; break; }              /* lru_order_.front() */
-        int cell = CELL(c, b, l), cbest = best < 0 ? 0 : CELL(c, c->lru_b[best], c->lru_l[best]);
-        float s = cell < c->nscores ? c->scores[cell] : 0.0f;
-        float sb = best < 0 ? 0.0f : (cbest < c->nscores ? c->scores[cbest] : 0.0f);
-        if (best < 0 || s < sb) best = i;                 /* first minimum */
+    for (int pass = 0; pass < 2; pass++) {
+        int best = -1;
+        for (int i = 0; i < c->lru_n; i++) {
+            int b = c->lru_b[i], l = c->lru_l[i];
+            int phys = c->table[CELL(c, b, l)];
+            if (c->loc[CELL(c, b, l)] != 0 || phys < 0 || c->refcount[phys] != 1 || c->pin[phys] > 0) continue;
+            if ((c->held[CELL(c, b, l)] != 0) != (pass == 1)) continue;
+            if (pass == 1 && for_branch >= 0 && b != for_branch) continue;
+            if (!c->scores) { best = i; break; }              /* lru_order_.front() */
+            int cell = CELL(c, b, l), cbest = best < 0 ? 0 : CELL(c, c->lru_b[best], c->lru_l[best]);
+            float s = cell < c->nscores ? c->scores[cell] : 0.0f;
+            float sb = best < 0 ? 0.0f : (cbest < c->nscores ? c->scores[cbest] : 0.0f);
+            if (best < 0 || s < sb) best = i;                 /* first minimum */
+        }
+        if (best >= 0) {
+            *vb = c->lru_b[best]; *vl = c->lru_l[best];
+            return 1;
+        }
     }
-    if (best < 0) return 0;
-    *vb = c->lru_b[best]; *vl = c->lru_l[best];
-    return 1;
+    return 0;
 }
 
 /* cache_manager.cpp:118-156 without a swapper: discard */
-int orc_cm_evict_blocks(orc_cm *c, int n)
+static int evict_for(orc_cm *c, int n, int for_branch)
 {
     int evicted = 0;
     while (evicted < n && c->lru_n > 0) {
         int b, l;
-        if (!pick_victim(c, &b, &l)) break;
+        if (!pick_victim(c, &b, &l, for_branch)) break;
         lru_remove(c, b, l);
         int phys = c->table[CELL(c, b, l)];
         drop_ref(c, phys);
@@ -870,22 +892,24 @@ int orc_cm_evict_blocks(orc_cm *c, int n)
     }
     return evicted;
 }
+int orc_cm_evict_blocks(orc_cm *c, int n) { return evict_for(c, n, -1); }
 
 /* cache_manager.cpp:158-164 */
-int orc_cm_ensure_free_blocks(orc_cm *c, int n_free)
+static int ensure_free_for(orc_cm *c, int n_free, int for_branch)
 {
     while (c->free_n < n_free) {
         if (c->lru_n == 0) return 0;
-        if (orc_cm_evict_blocks(c, 1) == 0) return 0;
+        if (evict_for(c, 1, for_branch) == 0) return 0;
     }
     return 1;
 }
+int orc_cm_ensure_free_blocks(orc_cm *c, int n_free) { return ensure_free_for(c, n_free, -1); }
 
-static int alloc_phys(orc_cm *c)                         /* cache_manager.cpp:306-319 */
+static int alloc_phys(orc_cm *c, int for_branch)         /* cache_manager.cpp:306-319 */
 {
     int phys = orc_cm_alloc_block(c);
     if (phys < 0) {
-        if (!orc_cm_ensure_free_blocks(c, 1)) return -1;
+        if (!ensure_free_for(c, 1, for_branch)) return -1;
         phys = orc_cm_alloc_block(c);
     }
     return phys;
@@ -903,8 +927,9 @@ int orc_cm_ensure(orc_cm *c, int b, int pos)
     size_t cell = CELL(c, b, l);
     if (c->loc[cell] == 0) {
         int phys = c->table[cell];
+        c->held[cell] = 1;                                /* before the allocation below looks for a victim */
         if (c->refcount[phys] > 1) {
-            int np = alloc_phys(c);
+            int np = alloc_phys(c, b);
             if (np < 0) return 0;
             if (c->cp_n == c->cp_cap) {
                 c->cp_cap *= 2;
@@ -912,15 +937,17 @@ int orc_cm_ensure(orc_cm *c, int b, int pos)
                 c->cp_dst = (int32_t *)realloc(c->cp_dst, sizeof(int32_t) * c->cp_cap);
             }
             c->cp_src[c->cp_n] = phys; c->cp_dst[c->cp_n] = np; c->cp_n++;
+            c->pin[phys]++; c->pin[np]++;
             c->refcount[phys]--;
             c->table[cell] = np;
         }
         return 1;
     }
-    int phys = alloc_phys(c);
+    int phys = alloc_phys(c, b);
     if (phys < 0) return 0;
     c->table[cell] = phys;                                /* cache_manager.cpp:321-323 */
     c->loc[cell] = 0;
+    c->held[cell] = 1;
     lru_push(c, b, l);
     return 1;
 }
@@ -1008,6 +1035,11 @@ int orc_cm_drain_copies(orc_cm *c, int32_t *so, int32_t *dn, int cap)
     memcpy(so, c->cp_src, sizeof(int32_t) * n);
     memcpy(dn, c->cp_dst, sizeof(int32_t) * n);
     int total = c->cp_n;
+    /* the copies count as issued: pins, deferred frees (in the order they were deferred) and holds end */
+    for (int i = 0; i < c->cp_n; i++) { c->pin[c->cp_src[i]]--; c->pin[c->cp_dst[i]]--; }
     c->cp_n = 0;
+    for (int i = 0; i < c->deferred_n; i++) drop_ref(c, c->deferred[i]);
+    c->deferred_n = 0;
+    memset(c->held, 0, (size_t)c->max_branches * c->max_logical);
     return total;
 }

@@ -1,5 +1,5 @@
 """The built libraries load without a GPU and export every symbol that
-include/drk_kv.h and include/drk_host.h declare; the layout arithmetic (host
+include/drk_kv.h, include/drk_debug.h and include/drk_host.h declare; the layout arithmetic (host
 only) agrees with the oracle's.  No kernel is launched here."""
 import ctypes as C
 import os
@@ -22,9 +22,13 @@ def declared(header, prefix):
 def test_drk_kv_symbols_are_exported_and_bound():
     names = declared("drk_kv.h", "drk_")
     assert len(names) > 30
+    assert not [n for n in names if n.startswith("drk_debug_")], "diagnostic switches belong in drk_debug.h"
+    debug = declared("drk_debug.h", "drk_debug_")
+    assert len(debug) >= 9
+    names = sorted(names + debug)
     raw = C.CDLL(cabi.LIB_PATH)
     for n in names:
-        assert hasattr(raw, n), f"{n} declared in drk_kv.h but not exported"
+        assert hasattr(raw, n), f"{n} declared in drk_kv.h / drk_debug.h but not exported"
     assert sorted(cabi.SIGNATURES) == names, "the ctypes table and the header differ"
     assert cabi.lib().drk_abi_version() == 1
 
@@ -65,3 +69,16 @@ def test_errors_are_reported_without_a_gpu():
     g = cabi.layout(1, 4, 16, 128, 16, 8, cabi.F16)
     need = L.drk_decode_workspace_bytes(C.byref(g), 1, 512)
     assert need >= 16 * (512 // L.drk_decode_default_split(C.byref(g), 1, 512)) * 130 * 4 and need % (130 * 4) == 0
+
+
+def test_decode_refuses_a_split_longer_than_the_kernels_run():
+    """split_tokens above 16 384 would overrun the persistent kernel's descriptor table: the call
+    returns DRK_ERR_INVALID before anything is launched (no GPU needed: the pointers are never used)."""
+    g = cabi.layout(1, 8, 32, 128, 16, 4096, cabi.BF16)
+    fake = C.c_void_p(0x1000)
+    L = cabi.lib()
+    for split, want in ((16384 + 64, cabi.ERR_INVALID), (100, cabi.ERR_INVALID)):
+        rc = L.drk_paged_decode_attention_branches(C.byref(g), fake, fake, fake, 4096, fake, 2, 65536, fake, 0, 0.1, cabi.BF16,
+                                                   split, fake, 1 << 30, None)
+        assert rc == want, (split, rc)
+    assert b"split_tokens" in L.drk_last_error()

@@ -166,3 +166,56 @@ def test_without_a_swapper_eviction_discards(dev, tmp_path):
         assert cm.ensure_blocks_for(0, blk * bs)
     assert cm.ssd_blocks_used() == 0
     assert [cm.block_location(0, i) for i in range(6)] == [host.CacheManager.INVALID] * 2 + [host.CacheManager.GPU] * 4
+
+
+def test_batch_eviction_pipelines_behind_the_writers_stream(dev, tmp_path):
+    """ensure_free_blocks() under the overflow tier: every victim's swap-out is queued at once and the
+    swapper overlaps one block's copy with its neighbour's file write.  The blocks are written by a
+    kernel on a stream of its own right before the request, with no wait in between: the copies order
+    themselves behind that stream (it was announced by sync_block_table) instead of stalling the device.
+    Every file holds its block's image; every block comes back bit for bit."""
+    import torch
+    L, KVH, QH, D, bs = 4, 8, 32, 128, 16
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    cm, sw = host.CacheManager(), host.KVSwapper()
+    block_bytes = L * 2 * KVH * bs * D * 2
+    NBLK = 24
+    assert cm.init_ssd(NBLK * block_bytes, tmp_path / "batch", bs, sw)
+    assert sw.init(cm, tmp_path / "batch", 3)
+    L_ = host.lib()
+    side = torch.cuda.Stream()
+    sp = C.c_void_p(side.cuda_stream)
+    try:
+        NB = cm.pool_max_blocks()
+        og = orc.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+        T = NBLK * bs
+        rng = np.random.default_rng(113)
+        k = U.normal_bits(rng, (L, T, KVH, D), cabi.BF16)
+        v = U.normal_bits(rng, (L, T, KVH, D), cabi.BF16)
+        dk, dv = [U.dev_bytes(k[l]) for l in range(L)], [U.dev_bytes(v[l]) for l in range(L)]
+        torch.cuda.synchronize()
+        assert cm.ensure_blocks_for_range(0, 0, T)
+        cm.sync_block_table(sp)
+        table = cm.h_block_table(0).copy()
+        for l in range(L):
+            L_.drkh_paged_kv_cache_write_batch(U.p(dk[l]), U.p(dv[l]), cm.pool_ptr(), cm.d_block_table(0), l, 0, T, NB, bs, sp)
+        cm.set_seq_len(0, T)
+        assert cm.ensure_free_blocks(NBLK)                               # all 24 go out in one batch, no sync before
+        assert cm.ssd_blocks_used() == NBLK and cm.free_blocks() == NBLK and sw.pending() == 0
+        opool = orc.new_pool(og)
+        for l in range(L):
+            orc.append_batch(og, opool, table, l, 0, k[l], v[l], cabi.BF16)
+        for blk in range(NBLK):
+            img = np.fromfile(tmp_path / "batch" / ("block_%d.kv" % blk), dtype=np.uint8)
+            assert np.array_equal(img, orc.block_image(og, opool, int(table[blk]))), blk
+        # ... and back, into whatever blocks are free
+        for blk in range(NBLK):
+            assert cm.ensure_blocks_for(0, blk * bs)
+        cm.sync_block_table(sp)
+        flat = U.dev_zeros(L * 2 * T * KVH * D * 2)
+        L_.drkh_invoke_extract_kv_from_pages(U.p(flat), cm.pool_ptr(), cm.d_block_table(0), 0, T, L, KVH, D, bs, NB, sp)
+        side.synchronize()
+        got = U.host(flat, np.uint16, (L, 2, T, KVH, D))
+        assert np.array_equal(got[:, 0], k) and np.array_equal(got[:, 1], v)
+    finally:
+        sw.shutdown()
