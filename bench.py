@@ -13,6 +13,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -22,11 +23,32 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the decode kernel from two `rocprofv3 --pmc` runs of this
-# script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), scaled by what the same
-# counters read for a plain 32 GiB read (x2.0) and a bulk append of known size
-# (x1.0).  Keyed by the algorithmic bytes of the launch it was measured on.
-MEASURED_TRAFFIC_BYTES = {1073741824: int((524763.5 * 2 + 1850.5) * 1024)}
+# HBM bytes per launch of the decode kernel come from the counter runs recorded in this
+# profile summary (two `rocprofv3 --pmc` runs of this script: FETCH_SIZE, then WRITE_SIZE).
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "decode_stream_bf16_config2_8x32k.md")
+
+
+def measured_traffic(launch_bytes):
+    """(bytes per launch, source) from the profile summary, when it was taken on a launch of
+    exactly these algorithmic bytes; (None, reason) otherwise.  The summary carries two lines,
+    `algorithmic_bytes_per_launch: N` and `traffic_bytes_per_launch: N`."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, "no profile summary"
+    alg = re.search(r"^algorithmic_bytes_per_launch:\s*(\d+)", text, re.M)
+    tr = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    if not alg or not tr:
+        return None, "profile summary carries no traffic figure"
+    if int(alg.group(1)) != launch_bytes:
+        return None, "profile summary was taken on another launch size"
+    return int(tr.group(1)), os.path.relpath(TRAFFIC_PROFILE, ROOT)
+
+
+def bf16_bits(rng, shape, mul):
+    """N(0,1) * mul as bf16 bit patterns (round to nearest even), for the CPU sample."""
+    u = (rng.standard_normal(shape).astype(np.float32) * np.float32(mul)).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
 def parse():
@@ -42,6 +64,8 @@ def parse():
     ap.add_argument("--pool-gb", type=float, default=40.0)
     ap.add_argument("--split", type=int, default=0, help="tokens per split-K workgroup (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the kernel measurements of configs 3, 4 and 5 that the default line carries")
     ap.add_argument("--no-ragged", action="store_true", help="skip the side measurements that launch the headline kernel on other shapes (profiling: one shape per kernel name)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="context per branch for the CPU sample (0 = auto)")
     ap.add_argument("--bulk-append-tokens", type=int, default=2048)
@@ -67,7 +91,6 @@ def main():
         sys.exit(2)
     import torch
     from deusridet_amd import cabi
-    from tests import util as U
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if args.config != 2:
@@ -116,8 +139,8 @@ def main():
             m = min(chunk, n - p0)
             k = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
             v = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
-            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(dtab[b].data_ptr()), 0, L, p0, m,
-                      U.p(k), U.p(v), cabi.BF16, sp)
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(pool), C.c_void_p(dtab[b].data_ptr()), 0, L, p0, m,
+                      cabi.p(k), cabi.p(v), cabi.BF16, sp)
             del k, v
     torch.cuda.synchronize()
     t_fill = time.time() - t_fill
@@ -142,11 +165,11 @@ def main():
         dpos = C.c_void_p(pos_steps[s].data_ptr())
         dlen = C.c_void_p(len_steps[s].data_ptr())
         for l in range(L):
-            cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), stride, dpos, B, l, 1,
+            cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos, B, l, 1,
                       C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, sp)
             cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow),
-                      U.p(pool), U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
-                      float(scale), cabi.BF16, split, U.p(ws), wsb, sp)
+                      cabi.p(pool), cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
+                      float(scale), cabi.BF16, split, cabi.p(ws), wsb, sp)
 
     use_graph = not args.no_graph
     if use_graph:
@@ -158,11 +181,11 @@ def main():
             dpos, dlen = C.c_void_p(pos_cur.data_ptr()), C.c_void_p(len_cur.data_ptr())
             gsp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
             for l in range(L):
-                cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), stride, dpos, B, l, 1,
+                cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos, B, l, 1,
                           C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, gsp)
                 cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow),
-                          U.p(pool), U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
-                          float(scale), cabi.BF16, split, U.p(ws), wsb, gsp)
+                          cabi.p(pool), cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
+                          float(scale), cabi.BF16, split, cabi.p(ws), wsb, gsp)
             pos_cur.add_(1)
             len_cur.add_(1)
 
@@ -213,9 +236,9 @@ def main():
     def attn_only(n):
         for it in range(n):
             l = it % L
-            cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
-                      U.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
-                      cabi.BF16, split, U.p(ws), wsb, sp)
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), cabi.p(pool),
+                      cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
+                      cabi.BF16, split, cabi.p(ws), wsb, sp)
 
     attn_only(8)
     lib.drk_debug_time_decode_kernel(1)
@@ -239,9 +262,9 @@ def main():
         def ragged_only(n):
             for it in range(n):
                 l = it % L
-                cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
-                          U.p(dtab), stride, U.p(rlen), B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
-                          cabi.BF16, split, U.p(ws), wsb, sp)
+                cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), cabi.p(pool),
+                          cabi.p(dtab), stride, cabi.p(rlen), B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
+                          cabi.BF16, split, cabi.p(ws), wsb, sp)
 
         ragged_only(8)
         lib.drk_debug_time_decode_kernel(1)
@@ -258,8 +281,14 @@ def main():
     sink = torch.zeros(16, dtype=torch.uint8, device="cuda")
     gb = C.c_float(0)
     torch.cuda.synchronize()
-    cabi.call("drk_probe_read_bandwidth", U.p(pool), probe_bytes, 5, U.p(sink), C.byref(gb))
+    cabi.call("drk_probe_read_bandwidth", cabi.p(pool), probe_bytes, 5, cabi.p(sink), C.byref(gb))
     read_probe_gbps = float(gb.value)
+    # ... and the decode kernels' own access pattern: 4 KiB granules in a scattered order
+    cabi.call("drk_probe_read_bandwidth_permuted", cabi.p(pool), probe_bytes, 4096, 5, cabi.p(sink), C.byref(gb))
+    permuted_probe_gbps = float(gb.value)
+    # the dense bf16 rate the matrix cores sustain with no memory traffic at all
+    cabi.call("drk_probe_mfma_rate", 20, cabi.p(sink), C.byref(gb))
+    mfma_probe_tflops = float(gb.value)
 
     # ---- bulk append bandwidth (read source + write pages), all layers in one launch
     m = args.bulk_append_tokens
@@ -269,13 +298,13 @@ def main():
         k = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
         v = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
         for _ in range(3):
-            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(scratch_tab), 0, L, 0, m, U.p(k), U.p(v),
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(pool), cabi.p(scratch_tab), 0, L, 0, m, cabi.p(k), cabi.p(v),
                       cabi.BF16, sp)
         a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a0.record(stream)
         reps = 10
         for _ in range(reps):
-            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(scratch_tab), 0, L, 0, m, U.p(k), U.p(v),
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(pool), cabi.p(scratch_tab), 0, L, 0, m, cabi.p(k), cabi.p(v),
                       cabi.BF16, sp)
         a1.record(stream)
         torch.cuda.synchronize()
@@ -289,9 +318,9 @@ def main():
         for name in ("drk_kv_extract", "drk_kv_inject"):
             def go():
                 if name == "drk_kv_extract":
-                    cabi.call(name, C.byref(g), U.p(flat), None, U.p(pool), U.p(scratch_tab), 0, m, L, sp)
+                    cabi.call(name, C.byref(g), cabi.p(flat), None, cabi.p(pool), cabi.p(scratch_tab), 0, m, L, sp)
                 else:
-                    cabi.call(name, C.byref(g), U.p(pool), U.p(flat), None, U.p(scratch_tab), 0, m, L, sp)
+                    cabi.call(name, C.byref(g), cabi.p(pool), cabi.p(flat), None, cabi.p(scratch_tab), 0, m, L, sp)
             for _ in range(3):
                 go()
             a0.record(stream)
@@ -318,7 +347,7 @@ def main():
         ktmp = torch.empty_like(newk)
         npos = max_ctx + 1
         rtab = torch.empty(npos * (rd // 2) * 2, dtype=torch.float32, device="cuda")
-        cabi.call("drk_rope_table_fill", U.p(rtab), npos, rd, theta, sp)
+        cabi.call("drk_rope_table_fill", cabi.p(rtab), npos, rd, theta, sp)
         dpos_l, dlen_l = C.c_void_p(pos_steps[last].data_ptr()), C.c_void_p(len_steps[last].data_ptr())
         qgrow = B * QH * 2 * D * 2
         wsb_g = lib.drk_decode_workspace_bytes(C.byref(g), B, max_ctx)
@@ -329,24 +358,24 @@ def main():
                 qp, gp, op = (C.c_void_p(t.data_ptr() + l * qrow) for t in (qsep, gsep, out))
                 kp = C.c_void_p(ktmp.data_ptr() + l * krow)
                 cabi.call("drk_split_q_gate", C.c_void_p(qg.data_ptr() + l * qgrow), qp, gp, B, QH, D, gsp)
-                cabi.call("drk_head_norm", qp, U.p(qw), qp, B * QH, D, eps, cabi.BF16, gsp)
-                cabi.call("drk_head_norm", C.c_void_p(newk.data_ptr() + l * krow), U.p(kw), kp, B * KVH, D, eps, cabi.BF16, gsp)
-                cabi.call("drk_apply_rope", qp, kp, B, QH, KVH, D, rd, dpos_l, 0, theta, U.p(rtab), npos, cabi.BF16, gsp)
-                cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), stride, dpos_l, B, l, 1, kp,
+                cabi.call("drk_head_norm", qp, cabi.p(qw), qp, B * QH, D, eps, cabi.BF16, gsp)
+                cabi.call("drk_head_norm", C.c_void_p(newk.data_ptr() + l * krow), cabi.p(kw), kp, B * KVH, D, eps, cabi.BF16, gsp)
+                cabi.call("drk_apply_rope", qp, kp, B, QH, KVH, D, rd, dpos_l, 0, theta, cabi.p(rtab), npos, cabi.BF16, gsp)
+                cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos_l, B, l, 1, kp,
                           C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, gsp)
-                cabi.call("drk_paged_decode_attention_branches", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen_l, B,
-                          max_ctx, op, l, float(scale), cabi.BF16, split, U.p(ws), wsb, gsp)
+                cabi.call("drk_paged_decode_attention_branches", C.byref(g), qp, cabi.p(pool), cabi.p(dtab), stride, dlen_l, B,
+                          max_ctx, op, l, float(scale), cabi.BF16, split, cabi.p(ws), wsb, gsp)
                 cabi.call("drk_sigmoid_gate", op, gp, op, B * QH, D, D, cabi.BF16, gsp)
 
         def fused(gsp):
             for l in range(L):
                 qp, op = (C.c_void_p(t.data_ptr() + l * qrow) for t in (qsep, out))
                 qgp = qg.data_ptr() + l * qgrow
-                cabi.call("drk_qk_norm_rope_append", C.byref(g), U.p(pool), U.p(dtab), stride, dpos_l, 0, B, l,
+                cabi.call("drk_qk_norm_rope_append", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos_l, 0, B, l,
                           C.c_void_p(qgp), C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow),
-                          U.p(qw), U.p(kw), eps, rd, theta, U.p(rtab), npos, qp, cabi.BF16, gsp)
-                cabi.call("drk_paged_decode_attention_gated", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen_l, B, max_ctx,
-                          op, l, float(scale), cabi.BF16, C.c_void_p(qgp + D * 2), 2 * D, U.p(ws_g), wsb_g, gsp)
+                          cabi.p(qw), cabi.p(kw), eps, rd, theta, cabi.p(rtab), npos, qp, cabi.BF16, gsp)
+                cabi.call("drk_paged_decode_attention_gated", C.byref(g), qp, cabi.p(pool), cabi.p(dtab), stride, dlen_l, B, max_ctx,
+                          op, l, float(scale), cabi.BF16, C.c_void_p(qgp + D * 2), 2 * D, cabi.p(ws_g), wsb_g, gsp)
 
         res = {}
         for name, fn in (("separate", separate), ("fused", fused)):
@@ -391,11 +420,11 @@ def main():
                     l = it % L
                     qp, op = C.c_void_p(q.data_ptr() + l * qrow), C.c_void_p(out.data_ptr() + l * qrow)
                     if name == "plain":
-                        cabi.call("drk_paged_decode_attention_branches", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen, B,
-                                  max_ctx, op, l, float(scale), cabi.BF16, 0, U.p(mws), mass_wsb, sp)
+                        cabi.call("drk_paged_decode_attention_branches", C.byref(g), qp, cabi.p(pool), cabi.p(dtab), stride, dlen, B,
+                                  max_ctx, op, l, float(scale), cabi.BF16, 0, cabi.p(mws), mass_wsb, sp)
                     else:
-                        cabi.call("drk_paged_decode_attention_mass", C.byref(g), qp, U.p(pool), U.p(dtab), stride, dlen, B,
-                                  max_ctx, op, l, float(scale), cabi.BF16, U.p(mass), mstride, 1 if l else 0, U.p(mws),
+                        cabi.call("drk_paged_decode_attention_mass", C.byref(g), qp, cabi.p(pool), cabi.p(dtab), stride, dlen, B,
+                                  max_ctx, op, l, float(scale), cabi.BF16, cabi.p(mass), mstride, 1 if l else 0, cabi.p(mws),
                                   mass_wsb, sp)
             go(4)
             a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -417,7 +446,7 @@ def main():
         for name in ("drk_kv_block_to_host", "drk_kv_block_from_host"):
             def go(n):
                 for i in range(n):
-                    cabi.call(name, C.byref(g), U.p(pool), int(perm[i % NB]), C.c_void_p(hp.value + (i % 4) * blk_bytes), sp)
+                    cabi.call(name, C.byref(g), cabi.p(pool), int(perm[i % NB]), C.c_void_p(hp.value + (i % 4) * blk_bytes), sp)
             go(4)
             torch.cuda.synchronize()
             t0 = time.time()
@@ -441,10 +470,10 @@ def main():
         htab = np.arange(B * nb1, dtype=np.int32).reshape(B, nb1)
         crng = np.random.default_rng(7)
         for b in range(B):
-            kk = U.normal_bits(crng, (n_cpu, KVH, D), cabi.BF16, 0.5)
-            vv = U.normal_bits(crng, (n_cpu, KVH, D), cabi.BF16, 0.5)
+            kk = bf16_bits(crng, (n_cpu, KVH, D), 0.5)
+            vv = bf16_bits(crng, (n_cpu, KVH, D), 0.5)
             orc.append_batch(og, hp, htab[b], 0, 0, kk, vv, orc.BF16)
-        hq = U.normal_bits(crng, (B, QH, D), cabi.BF16, 0.5)
+        hq = bf16_bits(crng, (B, QH, D), 0.5)
         lens = np.full(B, n_cpu, dtype=np.int32)
         t0 = time.time()
         reps = 0
@@ -465,7 +494,15 @@ def main():
                          f"oracle's reference-order loop, OpenMP over (branch, q head)",
                "single_thread_value": reps1 * B * n_cpu * kv_bytes_per_token / dt1 / 1e9}
 
+    # ---- the dominant kernels of configs 3, 4 and 5 on their own shapes, in the same buffer
+    other = None
+    if not args.no_other_configs:
+        import bench_extra
+        del ws
+        other = bench_extra.kernel_fractions(pool)
+
     tokens_per_s = B * K / (total_ms * 1e-3)
+    traffic, traffic_source = measured_traffic(launch_bytes)
     line = {
         "metric": "paged_decode_attention_GBps",
         "value": round(value_gbps, 2),
@@ -494,6 +531,9 @@ def main():
         "bulk_gather_GBps": None if gather_gbps is None else round(gather_gbps, 1),
         "bulk_scatter_GBps": None if scatter_gbps is None else round(scatter_gbps, 1),
         "hbm_read_probe_GBps": round(read_probe_gbps, 1),
+        "hbm_read_probe_permuted_4KiB_GBps": round(permuted_probe_gbps, 1),
+        "mfma_bf16_probe_TFLOPs": round(mfma_probe_tflops, 1),
+        "other_configs": other,
         "ragged_ctx_decode": ragged,
         "fill_seconds": round(t_fill, 2),
         "layer_steps": layer_steps,
@@ -502,7 +542,7 @@ def main():
         "roofline": {
             "kernel": "decode_stream_kernel<bf16>", "bound": "hbm", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(launch_bytes), "avg_launch_us": round(ker_avg_ms * 1e3, 2), "bytes_per_launch": launch_bytes,
+            "traffic": traffic, "traffic_source": traffic_source, "avg_launch_us": round(ker_avg_ms * 1e3, 2), "bytes_per_launch": launch_bytes,
         },
         "cpu_baseline": cpu,
     }

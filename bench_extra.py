@@ -17,11 +17,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 def _common(args):
     import torch
     from deusridet_amd import cabi
-    from tests import util as U
     lib = cabi.lib()
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
-    return torch, cabi, U, lib, stream, C.c_void_p(stream.cuda_stream)
+    return torch, cabi, None, lib, stream, C.c_void_p(stream.cuda_stream)
 
 
 def _timed_decode(lib, cabi, call, n):
@@ -67,8 +66,8 @@ def config4(args):
             v = torch.randn(L, m, KVH, D, device="cuda")
             v = torch.where(torch.rand_like(v) < 0.01, v * 20, v).to(torch.bfloat16)
             a0.record(stream)
-            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(dtab[b].data_ptr()), 0, L, p0, m,
-                      U.p(k), U.p(v), cabi.BF16, sp)
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(pool), C.c_void_p(dtab[b].data_ptr()), 0, L, p0, m,
+                      cabi.p(k), cabi.p(v), cabi.BF16, sp)
             a1.record(stream)
             torch.cuda.synchronize()
             if m == chunk and p0 > 0:
@@ -88,14 +87,14 @@ def config4(args):
     qrow, krow = B * QH * D * 2, B * KVH * D * 2
 
     def attn(l, dlen):
-        cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), U.p(pool),
-                  U.p(dtab), nblk, dlen, B, ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.BF16, 0,
-                  U.p(ws), wsb, sp)
+        cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), cabi.p(pool),
+                  cabi.p(dtab), nblk, dlen, B, ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.BF16, 0,
+                  cabi.p(ws), wsb, sp)
 
     def step(s):
         dpos, dlen = C.c_void_p(pos_steps[s].data_ptr()), C.c_void_p(len_steps[s].data_ptr())
         for l in range(L):
-            cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(dtab), nblk, dpos, B, l, 1,
+            cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), nblk, dpos, B, l, 1,
                       C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
             attn(l, dlen)
 
@@ -161,7 +160,7 @@ def config3(args):
         v = (torch.randn(L, m, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
         g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
         cabi.call("drk_kv_append_batch", C.byref(g), pool_ptr, C.c_void_p(cm.d_block_table(branch)), 0, L, p0, m,
-                  U.p(k), U.p(v), cabi.BF16, sp)
+                  cabi.p(k), cabi.p(v), cabi.BF16, sp)
         torch.cuda.synchronize()
         cm.set_seq_len(branch, p0 + m)
 
@@ -217,11 +216,11 @@ def config3(args):
         dpos.copy_(torch.from_numpy(lens))
         dlen.copy_(torch.from_numpy(lens + 1))
         for l in range(L):
-            cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, U.p(dpos), B, l, 1,
+            cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, cabi.p(dpos), B, l, 1,
                       C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
             cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr,
-                      dtabs, stride, U.p(dlen), B, max_ctx, shared_now[0], C.c_void_p(out.data_ptr() + l * qrow), l,
-                      float(scale), cabi.BF16, U.p(ws), wsb, sp)
+                      dtabs, stride, cabi.p(dlen), B, max_ctx, shared_now[0], C.c_void_p(out.data_ptr() + l * qrow), l,
+                      float(scale), cabi.BF16, cabi.p(ws), wsb, sp)
         for i, b in enumerate(forks):
             cm.set_seq_len(b, int(lens[i]) + 1)
 
@@ -241,11 +240,11 @@ def config3(args):
     per_tok = 2 * KVH * D * 2
     unique_tokens = cm.gpu_blocks_used() * bs
     value = logical * per_tok * L / (total_ms * 1e-3) / 1e9
-    dl = U.p(dlen)
+    dl = cabi.p(dlen)
     ker_ms = _timed_decode(lib, cabi, lambda n: [cabi.call(
         "drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + (i % L) * qrow), pool_ptr, dtabs,
         stride, dl, B, max_ctx, shared_now[0], C.c_void_p(out.data_ptr() + (i % L) * qrow), i % L, float(scale),
-        cabi.BF16, U.p(ws), wsb, sp) for i in range(n)], 60)
+        cabi.BF16, cabi.p(ws), wsb, sp) for i in range(n)], 60)
     launch_logical = int(lens.sum()) * per_tok
     # bytes the launch must fetch: shared pages once, private pages once each
     launch_unique = (shared_now[0] + int((lens - shared_now[0]).sum())) * per_tok
@@ -299,8 +298,8 @@ def config5(args):
         for p0 in range(0, dctx, chunk):
             k = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
             v = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
-            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), C.c_void_p(tab_dec[b].data_ptr()), 0, L, p0, chunk,
-                      U.p(k), U.p(v), cabi.BF16, sp)
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(pool), C.c_void_p(tab_dec[b].data_ptr()), 0, L, p0, chunk,
+                      cabi.p(k), cabi.p(v), cabi.BF16, sp)
             torch.cuda.synchronize()
     qd = torch.randn(L, DB, QH, D, device="cuda").to(torch.bfloat16)
     od = torch.zeros_like(qd)
@@ -321,20 +320,20 @@ def config5(args):
             q = torch.randn(L, chunk, QH, D, device="cuda").to(torch.bfloat16)
             o = torch.empty_like(q)
             ev[0].record(stream)
-            cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(tab_seq), 0, L, c * chunk, chunk, U.p(k), U.p(v),
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(pool), cabi.p(tab_seq), 0, L, c * chunk, chunk, cabi.p(k), cabi.p(v),
                       cabi.BF16, sp)
             ev[1].record(stream)
             for l in range(L):
                 cabi.call("drk_paged_prefill_attention", C.byref(g), C.c_void_p(q.data_ptr() + l * chunk * QH * D * 2),
-                          U.p(pool), U.p(tab_seq), C.c_void_p(o.data_ptr() + l * chunk * QH * D * 2), l, c * chunk, chunk,
+                          cabi.p(pool), cabi.p(tab_seq), C.c_void_p(o.data_ptr() + l * chunk * QH * D * 2), l, c * chunk, chunk,
                           float(scale), cabi.BF16, None, 0, sp)
             ev[2].record(stream)
             for l in range(L):                                   # one interleaved decode step of the 4 branches
-                cabi.call("drk_kv_append_branches", C.byref(g), U.p(pool), U.p(tab_dec), nb_dec, U.p(dpos), DB, l, 1,
+                cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(tab_dec), nb_dec, cabi.p(dpos), DB, l, 1,
                           C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
                 cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(qd.data_ptr() + l * qrow),
-                          U.p(pool), U.p(tab_dec), nb_dec, U.p(dlen), DB, dctx + 64, C.c_void_p(od.data_ptr() + l * qrow),
-                          l, float(scale), cabi.BF16, 0, U.p(ws), wsb, sp)
+                          cabi.p(pool), cabi.p(tab_dec), nb_dec, cabi.p(dlen), DB, dctx + 64, C.c_void_p(od.data_ptr() + l * qrow),
+                          l, float(scale), cabi.BF16, 0, cabi.p(ws), wsb, sp)
             ev[3].record(stream)
             torch.cuda.synchronize()
             if ps > 0:
@@ -360,8 +359,8 @@ def config5(args):
 
             def go(n):
                 for i in range(n):
-                    cabi.call("drk_paged_prefill_attention", C.byref(g), U.p(qs), U.p(pool), U.p(tab_seq), U.p(os_), i % L, pos, rows,
-                              float(scale), cabi.BF16, U.p(ws_s), wsb_s, sp)
+                    cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qs), cabi.p(pool), cabi.p(tab_seq), cabi.p(os_), i % L, pos, rows,
+                              float(scale), cabi.BF16, cabi.p(ws_s), wsb_s, sp)
             go(3)
             ev[0].record(stream)
             go(20)
@@ -408,9 +407,9 @@ def config6(args):
     blocks = prefix // bs + NBR * ((2 * (W + K)) // bs + 3) + 64
     assert cm.init(blocks * L * 2 * KVH * bs * D * 2, bs, None, NBR + 1), "CacheManager.init failed"
     table = torch.empty(max_ctx * RD, dtype=torch.float32, device="cuda")
-    cabi.call("drk_rope_table_fill", U.p(table), max_ctx, RD, THETA, sp)
+    cabi.call("drk_rope_table_fill", cabi.p(table), max_ctx, RD, THETA, sp)
     ks = host.KvStream()
-    assert ks.init(cm, max_ctx, None, U.p(table), max_ctx)
+    assert ks.init(cm, max_ctx, None, cabi.p(table), max_ctx)
     bf = torch.bfloat16
     qw = (1 + 0.1 * torch.randn(D, device="cuda")).to(bf)
     kw = (1 + 0.1 * torch.randn(D, device="cuda")).to(bf)
@@ -419,7 +418,7 @@ def config6(args):
     k = (torch.randn(chunk, KVH, D, device="cuda") * 0.7).to(bf)
     v = (torch.randn(chunk, KVH, D, device="cuda") * 0.5).to(bf)
     qs, ao = torch.empty(chunk, QH, D, device="cuda", dtype=bf), torch.empty(chunk, QH, D, device="cuda", dtype=bf)
-    io = (U.p(qg), U.p(k), U.p(v), U.p(qw), U.p(kw), U.p(qs), U.p(ao))
+    io = (cabi.p(qg), cabi.p(k), cabi.p(v), cabi.p(qw), cabi.p(kw), cabi.p(qs), cabi.p(ao))
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
@@ -444,7 +443,7 @@ def config6(args):
     def layers(st):
         for l in range(L):
             b = lay[l]
-            ks.decode_layer(l, (U.p(b["qg"]), U.p(b["k"]), U.p(b["v"]), U.p(qw), U.p(kw), U.p(b["q"]), U.p(b["out"])), st)
+            ks.decode_layer(l, (cabi.p(b["qg"]), cabi.p(b["k"]), cabi.p(b["v"]), cabi.p(qw), cabi.p(kw), cabi.p(b["q"]), cabi.p(b["out"])), st)
 
     per_tok = 2 * KVH * D * 2
 
@@ -519,23 +518,23 @@ def config7(args):
     qs = torch.empty(L, B, QH, D, device="cuda", dtype=h)
     out = torch.empty(L, B, QH, D, device="cuda", dtype=h)
     table = torch.empty(ctx * RD, dtype=torch.float32, device="cuda")
-    cabi.call("drk_rope_table_fill", U.p(table), ctx, RD, 1.0e7, sp)
+    cabi.call("drk_rope_table_fill", cabi.p(table), ctx, RD, 1.0e7, sp)
     wsb = lib.drk_decode_workspace_bytes(C.byref(g), B, ctx)
     ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
     scale = 1.0 / np.sqrt(D)
     qgrow, krow, qrow = B * QH * 2 * D * 2, B * KVH * D * 2, B * QH * D * 2
 
     def attn(l, dlen):
-        cabi.call("drk_paged_decode_attention_gated", C.byref(g), C.c_void_p(qs.data_ptr() + l * qrow), U.p(pool), U.p(dtab),
+        cabi.call("drk_paged_decode_attention_gated", C.byref(g), C.c_void_p(qs.data_ptr() + l * qrow), cabi.p(pool), cabi.p(dtab),
                   nblk, dlen, B, ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.F16,
-                  C.c_void_p(qg.data_ptr() + l * qgrow + D * 2), 2 * D, U.p(ws), wsb, sp)
+                  C.c_void_p(qg.data_ptr() + l * qgrow + D * 2), 2 * D, cabi.p(ws), wsb, sp)
 
     def step(s):
         dpos, dlen = C.c_void_p(pos_steps[s].data_ptr()), C.c_void_p(len_steps[s].data_ptr())
         for l in range(L):
-            cabi.call("drk_qk_norm_rope_append", C.byref(g), U.p(pool), U.p(dtab), nblk, dpos, 0, B, l,
+            cabi.call("drk_qk_norm_rope_append", C.byref(g), cabi.p(pool), cabi.p(dtab), nblk, dpos, 0, B, l,
                       C.c_void_p(qg.data_ptr() + l * qgrow), C.c_void_p(k.data_ptr() + l * krow),
-                      C.c_void_p(v.data_ptr() + l * krow), U.p(qn), U.p(kn), 1e-6, RD, 1.0e7, U.p(table), ctx,
+                      C.c_void_p(v.data_ptr() + l * krow), cabi.p(qn), cabi.p(kn), 1e-6, RD, 1.0e7, cabi.p(table), ctx,
                       C.c_void_p(qs.data_ptr() + l * qrow), cabi.F16, sp)
             attn(l, dlen)
 
@@ -574,3 +573,192 @@ def config7(args):
 
 def run(args):
     return {3: config3, 4: config4, 5: config5, 6: config6, 7: config7}[args.config](args)
+
+
+# ---------------------------------------------------------------------------------------------
+# Short kernel measurements of configs 3, 4 and 5 for bench.py's default line: the dominant kernel
+# of each configuration on its real shape, in a pool carved out of the device buffer the headline
+# run leaves behind.  Every figure is algorithmic bytes (or flops) per launch over the average
+# launch duration from HIP events recorded on the launch stream.
+# ---------------------------------------------------------------------------------------------
+def _entry(kernel, bound, per_launch, ms, what, extra=None):
+    peak = HBM_PEAK_GBPS if bound == "hbm" else MFMA_BF16_PEAK_TFLOPS
+    ach = per_launch / (ms * 1e-3) / (1e9 if bound == "hbm" else 1e12)
+    e = {"kernel": kernel, "bound": bound, "avg_launch_us": round(ms * 1e3, 2),
+         ("bytes_per_launch" if bound == "hbm" else "flops_per_launch"): int(per_launch),
+         "achieved": round(ach, 1), "peak": peak, "unit": "GB/s" if bound == "hbm" else "TFLOP/s",
+         "frac": round(ach / peak, 4), "workload": what}
+    if extra:
+        e.update(extra)
+    return e
+
+
+def _shuffled_rows(rng, NB, nblk_per_row):
+    perm = rng.permutation(NB).astype(np.int32)
+    stride = max(nblk_per_row) + 1
+    tab = np.full((len(nblk_per_row), stride), -1, dtype=np.int32)
+    o = 0
+    for i, n in enumerate(nblk_per_row):
+        tab[i, :n] = perm[o:o + n]
+        o += n
+    return tab, stride, perm[o:]
+
+
+def kernel_fractions(buf, seed=11):
+    """buf: a torch uint8 device tensor of at least 16 GiB that may be overwritten."""
+    import torch
+    from deusridet_amd import cabi
+    lib = cabi.lib()
+    stream = torch.cuda.current_stream()
+    sp = C.c_void_p(stream.cuda_stream)
+    KVH, QH, D, bs = 8, 32, 128, 16
+    scale = float(1.0 / np.sqrt(D))
+    rng = np.random.default_rng(seed)
+    res = {}
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+
+    def fit_blocks(L, dt, want):
+        probe = cabi.layout(L, KVH, QH, D, bs, 1, dt)
+        nb = lib.drk_kv_max_blocks_for_budget(C.byref(probe), buf.numel())
+        return min(nb, want)
+
+    def fill(g, table_row_ptr, n_tokens, L, outliers, timed=None, chunk=8192):
+        """append n_tokens N(0,1) tokens (x20 outliers on 1 % of the elements if asked) to one table row"""
+        for p0 in range(0, n_tokens, chunk):
+            m = min(chunk, n_tokens - p0)
+            k = torch.randn(L, m, KVH, D, device="cuda")
+            v = torch.randn(L, m, KVH, D, device="cuda")
+            if outliers:
+                k = torch.where(torch.rand_like(k) < 0.01, k * 20, k)
+                v = torch.where(torch.rand_like(v) < 0.01, v * 20, v)
+            k, v = k.to(torch.bfloat16), v.to(torch.bfloat16)
+            a0, a1 = ev(), ev()
+            a0.record(stream)
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), table_row_ptr, 0, L, p0, m, cabi.p(k), cabi.p(v),
+                      cabi.BF16, sp)
+            a1.record(stream)
+            torch.cuda.synchronize()
+            if timed is not None and m == chunk and p0 > 0:
+                timed.append((a0.elapsed_time(a1), m))
+
+    # ---- config 4: 4 branches x 131 072 tokens of int8 (+ fp16 scales) / fp8 pages ---------------------
+    for name, dt in (("int8", cabi.INT8), ("fp8", cabi.FP8_E4M3)):
+        L, B, ctx = 2, 4, 131072
+        NB = fit_blocks(L, dt, 200000)
+        g = cabi.layout(L, KVH, QH, D, bs, NB, dt)
+        tab, stride, _ = _shuffled_rows(rng, NB, [ctx // bs] * B)
+        dtab = torch.from_numpy(tab).cuda()
+        timed = []
+        for b in range(B):
+            fill(g, C.c_void_p(dtab[b].data_ptr()), ctx, L, True, timed)
+        code = 2 * KVH * D + (2 * KVH * 2 if dt == cabi.INT8 else 0)              # bytes per token and layer
+        ap_ms = float(np.mean([t for t, _ in timed]))
+        ap_bytes = timed[0][1] * L * (2 * KVH * D * 2 + code)
+        res["config4_%s_append" % name] = _entry(
+            "append_kernel<%s>" % name, "hbm", ap_bytes, ap_ms,
+            "quantising bulk append: %d tokens x %d layers per launch, reads 4096 B bf16 and writes %d B per token and layer"
+            % (timed[0][1], L, code))
+        q = torch.randn(L, B, QH, D, device="cuda").to(torch.bfloat16)
+        out = torch.zeros_like(q)
+        wsb = lib.drk_decode_workspace_bytes(C.byref(g), B, ctx)
+        ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+        dlen = torch.full((B,), ctx, dtype=torch.int32, device="cuda")
+        row = B * QH * D * 2
+        ms = _timed_decode(lib, cabi, lambda n: [cabi.call(
+            "drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + (i % L) * row), cabi.p(buf),
+            cabi.p(dtab), stride, cabi.p(dlen), B, ctx, C.c_void_p(out.data_ptr() + (i % L) * row), i % L, scale, cabi.BF16, 0,
+            cabi.p(ws), wsb, sp) for i in range(n)], 40)
+        res["config4_%s" % name] = _entry(
+            "decode_stream_kernel<%s>" % name, "hbm", B * ctx * code, ms,
+            "config 4: 4 branches x 131072 tokens, %s pages (%d B per token and layer), K/V N(0,1) with 1 %% x20 outliers "
+            "quantised on append, pages shuffled over %d blocks" % (name, code, NB))
+        del q, out, ws, dtab
+
+    # ---- config 3: 65 536-token prefix shared by 16 branches + private tails U{0..4096} -------------------
+    L, B, prefix = 2, 16, 65536
+    NB = fit_blocks(L, cabi.BF16, 200000)
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    tails = rng.integers(0, 4097, size=B)
+    rows, stride, _ = _shuffled_rows(rng, NB, [prefix // bs] + [int(t + bs - 1) // bs + 1 for t in tails])
+    stride = prefix // bs + max(int(t + bs - 1) // bs + 1 for t in tails) + 1
+    tab = np.full((B, stride), -1, dtype=np.int32)
+    for b in range(B):
+        nt = int(tails[b] + bs - 1) // bs + 1
+        tab[b, :prefix // bs] = rows[0, :prefix // bs]                            # the same physical pages in every row
+        tab[b, prefix // bs:prefix // bs + nt] = rows[1 + b, :nt]
+    dtab = torch.from_numpy(tab).cuda()
+    fill(g, C.c_void_p(dtab[0].data_ptr()), prefix, L, False)
+    # private tails: appended past the prefix through each branch's own row
+    for b in range(B):
+        n = int(tails[b])
+        if n:
+            k = (torch.randn(L, n, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+            v = (torch.randn(L, n, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), C.c_void_p(dtab[b].data_ptr()), 0, L, prefix, n, cabi.p(k),
+                      cabi.p(v), cabi.BF16, sp)
+            torch.cuda.synchronize()
+    lens = (prefix + tails).astype(np.int32)
+    dlen = torch.from_numpy(lens).cuda()
+    max_ctx = int(lens.max())
+    q = (torch.randn(L, B, QH, D, device="cuda") * 0.5).to(torch.bfloat16)
+    out = torch.zeros_like(q)
+    wsb = lib.drk_decode_shared_workspace_bytes(C.byref(g), B, max_ctx, prefix)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    row = B * QH * D * 2
+
+    def shared_call(n):
+        for i in range(n):
+            l = i % L
+            cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * row), cabi.p(buf), cabi.p(dtab),
+                      stride, cabi.p(dlen), B, max_ctx, prefix, C.c_void_p(out.data_ptr() + l * row), l, scale, cabi.BF16,
+                      cabi.p(ws), wsb, sp)
+
+    pair_ms = _timed_decode(lib, cabi, shared_call, 40)                           # prefix pass + tails, without the merge
+    a0, a1 = ev(), ev()
+    a0.record(stream)
+    shared_call(40)
+    a1.record(stream)
+    torch.cuda.synchronize()
+    call_ms = a0.elapsed_time(a1) / 40
+    distinct = (prefix + int(tails.sum())) * 2 * KVH * D * 2
+    res["config3_shared_prefix"] = _entry(
+        "prefill_mfma_kernel<bf16,shared> + decode_stream_kernel<bf16>", "hbm", distinct, pair_ms,
+        "config 3: 65536-token prefix shared by 16 branches + private tails U{0..4096} (sum %d), bf16; DISTINCT bytes (shared "
+        "pages counted once) over the prefix pass and the tail kernel together" % int(tails.sum()),
+        {"with_merge_us": round(call_ms * 1e3, 2), "with_merge_frac": round(distinct / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+         "logical_bytes_per_launch": int(lens.sum()) * 2 * KVH * D * 2})
+    del q, out, ws, dtab
+
+    # ---- config 5: chunked causal prefill to 32 768 tokens in 2 048-token chunks -------------------------
+    L, chunk, total = 1, 2048, 32768
+    NB = fit_blocks(L, cabi.BF16, 65536)
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    tab, stride, _ = _shuffled_rows(rng, NB, [total // bs])
+    dtab = torch.from_numpy(tab).cuda()
+    per_chunk = []
+    for ps in range(2):                                                           # the first pass warms up
+        per_chunk = []
+        for c in range(total // chunk):
+            k = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+            v = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+            q = torch.randn(chunk, QH, D, device="cuda").to(torch.bfloat16)
+            o = torch.empty_like(q)
+            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), cabi.p(dtab), 0, L, c * chunk, chunk, cabi.p(k), cabi.p(v),
+                      cabi.BF16, sp)
+            a0, a1 = ev(), ev()
+            a0.record(stream)
+            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, c * chunk, chunk,
+                      scale, cabi.BF16, None, 0, sp)
+            a1.record(stream)
+            torch.cuda.synchronize()
+            per_chunk.append((a0.elapsed_time(a1), 4.0 * chunk * (c * chunk + (chunk + 1) / 2.0) * D * QH))
+    tot_ms, tot_fl = sum(t for t, _ in per_chunk), sum(f for _, f in per_chunk)
+    res["config5_prefill"] = _entry(
+        "prefill_mfma_kernel<bf16>", "mfma", tot_fl / len(per_chunk), tot_ms / len(per_chunk),
+        "config 5: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV x 128 bf16; average "
+        "over the 16 launches (flops = 4 M (pos_start + (M+1)/2) D QH per chunk)",
+        {"last_chunk_us": round(per_chunk[-1][0] * 1e3, 1),
+         "last_chunk_TFLOPs": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12, 1),
+         "last_chunk_frac": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+         "first_chunk_TFLOPs": round(per_chunk[0][1] / (per_chunk[0][0] * 1e-3) / 1e12, 1)})
+    return res

@@ -163,3 +163,15 @@ def check(code):
 def call(name, *args):
     """Call an int-returning entry point and raise DrkError on failure."""
     return check(getattr(lib(), name)(*args))
+
+
+# ---- plumbing for callers that keep device memory in torch tensors -------------------
+def p(t):
+    """Device pointer of a torch tensor as a ctypes void pointer (None stays None)."""
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def stream_ptr():
+    """The hipStream_t of torch's current stream, as the entry points take it."""
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
