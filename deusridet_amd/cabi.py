@@ -93,6 +93,7 @@ SIGNATURES = {
     "drk_debug_set_decode_lds_pad": (None, [_i32]),
     "drk_debug_set_append_chunks": (None, [_i32, _i32, _i32]),
     "drk_debug_set_prefill_split": (None, [_i32]),
+    "drk_debug_set_prefill_two_phase": (None, [_i32]),
     "drk_probe_read_bandwidth": (_i32, [_vp, _sz, _i32, _vp, C.POINTER(C.c_float)]),
     "drk_probe_read_bandwidth_permuted": (_i32, [_vp, _sz, _i32, _i32, _vp, C.POINTER(C.c_float)]),
     "drk_probe_mfma_rate": (_i32, [_i32, _vp, C.POINTER(C.c_float)]),

@@ -143,23 +143,23 @@ __device__ __forceinline__ void pf_sched_barrier()
 #endif
 }
 
-// one wave's 16-token group of a tile: 16 rows of RB bytes = NL 128-bit loads per lane
-template <int RB>
+// one wave's group of ROWS consecutive tokens of a tile: ROWS rows of RB bytes = NL 128-bit loads per lane
+template <int RB, int ROWS = 16>
 struct PfGroup {
-    static constexpr int NL = RB / 64;
+    static constexpr int NL = RB * ROWS / 1024;
     uint4 r[NL];
 };
 
-template <bool ONCE, int RB>
-__device__ __forceinline__ PfGroup<RB> pf_load_group(const uint8_t *__restrict__ base, bool valid, size_t off, int lane)
+template <bool ONCE, int RB, int ROWS = 16>
+__device__ __forceinline__ PfGroup<RB, ROWS> pf_load_group(const uint8_t *__restrict__ base, bool valid, size_t off, int lane)
 {
-    PfGroup<RB> g;
+    PfGroup<RB, ROWS> g;
 #pragma unroll
-    for (int j = 0; j < PfGroup<RB>::NL; j++) g.r[j] = make_uint4(0, 0, 0, 0);
+    for (int j = 0; j < PfGroup<RB, ROWS>::NL; j++) g.r[j] = make_uint4(0, 0, 0, 0);
     if (valid) {
         const uint8_t *p = base + off + (size_t)lane * 16;
 #pragma unroll
-        for (int j = 0; j < PfGroup<RB>::NL; j++) {
+        for (int j = 0; j < PfGroup<RB, ROWS>::NL; j++) {
             if constexpr (ONCE) g.r[j] = ld_stream128(p + 1024 * j);   // every page is read by one workgroup only: stream it
             else g.r[j] = *(const uint4 *)(p + 1024 * j);              // the row tiles of a chunk share each page through the L2
         }
@@ -169,18 +169,18 @@ __device__ __forceinline__ PfGroup<RB> pf_load_group(const uint8_t *__restrict__
 
 // 16-bit pages: the 16-byte chunk j of a lane belongs to row (lane * 16 + 1024 j) / RB of the group.
 // Rows at or past `lim` may hold anything and are stored as zeros.
-template <int PITCH, int RB>
-__device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup<RB> &g, int w, int lane, int lim)
+template <int PITCH, int RB, int ROWS = 16>
+__device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup<RB, ROWS> &g, int w, int lane, int lim)
 {
     const int bp0 = lane * 16, row0 = bp0 / RB;
-    uint8_t *dst = lds + (w * 16 + row0) * PITCH + bp0 % RB;
+    uint8_t *dst = lds + (w * ROWS + row0) * PITCH + bp0 % RB;
     constexpr int RSTEP = 1024 / RB;                          // rows between a lane's consecutive chunks
-    if (lim >= 16) {                                          // the common case, wave-uniform
+    if (lim >= ROWS) {                                        // the common case, wave-uniform
 #pragma unroll
-        for (int j = 0; j < PfGroup<RB>::NL; j++) *(uint4 *)(dst + j * RSTEP * PITCH) = g.r[j];
+        for (int j = 0; j < PfGroup<RB, ROWS>::NL; j++) *(uint4 *)(dst + j * RSTEP * PITCH) = g.r[j];
     } else {
 #pragma unroll
-        for (int j = 0; j < PfGroup<RB>::NL; j++)
+        for (int j = 0; j < PfGroup<RB, ROWS>::NL; j++)
             *(uint4 *)(dst + j * RSTEP * PITCH) = row0 + j * RSTEP < lim ? g.r[j] : make_uint4(0, 0, 0, 0);
     }
 }
@@ -188,13 +188,13 @@ __device__ __forceinline__ void pf_store_group(uint8_t *lds, const PfGroup<RB> &
 // 8-bit pages: chunk j of a lane holds 16 codes of row (lane * 16 + 1024 j) / RB; they are stored as
 // the fp16 values code * scale (int8; sc[j] = the row's fp16 scale) or as the fp8 values themselves.
 // Rows at or past `lim` may hold anything -- codes and scales -- and are stored as zeros.
-template <int PITCH, int KV, int RB>
-__device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup<RB> &g, int w, int lane,
-                                                  const uint16_t (&sc)[PfGroup<RB>::NL], int lim)
+template <int PITCH, int KV, int RB, int ROWS = 16>
+__device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup<RB, ROWS> &g, int w, int lane,
+                                                  const uint16_t (&sc)[PfGroup<RB, ROWS>::NL], int lim)
 {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-    for (int j = 0; j < PfGroup<RB>::NL; j++) {
+    for (int j = 0; j < PfGroup<RB, ROWS>::NL; j++) {
         const int bp = lane * 16 + 1024 * j, row = bp / RB, col = bp % RB;
         uint32_t h[8];
         if constexpr (KV == DRK_INT8) {
@@ -220,7 +220,7 @@ __device__ __forceinline__ void pf_store_group_q8(uint8_t *lds, const PfGroup<RB
 #pragma unroll
             for (int i = 0; i < 8; i++) h[i] = 0u;
         }
-        uint8_t *dst = lds + (w * 16 + row) * PITCH + col * 2;
+        uint8_t *dst = lds + (w * ROWS + row) * PITCH + col * 2;
         *(uint4 *)(dst) = make_uint4(h[0], h[1], h[2], h[3]);
         *(uint4 *)(dst + 16) = make_uint4(h[4], h[5], h[6], h[7]);
     }
@@ -540,6 +540,372 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(Pre
     }
 }
 
+// As pf_store_group, without a branch: every chunk is a select between the loaded bytes and zeros.
+template <int PITCH, int RB, int ROWS>
+__device__ __forceinline__ void pf_store_group_sel(uint8_t *lds, const PfGroup<RB, ROWS> &g, int w, int lane, int lim)
+{
+    const int bp0 = lane * 16, row0 = bp0 / RB;
+    uint8_t *dst = lds + (w * ROWS + row0) * PITCH + bp0 % RB;
+    constexpr int RSTEP = 1024 / RB;
+#pragma unroll
+    for (int j = 0; j < PfGroup<RB, ROWS>::NL; j++) {
+        const bool ok = row0 + j * RSTEP < lim;
+        const uint4 v = g.r[j];
+        *(uint4 *)(dst + j * RSTEP * PITCH) = make_uint4(ok ? v.x : 0u, ok ? v.y : 0u, ok ? v.z : 0u, ok ? v.w : 0u);
+    }
+}
+
+// max(x of lane n, x of lane n ^ 32) without a trip through LDS
+__device__ __forceinline__ float pf_max_halves(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// ---- the chunk kernel in two phases ("ping-pong") ---------------------------------------------
+// In the kernel above the matrix cores and the vector ALU mostly take turns: the two waves that
+// share a SIMD (from two independent workgroups) drift into the same phase and then wait for the
+// same unit.  Here ONE workgroup of eight waves holds 256 rows (wave w: rows 32 w .. 32 w + 31),
+// waves w and w + 4 share a SIMD, and the two halves of the workgroup are kept half a tile apart
+// by the workgroup barrier itself: between two barriers waves 0-3 run the softmax of tile t on the
+// vector ALU while waves 4-7 run their matrix products (PV of tile t-1, QK^T of tile t); after the
+// next barrier the roles swap.  The matrix pipe of every SIMD always has one wave to take work from.
+//
+//   even phase 2t    A (waves 0-3): its share of K(t+1), V(t) -> LDS; softmax(t)
+//                    B (waves 4-7): PV(t-1), QK^T(t)
+//   odd phase 2t+1   A: PV(t), QK^T(t+1)
+//                    B: softmax(t); its share of K(t+2), V(t+1) -> LDS
+//
+// The memory side of a tile rides in the wave's vector phase (registers -> LDS, then the global loads
+// of the next tile into the same registers); it is straight-line code -- a taken branch costs a wave
+// tens of cycles, and a staging step with a dozen of them cost more than the softmax.  A buffer is
+// rewritten between its last reader's barrier and its next reader's: K(x) in phase 2x-3 or 2x-2,
+// V(x) in phase 2x-1 or 2x.  One set of score registers per wave is enough: the scores of a tile are
+// dead once its weights are packed.
+// grid = ceil(M / TPW) * KVH with TPW = 256 / (QH/KVH) query tokens per workgroup, longest walk
+// first; block = 512; one workgroup per CU.  head_dim 128; causal chunks only.
+template <int DT, int KV = DT, int IO = DT>
+__global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
+{
+    constexpr int D = 128;
+    constexpr bool Q8 = KV == DRK_INT8 || KV == DRK_FP8_E4M3;
+    constexpr int RB = D * (Q8 ? 1 : 2);
+    constexpr int kPitchK = D * 2 + 16, kPitchV = D * 2 + 32;
+    constexpr int NKS = D / 16, NDT = D / 32;
+    constexpr int ROWS = 8;                                 // tokens of a tile one wave stages
+    __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPitchK];
+    __shared__ __align__(16) uint8_t v_lds2[2][kPfBN * kPitchV];
+
+    const int kvh = (int)blockIdx.x % A.KVH;
+    const int nqt = (int)gridDim.x / A.KVH;
+    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, g = lane >> 5;
+    const bool grpA = w < 4;
+
+    const int G = A.QH / A.KVH, TPW = A.tpw;
+    const int r = w * 32 + n, rt = r / G;
+    const int tq = qt * TPW + rt;
+    const int head = kvh * G + (r - rt * G);
+    const bool row_live = rt < TPW && tq < A.M;
+    const int vis = A.pos_start + tq + 1;
+    const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
+    const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
+    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+
+    // Q as the B operand, multiplied by scale * log2(e) on the way in (rounded once more to the 16-bit
+    // type): the products then are the exponents themselves and the softmax needs no multiply per score.
+    uint4 qf[NKS];
+    {
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
+        const float c = A.scale_log2e;
+        auto scaled = [&](uint32_t w2) -> uint32_t {
+            return pack2<DT>(elem16_to_f((uint16_t)(w2 & 0xffffu), IO) * c, elem16_to_f((uint16_t)(w2 >> 16), IO) * c);
+        };
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            const uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+            qf[ks] = make_uint4(scaled(v.x), scaled(v.y), scaled(v.z), scaled(v.w));
+        }
+    }
+
+    const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+    // ---- pages -------------------------------------------------------------------------------------
+    // The block size is a power of two >= 16 (the host dispatches other sizes to the kernel above), so the
+    // 8 tokens a wave stages lie in one block, a 16-token run has one page, and a tile's blocks never
+    // straddle a multiple of 64.  Table entries come in windows of 64, one per lane, by a vector load (a
+    // scalar load would be waited for at every barrier, whose LDS wait counts on the same counter); two
+    // windows are held, so an entry is in a register long before its tile is reached.  Everything here is
+    // wave-uniform, straight-line code: the only branch is the change of window, every 64 blocks.
+    const int sh = A.bs_shift;
+    const int tgw = w * ROWS;                                 // the wave's first token within a tile
+    const int nblk_needed = (lim_wg + A.bs - 1) >> sh;
+    auto load_window = [&](int lb0) -> int {
+        const int i = lb0 + lane;
+        return i < nblk_needed ? A.table[i] : -1;             // entries past the chunk's last block are never read
+    };
+    auto pages_of = [&](int win) -> unsigned long long { return __builtin_amdgcn_ballot_w64(win >= 0 && win < A.NB); };
+    int win_lb0 = 0;
+    int win_a = load_window(0), win_b = load_window(64);
+    unsigned long long present_a = pages_of(win_a);           // bit i: block win_lb0 + i has a page
+    // the wave's page in `tile` (-1: a hole, or past the end) and the tile's four page flags, one per 16-token run
+    auto lookup = [&](int tile, int &blk, int &flags) {
+        const int lb0 = (tile * kPfBN) >> sh;
+        if (__builtin_expect(lb0 >= win_lb0 + 64, 0)) {       // tiles are asked for in ascending order
+            win_lb0 += 64;
+            win_a = win_b;
+            win_b = load_window(win_lb0 + 64);
+            present_a = pages_of(win_a);
+        }
+        const uint32_t m = (uint32_t)(present_a >> (lb0 - win_lb0));
+        flags = (int)((m & 1u) | (((m >> (16 >> sh)) & 1u) << 1) | (((m >> (32 >> sh)) & 1u) << 2) | (((m >> (48 >> sh)) & 1u) << 3));
+        const int tg = tile * kPfBN + tgw;
+        const int li = (tg >> sh) - win_lb0;
+        const int b = __builtin_amdgcn_readlane(win_a, li);
+        blk = (((present_a >> li) & 1ull) != 0 && tg < lim_wg) ? b : -1;
+    };
+
+    pf_f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+    // The softmax reference m_ref (per row): the products start from -m_ref (the C operand), so a score
+    // arrives as its exponent relative to the reference.  The reference moves only when a tile's maximum
+    // exceeds it by more than kLazy (or is the row's first finite one): weights stay below 2^kLazy, and O
+    // and the row sum are rescaled on those rare occasions only.  out = O / l does not depend on it.
+    constexpr float kLazy = 8.0f;
+    float m_ref = 0.0f, l_run = 0.0f;
+    bool m_init = false;
+    pf_f32x16 negm;
+#pragma unroll
+    for (int i = 0; i < 16; i++) negm[i] = 0.0f;
+
+    // ---- staging -----------------------------------------------------------------------------------
+    // A wave moves 8 rows of K and of V per tile: global -> registers one tile ahead, registers -> LDS when
+    // the buffer's last readers have passed.  No branches: a missing page is read from block 0 instead and
+    // stored as zeros, like the rows past the chunk's end (which may hold anything).
+    constexpr int NL = PfGroup<RB, ROWS>::NL;
+    PfGroup<RB, ROWS> kreg, vreg;
+    uint16_t ksc[NL], vsc[NL];
+    int klim = 0, vlim = 0;                                  // rows of kreg / vreg that are real
+    auto fetch = [&](PfGroup<RB, ROWS> &reg, uint16_t (&sc)[NL], int &lim, bool is_v, int tile, int blk) {
+        const int tg = tile * kPfBN + tgw;
+        const int tin = tg & (A.bs - 1);
+        const size_t boff = (size_t)max(blk, 0) * A.block_stride;
+        const uint8_t *p = kbase + (is_v ? A.kv_plane : 0) + boff + (size_t)tin * RB + (size_t)lane * 16;
+#pragma unroll
+        for (int j = 0; j < NL; j++) reg.r[j] = *(const uint4 *)(p + 1024 * j);   // the row tiles of a chunk share each page through the L2
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            if constexpr (KV == DRK_INT8) {
+                const int row = (lane * 16 + 1024 * j) / RB;
+                const size_t soff = boff + 2 * (size_t)A.kv_plane + (is_v ? A.scale_plane : 0) + ((size_t)kvh * A.bs + tin + row) * 2;
+                sc[j] = *(const uint16_t *)(A.pool_layer + soff);
+            } else {
+                sc[j] = 0;
+            }
+        }
+        lim = blk >= 0 ? lim_wg - tg : 0;
+    };
+    auto stage_k = [&](int tile) {
+        if constexpr (Q8) pf_store_group_q8<kPitchK, KV, RB, ROWS>(&k_lds2[tile & 1][0], kreg, w, lane, ksc, klim);
+        else pf_store_group_sel<kPitchK, RB, ROWS>(&k_lds2[tile & 1][0], kreg, w, lane, klim);
+    };
+    auto stage_v = [&](int tile) {
+        if constexpr (Q8) pf_store_group_q8<kPitchV, KV, RB, ROWS>(&v_lds2[tile & 1][0], vreg, w, lane, vsc, vlim);
+        else pf_store_group_sel<kPitchV, RB, ROWS>(&v_lds2[tile & 1][0], vreg, w, lane, vlim);
+    };
+
+    pf_f32x16 s[2];                 // scores of the tile in flight: [32-token half][16 per lane]
+    uint4 pb[2][2];                 // its weights, packed: [token half][k-half], the B operand of PV
+
+    // S^T = K Q^T.  The operand reads run two k-steps ahead of the products that use them; scheduling
+    // barriers pin that order, so that at most six operands are in registers at a time.
+    auto qk = [&](int tile) {
+        const uint8_t *ka = &k_lds2[tile & 1][0] + n * kPitchK + g * 16;
+        uint4 a[NKS][2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            a[ks][0] = *(const uint4 *)(ka + ks * 32);
+            a[ks][1] = *(const uint4 *)(ka + 32 * kPitchK + ks * 32);
+        }
+        pf_sched_barrier();
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            if (ks + 2 < NKS) {
+                a[ks + 2][0] = *(const uint4 *)(ka + (ks + 2) * 32);
+                a[ks + 2][1] = *(const uint4 *)(ka + 32 * kPitchK + (ks + 2) * 32);
+            }
+            if (ks == 0) {                                   // the products start from minus the row's reference
+                s[0] = mfma32<DT>(a[ks][0], qf[ks], negm);
+                s[1] = mfma32<DT>(a[ks][1], qf[ks], negm);
+            } else {
+                s[0] = mfma32<DT>(a[ks][0], qf[ks], s[0]);
+                s[1] = mfma32<DT>(a[ks][1], qf[ks], s[1]);
+            }
+            pf_sched_barrier();
+        }
+    };
+    // O^T += V^T P^T: 16 products, two transposed 8-byte reads each, the reads four products ahead
+    auto pv = [&](int tile) {
+        const uint8_t *v_lds = &v_lds2[tile & 1][0];
+        const int j16 = lane & 15;
+        const int dsub = 16 * ((lane >> 4) & 1) + 4 * (j16 & 3);
+        const uint8_t *vb = v_lds + (4 * g + (j16 >> 2)) * kPitchV + dsub * 2;
+        uint2 lo[16], hi[16];
+        auto rd = [&](int i) {                               // product i = (tt, mh, dt) = (i / 8, (i / 4) & 1, i & 3)
+            const uint8_t *vt = vb + ((i >> 3) * 32 + 16 * ((i >> 2) & 1)) * kPitchV + (i & 3) * 64;
+            lo[i] = lds_read_tr16(vt);
+            hi[i] = lds_read_tr16(vt + 8 * kPitchV);
+        };
+#pragma unroll
+        for (int i = 0; i < 4; i++) rd(i);
+        pf_sched_barrier();
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if (i + 4 < 16) rd(i + 4);
+            o[i & 3] = mfma32<DT>(make_uint4(lo[i].x, lo[i].y, hi[i].x, hi[i].y), pb[i >> 3][(i >> 2) & 1], o[i & 3]);
+            pf_sched_barrier();
+        }
+    };
+    // scores of tile `it` (page flags `flags`) -> packed weights, running maximum and sum, rescale of O^T
+    auto softmax = [&](int it, int flags) {
+        const int tile_t = it * kPfBN;
+        if (flags != 15 || it >= first_masked_tile) {
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    const bool ok = (tile_t + tl) < vis && ((flags >> (tl >> 4)) & 1) != 0;
+                    s[tt][i] = ok ? s[tt][i] : -INFINITY;
+                }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[tt][i]);
+        tmax = pf_max_halves(tmax);                          // a row's scores lie in lanes n and n + 32
+        const bool move = m_init ? tmax > kLazy : tmax > -INFINITY;
+        if (__any(move)) {
+            const float delta = move ? tmax : 0.0f;
+            m_init = m_init || move;
+            m_ref += delta;
+            const float alpha = __builtin_amdgcn_exp2f(-delta);
+            l_run *= alpha;
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[tt][i] -= delta;
+#pragma unroll
+            for (int i = 0; i < 16; i++) negm[i] = -m_ref;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+        }
+        float psum = 0.0f;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            float p[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) p[i] = __builtin_amdgcn_exp2f(s[tt][i]);
+            pb[tt][0] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+            pb[tt][1] = make_uint4(pack2<DT>(p[8], p[9]), pack2<DT>(p[10], p[11]), pack2<DT>(p[12], p[13]), pack2<DT>(p[14], p[15]));
+            psum = pf_sum2<DT>(pb[tt][0], psum);
+            psum = pf_sum2<DT>(pb[tt][1], psum);
+        }
+        l_run += psum;
+    };
+
+    // The memory side of tile t, this wave's share: K(t+1) and V(t) go from registers to LDS, then K(t+2)
+    // and V(t+1) are requested.  fl0 / fl1 / fl2 are the page flags of tiles t, t+1, t+2 afterwards.
+    int blk_next, fl0 = 15, fl1, fl2;                         // blk_next: the wave's page in tile t+1
+    auto stage = [&](int t) {
+        stage_k(t + 1);
+        stage_v(t);
+        int blk2, f;
+        lookup(t + 2, blk2, f);
+        fetch(kreg, ksc, klim, false, t + 2, blk2);
+        fetch(vreg, vsc, vlim, true, t + 1, blk_next);
+        blk_next = blk2;
+        fl0 = fl1;
+        fl1 = fl2;
+        fl2 = f;
+    };
+
+    // ---- prologue: K(0) in LDS; K(1) and V(0) in registers ----
+    {
+        int blk0;
+        lookup(0, blk0, fl1);
+        fetch(kreg, ksc, klim, false, 0, blk0);
+        stage_k(0);
+        lookup(1, blk_next, fl2);
+        fetch(kreg, ksc, klim, false, 1, blk_next);
+        fetch(vreg, vsc, vlim, true, 0, blk0);
+    }
+    __syncthreads();
+    // Both halves pass the same number of barriers, 2 ntiles + 1.  The loop bodies are straight-line code
+    // (the accumulators are updated in place): the product past the last tile multiplies whatever the other
+    // K buffer holds and its result is never read, and the staging past the last tile stores zeros.
+    // A buffer is rewritten only between its last reader's barrier and its next reader's: K(x) in phases
+    // 2x-3 or 2x-2, V(x) in phases 2x-1 or 2x (phase 2t: softmax of A / products of B for tile t).
+    if (grpA) {
+        qk(0);
+#pragma unroll 1
+        for (int t = 0; t < ntiles; t++) {
+            stage(t);                                        // phase 2t: K(t+1), V(t)
+            softmax(t, fl0);
+            __syncthreads();
+            pv(t);
+            qk(t + 1);
+            __syncthreads();
+        }
+        __syncthreads();
+    } else {
+        stage(0);                                            // phase 0: K(1), V(0)
+        qk(0);
+        __syncthreads();
+#pragma unroll 1
+        for (int t = 0; t < ntiles; t++) {
+            softmax(t, fl0);
+            stage(t + 1);                                    // phase 2t+1: K(t+2), V(t+1)
+            __syncthreads();
+            pv(t);
+            qk(t + 1);
+            __syncthreads();
+        }
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (row_live && (l_tot > 0.0f || A.gate)) {
+        const bool have = l_tot > 0.0f;
+        const float inv = have ? 1.0f / l_tot : 0.0f;
+        uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * (D * 2);
+        const uint16_t *grow = A.gate ? A.gate + ((size_t)tq * A.QH + head) * A.gate_stride : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; b4++) {
+                const int d0 = dt * 32 + 8 * b4 + 4 * g;
+                uint2 v = have ? make_uint2(pack2<IO>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
+                                            pack2<IO>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv))
+                               : *(const uint2 *)(orow + d0 * 2);
+                if (grow) {
+                    const uint2 gv = *(const uint2 *)(grow + d0);
+                    v.x = (uint32_t)gated_elem16((uint16_t)(v.x & 0xffffu), (uint16_t)(gv.x & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.x >> 16), (uint16_t)(gv.x >> 16), IO) << 16);
+                    v.y = (uint32_t)gated_elem16((uint16_t)(v.y & 0xffffu), (uint16_t)(gv.y & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.y >> 16), (uint16_t)(gv.y >> 16), IO) << 16);
+                }
+                *(uint2 *)(orow + d0 * 2) = v;
+            }
+    }
+}
+
 // ---- shared-prefix ("cascade") decode: host side of the prefix pass -------------------
 // One launch covers tokens [0, shared) for all B branches; the private tails go
 // through the stream kernel with start_tile = shared / 64.
@@ -599,6 +965,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 // pos_start + t + 1, all rows read one table -- so the kernel runs in that mode over tokens
 // [0, pos_start + M) with the context split over the whole chip, and a small kernel folds each
 // row's pieces (and applies the gate).
+int g_prefill_two_phase = 1;                   // 0: never; 1: by the rule in prefill_impl; 2: whenever the geometry allows (tests)
 int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
 constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
 
@@ -748,6 +1115,7 @@ using namespace drk;
 extern "C" {
 
 void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
+void drk_debug_set_prefill_two_phase(int mode) { g_prefill_two_phase = mode < 0 ? 1 : (mode > 2 ? 2 : mode); }
 
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 {
@@ -825,6 +1193,28 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = (const uint16_t *)gate; A.gate_stride = gate_stride;
     hipStream_t st = (hipStream_t)stream;
+    // Long chunks of head_dim 128 take the two-phase kernel (256 rows per workgroup, one workgroup per CU)
+    // when that still gives at least three quarters of the CUs a workgroup.  That kernel takes its pages
+    // without a branch, which wants a block size that is a power of two and at least 16.
+    const int G = a.QH / a.KVH;
+    if (a.D == 128 && G <= 256 && A.bs_shift >= 4 && g_prefill_two_phase != 0) {
+        const int tpw2 = 256 / G;
+        const long wgs2 = (long)((M + tpw2 - 1) / tpw2) * a.KVH;
+        if (wgs2 >= 192 || g_prefill_two_phase > 1) {
+            A.tpw = tpw2;
+            dim3 grid2((unsigned)wgs2);
+#define DRK_PP_LAUNCH(DT, KV, IO) hipLaunchKernelGGL((prefill_pp_kernel<DT, KV, IO>), grid2, dim3(512), 0, st, A)
+            if (a.dtype == DRK_BF16) DRK_PP_LAUNCH(DRK_BF16, DRK_BF16, DRK_BF16);
+            else if (a.dtype == DRK_F16) DRK_PP_LAUNCH(DRK_F16, DRK_F16, DRK_F16);
+            else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16) DRK_PP_LAUNCH(DRK_F16, DRK_INT8, DRK_BF16);
+            else if (a.dtype == DRK_INT8) DRK_PP_LAUNCH(DRK_F16, DRK_INT8, DRK_F16);
+            else if (io_dtype == DRK_BF16) DRK_PP_LAUNCH(DRK_F16, DRK_FP8_E4M3, DRK_BF16);
+            else DRK_PP_LAUNCH(DRK_F16, DRK_FP8_E4M3, DRK_F16);
+#undef DRK_PP_LAUNCH
+            DRK_LAUNCH_CHECK("prefill_pp_kernel");
+            return DRK_OK;
+        }
+    }
 #define DRK_PF_LAUNCH(DT, KV, IO)                                                                                        \
     do {                                                                                                                \
         if (a.D == 128) hipLaunchKernelGGL((prefill_mfma_kernel<DT, false, KV, IO, 128>), grid, dim3(256), 0, st, A);   \

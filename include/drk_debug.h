@@ -41,6 +41,10 @@ void drk_debug_set_decode_lds_pad(int bytes);
 /* Tuning: which prefill chunks run with the context split over the chip (they must stand behind 2 048 tokens
  * or more): negative = the library's cost rule (default); 0 = none; n = every chunk of up to n rows. */
 void drk_debug_set_prefill_split(int max_rows);
+/* Tuning: which causal chunks of head_dim 128 run on the two-phase chunk kernel (eight waves, 256 rows per
+ * workgroup): 0 = none (the four-wave kernel); 1 = the library's rule (default: chunks long enough to give
+ * most CUs a workgroup); 2 = every chunk the geometry allows. */
+void drk_debug_set_prefill_two_phase(int mode);
 /* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
  * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */
 void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chunks);

@@ -1,6 +1,6 @@
 """GPU parity: chunked causal prefill over pages (paged_attention.cu:465-554) --
-the MFMA kernel and the row-wise path against the fp64 oracle, tolerance
-|err| <= 2e-2 + 1e-2*|want|."""
+the MFMA kernels (the 128-row one and the two-phase 256-row one) and the row-wise
+path against the fp64 oracle, tolerance |err| <= 2e-2 + 1e-2*|want|."""
 import ctypes as C
 
 import numpy as np
@@ -11,6 +11,17 @@ from oracle import binding as orc
 from tests import util as U
 
 pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True, params=["by_rule", "two_phase"])
+def chunk_kernel(request):
+    """Every case runs twice: with the library's own choice of chunk kernel, and with the two-phase
+    kernel taken wherever its geometry allows (head_dim 128, blocks of 16 * 2^k tokens), whatever the
+    chunk's length."""
+    lib = cabi.lib()
+    lib.drk_debug_set_prefill_two_phase(2 if request.param == "two_phase" else 1)
+    yield request.param
+    lib.drk_debug_set_prefill_two_phase(1)
 
 
 def run_prefill(g, dq, dpool, dtab, layer, pos_start, M, scale, dtype, QH, D):
