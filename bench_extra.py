@@ -648,16 +648,9 @@ def kernel_fractions(buf, seed=11):
         g = cabi.layout(L, KVH, QH, D, bs, NB, dt)
         tab, stride, _ = _shuffled_rows(rng, NB, [ctx // bs] * B)
         dtab = torch.from_numpy(tab).cuda()
-        timed = []
         for b in range(B):
-            fill(g, C.c_void_p(dtab[b].data_ptr()), ctx, L, True, timed)
+            fill(g, C.c_void_p(dtab[b].data_ptr()), ctx, L, True)
         code = 2 * KVH * D + (2 * KVH * 2 if dt == cabi.INT8 else 0)              # bytes per token and layer
-        ap_ms = float(np.mean([t for t, _ in timed]))
-        ap_bytes = timed[0][1] * L * (2 * KVH * D * 2 + code)
-        res["config4_%s_append" % name] = _entry(
-            "append_kernel<%s>" % name, "hbm", ap_bytes, ap_ms,
-            "quantising bulk append: %d tokens x %d layers per launch, reads 4096 B bf16 and writes %d B per token and layer"
-            % (timed[0][1], L, code))
         q = torch.randn(L, B, QH, D, device="cuda").to(torch.bfloat16)
         out = torch.zeros_like(q)
         wsb = lib.drk_decode_workspace_bytes(C.byref(g), B, ctx)
@@ -673,6 +666,43 @@ def kernel_fractions(buf, seed=11):
             "config 4: 4 branches x 131072 tokens, %s pages (%d B per token and layer), K/V N(0,1) with 1 %% x20 outliers "
             "quantised on append, pages shuffled over %d blocks" % (name, code, NB))
         del q, out, ws, dtab
+
+    # ---- config 4's append: the quantising bulk append on a prefill chunk's shape -------------------------
+    # 2048 tokens x 36 layers of bf16 K and V per launch, four source sets in rotation (1.2 GB, so no launch
+    # finds its source in a cache), written to 16 successive positions of a shuffled table.
+    L, m, NSRC = 36, 2048, 4
+    srcs = []
+    for _ in range(NSRC):
+        kv = []
+        for _ in range(2):
+            x = torch.randn(L, m, KVH, D, device="cuda")
+            kv.append(torch.where(torch.rand_like(x) < 0.01, x * 20, x).to(torch.bfloat16))
+            del x
+        srcs.append(kv)
+    for name, dt in (("int8", cabi.INT8), ("fp8", cabi.FP8_E4M3)):
+        NB = fit_blocks(L, dt, 16 * m // bs + 8)
+        g = cabi.layout(L, KVH, QH, D, bs, NB, dt)
+        npos = min(16, (NB - 8) * bs // m)
+        tab = torch.from_numpy(rng.permutation(NB).astype(np.int32)).cuda()
+        code = 2 * KVH * D + (2 * KVH * 2 if dt == cabi.INT8 else 0)
+
+        def launches(n):
+            for it in range(n):
+                k, v = srcs[it % NSRC]
+                cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), cabi.p(tab), 0, L, (it % npos) * m, m, cabi.p(k), cabi.p(v),
+                          cabi.BF16, sp)
+        launches(4)
+        a0, a1 = ev(), ev()
+        torch.cuda.synchronize()
+        a0.record(stream)
+        launches(32)
+        a1.record(stream)
+        torch.cuda.synchronize()
+        res["config4_%s_append" % name] = _entry(
+            "append_quant_kernel<%s>" % name, "hbm", m * L * (2 * KVH * D * 2 + code), a0.elapsed_time(a1) / 32,
+            "quantising bulk append: %d tokens x %d layers per launch, reads 4096 B bf16 and writes %d B per token and layer; "
+            "four source sets in rotation" % (m, L, code))
+    del srcs
 
     # ---- config 3: 65 536-token prefix shared by 16 branches + private tails U{0..4096} -------------------
     L, B, prefix = 2, 16, 65536

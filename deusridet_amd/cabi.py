@@ -92,6 +92,8 @@ SIGNATURES = {
     "drk_debug_time_decode_kernel": (None, [_i32]),
     "drk_debug_set_decode_lds_pad": (None, [_i32]),
     "drk_debug_set_append_chunks": (None, [_i32, _i32, _i32]),
+    "drk_debug_check_int8_scale_math": (_i32, [_vp, _vp]),
+    "drk_debug_set_quant_append_pairs": (None, [_i32]),
     "drk_debug_set_prefill_split": (None, [_i32]),
     "drk_debug_set_prefill_two_phase": (None, [_i32]),
     "drk_probe_read_bandwidth": (_i32, [_vp, _sz, _i32, _vp, C.POINTER(C.c_float)]),

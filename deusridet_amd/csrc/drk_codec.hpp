@@ -67,6 +67,63 @@ __device__ __forceinline__ float row16_max(float v)
     return v;
 }
 
+// The int8 scale of a row from its largest magnitude, and the reciprocal the codes are made with:
+//   scale = fp16(amax / 127), saturated to the largest finite fp16;  rcp = 1 / scale  (0 for a zero scale),
+// both divisions correctly rounded in fp32.  IEEE = the compiler's full division sequences (about two dozen
+// instructions for the two); otherwise one multiply by the rounded reciprocal plus one residual correction
+// each, which gives the same bits for every input that occurs here: amax is the magnitude of a bf16 or fp16
+// number, and the scale is an fp16 number (so its significand is never all ones, the one case in which the
+// corrected reciprocal of a 1-ulp estimate can be off).  drk_debug_check_int8_scale_math compares the two
+// forms over all of those inputs on the device.
+template <bool IEEE>
+__device__ __forceinline__ void int8_row_scale(float amax, uint16_t &scale_bits, float &rcp)
+{
+    float s32;
+    if (IEEE) {
+        s32 = __fdiv_rn(amax, 127.0f);
+    } else {
+        const float c = 1.0f / 127.0f;
+        const float q = __fmul_rn(amax, c);
+        s32 = __fmaf_rn(__fmaf_rn(-q, 127.0f, amax), c, q);
+        s32 = amax == INFINITY ? amax : s32;                  // inf - inf in the residual
+    }
+    uint16_t sh = __half_as_ushort(__float2half_rn(s32));
+    if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
+    const float sf = f16_bits_to_f(sh);
+    if (IEEE) {
+        rcp = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
+    } else {
+#if defined(__HIP_DEVICE_COMPILE__)
+        const float y = __builtin_amdgcn_rcpf(sf);            // within 1 ulp
+        rcp = sf > 0.0f ? __fmaf_rn(__fmaf_rn(-sf, y, 1.0f), y, y) : 0.0f;
+#else
+        rcp = 0.0f;
+#endif
+    }
+    scale_bits = sh;
+}
+
+// int8 codes of 8 values: code = clamp(rint(x * rcp), -127, 127).  The clamp bounds are integers, so it may run
+// before the rounding, and adding 1.5 * 2^23 rounds to the nearest integer, ties to even, exactly as rint does --
+// and leaves the code's two's-complement byte as the low byte of the sum.
+__device__ __forceinline__ void int8_codes8(const float *x, float rcp, uint32_t &lo, uint32_t &hi)
+{
+    uint32_t u[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        float r = __fmul_rn(x[i], rcp);
+        r = fminf(fmaxf(r, -127.0f), 127.0f);
+        u[i] = __float_as_uint(__fadd_rn(r, 12582912.0f));
+    }
+    lo = s_perm(s_perm(u[3], u[2], 0x04000c0cu), s_perm(u[1], u[0], 0x0c0c0400u), 0x07060100u);
+    hi = s_perm(s_perm(u[7], u[6], 0x04000c0cu), s_perm(u[5], u[4], 0x0c0c0400u), 0x07060100u);
+}
+__device__ __forceinline__ void fp8_codes8(const float *x, uint32_t &lo, uint32_t &hi)
+{
+    lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
+    hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
+}
+
 // The 8 codes of chunk c of a row: the even lane of each lane pair takes its neighbour's
 // 8 bytes (chunks of one row sit in consecutive lanes, so both belong to the same row) and
 // stores 16 (fp8 bulk append 4.60 -> 5.02 TB/s against 8-byte stores from every lane);
@@ -111,28 +168,16 @@ __device__ __forceinline__ void store_page_chunk(uint8_t *__restrict__ pool, siz
                 for (unsigned off = rc >> 1; off > 0; off >>= 1)
                     amax = fmaxf(amax, __shfl_xor(amax, (int)off));
             }
-            float s32 = __fdiv_rn(amax, 127.0f);
-            uint16_t sh = __half_as_ushort(__float2half_rn(s32));
-            if ((sh & 0x7fffu) == 0x7c00u) sh = 0x7bffu;
-            float sf = f16_bits_to_f(sh);
-            float rcp = sf > 0.0f ? __fdiv_rn(1.0f, sf) : 0.0f;
-            // code = clamp(rint(x * rcp), -127, 127).  The clamp bounds are integers, so it may run before
-            // the rounding, and adding 1.5 * 2^23 rounds to the nearest integer, ties to even, exactly as
-            // rint does -- and leaves the code's two's-complement byte as the low byte of the sum.
-            uint32_t u[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                float r = __fmul_rn(x[i], rcp);
-                r = fminf(fmaxf(r, -127.0f), 127.0f);
-                u[i] = __float_as_uint(__fadd_rn(r, 12582912.0f));
-            }
-            const uint32_t lo = s_perm(s_perm(u[3], u[2], 0x04000c0cu), s_perm(u[1], u[0], 0x0c0c0400u), 0x07060100u);
-            const uint32_t hi = s_perm(s_perm(u[7], u[6], 0x04000c0cu), s_perm(u[5], u[4], 0x0c0c0400u), 0x07060100u);
+            uint16_t sh;
+            float rcp;
+            int8_row_scale<false>(amax, sh, rcp);
+            uint32_t lo, hi;
+            int8_codes8(x, rcp, lo, hi);
             store_codes(pool + poff, c, rc, lo, hi, ok);
             if (ok && c == 0) *(uint16_t *)(pool + soff) = sh;
         } else {
-            uint32_t lo = fp8_pair(x[0], x[1]) | (fp8_pair(x[2], x[3]) << 16);
-            uint32_t hi = fp8_pair(x[4], x[5]) | (fp8_pair(x[6], x[7]) << 16);
+            uint32_t lo, hi;
+            fp8_codes8(x, lo, hi);
             store_codes(pool + poff, c, rc, lo, hi, ok);
         }
     }

@@ -18,6 +18,7 @@ constexpr int kThreads = 256;
 // 5.94 / 5.80, inject 5.06 / 5.35 / 5.42 -- the quantising modes with four rounds of loads in
 // flight once per workgroup (1 024 chunks: int8 4.3 TB/s, fp8 5.0; 4.15 and 4.7 at 2 048).
 int g_copy_chunks = 256, g_flat_chunks = 512, g_quant_chunks = 1024;
+int g_quant_pairs = 1;                      // quantising append: 32 source bytes per thread (0: 16, the one-chunk kernel)
 static int tokens_per_group(unsigned chunks_per_token, int target_chunks)
 {
     const unsigned target = (unsigned)target_chunks;
@@ -159,6 +160,112 @@ __global__ __launch_bounds__(kThreads) void append_kernel(
     }
 }
 
+// The quantising append for rows of at least two chunks: one thread takes 32 source bytes (16 elements) and stores
+// their 16 codes with one 16-byte store -- half the index arithmetic, scale arithmetic and lane exchanges per byte
+// of the one-chunk form above, which is bound by instruction issue and not by memory.  Same grid and arguments;
+// row_div divides by the row's 32-byte items (head_dim / 16), tok_div by KVH times that.
+template <int QMODE>
+__global__ __launch_bounds__(kThreads) void append_quant_kernel(
+    Lay a, uint8_t *__restrict__ pool, const int32_t *__restrict__ tables, int table_stride,
+    const int32_t *__restrict__ d_pos, int pos_start, int ntokens, int layer0,
+    const uint8_t *__restrict__ src_k, const uint8_t *__restrict__ src_v, int src_dtype, int tpg, Div tok_div,
+    Div row_div, Div bs_div)
+{
+    static_assert(QMODE == 1 || QMODE == 2, "int8 or fp8");
+    const int tg = blockIdx.x, li = blockIdx.y, kv = blockIdx.z;
+    const int layer = layer0 + li;
+    const int t0 = tg * tpg;
+    const int ntok = min(tpg, ntokens - t0);
+    const unsigned rc2 = row_div.d;                      // 32-byte items per source row
+    const unsigned items = (unsigned)ntok * tok_div.d;
+    const uint8_t *sbase = (kv ? src_v : src_k) + ((size_t)li * ntokens + t0) * a.KVH * ((size_t)a.D * 2);
+    const unsigned rounds = (items + kThreads - 1) / kThreads;
+
+    constexpr int U = 2;                                 // four 16-byte loads in flight per thread
+    for (unsigned rnd0 = 0; rnd0 < rounds; rnd0 += U) {
+        uint4 va[U], vb[U];
+        size_t poff[U], soff[U];
+        bool ok[U], first[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const unsigned ci = (rnd0 + u) * kThreads + threadIdx.x;
+            va[u] = vb[u] = make_uint4(0, 0, 0, 0);
+            poff[u] = soff[u] = 0;
+            ok[u] = first[u] = false;
+            if (ci < items) {
+                const unsigned t = dv(ci, tok_div), r = ci - t * tok_div.d;
+                const unsigned h = dv(r, row_div), c2 = r - h * rc2;
+                const int ti = t0 + (int)t;
+                const int pos = d_pos ? d_pos[ti] : pos_start + ti;
+                const int32_t *tab = tables + (size_t)(d_pos ? ti : 0) * table_stride;
+                if (pos >= 0) {
+                    const unsigned lb = dv((unsigned)pos, bs_div);
+                    const int blk = tab[lb];
+                    if (blk >= 0 && blk < a.NB) {
+                        ok[u] = true;
+                        first[u] = c2 == 0;
+                        const int p = pos - lb * bs_div.d;
+                        poff[u] = row_off(a, layer, blk, kv, h, p) + (size_t)c2 * 16;
+                        if (QMODE == 1) soff[u] = scale_off(a, layer, blk, kv, h, p);
+                    }
+                }
+                const uint8_t *s = sbase + (size_t)ci * 32;
+                va[u] = ld_stream128(s);
+                vb[u] = ld_stream128(s + 16);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float x[16];
+            unpack8(va[u], src_dtype, x);
+            unpack8(vb[u], src_dtype, x + 8);
+            uint4 codes;
+            if (QMODE == 1) {
+                float amax = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 16; i++) amax = fmaxf(amax, fabsf(x[i]));
+                if (rc2 == 8) {                               // head_dim 128: a row is half a DPP row
+                    amax = fmaxf(amax, codec_dpp<0xB1>(amax));
+                    amax = fmaxf(amax, codec_dpp<0x4E>(amax));
+                    amax = fmaxf(amax, codec_dpp<0x141>(amax));
+                } else {
+                    for (unsigned off = rc2 >> 1; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, (int)off));
+                }
+                uint16_t sh;
+                float rcp;
+                int8_row_scale<false>(amax, sh, rcp);
+                int8_codes8(x, rcp, codes.x, codes.y);
+                int8_codes8(x + 8, rcp, codes.z, codes.w);
+                if (first[u]) *(uint16_t *)(pool + soff[u]) = sh;
+            } else {
+                fp8_codes8(x, codes.x, codes.y);
+                fp8_codes8(x + 8, codes.z, codes.w);
+            }
+            if (ok[u]) st_stream128(pool + poff[u], codes);
+        }
+    }
+}
+
+// Every input the int8 scale arithmetic can meet, through both of its forms (see int8_row_scale): thread i takes
+// the 16-bit pattern i as a bf16 and as an fp16 magnitude (scale bits must agree) and as an fp16 scale
+// (reciprocal bits must agree).  *mismatches counts the disagreements.
+__global__ void int8_scale_math_check_kernel(unsigned *__restrict__ mismatches)
+{
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= 65536u) return;
+    unsigned bad = 0;
+    for (int fmt = 0; fmt < 2; fmt++) {
+        const float x = fabsf(elem16_to_f((uint16_t)i, fmt == 0 ? DRK_BF16 : DRK_F16));
+        if (x != x) continue;                                 // a row maximum is never NaN (fmaxf drops it)
+        uint16_t s0, s1;
+        float r0, r1;
+        int8_row_scale<true>(x, s0, r0);
+        int8_row_scale<false>(x, s1, r1);
+        bad += (s0 != s1) || (__float_as_uint(r0) != __float_as_uint(r1));
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
 // ------------------------------------------------------------------------
 // copy-on-write: every layer of block src -> block dst
 // grid = (chunk groups, L, pairs)
@@ -226,9 +333,22 @@ static int launch_append(const drk_kv_layout *g, void *pool, const int32_t *tabl
             return fail(DRK_ERR_UNSUPPORTED, "append: quantising pools need head_dim in {8..512} power of two, got %d", a.D);
     }
     Div tok_div = mk_div((unsigned)a.KVH * rowc), row_div = mk_div(rowc), bs_div = mk_div((unsigned)a.bs);
-    const int tpg = tokens_per_group((unsigned)a.KVH * rowc, (a.dtype == DRK_INT8 || a.dtype == DRK_FP8_E4M3) ? g_quant_chunks : g_copy_chunks);
+    const bool quant = a.dtype == DRK_INT8 || a.dtype == DRK_FP8_E4M3;
+    const int tpg = tokens_per_group((unsigned)a.KVH * rowc, quant ? g_quant_chunks : g_copy_chunks);
     dim3 grid((ntokens + tpg - 1) / tpg, layer_count, 2);
     hipStream_t s = (hipStream_t)stream;
+    if (quant && rowc >= 2 && g_quant_pairs) {           // 32 source bytes per thread
+        const Div tok2 = mk_div((unsigned)a.KVH * (rowc / 2)), row2 = mk_div(rowc / 2);
+#define GO2(Q)                                                                                          \
+    hipLaunchKernelGGL(append_quant_kernel<Q>, grid, dim3(kThreads), 0, s, a, (uint8_t *)pool, tables,  \
+                       table_stride, d_pos, pos_start, ntokens, layer, (const uint8_t *)src_k,          \
+                       (const uint8_t *)src_v, src_dtype, tpg, tok2, row2, bs_div)
+        if (a.dtype == DRK_INT8) GO2(1);
+        else GO2(2);
+#undef GO2
+        DRK_LAUNCH_CHECK("append_quant_kernel");
+        return DRK_OK;
+    }
 #define GO(Q)                                                                                       \
     hipLaunchKernelGGL(append_kernel<Q>, grid, dim3(kThreads), 0, s, a, (uint8_t *)pool, tables,    \
                        table_stride, d_pos, pos_start, ntokens, layer, (const uint8_t *)src_k,      \
@@ -273,6 +393,16 @@ static int launch_flat(bool extract, const drk_kv_layout *g, void *pool, void *f
 using namespace drk;
 
 extern "C" {
+
+int drk_debug_check_int8_scale_math(unsigned *d_mismatches, void *stream)
+{
+    if (!d_mismatches) return fail(DRK_ERR_INVALID, "check_int8_scale_math: NULL counter");
+    hipLaunchKernelGGL(int8_scale_math_check_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream, d_mismatches);
+    DRK_LAUNCH_CHECK("int8_scale_math_check_kernel");
+    return DRK_OK;
+}
+
+void drk_debug_set_quant_append_pairs(int on) { g_quant_pairs = on ? 1 : 0; }
 
 void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chunks)
 {

@@ -48,6 +48,15 @@ void drk_debug_set_prefill_two_phase(int mode);
 /* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
  * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */
 void drk_debug_set_append_chunks(int copy_chunks, int flat_chunks, int quant_chunks);
+/* Tuning: the quantising append takes 32 source bytes per thread (1, the default) or 16 (0: the
+ * kernel it shares with the copying append; always used for head_dim 8). */
+void drk_debug_set_quant_append_pairs(int on);
+/* Self-check of the int8 scale arithmetic: the quantising kernels find a row's fp16 scale and its
+ * reciprocal with one multiply and one residual correction per division; this runs that form and
+ * the full IEEE divisions over every input that can occur (all bf16 and fp16 magnitudes, all fp16
+ * scales) and adds the number of disagreements to *d_mismatches (device memory, 4 bytes, zeroed
+ * by the caller).  Asynchronous on `stream`. */
+int drk_debug_check_int8_scale_math(unsigned *d_mismatches, void *stream);
 
 #ifdef __cplusplus
 }

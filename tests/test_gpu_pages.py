@@ -116,9 +116,17 @@ def test_append_token_and_branches_equal_batch(dev, dtype):
     assert np.array_equal(U.host(dpool2, np.uint8), opool)
 
 
+@pytest.fixture(params=["32B_per_thread", "16B_per_thread"])
+def quant_form(request):
+    """the quantising append has two kernels: 32 source bytes per thread (the default) and 16"""
+    cabi.lib().drk_debug_set_quant_append_pairs(1 if request.param == "32B_per_thread" else 0)
+    yield request.param
+    cabi.lib().drk_debug_set_quant_append_pairs(1)
+
+
 @pytest.mark.parametrize("dtype", [cabi.INT8, cabi.FP8_E4M3])
 @pytest.mark.parametrize("src_dtype", [cabi.F16, cabi.BF16])
-def test_quantising_append_bit_exact(dev, dtype, src_dtype):
+def test_quantising_append_bit_exact(dev, quant_form, dtype, src_dtype):
     """int8 codes + fp16 scales / fp8 codes equal the oracle's, with 1% outliers x20
     (BASELINE config 4) and a few crafted rows: zeros, ties, huge values."""
     L, KVH, QH, D, bs, NB = 2, 8, 32, 128, 16, 48
@@ -148,8 +156,61 @@ def test_quantising_append_bit_exact(dev, dtype, src_dtype):
     assert bad.size == 0, f"{bad.size} bytes differ, first at {bad[:8]}"
 
 
+@pytest.mark.parametrize("geom", [(2, 2, 4, 64, 32, 24), (1, 3, 6, 32, 16, 40), (2, 4, 24, 256, 256, 6), (1, 1, 1, 16, 16, 8),
+                                  (1, 2, 2, 512, 16, 12), (1, 5, 5, 128, 16, 20)])
+@pytest.mark.parametrize("dtype", [cabi.INT8, cabi.FP8_E4M3])
+def test_quantising_append_other_head_dims(dev, quant_form, geom, dtype):
+    """Rows of 1 to 32 lanes (head_dim 16 .. 512), odd head counts, a start inside a block: pool bytes
+    equal the oracle's for both kernels of the quantising append."""
+    bs = geom[4]
+    M = min(3 * bs + 5, (geom[5] - 1) * bs - 7)
+    g, og, table, opool, dpool, _ = _append_case(dev, geom, dtype, M=M, pos_start=7, seed=geom[3] + dtype, layer_count=geom[0])
+    assert np.array_equal(U.host(dpool, np.uint8), opool)
+
+
+def test_int8_scale_math_self_check(dev):
+    """The quantising kernels divide by multiply-and-correct; on the device that form and the IEEE
+    divisions give the same scale bits and the same reciprocal bits for every bf16 / fp16 magnitude."""
+    import torch
+    count = torch.zeros(1, dtype=torch.int32, device="cuda")
+    cabi.call("drk_debug_check_int8_scale_math", U.p(count), U.stream_ptr())
+    U.sync()
+    assert int(count.item()) == 0
+
+
 @pytest.mark.parametrize("src_dtype", [cabi.F16, cabi.BF16])
-def test_fp8_codes_exhaustive(dev, src_dtype):
+def test_int8_scales_exhaustive(dev, quant_form, src_dtype):
+    """Every non-NaN 16-bit magnitude as the largest element of a row: scale and codes of the int8
+    append equal the oracle's (which divides in IEEE fp32)."""
+    D = 128
+    top = 0x7C00 if src_dtype == cabi.F16 else 0x7F80                  # +inf
+    mags = np.arange(top + 1, dtype=np.uint16)
+    M = mags.size
+    rng = np.random.default_rng(8)
+    vals = U.from_bits(mags, src_dtype).astype(np.float64)
+    finite = np.where(np.isfinite(vals), vals, 60000.0 if src_dtype == cabi.F16 else 3e38)
+    rows = U.to_bits((finite[:, None] * rng.uniform(-1.0, 1.0, (M, D))).astype(np.float32), src_dtype)
+    rows[:, 5] = mags | np.where(rng.random(M) < 0.5, 0x8000, 0).astype(np.uint16)
+    assert np.all(np.abs(U.from_bits(rows, src_dtype)).max(axis=1) == vals)
+    L, KVH, QH, bs = 1, 1, 1, 16
+    NB = (M + bs - 1) // bs
+    g, og = U.both_layouts(L, KVH, QH, D, bs, NB, cabi.INT8)
+    table = np.arange(NB, dtype=np.int32)
+    src = np.ascontiguousarray(rows.reshape(M, 1, D))
+    opool = orc.new_pool(og)
+    orc.append_batch(og, opool, table, 0, 0, src, src, src_dtype)
+    dpool = U.dev_zeros(orc.pool_bytes(og))
+    d, dtab = U.dev_bytes(src), U.dev_i32(table)
+    cabi.call("drk_kv_append_batch", C.byref(g), U.p(dpool), U.p(dtab), 0, 1, 0, M, U.p(d), U.p(d), src_dtype,
+              U.stream_ptr())
+    U.sync()
+    got = U.host(dpool, np.uint8)
+    bad = np.nonzero(got != opool)[0]
+    assert bad.size == 0, f"{bad.size} bytes differ, first at {bad[:8]}"
+
+
+@pytest.mark.parametrize("src_dtype", [cabi.F16, cabi.BF16])
+def test_fp8_codes_exhaustive(dev, quant_form, src_dtype):
     """Every finite 16-bit input pattern through the fp8 append equals the oracle's
     E4M3FN round-half-even code (hardware conversion vs the C restatement)."""
     D = 128
