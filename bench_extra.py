@@ -267,7 +267,7 @@ def config3(args):
         "us_per_step": round(total_ms / K * 1e3, 1), "tokens_per_s": round(B * K / (total_ms * 1e-3), 1),
         "host_ns": {"fork_branch": round(fork_ns), "ensure_blocks_for": round(float(np.mean(ensure_ns))),
                     "evict_per_block": round(evict_ns / max(evicted, 1)), "blocks_evicted": int(evicted)},
-        "roofline": {"kernel": "prefill_mfma_kernel<bf16,shared> + decode_stream_kernel<bf16>", "bound": "hbm",
+        "roofline": {"kernel": "prefix_stream_kernel<bf16> + decode_stream_kernel<bf16>", "bound": "hbm",
                      "achieved": round(ach, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
                      "avg_launch_us": round(ker_ms * 1e3, 2), "bytes_per_launch": launch_unique,
@@ -752,7 +752,7 @@ def kernel_fractions(buf, seed=11):
     call_ms = a0.elapsed_time(a1) / 40
     distinct = (prefix + int(tails.sum())) * 2 * KVH * D * 2
     res["config3_shared_prefix"] = _entry(
-        "prefill_mfma_kernel<bf16,shared> + decode_stream_kernel<bf16>", "hbm", distinct, pair_ms,
+        "prefix_stream_kernel<bf16> + decode_stream_kernel<bf16>", "hbm", distinct, pair_ms,
         "config 3: 65536-token prefix shared by 16 branches + private tails U{0..4096} (sum %d), bf16; DISTINCT bytes (shared "
         "pages counted once) over the prefix pass and the tail kernel together" % int(tails.sum()),
         {"with_merge_us": round(call_ms * 1e3, 2), "with_merge_frac": round(distinct / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),

@@ -89,6 +89,7 @@ SIGNATURES = {
     "drk_debug_set_decode_kernel": (None, [_i32]),
     "drk_debug_set_stream_workgroups": (None, [_i32]),
     "drk_debug_set_shared_splits": (None, [_i32]),
+    "drk_debug_set_prefix_stream": (None, [_i32]),
     "drk_debug_time_decode_kernel": (None, [_i32]),
     "drk_debug_set_decode_lds_pad": (None, [_i32]),
     "drk_debug_set_append_chunks": (None, [_i32, _i32, _i32]),

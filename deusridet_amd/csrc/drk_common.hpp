@@ -71,6 +71,7 @@ constexpr int kStreamMaxUnits = 256;                          // 64-token tiles 
 constexpr int kStreamMaxSplitTokens = kStreamMaxUnits * 64;   // the longest explicit split: 16 384 tokens
 extern int g_stream_wgs;
 extern int g_shared_splits;
+extern int g_prefix_stream;
 bool stream_decode_supported(const Lay &a, int B);
 size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens, int start_tile = 0);
 int launch_decode_stream(const Lay &a, const void *q, const void *pool, const int32_t *tables, int table_stride,
@@ -88,7 +89,7 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
                          void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
                          void *stream, const void *gate = nullptr, size_t gate_stride = 0);
 // shared-prefix pass on the matrix cores (drk_prefill.hip)
-void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits);
+void shared_prefix_shape(const Lay &a, int B, int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,
                          const int32_t *d_seq_lens, int B, int shared, int layer, float scale, int io_dtype,
                          float *part_o, float *part_m, float *part_l, hipStream_t st, int chunk_tiles = 0,

@@ -612,7 +612,7 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
 static size_t shared_need(const Lay &a, int B, int max_seq_len, int shared, size_t *stream_part, bool exact)
 {
     int ct, ns;
-    shared_prefix_shape(shared, &ct, &ns);
+    shared_prefix_shape(a, B, shared, &ct, &ns);
     if (!exact && ns < g_shared_splits) ns = g_shared_splits;
     size_t sp = stream_workspace_need(a, B, max_seq_len, 0, exact ? shared / kTile : 0);
     sp = (sp + 255) & ~(size_t)255;
@@ -649,7 +649,7 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
         return fail(DRK_ERR_WORKSPACE, "decode: workspace of %zu bytes, need %zu", workspace_bytes, need);
     if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode: workspace must be 16-byte aligned");
     int ct, ns;
-    shared_prefix_shape(shared, &ct, &ns);
+    shared_prefix_shape(a, B, shared, &ct, &ns);
     float *pre_o = (float *)((uint8_t *)workspace + sp);
     float *pre_m = pre_o + (size_t)B * a.QH * ns * a.D;
     float *pre_l = pre_m + (size_t)B * a.QH * ns;
@@ -714,6 +714,7 @@ void drk_debug_force_portable_decode(int on) { g_force_portable = on ? 1 : 0; }
 void drk_debug_set_decode_kernel(int which) { g_decode_kernel = which; }
 void drk_debug_set_stream_workgroups(int n) { g_stream_wgs = n > 0 ? n : 0; }
 void drk_debug_set_shared_splits(int n) { g_shared_splits = n > 0 ? (n < 256 ? n : 256) : 64; }
+void drk_debug_set_prefix_stream(int on) { g_prefix_stream = on ? 1 : 0; }
 
 void drk_debug_time_decode_kernel(int on)
 {

@@ -906,15 +906,340 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     }
 }
 
+// Global loads the compiler does not count (see prefix_stream_kernel): issue, and wait until at most N of the
+// wave's loads are outstanding -- the values named become usable then, and only then.
+typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ pf_u32x4 pf_async_load128(const uint8_t *p)
+{
+    pf_u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=&v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ uint32_t pf_async_load16(const uint8_t *p)
+{
+    uint32_t v;
+    asm volatile("global_load_ushort %0, %1, off" : "=&v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void pf_async_wait(pf_u32x4 &a, pf_u32x4 &b)
+{
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void pf_async_wait16(uint32_t &a, uint32_t &b)
+{
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
+}
+__device__ __forceinline__ void pf_async_drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// ---- shared-prefix pass for few rows: producer and consumer waves ---------------------------------
+// With at most 64 rows (branches x query heads of one kv head) the pass is bound by HBM, and the kernel above
+// -- every wave stages one tile ahead in its own registers, next to its accumulators -- keeps only 64 KB per
+// CU in flight: each trip of its loop waits out a full memory latency (16 trips of 3.3 us for 1 024 tokens).
+// Here a workgroup has eight waves.  Waves 4-7 only move data: wave 4 + p owns the 16-token run p of every
+// tile and keeps four tiles' worth of it in registers (64 data registers), requesting tile t + 5 the moment
+// tile t + 1 has gone to LDS: 128 KB in flight per CU, loads issued four steps before their use.  (One wave
+// moving whole tiles was tried first: 64 memory instructions from one wave per step took 3.4 us.)
+// Waves 0-3 multiply: wave = (row half, key half) of the 64 x 64 tile, each with its own running maximum and
+// sum; the two key halves of a row are folded through LDS at the end.  One barrier per tile: the tile
+// written in a step is read in the next.  grid = (KVH * ceil(B / TPW), 1, splits), TPW = 64 / (QH/KVH);
+// block = 512, one workgroup per CU; leaves (o, m, l) per (branch, q head, split) like the kernel above.
+template <int DT, int KV = DT, int IO = DT>
+__global__ __launch_bounds__(512, 1) void prefix_stream_kernel(PrefillArgs A)
+{
+    constexpr int D = 128;
+    constexpr bool Q8 = KV == DRK_INT8 || KV == DRK_FP8_E4M3;
+    constexpr int RB = D * (Q8 ? 1 : 2);
+    constexpr int kPitchK = D * 2 + 16, kPitchV = D * 2 + 32;
+    constexpr int NKS = D / 16, NDT = D / 32;
+    __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPitchK];
+    __shared__ __align__(16) uint8_t v_lds2[2][kPfBN * kPitchV];
+    __shared__ int runs_lds[2][4];                           // the 16-token run of the tile in this slot has a page
+
+    const int kvh = (int)blockIdx.x % A.KVH;
+    const int qt = (int)blockIdx.x / A.KVH;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int t_begin = (int)blockIdx.z * A.chunk_tiles;
+    const int lim_wg = min(A.shared, (t_begin + A.chunk_tiles) * kPfBN);
+    const int nt = max(0, (lim_wg + kPfBN - 1) / kPfBN - t_begin);     // tiles of this workgroup
+
+    if (w >= 4) {
+        // ---------------- producer: the 16-token run p of every tile, kDepth tiles ahead ----------------
+        const int p = w - 4;
+        constexpr int kDepth = 4;
+        constexpr int NLR = PfGroup<RB, 16>::NL;             // 16-byte chunks per lane, operand and run: 4 (16-bit) or 2
+        // The loads are written as inline assembly and waited for by count: the compiler's own bookkeeping gives up
+        // at the loop's head (it cannot tell which of the rotating buffers a pending load belongs to) and drains
+        // every load there, the three tiles meant to stay in flight included.  Loads return in order, so "all but
+        // the last 3 fetches" is exactly "the buffer about to be stored".
+        pf_u32x4 kx[kDepth][NLR], vx[kDepth][NLR];           // tile t waits in buffer t % kDepth
+        uint32_t ksx[kDepth][NLR], vsx[kDepth][NLR];         // int8: the fp16 scales of the rows of this lane's chunks
+        constexpr int kLoadsPerFetch = 2 * NLR + (KV == DRK_INT8 ? 2 * NLR : 0);
+        int limq[kDepth];                                    // rows of the buffered run that are real (0: no page)
+        const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+        // Read through the scalar cache (the table is not written while the kernel runs).
+        typedef const int32_t __attribute__((address_space(4))) *const_table_t;
+        const const_table_t table_k = (const_table_t)(uintptr_t)A.table;
+        // the run's page in local tile i: the table entry, or -1 (past the end)
+        auto page_of = [&](int i) -> int {
+            const int tg = (t_begin + i) * kPfBN + p * 16;
+            if (i >= nt || tg >= lim_wg) return -1;
+            return table_k[A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs)];
+        };
+        auto fetch = [&](int d, int i, int blk) {            // local tile i into buffer d
+            const int tg = (t_begin + i) * kPfBN + p * 16;
+            const bool ok = blk >= 0 && blk < A.NB;
+            const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
+            const int tin = ok ? tg - lb * A.bs : 0;
+            const size_t boff = (size_t)(ok ? blk : 0) * A.block_stride;      // no page: block 0 is read and zeros are stored
+            const uint8_t *src = kbase + boff + (size_t)tin * RB + (size_t)lane * 16;
+#pragma unroll
+            for (int j = 0; j < NLR; j++) {
+                kx[d][j] = pf_async_load128(src + 1024 * j);
+                vx[d][j] = pf_async_load128(src + A.kv_plane + 1024 * j);
+                if constexpr (KV == DRK_INT8) {
+                    const int row = (lane * 16 + 1024 * j) / RB;
+                    const uint8_t *sp = A.pool_layer + boff + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + tin + row) * 2;
+                    ksx[d][j] = pf_async_load16(sp);
+                    vsx[d][j] = pf_async_load16(sp + A.scale_plane);
+                } else {
+                    ksx[d][j] = vsx[d][j] = 0;
+                }
+            }
+            limq[d] = ok ? lim_wg - tg : 0;
+        };
+        auto store = [&](int d, int slot) {
+            // everything but the last three fetches has arrived: buffer d
+#pragma unroll
+            for (int j = 0; j < NLR; j++) {
+                pf_async_wait<3 * kLoadsPerFetch>(kx[d][j], vx[d][j]);
+                if constexpr (KV == DRK_INT8) pf_async_wait16<3 * kLoadsPerFetch>(ksx[d][j], vsx[d][j]);
+            }
+            PfGroup<RB, 16> kq, vq;
+            uint16_t ksc[NLR], vsc[NLR];
+#pragma unroll
+            for (int j = 0; j < NLR; j++) {
+                kq.r[j] = make_uint4(kx[d][j].x, kx[d][j].y, kx[d][j].z, kx[d][j].w);
+                vq.r[j] = make_uint4(vx[d][j].x, vx[d][j].y, vx[d][j].z, vx[d][j].w);
+                ksc[j] = (uint16_t)ksx[d][j];
+                vsc[j] = (uint16_t)vsx[d][j];
+            }
+            if constexpr (Q8) {
+                pf_store_group_q8<kPitchK, KV, RB, 16>(&k_lds2[slot][0], kq, p, lane, ksc, limq[d]);
+                pf_store_group_q8<kPitchV, KV, RB, 16>(&v_lds2[slot][0], vq, p, lane, vsc, limq[d]);
+            } else {
+                pf_store_group_sel<kPitchK, RB, 16>(&k_lds2[slot][0], kq, p, lane, limq[d]);
+                pf_store_group_sel<kPitchV, RB, 16>(&v_lds2[slot][0], vq, p, lane, limq[d]);
+            }
+            if (lane == 0) runs_lds[slot][p] = limq[d] > 0 ? 1 : 0;
+        };
+        int first_pages[kDepth + 2];                         // all six table reads go out before the first is waited for
+#pragma unroll
+        for (int d = 0; d < kDepth + 2; d++) first_pages[d] = page_of(d);
+#pragma unroll
+        for (int d = 0; d < kDepth; d++) fetch(d, d, first_pages[d]);
+        store(0, 0);
+        fetch(0, kDepth, first_pages[kDepth]);
+        int blk_pf = first_pages[kDepth + 1];                // looked up one step before its loads are issued
+        __syncthreads();
+#pragma unroll 1
+        for (int i0 = 0; i0 < nt; i0 += kDepth) {
+#pragma unroll
+            for (int d = 0; d < kDepth; d++) {
+                const int i = i0 + d;
+                if (i < nt) {
+                    constexpr int kNextMask = kDepth - 1;
+                    const int nx = i + 1;                    // the tile the next step reads: buffer nx % kDepth = (d + 1) % kDepth
+                    store((d + 1) & kNextMask, nx & 1);
+                    fetch((d + 1) & kNextMask, nx + kDepth, blk_pf);
+                    blk_pf = page_of(nx + kDepth + 1);
+                    __syncthreads();
+                }
+            }
+        }
+        __syncthreads();                                     // the consumers' fold
+        pf_async_drain();
+        return;
+    }
+
+    // ---------------- consumer: rows 32 rh .. +31, keys 32 kh .. +31 of every tile ----------------
+    const int n = lane & 31, g = lane >> 5;
+    const int rh = w & 1, kh = w >> 1;
+    const int G = A.QH / A.KVH, TPW = A.tpw;
+    const int r = rh * 32 + n, rt = r / G;
+    const int tq = qt * TPW + rt;
+    const int head = kvh * G + (r - rt * G);
+    const bool row_live = rt < TPW && tq < A.M;
+    const int len = row_live ? (A.seq_lens ? A.seq_lens[tq] : A.pos_start + tq + 1) : 0;
+    const int vis = row_live ? min(len, A.shared) : 0x7fffffff;      // an idle row multiplies zeros and masks nothing
+
+    uint4 qf[NKS];
+    {
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+#if defined(__HIP_DEVICE_COMPILE__)
+            if constexpr (IO == DRK_BF16 && DT == DRK_F16) {      // 8-bit pages multiply in fp16
+                v.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.x), bf16_hi(v.x)));
+                v.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.y), bf16_hi(v.y)));
+                v.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.z), bf16_hi(v.z)));
+                v.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.w), bf16_hi(v.w)));
+            }
+#endif
+            qf[ks] = v;
+        }
+    }
+    pf_f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    __syncthreads();
+#pragma unroll 1
+    for (int i = 0; i < nt; i++) {
+        const int slot = i & 1;
+        const int tile_t = (t_begin + i) * kPfBN + kh * 32;  // first token of this wave's key half
+        // Every operand of the step is requested first -- one wave per SIMD multiplies, so nothing else would
+        // hide the LDS latency: 8 reads of K and 16 of V, then the products.  S^T = K Q^T in two chains of four
+        // (even and odd k-steps); register i4 of a lane is token tile_t + 8 (i4 / 4) + 4 g + i4 % 4.
+        uint4 ka4[NKS];
+        uint2 vlo[2][NDT], vhi[2][NDT];
+        {
+            const uint8_t *ka = &k_lds2[slot][0] + (kh * 32 + n) * kPitchK + g * 16;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ks++) ka4[ks] = *(const uint4 *)(ka + ks * 32);
+            const int j16 = lane & 15;
+            const int dsub = 16 * ((lane >> 4) & 1) + 4 * (j16 & 3);
+            const uint8_t *vb = &v_lds2[slot][0] + (kh * 32 + 4 * g + (j16 >> 2)) * kPitchV + dsub * 2;
+#pragma unroll
+            for (int mh = 0; mh < 2; mh++)
+#pragma unroll
+                for (int dt = 0; dt < NDT; dt++) {
+                    vlo[mh][dt] = lds_read_tr16(vb + 16 * mh * kPitchV + dt * 64);
+                    vhi[mh][dt] = lds_read_tr16(vb + (16 * mh + 8) * kPitchV + dt * 64);
+                }
+        }
+        pf_f32x16 s;
+        {
+            const pf_f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            pf_f32x16 s1;
+            s = mfma32<DT>(ka4[0], qf[0], zero);
+            s1 = mfma32<DT>(ka4[1], qf[1], zero);
+#pragma unroll
+            for (int ks = 2; ks < NKS; ks += 2) {
+                s = mfma32<DT>(ka4[ks], qf[ks], s);
+                s1 = mfma32<DT>(ka4[ks + 1], qf[ks + 1], s1);
+            }
+#pragma unroll
+            for (int i4 = 0; i4 < 16; i4++) s[i4] += s1[i4];
+        }
+        const int runs = runs_lds[slot][2 * kh] | (runs_lds[slot][2 * kh + 1] << 1);   // the two runs of this key half
+        if (runs != 3 || __any(tile_t + 32 > vis)) {
+#pragma unroll
+            for (int i4 = 0; i4 < 16; i4++) {
+                const int tl = 8 * (i4 >> 2) + 4 * g + (i4 & 3);
+                const bool ok = (tile_t + tl) < vis && ((runs >> (tl >> 4)) & 1) != 0;
+                s[i4] = ok ? s[i4] : -INFINITY;
+            }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i4 = 0; i4 < 16; i4++) tmax = fmaxf(tmax, s[i4]);
+        tmax = pf_max_halves(tmax);
+        const float m_new = fmaxf(m_run, tmax * A.scale_log2e);
+        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        float pr[16];
+#pragma unroll
+        for (int i4 = 0; i4 < 16; i4++) pr[i4] = __builtin_amdgcn_exp2f(fmaf(s[i4], A.scale_log2e, -m_use));
+        uint4 pb[2];                                         // [16-token half]: the B operand of PV
+        pb[0] = make_uint4(pack2<DT>(pr[0], pr[1]), pack2<DT>(pr[2], pr[3]), pack2<DT>(pr[4], pr[5]), pack2<DT>(pr[6], pr[7]));
+        pb[1] = make_uint4(pack2<DT>(pr[8], pr[9]), pack2<DT>(pr[10], pr[11]), pack2<DT>(pr[12], pr[13]), pack2<DT>(pr[14], pr[15]));
+        float psum = pf_sum2<DT>(pb[0], 0.0f);               // the row sum is taken over the rounded weights
+        psum = pf_sum2<DT>(pb[1], psum);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (!__all(alpha == 1.0f)) {
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int i4 = 0; i4 < 16; i4++) o[dt][i4] *= alpha;
+        }
+        // O^T += V^T P^T over this wave's 32 tokens
+#pragma unroll
+        for (int mh = 0; mh < 2; mh++)
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+                o[dt] = mfma32<DT>(make_uint4(vlo[mh][dt].x, vlo[mh][dt].y, vhi[mh][dt].x, vhi[mh][dt].y), pb[mh], o[dt]);
+        __syncthreads();
+    }
+
+    // fold the two key halves of every row: the waves of the second half leave theirs in LDS (the tiles are done)
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    float *xo = (float *)&k_lds2[0][0];                      // [dt * 16 + i4][rh][lane]: 32 KB
+    float *xm = (float *)&v_lds2[0][0];                      // [rh][lane], then l
+    if (kh == 1) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int i4 = 0; i4 < 16; i4++) xo[((dt * 16 + i4) * 2 + rh) * 64 + lane] = o[dt][i4];
+        xm[rh * 64 + lane] = m_run;
+        xm[128 + rh * 64 + lane] = l_tot;
+    }
+    __syncthreads();
+    if (kh == 0 && row_live) {
+        const float m1 = xm[rh * 64 + lane], l1 = xm[128 + rh * 64 + lane];
+        const float m = fmaxf(m_run, m1);
+        const float m_use = (m == -INFINITY) ? 0.0f : m;
+        const float a0 = __builtin_amdgcn_exp2f(m_run - m_use), a1 = __builtin_amdgcn_exp2f(m1 - m_use);
+        const size_t pi = ((size_t)tq * A.QH + head) * A.nsplits + blockIdx.z;
+        float *orow = A.part_o + pi * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; b4++) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    v[e] = o[dt][4 * b4 + e] * a0 + xo[((dt * 16 + 4 * b4 + e) * 2 + rh) * 64 + lane] * a1;
+                *(float4 *)(orow + dt * 32 + 8 * b4 + 4 * g) = make_float4(v[0], v[1], v[2], v[3]);
+            }
+        if (g == 0) {
+            A.part_m[pi] = m;
+            A.part_l[pi] = l_tot * a0 + l1 * a1;
+        }
+    }
+}
+
 // ---- shared-prefix ("cascade") decode: host side of the prefix pass -------------------
 // One launch covers tokens [0, shared) for all B branches; the private tails go
 // through the stream kernel with start_tile = shared / 64.
 int g_shared_splits = 64;              // context splits of the prefix pass: 8 kv heads x 64 = two workgroups per CU
+int g_prefix_stream = 1;               // few rows: the producer / consumer kernel (0: the kernel every wave stages in)
+int g_prefix_stream_wgs = 256;         // ... with this many workgroups in all: one per CU
 
-void shared_prefix_shape(int shared, int *chunk_tiles, int *nsplits)
+// the producer / consumer pass takes head_dim 128 and at most 64 rows per kv head (branches x query heads)
+static bool prefix_stream_applies(const Lay &a, int B)
+{
+    const int G = a.QH / a.KVH;
+    return g_prefix_stream && a.D == 128 && G >= 1 && G <= 64 && B * G <= 64;
+}
+
+void shared_prefix_shape(const Lay &a, int B, int shared, int *chunk_tiles, int *nsplits)
 {
     const int tiles = shared / kPfBN;
-    int ns = tiles < g_shared_splits ? tiles : g_shared_splits;
+    int target = g_shared_splits;
+    if (prefix_stream_applies(a, B)) {
+        target = g_prefix_stream_wgs / a.KVH;
+        if (target < 1) target = 1;
+        if (target > g_shared_splits) target = g_shared_splits;      // workspaces are sized for at most that many pieces
+    }
+    int ns = tiles < target ? tiles : target;
     if (ns < 1) ns = 1;
     *chunk_tiles = (tiles + ns - 1) / ns;
     if (*chunk_tiles < 1) *chunk_tiles = 1;
@@ -938,9 +1263,23 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     A.scale_log2e = scale * kLog2eP;
     A.seq_lens = d_seq_lens; A.shared = shared;
     if (nsplits > 0) { A.chunk_tiles = chunk_tiles; A.nsplits = nsplits; }      // the caller's split (shared need not be whole tiles)
-    else shared_prefix_shape(shared, &A.chunk_tiles, &A.nsplits);
+    else shared_prefix_shape(a, B, shared, &A.chunk_tiles, &A.nsplits);
     A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
     A.gate = nullptr; A.gate_stride = 0;
+    if (nsplits <= 0 && prefix_stream_applies(a, B)) {
+        A.tpw = 64 / (a.QH / a.KVH);
+        dim3 grid2(((B + A.tpw - 1) / A.tpw) * a.KVH, 1, A.nsplits);
+#define DRK_PS(DT, KV, IO) hipLaunchKernelGGL((prefix_stream_kernel<DT, KV, IO>), grid2, dim3(512), 0, st, A)
+        if (a.dtype == DRK_BF16) DRK_PS(DRK_BF16, DRK_BF16, DRK_BF16);
+        else if (a.dtype == DRK_F16) DRK_PS(DRK_F16, DRK_F16, DRK_F16);
+        else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16) DRK_PS(DRK_F16, DRK_INT8, DRK_BF16);
+        else if (a.dtype == DRK_INT8) DRK_PS(DRK_F16, DRK_INT8, DRK_F16);
+        else if (io_dtype == DRK_BF16) DRK_PS(DRK_F16, DRK_FP8_E4M3, DRK_BF16);
+        else DRK_PS(DRK_F16, DRK_FP8_E4M3, DRK_F16);
+#undef DRK_PS
+        DRK_LAUNCH_CHECK("prefix_stream_kernel");
+        return DRK_OK;
+    }
     dim3 grid(((B + A.tpw - 1) / A.tpw) * a.KVH, 1, A.nsplits);
 #define DRK_PF_SHARED(DT, KV, IO)                                                                                        \
     do {                                                                                                                \

@@ -27,6 +27,9 @@ void drk_debug_set_stream_workgroups(int n);
 /* Diagnostic: context splits of the shared-prefix pass (default 64, at most 256; 0 restores the
  * default).  Changes drk_decode_shared_workspace_bytes. */
 void drk_debug_set_shared_splits(int n);
+/* Tuning: the shared-prefix pass for at most 64 rows per kv head and head_dim 128 runs on the
+ * producer / consumer kernel (1, the default) or on the kernel every wave stages in (0). */
+void drk_debug_set_prefix_stream(int on);
 /* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
  * session; switching it on starts a new session) records a HIP event on its
  * stream right before and right after the split-K partial kernel; the merge

@@ -344,11 +344,21 @@ def test_workspace_too_small_is_refused(dev):
     assert rc == cabi.ERR_WORKSPACE
 
 
+@pytest.fixture(params=["producer_consumer", "every_wave_stages"])
+def prefix_kernel(request):
+    """the shared-prefix pass has two kernels for up to 64 rows per kv head of head_dim 128"""
+    cabi.lib().drk_debug_set_prefix_stream(1 if request.param == "producer_consumer" else 0)
+    yield request.param
+    cabi.lib().drk_debug_set_prefix_stream(1)
+
+
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
 @pytest.mark.parametrize("shared,extra,heads", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17], (8, 32, 128)), (960 + 16, [5, 300], (8, 32, 128)),
                                                 (64, [0], (8, 32, 128)), (4096, list(range(0, 400, 10)), (8, 32, 128)),
-                                                (1024, [3, 200, 64, 700, 1], (2, 16, 128)), (512, [9, 100, 33], (4, 24, 256))])
-def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
+                                                (1024, [3, 200, 64, 700, 1], (2, 16, 128)), (512, [9, 100, 33], (4, 24, 256)),
+                                                (8192 + 64, [(37 * i) % 900 for i in range(16)], (8, 32, 128)),
+                                                (192, [0, 5, 70], (1, 16, 128))])
+def test_shared_prefix_decode(dev, prefix_kernel, dtype, shared, extra, heads):
     """Branches whose leading pages are the same physical blocks (BASELINE config 3
     in small): the shared pass + private tails must agree with the fp64 oracle run
     per branch, and with the plain per-branch call.  Also with 8 and 6 query heads per kv head,
@@ -382,6 +392,9 @@ def test_shared_prefix_decode(dev, dtype, shared, extra, heads):
             kk = U.normal_bits(rng, (n, KVH, D), io, 0.7)
             vv = U.normal_bits(rng, (n, KVH, D), io, 0.7)
             orc.append_batch(og, opool, tables[b], 0, n_shared_blk * bs, kk, vv, io)
+    if shared >= 1024:                                   # a page of the prefix is missing (evicted) in every branch
+        tables[:, 2] = -1
+        tables[:, n_shared_blk - 5] = -1
     q = U.normal_bits(rng, (B, QH, D), io, 0.7)
     scale = 1 / np.sqrt(D)
     dq, dpool, dtab, dl = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(tables), U.dev_i32(lens)
