@@ -190,6 +190,31 @@ def test_config5_full_chunk_prefill_rows(dev):
     U.sync()
     ok, ma, _ = U.rel_abs_ok(out[rows].float().cpu().numpy(), od.float().cpu().numpy())
     assert ok, ma
+    # fp32 causal attention in torch over the stored K and V (gathered through the C ABI): the sampled rows
+    # of the chunk, for both chunk kernels
+    flat = torch.empty(2 * total * KVH * D, dtype=torch.bfloat16, device="cuda")
+    cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(pool), U.p(table), 0, total, 1, sp)
+    U.sync()
+    kv = flat.view(2, total, KVH, D).float()
+    want = torch.empty(len(rows), QH, D, dtype=torch.float32, device="cuda")
+    for i, t in enumerate(rows):
+        n = pos_start + t + 1
+        s = torch.einsum("hgd,thd->hgt", q[t].float().view(KVH, QH // KVH, D), kv[0, :n]) * scale
+        want[i] = torch.einsum("hgt,thd->hgd", torch.softmax(s, dim=-1), kv[1, :n]).reshape(QH, D)
+    want = want.cpu().numpy()
+    for mode in (1, 0, 2):                                   # the library's choice (two-phase kernel here), four-wave kernel, forced
+        lib.drk_debug_set_prefill_two_phase(mode)
+        try:
+            out2 = torch.zeros_like(q)
+            cabi.call("drk_paged_prefill_attention", C.byref(g), U.p(q), U.p(pool), U.p(table), U.p(out2), 0, pos_start, M,
+                      float(scale), cabi.BF16, None, 0, sp)
+            U.sync()
+        finally:
+            lib.drk_debug_set_prefill_two_phase(1)
+        ok, ma, _ = U.rel_abs_ok(out2[rows].float().cpu().numpy(), want)
+        assert ok, (mode, ma)
+    ok, ma, _ = U.rel_abs_ok(od.float().cpu().numpy(), want)
+    assert ok, ma
 
 
 @pytest.mark.parametrize("dtype", [cabi.BF16, cabi.INT8])
@@ -345,6 +370,24 @@ def test_config3_full_size_properties(dev):
     once, per_branch = attend(True), attend(False)
     ok, ma, _ = U.rel_abs_ok(once, per_branch)
     assert ok, ma
+    # torch fp32 attention over what the pool holds (prefix + private tail, gathered through the C ABI) for
+    # three branches: no tail, the longest tail, the last one -- against both prefix kernels and the per-branch call
+    lib.drk_debug_set_prefix_stream(0)
+    try:
+        once_staged = attend(True)
+    finally:
+        lib.drk_debug_set_prefix_stream(1)
+    for i in (0, 1, B - 1):
+        n = int(lens[i])
+        flat = torch.empty(2 * n * KVH * D, dtype=torch.bfloat16, device="cuda")
+        cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, pool_ptr, U.p(dt[i]), 0, n, 1, st)
+        U.sync()
+        kv = flat.view(2, n, KVH, D).float()
+        s = torch.einsum("hgd,thd->hgt", q[i].float().view(KVH, QH // KVH, D), kv[0]) * scale
+        want = torch.einsum("hgt,thd->hgd", torch.softmax(s, dim=-1), kv[1]).reshape(QH, D).cpu().numpy()
+        for name, got in (("prefix once", once), ("prefix once, every wave stages", once_staged), ("per branch", per_branch)):
+            ok, ma, _ = U.rel_abs_ok(got[i], want)
+            assert ok, (name, i, ma)
     # make room for 500 more blocks: private pages go (oldest first), the prefix stays
     private_blocks = int(sum((int(n) + bs - 1) // bs for n in priv))
     assert private_blocks > 600
@@ -367,3 +410,115 @@ def test_config3_full_size_properties(dev):
               scale, cabi.BF16, U.p(ws), wsb, st)
     U.sync()
     assert torch.equal(out_a, out_b)
+
+
+def test_config3_sustained_eviction(dev):
+    """BASELINE config 3 run for 520 decode steps on two layers: a 65 536-token prefix shared by 16 copy-on-write
+    branches with private tails of up to 4 096 tokens, every step appends one token per branch and layer and
+    attends with the prefix streamed once; at steps 256 and 512 the pool is brought to 25 % free blocks.  After
+    each eviction: the free count, the references on the prefix pages (parent + 16 forks), the prefix rows of
+    every table and the bytes of the prefix are what they were; at the end two branches are checked against
+    torch fp32 attention over the pages their tables still name."""
+    torch = _torch()
+    from deusridet_amd import host
+    L, KVH, QH, D, bs, B, P = 2, 8, 32, 128, 16, 16, 65536
+    steps, evict_at = 520, (256, 512)
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    rng = np.random.default_rng(33)
+    priv = rng.integers(0, 4097, size=B)
+    priv[0], priv[1] = 0, 4096
+    cm = host.CacheManager()
+    want_blocks = int((P // bs + int(priv.sum()) // bs + 4 * B + steps * B // bs) / 0.8)     # ~80 % full when everything is resident
+    assert cm.init(want_blocks * L * 2 * KVH * bs * D * 2, bs, None, 1 + B)
+    NB, stride = cm.pool_max_blocks(), cm.table_stride()
+    st = U.stream_ptr()
+    lib = cabi.lib()
+    pool_ptr = C.c_void_p(cm.pool_ptr())
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    gen = torch.Generator(device="cuda").manual_seed(34)
+
+    def bulk(branch, p0, m):
+        assert cm.ensure_blocks_for_range(branch, p0, m)
+        cm.sync_block_table(st)
+        k = (torch.randn(L, m, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        v = (torch.randn(L, m, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        cabi.call("drk_kv_append_batch", C.byref(g), pool_ptr, C.c_void_p(cm.d_block_table(branch)), 0, L, p0, m, U.p(k), U.p(v),
+                  cabi.BF16, st)
+        U.sync()
+        cm.set_seq_len(branch, p0 + m)
+
+    for p0 in range(0, P, 8192):
+        bulk(0, p0, 8192)
+    kids = [cm.fork_branch(0, P) for _ in range(B)]
+    assert min(kids) > 0 and kids == list(range(kids[0], kids[0] + B))
+    for b, n in zip(kids, priv):
+        for p0 in range(0, int(n), 2048):
+            bulk(b, P + p0, min(2048, int(n) - p0))
+    prefix_blocks = cm.h_block_table(0)[:P // bs].copy()
+
+    def prefix_bytes():
+        flat = torch.empty(L * 2 * P * KVH * D, dtype=torch.bfloat16, device="cuda")
+        cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, pool_ptr, C.c_void_p(cm.d_block_table(0)), 0, P, L, st)
+        U.sync()
+        return flat
+
+    prefix0 = prefix_bytes()
+    scale = float(1 / np.sqrt(D))
+    q = (torch.randn(L, B, QH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+    nk = (torch.randn(L, B, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+    nv = (torch.randn(L, B, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+    out = torch.zeros(L, B, QH, D, device="cuda", dtype=torch.bfloat16)
+    lens = np.array([cm.seq_len(b) for b in kids], dtype=np.int32)
+    max_ctx = int(lens.max()) + steps + 1
+    wsb = lib.drk_decode_shared_workspace_bytes(C.byref(g), B, max_ctx, P)
+    ws = U.dev_zeros(wsb)
+    dpos = torch.zeros(B, dtype=torch.int32, device="cuda")
+    dlen = torch.zeros(B, dtype=torch.int32, device="cuda")
+    dtabs = C.c_void_p(cm.d_block_table(kids[0]))
+    qrow, krow = B * QH * D * 2, B * KVH * D * 2
+    evictions = 0
+    for s in range(1, steps + 1):
+        for i, b in enumerate(kids):
+            assert cm.ensure_blocks_for(b, int(lens[i]))
+        if s in evict_at:
+            before = cm.free_blocks()
+            assert cm.ensure_free_blocks(NB // 4)
+            assert cm.free_blocks() >= NB // 4 and cm.free_blocks() > before      # the pool was fuller than that: pages went
+            evictions += 1
+            assert all(cm.pool_refcount(int(x)) == 1 + B for x in prefix_blocks[[0, 1, 1000, 2047, 4095]])
+            for b in kids:
+                assert np.array_equal(cm.h_block_table(b)[:P // bs], prefix_blocks)
+                assert cm.h_block_table(b)[int(lens[kids.index(b)]) // bs] >= 0    # the page this step writes stayed
+            assert cm.common_prefix_tokens(kids) == P
+        cm.sync_block_table(st)
+        if s in evict_at:
+            assert torch.equal(prefix_bytes(), prefix0)
+        dpos.copy_(torch.from_numpy(lens))
+        dlen.copy_(torch.from_numpy(lens + 1))
+        for l in range(L):
+            cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, U.p(dpos), B, l, 1,
+                      C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, st)
+            cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr, dtabs, stride,
+                      U.p(dlen), B, max_ctx, P, C.c_void_p(out.data_ptr() + l * qrow), l, scale, cabi.BF16, U.p(ws), wsb, st)
+        U.sync()                                                  # the device arrays are rewritten by the next step
+        lens += 1
+        for i, b in enumerate(kids):
+            cm.set_seq_len(b, int(lens[i]))
+    assert evictions == 2
+    holes = sum(int((cm.h_block_table(b)[:(int(lens[i]) + bs - 1) // bs] < 0).sum()) for i, b in enumerate(kids))
+    assert holes > 0                                              # private pages did go
+    # the last step's output of layer 1 for two branches, against fp32 attention over the pages still present
+    l = L - 1
+    for i in (1, B - 1):
+        n = int(lens[i])
+        table = cm.h_block_table(kids[i])
+        present = torch.from_numpy(np.repeat(table[:(n + bs - 1) // bs] >= 0, bs)[:n]).cuda()
+        flat = torch.empty(L * 2 * n * KVH * D, dtype=torch.bfloat16, device="cuda")
+        cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, pool_ptr, C.c_void_p(cm.d_block_table(kids[i])), 0, n, L, st)
+        U.sync()
+        kv = flat.view(L, 2, n, KVH, D)[l].float()
+        sc = torch.einsum("hgd,thd->hgt", q[l, i].float().view(KVH, QH // KVH, D), kv[0]) * scale
+        sc = sc.masked_fill(~present, float("-inf"))
+        want = torch.einsum("hgt,thd->hgd", torch.softmax(sc, dim=-1), kv[1]).reshape(QH, D).cpu().numpy()
+        ok, ma, _ = U.rel_abs_ok(out[l, i].float().cpu().numpy(), want)
+        assert ok, (i, ma)
