@@ -93,6 +93,7 @@ bool KvStream::begin_prefill(int M, hipStream_t stream)
         return false;
     }
     cm_->sync_block_table(stream);                                        // stream.cpp:156
+    first_layer_of_frame_ = -1;
     return true;
 }
 
@@ -107,10 +108,28 @@ void KvStream::prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipSt
     paged_prefill_attention_gated(ws_prefill_, io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), io.qg + hd, 2 * hd, io.attn_out,
                                   fa_layer_idx, current_pos_, M, pool.max_blocks(), pool.block_size(),
                                   1.0f / std::sqrt((float)hd), stream);
+    // what the frame's rows looked at, block by block, into the stream's own row of the scorer's new scores
+    // ("after each Prefill frame, record cumulative attention weight received by each KV block",
+    // docs/en/architecture/02-memoria.md:40-44): a pass over Q and K behind the layer's attention
+    if (scorer_ && scorer_->d_new_scores()) {
+        const bool first = first_layer_of_frame_ < 0;
+        if (first) first_layer_of_frame_ = fa_layer_idx;
+        paged_prefill_attention_mass(io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), fa_layer_idx, current_pos_, M,
+                                     pool.max_blocks(), pool.block_size(), 1.0f / std::sqrt((float)hd),
+                                     scorer_->d_new_scores(), cm_->table_stride(), !first, stream);
+    }
 }
 
-void KvStream::end_prefill(int M)
+void KvStream::end_prefill(int M, hipStream_t stream)
 {
+    if (scorer_ && first_layer_of_frame_ >= 0) {
+        // fold the frame's masses into the scores; the row is cleared behind that, or every decode step's fold
+        // would count the frame again
+        scorer_->apply_new_scores(stream);
+        if (drk_dev_memset_async(scorer_->d_new_scores(), 0, (size_t)cm_->table_stride() * sizeof(float), stream) != DRK_OK)
+            LOG_ERROR("Conscientia", "KvStream: clearing the frame's attention masses: %s", drk_last_error());
+        first_layer_of_frame_ = -1;
+    }
     current_pos_ += M;                                                    // stream.cpp:238-239
     cm_->set_seq_len(0, current_pos_);
 }

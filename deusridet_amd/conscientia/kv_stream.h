@@ -62,7 +62,8 @@ public:
     // pages they forked from, the stream copies a block it still shares before it writes into it.
     bool begin_prefill(int M, hipStream_t stream);
     void prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipStream_t stream);
-    void end_prefill(int M);
+    // with a scorer attached the frame's attention masses are folded into the scores here, on `stream`
+    void end_prefill(int M, hipStream_t stream = nullptr);
     int  current_pos() const { return current_pos_; }
 
     // ---- decode branches ---------------------------------------------------------------------
@@ -120,6 +121,7 @@ private:
     AttentionWorkspace ws_prefill_, ws_decode_;
     int max_prefill_rows_ = 0;
     int first_layer_of_step_ = -1;   // the layer whose scored call overwrites instead of accumulating
+    int first_layer_of_frame_ = -1;  // the same for the mass pass of a perception frame
 
     bool host_begin(hipStream_t stream);
     void host_end();

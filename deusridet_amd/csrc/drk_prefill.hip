@@ -906,6 +906,207 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     }
 }
 
+// ---- attention mass of a chunk ------------------------------------------------------------------
+// mass[lb] += sum over the chunk's rows (query tokens x query heads) and over the tokens of logical block lb of
+// the row's softmax probability: what each page of the context received from a perception frame (the
+// importance scorer's input, computed for decode steps by the stream kernel).  The chunk kernels cannot give
+// it -- a row's normaliser is known only when its walk ends -- so this kernel walks the keys twice and never
+// touches V: the first walk finds every row's log-sum-exp, the second adds exp2(score - lse) up by key.
+// The products are S = Q K^T, the transpose of the chunk kernel's: a lane stands for a key (n = lane & 31
+// of each 32-token half tile) and its 16 registers for rows 8 (i / 4) + 4 g + i % 4 of the wave's 32, so a
+// key's sum over rows is a sum over registers plus one exchange between the lane halves, and a page's is a
+// 16-lane DPP sum.  A lane keeps its own running maximum and sum per row over the keys it sees (no exchange
+// per tile); the 32 lanes of a row meet once, between the walks.
+// grid = ceil(M / TPW) * KVH, TPW = 128 / (QH/KVH); block = 256.  mass is added to with float atomics
+// (several workgroups -- row tiles and kv heads -- meet in every page): sums differ by rounding from run to run.
+__device__ __forceinline__ float pf_row16_sum(float v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    auto dpp = [](float x, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false));
+    };
+    v += dpp(v, std::integral_constant<int, 0xB1>{});
+    v += dpp(v, std::integral_constant<int, 0x4E>{});
+    v += dpp(v, std::integral_constant<int, 0x141>{});
+    v += dpp(v, std::integral_constant<int, 0x140>{});
+#endif
+    return v;
+}
+
+template <int DT, int KV = DT, int IO = DT, int D = 128>
+__global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(PrefillArgs A, float *__restrict__ mass, int mass_len)
+{
+    constexpr bool Q8 = KV == DRK_INT8 || KV == DRK_FP8_E4M3;
+    constexpr int RB = D * (Q8 ? 1 : 2);
+    constexpr int kPitchK = D * 2 + 16;
+    constexpr int NKS = D / 16;
+    __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPitchK];
+    __shared__ int valid_lds2[2][4];                        // page present, per (buffer, 16-token run)
+
+    const int kvh = (int)blockIdx.x % A.KVH;
+    const int qt = (int)blockIdx.x / A.KVH;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, g = lane >> 5;
+    const int G = A.QH / A.KVH, TPW = A.tpw;
+    const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
+    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+
+    // Q as the A operand: this lane's fragment belongs to row w * 32 + n
+    uint4 qf[NKS];
+    {
+        const int r = w * 32 + n, rt = r / G;
+        const int tq = qt * TPW + rt;
+        const int head = kvh * G + (r - rt * G);
+        const bool row_live = rt < TPW && tq < A.M;
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+#if defined(__HIP_DEVICE_COMPILE__)
+            if constexpr (IO == DRK_BF16 && DT == DRK_F16) {      // 8-bit pages multiply in fp16
+                v.x = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.x), bf16_hi(v.x)));
+                v.y = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.y), bf16_hi(v.y)));
+                v.z = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.z), bf16_hi(v.z)));
+                v.w = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.w), bf16_hi(v.w)));
+            }
+#endif
+            qf[ks] = v;
+        }
+    }
+    // the rows this lane's registers stand for: tokens [0, vis[i]) are visible to row i (0: an idle row)
+    int vis[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int r = w * 32 + 8 * (i >> 2) + 4 * g + (i & 3), rt = r / G;
+        const int tq = qt * TPW + rt;
+        vis[i] = (rt < TPW && tq < A.M) ? A.pos_start + tq + 1 : 0;
+    }
+
+    const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+    bool kreg_valid = false;
+    int kreg_lim = 0;
+    PfGroup<RB> kreg;
+    constexpr int NL = PfGroup<RB>::NL;
+    uint16_t ksc[NL];
+    auto fetch_k = [&](int tile) {                           // the wave's 16-token run of the tile -> registers
+        const int tg = tile * kPfBN + w * 16;
+        kreg_valid = false;
+        kreg_lim = lim_wg - tg;
+        size_t off = 0, soff = 0;
+        if (tg < lim_wg) {
+            const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
+            const int blk = A.table[lb];
+            if (blk >= 0 && blk < A.NB) {
+                kreg_valid = true;
+                const size_t base = (size_t)blk * A.block_stride;
+                soff = base + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + (tg - lb * A.bs)) * 2;
+                off = base + (size_t)(tg - lb * A.bs) * RB;
+            }
+        }
+        kreg = pf_load_group<false, RB>(kbase, kreg_valid, off, lane);
+#pragma unroll
+        for (int j = 0; j < NL; j++) {
+            const int row = (lane * 16 + 1024 * j) / RB;
+            ksc[j] = (KV == DRK_INT8 && kreg_valid) ? *(const uint16_t *)(A.pool_layer + soff + row * 2) : (uint16_t)0;
+        }
+    };
+    auto stage_k = [&](int buf) {
+        if constexpr (Q8) pf_store_group_q8<kPitchK, KV, RB>(&k_lds2[buf][0], kreg, w, lane, ksc, kreg_lim);
+        else pf_store_group<kPitchK, RB>(&k_lds2[buf][0], kreg, w, lane, kreg_lim);
+        if (lane == 0) valid_lds2[buf][w] = kreg_valid ? 1 : 0;
+    };
+
+    constexpr float kLazy = 8.0f, kNone = -1.0e30f;
+    float m[16], l[16], lse[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) { m[i] = kNone; l[i] = 0.0f; lse[i] = INFINITY; }
+
+    auto walk = [&](auto second) {
+        constexpr bool MASS = decltype(second)::value;
+        fetch_k(0);
+        stage_k(0);
+        if (1 < ntiles) fetch_k(1);
+        __syncthreads();
+#pragma unroll 1
+        for (int it = 0; it < ntiles; it++) {
+            if (it + 1 < ntiles) {
+                stage_k((it + 1) & 1);                       // the buffer tile it - 1 was read from, a barrier ago
+                if (it + 2 < ntiles) fetch_k(it + 2);
+            }
+            pf_f32x16 s[2];
+            {
+                const uint8_t *kb = &k_lds2[it & 1][0] + n * kPitchK + g * 16;
+                const pf_f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int ks = 0; ks < NKS; ks++) {
+                    const uint4 b0 = *(const uint4 *)(kb + ks * 32);
+                    const uint4 b1 = *(const uint4 *)(kb + 32 * kPitchK + ks * 32);
+                    s[0] = mfma32<DT>(qf[ks], b0, ks == 0 ? zero : s[0]);
+                    s[1] = mfma32<DT>(qf[ks], b1, ks == 0 ? zero : s[1]);
+                }
+            }
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                const int key = it * kPfBN + tt * 32 + n;
+                const bool kvalid = valid_lds2[it & 1][tt * 2 + (n >> 4)] != 0;
+                float x[16];
+                bool any_move = false;
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    x[i] = (kvalid && key < vis[i]) ? s[tt][i] * A.scale_log2e : -INFINITY;
+                    if (!MASS) any_move = any_move || x[i] > m[i] + kLazy;
+                }
+                if constexpr (!MASS) {
+                    if (__any(any_move)) {
+#pragma unroll
+                        for (int i = 0; i < 16; i++) {
+                            const float m_new = x[i] > m[i] + kLazy ? x[i] : m[i];
+                            l[i] = l[i] * __builtin_amdgcn_exp2f(m[i] - m_new) + __builtin_amdgcn_exp2f(x[i] - m_new);
+                            m[i] = m_new;
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 16; i++) l[i] += __builtin_amdgcn_exp2f(x[i] - m[i]);
+                    }
+                } else {
+                    float cs = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) cs += __builtin_amdgcn_exp2f(x[i] - lse[i]);
+                    cs += __shfl_xor(cs, 32);                // the key's other 16 rows
+                    cs = pf_row16_sum(cs);                   // the 16 keys of a run
+                    const int run0 = it * kPfBN + tt * 32 + (n & 16);
+                    if (g == 0 && (n & 15) == 0 && run0 < lim_wg) {
+                        const int lb = A.bs_shift >= 0 ? (run0 >> A.bs_shift) : (run0 / A.bs);
+                        if (lb < mass_len && cs != 0.0f) unsafeAtomicAdd(mass + lb, cs);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    };
+    walk(std::false_type{});
+    // a row's lanes (the 32 of its half of the wave) meet: lse = M + log2(sum l 2^(m - M)); +inf for a row that saw nothing
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float mm = m[i];
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) mm = fmaxf(mm, __shfl_xor(mm, off));
+        float ll = l[i] * __builtin_amdgcn_exp2f(m[i] - mm);
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) ll += __shfl_xor(ll, off);
+        lse[i] = ll > 0.0f ? mm + __builtin_log2f(ll) : INFINITY;
+    }
+    walk(std::true_type{});
+}
+
+// mass[0 .. n) = 0
+__global__ void pf_zero_kernel(float *__restrict__ p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
 // Global loads the compiler does not count (see prefix_stream_kernel): issue, and wait until at most N of the
 // wave's loads are outstanding -- the values named become usable then, and only then.
 typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
@@ -1454,6 +1655,60 @@ using namespace drk;
 extern "C" {
 
 void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
+int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
+                                     int layer, int pos_start, int M, float scale, int io_dtype, float *d_block_mass,
+                                     int mass_len, int accumulate, void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (pos_start < 0 || M < 0 || mass_len < 0) return fail(DRK_ERR_INVALID, "prefill_mass: negative pos_start, M or mass_len");
+    if (!q || !pool || !d_block_table || !d_block_mass) return fail(DRK_ERR_INVALID, "prefill_mass: NULL pointer");
+    if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "prefill_mass: io_dtype must be F16 or BF16");
+    if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
+        return fail(DRK_ERR_INVALID, "prefill_mass: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
+    if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill_mass: layer %d outside [0,%d)", layer, a.L);
+    if (!((a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 && (a.bs % 16) == 0 && scale > 0.0f))
+        return fail(DRK_ERR_UNSUPPORTED, "prefill_mass: needs head_dim 128 or 256, at most 128 query heads per kv head, block_size %% 16 == 0, scale > 0");
+    if (a.KVH > 65535) return fail(DRK_ERR_INVALID, "prefill_mass: more than 65535 kv heads");
+    if (M > 0 && mass_len < (pos_start + M + a.bs - 1) / a.bs)
+        return fail(DRK_ERR_INVALID, "prefill_mass: mass_len %d is less than the %d blocks of pos_start + M", mass_len,
+                    (pos_start + M + a.bs - 1) / a.bs);
+    hipStream_t st = (hipStream_t)stream;
+    if (!accumulate && mass_len > 0) {
+        hipLaunchKernelGGL(pf_zero_kernel, dim3((mass_len + 255) / 256), dim3(256), 0, st, d_block_mass, mass_len);
+        DRK_LAUNCH_CHECK("pf_zero_kernel");
+    }
+    if (M == 0) return DRK_OK;
+    PrefillArgs A;
+    A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
+    A.table = d_block_table;
+    A.q = (const uint8_t *)q;
+    A.out = nullptr;
+    A.pos_start = pos_start; A.M = M; A.QH = a.QH; A.KVH = a.KVH; A.NB = a.NB; A.bs = a.bs;
+    A.tpw = 128 / (a.QH / a.KVH);
+    A.bs_shift = ilog2_exact((unsigned)a.bs);
+    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride; A.scale_plane = a.scale_plane;
+    A.scale_log2e = scale * kLog2eP;
+    A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
+    A.gate = nullptr; A.gate_stride = 0;
+    dim3 grid(((M + A.tpw - 1) / A.tpw) * a.KVH);
+#define DRK_PM(DT, KV, IO)                                                                                                      \
+    do {                                                                                                                       \
+        if (a.D == 128) hipLaunchKernelGGL((prefill_mass_kernel<DT, KV, IO, 128>), grid, dim3(256), 0, st, A, d_block_mass, mass_len); \
+        else hipLaunchKernelGGL((prefill_mass_kernel<DT, KV, IO, 256>), grid, dim3(256), 0, st, A, d_block_mass, mass_len);    \
+    } while (0)
+    if (a.dtype == DRK_BF16) DRK_PM(DRK_BF16, DRK_BF16, DRK_BF16);
+    else if (a.dtype == DRK_F16) DRK_PM(DRK_F16, DRK_F16, DRK_F16);
+    else if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16) DRK_PM(DRK_F16, DRK_INT8, DRK_BF16);
+    else if (a.dtype == DRK_INT8) DRK_PM(DRK_F16, DRK_INT8, DRK_F16);
+    else if (io_dtype == DRK_BF16) DRK_PM(DRK_F16, DRK_FP8_E4M3, DRK_BF16);
+    else DRK_PM(DRK_F16, DRK_FP8_E4M3, DRK_F16);
+#undef DRK_PM
+    DRK_LAUNCH_CHECK("prefill_mass_kernel");
+    return DRK_OK;
+}
+
 void drk_debug_set_prefill_two_phase(int mode) { g_prefill_two_phase = mode < 0 ? 1 : (mode > 2 ? 2 : mode); }
 
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)

@@ -81,7 +81,7 @@ SIGNATURES = {
     "drkh_kvs_init": (_i32, [_vp, _vp, _i32, _vp, _vp, _i32, _i32]),
     "drkh_kvs_begin_prefill": (_i32, [_vp, _i32, _vp]),
     "drkh_kvs_prefill_layer": (None, [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp]),
-    "drkh_kvs_end_prefill": (None, [_vp, _i32]),
+    "drkh_kvs_end_prefill": (None, [_vp, _i32, _vp]),
     "drkh_kvs_current_pos": (_i32, [_vp]),
     "drkh_kvs_open_branches": (_i32, [_vp, _i32]),
     "drkh_kvs_set_branch_count": (_i32, [_vp, _i32]),
@@ -191,7 +191,7 @@ class KvStream:
 
     def begin_prefill(self, M, stream=None): return bool(lib().drkh_kvs_begin_prefill(self._h, M, stream))
     def prefill_layer(self, layer, io, M, stream=None): lib().drkh_kvs_prefill_layer(self._h, layer, *io, M, stream)
-    def end_prefill(self, M): lib().drkh_kvs_end_prefill(self._h, M)
+    def end_prefill(self, M, stream=None): lib().drkh_kvs_end_prefill(self._h, M, stream)
     def current_pos(self): return lib().drkh_kvs_current_pos(self._h)
     def open_branches(self, n): return lib().drkh_kvs_open_branches(self._h, n)
     def set_branch_count(self, n): return lib().drkh_kvs_set_branch_count(self._h, n)

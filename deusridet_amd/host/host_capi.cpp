@@ -259,7 +259,7 @@ void drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const vo
 {
     KS(ks)->prefill_layer(fa_layer_idx, make_io(qg, k, v, q_norm, k_norm, q_scratch, attn_out), M, (hipStream_t)stream);
 }
-void drkh_kvs_end_prefill(void *ks, int M) { KS(ks)->end_prefill(M); }
+void drkh_kvs_end_prefill(void *ks, int M, void *stream) { KS(ks)->end_prefill(M, (hipStream_t)stream); }
 int drkh_kvs_current_pos(void *ks) { return KS(ks)->current_pos(); }
 int drkh_kvs_open_branches(void *ks, int n) { return KS(ks)->open_branches(n); }
 int drkh_kvs_set_branch_count(void *ks, int n) { return KS(ks)->set_branch_count(n); }

@@ -145,6 +145,15 @@ void paged_gqa_decode_attention_branches_scored(const __half* Q, __half* kv_pool
                                                 int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
                                                 float* d_block_mass, bool accumulate, hipStream_t stream = 0);
 
+// The attention mass a prefill chunk gives to each block of the context (sum of the softmax
+// probabilities of the block's tokens over the chunk's rows and all query heads) into
+// d_block_mass [mass_len] -- the stream's row of ImportanceScorer::d_new_scores().  A pass of its
+// own after the chunk's attention: Q (normed, with RoPE) and the pool only, no workspace.
+// accumulate = false on the first full-attention layer of a frame, true on the others.
+void paged_prefill_attention_mass(const __half* Q, const __half* kv_pool, const int* d_block_table, int fa_layer_idx,
+                                  int pos_start, int M, int max_phys_blocks, int block_size, float scale,
+                                  float* d_block_mass, int mass_len, bool accumulate, hipStream_t stream = 0);
+
 // ---- the same attention calls on a workspace of the caller's ---------------------
 void paged_gqa_decode_attention(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
                                 __half* out, int fa_layer_idx, int seq_len, int max_phys_blocks, int block_size,

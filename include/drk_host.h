@@ -146,7 +146,7 @@ int   drkh_kvs_init(void *ks, void *cm, int max_context_len, void *scorer, const
 int   drkh_kvs_begin_prefill(void *ks, int M, void *stream);
 void  drkh_kvs_prefill_layer(void *ks, int fa_layer_idx, const void *qg, const void *k, const void *v, const void *q_norm,
                              const void *k_norm, void *q_scratch, void *attn_out, int M, void *stream);
-void  drkh_kvs_end_prefill(void *ks, int M);
+void  drkh_kvs_end_prefill(void *ks, int M, void *stream);
 int   drkh_kvs_current_pos(void *ks);
 int   drkh_kvs_open_branches(void *ks, int n);
 int   drkh_kvs_set_branch_count(void *ks, int n);

@@ -357,6 +357,22 @@ int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const
                                     int layer, float scale, int io_dtype, float *d_block_mass,
                                     int mass_stride, int accumulate, void *workspace,
                                     size_t workspace_bytes, void *stream);
+/* The attention mass a perception frame gives to every block of the context: for the chunk of M
+ * query tokens at pos_start (rows and visibility as in drk_paged_prefill_attention),
+ *   d_block_mass[lb] (+)= sum over the chunk's tokens, all query heads, and the tokens of logical
+ *   block lb of the row's softmax probability
+ * so the entries add up to M * num_q_heads.  "After each Prefill frame, record cumulative attention
+ * weight received by each KV block" (docs/en/architecture/02-memoria.md:40-44); the reference's
+ * scorer takes such an array (importance_scorer.h:37-41) and nothing in the reference fills it.
+ * A separate pass after the frame's attention, as the reference schedules it: it reads Q and K
+ * only (K twice), takes no workspace and writes no attention output.  accumulate != 0 adds to
+ * d_block_mass (sum over layers); 0 clears its mass_len entries first.  mass_len >=
+ * ceil((pos_start + M) / block_size).  The sums are made with float atomics: they differ in
+ * the last bits from run to run.  Geometry: head_dim 128 or 256, block_size % 16 == 0. */
+int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, const void *pool,
+                                     const int32_t *d_block_table, int layer, int pos_start, int M,
+                                     float scale, int io_dtype, float *d_block_mass, int mass_len,
+                                     int accumulate, void *stream);
 /* importance_update_kernel, importance_scorer.cu:27-36, 67-73 */
 int drk_importance_update(float *d_scores, const float *d_new_scores, int n, float decay,
                           void *stream);

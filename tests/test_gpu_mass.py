@@ -109,3 +109,90 @@ def test_block_mass_argument_errors(dev):
     with pytest.raises(cabi.DrkError):
         cabi.call("drk_paged_decode_attention_mass", C.byref(g2), U.p(x), U.p(x), U.p(x), 8, U.p(x), 1, 100, U.p(x), 0,
                   0.1, cabi.F16, U.p(x), 8, 0, U.p(x), 1 << 16, U.stream_ptr())
+
+
+# ---- perception frames: the mass a chunk of query tokens gives to the pages of the context ----------------
+
+def _frame_case(dtype, bs, seed, pos_start, M, heads=(8, 32, 128), holes=()):
+    L = 2
+    KVH, QH, D = heads
+    total = pos_start + M
+    nblk = (total + bs - 1) // bs
+    NB = nblk + 3
+    g, og = U.both_layouts(L, KVH, QH, D, bs, NB, dtype)
+    io = dtype if dtype in (cabi.F16, cabi.BF16) else cabi.BF16
+    rng = np.random.default_rng(seed)
+    table = np.full(nblk + 2, -1, np.int32)
+    table[:nblk] = rng.permutation(NB).astype(np.int32)[:nblk]
+    opool = orc.new_pool(og)
+    kf = rng.standard_normal((total, KVH, D)).astype(np.float32) * 0.5
+    kf[rng.integers(0, total, size=max(1, total // 50))] *= 4.0             # a few sharp keys: mass far from uniform
+    orc.append_batch(og, opool, table, 1, 0, U.to_bits(kf, io), U.normal_bits(rng, (total, KVH, D), io, 0.5), io)
+    for h in holes:
+        table[h] = -1
+    q = U.normal_bits(rng, (M, QH, D), io, 0.7)
+    return g, og, io, table, opool, q
+
+
+def _frame_want(og, io, table, opool, q, pos_start, scale):
+    """fp64: every row of the frame is a branch of length pos_start + t + 1 over the same table"""
+    M = q.shape[0]
+    tables = np.ascontiguousarray(np.broadcast_to(table, (M, table.size)))
+    lens = (pos_start + 1 + np.arange(M)).astype(np.int32)
+    return orc.block_attention_mass(og, q, opool, tables, lens, 1, scale, io, table.size).sum(axis=0)
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
+@pytest.mark.parametrize("bs,pos_start,M,heads", [(16, 0, 1, (8, 32, 128)), (16, 0, 70, (8, 32, 128)), (16, 333, 45, (8, 32, 128)),
+                                                  (32, 500, 130, (2, 12, 128)), (256, 100, 33, (4, 24, 256)), (48, 64, 64, (2, 2, 128))])
+def test_frame_mass_matches_fp64(dev, dtype, bs, pos_start, M, heads):
+    """drk_paged_prefill_attention_mass against the fp64 oracle (rows of the frame as causal branches): 8-bit
+    pages, head_dim 256, 1 / 4 / 6 query heads per kv head, block sizes that are not powers of two, a missing
+    page, stale entries in the output array; the entries add up to M x num_q_heads minus nothing."""
+    total = pos_start + M
+    holes = (1,) if total > 3 * bs else ()
+    g, og, io, table, opool, q = _frame_case(dtype, bs, seed=bs + pos_start + M, pos_start=pos_start, M=M, heads=heads, holes=holes)
+    scale = 1.0 / np.sqrt(heads[2])
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    mass = U.dev_bytes(np.full(table.size, 7.0, np.float32))
+    cabi.call("drk_paged_prefill_attention_mass", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale), io,
+              U.p(mass), table.size, 0, U.stream_ptr())
+    U.sync()
+    got = U.host(mass, np.float32).astype(np.float64)
+    want = _frame_want(og, io, table, opool, q, pos_start, scale)
+    assert np.all(np.abs(got - want) <= 2e-3 * M + 2e-3 * np.abs(want)), np.abs(got - want).max()
+    # every row that sees a token gives all of its probability away
+    seen = sum(1 for t in range(M) if any(table[p // bs] >= 0 for p in range(pos_start + t + 1)))
+    assert abs(got.sum() - seen * heads[1]) <= 1e-3 * M * heads[1]
+    # accumulate: a second layer's pass adds to the first's
+    cabi.call("drk_paged_prefill_attention_mass", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale), io,
+              U.p(mass), table.size, 1, U.stream_ptr())
+    U.sync()
+    assert np.all(np.abs(U.host(mass, np.float32) - 2 * want) <= 4e-3 * M + 4e-3 * np.abs(want))
+
+
+def test_frame_mass_of_a_long_chunk(dev):
+    """A 300-token frame behind 3 000 tokens (several row tiles per kv head meeting in every page)."""
+    pos_start, M, bs = 3000, 300, 16
+    g, og, io, table, opool, q = _frame_case(cabi.BF16, bs, seed=5, pos_start=pos_start, M=M, holes=(7, 150))
+    scale = 1.0 / np.sqrt(128)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    mass = U.dev_zeros(table.size * 4)
+    cabi.call("drk_paged_prefill_attention_mass", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale), io,
+              U.p(mass), table.size, 0, U.stream_ptr())
+    U.sync()
+    got = U.host(mass, np.float32).astype(np.float64)
+    want = _frame_want(og, io, table, opool, q, pos_start, scale)
+    assert np.all(np.abs(got - want) <= 2e-3 * M + 2e-3 * np.abs(want)), np.abs(got - want).max()
+    assert got[7] == 0.0 and got[150] == 0.0
+
+
+def test_frame_mass_argument_errors(dev):
+    g, og, io, table, opool, q = _frame_case(cabi.BF16, 16, seed=1, pos_start=10, M=5)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    mass = U.dev_zeros(64)
+    lib = cabi.lib()
+    args = (C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, 10, 5, 0.1, io, U.p(mass))
+    assert lib.drk_paged_prefill_attention_mass(*args, 0, 0, None) == cabi.ERR_INVALID          # mass_len too small
+    assert lib.drk_paged_prefill_attention_mass(C.byref(g), None, U.p(dpool), U.p(dtab), 1, 10, 5, 0.1, io, U.p(mass), 4, 0, None) == cabi.ERR_INVALID
+    assert lib.drk_paged_prefill_attention_mass(C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 9, 10, 5, 0.1, io, U.p(mass), 4, 0, None) == cabi.ERR_INVALID

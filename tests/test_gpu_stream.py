@@ -134,7 +134,7 @@ def run_session(nbranch, steps, mode, seed=120, scorer=False, shared_policy=None
             ok, mx, _ = U.rel_abs_ok(U.from_bits(got, DT), want)
             assert ok, (M, layer, mx)
             record["prefill"].append(got)
-        s.ks.end_prefill(M)
+        s.ks.end_prefill(M, st)
     assert s.ks.current_pos() == 100 and s.cm.seq_len(0) == 100
     assert np.array_equal(s.pool(), opool)
     # ---- decode branches ----
@@ -282,8 +282,52 @@ def test_stream_session_feeds_the_scorer(dev):
         tot = sum(s.sc.score(b * stride + lb) for lb in range(8))
         want = L * QH * (1 + 0.5 + 0.25)                               # three steps, decay 0.5
         assert abs(tot - want) < 0.05 * want, (b, tot, want)
-    assert sum(s.sc.score(lb) for lb in range(8)) == 0.0              # branch 0 took no decode step
+    # branch 0 took no decode step: its row holds what the two perception frames (64 and 36 tokens) left, folded
+    # once per frame and decayed by every fold since
+    tot0 = sum(s.sc.score(lb) for lb in range(8))
+    want0 = L * QH * (64 * 0.5 + 36) * 0.5 ** 3
+    assert abs(tot0 - want0) < 0.02 * want0, (tot0, want0)
     s.ks.close_branches()
+
+
+def test_perception_frames_feed_the_scorer(dev):
+    """With a scorer attached every perception frame leaves, block by block, the attention mass its rows gave to the
+    context (summed over the layers) in the stream's row of the scores -- against the fp64 oracle, frame after frame
+    (score = score * decay + mass)."""
+    s = Session(1, scorer=True)
+    rng = np.random.default_rng(77)
+    qw, kw = U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT)
+    s.set_weights(qw, kw)
+    st = U.stream_ptr()
+    og = orc.layout(L, KVH, QH, D, BS, s.NB, KVDT)
+    opool = orc.new_pool(og)
+    stride = s.cm.table_stride()
+    want = np.zeros(stride)
+    for M in (64, 5, 36):
+        pos0 = s.ks.current_pos()
+        assert s.ks.begin_prefill(M, st)
+        table0 = s.cm.h_block_table(0).copy()
+        pos = (pos0 + np.arange(M)).astype(np.int32)
+        frame = np.zeros(stride)
+        for layer in range(L):
+            qg, k, v = (U.normal_bits(rng, sh, DT, m) for sh, m in (((M, QH, 2 * D), 1.0), ((M, KVH, D), 0.7), ((M, KVH, D), 0.5)))
+            s.load(qg, k, v)
+            s.ks.prefill_layer(layer, s.io(), M, st)
+            q0, _ = orc.split_q_gate(qg, M, QH, D)
+            qr = orc.apply_rope(orc.head_norm(q0, qw, EPS, DT).reshape(M, QH, D), pos, s.tab, RD, DT)
+            kr = orc.apply_rope(orc.head_norm(k, kw, EPS, DT).reshape(M, KVH, D), pos, s.tab, RD, DT)
+            for tkn in range(M):
+                orc.append_token(og, opool, table0, layer, int(pos[tkn]), kr[tkn], v[tkn], DT)
+            tables = np.ascontiguousarray(np.broadcast_to(table0, (M, stride)))
+            frame += orc.block_attention_mass(og, qr, opool, tables, (pos + 1).astype(np.int32), layer, 1 / np.sqrt(D), DT, stride).sum(axis=0)
+        s.ks.end_prefill(M, st)
+        want = 0.5 * want + frame
+        U.sync()
+        s.sc.sync_to_host()
+        got = np.array([s.sc.score(lb) for lb in range(stride)])
+        assert np.all(np.abs(got - want) <= 4e-3 * M + 3e-3 * np.abs(want)), (M, float(np.abs(got - want).max()))
+        assert abs(frame.sum() - M * QH * L) < 1e-6 * M * QH * L
+    assert np.array_equal(s.pool(), opool)
 
 
 def test_time_division_perception_between_decode_steps_and_a_changing_branch_count(dev):
