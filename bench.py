@@ -273,8 +273,34 @@ def main():
         lib.drk_debug_time_decode_kernel(0)
         r_ms = float(np.mean(buf[:cnt.value]))
         r_bytes = int(rl.sum()) * kv_bytes_per_token
+        # what a launch pays before its first tile: the same launches with the kernel leaving once the branch
+        # lengths are scanned and the workgroup's unit descriptors (one table read per 16-token run) are built
+        lib.drk_debug_set_stream_descriptors_only(1)
+        ragged_only(8)
+        lib.drk_debug_time_decode_kernel(1)
+        ragged_only(n_timed)
+        cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
+        lib.drk_debug_time_decode_kernel(0)
+        lib.drk_debug_set_stream_descriptors_only(0)
+        ragged_pro_ms = float(np.mean(buf[:cnt.value]))
+        attn_only(8)
+        lib.drk_debug_set_stream_descriptors_only(1)
+        attn_only(8)
+        lib.drk_debug_time_decode_kernel(1)
+        attn_only(n_timed)
+        cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
+        lib.drk_debug_time_decode_kernel(0)
+        lib.drk_debug_set_stream_descriptors_only(0)
+        fixed_pro_ms = float(np.mean(buf[:cnt.value]))
+        attn_only(2)                                                 # leave real results behind
         ragged = {"ctx": [int(x) for x in rl], "kernel_us": round(r_ms * 1e3, 2), "bytes_per_launch": r_bytes,
-                  "GBps": round(r_bytes / (r_ms * 1e-3) / 1e9, 1), "hbm_frac": round(r_bytes / (r_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                  "GBps": round(r_bytes / (r_ms * 1e-3) / 1e9, 1), "hbm_frac": round(r_bytes / (r_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                  "prologue_only_us": round(ragged_pro_ms * 1e3, 2),
+                  "streaming_GBps": round(r_bytes / ((r_ms - ragged_pro_ms) * 1e-3) / 1e9, 1),
+                  "headline_prologue_only_us": round(fixed_pro_ms * 1e3, 2),
+                  "headline_streaming_GBps": round(launch_bytes / ((ker_avg_ms - fixed_pro_ms) * 1e-3) / 1e9, 1),
+                  "what": "prologue_only = the launch with the kernel leaving after its prologue (launch, scan of the lengths, "
+                          "unit descriptors); streaming = bytes over the rest of the launch"}
 
     # ---- achievable ceiling on this box: plain 128-bit streaming read of the pool
     probe_bytes = min(pool_bytes, 32 << 30)

@@ -88,6 +88,7 @@ SIGNATURES = {
     "drk_debug_force_portable_decode": (None, [_i32]),
     "drk_debug_set_decode_kernel": (None, [_i32]),
     "drk_debug_set_stream_workgroups": (None, [_i32]),
+    "drk_debug_set_stream_descriptors_only": (None, [_i32]),
     "drk_debug_set_shared_splits": (None, [_i32]),
     "drk_debug_set_prefix_stream": (None, [_i32]),
     "drk_debug_time_decode_kernel": (None, [_i32]),

@@ -70,6 +70,7 @@ int launch_sigmoid_gate(const void *x, const void *gate, void *out, size_t rows,
 constexpr int kStreamMaxUnits = 256;                          // 64-token tiles one workgroup may own (descriptor table in LDS)
 constexpr int kStreamMaxSplitTokens = kStreamMaxUnits * 64;   // the longest explicit split: 16 384 tokens
 extern int g_stream_wgs;
+extern int g_stream_stop_after_descriptors;
 extern int g_shared_splits;
 extern int g_prefix_stream;
 bool stream_decode_supported(const Lay &a, int B);

@@ -713,6 +713,7 @@ int drk_decode_default_split(const drk_kv_layout *g, int B, int max_seq_len)
 void drk_debug_force_portable_decode(int on) { g_force_portable = on ? 1 : 0; }
 void drk_debug_set_decode_kernel(int which) { g_decode_kernel = which; }
 void drk_debug_set_stream_workgroups(int n) { g_stream_wgs = n > 0 ? n : 0; }
+void drk_debug_set_stream_descriptors_only(int on) { g_stream_stop_after_descriptors = on ? 1 : 0; }
 void drk_debug_set_shared_splits(int n) { g_shared_splits = n > 0 ? (n < 256 ? n : 256) : 64; }
 void drk_debug_set_prefix_stream(int on) { g_prefix_stream = on ? 1 : 0; }
 

@@ -37,6 +37,7 @@ namespace drk {
 // for 16-bit pages (bandwidth-bound: fewer, longer runs stream best) and for head_dim
 // 256 (all that fit), 4 per CU for 8-bit pages of head_dim 128, whose tiles are half the bytes.
 int g_stream_wgs = 0;
+int g_stream_stop_after_descriptors = 0;   // measurement aid (drk_debug_set_stream_descriptors_only)
 static inline int stream_wgs(const Lay &a) { return g_stream_wgs > 0 ? g_stream_wgs : (a.E == 1 && a.D == 128 ? 1024 : 512); }
 
 constexpr int kSTile = 64;
@@ -127,6 +128,7 @@ struct StreamArgs {
     // (what the attention-mass pass needs; -inf for a group without a visible token)
     float *lse_groups;
     int lse_stride;
+    int stop_after_descriptors;     // measurement aid: leave once the workgroup's unit descriptors are built
 };
 
 constexpr int kMaxUnits = kStreamMaxUnits;    // units one workgroup may own (descriptor table in LDS)
@@ -362,6 +364,7 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
         }
     }
     __syncthreads();
+    if (A.stop_after_descriptors) return;
 
     uint8_t *const klds = &k_lds[w][0];
     // the 4 K scales and the 4 V scales of tokens 4g..4g+3 (int8 pages)
@@ -821,6 +824,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
         A.scale_log2e = scale * kSLog2e;
         A.lse_groups = lse_groups; A.lse_stride = lse_stride;
+        A.stop_after_descriptors = g_stream_stop_after_descriptors;
 #define DRK_STREAM_LAUNCH(DT)                                                                                           \
     do {                                                                                                                \
         const bool g4 = a.QH / a.KVH <= 4;                                                                              \

@@ -24,6 +24,11 @@ void drk_debug_set_decode_kernel(int which);
 /* Diagnostic: workgroups of the persistent decode grid; 0 restores the default (512; 1024 for
  * 8-bit pages of head_dim 128). */
 void drk_debug_set_stream_workgroups(int n);
+/* Measurement aid: the persistent decode kernel leaves after its prologue (the scan of the branch
+ * lengths and the workgroup's unit descriptors, one table read each) without reading a page or
+ * writing a result -- the launch then costs what every launch pays before its first tile.
+ * Outputs are garbage while this is on. */
+void drk_debug_set_stream_descriptors_only(int on);
 /* Diagnostic: context splits of the shared-prefix pass (default 64, at most 256; 0 restores the
  * default).  Changes drk_decode_shared_workspace_bytes. */
 void drk_debug_set_shared_splits(int n);
