@@ -315,6 +315,13 @@ def main():
     # the dense bf16 rate the matrix cores sustain with no memory traffic at all
     cabi.call("drk_probe_mfma_rate", 20, cabi.p(sink), C.byref(gb))
     mfma_probe_tflops = float(gb.value)
+    # ... and how much of a wave's matrix products hides another wave's vector work on the same SIMD
+    t_m, t_v, t_b = C.c_float(0), C.c_float(0), C.c_float(0)
+    cabi.call("drk_probe_mfma_valu_coexec", 3, cabi.p(sink), C.byref(t_m), C.byref(t_v), C.byref(t_b))
+    coexec = {"mfma_waves_ms": round(t_m.value, 3), "vector_waves_ms": round(t_v.value, 3), "both_ms": round(t_b.value, 3),
+              "hidden_share_of_mfma_time": round((t_m.value + t_v.value - t_b.value) / t_m.value, 3),
+              "what": "one workgroup of 8 waves per CU: waves 4-7 issue 32x32x16 bf16 products, waves 0-3 exp / fma / max3 / pack; "
+                      "perfect overlap gives both = max(alone), none gives the sum"}
 
     # ---- bulk append bandwidth (read source + write pages), all layers in one launch
     m = args.bulk_append_tokens
@@ -559,6 +566,7 @@ def main():
         "hbm_read_probe_GBps": round(read_probe_gbps, 1),
         "hbm_read_probe_permuted_4KiB_GBps": round(permuted_probe_gbps, 1),
         "mfma_bf16_probe_TFLOPs": round(mfma_probe_tflops, 1),
+        "mfma_valu_coexec_probe": coexec,
         "other_configs": other,
         "ragged_ctx_decode": ragged,
         "fill_seconds": round(t_fill, 2),

@@ -115,6 +115,47 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters, float *__res
 #endif
 }
 
+// Do matrix products from one wave and vector instructions from another wave of the same SIMD run at the same
+// time?  A workgroup of eight waves, one per CU: waves 4-7 issue v_mfma_f32_32x32x16_bf16 (four chains), waves 0-3 a
+// softmax-like mix (v_exp_f32, v_fma_f32, v_max3_f32, v_cvt_pk_bf16_f32), 32 vector instructions per four products
+// -- the same issue time on paper.  which: 1 = only the matrix waves work, 2 = only the vector waves, 3 = both.
+__global__ __launch_bounds__(512, 1) void coexec_probe_kernel(int which, int iters, float *__restrict__ sink)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int w = threadIdx.x >> 6;
+    float s = 0.0f;
+    if (w >= 4) {
+        if (!(which & 1)) return;
+        probe_bf16x8 a, b;
+        for (int i = 0; i < 8; i++) { a[i] = (__bf16)(0.001f * (float)(threadIdx.x + i)); b[i] = (__bf16)(0.002f * (float)(threadIdx.x ^ i)); }
+        probe_f32x16 c[4] = {};
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c[j]) : "v"(a), "v"(b));
+        }
+        for (int j = 0; j < 4; j++)
+            for (int i = 0; i < 16; i++) s += c[j][i];
+    } else {
+        if (!(which & 2)) return;
+        float v[8];
+        for (int i = 0; i < 8; i++) v[i] = 0.5f + 0.0001f * (float)threadIdx.x + (float)i;
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int k = 0; k < 32; k++) {
+                if (k % 4 == 0) asm volatile("v_exp_f32 %0, %0" : "+v"(v[k % 8]));
+                else if (k % 4 == 1) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v[k % 8]) : "v"(1.0001f), "v"(0.25f));
+                else if (k % 4 == 2) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(v[k % 8]) : "v"(v[(k + 1) % 8]), "v"(v[(k + 2) % 8]));
+                else asm volatile("v_cvt_pk_bf16_f32 %0, %0, %1" : "+v"(v[k % 8]) : "v"(v[(k + 3) % 8]));
+            }
+        }
+        for (int i = 0; i < 8; i++) s += v[i];
+    }
+    if (s == 12345.678f) *sink = s;                           // practically never: keeps the chains alive
+#else
+    (void)which; (void)iters; (void)sink;
+#endif
+}
+
 // positions and lengths of the decode branches move on by `delta` inside the stream (so that a
 // captured step advances them itself)
 __global__ void advance_i32_kernel(int32_t *__restrict__ a, int32_t *__restrict__ b, int n, int delta)
@@ -453,6 +494,30 @@ int drk_probe_mfma_rate(int iters, void *d_sink, float *tflops)
     DRK_HIP(hipEventDestroy(e1));
     const double flops = (double)iters * wgs * 4.0 /*waves*/ * loop * 4.0 /*chains*/ * (2.0 * 32 * 32 * 16);
     *tflops = (float)(flops / (ms * 1e-3) / 1e12);
+    return DRK_OK;
+}
+
+int drk_probe_mfma_valu_coexec(int iters, void *d_sink, float *ms_mfma, float *ms_valu, float *ms_both)
+{
+    if (!d_sink || !ms_mfma || !ms_valu || !ms_both || iters < 1) return fail(DRK_ERR_INVALID, "probe: bad argument");
+    const int loop = 20000;
+    hipEvent_t e0, e1;
+    DRK_HIP(hipEventCreate(&e0));
+    DRK_HIP(hipEventCreate(&e1));
+    float *out[3] = {ms_mfma, ms_valu, ms_both};
+    for (int which = 1; which <= 3; which++) {
+        hipLaunchKernelGGL(drk::coexec_probe_kernel, dim3(256), dim3(512), 0, 0, which, loop, (float *)d_sink);
+        DRK_HIP(hipEventRecord(e0, 0));
+        for (int i = 0; i < iters; i++)
+            hipLaunchKernelGGL(drk::coexec_probe_kernel, dim3(256), dim3(512), 0, 0, which, loop, (float *)d_sink);
+        DRK_HIP(hipEventRecord(e1, 0));
+        DRK_HIP(hipEventSynchronize(e1));
+        float ms = 0;
+        DRK_HIP(hipEventElapsedTime(&ms, e0, e1));
+        *out[which - 1] = ms / (float)iters;
+    }
+    DRK_HIP(hipEventDestroy(e0));
+    DRK_HIP(hipEventDestroy(e1));
     return DRK_OK;
 }
 

@@ -84,6 +84,13 @@ int drk_probe_read_bandwidth_permuted(const void *d_ptr, size_t bytes, int granu
  * the matrix cores of the part reach on their own.  d_sink is 4 bytes of device memory.
  * Synchronises. */
 int drk_probe_mfma_rate(int iters, void *d_sink, float *tflops);
+/* Measurement aid: how much of one wave's matrix products hides another wave's vector work on
+ * the same SIMD.  One workgroup of eight waves per CU; waves 4-7 issue 32x32x16 bf16 products,
+ * waves 0-3 a softmax-like mix of vector instructions (exp, fma, max3, pack), balanced to the
+ * same issue time.  Reports the milliseconds of a launch with only the matrix waves working,
+ * only the vector waves, and both: perfect overlap gives both = max, none gives the sum.
+ * d_sink is 4 bytes of device memory.  Synchronises. */
+int drk_probe_mfma_valu_coexec(int iters, void *d_sink, float *ms_mfma, float *ms_valu, float *ms_both);
 
 /* ---- layout arithmetic (host only, no GPU needed) --------------------- */
 /* block_pool.cpp:23-39: strides; block_pool.cpp:28-32: budget -> max_blocks */
