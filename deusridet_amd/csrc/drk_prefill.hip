@@ -110,6 +110,58 @@ __device__ __forceinline__ uint2 lds_read_tr16(const uint8_t *p)
 #endif
 }
 
+// 32-bit LDS addresses, for code that does its own address arithmetic (xor swizzles)
+typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
+typedef const pf_u32x4 __attribute__((address_space(3))) *pf_lds_u4_t;
+typedef pf_v4s __attribute__((address_space(3))) *pf_lds_v4s_t;
+__device__ __forceinline__ uint32_t pf_lds_addr(const void *p)
+{
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+__device__ __forceinline__ uint4 pf_lds_read128(uint32_t addr, int offset)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const pf_u32x4 v = *(pf_lds_u4_t)(uintptr_t)(addr + (uint32_t)offset);
+    return make_uint4(v.x, v.y, v.z, v.w);
+#else
+    (void)addr; (void)offset;
+    return make_uint4(0, 0, 0, 0);
+#endif
+}
+__device__ __forceinline__ uint2 pf_lds_read_tr16(uint32_t addr, int offset)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    pf_v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_lds_v4s_t)(uintptr_t)(addr + (uint32_t)offset));
+    return __builtin_bit_cast(uint2, r);
+#else
+    (void)addr; (void)offset;
+    return make_uint2(0, 0);
+#endif
+}
+
+// Workgroup barrier for kernels whose LDS is filled by direct loads from global memory: LDS reads and writes
+// of the wave are complete, its outstanding global loads are NOT waited for (__syncthreads would drain them,
+// the fence it carries covers every store into LDS) -- the caller counts those itself.
+__device__ __forceinline__ void pf_barrier_lds()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_sched_barrier(0);                       // nor may the scheduler move work from one side to the other
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+}
+// 16 bytes per lane from global memory straight into LDS: lane i's land at lds_addr + 16 i (lds_addr is the same
+// for the whole wave).  Written as assembly so that the compiler does not know of the store into LDS: it would
+// wait for every outstanding load ahead of the next LDS read.  The caller counts the loads (pf_async_wait).
+__device__ __forceinline__ void pf_load_to_lds16(const void *base, uint32_t lane_offset, uint32_t lds_addr)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory", "m0");
+#else
+    (void)base; (void)lane_offset; (void)lds_addr;
+#endif
+}
+
 struct PrefillArgs {
     const uint8_t *pool_layer;    // pool + layer * layer_stride
     const int32_t *table;
@@ -906,6 +958,414 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     }
 }
 
+// ---- the two-phase kernel for 16-bit pages: global -> LDS without registers -------------------------
+// As prefill_pp_kernel, but the tiles go from global memory straight into LDS (global_load_lds_dwordx4): a wave's
+// share of a tile is four memory instructions instead of four loads, four LDS writes and the selects between
+// them, and holds no registers, so the requests can run two tiles ahead of their use (four buffers per operand)
+// where registers allowed one.  Swizzled rows without padding instead of padded rows.  What bounds a wave's vector
+// phase is its instruction count -- a wave issues one instruction in about four clocks, scalar ones included --
+// so the phase is kept short: one straight path for whole pages, page addresses from scalar registers, the rare
+// cases (masked tiles, a moving softmax reference, pages in part) out of line.  8-bit pages keep the kernel above
+// (their codes are converted on the way).
+template <int DT, int IO = DT>
+__global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
+{
+    constexpr int D = 128;
+    constexpr int RB = D * 2;                                // bytes of a token row of one kv head, also the LDS row
+    constexpr int kTileBytes = kPfBN * RB;                   // 16 KB per operand and tile
+    constexpr int NKS = D / 16, NDT = D / 32;
+    constexpr int ROWS = 8;                                 // tokens of a tile one wave stages
+    constexpr int kRing = 4;                                // buffers per operand
+    __shared__ __align__(256) uint8_t k_lds3[kRing][kTileBytes];    // 256: the xor swizzle is applied to whole addresses
+    __shared__ __align__(256) uint8_t v_lds3[kRing][kTileBytes];
+
+    const int kvh = (int)blockIdx.x % A.KVH;
+    const int nqt = (int)gridDim.x / A.KVH;
+    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, g = lane >> 5;
+    const bool grpA = w < 4;
+
+    const int G = A.QH / A.KVH, TPW = A.tpw;
+    const int r = w * 32 + n, rt = r / G;
+    const int tq = qt * TPW + rt;
+    const int head = kvh * G + (r - rt * G);
+    const bool row_live = rt < TPW && tq < A.M;
+    const int vis = A.pos_start + tq + 1;
+    const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
+    const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
+    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+
+    // Q as the B operand, multiplied by scale * log2(e) on the way in (rounded once more to the 16-bit
+    // type): the products then are the exponents themselves and the softmax needs no multiply per score.
+    uint4 qf[NKS];
+    {
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
+        const float c = A.scale_log2e;
+        auto scaled = [&](uint32_t w2) -> uint32_t {
+            return pack2<DT>(elem16_to_f((uint16_t)(w2 & 0xffffu), IO) * c, elem16_to_f((uint16_t)(w2 >> 16), IO) * c);
+        };
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            const uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+            qf[ks] = make_uint4(scaled(v.x), scaled(v.y), scaled(v.z), scaled(v.w));
+        }
+    }
+
+    const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+    // ---- pages -------------------------------------------------------------------------------------
+    // The block size is a power of two >= 16 (the host dispatches other sizes to the kernel above), so the
+    // 8 tokens a wave stages lie in one block, a 16-token run has one page, and a tile's blocks never
+    // straddle a multiple of 64.  Table entries come in windows of 64, one per lane, by a vector load (a
+    // scalar load would be waited for at every barrier, whose LDS wait counts on the same counter); two
+    // windows are held, so an entry is in a register long before its tile is reached.  Everything here is
+    // wave-uniform, straight-line code: the only branch is the change of window, every 64 blocks.
+    const int sh = A.bs_shift;
+    const int tgw = w * ROWS;                                 // the wave's first token within a tile
+    const int nblk_needed = (lim_wg + A.bs - 1) >> sh;
+    auto load_window = [&](int lb0) -> int {
+        const int i = lb0 + lane;
+        return i < nblk_needed ? A.table[i] : -1;             // entries past the chunk's last block are never read
+    };
+    auto pages_of = [&](int win) -> unsigned long long { return __builtin_amdgcn_ballot_w64(win >= 0 && win < A.NB); };
+    int win_lb0 = 0;
+    int win_a = load_window(0), win_b = load_window(64);
+    unsigned long long present_a = pages_of(win_a);           // bit i: block win_lb0 + i has a page
+    // the wave's page in `tile` (-1: a hole, or past the end) and the tile's four page flags, one per 16-token run
+    auto lookup = [&](int tile, int &blk, int &flags) {
+        const int lb0 = (tile * kPfBN) >> sh;
+        if (__builtin_expect(lb0 >= win_lb0 + 64, 0)) {       // tiles are asked for in ascending order
+            win_lb0 += 64;
+            win_a = win_b;
+            win_b = load_window(win_lb0 + 64);
+            present_a = pages_of(win_a);
+        }
+        const uint32_t m = (uint32_t)(present_a >> (lb0 - win_lb0));
+        flags = (int)((m & 1u) | (((m >> (16 >> sh)) & 1u) << 1) | (((m >> (32 >> sh)) & 1u) << 2) | (((m >> (48 >> sh)) & 1u) << 3));
+        const int tg = tile * kPfBN + tgw;
+        const int li = (tg >> sh) - win_lb0;
+        const int b = __builtin_amdgcn_readlane(win_a, li);
+        blk = (((present_a >> li) & 1ull) != 0 && tg < lim_wg) ? b : -1;
+    };
+
+    pf_f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+    // The softmax reference m_ref (per row): the products start from -m_ref (the C operand), so a score
+    // arrives as its exponent relative to the reference.  The reference moves only when a tile's maximum
+    // exceeds it by more than kLazy (or is the row's first finite one): weights stay below 2^kLazy, and O
+    // and the row sum are rescaled on those rare occasions only.  out = O / l does not depend on it.
+    constexpr float kLazy = 8.0f;
+    float m_ref = 0.0f, l_run = 0.0f;
+    bool m_init = false;
+    pf_f32x16 negm;
+#pragma unroll
+    for (int i = 0; i < 16; i++) negm[i] = 0.0f;
+
+    // ---- staging -----------------------------------------------------------------------------------
+    // A wave moves 8 rows of K and of V per tile straight from global memory into LDS: two loads of 1 KB per
+    // operand, each landing as the wave's 64 lanes x 16 bytes in a row -- four token rows of 256 bytes.  The LDS
+    // rows have no padding; instead the 16-byte chunk c of row r sits at position c ^ sK(r) (K: sK = r & 15,
+    // whole-row reads by 16 consecutive rows) or c ^ sV(r) (V: sV = (r & 3) << 2, transposed reads of
+    // 4 rows x 64 bytes by 32 lanes), which the loading lane applies on the global side: the lane that fills
+    // position p of a row fetches chunk p ^ s(row).  Rows past the chunk's end and missing pages are not
+    // loaded at all: the buffers start out as zeros and only ever receive real rows, so what such a row holds
+    // is finite, and its scores are masked and its weights are exact zeros.
+    uint32_t goff_k[2], goff_v[2];                           // byte offset of this lane's chunk within the wave's 8 rows
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int rr = lane >> 4, cp = lane & 15, row = tgw + 4 * j + rr;
+        goff_k[j] = (uint32_t)((4 * j + rr) * RB + ((cp ^ (row & 15)) << 4));
+        goff_v[j] = (uint32_t)((4 * j + rr) * RB + ((cp ^ ((row & 3) << 2)) << 4));
+    }
+    // one request: four of the wave's 8 rows (j = which four) from `src`, the wave's first row of the tile in its
+    // page, to `lds`; `rows` of the 8 exist
+    auto request = [&](const uint8_t *src, uint32_t goff, uint32_t lds, int j, int rows) {
+        if (4 * j + (lane >> 4) < rows) pf_load_to_lds16(src, goff, lds);
+    };
+    // at most n of this wave's loads are still on their way (they land in order)
+    auto wait_loads = [&](auto n) {
+        constexpr int N = decltype(n)::value;
+        __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+    };
+
+    pf_f32x16 s[2];                 // scores of the tile in flight: [32-token half][16 per lane]
+    uint4 pb[2][2];                 // its weights, packed: [token half][k-half], the B operand of PV
+
+    // where this lane finds its operands in a tile (see the staging above for the two swizzles): K row n (and
+    // n + 32), chunk 2 ks + g, i.e. byte ((g ^ n & 15) << 4) ^ (ks << 5) of the row -- the xor with ks is made
+    // where it is used (an instruction the compiler may not hoist: eight more registers would spill); V rows
+    // 4 g + j16 / 4 + R (R a multiple of 8, which the swizzle does not see), 8 bytes at dims 32 dt + 16 (lane / 16 % 2)
+    // + 4 (j16 % 4).
+    uint32_t voff[NDT];
+    const uint32_t kx1 = (uint32_t)(n * RB + ((g ^ (n & 15)) << 4));     // row n, chunk g ^ sK(n): k-step 0
+    // the address of k-step ks = that of k-step 0 with ks xor-ed into bits 5-7 (the buffers are 256-byte aligned)
+    auto kaddr = [&](uint32_t base, int ks) -> uint32_t {
+        uint32_t r;
+        asm volatile("v_xor_b32 %0, %2, %1" : "=v"(r) : "v"(base), "s"((uint32_t)(ks << 5)));
+        return r;
+    };
+    {
+        const int j16 = lane & 15;
+        const int rowl = 4 * g + (j16 >> 2);
+        const int clane = 2 * ((lane >> 4) & 1) + ((j16 & 3) >> 1), half = j16 & 1;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+            voff[dt] = (uint32_t)(rowl * RB + ((((dt ^ (rowl & 3)) << 2) | clane) << 4) + (half << 3));
+    }
+
+    // S^T = K Q^T.  The operand reads run two k-steps ahead of the products that use them; scheduling
+    // barriers pin that order, so that at most six operands are in registers at a time.
+    auto qk = [&](int tile) {
+        const uint32_t ka0 = pf_lds_addr(&k_lds3[tile & (kRing - 1)][0]) + kx1;
+        uint4 a[NKS][2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const uint32_t ka = kaddr(ka0, ks);
+            a[ks][0] = pf_lds_read128(ka, 0);
+            a[ks][1] = pf_lds_read128(ka, 32 * RB);
+        }
+        pf_sched_barrier();
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            if (ks + 2 < NKS) {
+                const uint32_t ka = kaddr(ka0, ks + 2);
+                a[ks + 2][0] = pf_lds_read128(ka, 0);
+                a[ks + 2][1] = pf_lds_read128(ka, 32 * RB);
+            }
+            if (ks == 0) {                                   // the products start from minus the row's reference
+                s[0] = mfma32<DT>(a[ks][0], qf[ks], negm);
+                s[1] = mfma32<DT>(a[ks][1], qf[ks], negm);
+            } else {
+                s[0] = mfma32<DT>(a[ks][0], qf[ks], s[0]);
+                s[1] = mfma32<DT>(a[ks][1], qf[ks], s[1]);
+            }
+            pf_sched_barrier();
+        }
+    };
+    // O^T += V^T P^T: 16 products, two transposed 8-byte reads each, the reads four products ahead
+    auto pv = [&](int tile) {
+        const uint32_t v_lds = pf_lds_addr(&v_lds3[tile & (kRing - 1)][0]);
+        uint32_t va[NDT];
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++) va[dt] = v_lds + voff[dt];
+        uint2 lo[16], hi[16];
+        auto rd = [&](int i) {                               // product i = (tt, mh, dt) = (i / 8, (i / 4) & 1, i & 3)
+            const int roff = ((i >> 3) * 32 + 16 * ((i >> 2) & 1)) * RB;
+            lo[i] = pf_lds_read_tr16(va[i & 3], roff);
+            hi[i] = pf_lds_read_tr16(va[i & 3], roff + 8 * RB);
+        };
+#pragma unroll
+        for (int i = 0; i < 4; i++) rd(i);
+        pf_sched_barrier();
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            if (i + 4 < 16) rd(i + 4);
+            o[i & 3] = mfma32<DT>(make_uint4(lo[i].x, lo[i].y, hi[i].x, hi[i].y), pb[i >> 3][(i >> 2) & 1], o[i & 3]);
+            pf_sched_barrier();
+        }
+    };
+    // scores of tile `it` (page flags `flags`) -> packed weights, running maximum and sum, rescale of O^T
+    auto softmax = [&](int it, int flags) {
+        const int tile_t = it * kPfBN;
+        if (__builtin_expect(flags != 15 || it >= first_masked_tile, 0)) {
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    const bool ok = (tile_t + tl) < vis && ((flags >> (tl >> 4)) & 1) != 0;
+                    s[tt][i] = ok ? s[tt][i] : -INFINITY;
+                }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[tt][i]);
+        tmax = pf_max_halves(tmax);                          // a row's scores lie in lanes n and n + 32
+        const bool move = m_init ? tmax > kLazy : tmax > -INFINITY;
+        if (__builtin_expect(__any(move), 0)) {
+            const float delta = move ? tmax : 0.0f;
+            m_init = m_init || move;
+            m_ref += delta;
+            const float alpha = __builtin_amdgcn_exp2f(-delta);
+            l_run *= alpha;
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[tt][i] -= delta;
+#pragma unroll
+            for (int i = 0; i < 16; i++) negm[i] = -m_ref;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+        }
+        float psum = 0.0f;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            float p[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) p[i] = __builtin_amdgcn_exp2f(s[tt][i]);
+            pb[tt][0] = make_uint4(pack2<DT>(p[0], p[1]), pack2<DT>(p[2], p[3]), pack2<DT>(p[4], p[5]), pack2<DT>(p[6], p[7]));
+            pb[tt][1] = make_uint4(pack2<DT>(p[8], p[9]), pack2<DT>(p[10], p[11]), pack2<DT>(p[12], p[13]), pack2<DT>(p[14], p[15]));
+            // the row sum over the weights before rounding: the dot-product instructions that would sum the rounded
+            // pairs run on the matrix pipe and stall the products of the wave that shares the SIMD
+#pragma unroll
+            for (int i = 0; i < 16; i++) psum += p[i];
+        }
+        l_run += psum;
+    };
+
+    // The memory side: in its vector phase a wave requests its share of K(kt) and V(kt - 1) -- kt = t + 3 for the
+    // first half of the workgroup (phase 2t), t + 4 for the second (phase 2t + 1).  Four buffers per operand: the
+    // buffer of tile x is free once tile x's last reader has passed (K: phase 2x, V: phase 2x + 2) and is
+    // requested again for tile x + 4 from phase 2x + 1 (K) and 2x + 3 (V) on.  A request is first read five phases
+    // after it was made; a wave makes sure of its own requests of two vector phases ago at the end of every vector
+    // phase (wait_loads(8): all but the eight of this phase and the one before), ahead of the barrier.
+    const uint32_t k_ring = pf_lds_addr(&k_lds3[0][0]) + (uint32_t)(tgw * RB);   // the wave's rows in buffer 0
+    const uint32_t v_ring = pf_lds_addr(&v_lds3[0][0]) + (uint32_t)(tgw * RB);
+    const uint8_t *vsrc_prev = kbase;                        // where the V rows of the tile looked up last begin
+    int rows_prev = 0;                                       // how many of them exist
+    bool four_issued = false, four_before = false;           // the last stage() / the one before issued exactly four loads
+    // where the wave's K rows of tile kt begin and how many of the 8 exist; the tile's page flags
+    auto find = [&](int kt, int &f_new, const uint8_t *&ksrc, int &rows) {
+        int blk;
+        lookup(kt, blk, f_new);
+        const int tg = kt * kPfBN + tgw;
+        rows = blk >= 0 ? lim_wg - tg : 0;
+        ksrc = kbase + (size_t)max(blk, 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
+    };
+    auto stage = [&](int kt, int &f_new) {
+        const uint8_t *ksrc;
+        int rows;
+        find(kt, f_new, ksrc, rows);
+        const uint32_t lk = k_ring + ((uint32_t)(kt & (kRing - 1)) << 14);
+        const uint32_t lv = v_ring + ((uint32_t)((kt - 1) & (kRing - 1)) << 14);
+        const bool all = min(rows, rows_prev) >= ROWS;
+        if (__builtin_expect(all, 1)) {                      // whole pages: no lane is switched off
+            pf_load_to_lds16(ksrc, goff_k[0], lk);
+            pf_load_to_lds16(ksrc, goff_k[1], lk + 4 * RB);
+            pf_load_to_lds16(vsrc_prev, goff_v[0], lv);
+            pf_load_to_lds16(vsrc_prev, goff_v[1], lv + 4 * RB);
+        } else {
+            request(ksrc, goff_k[0], lk, 0, rows);
+            request(ksrc, goff_k[1], lk + 4 * RB, 1, rows);
+            request(vsrc_prev, goff_v[0], lv, 0, rows_prev);
+            request(vsrc_prev, goff_v[1], lv + 4 * RB, 1, rows_prev);
+        }
+        four_before = four_issued;
+        four_issued = all;
+        vsrc_prev = ksrc + A.kv_plane;
+        rows_prev = rows;
+    };
+    // everything this wave requested before its last stage() has landed (a stage that issued fewer than four
+    // loads -- the chunk's end, a missing page -- waits for everything)
+    auto wait_earlier_loads = [&]() {
+        if (four_issued && four_before) wait_loads(std::integral_constant<int, 8>{});
+        else wait_loads(std::integral_constant<int, 0>{});
+    };
+
+    // ---- prologue: the buffers cleared; K(0), K(1), K(2), V(0), V(1) (second half: also K(3), V(2)) in LDS ----
+    for (int i = threadIdx.x * 16; i < kRing * kTileBytes; i += 512 * 16) {
+        *(uint4 *)(&k_lds3[0][0] + i) = make_uint4(0, 0, 0, 0);
+        *(uint4 *)(&v_lds3[0][0] + i) = make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();
+    int f0, f1, f2, f3 = 15, f4 = 15;                        // page flags of the tiles ahead (see the loops)
+    {
+        auto both = [&](int kt, int &f_new, bool with_v) {   // K(kt) and, if asked for, V(kt)
+            const uint8_t *ksrc;
+            int rows;
+            find(kt, f_new, ksrc, rows);
+            const uint32_t lk = k_ring + ((uint32_t)kt << 14), lv = v_ring + ((uint32_t)kt << 14);
+            request(ksrc, goff_k[0], lk, 0, rows);
+            request(ksrc, goff_k[1], lk + 4 * RB, 1, rows);
+            vsrc_prev = ksrc + A.kv_plane;
+            rows_prev = rows;
+            if (with_v) {
+                request(vsrc_prev, goff_v[0], lv, 0, rows);
+                request(vsrc_prev, goff_v[1], lv + 4 * RB, 1, rows);
+            }
+        };
+        both(0, f0, true);
+        both(1, f1, true);
+        both(2, f2, false);
+        if (!grpA) stage(3, f3);                             // K(3), V(2)
+        wait_loads(std::integral_constant<int, 0>{});
+        four_issued = four_before = false;
+    }
+    __syncthreads();
+    // Both halves pass the same number of barriers.  The loop bodies are straight-line code (the accumulators are
+    // updated in place): the product past the last tile multiplies whatever that K buffer holds and its result is
+    // never read; requests past the last tile load nothing (no page).
+    if (grpA) {
+        // f0, f1, f2 = flags of tiles t, t + 1, t + 2 at the head of iteration t; stage(t + 3) adds tile t + 3's
+        qk(0);
+#pragma unroll 1
+        for (int t = 0; t < ntiles; t++) {
+            stage(t + 3, f3);                                // phase 2t: K(t+3), V(t+2)
+            softmax(t, f0);
+            f0 = f1;
+            f1 = f2;
+            f2 = f3;
+            wait_earlier_loads();
+            pf_barrier_lds();
+            pv(t);                                           // phase 2t+1
+            qk(t + 1);
+            pf_barrier_lds();
+        }
+        pf_barrier_lds();
+    } else {
+        // f0 .. f3 = flags of tiles t .. t + 3 at the head of iteration t; stage(t + 4) adds tile t + 4's
+        qk(0);                                               // phase 0
+        pf_barrier_lds();
+#pragma unroll 1
+        for (int t = 0; t < ntiles; t++) {
+            softmax(t, f0);                                  // phase 2t+1
+            stage(t + 4, f4);                                // K(t+4), V(t+3)
+            f0 = f1;
+            f1 = f2;
+            f2 = f3;
+            f3 = f4;
+            wait_earlier_loads();
+            pf_barrier_lds();
+            pv(t);                                           // phase 2t+2
+            qk(t + 1);
+            pf_barrier_lds();
+        }
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (row_live && (l_tot > 0.0f || A.gate)) {
+        const bool have = l_tot > 0.0f;
+        const float inv = have ? 1.0f / l_tot : 0.0f;
+        uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * (D * 2);
+        const uint16_t *grow = A.gate ? A.gate + ((size_t)tq * A.QH + head) * A.gate_stride : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; b4++) {
+                const int d0 = dt * 32 + 8 * b4 + 4 * g;
+                uint2 v = have ? make_uint2(pack2<IO>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
+                                            pack2<IO>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv))
+                               : *(const uint2 *)(orow + d0 * 2);
+                if (grow) {
+                    const uint2 gv = *(const uint2 *)(grow + d0);
+                    v.x = (uint32_t)gated_elem16((uint16_t)(v.x & 0xffffu), (uint16_t)(gv.x & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.x >> 16), (uint16_t)(gv.x >> 16), IO) << 16);
+                    v.y = (uint32_t)gated_elem16((uint16_t)(v.y & 0xffffu), (uint16_t)(gv.y & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.y >> 16), (uint16_t)(gv.y >> 16), IO) << 16);
+                }
+                *(uint2 *)(orow + d0 * 2) = v;
+            }
+    }
+}
+
 // ---- attention mass of a chunk ------------------------------------------------------------------
 // mass[lb] += sum over the chunk's rows (query tokens x query heads) and over the tokens of logical block lb of
 // the row's softmax probability: what each page of the context received from a perception frame (the
@@ -1109,7 +1569,6 @@ __global__ void pf_zero_kernel(float *__restrict__ p, int n)
 
 // Global loads the compiler does not count (see prefix_stream_kernel): issue, and wait until at most N of the
 // wave's loads are outstanding -- the values named become usable then, and only then.
-typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ pf_u32x4 pf_async_load128(const uint8_t *p)
 {
     pf_u32x4 v;
@@ -1505,7 +1964,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 // pos_start + t + 1, all rows read one table -- so the kernel runs in that mode over tokens
 // [0, pos_start + M) with the context split over the whole chip, and a small kernel folds each
 // row's pieces (and applies the gate).
-int g_prefill_two_phase = 1;                   // 0: never; 1: by the rule in prefill_impl; 2: whenever the geometry allows (tests)
+int g_prefill_two_phase = 1;                   // 0: never; 1: by the rule in prefill_impl; 2: whenever the geometry allows (tests); 3: as 2, with register staging also for 16-bit pages
 int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
 constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
 
@@ -1709,7 +2168,7 @@ int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, cons
     return DRK_OK;
 }
 
-void drk_debug_set_prefill_two_phase(int mode) { g_prefill_two_phase = mode < 0 ? 1 : (mode > 2 ? 2 : mode); }
+void drk_debug_set_prefill_two_phase(int mode) { g_prefill_two_phase = mode < 0 ? 1 : (mode > 3 ? 3 : mode); }
 
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
 {
@@ -1797,6 +2256,12 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         if (wgs2 >= 192 || g_prefill_two_phase > 1) {
             A.tpw = tpw2;
             dim3 grid2((unsigned)wgs2);
+            if ((a.dtype == DRK_BF16 || a.dtype == DRK_F16) && g_prefill_two_phase != 3) {    // 16-bit pages: global -> LDS directly
+                if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_ppd_kernel<DRK_BF16, DRK_BF16>), grid2, dim3(512), 0, st, A);
+                else hipLaunchKernelGGL((prefill_ppd_kernel<DRK_F16, DRK_F16>), grid2, dim3(512), 0, st, A);
+                DRK_LAUNCH_CHECK("prefill_ppd_kernel");
+                return DRK_OK;
+            }
 #define DRK_PP_LAUNCH(DT, KV, IO) hipLaunchKernelGGL((prefill_pp_kernel<DT, KV, IO>), grid2, dim3(512), 0, st, A)
             if (a.dtype == DRK_BF16) DRK_PP_LAUNCH(DRK_BF16, DRK_BF16, DRK_BF16);
             else if (a.dtype == DRK_F16) DRK_PP_LAUNCH(DRK_F16, DRK_F16, DRK_F16);

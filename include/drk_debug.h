@@ -49,9 +49,10 @@ void drk_debug_set_decode_lds_pad(int bytes);
 /* Tuning: which prefill chunks run with the context split over the chip (they must stand behind 2 048 tokens
  * or more): negative = the library's cost rule (default); 0 = none; n = every chunk of up to n rows. */
 void drk_debug_set_prefill_split(int max_rows);
-/* Tuning: which causal chunks of head_dim 128 run on the two-phase chunk kernel (eight waves, 256 rows per
+/* Tuning: which causal chunks of head_dim 128 run on the two-phase chunk kernels (eight waves, 256 rows per
  * workgroup): 0 = none (the four-wave kernel); 1 = the library's rule (default: chunks long enough to give
- * most CUs a workgroup); 2 = every chunk the geometry allows. */
+ * most CUs a workgroup); 2 = every chunk the geometry allows; 3 = as 2, and 16-bit pages too go through
+ * registers on their way into LDS (the kernel 8-bit pages always use) instead of straight from global memory. */
 void drk_debug_set_prefill_two_phase(int mode);
 /* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
  * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */

@@ -202,7 +202,7 @@ def test_config5_full_chunk_prefill_rows(dev):
         s = torch.einsum("hgd,thd->hgt", q[t].float().view(KVH, QH // KVH, D), kv[0, :n]) * scale
         want[i] = torch.einsum("hgt,thd->hgd", torch.softmax(s, dim=-1), kv[1, :n]).reshape(QH, D)
     want = want.cpu().numpy()
-    for mode in (1, 0, 2):                                   # the library's choice (two-phase kernel here), four-wave kernel, forced
+    for mode in (1, 0, 3):                                   # the library's choice (two-phase, global -> LDS), four-wave kernel, two-phase through registers
         lib.drk_debug_set_prefill_two_phase(mode)
         try:
             out2 = torch.zeros_like(q)

@@ -13,13 +13,14 @@ from tests import util as U
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["by_rule", "two_phase"])
+@pytest.fixture(autouse=True, params=["by_rule", "two_phase", "two_phase_through_registers"])
 def chunk_kernel(request):
-    """Every case runs twice: with the library's own choice of chunk kernel, and with the two-phase
-    kernel taken wherever its geometry allows (head_dim 128, blocks of 16 * 2^k tokens), whatever the
-    chunk's length."""
+    """Every case runs three times: with the library's own choice of chunk kernel, with the two-phase
+    kernels taken wherever their geometry allows (head_dim 128, blocks of 16 * 2^k tokens; 16-bit pages go
+    from global memory straight into LDS, 8-bit pages through registers), and with the register kind for
+    16-bit pages too, whatever the chunk's length."""
     lib = cabi.lib()
-    lib.drk_debug_set_prefill_two_phase(2 if request.param == "two_phase" else 1)
+    lib.drk_debug_set_prefill_two_phase({"by_rule": 1, "two_phase": 2, "two_phase_through_registers": 3}[request.param])
     yield request.param
     lib.drk_debug_set_prefill_two_phase(1)
 
