@@ -786,7 +786,7 @@ def kernel_fractions(buf, seed=11):
             per_chunk.append((a0.elapsed_time(a1), 4.0 * chunk * (c * chunk + (chunk + 1) / 2.0) * D * QH))
     tot_ms, tot_fl = sum(t for t, _ in per_chunk), sum(f for _, f in per_chunk)
     res["config5_prefill"] = _entry(
-        "prefill_pp_kernel<bf16>", "mfma", tot_fl / len(per_chunk), tot_ms / len(per_chunk),
+        "prefill_ppd_kernel<bf16>", "mfma", tot_fl / len(per_chunk), tot_ms / len(per_chunk),
         "config 5: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV x 128 bf16; average "
         "over the 16 launches (flops = 4 M (pos_start + (M+1)/2) D QH per chunk)",
         {"last_chunk_us": round(per_chunk[-1][0] * 1e3, 1),

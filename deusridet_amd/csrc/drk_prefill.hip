@@ -1128,6 +1128,10 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
             a[ks][0] = pf_lds_read128(ka, 0);
             a[ks][1] = pf_lds_read128(ka, 32 * RB);
         }
+        // The registers of the last tile's scores stay taken up to here, so that the first operands cannot land in
+        // them: the products below then write the new scores where the softmax expects them, instead of somewhere
+        // else with sixteen moves (and a wait for the last product) at the end.
+        asm volatile("" : : "v"(s[0]), "v"(s[1]));
         pf_sched_barrier();
 #pragma unroll
         for (int ks = 0; ks < NKS; ks++) {
@@ -1139,6 +1143,7 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
             if (ks == 0) {                                   // the products start from minus the row's reference
                 s[0] = mfma32<DT>(a[ks][0], qf[ks], negm);
                 s[1] = mfma32<DT>(a[ks][1], qf[ks], negm);
+                asm volatile("" : : "v"(negm));              // still in use: neither product may take its registers
             } else {
                 s[0] = mfma32<DT>(a[ks][0], qf[ks], s[0]);
                 s[1] = mfma32<DT>(a[ks][1], qf[ks], s[1]);
