@@ -323,6 +323,15 @@ def main():
               "what": "one workgroup of 8 waves per CU: waves 4-7 issue 32x32x16 bf16 products, waves 0-3 exp / fma / max3 / pack; "
                       "perfect overlap gives both = max(alone), none gives the sum"}
 
+    # ... and the same for two waves that take turns between barriers (the two-phase prefill kernels), one kind of
+    # vector instruction at a time: the share of the vector turns' time that the other wave's products hide
+    phase = {}
+    for op, name in enumerate(("v_exp_f32", "v_fma_f32", "v_dot2_f32_bf16", "v_cvt_pk_bf16_f32", "v_max3_f32", "v_cmp_gt_f32",
+                               "v_permlane32_swap_b32", "s_nop 3")):
+        cabi.call("drk_probe_phase_coexec", op, 2, cabi.p(sink), C.byref(t_m), C.byref(t_v), C.byref(t_b))
+        phase[name] = round(1.0 - (t_b.value - t_m.value) / t_v.value, 2)
+    coexec["hidden_share_by_instruction_in_turns"] = phase
+
     # ---- bulk append bandwidth (read source + write pages), all layers in one launch
     m = args.bulk_append_tokens
     scratch_tab = torch.from_numpy(perm[o:o + (m + bs - 1) // bs].copy()).cuda() if o + (m + bs - 1) // bs <= NB else None

@@ -102,6 +102,7 @@ SIGNATURES = {
     "drk_probe_read_bandwidth_permuted": (_i32, [_vp, _sz, _i32, _i32, _vp, C.POINTER(C.c_float)]),
     "drk_probe_mfma_rate": (_i32, [_i32, _vp, C.POINTER(C.c_float)]),
     "drk_probe_mfma_valu_coexec": (_i32, [_i32, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "drk_probe_phase_coexec": (_i32, [_i32, _i32, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "drk_prefill_workspace_bytes_max": (_sz, [_LP, _i32, _i32]),
     "drk_debug_decode_kernel_times": (_i32, [C.POINTER(C.c_float), _i32, C.POINTER(_i32)]),
     "drk_paged_decode_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),

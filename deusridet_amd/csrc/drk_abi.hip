@@ -156,6 +156,74 @@ __global__ __launch_bounds__(512, 1) void coexec_probe_kernel(int which, int ite
 #endif
 }
 
+// Which vector instructions of one wave run beside the matrix products of the wave it shares a SIMD with, when the
+// two take turns the way the two-phase prefill kernels do?  One workgroup of eight waves per CU; between two
+// barriers waves 0-3 issue 32 products (four chains) while waves 4-7 issue 32 x N vector instructions of ONE
+// kind, then the roles swap.  which: 1 = every wave only does its products (the vector turns are empty), 2 = only
+// the vector turns, 3 = both.
+template <int OP>
+__device__ __forceinline__ void phase_probe_op(float (&v)[8], int r)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (OP == 0) asm volatile("v_exp_f32 %0, %0" : "+v"(v[r]));
+    if constexpr (OP == 1) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(v[r]) : "v"(1.0001f), "v"(0.25f));
+    if constexpr (OP == 2) asm volatile("v_dot2_f32_bf16 %0, %1, %2, %0" : "+v"(v[r]) : "v"(v[(r + 1) & 7]), "v"(0x3f803f80u));
+    if constexpr (OP == 3) asm volatile("v_cvt_pk_bf16_f32 %0, %0, %1" : "+v"(v[r]) : "v"(v[(r + 3) & 7]));
+    if constexpr (OP == 4) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(v[r]) : "v"(v[(r + 3) & 7]), "v"(v[(r + 5) & 7]));
+    if constexpr (OP == 5) asm volatile("v_cmp_gt_f32 vcc, %0, %1" : : "v"(v[r]), "v"(v[(r + 3) & 7]) : "vcc");
+    if constexpr (OP == 6) asm volatile("v_permlane32_swap_b32 %0, %1" : "+v"(v[r]), "+v"(v[(r + 3) & 7]));
+    if constexpr (OP == 7) asm volatile("s_nop 3");
+#else
+    (void)v; (void)r;
+#endif
+}
+template <int OP, int N, int WHICH>
+__global__ __launch_bounds__(512, 1) void phase_probe_kernel(int iters, float *__restrict__ sink)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int w = threadIdx.x >> 6;
+    probe_bf16x8 a, b;
+    for (int i = 0; i < 8; i++) { a[i] = (__bf16)(0.001f * (float)(threadIdx.x + i)); b[i] = (__bf16)(0.002f * (float)(threadIdx.x ^ i)); }
+    probe_f32x16 c[4] = {};
+    float v[8];
+    for (int i = 0; i < 8; i++) v[i] = 0.5f + 0.0001f * (float)threadIdx.x + (float)i;
+    auto products = [&]() {
+        if constexpr ((WHICH & 1) != 0) {
+#pragma unroll
+            for (int i = 0; i < 32; i++) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c[i & 3]) : "v"(a), "v"(b));
+        }
+    };
+    auto vectors = [&]() {
+        if constexpr ((WHICH & 2) != 0) {
+#pragma unroll
+            for (int i = 0; i < 32; i++)
+#pragma unroll
+                for (int e = 0; e < N; e++) phase_probe_op<OP>(v, (i + e) & 7);
+        }
+    };
+    for (int it = 0; it < iters; it++) {
+        if (w < 4) products(); else vectors();
+        __builtin_amdgcn_s_barrier();
+        if (w < 4) vectors(); else products();
+        __builtin_amdgcn_s_barrier();
+    }
+    float s = 0.0f;
+    for (int j = 0; j < 4; j++)
+        for (int i = 0; i < 16; i++) s += c[j][i];
+    for (int i = 0; i < 8; i++) s += v[i];
+    if (s == 12345.678f) *sink = s;                           // practically never: keeps the chains alive
+#else
+    (void)iters; (void)sink;
+#endif
+}
+template <int OP, int N>
+static void phase_probe_launch(int which, int iters, float *sink)
+{
+    if (which == 1) hipLaunchKernelGGL((phase_probe_kernel<OP, N, 1>), dim3(256), dim3(512), 0, 0, iters, sink);
+    else if (which == 2) hipLaunchKernelGGL((phase_probe_kernel<OP, N, 2>), dim3(256), dim3(512), 0, 0, iters, sink);
+    else hipLaunchKernelGGL((phase_probe_kernel<OP, N, 3>), dim3(256), dim3(512), 0, 0, iters, sink);
+}
+
 // positions and lengths of the decode branches move on by `delta` inside the stream (so that a
 // captured step advances them itself)
 __global__ void advance_i32_kernel(int32_t *__restrict__ a, int32_t *__restrict__ b, int n, int delta)
@@ -510,6 +578,43 @@ int drk_probe_mfma_valu_coexec(int iters, void *d_sink, float *ms_mfma, float *m
         DRK_HIP(hipEventRecord(e0, 0));
         for (int i = 0; i < iters; i++)
             hipLaunchKernelGGL(drk::coexec_probe_kernel, dim3(256), dim3(512), 0, 0, which, loop, (float *)d_sink);
+        DRK_HIP(hipEventRecord(e1, 0));
+        DRK_HIP(hipEventSynchronize(e1));
+        float ms = 0;
+        DRK_HIP(hipEventElapsedTime(&ms, e0, e1));
+        *out[which - 1] = ms / (float)iters;
+    }
+    DRK_HIP(hipEventDestroy(e0));
+    DRK_HIP(hipEventDestroy(e1));
+    return DRK_OK;
+}
+
+int drk_probe_phase_coexec(int op, int iters, void *d_sink, float *ms_products, float *ms_vectors, float *ms_both)
+{
+    if (!d_sink || !ms_products || !ms_vectors || !ms_both || iters < 1 || op < 0 || op > 7)
+        return fail(DRK_ERR_INVALID, "probe: bad argument");
+    const int loop = 2000;
+    hipEvent_t e0, e1;
+    DRK_HIP(hipEventCreate(&e0));
+    DRK_HIP(hipEventCreate(&e1));
+    float *out[3] = {ms_products, ms_vectors, ms_both};
+    for (int which = 1; which <= 3; which++) {
+        auto launch = [&]() {
+            float *s = (float *)d_sink;
+            switch (op) {                                    // instructions per product: about 16 clocks of vector issue
+            case 0: drk::phase_probe_launch<0, 2>(which, loop, s); break;
+            case 1: drk::phase_probe_launch<1, 4>(which, loop, s); break;
+            case 2: drk::phase_probe_launch<2, 2>(which, loop, s); break;
+            case 3: drk::phase_probe_launch<3, 4>(which, loop, s); break;
+            case 4: drk::phase_probe_launch<4, 4>(which, loop, s); break;
+            case 5: drk::phase_probe_launch<5, 4>(which, loop, s); break;
+            case 6: drk::phase_probe_launch<6, 2>(which, loop, s); break;
+            default: drk::phase_probe_launch<7, 4>(which, loop, s); break;
+            }
+        };
+        launch();
+        DRK_HIP(hipEventRecord(e0, 0));
+        for (int i = 0; i < iters; i++) launch();
         DRK_HIP(hipEventRecord(e1, 0));
         DRK_HIP(hipEventSynchronize(e1));
         float ms = 0;

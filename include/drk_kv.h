@@ -91,6 +91,14 @@ int drk_probe_mfma_rate(int iters, void *d_sink, float *tflops);
  * only the vector waves, and both: perfect overlap gives both = max, none gives the sum.
  * d_sink is 4 bytes of device memory.  Synchronises. */
 int drk_probe_mfma_valu_coexec(int iters, void *d_sink, float *ms_mfma, float *ms_valu, float *ms_both);
+/* Measurement aid: the same question for two waves that take turns, as the halves of a two-phase
+ * prefill workgroup do: between two workgroup barriers waves 0-3 issue 32 products while waves 4-7
+ * issue vector instructions of ONE kind (about 16 clocks' worth per product), then the roles swap.
+ * op: 0 v_exp_f32, 1 v_fma_f32, 2 v_dot2_f32_bf16, 3 v_cvt_pk_bf16_f32, 4 v_max3_f32,
+ * 5 v_cmp_gt_f32 (writes vcc), 6 v_permlane32_swap_b32, 7 s_nop 3.  Reports the milliseconds of a
+ * launch with only the products, only the vector turns, and both; (both - products) / vectors is
+ * the share of the vector time that stays visible.  d_sink is 4 bytes of device memory.  Synchronises. */
+int drk_probe_phase_coexec(int op, int iters, void *d_sink, float *ms_products, float *ms_vectors, float *ms_both);
 
 /* ---- layout arithmetic (host only, no GPU needed) --------------------- */
 /* block_pool.cpp:23-39: strides; block_pool.cpp:28-32: budget -> max_blocks */
