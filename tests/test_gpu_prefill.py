@@ -241,6 +241,32 @@ def test_random_prefill_shapes(dev, seed):
     assert ok, f"max abs err {ma:.4g} ({D=} {KVH=} {G=} {bs=} {dtype=} {pos_start=} {M=} {holes=})"
 
 
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
+@pytest.mark.parametrize("bs,G,pos_start,M,holes", [
+    (16, 4, 700, 150, (3, 44)), (32, 1, 1, 300, (0,)), (64, 3, 640, 64, (9,)), (128, 8, 1023, 33, ()), (256, 2, 900, 257, (1,)),
+    (16, 16, 0, 600, (5, 6, 7, 8)), (32, 5, 2047, 2, ()), (16, 4, 4096, 256, (100, 255))])
+def test_ring_of_tiles_wraps_over_holes_and_ragged_ends(dev, chunk_kernel, dtype, bs, G, pos_start, M, holes):
+    """16-bit pages with head_dim 128 on the kernel that loads tiles straight into LDS (the forced two-phase run of
+    this case; the other two runs take the same inputs through the other kernels): walks of 10 to 70 tiles, so that
+    the ring of tile buffers wraps many times, with missing pages (whole tiles of them with 16-token blocks), chunks
+    that end inside a page and inside a tile, every block size the kernel takes and group sizes that are not powers of
+    two.  Rows behind holes only keep the caller's bytes; everything else against fp64 on the stored values."""
+    KVH, D = 2, 128
+    total = pos_start + M
+    nblk = (total + bs - 1) // bs
+    holes = tuple(h for h in holes if h < nblk)
+    geom = (2, KVH, KVH * G, D, bs, nblk + 3)
+    g, og, rng, table, opool = build(geom, dtype, total, seed=bs * 1000 + G, holes=holes, mul=0.7)
+    q = U.normal_bits(rng, (M, KVH * G, D), dtype, 0.7)
+    scale = 1 / np.sqrt(D)
+    got = run_prefill(g, U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table), 1, pos_start, M, scale, dtype, KVH * G, D)
+    want = orc.prefill_f64(og, q, opool, table, 1, pos_start, scale, dtype)
+    seen = np.array([any(table[t // bs] >= 0 for t in range(pos_start + r + 1)) for r in range(M)])
+    assert np.all(got[~seen].view(np.uint8) == 0x7B)
+    ok, ma, _ = U.rel_abs_ok(U.from_bits(got[seen], dtype), want[seen])
+    assert ok, f"max abs err {ma:.4g} ({chunk_kernel=} {bs=} {G=} {pos_start=} {M=} {holes=})"
+
+
 @pytest.mark.parametrize("geom,dtype,io", [((2, 8, 32, 128, 16, 300), cabi.BF16, cabi.BF16), ((2, 4, 24, 256, 256, 20), cabi.F16, cabi.F16),
                                            ((2, 2, 8, 128, 32, 150), cabi.INT8, cabi.BF16), ((2, 2, 12, 128, 16, 300), cabi.FP8_E4M3, cabi.F16)])
 @pytest.mark.parametrize("pos_start,M", [(2048, 1), (2049, 17), (3000, 64), (4095, 65), (2500, 130), (2048, 256)])
