@@ -784,6 +784,26 @@ def kernel_fractions(buf, seed=11):
             a1.record(stream)
             torch.cuda.synchronize()
             per_chunk.append((a0.elapsed_time(a1), 4.0 * chunk * (c * chunk + (chunk + 1) / 2.0) * D * QH))
+    # the same kernel at position 30 720 with fewer workgroups (shorter chunks): microseconds per 64-token tile of the
+    # longest walk.  One workgroup per CU either way -- what changes is how much of the chip draws power.
+    by_wgs = {}
+    for m in (64, 512, 1024, 2048):
+        q = torch.randn(m, QH, D, device="cuda").to(torch.bfloat16)
+        o = torch.empty_like(q)
+        pos = total - chunk
+        lib.drk_debug_set_prefill_two_phase(2)                                    # also where the rule would pick the four-wave kernel
+        for _ in range(2):
+            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, pos, m, scale,
+                      cabi.BF16, None, 0, sp)
+        a0, a1 = ev(), ev()
+        a0.record(stream)
+        for _ in range(4):
+            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, pos, m, scale,
+                      cabi.BF16, None, 0, sp)
+        a1.record(stream)
+        torch.cuda.synchronize()
+        lib.drk_debug_set_prefill_two_phase(1)
+        by_wgs[str(m // 64 * KVH)] = round(a0.elapsed_time(a1) / 4 * 1e3 / ((pos + m + 63) // 64), 3)
     tot_ms, tot_fl = sum(t for t, _ in per_chunk), sum(f for _, f in per_chunk)
     res["config5_prefill"] = _entry(
         "prefill_ppd_kernel<bf16>", "mfma", tot_fl / len(per_chunk), tot_ms / len(per_chunk),
@@ -792,5 +812,6 @@ def kernel_fractions(buf, seed=11):
         {"last_chunk_us": round(per_chunk[-1][0] * 1e3, 1),
          "last_chunk_TFLOPs": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12, 1),
          "last_chunk_frac": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-         "first_chunk_TFLOPs": round(per_chunk[0][1] / (per_chunk[0][0] * 1e-3) / 1e12, 1)})
+         "first_chunk_TFLOPs": round(per_chunk[0][1] / (per_chunk[0][0] * 1e-3) / 1e12, 1),
+         "us_per_tile_by_workgroups_at_30720": by_wgs})
     return res
