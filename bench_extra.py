@@ -557,7 +557,28 @@ def config7(args):
     ker_ms = _timed_decode(lib, cabi, lambda n: [attn(i % L, dlen) for i in range(n)], 60)
     launch_bytes = B * ctx * per_tok
     ach = launch_bytes / (ker_ms * 1e-3) / 1e9
+    # the same shape's chunked prefill: 2 048-token chunks at positions 0, 6 144 and 30 720 of branch 0's pages
+    M = 2048
+    qc = (torch.randn(M, QH, D, device="cuda") * 0.5).to(h)
+    oc = torch.empty_like(qc)
+    prefill = {}
+    for pos in (0, 3 * M, 15 * M):
+        for _ in range(2):
+            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(pool), cabi.p(dtab), cabi.p(oc), 0, pos, M,
+                      float(scale), cabi.F16, None, 0, sp)
+        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a0.record(stream)
+        for _ in range(4):
+            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(pool), cabi.p(dtab), cabi.p(oc), 0, pos, M,
+                      float(scale), cabi.F16, None, 0, sp)
+        a1.record(stream)
+        torch.cuda.synchronize()
+        ms = a0.elapsed_time(a1) / 4
+        fl = 4.0 * M * (pos + (M + 1) / 2.0) * D * QH
+        prefill["pos_%d" % pos] = {"us": round(ms * 1e3, 1), "TFLOPs": round(fl / (ms * 1e-3) / 1e12, 1),
+                                   "frac": round(fl / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
     return {
+        "prefill_chunks_2048": {"kernel": "prefill_d256_kernel<f16>", "bound": "mfma", "peak": MFMA_BF16_PEAK_TFLOPS, **prefill},
         "metric": "paged_decode_attention_GBps", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K,
         "warmup": W, "ms_per_step": round(total_ms / K, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",

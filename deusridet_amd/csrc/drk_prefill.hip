@@ -1371,6 +1371,313 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
     }
 }
 
+// ---- head_dim 256, 16-bit pages: one wave per SIMD, tiles straight into LDS -------------------------
+// 128 rows per workgroup as in prefill_mfma_kernel (a wave's 32 rows x 256 dims of output are 128 accumulator
+// registers, so a SIMD holds one wave), but the tiles go from global memory straight into LDS as in
+// prefill_ppd_kernel: no registers hold tile data (the register kind keeps 64 of them and, short of registers,
+// moves them and the Q operands between the two register files all the time), rows are swizzled instead of padded,
+// and with nothing else to overlap a wave's LDS latency and vector work with, the order of its instructions is
+// written out: the exponentials of tile t go between the k-steps of tile t + 1's scores, two per k-step, operand reads
+// run two k-steps / four products ahead, scheduling barriers pin it.  Per tile and wave 64 products (2 048 clocks).
+// Requests run one tile ahead, two buffers per operand, one barrier per tile: step t first takes the maximum of tile
+// t's scores (registers only), then waits for its requests of the step before and meets the other waves, then
+// requests K(t + 2) and V(t + 1) -- into the buffers of K(t) and V(t - 1) -- one request every four products of
+// QK(t + 1) and PV(t).
+template <int DT, int IO = DT>
+__global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
+{
+    constexpr int D = 256, RB = D * 2;                       // bytes of a token row of one kv head, also the LDS row
+    constexpr int kTileBytes = kPfBN * RB;                   // 32 KB per operand and tile
+    constexpr int NKS = D / 16, NDT = D / 32;
+    constexpr int ROWS = 16;                                 // tokens of a tile one wave requests
+    constexpr int XQ = 2, XP = 4;                            // operand reads ahead of their products: k-steps (QK), products (PV)
+    __shared__ __align__(512) uint8_t k_ldsd[2][kTileBytes]; // 512: the xor swizzle is applied to whole addresses
+    __shared__ __align__(512) uint8_t v_ldsd[2][kTileBytes];
+    __shared__ int valid_ldsd[4][4];                         // [tile & 3][wave]: the wave's 16-token run of the tile has a page
+
+    const int kvh = (int)blockIdx.x % A.KVH;
+    const int nqt = (int)gridDim.x / A.KVH;
+    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, g = lane >> 5;
+
+    const int G = A.QH / A.KVH, TPW = A.tpw;
+    const int r = w * 32 + n, rt = r / G;
+    const int tq = qt * TPW + rt;
+    const int head = kvh * G + (r - rt * G);
+    const bool row_live = rt < TPW && tq < A.M;
+    const int vis = A.pos_start + tq + 1;
+    const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
+    const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
+    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+
+    // Q as the B operand, multiplied by scale * log2(e) on the way in (rounded once more to the 16-bit
+    // type): the products then are the exponents themselves and the softmax needs no multiply per score.
+    uint4 qf[NKS];
+    {
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
+        const float c = A.scale_log2e;
+        auto scaled = [&](uint32_t w2) -> uint32_t {
+            return pack2<DT>(elem16_to_f((uint16_t)(w2 & 0xffffu), IO) * c, elem16_to_f((uint16_t)(w2 >> 16), IO) * c);
+        };
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            const uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+            qf[ks] = make_uint4(scaled(v.x), scaled(v.y), scaled(v.z), scaled(v.w));
+        }
+    }
+
+    const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+    const int sh = A.bs_shift;                               // blocks of 16 * 2^k tokens: a wave's 16 rows lie in one block
+    const int tgw = w * ROWS;                                // the wave's first token within a tile
+
+    // ---- requests ------------------------------------------------------------------------------------
+    // One request is 2 token rows (1 KB): lanes 0-31 the first, 32-63 the second; a wave has 8 per operand and tile.
+    // The 16-byte chunk c of row r sits at position c ^ (r & 15) (K, xor on the low four bits: whole-row reads by 16
+    // consecutive rows) or c ^ ((r & 3) << 2) (V: transposed reads of 4 rows x 64 bytes), which the requesting lane
+    // applies on the global side.  Rows past the chunk's end and missing pages are not requested: the buffers
+    // start out as zeros and only ever receive real rows.
+    uint32_t goff_k[8], goff_v[2];
+    {
+        const int rr = lane >> 5, cp = lane & 31;
+#pragma unroll
+        for (int j = 0; j < 8; j++) goff_k[j] = (uint32_t)(rr * RB + ((cp ^ ((2 * j + rr) & 15)) << 4));
+#pragma unroll
+        for (int j = 0; j < 2; j++) goff_v[j] = (uint32_t)(rr * RB + ((cp ^ (((2 * j + rr) & 3) << 2)) << 4));
+    }
+    auto wait_loads = [&]() { __builtin_amdgcn_s_waitcnt(0x0f70); };         // vmcnt(0): every request has landed
+    // the wave's page in `tile`, or -1; a vector load (a scalar one would share its counter with the LDS reads)
+    auto page_of = [&](int tile) -> int {
+        const int tg = tile * kPfBN + tgw;
+        return tg < lim_wg ? A.table[tg >> sh] : -1;
+    };
+    const uint8_t *vsrc_prev = kbase;                        // where the V rows of the tile requested last begin
+    int rows_prev = 0;                                       // how many of them exist
+    const uint32_t k_ring = pf_lds_addr(&k_ldsd[0][0]) + (uint32_t)(tgw * RB);
+    const uint32_t v_ring = pf_lds_addr(&v_ldsd[0][0]) + (uint32_t)(tgw * RB);
+    // A tile's requests in two steps.  plan(kt, page): where K(kt) comes from and where it and V(kt - 1) go (scalar
+    // work).  dma_k(j) / dma_v(j): request j of 8.  A wave's next memory instruction waits until the one before has
+    // passed the address unit (some 130 clocks for these), so the 16 requests of a tile are spread over the tile's
+    // products, one every four, instead of being issued in a row.
+    const uint8_t *p_ksrc = kbase, *p_vsrc = kbase;
+    int p_rows = 0, p_vrows = 0;
+    uint32_t p_lk = 0, p_lv = 0;
+    auto plan = [&](int kt, int blk_raw) {
+        const int blk0 = __builtin_amdgcn_readfirstlane(blk_raw);
+        const int tg = kt * kPfBN + tgw;
+        const bool ok = blk0 >= 0 && blk0 < A.NB && tg < lim_wg;
+        p_vsrc = vsrc_prev;
+        p_vrows = rows_prev;
+        p_rows = ok ? lim_wg - tg : 0;
+        p_ksrc = kbase + (size_t)(ok ? blk0 : 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
+        p_lk = k_ring + ((uint32_t)(kt & 1) << 15);
+        p_lv = v_ring + ((uint32_t)((kt - 1) & 1) << 15);
+        if (lane == 0) valid_ldsd[kt & 3][w] = ok ? 1 : 0;
+        vsrc_prev = p_ksrc + A.kv_plane;
+        rows_prev = p_rows;
+    };
+    auto dma_k = [&](int j) {
+        if (__builtin_expect(p_rows >= ROWS, 1)) pf_load_to_lds16(p_ksrc + 1024 * j, goff_k[j], p_lk + 1024 * j);
+        else if (2 * j + (lane >> 5) < p_rows) pf_load_to_lds16(p_ksrc + 1024 * j, goff_k[j], p_lk + 1024 * j);
+    };
+    auto dma_v = [&](int j) {
+        if (__builtin_expect(p_vrows >= ROWS, 1)) pf_load_to_lds16(p_vsrc + 1024 * j, goff_v[j & 1], p_lv + 1024 * j);
+        else if (2 * j + (lane >> 5) < p_vrows) pf_load_to_lds16(p_vsrc + 1024 * j, goff_v[j & 1], p_lv + 1024 * j);
+    };
+
+    pf_f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+    // the lazy softmax reference of prefill_pp_kernel: the products start from -m_ref (the C operand)
+    pf_f32x16 negm;
+#pragma unroll
+    for (int i = 0; i < 16; i++) negm[i] = 0.0f;
+    float m_ref = 0.0f, l_run = 0.0f;
+    bool m_init = false;
+    constexpr float kLazy = 8.0f;
+
+    // where this lane finds its operands: K row n (and n + 32), chunk 2 ks + g at byte ((g ^ n & 15) << 4) ^ (ks << 5)
+    // of the row; V rows 4 g + j16 / 4 (+ multiples of 8), 8 bytes at dims 32 dt + 16 (lane / 16 % 2) + 4 (j16 % 4)
+    const uint32_t kx1 = (uint32_t)(n * RB + ((g ^ (n & 15)) << 4));
+    uint32_t vx1;
+    {
+        const int j16 = lane & 15;
+        const int rowl = 4 * g + (j16 >> 2);
+        const int clane = 2 * ((lane >> 4) & 1) + ((j16 & 3) >> 1), half = j16 & 1;
+        vx1 = (uint32_t)(rowl * RB + (((rowl & 3) << 6) | (clane << 4)) + (half << 3));
+    }
+
+    // S^T = K Q^T for the tile in buffer `slot`; between(ks): the caller's vector work for that k-step
+    auto qk = [&](int slot, pf_f32x16 (&s)[2], auto &&between) {
+        const uint32_t ka0 = pf_lds_addr(&k_ldsd[0][0]) + ((uint32_t)slot << 15) + kx1;
+        uint4 a[NKS][2];
+#pragma unroll
+        for (int ks = 0; ks < XQ; ks++) {
+            a[ks][0] = pf_lds_read128(ka0 ^ (uint32_t)(ks << 5), 0);
+            a[ks][1] = pf_lds_read128(ka0 ^ (uint32_t)(ks << 5), 32 * RB);
+        }
+        pf_sched_barrier();
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            if (ks + XQ < NKS) {
+                a[ks + XQ][0] = pf_lds_read128(ka0 ^ (uint32_t)((ks + XQ) << 5), 0);
+                a[ks + XQ][1] = pf_lds_read128(ka0 ^ (uint32_t)((ks + XQ) << 5), 32 * RB);
+            }
+            between(ks);
+            if (ks == 0) {
+                s[0] = mfma32<DT>(a[ks][0], qf[ks], negm);
+                s[1] = mfma32<DT>(a[ks][1], qf[ks], negm);
+            } else {
+                s[0] = mfma32<DT>(a[ks][0], qf[ks], s[0]);
+                s[1] = mfma32<DT>(a[ks][1], qf[ks], s[1]);
+            }
+            pf_sched_barrier();
+        }
+    };
+    // O^T += V^T P^T over the tile in buffer `slot`: 32 products, two transposed 8-byte reads each, four products ahead
+    auto pv = [&](int slot, const uint4 (&pb)[2][2], auto &&between) {
+        const uint32_t vb = pf_lds_addr(&v_ldsd[0][0]) + ((uint32_t)slot << 15) + vx1;
+        constexpr int NP = 4 * NDT;
+        uint2 lo[NP], hi[NP];
+        auto rd = [&](int i) {                               // product i = (tt, mh, dt) = (i / 16, (i / 8) & 1, i % 8)
+            const int roff = ((i / (2 * NDT)) * 32 + 16 * ((i / NDT) & 1)) * RB;
+            const uint32_t va = vb ^ (uint32_t)((i % NDT) << 6);
+            lo[i] = pf_lds_read_tr16(va, roff);
+            hi[i] = pf_lds_read_tr16(va, roff + 8 * RB);
+        };
+#pragma unroll
+        for (int i = 0; i < XP; i++) rd(i);
+        pf_sched_barrier();
+#pragma unroll
+        for (int i = 0; i < NP; i++) {
+            if (i + XP < NP) rd(i + XP);
+            between(i);
+            o[i % NDT] = mfma32<DT>(make_uint4(lo[i].x, lo[i].y, hi[i].x, hi[i].y), pb[i / (2 * NDT)][(i / NDT) & 1], o[i % NDT]);
+            pf_sched_barrier();
+        }
+    };
+
+    // ---- prologue: the buffers cleared; K(0), V(0), K(1) in LDS; the scores of tile 0 ----
+    for (int i = threadIdx.x * 16; i < 2 * kTileBytes; i += 256 * 16) {
+        *(uint4 *)(&k_ldsd[0][0] + i) = make_uint4(0, 0, 0, 0);
+        *(uint4 *)(&v_ldsd[0][0] + i) = make_uint4(0, 0, 0, 0);
+    }
+    int blk_ahead;                                           // the wave's page two tiles ahead of the step
+    {
+        const int b0 = page_of(0), b1 = page_of(1);
+        blk_ahead = page_of(2);
+        __syncthreads();                                     // the clearing is done (and the table entries are here)
+        plan(0, b0);
+#pragma unroll
+        for (int j = 0; j < 8; j++) dma_k(j);
+        plan(1, b1);                                         // K(1), V(0)
+#pragma unroll
+        for (int j = 0; j < 8; j++) { dma_k(j); dma_v(j); }
+        wait_loads();
+    }
+    __syncthreads();
+    pf_f32x16 s_even[2], s_odd[2];
+    qk(0, s_even, [](int) {});
+
+    auto tile_step = [&](int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
+        // here: s = scores of tile it; every wave's requests of the step before are on their way or there
+        plan(it + 2, blk_ahead);                             // K(it + 2), V(it + 1): requested between the products below
+        blk_ahead = page_of(it + 3);
+        const int tile_t = it * kPfBN;
+        const int *vl = &valid_ldsd[it & 3][0];
+        const int flags = vl[0] | (vl[1] << 1) | (vl[2] << 2) | (vl[3] << 3);
+        if (__builtin_expect(flags != 15 || it >= first_masked_tile, 0)) {
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    const bool ok = (tile_t + tl) < vis && ((flags >> (tl >> 4)) & 1) != 0;
+                    s[tt][i] = ok ? s[tt][i] : -INFINITY;
+                }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[tt][i]);
+        tmax = pf_max_halves(tmax);                          // a row's scores lie in lanes n and n + 32
+        const bool move = m_init ? tmax > kLazy : tmax > -INFINITY;
+        if (__builtin_expect(__any(move), 0)) {
+            const float delta = move ? tmax : 0.0f;
+            m_init = m_init || move;
+            m_ref += delta;
+            const float alpha = __builtin_amdgcn_exp2f(-delta);
+            l_run *= alpha;
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[tt][i] -= delta;
+#pragma unroll
+            for (int i = 0; i < 16; i++) negm[i] = -m_ref;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+        }
+        // the exponentials of this tile between the k-steps of the next tile's scores, two per k-step, packed as
+        // soon as eight are there; the row sum over the weights before rounding (see prefill_ppd_kernel).  The
+        // products are unconditional: past the last tile they multiply whatever that buffer holds, never read.
+        float psum = 0.0f, p8[8];
+        uint4 pb[2][2];
+        // K(it + 1) and V(it) have landed, and every wave is done with K(it) and V(it - 1), whose buffers the
+        // requests below write
+        wait_loads();
+        pf_barrier_lds();
+        qk((it + 1) & 1, s_next, [&](int ks) {
+            if ((ks & 1) == 0) dma_k(ks >> 1);
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int j = ks * 2 + u, tt = j >> 4, i = j & 15;
+                const float e = __builtin_amdgcn_exp2f(s[tt][i]);
+                p8[j & 7] = e;
+                psum += e;
+                if ((j & 7) == 7)
+                    pb[tt][(i >> 3) & 1] = make_uint4(pack2<DT>(p8[0], p8[1]), pack2<DT>(p8[2], p8[3]), pack2<DT>(p8[4], p8[5]), pack2<DT>(p8[6], p8[7]));
+            }
+        });
+        l_run += psum;
+        pv(it & 1, pb, [&](int i) { if ((i & 3) == 0) dma_v(i >> 2); });
+    };
+    for (int it = 0; it < ntiles; it += 2) {                 // two tiles per trip, the score registers swapping roles
+        tile_step(it, s_even, s_odd);
+        if (it + 1 < ntiles) tile_step(it + 1, s_odd, s_even);
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (row_live && (l_tot > 0.0f || A.gate)) {
+        const bool have = l_tot > 0.0f;
+        const float inv = have ? 1.0f / l_tot : 0.0f;
+        uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * (D * 2);
+        const uint16_t *grow = A.gate ? A.gate + ((size_t)tq * A.QH + head) * A.gate_stride : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; b4++) {
+                const int d0 = dt * 32 + 8 * b4 + 4 * g;
+                uint2 v = have ? make_uint2(pack2<IO>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
+                                            pack2<IO>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv))
+                               : *(const uint2 *)(orow + d0 * 2);
+                if (grow) {
+                    const uint2 gv = *(const uint2 *)(grow + d0);
+                    v.x = (uint32_t)gated_elem16((uint16_t)(v.x & 0xffffu), (uint16_t)(gv.x & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.x >> 16), (uint16_t)(gv.x >> 16), IO) << 16);
+                    v.y = (uint32_t)gated_elem16((uint16_t)(v.y & 0xffffu), (uint16_t)(gv.y & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.y >> 16), (uint16_t)(gv.y >> 16), IO) << 16);
+                }
+                *(uint2 *)(orow + d0 * 2) = v;
+            }
+    }
+}
+
 // ---- attention mass of a chunk ------------------------------------------------------------------
 // mass[lb] += sum over the chunk's rows (query tokens x query heads) and over the tokens of logical block lb of
 // the row's softmax probability: what each page of the context received from a perception frame (the
@@ -2278,6 +2585,14 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
             DRK_LAUNCH_CHECK("prefill_pp_kernel");
             return DRK_OK;
         }
+    }
+    // head_dim 256 on 16-bit pages: one wave per SIMD, tiles straight into LDS (same grid, same rows per workgroup)
+    if (a.D == 256 && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 && g_prefill_two_phase != 0 &&
+        g_prefill_two_phase != 3) {
+        if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_d256_kernel<DRK_BF16, DRK_BF16>), grid, dim3(256), 0, st, A);
+        else hipLaunchKernelGGL((prefill_d256_kernel<DRK_F16, DRK_F16>), grid, dim3(256), 0, st, A);
+        DRK_LAUNCH_CHECK("prefill_d256_kernel");
+        return DRK_OK;
     }
 #define DRK_PF_LAUNCH(DT, KV, IO)                                                                                        \
     do {                                                                                                                \

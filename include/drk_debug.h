@@ -52,7 +52,9 @@ void drk_debug_set_prefill_split(int max_rows);
 /* Tuning: which causal chunks of head_dim 128 run on the two-phase chunk kernels (eight waves, 256 rows per
  * workgroup): 0 = none (the four-wave kernel); 1 = the library's rule (default: chunks long enough to give
  * most CUs a workgroup); 2 = every chunk the geometry allows; 3 = as 2, and 16-bit pages too go through
- * registers on their way into LDS (the kernel 8-bit pages always use) instead of straight from global memory. */
+ * registers on their way into LDS (the kernel 8-bit pages always use) instead of straight from global memory.
+ * Head_dim 256 on 16-bit pages: 1 and 2 = the direct-to-LDS kernel with one wave per SIMD, 0 and 3 = the four-wave
+ * kernel that stages through registers. */
 void drk_debug_set_prefill_two_phase(int mode);
 /* Tuning: 16-byte chunks one workgroup moves per (layer, K|V) in the copying append, in
  * extract / inject, and in the quantising append (0 = default: 256, 512, 1024). */

@@ -18,7 +18,8 @@ def chunk_kernel(request):
     """Every case runs three times: with the library's own choice of chunk kernel, with the two-phase
     kernels taken wherever their geometry allows (head_dim 128, blocks of 16 * 2^k tokens; 16-bit pages go
     from global memory straight into LDS, 8-bit pages through registers), and with the register kind for
-    16-bit pages too, whatever the chunk's length."""
+    16-bit pages too, whatever the chunk's length.  Head_dim 256 on 16-bit pages takes its own direct-to-LDS kernel
+    in the first two runs and the register-staging kernel in the third."""
     lib = cabi.lib()
     lib.drk_debug_set_prefill_two_phase({"by_rule": 1, "two_phase": 2, "two_phase_through_registers": 3}[request.param])
     yield request.param
@@ -257,6 +258,32 @@ def test_ring_of_tiles_wraps_over_holes_and_ragged_ends(dev, chunk_kernel, dtype
     holes = tuple(h for h in holes if h < nblk)
     geom = (2, KVH, KVH * G, D, bs, nblk + 3)
     g, og, rng, table, opool = build(geom, dtype, total, seed=bs * 1000 + G, holes=holes, mul=0.7)
+    q = U.normal_bits(rng, (M, KVH * G, D), dtype, 0.7)
+    scale = 1 / np.sqrt(D)
+    got = run_prefill(g, U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table), 1, pos_start, M, scale, dtype, KVH * G, D)
+    want = orc.prefill_f64(og, q, opool, table, 1, pos_start, scale, dtype)
+    seen = np.array([any(table[t // bs] >= 0 for t in range(pos_start + r + 1)) for r in range(M)])
+    assert np.all(got[~seen].view(np.uint8) == 0x7B)
+    ok, ma, _ = U.rel_abs_ok(U.from_bits(got[seen], dtype), want[seen])
+    assert ok, f"max abs err {ma:.4g} ({chunk_kernel=} {bs=} {G=} {pos_start=} {M=} {holes=})"
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
+@pytest.mark.parametrize("bs,G,pos_start,M,holes", [
+    (256, 6, 900, 257, (1,)), (16, 2, 0, 300, (3, 4, 5, 6, 17)), (64, 6, 1500, 100, (20,)), (32, 1, 33, 130, ()),
+    (128, 12, 2047, 22, (0,)), (16, 6, 640, 64, (40, 43))])
+def test_head_dim_256_over_holes_and_ragged_ends(dev, chunk_kernel, dtype, bs, G, pos_start, M, holes):
+    """16-bit pages with head_dim 256 (the reference model's: 24 query over 4 kv heads, blocks of 256 tokens) on the
+    kernel that loads tiles straight into LDS with one wave per SIMD (the first two runs of this case; the third takes
+    the register-staging kernel): walks of up to 35 tiles over missing pages, chunk ends inside a page and inside a
+    tile, query tiles of 21, 64, 128, 10 tokens.  Rows behind holes only keep the caller's bytes; everything else
+    against fp64 on the stored values."""
+    KVH, D = 2, 256
+    total = pos_start + M
+    nblk = (total + bs - 1) // bs
+    holes = tuple(h for h in holes if h < nblk)
+    geom = (2, KVH, KVH * G, D, bs, nblk + 3)
+    g, og, rng, table, opool = build(geom, dtype, total, seed=bs * 1000 + G + 7, holes=holes, mul=0.7)
     q = U.normal_bits(rng, (M, KVH * G, D), dtype, 0.7)
     scale = 1 / np.sqrt(D)
     got = run_prefill(g, U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table), 1, pos_start, M, scale, dtype, KVH * G, D)
