@@ -4,7 +4,7 @@
 Workload (BASELINE config 2): 36 layers, 32 Q / 8 KV heads x 128, bf16 KV in
 16-token pages shuffled across a 40 GB pool, 8 decode branches at 32k context.
 One step = for every layer: append one token per branch, then paged GQA decode
-attention over all branches.  Prints ONE JSON line (see README / DESIGN).
+attention over all branches.  Prints ONE JSON line.
 
 Torch is used for device memory, streams and events only; every kernel is
 reached through the C ABI in include/drk_kv.h.
@@ -86,8 +86,7 @@ def parse():
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (sharding across GPUs is "
-              "described in DESIGN.md, not implemented)", file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (nothing here shards across GPUs)", file=sys.stderr)
         sys.exit(2)
     import torch
     from deusridet_amd import cabi
