@@ -152,7 +152,13 @@ __device__ __forceinline__ void pf_barrier_lds()
 }
 // 16 bytes per lane from global memory straight into LDS: lane i's land at lds_addr + 16 i (lds_addr is the same
 // for the whole wave).  Written as assembly so that the compiler does not know of the store into LDS: it would
-// wait for every outstanding load ahead of the next LDS read.  The caller counts the loads (pf_async_wait).
+// wait for every outstanding load ahead of the next LDS read.  The caller counts the loads (s_waitcnt vmcnt).
+// The LDS address travels in M0, which the compiler reserves for instructions of its own that need it (indirect
+// register indexing, its own direct loads) and loads right before each of them; the kernels that call this have
+// none of those -- their arrays are indexed by constants after unrolling -- so nothing else reads M0, and the
+// compiler's remark about the clobber is switched off here.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void pf_load_to_lds16(const void *base, uint32_t lane_offset, uint32_t lds_addr)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -161,6 +167,7 @@ __device__ __forceinline__ void pf_load_to_lds16(const void *base, uint32_t lane
     (void)base; (void)lane_offset; (void)lds_addr;
 #endif
 }
+#pragma clang diagnostic pop
 
 struct PrefillArgs {
     const uint8_t *pool_layer;    // pool + layer * layer_stride
