@@ -1388,8 +1388,8 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
 // run two k-steps / four products ahead, scheduling barriers pin it.  Per tile and wave 64 products (2 048 clocks).
 // Requests run one tile ahead, two buffers per operand, one barrier per tile: step t first takes the maximum of tile
 // t's scores (registers only), then waits for its requests of the step before and meets the other waves, then
-// requests K(t + 2) and V(t + 1) -- into the buffers of K(t) and V(t - 1) -- one request every four products of
-// QK(t + 1) and PV(t).
+// requests K(t + 2) and V(t + 1) -- into the buffers of K(t) and V(t - 1) -- one request per k-step of QK(t + 1)
+// (between the transposed reads of PV a request holds the wave up for over a hundred clocks).
 template <int DT, int IO = DT>
 __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
 {
@@ -1454,10 +1454,15 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
         for (int j = 0; j < 2; j++) goff_v[j] = (uint32_t)(rr * RB + ((cp ^ (((2 * j + rr) & 3) << 2)) << 4));
     }
     auto wait_loads = [&]() { __builtin_amdgcn_s_waitcnt(0x0f70); };         // vmcnt(0): every request has landed
-    // the wave's page in `tile`, or -1; a vector load (a scalar one would share its counter with the LDS reads)
+    // the wave's page in `tile`, or -1.  Read through the scalar cache (the table is not written while the kernel
+    // runs): a vector load would be waited for together with the requests, which the kernel counts itself.  The
+    // step makes sure the entry is there before its products begin -- scalar loads return out of order, and with
+    // one outstanding the compiler could not count the LDS reads it waits for.
+    typedef const int32_t __attribute__((address_space(4))) *const_table_t;
+    const const_table_t table_k = (const_table_t)(uintptr_t)A.table;
     auto page_of = [&](int tile) -> int {
         const int tg = tile * kPfBN + tgw;
-        return tg < lim_wg ? A.table[tg >> sh] : -1;
+        return tg < lim_wg ? table_k[tg >> sh] : -1;
     };
     const uint8_t *vsrc_prev = kbase;                        // where the V rows of the tile requested last begin
     int rows_prev = 0;                                       // how many of them exist
@@ -1639,8 +1644,10 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
         // requests below write
         wait_loads();
         pf_barrier_lds();
-        qk((it + 1) & 1, s_next, [&](int ks) {
+        asm volatile("" : : "s"(blk_ahead));                 // the table entry read at the head of the step is here
+        qk((it + 1) & 1, s_next, [&](int ks) {               // all 16 requests between the k-steps: there they cost nothing
             if ((ks & 1) == 0) dma_k(ks >> 1);
+            else dma_v(ks >> 1);
 #pragma unroll
             for (int u = 0; u < 2; u++) {
                 const int j = ks * 2 + u, tt = j >> 4, i = j & 15;
@@ -1652,7 +1659,7 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
             }
         });
         l_run += psum;
-        pv(it & 1, pb, [&](int i) { if ((i & 3) == 0) dma_v(i >> 2); });
+        pv(it & 1, pb, [](int) {});
     };
     for (int it = 0; it < ntiles; it += 2) {                 // two tiles per trip, the score registers swapping roles
         tile_step(it, s_even, s_odd);
