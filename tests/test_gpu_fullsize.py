@@ -217,6 +217,53 @@ def test_config5_full_chunk_prefill_rows(dev):
     assert ok, ma
 
 
+def test_reference_model_shape_full_chunk_prefill_rows(dev):
+    """The reference model's head shape (24 query over 4 kv heads x 256, blocks of 256 tokens, fp16): a 2 048-token chunk at
+    position 30 720, sampled rows (first and last of a 21-token query tile among them) against fp32 causal attention in
+    torch over the stored K and V, for the direct-to-LDS kernel (the library's choice) and the register-staging one."""
+    torch = _torch()
+    L, KVH, QH, D, bs = 1, 4, 24, 256, 256
+    total, M = 32768, 2048
+    pos_start = total - M
+    NB = total // bs
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.F16)
+    lib = cabi.lib()
+    rng = np.random.default_rng(7)
+    table = torch.from_numpy(rng.permutation(NB).astype(np.int32)).cuda()
+    pool = torch.zeros(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    sp = U.stream_ptr()
+    for p0 in range(0, total, 8192):
+        k = (torch.randn(8192, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.float16)
+        v = (torch.randn(8192, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.float16)
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(table), 0, 1, p0, 8192, U.p(k), U.p(v), cabi.F16, sp)
+        U.sync()
+    q = (torch.randn(M, QH, D, device="cuda", generator=gen) * 0.5).to(torch.float16)
+    scale = 1 / np.sqrt(D)
+    rows = [0, 1, 20, 21, 1000, 2046, 2047]
+    flat = torch.empty(2 * total * KVH * D, dtype=torch.float16, device="cuda")
+    cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(pool), U.p(table), 0, total, 1, sp)
+    U.sync()
+    kv = flat.view(2, total, KVH, D).float()
+    want = torch.empty(len(rows), QH, D, dtype=torch.float32, device="cuda")
+    for i, tq in enumerate(rows):
+        n = pos_start + tq + 1
+        s = torch.einsum("hgd,thd->hgt", q[tq].float().view(KVH, QH // KVH, D), kv[0, :n]) * scale
+        want[i] = torch.einsum("hgt,thd->hgd", torch.softmax(s, dim=-1), kv[1, :n]).reshape(QH, D)
+    want = want.cpu().numpy()
+    for mode in (1, 3):
+        lib.drk_debug_set_prefill_two_phase(mode)
+        try:
+            out = torch.zeros_like(q)
+            cabi.call("drk_paged_prefill_attention", C.byref(g), U.p(q), U.p(pool), U.p(table), U.p(out), 0, pos_start, M,
+                      float(scale), cabi.F16, None, 0, sp)
+            U.sync()
+        finally:
+            lib.drk_debug_set_prefill_two_phase(1)
+        ok, ma, _ = U.rel_abs_ok(out[rows].float().cpu().numpy(), want)
+        assert ok, (mode, ma)
+
+
 @pytest.mark.parametrize("dtype", [cabi.BF16, cabi.INT8])
 def test_pages_beyond_4GiB_of_a_layer(dev, dtype):
     """A pool whose single layer holds more than 4 GiB (a 288 GB part at 36 layers has 7 GiB per
