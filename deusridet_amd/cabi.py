@@ -32,8 +32,22 @@ def layout(L, KVH, QH, D, bs, NB, dtype):
     return Layout(L, KVH, QH, D, bs, NB, dtype, 0)
 
 
+class PrefixGroup(C.Structure):
+    """drk_prefix_group: branches [first_branch, +n_branches) hold tokens [tok_begin, tok_end) in the same pages"""
+    _fields_ = [(n, C.c_int32) for n in ("first_branch", "n_branches", "tok_begin", "tok_end")]
+
+
+def prefix_groups(groups):
+    """ctypes array of drk_prefix_group from (first_branch, n_branches, tok_begin, tok_end) tuples"""
+    arr = (PrefixGroup * max(len(groups), 1))()
+    for i, gr in enumerate(groups):
+        arr[i] = PrefixGroup(*[int(x) for x in gr])
+    return arr
+
+
 _vp, _i32, _sz, _f32 = C.c_void_p, C.c_int32, C.c_size_t, C.c_float
 _LP = C.POINTER(Layout)
+_GP = C.POINTER(PrefixGroup)
 
 # name -> (restype, argtypes); mirrors include/drk_kv.h and include/drk_debug.h one to one
 SIGNATURES = {
@@ -113,6 +127,11 @@ SIGNATURES = {
     "drk_decode_shared_workspace_bytes": (_sz, [_LP, _i32, _i32, _i32]),
     "drk_paged_decode_attention_shared": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _i32, _f32,
                                                  _i32, _vp, _sz, _vp]),
+    "drk_decode_grouped_workspace_bytes": (_sz, [_LP, _i32, _i32, _GP, _i32]),
+    "drk_decode_grouped_workspace_bytes_max": (_sz, [_LP, _i32, _i32, _i32]),
+    "drk_paged_decode_attention_grouped": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _GP, _i32, _vp, _i32, _f32,
+                                                  _i32, _vp, _sz, _vp, _sz, _vp]),
+    "drk_debug_set_grouped_decode": (None, [_i32]),
     "drk_prefill_workspace_bytes": (_sz, [_LP, _i32, _i32]),
     "drk_paged_prefill_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
     "drk_rope_table_fill": (_i32, [_vp, _i32, _i32, _f32, _vp]),

@@ -89,6 +89,15 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
                          int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, int shared_tokens,
                          void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
                          void *stream, const void *gate = nullptr, size_t gate_stride = 0);
+// branches that share pages as a tree: one launch over shared and private tiles (drk_decode_group.hip)
+extern int g_grouped_mode;
+bool grouped_decode_supported(const Lay &a, int B);
+size_t grouped_workspace_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups);
+size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_depth);
+int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables, int table_stride,
+                          const int32_t *d_seq_lens, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups,
+                          void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
+                          void *stream, const void *gate = nullptr, size_t gate_stride = 0);
 // shared-prefix pass on the matrix cores (drk_prefill.hip)
 void shared_prefix_shape(const Lay &a, int B, int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,

@@ -643,6 +643,12 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
     if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
         return fail(DRK_ERR_INVALID, "decode: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "decode: layer %d outside [0,%d)", layer, a.L);
+    // one prefix for all branches is the simplest tree: shared and private tiles in one launch
+    if (grouped_decode_supported(a, B) && B * (a.QH / a.KVH) <= 64) {
+        const drk_prefix_group all = {0, B, 0, shared};
+        return launch_decode_grouped(g, q, pool, tables, table_stride, d_seq_lens, B, max_seq_len, &all, 1, out, layer, scale,
+                                     io_dtype, workspace, workspace_bytes, stream, gate, gate_stride);
+    }
     size_t sp;
     const size_t need = shared_need(a, B, max_seq_len, shared, &sp, true);
     if (!workspace || workspace_bytes < need)
@@ -754,6 +760,10 @@ size_t drk_decode_shared_workspace_bytes(const drk_kv_layout *g, int B, int max_
     if (stream_decode_supported(a, B) && shared >= kTile) {
         size_t s2 = shared_need(a, B, max_seq_len, shared, nullptr, false);
         if (s2 > need) need = s2;
+        if (a.D == 128 && B * (a.QH / a.KVH) <= 64) {        // the grouped kernel may take the call
+            s2 = grouped_workspace_need_max(a, B, max_seq_len, 1);
+            if (s2 > need) need = s2;
+        }
     }
     return need;
 }

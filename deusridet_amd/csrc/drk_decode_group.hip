@@ -1,0 +1,897 @@
+// drk_decode_group.hip -- paged GQA decode for branches that share pages: one persistent,
+// stream-K style launch over shared and private tiles alike.
+//
+// Decode branches forked copy-on-write from one context hold the same physical pages for
+// the tokens before their fork points: a tree of shared ranges ("groups": branches
+// [first, first + count) hold tokens [begin, end) in the same pages) with a private tail
+// per branch behind it.  A shared range is streamed from HBM once for all its branches:
+// the unit of work is, as in decode_stream_kernel, one 64-token tile of one kv head, and
+// a tile of a shared range serves up to 64 query rows (branches x query heads of the kv
+// head, in row groups of 16 = one matrix-core operand each) where a private tile serves
+// the one branch's heads.  Units are numbered groups first (kv head, then tile), then the
+// tails (branch, kv head, tile); workgroup g owns the run [g*U, (g+1)*U), so every
+// workgroup streams the same number of bytes whatever the shape of the tree is, the grid is
+// resident in one round, and shared and private tiles are in flight side by side.
+//
+// Per wave and tile (the wave owns 16 of the tile's 64 tokens, as in the stream kernel):
+//   K rows through the wave's LDS region into the A operand, once for all row groups;
+//   per row group: S = K Q^T (Q from LDS, loaded once per segment), softmax state of its
+//   own, P packed in place; V operands by byte permutes, once; per row group O += P V.
+// A segment (the run's tiles of one kv head of one group or tail) ends with the four waves'
+// states folded through LDS, 16 rows per round, and (o, m, l) per query row left in the
+// workspace slot of this piece; group_merge_kernel folds a row's pieces -- those of every
+// group the branch belongs to and those of its tail.
+#include "drk_stream_tile.hpp"
+
+#include <type_traits>
+#include <stdlib.h>
+
+namespace drk {
+
+int g_grouped_mode = 0;                        // diagnostic: 0 auto, 1 never (the prefix pass + tail kernel pair), see drk_debug.h
+
+constexpr int kGMaxGroups = DRK_MAX_PREFIX_GROUPS;
+constexpr int kGMaxUnits = 128;                // 64-token tiles one workgroup may own (descriptor table in LDS)
+constexpr int kGMaxPieces = 2048;              // pieces the merge folds for one query row
+constexpr int kGWgs = 512;                     // two workgroups per CU of a 256-CU part: all that fit
+
+struct GSeg {                                  // one shared range, in tiles
+    int first, count;                          // branches [first, first + count)
+    int tile0, ntile;                          // tiles [tile0, tile0 + ntile)
+    int slot;                                  // first workspace slot of its pieces in each of its rows
+    int unit0;                                 // its first unit: kv head h's tiles are units [unit0 + h*ntile, +ntile)
+};
+
+struct GroupedArgs {
+    const uint8_t *pool_layer;                 // pool + layer * layer_stride
+    const int32_t *tables;
+    const int32_t *seq_lens;                   // [B], on the device
+    const uint8_t *q;
+    float *part_o, *part_m, *part_l;
+    int table_stride, B, KVH, QH, NB, bs, bs_shift, io_dtype;
+    int Ptot;                                  // workspace slots per (branch, q head)
+    int ngroups, group_units;                  // units of all groups together
+    unsigned head_stride, kv_plane, block_stride, scale_plane, row_bytes;
+    float scale_log2e;
+    int dbg;
+    GSeg seg[kGMaxGroups];
+    int b_start[64];                           // first tile of each branch's private tail
+    int b_slot[64];                            // first workspace slot of the tail's pieces
+};
+
+struct GUnit {                                 // one 64-token tile of one kv head of a group or a tail
+    int tile_lim;                              // tokens of the tile that exist for every row (may exceed 64)
+    int flags;                                 // bit 0: first tile of a segment of this workgroup, bit 1: last; bits 8..15: query rows
+    int row0;                                  // first_branch*QH + kvh*(QH/KVH): query row R is row0 + (R / GQ)*QH + R % GQ
+    int slot;                                  // workspace slot of the segment's piece in each of its rows
+};
+
+// Reductions over the four lane groups (lanes c, c + 16, c + 32, c + 48) with the row swaps of gfx950:
+// no trip through LDS.
+__device__ __forceinline__ float max_lane_groups(float x)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+#endif
+    return x;
+}
+__device__ __forceinline__ float sum_lane_groups(float x)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(b[0]) + __uint_as_float(b[1]);
+#endif
+    return x;
+}
+
+// Maximum of the four scores a lane holds, read straight out of the matrix cores' result registers.  Written as
+// assembly to spare the canonicalising copy the compiler puts in front of every fmaxf of a value it has not
+// produced with a vector instruction -- but the compiler does not look into assembly for the wait states a read of
+// a matrix result needs behind the product that writes it (it pads its own reads with s_nop), so they are here:
+// without them the maximum is taken of what the registers held before.
+__device__ __forceinline__ float max4_of_product(float a, float b, float c, float d)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    float r;
+    asm volatile("s_nop 7\n\ts_nop 7\n\tv_max3_f32 %0, %1, %2, %3\n\tv_max3_f32 %0, %0, %4, %4" : "=&v"(r) : "v"(a), "v"(b), "v"(c), "v"(d));
+    return r;
+#else
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+#endif
+}
+
+// how far (in bits of the exponent) a row's maximum may run ahead of the reference its weights are taken to
+constexpr float kLazy = 5.0f;
+
+template <int DT, int D, int NG, bool DMA>
+__global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
+{
+    using Geo = StreamGeo<DT, D>;
+    [[maybe_unused]] constexpr bool Q8 = Geo::q8;
+    constexpr int DOT = KvTraits<DT>::dot;
+    constexpr uint32_t kNone = 0xffffffffu;
+    constexpr int QP = D * 2 + 16;                               // LDS pitch of a query row (16-bit values)
+    constexpr int NR = NG * 16;                                  // query rows a unit may serve
+    constexpr int CPR = D * 2 / 16;                              // 16-byte chunks per query row
+    constexpr int RPP = 256 / CPR;                               // rows the workgroup moves per pass
+    constexpr int QPASS = NR / RPP;
+    // K of 16-bit pages goes from global memory straight into LDS (no registers hold it): two buffers of a wave's
+    // 16 token rows, unpadded, 16-byte chunk x of row r at position x ^ r -- applied on the global side by the lane
+    // that fills the position, undone by the reader.  8-bit codes pass through registers (they are widened on the
+    // way) into one buffer of padded rows.
+    constexpr bool DIRECT = DMA && !Q8;
+    constexpr int KBUF = DIRECT ? 16 * D * 2 : 16 * Geo::PITCH;  // one wave's K rows of one tile
+    __shared__ __align__(256) uint8_t k_lds[DIRECT ? 2 : 1][4][KBUF];
+    __shared__ __align__(16) uint8_t q_lds[NR * QP];
+    __shared__ __align__(16) float o_lds[4][8][D];               // [wave][row of the round][dim], segment ends only
+    __shared__ float mw_lds[4][NR], lw_lds[4][NR];
+    __shared__ __align__(16) GUnit udesc[kGMaxUnits];
+    __shared__ __align__(16) uint2 gdesc[kGMaxUnits][4];
+    __shared__ int s_incl[64], s_len[64], s_gmin[kGMaxGroups];
+
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int g = lane >> 4, c = lane & 15;
+    const int GQ = A.QH / A.KVH;
+    // ---- the workgroup's run of units and one descriptor per unit ---------------------
+    const int len_i = lane < A.B ? A.seq_lens[lane] : 0;
+    const int nt_i = len_i > 0 ? max((len_i + kSTile - 1) / kSTile - A.b_start[lane], 0) : 0;
+    int incl = nt_i;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int t = __shfl_up(incl, off);
+        if (lane >= off) incl += t;
+    }
+    const int T = A.group_units + __builtin_amdgcn_readlane(incl, 63) * A.KVH;
+    if (T == 0) return;
+    const int U = (T + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int u0 = (int)blockIdx.x * U;
+    if (u0 >= T) return;
+    // the host sizes the grid from max_seq_len; lengths on the device beyond that bound must not overrun
+    // the descriptor table (the tiles past it are then left out: the caller broke its promise)
+    const int nunits = min(min(U, T - u0), kGMaxUnits);
+    if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
+    __syncthreads();
+    if ((int)threadIdx.x < A.ngroups) {
+        // a shared tile is visible to all its rows: no further than the shortest member reaches
+        const GSeg sg = A.seg[threadIdx.x];
+        int mn = 0x7fffffff;
+        for (int i = 0; i < sg.count; i++) mn = min(mn, s_len[sg.first + i]);
+        s_gmin[threadIdx.x] = max(mn, 0);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nunits * 4; i += 256) {
+        const int ui = i >> 2, grp = i & 3, u = u0 + ui;
+        int b, kvh, trel, nt, tile, len, nrows, slot0, run0;
+        if (u < A.group_units) {
+            int gi = 0;
+            while (gi + 1 < A.ngroups && A.seg[gi + 1].unit0 <= u) gi++;
+            const GSeg sg = A.seg[gi];
+            const int rem = u - sg.unit0;
+            nt = sg.ntile; kvh = rem / nt; trel = rem - kvh * nt;
+            tile = sg.tile0 + trel; b = sg.first; len = s_gmin[gi]; nrows = sg.count * GQ;
+            slot0 = sg.slot; run0 = sg.unit0 + kvh * nt;
+        } else {
+            const int v = u - A.group_units;
+            int lo = 0, hi = A.B - 1;                              // first branch whose cumulative units exceed v
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (A.KVH * s_incl[mid] > v) hi = mid; else lo = mid + 1;
+            }
+            b = lo;
+            const int excl = b ? s_incl[b - 1] : 0;
+            nt = s_incl[b] - excl; len = s_len[b];
+            const int rem = v - A.KVH * excl;
+            kvh = rem / nt; trel = rem - kvh * nt;
+            tile = trel + A.b_start[b]; nrows = GQ;
+            slot0 = A.b_slot[b]; run0 = A.group_units + A.KVH * excl + kvh * nt;
+        }
+        const int tg = tile * kSTile + grp * 16;
+        uint2 gd = make_uint2(kNone, 0u);
+        if (tg < len) {
+            const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
+            const int blk = A.tables[(size_t)b * A.table_stride + lb];
+            if (blk >= 0 && blk < A.NB) {
+                // every term is a multiple of 16 bytes (pp is a multiple of 16, plane sizes of 16 * 16)
+                const unsigned pp = (unsigned)(tg - lb * A.bs);
+                const size_t base = (size_t)blk * A.block_stride;
+                gd.x = (unsigned)((base + (size_t)kvh * A.head_stride + (size_t)pp * A.row_bytes) >> 4);
+                gd.y = (unsigned)((base + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + pp) * 2) >> 4);
+            }
+        }
+        gdesc[ui][grp] = gd;
+        if (grp == 0) {
+            GUnit d;
+            d.tile_lim = len - tile * kSTile;
+            d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0) | (nrows << 8);
+            d.row0 = b * A.QH + kvh * GQ;
+            d.slot = slot0 + ((int)blockIdx.x - run0 / U);
+            udesc[ui] = d;
+        }
+    }
+    __syncthreads();
+
+    // the 4 K scales and the 4 V scales of tokens 4g..4g+3 (int8 pages)
+    auto load_scales = [&](uint2 gd, uint2 &ks, uint2 &vs) {
+        if (DT != DRK_INT8) return;
+        const uint8_t *p = A.pool_layer + ((size_t)(gd.x == kNone ? 0u : gd.y) << 4) + g * 8;
+        ks = *(const uint2 *)p;
+        vs = *(const uint2 *)(p + A.scale_plane);
+    };
+    // A segment's query rows: requested into registers (the segment before is still being folded),
+    // then stored to LDS as the 16-bit type the products run in; rows past the segment's are zeros.
+    const int qr = (int)threadIdx.x / CPR, qc = (int)threadIdx.x % CPR;
+    auto q_issue = [&](const GUnit &d, uint4 (&qn)[QPASS]) {
+        const int nrows = (d.flags >> 8) & 0xff;
+#pragma unroll
+        for (int i = 0; i < QPASS; i++) {
+            const int R = i * RPP + qr;
+            qn[i] = make_uint4(0u, 0u, 0u, 0u);
+            if (R < nrows) {
+                const int bl = R / GQ, hd = R - bl * GQ;
+                qn[i] = *(const uint4 *)(A.q + (size_t)(d.row0 + bl * A.QH + hd) * (D * 2) + qc * 16);
+            }
+        }
+    };
+    // (times scale * log2 e, rounded to the 16-bit type once: a product then arrives as its exponent)
+    auto scaled16 = [&](uint32_t v) -> uint32_t {
+        float lo, hi;
+        if (A.io_dtype == DRK_BF16) { lo = bf16_lo(v); hi = bf16_hi(v); }
+        else { lo = f16_bits_to_f((uint16_t)(v & 0xffffu)); hi = f16_bits_to_f((uint16_t)(v >> 16)); }
+        lo *= A.scale_log2e; hi *= A.scale_log2e;
+        if constexpr (DOT == DRK_BF16) return (uint32_t)f_to_bf16_bits(lo) | ((uint32_t)f_to_bf16_bits(hi) << 16);
+        else return (uint32_t)__half_as_ushort(__float2half_rn(lo)) | ((uint32_t)__half_as_ushort(__float2half_rn(hi)) << 16);
+    };
+    auto q_store = [&](uint4 (&qn)[QPASS]) {
+#pragma unroll
+        for (int i = 0; i < QPASS; i++) {
+            uint4 v = qn[i];
+            v.x = scaled16(v.x); v.y = scaled16(v.y); v.z = scaled16(v.z); v.w = scaled16(v.w);
+            *(uint4 *)(q_lds + (i * RPP + qr) * QP + qc * 16) = v;
+        }
+    };
+    // Q^T as the B operand of row group rg: lane (row c of the group, dims 32 kk + 8 g ..)
+    auto q_operand = [&](int rg, int kk) -> uint4 { return *(const uint4 *)(q_lds + (rg * 16 + c) * QP + kk * 64 + g * 16); };
+
+    w_f32x4 o[NG][Geo::NPV];
+    float m_run[NG], l_lane[NG], ps_lane[NG], qbias[NG];
+#pragma unroll
+    for (int rg = 0; rg < NG; rg++) {
+#pragma unroll
+        for (int e = 0; e < Geo::NPV; e++) o[rg][e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        m_run[rg] = -INFINITY; l_lane[rg] = 0.0f; ps_lane[rg] = 0.0f; qbias[rg] = 0.0f;
+    }
+    // int8 pages: the sum of every row's query values, for the code offset
+    auto q_bias = [&]() {
+        if (DT != DRK_INT8) return;
+#pragma unroll
+        for (int rg = 0; rg < NG; rg++) {
+            float sq = 0.0f;
+#pragma unroll
+            for (int kk = 0; kk < Geo::NQK; kk++) {
+                const uint4 v = q_operand(rg, kk);
+                sq = s_dot2<DOT>(v.x, kF16Ones, sq);
+                sq = s_dot2<DOT>(v.y, kF16Ones, sq);
+                sq = s_dot2<DOT>(v.z, kF16Ones, sq);
+                sq = s_dot2<DOT>(v.w, kF16Ones, sq);
+            }
+            qbias[rg] = kI8Bias * sum_lane_groups(sq);
+        }
+    };
+
+    // K of a unit on its way into the wave's LDS buffer `buf`: four direct loads of 64 x 16 bytes; lane l of load j
+    // fills position l % 16 of row 4j + l / 16 with the row's chunk (l % 16) ^ row
+    // (row r = 4j + l / 16 and l / 16 < 4, so the chunk is ((l % 16) ^ (l / 16)) ^ 4j: load j's offset is load 0's
+    // with j xor-ed into bits 6-7, plus 1024 j)
+    const uint32_t kdma_row = (uint32_t)((lane >> 4) * (D * 2)), kdma_x = (uint32_t)(((lane & 15) ^ (lane >> 4)) << 4);
+    static_assert(!DIRECT || D == 128, "the direct K path is laid out for 256-byte rows");
+    auto k_request = [&](uint32_t off, int buf) {
+        if constexpr (DIRECT) {
+            const uint8_t *base = A.pool_layer + ((size_t)(off == kNone ? 0u : off) << 4);     // uniform: one run per wave
+            const uint32_t lds = lds_addr32(&k_lds[DIRECT ? buf : 0][w][0]);
+            uint32_t kx = kdma_x;
+#if defined(__HIP_DEVICE_COMPILE__)
+            asm volatile("" : "+v"(kx));                     // computed here, each time: four more registers held across the loop would spill
+#endif
+#pragma unroll
+            for (int j = 0; j < Geo::NK; j++) lds_dma16(base, (kx ^ (uint32_t)(j << 6)) + kdma_row + 1024u * j, lds + 1024 * j);
+        }
+    };
+    // V of a unit: the run's address is the same for the whole wave (scalar registers), the lane adds 32 bits
+    const uint32_t v_lane_off = (uint32_t)((lane >> 4) * (4 * Geo::RB) + (lane & 15) * (Q8 ? 8 : 16));
+    auto load_v_uniform = [&](uint32_t off) -> VRegs<DT, D> {
+        VRegs<DT, D> v;
+        const uint8_t *base = A.pool_layer + ((size_t)(off == kNone ? 0u : off) << 4) + A.kv_plane;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int ch = 0; ch < Geo::NCH; ch++) {
+                if constexpr (Q8) v.r[j][ch] = ld_stream64(base + (v_lane_off + (uint32_t)(j * Geo::RB + ch * 128)));
+                else v.r[j][ch] = ld_stream128(base + (v_lane_off + (uint32_t)(j * Geo::RB + ch * 256)));
+            }
+        return v;
+    };
+    uint2 gd = gdesc[0][w], ksr = {}, vsr = {};
+    KRegs<DT, D> kreg;
+    if constexpr (DIRECT) k_request(__builtin_amdgcn_readfirstlane(gd.x), 0);
+    else kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
+    VRegs<DT, D> vreg = load_v_uniform(__builtin_amdgcn_readfirstlane(gd.x));
+    load_scales(gd, ksr, vsr);
+    {
+        uint4 qn[QPASS];
+        q_issue(udesc[0], qn);
+        q_store(qn);
+        __syncthreads();
+        q_bias();
+    }
+
+    for (int it = 0; it < nunits; it++) {
+        const GUnit ud = udesc[it];
+        const int flags = __builtin_amdgcn_readfirstlane(ud.flags);
+        const int tile_lim = __builtin_amdgcn_readfirstlane(ud.tile_lim);
+        const int nrows = (flags >> 8) & 0xff;
+        const int nga = (nrows + 15) >> 4;                      // row groups of this unit
+        const bool hole = __builtin_amdgcn_readfirstlane((int)gd.x) == (int)kNone;   // the group the registers were loaded for
+        const int lim = hole ? 0 : tile_lim;                    // tokens of the tile this wave may look at
+        const bool has_next = it + 1 < nunits;
+        const bool partial = w * 16 + 16 > lim;                 // some of the wave's 16 tokens do not exist
+
+        // ---- K: registers -> the wave's LDS rows -> one token row per lane; V: registers -> B operands;
+        // then the loads of the next unit's K and V, so that they travel during all of this unit's arithmetic
+        if constexpr (DIRECT) vm_wait_all();                    // this unit's K has landed (its V too: requested before it)
+        if (A.dbg & 2) __builtin_amdgcn_s_sleep(8);
+        if (A.dbg & 8) __syncthreads();
+        else stage_k<DT, D>(&k_lds[0][w][0], kreg, lane);
+        float ks[4] = {1.0f, 1.0f, 1.0f, 1.0f}, vs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+        if (DT == DRK_INT8) {
+            ks[0] = f16_bits_to_f((uint16_t)(ksr.x & 0xffffu)); ks[1] = f16_bits_to_f((uint16_t)(ksr.x >> 16));
+            ks[2] = f16_bits_to_f((uint16_t)(ksr.y & 0xffffu)); ks[3] = f16_bits_to_f((uint16_t)(ksr.y >> 16));
+            vs[0] = f16_bits_to_f((uint16_t)(vsr.x & 0xffffu)); vs[1] = f16_bits_to_f((uint16_t)(vsr.x >> 16));
+            vs[2] = f16_bits_to_f((uint16_t)(vsr.y & 0xffffu)); vs[3] = f16_bits_to_f((uint16_t)(vsr.y >> 16));
+        }
+        const int t0 = w * 16 + g * 4;
+        if (DT != DRK_INT8 && partial) {                        // rows without a token may hold anything (NaN)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (t0 + j >= lim) {
+#pragma unroll
+                    for (int ch = 0; ch < Geo::NCH; ch++) vreg.r[j][ch] = {};
+                }
+        }
+        uint2 vb[Geo::NCH][8];
+#pragma unroll
+        for (int ch = 0; ch < Geo::NCH; ch++) v_operands<DT>(vreg.r[0][ch], vreg.r[1][ch], vreg.r[2][ch], vreg.r[3][ch], vb[ch]);
+        if (has_next) {
+            gd = gdesc[it + 1][w];
+            vreg = load_v_uniform(__builtin_amdgcn_readfirstlane(gd.x));
+            if constexpr (DIRECT) k_request(__builtin_amdgcn_readfirstlane(gd.x), (it + 1) & 1);
+            else kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
+            load_scales(gd, ksr, vsr);
+        }
+        if (A.dbg & 16) __builtin_amdgcn_s_sleep(20);
+        if (A.dbg & 32) vm_wait_all();
+        // the A operand: dims 32 kk + 8 g .. of token row c of the wave's 16
+        const uint8_t *const krows = &k_lds[DIRECT ? (it & 1) : 0][w][0];
+        auto k_operand = [&](int kk) -> uint4 {
+            if constexpr (DIRECT) return *(const uint4 *)(krows + c * (D * 2) + ((((g ^ c) & 15) << 4) ^ (kk << 6)) + (((kk * 4 + g) & ~15) << 4));
+            else return *(const uint4 *)(krows + c * Geo::PITCH + g * 16 + kk * 64);
+        };
+
+        // ---- scores, softmax, O += P V: for the unit's row groups (one, or all NG: a group of padding rows
+        // multiplies zeros and its state is never stored) ----------------------------------------------
+        auto tile_body = [&](auto NC) {
+            constexpr int N = decltype(NC)::value;
+            // S = K Q^T - m: the reference of row c's exponentials is the products' C operand, so a score arrives
+            // as the exponent of its weight; N independent chains, so that a product never waits for the one before
+            w_f32x4 s[N];
+#pragma unroll
+            for (int rg = 0; rg < N; rg++) {
+                const float nm = (DT == DRK_INT8 || m_run[rg] == -INFINITY) ? 0.0f : -m_run[rg];
+                s[rg] = w_f32x4{nm, nm, nm, nm};
+            }
+#pragma unroll
+            for (int kk = 0; kk < Geo::NQK; kk++) {
+                const uint4 ka = k_operand(kk);
+#pragma unroll
+                for (int rg = 0; rg < N; rg++) s[rg] = w_mfma_qk<DOT>(ka, q_operand(rg, kk), s[rg]);
+            }
+            uint2 pa[N];                                      // A operands of the second product: P[row c][tokens 4g..4g+3]
+#pragma unroll
+            for (int rg = 0; rg < N; rg++) {
+                if (DT == DRK_INT8) {                           // codes carry an offset and the token's scale
+                    const float nm = m_run[rg] == -INFINITY ? 0.0f : -m_run[rg];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) s[rg][j] = fmaf(s[rg][j] - qbias[rg], ks[j], nm);
+                }
+                if (partial) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) s[rg][j] = t0 + j < lim ? s[rg][j] : -INFINITY;
+                }
+                // row c's maximum over this wave's 16 tokens, relative to the reference.  The reference moves only
+                // when that exceeds kLazy (weights stay below 2^kLazy) or is the row's first; the output rows and
+                // sums are rescaled on those occasions only.
+                const float mrel = max_lane_groups(max4_of_product(s[rg][0], s[rg][1], s[rg][2], s[rg][3]));
+                const bool move = m_run[rg] == -INFINITY ? mrel > -INFINITY : mrel > kLazy;
+                if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                    const float delta = move ? mrel : 0.0f;
+                    const float alpha = (m_run[rg] == -INFINITY) ? 1.0f : s_exp2(-delta);    // nothing summed yet: nothing to rescale
+                    m_run[rg] = move ? (m_run[rg] == -INFINITY ? mrel : m_run[rg] + mrel) : m_run[rg];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) s[rg][j] -= delta;
+                    l_lane[rg] *= alpha;
+                    if constexpr (DT == DRK_INT8) ps_lane[rg] *= alpha;
+                    // register j of lane group g holds row 4g + j of the group
+                    const float a0 = __shfl(alpha, 4 * g), a1 = __shfl(alpha, 4 * g + 1);
+                    const float a2 = __shfl(alpha, 4 * g + 2), a3 = __shfl(alpha, 4 * g + 3);
+#pragma unroll
+                    for (int e = 0; e < Geo::NPV; e++) { o[rg][e][0] *= a0; o[rg][e][1] *= a1; o[rg][e][2] *= a2; o[rg][e][3] *= a3; }
+                }
+                float p[4], pw[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) p[j] = s_exp2(s[rg][j]);
+#pragma unroll
+                for (int j = 0; j < 4; j++) pw[j] = (DT == DRK_INT8) ? (t0 + j < lim ? p[j] * vs[j] : 0.0f) : p[j];
+                uint2 pk;
+                if constexpr (DOT == DRK_BF16) {
+                    pk.x = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[1]) << 16);
+                    pk.y = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[3]) << 16);
+                } else {
+                    pk.x = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[1]) << 16);
+                    pk.y = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[3]) << 16);
+                }
+                pa[rg] = pk;
+                // The row's denominator is the sum of the weights the second product multiplies -- the rounded
+                // ones -- so that numerator and denominator carry the same rounding.  (int8: the product
+                // multiplies p times the V scale, rounded; its sum of plain p stays exact, and the sum of the
+                // rounded weights is kept for the code offset.)
+                if (DT == DRK_INT8) {
+                    float t = s_dot2<DOT>(pk.x, kF16Ones, 0.0f);
+                    ps_lane[rg] += s_dot2<DOT>(pk.y, kF16Ones, t);
+                    l_lane[rg] += (p[0] + p[1]) + (p[2] + p[3]);
+                } else {
+                    l_lane[rg] += s_dot2<DOT>(pk.y, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, s_dot2<DOT>(pk.x, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, 0.0f));
+                }
+            }
+            // O += P V; the V operands serve all row groups
+#pragma unroll
+            for (int ch = 0; ch < Geo::NCH; ch++)
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+#pragma unroll
+                    for (int rg = 0; rg < N; rg++) o[rg][ch * 8 + e] = w_mfma_pv<DOT>(pa[rg], vb[ch][e], o[rg][ch * 8 + e]);
+        };
+        if (nga > 1 || (A.dbg & 1)) tile_body(std::integral_constant<int, NG>{});
+        else tile_body(std::integral_constant<int, 1>{});
+        // ---- the segment's last tile: fold the four waves, leave (o, m, l) for the merge ----
+        if (flags & 2) {
+            uint4 qn[QPASS];
+            if (has_next && !(A.dbg & 4)) q_issue(udesc[it + 1], qn);          // the next segment's query rows travel during the fold
+            float pwv[NG];
+#pragma unroll
+            for (int rg = 0; rg < NG; rg++) {
+                pwv[rg] = 0.0f;
+                if (rg < nga) {
+                    const float lw = sum_lane_groups(l_lane[rg]);
+                    if (DT == DRK_INT8) pwv[rg] = sum_lane_groups(ps_lane[rg]);
+                    if (lane < 16) { mw_lds[w][rg * 16 + lane] = m_run[rg]; lw_lds[w][rg * 16 + lane] = lw; }   // padded rows too: defined values
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int rg = 0; rg < NG; rg++) {
+                if (rg < nga) {
+                    float bias[4];                                   // code offset of row 4g + j (read from its lane while every lane is on)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) bias[j] = DT == DRK_INT8 ? kI8Bias * __shfl(pwv[rg], 4 * g + j) : 0.0f;
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {                    // rows 8t .. 8t + 7 of the group
+                        // this wave's rows 4g + j of the group, weighted for the fold and freed of the code offset
+                        if ((g >> 1) == t) {
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                const int h = rg * 16 + 4 * g + j;
+                                const float M = fmaxf(fmaxf(mw_lds[0][h], mw_lds[1][h]), fmaxf(mw_lds[2][h], mw_lds[3][h]));
+                                const float mo = mw_lds[w][h];
+                                const float f_own = mo == -INFINITY ? 0.0f : s_exp2(mo - M);
+#pragma unroll
+                                for (int ch = 0; ch < Geo::NCH; ch++) {
+                                    float *dst = &o_lds[w][4 * (g & 1) + j][ch * 128 + c * 8];
+                                    const w_f32x4 *oc = &o[rg][ch * 8];
+                                    *(float4 *)dst = make_float4((oc[0][j] - bias[j]) * f_own, (oc[1][j] - bias[j]) * f_own,
+                                                                 (oc[2][j] - bias[j]) * f_own, (oc[3][j] - bias[j]) * f_own);
+                                    *(float4 *)(dst + 4) = make_float4((oc[4][j] - bias[j]) * f_own, (oc[5][j] - bias[j]) * f_own,
+                                                                       (oc[6][j] - bias[j]) * f_own, (oc[7][j] - bias[j]) * f_own);
+                                }
+                            }
+                        }
+                        __syncthreads();
+                        // wave w sums rows 8t + w and 8t + w + 4 of the group over the four waves
+#pragma unroll
+                        for (int i = 0; i < 2; i++) {
+                            const int hl = w + 4 * i, R = rg * 16 + 8 * t + hl;
+                            if (R < nrows) {
+                                const float M = fmaxf(fmaxf(mw_lds[0][R], mw_lds[1][R]), fmaxf(mw_lds[2][R], mw_lds[3][R]));
+                                float L = 0.0f;
+#pragma unroll
+                                for (int ww = 0; ww < 4; ww++) {
+                                    const float mm = mw_lds[ww][R];
+                                    if (mm != -INFINITY) L = fmaf(lw_lds[ww][R], s_exp2(mm - M), L);
+                                }
+                                constexpr int VEC = D / 64;
+                                const int d = lane * VEC;
+                                float acc[VEC];
+#pragma unroll
+                                for (int x = 0; x < VEC; x++) acc[x] = 0.0f;
+#pragma unroll
+                                for (int ww = 0; ww < 4; ww++)
+#pragma unroll
+                                    for (int x = 0; x < VEC; x++) acc[x] += o_lds[ww][hl][d + x];
+                                const int bl = R / GQ, hd = R - bl * GQ;
+                                const size_t pi = (size_t)(ud.row0 + bl * A.QH + hd) * A.Ptot + ud.slot;
+#pragma unroll
+                                for (int x = 0; x < VEC; x++) A.part_o[pi * D + d + x] = acc[x];
+                                if (lane == 0) {
+                                    A.part_m[pi] = M;
+                                    A.part_l[pi] = L;
+                                }
+                            }
+                        }
+                        __syncthreads();
+                    }
+                }
+            }
+#pragma unroll
+            for (int rg = 0; rg < NG; rg++) {
+#pragma unroll
+                for (int e = 0; e < Geo::NPV; e++) o[rg][e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                m_run[rg] = -INFINITY; l_lane[rg] = 0.0f; ps_lane[rg] = 0.0f;
+            }
+            if (has_next) {
+                if (A.dbg & 4) q_issue(udesc[it + 1], qn);
+                q_store(qn);
+                __syncthreads();
+                q_bias();
+            }
+        }
+    }
+}
+
+// grid (QH, B), block 256: fold the pieces of (branch, q head): those of every group the branch
+// belongs to and those of its tail; out is written only when some token took part
+// (paged_attention.cu:266).  The piece list is put together first (which slots hold pieces follows
+// from the lengths, exactly as the kernel above cut its runs); then lane s of every wave owns the
+// (m, l) of piece s (+64, ...), wave w folds the o rows of pieces w, w+4, ... eight at a time, and
+// the four waves' sums meet in LDS.
+template <int D>
+__global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_t *__restrict__ out, int grid_wgs,
+                                                          const uint16_t *__restrict__ gate, size_t gate_stride)
+{
+    constexpr int VEC = D / 64;                                  // dims per lane: 2 or 4
+    typedef float fvec __attribute__((ext_vector_type(VEC)));
+    __shared__ fvec red[4][64];
+    __shared__ int seg_base[kGMaxGroups + 1], seg_cnt[kGMaxGroups + 1], seg_off[kGMaxGroups + 2], nseg_s;
+    __shared__ short slot_of[kGMaxPieces];
+    const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * VEC;
+    if (threadIdx.x == 0) {
+        int excl = 0, total = 0, nt_b = 0;
+        for (int i = 0; i < A.B; i++) {
+            const int len = A.seq_lens[i];
+            const int nt = len > 0 ? max((len + kSTile - 1) / kSTile - A.b_start[i], 0) : 0;
+            if (i < b) excl += nt;
+            if (i == b) nt_b = nt;
+            total += nt;
+        }
+        const int T = A.group_units + total * A.KVH;
+        int n = 0, off = 0;
+        if (T > 0) {
+            const int U = (T + grid_wgs - 1) / grid_wgs;
+            const int kvh = h / (A.QH / A.KVH);
+            for (int gi = 0; gi < A.ngroups; gi++) {
+                const GSeg sg = A.seg[gi];
+                if (b < sg.first || b >= sg.first + sg.count) continue;
+                const int first = sg.unit0 + kvh * sg.ntile, last = first + sg.ntile - 1;
+                seg_base[n] = sg.slot; seg_cnt[n] = last / U - first / U + 1; seg_off[n] = off;
+                off += seg_cnt[n]; n++;
+            }
+            if (nt_b > 0) {
+                const int first = A.group_units + A.KVH * excl + kvh * nt_b, last = first + nt_b - 1;
+                seg_base[n] = A.b_slot[b]; seg_cnt[n] = last / U - first / U + 1; seg_off[n] = off;
+                off += seg_cnt[n]; n++;
+            }
+        }
+        seg_off[n] = min(off, kGMaxPieces);
+        nseg_s = n;
+    }
+    __syncthreads();
+    const int nseg = nseg_s, n_all = seg_off[nseg];
+    for (int k = 0; k < nseg; k++)
+        for (int i = threadIdx.x; i < seg_cnt[k] && seg_off[k] + i < kGMaxPieces; i += 256) slot_of[seg_off[k] + i] = (short)(seg_base[k] + i);
+    __syncthreads();
+    const size_t base = ((size_t)b * A.QH + h) * A.Ptot;
+    float M = -INFINITY;
+    for (int s = lane; s < n_all; s += 64) {
+        const size_t pi = base + slot_of[s];
+        if (A.part_l[pi] > 0.0f) M = fmaxf(M, A.part_m[pi]);
+    }
+    M = s_wave_max(M);
+    fvec acc = {};
+    float L = 0.0f;
+    for (int c0 = 0; c0 < n_all; c0 += 64) {
+        const int s = c0 + lane, cnt = min(64, n_all - c0);
+        float wt = 0.0f;
+        if (s < n_all) {
+            const size_t pi = base + slot_of[s];
+            const float pl = A.part_l[pi];
+            if (pl > 0.0f) { wt = s_exp2(A.part_m[pi] - M); L = fmaf(pl, wt, L); }
+        }
+        for (int j = wv; j < cnt; j += 32) {
+            fvec o[8];
+            float wj[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int jj = min(j + 4 * u, cnt - 1);
+                wj[u] = j + 4 * u < cnt ? s_lane(wt, jj) : 0.0f;
+                o[u] = *(const fvec *)(A.part_o + (base + slot_of[c0 + jj]) * D + d);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (wj[u] != 0.0f) {                                  // a piece without tokens may hold anything
+#pragma unroll
+                    for (int x = 0; x < VEC; x++) acc[x] = fmaf(o[u][x], wj[u], acc[x]);
+                }
+        }
+    }
+    L = s_wave_sum(L);
+    red[wv][lane] = acc;
+    __syncthreads();
+    if (wv == 0) {
+        // with a gate the row is always rewritten: the reference gates whatever the attention
+        // kernel left in out, also when no token took part (paged_attention.cu:266, 368-370)
+        uint16_t *dst = out + ((size_t)b * A.QH + h) * D + d;
+        uint16_t vals[VEC];
+        if (L > 0.0f) {
+            const fvec a1 = red[1][lane], a2 = red[2][lane], a3 = red[3][lane];
+#pragma unroll
+            for (int x = 0; x < VEC; x++) vals[x] = f_to_elem16(((acc[x] + a1[x]) + (a2[x] + a3[x])) / L, A.io_dtype);
+        } else {
+            if (!gate) return;
+#pragma unroll
+            for (int x = 0; x < VEC; x++) vals[x] = dst[x];
+        }
+        if (gate) {
+            const uint16_t *gp = gate + ((size_t)b * A.QH + h) * gate_stride + d;
+#pragma unroll
+            for (int x = 0; x < VEC; x++) vals[x] = gated_elem16(vals[x], gp[x], A.io_dtype);
+        }
+        if constexpr (VEC == 2) {
+            *(uint32_t *)dst = (uint32_t)vals[0] | ((uint32_t)vals[1] << 16);
+        } else {
+            *(uint2 *)dst = make_uint2((uint32_t)vals[0] | ((uint32_t)vals[1] << 16), (uint32_t)vals[2] | ((uint32_t)vals[3] << 16));
+        }
+    }
+}
+
+// ---- host side ------------------------------------------------------------------------------
+bool grouped_decode_supported(const Lay &a, int B)
+{
+    return !g_force_portable && g_grouped_mode != 1 && a.D == 128 && stream_decode_supported(a, B);
+}
+
+struct GroupPlan {
+    int ngroups, group_units, grid, Ptot;
+    GSeg seg[kGMaxGroups];
+    int b_start[64], b_slot[64];
+};
+
+// Shared ranges in tokens -> tiles, checked: for every branch the ranges it belongs to must follow
+// one another from token 0 without gap or overlap (then every token of a branch is read exactly once:
+// by one range or by the branch's tail).  Ranges are cut down to whole 64-token tiles; what a range
+// loses at its end, the range or tail behind it reads.
+static int plan_groups(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_in, GroupPlan *P)
+{
+    if (n_in < 0 || n_in > kGMaxGroups) return fail(DRK_ERR_INVALID, "decode_grouped: %d groups (0..%d)", n_in, kGMaxGroups);
+    if (n_in > 0 && !groups) return fail(DRK_ERR_INVALID, "decode_grouped: groups is NULL");
+    const int GQ = a.QH / a.KVH;
+    const int max_tiles = (max_seq_len + kSTile - 1) / kSTile;
+    int n = 0;
+    for (int i = 0; i < n_in; i++) {
+        const drk_prefix_group &gr = groups[i];
+        if (gr.first_branch < 0 || gr.n_branches < 1 || gr.first_branch + gr.n_branches > B || gr.tok_begin < 0 ||
+            gr.tok_end < gr.tok_begin || gr.tok_end > max_seq_len)
+            return fail(DRK_ERR_INVALID, "decode_grouped: group %d = branches [%d, +%d) tokens [%d, %d) does not fit %d branches of up to %d tokens",
+                        i, gr.first_branch, gr.n_branches, gr.tok_begin, gr.tok_end, B, max_seq_len);
+        const int t0 = gr.tok_begin / kSTile, t1 = gr.tok_end / kSTile;
+        if (t1 <= t0) continue;
+        if (gr.n_branches * GQ > 64)
+            return fail(DRK_ERR_UNSUPPORTED, "decode_grouped: group %d has %d branches x %d query heads per kv head (at most 64 rows: split it)",
+                        i, gr.n_branches, GQ);
+        GSeg s;
+        s.first = gr.first_branch; s.count = gr.n_branches; s.tile0 = t0; s.ntile = t1 - t0; s.slot = -1; s.unit0 = 0;
+        int k = n++;
+        while (k > 0 && P->seg[k - 1].tile0 > s.tile0) { P->seg[k] = P->seg[k - 1]; k--; }   // ordered by first tile
+        P->seg[k] = s;
+    }
+    P->ngroups = n;
+    int units = 0;
+    for (int k = 0; k < n; k++) { P->seg[k].unit0 = units; units += a.KVH * P->seg[k].ntile; }
+    P->group_units = units;
+    long t_upper = units;
+    for (int b = 0; b < B; b++) {
+        int start = 0;
+        for (int k = 0; k < n; k++) {
+            const GSeg &s = P->seg[k];
+            if (b < s.first || b >= s.first + s.count) continue;
+            if (s.tile0 != start)
+                return fail(DRK_ERR_INVALID, "decode_grouped: the ranges of branch %d do not follow one another from token 0 (tile %d after tile %d)",
+                            b, s.tile0, start);
+            start = s.tile0 + s.ntile;
+        }
+        P->b_start[b] = start;
+        t_upper += (long)a.KVH * (max_tiles > start ? max_tiles - start : 0);
+    }
+    for (int b = B; b < 64; b++) P->b_start[b] = P->b_slot[b] = 0;
+    long G = t_upper < kGWgs ? t_upper : kGWgs;
+    if (G < 1) G = 1;
+    if ((t_upper + G - 1) / G > kGMaxUnits) G = (t_upper + kGMaxUnits - 1) / kGMaxUnits;   // descriptor table size
+    P->grid = (int)G;
+    // a run of n tiles of one kv head meets at most min(n, G / KVH + 2) workgroups
+    const int cap = (int)(G / a.KVH) + 2;
+    auto pub = [&](int tiles) { return tiles <= 0 ? 0 : (tiles < cap ? tiles : cap); };
+    int Ptot = 1;
+    for (int b = 0; b < B; b++) {
+        int slot = 0;
+        for (int k = 0; k < n; k++) {
+            GSeg &s = P->seg[k];
+            if (b < s.first || b >= s.first + s.count) continue;
+            if (s.slot < 0) s.slot = slot;
+            else if (s.slot != slot)
+                return fail(DRK_ERR_INVALID, "decode_grouped: the branches of a group must belong to the same groups before it (branch %d)", b);
+            slot += pub(s.ntile);
+        }
+        P->b_slot[b] = slot;
+        slot += pub(max_tiles - P->b_start[b]);
+        if (slot > Ptot) Ptot = slot;
+    }
+    if (Ptot > kGMaxPieces)
+        return fail(DRK_ERR_UNSUPPORTED, "decode_grouped: %d pieces per query row (at most %d)", Ptot, kGMaxPieces);
+    P->Ptot = Ptot;
+    return DRK_OK;
+}
+
+size_t grouped_workspace_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups)
+{
+    GroupPlan P;
+    if (B < 1 || B > 64 || plan_groups(a, B, max_seq_len, groups, n_groups, &P) != DRK_OK) return 0;
+    return (size_t)B * a.QH * P.Ptot * (a.D + 2) * sizeof(float);
+}
+
+// every plan with ranges nested at most max_depth deep fits: each level and the tail take at most kGWgs / KVH + 2 slots
+size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_depth)
+{
+    const int max_tiles = (max_seq_len + kSTile - 1) / kSTile;
+    long G = kGWgs;
+    const long t_upper = (long)a.KVH * B * max_tiles;
+    if ((t_upper + G - 1) / G > kGMaxUnits) G = (t_upper + kGMaxUnits - 1) / kGMaxUnits;
+    long cap = G / a.KVH + 2;
+    if (cap > max_tiles) cap = max_tiles;
+    long P = (long)(max_depth + 1) * cap;
+    if (P > max_tiles + 2L * (max_depth + 1)) P = max_tiles + 2L * (max_depth + 1);
+    if (P < 1) P = 1;
+    return (size_t)B * a.QH * (size_t)P * (a.D + 2) * sizeof(float);
+}
+
+int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables, int table_stride,
+                          const int32_t *d_seq_lens, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups,
+                          void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
+                          void *stream, const void *gate, size_t gate_stride)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (!q || !pool || !tables || !out || !d_seq_lens) return fail(DRK_ERR_INVALID, "decode_grouped: NULL pointer");
+    if (gate && (gate_stride < (size_t)a.D || (gate_stride % 8) || ((uintptr_t)gate % 16)))
+        return fail(DRK_ERR_INVALID, "decode_grouped: gate rows must be 16-byte aligned and at least head_dim apart");
+    if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode_grouped: io_dtype must be F16 or BF16");
+    if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
+        return fail(DRK_ERR_INVALID, "decode_grouped: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
+    if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "decode_grouped: layer %d outside [0,%d)", layer, a.L);
+    if (B < 0 || max_seq_len < 0 || table_stride < 0) return fail(DRK_ERR_INVALID, "decode_grouped: negative size");
+    if (B == 0 || max_seq_len == 0) return DRK_OK;
+    if (!grouped_decode_supported(a, B) || !(scale > 0.0f))
+        return fail(DRK_ERR_UNSUPPORTED, "decode_grouped: needs head_dim 128, at most 16 query heads per kv head, block_size %% 16 == 0, at most 64 branches, scale > 0");
+    GroupPlan P;
+    if ((rc = plan_groups(a, B, max_seq_len, groups, n_groups, &P))) return rc;
+    if (P.ngroups == 0)                                            // nothing shared (after rounding to tiles): the plain kernel
+        return launch_decode(g, q, pool, tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale, io_dtype,
+                             0, workspace, workspace_bytes, stream, gate, gate_stride);
+    const size_t need = (size_t)B * a.QH * P.Ptot * (a.D + 2) * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+        return fail(DRK_ERR_WORKSPACE, "decode_grouped: workspace of %zu bytes, need %zu", workspace_bytes, need);
+    if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode_grouped: workspace must be 16-byte aligned");
+
+    GroupedArgs A;
+    A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
+    A.tables = tables; A.seq_lens = d_seq_lens; A.q = (const uint8_t *)q;
+    A.part_o = (float *)workspace;
+    A.part_m = A.part_o + (size_t)B * a.QH * P.Ptot * a.D;
+    A.part_l = A.part_m + (size_t)B * a.QH * P.Ptot;
+    A.table_stride = table_stride; A.B = B; A.KVH = a.KVH; A.QH = a.QH; A.NB = a.NB; A.bs = a.bs;
+    A.bs_shift = ilog2_exact((unsigned)a.bs); A.io_dtype = io_dtype; A.Ptot = P.Ptot;
+    A.ngroups = P.ngroups; A.group_units = P.group_units;
+    A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
+    A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
+    A.scale_log2e = scale * kSLog2e;
+    A.dbg = getenv("DRK_GDBG") ? atoi(getenv("DRK_GDBG")) : 0;
+    for (int k = 0; k < kGMaxGroups; k++) A.seg[k] = k < P.ngroups ? P.seg[k] : GSeg{0, 0, 0, 0, 0, 0x7fffffff};
+    for (int b = 0; b < 64; b++) { A.b_start[b] = P.b_start[b]; A.b_slot[b] = P.b_slot[b]; }
+    hipStream_t st = (hipStream_t)stream;
+    const bool dma = g_grouped_mode != 2;
+    switch (a.dtype) {
+    case DRK_F16:
+        if (dma) hipLaunchKernelGGL((decode_group_kernel<DRK_F16, 128, 4, true>), dim3(P.grid), dim3(256), 0, st, A);
+        else hipLaunchKernelGGL((decode_group_kernel<DRK_F16, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A);
+        break;
+    case DRK_BF16:
+        if (dma) hipLaunchKernelGGL((decode_group_kernel<DRK_BF16, 128, 4, true>), dim3(P.grid), dim3(256), 0, st, A);
+        else hipLaunchKernelGGL((decode_group_kernel<DRK_BF16, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A);
+        break;
+    case DRK_INT8: hipLaunchKernelGGL((decode_group_kernel<DRK_INT8, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A); break;
+    default: hipLaunchKernelGGL((decode_group_kernel<DRK_FP8_E4M3, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A); break;
+    }
+    DRK_LAUNCH_CHECK("decode_group_kernel");
+    hipLaunchKernelGGL(group_merge_kernel<128>, dim3(a.QH, B), dim3(256), 0, st, A, (uint16_t *)out, P.grid,
+                       (const uint16_t *)gate, gate_stride);
+    DRK_LAUNCH_CHECK("group_merge_kernel");
+    return DRK_OK;
+}
+
+} // namespace drk
+
+using namespace drk;
+
+extern "C" {
+
+void drk_debug_set_grouped_decode(int mode) { g_grouped_mode = (mode == 1 || mode == 2) ? mode : 0; }
+
+size_t drk_decode_grouped_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len, const drk_prefix_group *groups,
+                                          int n_groups)
+{
+    Lay a;
+    if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0) return 0;
+    size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);      // no group left after rounding: the plain kernel
+    if (a.D == 128 && stream_decode_supported(a, B)) {
+        const size_t s2 = grouped_workspace_need(a, B, max_seq_len, groups, n_groups);
+        if (s2 == 0) return 0;
+        if (s2 > need) need = s2;
+    }
+    return need;
+}
+
+size_t drk_decode_grouped_workspace_bytes_max(const drk_kv_layout *g, int B, int max_seq_len, int max_depth)
+{
+    Lay a;
+    if (make_lay(g, &a) != DRK_OK || B <= 0 || max_seq_len <= 0 || max_depth < 0) return 0;
+    size_t need = drk_decode_workspace_bytes(g, B, max_seq_len);
+    if (a.D == 128 && stream_decode_supported(a, B)) {
+        const size_t s2 = grouped_workspace_need_max(a, B, max_seq_len, max_depth);
+        if (s2 > need) need = s2;
+    }
+    return need;
+}
+
+int drk_paged_decode_attention_grouped(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_tables,
+                                       int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len,
+                                       const drk_prefix_group *groups, int n_groups, void *out, int layer, float scale,
+                                       int io_dtype, const void *gate, size_t gate_stride, void *workspace,
+                                       size_t workspace_bytes, void *stream)
+{
+    return launch_decode_grouped(g, q, pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups, n_groups, out, layer,
+                                 scale, io_dtype, workspace, workspace_bytes, stream, gate, gate_stride);
+}
+
+} // extern "C"

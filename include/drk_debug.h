@@ -35,6 +35,9 @@ void drk_debug_set_shared_splits(int n);
 /* Tuning: the shared-prefix pass for at most 64 rows per kv head and head_dim 128 runs on the
  * producer / consumer kernel (1, the default) or on the kernel every wave stages in (0). */
 void drk_debug_set_prefix_stream(int on);
+/* Diagnostic: 1 = drk_paged_decode_attention_shared never takes the grouped kernel (one launch over
+ * shared and private tiles) but always the prefix pass + tail kernel pair; 0 = the library's choice. */
+void drk_debug_set_grouped_decode(int mode);
 /* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
  * session; switching it on starts a new session) records a HIP event on its
  * stream right before and right after the split-K partial kernel; the merge

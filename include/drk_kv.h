@@ -268,6 +268,37 @@ int drk_paged_decode_attention_shared(const drk_kv_layout *g, const void *q, con
                                       int io_dtype, void *workspace, size_t workspace_bytes,
                                       void *stream);
 
+/* Branches that share pages as a tree (no reference counterpart; intent
+ * docs/en/architecture/03-cogitatio.md:8-22: the Action / Speech / Thinking / Daydream branches fork from one
+ * context and from one another; src/conscientia/scheduler.h:53-56).  A group says: branches
+ * [first_branch, first_branch + n_branches) hold tokens [tok_begin, tok_end) in the same physical blocks, and every
+ * one of them is at least tok_end tokens long (CacheManager::common_prefix_groups computes the groups from the
+ * tables).  For every branch the groups it belongs to must follow one another from token 0 without gap or overlap
+ * -- a fork tree: the whole set over the persistent prefix, subsets over what they wrote before they split again --
+ * and a group takes at most 64 / (num_q_heads / num_kv_heads) branches.  Group boundaries are rounded down to
+ * multiples of 64 tokens; what a group loses at its end is read by the group or the private tail behind it.  All
+ * shared and private pages are streamed once, in ONE launch whose workgroups take equal shares of the bytes, and
+ * one merge.  head_dim 128, block_size % 16 == 0, at most 64 branches, at most 16 query heads per kv head, every
+ * storage type; DRK_ERR_UNSUPPORTED otherwise (use drk_paged_decode_attention_shared / _branches).  gate may be
+ * NULL; otherwise as in drk_paged_decode_attention_gated.  Results equal the per-branch call up to summation order.
+ * Workspace: drk_decode_grouped_workspace_bytes for these very groups, or _max for any tree nested at most
+ * max_depth groups deep (what a caller reserves once). */
+#define DRK_MAX_PREFIX_GROUPS 16
+typedef struct drk_prefix_group {
+    int32_t first_branch, n_branches;
+    int32_t tok_begin, tok_end;
+} drk_prefix_group;
+size_t drk_decode_grouped_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len,
+                                          const drk_prefix_group *groups, int n_groups);
+size_t drk_decode_grouped_workspace_bytes_max(const drk_kv_layout *g, int B, int max_seq_len, int max_depth);
+int drk_paged_decode_attention_grouped(const drk_kv_layout *g, const void *q, const void *pool,
+                                       const int32_t *d_tables, int table_stride,
+                                       const int32_t *d_seq_lens, int B, int max_seq_len,
+                                       const drk_prefix_group *groups, int n_groups, void *out,
+                                       int layer, float scale, int io_dtype, const void *gate,
+                                       size_t gate_stride, void *workspace, size_t workspace_bytes,
+                                       void *stream);
+
 /* ---- paged causal prefill attention ------------------------------------ */
 /* paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630:
  * q/out [M, num_q_heads, head_dim]; row t attends to tokens 0..pos_start+t (the

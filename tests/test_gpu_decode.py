@@ -344,12 +344,16 @@ def test_workspace_too_small_is_refused(dev):
     assert rc == cabi.ERR_WORKSPACE
 
 
-@pytest.fixture(params=["producer_consumer", "every_wave_stages"])
+@pytest.fixture(params=["grouped", "producer_consumer", "every_wave_stages"])
 def prefix_kernel(request):
-    """the shared-prefix pass has two kernels for up to 64 rows per kv head of head_dim 128"""
-    cabi.lib().drk_debug_set_prefix_stream(1 if request.param == "producer_consumer" else 0)
+    """Shared pages are read by the grouped kernel (shared and private tiles in one launch: head_dim 128, up to
+    64 rows per kv head) or by a prefix pass + the tail kernel; the prefix pass has two kernels for up to 64 rows
+    per kv head of head_dim 128."""
+    cabi.lib().drk_debug_set_grouped_decode(0 if request.param == "grouped" else 1)
+    cabi.lib().drk_debug_set_prefix_stream(0 if request.param == "every_wave_stages" else 1)
     yield request.param
     cabi.lib().drk_debug_set_prefix_stream(1)
+    cabi.lib().drk_debug_set_grouped_decode(0)
 
 
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
