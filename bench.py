@@ -80,6 +80,9 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "
                                                             "replaying one captured HIP graph per step")
     ap.add_argument("--no-cascade", action="store_true", help="config 3: read the shared prefix once per branch")
+    ap.add_argument("--shared-kernel", choices=["auto", "pair"], default="auto",
+                    help="config 3: how shared pages are read: auto = one launch over shared and private tiles where the "
+                         "geometry allows; pair = always the prefix pass followed by the tail kernel")
     return ap.parse_args()
 
 
@@ -92,6 +95,7 @@ def main():
     from deusridet_amd import cabi
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    cabi.lib().drk_debug_set_grouped_decode(1 if args.shared_kernel == "pair" else 0)
     if args.config != 2:
         import bench_extra
         print(json.dumps(bench_extra.run(args)))
@@ -239,15 +243,14 @@ def main():
                       cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
                       cabi.BF16, split, cabi.p(ws), wsb, sp)
 
-    attn_only(8)
-    lib.drk_debug_time_decode_kernel(1)
-    attn_only(n_timed)
-    buf = (C.c_float * 256)()
-    cnt = C.c_int32(0)
-    cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
-    lib.drk_debug_time_decode_kernel(0)
-    ker_ms = np.array(buf[:cnt.value])
-    ker_avg_ms = float(ker_ms.mean())
+    # (event pairs recorded here, around calls that leave the merge kernel out: cabi.time_partial_kernels)
+    def attn_one(it, lens=dlen):
+        l = it % L
+        cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), cabi.p(pool),
+                  cabi.p(dtab), stride, lens, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
+                  cabi.BF16, split, cabi.p(ws), wsb, sp)
+
+    ker_avg_ms = cabi.time_partial_kernels(attn_one, n_timed, warm=8)
     launch_bytes = int((start + last + 1).sum()) * kv_bytes_per_token               # one layer, one launch
     achieved = launch_bytes / (ker_avg_ms * 1e-3) / 1e9
 
@@ -265,32 +268,14 @@ def main():
                           cabi.p(dtab), stride, cabi.p(rlen), B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
                           cabi.BF16, split, cabi.p(ws), wsb, sp)
 
-        ragged_only(8)
-        lib.drk_debug_time_decode_kernel(1)
-        ragged_only(n_timed)
-        cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
-        lib.drk_debug_time_decode_kernel(0)
-        r_ms = float(np.mean(buf[:cnt.value]))
+        r_ms = cabi.time_partial_kernels(lambda it: attn_one(it, cabi.p(rlen)), n_timed, warm=8)
         r_bytes = int(rl.sum()) * kv_bytes_per_token
         # what a launch pays before its first tile: the same launches with the kernel leaving once the branch
         # lengths are scanned and the workgroup's unit descriptors (one table read per 16-token run) are built
         lib.drk_debug_set_stream_descriptors_only(1)
-        ragged_only(8)
-        lib.drk_debug_time_decode_kernel(1)
-        ragged_only(n_timed)
-        cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
-        lib.drk_debug_time_decode_kernel(0)
+        ragged_pro_ms = cabi.time_partial_kernels(lambda it: attn_one(it, cabi.p(rlen)), n_timed, warm=8)
+        fixed_pro_ms = cabi.time_partial_kernels(attn_one, n_timed, warm=8)
         lib.drk_debug_set_stream_descriptors_only(0)
-        ragged_pro_ms = float(np.mean(buf[:cnt.value]))
-        attn_only(8)
-        lib.drk_debug_set_stream_descriptors_only(1)
-        attn_only(8)
-        lib.drk_debug_time_decode_kernel(1)
-        attn_only(n_timed)
-        cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
-        lib.drk_debug_time_decode_kernel(0)
-        lib.drk_debug_set_stream_descriptors_only(0)
-        fixed_pro_ms = float(np.mean(buf[:cnt.value]))
         attn_only(2)                                                 # leave real results behind
         ragged = {"ctx": [int(x) for x in rl], "kernel_us": round(r_ms * 1e3, 2), "bytes_per_launch": r_bytes,
                   "GBps": round(r_bytes / (r_ms * 1e-3) / 1e9, 1), "hbm_frac": round(r_bytes / (r_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),

@@ -24,15 +24,9 @@ def _common(args):
 
 
 def _timed_decode(lib, cabi, call, n):
-    """average duration of the partial kernel over n back-to-back launches"""
-    call(6)
-    lib.drk_debug_time_decode_kernel(1)
-    call(n)
-    buf = (C.c_float * 256)()
-    cnt = C.c_int32(0)
-    cabi.call("drk_debug_decode_kernel_times", buf, 256, C.byref(cnt))
-    lib.drk_debug_time_decode_kernel(0)
-    return float(np.mean(buf[:cnt.value]))
+    """average duration (ms) of the kernels that read the pages over n back-to-back calls, merge left out;
+    call(i) makes the i-th call"""
+    return cabi.time_partial_kernels(call, n)
 
 
 def config4(args):
@@ -111,7 +105,7 @@ def config4(args):
     toks = sum(B * (start + s + 1) for s in range(W, W + K))
     value = toks * code_bytes * L / (total_ms * 1e-3) / 1e9
     dlen = C.c_void_p(len_steps[W + K - 1].data_ptr())
-    ker_ms = _timed_decode(lib, cabi, lambda n: [attn(i % L, dlen) for i in range(n)], 60)
+    ker_ms = _timed_decode(lib, cabi, lambda i: attn(i % L, dlen), 60)
     launch_bytes = B * ctx * code_bytes
     ach = launch_bytes / (ker_ms * 1e-3) / 1e9
     return {
@@ -243,10 +237,10 @@ def config3(args):
     unique_tokens = cm.gpu_blocks_used() * bs
     value = logical * per_tok * L / (total_ms * 1e-3) / 1e9
     dl = cabi.p(dlen)
-    ker_ms = _timed_decode(lib, cabi, lambda n: [cabi.call(
+    ker_ms = _timed_decode(lib, cabi, lambda i: cabi.call(
         "drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + (i % L) * qrow), pool_ptr, dtabs,
         stride, dl, B, max_ctx, shared_now[0], C.c_void_p(out.data_ptr() + (i % L) * qrow), i % L, float(scale),
-        cabi.BF16, cabi.p(ws), wsb, sp) for i in range(n)], 60)
+        cabi.BF16, cabi.p(ws), wsb, sp), 60)
     launch_logical = int(lens.sum()) * per_tok
     # bytes the launch must fetch: shared pages once, private pages once each
     launch_unique = (shared_now[0] + int((lens - shared_now[0]).sum())) * per_tok
@@ -554,7 +548,7 @@ def config7(args):
     toks = sum(B * (start + s + 1) for s in range(W, W + K))
     value = toks * per_tok * L / (total_ms * 1e-3) / 1e9
     dlen = C.c_void_p(len_steps[W + K - 1].data_ptr())
-    ker_ms = _timed_decode(lib, cabi, lambda n: [attn(i % L, dlen) for i in range(n)], 60)
+    ker_ms = _timed_decode(lib, cabi, lambda i: attn(i % L, dlen), 60)
     launch_bytes = B * ctx * per_tok
     ach = launch_bytes / (ker_ms * 1e-3) / 1e9
     # the same shape's chunked prefill: 2 048-token chunks at positions 0, 6 144 and 30 720 of branch 0's pages
@@ -680,10 +674,10 @@ def kernel_fractions(buf, seed=11):
         ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
         dlen = torch.full((B,), ctx, dtype=torch.int32, device="cuda")
         row = B * QH * D * 2
-        ms = _timed_decode(lib, cabi, lambda n: [cabi.call(
+        ms = _timed_decode(lib, cabi, lambda i: cabi.call(
             "drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + (i % L) * row), cabi.p(buf),
             cabi.p(dtab), stride, cabi.p(dlen), B, ctx, C.c_void_p(out.data_ptr() + (i % L) * row), i % L, scale, cabi.BF16, 0,
-            cabi.p(ws), wsb, sp) for i in range(n)], 40)
+            cabi.p(ws), wsb, sp), 40)
         res["config4_%s" % name] = _entry(
             "decode_stream_kernel<%s>" % name, "hbm", B * ctx * code, ms,
             "config 4: 4 branches x 131072 tokens, %s pages (%d B per token and layer), K/V N(0,1) with 1 %% x20 outliers "
@@ -759,14 +753,17 @@ def kernel_fractions(buf, seed=11):
     ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
     row = B * QH * D * 2
 
+    def shared_one(i):
+        l = i % L
+        cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * row), cabi.p(buf), cabi.p(dtab),
+                  stride, cabi.p(dlen), B, max_ctx, prefix, C.c_void_p(out.data_ptr() + l * row), l, scale, cabi.BF16,
+                  cabi.p(ws), wsb, sp)
+
     def shared_call(n):
         for i in range(n):
-            l = i % L
-            cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * row), cabi.p(buf), cabi.p(dtab),
-                      stride, cabi.p(dlen), B, max_ctx, prefix, C.c_void_p(out.data_ptr() + l * row), l, scale, cabi.BF16,
-                      cabi.p(ws), wsb, sp)
+            shared_one(i)
 
-    pair_ms = _timed_decode(lib, cabi, shared_call, 40)                           # prefix pass + tails, without the merge
+    pair_ms = _timed_decode(lib, cabi, shared_one, 40)                           # prefix pass + tails, without the merge
     a0, a1 = ev(), ev()
     a0.record(stream)
     shared_call(40)

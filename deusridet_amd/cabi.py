@@ -105,7 +105,7 @@ SIGNATURES = {
     "drk_debug_set_stream_descriptors_only": (None, [_i32]),
     "drk_debug_set_shared_splits": (None, [_i32]),
     "drk_debug_set_prefix_stream": (None, [_i32]),
-    "drk_debug_time_decode_kernel": (None, [_i32]),
+    "drk_debug_set_skip_merge": (None, [_i32]),
     "drk_debug_set_decode_lds_pad": (None, [_i32]),
     "drk_debug_set_append_chunks": (None, [_i32, _i32, _i32]),
     "drk_debug_check_int8_scale_math": (_i32, [_vp, _vp]),
@@ -118,7 +118,6 @@ SIGNATURES = {
     "drk_probe_mfma_valu_coexec": (_i32, [_i32, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "drk_probe_phase_coexec": (_i32, [_i32, _i32, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "drk_prefill_workspace_bytes_max": (_sz, [_LP, _i32, _i32]),
-    "drk_debug_decode_kernel_times": (_i32, [C.POINTER(C.c_float), _i32, C.POINTER(_i32)]),
     "drk_paged_decode_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
     "drk_paged_decode_attention_branches": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32,
                                                    _f32, _i32, _i32, _vp, _sz, _vp]),
@@ -196,6 +195,26 @@ def call(name, *args):
 def p(t):
     """Device pointer of a torch tensor as a ctypes void pointer (None stays None)."""
     return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def time_partial_kernels(call_one, n, warm=6):
+    """Average milliseconds of the kernels that read the pages in one decode call, merge left out: n calls back
+    to back on torch's current stream (which the calls must use), one event pair around each."""
+    import torch
+    for i in range(warm):
+        call_one(i)
+    lib().drk_debug_set_skip_merge(1)
+    try:
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for i, (e0, e1) in enumerate(ev):
+            e0.record()
+            call_one(i)
+            e1.record()
+        torch.cuda.synchronize()
+    finally:
+        lib().drk_debug_set_skip_merge(0)
+    call_one(0)                                      # leave real results behind
+    return sum(e0.elapsed_time(e1) for e0, e1 in ev) / n
 
 
 def stream_ptr():

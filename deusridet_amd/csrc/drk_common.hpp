@@ -57,6 +57,7 @@ inline int ilog2_exact(unsigned v)                 // -1 when v is not a power o
 
 // ---- shared between the decode and prefill translation units ---------------
 extern int g_force_portable;
+extern int g_skip_merge;
 int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                   int table_stride, const int32_t *d_seq_lens, int seq_len_host, int causal_base, int B,
                   int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,

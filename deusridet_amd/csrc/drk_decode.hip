@@ -40,11 +40,7 @@ namespace drk {
 
 int g_force_portable = 0;                    // diagnostic, shared with the prefill unit
 static int g_decode_kernel = 0;               // diagnostic: 0 auto, 2 fixed-split tiled kernel, 3 stream kernel
-static int g_time_kernel = 0;                 // diagnostic: bracket the partial kernel with events
-constexpr int kMaxTimed = 256;                // event pairs kept per timing session
-static hipEvent_t g_ev[2 * kMaxTimed];
-static bool g_ev_made = false;
-static int g_ev_count = 0;
+int g_skip_merge = 0;                         // measurement aid: leave the partials unmerged (drk_debug_set_skip_merge)
 static int g_lds_pad = 0;                     // diagnostic: extra dynamic LDS per workgroup (caps occupancy)
 
 constexpr int kTile = 64;            // tokens per tile
@@ -540,14 +536,6 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     hipStream_t st = (hipStream_t)stream;
     dim3 grid(S, a.KVH, B);
 
-    const bool timed = g_time_kernel && g_ev_count < kMaxTimed;
-    if (timed) {
-        if (!g_ev_made) {
-            for (int i = 0; i < 2 * kMaxTimed; i++) DRK_HIP(hipEventCreate(&g_ev[i]));
-            g_ev_made = true;
-        }
-        DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count], st));
-    }
     const bool tiled = !g_force_portable && a.D == 128 && a.E == 2 && G == 4 && (a.bs % 16) == 0;
     if (use_stream) {
         rc = launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, seq_len_host, B, max_seq_len, out, layer,
@@ -592,7 +580,7 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
 #undef GO
         DRK_LAUNCH_CHECK("decode_portable_kernel");
     }
-    if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
+    if (g_skip_merge) return DRK_OK;
     if (use_stream)
         return launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, seq_len_host, B, max_seq_len, out, layer,
                                     scale, io_dtype, split_tokens, workspace, true, st, 0, nullptr, nullptr, nullptr, 0,
@@ -660,19 +648,11 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
     float *pre_m = pre_o + (size_t)B * a.QH * ns * a.D;
     float *pre_l = pre_m + (size_t)B * a.QH * ns;
     hipStream_t st = (hipStream_t)stream;
-    const bool timed = g_time_kernel && g_ev_count < kMaxTimed;
-    if (timed) {
-        if (!g_ev_made) {
-            for (int i = 0; i < 2 * kMaxTimed; i++) DRK_HIP(hipEventCreate(&g_ev[i]));
-            g_ev_made = true;
-        }
-        DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count], st));
-    }
     // branch 0's table addresses the shared pages (identical in every row by the caller's promise)
     if ((rc = launch_shared_prefix(a, q, pool, tables, d_seq_lens, B, shared, layer, scale, io_dtype, pre_o, pre_m, pre_l, st))) return rc;
     if ((rc = launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
                                    io_dtype, 0, workspace, false, st, shared / kTile))) return rc;
-    if (timed) { DRK_HIP(hipEventRecord(g_ev[2 * g_ev_count + 1], st)); g_ev_count++; }
+    if (g_skip_merge) return DRK_OK;
     return launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
                                 io_dtype, 0, workspace, true, st, shared / kTile, pre_o, pre_m, pre_l, ns, gate, gate_stride);
 }
@@ -723,24 +703,8 @@ void drk_debug_set_stream_descriptors_only(int on) { g_stream_stop_after_descrip
 void drk_debug_set_shared_splits(int n) { g_shared_splits = n > 0 ? (n < 256 ? n : 256) : 64; }
 void drk_debug_set_prefix_stream(int on) { g_prefix_stream = on ? 1 : 0; }
 
-void drk_debug_time_decode_kernel(int on)
-{
-    g_time_kernel = on ? 1 : 0;
-    if (on) g_ev_count = 0;
-}
+void drk_debug_set_skip_merge(int on) { g_skip_merge = on ? 1 : 0; }
 void drk_debug_set_decode_lds_pad(int bytes) { g_lds_pad = bytes > 0 ? bytes : 0; }
-
-int drk_debug_decode_kernel_times(float *ms, int cap, int *count)
-{
-    if (!ms || !count || cap < 0) return fail(DRK_ERR_INVALID, "decode_kernel_times: bad argument");
-    int n = g_ev_count < cap ? g_ev_count : cap;
-    for (int i = 0; i < n; i++) {
-        DRK_HIP(hipEventSynchronize(g_ev[2 * i + 1]));
-        DRK_HIP(hipEventElapsedTime(&ms[i], g_ev[2 * i], g_ev[2 * i + 1]));
-    }
-    *count = n;
-    return DRK_OK;
-}
 
 int drk_paged_decode_attention(const drk_kv_layout *g, const void *q, const void *pool,
                                const int32_t *d_block_table, void *out, int layer, int seq_len, float scale,

@@ -24,7 +24,6 @@
 #include "drk_stream_tile.hpp"
 
 #include <type_traits>
-#include <stdlib.h>
 
 namespace drk {
 
@@ -53,7 +52,6 @@ struct GroupedArgs {
     int ngroups, group_units;                  // units of all groups together
     unsigned head_stride, kv_plane, block_stride, scale_plane, row_bytes;
     float scale_log2e;
-    int dbg;
     GSeg seg[kGMaxGroups];
     int b_start[64];                           // first tile of each branch's private tail
     int b_slot[64];                            // first workspace slot of the tail's pieces
@@ -89,12 +87,13 @@ __device__ __forceinline__ float sum_lane_groups(float x)
     return x;
 }
 
-// Maximum of the four scores a lane holds, read straight out of the matrix cores' result registers.  Written as
-// assembly to spare the canonicalising copy the compiler puts in front of every fmaxf of a value it has not
-// produced with a vector instruction -- but the compiler does not look into assembly for the wait states a read of
-// a matrix result needs behind the product that writes it (it pads its own reads with s_nop), so they are here:
-// without them the maximum is taken of what the registers held before.
-__device__ __forceinline__ float max4_of_product(float a, float b, float c, float d)
+// Maximum of the four scores a lane holds, read straight out of the matrix cores' result registers.  Assembly
+// spares the canonicalising copy the compiler puts in front of every fmaxf of a value it has not produced with
+// a vector instruction -- but the compiler does not look into assembly for the wait states a read of a matrix
+// result needs behind the product that writes it (it pads its own reads with s_nop), and it is free to place
+// that product right in front of this statement, so the wait states are here: without them the maximum is
+// taken of what the registers held before the product.
+__device__ __forceinline__ float max4_asm(float a, float b, float c, float d)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     float r;
@@ -104,39 +103,29 @@ __device__ __forceinline__ float max4_of_product(float a, float b, float c, floa
     return fmaxf(fmaxf(a, b), fmaxf(c, d));
 #endif
 }
+// two fp32 -> one dword of the 16-bit type the products run in, round to nearest even, one instruction
+typedef float g_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 g_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 g_f16x2 __attribute__((ext_vector_type(2)));
+template <int DOT>
+__device__ __forceinline__ uint32_t pack16(float a, float b)
+{
+    const g_f32x2 v = {a, b};
+    if constexpr (DOT == DRK_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, g_bf16x2));
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, g_f16x2));
+}
 
 // how far (in bits of the exponent) a row's maximum may run ahead of the reference its weights are taken to
 constexpr float kLazy = 5.0f;
 
-template <int DT, int D, int NG, bool DMA>
-__global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
+// The workgroup's run of units and one descriptor per unit, in LDS: returns how many (0: nothing to do).
+// Every thread of the workgroup must call it (it holds barriers).
+template <int MAXU>
+__device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, uint2 (*gdesc)[4], int *s_incl, int *s_len, int *s_gmin)
 {
-    using Geo = StreamGeo<DT, D>;
-    [[maybe_unused]] constexpr bool Q8 = Geo::q8;
-    constexpr int DOT = KvTraits<DT>::dot;
     constexpr uint32_t kNone = 0xffffffffu;
-    constexpr int QP = D * 2 + 16;                               // LDS pitch of a query row (16-bit values)
-    constexpr int NR = NG * 16;                                  // query rows a unit may serve
-    constexpr int CPR = D * 2 / 16;                              // 16-byte chunks per query row
-    constexpr int RPP = 256 / CPR;                               // rows the workgroup moves per pass
-    constexpr int QPASS = NR / RPP;
-    // K of 16-bit pages goes from global memory straight into LDS (no registers hold it): two buffers of a wave's
-    // 16 token rows, unpadded, 16-byte chunk x of row r at position x ^ r -- applied on the global side by the lane
-    // that fills the position, undone by the reader.  8-bit codes pass through registers (they are widened on the
-    // way) into one buffer of padded rows.
-    constexpr bool DIRECT = DMA && !Q8;
-    constexpr int KBUF = DIRECT ? 16 * D * 2 : 16 * Geo::PITCH;  // one wave's K rows of one tile
-    __shared__ __align__(256) uint8_t k_lds[DIRECT ? 2 : 1][4][KBUF];
-    __shared__ __align__(16) uint8_t q_lds[NR * QP];
-    __shared__ __align__(16) float o_lds[4][8][D];               // [wave][row of the round][dim], segment ends only
-    __shared__ float mw_lds[4][NR], lw_lds[4][NR];
-    __shared__ __align__(16) GUnit udesc[kGMaxUnits];
-    __shared__ __align__(16) uint2 gdesc[kGMaxUnits][4];
-    __shared__ int s_incl[64], s_len[64], s_gmin[kGMaxGroups];
-
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
-    const int g = lane >> 4, c = lane & 15;
     const int GQ = A.QH / A.KVH;
     // ---- the workgroup's run of units and one descriptor per unit ---------------------
     const int len_i = lane < A.B ? A.seq_lens[lane] : 0;
@@ -148,13 +137,13 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
         if (lane >= off) incl += t;
     }
     const int T = A.group_units + __builtin_amdgcn_readlane(incl, 63) * A.KVH;
-    if (T == 0) return;
+    if (T == 0) return 0;
     const int U = (T + (int)gridDim.x - 1) / (int)gridDim.x;
     const int u0 = (int)blockIdx.x * U;
-    if (u0 >= T) return;
+    if (u0 >= T) return 0;
     // the host sizes the grid from max_seq_len; lengths on the device beyond that bound must not overrun
     // the descriptor table (the tiles past it are then left out: the caller broke its promise)
-    const int nunits = min(min(U, T - u0), kGMaxUnits);
+    const int nunits = min(min(U, T - u0), MAXU);
     if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
     __syncthreads();
     if ((int)threadIdx.x < A.ngroups) {
@@ -215,6 +204,339 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
         }
     }
     __syncthreads();
+    return nunits;
+}
+
+// ---- 16-bit pages: the tile in LDS, rows dealt to the waves -------------------------------------------
+// decode_group_kernel below gives every wave 16 of a tile's tokens and ALL of a unit's query rows: 64 rows are
+// 128 accumulator registers per lane, K and V wait in registers besides, and the compiler spills.  For 16-bit
+// pages a tile needs no registers on its way: each wave requests its 16-token slice of K and of V straight
+// into LDS (global_load_lds_dwordx4, two buffers, the next unit's slices travel while this one is computed),
+// and a unit of a shared range with more than 16 rows is then split by ROWS: wave w multiplies row group w
+// (16 rows: 32 accumulator registers) against all four slices -- S = K Q^T with Q in registers for the whole
+// segment, O += P V as v_mfma_f32_16x16x32 over token pairs of slices with V read transposed from LDS
+// (ds_read_b64_tr_b16), half the matrix instructions of the token split and no byte permutes.  A wave then
+// holds complete rows: a segment ends without a fold.  The price is one workgroup barrier per tile (every wave
+// reads every slice).  Units of one row group (private tails, small groups) keep the token split -- wave w
+// multiplies its own slice, the four waves fold at the segment's end -- and need no barrier.
+// LDS rows are unpadded 256 bytes; K: 16-byte chunk x of row r at position x ^ r (whole-row reads by 16 rows);
+// V: 32-byte slot y of row r at position y ^ (r & 7) (transposed reads touch 4 rows x 32 bytes per 16 lanes) --
+// applied on the global side by the lane that fills the position.
+constexpr int kG16MaxUnits = 64;
+
+__device__ __forceinline__ uint2 lds_read_tr16_b64(const uint8_t *p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef short tr_v4s __attribute__((ext_vector_type(4)));
+    const tr_v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3))) *)p);
+    return __builtin_bit_cast(uint2, r);
+#else
+    (void)p;
+    return make_uint2(0u, 0u);
+#endif
+}
+
+template <int DT>
+__global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
+{
+    constexpr int D = 128;
+    constexpr int DOT = DT;
+    constexpr uint32_t kNone = 0xffffffffu;
+    constexpr uint32_t kOnes = DT == DRK_BF16 ? kBf16Ones : kF16Ones;
+    __shared__ __align__(256) uint8_t ring[2][2][4][4096];       // [buffer][K | V][slice = wave that requests it][16 rows x 256 B]
+    __shared__ __align__(16) float o_lds[4][4][D];               // token split: [wave][row of the round][dim], segment ends only
+    __shared__ float mw_lds[4][16], lw_lds[4][16];
+    __shared__ __align__(16) GUnit udesc[kG16MaxUnits];
+    __shared__ __align__(16) uint2 gdesc[kG16MaxUnits][4];
+    __shared__ int s_incl[64], s_len[64], s_gmin[kGMaxGroups];
+
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int g = lane >> 4, c = lane & 15;
+    const int GQ = A.QH / A.KVH;
+    const int nunits = build_units<kG16MaxUnits>(A, udesc, gdesc, s_incl, s_len, s_gmin);
+    if (nunits == 0) return;
+
+    // ---- requests: lane l of load j fills position l % 16 of row 4j + l / 16 of the wave's slice ----
+    const uint32_t dma_row = (uint32_t)((lane >> 4) * 256);
+    const uint32_t kdma_x = (uint32_t)(((lane & 15) ^ (lane >> 4)) << 4);            // K: chunk (l % 16) ^ row, row = 4j | l / 16
+    const uint32_t vdma_x = (uint32_t)(((lane & 15) ^ ((lane >> 4) << 1)) << 4);     // V: slot (l % 16 / 2) ^ (row & 7), row & 7 = 4 (j & 1) | l / 16
+    auto request = [&](int un) {
+        const uint32_t off = (uint32_t)__builtin_amdgcn_readfirstlane((int)gdesc[un][w].x);
+        const uint8_t *base = A.pool_layer + ((size_t)(off == kNone ? 0u : off) << 4);   // no page: any mapped bytes (the rows are masked)
+        const uint32_t lk = lds_addr32(&ring[un & 1][0][w][0]), lv = lds_addr32(&ring[un & 1][1][w][0]);
+        uint32_t kx = kdma_x, vx = vdma_x;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "+v"(kx), "+v"(vx));               // computed here, each time: offsets held across the loop would cost registers
+#endif
+#pragma unroll
+        for (int j = 0; j < 4; j++) lds_dma16(base, (kx ^ (uint32_t)(j << 6)) + dma_row + 1024u * j, lk + 1024 * j);
+        const uint8_t *vbase = base + A.kv_plane;
+#pragma unroll
+        for (int j = 0; j < 4; j++) lds_dma16(vbase, (vx ^ (uint32_t)((j & 1) << 7)) + dma_row + 1024u * j, lv + 1024 * j);
+    };
+
+    // ---- Q^T of the segment as the B operand, in registers: lane (row c, dims 32 kk + 8 g ..), times scale * log2 e
+    // (rounded to the 16-bit type once: a product then arrives as its exponent) ----
+    uint4 qop[4];
+    auto scaled16 = [&](uint32_t v) -> uint32_t {
+        float lo, hi;
+        if constexpr (DT == DRK_BF16) { lo = bf16_lo(v); hi = bf16_hi(v); }
+        else { lo = f16_bits_to_f((uint16_t)(v & 0xffffu)); hi = f16_bits_to_f((uint16_t)(v >> 16)); }
+        return pack16<DOT>(lo * A.scale_log2e, hi * A.scale_log2e);
+    };
+    auto load_q = [&](const GUnit &d) {
+        const int nrows = (d.flags >> 8) & 0xff;
+        const int R = nrows > 16 ? 16 * w + c : c;           // row split: the wave's row group; token split: the one group
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            uint4 v = make_uint4(0u, 0u, 0u, 0u);
+            if (R < nrows) {
+                const int bl = R / GQ, hd = R - bl * GQ;
+                v = *(const uint4 *)(A.q + (size_t)(d.row0 + bl * A.QH + hd) * (D * 2) + kk * 64 + g * 16);
+                v.x = scaled16(v.x); v.y = scaled16(v.y); v.z = scaled16(v.z); v.w = scaled16(v.w);
+            }
+            qop[kk] = v;
+        }
+    };
+
+    // where this lane finds its operands in a slice
+    const uint32_t k_lane = (uint32_t)(c * 256 + (((g ^ c) & 15) << 4));             // row c, chunk g ^ c: k-step 0 (k-step kk: ^ kk << 6)
+    const int vrow = 4 * g + (c >> 2);                                               // transposed read: row 4g + c / 4, dims 16 e + 4 (c % 4) ..
+    const uint32_t v_lane = (uint32_t)(vrow * 256 + 8 * (c & 3)), v_x = (uint32_t)((vrow & 7) << 5);
+
+    w_f32x4 o[8];                                            // O[row 4g + j][dim 16 e + c] = o[e][j]
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    // row c: minus the reference of the exponentials (0 until the row has one), what a score must exceed for the
+    // reference to move (-inf until the row has one), this lane's share of the sum of the weights
+    float negm = 0.0f, thr = -INFINITY, l_lane = 0.0f;
+
+    // The reference moves only when a score exceeds it by more than kLazy (weights stay below 2^kLazy), or for the
+    // row's first tokens; the output rows and the sum are rescaled on those occasions only -- rare enough that the
+    // common path does not even fold the maximum across lanes.  Returns what to take off the scores.
+    auto move_reference = [&](float lmax) -> float {
+        const float mrel = max_lane_groups(lmax);            // row c's maximum over the wave's tokens of this tile
+        const bool move = mrel > thr;
+        const float delta = move ? mrel : 0.0f;
+        const float alpha = thr == -INFINITY ? 1.0f : s_exp2(-delta);     // nothing summed yet: nothing to rescale
+        negm -= delta;
+        thr = move ? kLazy : thr;
+        l_lane *= alpha;
+        // register j of lane group g holds row 4g + j
+        const float a0 = __shfl(alpha, 4 * g), a1 = __shfl(alpha, 4 * g + 1);
+        const float a2 = __shfl(alpha, 4 * g + 2), a3 = __shfl(alpha, 4 * g + 3);
+#pragma unroll
+        for (int e = 0; e < 8; e++) { o[e][0] *= a0; o[e][1] *= a1; o[e][2] *= a2; o[e][3] *= a3; }
+        return delta;
+    };
+
+    request(0);
+    load_q(udesc[0]);
+    for (int it = 0; it < nunits; it++) {
+        const GUnit ud = udesc[it];
+        const int flags = __builtin_amdgcn_readfirstlane(ud.flags);
+        const int tile_lim = __builtin_amdgcn_readfirstlane(ud.tile_lim);
+        const int nrows = (flags >> 8) & 0xff;
+        const bool split_rows = nrows > 16;
+        const bool has_next = it + 1 < nunits;
+        // tokens of slice tg that exist (a slice without a page has none)
+        int limt[4];
+#pragma unroll
+        for (int tg = 0; tg < 4; tg++)
+            limt[tg] = __builtin_amdgcn_readfirstlane((int)gdesc[it][tg].x) == (int)kNone ? 0 : tile_lim - 16 * tg;
+
+        vm_wait_all();                                       // the wave's slices of this unit have landed
+        uint8_t *const kbuf = &ring[it & 1][0][0][0];
+        uint8_t *const vbuf = &ring[it & 1][1][0][0];
+        if (limt[w] < 16) {
+            // rows without a token may hold anything (NaN): their weights are exact zeros, their V rows are cleared
+            // (by the wave that owns the slice, before anyone multiplies)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int row = 4 * j + (lane >> 4);
+                if (row >= limt[w]) *(uint4 *)(vbuf + w * 4096 + row * 256 + (lane & 15) * 16) = make_uint4(0u, 0u, 0u, 0u);
+            }
+        }
+        // The next unit's slices are requested the moment this unit's have landed, so that a request is on its way
+        // at all times.  They overwrite the buffer the unit before was read from -- by every wave, if it was split
+        // by rows: such a unit ends with a barrier (below).  Row split: every wave reads every slice.
+        if (has_next) request(it + 1);
+        if (split_rows) __syncthreads();
+
+        if (split_rows) {
+            // ---- wave w: rows 16 w .. 16 w + 15 against the tile's 64 tokens --------------------------
+            w_f32x4 s[4];                                     // s[tg][j]: row c, token 16 tg + 4 g + j, minus the reference
+#pragma unroll
+            for (int tg = 0; tg < 4; tg++) s[tg] = w_f32x4{negm, negm, negm, negm};
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+#pragma unroll
+                for (int tg = 0; tg < 4; tg++)
+                    s[tg] = w_mfma_qk<DOT>(*(const uint4 *)(kbuf + tg * 4096 + (k_lane ^ (uint32_t)(kk << 6))), qop[kk], s[tg]);
+            if (limt[0] < 16 || limt[1] < 16 || limt[2] < 16 || limt[3] < 16) {
+#pragma unroll
+                for (int tg = 0; tg < 4; tg++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) s[tg][j] = 4 * g + j < limt[tg] ? s[tg][j] : -INFINITY;
+            }
+            const float lmax = fmaxf(fmaxf(max4_asm(s[0][0], s[0][1], s[0][2], s[0][3]), max4_asm(s[1][0], s[1][1], s[1][2], s[1][3])),
+                                     fmaxf(max4_asm(s[2][0], s[2][1], s[2][2], s[2][3]), max4_asm(s[3][0], s[3][1], s[3][2], s[3][3])));
+            if (__builtin_amdgcn_ballot_w64(lmax > thr) != 0) {
+                const float delta = move_reference(lmax);
+#pragma unroll
+                for (int tg = 0; tg < 4; tg++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) s[tg][j] -= delta;
+            }
+            uint2 pk[4];
+#pragma unroll
+            for (int tg = 0; tg < 4; tg++) {
+                pk[tg] = make_uint2(pack16<DOT>(s_exp2(s[tg][0]), s_exp2(s[tg][1])), pack16<DOT>(s_exp2(s[tg][2]), s_exp2(s[tg][3])));
+                // the row's denominator is the sum of the weights the second product multiplies -- the rounded ones
+                l_lane = s_dot2<DOT>(pk[tg].y, kOnes, s_dot2<DOT>(pk[tg].x, kOnes, l_lane));
+            }
+            // O += P V over token pairs of slices: k-index 8 g + j is token 4 g + j of the pair's first slice (j < 4) or second
+#pragma unroll
+            for (int pr = 0; pr < 2; pr++) {
+                const uint4 pa = make_uint4(pk[2 * pr].x, pk[2 * pr].y, pk[2 * pr + 1].x, pk[2 * pr + 1].y);
+                const uint8_t *va = vbuf + (2 * pr) * 4096 + v_lane;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const uint2 b0 = lds_read_tr16_b64(va + (v_x ^ (uint32_t)(e << 5)));
+                    const uint2 b1 = lds_read_tr16_b64(va + 4096 + (v_x ^ (uint32_t)(e << 5)));
+                    o[e] = w_mfma_qk<DOT>(pa, make_uint4(b0.x, b0.y, b1.x, b1.y), o[e]);
+                }
+            }
+            __syncthreads();                                 // every wave is done with this buffer
+        } else {
+            // ---- wave w: its own 16 tokens against the unit's one row group ----------------------------
+            w_f32x4 s = {negm, negm, negm, negm};
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++)
+                s = w_mfma_qk<DOT>(*(const uint4 *)(kbuf + w * 4096 + (k_lane ^ (uint32_t)(kk << 6))), qop[kk], s);
+            if (limt[w] < 16) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) s[j] = 4 * g + j < limt[w] ? s[j] : -INFINITY;
+            }
+            const float lmax = max4_asm(s[0], s[1], s[2], s[3]);
+            if (__builtin_amdgcn_ballot_w64(lmax > thr) != 0) {
+                const float delta = move_reference(lmax);
+#pragma unroll
+                for (int j = 0; j < 4; j++) s[j] -= delta;
+            }
+            const uint2 pk = make_uint2(pack16<DOT>(s_exp2(s[0]), s_exp2(s[1])), pack16<DOT>(s_exp2(s[2]), s_exp2(s[3])));
+            l_lane = s_dot2<DOT>(pk.y, kOnes, s_dot2<DOT>(pk.x, kOnes, l_lane));
+            const uint8_t *va = vbuf + w * 4096 + v_lane;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = w_mfma_pv<DOT>(pk, lds_read_tr16_b64(va + (v_x ^ (uint32_t)(e << 5))), o[e]);
+        }
+
+        // ---- the segment's last tile: leave (o, m, l) per query row for the merge ----------------------
+        if (flags & 2) {
+            const float lw = sum_lane_groups(l_lane);
+            const float mw = thr == -INFINITY ? -INFINITY : -negm;
+            if (split_rows) {
+                // the wave has seen every token of the segment for its rows: no fold
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int R = 16 * w + 4 * g + j;
+                    const float mj = __shfl(mw, 4 * g + j), lj = __shfl(lw, 4 * g + j);
+                    if (R < nrows) {
+                        const int bl = R / GQ, hd = R - bl * GQ;
+                        const size_t pi = (size_t)(ud.row0 + bl * A.QH + hd) * A.Ptot + ud.slot;
+#pragma unroll
+                        for (int e = 0; e < 8; e++) A.part_o[pi * D + 16 * e + c] = o[e][j];
+                        if (c == 0) {
+                            A.part_m[pi] = mj;
+                            A.part_l[pi] = lj;
+                        }
+                    }
+                }
+            } else {
+                // fold the four waves, four rows a round: row 4 r + w is stored by wave w
+                if (lane < 16) { mw_lds[w][lane] = mw; lw_lds[w][lane] = lw; }       // padded rows too: defined values
+                __syncthreads();
+                const int rounds = (nrows + 3) >> 2;
+                for (int r = 0; r < rounds; r++) {
+                    if (r > 0) __syncthreads();                  // the previous round's sums have been read
+                    if (g == r) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const int h = 4 * g + j;
+                            const float M = fmaxf(fmaxf(mw_lds[0][h], mw_lds[1][h]), fmaxf(mw_lds[2][h], mw_lds[3][h]));
+                            const float mo = mw_lds[w][h];
+                            const float f_own = mo == -INFINITY ? 0.0f : s_exp2(mo - M);
+#pragma unroll
+                            for (int e = 0; e < 8; e++) o_lds[w][j][16 * e + c] = o[e][j] * f_own;
+                        }
+                    }
+                    // (m, l) of row 4 r + w over the four waves; read here, before the barrier, because a wave
+                    // that is through with this segment may overwrite its slots for the next one
+                    const int h = 4 * r + w;
+                    const float M = fmaxf(fmaxf(mw_lds[0][h], mw_lds[1][h]), fmaxf(mw_lds[2][h], mw_lds[3][h]));
+                    float L = 0.0f;
+#pragma unroll
+                    for (int ww = 0; ww < 4; ww++) {
+                        const float mm = mw_lds[ww][h];
+                        if (mm != -INFINITY) L = fmaf(lw_lds[ww][h], s_exp2(mm - M), L);
+                    }
+                    __syncthreads();
+                    if (h < nrows) {
+                        const int d = lane * 2;
+                        float acc0 = 0.0f, acc1 = 0.0f;
+#pragma unroll
+                        for (int ww = 0; ww < 4; ww++) { acc0 += o_lds[ww][w][d]; acc1 += o_lds[ww][w][d + 1]; }
+                        const int bl = h / GQ, hd = h - bl * GQ;
+                        const size_t pi = (size_t)(ud.row0 + bl * A.QH + hd) * A.Ptot + ud.slot;
+                        *(float2 *)(A.part_o + pi * D + d) = make_float2(acc0, acc1);
+                        if (lane == 0) {
+                            A.part_m[pi] = M;
+                            A.part_l[pi] = L;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            negm = 0.0f; thr = -INFINITY; l_lane = 0.0f;
+            if (has_next) load_q(udesc[it + 1]);
+        }
+    }
+}
+
+template <int DT, int D, int NG, bool DMA>
+__global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
+{
+    using Geo = StreamGeo<DT, D>;
+    [[maybe_unused]] constexpr bool Q8 = Geo::q8;
+    constexpr int DOT = KvTraits<DT>::dot;
+    constexpr uint32_t kNone = 0xffffffffu;
+    constexpr int QP = D * 2 + 16;                               // LDS pitch of a query row (16-bit values)
+    constexpr int NR = NG * 16;                                  // query rows a unit may serve
+    constexpr int CPR = D * 2 / 16;                              // 16-byte chunks per query row
+    constexpr int RPP = 256 / CPR;                               // rows the workgroup moves per pass
+    constexpr int QPASS = NR / RPP;
+    // K of 16-bit pages goes from global memory straight into LDS (no registers hold it): two buffers of a wave's
+    // 16 token rows, unpadded, 16-byte chunk x of row r at position x ^ r -- applied on the global side by the lane
+    // that fills the position, undone by the reader.  8-bit codes pass through registers (they are widened on the
+    // way) into one buffer of padded rows.
+    constexpr bool DIRECT = DMA && !Q8;
+    constexpr int KBUF = DIRECT ? 16 * D * 2 : 16 * Geo::PITCH;  // one wave's K rows of one tile
+    __shared__ __align__(256) uint8_t k_lds[DIRECT ? 2 : 1][4][KBUF];
+    __shared__ __align__(16) uint8_t q_lds[NR * QP];
+    __shared__ __align__(16) float o_lds[4][8][D];               // [wave][row of the round][dim], segment ends only
+    __shared__ float mw_lds[4][NR], lw_lds[4][NR];
+    __shared__ __align__(16) GUnit udesc[kGMaxUnits];
+    __shared__ __align__(16) uint2 gdesc[kGMaxUnits][4];
+    __shared__ int s_incl[64], s_len[64], s_gmin[kGMaxGroups];
+
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int g = lane >> 4, c = lane & 15;
+    const int GQ = A.QH / A.KVH;
+    const int nunits = build_units<kGMaxUnits>(A, udesc, gdesc, s_incl, s_len, s_gmin);
+    if (nunits == 0) return;
 
     // the 4 K scales and the 4 V scales of tokens 4g..4g+3 (int8 pages)
     auto load_scales = [&](uint2 gd, uint2 &ks, uint2 &vs) {
@@ -259,12 +581,14 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
     auto q_operand = [&](int rg, int kk) -> uint4 { return *(const uint4 *)(q_lds + (rg * 16 + c) * QP + kk * 64 + g * 16); };
 
     w_f32x4 o[NG][Geo::NPV];
-    float m_run[NG], l_lane[NG], ps_lane[NG], qbias[NG];
+    // per row group and row c: minus the reference of the exponentials (0 until the row has one), what a score
+    // must exceed for the reference to move (-inf until the row has one), the sum of the weights
+    float negm[NG], thr[NG], l_lane[NG], ps_lane[NG], qbias[NG];
 #pragma unroll
     for (int rg = 0; rg < NG; rg++) {
 #pragma unroll
         for (int e = 0; e < Geo::NPV; e++) o[rg][e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        m_run[rg] = -INFINITY; l_lane[rg] = 0.0f; ps_lane[rg] = 0.0f; qbias[rg] = 0.0f;
+        negm[rg] = 0.0f; thr[rg] = -INFINITY; l_lane[rg] = 0.0f; ps_lane[rg] = 0.0f; qbias[rg] = 0.0f;
     }
     // int8 pages: the sum of every row's query values, for the code offset
     auto q_bias = [&]() {
@@ -344,8 +668,6 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
         // ---- K: registers -> the wave's LDS rows -> one token row per lane; V: registers -> B operands;
         // then the loads of the next unit's K and V, so that they travel during all of this unit's arithmetic
         if constexpr (DIRECT) vm_wait_all();                    // this unit's K has landed (its V too: requested before it)
-        if (A.dbg & 2) __builtin_amdgcn_s_sleep(8);
-        if (A.dbg & 8) __syncthreads();
         else stage_k<DT, D>(&k_lds[0][w][0], kreg, lane);
         float ks[4] = {1.0f, 1.0f, 1.0f, 1.0f}, vs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
         if (DT == DRK_INT8) {
@@ -373,8 +695,6 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
             else kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
             load_scales(gd, ksr, vsr);
         }
-        if (A.dbg & 16) __builtin_amdgcn_s_sleep(20);
-        if (A.dbg & 32) vm_wait_all();
         // the A operand: dims 32 kk + 8 g .. of token row c of the wave's 16
         const uint8_t *const krows = &k_lds[DIRECT ? (it & 1) : 0][w][0];
         auto k_operand = [&](int kk) -> uint4 {
@@ -391,7 +711,7 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
             w_f32x4 s[N];
 #pragma unroll
             for (int rg = 0; rg < N; rg++) {
-                const float nm = (DT == DRK_INT8 || m_run[rg] == -INFINITY) ? 0.0f : -m_run[rg];
+                const float nm = DT == DRK_INT8 ? 0.0f : negm[rg];
                 s[rg] = w_f32x4{nm, nm, nm, nm};
             }
 #pragma unroll
@@ -404,23 +724,25 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
 #pragma unroll
             for (int rg = 0; rg < N; rg++) {
                 if (DT == DRK_INT8) {                           // codes carry an offset and the token's scale
-                    const float nm = m_run[rg] == -INFINITY ? 0.0f : -m_run[rg];
 #pragma unroll
-                    for (int j = 0; j < 4; j++) s[rg][j] = fmaf(s[rg][j] - qbias[rg], ks[j], nm);
+                    for (int j = 0; j < 4; j++) s[rg][j] = fmaf(s[rg][j] - qbias[rg], ks[j], negm[rg]);
                 }
                 if (partial) {
 #pragma unroll
                     for (int j = 0; j < 4; j++) s[rg][j] = t0 + j < lim ? s[rg][j] : -INFINITY;
                 }
-                // row c's maximum over this wave's 16 tokens, relative to the reference.  The reference moves only
-                // when that exceeds kLazy (weights stay below 2^kLazy) or is the row's first; the output rows and
-                // sums are rescaled on those occasions only.
-                const float mrel = max_lane_groups(max4_of_product(s[rg][0], s[rg][1], s[rg][2], s[rg][3]));
-                const bool move = m_run[rg] == -INFINITY ? mrel > -INFINITY : mrel > kLazy;
-                if (__builtin_amdgcn_ballot_w64(move) != 0) {
+                // The reference moves only when a score exceeds it by more than kLazy (weights stay below 2^kLazy), or
+                // for the row's first tokens (thr = -inf until then); the output rows and sums are rescaled on those
+                // occasions only -- rare enough that the common path does not even fold the maximum across lanes.
+                const float lmax = max4_asm(s[rg][0], s[rg][1], s[rg][2], s[rg][3]);
+                if (__builtin_amdgcn_ballot_w64(lmax > thr[rg]) != 0) {
+                    const float mrel = max_lane_groups(lmax);       // row c's maximum over this wave's 16 tokens
+                    const bool move = mrel > thr[rg];
+                    const bool first = thr[rg] == -INFINITY;
                     const float delta = move ? mrel : 0.0f;
-                    const float alpha = (m_run[rg] == -INFINITY) ? 1.0f : s_exp2(-delta);    // nothing summed yet: nothing to rescale
-                    m_run[rg] = move ? (m_run[rg] == -INFINITY ? mrel : m_run[rg] + mrel) : m_run[rg];
+                    const float alpha = first ? 1.0f : s_exp2(-delta);    // nothing summed yet: nothing to rescale
+                    negm[rg] -= delta;
+                    thr[rg] = move ? kLazy : thr[rg];
 #pragma unroll
                     for (int j = 0; j < 4; j++) s[rg][j] -= delta;
                     l_lane[rg] *= alpha;
@@ -436,14 +758,7 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
                 for (int j = 0; j < 4; j++) p[j] = s_exp2(s[rg][j]);
 #pragma unroll
                 for (int j = 0; j < 4; j++) pw[j] = (DT == DRK_INT8) ? (t0 + j < lim ? p[j] * vs[j] : 0.0f) : p[j];
-                uint2 pk;
-                if constexpr (DOT == DRK_BF16) {
-                    pk.x = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[1]) << 16);
-                    pk.y = (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)pw[3]) << 16);
-                } else {
-                    pk.x = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[0]) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[1]) << 16);
-                    pk.y = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[2]) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)pw[3]) << 16);
-                }
+                const uint2 pk = make_uint2(pack16<DOT>(pw[0], pw[1]), pack16<DOT>(pw[2], pw[3]));
                 pa[rg] = pk;
                 // The row's denominator is the sum of the weights the second product multiplies -- the rounded
                 // ones -- so that numerator and denominator carry the same rounding.  (int8: the product
@@ -454,7 +769,7 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
                     ps_lane[rg] += s_dot2<DOT>(pk.y, kF16Ones, t);
                     l_lane[rg] += (p[0] + p[1]) + (p[2] + p[3]);
                 } else {
-                    l_lane[rg] += s_dot2<DOT>(pk.y, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, s_dot2<DOT>(pk.x, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, 0.0f));
+                    l_lane[rg] = s_dot2<DOT>(pk.y, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, s_dot2<DOT>(pk.x, DOT == DRK_BF16 ? kBf16Ones : kF16Ones, l_lane[rg]));
                 }
             }
             // O += P V; the V operands serve all row groups
@@ -465,12 +780,12 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
 #pragma unroll
                     for (int rg = 0; rg < N; rg++) o[rg][ch * 8 + e] = w_mfma_pv<DOT>(pa[rg], vb[ch][e], o[rg][ch * 8 + e]);
         };
-        if (nga > 1 || (A.dbg & 1)) tile_body(std::integral_constant<int, NG>{});
+        if (nga > 1) tile_body(std::integral_constant<int, NG>{});
         else tile_body(std::integral_constant<int, 1>{});
         // ---- the segment's last tile: fold the four waves, leave (o, m, l) for the merge ----
         if (flags & 2) {
             uint4 qn[QPASS];
-            if (has_next && !(A.dbg & 4)) q_issue(udesc[it + 1], qn);          // the next segment's query rows travel during the fold
+            if (has_next) q_issue(udesc[it + 1], qn);          // the next segment's query rows travel during the fold
             float pwv[NG];
 #pragma unroll
             for (int rg = 0; rg < NG; rg++) {
@@ -478,7 +793,7 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
                 if (rg < nga) {
                     const float lw = sum_lane_groups(l_lane[rg]);
                     if (DT == DRK_INT8) pwv[rg] = sum_lane_groups(ps_lane[rg]);
-                    if (lane < 16) { mw_lds[w][rg * 16 + lane] = m_run[rg]; lw_lds[w][rg * 16 + lane] = lw; }   // padded rows too: defined values
+                    if (lane < 16) { mw_lds[w][rg * 16 + lane] = thr[rg] == -INFINITY ? -INFINITY : -negm[rg]; lw_lds[w][rg * 16 + lane] = lw; }   // padded rows too: defined values
                 }
             }
             __syncthreads();
@@ -549,10 +864,9 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
             for (int rg = 0; rg < NG; rg++) {
 #pragma unroll
                 for (int e = 0; e < Geo::NPV; e++) o[rg][e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                m_run[rg] = -INFINITY; l_lane[rg] = 0.0f; ps_lane[rg] = 0.0f;
+                negm[rg] = 0.0f; thr[rg] = -INFINITY; l_lane[rg] = 0.0f; ps_lane[rg] = 0.0f;
             }
             if (has_next) {
-                if (A.dbg & 4) q_issue(udesc[it + 1], qn);
                 q_store(qn);
                 __syncthreads();
                 q_bias();
@@ -576,16 +890,25 @@ __global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_
     __shared__ fvec red[4][64];
     __shared__ int seg_base[kGMaxGroups + 1], seg_cnt[kGMaxGroups + 1], seg_off[kGMaxGroups + 2], nseg_s;
     __shared__ short slot_of[kGMaxPieces];
+    __shared__ int scan_s[3];
     const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * VEC;
-    if (threadIdx.x == 0) {
-        int excl = 0, total = 0, nt_b = 0;
-        for (int i = 0; i < A.B; i++) {
-            const int len = A.seq_lens[i];
-            const int nt = len > 0 ? max((len + kSTile - 1) / kSTile - A.b_start[i], 0) : 0;
-            if (i < b) excl += nt;
-            if (i == b) nt_b = nt;
-            total += nt;
+    // tail tiles of every branch: one lane each (one round of loads), folded by the first wave
+    if (wv == 0) {
+        const int len = lane < A.B ? A.seq_lens[lane] : 0;
+        const int nt = len > 0 ? max((len + kSTile - 1) / kSTile - A.b_start[lane], 0) : 0;
+        int incl = nt;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
         }
+        const int total_all = __builtin_amdgcn_readlane(incl, 63);
+        const int incl_b = __shfl(incl, b), nt_bb = __shfl(nt, b);
+        if (lane == 0) { scan_s[0] = incl_b - nt_bb; scan_s[1] = total_all; scan_s[2] = nt_bb; }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int excl = scan_s[0], total = scan_s[1], nt_b = scan_s[2];
         const int T = A.group_units + total * A.KVH;
         int n = 0, off = 0;
         if (T > 0) {
@@ -692,8 +1015,12 @@ struct GroupPlan {
 // one another from token 0 without gap or overlap (then every token of a branch is read exactly once:
 // by one range or by the branch's tail).  Ranges are cut down to whole 64-token tiles; what a range
 // loses at its end, the range or tail behind it reads.
+// units one workgroup may own: the descriptor table of the kernel that takes the call
+static int group_max_units(const Lay &a) { return a.E == 2 && g_grouped_mode != 2 ? kG16MaxUnits : kGMaxUnits; }
+
 static int plan_groups(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_in, GroupPlan *P)
 {
+    const int max_units = group_max_units(a);
     if (n_in < 0 || n_in > kGMaxGroups) return fail(DRK_ERR_INVALID, "decode_grouped: %d groups (0..%d)", n_in, kGMaxGroups);
     if (n_in > 0 && !groups) return fail(DRK_ERR_INVALID, "decode_grouped: groups is NULL");
     const int GQ = a.QH / a.KVH;
@@ -737,7 +1064,7 @@ static int plan_groups(const Lay &a, int B, int max_seq_len, const drk_prefix_gr
     for (int b = B; b < 64; b++) P->b_start[b] = P->b_slot[b] = 0;
     long G = t_upper < kGWgs ? t_upper : kGWgs;
     if (G < 1) G = 1;
-    if ((t_upper + G - 1) / G > kGMaxUnits) G = (t_upper + kGMaxUnits - 1) / kGMaxUnits;   // descriptor table size
+    if ((t_upper + G - 1) / G > max_units) G = (t_upper + max_units - 1) / max_units;   // descriptor table size
     P->grid = (int)G;
     // a run of n tiles of one kv head meets at most min(n, G / KVH + 2) workgroups
     const int cap = (int)(G / a.KVH) + 2;
@@ -776,7 +1103,8 @@ size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_
     const int max_tiles = (max_seq_len + kSTile - 1) / kSTile;
     long G = kGWgs;
     const long t_upper = (long)a.KVH * B * max_tiles;
-    if ((t_upper + G - 1) / G > kGMaxUnits) G = (t_upper + kGMaxUnits - 1) / kGMaxUnits;
+    const int max_units = kG16MaxUnits;                          // the smaller table gives the larger grid, and so the larger bound
+    if ((t_upper + G - 1) / G > max_units) G = (t_upper + max_units - 1) / max_units;
     long cap = G / a.KVH + 2;
     if (cap > max_tiles) cap = max_tiles;
     long P = (long)(max_depth + 1) * cap;
@@ -826,24 +1154,26 @@ int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *poo
     A.head_stride = a.head_stride; A.kv_plane = a.kv_plane; A.block_stride = a.block_stride;
     A.scale_plane = a.scale_plane; A.row_bytes = a.row_bytes;
     A.scale_log2e = scale * kSLog2e;
-    A.dbg = getenv("DRK_GDBG") ? atoi(getenv("DRK_GDBG")) : 0;
     for (int k = 0; k < kGMaxGroups; k++) A.seg[k] = k < P.ngroups ? P.seg[k] : GSeg{0, 0, 0, 0, 0, 0x7fffffff};
     for (int b = 0; b < 64; b++) { A.b_start[b] = P.b_start[b]; A.b_slot[b] = P.b_slot[b]; }
     hipStream_t st = (hipStream_t)stream;
-    const bool dma = g_grouped_mode != 2;
+    // 16-bit pages: the tile in LDS, rows dealt to the waves; 8-bit pages (and, as a cross-check, 16-bit pages in
+    // diagnostic mode 2): tokens dealt to the waves, K and V through registers
+    const bool tile16 = a.E == 2 && g_grouped_mode != 2;
     switch (a.dtype) {
     case DRK_F16:
-        if (dma) hipLaunchKernelGGL((decode_group_kernel<DRK_F16, 128, 4, true>), dim3(P.grid), dim3(256), 0, st, A);
+        if (tile16) hipLaunchKernelGGL((decode_group16_kernel<DRK_F16>), dim3(P.grid), dim3(256), 0, st, A);
         else hipLaunchKernelGGL((decode_group_kernel<DRK_F16, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A);
         break;
     case DRK_BF16:
-        if (dma) hipLaunchKernelGGL((decode_group_kernel<DRK_BF16, 128, 4, true>), dim3(P.grid), dim3(256), 0, st, A);
+        if (tile16) hipLaunchKernelGGL((decode_group16_kernel<DRK_BF16>), dim3(P.grid), dim3(256), 0, st, A);
         else hipLaunchKernelGGL((decode_group_kernel<DRK_BF16, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A);
         break;
     case DRK_INT8: hipLaunchKernelGGL((decode_group_kernel<DRK_INT8, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A); break;
     default: hipLaunchKernelGGL((decode_group_kernel<DRK_FP8_E4M3, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A); break;
     }
     DRK_LAUNCH_CHECK("decode_group_kernel");
+    if (g_skip_merge) return DRK_OK;
     hipLaunchKernelGGL(group_merge_kernel<128>, dim3(a.QH, B), dim3(256), 0, st, A, (uint16_t *)out, P.grid,
                        (const uint16_t *)gate, gate_stride);
     DRK_LAUNCH_CHECK("group_merge_kernel");

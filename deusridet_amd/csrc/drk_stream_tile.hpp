@@ -247,7 +247,7 @@ __device__ __forceinline__ uint32_t lds_addr32(const void *p)
 __device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_offset, uint32_t lds_addr)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" : : "v"(lane_offset), "s"(base), "s"(lds_addr) : "memory", "m0");
 #else
     (void)base; (void)lane_offset; (void)lds_addr;
 #endif

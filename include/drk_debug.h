@@ -38,15 +38,10 @@ void drk_debug_set_prefix_stream(int on);
 /* Diagnostic: 1 = drk_paged_decode_attention_shared never takes the grouped kernel (one launch over
  * shared and private tiles) but always the prefix pass + tail kernel pair; 0 = the library's choice. */
 void drk_debug_set_grouped_decode(int mode);
-/* Diagnostic for benchmarks: while on, every decode launch (up to 256 per
- * session; switching it on starts a new session) records a HIP event on its
- * stream right before and right after the split-K partial kernel; the merge
- * kernel is outside the pair.  drk_debug_decode_kernel_times waits for the pairs
- * recorded so far and returns their elapsed milliseconds.  Launch back to back
- * (no host sync in between) so that the queue stays busy and the pairs bracket
- * the kernel tightly.  Process-wide. */
-void drk_debug_time_decode_kernel(int on);
-int  drk_debug_decode_kernel_times(float *ms, int cap, int *count);
+/* Measurement aid for benchmarks: while on, the decode entry points launch the kernels that read the
+ * pages and leave their partial results unmerged (no merge kernel: out is not written), so that an event
+ * pair the caller records around a call brackets the dominant kernel(s) alone.  Process-wide. */
+void drk_debug_set_skip_merge(int on);
 /* Diagnostic: extra dynamic LDS bytes per decode workgroup (lowers occupancy). */
 void drk_debug_set_decode_lds_pad(int bytes);
 /* Tuning: which prefill chunks run with the context split over the chip (they must stand behind 2 048 tokens
@@ -71,6 +66,38 @@ void drk_debug_set_quant_append_pairs(int on);
  * scales) and adds the number of disagreements to *d_mismatches (device memory, 4 bytes, zeroed
  * by the caller).  Asynchronous on `stream`. */
 int drk_debug_check_int8_scale_math(unsigned *d_mismatches, void *stream);
+
+/* ---- probes: what the part reaches on its own (bench.py reports them beside the kernels) ---- */
+/* Measurement aid (precedent tools/probe_bw.cu:74-97): sustained GB/s of a plain
+ * 128-bit streaming read of `bytes` of device memory on the default stream,
+ * 5 warm-up + `iters` timed passes; d_sink is 4 bytes of device memory.
+ * Synchronises. */
+int drk_probe_read_bandwidth(const void *d_ptr, size_t bytes, int iters, void *d_sink, float *gbps);
+/* Same, with the decode kernels' access pattern: aligned granules of granule_bytes (a multiple of
+ * 4096; 4096 = one 16-token K or V run of one kv head at head_dim 128, 16-bit) read in a
+ * scattered order over the largest power-of-two number of granules that fits in `bytes`. */
+int drk_probe_read_bandwidth_permuted(const void *d_ptr, size_t bytes, int granule_bytes, int iters,
+                                      void *d_sink, float *gbps);
+/* Measurement aid: dense bf16 TFLOP/s a registers-only v_mfma_f32_32x32x16_bf16 loop sustains
+ * (8 waves per CU, four independent accumulator chains per wave, no memory traffic): the rate
+ * the matrix cores of the part reach on their own.  d_sink is 4 bytes of device memory.
+ * Synchronises. */
+int drk_probe_mfma_rate(int iters, void *d_sink, float *tflops);
+/* Measurement aid: how much of one wave's matrix products hides another wave's vector work on
+ * the same SIMD.  One workgroup of eight waves per CU; waves 4-7 issue 32x32x16 bf16 products,
+ * waves 0-3 a softmax-like mix of vector instructions (exp, fma, max3, pack), balanced to the
+ * same issue time.  Reports the milliseconds of a launch with only the matrix waves working,
+ * only the vector waves, and both: perfect overlap gives both = max, none gives the sum.
+ * d_sink is 4 bytes of device memory.  Synchronises. */
+int drk_probe_mfma_valu_coexec(int iters, void *d_sink, float *ms_mfma, float *ms_valu, float *ms_both);
+/* Measurement aid: the same question for two waves that take turns, as the halves of a two-phase
+ * prefill workgroup do: between two workgroup barriers waves 0-3 issue 32 products while waves 4-7
+ * issue vector instructions of ONE kind (about 16 clocks' worth per product), then the roles swap.
+ * op: 0 v_exp_f32, 1 v_fma_f32, 2 v_dot2_f32_bf16, 3 v_cvt_pk_bf16_f32, 4 v_max3_f32,
+ * 5 v_cmp_gt_f32 (writes vcc), 6 v_permlane32_swap_b32, 7 s_nop 3.  Reports the milliseconds of a
+ * launch with only the products, only the vector turns, and both; (both - products) / vectors is
+ * the share of the vector time that stays visible.  d_sink is 4 bytes of device memory.  Synchronises. */
+int drk_probe_phase_coexec(int op, int iters, void *d_sink, float *ms_products, float *ms_vectors, float *ms_both);
 
 #ifdef __cplusplus
 }

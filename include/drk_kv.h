@@ -69,37 +69,6 @@ const char *drk_last_error(void);
 const char *drk_strerror(int code);
 int         drk_device_count(int *count);
 
-/* Measurement aid (precedent tools/probe_bw.cu:74-97): sustained GB/s of a plain
- * 128-bit streaming read of `bytes` of device memory on the default stream,
- * 5 warm-up + `iters` timed passes; d_sink is 4 bytes of device memory.
- * Synchronises. */
-int drk_probe_read_bandwidth(const void *d_ptr, size_t bytes, int iters, void *d_sink, float *gbps);
-/* Same, with the decode kernels' access pattern: aligned granules of granule_bytes (a multiple of
- * 4096; 4096 = one 16-token K or V run of one kv head at head_dim 128, 16-bit) read in a
- * scattered order over the largest power-of-two number of granules that fits in `bytes`. */
-int drk_probe_read_bandwidth_permuted(const void *d_ptr, size_t bytes, int granule_bytes, int iters,
-                                      void *d_sink, float *gbps);
-/* Measurement aid: dense bf16 TFLOP/s a registers-only v_mfma_f32_32x32x16_bf16 loop sustains
- * (8 waves per CU, four independent accumulator chains per wave, no memory traffic): the rate
- * the matrix cores of the part reach on their own.  d_sink is 4 bytes of device memory.
- * Synchronises. */
-int drk_probe_mfma_rate(int iters, void *d_sink, float *tflops);
-/* Measurement aid: how much of one wave's matrix products hides another wave's vector work on
- * the same SIMD.  One workgroup of eight waves per CU; waves 4-7 issue 32x32x16 bf16 products,
- * waves 0-3 a softmax-like mix of vector instructions (exp, fma, max3, pack), balanced to the
- * same issue time.  Reports the milliseconds of a launch with only the matrix waves working,
- * only the vector waves, and both: perfect overlap gives both = max, none gives the sum.
- * d_sink is 4 bytes of device memory.  Synchronises. */
-int drk_probe_mfma_valu_coexec(int iters, void *d_sink, float *ms_mfma, float *ms_valu, float *ms_both);
-/* Measurement aid: the same question for two waves that take turns, as the halves of a two-phase
- * prefill workgroup do: between two workgroup barriers waves 0-3 issue 32 products while waves 4-7
- * issue vector instructions of ONE kind (about 16 clocks' worth per product), then the roles swap.
- * op: 0 v_exp_f32, 1 v_fma_f32, 2 v_dot2_f32_bf16, 3 v_cvt_pk_bf16_f32, 4 v_max3_f32,
- * 5 v_cmp_gt_f32 (writes vcc), 6 v_permlane32_swap_b32, 7 s_nop 3.  Reports the milliseconds of a
- * launch with only the products, only the vector turns, and both; (both - products) / vectors is
- * the share of the vector time that stays visible.  d_sink is 4 bytes of device memory.  Synchronises. */
-int drk_probe_phase_coexec(int op, int iters, void *d_sink, float *ms_products, float *ms_vectors, float *ms_both);
-
 /* ---- layout arithmetic (host only, no GPU needed) --------------------- */
 /* block_pool.cpp:23-39: strides; block_pool.cpp:28-32: budget -> max_blocks */
 int drk_kv_layout_check(const drk_kv_layout *g);

@@ -22,9 +22,10 @@ def declared(header, prefix):
 def test_drk_kv_symbols_are_exported_and_bound():
     names = declared("drk_kv.h", "drk_")
     assert len(names) > 30
-    assert not [n for n in names if n.startswith("drk_debug_")], "diagnostic switches belong in drk_debug.h"
-    debug = declared("drk_debug.h", "drk_debug_")
-    assert len(debug) >= 9
+    assert not [n for n in names if n.startswith(("drk_debug_", "drk_probe_"))], \
+        "diagnostic switches and measurement probes belong in drk_debug.h, out of the boundary a drop-in binds"
+    debug = declared("drk_debug.h", "drk_debug_") + declared("drk_debug.h", "drk_probe_")
+    assert len(debug) >= 14
     names = sorted(names + debug)
     raw = C.CDLL(cabi.LIB_PATH)
     for n in names:
