@@ -80,6 +80,9 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "
                                                             "replaying one captured HIP graph per step")
     ap.add_argument("--no-cascade", action="store_true", help="config 3: read the shared prefix once per branch")
+    ap.add_argument("--forks", choices=["tree", "prefix"], default="tree",
+                    help="config 3: branches fork from the prefix or from one another at random block boundaries (tree), "
+                         "or all from the prefix's end (prefix)")
     ap.add_argument("--shared-kernel", choices=["auto", "pair"], default="auto",
                     help="config 3: how shared pages are read: auto = one launch over shared and private tiles where the "
                          "geometry allows; pair = always the prefix pass followed by the tail kernel")

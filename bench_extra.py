@@ -160,18 +160,41 @@ def config3(args):
 
     for p0 in range(0, prefix, chunk):
         bulk(0, p0, chunk)
-    t0 = time.perf_counter()
-    forks = []
-    for i in range(NBR):
-        # block boundaries, except every fourth fork lands inside a block (forces a copy-on-write)
-        fp = prefix if i % 4 else prefix - int(rng.integers(1, bs))
-        forks.append(cm.fork_branch(0, fp))
-    fork_ns = (time.perf_counter() - t0) / NBR * 1e9
-    assert min(forks) > 0
-    for b, n in zip(forks, private):
-        base = cm.seq_len(b)
-        for p0 in range(0, int(n), chunk):
-            bulk(b, base + p0, min(chunk, int(n) - p0))
+    # The fork tree.  "prefix": every branch forks from the prefix's end.  "tree": a branch forks from the prefix or
+    # from an earlier branch, at a random block boundary of what that branch holds beyond the prefix, so the 16
+    # branches share the prefix and subsets of them share what they wrote before they split again.  Every fourth
+    # fork lands inside a block instead (forces a copy-on-write).  Branches are created parents first, then their
+    # children from the latest fork point to the earliest, so that branches which share pages are neighbours in the
+    # table.
+    tree = getattr(args, "forks", "tree") == "tree"
+    parent = [-1] + [int(rng.integers(-1, i)) if tree else -1 for i in range(1, NBR)]
+    forks, fork_points, order, fork_s = [], [], [], 0.0
+
+    def grow(node, par_branch, fp):
+        nonlocal fork_s
+        if node % 4 == 0:
+            fp -= int(rng.integers(1, bs))
+        t0 = time.perf_counter()
+        b = cm.fork_branch(par_branch, fp)
+        fork_s += time.perf_counter() - t0
+        assert b > 0
+        forks.append(b)
+        fork_points.append(fp)
+        order.append(node)
+        for p0 in range(0, int(private[node]), chunk):
+            bulk(b, fp + p0, min(chunk, int(private[node]) - p0))
+        descend(node, b)
+
+    def descend(node, branch):
+        held = cm.seq_len(branch)
+        kids = [(prefix + bs * int(rng.integers(0, (held - prefix) // bs + 1)) if branch else prefix, c)
+                for c in range(node + 1, NBR) if parent[c] == node]
+        for fp, c in sorted(kids, key=lambda k: -k[0]):           # the latest fork first
+            grow(c, branch, fp)
+
+    descend(-1, 0)
+    fork_ns = fork_s / NBR * 1e9
+    parent = [-1 if parent[n] < 0 else order.index(parent[n]) for n in order]          # in table-row numbering
     lens0 = np.array([cm.seq_len(b) for b in forks], dtype=np.int32)
     g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
     B = NBR
@@ -182,9 +205,11 @@ def config3(args):
     out = torch.zeros(L, B, QH, D, device="cuda", dtype=torch.bfloat16)
     max_ctx = int(lens0.max()) + W + K + 1
     cascade = not getattr(args, "no_cascade", False)
-    wsb = lib.drk_decode_shared_workspace_bytes(C.byref(g), B, max_ctx, prefix)
+    grouped = cascade and getattr(args, "shared_kernel", "auto") != "pair"       # else: the common prefix alone, as a kernel pair
+    wsb = max(lib.drk_decode_shared_workspace_bytes(C.byref(g), B, max_ctx, prefix),
+              lib.drk_decode_grouped_workspace_bytes_max(C.byref(g), B, max_ctx, cabi.MAX_PREFIX_GROUPS) if grouped else 0)
     ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
-    shared_now = [0]
+    shared_now, groups_now = [0], [[], cabi.prefix_groups([])]
     dpos = torch.zeros(B, dtype=torch.int32, device="cuda")
     dlen = torch.zeros(B, dtype=torch.int32, device="cuda")
     # the forked branches' rows are consecutive in the device table: branch ids forks[0]..forks[-1]
@@ -192,6 +217,16 @@ def config3(args):
     dtabs = C.c_void_p(cm.d_block_table(forks[0]))
     qrow, krow = B * QH * D * 2, B * KVH * D * 2
     ensure_ns, evicted, evict_ns = [], 0, 0.0
+
+    def attend(l, dl):
+        if grouped:
+            cabi.call("drk_paged_decode_attention_grouped", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr,
+                      dtabs, stride, dl, B, max_ctx, groups_now[1], len(groups_now[0]), C.c_void_p(out.data_ptr() + l * qrow),
+                      l, float(scale), cabi.BF16, None, 0, cabi.p(ws), wsb, sp)
+        else:
+            cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr,
+                      dtabs, stride, dl, B, max_ctx, shared_now[0], C.c_void_p(out.data_ptr() + l * qrow), l,
+                      float(scale), cabi.BF16, cabi.p(ws), wsb, sp)
 
     def step(s, lens):
         nonlocal evicted, evict_ns
@@ -209,14 +244,15 @@ def config3(args):
             evict_ns += (time.perf_counter() - t) * 1e9
         cm.sync_block_table(sp)                               # COW copies, then table deltas
         shared_now[0] = cm.common_prefix_tokens(forks) if cascade else 0
+        if grouped:
+            groups_now[0] = cm.common_prefix_groups(forks, 64 // (QH // KVH), 256, cabi.MAX_PREFIX_GROUPS)
+            groups_now[1] = cabi.prefix_groups(groups_now[0])
         dpos.copy_(torch.from_numpy(lens))
         dlen.copy_(torch.from_numpy(lens + 1))
         for l in range(L):
             cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, cabi.p(dpos), B, l, 1,
                       C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
-            cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr,
-                      dtabs, stride, cabi.p(dlen), B, max_ctx, shared_now[0], C.c_void_p(out.data_ptr() + l * qrow), l,
-                      float(scale), cabi.BF16, cabi.p(ws), wsb, sp)
+            attend(l, cabi.p(dlen))
         for i, b in enumerate(forks):
             cm.set_seq_len(b, int(lens[i]) + 1)
 
@@ -237,13 +273,19 @@ def config3(args):
     unique_tokens = cm.gpu_blocks_used() * bs
     value = logical * per_tok * L / (total_ms * 1e-3) / 1e9
     dl = cabi.p(dlen)
-    ker_ms = _timed_decode(lib, cabi, lambda i: cabi.call(
-        "drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + (i % L) * qrow), pool_ptr, dtabs,
-        stride, dl, B, max_ctx, shared_now[0], C.c_void_p(out.data_ptr() + (i % L) * qrow), i % L, float(scale),
-        cabi.BF16, cabi.p(ws), wsb, sp), 60)
+    ker_ms = _timed_decode(lib, cabi, lambda i: attend(i % L, dl), 60)
     launch_logical = int(lens.sum()) * per_tok
-    # bytes the launch must fetch: shared pages once, private pages once each
-    launch_unique = (shared_now[0] + int((lens - shared_now[0]).sum())) * per_tok
+    # bytes the launch must fetch: every physical page some branch reads, once, up to the last token read in it
+    held = {}
+    for b, n in zip(forks, lens):
+        tab = cm.h_block_table(b)
+        for k in range((int(n) + bs - 1) // bs):
+            if tab[k] >= 0:
+                held[int(tab[k])] = max(held.get(int(tab[k]), 0), min(bs, int(n) - k * bs))
+    launch_unique = sum(held.values()) * per_tok
+    # what the launch streams once: the ranges it was given as groups, and every branch's remainder
+    in_groups = sum((e - b0) // 64 * 64 * (nb - 1) for _, nb, b0, e in groups_now[0]) if grouped else shared_now[0] // 64 * 64 * (B - 1)
+    launch_streamed = launch_logical - in_groups * per_tok
     ach = launch_unique / (ker_ms * 1e-3) / 1e9
     value_unique = value * launch_unique / launch_logical
     return {
@@ -255,6 +297,8 @@ def config3(args):
                                f"value counts LOGICAL bytes (every branch's whole context); shared pages streamed "
                                f"{'once for all branches' if cascade else 'once per branch'}",
                    "branches": B, "layers": L, "ctx_final": [int(x) for x in lens], "shared_tokens": int(shared_now[0]),
+                   "forks": "tree" if tree else "prefix", "fork_parent": parent, "fork_points": fork_points,
+                   "shared_ranges": [list(x) for x in groups_now[0]] if grouped else [[0, B, 0, int(shared_now[0])]],
                    "pool_blocks": NB},
         "logical_GB_per_layer_step": round(launch_logical / 1e9, 3),
         "unique_GB_per_layer_step": round(launch_unique / 1e9, 3),
@@ -263,12 +307,16 @@ def config3(args):
         "us_per_step": round(total_ms / K * 1e3, 1), "tokens_per_s": round(B * K / (total_ms * 1e-3), 1),
         "host_ns": {"fork_branch": round(fork_ns), "ensure_blocks_for": round(float(np.mean(ensure_ns))),
                     "evict_per_block": round(evict_ns / max(evicted, 1)), "blocks_evicted": int(evicted)},
-        "roofline": {"kernel": "prefix_stream_kernel<bf16> + decode_stream_kernel<bf16>", "bound": "hbm",
+        "roofline": {"kernel": "decode_group16_kernel<bf16>" if grouped else
+                               "prefix_stream_kernel<bf16> + decode_stream_kernel<bf16>", "bound": "hbm",
                      "achieved": round(ach, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
                      "avg_launch_us": round(ker_ms * 1e3, 2), "bytes_per_launch": launch_unique,
-                     "note": "UNIQUE bytes (shared pages counted once); the pair prefill_mfma_kernel<shared> + "
-                             "decode_stream_kernel is timed as one unit"},
+                     "streamed_bytes_per_launch": launch_streamed,
+                     "note": "DISTINCT bytes: every physical page some branch reads, counted once.  streamed_bytes is what "
+                             "the launch reads given the shared ranges it was handed (ranges under 256 tokens and what "
+                             "rounding to 64-token tiles cuts off are read once per branch).  The merge is not in "
+                             "avg_launch_us" + ("" if grouped else "; the prefix pass and the tail kernel are timed as one unit")},
         "cpu_baseline": None,
     }
 
@@ -621,6 +669,51 @@ def _shuffled_rows(rng, NB, nblk_per_row):
     return tab, stride, perm[o:]
 
 
+def _fork_tree(rng, n_blocks, prefix, private, bs, tree, per_group):
+    """Block tables of len(private) branches over one prefix, built by a bookkeeping-only CacheManager (forks and the
+    shared ranges are the host classes' own), with the page ids sent through a random permutation of the pool.
+    Returns (tables [B, stride], lengths, fork points, parents, shared ranges)."""
+    from deusridet_amd import cabi, host
+    B = len(private)
+    cm = host.CacheManager()
+    assert cm.init_detached(n_blocks, bs, None, B + 1), "CacheManager.init_detached failed"
+    assert cm.ensure_blocks_for_range(0, 0, prefix)
+    cm.set_seq_len(0, prefix)
+    parent = [-1] + [int(rng.integers(-1, i)) if tree else -1 for i in range(1, B)]
+    ids, points, order = [], [], []
+
+    def grow(node, par_branch, fp):
+        b = cm.fork_branch(par_branch, fp)
+        assert b > 0
+        if private[node]:
+            assert cm.ensure_blocks_for_range(b, fp, int(private[node]))
+        cm.set_seq_len(b, fp + int(private[node]))
+        ids.append(b)
+        points.append(fp)
+        order.append(node)
+        descend(node, b)
+
+    def descend(node, branch):
+        # the children of a node, the latest fork first: then branches that share pages are neighbours in the table
+        held = cm.seq_len(branch)
+        kids = [(prefix + bs * int(rng.integers(0, (held - prefix) // bs + 1)) if branch else prefix, c)
+                for c in range(node + 1, B) if parent[c] == node]
+        for fp, c in sorted(kids, key=lambda k: -k[0]):
+            grow(c, branch, fp)
+
+    descend(-1, 0)
+    perm = rng.permutation(n_blocks).astype(np.int32)
+    lens = np.array([cm.seq_len(b) for b in ids], dtype=np.int32)
+    stride = (int(lens.max()) + bs - 1) // bs + 1
+    tab = np.full((B, stride), -1, dtype=np.int32)
+    for i, b in enumerate(ids):
+        row = cm.h_block_table(b)[:stride]
+        tab[i, :len(row)] = np.where(row >= 0, perm[np.maximum(row, 0)], -1)
+    groups = cm.common_prefix_groups(ids, per_group, 256, cabi.MAX_PREFIX_GROUPS)
+    parent_row = [-1 if parent[n] < 0 else order.index(parent[n]) for n in order]      # in table-row numbering
+    return tab, lens, points, parent_row, groups
+
+
 def kernel_fractions(buf, seed=11):
     """buf: a torch uint8 device tensor of at least 16 GiB that may be overwritten."""
     import torch
@@ -721,87 +814,115 @@ def kernel_fractions(buf, seed=11):
             "four source sets in rotation" % (m, L, code))
     del srcs
 
-    # ---- config 3: 65 536-token prefix shared by 16 branches + private tails U{0..4096} -------------------
-    L, B, prefix = 2, 16, 65536
+    # ---- config 3: 65 536-token prefix shared by 16 branches + private tokens U{0..4096}, 36 layers of pages ----
+    # Two draws of the fork points: every branch from the prefix's end, and a tree (a branch forks from the prefix or
+    # from an earlier branch at a random block boundary of what that branch wrote).
+    L, B, prefix = 36, 16, 65536
     NB = fit_blocks(L, cabi.BF16, 200000)
     g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
-    tails = rng.integers(0, 4097, size=B)
-    rows, stride, _ = _shuffled_rows(rng, NB, [prefix // bs] + [int(t + bs - 1) // bs + 1 for t in tails])
-    stride = prefix // bs + max(int(t + bs - 1) // bs + 1 for t in tails) + 1
-    tab = np.full((B, stride), -1, dtype=np.int32)
-    for b in range(B):
-        nt = int(tails[b] + bs - 1) // bs + 1
-        tab[b, :prefix // bs] = rows[0, :prefix // bs]                            # the same physical pages in every row
-        tab[b, prefix // bs:prefix // bs + nt] = rows[1 + b, :nt]
-    dtab = torch.from_numpy(tab).cuda()
-    fill(g, C.c_void_p(dtab[0].data_ptr()), prefix, L, False)
-    # private tails: appended past the prefix through each branch's own row
-    for b in range(B):
-        n = int(tails[b])
-        if n:
-            k = (torch.randn(L, n, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
-            v = (torch.randn(L, n, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
-            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), C.c_void_p(dtab[b].data_ptr()), 0, L, prefix, n, cabi.p(k),
-                      cabi.p(v), cabi.BF16, sp)
-            torch.cuda.synchronize()
-    lens = (prefix + tails).astype(np.int32)
-    dlen = torch.from_numpy(lens).cuda()
-    max_ctx = int(lens.max())
-    q = (torch.randn(L, B, QH, D, device="cuda") * 0.5).to(torch.bfloat16)
-    out = torch.zeros_like(q)
-    wsb = lib.drk_decode_shared_workspace_bytes(C.byref(g), B, max_ctx, prefix)
-    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
-    row = B * QH * D * 2
+    per_tok = 2 * KVH * D * 2
+    for key, tree in (("config3_shared_prefix", False), ("config3_fork_tree", True)):
+        private = rng.integers(0, 4097, size=B)
+        tab, lens, points, parent, groups = _fork_tree(rng, NB, prefix, private, bs, tree, 64 // (QH // KVH))
+        stride = tab.shape[1]
+        dtab = torch.from_numpy(tab).cuda()
+        fill(g, C.c_void_p(dtab[0].data_ptr()), prefix, L, False, chunk=4096)
+        for b in range(B):                                                        # private tokens, through the branch's own row
+            n = int(lens[b]) - points[b]
+            if n:
+                k = (torch.randn(L, n, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+                v = (torch.randn(L, n, KVH, D, device="cuda") * 0.5).to(torch.bfloat16)
+                cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), C.c_void_p(dtab[b].data_ptr()), 0, L, points[b], n,
+                          cabi.p(k), cabi.p(v), cabi.BF16, sp)
+                torch.cuda.synchronize()
+        dlen = torch.from_numpy(lens).cuda()
+        max_ctx = int(lens.max())
+        q = (torch.randn(L, B, QH, D, device="cuda") * 0.5).to(torch.bfloat16)
+        out = torch.zeros_like(q)
+        wsb = max(lib.drk_decode_shared_workspace_bytes(C.byref(g), B, max_ctx, prefix),
+                  lib.drk_decode_grouped_workspace_bytes_max(C.byref(g), B, max_ctx, cabi.MAX_PREFIX_GROUPS))
+        ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+        row = B * QH * D * 2
+        garr = cabi.prefix_groups(groups)
 
-    def shared_one(i):
-        l = i % L
-        cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * row), cabi.p(buf), cabi.p(dtab),
-                  stride, cabi.p(dlen), B, max_ctx, prefix, C.c_void_p(out.data_ptr() + l * row), l, scale, cabi.BF16,
-                  cabi.p(ws), wsb, sp)
+        def shared_one(i):
+            l = i % L
+            if tree:
+                cabi.call("drk_paged_decode_attention_grouped", C.byref(g), C.c_void_p(q.data_ptr() + l * row), cabi.p(buf),
+                          cabi.p(dtab), stride, cabi.p(dlen), B, max_ctx, garr, len(groups), C.c_void_p(out.data_ptr() + l * row),
+                          l, scale, cabi.BF16, None, 0, cabi.p(ws), wsb, sp)
+            else:
+                cabi.call("drk_paged_decode_attention_shared", C.byref(g), C.c_void_p(q.data_ptr() + l * row), cabi.p(buf),
+                          cabi.p(dtab), stride, cabi.p(dlen), B, max_ctx, prefix, C.c_void_p(out.data_ptr() + l * row), l, scale,
+                          cabi.BF16, cabi.p(ws), wsb, sp)
 
-    def shared_call(n):
-        for i in range(n):
+        ker_ms = _timed_decode(lib, cabi, shared_one, 72)                         # without the merge
+        for i in range(6):
             shared_one(i)
-
-    pair_ms = _timed_decode(lib, cabi, shared_one, 40)                           # prefix pass + tails, without the merge
-    a0, a1 = ev(), ev()
-    a0.record(stream)
-    shared_call(40)
-    a1.record(stream)
-    torch.cuda.synchronize()
-    call_ms = a0.elapsed_time(a1) / 40
-    distinct = (prefix + int(tails.sum())) * 2 * KVH * D * 2
-    res["config3_shared_prefix"] = _entry(
-        "prefix_stream_kernel<bf16> + decode_stream_kernel<bf16>", "hbm", distinct, pair_ms,
-        "config 3: 65536-token prefix shared by 16 branches + private tails U{0..4096} (sum %d), bf16; DISTINCT bytes (shared "
-        "pages counted once) over the prefix pass and the tail kernel together" % int(tails.sum()),
-        {"with_merge_us": round(call_ms * 1e3, 2), "with_merge_frac": round(distinct / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-         "logical_bytes_per_launch": int(lens.sum()) * 2 * KVH * D * 2})
-    del q, out, ws, dtab
+        a0, a1 = ev(), ev()
+        a0.record(stream)
+        for i in range(72):
+            shared_one(i)
+        a1.record(stream)
+        torch.cuda.synchronize()
+        call_ms = a0.elapsed_time(a1) / 72
+        distinct = (prefix + int(private.sum())) * per_tok
+        in_groups = sum((e - b0) // 64 * 64 * (nb - 1) for _, nb, b0, e in groups)
+        res[key] = _entry(
+            "decode_group16_kernel<bf16>", "hbm", distinct, ker_ms,
+            "config 3: 65536-token prefix shared by 16 branches + private tokens U{0..4096} (sum %d), bf16, %d layers of pages "
+            "in the pool; %s; DISTINCT bytes (a page that several branches read is counted once)"
+            % (int(private.sum()), L, "a branch forks from the prefix or from an earlier branch at a random block boundary"
+               if tree else "every branch forks at the prefix's end"),
+            {"with_merge_us": round(call_ms * 1e3, 2), "with_merge_frac": round(distinct / (call_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+             "logical_bytes_per_launch": int(lens.sum()) * per_tok,
+             "streamed_bytes_per_launch": (int(lens.sum()) - in_groups) * per_tok,
+             "fork_parent": parent, "fork_points": points, "shared_ranges": [list(x) for x in groups]})
+        del q, out, ws, dtab
 
     # ---- config 5: chunked causal prefill to 32 768 tokens in 2 048-token chunks -------------------------
     L, chunk, total = 1, 2048, 32768
-    NB = fit_blocks(L, cabi.BF16, 65536)
-    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
-    tab, stride, _ = _shuffled_rows(rng, NB, [total // bs])
-    dtab = torch.from_numpy(tab).cuda()
-    per_chunk = []
-    for ps in range(2):                                                           # the first pass warms up
+
+    def chunk_flops(pos, m, qh, d):
+        return 4.0 * m * (pos + (m + 1) / 2.0) * d * qh
+
+    def prefill_entry(key, kernel, per_chunk, what, extra=None):
+        tot_ms, tot_fl = sum(t for t, _ in per_chunk), sum(f for _, f in per_chunk)
+        e = {"last_chunk_us": round(per_chunk[-1][0] * 1e3, 1),
+             "last_chunk_TFLOPs": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12, 1),
+             "last_chunk_frac": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+             "first_chunk_TFLOPs": round(per_chunk[0][1] / (per_chunk[0][0] * 1e-3) / 1e12, 1)}
+        e.update(extra or {})
+        res[key] = _entry(kernel, "mfma", tot_fl / len(per_chunk), tot_ms / len(per_chunk), what +
+                          "; average over the 16 launches (flops = 4 M (pos_start + (M+1)/2) D QH per chunk)", e)
+
+    for key, name, dt in (("config5_prefill_int8", "int8", cabi.INT8), ("config5_prefill_fp8", "fp8", cabi.FP8_E4M3),
+                          ("config5_prefill", "bf16", cabi.BF16)):
+        NB = fit_blocks(L, dt, 65536)
+        g = cabi.layout(L, KVH, QH, D, bs, NB, dt)
+        tab, stride, _ = _shuffled_rows(rng, NB, [total // bs])
+        dtab = torch.from_numpy(tab).cuda()
         per_chunk = []
-        for c in range(total // chunk):
-            k = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
-            v = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
-            q = torch.randn(chunk, QH, D, device="cuda").to(torch.bfloat16)
-            o = torch.empty_like(q)
-            cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), cabi.p(dtab), 0, L, c * chunk, chunk, cabi.p(k), cabi.p(v),
-                      cabi.BF16, sp)
-            a0, a1 = ev(), ev()
-            a0.record(stream)
-            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, c * chunk, chunk,
-                      scale, cabi.BF16, None, 0, sp)
-            a1.record(stream)
-            torch.cuda.synchronize()
-            per_chunk.append((a0.elapsed_time(a1), 4.0 * chunk * (c * chunk + (chunk + 1) / 2.0) * D * QH))
+        for ps in range(2):                                                       # the first pass warms up
+            per_chunk = []
+            for c in range(total // chunk):
+                k = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+                v = torch.randn(L, chunk, KVH, D, device="cuda").to(torch.bfloat16)
+                q = torch.randn(chunk, QH, D, device="cuda").to(torch.bfloat16)
+                o = torch.empty_like(q)
+                cabi.call("drk_kv_append_batch", C.byref(g), cabi.p(buf), cabi.p(dtab), 0, L, c * chunk, chunk, cabi.p(k), cabi.p(v),
+                          cabi.BF16, sp)
+                a0, a1 = ev(), ev()
+                a0.record(stream)
+                cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, c * chunk, chunk,
+                          scale, cabi.BF16, None, 0, sp)
+                a1.record(stream)
+                torch.cuda.synchronize()
+                per_chunk.append((a0.elapsed_time(a1), chunk_flops(c * chunk, chunk, QH, D)))
+        if dt != cabi.BF16:
+            prefill_entry(key, "prefill_pp_kernel<%s>" % name, per_chunk,
+                          "config 5 over %s pages: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV "
+                          "x 128, bf16 queries, codes turned into 16-bit MFMA operands on the way into LDS" % name)
     # the same kernel at position 30 720 with fewer workgroups (shorter chunks): microseconds per 64-token tile of the
     # longest walk.  One workgroup per CU either way -- what changes is how much of the chip draws power.
     by_wgs = {}
@@ -822,14 +943,51 @@ def kernel_fractions(buf, seed=11):
         torch.cuda.synchronize()
         lib.drk_debug_set_prefill_two_phase(1)
         by_wgs[str(m // 64 * KVH)] = round(a0.elapsed_time(a1) / 4 * 1e3 / ((pos + m + 63) // 64), 3)
-    tot_ms, tot_fl = sum(t for t, _ in per_chunk), sum(f for _, f in per_chunk)
-    res["config5_prefill"] = _entry(
-        "prefill_ppd_kernel<bf16>", "mfma", tot_fl / len(per_chunk), tot_ms / len(per_chunk),
-        "config 5: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV x 128 bf16; average "
-        "over the 16 launches (flops = 4 M (pos_start + (M+1)/2) D QH per chunk)",
-        {"last_chunk_us": round(per_chunk[-1][0] * 1e3, 1),
-         "last_chunk_TFLOPs": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12, 1),
-         "last_chunk_frac": round(per_chunk[-1][1] / (per_chunk[-1][0] * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-         "first_chunk_TFLOPs": round(per_chunk[0][1] / (per_chunk[0][0] * 1e-3) / 1e12, 1),
-         "us_per_tile_by_workgroups_at_30720": by_wgs})
+    prefill_entry("config5_prefill", "prefill_ppd_kernel<bf16>", per_chunk,
+                  "config 5: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV x 128 bf16",
+                  {"us_per_tile_by_workgroups_at_30720": by_wgs})
+    del dtab
+
+    # ---- the reference's model shape: 24 Q / 4 KV heads x 256, fp16, 256-token blocks, 16 layers --------------
+    L7, KVH7, QH7, D7, bs7, B7, ctx7 = 16, 4, 24, 256, 256, 8, 32768
+    nblk = ctx7 // bs7 + 1
+    NB7 = B7 * nblk + 8
+    g = cabi.layout(L7, KVH7, QH7, D7, bs7, NB7, cabi.F16)
+    pool_bytes = lib.drk_kv_pool_bytes(C.byref(g))
+    assert pool_bytes <= buf.numel()
+    buf[:pool_bytes].view(torch.float16).normal_(0, 0.5)
+    dtab = torch.from_numpy(np.stack(np.split(rng.permutation(NB7).astype(np.int32)[:B7 * nblk], B7))).cuda()
+    h = torch.float16
+    q = (torch.randn(L7, B7, QH7, D7, device="cuda") * 0.5).to(h)
+    gate = (torch.randn(L7, B7, QH7, D7, device="cuda") * 0.5).to(h)
+    out = torch.empty_like(q)
+    dlen = torch.full((B7,), ctx7, dtype=torch.int32, device="cuda")
+    wsb = lib.drk_decode_workspace_bytes(C.byref(g), B7, ctx7)
+    ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
+    scale7 = float(1.0 / np.sqrt(D7))
+    row = B7 * QH7 * D7 * 2
+    ms = _timed_decode(lib, cabi, lambda i: cabi.call(
+        "drk_paged_decode_attention_gated", C.byref(g), C.c_void_p(q.data_ptr() + (i % L7) * row), cabi.p(buf), cabi.p(dtab), nblk,
+        cabi.p(dlen), B7, ctx7, C.c_void_p(out.data_ptr() + (i % L7) * row), i % L7, scale7, cabi.F16,
+        C.c_void_p(gate.data_ptr() + (i % L7) * row), D7, cabi.p(ws), wsb, sp), 48)
+    res["config7_decode_d256"] = _entry(
+        "decode_stream_kernel<f16, 256>", "hbm", B7 * ctx7 * 2 * KVH7 * D7 * 2, ms,
+        "the reference's model shape: 24 Q / 4 KV heads x 256, fp16, 256-token blocks shuffled over %d, %d layers of pages; decode "
+        "attention of 8 branches x 32768 tokens with the sigmoid gate (applied in the merge, not in this kernel)" % (NB7, L7))
+    qc = (torch.randn(chunk, QH7, D7, device="cuda") * 0.5).to(h)
+    oc = torch.empty_like(qc)
+    per_chunk = []
+    for ps in range(2):
+        per_chunk = []
+        for c in range(total // chunk):
+            a0, a1 = ev(), ev()
+            a0.record(stream)
+            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(buf), cabi.p(dtab), cabi.p(oc), c % L7, c * chunk, chunk,
+                      scale7, cabi.F16, None, 0, sp)
+            a1.record(stream)
+            torch.cuda.synchronize()
+            per_chunk.append((a0.elapsed_time(a1), chunk_flops(c * chunk, chunk, QH7, D7)))
+    prefill_entry("config7_prefill_d256", "prefill_d256_kernel<f16>", per_chunk,
+                  "the reference's model shape: causal prefill of 32768 tokens in 16 chunks of 2048 over 256-token blocks, 24 Q / 4 KV "
+                  "heads x 256, fp16 (the pages hold N(0, 0.5), written beforehand)")
     return res

@@ -32,6 +32,9 @@ def layout(L, KVH, QH, D, bs, NB, dtype):
     return Layout(L, KVH, QH, D, bs, NB, dtype, 0)
 
 
+MAX_PREFIX_GROUPS = 16             # DRK_MAX_PREFIX_GROUPS
+
+
 class PrefixGroup(C.Structure):
     """drk_prefix_group: branches [first_branch, +n_branches) hold tokens [tok_begin, tok_end) in the same pages"""
     _fields_ = [(n, C.c_int32) for n in ("first_branch", "n_branches", "tok_begin", "tok_end")]

@@ -165,11 +165,27 @@ int KvStream::set_branch_count(int n)
     }
     positions_on_device_ = false;
     shared_tokens_ = branches_.empty() ? 0 : cm_->common_prefix_tokens(branches_.data(), (int)branches_.size());
+    find_shared_groups();
     if (graph_) {                        // a captured step is tied to the branch set it was recorded for
         drk_graph_destroy(graph_);
         graph_ = nullptr;
     }
     return (int)branches_.size();
+}
+
+// Branches forked at different moments form a tree: all of them share the context up to the oldest fork, the
+// younger ones what the stream took in since.  (Forks never change a shared page -- a write takes a private copy
+// -- so the tree found here holds until the branch set changes.)
+void KvStream::find_shared_groups()
+{
+    groups_.clear();
+    const int B = (int)branches_.size();
+    if (B < 2 || !paged_gqa_decode_grouped_supported(cm_->block_pool().block_size()) || ModelConfig::KV_DTYPE > DRK_BF16) return;
+    const int per_group = 64 / (ModelConfig::NUM_ATTN_HEADS / ModelConfig::NUM_KV_HEADS);     // 64 query rows per kv head and group
+    if (per_group < 2) return;
+    groups_.resize(DRK_MAX_PREFIX_GROUPS);
+    const int n = cm_->common_prefix_groups(branches_.data(), B, per_group, 256, groups_.data(), DRK_MAX_PREFIX_GROUPS);
+    groups_.resize((size_t)n);
 }
 
 // The scorer folds its whole new-score buffer into the scores on every step.  The rows of a branch
@@ -195,6 +211,7 @@ void KvStream::close_branches()
     pos_.clear();
     positions_on_device_ = false;
     shared_tokens_ = 0;
+    groups_.clear();
     if (graph_) {                        // a captured step is tied to the branch set it was recorded for
         drk_graph_destroy(graph_);
         graph_ = nullptr;
@@ -269,6 +286,11 @@ void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t s
         if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
                              ModelConfig::IO_DTYPE, stream) != DRK_OK)
             LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
+    } else if (B >= shared_min_branches_ && !groups_.empty() && groups_[0].tok_end - groups_[0].tok_begin >= shared_min_tokens_) {
+        // every range some of the branches share is streamed once for them, the gate rides on the merge
+        paged_gqa_decode_attention_grouped(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
+                                           groups_.data(), (int)groups_.size(), gate, 2 * hd, io.attn_out, fa_layer_idx,
+                                           pool.max_blocks(), pool.block_size(), scale, stream);
     } else if (B >= shared_min_branches_ && shared_tokens_ >= shared_min_tokens_) {
         // the branches' common prefix is streamed once for all of them
         paged_gqa_decode_attention_shared(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, shared_tokens_,

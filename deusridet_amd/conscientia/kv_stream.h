@@ -82,6 +82,8 @@ public:
     // at least min_tokens shared, decode streams that prefix once for all branches instead of
     // once per branch.  Defaults: 4 branches, 4096 tokens.
     int  shared_tokens() const { return shared_tokens_; }
+    // the open branches' fork tree as decode reads it: shared ranges, parents first (empty: nothing shared)
+    const std::vector<drk_prefix_group>& shared_groups() const { return groups_; }
     void set_shared_prefix_policy(int min_branches, int min_tokens) { shared_min_branches_ = min_branches; shared_min_tokens_ = min_tokens; }
 
     // One decode step = begin, decode_layer for every full-attention layer, end.
@@ -115,6 +117,7 @@ private:
     int* d_len_ = nullptr;
     bool positions_on_device_ = false;
     int shared_tokens_ = 0;          // prefix the open branches share (whole blocks)
+    std::vector<drk_prefix_group> groups_;   // their fork tree: the ranges some of them share (CacheManager::common_prefix_groups)
     int shared_min_branches_ = 4;
     int shared_min_tokens_ = 4096;
     void* graph_ = nullptr;
@@ -126,6 +129,7 @@ private:
     bool host_begin(hipStream_t stream);
     void host_end();
     void clear_mass_rows(int first_branch, int count);
+    void find_shared_groups();
 };
 
 } // namespace deusridet

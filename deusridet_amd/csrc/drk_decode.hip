@@ -632,7 +632,8 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
         return fail(DRK_ERR_INVALID, "decode: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "decode: layer %d outside [0,%d)", layer, a.L);
     // one prefix for all branches is the simplest tree: shared and private tiles in one launch
-    if (grouped_decode_supported(a, B) && B * (a.QH / a.KVH) <= 64) {
+    // (16-bit pages; 8-bit pages are faster on the prefix pass + tail kernel pair below)
+    if (grouped_decode_supported(a, B) && a.E == 2 && B * (a.QH / a.KVH) <= 64) {
         const drk_prefix_group all = {0, B, 0, shared};
         return launch_decode_grouped(g, q, pool, tables, table_stride, d_seq_lens, B, max_seq_len, &all, 1, out, layer, scale,
                                      io_dtype, workspace, workspace_bytes, stream, gate, gate_stride);

@@ -118,6 +118,27 @@ __device__ __forceinline__ uint32_t pack16(float a, float b)
 // how far (in bits of the exponent) a row's maximum may run ahead of the reference its weights are taken to
 constexpr float kLazy = 5.0f;
 
+// The grid is dealt to the two kinds of units by what they cost: a tile of a shared range (its waves meet at two
+// barriers) takes about 13 parts of time where a tile of a private tail takes 12.  Workgroups [0, Gs) take runs of
+// Us units of the shared ranges, the others runs of Ut units of the tails.  Kernel and merge compute it alike.
+struct RegionSplit { int Gs, Us, Ut; };
+__host__ __device__ inline RegionSplit region_split(int group_units, int tail_units, int grid)
+{
+    RegionSplit r;
+    const long long cs = 13LL * group_units, ct = 12LL * tail_units;
+    if (group_units <= 0) r.Gs = 0;
+    else if (tail_units <= 0 || grid < 2) r.Gs = grid;
+    else {
+        long long gs = (cs * grid + (cs + ct) / 2) / (cs + ct);
+        r.Gs = (int)(gs < 1 ? 1 : (gs > grid - 1 ? grid - 1 : gs));
+    }
+    r.Us = r.Gs > 0 ? (group_units + r.Gs - 1) / r.Gs : 1;
+    r.Ut = grid - r.Gs > 0 ? (tail_units + (grid - r.Gs) - 1) / (grid - r.Gs) : 1;
+    if (r.Us < 1) r.Us = 1;
+    if (r.Ut < 1) r.Ut = 1;
+    return r;
+}
+
 // The workgroup's run of units and one descriptor per unit, in LDS: returns how many (0: nothing to do).
 // Every thread of the workgroup must call it (it holds barriers).
 template <int MAXU>
@@ -136,14 +157,18 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
         const int t = __shfl_up(incl, off);
         if (lane >= off) incl += t;
     }
-    const int T = A.group_units + __builtin_amdgcn_readlane(incl, 63) * A.KVH;
-    if (T == 0) return 0;
-    const int U = (T + (int)gridDim.x - 1) / (int)gridDim.x;
-    const int u0 = (int)blockIdx.x * U;
-    if (u0 >= T) return 0;
+    const int tail_units = __builtin_amdgcn_readlane(incl, 63) * A.KVH;
+    if (A.group_units + tail_units == 0) return 0;
+    const RegionSplit rs = region_split(A.group_units, tail_units, (int)gridDim.x);
+    const bool tail_wg = (int)blockIdx.x >= rs.Gs;
+    const int U = tail_wg ? rs.Ut : rs.Us;
+    const int wg_rel = tail_wg ? (int)blockIdx.x - rs.Gs : (int)blockIdx.x;      // the workgroup's place among those of its kind
+    const int region_units = tail_wg ? tail_units : A.group_units;
+    const int u0 = wg_rel * U;                                   // its first unit, counted within its kind
+    if (u0 >= region_units) return 0;
     // the host sizes the grid from max_seq_len; lengths on the device beyond that bound must not overrun
     // the descriptor table (the tiles past it are then left out: the caller broke its promise)
-    const int nunits = min(min(U, T - u0), MAXU);
+    const int nunits = min(min(U, region_units - u0), MAXU);
     if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
     __syncthreads();
     if ((int)threadIdx.x < A.ngroups) {
@@ -156,8 +181,8 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
     __syncthreads();
     for (int i = threadIdx.x; i < nunits * 4; i += 256) {
         const int ui = i >> 2, grp = i & 3, u = u0 + ui;
-        int b, kvh, trel, nt, tile, len, nrows, slot0, run0;
-        if (u < A.group_units) {
+        int b, kvh, trel, nt, tile, len, nrows, slot0, run0;     // run0: first unit of the run (one kv head of a range or tail), within its kind
+        if (!tail_wg) {
             int gi = 0;
             while (gi + 1 < A.ngroups && A.seg[gi + 1].unit0 <= u) gi++;
             const GSeg sg = A.seg[gi];
@@ -166,7 +191,7 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
             tile = sg.tile0 + trel; b = sg.first; len = s_gmin[gi]; nrows = sg.count * GQ;
             slot0 = sg.slot; run0 = sg.unit0 + kvh * nt;
         } else {
-            const int v = u - A.group_units;
+            const int v = u;
             int lo = 0, hi = A.B - 1;                              // first branch whose cumulative units exceed v
             while (lo < hi) {
                 const int mid = (lo + hi) >> 1;
@@ -178,7 +203,7 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
             const int rem = v - A.KVH * excl;
             kvh = rem / nt; trel = rem - kvh * nt;
             tile = trel + A.b_start[b]; nrows = GQ;
-            slot0 = A.b_slot[b]; run0 = A.group_units + A.KVH * excl + kvh * nt;
+            slot0 = A.b_slot[b]; run0 = A.KVH * excl + kvh * nt;
         }
         const int tg = tile * kSTile + grp * 16;
         uint2 gd = make_uint2(kNone, 0u);
@@ -199,7 +224,7 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
             d.tile_lim = len - tile * kSTile;
             d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0) | (nrows << 8);
             d.row0 = b * A.QH + kvh * GQ;
-            d.slot = slot0 + ((int)blockIdx.x - run0 / U);
+            d.slot = slot0 + (wg_rel - run0 / U);
             udesc[ui] = d;
         }
     }
@@ -505,7 +530,7 @@ __global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
     }
 }
 
-template <int DT, int D, int NG, bool DMA>
+template <int DT, int D, int NG>
 __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
 {
     using Geo = StreamGeo<DT, D>;
@@ -517,13 +542,7 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
     constexpr int CPR = D * 2 / 16;                              // 16-byte chunks per query row
     constexpr int RPP = 256 / CPR;                               // rows the workgroup moves per pass
     constexpr int QPASS = NR / RPP;
-    // K of 16-bit pages goes from global memory straight into LDS (no registers hold it): two buffers of a wave's
-    // 16 token rows, unpadded, 16-byte chunk x of row r at position x ^ r -- applied on the global side by the lane
-    // that fills the position, undone by the reader.  8-bit codes pass through registers (they are widened on the
-    // way) into one buffer of padded rows.
-    constexpr bool DIRECT = DMA && !Q8;
-    constexpr int KBUF = DIRECT ? 16 * D * 2 : 16 * Geo::PITCH;  // one wave's K rows of one tile
-    __shared__ __align__(256) uint8_t k_lds[DIRECT ? 2 : 1][4][KBUF];
+    __shared__ __align__(16) uint8_t k_lds[4][16 * Geo::PITCH];  // a wave's 16 K rows as 16-bit values, padded rows
     __shared__ __align__(16) uint8_t q_lds[NR * QP];
     __shared__ __align__(16) float o_lds[4][8][D];               // [wave][row of the round][dim], segment ends only
     __shared__ float mw_lds[4][NR], lw_lds[4][NR];
@@ -608,24 +627,6 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
         }
     };
 
-    // K of a unit on its way into the wave's LDS buffer `buf`: four direct loads of 64 x 16 bytes; lane l of load j
-    // fills position l % 16 of row 4j + l / 16 with the row's chunk (l % 16) ^ row
-    // (row r = 4j + l / 16 and l / 16 < 4, so the chunk is ((l % 16) ^ (l / 16)) ^ 4j: load j's offset is load 0's
-    // with j xor-ed into bits 6-7, plus 1024 j)
-    const uint32_t kdma_row = (uint32_t)((lane >> 4) * (D * 2)), kdma_x = (uint32_t)(((lane & 15) ^ (lane >> 4)) << 4);
-    static_assert(!DIRECT || D == 128, "the direct K path is laid out for 256-byte rows");
-    auto k_request = [&](uint32_t off, int buf) {
-        if constexpr (DIRECT) {
-            const uint8_t *base = A.pool_layer + ((size_t)(off == kNone ? 0u : off) << 4);     // uniform: one run per wave
-            const uint32_t lds = lds_addr32(&k_lds[DIRECT ? buf : 0][w][0]);
-            uint32_t kx = kdma_x;
-#if defined(__HIP_DEVICE_COMPILE__)
-            asm volatile("" : "+v"(kx));                     // computed here, each time: four more registers held across the loop would spill
-#endif
-#pragma unroll
-            for (int j = 0; j < Geo::NK; j++) lds_dma16(base, (kx ^ (uint32_t)(j << 6)) + kdma_row + 1024u * j, lds + 1024 * j);
-        }
-    };
     // V of a unit: the run's address is the same for the whole wave (scalar registers), the lane adds 32 bits
     const uint32_t v_lane_off = (uint32_t)((lane >> 4) * (4 * Geo::RB) + (lane & 15) * (Q8 ? 8 : 16));
     auto load_v_uniform = [&](uint32_t off) -> VRegs<DT, D> {
@@ -641,9 +642,7 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
         return v;
     };
     uint2 gd = gdesc[0][w], ksr = {}, vsr = {};
-    KRegs<DT, D> kreg;
-    if constexpr (DIRECT) k_request(__builtin_amdgcn_readfirstlane(gd.x), 0);
-    else kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
+    KRegs<DT, D> kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
     VRegs<DT, D> vreg = load_v_uniform(__builtin_amdgcn_readfirstlane(gd.x));
     load_scales(gd, ksr, vsr);
     {
@@ -667,8 +666,7 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
 
         // ---- K: registers -> the wave's LDS rows -> one token row per lane; V: registers -> B operands;
         // then the loads of the next unit's K and V, so that they travel during all of this unit's arithmetic
-        if constexpr (DIRECT) vm_wait_all();                    // this unit's K has landed (its V too: requested before it)
-        else stage_k<DT, D>(&k_lds[0][w][0], kreg, lane);
+        stage_k<DT, D>(&k_lds[w][0], kreg, lane);
         float ks[4] = {1.0f, 1.0f, 1.0f, 1.0f}, vs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
         if (DT == DRK_INT8) {
             ks[0] = f16_bits_to_f((uint16_t)(ksr.x & 0xffffu)); ks[1] = f16_bits_to_f((uint16_t)(ksr.x >> 16));
@@ -691,16 +689,12 @@ __global__ __launch_bounds__(256, 2) void decode_group_kernel(GroupedArgs A)
         if (has_next) {
             gd = gdesc[it + 1][w];
             vreg = load_v_uniform(__builtin_amdgcn_readfirstlane(gd.x));
-            if constexpr (DIRECT) k_request(__builtin_amdgcn_readfirstlane(gd.x), (it + 1) & 1);
-            else kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
+            kreg = load_k<DT, D>(A.pool_layer, gd.x, lane);
             load_scales(gd, ksr, vsr);
         }
         // the A operand: dims 32 kk + 8 g .. of token row c of the wave's 16
-        const uint8_t *const krows = &k_lds[DIRECT ? (it & 1) : 0][w][0];
-        auto k_operand = [&](int kk) -> uint4 {
-            if constexpr (DIRECT) return *(const uint4 *)(krows + c * (D * 2) + ((((g ^ c) & 15) << 4) ^ (kk << 6)) + (((kk * 4 + g) & ~15) << 4));
-            else return *(const uint4 *)(krows + c * Geo::PITCH + g * 16 + kk * 64);
-        };
+        const uint8_t *const krows = &k_lds[w][0];
+        auto k_operand = [&](int kk) -> uint4 { return *(const uint4 *)(krows + c * Geo::PITCH + g * 16 + kk * 64); };
 
         // ---- scores, softmax, O += P V: for the unit's row groups (one, or all NG: a group of padding rows
         // multiplies zeros and its state is never stored) ----------------------------------------------
@@ -909,21 +903,20 @@ __global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_
     __syncthreads();
     if (threadIdx.x == 0) {
         const int excl = scan_s[0], total = scan_s[1], nt_b = scan_s[2];
-        const int T = A.group_units + total * A.KVH;
         int n = 0, off = 0;
-        if (T > 0) {
-            const int U = (T + grid_wgs - 1) / grid_wgs;
+        if (A.group_units + total * A.KVH > 0) {
+            const RegionSplit rs = region_split(A.group_units, total * A.KVH, grid_wgs);
             const int kvh = h / (A.QH / A.KVH);
             for (int gi = 0; gi < A.ngroups; gi++) {
                 const GSeg sg = A.seg[gi];
                 if (b < sg.first || b >= sg.first + sg.count) continue;
                 const int first = sg.unit0 + kvh * sg.ntile, last = first + sg.ntile - 1;
-                seg_base[n] = sg.slot; seg_cnt[n] = last / U - first / U + 1; seg_off[n] = off;
+                seg_base[n] = sg.slot; seg_cnt[n] = last / rs.Us - first / rs.Us + 1; seg_off[n] = off;
                 off += seg_cnt[n]; n++;
             }
             if (nt_b > 0) {
-                const int first = A.group_units + A.KVH * excl + kvh * nt_b, last = first + nt_b - 1;
-                seg_base[n] = A.b_slot[b]; seg_cnt[n] = last / U - first / U + 1; seg_off[n] = off;
+                const int first = A.KVH * excl + kvh * nt_b, last = first + nt_b - 1;
+                seg_base[n] = A.b_slot[b]; seg_cnt[n] = last / rs.Ut - first / rs.Ut + 1; seg_off[n] = off;
                 off += seg_cnt[n]; n++;
             }
         }
@@ -1016,7 +1009,8 @@ struct GroupPlan {
 // by one range or by the branch's tail).  Ranges are cut down to whole 64-token tiles; what a range
 // loses at its end, the range or tail behind it reads.
 // units one workgroup may own: the descriptor table of the kernel that takes the call
-static int group_max_units(const Lay &a) { return a.E == 2 && g_grouped_mode != 2 ? kG16MaxUnits : kGMaxUnits; }
+// (times 12 / 13: the workgroups of the tails take runs up to 13 / 12 of the even share, see region_split)
+static int group_max_units(const Lay &a) { return (a.E == 2 && g_grouped_mode != 2 ? kG16MaxUnits : kGMaxUnits) * 12 / 13; }
 
 static int plan_groups(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_in, GroupPlan *P)
 {
@@ -1103,7 +1097,7 @@ size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_
     const int max_tiles = (max_seq_len + kSTile - 1) / kSTile;
     long G = kGWgs;
     const long t_upper = (long)a.KVH * B * max_tiles;
-    const int max_units = kG16MaxUnits;                          // the smaller table gives the larger grid, and so the larger bound
+    const int max_units = kG16MaxUnits * 12 / 13;                // the smaller table gives the larger grid, and so the larger bound
     if ((t_upper + G - 1) / G > max_units) G = (t_upper + max_units - 1) / max_units;
     long cap = G / a.KVH + 2;
     if (cap > max_tiles) cap = max_tiles;
@@ -1163,14 +1157,14 @@ int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *poo
     switch (a.dtype) {
     case DRK_F16:
         if (tile16) hipLaunchKernelGGL((decode_group16_kernel<DRK_F16>), dim3(P.grid), dim3(256), 0, st, A);
-        else hipLaunchKernelGGL((decode_group_kernel<DRK_F16, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A);
+        else hipLaunchKernelGGL((decode_group_kernel<DRK_F16, 128, 4>), dim3(P.grid), dim3(256), 0, st, A);
         break;
     case DRK_BF16:
         if (tile16) hipLaunchKernelGGL((decode_group16_kernel<DRK_BF16>), dim3(P.grid), dim3(256), 0, st, A);
-        else hipLaunchKernelGGL((decode_group_kernel<DRK_BF16, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A);
+        else hipLaunchKernelGGL((decode_group_kernel<DRK_BF16, 128, 4>), dim3(P.grid), dim3(256), 0, st, A);
         break;
-    case DRK_INT8: hipLaunchKernelGGL((decode_group_kernel<DRK_INT8, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A); break;
-    default: hipLaunchKernelGGL((decode_group_kernel<DRK_FP8_E4M3, 128, 4, false>), dim3(P.grid), dim3(256), 0, st, A); break;
+    case DRK_INT8: hipLaunchKernelGGL((decode_group_kernel<DRK_INT8, 128, 4>), dim3(P.grid), dim3(256), 0, st, A); break;
+    default: hipLaunchKernelGGL((decode_group_kernel<DRK_FP8_E4M3, 128, 4>), dim3(P.grid), dim3(256), 0, st, A); break;
     }
     DRK_LAUNCH_CHECK("decode_group_kernel");
     if (g_skip_merge) return DRK_OK;

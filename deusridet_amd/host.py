@@ -48,7 +48,8 @@ SIGNATURES = {
     "drkh_cm_num_logical_blocks": (_i32, [_vp, _i32]),
     "drkh_cm_fork_branch": (_i32, [_vp, _i32, _i32]), "drkh_cm_release_branch": (None, [_vp, _i32]),
     "drkh_cm_touch_block": (None, [_vp, _i32, _i32]),
-    "drkh_cm_common_prefix_tokens": (_i32, [_vp, _vp, _i32]), "drkh_cm_block_location": (_i32, [_vp, _i32, _i32]),
+    "drkh_cm_common_prefix_tokens": (_i32, [_vp, _vp, _i32]),
+    "drkh_cm_common_prefix_groups": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _i32]), "drkh_cm_block_location": (_i32, [_vp, _i32, _i32]),
     "drkh_cm_evict_blocks": (_i32, [_vp, _i32]), "drkh_cm_ensure_free_blocks": (_i32, [_vp, _i32]),
     "drkh_cm_gpu_blocks_used": (_i32, [_vp]), "drkh_cm_free_blocks": (_i32, [_vp]),
     "drkh_cm_lru_snapshot": (_i32, [_vp, _vp, _vp, _i32]),
@@ -67,6 +68,9 @@ SIGNATURES = {
                                                         _i32, _f32, _vp]),
     "drkh_paged_gqa_decode_attention_shared": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _i32, _vp, _i32, _i32, _i32,
                                                       _f32, _vp]),
+    "drkh_paged_gqa_decode_grouped_supported": (_i32, [_i32]),
+    "drkh_paged_gqa_decode_attention_grouped": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _vp, _i32, _i32, _i32,
+                                                       _f32, _vp]),
     "drkh_paged_prefill_attention": (None, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _vp]),
     "drkh_paged_attention_reserve_workspace": (_i32, [_i32, _i32, _i32, _i32, _vp]),
     "drkh_paged_attention_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
@@ -274,6 +278,13 @@ class CacheManager:
     def fork_branch(self, parent, pos): return lib().drkh_cm_fork_branch(self._h, parent, pos)
     def release_branch(self, branch): lib().drkh_cm_release_branch(self._h, branch)
     def touch_block(self, branch, logical): lib().drkh_cm_touch_block(self._h, branch, logical)
+
+    def common_prefix_groups(self, branches, max_group_branches=16, min_tokens=64, max_groups=16):
+        """the fork tree of the branches as (first_branch, n_branches, tok_begin, tok_end) tuples, parents first"""
+        a = np.ascontiguousarray(branches, dtype=np.int32)
+        out = np.zeros((max_groups, 4), dtype=np.int32)
+        n = lib().drkh_cm_common_prefix_groups(self._h, _p(a), a.shape[0], max_group_branches, min_tokens, _p(out), max_groups)
+        return [tuple(int(x) for x in out[i]) for i in range(n)]
 
     def common_prefix_tokens(self, branches):
         a = np.ascontiguousarray(branches, dtype=np.int32)

@@ -98,6 +98,10 @@ int drkh_cm_fork_branch(void *cm, int parent, int pos) { return CM(cm)->fork_bra
 void drkh_cm_release_branch(void *cm, int branch) { CM(cm)->release_branch(branch); }
 void drkh_cm_touch_block(void *cm, int branch, int logical) { CM(cm)->touch_block(branch, logical); }
 int drkh_cm_common_prefix_tokens(void *cm, const int32_t *branches, int n) { return CM(cm)->common_prefix_tokens(branches, n); }
+int drkh_cm_common_prefix_groups(void *cm, const int32_t *branches, int n, int max_group_branches, int min_tokens, int32_t *out, int max_groups)
+{
+    return CM(cm)->common_prefix_groups(branches, n, max_group_branches, min_tokens, (drk_prefix_group *)out, max_groups);
+}
 int drkh_cm_block_location(void *cm, int branch, int logical) { return (int)CM(cm)->block_location(branch, logical); }
 int drkh_cm_evict_blocks(void *cm, int n) { return CM(cm)->evict_blocks(n); }
 int drkh_cm_ensure_free_blocks(void *cm, int n_free) { return CM(cm)->ensure_free_blocks(n_free) ? 1 : 0; }
@@ -181,6 +185,16 @@ void drkh_paged_gqa_decode_attention_shared(const void *Q, void *kv_pool, const 
     paged_gqa_decode_attention_shared(CH(Q), H(kv_pool), d_tables, table_stride, d_seq_lens, B, max_seq_len,
                                       shared_tokens, H(out), fa_layer_idx, max_phys_blocks, block_size, scale,
                                       ST(stream));
+}
+int drkh_paged_gqa_decode_grouped_supported(int block_size) { return paged_gqa_decode_grouped_supported(block_size) ? 1 : 0; }
+void drkh_paged_gqa_decode_attention_grouped(const void *Q, void *kv_pool, const int32_t *d_tables, int table_stride,
+                                             const int32_t *d_seq_lens, int B, int max_seq_len,
+                                             const int32_t *groups, int n_groups, void *out, int fa_layer_idx,
+                                             int max_phys_blocks, int block_size, float scale, void *stream)
+{
+    paged_gqa_decode_attention_grouped(CH(Q), H(kv_pool), d_tables, table_stride, d_seq_lens, B, max_seq_len,
+                                       reinterpret_cast<const drk_prefix_group *>(groups),
+                                       n_groups, H(out), fa_layer_idx, max_phys_blocks, block_size, scale, ST(stream));
 }
 void drkh_paged_prefill_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
                                   int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,

@@ -32,6 +32,10 @@ bool AttentionWorkspace::reserve(size_t bytes)
     return true;
 }
 
+// shared ranges nested deeper than this fall to the private tails (CacheManager::common_prefix_groups emits
+// parents first, so the callers simply stop there)
+static constexpr int kMaxForkTreeDepth = 4;
+
 size_t paged_attention_workspace_bytes(int max_branches, int max_seq_len, int max_prefill_rows, int block_size)
 {
     drk_kv_layout g = ModelConfig::layout(1, block_size);
@@ -41,6 +45,8 @@ size_t paged_attention_workspace_bytes(int max_branches, int max_seq_len, int ma
     size_t s = drk_decode_shared_workspace_bytes(&g, B, max_seq_len, max_seq_len);
     if (s > need) need = s;
     s = drk_decode_mass_workspace_bytes(&g, B, max_seq_len);
+    if (s > need) need = s;
+    s = drk_decode_grouped_workspace_bytes_max(&g, B, max_seq_len, kMaxForkTreeDepth);
     if (s > need) need = s;
     if (max_prefill_rows > 0) {
         // a short chunk behind a long context runs with the context split over the chip and keeps
@@ -198,6 +204,26 @@ void paged_gqa_decode_attention_shared(AttentionWorkspace& ws, const __half* Q, 
         LOG_ERROR("Machina", "paged_gqa_decode_attention_shared: %s", drk_last_error());
 }
 
+bool paged_gqa_decode_grouped_supported(int block_size)
+{
+    return ModelConfig::HEAD_DIM == 128 && block_size % 16 == 0 && ModelConfig::NUM_KV_HEADS > 0 &&
+           ModelConfig::NUM_ATTN_HEADS / ModelConfig::NUM_KV_HEADS <= 16;
+}
+
+void paged_gqa_decode_attention_grouped(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_tables,
+                                        int table_stride, const int* d_seq_lens, int B, int max_seq_len,
+                                        const drk_prefix_group* groups, int n_groups, const __half* gate,
+                                        int gate_stride, __half* out, int fa_layer_idx, int max_phys_blocks,
+                                        int block_size, float scale, hipStream_t stream)
+{
+    if (B <= 0 || max_seq_len <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    if (drk_paged_decode_attention_grouped(&g, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups,
+                                           n_groups, out, fa_layer_idx, scale, ModelConfig::IO_DTYPE, gate,
+                                           (size_t)gate_stride, ws.ptr(), ws.bytes(), stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_gqa_decode_attention_grouped: %s", drk_last_error());
+}
+
 void paged_gqa_decode_attention_shared(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
                                        const int* d_seq_lens, int B, int max_seq_len, int shared_tokens,
                                        __half* out, int fa_layer_idx, int max_phys_blocks, int block_size,
@@ -209,6 +235,19 @@ void paged_gqa_decode_attention_shared(const __half* Q, __half* kv_pool, const i
                                               "paged_gqa_decode_attention_shared");
     if (ws) paged_gqa_decode_attention_shared(*ws, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, shared_tokens,
                                               out, fa_layer_idx, max_phys_blocks, block_size, scale, stream);
+}
+
+void paged_gqa_decode_attention_grouped(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                        const int* d_seq_lens, int B, int max_seq_len, const drk_prefix_group* groups,
+                                        int n_groups, __half* out, int fa_layer_idx, int max_phys_blocks, int block_size,
+                                        float scale, hipStream_t stream)
+{
+    if (B <= 0 || max_seq_len <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    AttentionWorkspace* ws = stream_workspace(stream, drk_decode_grouped_workspace_bytes(&g, B, max_seq_len, groups, n_groups),
+                                              "paged_gqa_decode_attention_grouped");
+    if (ws) paged_gqa_decode_attention_grouped(*ws, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups,
+                                               n_groups, nullptr, 0, out, fa_layer_idx, max_phys_blocks, block_size, scale, stream);
 }
 
 void paged_prefill_attention(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,

@@ -103,6 +103,15 @@ void paged_gqa_decode_attention_shared(const __half* Q, __half* kv_pool, const i
                                        __half* out, int fa_layer_idx, int max_phys_blocks, int block_size,
                                        float scale, hipStream_t stream = 0);
 
+// Same, for branches that share pages as a fork tree (CacheManager::common_prefix_groups): every shared range and
+// every private tail is read once, in one launch.  head_dim 128 only (the call logs and leaves out untouched
+// otherwise: check paged_gqa_decode_grouped_supported()).
+bool paged_gqa_decode_grouped_supported(int block_size);
+void paged_gqa_decode_attention_grouped(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
+                                        const int* d_seq_lens, int B, int max_seq_len, const drk_prefix_group* groups,
+                                        int n_groups, __half* out, int fa_layer_idx, int max_phys_blocks, int block_size,
+                                        float scale, hipStream_t stream = 0);
+
 // ---- fused layer steps (not in the reference as single functions) ---------------
 // Steps 1b-5 of full_attention_forward_paged (paged_attention.cu:331-360) in one launch:
 // qg is the interleaved Q|gate projection [T, NUM_ATTN_HEADS, 2*HEAD_DIM], k / v the K and
@@ -169,6 +178,12 @@ void paged_gqa_decode_attention_shared(AttentionWorkspace& ws, const __half* Q, 
                                        int table_stride, const int* d_seq_lens, int B, int max_seq_len,
                                        int shared_tokens, __half* out, int fa_layer_idx, int max_phys_blocks,
                                        int block_size, float scale, hipStream_t stream = 0);
+// The fork-tree call; gate may be null, otherwise as in the gated call below.
+void paged_gqa_decode_attention_grouped(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_tables,
+                                        int table_stride, const int* d_seq_lens, int B, int max_seq_len,
+                                        const drk_prefix_group* groups, int n_groups, const __half* gate,
+                                        int gate_stride, __half* out, int fa_layer_idx, int max_phys_blocks,
+                                        int block_size, float scale, hipStream_t stream = 0);
 void paged_gqa_decode_attention_gated_branches(AttentionWorkspace& ws, const __half* Q, __half* kv_pool,
                                                const int* d_tables, int table_stride, const int* d_seq_lens, int B,
                                                int max_seq_len, const __half* gate, int gate_stride, __half* out,

@@ -1,6 +1,7 @@
 // cache_manager.cpp -- see cache_manager.h.  Host bookkeeping only; the device is
 // reached through the C ABI (table upload, copy-on-write block copies).
 #include "cache_manager.h"
+#include <vector>
 #include "kv_swapper.h"
 #include "../communis/log.h"
 
@@ -535,6 +536,66 @@ int CacheManager::common_prefix_tokens(const int* branches, int n) const
         if (!same) break;
     }
     return blocks * block_size_;
+}
+
+int CacheManager::common_prefix_groups(const int* branches, int n, int max_group_branches, int min_tokens,
+                                       drk_prefix_group* out, int max_groups) const
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (!branches || !out || n < 2 || max_groups <= 0 || max_group_branches < 2) return 0;
+    for (int i = 0; i < n; i++) {
+        const int b = branches[i];
+        if (b < 0 || b >= max_branches_ || !alive_[b]) return 0;
+    }
+    // blocks neighbours i and i + 1 hold in common, from block 0 on (a missing page ends the run)
+    std::vector<int> lcp((size_t)n - 1);
+    for (int i = 0; i + 1 < n; i++) {
+        const int limit = std::min(std::min(seq_len_[branches[i]], seq_len_[branches[i + 1]]) / block_size_, max_logical_blocks_);
+        int k = 0;
+        for (; k < limit; k++) {
+            const int phys = h_tables_[cell(branches[i], k)];
+            if (phys < 0 || h_tables_[cell(branches[i + 1], k)] != phys) break;
+        }
+        lcp[(size_t)i] = k;
+    }
+    const int min_blocks = std::max(1, (min_tokens + block_size_ - 1) / block_size_);
+    struct Range { int lo, hi, base; };                       // positions [lo, hi) share blocks [0, base) through their ancestors
+    std::vector<Range> queue{{0, n, 0}};
+    int count = 0;
+    for (size_t qi = 0; qi < queue.size() && count < max_groups; qi++) {      // breadth first: parents before children
+        const Range r = queue[qi];
+        if (r.hi - r.lo < 2) continue;
+        int m = 0x7fffffff;
+        for (int i = r.lo; i + 1 < r.hi; i++) m = std::min(m, lcp[(size_t)i]);
+        int base = r.base;
+        if (m - base >= min_blocks) {
+            // the whole range shares blocks [base, m): one group, or several over the same blocks when it is too wide
+            const int width = r.hi - r.lo;
+            const int parts = (width + max_group_branches - 1) / max_group_branches;
+            if (count + parts > max_groups) break;
+            if (parts > 1) {
+                // each part is a tree of its own from here on
+                for (int p = 0; p < parts; p++) {
+                    const int lo = r.lo + p * max_group_branches, hi = std::min(lo + max_group_branches, r.hi);
+                    if (hi - lo < 2) continue;                     // a part of one branch: its tail reads the range
+                    out[count++] = drk_prefix_group{lo, hi - lo, base * block_size_, m * block_size_};
+                    queue.push_back({lo, hi, m});
+                }
+                continue;
+            }
+            out[count++] = drk_prefix_group{r.lo, width, base * block_size_, m * block_size_};
+            base = m;
+        }
+        // neighbours that share more than the whole range does form the children
+        int lo = r.lo;
+        for (int i = r.lo; i + 1 <= r.hi; i++) {
+            if (i + 1 == r.hi || lcp[(size_t)i] <= std::max(m, base)) {
+                if (i + 1 - lo >= 2) queue.push_back({lo, i + 1, base});
+                lo = i + 1;
+            }
+        }
+    }
+    return count;
 }
 
 bool CacheManager::branch_alive(int branch) const

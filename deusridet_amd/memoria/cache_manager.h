@@ -30,6 +30,7 @@
 // (cache_manager.cpp:143-147).  Only unshared blocks are ever evicted, so a block
 // on SSD belongs to exactly one table entry; fork_branch() treats it as a hole.
 #pragma once
+#include "drk_kv.h"
 
 #include "block_pool.h"
 #include "importance_scorer.h"
@@ -101,6 +102,15 @@ public:
     // (whole blocks only, capped by the shortest seq_len): what
     // paged_gqa_decode_attention_shared() may stream once for all of them.
     int  common_prefix_tokens(const int* branches, int n) const;
+    // The fork tree of the listed branches (consecutive ids: their table rows are one [n, stride] array) as
+    // the shared ranges paged_gqa_decode_attention_grouped() takes: group = branches [first_branch,
+    // first_branch + n_branches) (positions in `branches`) hold tokens [tok_begin, tok_end) in the same
+    // physical blocks.  Ranges are whole blocks, at least min_tokens long, over at most max_group_branches
+    // neighbours (a wider set is cut into several groups over the same range); parents come before their
+    // children, so that cutting the list short (max_groups) leaves a valid tree.  Only neighbours in the list
+    // are compared: fork branches that belong together one after the other.  Returns the number of groups.
+    int  common_prefix_groups(const int* branches, int n, int max_group_branches, int min_tokens,
+                              drk_prefix_group* out, int max_groups) const;
     // Recency update: move the entry to the back of the LRU order.
     void touch_block(int branch, int logical_idx);
     int  refcount(int phys_block) const { return pool_.refcount(phys_block); }

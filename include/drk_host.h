@@ -69,6 +69,9 @@ int   drkh_cm_fork_branch(void *cm, int parent, int pos);
 void  drkh_cm_release_branch(void *cm, int branch);
 void  drkh_cm_touch_block(void *cm, int branch, int logical);
 int   drkh_cm_common_prefix_tokens(void *cm, const int32_t *branches, int n);
+/* CacheManager::common_prefix_groups: out holds max_groups drk_prefix_group (4 x int32 each); returns the count */
+int   drkh_cm_common_prefix_groups(void *cm, const int32_t *branches, int n, int max_group_branches, int min_tokens,
+                                   int32_t *out, int max_groups);
 int   drkh_cm_block_location(void *cm, int branch, int logical);
 int   drkh_cm_evict_blocks(void *cm, int n);
 int   drkh_cm_ensure_free_blocks(void *cm, int n_free);
@@ -110,6 +113,13 @@ void drkh_paged_gqa_decode_attention_shared(const void *Q, void *kv_pool, const 
                                             const int32_t *d_seq_lens, int B, int max_seq_len, int shared_tokens,
                                             void *out, int fa_layer_idx, int max_phys_blocks, int block_size,
                                             float scale, void *stream);
+/* branches that share pages as a fork tree (groups: n_groups x 4 int32 as drkh_cm_common_prefix_groups wrote them;
+ * no reference counterpart) */
+int  drkh_paged_gqa_decode_grouped_supported(int block_size);
+void drkh_paged_gqa_decode_attention_grouped(const void *Q, void *kv_pool, const int32_t *d_tables, int table_stride,
+                                             const int32_t *d_seq_lens, int B, int max_seq_len,
+                                             const int32_t *groups, int n_groups, void *out, int fa_layer_idx,
+                                             int max_phys_blocks, int block_size, float scale, void *stream);
 void drkh_paged_prefill_attention(const void *Q, void *kv_pool, const int32_t *d_block_table, void *out,
                                   int fa_layer_idx, int pos_start, int M, int max_phys_blocks, int block_size,
                                   float scale, void *stream);

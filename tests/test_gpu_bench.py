@@ -15,7 +15,8 @@ KEYS = {"metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "
         "dtype", "data", "config", "roofline", "cpu_baseline"}
 
 
-@pytest.mark.parametrize("extra", [[], ["--ctx-mode", "uniform", "--no-other-configs"], ["--config", "3"], ["--config", "4"], ["--config", "4", "--kv-dtype", "fp8"],
+@pytest.mark.parametrize("extra", [[], ["--ctx-mode", "uniform", "--no-other-configs"], ["--config", "3"], ["--config", "3", "--forks", "prefix"],
+                                   ["--config", "3", "--shared-kernel", "pair"], ["--config", "4"], ["--config", "4", "--kv-dtype", "fp8"],
                                    ["--config", "5"], ["--config", "5", "--kv-dtype", "int8"], ["--config", "6"], ["--config", "7"]],
                          ids=lambda e: "-".join(x.strip("-") for x in e) or "default")
 def test_bench_workload_runs(dev, extra):
@@ -29,8 +30,10 @@ def test_bench_workload_runs(dev, extra):
     if not extra:
         # the default line carries the dominant kernel of every other configuration, each with its own roofline entry
         other = j["other_configs"]
-        assert set(other) == {"config3_shared_prefix", "config4_int8", "config4_fp8", "config4_int8_append", "config4_fp8_append",
-                              "config5_prefill"}
+        assert set(other) == {"config3_shared_prefix", "config3_fork_tree", "config4_int8", "config4_fp8", "config4_int8_append",
+                              "config4_fp8_append", "config5_prefill", "config5_prefill_int8", "config5_prefill_fp8",
+                              "config7_decode_d256", "config7_prefill_d256"}
+        assert len(other["config3_fork_tree"]["shared_ranges"]) >= 3
         for name, e in other.items():
             assert 0 < e["frac"] < 1 and e["avg_launch_us"] > 0 and e["peak"] in (8000.0, 2500.0), name
         assert j["hbm_read_probe_permuted_4KiB_GBps"] > 1000 and j["mfma_bf16_probe_TFLOPs"] > 500

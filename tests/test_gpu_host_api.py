@@ -200,6 +200,82 @@ def test_shared_prefix_branches_copy_on_write(dev):
         assert ok, (b, ma)
 
 
+def test_fork_tree_through_the_host_classes(dev):
+    """Branches that fork from one another at different block boundaries (and once inside a block): the groups
+    CacheManager::common_prefix_groups finds, handed to the grouped decode call, against the fp64 oracle on a
+    model in which every branch owns a private copy of its context."""
+    L, KVH, QH, D, bs = 2, 8, 32, 128, 16
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    lib = host.lib()
+    assert lib.drkh_paged_gqa_decode_grouped_supported(bs)
+    cm = host.CacheManager()
+    assert cm.init(160 * L * 2 * KVH * bs * D * 2, bs, None, 8)
+    NB, stride = cm.pool_max_blocks(), cm.table_stride()
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    rng = np.random.default_rng(71)
+    model = {0: (np.zeros((L, 0, KVH, D), np.uint16), np.zeros((L, 0, KVH, D), np.uint16))}
+
+    def bulk(b, m):
+        p0 = cm.seq_len(b)
+        assert model[b][0].shape[1] == p0 and cm.ensure_blocks_for_range(b, p0, m)
+        cm.sync_block_table(U.stream_ptr())               # copy-on-write copies, table upload
+        k, v = U.normal_bits(rng, (L, m, KVH, D), cabi.BF16), U.normal_bits(rng, (L, m, KVH, D), cabi.BF16)
+        dk, dv = U.dev_bytes(k), U.dev_bytes(v)
+        cabi.call("drk_kv_append_batch", C.byref(g), C.c_void_p(cm.pool_ptr()), C.c_void_p(cm.d_block_table(b)), 0, L, p0, m,
+                  U.p(dk), U.p(dv), cabi.BF16, U.stream_ptr())
+        U.sync()
+        model[b] = (np.concatenate([model[b][0], k], axis=1), np.concatenate([model[b][1], v], axis=1))
+        cm.set_seq_len(b, p0 + m)
+
+    def fork(parent, pos):
+        b = cm.fork_branch(parent, pos)
+        assert b > 0
+        model[b] = (model[parent][0][:, :pos].copy(), model[parent][1][:, :pos].copy())
+        return b
+
+    bulk(0, 20 * bs + 5)                                   # the persistent context: 325 tokens
+    b1 = fork(0, 20 * bs)                                  # at a block boundary
+    bulk(b1, 9 * bs + 3)
+    b2 = fork(b1, 28 * bs)                                 # 8 blocks into what b1 wrote
+    bulk(b2, 6 * bs)
+    b3 = fork(b2, 32 * bs)                                 # 4 blocks into what b2 wrote
+    bulk(b3, 2 * bs + 9)
+    b4 = fork(b1, 24 * bs + 7)                             # inside a block of b1: shares 24 whole blocks with it
+    bulk(b4, 3 * bs)
+    bulk(b2, 11)                                           # the parents go on after their children left
+    bulk(0, 2 * bs)
+    branches = [0, b1, b2, b3, b4]
+    assert branches == list(range(5))
+    groups = cm.common_prefix_groups(branches, 64 // (QH // KVH), 4 * bs)
+    assert groups == [(0, 5, 0, 20 * bs), (1, 4, 20 * bs, 24 * bs), (1, 3, 24 * bs, 28 * bs), (2, 2, 28 * bs, 32 * bs)]
+
+    B = len(branches)
+    lens = np.array([cm.seq_len(b) for b in branches], dtype=np.int32)
+    q = U.normal_bits(rng, (B, QH, D), cabi.BF16)
+    dq, dl = U.dev_bytes(q), U.dev_i32(lens)
+    scale = 1 / np.sqrt(D)
+    cm.sync_block_table(U.stream_ptr())
+    garr = np.array(groups, dtype=np.int32)
+    outs = []
+    for n_groups in (len(groups), 2, 0):                   # the whole tree, its first two levels, no sharing at all
+        out = U.dev_zeros(B * QH * D * 2)
+        lib.drkh_paged_gqa_decode_attention_grouped(U.p(dq), cm.pool_ptr(), cm.d_block_table(0), stride, U.p(dl), B,
+                                                    int(lens.max()), garr.ctypes.data_as(C.c_void_p), n_groups, U.p(out), 1,
+                                                    NB, bs, float(scale), U.stream_ptr())
+        U.sync()
+        outs.append(U.from_bits(U.host(out, np.uint16, (B, QH, D)), cabi.BF16))
+    for i, b in enumerate(branches):
+        n = int(lens[i])
+        pg = orc.layout(L, KVH, QH, D, bs, (n + bs - 1) // bs, orc.BF16)
+        ppool = orc.new_pool(pg)
+        ptab = np.arange((n + bs - 1) // bs, dtype=np.int32)
+        orc.append_batch(pg, ppool, ptab, 1, 0, model[b][0][1], model[b][1][1], orc.BF16)
+        want = orc.decode_f64(pg, q[i], ppool, ptab, 1, n, scale, orc.BF16)
+        for got in outs:
+            ok, ma, _ = U.rel_abs_ok(got[i], want)
+            assert ok, (b, ma)
+
+
 def test_importance_scorer_on_device(dev):
     sc = host.ImportanceScorer()
     assert sc.init(64, 0.5)
