@@ -11,6 +11,7 @@ reached through the C ABI in include/drk_kv.h.
 """
 import argparse
 import ctypes as C
+import gc
 import json
 import os
 import re
@@ -98,6 +99,11 @@ def main():
     from deusridet_amd import cabi
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    # The interpreter's cycle collector stays off while anything is timed: a full collection over torch's and numpy's
+    # objects takes tens of milliseconds, and the workloads that launch every kernel from Python (config 3: some 110
+    # calls a step) reach its threshold in the middle of their timed steps.
+    gc.collect()
+    gc.disable()
     cabi.lib().drk_debug_set_grouped_decode(1 if args.shared_kernel == "pair" else 0)
     if args.config != 2:
         import bench_extra

@@ -6,6 +6,7 @@ for memory, streams and events; kernels go through the C ABI, block tables of
 config 3 through the C++ CacheManager.
 """
 import ctypes as C
+import sys
 import time
 
 import numpy as np

@@ -114,6 +114,7 @@ void KvStream::prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipSt
     if (scorer_ && scorer_->d_new_scores()) {
         const bool first = first_layer_of_frame_ < 0;
         if (first) first_layer_of_frame_ = fa_layer_idx;
+        frame_stream_ = stream;
         paged_prefill_attention_mass(io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), fa_layer_idx, current_pos_, M,
                                      pool.max_blocks(), pool.block_size(), 1.0f / std::sqrt((float)hd),
                                      scorer_->d_new_scores(), cm_->table_stride(), !first, stream);
@@ -123,11 +124,12 @@ void KvStream::prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipSt
 void KvStream::end_prefill(int M, hipStream_t stream)
 {
     if (scorer_ && first_layer_of_frame_ >= 0) {
-        // fold the frame's masses into the scores; the row is cleared behind that, or every decode step's fold
-        // would count the frame again
-        scorer_->apply_new_scores(stream);
-        if (drk_dev_memset_async(scorer_->d_new_scores(), 0, (size_t)cm_->table_stride() * sizeof(float), stream) != DRK_OK)
-            LOG_ERROR("Conscientia", "KvStream: clearing the frame's attention masses: %s", drk_last_error());
+        // Fold the frame's masses into the scores of the stream's own row, and clear them in the same pass (or
+        // every later fold would count the frame again).  Only that row: the rows of open decode branches still
+        // hold their last step's masses, which that step has folded in already.  The fold goes behind the mass
+        // passes, on the stream they ran on, whatever the caller passes (or leaves out) here.
+        (void)stream;
+        scorer_->apply_new_scores(0, cm_->table_stride(), frame_stream_);
         first_layer_of_frame_ = -1;
     }
     current_pos_ += M;                                                    // stream.cpp:238-239
@@ -344,10 +346,12 @@ bool KvStream::replay_decode_step(hipStream_t stream)
 {
     if (!graph_) return false;
     if (!host_begin(stream)) return false;
+    if (scorer_) scorer_->wait_for_last_fold(stream);     // the recorded fold could not wait for a frame's by itself
     if (drk_graph_launch(graph_, stream) != DRK_OK) {
         LOG_ERROR("Conscientia", "KvStream: graph launch: %s", drk_last_error());
         return false;
     }
+    if (scorer_ && scorer_->d_new_scores()) scorer_->note_fold_on(stream);
     host_end();
     return true;
 }

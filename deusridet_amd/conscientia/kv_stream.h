@@ -62,7 +62,9 @@ public:
     // pages they forked from, the stream copies a block it still shares before it writes into it.
     bool begin_prefill(int M, hipStream_t stream);
     void prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipStream_t stream);
-    // with a scorer attached the frame's attention masses are folded into the scores here, on `stream`
+    // With a scorer attached the frame's attention masses are folded into the scores of the stream's own row here
+    // (and cleared), on the stream the frame's prefill_layer calls ran on -- not on `stream`, which only keeps the
+    // reference's call shape: a fold on another stream could overtake the mass passes.
     void end_prefill(int M, hipStream_t stream = nullptr);
     int  current_pos() const { return current_pos_; }
 
@@ -125,6 +127,7 @@ private:
     int max_prefill_rows_ = 0;
     int first_layer_of_step_ = -1;   // the layer whose scored call overwrites instead of accumulating
     int first_layer_of_frame_ = -1;  // the same for the mass pass of a perception frame
+    hipStream_t frame_stream_ = nullptr;   // stream of the frame's mass passes
 
     bool host_begin(hipStream_t stream);
     void host_end();

@@ -305,6 +305,17 @@ __global__ void importance_update_kernel(float *__restrict__ scores, const float
     if (b < n) scores[b] = __builtin_fmaf(scores[b], decay, new_scores[b]);
 }
 
+// The same fold for a range whose new scores are spent with it: they are cleared in the same pass
+// (a fill kernel of its own would be one more launch; a memset node may not be recorded into a graph).
+__global__ void importance_fold_clear_kernel(float *__restrict__ scores, float *__restrict__ new_scores, int n, float decay)
+{
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < n) {
+        scores[b] = __builtin_fmaf(scores[b], decay, new_scores[b]);
+        new_scores[b] = 0.0f;
+    }
+}
+
 static int check_src_dtype(int d)
 {
     if (d != DRK_F16 && d != DRK_BF16) return fail(DRK_ERR_INVALID, "src_dtype must be F16 or BF16");
@@ -480,6 +491,16 @@ int drk_importance_update(float *d_scores, const float *d_new_scores, int n, flo
     hipLaunchKernelGGL(importance_update_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
                        d_scores, d_new_scores, n, decay);
     DRK_LAUNCH_CHECK("importance_update_kernel");
+    return DRK_OK;
+}
+
+int drk_importance_fold_clear(float *d_scores, float *d_new_scores, int n, float decay, void *stream)
+{
+    if (n <= 0) return DRK_OK;
+    if (!d_scores || !d_new_scores) return fail(DRK_ERR_INVALID, "importance_fold_clear: NULL pointer");
+    hipLaunchKernelGGL(importance_fold_clear_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       d_scores, d_new_scores, n, decay);
+    DRK_LAUNCH_CHECK("importance_fold_clear_kernel");
     return DRK_OK;
 }
 

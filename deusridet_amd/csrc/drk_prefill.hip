@@ -2516,7 +2516,9 @@ size_t drk_prefill_workspace_bytes_max(const drk_kv_layout *g, int max_seq_len, 
     if (!mfma) return drk_decode_workspace_bytes(g, max_rows, max_seq_len);
     // the pieces per row grow with the context: the chunk that ends at max_seq_len needs the most for its length
     size_t need = 0;
-    const int top = max_rows < kSplitMaxM ? max_rows : kSplitMaxM;
+    // (the debug switch drk_debug_set_prefill_split(n) lets chunks of up to n rows take the split path)
+    const int widest = g_prefill_split > kSplitMaxM ? g_prefill_split : kSplitMaxM;
+    const int top = max_rows < widest ? max_rows : widest;
     for (int M = 1; M <= top; M++) {
         const size_t n = drk_prefill_workspace_bytes(g, max_seq_len - M, M);
         if (n > need) need = n;
@@ -2543,9 +2545,12 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
         return fail(DRK_ERR_INVALID, "prefill: io_dtype %d differs from the pool's %d", io_dtype, a.dtype);
     if (layer < 0 || layer >= a.L) return fail(DRK_ERR_INVALID, "prefill: layer %d outside [0,%d)", layer, a.L);
+    // the MFMA kernels fold the scale into the exponent's base-2 factor and assume it positive; a softmax scale
+    // is 1/sqrt(head_dim) or close to it
+    if (!(scale > 0.0f)) return fail(DRK_ERR_INVALID, "prefill: scale must be positive (got %g)", (double)scale);
 
     const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 &&
-                      a.QH / a.KVH <= 128 && (a.bs % 16) == 0 && scale > 0.0f;
+                      a.QH / a.KVH <= 128 && (a.bs % 16) == 0;
     if (!mfma)
         return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
                              io_dtype, 0, workspace, workspace_bytes, stream, gate, gate_stride);

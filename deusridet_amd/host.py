@@ -38,10 +38,13 @@ SIGNATURES = {
     "drkh_swapper_is_prefetched": (_i32, [_vp, _i32]),
     "drkh_swapper_block_bytes": (_sz, [_vp]),
     "drkh_swapper_swap": (_i32, [_vp, _i32, _i32, _i32, C.c_char_p]),
+    "drkh_swapper_swap_many": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "drkh_swapper_remove_writer_stream": (None, [_vp, _vp]),
     "drkh_cm_init_detached": (_i32, [_vp, _i32, _i32, _vp, _i32]),
     "drkh_cm_ensure_blocks_for": (_i32, [_vp, _i32, _i32]),
     "drkh_cm_ensure_blocks_for_range": (_i32, [_vp, _i32, _i32, _i32]),
     "drkh_cm_sync_block_table": (None, [_vp, _vp]),
+    "drkh_cm_forget_stream": (None, [_vp, _vp]),
     "drkh_cm_d_block_table": (_vp, [_vp, _i32]), "drkh_cm_h_block_table": (_ip, [_vp, _i32]),
     "drkh_cm_table_stride": (_i32, [_vp]),
     "drkh_cm_seq_len": (_i32, [_vp, _i32]), "drkh_cm_set_seq_len": (None, [_vp, _i32, _i32]),
@@ -102,6 +105,7 @@ SIGNATURES = {
     "drkh_kvs_replay_decode_step": (_i32, [_vp, _vp]),
     "drkh_scorer_d_new_scores": (_vp, [_vp]),
     "drkh_scorer_apply_new_scores": (None, [_vp, _vp]),
+    "drkh_scorer_apply_new_scores_range": (None, [_vp, _i32, _i32, _vp]),
     "drkh_paged_gqa_decode_attention_branches_scored": (None, [_vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32,
                                                                _f32, _vp, _i32, _vp]),
     "drkh_set_rope": (_i32, [_i32, _f32, _f32]),
@@ -166,6 +170,7 @@ class ImportanceScorer:
     def sync_to_host(self): lib().drkh_scorer_sync_to_host(self._h)
     def d_new_scores(self): return lib().drkh_scorer_d_new_scores(self._h)
     def apply_new_scores(self, stream=None): lib().drkh_scorer_apply_new_scores(self._h, stream)
+    def apply_new_scores_range(self, first, count, stream=None): lib().drkh_scorer_apply_new_scores_range(self._h, first, count, stream)
 
     def least_important(self, ids):
         a = np.ascontiguousarray(ids, dtype=np.int32)
@@ -235,6 +240,19 @@ class KVSwapper:
     def prefetch(self, idx, path): lib().drkh_swapper_prefetch(self._h, idx, str(path).encode())
     def is_prefetched(self, idx): return bool(lib().drkh_swapper_is_prefetched(self._h, idx))
     def block_bytes(self): return lib().drkh_swapper_block_bytes(self._h)
+    def remove_writer_stream(self, stream): lib().drkh_swapper_remove_writer_stream(self._h, stream)
+
+    def swap_many(self, requests):
+        """requests: (direction 0 out / 1 in, logical idx, physical block or -1 for a prefetch, path); submitted in order,
+        then drained.  Returns (completion order, ok per request)."""
+        n = len(requests)
+        d = np.array([r[0] for r in requests], dtype=np.int32)
+        lg = np.array([r[1] for r in requests], dtype=np.int32)
+        ph = np.array([r[2] for r in requests], dtype=np.int32)
+        paths = (C.c_char_p * n)(*[str(r[3]).encode() for r in requests])
+        order, ok = np.full(n, -1, dtype=np.int32), np.zeros(n, dtype=np.int32)
+        done = lib().drkh_swapper_swap_many(self._h, n, _p(d), _p(lg), _p(ph), C.cast(paths, C.c_void_p), _p(order), _p(ok))
+        return [int(x) for x in order[:done]], [bool(x) for x in ok]
     def swap_out(self, idx, phys, path): return bool(lib().drkh_swapper_swap(self._h, 0, idx, phys, str(path).encode()))
     def swap_in(self, idx, phys, path): return bool(lib().drkh_swapper_swap(self._h, 1, idx, phys, str(path).encode()))
 
@@ -270,6 +288,7 @@ class CacheManager:
     def ensure_blocks_for(self, branch, pos): return bool(lib().drkh_cm_ensure_blocks_for(self._h, branch, pos))
     def ensure_blocks_for_range(self, branch, pos, M): return bool(lib().drkh_cm_ensure_blocks_for_range(self._h, branch, pos, M))
     def sync_block_table(self, stream=None): lib().drkh_cm_sync_block_table(self._h, stream)
+    def forget_stream(self, stream): lib().drkh_cm_forget_stream(self._h, stream)
     def d_block_table(self, branch=0): return lib().drkh_cm_d_block_table(self._h, branch)
     def table_stride(self): return lib().drkh_cm_table_stride(self._h)
     def seq_len(self, branch=0): return lib().drkh_cm_seq_len(self._h, branch)

@@ -1,5 +1,6 @@
 // host_capi.cpp -- the C shim declared in include/drk_host.h: one-line forwarders
 // to the C++ host classes.
+#include <mutex>
 #include "drk_host.h"
 
 #include "../machina/paged_attention.h"
@@ -78,6 +79,31 @@ int drkh_swapper_swap(void *sw, int direction, int logical_block_idx, int physic
     SW(sw)->drain();
     return success ? 1 : 0;
 }
+int drkh_swapper_swap_many(void *sw, int n, const int32_t *direction, const int32_t *logical_block_idx,
+                           const int32_t *physical_block_id, const char *const *path, int32_t *completion_order,
+                           int32_t *ok)
+{
+    std::mutex mu;
+    int done = 0;
+    for (int i = 0; i < n; i++) {
+        SwapRequest req;
+        req.direction = direction[i] == 0 ? SwapDirection::GPU_TO_SSD : SwapDirection::SSD_TO_GPU;
+        req.logical_block_idx = logical_block_idx[i];
+        req.physical_block_id = physical_block_id[i];
+        req.ssd_path = path[i] ? path[i] : "";
+        req.callback = [&, i](bool success) {
+            std::lock_guard<std::mutex> lock(mu);
+            if (completion_order) completion_order[done] = i;
+            if (ok) ok[i] = success ? 1 : 0;
+            done++;
+        };
+        SW(sw)->submit(std::move(req));
+    }
+    SW(sw)->drain();
+    std::lock_guard<std::mutex> lock(mu);
+    return done;
+}
+void drkh_swapper_remove_writer_stream(void *sw, void *stream) { SW(sw)->remove_writer_stream(ST(stream)); }
 int drkh_cm_init_detached(void *cm, int max_blocks, int block_size, void *scorer, int max_branches)
 {
     return CM(cm)->init_detached(max_blocks, block_size, SC(scorer), max_branches) ? 1 : 0;
@@ -88,6 +114,7 @@ int drkh_cm_ensure_blocks_for_range(void *cm, int branch, int pos_start, int M)
     return CM(cm)->ensure_blocks_for_range(branch, pos_start, M) ? 1 : 0;
 }
 void drkh_cm_sync_block_table(void *cm, void *stream) { CM(cm)->sync_block_table(ST(stream)); }
+void drkh_cm_forget_stream(void *cm, void *stream) { CM(cm)->forget_stream(ST(stream)); }
 const int32_t *drkh_cm_d_block_table(void *cm, int branch) { return CM(cm)->d_block_table(branch); }
 const int32_t *drkh_cm_h_block_table(void *cm, int branch) { return CM(cm)->h_block_table(branch); }
 int drkh_cm_table_stride(void *cm) { return CM(cm)->table_stride(); }
@@ -297,6 +324,7 @@ int drkh_kvs_capture_decode_step(void *ks, void (*layers)(void *stream, void *us
 int drkh_kvs_replay_decode_step(void *ks, void *stream) { return KS(ks)->replay_decode_step((hipStream_t)stream) ? 1 : 0; }
 void *drkh_scorer_d_new_scores(void *s) { return SC(s)->d_new_scores(); }
 void drkh_scorer_apply_new_scores(void *s, void *stream) { SC(s)->apply_new_scores((hipStream_t)stream); }
+void drkh_scorer_apply_new_scores_range(void *sc, int first, int count, void *stream) { SC(sc)->apply_new_scores(first, count, ST(stream)); }
 void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_pool, const int32_t *d_tables,
                                                      int table_stride, const int32_t *d_seq_lens, int B,
                                                      int max_seq_len, void *out, int fa_layer_idx,

@@ -426,6 +426,12 @@ void CacheManager::flush_copies(hipStream_t stream)
     pending_copies_.clear();
 }
 
+void CacheManager::forget_stream(hipStream_t stream)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    if (swapper_) swapper_->remove_writer_stream(stream);
+}
+
 void CacheManager::sync_block_table(hipStream_t stream)
 {
     std::lock_guard<std::mutex> lock(mu_);

@@ -80,6 +80,9 @@ public:
     // Issue queued copy-on-write copies, then upload changed table ranges, both on
     // `stream`, asynchronously (cache_manager.cpp:108-112).
     void sync_block_table(hipStream_t stream = 0);
+    // With an overflow tier every stream passed to sync_block_table() is remembered (swaps order themselves behind
+    // it); call this before such a stream is destroyed.
+    void forget_stream(hipStream_t stream);
     const int* h_block_table(int branch = 0) const;
 
     int  seq_len() const { return seq_len(0); }

@@ -71,13 +71,51 @@ float* ImportanceScorer::d_new_scores()
     return d_new_;
 }
 
+namespace {
+bool stream_is_capturing(hipStream_t stream)
+{
+    int capturing = 0;
+    return stream && drk_stream_is_capturing(stream, &capturing) == DRK_OK && capturing;
+}
+}
+
+void ImportanceScorer::wait_for_last_fold(hipStream_t stream)
+{
+    if (!fold_marked_ || stream == last_apply_stream_) return;
+    if (drk_stream_wait_event(stream, fold_done_) != DRK_OK)
+        LOG_ERROR("Memoria", "ImportanceScorer: waiting for the last fold: %s", drk_last_error());
+}
+
+void ImportanceScorer::note_fold_on(hipStream_t stream)
+{
+    if (!fold_done_ && drk_event_create(&fold_done_) != DRK_OK) {
+        LOG_ERROR("Memoria", "ImportanceScorer: event: %s", drk_last_error());
+        fold_done_ = nullptr;
+    }
+    last_apply_stream_ = stream;
+    applied_ = true;
+    fold_marked_ = fold_done_ && drk_event_record(fold_done_, stream) == DRK_OK;
+}
+
 void ImportanceScorer::apply_new_scores(hipStream_t stream)
 {
     if (!d_scores_ || !d_new_) return;
+    const bool captured = stream_is_capturing(stream);
+    if (!captured) wait_for_last_fold(stream);
     if (drk_importance_update(d_scores_, d_new_, max_blocks_, decay_, stream) != DRK_OK)
         LOG_ERROR("Memoria", "ImportanceScorer: apply_new_scores: %s", drk_last_error());
-    last_apply_stream_ = stream;
-    applied_ = true;
+    if (!captured) note_fold_on(stream);
+}
+
+void ImportanceScorer::apply_new_scores(int first, int count, hipStream_t stream)
+{
+    if (!d_scores_ || !d_new_ || first < 0 || count <= 0 || first >= max_blocks_) return;
+    if (count > max_blocks_ - first) count = max_blocks_ - first;
+    const bool captured = stream_is_capturing(stream);
+    if (!captured) wait_for_last_fold(stream);
+    if (drk_importance_fold_clear(d_scores_ + first, d_new_ + first, count, decay_, stream) != DRK_OK)
+        LOG_ERROR("Memoria", "ImportanceScorer: apply_new_scores(range): %s", drk_last_error());
+    if (!captured) note_fold_on(stream);
 }
 
 int ImportanceScorer::least_important(const int* gpu_resident, int n) const
@@ -130,6 +168,11 @@ void ImportanceScorer::destroy()
         d_new_ = nullptr;
     }
     applied_ = false;
+    fold_marked_ = false;
+    if (fold_done_) {
+        drk_event_destroy(fold_done_);
+        fold_done_ = nullptr;
+    }
     if (scorer_stream_) {
         drk_stream_destroy(scorer_stream_);
         scorer_stream_ = nullptr;

@@ -35,6 +35,16 @@ public:
     // branch * table_stride + logical block, so max_blocks must cover max_branches * table_stride.
     float* d_new_scores();
     void apply_new_scores(hipStream_t stream);
+    // The same fold for cells [first, first + count) only, whose new scores are cleared with it: what a
+    // perception frame does with the stream's own row while the rows of open decode branches keep the
+    // masses of their last step (those were folded in by that step and must not be counted again).
+    void apply_new_scores(int first, int count, hipStream_t stream);
+    // Folds read and write the scores, so two of them must not run at once.  Each fold waits for the one
+    // before it when that ran on another stream, and marks its own end for the next.  A fold recorded into a
+    // graph cannot do either (the capture may not wait on work outside it): whoever replays such a graph calls
+    // wait_for_last_fold(stream) before the launch and note_fold_on(stream) behind it.
+    void wait_for_last_fold(hipStream_t stream);
+    void note_fold_on(hipStream_t stream);
 
     // First minimum over the given logical block ids in list order, from the host
     // mirror (importance_scorer.cu:75-87).  -1 when n <= 0.
@@ -55,6 +65,8 @@ private:
     float* d_new_ = nullptr;
     hipStream_t last_apply_stream_ = nullptr;
     bool applied_ = false;
+    void* fold_done_ = nullptr;          // event: end of the last fold that was launched (not captured)
+    bool fold_marked_ = false;
     std::vector<float> h_scores_;
     int max_blocks_ = 0;
     float decay_ = 0.95f;

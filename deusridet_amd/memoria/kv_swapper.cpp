@@ -94,6 +94,12 @@ void KVSwapper::add_writer_stream(hipStream_t stream)
     if (std::find(writers_.begin(), writers_.end(), stream) == writers_.end()) writers_.push_back(stream);
 }
 
+void KVSwapper::remove_writer_stream(hipStream_t stream)
+{
+    std::lock_guard<std::mutex> lock(mu_);
+    writers_.erase(std::remove(writers_.begin(), writers_.end(), stream), writers_.end());
+}
+
 // Called on the requester's thread: the events mark what the pool's users have been given up
 // to now -- everything that wrote, or may still read, the block of this request.
 void KVSwapper::submit(SwapRequest req)
@@ -101,7 +107,13 @@ void KVSwapper::submit(SwapRequest req)
     Ticket t;
     t.req = std::move(req);
     {
-        std::lock_guard<std::mutex> lock(mu_);
+        std::unique_lock<std::mutex> lock(mu_);
+        if (!running_) {                              // no worker would ever take it: fail it here
+            lock.unlock();
+            LOG_ERROR("Memoria", "KVSwapper: submit() on a swapper that is not running (block %d)", t.req.logical_block_idx);
+            if (t.req.callback) t.req.callback(false);
+            return;
+        }
         if (t.req.physical_block_id >= 0) {
             for (hipStream_t w : writers_) {
                 int capturing = 0;
@@ -133,6 +145,17 @@ void KVSwapper::shutdown()
     }
     cv_.notify_all();
     if (worker_.joinable()) worker_.join();          // the worker empties the queue before it leaves
+    // what a worker that never started (init failed half-way) or a late submit() left behind fails here
+    std::deque<Ticket> left;
+    {
+        std::lock_guard<std::mutex> lock(mu_);
+        left.swap(queue_);
+    }
+    for (Ticket& t : left) complete(t, false);
+    {
+        std::lock_guard<std::mutex> lock(mu_);
+        unfinished_ = 0;
+    }
     for (void* h : slots_)
         if (h) drk_host_free(h);
     for (void* e : slot_done_)
@@ -313,6 +336,7 @@ void KVSwapper::run()
                     host_cache_[t.req.logical_block_idx] = std::move(image);
             }
             if (!ok) LOG_ERROR("Memoria", "KVSwapper: prefetch of %s failed", t.req.ssd_path.c_str());
+            while (!flying.empty()) finish_oldest();      // completion order is submission order
             complete(t, ok);
             continue;
         }
@@ -324,6 +348,7 @@ void KVSwapper::run()
             flying.push_back(std::move(f));
         } else {
             free_slots.push_back(f.slot);
+            while (!flying.empty()) finish_oldest();      // the older requests call back first
             complete(f.t, false);
         }
     }

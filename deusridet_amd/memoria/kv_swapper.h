@@ -56,7 +56,7 @@ public:
     bool init(BlockPool& pool, const std::string& ssd_dir, int staging_blocks = 2);
     bool ready() const { return running_; }
 
-    void submit(SwapRequest req);          // non-blocking
+    void submit(SwapRequest req);          // non-blocking; on a swapper that is not running the callback gets false at once
     void drain();                          // until every submitted request has completed
     void shutdown();
     int  pending() const;
@@ -68,6 +68,8 @@ public:
     // A stream whose kernels write or read the pool: requests submitted from now on wait for what
     // that stream had been given when they were submitted.  Idempotent.
     void add_writer_stream(hipStream_t stream);
+    // Before such a stream is destroyed: later requests must not record events on a dead handle.
+    void remove_writer_stream(hipStream_t stream);
 
     size_t block_bytes() const { return block_bytes_; }
 

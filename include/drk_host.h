@@ -55,10 +55,18 @@ int   drkh_swapper_is_prefetched(void *sw, int logical_block_idx);
 size_t drkh_swapper_block_bytes(void *sw);
 /* one synchronous request through the queue: direction 0 = GPU -> file, 1 = file -> GPU; returns success */
 int   drkh_swapper_swap(void *sw, int direction, int logical_block_idx, int physical_block_id, const char *path);
+/* n requests submitted one after the other, then drain(): completion_order[k] = index of the k-th request whose
+ * callback ran, ok[i] = its result (either may be NULL); returns the number of callbacks.  physical_block_id < 0 with
+ * direction 1 is a prefetch (file -> host cache). */
+int   drkh_swapper_swap_many(void *sw, int n, const int32_t *direction, const int32_t *logical_block_idx,
+                             const int32_t *physical_block_id, const char *const *path, int32_t *completion_order,
+                             int32_t *ok);
+void  drkh_swapper_remove_writer_stream(void *sw, void *stream);     /* KVSwapper::remove_writer_stream */
 int   drkh_cm_init_detached(void *cm, int max_blocks, int block_size, void *scorer, int max_branches);
 int   drkh_cm_ensure_blocks_for(void *cm, int branch, int pos);
 int   drkh_cm_ensure_blocks_for_range(void *cm, int branch, int pos_start, int M);
 void  drkh_cm_sync_block_table(void *cm, void *stream);
+void  drkh_cm_forget_stream(void *cm, void *stream);      /* CacheManager::forget_stream: before the stream is destroyed */
 const int32_t *drkh_cm_d_block_table(void *cm, int branch);
 const int32_t *drkh_cm_h_block_table(void *cm, int branch);
 int   drkh_cm_table_stride(void *cm);
@@ -175,6 +183,7 @@ int   drkh_kvs_capture_decode_step(void *ks, void (*layers)(void *stream, void *
 int   drkh_kvs_replay_decode_step(void *ks, void *stream);
 void *drkh_scorer_d_new_scores(void *s);
 void drkh_scorer_apply_new_scores(void *s, void *stream);
+void  drkh_scorer_apply_new_scores_range(void *sc, int first, int count, void *stream);   /* cells [first, first + count): folded and their new scores cleared */
 void drkh_paged_gqa_decode_attention_branches_scored(const void *Q, void *kv_pool, const int32_t *d_tables,
                                                      int table_stride, const int32_t *d_seq_lens, int B,
                                                      int max_seq_len, void *out, int fa_layer_idx,

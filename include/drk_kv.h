@@ -283,7 +283,9 @@ int drk_paged_decode_attention_grouped(const drk_kv_layout *g, const void *q, co
  * the workspace. */
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M);
 /* The most drk_prefill_workspace_bytes reports for any chunk of up to max_rows rows that
- * ends at or before max_seq_len tokens: what a caller reserves once, up front. */
+ * ends at or before max_seq_len tokens: what a caller reserves once, up front.  (Both sizes follow the
+ * debug switches of drk_debug.h as they stand at the time of the call: reserve after setting them.)
+ * scale must be positive: DRK_ERR_INVALID otherwise. */
 size_t drk_prefill_workspace_bytes_max(const drk_kv_layout *g, int max_seq_len, int max_rows);
 int drk_paged_prefill_attention(const drk_kv_layout *g, const void *q, const void *pool,
                                 const int32_t *d_block_table, void *out, int layer,
@@ -391,6 +393,9 @@ int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, cons
 /* importance_update_kernel, importance_scorer.cu:27-36, 67-73 */
 int drk_importance_update(float *d_scores, const float *d_new_scores, int n, float decay,
                           void *stream);
+/* The same fold over a range whose new scores are spent with it: d_new_scores[0..n) is zero afterwards (no
+ * reference counterpart: the reference's scorer is never fed).  One launch, no memset node: may be captured. */
+int drk_importance_fold_clear(float *d_scores, float *d_new_scores, int n, float decay, void *stream);
 
 #ifdef __cplusplus
 }

@@ -330,3 +330,24 @@ def test_short_chunks_behind_a_long_context(dev, geom, dtype, io, pos_start, M):
     U.sync()
     gated = orc.sigmoid_gate(raw, np.ascontiguousarray(qg[:, :, D:]), io)
     assert U.ulp_distance(U.host(out, np.uint16, (M, QH, D)), gated).max() <= 1
+
+
+def test_prefill_refuses_a_scale_that_is_not_positive_and_sizes_follow_the_debug_switch(dev):
+    """The size a caller reserves once must cover what the split path asks for also when the debug switch widens
+    that path; a softmax scale of zero or less is refused before anything is launched."""
+    lib = cabi.lib()
+    geom = (1, 8, 32, 128, 16, 600)
+    g = cabi.layout(*geom, cabi.BF16)
+    try:
+        lib.drk_debug_set_prefill_split(1500)
+        top = lib.drk_prefill_workspace_bytes_max(C.byref(g), 8192, 2048)
+        assert top >= lib.drk_prefill_workspace_bytes(C.byref(g), 8192 - 1500, 1500) > 0
+    finally:
+        lib.drk_debug_set_prefill_split(-1)
+    buf = U.dev_zeros(64 * 32 * 128 * 2)
+    pool = U.dev_zeros(lib.drk_kv_pool_bytes(C.byref(g)))
+    tab = U.dev_i32(np.arange(600, dtype=np.int32))
+    for scale in (0.0, -0.1, float("nan")):
+        rc = lib.drk_paged_prefill_attention(C.byref(g), U.p(buf), U.p(pool), U.p(tab), U.p(buf), 0, 0, 64, scale, cabi.BF16,
+                                             None, 0, U.stream_ptr())
+        assert rc == cabi.ERR_INVALID and b"scale" in lib.drk_last_error()

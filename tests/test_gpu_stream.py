@@ -330,6 +330,77 @@ def test_perception_frames_feed_the_scorer(dev):
     assert np.array_equal(s.pool(), opool)
 
 
+@pytest.mark.parametrize("mode", ["eager", "graph"])
+def test_scorer_with_branches_open_across_perception_frames(dev, mode):
+    """A frame folds its masses into the stream's own row only: the rows of open branches still hold their last
+    step's masses, which that step folded in already -- a frame must neither count them again nor age them.
+    Frames and decode steps run on two streams (the folds order themselves); in graph mode the step's fold is
+    part of the replayed graph.  Per row, mass sums are known in closed form: a decode step gives every branch
+    L * QH, a frame of M tokens gives the stream M * L * QH; every fold of a row halves what it held."""
+    import torch
+    nbranch = 2
+    s = Session(nbranch, scorer=True)
+    rng = np.random.default_rng(133)
+    s.set_weights(U.normal_bits(rng, (D,), DT), U.normal_bits(rng, (D,), DT))
+    frames, steps = torch.cuda.Stream(), torch.cuda.Stream()
+    fp, sp = C.c_void_p(frames.cuda_stream), C.c_void_p(steps.cuda_stream)
+    stride = s.cm.table_stride()
+    LQ = L * QH
+
+    def frame(M):
+        assert s.ks.begin_prefill(M, fp)
+        for layer in range(L):
+            qg, k, v = (U.normal_bits(rng, sh, DT, m) for sh, m in (((M, QH, 2 * D), 1.0), ((M, KVH, D), 0.7), ((M, KVH, D), 0.5)))
+            frames.synchronize()                           # the previous layer has read the buffers
+            s.load(qg, k, v)
+            torch.cuda.current_stream().synchronize()      # the copies ran on torch's stream; the step's stream is not waited for
+            s.ks.prefill_layer(layer, s.io(), M, fp)
+        s.ks.end_prefill(M)                                # no stream given: the fold follows the layers' stream
+
+    lay_bufs = [dict(qg=U.dev_zeros(nbranch * QH * 2 * D * 2), k=U.dev_zeros(nbranch * KVH * D * 2), v=U.dev_zeros(nbranch * KVH * D * 2),
+                     q=U.dev_zeros(nbranch * QH * D * 2), out=U.dev_zeros(nbranch * QH * D * 2)) for _ in range(L)]
+
+    def layers(stream):
+        for layer in range(L):
+            b = lay_bufs[layer]
+            s.ks.decode_layer(layer, (U.p(b["qg"]), U.p(b["k"]), U.p(b["v"]), U.p(s.dqw), U.p(s.dkw), U.p(b["q"]), U.p(b["out"])), stream)
+
+    def step():
+        steps.synchronize()                                # the previous step has read its inputs
+        for layer in range(L):
+            for name, sh, m in (("qg", (nbranch, QH, 2 * D), 1.0), ("k", (nbranch, KVH, D), 0.7), ("v", (nbranch, KVH, D), 0.5)):
+                a = U.normal_bits(rng, sh, DT, m)
+                lay_bufs[layer][name].copy_(torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(-1)))
+        torch.cuda.current_stream().synchronize()          # the frame's last layers and its fold may still be running
+        if mode == "graph":
+            assert s.ks.replay_decode_step(sp)
+        else:
+            assert s.ks.begin_decode_step(sp)
+            layers(sp)
+            s.ks.end_decode_step(sp)
+
+    frame(40)
+    assert s.ks.open_branches(nbranch) == nbranch
+    if mode == "graph":
+        assert s.ks.capture_decode_step(layers, sp)
+    want0, wantb = 40.0 * LQ, 0.0
+    for M in (20, 10, 33):
+        step()                                             # folds every row
+        want0, wantb = 0.5 * want0, 0.5 * wantb + LQ
+        frame(M)                                           # folds the stream's row; not ordered against the step by the caller
+        want0 = 0.5 * want0 + M * LQ
+    step()
+    want0, wantb = 0.5 * want0, 0.5 * wantb + LQ
+    torch.cuda.synchronize()
+    s.sc.sync_to_host()
+    got0 = sum(s.sc.score(lb) for lb in range(stride))
+    assert abs(got0 - want0) < 0.02 * want0, (got0, want0)
+    for b in (1, 2):
+        got = sum(s.sc.score(b * stride + lb) for lb in range(stride))
+        assert abs(got - wantb) < 0.02 * wantb, (b, got, wantb)
+    s.ks.close_branches()
+
+
 def test_time_division_perception_between_decode_steps_and_a_changing_branch_count(dev):
     """The scheduler's regime (scheduler.h:8-24, 53-56): perception goes on while branches think, and
     the number of branches follows the wakefulness state.  The stream writes into a block it still

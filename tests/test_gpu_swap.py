@@ -84,6 +84,33 @@ def test_swapper_file_image_swap_in_and_prefetch(dev, dtype, tmp_path):
         sw.shutdown()
 
 
+def test_swapper_calls_back_in_submission_order_and_refuses_work_after_shutdown(dev, tmp_path):
+    """Requests that have no device phase (a prefetch) or whose first phase fails (a swap-in of a missing file)
+    complete at once -- but not before the copies submitted ahead of them; after shutdown() a request fails
+    immediately and leaves nothing pending."""
+    L, KVH, QH, D, bs = 3, 4, 16, 128, 16
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.F16)
+    cm, sw = host.CacheManager(), host.KVSwapper()
+    og1 = orc.layout(L, KVH, QH, D, bs, 1, cabi.F16)
+    block_bytes = L * orc.lib().orc_block_stride_bytes(C.byref(og1))
+    assert cm.init_ssd(8 * block_bytes, tmp_path / "kv", bs, sw)
+    assert sw.init(cm, tmp_path / "kv", 3)
+    try:
+        d = tmp_path / "kv"
+        assert sw.swap_out(9, 0, d / "seed.kv")
+        reqs = [(0, 0, 0, d / "a.kv"), (0, 1, 1, d / "b.kv"), (1, 7, 2, d / "missing.kv"), (0, 2, 3, d / "c.kv"),
+                (1, 9, -1, d / "seed.kv"), (0, 3, 4, d / "d.kv"), (1, 8, -1, d / "missing2.kv")]
+        order, ok = sw.swap_many(reqs)
+        assert order == list(range(len(reqs)))
+        assert ok == [True, True, False, True, True, True, False]
+        assert sw.pending() == 0
+        sw.remove_writer_stream(U.stream_ptr())
+        assert sw.swap_out(4, 5, d / "e.kv")
+    finally:
+        sw.shutdown()
+    assert not sw.swap_out(5, 5, tmp_path / "kv" / "late.kv") and sw.pending() == 0
+
+
 def test_cache_manager_spills_to_the_overflow_tier_and_brings_blocks_back(dev, tmp_path):
     """A sequence twice the size of the pool: the oldest blocks go to <dir>/block_<i>.kv
     (cache_manager.cpp:132-141, 207-243), come back on demand into other physical blocks

@@ -53,3 +53,35 @@ def test_static_scratch_rejects_what_does_not_fit(dev):
                                                                B, mx, U.p(buf), 0, 0.1, cabi.BF16, U.stream_ptr())
     assert rc == cabi.ERR_WORKSPACE
     assert b"static scratch" in cabi.lib().drk_last_error()
+
+
+def test_static_scratch_decode_under_graph_capture(dev):
+    """What the entry point is for: a caller that may not allocate.  One warm call outside any capture (it looks
+    the scratch array's address up), then the call is recorded into a graph and replayed: every replay equals the
+    workspace call, with other launches that use the scratch array in between."""
+    import torch
+    geom = (2, 8, 32, 128, 16, 900)
+    case = Case(geom, cabi.BF16, [2000, 777, 64, 1301], seed=73)
+    other = Case(geom, cabi.BF16, [500, 3000], seed=74)
+    want = case.run_branches()
+    assert np.array_equal(_static(case), want)                 # the warm call
+    B = len(case.seq_lens)
+    QH, D = case.geom[2], case.geom[3]
+    out = U.dev_bytes(np.full(B * QH * D * 2, 0x7B, dtype=np.uint8))
+    side = torch.cuda.Stream()
+    sp = C.c_void_p(side.cuda_stream)
+    cabi.call("drk_graph_begin_capture", sp)
+    cabi.call("drk_paged_decode_attention_branches_static", C.byref(case.g), U.p(case.dq), U.p(case.dpool), U.p(case.dtab),
+              case.stride, U.p(case.dlens), B, int(case.seq_lens.max()), U.p(out), case.layer, float(case.scale), case.io, sp)
+    graph = C.c_void_p()
+    cabi.call("drk_graph_end_capture", sp, C.byref(graph))
+    try:
+        for replay in range(3):
+            out.fill_(0x7B)
+            torch.cuda.synchronize()
+            cabi.call("drk_graph_launch", graph, sp)
+            side.synchronize()
+            assert np.array_equal(U.host(out, np.uint16, (B, QH, D)), want), f"replay {replay}"
+            assert np.array_equal(_static(other), other.run_branches())     # eager work on the same scratch array
+    finally:
+        cabi.call("drk_graph_destroy", graph)
