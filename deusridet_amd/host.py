@@ -11,7 +11,9 @@ import numpy as np
 from . import cabi
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libdeusridet_memoria.so")
+# DRK_HOST_SAN=asan / tsan: the sanitizer build of deusridet_amd/host/Makefile (SAN=1 / SAN=thread), made beforehand
+_SAN = os.environ.get("DRK_HOST_SAN", "")
+LIB_PATH = os.path.join(_HERE, "lib", "libdeusridet_memoria%s.so" % ("_" + _SAN if _SAN in ("asan", "tsan") else ""))
 
 _vp, _i32, _sz, _f32 = C.c_void_p, C.c_int32, C.c_size_t, C.c_float
 _ip = C.POINTER(C.c_int32)

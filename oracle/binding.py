@@ -9,7 +9,9 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "liboracle.so")
+# DRK_ORACLE_SAN=asan / tsan: the sanitizer build of oracle/Makefile (SAN=1 / SAN=thread), made beforehand
+_SAN = os.environ.get("DRK_ORACLE_SAN", "")
+_SO = os.path.join(_HERE, "liboracle%s.so" % ("_" + _SAN if _SAN in ("asan", "tsan") else ""))
 
 F16, BF16, INT8, FP8 = 0, 1, 2, 3
 
@@ -20,7 +22,8 @@ class Layout(C.Structure):
 
 def build(force=False):
     if force or not os.path.exists(_SO):
-        subprocess.check_call(["make", "-B", "-C", _HERE, "liboracle.so"])
+        subprocess.check_call(["make", "-B", "-C", _HERE, os.path.basename(_SO)] +
+                              ({"asan": ["SAN=1"], "tsan": ["SAN=thread"]}.get(_SAN, [])))
     return _SO
 
 
