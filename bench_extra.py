@@ -257,10 +257,25 @@ def config3(args):
         for i, b in enumerate(forks):
             cm.set_seq_len(b, int(lens[i]) + 1)
 
+    per_tok = 2 * KVH * D * 2
+
+    def distinct_bytes(lens_now):
+        """bytes a launch must fetch: every physical page some branch reads, once, up to the last token read in it"""
+        held = {}
+        for b, n in zip(forks, lens_now):
+            tab = cm.h_block_table(b)
+            for k in range((int(n) + bs - 1) // bs):
+                if tab[k] >= 0:
+                    held[int(tab[k])] = max(held.get(int(tab[k]), 0), min(bs, int(n) - k * bs))
+        return sum(held.values()) * per_tok
+
     lens = lens0.copy()
     for s in range(W):
         step(s, lens); lens += 1
     torch.cuda.synchronize()
+    # the launch as the warm-up left it: every page resident (the timed steps evict)
+    full_ms = _timed_decode(lib, cabi, lambda i: attend(i % L, cabi.p(dlen)), 60)
+    full_bytes = distinct_bytes(lens)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     logical = 0
@@ -270,20 +285,12 @@ def config3(args):
     e1.record(stream)
     torch.cuda.synchronize()
     total_ms = e0.elapsed_time(e1)
-    per_tok = 2 * KVH * D * 2
     unique_tokens = cm.gpu_blocks_used() * bs
     value = logical * per_tok * L / (total_ms * 1e-3) / 1e9
     dl = cabi.p(dlen)
     ker_ms = _timed_decode(lib, cabi, lambda i: attend(i % L, dl), 60)
     launch_logical = int(lens.sum()) * per_tok
-    # bytes the launch must fetch: every physical page some branch reads, once, up to the last token read in it
-    held = {}
-    for b, n in zip(forks, lens):
-        tab = cm.h_block_table(b)
-        for k in range((int(n) + bs - 1) // bs):
-            if tab[k] >= 0:
-                held[int(tab[k])] = max(held.get(int(tab[k]), 0), min(bs, int(n) - k * bs))
-    launch_unique = sum(held.values()) * per_tok
+    launch_unique = distinct_bytes(lens)
     # what the launch streams once: the ranges it was given as groups, and every branch's remainder
     in_groups = sum((e - b0) // 64 * 64 * (nb - 1) for _, nb, b0, e in groups_now[0]) if grouped else shared_now[0] // 64 * 64 * (B - 1)
     launch_streamed = launch_logical - in_groups * per_tok
@@ -314,6 +321,11 @@ def config3(args):
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
                      "avg_launch_us": round(ker_ms * 1e3, 2), "bytes_per_launch": launch_unique,
                      "streamed_bytes_per_launch": launch_streamed,
+                     "all_pages_resident": {"avg_launch_us": round(full_ms * 1e3, 2), "bytes_per_launch": full_bytes,
+                                            "frac": round(full_bytes / (full_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                                            "what": "the same launch after the warm-up steps, before the timed steps evicted "
+                                                    "%d blocks (an evicted page is a hole the kernel skips: its tile still "
+                                                    "takes a turn, its bytes are not counted)" % evicted},
                      "note": "DISTINCT bytes: every physical page some branch reads, counted once.  streamed_bytes is what "
                              "the launch reads given the shared ranges it was handed (ranges under 256 tokens and what "
                              "rounding to 64-token tiles cuts off are read once per branch).  The merge is not in "
