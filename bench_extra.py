@@ -956,6 +956,63 @@ def kernel_fractions(buf, seed=11):
         torch.cuda.synchronize()
         lib.drk_debug_set_prefill_two_phase(1)
         by_wgs[str(m // 64 * KVH)] = round(a0.elapsed_time(a1) / 4 * 1e3 / ((pos + m + 63) // 64), 3)
+    # ---- the attention mass of a perception frame: the last chunk (2 048 rows at 30 720) with and without it ----
+    q = torch.randn(chunk, QH, D, device="cuda").to(torch.bfloat16)
+    o = torch.empty_like(q)
+    lse = torch.empty(chunk * QH, dtype=torch.float32, device="cuda")
+    mass = torch.zeros(total // bs, dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    ssp = C.c_void_p(side.cuda_stream)
+    pos = total - chunk
+    ev_a, ev_m = C.c_void_p(), C.c_void_p()
+    cabi.call("drk_event_create", C.byref(ev_a))
+    cabi.call("drk_event_create", C.byref(ev_m))
+
+    def attn_plain():
+        cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, pos, chunk, scale,
+                  cabi.BF16, None, 0, sp)
+
+    def attn_two_walks():
+        attn_plain()
+        cabi.call("drk_paged_prefill_attention_mass", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), 0, pos, chunk, scale, cabi.BF16,
+                  cabi.p(mass), total // bs, 1, sp)
+
+    def attn_lse(mass_stream):
+        if mass_stream is not sp:
+            cabi.call("drk_stream_wait_event", sp, ev_m)                           # the pass before still reads q
+        cabi.call("drk_paged_prefill_attention_lse", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, pos, chunk, scale,
+                  cabi.BF16, None, 0, cabi.p(lse), None, 0, sp)
+        if mass_stream is not sp:
+            cabi.call("drk_event_record", ev_a, sp)
+            cabi.call("drk_stream_wait_event", mass_stream, ev_a)
+        cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), 0, pos, chunk, scale,
+                  cabi.BF16, cabi.p(lse), cabi.p(mass), total // bs, 1, mass_stream)
+        if mass_stream is not sp:
+            cabi.call("drk_event_record", ev_m, mass_stream)
+
+    def timed(fn, n=6):
+        cabi.call("drk_event_record", ev_m, ssp)
+        fn(); fn()
+        torch.cuda.synchronize()
+        a0, a1 = ev(), ev()
+        a0.record(stream)
+        for _ in range(n):
+            fn()
+        cabi.call("drk_stream_wait_event", sp, ev_m)
+        a1.record(stream)
+        torch.cuda.synchronize()
+        return round(a0.elapsed_time(a1) / n * 1e3, 1)
+
+    frame_mass = {"attention_us": timed(attn_plain), "with_two_walk_mass_us": timed(attn_two_walks),
+                  "with_one_walk_mass_same_stream_us": timed(lambda: attn_lse(sp)),
+                  "with_one_walk_mass_second_stream_us": timed(lambda: attn_lse(ssp)),
+                  "what": "config 5's last chunk (2048 rows behind 30720 tokens, 32 Q / 8 KV x 128 bf16), per layer: the chunk's "
+                          "attention alone; followed by the mass pass that walks the keys twice; by the pass that takes the rows' "
+                          "log-sum-exps from the attention call and walks once; and with that pass on a second stream behind an "
+                          "event, back to back launches (the next attention call waits for the pass, which reads its Q)"}
+    cabi.call("drk_event_destroy", ev_a)
+    cabi.call("drk_event_destroy", ev_m)
+    res["frame_mass"] = frame_mass
     prefill_entry("config5_prefill", "prefill_ppd_kernel<bf16>", per_chunk,
                   "config 5: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV x 128 bf16",
                   {"us_per_tile_by_workgroups_at_30720": by_wgs})

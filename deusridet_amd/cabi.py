@@ -151,6 +151,10 @@ SIGNATURES = {
     "drk_paged_decode_attention_mass": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _f32, _i32, _vp,
                                                _i32, _i32, _vp, _sz, _vp]),
     "drk_paged_prefill_attention_mass": (_i32, [_LP, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _i32, _i32, _vp]),
+    "drk_paged_prefill_attention_lse": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp, _vp, _sz,
+                                               _vp]),
+    "drk_paged_prefill_attention_mass_lse": (_i32, [_LP, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _i32, _i32,
+                                                    _vp]),
     "drk_importance_update": (_i32, [_vp, _vp, _i32, _f32, _vp]),
     "drk_importance_fold_clear": (_i32, [_vp, _vp, _i32, _f32, _vp]),
 }

@@ -41,6 +41,25 @@ bool KvStream::init(CacheManager& cm, int max_context_len, ImportanceScorer* sco
         return false;
     }
     d_len_ = static_cast<int*>(p);
+    if (scorer && scorer->d_new_scores()) {
+        // perception frames: two sets of row log-sum-exps (the attention call of one layer may run while the mass
+        // pass of the layer before still reads its set) and the two events that order the passes
+        // and the frame's masses, one per table entry of the stream's row (zero between frames)
+        const size_t lse_floats = 2 * (size_t)max_prefill_rows * ModelConfig::NUM_ATTN_HEADS;
+        const size_t mass_floats = (size_t)cm.table_stride();
+        p = nullptr;
+        if (drk_dev_malloc(&p, (lse_floats + mass_floats) * sizeof(float)) != DRK_OK || drk_event_create(&ev_attn_) != DRK_OK ||
+            drk_event_create(&ev_mass_) != DRK_OK ||
+            drk_dev_memset_async(static_cast<float*>(p) + lse_floats, 0, mass_floats * sizeof(float), nullptr) != DRK_OK ||
+            drk_stream_synchronize(nullptr) != DRK_OK) {
+            LOG_ERROR("Conscientia", "KvStream: buffers of the mass pass: %s", drk_last_error());
+            d_row_lse_ = static_cast<float*>(p);
+            destroy();
+            return false;
+        }
+        d_row_lse_ = static_cast<float*>(p);
+        d_frame_mass_ = d_row_lse_ + lse_floats;
+    }
     // every attention call below finds its split-K workspace ready: nothing allocates later
     const int bs = cm.block_pool().block_size();
     if (!ws_decode_.reserve_for(cm.max_branches(), max_context_len, 0, bs) ||
@@ -61,6 +80,15 @@ void KvStream::destroy()
     if (cm_) close_branches();
     if (d_pos_) drk_dev_free(d_pos_);
     if (d_len_) drk_dev_free(d_len_);
+    if (d_row_lse_ || ev_attn_ || ev_mass_) {
+        drk_device_synchronize();                 // a mass pass may still be reading
+        if (d_row_lse_) drk_dev_free(d_row_lse_);
+        if (ev_attn_) drk_event_destroy(ev_attn_);
+        if (ev_mass_) drk_event_destroy(ev_mass_);
+        d_row_lse_ = d_frame_mass_ = nullptr;
+        ev_attn_ = ev_mass_ = nullptr;
+        mass_pending_ = false;
+    }
     if (ws_decode_.ptr() || ws_prefill_.ptr()) {
         drk_device_synchronize();                 // launches that use the partials may still be running
         ws_decode_.release();
@@ -101,35 +129,55 @@ void KvStream::prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipSt
 {
     const BlockPool& pool = cm_->block_pool();
     const int hd = ModelConfig::HEAD_DIM;
+    const float scale = 1.0f / std::sqrt((float)hd);
+    const bool scored = scorer_ && scorer_->d_new_scores() && d_row_lse_;
+    // the mass pass of the layer before reads q_scratch on the scorer's stream: this layer's first launch rewrites it
+    if (scored && mass_pending_ && drk_stream_wait_event(stream, ev_mass_) != DRK_OK)
+        LOG_ERROR("Conscientia", "KvStream: waiting for the mass pass: %s", drk_last_error());
     // steps 4-9 of full_attention_forward_paged_prefill (paged_attention.cu:589-634) in two launches
     paged_qk_norm_rope_write_batch(io.qg, io.k, io.v, io.q_norm, io.k_norm, io.q_scratch, pool.pool_ptr(),
                                    cm_->d_block_table(0), fa_layer_idx, current_pos_, M, pool.max_blocks(),
                                    pool.block_size(), d_rope_table_, table_positions_, stream);
-    paged_prefill_attention_gated(ws_prefill_, io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), io.qg + hd, 2 * hd, io.attn_out,
-                                  fa_layer_idx, current_pos_, M, pool.max_blocks(), pool.block_size(),
-                                  1.0f / std::sqrt((float)hd), stream);
-    // what the frame's rows looked at, block by block, into the stream's own row of the scorer's new scores
-    // ("after each Prefill frame, record cumulative attention weight received by each KV block",
-    // docs/en/architecture/02-memoria.md:40-44): a pass over Q and K behind the layer's attention
-    if (scorer_ && scorer_->d_new_scores()) {
-        const bool first = first_layer_of_frame_ < 0;
-        if (first) first_layer_of_frame_ = fa_layer_idx;
-        frame_stream_ = stream;
-        paged_prefill_attention_mass(io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), fa_layer_idx, current_pos_, M,
-                                     pool.max_blocks(), pool.block_size(), 1.0f / std::sqrt((float)hd),
-                                     scorer_->d_new_scores(), cm_->table_stride(), !first, stream);
+    if (!scored) {
+        paged_prefill_attention_gated(ws_prefill_, io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), io.qg + hd, 2 * hd, io.attn_out,
+                                      fa_layer_idx, current_pos_, M, pool.max_blocks(), pool.block_size(), scale, stream);
+        return;
     }
+    // What the frame's rows looked at, block by block, into a buffer of the stream's own
+    // ("after each Prefill frame, record cumulative attention weight received by each KV block",
+    // docs/en/architecture/02-memoria.md:40-44).  The attention call leaves every row's log-sum-exp; the mass pass
+    // -- Q and K once more, no V -- runs on the scorer's stream behind an event, beside whatever the caller puts on
+    // `stream` next (the layer's output projection and MLP).
+    float* lse = d_row_lse_ + (size_t)(lse_turn_ & 1) * max_prefill_rows_ * ModelConfig::NUM_ATTN_HEADS;
+    lse_turn_++;
+    paged_prefill_attention_gated(ws_prefill_, io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), io.qg + hd, 2 * hd, io.attn_out,
+                                  lse, fa_layer_idx, current_pos_, M, pool.max_blocks(), pool.block_size(), scale, stream);
+    const bool first = first_layer_of_frame_ < 0;
+    if (first) first_layer_of_frame_ = fa_layer_idx;
+    frame_stream_ = stream;
+    hipStream_t ms = scorer_->stream();
+    if (drk_event_record(ev_attn_, stream) != DRK_OK || drk_stream_wait_event(ms, ev_attn_) != DRK_OK) {
+        LOG_ERROR("Conscientia", "KvStream: ordering the mass pass: %s", drk_last_error());
+        ms = stream;                                    // in line, then
+    }
+    paged_prefill_attention_mass(io.q_scratch, pool.pool_ptr(), cm_->d_block_table(0), fa_layer_idx, current_pos_, M,
+                                 pool.max_blocks(), pool.block_size(), scale, lse, d_frame_mass_, cm_->table_stride(), !first, ms);
+    mass_stream_ = ms;
+    mass_pending_ = drk_event_record(ev_mass_, ms) == DRK_OK;
 }
 
 void KvStream::end_prefill(int M, hipStream_t stream)
 {
     if (scorer_ && first_layer_of_frame_ >= 0) {
-        // Fold the frame's masses into the scores of the stream's own row, and clear them in the same pass (or
-        // every later fold would count the frame again).  Only that row: the rows of open decode branches still
-        // hold their last step's masses, which that step has folded in already.  The fold goes behind the mass
-        // passes, on the stream they ran on, whatever the caller passes (or leaves out) here.
+        // Fold the frame's masses into the scores of the stream's own row, and clear them in the same pass.  Only
+        // that row: the rows of open decode branches still hold their last step's masses, which that step has
+        // folded in already.  The fold goes behind the mass passes, on the stream they ran on, whatever the caller
+        // passes (or leaves out) here; the caller's stream waits for the last pass, which still reads q_scratch.
         (void)stream;
-        scorer_->apply_new_scores(0, cm_->table_stride(), frame_stream_);
+        scorer_->fold_masses(0, cm_->table_stride(), d_frame_mass_, mass_stream_);
+        if (mass_pending_ && mass_stream_ != frame_stream_ && drk_stream_wait_event(frame_stream_, ev_mass_) != DRK_OK)
+            LOG_ERROR("Conscientia", "KvStream: waiting for the mass pass: %s", drk_last_error());
+        mass_pending_ = false;
         first_layer_of_frame_ = -1;
     }
     current_pos_ += M;                                                    // stream.cpp:238-239

@@ -62,9 +62,11 @@ public:
     // pages they forked from, the stream copies a block it still shares before it writes into it.
     bool begin_prefill(int M, hipStream_t stream);
     void prefill_layer(int fa_layer_idx, const KvLayerIO& io, int M, hipStream_t stream);
-    // With a scorer attached the frame's attention masses are folded into the scores of the stream's own row here
-    // (and cleared), on the stream the frame's prefill_layer calls ran on -- not on `stream`, which only keeps the
-    // reference's call shape: a fold on another stream could overtake the mass passes.
+    // With a scorer attached every layer's attention call also leaves its rows' log-sum-exps, and a pass over Q and
+    // K on the scorer's stream (behind an event) turns them into the attention mass every block received; the next
+    // layer's first launch waits for that pass, which reads q_scratch.  end_prefill folds the frame's masses into the
+    // scores of the stream's own row (and clears them) on the scorer's stream, behind the passes, and makes the
+    // layers' stream wait for the last pass; `stream` only keeps the reference's call shape.
     void end_prefill(int M, hipStream_t stream = nullptr);
     int  current_pos() const { return current_pos_; }
 
@@ -127,7 +129,14 @@ private:
     int max_prefill_rows_ = 0;
     int first_layer_of_step_ = -1;   // the layer whose scored call overwrites instead of accumulating
     int first_layer_of_frame_ = -1;  // the same for the mass pass of a perception frame
-    hipStream_t frame_stream_ = nullptr;   // stream of the frame's mass passes
+    hipStream_t frame_stream_ = nullptr;   // stream of the frame's layers
+    hipStream_t mass_stream_ = nullptr;    // stream of the frame's mass passes (the scorer's)
+    float* d_row_lse_ = nullptr;           // [2][max_prefill_rows][num_q_heads]: the rows' log-sum-exps, by turns
+    float* d_frame_mass_ = nullptr;        // [table_stride]: the masses of the frame under way (same allocation)
+    unsigned lse_turn_ = 0;
+    void* ev_attn_ = nullptr;              // a layer's attention call has been issued (recorded on the caller's stream)
+    void* ev_mass_ = nullptr;              // its mass pass has been issued (recorded on the scorer's stream)
+    bool mass_pending_ = false;
 
     bool host_begin(hipStream_t stream);
     void host_end();

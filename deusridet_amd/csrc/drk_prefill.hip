@@ -185,6 +185,9 @@ struct PrefillArgs {
     // optional epilogue: out *= sigmoid(gate), gate rows gate_stride elements apart
     const uint16_t *gate;
     size_t gate_stride;
+    // optional: the row's log2-sum-exp of its scaled scores, [M][QH] (+inf for a row that saw no token).  Written
+    // by the chunk kernels where a row's walk ends; read by the mass kernel, which then walks the keys once.
+    float *lse_rows;
 };
 
 // scheduling hints: order instruction groups inside one basic block
@@ -557,6 +560,8 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mfma_kernel(Pre
 
     // ---- register i of tile dt is d = dt*32 + 8*(i/4) + 4*g + i%4 ----
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (!SHARED && A.lse_rows && row_live && g == 0)
+        A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_run + __builtin_log2f(l_tot) : INFINITY;
     if (SHARED) {
         if (row_live) {                      // unnormalised partial; an empty range leaves (0, -inf, 0)
             const size_t pi = ((size_t)tq * A.QH + head) * A.nsplits + blockIdx.z;
@@ -940,6 +945,8 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (A.lse_rows && row_live && g == 0)      // m_ref is the reference the weights were taken against, in log2 units
+        A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_ref + __builtin_log2f(l_tot) : INFINITY;
     if (row_live && (l_tot > 0.0f || A.gate)) {
         const bool have = l_tot > 0.0f;
         const float inv = have ? 1.0f / l_tot : 0.0f;
@@ -1353,6 +1360,8 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (A.lse_rows && row_live && g == 0)      // m_ref is the reference the weights were taken against, in log2 units
+        A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_ref + __builtin_log2f(l_tot) : INFINITY;
     if (row_live && (l_tot > 0.0f || A.gate)) {
         const bool have = l_tot > 0.0f;
         const float inv = have ? 1.0f / l_tot : 0.0f;
@@ -1667,6 +1676,8 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (A.lse_rows && row_live && g == 0)      // m_ref is the reference the weights were taken against, in log2 units
+        A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_ref + __builtin_log2f(l_tot) : INFINITY;
     if (row_live && (l_tot > 0.0f || A.gate)) {
         const bool have = l_tot > 0.0f;
         const float inv = have ? 1.0f / l_tot : 0.0f;
@@ -1871,17 +1882,27 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
             __syncthreads();
         }
     };
-    walk(std::false_type{});
-    // a row's lanes (the 32 of its half of the wave) meet: lse = M + log2(sum l 2^(m - M)); +inf for a row that saw nothing
+    if (A.lse_rows) {
+        // the chunk's attention kernel left every row's log-sum-exp: one walk
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        float mm = m[i];
+        for (int i = 0; i < 16; i++) {
+            const int r = w * 32 + 8 * (i >> 2) + 4 * g + (i & 3), rt = r / G;
+            const int tq = qt * TPW + rt;
+            lse[i] = vis[i] > 0 ? A.lse_rows[(size_t)tq * A.QH + kvh * G + (r - rt * G)] : INFINITY;
+        }
+    } else {
+        walk(std::false_type{});
+        // a row's lanes (the 32 of its half of the wave) meet: lse = M + log2(sum l 2^(m - M)); +inf for a row that saw nothing
 #pragma unroll
-        for (int off = 1; off < 32; off <<= 1) mm = fmaxf(mm, __shfl_xor(mm, off));
-        float ll = l[i] * __builtin_amdgcn_exp2f(m[i] - mm);
+        for (int i = 0; i < 16; i++) {
+            float mm = m[i];
 #pragma unroll
-        for (int off = 1; off < 32; off <<= 1) ll += __shfl_xor(ll, off);
-        lse[i] = ll > 0.0f ? mm + __builtin_log2f(ll) : INFINITY;
+            for (int off = 1; off < 32; off <<= 1) mm = fmaxf(mm, __shfl_xor(mm, off));
+            float ll = l[i] * __builtin_amdgcn_exp2f(m[i] - mm);
+#pragma unroll
+            for (int off = 1; off < 32; off <<= 1) ll += __shfl_xor(ll, off);
+            lse[i] = ll > 0.0f ? mm + __builtin_log2f(ll) : INFINITY;
+        }
     }
     walk(std::true_type{});
 }
@@ -2252,6 +2273,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
     else shared_prefix_shape(a, B, shared, &A.chunk_tiles, &A.nsplits);
     A.part_o = part_o; A.part_m = part_m; A.part_l = part_l;
     A.gate = nullptr; A.gate_stride = 0;
+    A.lse_rows = nullptr;
     if (nsplits <= 0 && prefix_stream_applies(a, B)) {
         A.tpw = 64 / (a.QH / a.KVH);
         dim3 grid2(((B + A.tpw - 1) / A.tpw) * a.KVH, 1, A.nsplits);
@@ -2312,7 +2334,7 @@ template <int D>
 __global__ __launch_bounds__(64) void prefill_merge_kernel(const float *__restrict__ part_o, const float *__restrict__ part_m,
                                                            const float *__restrict__ part_l, uint16_t *__restrict__ out,
                                                            int nsplits, int io_dtype, const uint16_t *__restrict__ gate,
-                                                           size_t gate_stride)
+                                                           size_t gate_stride, float *__restrict__ lse_rows)
 {
     constexpr int VEC = D / 64;
     typedef float fvec __attribute__((ext_vector_type(VEC)));
@@ -2336,6 +2358,7 @@ __global__ __launch_bounds__(64) void prefill_merge_kernel(const float *__restri
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off);
+    if (lse_rows && lane == 0) lse_rows[row] = L > 0.0f ? M + __builtin_log2f(L) : INFINITY;
     fvec acc = {};
     const float *obase = part_o + row * nsplits * D + d;
     for (int j = 0; j < nsplits; j += 8) {
@@ -2412,7 +2435,7 @@ static size_t prefill_split_need(const Lay &a, int pos_start, int M)
 
 static int prefill_split(const Lay &a, const void *q, const void *pool, const int32_t *table, void *out, int layer,
                          int pos_start, int M, float scale, int io_dtype, void *workspace, hipStream_t st,
-                         const void *gate, size_t gate_stride)
+                         const void *gate, size_t gate_stride, float *lse_rows)
 {
     int ct, ns;
     prefill_split_shape(a, pos_start, M, &ct, &ns);
@@ -2425,10 +2448,10 @@ static int prefill_split(const Lay &a, const void *q, const void *pool, const in
     const dim3 grid((unsigned)((size_t)M * a.QH));
     if (a.D == 128)
         hipLaunchKernelGGL(prefill_merge_kernel<128>, grid, dim3(64), 0, st, part_o, part_m, part_l, (uint16_t *)out, ns, io_dtype,
-                           (const uint16_t *)gate, gate_stride);
+                           (const uint16_t *)gate, gate_stride, lse_rows);
     else
         hipLaunchKernelGGL(prefill_merge_kernel<256>, grid, dim3(64), 0, st, part_o, part_m, part_l, (uint16_t *)out, ns, io_dtype,
-                           (const uint16_t *)gate, gate_stride);
+                           (const uint16_t *)gate, gate_stride, lse_rows);
     DRK_LAUNCH_CHECK("prefill_merge_kernel");
     return DRK_OK;
 }
@@ -2440,9 +2463,9 @@ using namespace drk;
 extern "C" {
 
 void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
-int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
-                                     int layer, int pos_start, int M, float scale, int io_dtype, float *d_block_mass,
-                                     int mass_len, int accumulate, void *stream)
+static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
+                             int layer, int pos_start, int M, float scale, int io_dtype, const float *d_row_lse,
+                             float *d_block_mass, int mass_len, int accumulate, void *stream)
 {
     Lay a;
     int rc = make_lay(g, &a);
@@ -2477,6 +2500,7 @@ int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, cons
     A.scale_log2e = scale * kLog2eP;
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = nullptr; A.gate_stride = 0;
+    A.lse_rows = const_cast<float *>(d_row_lse);             // read only here: the rows' log-sum-exps, or NULL (first walk finds them)
     dim3 grid(((M + A.tpw - 1) / A.tpw) * a.KVH);
 #define DRK_PM(DT, KV, IO)                                                                                                      \
     do {                                                                                                                       \
@@ -2492,6 +2516,24 @@ int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, cons
 #undef DRK_PM
     DRK_LAUNCH_CHECK("prefill_mass_kernel");
     return DRK_OK;
+}
+
+int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
+                                     int layer, int pos_start, int M, float scale, int io_dtype, float *d_block_mass,
+                                     int mass_len, int accumulate, void *stream)
+{
+    return prefill_mass_impl(g, q, pool, d_block_table, layer, pos_start, M, scale, io_dtype, nullptr, d_block_mass, mass_len,
+                             accumulate, stream);
+}
+
+int drk_paged_prefill_attention_mass_lse(const drk_kv_layout *g, const void *q, const void *pool,
+                                         const int32_t *d_block_table, int layer, int pos_start, int M, float scale,
+                                         int io_dtype, const float *d_row_lse, float *d_block_mass, int mass_len,
+                                         int accumulate, void *stream)
+{
+    if (!d_row_lse) return fail(DRK_ERR_INVALID, "prefill_mass: d_row_lse is NULL");
+    return prefill_mass_impl(g, q, pool, d_block_table, layer, pos_start, M, scale, io_dtype, d_row_lse, d_block_mass, mass_len,
+                             accumulate, stream);
 }
 
 void drk_debug_set_prefill_two_phase(int mode) { g_prefill_two_phase = mode < 0 ? 1 : (mode > 3 ? 3 : mode); }
@@ -2533,7 +2575,7 @@ size_t drk_prefill_workspace_bytes_max(const drk_kv_layout *g, int max_seq_len, 
 // verbatim (paged_attention.cu:481, 506-549) -- and needs the workspace.
 static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
                         void *out, int layer, int pos_start, int M, float scale, int io_dtype, void *workspace,
-                        size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
+                        size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride, float *lse_rows = nullptr)
 {
     Lay a;
     int rc = make_lay(g, &a);
@@ -2551,6 +2593,8 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
 
     const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 &&
                       a.QH / a.KVH <= 128 && (a.bs % 16) == 0;
+    if (!mfma && lse_rows)
+        return fail(DRK_ERR_UNSUPPORTED, "prefill: row log-sum-exps need head_dim 128 or 256 and block_size %% 16 == 0");
     if (!mfma)
         return launch_decode(g, q, pool, d_block_table, 0, nullptr, 0, pos_start, M, pos_start + M, out, layer, scale,
                              io_dtype, 0, workspace, workspace_bytes, stream, gate, gate_stride);
@@ -2562,7 +2606,7 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     if (prefill_split_applies(a, pos_start, M) && workspace && ((uintptr_t)workspace % 16) == 0 &&
         workspace_bytes >= prefill_split_need(a, pos_start, M))
         return prefill_split(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
-                             (hipStream_t)stream, gate, gate_stride);
+                             (hipStream_t)stream, gate, gate_stride, lse_rows);
     PrefillArgs A;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
     A.table = d_block_table;
@@ -2576,6 +2620,7 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     dim3 grid(((M + A.tpw - 1) / A.tpw) * a.KVH);
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = (const uint16_t *)gate; A.gate_stride = gate_stride;
+    A.lse_rows = lse_rows;
     hipStream_t st = (hipStream_t)stream;
     // Long chunks of head_dim 128 take the two-phase kernel (256 rows per workgroup, one workgroup per CU)
     // when that still gives at least three quarters of the CUs a workgroup.  That kernel takes its pages
@@ -2647,6 +2692,17 @@ int drk_paged_prefill_attention_gated(const drk_kv_layout *g, const void *q, con
     if (!gate) return fail(DRK_ERR_INVALID, "prefill: gate is NULL");
     return prefill_impl(g, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
                         workspace_bytes, stream, gate, gate_stride);
+}
+
+// the same call (gate may be NULL) that also leaves every row's log2-sum-exp, for the single-walk mass pass
+int drk_paged_prefill_attention_lse(const drk_kv_layout *g, const void *q, const void *pool,
+                                    const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
+                                    float scale, int io_dtype, const void *gate, size_t gate_stride, float *d_row_lse,
+                                    void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!d_row_lse) return fail(DRK_ERR_INVALID, "prefill: d_row_lse is NULL");
+    return prefill_impl(g, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
+                        workspace_bytes, stream, gate, gate_stride, d_row_lse);
 }
 
 } // extern "C"

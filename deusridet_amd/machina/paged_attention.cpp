@@ -391,6 +391,31 @@ void paged_prefill_attention_mass(const __half* Q, const __half* kv_pool, const 
         LOG_ERROR("Machina", "paged_prefill_attention_mass: %s", drk_last_error());
 }
 
+void paged_prefill_attention_mass(const __half* Q, const __half* kv_pool, const int* d_block_table, int fa_layer_idx,
+                                  int pos_start, int M, int max_phys_blocks, int block_size, float scale,
+                                  const float* d_row_lse, float* d_block_mass, int mass_len, bool accumulate,
+                                  hipStream_t stream)
+{
+    if (M <= 0 && accumulate) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    if (drk_paged_prefill_attention_mass_lse(&g, Q, kv_pool, d_block_table, fa_layer_idx, pos_start, M, scale,
+                                             ModelConfig::IO_DTYPE, d_row_lse, d_block_mass, mass_len, accumulate ? 1 : 0,
+                                             stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_prefill_attention_mass: %s", drk_last_error());
+}
+
+void paged_prefill_attention_gated(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
+                                   const __half* gate, int gate_stride, __half* out, float* d_row_lse, int fa_layer_idx,
+                                   int pos_start, int M, int max_phys_blocks, int block_size, float scale, hipStream_t stream)
+{
+    if (M <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    if (drk_paged_prefill_attention_lse(&g, Q, kv_pool, d_block_table, out, fa_layer_idx, pos_start, M, scale,
+                                        ModelConfig::IO_DTYPE, gate, (size_t)gate_stride, d_row_lse, ws.ptr(), ws.bytes(),
+                                        stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_prefill_attention_gated: %s", drk_last_error());
+}
+
 void paged_prefill_attention_gated(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
                                    const __half* gate, int gate_stride, __half* out, int fa_layer_idx, int pos_start,
                                    int M, int max_phys_blocks, int block_size, float scale, hipStream_t stream)

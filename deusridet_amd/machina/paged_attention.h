@@ -162,6 +162,13 @@ void paged_gqa_decode_attention_branches_scored(const __half* Q, __half* kv_pool
 void paged_prefill_attention_mass(const __half* Q, const __half* kv_pool, const int* d_block_table, int fa_layer_idx,
                                   int pos_start, int M, int max_phys_blocks, int block_size, float scale,
                                   float* d_block_mass, int mass_len, bool accumulate, hipStream_t stream = 0);
+// The same measurement without the second walk over the keys: the gated attention call below leaves every row's
+// log-sum-exp in d_row_lse [M * num_q_heads], this pass reads it.  The pass may run on another stream behind an
+// event recorded after the attention call: it reads Q, the pages and d_row_lse only.
+void paged_prefill_attention_mass(const __half* Q, const __half* kv_pool, const int* d_block_table, int fa_layer_idx,
+                                  int pos_start, int M, int max_phys_blocks, int block_size, float scale,
+                                  const float* d_row_lse, float* d_block_mass, int mass_len, bool accumulate,
+                                  hipStream_t stream = 0);
 
 // ---- the same attention calls on a workspace of the caller's ---------------------
 void paged_gqa_decode_attention(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
@@ -192,6 +199,10 @@ void paged_gqa_decode_attention_gated_branches(AttentionWorkspace& ws, const __h
 void paged_prefill_attention_gated(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
                                    const __half* gate, int gate_stride, __half* out, int fa_layer_idx, int pos_start,
                                    int M, int max_phys_blocks, int block_size, float scale, hipStream_t stream = 0);
+void paged_prefill_attention_gated(AttentionWorkspace& ws, const __half* Q, __half* kv_pool, const int* d_block_table,
+                                   const __half* gate, int gate_stride, __half* out, float* d_row_lse, int fa_layer_idx,
+                                   int pos_start, int M, int max_phys_blocks, int block_size, float scale,
+                                   hipStream_t stream = 0);
 void paged_gqa_decode_attention_branches_scored(AttentionWorkspace& ws, const __half* Q, __half* kv_pool,
                                                 const int* d_tables, int table_stride, const int* d_seq_lens, int B,
                                                 int max_seq_len, __half* out, int fa_layer_idx, int max_phys_blocks,

@@ -109,12 +109,18 @@ void ImportanceScorer::apply_new_scores(hipStream_t stream)
 
 void ImportanceScorer::apply_new_scores(int first, int count, hipStream_t stream)
 {
-    if (!d_scores_ || !d_new_ || first < 0 || count <= 0 || first >= max_blocks_) return;
+    if (!d_new_ || first < 0 || first >= max_blocks_) return;
+    fold_masses(first, count, d_new_ + first, stream);
+}
+
+void ImportanceScorer::fold_masses(int first, int count, float* d_masses, hipStream_t stream)
+{
+    if (!d_scores_ || !d_masses || first < 0 || count <= 0 || first >= max_blocks_) return;
     if (count > max_blocks_ - first) count = max_blocks_ - first;
     const bool captured = stream_is_capturing(stream);
     if (!captured) wait_for_last_fold(stream);
-    if (drk_importance_fold_clear(d_scores_ + first, d_new_ + first, count, decay_, stream) != DRK_OK)
-        LOG_ERROR("Memoria", "ImportanceScorer: apply_new_scores(range): %s", drk_last_error());
+    if (drk_importance_fold_clear(d_scores_ + first, d_masses, count, decay_, stream) != DRK_OK)
+        LOG_ERROR("Memoria", "ImportanceScorer: fold_masses: %s", drk_last_error());
     if (!captured) note_fold_on(stream);
 }
 

@@ -39,6 +39,10 @@ public:
     // perception frame does with the stream's own row while the rows of open decode branches keep the
     // masses of their last step (those were folded in by that step and must not be counted again).
     void apply_new_scores(int first, int count, hipStream_t stream);
+    // The same for masses that live in a buffer of the caller's (count floats, cleared by the fold): a perception
+    // frame gathers its masses there, so that a decode step's fold over the whole array, issued while the frame is
+    // under way, neither reads half a frame nor counts it twice.
+    void fold_masses(int first, int count, float* d_masses, hipStream_t stream);
     // Folds read and write the scores, so two of them must not run at once.  Each fold waits for the one
     // before it when that ran on another stream, and marks its own end for the next.  A fold recorded into a
     // graph cannot do either (the capture may not wait on work outside it): whoever replays such a graph calls

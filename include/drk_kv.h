@@ -390,6 +390,22 @@ int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, cons
                                      const int32_t *d_block_table, int layer, int pos_start, int M,
                                      float scale, int io_dtype, float *d_block_mass, int mass_len,
                                      int accumulate, void *stream);
+/* The two halves of the same measurement without the second walk over the keys (no reference counterpart).
+ * drk_paged_prefill_attention_lse is drk_paged_prefill_attention_gated (gate may be NULL here) that also writes
+ * every row's log2-sum-exp of its scaled scores to d_row_lse[M * num_q_heads] (+inf for a row without a visible
+ * token) -- the chunk kernels know it where a row's walk ends.  drk_paged_prefill_attention_mass_lse is the mass
+ * pass given those values: it reads K once.  It may run on another stream behind an event (it reads q, the pages
+ * and d_row_lse; nothing the attention call wrote except d_row_lse).  Head_dim 128 or 256, block_size % 16 == 0;
+ * DRK_ERR_UNSUPPORTED otherwise.  The two calls round Q differently for some chunk lengths (the long-chunk kernels
+ * fold the scale into Q in its 16-bit type): a row's masses then sum to 1 within 2e-3 instead of 1e-6. */
+int drk_paged_prefill_attention_lse(const drk_kv_layout *g, const void *q, const void *pool,
+                                    const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
+                                    float scale, int io_dtype, const void *gate, size_t gate_stride,
+                                    float *d_row_lse, void *workspace, size_t workspace_bytes, void *stream);
+int drk_paged_prefill_attention_mass_lse(const drk_kv_layout *g, const void *q, const void *pool,
+                                         const int32_t *d_block_table, int layer, int pos_start, int M,
+                                         float scale, int io_dtype, const float *d_row_lse, float *d_block_mass,
+                                         int mass_len, int accumulate, void *stream);
 /* importance_update_kernel, importance_scorer.cu:27-36, 67-73 */
 int drk_importance_update(float *d_scores, const float *d_new_scores, int n, float decay,
                           void *stream);

@@ -32,8 +32,10 @@ def test_bench_workload_runs(dev, extra):
         other = j["other_configs"]
         assert set(other) == {"config3_shared_prefix", "config3_fork_tree", "config4_int8", "config4_fp8", "config4_int8_append",
                               "config4_fp8_append", "config5_prefill", "config5_prefill_int8", "config5_prefill_fp8",
-                              "config7_decode_d256", "config7_prefill_d256"}
+                              "config7_decode_d256", "config7_prefill_d256", "frame_mass"}
         assert len(other["config3_fork_tree"]["shared_ranges"]) >= 3
+        fm = other.pop("frame_mass")
+        assert fm["attention_us"] < fm["with_one_walk_mass_same_stream_us"] < fm["with_two_walk_mass_us"]
         for name, e in other.items():
             assert 0 < e["frac"] < 1 and e["avg_launch_us"] > 0 and e["peak"] in (8000.0, 2500.0), name
         assert j["hbm_read_probe_permuted_4KiB_GBps"] > 1000 and j["mfma_bf16_probe_TFLOPs"] > 500

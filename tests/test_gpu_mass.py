@@ -171,6 +171,58 @@ def test_frame_mass_matches_fp64(dev, dtype, bs, pos_start, M, heads):
     assert np.all(np.abs(U.host(mass, np.float32) - 2 * want) <= 4e-3 * M + 4e-3 * np.abs(want))
 
 
+@pytest.fixture(params=["by_rule", "two_phase", "two_phase_through_registers", "context_split"])
+def chunk_path(request):
+    """the chunk kernels that can leave the rows' log-sum-exps: the four-wave kernel and the head_dim 256 one (by the
+    rule, for these sizes), the two-phase kernels, and the context-split pass with its merge"""
+    lib = cabi.lib()
+    if request.param == "context_split":
+        lib.drk_debug_set_prefill_split(4096)
+    else:
+        lib.drk_debug_set_prefill_two_phase({"by_rule": 1, "two_phase": 2, "two_phase_through_registers": 3}[request.param])
+    yield request.param
+    lib.drk_debug_set_prefill_two_phase(1)
+    lib.drk_debug_set_prefill_split(-1)
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
+@pytest.mark.parametrize("bs,pos_start,M,heads", [(16, 0, 70, (8, 32, 128)), (16, 333, 45, (8, 32, 128)), (32, 2500, 130, (2, 12, 128)),
+                                                  (256, 2100, 33, (4, 24, 256)), (16, 64, 300, (2, 2, 128))])
+def test_frame_mass_from_the_attention_calls_row_sums(dev, chunk_path, dtype, bs, pos_start, M, heads):
+    """The attention call leaves every row's log-sum-exp, the mass pass then walks the keys once: same masses as the
+    two-walk pass within the tolerance of the fp64 oracle, same attention output as the call without the extra result."""
+    total = pos_start + M
+    holes = (1,) if total > 3 * bs else ()
+    g, og, io, table, opool, q = _frame_case(dtype, bs, seed=bs + pos_start + M, pos_start=pos_start, M=M, heads=heads, holes=holes)
+    KVH, QH, D = heads
+    scale = 1.0 / np.sqrt(D)
+    lib = cabi.lib()
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    ws = U.dev_zeros(max(wsb, 16))
+    out0 = U.dev_bytes(np.full(M * QH * D * 2, 0x7B, dtype=np.uint8))
+    out1 = U.dev_bytes(np.full(M * QH * D * 2, 0x7B, dtype=np.uint8))
+    lse = U.dev_bytes(np.full(M * QH, 123.0, np.float32))
+    cabi.call("drk_paged_prefill_attention", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out0), 1, pos_start, M, float(scale), io,
+              U.p(ws), wsb, U.stream_ptr())
+    cabi.call("drk_paged_prefill_attention_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out1), 1, pos_start, M, float(scale),
+              io, None, 0, U.p(lse), U.p(ws), wsb, U.stream_ptr())
+    mass = U.dev_bytes(np.full(table.size, 7.0, np.float32))
+    cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale), io,
+              U.p(lse), U.p(mass), table.size, 0, U.stream_ptr())
+    U.sync()
+    assert np.array_equal(U.host(out0, np.uint16), U.host(out1, np.uint16))
+    got = U.host(mass, np.float32).astype(np.float64)
+    want = _frame_want(og, io, table, opool, q, pos_start, scale)
+    assert np.all(np.abs(got - want) <= 2e-3 * M + 3e-3 * np.abs(want)), np.abs(got - want).max()
+    seen = sum(1 for t in range(M) if any(table[p // bs] >= 0 for p in range(pos_start + t + 1)))
+    assert abs(got.sum() - seen * QH) <= 2e-3 * M * QH
+    rows = U.host(lse, np.float32).reshape(M, QH)
+    for t in range(M):                                     # rows without a visible token say so
+        sees = any(table[p // bs] >= 0 for p in range(pos_start + t + 1))
+        assert np.all(np.isfinite(rows[t])) if sees else np.all(np.isposinf(rows[t]))
+
+
 def test_frame_mass_of_a_long_chunk(dev):
     """A 300-token frame behind 3 000 tokens (several row tiles per kv head meeting in every page)."""
     pos_start, M, bs = 3000, 300, 16
