@@ -80,6 +80,8 @@ def parse():
                     help="storage type of the pages: config 4 int8 (default) | fp8; config 5 bf16 (default) | int8 | fp8")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "
                                                             "replaying one captured HIP graph per step")
+    ap.add_argument("--no-plan", action="store_true", help="build the decode kernel's unit descriptors in every layer's launch "
+                                                           "instead of once per step (drk_decode_plan_build)")
     ap.add_argument("--no-cascade", action="store_true", help="config 3: read the shared prefix once per branch")
     ap.add_argument("--forks", choices=["tree", "prefix"], default="tree",
                     help="config 3: branches fork from the prefix or from one another at random block boundaries (tree), "
@@ -172,16 +174,33 @@ def main():
     pos_steps = torch.from_numpy(np.stack([start + s for s in range(W + K)]).astype(np.int32)).cuda()
     len_steps = pos_steps + 1                                 # write-then-attend: the new token is visible
     qrow, krow = B * QH * D * 2, B * KVH * D * 2
+    # The layers of a step read the same tables and lengths: the decode kernel's unit descriptors are built once per
+    # step (one small launch) and read by the 36 attention launches.
+    plan_bytes = 0 if (split or args.no_plan) else lib.drk_decode_plan_bytes(C.byref(g), B, max_ctx, 0)
+    plan = torch.empty(max(plan_bytes, 16), dtype=torch.uint8, device="cuda")
+
+    def build_plan(dlen, spx):
+        if plan_bytes:
+            cabi.call("drk_decode_plan_build", C.byref(g), cabi.p(dtab), stride, dlen, B, max_ctx, None, 0, cabi.p(plan), plan_bytes, spx)
+
+    def attend(l, dlen, spx):
+        if plan_bytes:
+            cabi.call("drk_paged_decode_attention_planned", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), cabi.p(pool),
+                      cabi.p(dtab), stride, dlen, B, max_ctx, None, 0, cabi.p(plan), C.c_void_p(out.data_ptr() + l * qrow), l,
+                      float(scale), cabi.BF16, None, 0, cabi.p(ws), wsb, spx)
+        else:
+            cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow),
+                      cabi.p(pool), cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
+                      float(scale), cabi.BF16, split, cabi.p(ws), wsb, spx)
 
     def step(s):
         dpos = C.c_void_p(pos_steps[s].data_ptr())
         dlen = C.c_void_p(len_steps[s].data_ptr())
+        build_plan(dlen, sp)
         for l in range(L):
             cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos, B, l, 1,
                       C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, sp)
-            cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow),
-                      cabi.p(pool), cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
-                      float(scale), cabi.BF16, split, cabi.p(ws), wsb, sp)
+            attend(l, dlen, sp)
 
     use_graph = not args.no_graph
     if use_graph:
@@ -192,12 +211,11 @@ def main():
         def graph_step():
             dpos, dlen = C.c_void_p(pos_cur.data_ptr()), C.c_void_p(len_cur.data_ptr())
             gsp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            build_plan(dlen, gsp)
             for l in range(L):
                 cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos, B, l, 1,
                           C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, gsp)
-                cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow),
-                          cabi.p(pool), cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
-                          float(scale), cabi.BF16, split, cabi.p(ws), wsb, gsp)
+                attend(l, dlen, gsp)
             pos_cur.add_(1)
             len_cur.add_(1)
 
@@ -253,11 +271,13 @@ def main():
                       cabi.BF16, split, cabi.p(ws), wsb, sp)
 
     # (event pairs recorded here, around calls that leave the merge kernel out: cabi.time_partial_kernels)
+    planned_for = [None]
+
     def attn_one(it, lens=dlen):
-        l = it % L
-        cabi.call("drk_paged_decode_attention_branches", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), cabi.p(pool),
-                  cabi.p(dtab), stride, lens, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l, float(scale),
-                  cabi.BF16, split, cabi.p(ws), wsb, sp)
+        if planned_for[0] != lens.value:                     # the timed launches read the plan of their lengths
+            build_plan(lens, sp)
+            planned_for[0] = lens.value
+        attend(it % L, lens, sp)
 
     ker_avg_ms = cabi.time_partial_kernels(attn_one, n_timed, warm=8)
     launch_bytes = int((start + last + 1).sum()) * kv_bytes_per_token               # one layer, one launch
@@ -285,6 +305,7 @@ def main():
         ragged_pro_ms = cabi.time_partial_kernels(lambda it: attn_one(it, cabi.p(rlen)), n_timed, warm=8)
         fixed_pro_ms = cabi.time_partial_kernels(attn_one, n_timed, warm=8)
         lib.drk_debug_set_stream_descriptors_only(0)
+        planned_for[0] = None
         attn_only(2)                                                 # leave real results behind
         ragged = {"ctx": [int(x) for x in rl], "kernel_us": round(r_ms * 1e3, 2), "bytes_per_launch": r_bytes,
                   "GBps": round(r_bytes / (r_ms * 1e-3) / 1e9, 1), "hbm_frac": round(r_bytes / (r_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
@@ -557,6 +578,7 @@ def main():
                         f"{int(final.min())}..{int(final.max())}; step = per layer: append 1 token/branch + paged decode attention",
             "branches": B, "layers": L, "ctx_final": [int(x) for x in final],
             "launch": "one captured HIP graph per step" if use_graph else "host launches",
+            "unit_descriptors": "built once per step" if plan_bytes else "built by every launch",
         },
         "hbm_frac_step": round(value_gbps / HBM_PEAK_GBPS, 4),
         "us_per_step": round(ms_per_step * 1e3, 1),

@@ -211,6 +211,9 @@ def config3(args):
               lib.drk_decode_grouped_workspace_bytes_max(C.byref(g), B, max_ctx, cabi.MAX_PREFIX_GROUPS) if grouped else 0)
     ws = torch.empty(wsb, dtype=torch.uint8, device="cuda")
     shared_now, groups_now = [0], [[], cabi.prefix_groups([])]
+    # the unit descriptors of the grouped kernel, built once per step for the 36 layers
+    plan_bytes = lib.drk_decode_plan_bytes(C.byref(g), B, max_ctx, cabi.MAX_PREFIX_GROUPS) if grouped and not getattr(args, "no_plan", False) else 0
+    plan = torch.empty(max(plan_bytes, 16), dtype=torch.uint8, device="cuda")
     dpos = torch.zeros(B, dtype=torch.int32, device="cuda")
     dlen = torch.zeros(B, dtype=torch.int32, device="cuda")
     # the forked branches' rows are consecutive in the device table: branch ids forks[0]..forks[-1]
@@ -220,7 +223,11 @@ def config3(args):
     ensure_ns, evicted, evict_ns = [], 0, 0.0
 
     def attend(l, dl):
-        if grouped:
+        if plan_bytes:
+            cabi.call("drk_paged_decode_attention_planned", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr,
+                      dtabs, stride, dl, B, max_ctx, groups_now[1], len(groups_now[0]), cabi.p(plan),
+                      C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.BF16, None, 0, cabi.p(ws), wsb, sp)
+        elif grouped:
             cabi.call("drk_paged_decode_attention_grouped", C.byref(g), C.c_void_p(q.data_ptr() + l * qrow), pool_ptr,
                       dtabs, stride, dl, B, max_ctx, groups_now[1], len(groups_now[0]), C.c_void_p(out.data_ptr() + l * qrow),
                       l, float(scale), cabi.BF16, None, 0, cabi.p(ws), wsb, sp)
@@ -250,6 +257,9 @@ def config3(args):
             groups_now[1] = cabi.prefix_groups(groups_now[0])
         dpos.copy_(torch.from_numpy(lens))
         dlen.copy_(torch.from_numpy(lens + 1))
+        if plan_bytes:
+            cabi.call("drk_decode_plan_build", C.byref(g), dtabs, stride, cabi.p(dlen), B, max_ctx, groups_now[1],
+                      len(groups_now[0]), cabi.p(plan), plan_bytes, sp)
         for l in range(L):
             cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, cabi.p(dpos), B, l, 1,
                       C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)

@@ -62,6 +62,17 @@ bool KvStream::init(CacheManager& cm, int max_context_len, ImportanceScorer* sco
     }
     // every attention call below finds its split-K workspace ready: nothing allocates later
     const int bs = cm.block_pool().block_size();
+    // the decode kernels' unit descriptors, built once per step for all layers (where the kernels take a plan)
+    plan_bytes_ = paged_decode_plan_bytes(cm.max_branches(), max_context_len, cm.block_pool().max_blocks(), bs, DRK_MAX_PREFIX_GROUPS);
+    if (plan_bytes_) {
+        p = nullptr;
+        if (drk_dev_malloc(&p, plan_bytes_) != DRK_OK) {
+            LOG_ERROR("Conscientia", "KvStream: plan buffer: %s", drk_last_error());
+            destroy();
+            return false;
+        }
+        d_plan_ = p;
+    }
     if (!ws_decode_.reserve_for(cm.max_branches(), max_context_len, 0, bs) ||
         !ws_prefill_.reserve_for(1, max_context_len, max_prefill_rows, bs)) {
         destroy();
@@ -80,6 +91,12 @@ void KvStream::destroy()
     if (cm_) close_branches();
     if (d_pos_) drk_dev_free(d_pos_);
     if (d_len_) drk_dev_free(d_len_);
+    if (d_plan_) {
+        drk_device_synchronize();                 // a launch may still be reading it
+        drk_dev_free(d_plan_);
+        d_plan_ = nullptr;
+    }
+    plan_bytes_ = 0;
     if (d_row_lse_ || ev_attn_ || ev_mass_) {
         drk_device_synchronize();                 // a mass pass may still be reading
         if (d_row_lse_) drk_dev_free(d_row_lse_);
@@ -308,6 +325,7 @@ void KvStream::host_end()
 bool KvStream::begin_decode_step(hipStream_t stream)
 {
     first_layer_of_step_ = -1;
+    plan_built_ = false;
     return host_begin(stream);
 }
 
@@ -338,9 +356,14 @@ void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t s
             LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
     } else if (B >= shared_min_branches_ && !groups_.empty() && groups_[0].tok_end - groups_[0].tok_begin >= shared_min_tokens_) {
         // every range some of the branches share is streamed once for them, the gate rides on the merge
-        paged_gqa_decode_attention_grouped(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
-                                           groups_.data(), (int)groups_.size(), gate, 2 * hd, io.attn_out, fa_layer_idx,
-                                           pool.max_blocks(), pool.block_size(), scale, stream);
+        if (step_plan(tables, stride, B, max_len, groups_.data(), (int)groups_.size(), stream))
+            paged_gqa_decode_attention_planned(ws_decode_, d_plan_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
+                                               groups_.data(), (int)groups_.size(), gate, 2 * hd, io.attn_out, fa_layer_idx,
+                                               pool.max_blocks(), pool.block_size(), scale, stream);
+        else
+            paged_gqa_decode_attention_grouped(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
+                                               groups_.data(), (int)groups_.size(), gate, 2 * hd, io.attn_out, fa_layer_idx,
+                                               pool.max_blocks(), pool.block_size(), scale, stream);
     } else if (B >= shared_min_branches_ && shared_tokens_ >= shared_min_tokens_) {
         // the branches' common prefix is streamed once for all of them
         paged_gqa_decode_attention_shared(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, shared_tokens_,
@@ -348,11 +371,30 @@ void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t s
         if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
                              ModelConfig::IO_DTYPE, stream) != DRK_OK)
             LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
+    } else if (step_plan(tables, stride, B, max_len, nullptr, 0, stream)) {
+        paged_gqa_decode_attention_planned(ws_decode_, d_plan_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
+                                           nullptr, 0, gate, 2 * hd, io.attn_out, fa_layer_idx, pool.max_blocks(),
+                                           pool.block_size(), scale, stream);
     } else {
         paged_gqa_decode_attention_gated_branches(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len, gate,
                                                   2 * hd, io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(),
                                                   scale, stream);
     }
+}
+
+// The step's unit descriptors: built by the first layer that asks, read by the others (the tables and lengths do not
+// change within a step).  False where the kernels take no plan.
+bool KvStream::step_plan(const int* tables, int stride, int B, int max_len, const drk_prefix_group* groups, int n_groups,
+                         hipStream_t stream)
+{
+    if (!d_plan_ || B > 64) return false;
+    if (plan_built_) return true;
+    const BlockPool& pool = cm_->block_pool();
+    if (!paged_decode_plan_build(d_plan_, plan_bytes_, tables, stride, d_len_, B, max_len, groups, n_groups, pool.max_blocks(),
+                                 pool.block_size(), stream))
+        return false;
+    plan_built_ = true;
+    return true;
 }
 
 void KvStream::end_decode_step(hipStream_t stream)
@@ -374,6 +416,7 @@ bool KvStream::capture_decode_step(const std::function<void(hipStream_t)>& layer
     }
     // host part first: the capture must not contain table uploads or the position upload
     first_layer_of_step_ = -1;
+    plan_built_ = false;
     if (!host_begin(stream)) return false;
     if (drk_graph_begin_capture(stream) != DRK_OK) {
         LOG_ERROR("Conscientia", "KvStream: begin capture: %s", drk_last_error());

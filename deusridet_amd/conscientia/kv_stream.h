@@ -129,6 +129,11 @@ private:
     int max_prefill_rows_ = 0;
     int first_layer_of_step_ = -1;   // the layer whose scored call overwrites instead of accumulating
     int first_layer_of_frame_ = -1;  // the same for the mass pass of a perception frame
+    void* d_plan_ = nullptr;               // the decode kernels' unit descriptors of the step under way
+    size_t plan_bytes_ = 0;
+    bool plan_built_ = false;
+    bool step_plan(const int* tables, int stride, int B, int max_len, const drk_prefix_group* groups, int n_groups,
+                   hipStream_t stream);
     hipStream_t frame_stream_ = nullptr;   // stream of the frame's layers
     hipStream_t mass_stream_ = nullptr;    // stream of the frame's mass passes (the scorer's)
     float* d_row_lse_ = nullptr;           // [2][max_prefill_rows][num_q_heads]: the rows' log-sum-exps, by turns

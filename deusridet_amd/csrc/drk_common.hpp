@@ -56,13 +56,22 @@ inline int ilog2_exact(unsigned v)                 // -1 when v is not a power o
 }
 
 // ---- shared between the decode and prefill translation units ---------------
+// The unit descriptors of the persistent decode kernels, built once and read by every launch on the same tables and
+// lengths (the layers of one step).  mode 1: the launch only builds and stores them; 2: it reads them.  One record per
+// workgroup: {units, 0, 0, 0}, max_units unit descriptors of 16 bytes, max_units x 4 page descriptors of 8 bytes.
+struct DecodePlan {
+    uint8_t *ptr = nullptr;
+    int mode = 0;
+};
+constexpr size_t plan_record_bytes(int max_units) { return 16 + 48 * (size_t)max_units; }
+size_t decode_plan_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups);
 extern int g_force_portable;
 extern int g_skip_merge;
 int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                   int table_stride, const int32_t *d_seq_lens, int seq_len_host, int causal_base, int B,
                   int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
                   void *workspace, size_t workspace_bytes, void *stream, const void *gate = nullptr,
-                  size_t gate_stride = 0);
+                  size_t gate_stride = 0, DecodePlan plan = {});
 // out[row][d] *= sigmoid(gate[row * gate_stride + d]), rows of D elements (drk_layer.hip)
 int launch_sigmoid_gate(const void *x, const void *gate, void *out, size_t rows, int D, size_t gate_stride_elems,
                         int dtype, hipStream_t st);
@@ -82,7 +91,8 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
                          int start_tile = 0, const float *pre_o = nullptr, const float *pre_m = nullptr,
                          const float *pre_l = nullptr, int pre_splits = 0, const void *gate = nullptr,
                          size_t gate_stride = 0, float *lse_groups = nullptr, float *lse_rows = nullptr,
-                         int lse_stride = 0);
+                         int lse_stride = 0, DecodePlan plan = {});
+size_t stream_plan_need(const Lay &a, int B, int max_seq_len);
 int launch_block_mass(const float *lse_groups, const float *lse_rows, const int32_t *d_seq_lens, int B, int QH,
                       int lse_stride, int bs, float *mass, int mass_stride, int accumulate, hipStream_t st);
 // branches over a shared prefix: prefix pass + tails + one merge (drk_decode.hip); table_stride 0 = one table for all
@@ -98,7 +108,8 @@ size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_
 int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables, int table_stride,
                           const int32_t *d_seq_lens, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups,
                           void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
-                          void *stream, const void *gate = nullptr, size_t gate_stride = 0);
+                          void *stream, const void *gate = nullptr, size_t gate_stride = 0, DecodePlan plan = {});
+size_t grouped_plan_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups);
 // shared-prefix pass on the matrix cores (drk_prefill.hip)
 void shared_prefix_shape(const Lay &a, int B, int shared, int *chunk_tiles, int *nsplits);
 int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const int32_t *table0,

@@ -484,12 +484,14 @@ static size_t workspace_need(const Lay &a, int B, int max_seq_len, int split)
 int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables,
                          int table_stride, const int32_t *d_seq_lens, int seq_len_host, int causal_base,
                          int B, int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
-                         void *workspace, size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride)
+                         void *workspace, size_t workspace_bytes, void *stream, const void *gate, size_t gate_stride,
+                         DecodePlan plan)
 {
     Lay a;
     int rc = make_lay(g, &a);
     if (rc) return rc;
-    if (!q || !pool || !tables || !out) return fail(DRK_ERR_INVALID, "decode: NULL pointer");
+    const bool plan_only = plan.ptr && plan.mode == 1;              // builds the unit descriptors: reads tables and lengths only
+    if (!tables || (!plan_only && (!q || !pool || !out))) return fail(DRK_ERR_INVALID, "decode: NULL pointer");
     if (gate && (gate_stride < (size_t)a.D || (gate_stride % 8) || ((uintptr_t)gate % 16)))
         return fail(DRK_ERR_INVALID, "decode: gate rows must be 16-byte aligned and at least head_dim apart");
     if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode: io_dtype must be F16 or BF16");
@@ -506,6 +508,7 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     // more branches than one launch of the tiled kernel takes: 64 at a time, one after the other
     // through the same workspace (the launches are ordered by the stream)
     if (B > 64 && d_seq_lens && !g_force_portable && g_decode_kernel != 2 && causal_base < 0 && stream_decode_supported(a, 64)) {
+        if (plan.ptr) return fail(DRK_ERR_UNSUPPORTED, "decode: a plan covers at most 64 branches");
         const size_t row = (size_t)a.QH * a.D * 2;
         for (int b0 = 0; b0 < B; b0 += 64) {
             const int nb = B - b0 < 64 ? B - b0 : 64;
@@ -524,7 +527,13 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     if (use_stream && split_tokens > kStreamMaxSplitTokens)
         return fail(DRK_ERR_INVALID, "decode: split_tokens %d exceeds %d (the tiled kernel's run length)", split_tokens,
                     kStreamMaxSplitTokens);
+    if (plan.ptr && (!use_stream || split_tokens))
+        return fail(DRK_ERR_UNSUPPORTED, "decode: plans are for the tiled kernel with its own split");
     const size_t need = use_stream ? stream_workspace_need(a, B, max_seq_len, split_tokens) : workspace_need(a, B, max_seq_len, split);
+    if (plan_only)
+        return launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, seq_len_host, B, max_seq_len, out, layer,
+                                    scale, io_dtype, split_tokens, workspace, false, (hipStream_t)stream, 0, nullptr, nullptr,
+                                    nullptr, 0, nullptr, 0, nullptr, nullptr, 0, plan);
     if (!workspace || workspace_bytes < need)
         return fail(DRK_ERR_WORKSPACE, "decode: workspace of %zu bytes, need %zu", workspace_bytes, need);
     if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode: workspace must be 16-byte aligned");
@@ -539,7 +548,8 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
     const bool tiled = !g_force_portable && a.D == 128 && a.E == 2 && G == 4 && (a.bs % 16) == 0;
     if (use_stream) {
         rc = launch_decode_stream(a, q, pool, tables, table_stride, d_seq_lens, seq_len_host, B, max_seq_len, out, layer,
-                                  scale, io_dtype, split_tokens, workspace, false, st);
+                                  scale, io_dtype, split_tokens, workspace, false, st, 0, nullptr, nullptr, nullptr, 0, nullptr,
+                                  0, nullptr, nullptr, 0, plan);
         if (rc) return rc;
     } else if (tiled) {
         TiledArgs A;
@@ -658,11 +668,74 @@ int launch_decode_shared(const drk_kv_layout *g, const void *q, const void *pool
                                 io_dtype, 0, workspace, true, st, shared / kTile, pre_o, pre_m, pre_l, ns, gate, gate_stride);
 }
 
+size_t decode_plan_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups)
+{
+    if (g_force_portable || g_decode_kernel == 2 || B < 1 || B > 64 || max_seq_len < 1 || !stream_decode_supported(a, B)) return 0;
+    size_t need = stream_plan_need(a, B, max_seq_len);
+    if (n_groups > 0 && grouped_decode_supported(a, B)) {
+        const size_t g2 = grouped_plan_need(a, B, max_seq_len, groups, n_groups);
+        if (g2 > need) need = g2;
+    }
+    return need;
+}
+
 } // namespace drk
 
 using namespace drk;
 
 extern "C" {
+
+size_t drk_decode_plan_bytes(const drk_kv_layout *g, int B, int max_seq_len, int n_groups)
+{
+    Lay a;
+    if (make_lay(g, &a) != DRK_OK) return 0;
+    return decode_plan_need(a, B, max_seq_len, nullptr, n_groups);
+}
+
+int drk_decode_plan_build(const drk_kv_layout *g, const int32_t *d_tables, int table_stride, const int32_t *d_seq_lens, int B,
+                          int max_seq_len, const drk_prefix_group *groups, int n_groups, void *d_plan, size_t plan_bytes,
+                          void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (!d_tables || !d_seq_lens || !d_plan) return fail(DRK_ERR_INVALID, "decode_plan: NULL pointer");
+    if (((uintptr_t)d_plan) % 16) return fail(DRK_ERR_INVALID, "decode_plan: the plan must be 16-byte aligned");
+    const size_t need = decode_plan_need(a, B, max_seq_len, groups, n_groups);
+    if (need == 0) return fail(DRK_ERR_UNSUPPORTED, "decode_plan: this geometry or number of branches takes no plan");
+    if (plan_bytes < need) return fail(DRK_ERR_WORKSPACE, "decode_plan: plan of %zu bytes, need %zu", plan_bytes, need);
+    DecodePlan plan;
+    plan.ptr = (uint8_t *)d_plan;
+    plan.mode = 1;
+    const int io = a.dtype == DRK_F16 ? DRK_F16 : DRK_BF16;
+    if (n_groups > 0 && grouped_decode_supported(a, B))
+        return launch_decode_grouped(g, nullptr, nullptr, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups, n_groups,
+                                     nullptr, 0, 1.0f, io, nullptr, 0, stream, nullptr, 0, plan);
+    return launch_decode(g, nullptr, nullptr, d_tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, nullptr, 0, 1.0f, io, 0,
+                         nullptr, 0, stream, nullptr, 0, plan);
+}
+
+int drk_paged_decode_attention_planned(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_tables,
+                                       int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len,
+                                       const drk_prefix_group *groups, int n_groups, const void *d_plan, void *out, int layer,
+                                       float scale, int io_dtype, const void *gate, size_t gate_stride, void *workspace,
+                                       size_t workspace_bytes, void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (!d_plan) return fail(DRK_ERR_INVALID, "decode_planned: d_plan is NULL");
+    if (decode_plan_need(a, B, max_seq_len, groups, n_groups) == 0)
+        return fail(DRK_ERR_UNSUPPORTED, "decode_planned: this geometry or number of branches takes no plan");
+    DecodePlan plan;
+    plan.ptr = (uint8_t *)const_cast<void *>(d_plan);
+    plan.mode = 2;
+    if (n_groups > 0 && grouped_decode_supported(a, B))
+        return launch_decode_grouped(g, q, pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups, n_groups, out, layer,
+                                     scale, io_dtype, workspace, workspace_bytes, stream, gate, gate_stride, plan);
+    return launch_decode(g, q, pool, d_tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale, io_dtype, 0,
+                         workspace, workspace_bytes, stream, gate, gate_stride, plan);
+}
 
 size_t drk_decode_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len)
 {

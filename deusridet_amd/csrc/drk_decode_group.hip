@@ -55,6 +55,8 @@ struct GroupedArgs {
     GSeg seg[kGMaxGroups];
     int b_start[64];                           // first tile of each branch's private tail
     int b_slot[64];                            // first workspace slot of the tail's pieces
+    uint8_t *plan;                             // the descriptors of every workgroup in global memory, see DecodePlan
+    int plan_mode;                             // 0: build and use; 1: build, store, leave (build_units returns 0); 2: read
 };
 
 struct GUnit {                                 // one 64-token tile of one kv head of a group or a tail
@@ -148,6 +150,7 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int GQ = A.QH / A.KVH;
+    if (A.plan_mode == 2) return plan_load<GUnit, MAXU>(A.plan, udesc, gdesc);
     // ---- the workgroup's run of units and one descriptor per unit ---------------------
     const int len_i = lane < A.B ? A.seq_lens[lane] : 0;
     const int nt_i = len_i > 0 ? max((len_i + kSTile - 1) / kSTile - A.b_start[lane], 0) : 0;
@@ -158,17 +161,15 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
         if (lane >= off) incl += t;
     }
     const int tail_units = __builtin_amdgcn_readlane(incl, 63) * A.KVH;
-    if (A.group_units + tail_units == 0) return 0;
     const RegionSplit rs = region_split(A.group_units, tail_units, (int)gridDim.x);
     const bool tail_wg = (int)blockIdx.x >= rs.Gs;
     const int U = tail_wg ? rs.Ut : rs.Us;
     const int wg_rel = tail_wg ? (int)blockIdx.x - rs.Gs : (int)blockIdx.x;      // the workgroup's place among those of its kind
     const int region_units = tail_wg ? tail_units : A.group_units;
     const int u0 = wg_rel * U;                                   // its first unit, counted within its kind
-    if (u0 >= region_units) return 0;
     // the host sizes the grid from max_seq_len; lengths on the device beyond that bound must not overrun
     // the descriptor table (the tiles past it are then left out: the caller broke its promise)
-    const int nunits = min(min(U, region_units - u0), MAXU);
+    const int nunits = u0 >= region_units ? 0 : min(min(U, region_units - u0), MAXU);
     if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
     __syncthreads();
     if ((int)threadIdx.x < A.ngroups) {
@@ -229,6 +230,10 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
         }
     }
     __syncthreads();
+    if (A.plan_mode == 1) {
+        plan_store<GUnit, MAXU>(A.plan, nunits, udesc, gdesc);
+        return 0;
+    }
     return nunits;
 }
 
@@ -1110,12 +1115,13 @@ size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_
 int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables, int table_stride,
                           const int32_t *d_seq_lens, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups,
                           void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
-                          void *stream, const void *gate, size_t gate_stride)
+                          void *stream, const void *gate, size_t gate_stride, DecodePlan plan)
 {
     Lay a;
     int rc = make_lay(g, &a);
     if (rc) return rc;
-    if (!q || !pool || !tables || !out || !d_seq_lens) return fail(DRK_ERR_INVALID, "decode_grouped: NULL pointer");
+    const bool plan_only = plan.ptr && plan.mode == 1;              // builds the unit descriptors: reads tables and lengths only
+    if (!tables || !d_seq_lens || (!plan_only && (!q || !pool || !out))) return fail(DRK_ERR_INVALID, "decode_grouped: NULL pointer");
     if (gate && (gate_stride < (size_t)a.D || (gate_stride % 8) || ((uintptr_t)gate % 16)))
         return fail(DRK_ERR_INVALID, "decode_grouped: gate rows must be 16-byte aligned and at least head_dim apart");
     if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode_grouped: io_dtype must be F16 or BF16");
@@ -1130,9 +1136,9 @@ int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *poo
     if ((rc = plan_groups(a, B, max_seq_len, groups, n_groups, &P))) return rc;
     if (P.ngroups == 0)                                            // nothing shared (after rounding to tiles): the plain kernel
         return launch_decode(g, q, pool, tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale, io_dtype,
-                             0, workspace, workspace_bytes, stream, gate, gate_stride);
+                             0, workspace, workspace_bytes, stream, gate, gate_stride, plan);
     const size_t need = (size_t)B * a.QH * P.Ptot * (a.D + 2) * sizeof(float);
-    if (!workspace || workspace_bytes < need)
+    if (!plan_only && (!workspace || workspace_bytes < need))
         return fail(DRK_ERR_WORKSPACE, "decode_grouped: workspace of %zu bytes, need %zu", workspace_bytes, need);
     if (((uintptr_t)workspace) % 16) return fail(DRK_ERR_INVALID, "decode_grouped: workspace must be 16-byte aligned");
 
@@ -1150,6 +1156,7 @@ int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *poo
     A.scale_log2e = scale * kSLog2e;
     for (int k = 0; k < kGMaxGroups; k++) A.seg[k] = k < P.ngroups ? P.seg[k] : GSeg{0, 0, 0, 0, 0, 0x7fffffff};
     for (int b = 0; b < 64; b++) { A.b_start[b] = P.b_start[b]; A.b_slot[b] = P.b_slot[b]; }
+    A.plan = plan.ptr; A.plan_mode = plan.ptr ? plan.mode : 0;
     hipStream_t st = (hipStream_t)stream;
     // 16-bit pages: the tile in LDS, rows dealt to the waves; 8-bit pages (and, as a cross-check, 16-bit pages in
     // diagnostic mode 2): tokens dealt to the waves, K and V through registers
@@ -1167,11 +1174,17 @@ int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *poo
     default: hipLaunchKernelGGL((decode_group_kernel<DRK_FP8_E4M3, 128, 4>), dim3(P.grid), dim3(256), 0, st, A); break;
     }
     DRK_LAUNCH_CHECK("decode_group_kernel");
-    if (g_skip_merge) return DRK_OK;
+    if (g_skip_merge || plan_only) return DRK_OK;
     hipLaunchKernelGGL(group_merge_kernel<128>, dim3(a.QH, B), dim3(256), 0, st, A, (uint16_t *)out, P.grid,
                        (const uint16_t *)gate, gate_stride);
     DRK_LAUNCH_CHECK("group_merge_kernel");
     return DRK_OK;
+}
+
+size_t grouped_plan_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups)
+{
+    (void)a; (void)B; (void)max_seq_len; (void)groups; (void)n_groups;
+    return (size_t)kGWgs * plan_record_bytes(kGMaxUnits);          // either kernel's records fit
 }
 
 } // namespace drk

@@ -55,6 +55,8 @@ struct StreamArgs {
     float *lse_groups;
     int lse_stride;
     int stop_after_descriptors;     // measurement aid: leave once the workgroup's unit descriptors are built
+    uint8_t *plan;                  // the descriptors of every workgroup in global memory, see DecodePlan
+    int plan_mode;                  // 0: build and use; 1: build, store, leave; 2: read
 };
 
 constexpr int kMaxUnits = kStreamMaxUnits;    // units one workgroup may own (descriptor table in LDS)
@@ -87,59 +89,67 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
     const int g = lane >> 4, c = lane & 15;
     const int GQ = A.QH / A.KVH;                               // query heads per kv head, 1..16
     // ---- the workgroup's run of units and one descriptor per unit ---------------------
-    const int len_i = lane < A.B ? (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host) : 0;
-    const int nt_i = len_i > 0 ? max((len_i + kSTile - 1) / kSTile - A.start_tile, 0) : 0;
-    int incl = nt_i;
+    int nunits = 0;
+    if (A.plan_mode == 2) {
+        nunits = plan_load<UnitDesc, kMaxUnits>(A.plan, udesc, gdesc);
+    } else {
+        const int len_i = lane < A.B ? (A.seq_lens ? A.seq_lens[lane] : A.seq_len_host) : 0;
+        const int nt_i = len_i > 0 ? max((len_i + kSTile - 1) / kSTile - A.start_tile, 0) : 0;
+        int incl = nt_i;
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const int t = __shfl_up(incl, off);
-        if (lane >= off) incl += t;
-    }
-    const int T = __builtin_amdgcn_readlane(incl, 63) * A.KVH;
-    if (T == 0) return;
-    const int U = A.unit_tiles > 0 ? A.unit_tiles : (T + (int)gridDim.x - 1) / (int)gridDim.x;
-    const int u0 = (int)blockIdx.x * U;
-    if (u0 >= T) return;
-    // the host sizes U from max_seq_len; a length on the device beyond that bound must not overrun the
-    // descriptor table (the tiles past it are then left out: the caller broke its promise)
-    const int nunits = min(min(U, T - u0), kMaxUnits);
-    if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
-    __syncthreads();
-    for (int i = threadIdx.x; i < nunits * 4; i += 256) {
-        const int ui = i >> 2, grp = i & 3, u = u0 + ui;
-        int lo = 0, hi = A.B - 1;                              // first branch whose cumulative units exceed u
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (A.KVH * s_incl[mid] > u) hi = mid; else lo = mid + 1;
+        for (int off = 1; off < 64; off <<= 1) {
+            const int t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
         }
-        const int b = lo;
-        const int excl = b ? s_incl[b - 1] : 0, nt = s_incl[b] - excl, len = s_len[b];
-        const int rem = u - A.KVH * excl, kvh = rem / nt, trel = rem - kvh * nt;
-        const int tile = trel + A.start_tile;                  // absolute tile of the branch
-        const int tg = tile * kSTile + grp * 16;
-        uint2 gd = make_uint2(kNone, 0u);
-        if (tg < len) {
-            const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
-            const int blk = A.tables[(size_t)b * A.table_stride + lb];
-            if (blk >= 0 && blk < A.NB) {
-                // every term is a multiple of 16 bytes (pp is a multiple of 16, plane sizes of 16 * 16)
-                const unsigned pp = (unsigned)(tg - lb * A.bs);
-                const size_t base = (size_t)blk * A.block_stride;
-                gd.x = (unsigned)((base + (size_t)kvh * A.head_stride + (size_t)pp * A.row_bytes) >> 4);
-                gd.y = (unsigned)((base + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + pp) * 2) >> 4);
+        const int T = __builtin_amdgcn_readlane(incl, 63) * A.KVH;
+        const int U = A.unit_tiles > 0 ? A.unit_tiles : (T + (int)gridDim.x - 1) / (int)gridDim.x;
+        const int u0 = (int)blockIdx.x * U;
+        // the host sizes U from max_seq_len; a length on the device beyond that bound must not overrun the
+        // descriptor table (the tiles past it are then left out: the caller broke its promise)
+        nunits = (T == 0 || u0 >= T) ? 0 : min(min(U, T - u0), kMaxUnits);
+        if (w == 0) { s_incl[lane] = incl; s_len[lane] = len_i; }
+        __syncthreads();
+        for (int i = threadIdx.x; i < nunits * 4; i += 256) {
+            const int ui = i >> 2, grp = i & 3, u = u0 + ui;
+            int lo = 0, hi = A.B - 1;                              // first branch whose cumulative units exceed u
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (A.KVH * s_incl[mid] > u) hi = mid; else lo = mid + 1;
+            }
+            const int b = lo;
+            const int excl = b ? s_incl[b - 1] : 0, nt = s_incl[b] - excl, len = s_len[b];
+            const int rem = u - A.KVH * excl, kvh = rem / nt, trel = rem - kvh * nt;
+            const int tile = trel + A.start_tile;                  // absolute tile of the branch
+            const int tg = tile * kSTile + grp * 16;
+            uint2 gd = make_uint2(kNone, 0u);
+            if (tg < len) {
+                const int lb = A.bs_shift >= 0 ? (tg >> A.bs_shift) : (tg / A.bs);
+                const int blk = A.tables[(size_t)b * A.table_stride + lb];
+                if (blk >= 0 && blk < A.NB) {
+                    // every term is a multiple of 16 bytes (pp is a multiple of 16, plane sizes of 16 * 16)
+                    const unsigned pp = (unsigned)(tg - lb * A.bs);
+                    const size_t base = (size_t)blk * A.block_stride;
+                    gd.x = (unsigned)((base + (size_t)kvh * A.head_stride + (size_t)pp * A.row_bytes) >> 4);
+                    gd.y = (unsigned)((base + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + pp) * 2) >> 4);
+                }
+            }
+            gdesc[ui][grp] = gd;
+            if (grp == 0) {
+                UnitDesc d;
+                d.tile_lim = len - tile * kSTile;
+                d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0) | (tile << 2);
+                d.bq = b * A.QH + kvh * GQ;
+                d.piece = (int)blockIdx.x - (A.KVH * excl + kvh * nt) / U;
+                udesc[ui] = d;
             }
         }
-        gdesc[ui][grp] = gd;
-        if (grp == 0) {
-            UnitDesc d;
-            d.tile_lim = len - tile * kSTile;
-            d.flags = ((ui == 0 || trel == 0) ? 1 : 0) | ((ui == nunits - 1 || trel + 1 == nt) ? 2 : 0) | (tile << 2);
-            d.bq = b * A.QH + kvh * GQ;
-            d.piece = (int)blockIdx.x - (A.KVH * excl + kvh * nt) / U;
-            udesc[ui] = d;
+        __syncthreads();
+        if (A.plan_mode == 1) {
+            plan_store<UnitDesc, kMaxUnits>(A.plan, nunits, udesc, gdesc);
+            return;
         }
     }
-    __syncthreads();
+    if (nunits == 0) return;
     if (A.stop_after_descriptors) return;
 
     uint8_t *const klds = &k_lds[w][0];
@@ -569,6 +579,13 @@ static void stream_shape(const Lay &a, int B, int max_seq_len, int split_tokens,
     }
 }
 
+size_t stream_plan_need(const Lay &a, int B, int max_seq_len)
+{
+    int grid, U, Pmax;
+    stream_shape(a, B, max_seq_len, 0, 0, &grid, &U, &Pmax);
+    return (size_t)grid * plan_record_bytes(kMaxUnits);
+}
+
 size_t stream_workspace_need(const Lay &a, int B, int max_seq_len, int split_tokens, int start_tile)
 {
     int grid, U, Pmax;
@@ -581,7 +598,8 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
                          const int32_t *d_seq_lens, int seq_len_host, int B, int max_seq_len, void *out, int layer,
                          float scale, int io_dtype, int split_tokens, void *workspace, bool merge_only, hipStream_t st,
                          int start_tile, const float *pre_o, const float *pre_m, const float *pre_l, int pre_splits,
-                         const void *gate, size_t gate_stride, float *lse_groups, float *lse_rows, int lse_stride)
+                         const void *gate, size_t gate_stride, float *lse_groups, float *lse_rows, int lse_stride,
+                         DecodePlan plan)
 {
     int grid, U, Pmax;
     stream_shape(a, B, max_seq_len, split_tokens, start_tile, &grid, &U, &Pmax);
@@ -601,6 +619,7 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         A.scale_log2e = scale * kSLog2e;
         A.lse_groups = lse_groups; A.lse_stride = lse_stride;
         A.stop_after_descriptors = g_stream_stop_after_descriptors;
+        A.plan = plan.ptr; A.plan_mode = plan.ptr ? plan.mode : 0;
 #define DRK_STREAM_LAUNCH(DT)                                                                                           \
     do {                                                                                                                \
         const bool g4 = a.QH / a.KVH <= 4;                                                                              \

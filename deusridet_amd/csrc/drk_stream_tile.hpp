@@ -232,6 +232,36 @@ __device__ __forceinline__ void v_operands(const uint4 &r0, const uint4 &r1, con
     }
 }
 
+// ---- a workgroup's unit descriptors to and from a plan in global memory ---------------------------------
+// UD is the kernel's 16-byte unit descriptor; udesc / gdesc are its tables in LDS, complete (a barrier has passed).
+template <typename UD, int MAXU>
+__device__ __forceinline__ void plan_store(uint8_t *plan, int nunits, const UD *udesc, const uint2 (*gdesc)[4])
+{
+    static_assert(sizeof(UD) == 16, "unit descriptors are 16 bytes");
+    uint8_t *rec = plan + (size_t)blockIdx.x * plan_record_bytes(MAXU);
+    if (threadIdx.x == 0) *(int4 *)rec = make_int4(nunits, 0, 0, 0);
+    for (int i = threadIdx.x; i < nunits * 3; i += blockDim.x) {
+        const int u = i / 3, part = i - 3 * u;
+        if (part == 0) *(uint4 *)(rec + 16 + 16 * u) = *(const uint4 *)&udesc[u];
+        else *(uint4 *)(rec + 16 + 16 * MAXU + 32 * u + 16 * (part - 1)) = *(const uint4 *)&gdesc[u][2 * (part - 1)];
+    }
+}
+// returns the number of units (the same for every thread); holds a barrier
+template <typename UD, int MAXU>
+__device__ __forceinline__ int plan_load(const uint8_t *plan, UD *udesc, uint2 (*gdesc)[4])
+{
+    const uint8_t *rec = plan + (size_t)blockIdx.x * plan_record_bytes(MAXU);
+    int nunits = __builtin_amdgcn_readfirstlane(*(const int *)rec);
+    nunits = nunits < 0 ? 0 : (nunits > MAXU ? MAXU : nunits);
+    for (int i = threadIdx.x; i < nunits * 3; i += blockDim.x) {
+        const int u = i / 3, part = i - 3 * u;
+        if (part == 0) *(uint4 *)&udesc[u] = *(const uint4 *)(rec + 16 + 16 * u);
+        else *(uint4 *)&gdesc[u][2 * (part - 1)] = *(const uint4 *)(rec + 16 + 16 * MAXU + 32 * u + 16 * (part - 1));
+    }
+    __syncthreads();
+    return nunits;
+}
+
 // ---- global memory straight into LDS ------------------------------------------------------------
 __device__ __forceinline__ uint32_t lds_addr32(const void *p)
 {

@@ -204,6 +204,39 @@ void paged_gqa_decode_attention_shared(AttentionWorkspace& ws, const __half* Q, 
         LOG_ERROR("Machina", "paged_gqa_decode_attention_shared: %s", drk_last_error());
 }
 
+size_t paged_decode_plan_bytes(int B, int max_seq_len, int max_phys_blocks, int block_size, int n_groups)
+{
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    return drk_decode_plan_bytes(&g, B, max_seq_len, n_groups);
+}
+
+bool paged_decode_plan_build(void* d_plan, size_t plan_bytes, const int* d_tables, int table_stride, const int* d_seq_lens,
+                             int B, int max_seq_len, const drk_prefix_group* groups, int n_groups, int max_phys_blocks,
+                             int block_size, hipStream_t stream)
+{
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    if (drk_decode_plan_build(&g, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups, n_groups, d_plan, plan_bytes,
+                              stream) != DRK_OK) {
+        LOG_ERROR("Machina", "paged_decode_plan_build: %s", drk_last_error());
+        return false;
+    }
+    return true;
+}
+
+void paged_gqa_decode_attention_planned(AttentionWorkspace& ws, const void* d_plan, const __half* Q, __half* kv_pool,
+                                        const int* d_tables, int table_stride, const int* d_seq_lens, int B, int max_seq_len,
+                                        const drk_prefix_group* groups, int n_groups, const __half* gate, int gate_stride,
+                                        __half* out, int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                        hipStream_t stream)
+{
+    if (B <= 0 || max_seq_len <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    if (drk_paged_decode_attention_planned(&g, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups, n_groups,
+                                           d_plan, out, fa_layer_idx, scale, ModelConfig::IO_DTYPE, gate, (size_t)gate_stride,
+                                           ws.ptr(), ws.bytes(), stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_gqa_decode_attention_planned: %s", drk_last_error());
+}
+
 bool paged_gqa_decode_grouped_supported(int block_size)
 {
     return ModelConfig::HEAD_DIM == 128 && block_size % 16 == 0 && ModelConfig::NUM_KV_HEADS > 0 &&

@@ -191,6 +191,20 @@ void paged_gqa_decode_attention_grouped(AttentionWorkspace& ws, const __half* Q,
                                         const drk_prefix_group* groups, int n_groups, const __half* gate,
                                         int gate_stride, __half* out, int fa_layer_idx, int max_phys_blocks,
                                         int block_size, float scale, hipStream_t stream = 0);
+// The layers of one decode step read the same tables and lengths: the decode kernels' unit descriptors can be built
+// once per step (paged_decode_plan_build, one small launch) and read by every layer's attention call
+// (paged_gqa_decode_attention_planned: the grouped call, or with n_groups = 0 the gated one; gate may be null).
+// The plan must come from the same tables, lengths, B, max_seq_len and groups.  paged_decode_plan_bytes is 0 where
+// the kernels take no plan (more than 64 branches, head dims other than 128 / 256).
+size_t paged_decode_plan_bytes(int B, int max_seq_len, int max_phys_blocks, int block_size, int n_groups);
+bool paged_decode_plan_build(void* d_plan, size_t plan_bytes, const int* d_tables, int table_stride, const int* d_seq_lens,
+                             int B, int max_seq_len, const drk_prefix_group* groups, int n_groups, int max_phys_blocks,
+                             int block_size, hipStream_t stream = 0);
+void paged_gqa_decode_attention_planned(AttentionWorkspace& ws, const void* d_plan, const __half* Q, __half* kv_pool,
+                                        const int* d_tables, int table_stride, const int* d_seq_lens, int B, int max_seq_len,
+                                        const drk_prefix_group* groups, int n_groups, const __half* gate, int gate_stride,
+                                        __half* out, int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                        hipStream_t stream = 0);
 void paged_gqa_decode_attention_gated_branches(AttentionWorkspace& ws, const __half* Q, __half* kv_pool,
                                                const int* d_tables, int table_stride, const int* d_seq_lens, int B,
                                                int max_seq_len, const __half* gate, int gate_stride, __half* out,

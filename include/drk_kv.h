@@ -268,6 +268,29 @@ int drk_paged_decode_attention_grouped(const drk_kv_layout *g, const void *q, co
                                        size_t gate_stride, void *workspace, size_t workspace_bytes,
                                        void *stream);
 
+/* The layers of one decode step read the same tables and lengths: the tiled decode kernels' per-workgroup
+ * unit descriptors (which 64-token tile of which branch and kv head, where its pages lie) can be built once
+ * per step instead of once per layer (no reference counterpart; the reference's kernel takes one workgroup per
+ * (head, branch) and needs none).  drk_decode_plan_build writes them to d_plan -- a launch of its own that reads
+ * d_tables and d_seq_lens only -- and drk_paged_decode_attention_planned is drk_paged_decode_attention_grouped
+ * (n_groups = 0: drk_paged_decode_attention_gated, gate may be NULL) reading them.  The caller promises that the
+ * plan was built with the same g (any layer), d_tables contents, d_seq_lens contents, B, max_seq_len and groups,
+ * and with the debug switches of drk_debug.h unchanged; the results are then bit for bit those of the unplanned
+ * call.  At most 64 branches, head_dim 128 or 256 with block_size % 16 == 0 (drk_decode_plan_bytes returns 0
+ * otherwise and both calls DRK_ERR_UNSUPPORTED).  drk_decode_plan_bytes: up to 12.6 MB; 16-byte aligned. */
+size_t drk_decode_plan_bytes(const drk_kv_layout *g, int B, int max_seq_len, int n_groups);
+int drk_decode_plan_build(const drk_kv_layout *g, const int32_t *d_tables, int table_stride,
+                          const int32_t *d_seq_lens, int B, int max_seq_len,
+                          const drk_prefix_group *groups, int n_groups, void *d_plan, size_t plan_bytes,
+                          void *stream);
+int drk_paged_decode_attention_planned(const drk_kv_layout *g, const void *q, const void *pool,
+                                       const int32_t *d_tables, int table_stride,
+                                       const int32_t *d_seq_lens, int B, int max_seq_len,
+                                       const drk_prefix_group *groups, int n_groups, const void *d_plan,
+                                       void *out, int layer, float scale, int io_dtype, const void *gate,
+                                       size_t gate_stride, void *workspace, size_t workspace_bytes,
+                                       void *stream);
+
 /* ---- paged causal prefill attention ------------------------------------ */
 /* paged_prefill_attention_kernel, paged_attention.cu:465-554, 621-630:
  * q/out [M, num_q_heads, head_dim]; row t attends to tokens 0..pos_start+t (the

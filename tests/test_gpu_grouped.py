@@ -209,3 +209,63 @@ def test_more_rows_than_one_group_takes_is_refused(dev):
     t.groups = [(0, 4, 0, 128)]
     ok, ma, _ = U.rel_abs_ok(U.from_bits(t.run_grouped(), t.io), t.want(), REL, ABS)
     assert ok, ma
+
+
+@pytest.mark.parametrize("dtype", [cabi.BF16, cabi.INT8])
+@pytest.mark.parametrize("tree,heads", [(TREE8, (8, 32, 128)), (ONE, (8, 32, 128)), (SPREAD, (1, 10, 128)), (([], TREE8[1]), (8, 32, 128)),
+                                        (([], SPREAD[1]), (4, 24, 256))])
+def test_unit_descriptors_built_once_for_the_layers_of_a_step(dev, dtype, tree, heads):
+    """drk_decode_plan_build + drk_paged_decode_attention_planned against the unplanned calls: the same bits, with
+    and without groups (no groups: the plain tiled kernel, also at head_dim 256), with the plan reused by a second
+    call and a gate."""
+    if heads[2] == 256:
+        dtype = cabi.F16 if dtype == cabi.BF16 else dtype
+    t = Tree(heads, dtype, tree[0], tree[1], seed=31, holes=() if tree[0] else ((1, 5),))     # a missing page where nothing is shared
+    lib = cabi.lib()
+    arr = cabi.prefix_groups(t.groups)
+    n_groups = len(t.groups)
+    mx = int(t.lens.max())
+    pb = lib.drk_decode_plan_bytes(C.byref(t.g), t.B, mx, n_groups)
+    assert pb > 0
+    plan = U.dev_bytes(np.full(pb, 0xEE, dtype=np.uint8))
+    cabi.call("drk_decode_plan_build", C.byref(t.g), U.p(t.dtab), t.stride, U.p(t.dl), t.B, mx, arr, n_groups, U.p(plan), pb,
+              U.stream_ptr())
+    wsb = lib.drk_decode_grouped_workspace_bytes(C.byref(t.g), t.B, mx, arr, n_groups)
+    rng = np.random.default_rng(5)
+    gate = U.normal_bits(rng, (t.B, t.QH, 2 * t.D), t.io)
+    dgate = U.dev_bytes(gate)
+    for use_gate in ((False, True, False) if t.D == 128 else (False, False)):
+        ws = U.dev_bytes(np.full(wsb, 0xFF, dtype=np.uint8))
+        outs = []
+        for planned in (True, False):
+            out = U.dev_bytes(np.full(t.B * t.QH * t.D * 2, 0x7B, dtype=np.uint8))
+            tail = (U.p(out), 0, float(t.scale), t.io, U.p(dgate) if use_gate else None, 2 * t.D if use_gate else 0, U.p(ws), wsb,
+                    U.stream_ptr())
+            if planned:
+                cabi.call("drk_paged_decode_attention_planned", C.byref(t.g), U.p(t.dq), U.p(t.dpool), U.p(t.dtab), t.stride,
+                          U.p(t.dl), t.B, mx, arr, n_groups, U.p(plan), *tail)
+            elif t.D == 128:
+                cabi.call("drk_paged_decode_attention_grouped", C.byref(t.g), U.p(t.dq), U.p(t.dpool), U.p(t.dtab), t.stride,
+                          U.p(t.dl), t.B, mx, arr, n_groups, *tail)
+            else:                                              # the grouped entry point is for head_dim 128
+                cabi.call("drk_paged_decode_attention_branches", C.byref(t.g), U.p(t.dq), U.p(t.dpool), U.p(t.dtab), t.stride,
+                          U.p(t.dl), t.B, mx, U.p(out), 0, float(t.scale), t.io, 0, U.p(ws), wsb, U.stream_ptr())
+            U.sync()
+            outs.append(U.host(out, np.uint16, (t.B, t.QH, t.D)))
+        assert np.array_equal(outs[0], outs[1]), "the planned call differs from the unplanned one"
+    got = U.from_bits(outs[0], t.io)
+    ok, ma, _ = U.rel_abs_ok(got, t.want())
+    assert ok, ma
+
+
+def test_plan_argument_errors(dev):
+    g = cabi.layout(1, 8, 32, 128, 16, 64, cabi.BF16)
+    lib = cabi.lib()
+    assert lib.drk_decode_plan_bytes(C.byref(g), 65, 1000, 0) == 0                 # more than 64 branches
+    g64 = cabi.layout(1, 4, 16, 64, 16, 64, cabi.F16)                              # a geometry of the portable kernel
+    assert lib.drk_decode_plan_bytes(C.byref(g64), 4, 1000, 0) == 0
+    x = U.dev_zeros(1 << 16)
+    rc = lib.drk_decode_plan_build(C.byref(g), U.p(x), 8, U.p(x), 4, 1000, None, 0, U.p(x), 64, U.stream_ptr())
+    assert rc == cabi.ERR_WORKSPACE
+    rc = lib.drk_decode_plan_build(C.byref(g64), U.p(x), 8, U.p(x), 4, 1000, None, 0, U.p(x), 1 << 16, U.stream_ptr())
+    assert rc == cabi.ERR_UNSUPPORTED
