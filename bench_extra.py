@@ -244,7 +244,7 @@ def config3(args):
         ensure_ns.append((time.perf_counter() - t) / B * 1e9)
         # pressure: free 25 % of the pool, oldest private pages first -- every 256 steps, as the configuration says,
         # and once in the middle of a timed region too short to reach step 256
-        if (s - W) % 256 == 255 or (K < 256 and s == W + K // 2):
+        if s >= W and ((s - W) % 256 == 255 or (K < 256 and s == W + K // 2)):
             t = time.perf_counter()
             before = cm.free_blocks()
             cm.ensure_free_blocks(NB // 4)
