@@ -626,16 +626,18 @@ def config7(args):
     M = 2048
     qc = (torch.randn(M, QH, D, device="cuda") * 0.5).to(h)
     oc = torch.empty_like(qc)
+    pwsb = lib.drk_prefill_workspace_bytes_max(C.byref(g), ctx, M)
+    pws = torch.empty(max(pwsb, 16), dtype=torch.uint8, device="cuda")
     prefill = {}
     for pos in (0, 3 * M, 15 * M):
         for _ in range(2):
             cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(pool), cabi.p(dtab), cabi.p(oc), 0, pos, M,
-                      float(scale), cabi.F16, None, 0, sp)
+                      float(scale), cabi.F16, cabi.p(pws), pwsb, sp)
         a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a0.record(stream)
         for _ in range(4):
             cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(pool), cabi.p(dtab), cabi.p(oc), 0, pos, M,
-                      float(scale), cabi.F16, None, 0, sp)
+                      float(scale), cabi.F16, cabi.p(pws), pwsb, sp)
         a1.record(stream)
         torch.cuda.synchronize()
         ms = a0.elapsed_time(a1) / 4
@@ -1056,6 +1058,8 @@ def kernel_fractions(buf, seed=11):
         "attention of 8 branches x 32768 tokens with the sigmoid gate (applied in the merge, not in this kernel)" % (NB7, L7))
     qc = (torch.randn(chunk, QH7, D7, device="cuda") * 0.5).to(h)
     oc = torch.empty_like(qc)
+    pwsb = lib.drk_prefill_workspace_bytes_max(C.byref(g), total, chunk)          # the pieces of the last round's walks
+    pws = torch.empty(max(pwsb, 16), dtype=torch.uint8, device="cuda")
     per_chunk = []
     for ps in range(2):
         per_chunk = []
@@ -1063,11 +1067,25 @@ def kernel_fractions(buf, seed=11):
             a0, a1 = ev(), ev()
             a0.record(stream)
             cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(buf), cabi.p(dtab), cabi.p(oc), c % L7, c * chunk, chunk,
-                      scale7, cabi.F16, None, 0, sp)
+                      scale7, cabi.F16, cabi.p(pws), pwsb, sp)
             a1.record(stream)
             torch.cuda.synchronize()
             per_chunk.append((a0.elapsed_time(a1), chunk_flops(c * chunk, chunk, QH7, D7)))
-    prefill_entry("config7_prefill_d256", "prefill_d256_kernel<f16>", per_chunk,
+    whole = []
+    lib.drk_debug_set_prefill_pieces(0)
+    for c in (0, total // chunk - 1):
+        for _ in range(2):
+            a0, a1 = ev(), ev()
+            a0.record(stream)
+            cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(buf), cabi.p(dtab), cabi.p(oc), 0, c * chunk, chunk,
+                      scale7, cabi.F16, cabi.p(pws), pwsb, sp)
+            a1.record(stream)
+            torch.cuda.synchronize()
+        whole.append(round(a0.elapsed_time(a1) * 1e3, 1))
+    lib.drk_debug_set_prefill_pieces(1)
+    prefill_entry("config7_prefill_d256", "prefill_d256_kernel<f16> + prefill_piece_merge_kernel", per_chunk,
                   "the reference's model shape: causal prefill of 32768 tokens in 16 chunks of 2048 over 256-token blocks, 24 Q / 4 KV "
-                  "heads x 256, fp16 (the pages hold N(0, 0.5), written beforehand)")
+                  "heads x 256, fp16 (the pages hold N(0, 0.5), written beforehand); 384 walks of 128 rows: 256 whole, the last 128 "
+                  "in two pieces each and a merge of their rows, timed together",
+                  {"first_and_last_chunk_us_with_whole_walks": whole})
     return res

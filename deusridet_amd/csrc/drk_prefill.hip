@@ -188,6 +188,10 @@ struct PrefillArgs {
     // optional: the row's log2-sum-exp of its scaled scores, [M][QH] (+inf for a row that saw no token).  Written
     // by the chunk kernels where a row's walk ends; read by the mass kernel, which then walks the keys once.
     float *lse_rows;
+    // prefill_d256_kernel only: a workgroup's 128 rows are 128 / gh query tokens x gh query heads (gh divides the
+    // heads per kv head); nqt row blocks of tokens; workgroups [0, n_full) take whole walks, the others one of
+    // kparts pieces of a walk each (tile ranges) and leave (o, m, l) per row and piece in part_o / part_m / part_l
+    int gh, nqt, n_full, kparts;
 };
 
 // scheduling hints: order instruction groups inside one basic block
@@ -1411,22 +1415,43 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
     __shared__ __align__(512) uint8_t v_ldsd[2][kTileBytes];
     __shared__ int valid_ldsd[4][4];                         // [tile & 3][wave]: the wave's 16-token run of the tile has a page
 
-    const int kvh = (int)blockIdx.x % A.KVH;
-    const int nqt = (int)gridDim.x / A.KVH;
-    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    // walk = (row block of tokens, kv head, group of gh query heads), the longest walks first; workgroups past
+    // n_full take one piece of a walk each
+    int walk = (int)blockIdx.x, part = 0, nparts = 1;
+    if (walk >= A.n_full) {
+        const int p = walk - A.n_full;
+        walk = A.n_full + p / A.kparts;
+        part = p - (p / A.kparts) * A.kparts;
+        nparts = A.kparts;
+    }
+    const int G = A.QH / A.KVH, GH = A.gh, TPW = A.tpw, NHG = G / GH;
+    const int kvh = walk % A.KVH;
+    const int hg = (walk / A.KVH) % NHG;
+    const int qt = A.nqt - 1 - walk / (A.KVH * NHG);
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
 
-    const int G = A.QH / A.KVH, TPW = A.tpw;
-    const int r = w * 32 + n, rt = r / G;
+    const int r = w * 32 + n, rt = r / GH;
     const int tq = qt * TPW + rt;
-    const int head = kvh * G + (r - rt * G);
+    const int head = kvh * G + hg * GH + (r - rt * GH);
     const bool row_live = rt < TPW && tq < A.M;
     const int vis = A.pos_start + tq + 1;
-    const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
+    const int lim_walk = A.pos_start + min((qt + 1) * TPW, A.M);
     const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
-    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+    const int nt_walk = (lim_walk + kPfBN - 1) / kPfBN;
+    // a piece is a range of tiles that begins at an even tile (the two score register sets and the LDS buffers
+    // take turns by the tile's parity); the last piece ends where the walk ends
+    // (the same value in every lane; the divisions run on the vector unit, and the LDS addresses derived from the
+    // tile number must be scalars)
+    const int t0 = __builtin_amdgcn_readfirstlane(part == 0 ? 0 : ((part * nt_walk / nparts) & ~1));
+    const int ntiles = __builtin_amdgcn_readfirstlane(part == nparts - 1 ? nt_walk : (((part + 1) * nt_walk / nparts) & ~1));
+    const int lim_wg = min(lim_walk, ntiles * kPfBN);        // nothing past the piece's end is requested
+    const size_t prow = nparts > 1 ? ((size_t)(walk - A.n_full) * 128 + r) * nparts + part : 0;   // the row's slot among the pieces
+    if (t0 >= ntiles) {                                      // an empty piece (a walk of fewer tiles than pieces)
+        if (row_live && g == 0) A.part_l[prow] = 0.0f;
+        return;
+    }
 
     // Q as the B operand, multiplied by scale * log2(e) on the way in (rounded once more to the 16-bit
     // type): the products then are the exponents themselves and the softmax needs no multiply per score.
@@ -1588,13 +1613,13 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
     }
     int blk_ahead;                                           // the wave's page two tiles ahead of the step
     {
-        const int b0 = page_of(0), b1 = page_of(1);
-        blk_ahead = page_of(2);
+        const int b0 = page_of(t0), b1 = page_of(t0 + 1);
+        blk_ahead = page_of(t0 + 2);
         __syncthreads();                                     // the clearing is done (and the table entries are here)
-        plan(0, b0);
+        plan(t0, b0);
 #pragma unroll
         for (int j = 0; j < 8; j++) dma_k(j);
-        plan(1, b1);                                         // K(1), V(0)
+        plan(t0 + 1, b1);                                    // K(t0 + 1), V(t0)
 #pragma unroll
         for (int j = 0; j < 8; j++) { dma_k(j); dma_v(j); }
         wait_loads();
@@ -1670,12 +1695,29 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
         l_run += psum;
         pv(it & 1, pb, [](int) {});
     };
-    for (int it = 0; it < ntiles; it += 2) {                 // two tiles per trip, the score registers swapping roles
+    for (int it = t0; it < ntiles; it += 2) {                // two tiles per trip, the score registers swapping roles
         tile_step(it, s_even, s_odd);
         if (it + 1 < ntiles) tile_step(it + 1, s_odd, s_even);
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (nparts > 1) {
+        // a piece of a walk: the unnormalised sums (register i of tile dt is d = dt*32 + 8*(i/4) + 4*g + i%4)
+        if (row_live) {
+            float *orow = A.part_o + prow * D;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int b4 = 0; b4 < 4; b4++)
+                    *(float4 *)(orow + dt * 32 + 8 * b4 + 4 * g) =
+                        make_float4(o[dt][4 * b4], o[dt][4 * b4 + 1], o[dt][4 * b4 + 2], o[dt][4 * b4 + 3]);
+            if (g == 0) {
+                A.part_m[prow] = m_ref;
+                A.part_l[prow] = l_tot;
+            }
+        }
+        return;
+    }
     if (A.lse_rows && row_live && g == 0)      // m_ref is the reference the weights were taken against, in log2 units
         A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_ref + __builtin_log2f(l_tot) : INFINITY;
     if (row_live && (l_tot > 0.0f || A.gate)) {
@@ -2313,6 +2355,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 // [0, pos_start + M) with the context split over the whole chip, and a small kernel folds each
 // row's pieces (and applies the gate).
 int g_prefill_two_phase = 1;                   // 0: never; 1: by the rule in prefill_impl; 2: whenever the geometry allows (tests); 3: as 2, with register staging also for 16-bit pages
+int g_prefill_pieces = 1;                      // head_dim 256, pieces for the walks of the last round: 0 never, 1 when they are worth it, 2 whenever there are any (tests)
 int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
 constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
 
@@ -2399,6 +2442,90 @@ __global__ __launch_bounds__(64) void prefill_merge_kernel(const float *__restri
     for (int x = 0; x < VEC; x++) dst[x] = vals[x];
 }
 
+// ---- head_dim 256: walks beyond a whole number of rounds are cut into pieces --------------------------
+// prefill_d256_kernel holds one workgroup per CU, so W walks of about equal length take ceil(W / 256) rounds
+// however few workgroups the last round has.  The walks of that last round (the shortest: they are dispatched
+// last) are cut into k = floor(256 / their number) pieces each, which still fit one round and take a k-th of
+// the time; their rows are then folded from the pieces by prefill_piece_merge_kernel.  gh query heads per
+// workgroup (the largest divisor of the heads per kv head that divides 128), so that no row of a workgroup idles.
+struct D256Shape { int gh, tpw, nqt, walks, n_full, tail, kparts; };
+static D256Shape d256_shape(const Lay &a, int pos_start, int M, int pieces)      // pieces: 0 none, 1 by the rule, 2 whenever a last round exists
+{
+    D256Shape s;
+    const int G = a.QH / a.KVH;
+    s.gh = 1;
+    for (int d = 1; d <= G && d <= 128; d++)
+        if (G % d == 0 && 128 % d == 0) s.gh = d;
+    s.tpw = 128 / s.gh;
+    s.nqt = (M + s.tpw - 1) / s.tpw;
+    s.walks = s.nqt * a.KVH * (G / s.gh);
+    s.tail = s.walks % 256;
+    s.kparts = (pieces && s.tail > 0) ? 256 / s.tail : 1;
+    if (s.kparts > 8) s.kparts = 8;
+    // a piece should be worth its start-up and the merge: eight tiles or more of the longest walk that is cut
+    // (the last round holds the shortest walks: the first row blocks of the chunk)
+    const int qt_tail = s.nqt - 1 - (s.walks - s.tail) / (a.KVH * (G / s.gh));
+    const int rows_to = (qt_tail + 1) * s.tpw < M ? (qt_tail + 1) * s.tpw : M;
+    const int tiles = (pos_start + rows_to + kPfBN - 1) / kPfBN;
+    if (pieces == 1 && s.kparts > tiles / 8) s.kparts = tiles / 8;
+    if (s.kparts < 2) { s.kparts = 1; s.tail = 0; }
+    s.n_full = s.walks - s.tail;
+    return s;
+}
+static size_t d256_pieces_need(const D256Shape &s) { return (size_t)s.tail * 128 * s.kparts * (256 + 2) * sizeof(float); }
+
+// grid = tail walks x 128 rows, block = 64: the row's pieces (at most 8) folded as in prefill_merge_kernel
+__global__ __launch_bounds__(64) void prefill_piece_merge_kernel(PrefillArgs A, int io_dtype)
+{
+    constexpr int D = 256, VEC = 4;
+    typedef float fvec __attribute__((ext_vector_type(VEC)));
+    const int walk = A.n_full + (int)blockIdx.x / 128, r = (int)blockIdx.x % 128;
+    const int lane = threadIdx.x, d = lane * VEC;
+    const int G = A.QH / A.KVH, GH = A.gh, NHG = G / GH;
+    const int kvh = walk % A.KVH, hg = (walk / A.KVH) % NHG, qt = A.nqt - 1 - walk / (A.KVH * NHG);
+    const int rt = r / GH, tq = qt * A.tpw + rt;
+    if (rt >= A.tpw || tq >= A.M) return;
+    const size_t row = (size_t)tq * A.QH + kvh * G + hg * GH + (r - rt * GH);
+    const size_t p0 = (size_t)blockIdx.x * A.kparts;
+    const float pl = lane < A.kparts ? A.part_l[p0 + lane] : 0.0f;
+    const float pm = (lane < A.kparts && pl > 0.0f) ? A.part_m[p0 + lane] : -INFINITY;
+    float M = pm;
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
+    const float w = pl > 0.0f ? __builtin_amdgcn_exp2f(pm - M) : 0.0f;
+    float L = pl * w;
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) L += __shfl_xor(L, off);
+    M = pm_lane(M, 0);
+    L = pm_lane(L, 0);
+    if (A.lse_rows && lane == 0) A.lse_rows[row] = L > 0.0f ? M + __builtin_log2f(L) : INFINITY;
+    fvec acc = {};
+    for (int j = 0; j < A.kparts; j++) {
+        const float wj = pm_lane(w, j);
+        if (wj != 0.0f) {                                    // an empty piece may hold anything
+            const fvec o = *(const fvec *)(A.part_o + (p0 + j) * D + d);
+#pragma unroll
+            for (int x = 0; x < VEC; x++) acc[x] = fmaf(o[x], wj, acc[x]);
+        }
+    }
+    uint16_t *dst = (uint16_t *)A.out + row * D + d;
+    uint16_t vals[VEC];
+    if (L > 0.0f) {
+#pragma unroll
+        for (int x = 0; x < VEC; x++) vals[x] = f_to_elem16(acc[x] / L, io_dtype);
+    } else {
+        if (!A.gate) return;
+#pragma unroll
+        for (int x = 0; x < VEC; x++) vals[x] = dst[x];
+    }
+    if (A.gate) {
+        const uint16_t *gp = A.gate + row * A.gate_stride + d;
+#pragma unroll
+        for (int x = 0; x < VEC; x++) vals[x] = gated_elem16(vals[x], gp[x], io_dtype);
+    }
+    *(uint2 *)dst = make_uint2((uint32_t)vals[0] | ((uint32_t)vals[1] << 16), (uint32_t)vals[2] | ((uint32_t)vals[3] << 16));
+}
+
 // context splits: two workgroups per CU over the whole grid -- one resident round -- of whole tiles each
 static void prefill_split_shape(const Lay &a, int pos_start, int M, int *chunk_tiles, int *nsplits)
 {
@@ -2424,6 +2551,13 @@ static bool prefill_split_applies(const Lay &a, int pos_start, int M)
     if (g_prefill_split == 0 || pos_start < kSplitMinPos) return false;
     if (g_prefill_split > 0) return M <= g_prefill_split;
     return M <= 512 || (M <= kSplitMaxM && pos_start >= 2 * kSplitMinPos);
+}
+
+// head_dim 256 on 16-bit pages takes prefill_d256_kernel (tiles straight into LDS)
+static bool d256_direct(const Lay &a)
+{
+    return a.D == 256 && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && a.bs >= 16 && ilog2_exact((unsigned)a.bs) >= 4 &&
+           g_prefill_two_phase != 0 && g_prefill_two_phase != 3;
 }
 
 static size_t prefill_split_need(const Lay &a, int pos_start, int M)
@@ -2463,6 +2597,7 @@ using namespace drk;
 extern "C" {
 
 void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
+void drk_debug_set_prefill_pieces(int mode) { g_prefill_pieces = mode < 0 ? 1 : (mode > 2 ? 2 : mode); }
 static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
                              int layer, int pos_start, int M, float scale, int io_dtype, const float *d_row_lse,
                              float *d_block_mass, int mass_len, int accumulate, void *stream)
@@ -2544,7 +2679,11 @@ size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M)
     if (make_lay(g, &a) != DRK_OK || M <= 0 || pos_start < 0) return 0;
     const bool mfma = !g_force_portable && (a.D == 128 || a.D == 256) && a.QH % a.KVH == 0 && a.QH / a.KVH <= 128 &&
                       (a.bs % 16) == 0;
-    if (mfma) return prefill_split_applies(a, pos_start, M) ? prefill_split_need(a, pos_start, M) : 0;
+    if (mfma) {
+        if (prefill_split_applies(a, pos_start, M)) return prefill_split_need(a, pos_start, M);
+        if (d256_direct(a) && g_prefill_pieces) return d256_pieces_need(d256_shape(a, pos_start, M, g_prefill_pieces));
+        return 0;
+    }
     return drk_decode_workspace_bytes(g, M, pos_start + M);
 }
 
@@ -2563,6 +2702,11 @@ size_t drk_prefill_workspace_bytes_max(const drk_kv_layout *g, int max_seq_len, 
     const int top = max_rows < widest ? max_rows : widest;
     for (int M = 1; M <= top; M++) {
         const size_t n = drk_prefill_workspace_bytes(g, max_seq_len - M, M);
+        if (n > need) need = n;
+    }
+    if (d256_direct(a) && g_prefill_pieces) {
+        // the pieces of the last round's walks: at most 256 pieces of 128 rows whatever the chunk's length
+        const size_t n = (size_t)256 * 128 * (256 + 2) * sizeof(float);
         if (n > need) need = n;
     }
     return need;
@@ -2651,11 +2795,25 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         }
     }
     // head_dim 256 on 16-bit pages: one wave per SIMD, tiles straight into LDS (same grid, same rows per workgroup)
-    if (a.D == 256 && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 && g_prefill_two_phase != 0 &&
-        g_prefill_two_phase != 3) {
-        if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_d256_kernel<DRK_BF16, DRK_BF16>), grid, dim3(256), 0, st, A);
-        else hipLaunchKernelGGL((prefill_d256_kernel<DRK_F16, DRK_F16>), grid, dim3(256), 0, st, A);
+    if (d256_direct(a)) {
+        // pieces for the walks of the last round when the caller brought the workspace for them
+        D256Shape sh = d256_shape(a, pos_start, M, g_prefill_pieces);
+        if (sh.kparts > 1 && (!workspace || ((uintptr_t)workspace % 16) || workspace_bytes < d256_pieces_need(sh)))
+            sh = d256_shape(a, pos_start, M, 0);
+        A.gh = sh.gh; A.tpw = sh.tpw; A.nqt = sh.nqt; A.n_full = sh.n_full; A.kparts = sh.kparts;
+        if (sh.kparts > 1) {
+            A.part_o = (float *)workspace;
+            A.part_m = A.part_o + (size_t)sh.tail * 128 * sh.kparts * 256;
+            A.part_l = A.part_m + (size_t)sh.tail * 128 * sh.kparts;
+        }
+        const dim3 gridp((unsigned)(sh.n_full + sh.tail * sh.kparts));
+        if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_d256_kernel<DRK_BF16, DRK_BF16>), gridp, dim3(256), 0, st, A);
+        else hipLaunchKernelGGL((prefill_d256_kernel<DRK_F16, DRK_F16>), gridp, dim3(256), 0, st, A);
         DRK_LAUNCH_CHECK("prefill_d256_kernel");
+        if (sh.kparts > 1) {
+            hipLaunchKernelGGL(prefill_piece_merge_kernel, dim3((unsigned)(sh.tail * 128)), dim3(64), 0, st, A, io_dtype);
+            DRK_LAUNCH_CHECK("prefill_piece_merge_kernel");
+        }
         return DRK_OK;
     }
 #define DRK_PF_LAUNCH(DT, KV, IO)                                                                                        \

@@ -47,6 +47,10 @@ void drk_debug_set_decode_lds_pad(int bytes);
 /* Tuning: which prefill chunks run with the context split over the chip (they must stand behind 2 048 tokens
  * or more): negative = the library's cost rule (default); 0 = none; n = every chunk of up to n rows. */
 void drk_debug_set_prefill_split(int max_rows);
+/* head_dim 256 chunk kernel: 0 = never cut the walks of the last round of workgroups into pieces (what it does
+ * without a workspace); 1 (default) = cut them when a piece is eight tiles or more and the workspace
+ * drk_prefill_workspace_bytes reports is passed; 2 = whenever a last round exists (tests). */
+void drk_debug_set_prefill_pieces(int mode);
 /* Tuning: which causal chunks of head_dim 128 run on the two-phase chunk kernels (eight waves, 256 rows per
  * workgroup): 0 = none (the four-wave kernel); 1 = the library's rule (default: chunks long enough to give
  * most CUs a workgroup); 2 = every chunk the geometry allows; 3 = as 2, and 16-bit pages too go through

@@ -294,6 +294,50 @@ def test_head_dim_256_over_holes_and_ragged_ends(dev, chunk_kernel, dtype, bs, G
     assert ok, f"max abs err {ma:.4g} ({chunk_kernel=} {bs=} {G=} {pos_start=} {M=} {holes=})"
 
 
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
+@pytest.mark.parametrize("bs,KVH,G,pos_start,M,holes", [
+    (256, 4, 6, 900, 257, (1,)), (16, 2, 2, 0, 300, (3, 4, 5, 6, 17)), (64, 2, 6, 1500, 100, (20,)), (32, 2, 1, 33, 130, ()),
+    (128, 1, 12, 2047, 22, (0,)), (16, 2, 6, 640, 64, (40, 43)), (16, 4, 6, 64, 2048, (7,)), (16, 3, 5, 3, 50, ())])
+def test_head_dim_256_walks_cut_into_pieces(dev, dtype, bs, KVH, G, pos_start, M, holes):
+    """The workgroups of the head_dim 256 kernel's last round take pieces of their walks (ranges of tiles) and a merge
+    folds them: forced here for every shape (2 to 8 pieces, walks shorter than their number of pieces, the reference
+    model's 24 / 4 heads on a full 2 048-row chunk: 384 walks, the last 128 in two pieces each), against fp64 and
+    against the same call with whole walks; rows behind holes only keep the caller's bytes."""
+    lib = cabi.lib()
+    D = 256
+    total = pos_start + M
+    nblk = (total + bs - 1) // bs
+    holes = tuple(h for h in holes if h < nblk)
+    geom = (2, KVH, KVH * G, D, bs, nblk + 3)
+    g, og, rng, table, opool = build(geom, dtype, total, seed=bs * 1000 + G + 11, holes=holes, mul=0.7)
+    q = U.normal_bits(rng, (M, KVH * G, D), dtype, 0.7)
+    scale = 1 / np.sqrt(D)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    try:
+        lib.drk_debug_set_prefill_two_phase(1)              # whatever the fixture chose: the kernel that loads tiles straight into LDS
+        lib.drk_debug_set_prefill_pieces(2)
+        assert lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M) > 0
+        got = run_prefill(g, dq, dpool, dtab, 1, pos_start, M, scale, dtype, KVH * G, D)
+        lib.drk_debug_set_prefill_pieces(0)
+        whole = run_prefill(g, dq, dpool, dtab, 1, pos_start, M, scale, dtype, KVH * G, D)
+    finally:
+        lib.drk_debug_set_prefill_pieces(1)
+    seen = np.array([any(table[t // bs] >= 0 for t in range(pos_start + r + 1)) for r in range(M)])
+    assert np.all(got[~seen].view(np.uint8) == 0x7B)
+    a, b = U.from_bits(got[seen], dtype), U.from_bits(whole[seen], dtype)
+    assert np.abs(a - b).max() <= 2e-2 * max(1.0, np.abs(b).max())
+    if M <= 300:
+        want = orc.prefill_f64(og, q, opool, table, 1, pos_start, scale, dtype)
+        ok, ma, _ = U.rel_abs_ok(a, want[seen])
+        assert ok, f"max abs err {ma:.4g}"
+    else:                                                   # the long chunk: a sample of rows against fp64
+        rows = np.array([0, 1, 63, 64, 1000, 1343, 1344, 2047])
+        for rsel in rows:
+            w1 = orc.decode_f64(og, q[rsel], opool, table, 1, pos_start + int(rsel) + 1, scale, dtype)
+            ok, ma, _ = U.rel_abs_ok(U.from_bits(got[rsel], dtype), w1)
+            assert ok, (int(rsel), ma)
+
+
 @pytest.mark.parametrize("geom,dtype,io", [((2, 8, 32, 128, 16, 300), cabi.BF16, cabi.BF16), ((2, 4, 24, 256, 256, 20), cabi.F16, cabi.F16),
                                            ((2, 2, 8, 128, 32, 150), cabi.INT8, cabi.BF16), ((2, 2, 12, 128, 16, 300), cabi.FP8_E4M3, cabi.F16)])
 @pytest.mark.parametrize("pos_start,M", [(2048, 1), (2049, 17), (3000, 64), (4095, 65), (2500, 130), (2048, 256)])
@@ -316,11 +360,13 @@ def test_short_chunks_behind_a_long_context(dev, geom, dtype, io, pos_start, M):
     ok, ma, _ = U.rel_abs_ok(got, want)
     assert ok, ma
     lib.drk_debug_set_prefill_split(0)
+    lib.drk_debug_set_prefill_pieces(0)                    # head_dim 256 would cut its walks into pieces otherwise
     try:
         assert lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M) == 0
         chunk = U.from_bits(run_prefill(g, dq, dpool, dtab, L - 1, pos_start, M, scale, io, QH, D), io)
     finally:
         lib.drk_debug_set_prefill_split(-1)
+        lib.drk_debug_set_prefill_pieces(1)
     assert np.max(np.abs(chunk - got)) <= 2e-2                      # two summation orders of the same sums
     ws = U.dev_zeros(wsb)
     out = U.dev_zeros(M * QH * D * 2)
