@@ -1410,7 +1410,7 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
     constexpr int kTileBytes = kPfBN * RB;                   // 32 KB per operand and tile
     constexpr int NKS = D / 16, NDT = D / 32;
     constexpr int ROWS = 16;                                 // tokens of a tile one wave requests
-    constexpr int XQ = 2, XP = 4;                            // operand reads ahead of their products: k-steps (QK), products (PV)
+    constexpr int XQ = 3, XP = 6;                            // operand reads ahead of their products: k-steps (QK), products (PV)
     __shared__ __align__(512) uint8_t k_ldsd[2][kTileBytes]; // 512: the xor swizzle is applied to whole addresses
     __shared__ __align__(512) uint8_t v_ldsd[2][kTileBytes];
     __shared__ int valid_ldsd[4][4];                         // [tile & 3][wave]: the wave's 16-token run of the tile has a page
