@@ -80,6 +80,8 @@ def parse():
                     help="storage type of the pages: config 4 int8 (default) | fp8; config 5 bf16 (default) | int8 | fp8")
     ap.add_argument("--no-graph", action="store_true", help="launch every kernel of a step from the host instead of "
                                                             "replaying one captured HIP graph per step")
+    ap.add_argument("--no-fused-append", action="store_true", help="launch the one-token append of every layer by itself instead of "
+                                                                   "letting the attention launch write the new rows")
     ap.add_argument("--no-plan", action="store_true", help="build the decode kernel's unit descriptors in every layer's launch "
                                                            "instead of once per step (drk_decode_plan_build)")
     ap.add_argument("--no-cascade", action="store_true", help="config 3: read the shared prefix once per branch")
@@ -193,14 +195,26 @@ def main():
                       cabi.p(pool), cabi.p(dtab), stride, dlen, B, max_ctx, C.c_void_p(out.data_ptr() + l * qrow), l,
                       float(scale), cabi.BF16, split, cabi.p(ws), wsb, spx)
 
+    fused_append = bool(plan_bytes) and not args.no_fused_append
+
+    def layer_step(l, dpos, dlen, spx):
+        """append one token per branch, then attend: one call (one launch for these bf16 pages) or two"""
+        if fused_append:
+            cabi.call("drk_kv_append_decode_planned", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dlen, B, max_ctx, None, 0,
+                      cabi.p(plan), C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16,
+                      C.c_void_p(q.data_ptr() + l * qrow), C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.BF16,
+                      None, 0, cabi.p(ws), wsb, spx)
+        else:
+            cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos, B, l, 1,
+                      C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, spx)
+            attend(l, dlen, spx)
+
     def step(s):
         dpos = C.c_void_p(pos_steps[s].data_ptr())
         dlen = C.c_void_p(len_steps[s].data_ptr())
         build_plan(dlen, sp)
         for l in range(L):
-            cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos, B, l, 1,
-                      C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, sp)
-            attend(l, dlen, sp)
+            layer_step(l, dpos, dlen, sp)
 
     use_graph = not args.no_graph
     if use_graph:
@@ -213,9 +227,7 @@ def main():
             gsp = C.c_void_p(torch.cuda.current_stream().cuda_stream)
             build_plan(dlen, gsp)
             for l in range(L):
-                cabi.call("drk_kv_append_branches", C.byref(g), cabi.p(pool), cabi.p(dtab), stride, dpos, B, l, 1,
-                          C.c_void_p(newk.data_ptr() + l * krow), C.c_void_p(newv.data_ptr() + l * krow), cabi.BF16, gsp)
-                attend(l, dlen, gsp)
+                layer_step(l, dpos, dlen, gsp)
             pos_cur.add_(1)
             len_cur.add_(1)
 
@@ -579,6 +591,7 @@ def main():
             "branches": B, "layers": L, "ctx_final": [int(x) for x in final],
             "launch": "one captured HIP graph per step" if use_graph else "host launches",
             "unit_descriptors": "built once per step" if plan_bytes else "built by every launch",
+            "append": "written by the attention launch" if fused_append else "a launch of its own",
         },
         "hbm_frac_step": round(value_gbps / HBM_PEAK_GBPS, 4),
         "us_per_step": round(ms_per_step * 1e3, 1),

@@ -138,6 +138,8 @@ SIGNATURES = {
     "drk_decode_plan_build": (_i32, [_LP, _vp, _i32, _vp, _i32, _i32, _GP, _i32, _vp, _sz, _vp]),
     "drk_paged_decode_attention_planned": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _GP, _i32, _vp, _vp, _i32, _f32,
                                                   _i32, _vp, _sz, _vp, _sz, _vp]),
+    "drk_kv_append_decode_planned": (_i32, [_LP, _vp, _vp, _i32, _vp, _i32, _i32, _GP, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _i32,
+                                            _f32, _i32, _vp, _sz, _vp, _sz, _vp]),
     "drk_debug_set_grouped_decode": (None, [_i32]),
     "drk_prefill_workspace_bytes": (_sz, [_LP, _i32, _i32]),
     "drk_paged_prefill_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),

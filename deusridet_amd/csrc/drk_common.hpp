@@ -62,6 +62,9 @@ inline int ilog2_exact(unsigned v)                 // -1 when v is not a power o
 struct DecodePlan {
     uint8_t *ptr = nullptr;
     int mode = 0;
+    // optional (plain tiled kernel, 16-bit pages): the step's new token of every branch, [B][KVH][D] in the pages'
+    // own type, written at position seq_len - 1 by the workgroup that owns the branch's last tile before it reads it
+    const uint8_t *new_k = nullptr, *new_v = nullptr;
 };
 constexpr size_t plan_record_bytes(int max_units) { return 16 + 48 * (size_t)max_units; }
 size_t decode_plan_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups);
@@ -72,6 +75,10 @@ int launch_decode(const drk_kv_layout *g, const void *q, const void *pool, const
                   int max_seq_len, void *out, int layer, float scale, int io_dtype, int split_tokens,
                   void *workspace, size_t workspace_bytes, void *stream, const void *gate = nullptr,
                   size_t gate_stride = 0, DecodePlan plan = {});
+// bulk / per-branch append (drk_pages.hip); branch mode (d_pos != NULL) writes at d_pos[i] + pos_start
+int launch_append(const drk_kv_layout *g, void *pool, const int32_t *tables, int table_stride, const int32_t *d_pos,
+                  int pos_start, int ntokens, int layer, int layer_count, const void *src_k, const void *src_v,
+                  int src_dtype, void *stream);
 // out[row][d] *= sigmoid(gate[row * gate_stride + d]), rows of D elements (drk_layer.hip)
 int launch_sigmoid_gate(const void *x, const void *gate, void *out, size_t rows, int D, size_t gate_stride_elems,
                         int dtype, hipStream_t st);

@@ -737,6 +737,38 @@ int drk_paged_decode_attention_planned(const drk_kv_layout *g, const void *q, co
                          workspace, workspace_bytes, stream, gate, gate_stride, plan);
 }
 
+int drk_kv_append_decode_planned(const drk_kv_layout *g, void *pool, const int32_t *d_tables, int table_stride,
+                                 const int32_t *d_seq_lens, int B, int max_seq_len, const drk_prefix_group *groups,
+                                 int n_groups, const void *d_plan, const void *new_k, const void *new_v, int src_dtype,
+                                 const void *q, void *out, int layer, float scale, int io_dtype, const void *gate,
+                                 size_t gate_stride, void *workspace, size_t workspace_bytes, void *stream)
+{
+    Lay a;
+    int rc = make_lay(g, &a);
+    if (rc) return rc;
+    if (!d_plan || !new_k || !new_v || !d_seq_lens || !pool) return fail(DRK_ERR_INVALID, "append_decode: NULL pointer");
+    if (decode_plan_need(a, B, max_seq_len, groups, n_groups) == 0)
+        return fail(DRK_ERR_UNSUPPORTED, "append_decode: this geometry or number of branches takes no plan");
+    DecodePlan plan;
+    plan.ptr = (uint8_t *)const_cast<void *>(d_plan);
+    plan.mode = 2;
+    const bool grouped = n_groups > 0 && grouped_decode_supported(a, B);
+    // the plain tiled kernel writes the new rows itself when they are in the pages' own 16-bit type; otherwise the
+    // append is a launch of its own, at position length - 1
+    const bool fused = !grouped && a.E == 2 && src_dtype == a.dtype;
+    if (fused) {
+        plan.new_k = (const uint8_t *)new_k;
+        plan.new_v = (const uint8_t *)new_v;
+    } else if ((rc = launch_append(g, pool, d_tables, table_stride, d_seq_lens, -1, B, layer, 1, new_k, new_v, src_dtype, stream))) {
+        return rc;
+    }
+    if (grouped)
+        return launch_decode_grouped(g, q, pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, groups, n_groups, out, layer,
+                                     scale, io_dtype, workspace, workspace_bytes, stream, gate, gate_stride, plan);
+    return launch_decode(g, q, pool, d_tables, table_stride, d_seq_lens, 0, -1, B, max_seq_len, out, layer, scale, io_dtype, 0,
+                         workspace, workspace_bytes, stream, gate, gate_stride, plan);
+}
+
 size_t drk_decode_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len)
 {
     Lay a;

@@ -57,6 +57,9 @@ struct StreamArgs {
     int stop_after_descriptors;     // measurement aid: leave once the workgroup's unit descriptors are built
     uint8_t *plan;                  // the descriptors of every workgroup in global memory, see DecodePlan
     int plan_mode;                  // 0: build and use; 1: build, store, leave; 2: read
+    const uint8_t *new_k, *new_v;   // or NULL: one new token per branch, [B][KVH][D] of the pages' 16-bit type, to be
+                                    // written at position seq_len - 1 before the tile that holds it is read
+    uint8_t *pool_layer_w;          // the layer's pages, writable (with new_k)
 };
 
 constexpr int kMaxUnits = kStreamMaxUnits;    // units one workgroup may own (descriptor table in LDS)
@@ -150,6 +153,29 @@ __global__ __launch_bounds__(256, D == 128 ? 4 : 2) void decode_stream_kernel(St
         }
     }
     if (nunits == 0) return;
+    if (A.new_k) {
+        // The step's append, folded in: the unit that is a (branch, kv head)'s last tile holds the new token's
+        // position, and only this workgroup reads that tile -- so it writes the row itself, K and V, 16 bytes per
+        // thread, before its first request.  The barrier below orders the stores before the loads of every wave of
+        // the workgroup (one CU, one vector cache in front of the L2 the stores went to).  A missing page is
+        // skipped, as the append kernel skips it.
+        if constexpr (!KvTraits<DT>::q8) {
+            constexpr int CH = D * 2 / 16;                       // 16-byte chunks per row
+            for (int i = threadIdx.x; i < nunits * 2 * CH; i += 256) {
+                const int ui = i / (2 * CH), rest = i - ui * (2 * CH), kv = rest / CH, ch = rest - kv * CH;
+                const UnitDesc ud = udesc[ui];
+                if (ud.tile_lim < 1 || ud.tile_lim > kSTile) continue;           // not the last tile of its run
+                const int r = ud.tile_lim - 1;
+                const uint32_t gx = gdesc[ui][r >> 4].x;
+                if (gx == kNone) continue;
+                const int b = ud.bq / A.QH, kvh = (ud.bq - b * A.QH) / GQ;
+                const uint8_t *src = (kv ? A.new_v : A.new_k) + ((size_t)(b * A.KVH + kvh) * D * 2) + ch * 16;
+                uint8_t *dst = A.pool_layer_w + ((size_t)gx << 4) + (size_t)(r & 15) * A.row_bytes + (kv ? A.kv_plane : 0) + ch * 16;
+                *(uint4 *)dst = *(const uint4 *)src;
+            }
+        }
+        __syncthreads();
+    }
     if (A.stop_after_descriptors) return;
 
     uint8_t *const klds = &k_lds[w][0];
@@ -620,6 +646,10 @@ int launch_decode_stream(const Lay &a, const void *q, const void *pool, const in
         A.lse_groups = lse_groups; A.lse_stride = lse_stride;
         A.stop_after_descriptors = g_stream_stop_after_descriptors;
         A.plan = plan.ptr; A.plan_mode = plan.ptr ? plan.mode : 0;
+        const bool fused_append = plan.new_k && plan.new_v && a.E == 2 && start_tile == 0 && plan.mode != 1;
+        A.new_k = fused_append ? plan.new_k : nullptr;
+        A.new_v = fused_append ? plan.new_v : nullptr;
+        A.pool_layer_w = (uint8_t *)const_cast<void *>(pool) + (size_t)layer * a.layer_stride;
 #define DRK_STREAM_LAUNCH(DT)                                                                                           \
     do {                                                                                                                \
         const bool g4 = a.QH / a.KVH <= 4;                                                                              \

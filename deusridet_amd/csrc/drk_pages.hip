@@ -99,7 +99,8 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(
 // grid = (token groups, layer_count, 2); source [layer][token][head][dim] of
 // 16-bit elements, one 16-byte chunk (8 elements) per thread.
 // "token" i is position pos_start+i of one table (batch mode, d_pos == NULL) or
-// the single new token of branch i at d_pos[i] with table row i (branch mode).
+// the single new token of branch i at d_pos[i] + pos_start with table row i (branch mode; pos_start is 0 there,
+// or -1 when the array holds lengths that already count the token).
 // QMODE 0: copy.  1: int8 codes + fp16 scale per row.  2: fp8 e4m3 codes.
 // ------------------------------------------------------------------------
 template <int QMODE>
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(kThreads) void append_kernel(
                 unsigned h = dv(r, row_div);
                 cc[u] = r - h * rc;
                 int ti = t0 + (int)t;
-                int pos = d_pos ? d_pos[ti] : pos_start + ti;
+                int pos = d_pos ? d_pos[ti] + pos_start : pos_start + ti;
                 const int32_t *tab = tables + (size_t)(d_pos ? ti : 0) * table_stride;
                 if (pos >= 0) {
                     unsigned lb = dv((unsigned)pos, bs_div);
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(kThreads) void append_quant_kernel(
                 const unsigned t = dv(ci, tok_div), r = ci - t * tok_div.d;
                 const unsigned h = dv(r, row_div), c2 = r - h * rc2;
                 const int ti = t0 + (int)t;
-                const int pos = d_pos ? d_pos[ti] : pos_start + ti;
+                const int pos = d_pos ? d_pos[ti] + pos_start : pos_start + ti;
                 const int32_t *tab = tables + (size_t)(d_pos ? ti : 0) * table_stride;
                 if (pos >= 0) {
                     const unsigned lb = dv((unsigned)pos, bs_div);
@@ -322,9 +323,9 @@ static int check_src_dtype(int d)
     return DRK_OK;
 }
 
-static int launch_append(const drk_kv_layout *g, void *pool, const int32_t *tables, int table_stride,
-                         const int32_t *d_pos, int pos_start, int ntokens, int layer, int layer_count,
-                         const void *src_k, const void *src_v, int src_dtype, void *stream)
+int launch_append(const drk_kv_layout *g, void *pool, const int32_t *tables, int table_stride,
+                  const int32_t *d_pos, int pos_start, int ntokens, int layer, int layer_count,
+                  const void *src_k, const void *src_v, int src_dtype, void *stream)
 {
     Lay a;
     int rc = make_lay(g, &a);
@@ -334,7 +335,8 @@ static int launch_append(const drk_kv_layout *g, void *pool, const int32_t *tabl
     if (layer < 0 || layer_count < 1 || layer + layer_count > a.L)
         return fail(DRK_ERR_INVALID, "append: layers [%d,%d) outside [0,%d)", layer, layer + layer_count, a.L);
     if (layer_count > 65535) return fail(DRK_ERR_INVALID, "append: layer_count > 65535");
-    if (ntokens < 0 || pos_start < 0) return fail(DRK_ERR_INVALID, "append: negative token count or position");
+    if (ntokens < 0 || (pos_start < 0 && !(d_pos && pos_start == -1)))
+        return fail(DRK_ERR_INVALID, "append: negative token count or position");
     if (ntokens == 0) return DRK_OK;
     if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && src_dtype != a.dtype)
         return fail(DRK_ERR_INVALID, "append: src_dtype %d differs from the pool's %d", src_dtype, a.dtype);

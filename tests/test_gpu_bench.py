@@ -15,7 +15,8 @@ KEYS = {"metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "
         "dtype", "data", "config", "roofline", "cpu_baseline"}
 
 
-@pytest.mark.parametrize("extra", [[], ["--ctx-mode", "uniform", "--no-other-configs"], ["--config", "3"], ["--config", "3", "--forks", "prefix"],
+@pytest.mark.parametrize("extra", [[], ["--ctx-mode", "uniform", "--no-other-configs"], ["--no-plan", "--no-other-configs"],
+                                   ["--no-fused-append", "--no-graph", "--no-other-configs"], ["--config", "3"], ["--config", "3", "--forks", "prefix"],
                                    ["--config", "3", "--shared-kernel", "pair"], ["--config", "4"], ["--config", "4", "--kv-dtype", "fp8"],
                                    ["--config", "5"], ["--config", "5", "--kv-dtype", "int8"], ["--config", "6"], ["--config", "7"]],
                          ids=lambda e: "-".join(x.strip("-") for x in e) or "default")

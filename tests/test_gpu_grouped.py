@@ -269,3 +269,48 @@ def test_plan_argument_errors(dev):
     assert rc == cabi.ERR_WORKSPACE
     rc = lib.drk_decode_plan_build(C.byref(g64), U.p(x), 8, U.p(x), 4, 1000, None, 0, U.p(x), 1 << 16, U.stream_ptr())
     assert rc == cabi.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("dtype,heads,tree", [(cabi.BF16, (8, 32, 128), ([], TREE8[1])), (cabi.F16, (4, 24, 256), ([], SPREAD[1])),
+                                              (cabi.INT8, (8, 32, 128), ([], TREE8[1])), (cabi.BF16, (8, 32, 128), TREE8),
+                                              (cabi.F16, (2, 16, 128), ([], [1, 64, 65, 128, 1000]))])
+def test_append_and_attention_of_a_layer_in_one_call(dev, dtype, heads, tree):
+    """drk_kv_append_decode_planned against drk_kv_append_branches + drk_paged_decode_attention_planned: the same bytes
+    in the pool and the same output bits -- in one launch for 16-bit pages without groups (the workgroup that owns a
+    branch's last tile writes the new rows), in two otherwise; a branch whose last page is missing keeps it missing."""
+    import torch
+    holes = () if tree[0] else ((1, (int(tree[1][1]) - 1) // 16),)
+    t = Tree(heads, dtype, tree[0], tree[1], seed=47, holes=holes)
+    lib = cabi.lib()
+    arr = cabi.prefix_groups(t.groups)
+    n_groups = len(t.groups)
+    mx = int(t.lens.max())
+    KVH = heads[0]
+    pb = lib.drk_decode_plan_bytes(C.byref(t.g), t.B, mx, n_groups)
+    plan = U.dev_zeros(pb)
+    cabi.call("drk_decode_plan_build", C.byref(t.g), U.p(t.dtab), t.stride, U.p(t.dl), t.B, mx, arr, n_groups, U.p(plan), pb,
+              U.stream_ptr())
+    wsb = lib.drk_decode_grouped_workspace_bytes(C.byref(t.g), t.B, mx, arr, n_groups)
+    rng = np.random.default_rng(9)
+    nk, nv = U.normal_bits(rng, (t.B, KVH, t.D), t.io, 0.7), U.normal_bits(rng, (t.B, KVH, t.D), t.io, 0.7)
+    dnk, dnv = U.dev_bytes(nk), U.dev_bytes(nv)
+    dpos = U.dev_i32(t.lens - 1)
+    results = []
+    for fused in (False, True):
+        pool = U.dev_bytes(t.opool)
+        ws = U.dev_bytes(np.full(wsb, 0xFF, dtype=np.uint8))
+        out = U.dev_bytes(np.full(t.B * t.QH * t.D * 2, 0x7B, dtype=np.uint8))
+        if fused:
+            cabi.call("drk_kv_append_decode_planned", C.byref(t.g), U.p(pool), U.p(t.dtab), t.stride, U.p(t.dl), t.B, mx, arr,
+                      n_groups, U.p(plan), U.p(dnk), U.p(dnv), t.io, U.p(t.dq), U.p(out), 0, float(t.scale), t.io, None, 0,
+                      U.p(ws), wsb, U.stream_ptr())
+        else:
+            cabi.call("drk_kv_append_branches", C.byref(t.g), U.p(pool), U.p(t.dtab), t.stride, U.p(dpos), t.B, 0, 1, U.p(dnk),
+                      U.p(dnv), t.io, U.stream_ptr())
+            cabi.call("drk_paged_decode_attention_planned", C.byref(t.g), U.p(t.dq), U.p(pool), U.p(t.dtab), t.stride, U.p(t.dl),
+                      t.B, mx, arr, n_groups, U.p(plan), U.p(out), 0, float(t.scale), t.io, None, 0, U.p(ws), wsb, U.stream_ptr())
+        U.sync()
+        results.append((U.host(out, np.uint16, (t.B, t.QH, t.D)).copy(), U.host(pool, np.uint8).copy()))
+    assert np.array_equal(results[0][1], results[1][1]), "the pools differ"
+    assert not np.array_equal(results[0][1], t.opool), "nothing was appended"
+    assert np.array_equal(results[0][0], results[1][0]), "the outputs differ"
