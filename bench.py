@@ -91,6 +91,9 @@ def parse():
     ap.add_argument("--shared-kernel", choices=["auto", "pair"], default="auto",
                     help="config 3: how shared pages are read: auto = one launch over shared and private tiles where the "
                          "geometry allows; pair = always the prefix pass followed by the tail kernel")
+    ap.add_argument("--d256-waves", type=int, choices=[0, 1], default=None,
+                    help="head_dim 256 chunk kernel: 0 = four waves that do both products, 1 = score waves and value waves "
+                         "(default: the library's choice)")
     return ap.parse_args()
 
 
@@ -109,6 +112,8 @@ def main():
     gc.collect()
     gc.disable()
     cabi.lib().drk_debug_set_grouped_decode(1 if args.shared_kernel == "pair" else 0)
+    if args.d256_waves is not None:
+        cabi.lib().drk_debug_set_prefill_d256_waves(args.d256_waves)
     if args.config != 2:
         import bench_extra
         print(json.dumps(bench_extra.run(args)))

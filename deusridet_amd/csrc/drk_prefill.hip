@@ -1745,6 +1745,389 @@ __global__ __launch_bounds__(256, 1) void prefill_d256_kernel(PrefillArgs A)
     }
 }
 
+// ---- head_dim 256, 16-bit pages: two kinds of waves, two per SIMD ------------------------------------
+// prefill_d256_kernel holds one wave per SIMD because a wave's 32 rows x 256 dims of output are 128 accumulator
+// registers, beside its 64 of Q and 64 of scores: nothing overlaps that wave's LDS latency, its softmax and the issue
+// time of its requests.  Here the two products of a row group belong to two waves of the same SIMD:
+//   wave w (0-3), the SCORE wave of row group w: Q in registers, S^T = K Q^T for tile t + 1 with the exponentials of
+//     tile t between the k-steps, mask, lazy maximum, row sums; it hands the tile's weights P (16 registers per lane,
+//     already in the layout of the second product's B operand) and, when the reference moved, the rows' factors to
+//     its partner through LDS;
+//   wave w + 4, the VALUE wave of row group w: the 128 accumulators, O^T += V^T P^T.
+// Neither holds more than 256 registers, so both fit a SIMD, and each one's stalls are the other's issue slots.
+// The score waves request K (their 16-token run of every tile, two tiles ahead), the value waves V (one tile ahead).
+// Two barriers per tile, A and B, passed by all eight waves:
+//   score wave, step t:  mask / maximum of tile t;  wait for its K requests;  A_t;  scores of tile t + 1 with the
+//                        exponentials of tile t and the requests for K(t + 2) between the k-steps;  write P(t);  B_t.
+//   value wave, step t:  (B_t passed: P(t) and V(t) are in LDS)  read P(t);  the first products of PV(t);  A_{t+1};
+//                        the other products with the requests for V(t + 1) between them;  wait for those;  B_{t+1}.
+// P has one buffer: the value wave reads P(t) ahead of A_{t+1}, the score wave writes P(t + 1) behind it.  K(t + 2)
+// is requested behind A_t into the buffer of K(t), which the scores of tile t read ahead of B_{t-1}; V(t + 1) behind
+// B_t into the buffer of V(t - 1), which PV(t - 1) read ahead of B_t.  Same walks, pieces, gate and row log-sum-exp
+// as prefill_d256_kernel, and the same arithmetic in the same order: the two give the same bits.
+// What it gains is overlap, not fewer clocks of work: a tile takes 3 900 clocks against 5 100, with the matrix pipe
+// busy 57 % of them; the part then runs at 1.8 GHz instead of 2.4.  Variants that take fewer clocks per tile (all
+// requests from the score waves, K from the value waves and V from the score waves, requests earlier in the step)
+// ran at lower clocks still and took as long or longer; without the tile requests (wrong results, a probe) the same
+// schedule takes two thirds of the time.
+template <int DT, int IO = DT>
+__global__ __launch_bounds__(512, 1) void prefill_d256w_kernel(PrefillArgs A)
+{
+    constexpr int D = 256, RB = D * 2;
+    constexpr int kTileBytes = kPfBN * RB;                   // 32 KB per operand and tile
+    constexpr int NKS = D / 16, NDT = D / 32;
+    constexpr int ROWS = 16;
+    constexpr int XQ = 3, XP = 6;
+    constexpr int kFirst = 4;                                // products of PV(t) ahead of barrier A
+    __shared__ __align__(512) uint8_t k_ldsw[2][kTileBytes];
+    __shared__ __align__(512) uint8_t v_ldsw[2][kTileBytes];
+    __shared__ __align__(16) uint4 p_ldsw[4][4][64];         // [row group][register quad][lane]: the tile's weights
+    __shared__ float alpha_ldsw[4][64], l_ldsw[4][64];
+    __shared__ int moved_ldsw[4];
+    __shared__ int valid_ldsw[4][4];                         // [tile & 3][run]: the 16-token run of the tile has a page
+
+    int walk = (int)blockIdx.x, part = 0, nparts = 1;
+    if (walk >= A.n_full) {
+        const int p = walk - A.n_full;
+        walk = A.n_full + p / A.kparts;
+        part = p - (p / A.kparts) * A.kparts;
+        nparts = A.kparts;
+    }
+    const int G = A.QH / A.KVH, GH = A.gh, TPW = A.tpw, NHG = G / GH;
+    const int kvh = walk % A.KVH;
+    const int hg = (walk / A.KVH) % NHG;
+    const int qt = A.nqt - 1 - walk / (A.KVH * NHG);
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const bool value_wave = wave >= 4;
+    const int w = wave & 3;                                  // row group, and the 16-token run this wave requests
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, g = lane >> 5;
+
+    const int r = w * 32 + n, rt = r / GH;
+    const int tq = qt * TPW + rt;
+    const int head = kvh * G + hg * GH + (r - rt * GH);
+    const bool row_live = rt < TPW && tq < A.M;
+    const int vis = A.pos_start + tq + 1;
+    const int lim_walk = A.pos_start + min((qt + 1) * TPW, A.M);
+    const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
+    const int nt_walk = (lim_walk + kPfBN - 1) / kPfBN;
+    const int t0 = __builtin_amdgcn_readfirstlane(part == 0 ? 0 : ((part * nt_walk / nparts) & ~1));
+    const int ntiles = __builtin_amdgcn_readfirstlane(part == nparts - 1 ? nt_walk : (((part + 1) * nt_walk / nparts) & ~1));
+    const int lim_wg = min(lim_walk, ntiles * kPfBN);
+    const size_t prow = nparts > 1 ? ((size_t)(walk - A.n_full) * 128 + r) * nparts + part : 0;
+    if (t0 >= ntiles) {
+        if (!value_wave && row_live && g == 0) A.part_l[prow] = 0.0f;
+        return;
+    }
+
+    const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+    const int sh = A.bs_shift;
+    const int tgw = w * ROWS;
+    auto wait_loads = [&]() { __builtin_amdgcn_s_waitcnt(0x0f70); };         // vmcnt(0)
+    typedef const int32_t __attribute__((address_space(4))) *const_table_t;
+    const const_table_t table_k = (const_table_t)(uintptr_t)A.table;
+    auto page_of = [&](int tile) -> int {
+        const int tg = tile * kPfBN + tgw;
+        return tg < lim_wg ? table_k[tg >> sh] : -1;
+    };
+    // where the wave's run of tile kt comes from, how many of its rows exist
+    const uint8_t *p_src = kbase;
+    int p_rows = 0;
+    uint32_t p_lds = 0;
+    const uint32_t k_ring = pf_lds_addr(&k_ldsw[0][0]) + (uint32_t)(tgw * RB);
+    const uint32_t v_ring = pf_lds_addr(&v_ldsw[0][0]) + (uint32_t)(tgw * RB);
+    auto plan = [&](int kt, int blk_raw) {
+        const int blk0 = __builtin_amdgcn_readfirstlane(blk_raw);
+        const int tg = kt * kPfBN + tgw;
+        const bool ok = blk0 >= 0 && blk0 < A.NB && tg < lim_wg;
+        p_rows = ok ? lim_wg - tg : 0;
+        p_src = kbase + (size_t)(ok ? blk0 : 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB) + (value_wave ? A.kv_plane : 0);
+        p_lds = (value_wave ? v_ring : k_ring) + ((uint32_t)(kt & 1) << 15);
+        if (!value_wave && lane == 0) valid_ldsw[kt & 3][w] = ok ? 1 : 0;
+    };
+    // request j of 8: two token rows (1 KB); K chunk c of row r at c ^ (r & 15), V at c ^ ((r & 3) << 2)
+    uint32_t goff[8];
+    {
+        const int rr = lane >> 5, cp = lane & 31;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            goff[j] = value_wave ? (uint32_t)(rr * RB + ((cp ^ (((2 * j + rr) & 3) << 2)) << 4))
+                                 : (uint32_t)(rr * RB + ((cp ^ ((2 * j + rr) & 15)) << 4));
+    }
+    auto dma = [&](int j) {
+        if (__builtin_expect(p_rows >= ROWS, 1)) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
+        else if (2 * j + (lane >> 5) < p_rows) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
+    };
+
+    // ---- prologue: the buffers cleared; K(t0), K(t0 + 1), V(t0) in LDS ----
+    for (int i = threadIdx.x * 16; i < 2 * kTileBytes; i += 512 * 16) {
+        *(uint4 *)(&k_ldsw[0][0] + i) = make_uint4(0, 0, 0, 0);
+        *(uint4 *)(&v_ldsw[0][0] + i) = make_uint4(0, 0, 0, 0);
+    }
+    int blk_ahead;
+    {
+        const int b0 = page_of(t0), b1 = page_of(t0 + 1);
+        blk_ahead = value_wave ? b1 : page_of(t0 + 2);       // the next page this wave will ask for
+        __syncthreads();
+        plan(t0, b0);
+#pragma unroll
+        for (int j = 0; j < 8; j++) dma(j);
+        if (!value_wave) {
+            plan(t0 + 1, b1);
+#pragma unroll
+            for (int j = 0; j < 8; j++) dma(j);
+        }
+        wait_loads();
+    }
+    __syncthreads();
+
+    const float kLazy = 8.0f;
+    if (!value_wave) {
+        // ================================ score wave ================================
+        uint4 qf[NKS];
+        {
+            const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
+            const float c = A.scale_log2e;
+            auto scaled = [&](uint32_t w2) -> uint32_t {
+                return pack2<DT>(elem16_to_f((uint16_t)(w2 & 0xffffu), IO) * c, elem16_to_f((uint16_t)(w2 >> 16), IO) * c);
+            };
+#pragma unroll
+            for (int ks = 0; ks < NKS; ks++) {
+                const uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+                qf[ks] = make_uint4(scaled(v.x), scaled(v.y), scaled(v.z), scaled(v.w));
+            }
+        }
+        pf_f32x16 negm;
+#pragma unroll
+        for (int i = 0; i < 16; i++) negm[i] = 0.0f;
+        float m_ref = 0.0f, l_run = 0.0f;
+        bool m_init = false;
+        const uint32_t kx1 = (uint32_t)(n * RB + ((g ^ (n & 15)) << 4));
+        auto qk = [&](int slot, pf_f32x16 (&s)[2], auto &&between) {
+            const uint32_t ka0 = pf_lds_addr(&k_ldsw[0][0]) + ((uint32_t)slot << 15) + kx1;
+            uint4 a[NKS][2];
+#pragma unroll
+            for (int ks = 0; ks < XQ; ks++) {
+                a[ks][0] = pf_lds_read128(ka0 ^ (uint32_t)(ks << 5), 0);
+                a[ks][1] = pf_lds_read128(ka0 ^ (uint32_t)(ks << 5), 32 * RB);
+            }
+            pf_sched_barrier();
+#pragma unroll
+            for (int ks = 0; ks < NKS; ks++) {
+                if (ks + XQ < NKS) {
+                    a[ks + XQ][0] = pf_lds_read128(ka0 ^ (uint32_t)((ks + XQ) << 5), 0);
+                    a[ks + XQ][1] = pf_lds_read128(ka0 ^ (uint32_t)((ks + XQ) << 5), 32 * RB);
+                }
+                between(ks);
+                if (ks == 0) {
+                    s[0] = mfma32<DT>(a[ks][0], qf[ks], negm);
+                    s[1] = mfma32<DT>(a[ks][1], qf[ks], negm);
+                } else {
+                    s[0] = mfma32<DT>(a[ks][0], qf[ks], s[0]);
+                    s[1] = mfma32<DT>(a[ks][1], qf[ks], s[1]);
+                }
+                pf_sched_barrier();
+            }
+        };
+        pf_f32x16 s_even[2], s_odd[2];
+        qk(t0 & 1, s_even, [](int) {});
+        // bit r: run r of the tile has a page; read one tile ahead, between the products
+        auto flags_of = [&](const int4 &v) -> int {
+            return __builtin_amdgcn_readfirstlane(v.x | (v.y << 1) | (v.z << 2) | (v.w << 3));
+        };
+        int flags = flags_of(*(const int4 *)&valid_ldsw[t0 & 3][0]);
+
+        auto step = [&](int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
+            plan(it + 2, blk_ahead);                             // K(it + 2): requested between the products below
+            blk_ahead = page_of(it + 3);
+            const int tile_t = it * kPfBN;
+            if (__builtin_expect(flags != 15 || it >= first_masked_tile, 0)) {
+#pragma unroll
+                for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int tl = tt * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                        const bool ok = (tile_t + tl) < vis && ((flags >> (tl >> 4)) & 1) != 0;
+                        s[tt][i] = ok ? s[tt][i] : -INFINITY;
+                    }
+            }
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[tt][i]);
+            tmax = pf_max_halves(tmax);
+            const bool move = m_init ? tmax > kLazy : tmax > -INFINITY;
+            float alpha = 1.0f;
+            const bool any_move = __any(move);
+            if (__builtin_expect(any_move, 0)) {
+                const float delta = move ? tmax : 0.0f;
+                m_init = m_init || move;
+                m_ref += delta;
+                alpha = __builtin_amdgcn_exp2f(-delta);
+                l_run *= alpha;
+#pragma unroll
+                for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) s[tt][i] -= delta;
+#pragma unroll
+                for (int i = 0; i < 16; i++) negm[i] = -m_ref;
+            }
+            float psum = 0.0f, p8[8];
+            uint4 pb[2][2];
+            int4 flags_ahead;
+            wait_loads();                                        // K(it + 1) of this wave's run has landed
+            pf_barrier_lds();                                    // A_it
+            asm volatile("" : : "s"(blk_ahead));
+            qk((it + 1) & 1, s_next, [&](int ks) {
+                if (ks == 0) flags_ahead = *(const int4 *)&valid_ldsw[(it + 1) & 3][0];
+                if ((ks & 1) == 0) dma(ks >> 1);
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int j = ks * 2 + u, tt = j >> 4, i = j & 15;
+                    const float e = __builtin_amdgcn_exp2f(s[tt][i]);
+                    p8[j & 7] = e;
+                    psum += e;
+                    asm volatile("" : "+v"(psum));               // the sum stays here, in the shadow of the products
+                    if ((j & 7) == 7)
+                        pb[tt][(i >> 3) & 1] = make_uint4(pack2<DT>(p8[0], p8[1]), pack2<DT>(p8[2], p8[3]), pack2<DT>(p8[4], p8[5]), pack2<DT>(p8[6], p8[7]));
+                }
+            });
+            l_run += psum;
+            flags = flags_of(flags_ahead);
+            // the tile's weights and, if the reference moved, the rows' factors, to the value wave
+            p_ldsw[w][0][lane] = pb[0][0];
+            p_ldsw[w][1][lane] = pb[0][1];
+            p_ldsw[w][2][lane] = pb[1][0];
+            p_ldsw[w][3][lane] = pb[1][1];
+            if (any_move) alpha_ldsw[w][lane] = alpha;
+            if (lane == 0) moved_ldsw[w] = any_move ? 1 : 0;
+            pf_barrier_lds();                                    // B_it
+        };
+        for (int it = t0; it < ntiles; it += 2) {
+            step(it, s_even, s_odd);
+            if (it + 1 < ntiles) step(it + 1, s_odd, s_even);
+        }
+        l_ldsw[w][lane] = l_run;
+        pf_barrier_lds();                                        // E: the value wave may read the row sums
+        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        if (nparts > 1) {
+            if (row_live && g == 0) {
+                A.part_m[prow] = m_ref;
+                A.part_l[prow] = l_tot;
+            }
+            return;
+        }
+        if (A.lse_rows && row_live && g == 0)
+            A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_ref + __builtin_log2f(l_tot) : INFINITY;
+        return;
+    }
+
+    // ================================ value wave ================================
+    pf_f32x16 o[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[dt][i] = 0.0f;
+    uint32_t vx1;
+    {
+        const int j16 = lane & 15;
+        const int rowl = 4 * g + (j16 >> 2);
+        const int clane = 2 * ((lane >> 4) & 1) + ((j16 & 3) >> 1), half = j16 & 1;
+        vx1 = (uint32_t)(rowl * RB + (((rowl & 3) << 6) | (clane << 4)) + (half << 3));
+    }
+    pf_barrier_lds();                                            // A_t0 (the score waves' first scores follow it)
+    pf_barrier_lds();                                            // B_t0: P(t0) is there
+#pragma unroll 1
+    for (int it = t0; it < ntiles; it++) {
+        const bool last = it + 1 >= ntiles;
+        // the tile's weights, then the first V operands (V(it) is there since B_it); the wave waits once
+        uint4 pb[2][2];
+        pb[0][0] = p_ldsw[w][0][lane];
+        pb[0][1] = p_ldsw[w][1][lane];
+        pb[1][0] = p_ldsw[w][2][lane];
+        pb[1][1] = p_ldsw[w][3][lane];
+        const int moved = moved_ldsw[w];
+        const uint32_t vb = pf_lds_addr(&v_ldsw[0][0]) + ((uint32_t)(it & 1) << 15) + vx1;
+        constexpr int NP = 4 * NDT;
+        uint2 lo[NP], hi[NP];
+        auto rd = [&](int i) {                                   // product i = (tt, mh, dt) = (i / 16, (i / 8) & 1, i % 8)
+            const int roff = ((i / (2 * NDT)) * 32 + 16 * ((i / NDT) & 1)) * RB;
+            const uint32_t va = vb ^ (uint32_t)((i % NDT) << 6);
+            lo[i] = pf_lds_read_tr16(va, roff);
+            hi[i] = pf_lds_read_tr16(va, roff + 8 * RB);
+        };
+#pragma unroll
+        for (int i = 0; i < XP; i++) rd(i);
+        pf_sched_barrier();
+        if (__builtin_expect(moved != 0, 0)) {
+            const float alpha = alpha_ldsw[w][lane];
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[dt][i] *= alpha;
+        }
+        plan(it + 1, blk_ahead);                                 // V(it + 1): requested between the products below
+        blk_ahead = page_of(it + 2);
+        asm volatile("" : : "s"(blk_ahead));
+#pragma unroll
+        for (int i = 0; i < NP; i++) {
+            if (i + XP < NP) rd(i + XP);
+            // A_{it+1}: P(it) has been read -- the products before this one used it -- and the score wave may write
+            // P(it + 1); the V operands on their way are not waited for
+            if (i == kFirst && !last) {
+                pf_sched_barrier();
+                asm volatile("s_barrier" ::: "memory");
+                pf_sched_barrier();
+            }
+            if (i >= kFirst && (i - kFirst) % 3 == 0 && (i - kFirst) / 3 < 8 && !last) dma((i - kFirst) / 3);
+            o[i % NDT] = mfma32<DT>(make_uint4(lo[i].x, lo[i].y, hi[i].x, hi[i].y), pb[i / (2 * NDT)][(i / NDT) & 1], o[i % NDT]);
+            pf_sched_barrier();
+        }
+        if (!last) {
+            wait_loads();                                        // V(it + 1) of this wave's run has landed
+            pf_barrier_lds();                                    // B_{it+1}
+        }
+    }
+    pf_barrier_lds();                                            // E
+    const float l_tot = l_ldsw[w][lane] + l_ldsw[w][lane ^ 32];
+    if (nparts > 1) {
+        if (row_live) {
+            float *orow = A.part_o + prow * D;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int b4 = 0; b4 < 4; b4++)
+                    *(float4 *)(orow + dt * 32 + 8 * b4 + 4 * g) =
+                        make_float4(o[dt][4 * b4], o[dt][4 * b4 + 1], o[dt][4 * b4 + 2], o[dt][4 * b4 + 3]);
+        }
+        return;
+    }
+    if (row_live && (l_tot > 0.0f || A.gate)) {
+        const bool have = l_tot > 0.0f;
+        const float inv = have ? 1.0f / l_tot : 0.0f;
+        uint8_t *orow = A.out + ((size_t)tq * A.QH + head) * (D * 2);
+        const uint16_t *grow = A.gate ? A.gate + ((size_t)tq * A.QH + head) * A.gate_stride : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+            for (int b4 = 0; b4 < 4; b4++) {
+                const int d0 = dt * 32 + 8 * b4 + 4 * g;
+                uint2 v = have ? make_uint2(pack2<IO>(o[dt][4 * b4] * inv, o[dt][4 * b4 + 1] * inv),
+                                            pack2<IO>(o[dt][4 * b4 + 2] * inv, o[dt][4 * b4 + 3] * inv))
+                               : *(const uint2 *)(orow + d0 * 2);
+                if (grow) {
+                    const uint2 gv = *(const uint2 *)(grow + d0);
+                    v.x = (uint32_t)gated_elem16((uint16_t)(v.x & 0xffffu), (uint16_t)(gv.x & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.x >> 16), (uint16_t)(gv.x >> 16), IO) << 16);
+                    v.y = (uint32_t)gated_elem16((uint16_t)(v.y & 0xffffu), (uint16_t)(gv.y & 0xffffu), IO) |
+                          ((uint32_t)gated_elem16((uint16_t)(v.y >> 16), (uint16_t)(gv.y >> 16), IO) << 16);
+                }
+                *(uint2 *)(orow + d0 * 2) = v;
+            }
+    }
+}
+
 // ---- attention mass of a chunk ------------------------------------------------------------------
 // mass[lb] += sum over the chunk's rows (query tokens x query heads) and over the tokens of logical block lb of
 // the row's softmax probability: what each page of the context received from a perception frame (the
@@ -2355,6 +2738,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 // [0, pos_start + M) with the context split over the whole chip, and a small kernel folds each
 // row's pieces (and applies the gate).
 int g_prefill_two_phase = 1;                   // 0: never; 1: by the rule in prefill_impl; 2: whenever the geometry allows (tests); 3: as 2, with register staging also for 16-bit pages
+int g_prefill_d256_waves = 1;                  // head_dim 256 chunk kernel: 0 one wave per SIMD does both products, 1 a score wave and a value wave per SIMD
 int g_prefill_pieces = 1;                      // head_dim 256, pieces for the walks of the last round: 0 never, 1 when they are worth it, 2 whenever there are any (tests)
 int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
 constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
@@ -2597,6 +2981,7 @@ using namespace drk;
 extern "C" {
 
 void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
+void drk_debug_set_prefill_d256_waves(int mode) { g_prefill_d256_waves = mode != 0 ? 1 : 0; }
 void drk_debug_set_prefill_pieces(int mode) { g_prefill_pieces = mode < 0 ? 1 : (mode > 2 ? 2 : mode); }
 static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
                              int layer, int pos_start, int M, float scale, int io_dtype, const float *d_row_lse,
@@ -2807,8 +3192,13 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
             A.part_l = A.part_m + (size_t)sh.tail * 128 * sh.kparts;
         }
         const dim3 gridp((unsigned)(sh.n_full + sh.tail * sh.kparts));
-        if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_d256_kernel<DRK_BF16, DRK_BF16>), gridp, dim3(256), 0, st, A);
-        else hipLaunchKernelGGL((prefill_d256_kernel<DRK_F16, DRK_F16>), gridp, dim3(256), 0, st, A);
+        if (g_prefill_d256_waves) {
+            if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_d256w_kernel<DRK_BF16, DRK_BF16>), gridp, dim3(512), 0, st, A);
+            else hipLaunchKernelGGL((prefill_d256w_kernel<DRK_F16, DRK_F16>), gridp, dim3(512), 0, st, A);
+        } else {
+            if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_d256_kernel<DRK_BF16, DRK_BF16>), gridp, dim3(256), 0, st, A);
+            else hipLaunchKernelGGL((prefill_d256_kernel<DRK_F16, DRK_F16>), gridp, dim3(256), 0, st, A);
+        }
         DRK_LAUNCH_CHECK("prefill_d256_kernel");
         if (sh.kparts > 1) {
             hipLaunchKernelGGL(prefill_piece_merge_kernel, dim3((unsigned)(sh.tail * 128)), dim3(64), 0, st, A, io_dtype);

@@ -51,6 +51,10 @@ void drk_debug_set_prefill_split(int max_rows);
  * without a workspace); 1 (default) = cut them when a piece is eight tiles or more and the workspace
  * drk_prefill_workspace_bytes reports is passed; 2 = whenever a last round exists (tests). */
 void drk_debug_set_prefill_pieces(int mode);
+/* head_dim 256 chunk kernel on 16-bit pages: 1 (default) = eight waves per workgroup, a score wave (K Q^T, softmax)
+ * and a value wave (V^T P^T) per 32 rows; 0 = four waves, each does both products of its 32 rows.  Same walks,
+ * same pieces, same bits. */
+void drk_debug_set_prefill_d256_waves(int mode);
 /* Tuning: which causal chunks of head_dim 128 run on the two-phase chunk kernels (eight waves, 256 rows per
  * workgroup): 0 = none (the four-wave kernel); 1 = the library's rule (default: chunks long enough to give
  * most CUs a workgroup); 2 = every chunk the geometry allows; 3 = as 2, and 16-bit pages too go through

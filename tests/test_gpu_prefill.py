@@ -268,14 +268,24 @@ def test_ring_of_tiles_wraps_over_holes_and_ragged_ends(dev, chunk_kernel, dtype
     assert ok, f"max abs err {ma:.4g} ({chunk_kernel=} {bs=} {G=} {pos_start=} {M=} {holes=})"
 
 
+@pytest.fixture(params=["score_and_value_waves", "one_wave_per_simd"])
+def d256_waves(request):
+    """The two head_dim 256 chunk kernels for 16-bit pages: eight waves, a score wave and a value wave per 32 rows
+    (the library's default), and four waves that do both products."""
+    lib = cabi.lib()
+    lib.drk_debug_set_prefill_d256_waves(1 if request.param == "score_and_value_waves" else 0)
+    yield request.param
+    lib.drk_debug_set_prefill_d256_waves(1)
+
+
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
 @pytest.mark.parametrize("bs,G,pos_start,M,holes", [
     (256, 6, 900, 257, (1,)), (16, 2, 0, 300, (3, 4, 5, 6, 17)), (64, 6, 1500, 100, (20,)), (32, 1, 33, 130, ()),
     (128, 12, 2047, 22, (0,)), (16, 6, 640, 64, (40, 43))])
-def test_head_dim_256_over_holes_and_ragged_ends(dev, chunk_kernel, dtype, bs, G, pos_start, M, holes):
+def test_head_dim_256_over_holes_and_ragged_ends(dev, chunk_kernel, d256_waves, dtype, bs, G, pos_start, M, holes):
     """16-bit pages with head_dim 256 (the reference model's: 24 query over 4 kv heads, blocks of 256 tokens) on the
-    kernel that loads tiles straight into LDS with one wave per SIMD (the first two runs of this case; the third takes
-    the register-staging kernel): walks of up to 35 tiles over missing pages, chunk ends inside a page and inside a
+    kernels that load tiles straight into LDS (the first two runs of this case, each with both arrangements of waves;
+    the third takes the register-staging kernel): walks of up to 35 tiles over missing pages, chunk ends inside a page and inside a
     tile, query tiles of 21, 64, 128, 10 tokens.  Rows behind holes only keep the caller's bytes; everything else
     against fp64 on the stored values."""
     KVH, D = 2, 256
@@ -298,7 +308,7 @@ def test_head_dim_256_over_holes_and_ragged_ends(dev, chunk_kernel, dtype, bs, G
 @pytest.mark.parametrize("bs,KVH,G,pos_start,M,holes", [
     (256, 4, 6, 900, 257, (1,)), (16, 2, 2, 0, 300, (3, 4, 5, 6, 17)), (64, 2, 6, 1500, 100, (20,)), (32, 2, 1, 33, 130, ()),
     (128, 1, 12, 2047, 22, (0,)), (16, 2, 6, 640, 64, (40, 43)), (16, 4, 6, 64, 2048, (7,)), (16, 3, 5, 3, 50, ())])
-def test_head_dim_256_walks_cut_into_pieces(dev, dtype, bs, KVH, G, pos_start, M, holes):
+def test_head_dim_256_walks_cut_into_pieces(dev, d256_waves, dtype, bs, KVH, G, pos_start, M, holes):
     """The workgroups of the head_dim 256 kernel's last round take pieces of their walks (ranges of tiles) and a merge
     folds them: forced here for every shape (2 to 8 pieces, walks shorter than their number of pieces, the reference
     model's 24 / 4 heads on a full 2 048-row chunk: 384 walks, the last 128 in two pieces each), against fp64 and
@@ -336,6 +346,44 @@ def test_head_dim_256_walks_cut_into_pieces(dev, dtype, bs, KVH, G, pos_start, M
             w1 = orc.decode_f64(og, q[rsel], opool, table, 1, pos_start + int(rsel) + 1, scale, dtype)
             ok, ma, _ = U.rel_abs_ok(U.from_bits(got[rsel], dtype), w1)
             assert ok, (int(rsel), ma)
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16])
+@pytest.mark.parametrize("bs,KVH,G,pos_start,M,holes,pieces", [
+    (256, 4, 6, 900, 257, (1,), 0), (16, 2, 2, 0, 300, (3, 4, 5, 6, 17), 2), (64, 2, 6, 1500, 100, (20,), 0),
+    (128, 1, 12, 2047, 22, (0,), 2), (16, 4, 6, 4096, 2048, (7, 200), 1), (16, 3, 5, 3, 50, (), 2)])
+def test_head_dim_256_wave_arrangements_give_the_same_bits(dev, dtype, bs, KVH, G, pos_start, M, holes, pieces):
+    """The eight-wave kernel splits the work of the four-wave kernel between two waves per 32 rows and keeps its
+    arithmetic and its order: outputs and row log-sum-exps of the two are the same bits, with whole walks, with the
+    library's rule for pieces (a 2 048-row chunk behind 4 096 tokens) and with pieces forced."""
+    lib = cabi.lib()
+    D, QH = 256, KVH * G
+    total = pos_start + M
+    nblk = (total + bs - 1) // bs
+    holes = tuple(h for h in holes if h < nblk)
+    g, og, rng, table, opool = build((2, KVH, QH, D, bs, nblk + 3), dtype, total, seed=bs * 77 + G, holes=holes, mul=0.7)
+    q = U.normal_bits(rng, (M, QH, D), dtype, 0.7)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    res = []
+    try:
+        lib.drk_debug_set_prefill_two_phase(1)
+        lib.drk_debug_set_prefill_pieces(pieces)
+        wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+        ws = U.dev_zeros(max(wsb, 16))
+        for waves in (1, 0):
+            lib.drk_debug_set_prefill_d256_waves(waves)
+            out = U.dev_bytes(np.full(M * QH * D * 2, 0x7B, dtype=np.uint8))
+            lse = U.dev_bytes(np.full(M * QH * 4, 0x7B, dtype=np.uint8))
+            cabi.call("drk_paged_prefill_attention_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), 1, pos_start, M,
+                      float(1 / np.sqrt(D)), dtype, None, 0, U.p(lse), U.p(ws), wsb, U.stream_ptr())
+            U.sync()
+            res.append((U.host(out, np.uint16, (M, QH, D)), U.host(lse, np.uint32, (M, QH))))
+    finally:
+        lib.drk_debug_set_prefill_pieces(1)
+        lib.drk_debug_set_prefill_d256_waves(1)
+    assert np.array_equal(res[0][0], res[1][0])
+    assert np.array_equal(res[0][1], res[1][1])
+    assert not np.all(res[0][0].view(np.uint8) == 0x7B)
 
 
 @pytest.mark.parametrize("geom,dtype,io", [((2, 8, 32, 128, 16, 300), cabi.BF16, cabi.BF16), ((2, 4, 24, 256, 256, 20), cabi.F16, cabi.F16),
