@@ -645,7 +645,7 @@ def config7(args):
         prefill["pos_%d" % pos] = {"us": round(ms * 1e3, 1), "TFLOPs": round(fl / (ms * 1e-3) / 1e12, 1),
                                    "frac": round(fl / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
     return {
-        "prefill_chunks_2048": {"kernel": "prefill_d256_kernel<f16>", "bound": "mfma", "peak": MFMA_BF16_PEAK_TFLOPS, **prefill},
+        "prefill_chunks_2048": {"kernel": "prefill_d256w_kernel<f16>" if getattr(args, "d256_waves", None) != 0 else "prefill_d256_kernel<f16>", "bound": "mfma", "peak": MFMA_BF16_PEAK_TFLOPS, **prefill},
         "metric": "paged_decode_attention_GBps", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": K,
         "warmup": W, "ms_per_step": round(total_ms / K, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
@@ -1083,7 +1083,7 @@ def kernel_fractions(buf, seed=11):
             torch.cuda.synchronize()
         whole.append(round(a0.elapsed_time(a1) * 1e3, 1))
     lib.drk_debug_set_prefill_pieces(1)
-    prefill_entry("config7_prefill_d256", "prefill_d256_kernel<f16> + prefill_piece_merge_kernel", per_chunk,
+    prefill_entry("config7_prefill_d256", "prefill_d256w_kernel<f16> + prefill_piece_merge_kernel", per_chunk,
                   "the reference's model shape: causal prefill of 32768 tokens in 16 chunks of 2048 over 256-token blocks, 24 Q / 4 KV "
                   "heads x 256, fp16 (the pages hold N(0, 0.5), written beforehand); 384 walks of 128 rows: 256 whole, the last 128 "
                   "in two pieces each and a merge of their rows, timed together",
