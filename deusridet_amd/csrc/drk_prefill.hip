@@ -2332,6 +2332,245 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
     walk(std::true_type{});
 }
 
+// ---- attention mass of a chunk, 16-bit pages, the rows' log-sum-exps given: tiles straight into LDS ----------
+// The one-walk case of prefill_mass_kernel rebuilt on the chunk kernels' machinery: 256 rows per workgroup (eight
+// waves of 32, two per SIMD), K tiles from global memory straight into a ring of four swizzled LDS buffers,
+// requested two tiles ahead between the k-steps, one barrier per tile; the products start from minus the row's
+// log-sum-exp (the C operand), so a score arrives as the exponent of its probability, and the exponentials of tile t
+// sit between the k-steps of tile t + 1's products, the fold of tile t - 1's sums too.  The vector unit bounds it:
+// 32 exponentials and 32 additions per wave and tile beside 16 products (probes: without the products 584 of 715 us
+// on 2 048 rows behind 30 720 tokens at 32 / 8 heads x 128, without the vector work 300; half of the LDS operand
+// reads left out changes nothing).  S = Q K^T as
+// in prefill_mass_kernel: a lane stands for a key, its registers for 16 of the wave's rows, a key's sum over rows is
+// a sum over registers.  A page's sum goes to a table in LDS (one entry per logical block of the walk) and the
+// table to `mass` with one atomic per block and workgroup when the walk ends -- 256 workgroups adding to the same
+// four blocks tile after tile would queue up on them.  FOLD: the softmax scale goes into Q, rounded to the 16-bit
+// type, as in the chunk kernels that do so (their log-sum-exps belong to those scores); otherwise Q stays as it
+// is and the exponent is scaled.
+// grid = ceil(M / TPW) * KVH, TPW = 256 / (QH/KVH); block = 512; block size 16 * 2^k; at most kMassdBlocks<D>
+// logical blocks in pos_start + M tokens.
+template <int D>
+constexpr int kMassdBlocks = D == 128 ? 8192 : 6144;
+template <int DT, int IO, int D, bool FOLD>
+__global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, float *__restrict__ mass, int mass_len)
+{
+    constexpr int RB = D * 2;
+    constexpr int kTileBytes = kPfBN * RB, kTileShift = D == 128 ? 14 : 15;
+    constexpr int NKS = D / 16;
+    constexpr int kRing = 4, ROWS = 8;                       // buffers; tokens of a tile one wave requests
+    constexpr int LPR = RB / 16, RPQ = 64 / LPR, NREQ = ROWS / RPQ;   // lanes per token row, rows per request, requests per wave and tile
+    constexpr int XQ = 2;                                    // operand reads ahead of their products, k-steps
+    constexpr int EPK = 32 / NKS;                            // exponentials per k-step
+    __shared__ __align__(512) uint8_t k_ldsm[kRing][kTileBytes];
+    __shared__ float mass_ldsm[kMassdBlocks<D>];
+    __shared__ __align__(16) int valid_ldsm[kRing][8];                     // [tile & 3][wave]: the wave's 8-token run of the tile has a page
+
+    const int kvh = (int)blockIdx.x % A.KVH;
+    const int nqt = (int)gridDim.x / A.KVH;
+    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, g = lane >> 5;
+    const int G = A.QH / A.KVH, TPW = A.tpw;
+    const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
+    const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
+    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+    const int sh = A.bs_shift;
+    const int nblk_wg = (lim_wg + A.bs - 1) >> sh;
+
+    for (int i = threadIdx.x; i < nblk_wg; i += 512) mass_ldsm[i] = 0.0f;
+    for (int i = threadIdx.x * 16; i < kRing * kTileBytes; i += 512 * 16) *(uint4 *)(&k_ldsm[0][0] + i) = make_uint4(0, 0, 0, 0);
+
+    // Q as the A operand: this lane's fragment belongs to row w * 32 + n
+    uint4 qf[NKS];
+    {
+        const int r = w * 32 + n, rt = r / G;
+        const int tq = qt * TPW + rt;
+        const int head = kvh * G + (r - rt * G);
+        const bool row_live = rt < TPW && tq < A.M;
+        const uint8_t *qrow = A.q + ((size_t)tq * A.QH + head) * (D * 2) + g * 16;
+        const float c = A.scale_log2e;
+        auto scaled = [&](uint32_t w2) -> uint32_t {
+            return pack2<DT>(elem16_to_f((uint16_t)(w2 & 0xffffu), IO) * c, elem16_to_f((uint16_t)(w2 >> 16), IO) * c);
+        };
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            const uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
+            qf[ks] = FOLD ? make_uint4(scaled(v.x), scaled(v.y), scaled(v.z), scaled(v.w)) : v;
+        }
+    }
+    // the rows this lane's registers stand for: tokens [0, vis[i]) are visible to row i (0: an idle row); the
+    // products start from -lse (FOLD) or -lse / (scale log2 e), so that the scaled score comes out less the lse
+    int vis[16];
+    pf_f32x16 negl;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int r = w * 32 + 8 * (i >> 2) + 4 * g + (i & 3), rt = r / G;
+        const int tq = qt * TPW + rt;
+        const bool live = rt < TPW && tq < A.M;
+        vis[i] = live ? A.pos_start + tq + 1 : 0;
+        const float lse = live ? A.lse_rows[(size_t)tq * A.QH + kvh * G + (r - rt * G)] : INFINITY;
+        negl[i] = FOLD ? -lse : -lse / A.scale_log2e;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // from here on the kernel counts its loads itself
+
+    const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
+    const int tgw = w * ROWS;
+    typedef const int32_t __attribute__((address_space(4))) *const_table_t;
+    const const_table_t table_k = (const_table_t)(uintptr_t)A.table;
+    auto page_of = [&](int tile) -> int {                    // through the scalar cache: not counted with the requests
+        const int tg = tile * kPfBN + tgw;
+        return tg < lim_wg ? table_k[tg >> sh] : -1;
+    };
+    const uint8_t *p_src = kbase;
+    int p_rows = 0;
+    uint32_t p_lds = 0;
+    const uint32_t k_ring = pf_lds_addr(&k_ldsm[0][0]) + (uint32_t)(tgw * RB);
+    auto plan = [&](int kt, int blk_raw) {
+        const int blk0 = __builtin_amdgcn_readfirstlane(blk_raw);
+        const int tg = kt * kPfBN + tgw;
+        const bool ok = blk0 >= 0 && blk0 < A.NB && tg < lim_wg;
+        p_rows = ok ? lim_wg - tg : 0;
+        p_src = kbase + (size_t)(ok ? blk0 : 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
+        p_lds = k_ring + ((uint32_t)(kt & (kRing - 1)) << kTileShift);
+        if (lane == 0) valid_ldsm[kt & (kRing - 1)][w] = ok ? 1 : 0;
+    };
+    // request j: RPQ token rows (1 KB); the 16-byte chunk c of row r sits at position c ^ (r & 15)
+    uint32_t goff[NREQ];
+    {
+        const int rr = lane / LPR, cp = lane % LPR;
+#pragma unroll
+        for (int j = 0; j < NREQ; j++) goff[j] = (uint32_t)(rr * RB + ((cp ^ ((tgw + RPQ * j + rr) & 15)) << 4));
+    }
+    bool whole = false;                                      // the last tile requested made all NREQ requests
+    auto request = [&](int j) {
+        if (__builtin_expect(whole, 1)) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
+        else if (RPQ * j + lane / LPR < p_rows) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
+    };
+    auto request_tile = [&]() {
+        whole = p_rows >= ROWS;
+#pragma unroll
+        for (int j = 0; j < NREQ; j++) request(j);
+    };
+
+    // where this lane finds its B operands: K row n (and n + 32), chunk 2 ks + g at byte ((g ^ n & 15) << 4) ^ (ks << 5)
+    const uint32_t kx1 = (uint32_t)(n * RB + ((g ^ (n & 15)) << 4));
+    auto qk = [&](int slot, pf_f32x16 (&s)[2], auto &&between) {
+        const uint32_t ka0 = pf_lds_addr(&k_ldsm[0][0]) + ((uint32_t)slot << kTileShift) + kx1;
+        uint4 b[NKS][2];
+#pragma unroll
+        for (int ks = 0; ks < XQ; ks++) {
+            b[ks][0] = pf_lds_read128(ka0 ^ (uint32_t)(ks << 5), 0);
+            b[ks][1] = pf_lds_read128(ka0 ^ (uint32_t)(ks << 5), 32 * RB);
+        }
+        pf_sched_barrier();
+#pragma unroll
+        for (int ks = 0; ks < NKS; ks++) {
+            if (ks + XQ < NKS) {
+                b[ks + XQ][0] = pf_lds_read128(ka0 ^ (uint32_t)((ks + XQ) << 5), 0);
+                b[ks + XQ][1] = pf_lds_read128(ka0 ^ (uint32_t)((ks + XQ) << 5), 32 * RB);
+            }
+            between(ks);
+            if (ks == 0) {
+                s[0] = mfma32<DT>(qf[ks], b[ks][0], negl);
+                s[1] = mfma32<DT>(qf[ks], b[ks][1], negl);
+            } else {
+                s[0] = mfma32<DT>(qf[ks], b[ks][0], s[0]);
+                s[1] = mfma32<DT>(qf[ks], b[ks][1], s[1]);
+            }
+            pf_sched_barrier();
+        }
+    };
+
+    // ---- prologue: K(0), K(1), K(2) requested, K(0) there, its scores ----
+    int blk_ahead;
+    {
+        const int b0 = page_of(0), b1 = page_of(1), b2 = page_of(2);
+        blk_ahead = page_of(3);
+        __syncthreads();                                     // the clearing is done (and the table entries are here)
+        plan(0, b0);
+        request_tile();
+        plan(1, b1);
+        request_tile();
+        plan(2, b2);
+        request_tile();
+        __builtin_amdgcn_s_waitcnt(0x0f70);                  // vmcnt(0)
+    }
+    __syncthreads();
+    pf_f32x16 s_even[2], s_odd[2];
+    qk(0, s_even, [](int) {});
+    // bit r: the tile's 8-token run r has a page; read one tile ahead, between the products
+    auto flags_of = [&](const int4 &a, const int4 &b) -> int {
+        return __builtin_amdgcn_readfirstlane(a.x | (a.y << 1) | (a.z << 2) | (a.w << 3) | (b.x << 4) | (b.y << 5) | (b.z << 6) | (b.w << 7));
+    };
+    int flags = flags_of(*(const int4 *)&valid_ldsm[0][0], *(const int4 *)&valid_ldsm[0][4]);
+
+    // the page sums of tile `tile_t` from the lanes' key sums: a key's other 16 rows are in the other half of the
+    // wave; a block is 16 keys or more
+    auto fold = [&](int tile_t, const float (&cs)[2]) {
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            const auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(cs[tt]), __float_as_uint(cs[tt]), false, false);
+            const float c16 = pf_row16_sum(__uint_as_float(r2[0]) + __uint_as_float(r2[1]));
+            const int run0 = tile_t + tt * 32 + (n & 16);
+            if (g == 0 && (n & 15) == 0 && run0 >= 0 && run0 < lim_wg && c16 != 0.0f) atomicAdd(&mass_ldsm[run0 >> sh], c16);
+        }
+    };
+    float cs_prev[2] = {0.0f, 0.0f};                         // the key sums of the tile before, folded a step later
+    auto step = [&](int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
+        // here: s = exponents of tile it; K(it + 1) and K(it + 2) requested
+        const int tile_t = it * kPfBN;
+        if (__builtin_expect(flags != 255 || it >= first_masked_tile, 0)) {
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                const int key = tile_t + tt * 32 + n;
+                const bool kvalid = ((flags >> ((tt * 32 + n) >> 3)) & 1) != 0;
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[tt][i] = (kvalid && key < vis[i]) ? s[tt][i] : -INFINITY;
+            }
+        }
+        // K(it + 1) has landed (this wave's share; the requests of K(it + 2) came after it), then everybody's
+        if (__builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
+        else __builtin_amdgcn_s_waitcnt(0x0f70);
+        pf_barrier_lds();
+        asm volatile("" : : "s"(blk_ahead));
+        plan(it + 3, blk_ahead);                             // into the buffer of K(it - 1), read two steps ago
+        blk_ahead = page_of(it + 4);
+        whole = p_rows >= ROWS;                              // requested between the products below
+        float cs[2] = {0.0f, 0.0f};
+        int4 fa, fb;
+        qk((it + 1) & (kRing - 1), s_next, [&](int ks) {
+            if (ks == 0) {
+                fa = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][0];
+                fb = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][4];
+            }
+            if ((ks & 1) == 0 && (ks >> 1) < NREQ) request(ks >> 1);
+            if (ks == NKS / 2) fold(tile_t - kPfBN, cs_prev);
+#pragma unroll
+            for (int u = 0; u < EPK; u++) {
+                const int j = ks * EPK + u, tt = j >> 4, i = j & 15;
+                const float e = __builtin_amdgcn_exp2f(FOLD ? s[tt][i] : s[tt][i] * A.scale_log2e);
+                cs[tt] += e;
+                asm volatile("" : "+v"(cs[tt]));             // the sum stays here, in the shadow of the products
+            }
+        });
+        flags = flags_of(fa, fb);
+        cs_prev[0] = cs[0];
+        cs_prev[1] = cs[1];
+    };
+    for (int it = 0; it < ntiles; it += 2) {
+        step(it, s_even, s_odd);
+        if (it + 1 < ntiles) step(it + 1, s_odd, s_even);
+    }
+    fold((ntiles - 1) * kPfBN, cs_prev);
+    __builtin_amdgcn_s_waitcnt(0x0f70);                      // nothing is on its way when the workgroup ends
+    __syncthreads();
+    for (int i = threadIdx.x; i < nblk_wg; i += 512) {
+        const float v = mass_ldsm[i];
+        if (v != 0.0f && i < mass_len) unsafeAtomicAdd(mass + i, v);
+    }
+}
+
 // mass[0 .. n) = 0
 __global__ void pf_zero_kernel(float *__restrict__ p, int n)
 {
@@ -2739,6 +2978,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 // row's pieces (and applies the gate).
 int g_prefill_two_phase = 1;                   // 0: never; 1: by the rule in prefill_impl; 2: whenever the geometry allows (tests); 3: as 2, with register staging also for 16-bit pages
 int g_prefill_d256_waves = 1;                  // head_dim 256 chunk kernel: 0 one wave per SIMD does both products, 1 a score wave and a value wave per SIMD
+int g_prefill_mass_direct = 1;                 // one-walk mass pass over 16-bit pages: 1 the kernel that takes tiles straight into LDS, 0 the register-staging kernel
 int g_prefill_pieces = 1;                      // head_dim 256, pieces for the walks of the last round: 0 never, 1 when they are worth it, 2 whenever there are any (tests)
 int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
 constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
@@ -2944,6 +3184,22 @@ static bool d256_direct(const Lay &a)
            g_prefill_two_phase != 0 && g_prefill_two_phase != 3;
 }
 
+// Whether the chunk kernel that prefill_impl takes for this chunk folds the softmax scale into Q (rounded to the
+// 16-bit type): the two-phase kernels and the head_dim 256 kernels do, the four-wave kernel and the split path
+// (taken when the caller passes its workspace) do not.  The mass pass scores the way the attention call did.
+static bool chunk_kernel_scales_q(const Lay &a, int pos_start, int M)
+{
+    if (prefill_split_applies(a, pos_start, M)) return false;
+    if (d256_direct(a)) return true;
+    const int G = a.QH / a.KVH;
+    if (a.D == 128 && G <= 256 && a.bs >= 16 && ilog2_exact((unsigned)a.bs) >= 4 && g_prefill_two_phase != 0) {
+        const int tpw2 = 256 / G;
+        const long wgs2 = (long)((M + tpw2 - 1) / tpw2) * a.KVH;
+        return wgs2 >= 192 || g_prefill_two_phase > 1;
+    }
+    return false;
+}
+
 static size_t prefill_split_need(const Lay &a, int pos_start, int M)
 {
     int ct, ns;
@@ -2982,6 +3238,7 @@ extern "C" {
 
 void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
 void drk_debug_set_prefill_d256_waves(int mode) { g_prefill_d256_waves = mode != 0 ? 1 : 0; }
+void drk_debug_set_prefill_mass_direct(int on) { g_prefill_mass_direct = on != 0 ? 1 : 0; }
 void drk_debug_set_prefill_pieces(int mode) { g_prefill_pieces = mode < 0 ? 1 : (mode > 2 ? 2 : mode); }
 static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
                              int layer, int pos_start, int M, float scale, int io_dtype, const float *d_row_lse,
@@ -3021,6 +3278,25 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = nullptr; A.gate_stride = 0;
     A.lse_rows = const_cast<float *>(d_row_lse);             // read only here: the rows' log-sum-exps, or NULL (first walk finds them)
+    // 16-bit pages with the rows' log-sum-exps given: the kernel that takes its tiles straight into LDS
+    if (g_prefill_mass_direct && d_row_lse && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 &&
+        (pos_start + M + a.bs - 1) / a.bs <= (a.D == 128 ? kMassdBlocks<128> : kMassdBlocks<256>) && a.QH / a.KVH <= 128) {
+        A.tpw = 256 / (a.QH / a.KVH);
+        const dim3 gridd(((M + A.tpw - 1) / A.tpw) * a.KVH);
+        const bool fold = chunk_kernel_scales_q(a, pos_start, M);
+#define DRK_PMD(DT, DD)                                                                                                   \
+        do {                                                                                                             \
+            if (fold) hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, true>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
+            else hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, false>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
+        } while (0)
+        if (a.dtype == DRK_BF16 && a.D == 128) DRK_PMD(DRK_BF16, 128);
+        else if (a.dtype == DRK_BF16) DRK_PMD(DRK_BF16, 256);
+        else if (a.D == 128) DRK_PMD(DRK_F16, 128);
+        else DRK_PMD(DRK_F16, 256);
+#undef DRK_PMD
+        DRK_LAUNCH_CHECK("prefill_massd_kernel");
+        return DRK_OK;
+    }
     dim3 grid(((M + A.tpw - 1) / A.tpw) * a.KVH);
 #define DRK_PM(DT, KV, IO)                                                                                                      \
     do {                                                                                                                       \

@@ -185,12 +185,26 @@ def chunk_path(request):
     lib.drk_debug_set_prefill_split(-1)
 
 
+@pytest.fixture(params=["tiles_straight_into_lds", "tiles_through_registers"])
+def mass_kernel(request):
+    """The two one-walk mass kernels for 16-bit pages (8-bit pages have the second only)."""
+    lib = cabi.lib()
+    lib.drk_debug_set_prefill_mass_direct(1 if request.param == "tiles_straight_into_lds" else 0)
+    yield request.param
+    lib.drk_debug_set_prefill_mass_direct(1)
+
+
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
 @pytest.mark.parametrize("bs,pos_start,M,heads", [(16, 0, 70, (8, 32, 128)), (16, 333, 45, (8, 32, 128)), (32, 2500, 130, (2, 12, 128)),
-                                                  (256, 2100, 33, (4, 24, 256)), (16, 64, 300, (2, 2, 128))])
-def test_frame_mass_from_the_attention_calls_row_sums(dev, chunk_path, dtype, bs, pos_start, M, heads):
+                                                  (256, 2100, 33, (4, 24, 256)), (16, 64, 300, (2, 2, 128)), (16, 7, 200, (1, 5, 256)),
+                                                  (64, 1000, 260, (2, 14, 128))])
+def test_frame_mass_from_the_attention_calls_row_sums(dev, chunk_path, mass_kernel, dtype, bs, pos_start, M, heads):
     """The attention call leaves every row's log-sum-exp, the mass pass then walks the keys once: same masses as the
-    two-walk pass within the tolerance of the fp64 oracle, same attention output as the call without the extra result."""
+    two-walk pass within the tolerance of the fp64 oracle, same attention output as the call without the extra result.
+    Both one-walk kernels: the one that takes 256 rows per workgroup and its tiles straight into LDS (16-bit pages; head
+    counts that leave idle rows, walks that end inside a tile and inside a page, holes) and the register-staging one."""
+    if mass_kernel == "tiles_straight_into_lds" and dtype in (cabi.INT8, cabi.FP8_E4M3):
+        pytest.skip("8-bit pages have one mass kernel")
     total = pos_start + M
     holes = (1,) if total > 3 * bs else ()
     g, og, io, table, opool, q = _frame_case(dtype, bs, seed=bs + pos_start + M, pos_start=pos_start, M=M, heads=heads, holes=holes)
