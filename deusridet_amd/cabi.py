@@ -117,6 +117,7 @@ SIGNATURES = {
     "drk_debug_set_prefill_pieces": (None, [_i32]),
     "drk_debug_set_prefill_d256_waves": (None, [_i32]),
     "drk_debug_set_prefill_mass_direct": (None, [_i32]),
+    "drk_debug_set_prefill_mass_parts": (None, [_i32]),
     "drk_debug_set_prefill_two_phase": (None, [_i32]),
     "drk_probe_read_bandwidth": (_i32, [_vp, _sz, _i32, _vp, C.POINTER(C.c_float)]),
     "drk_probe_read_bandwidth_permuted": (_i32, [_vp, _sz, _i32, _i32, _vp, C.POINTER(C.c_float)]),

@@ -2365,18 +2365,25 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
     __shared__ float mass_ldsm[kMassdBlocks<D>];
     __shared__ __align__(16) int valid_ldsm[kRing][8];                     // [tile & 3][wave]: the wave's 8-token run of the tile has a page
 
-    const int kvh = (int)blockIdx.x % A.KVH;
-    const int nqt = (int)gridDim.x / A.KVH;
-    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    // workgroup = (walk, part): a walk is (row block of tokens, kv head), the longest first; a part is one of
+    // A.kparts ranges of the walk's tiles (a short chunk behind a long context has few walks: with the rows'
+    // log-sum-exps known the parts need no merge, their sums just add up)
+    const int walk = (int)blockIdx.x / A.kparts, part = (int)blockIdx.x - walk * A.kparts;
+    const int kvh = walk % A.KVH;
+    const int qt = A.nqt - 1 - walk / A.KVH;
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
     const int G = A.QH / A.KVH, TPW = A.tpw;
     const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
     const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
-    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+    const int nt_walk = (lim_wg + kPfBN - 1) / kPfBN;
+    const int t0 = __builtin_amdgcn_readfirstlane((int)((long)part * nt_walk / A.kparts));
+    const int ntiles = __builtin_amdgcn_readfirstlane((int)((long)(part + 1) * nt_walk / A.kparts));     // the part's tiles: [t0, ntiles)
+    if (t0 >= ntiles) return;                                // more parts than tiles
     const int sh = A.bs_shift;
-    const int nblk_wg = (lim_wg + A.bs - 1) >> sh;
+    const int lb0 = (t0 * kPfBN) >> sh;                      // the table in LDS begins at the part's first block
+    const int nblk_wg = ((min(lim_wg, ntiles * kPfBN) + A.bs - 1) >> sh) - lb0;
 
     for (int i = threadIdx.x; i < nblk_wg; i += 512) mass_ldsm[i] = 0.0f;
     for (int i = threadIdx.x * 16; i < kRing * kTileBytes; i += 512 * 16) *(uint4 *)(&k_ldsm[0][0] + i) = make_uint4(0, 0, 0, 0);
@@ -2418,9 +2425,10 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
     const int tgw = w * ROWS;
     typedef const int32_t __attribute__((address_space(4))) *const_table_t;
     const const_table_t table_k = (const_table_t)(uintptr_t)A.table;
+    const int lim_part = min(lim_wg, ntiles * kPfBN);        // nothing past the part's end is requested
     auto page_of = [&](int tile) -> int {                    // through the scalar cache: not counted with the requests
         const int tg = tile * kPfBN + tgw;
-        return tg < lim_wg ? table_k[tg >> sh] : -1;
+        return tg < lim_part ? table_k[tg >> sh] : -1;
     };
     const uint8_t *p_src = kbase;
     int p_rows = 0;
@@ -2429,8 +2437,8 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
     auto plan = [&](int kt, int blk_raw) {
         const int blk0 = __builtin_amdgcn_readfirstlane(blk_raw);
         const int tg = kt * kPfBN + tgw;
-        const bool ok = blk0 >= 0 && blk0 < A.NB && tg < lim_wg;
-        p_rows = ok ? lim_wg - tg : 0;
+        const bool ok = blk0 >= 0 && blk0 < A.NB && tg < lim_part;
+        p_rows = ok ? lim_part - tg : 0;
         p_src = kbase + (size_t)(ok ? blk0 : 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
         p_lds = k_ring + ((uint32_t)(kt & (kRing - 1)) << kTileShift);
         if (lane == 0) valid_ldsm[kt & (kRing - 1)][w] = ok ? 1 : 0;
@@ -2482,28 +2490,28 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         }
     };
 
-    // ---- prologue: K(0), K(1), K(2) requested, K(0) there, its scores ----
+    // ---- prologue: K(t0), K(t0 + 1), K(t0 + 2) requested and there, the scores of tile t0 ----
     int blk_ahead;
     {
-        const int b0 = page_of(0), b1 = page_of(1), b2 = page_of(2);
-        blk_ahead = page_of(3);
+        const int b0 = page_of(t0), b1 = page_of(t0 + 1), b2 = page_of(t0 + 2);
+        blk_ahead = page_of(t0 + 3);
         __syncthreads();                                     // the clearing is done (and the table entries are here)
-        plan(0, b0);
+        plan(t0, b0);
         request_tile();
-        plan(1, b1);
+        plan(t0 + 1, b1);
         request_tile();
-        plan(2, b2);
+        plan(t0 + 2, b2);
         request_tile();
         __builtin_amdgcn_s_waitcnt(0x0f70);                  // vmcnt(0)
     }
     __syncthreads();
     pf_f32x16 s_even[2], s_odd[2];
-    qk(0, s_even, [](int) {});
+    qk(t0 & (kRing - 1), s_even, [](int) {});
     // bit r: the tile's 8-token run r has a page; read one tile ahead, between the products
     auto flags_of = [&](const int4 &a, const int4 &b) -> int {
         return __builtin_amdgcn_readfirstlane(a.x | (a.y << 1) | (a.z << 2) | (a.w << 3) | (b.x << 4) | (b.y << 5) | (b.z << 6) | (b.w << 7));
     };
-    int flags = flags_of(*(const int4 *)&valid_ldsm[0][0], *(const int4 *)&valid_ldsm[0][4]);
+    int flags = flags_of(*(const int4 *)&valid_ldsm[t0 & (kRing - 1)][0], *(const int4 *)&valid_ldsm[t0 & (kRing - 1)][4]);
 
     // the page sums of tile `tile_t` from the lanes' key sums: a key's other 16 rows are in the other half of the
     // wave; a block is 16 keys or more
@@ -2513,7 +2521,7 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
             const auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(cs[tt]), __float_as_uint(cs[tt]), false, false);
             const float c16 = pf_row16_sum(__uint_as_float(r2[0]) + __uint_as_float(r2[1]));
             const int run0 = tile_t + tt * 32 + (n & 16);
-            if (g == 0 && (n & 15) == 0 && run0 >= 0 && run0 < lim_wg && c16 != 0.0f) atomicAdd(&mass_ldsm[run0 >> sh], c16);
+            if (g == 0 && (n & 15) == 0 && run0 >= t0 * kPfBN && run0 < lim_part && c16 != 0.0f) atomicAdd(&mass_ldsm[(run0 >> sh) - lb0], c16);
         }
     };
     float cs_prev[2] = {0.0f, 0.0f};                         // the key sums of the tile before, folded a step later
@@ -2558,7 +2566,7 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         cs_prev[0] = cs[0];
         cs_prev[1] = cs[1];
     };
-    for (int it = 0; it < ntiles; it += 2) {
+    for (int it = t0; it < ntiles; it += 2) {
         step(it, s_even, s_odd);
         if (it + 1 < ntiles) step(it + 1, s_odd, s_even);
     }
@@ -2567,7 +2575,7 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
     __syncthreads();
     for (int i = threadIdx.x; i < nblk_wg; i += 512) {
         const float v = mass_ldsm[i];
-        if (v != 0.0f && i < mass_len) unsafeAtomicAdd(mass + i, v);
+        if (v != 0.0f && lb0 + i < mass_len) unsafeAtomicAdd(mass + lb0 + i, v);
     }
 }
 
@@ -2979,6 +2987,7 @@ int launch_shared_prefix(const Lay &a, const void *q, const void *pool, const in
 int g_prefill_two_phase = 1;                   // 0: never; 1: by the rule in prefill_impl; 2: whenever the geometry allows (tests); 3: as 2, with register staging also for 16-bit pages
 int g_prefill_d256_waves = 1;                  // head_dim 256 chunk kernel: 0 one wave per SIMD does both products, 1 a score wave and a value wave per SIMD
 int g_prefill_mass_direct = 1;                 // one-walk mass pass over 16-bit pages: 1 the kernel that takes tiles straight into LDS, 0 the register-staging kernel
+int g_prefill_mass_parts = 0;                  // that kernel's parts per walk: 0 by its rule, n > 0 forced (tests)
 int g_prefill_pieces = 1;                      // head_dim 256, pieces for the walks of the last round: 0 never, 1 when they are worth it, 2 whenever there are any (tests)
 int g_prefill_split = -1;                      // -1: by the rule below; 0: never; n > 0: every chunk of up to n rows (tests)
 constexpr int kSplitMinPos = 2048, kSplitMaxM = 1024, kSplitMaxPieces = 128;
@@ -3072,6 +3081,7 @@ __global__ __launch_bounds__(64) void prefill_merge_kernel(const float *__restri
 // last) are cut into k = floor(256 / their number) pieces each, which still fit one round and take a k-th of
 // the time; their rows are then folded from the pieces by prefill_piece_merge_kernel.  gh query heads per
 // workgroup (the largest divisor of the heads per kv head that divides 128), so that no row of a workgroup idles.
+constexpr int kD256MaxPieces = 32;                  // per walk: the merge gives a piece a lane of half a wave
 struct D256Shape { int gh, tpw, nqt, walks, n_full, tail, kparts; };
 static D256Shape d256_shape(const Lay &a, int pos_start, int M, int pieces)      // pieces: 0 none, 1 by the rule, 2 whenever a last round exists
 {
@@ -3085,7 +3095,7 @@ static D256Shape d256_shape(const Lay &a, int pos_start, int M, int pieces)     
     s.walks = s.nqt * a.KVH * (G / s.gh);
     s.tail = s.walks % 256;
     s.kparts = (pieces && s.tail > 0) ? 256 / s.tail : 1;
-    if (s.kparts > 8) s.kparts = 8;
+    if (s.kparts > kD256MaxPieces) s.kparts = kD256MaxPieces;
     // a piece should be worth its start-up and the merge: eight tiles or more of the longest walk that is cut
     // (the last round holds the shortest walks: the first row blocks of the chunk)
     const int qt_tail = s.nqt - 1 - (s.walks - s.tail) / (a.KVH * (G / s.gh));
@@ -3115,11 +3125,11 @@ __global__ __launch_bounds__(64) void prefill_piece_merge_kernel(PrefillArgs A, 
     const float pm = (lane < A.kparts && pl > 0.0f) ? A.part_m[p0 + lane] : -INFINITY;
     float M = pm;
 #pragma unroll
-    for (int off = 4; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
+    for (int off = kD256MaxPieces / 2; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
     const float w = pl > 0.0f ? __builtin_amdgcn_exp2f(pm - M) : 0.0f;
     float L = pl * w;
 #pragma unroll
-    for (int off = 4; off > 0; off >>= 1) L += __shfl_xor(L, off);
+    for (int off = kD256MaxPieces / 2; off > 0; off >>= 1) L += __shfl_xor(L, off);
     M = pm_lane(M, 0);
     L = pm_lane(L, 0);
     if (A.lse_rows && lane == 0) A.lse_rows[row] = L > 0.0f ? M + __builtin_log2f(L) : INFINITY;
@@ -3169,11 +3179,15 @@ static void prefill_split_shape(const Lay &a, int pos_start, int M, int *chunk_t
 // keeps every CU busy.  Rows behind 2k / 32k / 128k tokens, chunk kernel -> split:
 //   16: 59 -> 18, 878 -> 42, 3 992 -> 115 us;  256: 66 -> 37, 868 -> 211, 3 857 -> 799 us;
 //   1 024: 92 -> 98, 928 -> 715, 3 896 -> 2 566 us.
+static bool d256_direct(const Lay &a);
 static bool prefill_split_applies(const Lay &a, int pos_start, int M)
 {
-    (void)a;
     if (g_prefill_split == 0 || pos_start < kSplitMinPos) return false;
     if (g_prefill_split > 0) return M <= g_prefill_split;
+    // head_dim 256 on 16-bit pages: the chunk kernel cuts its walks into up to 32 pieces each and fills the chip that
+    // way, faster than this path's kernel at every chunk length (16 rows behind 32k tokens 69 against 73 us, 256 rows
+    // 210 against 596, 1 024 rows 895 against 1 993)
+    if (d256_direct(a) && g_prefill_pieces != 0) return false;
     return M <= 512 || (M <= kSplitMaxM && pos_start >= 2 * kSplitMinPos);
 }
 
@@ -3239,6 +3253,7 @@ extern "C" {
 void drk_debug_set_prefill_split(int max_rows) { g_prefill_split = max_rows < 0 ? -1 : max_rows; }
 void drk_debug_set_prefill_d256_waves(int mode) { g_prefill_d256_waves = mode != 0 ? 1 : 0; }
 void drk_debug_set_prefill_mass_direct(int on) { g_prefill_mass_direct = on != 0 ? 1 : 0; }
+void drk_debug_set_prefill_mass_parts(int parts) { g_prefill_mass_parts = parts < 0 ? 0 : (parts > 4096 ? 4096 : parts); }
 void drk_debug_set_prefill_pieces(int mode) { g_prefill_pieces = mode < 0 ? 1 : (mode > 2 ? 2 : mode); }
 static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_block_table,
                              int layer, int pos_start, int M, float scale, int io_dtype, const float *d_row_lse,
@@ -3282,7 +3297,14 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
     if (g_prefill_mass_direct && d_row_lse && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 &&
         (pos_start + M + a.bs - 1) / a.bs <= (a.D == 128 ? kMassdBlocks<128> : kMassdBlocks<256>) && a.QH / a.KVH <= 128) {
         A.tpw = 256 / (a.QH / a.KVH);
-        const dim3 gridd(((M + A.tpw - 1) / A.tpw) * a.KVH);
+        A.nqt = (M + A.tpw - 1) / A.tpw;
+        // few walks (a short chunk): every walk's tiles in parts, so that the workgroups fill the chip once (one
+        // per CU: the LDS ring), a part no shorter than eight tiles
+        const int walks = A.nqt * a.KVH;
+        const int tiles = (pos_start + M + kPfBN - 1) / kPfBN;
+        A.kparts = g_prefill_mass_parts > 0 ? g_prefill_mass_parts : std::max(1, std::min(256 / walks, tiles / 8));
+        A.gh = 0; A.n_full = 0;
+        const dim3 gridd((unsigned)(walks * A.kparts));
         const bool fold = chunk_kernel_scales_q(a, pos_start, M);
 #define DRK_PMD(DT, DD)                                                                                                   \
         do {                                                                                                             \

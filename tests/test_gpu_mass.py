@@ -237,6 +237,43 @@ def test_frame_mass_from_the_attention_calls_row_sums(dev, chunk_path, mass_kern
         assert np.all(np.isfinite(rows[t])) if sees else np.all(np.isposinf(rows[t]))
 
 
+@pytest.mark.parametrize("parts", [0, 3, 40])
+@pytest.mark.parametrize("dtype,bs,pos_start,M,heads,holes", [
+    (cabi.BF16, 16, 3000, 20, (8, 32, 128), (7, 150)), (cabi.F16, 256, 2100, 33, (4, 24, 256), (2,)),
+    (cabi.F16, 32, 700, 260, (2, 14, 128), ()), (cabi.BF16, 64, 0, 130, (1, 6, 256), (1,))])
+def test_frame_mass_with_the_context_in_parts(dev, parts, dtype, bs, pos_start, M, heads, holes):
+    """A short frame behind a long context has few walks; the one-walk kernel for 16-bit pages cuts them into parts
+    (by its rule: 16-tile parts for the first case; forced: 3 and 40 per walk, more parts than some walks have tiles).
+    Masses against fp64 and against the same call with whole walks."""
+    lib = cabi.lib()
+    g, og, io, table, opool, q = _frame_case(dtype, bs, seed=bs + M, pos_start=pos_start, M=M, heads=heads, holes=holes)
+    KVH, QH, D = heads
+    scale = 1.0 / np.sqrt(D)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    ws = U.dev_zeros(max(wsb, 16))
+    out = U.dev_bytes(np.zeros(M * QH * D * 2, dtype=np.uint8))
+    lse = U.dev_bytes(np.zeros(M * QH, np.float32))
+    cabi.call("drk_paged_prefill_attention_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), 1, pos_start, M, float(scale),
+              io, None, 0, U.p(lse), U.p(ws), wsb, U.stream_ptr())
+    got = []
+    try:
+        for p in (parts, 1):
+            lib.drk_debug_set_prefill_mass_parts(p)
+            mass = U.dev_bytes(np.full(table.size, 7.0, np.float32))
+            cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale),
+                      io, U.p(lse), U.p(mass), table.size, 0, U.stream_ptr())
+            U.sync()
+            got.append(U.host(mass, np.float32).astype(np.float64))
+    finally:
+        lib.drk_debug_set_prefill_mass_parts(0)
+    want = _frame_want(og, io, table, opool, q, pos_start, scale)
+    assert np.all(np.abs(got[0] - want) <= 2e-3 * M + 3e-3 * np.abs(want)), np.abs(got[0] - want).max()
+    assert np.all(np.abs(got[0] - got[1]) <= 1e-4 * M + 1e-4 * np.abs(got[1])), np.abs(got[0] - got[1]).max()
+    for h in holes:
+        assert got[0][h] == 0.0
+
+
 def test_frame_mass_of_a_long_chunk(dev):
     """A 300-token frame behind 3 000 tokens (several row tiles per kv head meeting in every page)."""
     pos_start, M, bs = 3000, 300, 16
