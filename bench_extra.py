@@ -1022,6 +1022,28 @@ def kernel_fractions(buf, seed=11):
                           "attention alone; followed by the mass pass that walks the keys twice; by the pass that takes the rows' "
                           "log-sum-exps from the attention call and walks once; and with that pass on a second stream behind an "
                           "event, back to back launches (the next attention call waits for the pass, which reads its Q)"}
+    # a short frame behind the same context: 64 rows at 32 704 (the split path for the attention, the mass pass with its
+    # walks in parts)
+    big = (q, o, lse, chunk, pos)
+    chunk = 64
+    pos = total - chunk
+    q = torch.randn(chunk, QH, D, device="cuda").to(torch.bfloat16)
+    o = torch.empty_like(q)
+    lse = torch.empty(chunk * QH, dtype=torch.float32, device="cuda")
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos, chunk)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+
+    def short_attn():
+        cabi.call("drk_paged_prefill_attention_lse", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, pos, chunk, scale,
+                  cabi.BF16, None, 0, cabi.p(lse), cabi.p(ws), wsb, sp)
+
+    def short_both():
+        short_attn()
+        cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), 0, pos, chunk, scale,
+                  cabi.BF16, cabi.p(lse), cabi.p(mass), total // bs, 1, sp)
+
+    frame_mass["short_frame_64_rows"] = {"attention_us": timed(short_attn), "with_one_walk_mass_us": timed(short_both)}
+    q, o, lse, chunk, pos = big
     cabi.call("drk_event_destroy", ev_a)
     cabi.call("drk_event_destroy", ev_m)
     res["frame_mass"] = frame_mass

@@ -315,8 +315,11 @@ int drk_kv_append_decode_planned(const drk_kv_layout *g, void *pool, const int32
  * drk_paged_decode_attention_shared, rows = the chunk's tokens, then a merge -- when the
  * workspace drk_prefill_workspace_bytes reports for it is passed (16-byte aligned, up to
  * ~35 MB at 32 query heads x 128); without it the unsplit kernel does the work, up to 30
- * times slower for a chunk of a few tokens behind a long context.  Anything else runs row by row through the portable decode kernel, which needs
- * the workspace. */
+ * times slower for a chunk of a few tokens behind a long context.  Head_dim 256 on 16-bit pages
+ * (blocks of 16 * 2^k tokens) does not take that path: its chunk kernel cuts the walks of a round
+ * that does not fill the chip into up to 32 pieces each and merges them, with the same workspace
+ * call (up to 33.8 MB).  Anything else runs row by row through the portable decode kernel, which
+ * needs the workspace. */
 size_t drk_prefill_workspace_bytes(const drk_kv_layout *g, int pos_start, int M);
 /* The most drk_prefill_workspace_bytes reports for any chunk of up to max_rows rows that
  * ends at or before max_seq_len tokens: what a caller reserves once, up front.  (Both sizes follow the
@@ -432,8 +435,11 @@ int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, cons
  * token) -- the chunk kernels know it where a row's walk ends.  drk_paged_prefill_attention_mass_lse is the mass
  * pass given those values: it reads K once.  It may run on another stream behind an event (it reads q, the pages
  * and d_row_lse; nothing the attention call wrote except d_row_lse).  Head_dim 128 or 256, block_size % 16 == 0;
- * DRK_ERR_UNSUPPORTED otherwise.  The two calls round Q differently for some chunk lengths (the long-chunk kernels
- * fold the scale into Q in its 16-bit type): a row's masses then sum to 1 within 2e-3 instead of 1e-6. */
+ * DRK_ERR_UNSUPPORTED otherwise.  Over 16-bit pages (blocks of 16 * 2^k tokens, up to 8 192 / 6 144 blocks of context
+ * at head_dim 128 / 256) the pass scores the way the attention call did and a row's masses sum to 1 within 1e-6;
+ * over 8-bit pages the two calls round Q differently for some chunk lengths (the long-chunk kernels fold the scale
+ * into Q in its 16-bit type) and the sum is 1 within 2e-3.  d_row_lse must come from the attention call for the same
+ * chunk with the library's debug switches unchanged in between. */
 int drk_paged_prefill_attention_lse(const drk_kv_layout *g, const void *q, const void *pool,
                                     const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
                                     float scale, int io_dtype, const void *gate, size_t gate_stride,
