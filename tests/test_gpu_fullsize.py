@@ -264,6 +264,74 @@ def test_reference_model_shape_full_chunk_prefill_rows(dev):
         assert ok, (mode, ma)
 
 
+@pytest.mark.parametrize("shape", ["config5", "reference_model"])
+def test_full_chunk_frame_mass(dev, shape):
+    """The attention mass of a full 2 048-token chunk at position 30 720 (config 5's shape, and the reference model's):
+    the attention call leaves the rows' log-sum-exps, the one-walk pass adds every row's probabilities up by page.
+    Against fp32 softmax in torch over the stored K (all 2 048 x QH rows over 32 768 keys, summed per block), the
+    pages of the whole context sum to rows x heads, and the register-staging kernel gives the same masses."""
+    torch = _torch()
+    if shape == "config5":
+        L, KVH, QH, D, bs, dt, tdt, amp = 1, 8, 32, 128, 16, cabi.BF16, torch.bfloat16, 1.0
+    else:
+        L, KVH, QH, D, bs, dt, tdt, amp = 1, 4, 24, 256, 256, cabi.F16, torch.float16, 0.5
+    total, M = 32768, 2048
+    pos_start = total - M
+    NB = total // bs
+    g = cabi.layout(L, KVH, QH, D, bs, NB, dt)
+    lib = cabi.lib()
+    rng = np.random.default_rng(11)
+    table = torch.from_numpy(rng.permutation(NB).astype(np.int32)).cuda()
+    pool = torch.zeros(lib.drk_kv_pool_bytes(C.byref(g)), dtype=torch.uint8, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(23)
+    sp = U.stream_ptr()
+    for p0 in range(0, total, 8192):
+        k = (torch.randn(8192, KVH, D, device="cuda", generator=gen) * amp).to(tdt)
+        v = (torch.randn(8192, KVH, D, device="cuda", generator=gen) * amp).to(tdt)
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(table), 0, 1, p0, 8192, U.p(k), U.p(v), dt, sp)
+        U.sync()
+    q = (torch.randn(M, QH, D, device="cuda", generator=gen) * amp).to(tdt)
+    out = torch.zeros_like(q)
+    scale = 1 / np.sqrt(D)
+    lse = torch.zeros(M * QH, dtype=torch.float32, device="cuda")
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    ws = torch.zeros(max(wsb, 16), dtype=torch.uint8, device="cuda")
+    cabi.call("drk_paged_prefill_attention_lse", C.byref(g), U.p(q), U.p(pool), U.p(table), U.p(out), 0, pos_start, M,
+              float(scale), dt, None, 0, U.p(lse), U.p(ws), wsb, sp)
+    got = {}
+    try:
+        for direct in (1, 0):
+            lib.drk_debug_set_prefill_mass_direct(direct)
+            mass = torch.full((NB,), 7.0, dtype=torch.float32, device="cuda")
+            cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), U.p(q), U.p(pool), U.p(table), 0, pos_start, M,
+                      float(scale), dt, U.p(lse), U.p(mass), NB, 0, sp)
+            U.sync()
+            got[direct] = mass.double().cpu().numpy()
+    finally:
+        lib.drk_debug_set_prefill_mass_direct(1)
+    flat = torch.empty(2 * total * KVH * D, dtype=tdt, device="cuda")
+    cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(pool), U.p(table), 0, total, 1, sp)
+    U.sync()
+    kk = flat.view(2, total, KVH, D)[0].float()
+    G = QH // KVH
+    keys = torch.arange(total, device="cuda")
+    want = torch.zeros(total, dtype=torch.float64, device="cuda")
+    for h in range(KVH):
+        for r0 in range(0, M, 512):                          # 512 rows x G heads x 32 768 keys of fp32 scores at a time
+            qq = q[r0:r0 + 512, h * G:(h + 1) * G].float()
+            sc = torch.einsum("tgd,kd->tgk", qq, kk[:, h]) * scale
+            vis = keys[None, None, :] <= (pos_start + r0 + torch.arange(qq.shape[0], device="cuda"))[:, None, None]
+            sc = sc.masked_fill(~vis, float("-inf"))
+            want += torch.softmax(sc, dim=-1).double().sum(dim=(0, 1))
+    want = want.view(NB, bs).sum(dim=1).cpu().numpy()
+    assert abs(want.sum() - M * QH) < 1e-3 * M * QH
+    for direct in (1, 0):
+        err = np.abs(got[direct] - want)
+        assert np.all(err <= 2e-2 * np.abs(want) + 5e-2), (direct, err.max(), want[err.argmax()])
+    assert abs(got[1].sum() - M * QH) <= 1e-4 * M * QH       # scored as the attention call scored: the rows' masses sum to 1
+    assert abs(got[0].sum() - M * QH) <= 2e-3 * M * QH
+
+
 @pytest.mark.parametrize("dtype", [cabi.BF16, cabi.INT8])
 def test_pages_beyond_4GiB_of_a_layer(dev, dtype):
     """A pool whose single layer holds more than 4 GiB (a 288 GB part at 36 layers has 7 GiB per
