@@ -2332,8 +2332,10 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
     walk(std::true_type{});
 }
 
-// ---- attention mass of a chunk, 16-bit pages, the rows' log-sum-exps given: tiles straight into LDS ----------
-// The one-walk case of prefill_mass_kernel rebuilt on the chunk kernels' machinery: 256 rows per workgroup (eight
+// ---- attention mass of a chunk, 16-bit pages: tiles straight into LDS ----------------------------------------
+// prefill_mass_kernel rebuilt on the chunk kernels' machinery (one walk when the rows' log-sum-exps are given; TWO:
+// the workgroup first walks its keys for them, a lane keeping a lazy running maximum and sum per row over the keys
+// it sees, the 32 lanes of a row meeting once between the walks): 256 rows per workgroup (eight
 // waves of 32, two per SIMD), K tiles from global memory straight into a ring of four swizzled LDS buffers,
 // requested two tiles ahead between the k-steps, one barrier per tile; the products start from minus the row's
 // log-sum-exp (the C operand), so a score arrives as the exponent of its probability, and the exponentials of tile t
@@ -2351,7 +2353,7 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
 // logical blocks in pos_start + M tokens.
 template <int D>
 constexpr int kMassdBlocks = D == 128 ? 8192 : 6144;
-template <int DT, int IO, int D, bool FOLD>
+template <int DT, int IO, int D, bool FOLD, bool TWO>
 __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, float *__restrict__ mass, int mass_len)
 {
     constexpr int RB = D * 2;
@@ -2416,8 +2418,12 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         const int tq = qt * TPW + rt;
         const bool live = rt < TPW && tq < A.M;
         vis[i] = live ? A.pos_start + tq + 1 : 0;
-        const float lse = live ? A.lse_rows[(size_t)tq * A.QH + kvh * G + (r - rt * G)] : INFINITY;
-        negl[i] = FOLD ? -lse : -lse / A.scale_log2e;
+        if constexpr (!TWO) {
+            const float lse = live ? A.lse_rows[(size_t)tq * A.QH + kvh * G + (r - rt * G)] : INFINITY;
+            negl[i] = FOLD ? -lse : -lse / A.scale_log2e;
+        } else {
+            negl[i] = 0.0f;                                  // the first walk's products start from zero
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // from here on the kernel counts its loads itself
 
@@ -2490,87 +2496,138 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         }
     };
 
-    // ---- prologue: K(t0), K(t0 + 1), K(t0 + 2) requested and there, the scores of tile t0 ----
-    int blk_ahead;
-    {
-        const int b0 = page_of(t0), b1 = page_of(t0 + 1), b2 = page_of(t0 + 2);
-        blk_ahead = page_of(t0 + 3);
-        __syncthreads();                                     // the clearing is done (and the table entries are here)
-        plan(t0, b0);
-        request_tile();
-        plan(t0 + 1, b1);
-        request_tile();
-        plan(t0 + 2, b2);
-        request_tile();
-        __builtin_amdgcn_s_waitcnt(0x0f70);                  // vmcnt(0)
-    }
-    __syncthreads();
-    pf_f32x16 s_even[2], s_odd[2];
-    qk(t0 & (kRing - 1), s_even, [](int) {});
-    // bit r: the tile's 8-token run r has a page; read one tile ahead, between the products
-    auto flags_of = [&](const int4 &a, const int4 &b) -> int {
-        return __builtin_amdgcn_readfirstlane(a.x | (a.y << 1) | (a.z << 2) | (a.w << 3) | (b.x << 4) | (b.y << 5) | (b.z << 6) | (b.w << 7));
-    };
-    int flags = flags_of(*(const int4 *)&valid_ldsm[t0 & (kRing - 1)][0], *(const int4 *)&valid_ldsm[t0 & (kRing - 1)][4]);
-
-    // the page sums of tile `tile_t` from the lanes' key sums: a key's other 16 rows are in the other half of the
-    // wave; a block is 16 keys or more
-    auto fold = [&](int tile_t, const float (&cs)[2]) {
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++) {
-            const auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(cs[tt]), __float_as_uint(cs[tt]), false, false);
-            const float c16 = pf_row16_sum(__uint_as_float(r2[0]) + __uint_as_float(r2[1]));
-            const int run0 = tile_t + tt * 32 + (n & 16);
-            if (g == 0 && (n & 15) == 0 && run0 >= t0 * kPfBN && run0 < lim_part && c16 != 0.0f) atomicAdd(&mass_ldsm[(run0 >> sh) - lb0], c16);
+    // One walk over the part's tiles.  LSE: the first of two walks -- every lane keeps a running maximum and sum per
+    // row over the keys it sees, in units of the exponent; the second (or only) walk adds the probabilities up by key.
+    const float cexp = FOLD ? 1.0f : A.scale_log2e;
+    float m_run[16], l_run[16];
+    auto run_walk = [&](auto lse_mode) {
+        constexpr bool LSE = decltype(lse_mode)::value;
+        // ---- prologue: K(t0), K(t0 + 1), K(t0 + 2) requested and there, the scores of tile t0 ----
+        int blk_ahead;
+        {
+            const int b0 = page_of(t0), b1 = page_of(t0 + 1), b2 = page_of(t0 + 2);
+            blk_ahead = page_of(t0 + 3);
+            __syncthreads();                                     // the clearing is done (and the table entries are here)
+            plan(t0, b0);
+            request_tile();
+            plan(t0 + 1, b1);
+            request_tile();
+            plan(t0 + 2, b2);
+            request_tile();
+            __builtin_amdgcn_s_waitcnt(0x0f70);                  // vmcnt(0)
         }
-    };
-    float cs_prev[2] = {0.0f, 0.0f};                         // the key sums of the tile before, folded a step later
-    auto step = [&](int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
-        // here: s = exponents of tile it; K(it + 1) and K(it + 2) requested
-        const int tile_t = it * kPfBN;
-        if (__builtin_expect(flags != 255 || it >= first_masked_tile, 0)) {
+        __syncthreads();
+        pf_f32x16 s_even[2], s_odd[2];
+        qk(t0 & (kRing - 1), s_even, [](int) {});
+        // bit r: the tile's 8-token run r has a page; read one tile ahead, between the products
+        auto flags_of = [&](const int4 &a, const int4 &b) -> int {
+            return __builtin_amdgcn_readfirstlane(a.x | (a.y << 1) | (a.z << 2) | (a.w << 3) | (b.x << 4) | (b.y << 5) | (b.z << 6) | (b.w << 7));
+        };
+        int flags = flags_of(*(const int4 *)&valid_ldsm[t0 & (kRing - 1)][0], *(const int4 *)&valid_ldsm[t0 & (kRing - 1)][4]);
+
+        // the page sums of tile `tile_t` from the lanes' key sums: a key's other 16 rows are in the other half of the
+        // wave; a block is 16 keys or more
+        auto fold = [&](int tile_t, const float (&cs)[2]) {
 #pragma unroll
             for (int tt = 0; tt < 2; tt++) {
-                const int key = tile_t + tt * 32 + n;
-                const bool kvalid = ((flags >> ((tt * 32 + n) >> 3)) & 1) != 0;
-#pragma unroll
-                for (int i = 0; i < 16; i++) s[tt][i] = (kvalid && key < vis[i]) ? s[tt][i] : -INFINITY;
+                const auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(cs[tt]), __float_as_uint(cs[tt]), false, false);
+                const float c16 = pf_row16_sum(__uint_as_float(r2[0]) + __uint_as_float(r2[1]));
+                const int run0 = tile_t + tt * 32 + (n & 16);
+                if (g == 0 && (n & 15) == 0 && run0 >= t0 * kPfBN && run0 < lim_part && c16 != 0.0f) atomicAdd(&mass_ldsm[(run0 >> sh) - lb0], c16);
             }
+        };
+        float cs_prev[2] = {0.0f, 0.0f};                         // the key sums of the tile before, folded a step later
+        constexpr float kLazy = 8.0f;
+        auto step = [&](int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
+            // here: s = exponents of tile it; K(it + 1) and K(it + 2) requested
+            const int tile_t = it * kPfBN;
+            if (__builtin_expect(flags != 255 || it >= first_masked_tile, 0)) {
+#pragma unroll
+                for (int tt = 0; tt < 2; tt++) {
+                    const int key = tile_t + tt * 32 + n;
+                    const bool kvalid = ((flags >> ((tt * 32 + n) >> 3)) & 1) != 0;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) s[tt][i] = (kvalid && key < vis[i]) ? s[tt][i] : -INFINITY;
+                }
+            }
+            if constexpr (LSE) {
+                // a lane's running maximum per row over the keys it has seen moves only when a score exceeds it by kLazy
+                // (in units of the exponent): the common tile costs sixteen maxima and compares
+                bool mv = false;
+#pragma unroll
+                for (int i = 0; i < 16; i++) mv = mv || fmaxf(s[0][i], s[1][i]) * cexp > m_run[i] + kLazy;
+                if (__builtin_expect(__any(mv), 0)) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const float x = fmaxf(s[0][i], s[1][i]) * cexp;
+                        const float m_new = x > m_run[i] + kLazy ? x : m_run[i];
+                        l_run[i] *= __builtin_amdgcn_exp2f(m_run[i] - m_new);
+                        m_run[i] = m_new;
+                    }
+                }
+            }
+            // K(it + 1) has landed (this wave's share; the requests of K(it + 2) came after it), then everybody's
+            if (__builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
+            else __builtin_amdgcn_s_waitcnt(0x0f70);
+            pf_barrier_lds();
+            asm volatile("" : : "s"(blk_ahead));
+            plan(it + 3, blk_ahead);                             // into the buffer of K(it - 1), read two steps ago
+            blk_ahead = page_of(it + 4);
+            whole = p_rows >= ROWS;                              // requested between the products below
+            float cs[2] = {0.0f, 0.0f};
+            int4 fa, fb;
+            qk((it + 1) & (kRing - 1), s_next, [&](int ks) {
+                if (ks == 0) {
+                    fa = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][0];
+                    fb = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][4];
+                }
+                if ((ks & 1) == 0 && (ks >> 1) < NREQ) request(ks >> 1);
+                if constexpr (!LSE) {
+                    if (ks == NKS / 2) fold(tile_t - kPfBN, cs_prev);
+                }
+#pragma unroll
+                for (int u = 0; u < EPK; u++) {
+                    const int j = ks * EPK + u, tt = j >> 4, i = j & 15;
+                    if constexpr (LSE) {
+                        l_run[i] += __builtin_amdgcn_exp2f(s[tt][i] * cexp - m_run[i]);
+                        asm volatile("" : "+v"(l_run[i]));
+                    } else {
+                        const float e = __builtin_amdgcn_exp2f(FOLD ? s[tt][i] : s[tt][i] * A.scale_log2e);
+                        cs[tt] += e;
+                        asm volatile("" : "+v"(cs[tt]));         // the sum stays here, in the shadow of the products
+                    }
+                }
+            });
+            flags = flags_of(fa, fb);
+            cs_prev[0] = cs[0];
+            cs_prev[1] = cs[1];
+        };
+        for (int it = t0; it < ntiles; it += 2) {
+            step(it, s_even, s_odd);
+            if (it + 1 < ntiles) step(it + 1, s_odd, s_even);
         }
-        // K(it + 1) has landed (this wave's share; the requests of K(it + 2) came after it), then everybody's
-        if (__builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
-        else __builtin_amdgcn_s_waitcnt(0x0f70);
-        pf_barrier_lds();
-        asm volatile("" : : "s"(blk_ahead));
-        plan(it + 3, blk_ahead);                             // into the buffer of K(it - 1), read two steps ago
-        blk_ahead = page_of(it + 4);
-        whole = p_rows >= ROWS;                              // requested between the products below
-        float cs[2] = {0.0f, 0.0f};
-        int4 fa, fb;
-        qk((it + 1) & (kRing - 1), s_next, [&](int ks) {
-            if (ks == 0) {
-                fa = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][0];
-                fb = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][4];
-            }
-            if ((ks & 1) == 0 && (ks >> 1) < NREQ) request(ks >> 1);
-            if (ks == NKS / 2) fold(tile_t - kPfBN, cs_prev);
-#pragma unroll
-            for (int u = 0; u < EPK; u++) {
-                const int j = ks * EPK + u, tt = j >> 4, i = j & 15;
-                const float e = __builtin_amdgcn_exp2f(FOLD ? s[tt][i] : s[tt][i] * A.scale_log2e);
-                cs[tt] += e;
-                asm volatile("" : "+v"(cs[tt]));             // the sum stays here, in the shadow of the products
-            }
-        });
-        flags = flags_of(fa, fb);
-        cs_prev[0] = cs[0];
-        cs_prev[1] = cs[1];
+        if constexpr (!LSE) fold((ntiles - 1) * kPfBN, cs_prev);
     };
-    for (int it = t0; it < ntiles; it += 2) {
-        step(it, s_even, s_odd);
-        if (it + 1 < ntiles) step(it + 1, s_odd, s_even);
+    if constexpr (TWO) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) { m_run[i] = -1.0e30f; l_run[i] = 0.0f; }
+        run_walk(std::true_type{});
+        // a row's lanes (the 32 of its half of the wave) meet: lse = M + log2(sum l 2^(m - M)); +inf for a row that
+        // saw nothing.  The second walk's products start from -lse in units of the product.
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float mm = m_run[i];
+#pragma unroll
+            for (int off = 1; off < 32; off <<= 1) mm = fmaxf(mm, __shfl_xor(mm, off));
+            float ll = l_run[i] * __builtin_amdgcn_exp2f(m_run[i] - mm);
+#pragma unroll
+            for (int off = 1; off < 32; off <<= 1) ll += __shfl_xor(ll, off);
+            const float lse = (vis[i] > 0 && ll > 0.0f) ? mm + __builtin_log2f(ll) : INFINITY;
+            negl[i] = -lse / cexp;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
     }
-    fold((ntiles - 1) * kPfBN, cs_prev);
+    run_walk(std::false_type{});
     __builtin_amdgcn_s_waitcnt(0x0f70);                      // nothing is on its way when the workgroup ends
     __syncthreads();
     for (int i = threadIdx.x; i < nblk_wg; i += 512) {
@@ -3293,8 +3350,9 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
     A.seq_lens = nullptr; A.shared = 0; A.chunk_tiles = 0; A.nsplits = 0; A.part_o = A.part_m = A.part_l = nullptr;
     A.gate = nullptr; A.gate_stride = 0;
     A.lse_rows = const_cast<float *>(d_row_lse);             // read only here: the rows' log-sum-exps, or NULL (first walk finds them)
-    // 16-bit pages with the rows' log-sum-exps given: the kernel that takes its tiles straight into LDS
-    if (g_prefill_mass_direct && d_row_lse && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 &&
+    // 16-bit pages: the kernel that takes its tiles straight into LDS -- one walk when the rows' log-sum-exps are
+    // given, else two by the same workgroup (whole walks then: the first must see every key)
+    if (g_prefill_mass_direct && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 &&
         (pos_start + M + a.bs - 1) / a.bs <= (a.D == 128 ? kMassdBlocks<128> : kMassdBlocks<256>) && a.QH / a.KVH <= 128) {
         A.tpw = 256 / (a.QH / a.KVH);
         A.nqt = (M + A.tpw - 1) / A.tpw;
@@ -3302,14 +3360,15 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
         // per CU: the LDS ring), a part no shorter than eight tiles
         const int walks = A.nqt * a.KVH;
         const int tiles = (pos_start + M + kPfBN - 1) / kPfBN;
-        A.kparts = g_prefill_mass_parts > 0 ? g_prefill_mass_parts : std::max(1, std::min(256 / walks, tiles / 8));
+        A.kparts = !d_row_lse ? 1 : (g_prefill_mass_parts > 0 ? g_prefill_mass_parts : std::max(1, std::min(256 / walks, tiles / 8)));
         A.gh = 0; A.n_full = 0;
         const dim3 gridd((unsigned)(walks * A.kparts));
-        const bool fold = chunk_kernel_scales_q(a, pos_start, M);
+        const int kind = !d_row_lse ? 2 : (chunk_kernel_scales_q(a, pos_start, M) ? 1 : 0);
 #define DRK_PMD(DT, DD)                                                                                                   \
         do {                                                                                                             \
-            if (fold) hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, true>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
-            else hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, false>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
+            if (kind == 2) hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, false, true>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
+            else if (kind == 1) hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, true, false>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
+            else hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, false, false>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
         } while (0)
         if (a.dtype == DRK_BF16 && a.D == 128) DRK_PMD(DRK_BF16, 128);
         else if (a.dtype == DRK_BF16) DRK_PMD(DRK_BF16, 256);

@@ -55,7 +55,7 @@ void drk_debug_set_prefill_pieces(int mode);
  * and a value wave (V^T P^T) per 32 rows; 0 = four waves, each does both products of its 32 rows.  Same walks,
  * same pieces, same bits. */
 void drk_debug_set_prefill_d256_waves(int mode);
-/* One-walk mass pass (drk_paged_prefill_attention_mass_lse) over 16-bit pages: 1 (default) = the kernel that takes
+/* Mass passes (drk_paged_prefill_attention_mass[_lse]) over 16-bit pages: 1 (default) = the kernel that takes
  * 256 rows per workgroup and its K tiles straight into LDS (blocks of 16 * 2^k tokens, up to 8 192 / 6 144 logical
  * blocks at head_dim 128 / 256); 0 = the register-staging kernel, which also serves every other case. */
 void drk_debug_set_prefill_mass_direct(int on);

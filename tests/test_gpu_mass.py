@@ -113,6 +113,15 @@ def test_block_mass_argument_errors(dev):
 
 # ---- perception frames: the mass a chunk of query tokens gives to the pages of the context ----------------
 
+@pytest.fixture(params=["tiles_straight_into_lds", "tiles_through_registers"])
+def mass_kernel(request):
+    """The two one-walk mass kernels for 16-bit pages (8-bit pages have the second only)."""
+    lib = cabi.lib()
+    lib.drk_debug_set_prefill_mass_direct(1 if request.param == "tiles_straight_into_lds" else 0)
+    yield request.param
+    lib.drk_debug_set_prefill_mass_direct(1)
+
+
 def _frame_case(dtype, bs, seed, pos_start, M, heads=(8, 32, 128), holes=()):
     L = 2
     KVH, QH, D = heads
@@ -145,7 +154,7 @@ def _frame_want(og, io, table, opool, q, pos_start, scale):
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
 @pytest.mark.parametrize("bs,pos_start,M,heads", [(16, 0, 1, (8, 32, 128)), (16, 0, 70, (8, 32, 128)), (16, 333, 45, (8, 32, 128)),
                                                   (32, 500, 130, (2, 12, 128)), (256, 100, 33, (4, 24, 256)), (48, 64, 64, (2, 2, 128))])
-def test_frame_mass_matches_fp64(dev, dtype, bs, pos_start, M, heads):
+def test_frame_mass_matches_fp64(dev, mass_kernel, dtype, bs, pos_start, M, heads):
     """drk_paged_prefill_attention_mass against the fp64 oracle (rows of the frame as causal branches): 8-bit
     pages, head_dim 256, 1 / 4 / 6 query heads per kv head, block sizes that are not powers of two, a missing
     page, stale entries in the output array; the entries add up to M x num_q_heads minus nothing."""
@@ -183,15 +192,6 @@ def chunk_path(request):
     yield request.param
     lib.drk_debug_set_prefill_two_phase(1)
     lib.drk_debug_set_prefill_split(-1)
-
-
-@pytest.fixture(params=["tiles_straight_into_lds", "tiles_through_registers"])
-def mass_kernel(request):
-    """The two one-walk mass kernels for 16-bit pages (8-bit pages have the second only)."""
-    lib = cabi.lib()
-    lib.drk_debug_set_prefill_mass_direct(1 if request.param == "tiles_straight_into_lds" else 0)
-    yield request.param
-    lib.drk_debug_set_prefill_mass_direct(1)
 
 
 @pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
