@@ -213,6 +213,7 @@ def config3(args):
     shared_now, groups_now = [0], [[], cabi.prefix_groups([])]
     # the unit descriptors of the grouped kernel, built once per step for the 36 layers
     plan_bytes = lib.drk_decode_plan_bytes(C.byref(g), B, max_ctx, cabi.MAX_PREFIX_GROUPS) if grouped and not getattr(args, "no_plan", False) else 0
+    fused_append = bool(plan_bytes) and not getattr(args, "no_fused_append", False)
     plan = torch.empty(max(plan_bytes, 16), dtype=torch.uint8, device="cuda")
     dpos = torch.zeros(B, dtype=torch.int32, device="cuda")
     dlen = torch.zeros(B, dtype=torch.int32, device="cuda")
@@ -261,6 +262,12 @@ def config3(args):
             cabi.call("drk_decode_plan_build", C.byref(g), dtabs, stride, cabi.p(dlen), B, max_ctx, groups_now[1],
                       len(groups_now[0]), cabi.p(plan), plan_bytes, sp)
         for l in range(L):
+            if fused_append:                                      # the attention launch writes the new rows itself
+                cabi.call("drk_kv_append_decode_planned", C.byref(g), pool_ptr, dtabs, stride, cabi.p(dlen), B, max_ctx,
+                          groups_now[1], len(groups_now[0]), cabi.p(plan), C.c_void_p(nk.data_ptr() + l * krow),
+                          C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, C.c_void_p(q.data_ptr() + l * qrow),
+                          C.c_void_p(out.data_ptr() + l * qrow), l, float(scale), cabi.BF16, None, 0, cabi.p(ws), wsb, sp)
+                continue
             cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, cabi.p(dpos), B, l, 1,
                       C.c_void_p(nk.data_ptr() + l * krow), C.c_void_p(nv.data_ptr() + l * krow), cabi.BF16, sp)
             attend(l, cabi.p(dlen))
@@ -317,7 +324,9 @@ def config3(args):
                    "branches": B, "layers": L, "ctx_final": [int(x) for x in lens], "shared_tokens": int(shared_now[0]),
                    "forks": "tree" if tree else "prefix", "fork_parent": parent, "fork_points": fork_points,
                    "shared_ranges": [list(x) for x in groups_now[0]] if grouped else [[0, B, 0, int(shared_now[0])]],
-                   "pool_blocks": NB},
+                   "pool_blocks": NB,
+                   "unit_descriptors": "built once per step" if plan_bytes else "built by every launch",
+                   "append": "written by the attention launch" if fused_append else "a launch of its own"},
         "logical_GB_per_layer_step": round(launch_logical / 1e9, 3),
         "unique_GB_per_layer_step": round(launch_unique / 1e9, 3),
         "resident_GB_per_layer": round(unique_tokens * per_tok / 1e9, 3),

@@ -112,6 +112,7 @@ extern int g_grouped_mode;
 bool grouped_decode_supported(const Lay &a, int B);
 size_t grouped_workspace_need(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups);
 size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_depth);
+bool grouped_decode_writes_new_rows(const Lay &a);        // the grouped kernel for this layout takes DecodePlan::new_k / new_v
 int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables, int table_stride,
                           const int32_t *d_seq_lens, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups,
                           void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,

@@ -753,9 +753,10 @@ int drk_kv_append_decode_planned(const drk_kv_layout *g, void *pool, const int32
     plan.ptr = (uint8_t *)const_cast<void *>(d_plan);
     plan.mode = 2;
     const bool grouped = n_groups > 0 && grouped_decode_supported(a, B);
-    // the plain tiled kernel writes the new rows itself when they are in the pages' own 16-bit type; otherwise the
-    // append is a launch of its own, at position length - 1
-    const bool fused = !grouped && a.E == 2 && src_dtype == a.dtype && (((uintptr_t)new_k | (uintptr_t)new_v) % 16) == 0;
+    // the tiled kernels (plain and grouped) write the new rows themselves when they are in the pages' own 16-bit type;
+    // otherwise the append is a launch of its own, at position length - 1
+    const bool fused = a.E == 2 && src_dtype == a.dtype && (((uintptr_t)new_k | (uintptr_t)new_v) % 16) == 0 &&
+                       (!grouped || grouped_decode_writes_new_rows(a));
     if (fused) {
         plan.new_k = (const uint8_t *)new_k;
         plan.new_v = (const uint8_t *)new_v;

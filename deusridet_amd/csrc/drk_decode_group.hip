@@ -57,6 +57,10 @@ struct GroupedArgs {
     int b_slot[64];                            // first workspace slot of the tail's pieces
     uint8_t *plan;                             // the descriptors of every workgroup in global memory, see DecodePlan
     int plan_mode;                             // 0: build and use; 1: build, store, leave (build_units returns 0); 2: read
+    // or NULL: one new token per branch, [B][KVH][D] of the pages' 16-bit type, written by the workgroup that owns the
+    // last tile of the branch's tail before it reads that tile (decode_group16_kernel only)
+    const uint8_t *new_k, *new_v;
+    uint8_t *pool_layer_w;                     // the layer's pages, writable (with new_k)
 };
 
 struct GUnit {                                 // one 64-token tile of one kv head of a group or a tail
@@ -286,6 +290,26 @@ __global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
     const int GQ = A.QH / A.KVH;
     const int nunits = build_units<kG16MaxUnits>(A, udesc, gdesc, s_incl, s_len, s_gmin);
     if (nunits == 0) return;
+    if (A.new_k) {
+        // The step's append, folded in as in decode_stream_kernel: the unit that is the last tile of a branch's tail
+        // (a tail unit has the rows of one kv head, a shared one those of two branches or more) holds the new token's
+        // position, the page is the branch's own, and only this workgroup reads the tile -- so it writes the row
+        // itself, K and V, 16 bytes per thread, and the barrier orders the stores before every wave's requests.
+        constexpr int CH = D * 2 / 16;
+        for (int i = threadIdx.x; i < nunits * 2 * CH; i += 256) {
+            const int ui = i / (2 * CH), rest = i - ui * (2 * CH), kv = rest / CH, ch = rest - kv * CH;
+            const GUnit ud = udesc[ui];
+            if (((ud.flags >> 8) & 0xff) != GQ || ud.tile_lim < 1 || ud.tile_lim > kSTile) continue;
+            const int r = ud.tile_lim - 1;
+            const uint32_t gx = gdesc[ui][r >> 4].x;
+            if (gx == kNone) continue;
+            const int b = ud.row0 / A.QH, kvh = (ud.row0 - b * A.QH) / GQ;
+            const uint8_t *src = (kv ? A.new_v : A.new_k) + ((size_t)(b * A.KVH + kvh) * D * 2) + ch * 16;
+            uint8_t *dst = A.pool_layer_w + ((size_t)gx << 4) + (size_t)(r & 15) * A.row_bytes + (kv ? A.kv_plane : 0) + ch * 16;
+            *(uint4 *)dst = *(const uint4 *)src;
+        }
+        __syncthreads();
+    }
 
     // ---- requests: lane l of load j fills position l % 16 of row 4j + l / 16 of the wave's slice ----
     const uint32_t dma_row = (uint32_t)((lane >> 4) * 256);
@@ -1112,6 +1136,8 @@ size_t grouped_workspace_need_max(const Lay &a, int B, int max_seq_len, int max_
     return (size_t)B * a.QH * (size_t)P * (a.D + 2) * sizeof(float);
 }
 
+bool grouped_decode_writes_new_rows(const Lay &a) { return a.E == 2 && g_grouped_mode != 2; }
+
 int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *tables, int table_stride,
                           const int32_t *d_seq_lens, int B, int max_seq_len, const drk_prefix_group *groups, int n_groups,
                           void *out, int layer, float scale, int io_dtype, void *workspace, size_t workspace_bytes,
@@ -1161,6 +1187,11 @@ int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *poo
     // 16-bit pages: the tile in LDS, rows dealt to the waves; 8-bit pages (and, as a cross-check, 16-bit pages in
     // diagnostic mode 2): tokens dealt to the waves, K and V through registers
     const bool tile16 = a.E == 2 && g_grouped_mode != 2;
+    const bool fused_append = plan.new_k && plan.new_v && plan.mode != 1;
+    if (fused_append && !tile16) return fail(DRK_ERR_INVALID, "decode_grouped: only the 16-bit tile kernel writes the new rows itself");
+    A.new_k = fused_append ? plan.new_k : nullptr;
+    A.new_v = fused_append ? plan.new_v : nullptr;
+    A.pool_layer_w = (uint8_t *)const_cast<void *>(pool) + (size_t)layer * a.layer_stride;
     switch (a.dtype) {
     case DRK_F16:
         if (tile16) hipLaunchKernelGGL((decode_group16_kernel<DRK_F16>), dim3(P.grid), dim3(256), 0, st, A);

@@ -293,10 +293,12 @@ int drk_paged_decode_attention_planned(const drk_kv_layout *g, const void *q, co
 /* One layer of a decode step in one call: drk_kv_append_branches of one token per branch at position
  * d_seq_lens[b] - 1 (write then attend: the lengths already count the new token; new_k / new_v are
  * [B, num_kv_heads, head_dim] of src_dtype), then drk_paged_decode_attention_planned.  With 16-bit pages, src_dtype
- * equal to the pool's type and no groups it is ONE launch: the workgroup that owns a branch's last tile writes the
- * new rows before it reads the tile (no other workgroup reads them), which takes the append's launch out of every
- * layer; otherwise the append is launched by itself first.  Same bytes in the pool and same output bits as the
- * two calls (tested).  The plan must have been built from these lengths. */
+ * equal to the pool's type and 16-byte aligned sources it is ONE launch, with or without groups: the workgroup that
+ * owns a branch's last tile writes the new rows before it reads the tile, which takes the append's launch out of
+ * every layer; otherwise the append is launched by itself first.  Same bytes in the pool and same output bits as
+ * the two calls (tested).  As for any append, the page that receives a branch's new token must be mapped by that
+ * branch alone (copy-on-write done: CacheManager::ensure_blocks_for sees to it) -- here also because no other
+ * workgroup may be reading it.  The plan must have been built from these lengths. */
 int drk_kv_append_decode_planned(const drk_kv_layout *g, void *pool, const int32_t *d_tables,
                                  int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len,
                                  const drk_prefix_group *groups, int n_groups, const void *d_plan,

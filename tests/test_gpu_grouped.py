@@ -110,6 +110,8 @@ class Tree:
 
 TREE8 = ([(0, 8, 0, 1040), (0, 4, 1040, 2000), (4, 4, 1040, 1216), (0, 2, 2000, 2512)],
          [2512 + 300, 2512, 2000 + 5, 2000 + 700, 1216 + 64, 1216 + 1, 1216 + 1000, 1216 + 130])
+# the same tree with every branch's last token behind the ranges it shares (branch 1 above ends with its range)
+TREE8_OWN_LAST = (TREE8[0], [2512 + 300, 2512 + 1, 2000 + 5, 2000 + 700, 1216 + 64, 1216 + 1, 1216 + 1000, 1216 + 130])
 # forks spread over a prefix: every branch leaves the common context somewhere else
 SPREAD = ([(0, 6, 0, 512), (1, 5, 512, 1024), (2, 4, 1024, 2048), (3, 3, 2048, 2560), (4, 2, 2560, 4096)],
           [512 + 77, 1024 + 1, 2048 + 300, 2560 + 64, 4096 + 5, 4096 + 640])
@@ -272,12 +274,16 @@ def test_plan_argument_errors(dev):
 
 
 @pytest.mark.parametrize("dtype,heads,tree", [(cabi.BF16, (8, 32, 128), ([], TREE8[1])), (cabi.F16, (4, 24, 256), ([], SPREAD[1])),
-                                              (cabi.INT8, (8, 32, 128), ([], TREE8[1])), (cabi.BF16, (8, 32, 128), TREE8),
+                                              (cabi.INT8, (8, 32, 128), ([], TREE8[1])), (cabi.BF16, (8, 32, 128), TREE8_OWN_LAST),
+                                              (cabi.F16, (8, 32, 128), SPREAD), (cabi.FP8_E4M3, (8, 32, 128), TREE8_OWN_LAST),
                                               (cabi.F16, (2, 16, 128), ([], [1, 64, 65, 128, 1000]))])
 def test_append_and_attention_of_a_layer_in_one_call(dev, dtype, heads, tree):
     """drk_kv_append_decode_planned against drk_kv_append_branches + drk_paged_decode_attention_planned: the same bytes
-    in the pool and the same output bits -- in one launch for 16-bit pages without groups (the workgroup that owns a
-    branch's last tile writes the new rows), in two otherwise; a branch whose last page is missing keeps it missing."""
+    in the pool and the same output bits -- in one launch for 16-bit pages (the workgroup that owns a branch's last
+    tile writes the new rows; with fork trees that is a unit of the branch's private tail), in two for 8-bit pages; a
+    branch whose last page is missing keeps it missing.  Every branch's new token lies in a page of its own, as
+    copy-on-write leaves it: a branch that ends where a shared range ends would write into the other branches'
+    context."""
     import torch
     holes = () if tree[0] else ((1, (int(tree[1][1]) - 1) // 16),)
     t = Tree(heads, dtype, tree[0], tree[1], seed=47, holes=holes)
