@@ -913,9 +913,10 @@ __global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_
     __shared__ fvec red[4][64];
     __shared__ int seg_base[kGMaxGroups + 1], seg_cnt[kGMaxGroups + 1], seg_off[kGMaxGroups + 2], nseg_s;
     __shared__ short slot_of[kGMaxPieces];
-    __shared__ int scan_s[3];
     const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6, d = lane * VEC;
-    // tail tiles of every branch: one lane each (one round of loads), folded by the first wave
+    // The pieces of this row: those of every shared range the branch is a member of, in the order of the ranges, then
+    // those of its tail.  One lane per branch scans the tail tiles (one round of loads), then one lane per range (and
+    // one for the tail) works out how many workgroups its run of units was dealt to; a scan gives the offsets.
     if (wv == 0) {
         const int len = lane < A.B ? A.seq_lens[lane] : 0;
         const int nt = len > 0 ? max((len + kSTile - 1) / kSTile - A.b_start[lane], 0) : 0;
@@ -925,32 +926,31 @@ __global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_
             const int t = __shfl_up(incl, off);
             if (lane >= off) incl += t;
         }
-        const int total_all = __builtin_amdgcn_readlane(incl, 63);
-        const int incl_b = __shfl(incl, b), nt_bb = __shfl(nt, b);
-        if (lane == 0) { scan_s[0] = incl_b - nt_bb; scan_s[1] = total_all; scan_s[2] = nt_bb; }
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const int excl = scan_s[0], total = scan_s[1], nt_b = scan_s[2];
-        int n = 0, off = 0;
+        const int total = __builtin_amdgcn_readlane(incl, 63);
+        const int nt_b = __shfl(nt, b), excl = __shfl(incl, b) - nt_b;
+        int cnt = 0, slot0 = 0;
         if (A.group_units + total * A.KVH > 0) {
             const RegionSplit rs = region_split(A.group_units, total * A.KVH, grid_wgs);
             const int kvh = h / (A.QH / A.KVH);
-            for (int gi = 0; gi < A.ngroups; gi++) {
-                const GSeg sg = A.seg[gi];
-                if (b < sg.first || b >= sg.first + sg.count) continue;
-                const int first = sg.unit0 + kvh * sg.ntile, last = first + sg.ntile - 1;
-                seg_base[n] = sg.slot; seg_cnt[n] = last / rs.Us - first / rs.Us + 1; seg_off[n] = off;
-                off += seg_cnt[n]; n++;
-            }
-            if (nt_b > 0) {
+            if (lane < A.ngroups) {
+                const GSeg sg = A.seg[lane];
+                if (b >= sg.first && b < sg.first + sg.count) {
+                    const int first = sg.unit0 + kvh * sg.ntile, last = first + sg.ntile - 1;
+                    slot0 = sg.slot; cnt = last / rs.Us - first / rs.Us + 1;
+                }
+            } else if (lane == A.ngroups && nt_b > 0) {
                 const int first = A.KVH * excl + kvh * nt_b, last = first + nt_b - 1;
-                seg_base[n] = A.b_slot[b]; seg_cnt[n] = last / rs.Ut - first / rs.Ut + 1; seg_off[n] = off;
-                off += seg_cnt[n]; n++;
+                slot0 = A.b_slot[b]; cnt = last / rs.Ut - first / rs.Ut + 1;
             }
         }
-        seg_off[n] = min(off, kGMaxPieces);
-        nseg_s = n;
+        int cincl = cnt;
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) {                 // at most kGMaxGroups + 1 entries
+            const int t = __shfl_up(cincl, off);
+            if (lane >= off) cincl += t;
+        }
+        if (lane <= A.ngroups) { seg_base[lane] = slot0; seg_cnt[lane] = cnt; seg_off[lane] = cincl - cnt; }
+        if (lane == A.ngroups) { seg_off[lane + 1] = min(cincl, kGMaxPieces); nseg_s = lane + 1; }
     }
     __syncthreads();
     const int nseg = nseg_s, n_all = seg_off[nseg];
@@ -958,8 +958,15 @@ __global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_
         for (int i = threadIdx.x; i < seg_cnt[k] && seg_off[k] + i < kGMaxPieces; i += 256) slot_of[seg_off[k] + i] = (short)(seg_base[k] + i);
     __syncthreads();
     const size_t base = ((size_t)b * A.QH + h) * A.Ptot;
-    float M = -INFINITY;
-    for (int s = lane; s < n_all; s += 64) {
+    // the first 64 pieces' sums and maxima stay in registers for the second pass (a row rarely has more)
+    float M = -INFINITY, pl0 = 0.0f, pm0 = 0.0f;
+    if (lane < n_all) {
+        const size_t pi = base + slot_of[lane];
+        pl0 = A.part_l[pi];
+        pm0 = A.part_m[pi];
+        if (pl0 > 0.0f) M = pm0;
+    }
+    for (int s = lane + 64; s < n_all; s += 64) {
         const size_t pi = base + slot_of[s];
         if (A.part_l[pi] > 0.0f) M = fmaxf(M, A.part_m[pi]);
     }
@@ -971,8 +978,8 @@ __global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_
         float wt = 0.0f;
         if (s < n_all) {
             const size_t pi = base + slot_of[s];
-            const float pl = A.part_l[pi];
-            if (pl > 0.0f) { wt = s_exp2(A.part_m[pi] - M); L = fmaf(pl, wt, L); }
+            const float pl = c0 == 0 ? pl0 : A.part_l[pi];
+            if (pl > 0.0f) { wt = s_exp2((c0 == 0 ? pm0 : A.part_m[pi]) - M); L = fmaf(pl, wt, L); }
         }
         for (int j = wv; j < cnt; j += 32) {
             fvec o[8];
