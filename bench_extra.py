@@ -1114,9 +1114,39 @@ def kernel_fractions(buf, seed=11):
             torch.cuda.synchronize()
         whole.append(round(a0.elapsed_time(a1) * 1e3, 1))
     lib.drk_debug_set_prefill_pieces(1)
+    # the attention mass of a perception frame at this shape: the last chunk, and a 64-row frame behind 32 704 tokens
+    # (table of branch 0; the attention call leaves the rows' log-sum-exps, the pass walks the keys once)
+    fm7 = {}
+    mass7 = torch.zeros(nblk, dtype=torch.float32, device="cuda")
+    for rows7 in (chunk, 64):
+        pos7 = total - rows7
+        q7 = (torch.randn(rows7, QH7, D7, device="cuda") * 0.5).to(h)
+        o7 = torch.empty_like(q7)
+        lse7 = torch.empty(rows7 * QH7, dtype=torch.float32, device="cuda")
+
+        def attn7():
+            cabi.call("drk_paged_prefill_attention_lse", C.byref(g), cabi.p(q7), cabi.p(buf), cabi.p(dtab), cabi.p(o7), 0, pos7, rows7,
+                      scale7, cabi.F16, None, 0, cabi.p(lse7), cabi.p(pws), pwsb, sp)
+
+        def both7():
+            attn7()
+            cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), cabi.p(q7), cabi.p(buf), cabi.p(dtab), 0, pos7, rows7,
+                      scale7, cabi.F16, cabi.p(lse7), cabi.p(mass7), nblk, 1, sp)
+
+        t = []
+        for fn in (attn7, both7):
+            fn(); fn()
+            a0, a1 = ev(), ev()
+            a0.record(stream)
+            for _ in range(4):
+                fn()
+            a1.record(stream)
+            torch.cuda.synchronize()
+            t.append(round(a0.elapsed_time(a1) / 4 * 1e3, 1))
+        fm7["%d_rows" % rows7] = {"attention_us": t[0], "with_one_walk_mass_us": t[1]}
     prefill_entry("config7_prefill_d256", "prefill_d256w_kernel<f16> + prefill_piece_merge_kernel", per_chunk,
                   "the reference's model shape: causal prefill of 32768 tokens in 16 chunks of 2048 over 256-token blocks, 24 Q / 4 KV "
                   "heads x 256, fp16 (the pages hold N(0, 0.5), written beforehand); 384 walks of 128 rows: 256 whole, the last 128 "
                   "in two pieces each and a merge of their rows, timed together",
-                  {"first_and_last_chunk_us_with_whole_walks": whole})
+                  {"first_and_last_chunk_us_with_whole_walks": whole, "frame_mass_behind_32768_tokens": fm7})
     return res
