@@ -2165,14 +2165,19 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
     __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPitchK];
     __shared__ int valid_lds2[2][4];                        // page present, per (buffer, 16-token run)
 
-    const int kvh = (int)blockIdx.x % A.KVH;
-    const int qt = (int)blockIdx.x / A.KVH;
+    // workgroup = (row tile, kv head, part): with the rows' log-sum-exps given the launcher may cut every walk into
+    // A.kparts ranges of tiles (a short chunk behind a long context has few walks; the parts' sums just add up)
+    const int wg = (int)blockIdx.x / A.kparts, part = (int)blockIdx.x - wg * A.kparts;
+    const int kvh = wg % A.KVH;
+    const int qt = wg / A.KVH;
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
     const int G = A.QH / A.KVH, TPW = A.tpw;
     const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
-    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+    const int nt_walk = (lim_wg + kPfBN - 1) / kPfBN;
+    const int t0 = (int)((long)part * nt_walk / A.kparts), ntiles = (int)((long)(part + 1) * nt_walk / A.kparts);   // the part's tiles: [t0, ntiles)
+    if (t0 >= ntiles) return;
 
     // Q as the A operand: this lane's fragment belongs to row w * 32 + n
     uint4 qf[NKS];
@@ -2246,12 +2251,12 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
 
     auto walk = [&](auto second) {
         constexpr bool MASS = decltype(second)::value;
-        fetch_k(0);
-        stage_k(0);
-        if (1 < ntiles) fetch_k(1);
+        fetch_k(t0);
+        stage_k(t0 & 1);
+        if (t0 + 1 < ntiles) fetch_k(t0 + 1);
         __syncthreads();
 #pragma unroll 1
-        for (int it = 0; it < ntiles; it++) {
+        for (int it = t0; it < ntiles; it++) {
             if (it + 1 < ntiles) {
                 stage_k((it + 1) & 1);                       // the buffer tile it - 1 was read from, a barrier ago
                 if (it + 2 < ntiles) fetch_k(it + 2);
@@ -3378,7 +3383,15 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
         DRK_LAUNCH_CHECK("prefill_massd_kernel");
         return DRK_OK;
     }
-    dim3 grid(((M + A.tpw - 1) / A.tpw) * a.KVH);
+    // few walks and the rows' log-sum-exps given: every walk's tiles in parts, about 512 workgroups (two per CU at
+    // head_dim 128), a part no shorter than eight tiles
+    A.gh = 0; A.nqt = 0; A.n_full = 0;
+    {
+        const int walks = ((M + A.tpw - 1) / A.tpw) * a.KVH;
+        const int tiles = (pos_start + M + kPfBN - 1) / kPfBN;
+        A.kparts = !d_row_lse ? 1 : (g_prefill_mass_parts > 0 ? g_prefill_mass_parts : std::max(1, std::min(512 / walks, tiles / 8)));
+    }
+    dim3 grid(((M + A.tpw - 1) / A.tpw) * a.KVH * A.kparts);
 #define DRK_PM(DT, KV, IO)                                                                                                      \
     do {                                                                                                                       \
         if (a.D == 128) hipLaunchKernelGGL((prefill_mass_kernel<DT, KV, IO, 128>), grid, dim3(256), 0, st, A, d_block_mass, mass_len); \

@@ -59,9 +59,9 @@ void drk_debug_set_prefill_d256_waves(int mode);
  * 256 rows per workgroup and its K tiles straight into LDS (blocks of 16 * 2^k tokens, up to 8 192 / 6 144 logical
  * blocks at head_dim 128 / 256); 0 = the register-staging kernel, which also serves every other case. */
 void drk_debug_set_prefill_mass_direct(int on);
-/* That kernel cuts every walk into parts (ranges of tiles) when a chunk has few walks, so that a short frame
- * behind a long context fills the chip: 0 (default) = the library's rule (256 workgroups, a part no shorter
- * than eight tiles); n > 0 = n parts per walk, whatever their length (tests). */
+/* The one-walk mass kernels cut every walk into parts (ranges of tiles) when a chunk has few walks, so that a
+ * short frame behind a long context fills the chip: 0 (default) = the library's rule (256 or 512 workgroups, a
+ * part no shorter than eight tiles); n > 0 = n parts per walk, whatever their length (tests). */
 void drk_debug_set_prefill_mass_parts(int parts);
 /* Tuning: which causal chunks of head_dim 128 run on the two-phase chunk kernels (eight waves, 256 rows per
  * workgroup): 0 = none (the four-wave kernel); 1 = the library's rule (default: chunks long enough to give
