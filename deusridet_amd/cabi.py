@@ -160,6 +160,8 @@ SIGNATURES = {
     "drk_decode_mass_workspace_bytes": (_sz, [_LP, _i32, _i32]),
     "drk_paged_decode_attention_mass": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _i32, _f32, _i32, _vp,
                                                _i32, _i32, _vp, _sz, _vp]),
+    "drk_paged_decode_attention_mass_gated": (_i32, [_LP, _vp, _vp, _vp, _i32, _vp, _i32, _i32, _vp, _vp, _i32, _f32, _i32,
+                                                     _vp, _sz, _vp, _i32, _i32, _vp, _sz, _vp]),
     "drk_paged_prefill_attention_mass": (_i32, [_LP, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _i32, _i32, _vp]),
     "drk_paged_prefill_attention_lse": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp, _vp, _sz,
                                                _vp]),

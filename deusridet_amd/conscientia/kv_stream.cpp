@@ -348,12 +348,11 @@ void KvStream::decode_layer(int fa_layer_idx, const KvLayerIO& io, hipStream_t s
     if (scorer_ && scorer_->d_new_scores()) {
         if (first_layer_of_step_ < 0) first_layer_of_step_ = fa_layer_idx;
         float* mass = scorer_->d_new_scores() + (size_t)branches_[0] * stride;
-        paged_gqa_decode_attention_branches_scored(ws_decode_, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B, max_len,
-                                                   io.attn_out, fa_layer_idx, pool.max_blocks(), pool.block_size(), scale,
-                                                   mass, fa_layer_idx != first_layer_of_step_, stream);
-        if (drk_sigmoid_gate(io.attn_out, gate, io.attn_out, (size_t)B * ModelConfig::NUM_ATTN_HEADS, hd, 2 * (size_t)hd,
-                             ModelConfig::IO_DTYPE, stream) != DRK_OK)
-            LOG_ERROR("Conscientia", "sigmoid_gate: %s", drk_last_error());
+        // the step's unit descriptors where the kernel takes a plan, the gate on the merge
+        const void* plan = step_plan(tables, stride, B, max_len, nullptr, 0, stream) ? d_plan_ : nullptr;
+        paged_gqa_decode_attention_branches_scored(ws_decode_, plan, io.q_scratch, pool.pool_ptr(), tables, stride, d_len_, B,
+                                                   max_len, gate, 2 * hd, io.attn_out, fa_layer_idx, pool.max_blocks(),
+                                                   pool.block_size(), scale, mass, fa_layer_idx != first_layer_of_step_, stream);
     } else if (B >= shared_min_branches_ && !groups_.empty() && groups_[0].tok_end - groups_[0].tok_begin >= shared_min_tokens_) {
         // every range some of the branches share is streamed once for them, the gate rides on the merge
         if (step_plan(tables, stride, B, max_len, groups_.data(), (int)groups_.size(), stream))

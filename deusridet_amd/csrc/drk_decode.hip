@@ -883,14 +883,23 @@ size_t drk_decode_mass_workspace_bytes(const drk_kv_layout *g, int B, int max_se
 // block received: sum over its tokens and all query heads of the softmax probability --
 // the "new importance values from attention" ImportanceScorer::update takes
 // (importance_scorer.h:37-41; docs/en/architecture/02-memoria.md:40-44).
-int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_tables,
-                                    int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, void *out,
-                                    int layer, float scale, int io_dtype, float *d_block_mass, int mass_stride,
-                                    int accumulate, void *workspace, size_t workspace_bytes, void *stream)
+static int decode_mass_impl(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_tables,
+                            int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, const void *d_plan, void *out,
+                            int layer, float scale, int io_dtype, const void *gate, size_t gate_stride, float *d_block_mass,
+                            int mass_stride, int accumulate, void *workspace, size_t workspace_bytes, void *stream)
 {
     Lay a;
     int rc = make_lay(g, &a);
     if (rc) return rc;
+    if (gate && (gate_stride < (size_t)a.D || (gate_stride % 8) || ((uintptr_t)gate % 16)))
+        return fail(DRK_ERR_INVALID, "decode_mass: gate rows must be 16-byte aligned and at least head_dim apart");
+    DecodePlan plan;
+    if (d_plan) {
+        if (decode_plan_need(a, B, max_seq_len, nullptr, 0) == 0)
+            return fail(DRK_ERR_UNSUPPORTED, "decode_mass: this geometry or number of branches takes no plan");
+        plan.ptr = (uint8_t *)const_cast<void *>(d_plan);
+        plan.mode = 2;
+    }
     if (!q || !pool || !d_tables || !out || !d_seq_lens || !d_block_mass) return fail(DRK_ERR_INVALID, "decode_mass: NULL pointer");
     if (io_dtype != DRK_F16 && io_dtype != DRK_BF16) return fail(DRK_ERR_INVALID, "decode_mass: io_dtype must be F16 or BF16");
     if ((a.dtype == DRK_F16 || a.dtype == DRK_BF16) && io_dtype != a.dtype)
@@ -916,13 +925,32 @@ int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const
     hipStream_t st = (hipStream_t)stream;
     if ((rc = launch_decode_stream(a, q, pool, d_tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
                                    io_dtype, 0, workspace, false, st, 0, nullptr, nullptr, nullptr, 0, nullptr, 0,
-                                   lse_groups, lse_rows, ls)))
+                                   lse_groups, lse_rows, ls, plan)))
         return rc;
     if ((rc = launch_decode_stream(a, q, pool, d_tables, table_stride, d_seq_lens, 0, B, max_seq_len, out, layer, scale,
-                                   io_dtype, 0, workspace, true, st, 0, nullptr, nullptr, nullptr, 0, nullptr, 0,
+                                   io_dtype, 0, workspace, true, st, 0, nullptr, nullptr, nullptr, 0, gate, gate_stride,
                                    lse_groups, lse_rows, ls)))
         return rc;
     return launch_block_mass(lse_groups, lse_rows, d_seq_lens, B, a.QH, ls, a.bs, d_block_mass, mass_stride, accumulate, st);
+}
+
+int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_tables,
+                                    int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len, void *out,
+                                    int layer, float scale, int io_dtype, float *d_block_mass, int mass_stride,
+                                    int accumulate, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return decode_mass_impl(g, q, pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, nullptr, out, layer, scale, io_dtype,
+                            nullptr, 0, d_block_mass, mass_stride, accumulate, workspace, workspace_bytes, stream);
+}
+
+int drk_paged_decode_attention_mass_gated(const drk_kv_layout *g, const void *q, const void *pool, const int32_t *d_tables,
+                                          int table_stride, const int32_t *d_seq_lens, int B, int max_seq_len,
+                                          const void *d_plan, void *out, int layer, float scale, int io_dtype, const void *gate,
+                                          size_t gate_stride, float *d_block_mass, int mass_stride, int accumulate,
+                                          void *workspace, size_t workspace_bytes, void *stream)
+{
+    return decode_mass_impl(g, q, pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, d_plan, out, layer, scale, io_dtype,
+                            gate, gate_stride, d_block_mass, mass_stride, accumulate, workspace, workspace_bytes, stream);
 }
 
 // ---- decode that allocates nothing and takes no workspace ------------------------------

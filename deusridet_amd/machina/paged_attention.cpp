@@ -396,6 +396,21 @@ void paged_gqa_decode_attention_branches_scored(AttentionWorkspace& ws, const __
         LOG_ERROR("Machina", "paged_gqa_decode_attention_branches_scored: %s", drk_last_error());
 }
 
+void paged_gqa_decode_attention_branches_scored(AttentionWorkspace& ws, const void* d_plan, const __half* Q, __half* kv_pool,
+                                                const int* d_tables, int table_stride, const int* d_seq_lens, int B,
+                                                int max_seq_len, const __half* gate, int gate_stride, __half* out,
+                                                int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                                float* d_block_mass, bool accumulate, hipStream_t stream)
+{
+    if (B <= 0 || max_seq_len <= 0) return;
+    drk_kv_layout g = ModelConfig::layout(max_phys_blocks, block_size);
+    if (drk_paged_decode_attention_mass_gated(&g, Q, kv_pool, d_tables, table_stride, d_seq_lens, B, max_seq_len, d_plan, out,
+                                              fa_layer_idx, scale, ModelConfig::IO_DTYPE, gate, (size_t)gate_stride,
+                                              d_block_mass, table_stride, accumulate ? 1 : 0, ws.ptr(), ws.bytes(),
+                                              stream) != DRK_OK)
+        LOG_ERROR("Machina", "paged_gqa_decode_attention_branches_scored: %s", drk_last_error());
+}
+
 void paged_gqa_decode_attention_branches_scored(const __half* Q, __half* kv_pool, const int* d_tables, int table_stride,
                                                 const int* d_seq_lens, int B, int max_seq_len, __half* out,
                                                 int fa_layer_idx, int max_phys_blocks, int block_size, float scale,

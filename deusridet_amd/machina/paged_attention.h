@@ -222,6 +222,13 @@ void paged_gqa_decode_attention_branches_scored(AttentionWorkspace& ws, const __
                                                 int max_seq_len, __half* out, int fa_layer_idx, int max_phys_blocks,
                                                 int block_size, float scale, float* d_block_mass, bool accumulate,
                                                 hipStream_t stream = 0);
+// The same with the step's plan (or null: every launch builds its descriptors) and the gate (or null) applied in
+// the merge: what a layer of a decode step with a scorer attached needs in one call.
+void paged_gqa_decode_attention_branches_scored(AttentionWorkspace& ws, const void* d_plan, const __half* Q, __half* kv_pool,
+                                                const int* d_tables, int table_stride, const int* d_seq_lens, int B,
+                                                int max_seq_len, const __half* gate, int gate_stride, __half* out,
+                                                int fa_layer_idx, int max_phys_blocks, int block_size, float scale,
+                                                float* d_block_mass, bool accumulate, hipStream_t stream = 0);
 
 // ---- the per-stream workspaces behind the calls that take none ---------------------
 // Reserve the workspace of `stream` up front for the largest shapes, so that the steady

@@ -415,6 +415,18 @@ int drk_paged_decode_attention_mass(const drk_kv_layout *g, const void *q, const
                                     int layer, float scale, int io_dtype, float *d_block_mass,
                                     int mass_stride, int accumulate, void *workspace,
                                     size_t workspace_bytes, void *stream);
+/* The same with the two things a layer step of the reference model does around it folded in (no reference
+ * counterpart): d_plan, or NULL -- the step's unit descriptors from drk_decode_plan_build (built without groups),
+ * read instead of rebuilt by every layer's launch; gate, or NULL -- out = attention * sigmoid(gate) applied in the
+ * merge, as drk_paged_decode_attention_gated does (rows gate_stride elements apart).  Same output bits as
+ * drk_paged_decode_attention_mass followed by drk_sigmoid_gate, same masses. */
+int drk_paged_decode_attention_mass_gated(const drk_kv_layout *g, const void *q, const void *pool,
+                                          const int32_t *d_tables, int table_stride,
+                                          const int32_t *d_seq_lens, int B, int max_seq_len,
+                                          const void *d_plan, void *out, int layer, float scale,
+                                          int io_dtype, const void *gate, size_t gate_stride,
+                                          float *d_block_mass, int mass_stride, int accumulate,
+                                          void *workspace, size_t workspace_bytes, void *stream);
 /* The attention mass a perception frame gives to every block of the context: for the chunk of M
  * query tokens at pos_start (rows and visibility as in drk_paged_prefill_attention),
  *   d_block_mass[lb] (+)= sum over the chunk's tokens, all query heads, and the tokens of logical

@@ -97,6 +97,42 @@ def test_block_mass_accumulates_over_layers(dev):
     assert np.allclose(acc, base + once, rtol=0, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype,heads,bs", [(cabi.BF16, (8, 32, 128), 16), (cabi.F16, (4, 24, 256), 64), (cabi.INT8, (8, 32, 128), 16)])
+@pytest.mark.parametrize("with_plan", [False, True])
+def test_block_mass_with_the_gate_and_the_plan_folded_in(dev, dtype, heads, bs, with_plan):
+    """drk_paged_decode_attention_mass_gated -- the step's unit descriptors read from a plan, the sigmoid gate applied in
+    the merge -- against drk_paged_decode_attention_mass followed by drk_sigmoid_gate: same output bits, same masses."""
+    g, og, io, lens, tables, stride, opool, q, shape = _case(dtype, bs, seed=31, heads=heads)
+    B, QH, D, ctx = shape
+    lib = cabi.lib()
+    rng = np.random.default_rng(8)
+    gate = U.normal_bits(rng, (B, QH, 2 * D), io, 1.0)          # rows 2 D apart, as the second halves of a Q | gate projection
+    dpool, dq, dtab, dlens, dgate = U.dev_bytes(opool), U.dev_bytes(q), U.dev_i32(tables), U.dev_i32(lens), U.dev_bytes(gate)
+    wsb = lib.drk_decode_mass_workspace_bytes(C.byref(g), B, ctx)
+    ws = U.dev_zeros(wsb)
+    scale = 1.0 / np.sqrt(D)
+    plan = None
+    if with_plan:
+        pb = lib.drk_decode_plan_bytes(C.byref(g), B, ctx, 0)
+        assert pb > 0
+        plan = U.dev_zeros(pb)
+        cabi.call("drk_decode_plan_build", C.byref(g), U.p(dtab), stride, U.p(dlens), B, ctx, None, 0, U.p(plan), pb, U.stream_ptr())
+    out_a, out_b = U.dev_zeros(B * QH * D * 2), U.dev_zeros(B * QH * D * 2)
+    mass_a = U.dev_bytes(np.full((B, stride), 7.0, np.float32))
+    mass_b = U.dev_bytes(np.full((B, stride), 7.0, np.float32))
+    gate_ptr = C.c_void_p(U.p(dgate).value + D * 2)
+    cabi.call("drk_paged_decode_attention_mass", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dlens), B, ctx,
+              U.p(out_a), 1, scale, io, U.p(mass_a), stride, 0, U.p(ws), wsb, U.stream_ptr())
+    cabi.call("drk_sigmoid_gate", U.p(out_a), gate_ptr, U.p(out_a), B * QH, D, 2 * D, io, U.stream_ptr())
+    cabi.call("drk_paged_decode_attention_mass_gated", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), stride, U.p(dlens), B, ctx,
+              U.p(plan) if plan is not None else None, U.p(out_b), 1, scale, io, gate_ptr, 2 * D, U.p(mass_b), stride, 0,
+              U.p(ws), wsb, U.stream_ptr())
+    U.sync()
+    assert np.array_equal(U.host(out_a, np.uint16), U.host(out_b, np.uint16))
+    ma, mb = U.host(mass_a, np.float32), U.host(mass_b, np.float32)
+    assert np.allclose(ma, mb, rtol=1e-5, atol=1e-5) and not np.all(ma == 7.0)
+
+
 def test_block_mass_argument_errors(dev):
     g, og, io, lens, tables, stride, opool, q, shape = _case(cabi.BF16, 16, seed=8, B=2, ctx=100, holes=False)
     B, QH, D, ctx = shape
