@@ -527,6 +527,119 @@ def test_config3_full_size_properties(dev):
     assert torch.equal(out_a, out_b)
 
 
+def test_config3_fork_tree_layer_in_one_call(dev):
+    """Config 3 at its real sizes through the host classes: a 65 536-token prefix, 16 branches forked from it and from one
+    another at random block boundaries (every fourth inside a block: copy-on-write), private tails of up to 4 096
+    tokens.  Three decode steps, each as the caller runs it -- blocks for the new token (copies where a page is still
+    shared), table upload, CacheManager::common_prefix_groups, the step's plan -- then the layer twice from the same
+    pool bytes: append + planned attention as two calls, and drk_kv_append_decode_planned (the attention launch
+    writes the new rows).  Same pool bytes, same output bits; the new token's page is the branch's own in every
+    step."""
+    torch = _torch()
+    from deusridet_amd import host
+    L, KVH, QH, D, bs, B, P = 1, 8, 32, 128, 16, 16, 65536
+    assert host.set_attention_geometry(L, QH, KVH, D, cabi.BF16)
+    cm = host.CacheManager()
+    rng = np.random.default_rng(12)
+    private = rng.integers(0, 4097, size=B)
+    NBW = P // bs + int(private.sum()) // bs + 8 * B + 64
+    assert cm.init(NBW * L * 2 * KVH * bs * D * 2, bs, None, 1 + B)
+    NB, stride = cm.pool_max_blocks(), cm.table_stride()
+    st = U.stream_ptr()
+    lib = cabi.lib()
+    g = cabi.layout(L, KVH, QH, D, bs, NB, cabi.BF16)
+    pool_ptr = C.c_void_p(cm.pool_ptr())
+    pool_bytes = lib.drk_kv_pool_bytes(C.byref(g))
+    gen = torch.Generator(device="cuda").manual_seed(5)
+
+    def bulk(branch, p0, m):
+        assert cm.ensure_blocks_for_range(branch, p0, m)
+        cm.sync_block_table(st)
+        k = (torch.randn(L, m, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        v = (torch.randn(L, m, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        cabi.call("drk_kv_append_batch", C.byref(g), pool_ptr, C.c_void_p(cm.d_block_table(branch)), 0, L, p0, m, U.p(k), U.p(v),
+                  cabi.BF16, st)
+        U.sync()
+        cm.set_seq_len(branch, p0 + m)
+
+    for p0 in range(0, P, 8192):
+        bulk(0, p0, 8192)
+    parent = [-1] + [int(rng.integers(-1, i)) for i in range(1, B)]
+    forks = []
+
+    def grow(node, par_branch, fp):
+        if node % 4 == 0:
+            fp -= int(rng.integers(1, bs))
+        b = cm.fork_branch(par_branch, fp)
+        assert b > 0
+        forks.append(b)
+        for p0 in range(0, int(private[node]), 2048):
+            bulk(b, fp + p0, min(2048, int(private[node]) - p0))
+        descend(node, b)
+
+    def descend(node, branch):
+        held = cm.seq_len(branch)
+        kids = [(P + bs * int(rng.integers(0, (held - P) // bs + 1)) if branch else P, c)
+                for c in range(node + 1, B) if parent[c] == node]
+        for fp, c in sorted(kids, key=lambda k: -k[0]):
+            grow(c, branch, fp)
+
+    descend(-1, 0)
+    assert forks == list(range(forks[0], forks[0] + B))
+    dtabs = C.c_void_p(cm.d_block_table(forks[0]))
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    before = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    after_two = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+    after_one = torch.empty(pool_bytes, dtype=torch.uint8, device="cuda")
+
+    def copy(dst, src):
+        U.sync()
+        assert hip.hipMemcpy(dst, src, pool_bytes, 3) == 0
+
+    q = (torch.randn(B, QH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+    scale = float(1 / np.sqrt(D))
+    n_with_groups = 0
+    for step in range(3):
+        lens = np.array([cm.seq_len(b) for b in forks], dtype=np.int32)
+        for i, b in enumerate(forks):
+            assert cm.ensure_blocks_for(b, int(lens[i]))                 # the new token's block; a copy where it is shared
+        cm.sync_block_table(st)
+        groups = cm.common_prefix_groups(forks, 64 // (QH // KVH), 256, cabi.MAX_PREFIX_GROUPS)
+        n_with_groups += len(groups) >= 3
+        arr = cabi.prefix_groups(groups)
+        tabs = np.stack([cm.h_block_table(b) for b in forks])
+        for i in range(B):                                               # nobody else maps the page the new token goes to
+            blk = tabs[i, int(lens[i]) // bs]
+            assert blk >= 0 and (tabs[:, :] == blk).sum() == 1
+        mx = int(lens.max()) + 1
+        dlen, dpos = U.dev_i32(lens + 1), U.dev_i32(lens)
+        pb = lib.drk_decode_plan_bytes(C.byref(g), B, mx, len(groups))
+        plan = U.dev_zeros(pb)
+        cabi.call("drk_decode_plan_build", C.byref(g), dtabs, stride, U.p(dlen), B, mx, arr, len(groups), U.p(plan), pb, st)
+        wsb = lib.drk_decode_grouped_workspace_bytes(C.byref(g), B, mx, arr, len(groups))
+        ws = U.dev_zeros(wsb)
+        nk = (torch.randn(B, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        nv = (torch.randn(B, KVH, D, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+        out_two, out_one = torch.zeros_like(q), torch.zeros_like(q)
+        copy(U.p(before), pool_ptr)
+        cabi.call("drk_kv_append_branches", C.byref(g), pool_ptr, dtabs, stride, U.p(dpos), B, 0, 1, U.p(nk), U.p(nv), cabi.BF16, st)
+        cabi.call("drk_paged_decode_attention_planned", C.byref(g), U.p(q), pool_ptr, dtabs, stride, U.p(dlen), B, mx, arr,
+                  len(groups), U.p(plan), U.p(out_two), 0, scale, cabi.BF16, None, 0, U.p(ws), wsb, st)
+        copy(U.p(after_two), pool_ptr)
+        copy(pool_ptr, U.p(before))
+        cabi.call("drk_kv_append_decode_planned", C.byref(g), pool_ptr, dtabs, stride, U.p(dlen), B, mx, arr, len(groups),
+                  U.p(plan), U.p(nk), U.p(nv), cabi.BF16, U.p(q), U.p(out_one), 0, scale, cabi.BF16, None, 0, U.p(ws), wsb, st)
+        copy(U.p(after_one), pool_ptr)
+        assert torch.equal(after_one, after_two), step
+        assert not torch.equal(after_one, before), step
+        assert torch.equal(out_one, out_two), step
+        assert bool(torch.isfinite(out_one.float()).all())
+        for i, b in enumerate(forks):
+            cm.set_seq_len(b, int(lens[i]) + 1)
+    assert n_with_groups == 3
+
+
 def test_config3_sustained_eviction(dev):
     """BASELINE config 3 run for 520 decode steps on two layers: a 65 536-token prefix shared by 16 copy-on-write
     branches with private tails of up to 4 096 tokens, every step appends one token per branch and layer and
