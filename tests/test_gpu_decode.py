@@ -344,29 +344,15 @@ def test_workspace_too_small_is_refused(dev):
     assert rc == cabi.ERR_WORKSPACE
 
 
-@pytest.fixture(params=["grouped", "producer_consumer", "every_wave_stages"])
-def prefix_kernel(request):
-    """Shared pages are read by the grouped kernel (shared and private tiles in one launch: head_dim 128, up to
-    64 rows per kv head) or by a prefix pass + the tail kernel; the prefix pass has two kernels for up to 64 rows
-    per kv head of head_dim 128."""
-    cabi.lib().drk_debug_set_grouped_decode(0 if request.param == "grouped" else 1)
-    cabi.lib().drk_debug_set_prefix_stream(0 if request.param == "every_wave_stages" else 1)
-    yield request.param
-    cabi.lib().drk_debug_set_prefix_stream(1)
-    cabi.lib().drk_debug_set_grouped_decode(0)
+_SHARED_CASES = {}
 
 
-@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
-@pytest.mark.parametrize("shared,extra,heads", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17], (8, 32, 128)), (960 + 16, [5, 300], (8, 32, 128)),
-                                                (64, [0], (8, 32, 128)), (4096, list(range(0, 400, 10)), (8, 32, 128)),
-                                                (1024, [3, 200, 64, 700, 1], (2, 16, 128)), (512, [9, 100, 33], (4, 24, 256)),
-                                                (8192 + 64, [(37 * i) % 900 for i in range(16)], (8, 32, 128)),
-                                                (192, [0, 5, 70], (1, 16, 128))])
-def test_shared_prefix_decode(dev, prefix_kernel, dtype, shared, extra, heads):
-    """Branches whose leading pages are the same physical blocks (BASELINE config 3
-    in small): the shared pass + private tails must agree with the fp64 oracle run
-    per branch, and with the plain per-branch call.  Also with 8 and 6 query heads per kv head,
-    head_dim 256, and 8-bit pages."""
+def _shared_case(dtype, shared, extra, heads):
+    """The pool, tables and queries of a shared-prefix case and the fp64 oracle's outputs: the same for every kernel the
+    case runs on, built once (nothing writes to them afterwards)."""
+    key = (dtype, shared, tuple(extra), tuple(heads))
+    if key in _SHARED_CASES:
+        return _SHARED_CASES[key]
     L, bs = 1, 16
     KVH, QH, D = heads
     io = dtype if dtype in (cabi.F16, cabi.BF16) else cabi.BF16
@@ -401,6 +387,35 @@ def test_shared_prefix_decode(dev, prefix_kernel, dtype, shared, extra, heads):
         tables[:, n_shared_blk - 5] = -1
     q = U.normal_bits(rng, (B, QH, D), io, 0.7)
     scale = 1 / np.sqrt(D)
+    want = np.stack([orc.decode_f64(og, q[b], opool, tables[b], 0, int(lens[b]), scale, io) for b in range(B)])
+    _SHARED_CASES[key] = (bs, KVH, QH, D, io, B, lens, n_shared_blk, g, og, stride, tables, opool, q, scale, want)
+    return _SHARED_CASES[key]
+
+
+@pytest.fixture(params=["grouped", "producer_consumer", "every_wave_stages"])
+def prefix_kernel(request):
+    """Shared pages are read by the grouped kernel (shared and private tiles in one launch: head_dim 128, up to
+    64 rows per kv head) or by a prefix pass + the tail kernel; the prefix pass has two kernels for up to 64 rows
+    per kv head of head_dim 128."""
+    cabi.lib().drk_debug_set_grouped_decode(0 if request.param == "grouped" else 1)
+    cabi.lib().drk_debug_set_prefix_stream(0 if request.param == "every_wave_stages" else 1)
+    yield request.param
+    cabi.lib().drk_debug_set_prefix_stream(1)
+    cabi.lib().drk_debug_set_grouped_decode(0)
+
+
+@pytest.mark.parametrize("dtype", [cabi.F16, cabi.BF16, cabi.INT8, cabi.FP8_E4M3])
+@pytest.mark.parametrize("shared,extra,heads", [(1024, [0, 1, 63, 64, 65, 500, 1000, 17], (8, 32, 128)), (960 + 16, [5, 300], (8, 32, 128)),
+                                                (64, [0], (8, 32, 128)), (4096, list(range(0, 400, 10)), (8, 32, 128)),
+                                                (1024, [3, 200, 64, 700, 1], (2, 16, 128)), (512, [9, 100, 33], (4, 24, 256)),
+                                                (8192 + 64, [(37 * i) % 900 for i in range(16)], (8, 32, 128)),
+                                                (192, [0, 5, 70], (1, 16, 128))])
+def test_shared_prefix_decode(dev, prefix_kernel, dtype, shared, extra, heads):
+    """Branches whose leading pages are the same physical blocks (BASELINE config 3
+    in small): the shared pass + private tails must agree with the fp64 oracle run
+    per branch, and with the plain per-branch call.  Also with 8 and 6 query heads per kv head,
+    head_dim 256, and 8-bit pages."""
+    bs, KVH, QH, D, io, B, lens, n_shared_blk, g, og, stride, tables, opool, q, scale, want = _shared_case(dtype, shared, extra, heads)
     dq, dpool, dtab, dl = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(tables), U.dev_i32(lens)
     lib = cabi.lib()
     mx = int(lens.max())
@@ -416,7 +431,6 @@ def test_shared_prefix_decode(dev, prefix_kernel, dtype, shared, extra, heads):
     U.sync()
     got = U.from_bits(U.host(out, np.uint16, (B, QH, D)), io)
     plain = U.from_bits(U.host(out2, np.uint16, (B, QH, D)), io)
-    want = np.stack([orc.decode_f64(og, q[b], opool, tables[b], 0, int(lens[b]), scale, io) for b in range(B)])
     ok, ma, _ = U.rel_abs_ok(got, want, REL, ABS)
     assert ok, ma
     ok, ma, _ = U.rel_abs_ok(got, plain, REL, ABS)
