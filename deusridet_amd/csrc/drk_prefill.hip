@@ -2354,8 +2354,8 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
 // four blocks tile after tile would queue up on them.  FOLD: the softmax scale goes into Q, rounded to the 16-bit
 // type, as in the chunk kernels that do so (their log-sum-exps belong to those scores); otherwise Q stays as it
 // is and the exponent is scaled.
-// grid = ceil(M / TPW) * KVH, TPW = 256 / (QH/KVH); block = 512; block size 16 * 2^k; at most kMassdBlocks<D>
-// logical blocks in pos_start + M tokens.
+// grid = ceil(M / TPW) * KVH * parts, TPW = 256 / (QH/KVH); block = 512; block size 16 * 2^k; at most
+// kMassdBlocks<D> logical blocks in a part's range of tiles (the launcher sees to it).
 template <int D>
 constexpr int kMassdBlocks = D == 128 ? 8192 : 6144;
 template <int DT, int IO, int D, bool FOLD, bool TWO>
@@ -2390,7 +2390,7 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
     if (t0 >= ntiles) return;                                // more parts than tiles
     const int sh = A.bs_shift;
     const int lb0 = (t0 * kPfBN) >> sh;                      // the table in LDS begins at the part's first block
-    const int nblk_wg = ((min(lim_wg, ntiles * kPfBN) + A.bs - 1) >> sh) - lb0;
+    const int nblk_wg = min(((min(lim_wg, ntiles * kPfBN) + A.bs - 1) >> sh) - lb0, kMassdBlocks<D>);   // (the launcher keeps a part within the table)
 
     for (int i = threadIdx.x; i < nblk_wg; i += 512) mass_ldsm[i] = 0.0f;
     for (int i = threadIdx.x * 16; i < kRing * kTileBytes; i += 512 * 16) *(uint4 *)(&k_ldsm[0][0] + i) = make_uint4(0, 0, 0, 0);
@@ -2538,7 +2538,8 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
                 const auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(cs[tt]), __float_as_uint(cs[tt]), false, false);
                 const float c16 = pf_row16_sum(__uint_as_float(r2[0]) + __uint_as_float(r2[1]));
                 const int run0 = tile_t + tt * 32 + (n & 16);
-                if (g == 0 && (n & 15) == 0 && run0 >= t0 * kPfBN && run0 < lim_part && c16 != 0.0f) atomicAdd(&mass_ldsm[(run0 >> sh) - lb0], c16);
+                const int bi = (run0 >> sh) - lb0;
+            if (g == 0 && (n & 15) == 0 && run0 >= t0 * kPfBN && run0 < lim_part && bi < nblk_wg && c16 != 0.0f) atomicAdd(&mass_ldsm[bi], c16);
             }
         };
         float cs_prev[2] = {0.0f, 0.0f};                         // the key sums of the tile before, folded a step later
@@ -3357,15 +3358,20 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
     A.lse_rows = const_cast<float *>(d_row_lse);             // read only here: the rows' log-sum-exps, or NULL (first walk finds them)
     // 16-bit pages: the kernel that takes its tiles straight into LDS -- one walk when the rows' log-sum-exps are
     // given, else two by the same workgroup (whole walks then: the first must see every key)
+    // (the table of page sums in LDS holds the blocks of one part: a context of more blocks than it holds is cut into
+    // parts for that reason alone -- which the two-walk call cannot do)
+    const int massd_cap = (a.D == 128 ? kMassdBlocks<128> : kMassdBlocks<256>) - 8;      // a part's range is rounded to tiles and to blocks
+    const int massd_min_parts = ((pos_start + M + a.bs - 1) / a.bs + massd_cap - 1) / massd_cap;
     if (g_prefill_mass_direct && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 &&
-        (pos_start + M + a.bs - 1) / a.bs <= (a.D == 128 ? kMassdBlocks<128> : kMassdBlocks<256>) && a.QH / a.KVH <= 128) {
+        (d_row_lse || massd_min_parts == 1) && a.QH / a.KVH <= 128) {
         A.tpw = 256 / (a.QH / a.KVH);
         A.nqt = (M + A.tpw - 1) / A.tpw;
         // few walks (a short chunk): every walk's tiles in parts, so that the workgroups fill the chip once (one
         // per CU: the LDS ring), a part no shorter than eight tiles
         const int walks = A.nqt * a.KVH;
         const int tiles = (pos_start + M + kPfBN - 1) / kPfBN;
-        A.kparts = !d_row_lse ? 1 : (g_prefill_mass_parts > 0 ? g_prefill_mass_parts : std::max(1, std::min(256 / walks, tiles / 8)));
+        A.kparts = !d_row_lse ? 1 : std::max(massd_min_parts, g_prefill_mass_parts > 0 ? g_prefill_mass_parts
+                                                                                        : std::max(1, std::min(256 / walks, tiles / 8)));
         A.gh = 0; A.n_full = 0;
         const dim3 gridd((unsigned)(walks * A.kparts));
         const int kind = !d_row_lse ? 2 : (chunk_kernel_scales_q(a, pos_start, M) ? 1 : 0);

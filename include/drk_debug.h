@@ -56,8 +56,9 @@ void drk_debug_set_prefill_pieces(int mode);
  * same pieces, same bits. */
 void drk_debug_set_prefill_d256_waves(int mode);
 /* Mass passes (drk_paged_prefill_attention_mass[_lse]) over 16-bit pages: 1 (default) = the kernel that takes
- * 256 rows per workgroup and its K tiles straight into LDS (blocks of 16 * 2^k tokens, up to 8 192 / 6 144 logical
- * blocks at head_dim 128 / 256); 0 = the register-staging kernel, which also serves every other case. */
+ * 256 rows per workgroup and its K tiles straight into LDS (blocks of 16 * 2^k tokens; the two-walk call up to
+ * 8 184 / 6 136 logical blocks of context at head_dim 128 / 256); 0 = the register-staging kernel, which also
+ * serves every other case. */
 void drk_debug_set_prefill_mass_direct(int on);
 /* The one-walk mass kernels cut every walk into parts (ranges of tiles) when a chunk has few walks, so that a
  * short frame behind a long context fills the chip: 0 (default) = the library's rule (256 or 512 workgroups, a

@@ -333,6 +333,42 @@ def test_frame_mass_with_the_context_in_parts(dev, mass_kernel, parts, dtype, bs
         assert got[0][h] == 0.0
 
 
+@pytest.mark.parametrize("dtype,heads,total", [(cabi.BF16, (1, 2, 128), 8192 * 16 + 700), (cabi.F16, (1, 1, 256), 6144 * 16 + 300)])
+def test_frame_mass_behind_more_blocks_than_the_kernels_table_holds(dev, dtype, heads, total):
+    """A context of more 16-token blocks than the one-walk kernel's table of page sums in LDS holds (8 192 at head_dim
+    128, 6 144 at 256): the walk is cut into parts for that reason alone.  Five rows behind 131k / 98k tokens against
+    fp64; the masses of the whole context add up to rows x heads."""
+    bs, M = 16, 5
+    pos_start = total - M
+    g, og, io, table, opool, q = _frame_case(dtype, bs, seed=77, pos_start=pos_start, M=M, heads=heads, holes=(3, 4000))
+    KVH, QH, D = heads
+    scale = 1.0 / np.sqrt(D)
+    lib = cabi.lib()
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    ws = U.dev_zeros(max(wsb, 16))
+    out = U.dev_bytes(np.zeros(M * QH * D * 2, dtype=np.uint8))
+    lse = U.dev_bytes(np.zeros(M * QH, np.float32))
+    cabi.call("drk_paged_prefill_attention_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), 1, pos_start, M, float(scale),
+              io, None, 0, U.p(lse), U.p(ws), wsb, U.stream_ptr())
+    got = []
+    try:
+        for parts in (0, 1):                                # the rule's parts; "one part" asked for: still as many as the table needs
+            lib.drk_debug_set_prefill_mass_parts(parts)
+            mass = U.dev_bytes(np.full(table.size, 7.0, np.float32))
+            cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale),
+                      io, U.p(lse), U.p(mass), table.size, 0, U.stream_ptr())
+            U.sync()
+            got.append(U.host(mass, np.float32).astype(np.float64))
+    finally:
+        lib.drk_debug_set_prefill_mass_parts(0)
+    want = _frame_want(og, io, table, opool, q, pos_start, scale)
+    for m in got:
+        assert np.all(np.abs(m - want) <= 2e-3 * M + 3e-3 * np.abs(want)), np.abs(m - want).max()
+        assert abs(m.sum() - M * QH) <= 2e-3 * M * QH
+        assert m[3] == 0.0 and m[4000] == 0.0
+
+
 def test_frame_mass_of_a_long_chunk(dev):
     """A 300-token frame behind 3 000 tokens (several row tiles per kv head meeting in every page)."""
     pos_start, M, bs = 3000, 300, 16
