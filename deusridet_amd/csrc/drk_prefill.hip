@@ -2249,6 +2249,8 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
 #pragma unroll
     for (int i = 0; i < 16; i++) { m[i] = kNone; l[i] = 0.0f; lse[i] = INFINITY; }
 
+    int carry_lb = 0;                                        // second walk: the block this lane is adding up, and its sum so far
+    float carry = 0.0f;
     auto walk = [&](auto second) {
         constexpr bool MASS = decltype(second)::value;
         fetch_k(t0);
@@ -2304,8 +2306,16 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
                     cs = pf_row16_sum(cs);                   // the 16 keys of a run
                     const int run0 = it * kPfBN + tt * 32 + (n & 16);
                     if (g == 0 && (n & 15) == 0 && run0 < lim_wg) {
+                        // the lane keeps adding while its runs stay in one block (blocks of 32 tokens or more) and
+                        // goes to memory when the block changes: every workgroup of the launch adds to the same few
+                        // blocks at about the same time, and atomics to one address queue up
                         const int lb = A.bs_shift >= 0 ? (run0 >> A.bs_shift) : (run0 / A.bs);
-                        if (lb < mass_len && cs != 0.0f) unsafeAtomicAdd(mass + lb, cs);
+                        if (lb != carry_lb) {
+                            if (carry != 0.0f && carry_lb < mass_len) unsafeAtomicAdd(mass + carry_lb, carry);
+                            carry_lb = lb;
+                            carry = 0.0f;
+                        }
+                        carry += cs;
                     }
                 }
             }
@@ -2335,6 +2345,7 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
         }
     }
     walk(std::true_type{});
+    if (carry != 0.0f && carry_lb < mass_len) unsafeAtomicAdd(mass + carry_lb, carry);
 }
 
 // ---- attention mass of a chunk, 16-bit pages: tiles straight into LDS ----------------------------------------
