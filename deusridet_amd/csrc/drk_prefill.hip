@@ -2403,8 +2403,15 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
     const int lb0 = (t0 * kPfBN) >> sh;                      // the table in LDS begins at the part's first block
     const int nblk_wg = min(((min(lim_wg, ntiles * kPfBN) + A.bs - 1) >> sh) - lb0, kMassdBlocks<D>);   // (the launcher keeps a part within the table)
 
-    for (int i = threadIdx.x; i < nblk_wg; i += 512) mass_ldsm[i] = 0.0f;
+    // (while clearing the table: does every block of the part have a page?  Then most steps need no validity flags)
+    int no_page = 0;
+    for (int i = threadIdx.x; i < nblk_wg; i += 512) {
+        mass_ldsm[i] = 0.0f;
+        const int e = A.table[lb0 + i];
+        no_page |= (e < 0 || e >= A.NB) ? 1 : 0;
+    }
     for (int i = threadIdx.x * 16; i < kRing * kTileBytes; i += 512 * 16) *(uint4 *)(&k_ldsm[0][0] + i) = make_uint4(0, 0, 0, 0);
+    const bool holes = __syncthreads_or(no_page) != 0;
 
     // Q as the A operand: this lane's fragment belongs to row w * 32 + n
     uint4 qf[NKS];
@@ -2464,6 +2471,14 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         p_src = kbase + (size_t)(ok ? blk0 : 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
         p_lds = k_ring + ((uint32_t)(kt & (kRing - 1)) << kTileShift);
         if (lane == 0) valid_ldsm[kt & (kRing - 1)][w] = ok ? 1 : 0;
+    };
+    auto plan_whole = [&](int kt, int blk_raw) {             // a tile whose pages exist and whose rows are all wanted
+        const int blk0 = __builtin_amdgcn_readfirstlane(blk_raw);
+        const int tg = kt * kPfBN + tgw;
+        p_rows = ROWS;
+        p_src = kbase + (size_t)blk0 * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
+        p_lds = k_ring + ((uint32_t)(kt & (kRing - 1)) << kTileShift);
+        if (lane == 0) valid_ldsm[kt & (kRing - 1)][w] = 1;
     };
     // request j: RPQ token rows (1 KB); the 16-byte chunk c of row r sits at position c ^ (r & 15)
     uint32_t goff[NREQ];
@@ -2553,12 +2568,25 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
             if (g == 0 && (n & 15) == 0 && run0 >= t0 * kPfBN && run0 < lim_part && bi < nblk_wg && c16 != 0.0f) atomicAdd(&mass_ldsm[bi], c16);
             }
         };
+        // the same in a step's fast mode: every key of the tile counts and its blocks are the part's; the two halves of
+        // the wave add their 16 rows each
+        auto fold_whole = [&](int tile_t, const float (&cs)[2]) {
+            const int sb = __builtin_amdgcn_readfirstlane((tile_t >> sh) - lb0);
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+                const float c16 = pf_row16_sum(cs[tt]);
+                if ((n & 15) == 0 && c16 != 0.0f) atomicAdd(&mass_ldsm[sb + ((tt * 32 + (n & 16)) >> sh)], c16);
+            }
+        };
         float cs_prev[2] = {0.0f, 0.0f};                         // the key sums of the tile before, folded a step later
         constexpr float kLazy = 8.0f;
-        auto step = [&](int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
+        // FAST: a step in the part's interior -- no row of tile it is masked, every block has a page, tile it + 3 is
+        // whole for every wave: no flags, no conditions, and the plan behind the first operand reads
+        auto step = [&](auto fast_mode, int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
+            constexpr bool FAST = decltype(fast_mode)::value;
             // here: s = exponents of tile it; K(it + 1) and K(it + 2) requested
             const int tile_t = it * kPfBN;
-            if (__builtin_expect(flags != 255 || it >= first_masked_tile, 0)) {
+            if (!FAST && __builtin_expect(flags != 255 || it >= first_masked_tile, 0)) {
 #pragma unroll
                 for (int tt = 0; tt < 2; tt++) {
                     const int key = tile_t + tt * 32 + n;
@@ -2584,23 +2612,36 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
                 }
             }
             // K(it + 1) has landed (this wave's share; the requests of K(it + 2) came after it), then everybody's
-            if (__builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
+            if (FAST || __builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
             else __builtin_amdgcn_s_waitcnt(0x0f70);
             pf_barrier_lds();
-            asm volatile("" : : "s"(blk_ahead));
-            plan(it + 3, blk_ahead);                             // into the buffer of K(it - 1), read two steps ago
-            blk_ahead = page_of(it + 4);
-            whole = p_rows >= ROWS;                              // requested between the products below
+            if constexpr (!FAST) {
+                asm volatile("" : : "s"(blk_ahead));
+                plan(it + 3, blk_ahead);                         // into the buffer of K(it - 1), read two steps ago
+                blk_ahead = page_of(it + 4);
+                whole = p_rows >= ROWS;                          // requested between the products below
+            }
             float cs[2] = {0.0f, 0.0f};
             int4 fa, fb;
             qk((it + 1) & (kRing - 1), s_next, [&](int ks) {
-                if (ks == 0) {
-                    fa = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][0];
-                    fb = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][4];
+                if constexpr (FAST) {
+                    if (ks == 0) {
+                        plan_whole(it + 3, blk_ahead);
+                        whole = true;
+                    }
+                    if ((ks & 1) == 1 && (ks >> 1) < NREQ) pf_load_to_lds16(p_src + 1024 * (ks >> 1), goff[ks >> 1], p_lds + 1024 * (ks >> 1));
+                } else {
+                    if (ks == 0) {
+                        fa = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][0];
+                        fb = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][4];
+                    }
+                    if ((ks & 1) == 0 && (ks >> 1) < NREQ) request(ks >> 1);
                 }
-                if ((ks & 1) == 0 && (ks >> 1) < NREQ) request(ks >> 1);
                 if constexpr (!LSE) {
-                    if (ks == NKS / 2) fold(tile_t - kPfBN, cs_prev);
+                    if (ks == NKS / 2) {
+                        if constexpr (FAST) fold_whole(tile_t - kPfBN, cs_prev);
+                        else fold(tile_t - kPfBN, cs_prev);
+                    }
                 }
 #pragma unroll
                 for (int u = 0; u < EPK; u++) {
@@ -2615,13 +2656,25 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
                     }
                 }
             });
-            flags = flags_of(fa, fb);
+            if constexpr (FAST) {
+                flags = 255;
+                blk_ahead = page_of(it + 4);                     // the scalar load's wait falls into the barrier's
+            } else {
+                flags = flags_of(fa, fb);
+            }
             cs_prev[0] = cs[0];
             cs_prev[1] = cs[1];
         };
-        for (int it = t0; it < ntiles; it += 2) {
-            step(it, s_even, s_odd);
-            if (it + 1 < ntiles) step(it + 1, s_odd, s_even);
+        // steps [t0, fast_end) can run in the fast mode: tile it unmasked, tile it + 3 whole for every wave
+        const int fast_end = holes ? t0 : min(first_masked_tile, lim_part / kPfBN - 3);
+        int it = t0;
+        for (; it + 2 <= fast_end; it += 2) {
+            step(std::true_type{}, it, s_even, s_odd);
+            step(std::true_type{}, it + 1, s_odd, s_even);
+        }
+        for (; it < ntiles; it += 2) {
+            step(std::false_type{}, it, s_even, s_odd);
+            if (it + 1 < ntiles) step(std::false_type{}, it + 1, s_odd, s_even);
         }
         if constexpr (!LSE) fold((ntiles - 1) * kPfBN, cs_prev);
     };
