@@ -142,6 +142,17 @@ __device__ __forceinline__ uint2 pf_lds_read_tr16(uint32_t addr, int offset)
 // Workgroup barrier for kernels whose LDS is filled by direct loads from global memory: LDS reads and writes
 // of the wave are complete, its outstanding global loads are NOT waited for (__syncthreads would drain them,
 // the fence it carries covers every store into LDS) -- the caller counts those itself.
+// The same, with the wait written so that the compiler knows of it: a scalar load issued before the barrier counts as
+// arrived behind it (otherwise its first use drains the LDS reads issued since).
+__device__ __forceinline__ void pf_barrier_lgkm()
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xc07f);                      // lgkmcnt(0)
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+#endif
+}
 __device__ __forceinline__ void pf_barrier_lds()
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -2614,7 +2625,7 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
             // K(it + 1) has landed (this wave's share; the requests of K(it + 2) came after it), then everybody's
             if (FAST || __builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
             else __builtin_amdgcn_s_waitcnt(0x0f70);
-            pf_barrier_lds();
+            pf_barrier_lgkm();
             if constexpr (!FAST) {
                 asm volatile("" : : "s"(blk_ahead));
                 plan(it + 3, blk_ahead);                         // into the buffer of K(it - 1), read two steps ago

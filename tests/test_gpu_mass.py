@@ -292,6 +292,35 @@ def test_frame_mass_from_the_attention_calls_row_sums(dev, chunk_path, mass_kern
         assert np.all(np.isfinite(rows[t])) if sees else np.all(np.isposinf(rows[t]))
 
 
+@pytest.mark.parametrize("dtype,bs,pos_start,M,heads", [(cabi.BF16, 16, 1500, 100, (8, 32, 128)), (cabi.F16, 256, 2500, 70, (4, 24, 256)),
+                                                        (cabi.F16, 64, 900, 300, (2, 14, 128))])
+def test_frame_mass_where_every_block_has_a_page(dev, mass_kernel, dtype, bs, pos_start, M, heads):
+    """No holes: the kernel for 16-bit pages takes its lean steps through the interior of every walk (no validity flags,
+    no masks) and the general ones at the ends.  The two-walk call and the one-walk call against fp64."""
+    lib = cabi.lib()
+    g, og, io, table, opool, q = _frame_case(dtype, bs, seed=3 * bs + M, pos_start=pos_start, M=M, heads=heads, holes=())
+    KVH, QH, D = heads
+    scale = 1.0 / np.sqrt(D)
+    dq, dpool, dtab = U.dev_bytes(q), U.dev_bytes(opool), U.dev_i32(table)
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
+    ws = U.dev_zeros(max(wsb, 16))
+    out = U.dev_bytes(np.zeros(M * QH * D * 2, dtype=np.uint8))
+    lse = U.dev_bytes(np.zeros(M * QH, np.float32))
+    cabi.call("drk_paged_prefill_attention_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), U.p(out), 1, pos_start, M, float(scale),
+              io, None, 0, U.p(lse), U.p(ws), wsb, U.stream_ptr())
+    one = U.dev_bytes(np.full(table.size, 7.0, np.float32))
+    two = U.dev_bytes(np.full(table.size, 7.0, np.float32))
+    cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale),
+              io, U.p(lse), U.p(one), table.size, 0, U.stream_ptr())
+    cabi.call("drk_paged_prefill_attention_mass", C.byref(g), U.p(dq), U.p(dpool), U.p(dtab), 1, pos_start, M, float(scale), io,
+              U.p(two), table.size, 0, U.stream_ptr())
+    U.sync()
+    want = _frame_want(og, io, table, opool, q, pos_start, scale)
+    for got in (U.host(one, np.float32).astype(np.float64), U.host(two, np.float32).astype(np.float64)):
+        assert np.all(np.abs(got - want) <= 2e-3 * M + 3e-3 * np.abs(want)), np.abs(got - want).max()
+        assert abs(got.sum() - M * QH) <= 2e-3 * M * QH
+
+
 @pytest.mark.parametrize("parts", [0, 3, 40])
 @pytest.mark.parametrize("dtype,bs,pos_start,M,heads,holes", [
     (cabi.BF16, 16, 3000, 20, (8, 32, 128), (7, 150)), (cabi.F16, 256, 2100, 33, (4, 24, 256), (2,)),
