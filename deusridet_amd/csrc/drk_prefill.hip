@@ -2366,10 +2366,12 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
 // waves of 32, two per SIMD), K tiles from global memory straight into a ring of four swizzled LDS buffers,
 // requested two tiles ahead between the k-steps, one barrier per tile; the products start from minus the row's
 // log-sum-exp (the C operand), so a score arrives as the exponent of its probability, and the exponentials of tile t
-// sit between the k-steps of tile t + 1's products, the fold of tile t - 1's sums too.  The vector unit bounds it:
-// 32 exponentials and 32 additions per wave and tile beside 16 products (probes: without the products 584 of 715 us
-// on 2 048 rows behind 30 720 tokens at 32 / 8 heads x 128, without the vector work 300; half of the LDS operand
-// reads left out changes nothing).  S = Q K^T as
+// sit between the k-steps of tile t + 1's products, the fold of tile t - 1's sums too.  A wave's instruction
+// count bounds it -- 32 exponentials (8 clocks each on this chip, measured) and 32 additions per wave and tile beside
+// 16 products of 32 clocks -- so the steps in the interior of a part (no masked row, every block with a page, the
+// tile requested whole: all but the last three or four of a walk) run a lean form: no validity flags, no
+// conditions, the request's plan behind the first operand reads, the table entry loaded where the barrier's wait
+// covers it, page sums without the exchange between the wave's halves.  S = Q K^T as
 // in prefill_mass_kernel: a lane stands for a key, its registers for 16 of the wave's rows, a key's sum over rows is
 // a sum over registers.  A page's sum goes to a table in LDS (one entry per logical block of the walk) and the
 // table to `mass` with one atomic per block and workgroup when the walk ends -- 256 workgroups adding to the same
