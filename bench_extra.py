@@ -1053,12 +1053,29 @@ def kernel_fractions(buf, seed=11):
 
     frame_mass["short_frame_64_rows"] = {"attention_us": timed(short_attn), "with_one_walk_mass_us": timed(short_both)}
     q, o, lse, chunk, pos = big
+    # the last chunk's launch once more on constant data (every K and V element 0.5, every Q element 0.25): the same
+    # instructions on the same addresses -- what differs is how many bits toggle, i.e. the clock the part holds
+    buf[:lib.drk_kv_pool_bytes(C.byref(g))].view(torch.bfloat16).fill_(0.5)
+    qc = torch.full_like(q, 0.25)
+
+    def attn_const():
+        cabi.call("drk_paged_prefill_attention", C.byref(g), cabi.p(qc), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, pos, chunk, scale,
+                  cabi.BF16, None, 0, sp)
+
+    const_us = timed(attn_const)
+    last_fl = chunk_flops(pos, chunk, QH, D)
+    on_const = {"random_data_us": frame_mass["attention_us"], "constant_data_us": const_us,
+                "random_data_frac": round(last_fl / (frame_mass["attention_us"] * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "constant_data_frac": round(last_fl / (const_us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                "what": "the last chunk's launch six times back to back, on the pages of the run and on pages and queries that "
+                        "hold one constant: same kernel, same addresses, same instruction stream"}
+    del qc
     cabi.call("drk_event_destroy", ev_a)
     cabi.call("drk_event_destroy", ev_m)
     res["frame_mass"] = frame_mass
     prefill_entry("config5_prefill", "prefill_ppd_kernel<bf16>", per_chunk,
                   "config 5: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV x 128 bf16",
-                  {"us_per_tile_by_workgroups_at_30720": by_wgs})
+                  {"us_per_tile_by_workgroups_at_30720": by_wgs, "last_chunk_by_data": on_const})
     del dtab
 
     # ---- the reference's model shape: 24 Q / 4 KV heads x 256, fp16, 256-token blocks, 16 layers --------------

@@ -38,6 +38,8 @@ def test_bench_workload_runs(dev, extra):
         fm = other.pop("frame_mass")
         assert fm["attention_us"] < fm["with_one_walk_mass_same_stream_us"] < fm["with_two_walk_mass_us"]
         assert 0 < fm["short_frame_64_rows"]["attention_us"] < fm["short_frame_64_rows"]["with_one_walk_mass_us"]
+        by_data = other["config5_prefill"]["last_chunk_by_data"]                   # the same launch on constant data is not slower
+        assert 0 < by_data["constant_data_us"] <= by_data["random_data_us"] * 1.05
         for name, e in other.items():
             assert 0 < e["frac"] < 1 and e["avg_launch_us"] > 0 and e["peak"] in (8000.0, 2500.0), name
         assert j["hbm_read_probe_permuted_4KiB_GBps"] > 1000 and j["mfma_bf16_probe_TFLOPs"] > 500
