@@ -954,9 +954,33 @@ def kernel_fractions(buf, seed=11):
                 torch.cuda.synchronize()
                 per_chunk.append((a0.elapsed_time(a1), chunk_flops(c * chunk, chunk, QH, D)))
         if dt != cabi.BF16:
+            # the last chunk as a perception frame: attention that leaves the rows' log-sum-exps, then the one-walk mass pass
+            pos8 = total - chunk
+            lse8 = torch.empty(chunk * QH, dtype=torch.float32, device="cuda")
+            mass8 = torch.zeros(total // bs, dtype=torch.float32, device="cuda")
+
+            def frame8(with_mass):
+                cabi.call("drk_paged_prefill_attention_lse", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), cabi.p(o), 0, pos8, chunk,
+                          scale, cabi.BF16, None, 0, cabi.p(lse8), None, 0, sp)
+                if with_mass:
+                    cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), cabi.p(q), cabi.p(buf), cabi.p(dtab), 0, pos8, chunk,
+                              scale, cabi.BF16, cabi.p(lse8), cabi.p(mass8), total // bs, 1, sp)
+
+            frame_us = []
+            for with_mass in (False, True):
+                frame8(with_mass)
+                a0, a1 = ev(), ev()
+                a0.record(stream)
+                for _ in range(4):
+                    frame8(with_mass)
+                a1.record(stream)
+                torch.cuda.synchronize()
+                frame_us.append(round(a0.elapsed_time(a1) / 4 * 1e3, 1))
             prefill_entry(key, "prefill_pp_kernel<%s>" % name, per_chunk,
                           "config 5 over %s pages: causal prefill of 32768 tokens in 16 chunks of 2048 over 16-token pages, 32 Q / 8 KV "
-                          "x 128, bf16 queries, codes turned into 16-bit MFMA operands on the way into LDS" % name)
+                          "x 128, bf16 queries, codes turned into 16-bit MFMA operands on the way into LDS" % name,
+                          {"last_chunk_as_frame": {"attention_us": frame_us[0], "with_one_walk_mass_us": frame_us[1]}})
+            del lse8, mass8
     # the same kernel at position 30 720 with fewer workgroups (shorter chunks): microseconds per 64-token tile of the
     # longest walk.  One workgroup per CU either way -- what changes is how much of the chip draws power.
     by_wgs = {}

@@ -2359,7 +2359,7 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
     if (carry != 0.0f && carry_lb < mass_len) unsafeAtomicAdd(mass + carry_lb, carry);
 }
 
-// ---- attention mass of a chunk, 16-bit pages: tiles straight into LDS ----------------------------------------
+// ---- attention mass of a chunk: 256 rows per workgroup, 16-bit tiles straight into LDS ----------------------
 // prefill_mass_kernel rebuilt on the chunk kernels' machinery (one walk when the rows' log-sum-exps are given; TWO:
 // the workgroup first walks its keys for them, a lane keeping a lazy running maximum and sum per row over the keys
 // it sees, the 32 lanes of a row meeting once between the walks): 256 rows per workgroup (eight
@@ -2382,10 +2382,16 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
 // kMassdBlocks<D> logical blocks in a part's range of tiles (the launcher sees to it).
 template <int D>
 constexpr int kMassdBlocks = D == 128 ? 8192 : 6144;
-template <int DT, int IO, int D, bool FOLD, bool TWO>
+template <int DT, int IO, int D, bool FOLD, bool TWO, int KV = DT>
 __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, float *__restrict__ mass, int mass_len)
 {
+    // Q8: 8-bit pages (head_dim 128, one walk).  A tile's codes cannot go straight into LDS: a wave's 8 rows are one
+    // 16-byte load per lane into registers, requested where the 16-bit kind requests, and turned into fp16 rows of the
+    // same swizzled layout at the head of the next step (a step ahead of the barrier behind which they are read).
+    constexpr bool Q8 = KV == DRK_INT8 || KV == DRK_FP8_E4M3;
+    static_assert(!Q8 || (D == 128 && !TWO && DT == DRK_F16), "8-bit pages: head_dim 128, fp16 products, the rows' log-sum-exps given");
     constexpr int RB = D * 2;
+    constexpr int SRB = Q8 ? D : RB;                         // bytes of a token row of one kv head in its page
     constexpr int kTileBytes = kPfBN * RB, kTileShift = D == 128 ? 14 : 15;
     constexpr int NKS = D / 16;
     constexpr int kRing = 4, ROWS = 8;                       // buffers; tokens of a tile one wave requests
@@ -2441,7 +2447,18 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
 #pragma unroll
         for (int ks = 0; ks < NKS; ks++) {
             const uint4 v = row_live ? *(const uint4 *)(qrow + ks * 32) : make_uint4(0, 0, 0, 0);
-            qf[ks] = FOLD ? make_uint4(scaled(v.x), scaled(v.y), scaled(v.z), scaled(v.w)) : v;
+            if constexpr (FOLD) {
+                qf[ks] = make_uint4(scaled(v.x), scaled(v.y), scaled(v.z), scaled(v.w));
+            } else if constexpr (IO == DRK_BF16 && DT == DRK_F16) {     // 8-bit pages multiply in fp16
+#if defined(__HIP_DEVICE_COMPILE__)
+                qf[ks] = make_uint4(__builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.x), bf16_hi(v.x))),
+                                    __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.y), bf16_hi(v.y))),
+                                    __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.z), bf16_hi(v.z))),
+                                    __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(bf16_lo(v.w), bf16_hi(v.w))));
+#endif
+            } else {
+                qf[ks] = v;
+            }
         }
     }
     // the rows this lane's registers stand for: tokens [0, vis[i]) are visible to row i (0: an idle row); the
@@ -2473,6 +2490,7 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         return tg < lim_part ? table_k[tg >> sh] : -1;
     };
     const uint8_t *p_src = kbase;
+    const uint8_t *p_sc = kbase;                             // int8: the fp16 scales of the wave's rows
     int p_rows = 0;
     uint32_t p_lds = 0;
     const uint32_t k_ring = pf_lds_addr(&k_ldsm[0][0]) + (uint32_t)(tgw * RB);
@@ -2481,7 +2499,9 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         const int tg = kt * kPfBN + tgw;
         const bool ok = blk0 >= 0 && blk0 < A.NB && tg < lim_part;
         p_rows = ok ? lim_part - tg : 0;
-        p_src = kbase + (size_t)(ok ? blk0 : 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
+        p_src = kbase + (size_t)(ok ? blk0 : 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * SRB);
+        if constexpr (KV == DRK_INT8)
+            p_sc = A.pool_layer + (size_t)(ok ? blk0 : 0) * A.block_stride + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + (tg & (A.bs - 1))) * 2;
         p_lds = k_ring + ((uint32_t)(kt & (kRing - 1)) << kTileShift);
         if (lane == 0) valid_ldsm[kt & (kRing - 1)][w] = ok ? 1 : 0;
     };
@@ -2489,7 +2509,9 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         const int blk0 = __builtin_amdgcn_readfirstlane(blk_raw);
         const int tg = kt * kPfBN + tgw;
         p_rows = ROWS;
-        p_src = kbase + (size_t)blk0 * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
+        p_src = kbase + (size_t)blk0 * A.block_stride + (size_t)((tg & (A.bs - 1)) * SRB);
+        if constexpr (KV == DRK_INT8)
+            p_sc = A.pool_layer + (size_t)blk0 * A.block_stride + 2 * (size_t)A.kv_plane + ((size_t)kvh * A.bs + (tg & (A.bs - 1))) * 2;
         p_lds = k_ring + ((uint32_t)(kt & (kRing - 1)) << kTileShift);
         if (lane == 0) valid_ldsm[kt & (kRing - 1)][w] = 1;
     };
@@ -2501,14 +2523,64 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         for (int j = 0; j < NREQ; j++) goff[j] = (uint32_t)(rr * RB + ((cp ^ ((tgw + RPQ * j + rr) & 15)) << 4));
     }
     bool whole = false;                                      // the last tile requested made all NREQ requests
+    // 8-bit pages: the codes (and scale) of the tile requested last, 16 of row lane / 8 per lane; where they go, how
+    // many of the wave's rows exist
+    uint4 stg = make_uint4(0, 0, 0, 0);
+    uint32_t stg_sc = 0, c_lds = 0;
+    int c_rows = 0;
+    bool stg_live = false;
+    constexpr int NREQ_EFF = Q8 ? 1 : NREQ;
     auto request = [&](int j) {
-        if (__builtin_expect(whole, 1)) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
-        else if (RPQ * j + lane / LPR < p_rows) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
+        if constexpr (Q8) {
+            if (j == 0) {
+                const bool ok = whole || (lane >> 3) < p_rows;
+                stg = ok ? *(const uint4 *)(p_src + lane * 16) : make_uint4(0, 0, 0, 0);
+                if constexpr (KV == DRK_INT8) stg_sc = ok ? (uint32_t)*(const uint16_t *)(p_sc + (lane >> 3) * 2) : 0u;
+                c_lds = p_lds;
+                c_rows = p_rows;
+                stg_live = true;
+            }
+        } else {
+            if (__builtin_expect(whole, 1)) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
+            else if (RPQ * j + lane / LPR < p_rows) pf_load_to_lds16(p_src + 1024 * j, goff[j], p_lds + 1024 * j);
+        }
+    };
+    // 8-bit pages: the staged codes as fp16 values (code x scale, rounded once; fp8 exact) into the wave's rows of their
+    // buffer -- 16 dims = two 16-byte chunks 2 c, 2 c + 1 of row r, at positions chunk ^ (r & 15); rows past the end as zeros
+    auto commit = [&]() {
+        if constexpr (Q8) {
+            typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+            uint32_t h[8];
+            if constexpr (KV == DRK_INT8) {
+                int8x4_to_f16x4(stg.x, h[0], h[1]);
+                int8x4_to_f16x4(stg.y, h[2], h[3]);
+                int8x4_to_f16x4(stg.z, h[4], h[5]);
+                int8x4_to_f16x4(stg.w, h[6], h[7]);
+                const h2 scale = __builtin_bit_cast(h2, stg_sc | (stg_sc << 16));
+                const h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+#pragma unroll
+                for (int i = 0; i < 8; i++) h[i] = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(h2, h[i]) - bias) * scale);
+            } else {
+                fp8x4_to_f16x4(stg.x, h[0], h[1]);
+                fp8x4_to_f16x4(stg.y, h[2], h[3]);
+                fp8x4_to_f16x4(stg.z, h[4], h[5]);
+                fp8x4_to_f16x4(stg.w, h[6], h[7]);
+            }
+            const int row = lane >> 3, c0 = (lane & 7) * 2, sw = (tgw + row) & 15;
+            if (row >= c_rows) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) h[i] = 0u;
+            }
+            const uint32_t rb = c_lds - pf_lds_addr(&k_ldsm[0][0]) + (uint32_t)(row * RB);
+            *(uint4 *)(&k_ldsm[0][0] + rb + ((c0 ^ sw) << 4)) = make_uint4(h[0], h[1], h[2], h[3]);
+            *(uint4 *)(&k_ldsm[0][0] + rb + (((c0 + 1) ^ sw) << 4)) = make_uint4(h[4], h[5], h[6], h[7]);
+        }
     };
     auto request_tile = [&]() {
         whole = p_rows >= ROWS;
 #pragma unroll
-        for (int j = 0; j < NREQ; j++) request(j);
+        for (int j = 0; j < NREQ_EFF; j++) request(j);
+        if constexpr (Q8) commit();                          // (the prologue: straight into LDS)
     };
 
     // where this lane finds its B operands: K row n (and n + 32), chunk 2 ks + g at byte ((g ^ n & 15) << 4) ^ (ks << 5)
@@ -2559,6 +2631,7 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
             plan(t0 + 2, b2);
             request_tile();
             __builtin_amdgcn_s_waitcnt(0x0f70);                  // vmcnt(0)
+            stg_live = false;
         }
         __syncthreads();
         pf_f32x16 s_even[2], s_odd[2];
@@ -2625,9 +2698,14 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
                 }
             }
             // K(it + 1) has landed (this wave's share; the requests of K(it + 2) came after it), then everybody's
-            if (FAST || __builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
-            else __builtin_amdgcn_s_waitcnt(0x0f70);
+            if constexpr (!Q8) {
+                if (FAST || __builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
+                else __builtin_amdgcn_s_waitcnt(0x0f70);
+            }
             pf_barrier_lgkm();
+            if constexpr (Q8) {
+                if (stg_live) commit();                          // K(it + 2), requested a step ago, read behind the next barrier
+            }
             if constexpr (!FAST) {
                 asm volatile("" : : "s"(blk_ahead));
                 plan(it + 3, blk_ahead);                         // into the buffer of K(it - 1), read two steps ago
@@ -2642,13 +2720,17 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
                         plan_whole(it + 3, blk_ahead);
                         whole = true;
                     }
-                    if ((ks & 1) == 1 && (ks >> 1) < NREQ) pf_load_to_lds16(p_src + 1024 * (ks >> 1), goff[ks >> 1], p_lds + 1024 * (ks >> 1));
+                    if constexpr (Q8) {
+                        if (ks == 1) request(0);
+                    } else {
+                        if ((ks & 1) == 1 && (ks >> 1) < NREQ) pf_load_to_lds16(p_src + 1024 * (ks >> 1), goff[ks >> 1], p_lds + 1024 * (ks >> 1));
+                    }
                 } else {
                     if (ks == 0) {
                         fa = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][0];
                         fb = *(const int4 *)&valid_ldsm[(it + 1) & (kRing - 1)][4];
                     }
-                    if ((ks & 1) == 0 && (ks >> 1) < NREQ) request(ks >> 1);
+                    if ((ks & 1) == 0 && (ks >> 1) < NREQ_EFF) request(ks >> 1);
                 }
                 if constexpr (!LSE) {
                     if (ks == NKS / 2) {
@@ -3439,7 +3521,8 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
     // parts for that reason alone -- which the two-walk call cannot do)
     const int massd_cap = (a.D == 128 ? kMassdBlocks<128> : kMassdBlocks<256>) - 8;      // a part's range is rounded to tiles and to blocks
     const int massd_min_parts = ((pos_start + M + a.bs - 1) / a.bs + massd_cap - 1) / massd_cap;
-    if (g_prefill_mass_direct && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && A.bs_shift >= 4 &&
+    const bool q8 = a.dtype == DRK_INT8 || a.dtype == DRK_FP8_E4M3;       // 8-bit pages: head_dim 128, the one-walk call
+    if (g_prefill_mass_direct && (a.dtype == DRK_BF16 || a.dtype == DRK_F16 || (q8 && a.D == 128 && d_row_lse)) && A.bs_shift >= 4 &&
         (d_row_lse || massd_min_parts == 1) && a.QH / a.KVH <= 128) {
         A.tpw = 256 / (a.QH / a.KVH);
         A.nqt = (M + A.tpw - 1) / A.tpw;
@@ -3458,10 +3541,20 @@ static int prefill_mass_impl(const drk_kv_layout *g, const void *q, const void *
             else if (kind == 1) hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, true, false>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
             else hipLaunchKernelGGL((prefill_massd_kernel<DT, DT, DD, false, false>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
         } while (0)
-        if (a.dtype == DRK_BF16 && a.D == 128) DRK_PMD(DRK_BF16, 128);
+#define DRK_PMD8(KV, IO)                                                                                                  \
+        do {                                                                                                             \
+            if (kind == 1) hipLaunchKernelGGL((prefill_massd_kernel<DRK_F16, IO, 128, true, false, KV>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
+            else hipLaunchKernelGGL((prefill_massd_kernel<DRK_F16, IO, 128, false, false, KV>), gridd, dim3(512), 0, st, A, d_block_mass, mass_len);  \
+        } while (0)
+        if (a.dtype == DRK_INT8 && io_dtype == DRK_BF16) DRK_PMD8(DRK_INT8, DRK_BF16);
+        else if (a.dtype == DRK_INT8) DRK_PMD8(DRK_INT8, DRK_F16);
+        else if (a.dtype == DRK_FP8_E4M3 && io_dtype == DRK_BF16) DRK_PMD8(DRK_FP8_E4M3, DRK_BF16);
+        else if (a.dtype == DRK_FP8_E4M3) DRK_PMD8(DRK_FP8_E4M3, DRK_F16);
+        else if (a.dtype == DRK_BF16 && a.D == 128) DRK_PMD(DRK_BF16, 128);
         else if (a.dtype == DRK_BF16) DRK_PMD(DRK_BF16, 256);
         else if (a.D == 128) DRK_PMD(DRK_F16, 128);
         else DRK_PMD(DRK_F16, 256);
+#undef DRK_PMD8
 #undef DRK_PMD
         DRK_LAUNCH_CHECK("prefill_massd_kernel");
         return DRK_OK;

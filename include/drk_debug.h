@@ -55,10 +55,10 @@ void drk_debug_set_prefill_pieces(int mode);
  * and a value wave (V^T P^T) per 32 rows; 0 = four waves, each does both products of its 32 rows.  Same walks,
  * same pieces, same bits. */
 void drk_debug_set_prefill_d256_waves(int mode);
-/* Mass passes (drk_paged_prefill_attention_mass[_lse]) over 16-bit pages: 1 (default) = the kernel that takes
- * 256 rows per workgroup and its K tiles straight into LDS (blocks of 16 * 2^k tokens; the two-walk call up to
- * 8 184 / 6 136 logical blocks of context at head_dim 128 / 256); 0 = the register-staging kernel, which also
- * serves every other case. */
+/* Mass passes (drk_paged_prefill_attention_mass[_lse]): 1 (default) = the kernel that takes 256 rows per workgroup
+ * and, on 16-bit pages, its K tiles straight into LDS (blocks of 16 * 2^k tokens; the two-walk call up to
+ * 8 184 / 6 136 logical blocks of context at head_dim 128 / 256; 8-bit pages: the one-walk call at head_dim 128,
+ * codes staged through registers); 0 = the register-staging kernel, which also serves every other case. */
 void drk_debug_set_prefill_mass_direct(int on);
 /* The one-walk mass kernels cut every walk into parts (ranges of tiles) when a chunk has few walks, so that a
  * short frame behind a long context fills the chip: 0 (default) = the library's rule (256 or 512 workgroups, a

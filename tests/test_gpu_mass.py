@@ -151,7 +151,8 @@ def test_block_mass_argument_errors(dev):
 
 @pytest.fixture(params=["tiles_straight_into_lds", "tiles_through_registers"])
 def mass_kernel(request):
-    """The two one-walk mass kernels for 16-bit pages (8-bit pages have the second only)."""
+    """The two one-walk mass kernels (8-bit pages: the first at head_dim 128 with a power-of-two block size, staged
+    through registers on their way into LDS; the second otherwise)."""
     lib = cabi.lib()
     lib.drk_debug_set_prefill_mass_direct(1 if request.param == "tiles_straight_into_lds" else 0)
     yield request.param
@@ -256,10 +257,9 @@ def chunk_path(request):
 def test_frame_mass_from_the_attention_calls_row_sums(dev, chunk_path, mass_kernel, dtype, bs, pos_start, M, heads):
     """The attention call leaves every row's log-sum-exp, the mass pass then walks the keys once: same masses as the
     two-walk pass within the tolerance of the fp64 oracle, same attention output as the call without the extra result.
-    Both one-walk kernels: the one that takes 256 rows per workgroup and its tiles straight into LDS (16-bit pages; head
-    counts that leave idle rows, walks that end inside a tile and inside a page, holes) and the register-staging one."""
-    if mass_kernel == "tiles_straight_into_lds" and dtype in (cabi.INT8, cabi.FP8_E4M3):
-        pytest.skip("8-bit pages have one mass kernel")
+    Both one-walk kernels: the one that takes 256 rows per workgroup and its tiles straight into LDS (8-bit pages: by
+    way of registers; head counts that leave idle rows, walks that end inside a tile and inside a page, holes) and the
+    register-staging one."""
     total = pos_start + M
     holes = (1,) if total > 3 * bs else ()
     g, og, io, table, opool, q = _frame_case(dtype, bs, seed=bs + pos_start + M, pos_start=pos_start, M=M, heads=heads, holes=holes)
@@ -293,7 +293,8 @@ def test_frame_mass_from_the_attention_calls_row_sums(dev, chunk_path, mass_kern
 
 
 @pytest.mark.parametrize("dtype,bs,pos_start,M,heads", [(cabi.BF16, 16, 1500, 100, (8, 32, 128)), (cabi.F16, 256, 2500, 70, (4, 24, 256)),
-                                                        (cabi.F16, 64, 900, 300, (2, 14, 128))])
+                                                        (cabi.F16, 64, 900, 300, (2, 14, 128)), (cabi.INT8, 16, 1500, 100, (8, 32, 128)),
+                                                        (cabi.FP8_E4M3, 32, 1100, 260, (2, 8, 128))])
 def test_frame_mass_where_every_block_has_a_page(dev, mass_kernel, dtype, bs, pos_start, M, heads):
     """No holes: the kernel for 16-bit pages takes its lean steps through the interior of every walk (no validity flags,
     no masks) and the general ones at the ends.  The two-walk call and the one-walk call against fp64."""
@@ -329,10 +330,8 @@ def test_frame_mass_where_every_block_has_a_page(dev, mass_kernel, dtype, bs, po
 def test_frame_mass_with_the_context_in_parts(dev, mass_kernel, parts, dtype, bs, pos_start, M, heads, holes):
     """A short frame behind a long context has few walks; the one-walk kernels cut them into parts (by their rule:
     16-tile parts for the first case; forced: 3 and 40 per walk, more parts than some walks have tiles) -- the kernel
-    for 16-bit pages and the register-staging one, which 8-bit pages and block sizes that are no power of two take.
+    with 256 rows per workgroup and the register-staging one, which block sizes that are no power of two take.
     Masses against fp64 and against the same call with whole walks."""
-    if mass_kernel == "tiles_straight_into_lds" and dtype in (cabi.INT8, cabi.FP8_E4M3):
-        pytest.skip("8-bit pages have one mass kernel")
     lib = cabi.lib()
     g, og, io, table, opool, q = _frame_case(dtype, bs, seed=bs + M, pos_start=pos_start, M=M, heads=heads, holes=holes)
     KVH, QH, D = heads
