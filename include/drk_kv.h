@@ -449,10 +449,10 @@ int drk_paged_prefill_attention_mass(const drk_kv_layout *g, const void *q, cons
  * token) -- the chunk kernels know it where a row's walk ends.  drk_paged_prefill_attention_mass_lse is the mass
  * pass given those values: it reads K once.  It may run on another stream behind an event (it reads q, the pages
  * and d_row_lse; nothing the attention call wrote except d_row_lse).  Head_dim 128 or 256, block_size % 16 == 0;
- * DRK_ERR_UNSUPPORTED otherwise.  Over 16-bit pages (blocks of 16 * 2^k tokens) the pass scores the way the attention
- * call did and a row's masses sum to 1 within 1e-6;
- * over 8-bit pages the two calls round Q differently for some chunk lengths (the long-chunk kernels fold the scale
- * into Q in its 16-bit type) and the sum is 1 within 2e-3.  d_row_lse must come from the attention call for the same
+ * DRK_ERR_UNSUPPORTED otherwise.  Over 16-bit pages, and over 8-bit pages at head_dim 128 (blocks of 16 * 2^k tokens
+ * either way), the pass scores the way the attention call did and a row's masses sum to 1 within 1e-6;
+ * over 8-bit pages at head_dim 256, and with other block sizes, the two calls round Q differently for some chunk
+ * lengths (the long-chunk kernels fold the scale into Q in its 16-bit type) and the sum is 1 within 2e-3.  d_row_lse must come from the attention call for the same
  * chunk with the library's debug switches unchanged in between. */
 int drk_paged_prefill_attention_lse(const drk_kv_layout *g, const void *q, const void *pool,
                                     const int32_t *d_block_table, void *out, int layer, int pos_start, int M,
