@@ -1076,6 +1076,15 @@ def kernel_fractions(buf, seed=11):
                   cabi.BF16, cabi.p(lse), cabi.p(mass), total // bs, 1, sp)
 
     frame_mass["short_frame_64_rows"] = {"attention_us": timed(short_attn), "with_one_walk_mass_us": timed(short_both)}
+    # ... and 16 rows at 32 752: 64 of a workgroup's 256 rows exist, the other six waves only move tiles
+    chunk = 16
+    pos = total - chunk
+    q = torch.randn(chunk, QH, D, device="cuda").to(torch.bfloat16)
+    o = torch.empty_like(q)
+    lse = torch.empty(chunk * QH, dtype=torch.float32, device="cuda")
+    wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos, chunk)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda")
+    frame_mass["short_frame_16_rows"] = {"attention_us": timed(short_attn), "with_one_walk_mass_us": timed(short_both)}
     q, o, lse, chunk, pos = big
     # the last chunk's launch once more on constant data (every K and V element 0.5, every Q element 0.25): the same
     # instructions on the same addresses -- what differs is how many bits toggle, i.e. the clock the part holds

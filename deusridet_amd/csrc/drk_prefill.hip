@@ -2371,7 +2371,8 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void prefill_mass_kernel(Pre
 // 16 products of 32 clocks -- so the steps in the interior of a part (no masked row, every block with a page, the
 // tile requested whole: all but the last three or four of a walk) run a lean form: no validity flags, no
 // conditions, the request's plan behind the first operand reads, the table entry loaded where the barrier's wait
-// covers it, page sums without the exchange between the wave's halves.  S = Q K^T as
+// covers it, page sums without the exchange between the wave's halves.  A wave none of whose rows exists (a short
+// frame) only takes part in the barriers and the requests.  S = Q K^T as
 // in prefill_mass_kernel: a lane stands for a key, its registers for 16 of the wave's rows, a key's sum over rows is
 // a sum over registers.  A page's sum goes to a table in LDS (one entry per logical block of the walk) and the
 // table to `mass` with one atomic per block and workgroup when the walk ends -- 256 workgroups adding to the same
@@ -2479,6 +2480,11 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // from here on the kernel counts its loads itself
+    bool wave_live;                                          // one of the wave's 32 rows exists
+    {
+        const int rt = (w * 32 + n) / G;
+        wave_live = __builtin_amdgcn_ballot_w64(rt < TPW && qt * TPW + rt < A.M) != 0ull;
+    }
 
     const uint8_t *kbase = A.pool_layer + (size_t)kvh * A.head_stride;
     const int tgw = w * ROWS;
@@ -2668,6 +2674,30 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         constexpr float kLazy = 8.0f;
         // FAST: a step in the part's interior -- no row of tile it is masked, every block has a page, tile it + 3 is
         // whole for every wave: no flags, no conditions, and the plan behind the first operand reads
+        // a wave none of whose 32 rows exists (a short frame: 16 tokens x 4 heads fill two of the eight waves) does the
+        // step's memory side only -- the barrier, its share of the next tile's request -- and leaves the SIMD to its neighbour
+        auto idle_step = [&](auto fast_mode, int it) {
+            constexpr bool FAST = decltype(fast_mode)::value;
+            if constexpr (!Q8) {
+                if (FAST || __builtin_expect(whole, 1)) __builtin_amdgcn_s_waitcnt(NREQ == 2 ? 0x0f72 : 0x0f74);   // vmcnt(NREQ)
+                else __builtin_amdgcn_s_waitcnt(0x0f70);
+            }
+            pf_barrier_lgkm();
+            if constexpr (Q8) {
+                if (stg_live) commit();
+            }
+            if constexpr (FAST) {
+                plan_whole(it + 3, blk_ahead);
+                whole = true;
+            } else {
+                plan(it + 3, blk_ahead);
+                whole = p_rows >= ROWS;
+            }
+            blk_ahead = page_of(it + 4);
+#pragma unroll
+            for (int j = 0; j < NREQ_EFF; j++) request(j);
+            flags = 255;                                         // (its scores are never looked at)
+        };
         auto step = [&](auto fast_mode, int it, pf_f32x16 (&s)[2], pf_f32x16 (&s_next)[2]) {
             constexpr bool FAST = decltype(fast_mode)::value;
             // here: s = exponents of tile it; K(it + 1) and K(it + 2) requested
@@ -2763,6 +2793,11 @@ __global__ __launch_bounds__(512, 1) void prefill_massd_kernel(PrefillArgs A, fl
         // steps [t0, fast_end) can run in the fast mode: tile it unmasked, tile it + 3 whole for every wave
         const int fast_end = holes ? t0 : min(first_masked_tile, lim_part / kPfBN - 3);
         int it = t0;
+        if (__builtin_expect(!wave_live, 0)) {                   // the same steps, the same barriers
+            for (; it < fast_end; it++) idle_step(std::true_type{}, it);
+            for (; it < ntiles; it++) idle_step(std::false_type{}, it);
+            return;
+        }
         for (; it + 2 <= fast_end; it += 2) {
             step(std::true_type{}, it, s_even, s_odd);
             step(std::true_type{}, it + 1, s_odd, s_even);
