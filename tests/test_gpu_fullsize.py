@@ -264,15 +264,20 @@ def test_reference_model_shape_full_chunk_prefill_rows(dev):
         assert ok, (mode, ma)
 
 
-@pytest.mark.parametrize("shape", ["config5", "reference_model"])
+@pytest.mark.parametrize("shape", ["config5", "reference_model", "config5_int8", "config5_fp8"])
 def test_full_chunk_frame_mass(dev, shape):
-    """The attention mass of a full 2 048-token chunk at position 30 720 (config 5's shape, and the reference model's):
-    the attention call leaves the rows' log-sum-exps, the one-walk pass adds every row's probabilities up by page.
-    Against fp32 softmax in torch over the stored K (all 2 048 x QH rows over 32 768 keys, summed per block), the
-    pages of the whole context sum to rows x heads, and the register-staging kernel gives the same masses."""
+    """The attention mass of a full 2 048-token chunk at position 30 720 (config 5's shape over bf16, int8 and fp8
+    pages, and the reference model's): the attention call leaves the rows' log-sum-exps, the one-walk pass adds every
+    row's probabilities up by page.  Against fp32 softmax in torch over the stored K (dequantised for 8-bit pages; all
+    2 048 x QH rows over 32 768 keys, summed per block), the pages of the whole context sum to rows x heads, and the
+    register-staging kernel gives the same masses."""
     torch = _torch()
+    io = None
     if shape == "config5":
         L, KVH, QH, D, bs, dt, tdt, amp = 1, 8, 32, 128, 16, cabi.BF16, torch.bfloat16, 1.0
+    elif shape in ("config5_int8", "config5_fp8"):
+        L, KVH, QH, D, bs, dt, tdt, amp = 1, 8, 32, 128, 16, (cabi.INT8 if shape == "config5_int8" else cabi.FP8_E4M3), torch.bfloat16, 1.0
+        io = cabi.BF16
     else:
         L, KVH, QH, D, bs, dt, tdt, amp = 1, 4, 24, 256, 256, cabi.F16, torch.float16, 0.5
     total, M = 32768, 2048
@@ -288,8 +293,11 @@ def test_full_chunk_frame_mass(dev, shape):
     for p0 in range(0, total, 8192):
         k = (torch.randn(8192, KVH, D, device="cuda", generator=gen) * amp).to(tdt)
         v = (torch.randn(8192, KVH, D, device="cuda", generator=gen) * amp).to(tdt)
-        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(table), 0, 1, p0, 8192, U.p(k), U.p(v), dt, sp)
+        cabi.call("drk_kv_append_batch", C.byref(g), U.p(pool), U.p(table), 0, 1, p0, 8192, U.p(k), U.p(v), io if io is not None else dt, sp)
         U.sync()
+    q8 = io is not None
+    if not q8:
+        io = dt
     q = (torch.randn(M, QH, D, device="cuda", generator=gen) * amp).to(tdt)
     out = torch.zeros_like(q)
     scale = 1 / np.sqrt(D)
@@ -297,22 +305,33 @@ def test_full_chunk_frame_mass(dev, shape):
     wsb = lib.drk_prefill_workspace_bytes(C.byref(g), pos_start, M)
     ws = torch.zeros(max(wsb, 16), dtype=torch.uint8, device="cuda")
     cabi.call("drk_paged_prefill_attention_lse", C.byref(g), U.p(q), U.p(pool), U.p(table), U.p(out), 0, pos_start, M,
-              float(scale), dt, None, 0, U.p(lse), U.p(ws), wsb, sp)
+              float(scale), io, None, 0, U.p(lse), U.p(ws), wsb, sp)
     got = {}
     try:
         for direct in (1, 0):
             lib.drk_debug_set_prefill_mass_direct(direct)
             mass = torch.full((NB,), 7.0, dtype=torch.float32, device="cuda")
             cabi.call("drk_paged_prefill_attention_mass_lse", C.byref(g), U.p(q), U.p(pool), U.p(table), 0, pos_start, M,
-                      float(scale), dt, U.p(lse), U.p(mass), NB, 0, sp)
+                      float(scale), io, U.p(lse), U.p(mass), NB, 0, sp)
             U.sync()
             got[direct] = mass.double().cpu().numpy()
     finally:
         lib.drk_debug_set_prefill_mass_direct(1)
-    flat = torch.empty(2 * total * KVH * D, dtype=tdt, device="cuda")
-    cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(pool), U.p(table), 0, total, 1, sp)
-    U.sync()
-    kk = flat.view(2, total, KVH, D)[0].float()
+    if q8:                                                   # codes and scales through the C ABI, dequantised here
+        codes = torch.empty(2 * total * KVH * D, dtype=torch.uint8, device="cuda")
+        scales = torch.empty(2 * total * KVH, dtype=torch.float16, device="cuda") if dt == cabi.INT8 else None
+        cabi.call("drk_kv_extract", C.byref(g), U.p(codes), U.p(scales), U.p(pool), U.p(table), 0, total, 1, sp)
+        U.sync()
+        if dt == cabi.INT8:
+            kk = codes.view(torch.int8).view(2, total, KVH, D)[0].float() * scales.view(2, total, KVH, 1)[0].float()
+        else:
+            kk = codes.view(torch.float8_e4m3fn).view(2, total, KVH, D)[0].float()
+        del codes
+    else:
+        flat = torch.empty(2 * total * KVH * D, dtype=tdt, device="cuda")
+        cabi.call("drk_kv_extract", C.byref(g), U.p(flat), None, U.p(pool), U.p(table), 0, total, 1, sp)
+        U.sync()
+        kk = flat.view(2, total, KVH, D)[0].float()
     G = QH // KVH
     keys = torch.arange(total, device="cuda")
     want = torch.zeros(total, dtype=torch.float64, device="cuda")
