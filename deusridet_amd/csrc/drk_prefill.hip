@@ -1008,9 +1008,13 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
     __shared__ __align__(256) uint8_t k_lds3[kRing][kTileBytes];    // 256: the xor swizzle is applied to whole addresses
     __shared__ __align__(256) uint8_t v_lds3[kRing][kTileBytes];
 
-    const int kvh = (int)blockIdx.x % A.KVH;
-    const int nqt = (int)gridDim.x / A.KVH;
-    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    // workgroup = (walk, part): a walk is (row block, kv head); A.kparts > 1 (a chunk too short to fill the chip with its
+    // walks): a part is one of A.kparts ranges of the walk's tiles and leaves (o, m, l) per row for prefill_merge_kernel
+    const int kp = A.kparts;
+    const int walk = (int)blockIdx.x / kp, part = (int)blockIdx.x - walk * kp;
+    const int kvh = walk % A.KVH;
+    const int nqt = (int)gridDim.x / (A.KVH * kp);
+    const int qt = nqt - 1 - walk / A.KVH;                   // the longest walks are dispatched first
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
@@ -1024,7 +1028,14 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
     const int vis = A.pos_start + tq + 1;
     const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
     const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
-    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+    const int nt_walk = (lim_wg + kPfBN - 1) / kPfBN;
+    const int t_begin = __builtin_amdgcn_readfirstlane((int)((long)part * nt_walk / kp));
+    const int ntiles = __builtin_amdgcn_readfirstlane((int)((long)(part + 1) * nt_walk / kp));   // the part's tiles: [t_begin, ntiles)
+    const int lim_part = min(lim_wg, ntiles * kPfBN);        // nothing past the part's end is requested
+    if (t_begin >= ntiles) {                                 // more parts than tiles: an empty piece
+        if (row_live && g == 0) A.part_l[((size_t)tq * A.QH + head) * kp + part] = 0.0f;
+        return;
+    }
 
     // Q as the B operand, multiplied by scale * log2(e) on the way in (rounded once more to the 16-bit
     // type): the products then are the exponents themselves and the softmax needs no multiply per score.
@@ -1058,8 +1069,8 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
         return i < nblk_needed ? A.table[i] : -1;             // entries past the chunk's last block are never read
     };
     auto pages_of = [&](int win) -> unsigned long long { return __builtin_amdgcn_ballot_w64(win >= 0 && win < A.NB); };
-    int win_lb0 = 0;
-    int win_a = load_window(0), win_b = load_window(64);
+    int win_lb0 = (((t_begin * kPfBN) >> sh) >> 6) << 6;
+    int win_a = load_window(win_lb0), win_b = load_window(win_lb0 + 64);
     unsigned long long present_a = pages_of(win_a);           // bit i: block win_lb0 + i has a page
     // the wave's page in `tile` (-1: a hole, or past the end) and the tile's four page flags, one per 16-token run
     auto lookup = [&](int tile, int &blk, int &flags) {
@@ -1075,7 +1086,7 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
         const int tg = tile * kPfBN + tgw;
         const int li = (tg >> sh) - win_lb0;
         const int b = __builtin_amdgcn_readlane(win_a, li);
-        blk = (((present_a >> li) & 1ull) != 0 && tg < lim_wg) ? b : -1;
+        blk = (((present_a >> li) & 1ull) != 0 && tg < lim_part) ? b : -1;
     };
 
     pf_f32x16 o[NDT];
@@ -1271,7 +1282,7 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
         int blk;
         lookup(kt, blk, f_new);
         const int tg = kt * kPfBN + tgw;
-        rows = blk >= 0 ? lim_wg - tg : 0;
+        rows = blk >= 0 ? lim_part - tg : 0;
         ksrc = kbase + (size_t)max(blk, 0) * A.block_stride + (size_t)((tg & (A.bs - 1)) * RB);
     };
     auto stage = [&](int kt, int &f_new) {
@@ -1316,7 +1327,7 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
             const uint8_t *ksrc;
             int rows;
             find(kt, f_new, ksrc, rows);
-            const uint32_t lk = k_ring + ((uint32_t)kt << 14), lv = v_ring + ((uint32_t)kt << 14);
+            const uint32_t lk = k_ring + ((uint32_t)(kt & (kRing - 1)) << 14), lv = v_ring + ((uint32_t)(kt & (kRing - 1)) << 14);
             request(ksrc, goff_k[0], lk, 0, rows);
             request(ksrc, goff_k[1], lk + 4 * RB, 1, rows);
             vsrc_prev = ksrc + A.kv_plane;
@@ -1326,10 +1337,10 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
                 request(vsrc_prev, goff_v[1], lv + 4 * RB, 1, rows);
             }
         };
-        both(0, f0, true);
-        both(1, f1, true);
-        both(2, f2, false);
-        if (!grpA) stage(3, f3);                             // K(3), V(2)
+        both(t_begin, f0, true);
+        both(t_begin + 1, f1, true);
+        both(t_begin + 2, f2, false);
+        if (!grpA) stage(t_begin + 3, f3);                   // K(3), V(2) of the part
         wait_loads(std::integral_constant<int, 0>{});
         four_issued = four_before = false;
     }
@@ -1339,9 +1350,9 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
     // never read; requests past the last tile load nothing (no page).
     if (grpA) {
         // f0, f1, f2 = flags of tiles t, t + 1, t + 2 at the head of iteration t; stage(t + 3) adds tile t + 3's
-        qk(0);
+        qk(t_begin);
 #pragma unroll 1
-        for (int t = 0; t < ntiles; t++) {
+        for (int t = t_begin; t < ntiles; t++) {
             stage(t + 3, f3);                                // phase 2t: K(t+3), V(t+2)
             softmax(t, f0);
             f0 = f1;
@@ -1356,10 +1367,10 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
         pf_barrier_lds();
     } else {
         // f0 .. f3 = flags of tiles t .. t + 3 at the head of iteration t; stage(t + 4) adds tile t + 4's
-        qk(0);                                               // phase 0
+        qk(t_begin);                                         // phase 0
         pf_barrier_lds();
 #pragma unroll 1
-        for (int t = 0; t < ntiles; t++) {
+        for (int t = t_begin; t < ntiles; t++) {
             softmax(t, f0);                                  // phase 2t+1
             stage(t + 4, f4);                                // K(t+4), V(t+3)
             f0 = f1;
@@ -1375,6 +1386,22 @@ __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (kp > 1) {                                            // a piece: the sums as they are, relative to m_ref (log2 units)
+        if (row_live) {
+            const size_t slot = ((size_t)tq * A.QH + head) * kp + part;
+            if (g == 0) {
+                A.part_m[slot] = m_ref;
+                A.part_l[slot] = l_tot;
+            }
+            float *po = A.part_o + slot * D;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int b4 = 0; b4 < 4; b4++)
+                    *(float4 *)(po + dt * 32 + 8 * b4 + 4 * g) = make_float4(o[dt][4 * b4], o[dt][4 * b4 + 1], o[dt][4 * b4 + 2], o[dt][4 * b4 + 3]);
+        }
+        return;
+    }
     if (A.lse_rows && row_live && g == 0)      // m_ref is the reference the weights were taken against, in log2 units
         A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_ref + __builtin_log2f(l_tot) : INFINITY;
     if (row_live && (l_tot > 0.0f || A.gate)) {
@@ -3437,6 +3464,7 @@ static void prefill_split_shape(const Lay &a, int pos_start, int M, int *chunk_t
 //   16: 59 -> 18, 878 -> 42, 3 992 -> 115 us;  256: 66 -> 37, 868 -> 211, 3 857 -> 799 us;
 //   1 024: 92 -> 98, 928 -> 715, 3 896 -> 2 566 us.
 static bool d256_direct(const Lay &a);
+static int prefill_split_ppd_parts(const Lay &a, int pos_start, int M);
 static bool prefill_split_applies(const Lay &a, int pos_start, int M)
 {
     if (g_prefill_split == 0 || pos_start < kSplitMinPos) return false;
@@ -3460,7 +3488,7 @@ static bool d256_direct(const Lay &a)
 // (taken when the caller passes its workspace) do not.  The mass pass scores the way the attention call did.
 static bool chunk_kernel_scales_q(const Lay &a, int pos_start, int M)
 {
-    if (prefill_split_applies(a, pos_start, M)) return false;
+    if (prefill_split_applies(a, pos_start, M)) return prefill_split_ppd_parts(a, pos_start, M) != 0;
     if (d256_direct(a)) return true;
     const int G = a.QH / a.KVH;
     if (a.D == 128 && G <= 256 && a.bs >= 16 && ilog2_exact((unsigned)a.bs) >= 4 && g_prefill_two_phase != 0) {
@@ -3469,6 +3497,26 @@ static bool chunk_kernel_scales_q(const Lay &a, int pos_start, int M)
         return wgs2 >= 192 || g_prefill_two_phase > 1;
     }
     return false;
+}
+
+// A chunk of 16-bit pages at head_dim 128 with at least 256 rows per kv head takes the two-phase kernel on that path
+// too: every walk in parts, one workgroup per CU, the same (o, m, l) pieces and the same merge.  Returns the number of
+// parts per walk (never more than the pieces the workspace was sized for), or 0 for the four-wave kernel.
+static int prefill_split_ppd_parts(const Lay &a, int pos_start, int M)
+{
+    if (!(a.D == 128 && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && a.bs >= 16 && ilog2_exact((unsigned)a.bs) >= 4)) return 0;
+    if (g_prefill_two_phase == 0 || g_prefill_two_phase == 3) return 0;
+    const int G = a.QH / a.KVH;
+    if (G > 256 || (long)M * G < 256) return 0;
+    const int tpw2 = 256 / G;
+    const long walks = (long)((M + tpw2 - 1) / tpw2) * a.KVH;
+    int ct, ns;
+    prefill_split_shape(a, pos_start, M, &ct, &ns);
+    const int shortest = (pos_start + 1 + kPfBN - 1) / kPfBN;          // tiles of the first row block's walk, at least
+    long kp = 256 / walks;
+    if (kp > shortest / 8) kp = shortest / 8;
+    if (kp > ns) kp = ns;
+    return kp >= 2 ? (int)kp : 0;
 }
 
 static size_t prefill_split_need(const Lay &a, int pos_start, int M)
@@ -3713,11 +3761,16 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
         return fail(DRK_ERR_INVALID, "prefill: gate rows must be 16-byte aligned and at least head_dim apart");
     // a short chunk behind a long context: split the context over the chip (needs the workspace
     // drk_prefill_workspace_bytes reports; without it the chunk kernel below does the work)
+    int split_parts = 0;                                     // > 0: the two-phase kernel below, every walk in that many parts
     if (prefill_split_applies(a, pos_start, M) && workspace && ((uintptr_t)workspace % 16) == 0 &&
-        workspace_bytes >= prefill_split_need(a, pos_start, M))
-        return prefill_split(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
-                             (hipStream_t)stream, gate, gate_stride, lse_rows);
+        workspace_bytes >= prefill_split_need(a, pos_start, M)) {
+        split_parts = prefill_split_ppd_parts(a, pos_start, M);
+        if (split_parts == 0)
+            return prefill_split(a, q, pool, d_block_table, out, layer, pos_start, M, scale, io_dtype, workspace,
+                                 (hipStream_t)stream, gate, gate_stride, lse_rows);
+    }
     PrefillArgs A;
+    A.kparts = 1;
     A.pool_layer = (const uint8_t *)pool + (size_t)layer * a.layer_stride;
     A.table = d_block_table;
     A.q = (const uint8_t *)q;
@@ -3739,13 +3792,24 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
     if (a.D == 128 && G <= 256 && A.bs_shift >= 4 && g_prefill_two_phase != 0) {
         const int tpw2 = 256 / G;
         const long wgs2 = (long)((M + tpw2 - 1) / tpw2) * a.KVH;
-        if (wgs2 >= 192 || g_prefill_two_phase > 1) {
+        if (wgs2 >= 192 || g_prefill_two_phase > 1 || split_parts > 0) {
             A.tpw = tpw2;
-            dim3 grid2((unsigned)wgs2);
+            if (split_parts > 0) {                           // pieces into the caller's workspace, then the split path's merge
+                A.kparts = split_parts;
+                A.part_o = (float *)workspace;
+                A.part_m = A.part_o + (size_t)M * a.QH * split_parts * a.D;
+                A.part_l = A.part_m + (size_t)M * a.QH * split_parts;
+            }
+            dim3 grid2((unsigned)(wgs2 * A.kparts));
             if ((a.dtype == DRK_BF16 || a.dtype == DRK_F16) && g_prefill_two_phase != 3) {    // 16-bit pages: global -> LDS directly
                 if (a.dtype == DRK_BF16) hipLaunchKernelGGL((prefill_ppd_kernel<DRK_BF16, DRK_BF16>), grid2, dim3(512), 0, st, A);
                 else hipLaunchKernelGGL((prefill_ppd_kernel<DRK_F16, DRK_F16>), grid2, dim3(512), 0, st, A);
                 DRK_LAUNCH_CHECK("prefill_ppd_kernel");
+                if (split_parts > 0) {
+                    hipLaunchKernelGGL(prefill_merge_kernel<128>, dim3((unsigned)((size_t)M * a.QH)), dim3(64), 0, st, A.part_o, A.part_m,
+                                       A.part_l, (uint16_t *)out, split_parts, io_dtype, (const uint16_t *)gate, gate_stride, lse_rows);
+                    DRK_LAUNCH_CHECK("prefill_merge_kernel");
+                }
                 return DRK_OK;
             }
 #define DRK_PP_LAUNCH(DT, KV, IO) hipLaunchKernelGGL((prefill_pp_kernel<DT, KV, IO>), grid2, dim3(512), 0, st, A)
