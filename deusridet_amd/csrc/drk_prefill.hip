@@ -995,7 +995,9 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
 // phase is its instruction count -- a wave issues one instruction in about four clocks, scalar ones included --
 // so the phase is kept short: one straight path for whole pages, page addresses from scalar registers, the rare
 // cases (masked tiles, a moving softmax reference, pages in part) out of line.  8-bit pages keep the kernel above
-// (their codes are converted on the way).
+// (their codes are converted on the way).  A chunk too short to give every CU a walk (A.kparts > 1: the context-split
+// path, 256 or more rows per kv head) has every walk in parts -- ranges of its tiles, a workgroup each -- that leave
+// (o, m, l) per row for prefill_merge_kernel.
 template <int DT, int IO = DT>
 __global__ __launch_bounds__(512, 1) void prefill_ppd_kernel(PrefillArgs A)
 {
@@ -3463,6 +3465,8 @@ static void prefill_split_shape(const Lay &a, int pos_start, int M, int *chunk_t
 // keeps every CU busy.  Rows behind 2k / 32k / 128k tokens, chunk kernel -> split:
 //   16: 59 -> 18, 878 -> 42, 3 992 -> 115 us;  256: 66 -> 37, 868 -> 211, 3 857 -> 799 us;
 //   1 024: 92 -> 98, 928 -> 715, 3 896 -> 2 566 us.
+// (with the two-phase kernel walking its context in parts, prefill_split_ppd_parts, behind 32k tokens: 64 rows 70 -> 55,
+// 256 rows 211 -> 141, 1 024 rows 715 -> 487 us)
 static bool d256_direct(const Lay &a);
 static int prefill_split_ppd_parts(const Lay &a, int pos_start, int M);
 static bool prefill_split_applies(const Lay &a, int pos_start, int M)
