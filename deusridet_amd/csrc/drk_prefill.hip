@@ -675,9 +675,13 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     __shared__ __align__(16) uint8_t k_lds2[2][kPfBN * kPitchK];
     __shared__ __align__(16) uint8_t v_lds2[2][kPfBN * kPitchV];
 
-    const int kvh = (int)blockIdx.x % A.KVH;
-    const int nqt = (int)gridDim.x / A.KVH;
-    const int qt = nqt - 1 - (int)blockIdx.x / A.KVH;        // the longest walks are dispatched first
+    // workgroup = (walk, part), as in prefill_ppd_kernel: with A.kparts > 1 a part is one of A.kparts ranges of the
+    // walk's tiles and leaves (o, m, l) per row for prefill_merge_kernel
+    const int kp = A.kparts;
+    const int walk = (int)blockIdx.x / kp, part = (int)blockIdx.x - walk * kp;
+    const int kvh = walk % A.KVH;
+    const int nqt = (int)gridDim.x / (A.KVH * kp);
+    const int qt = nqt - 1 - walk / A.KVH;                   // the longest walks are dispatched first
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63;
     const int n = lane & 31, g = lane >> 5;
@@ -691,7 +695,14 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     const int vis = A.pos_start + tq + 1;
     const int lim_wg = A.pos_start + min((qt + 1) * TPW, A.M);
     const int first_masked_tile = (A.pos_start + qt * TPW + 1) / kPfBN;
-    const int ntiles = (lim_wg + kPfBN - 1) / kPfBN;
+    const int nt_walk = (lim_wg + kPfBN - 1) / kPfBN;
+    const int t_begin = __builtin_amdgcn_readfirstlane((int)((long)part * nt_walk / kp));
+    const int ntiles = __builtin_amdgcn_readfirstlane((int)((long)(part + 1) * nt_walk / kp));   // the part's tiles: [t_begin, ntiles)
+    const int lim_part = min(lim_wg, ntiles * kPfBN);        // rows past the part's end are stored as zeros
+    if (t_begin >= ntiles) {                                 // more parts than tiles: an empty piece
+        if (row_live && g == 0) A.part_l[((size_t)tq * A.QH + head) * kp + part] = 0.0f;
+        return;
+    }
 
     // Q as the B operand, multiplied by scale * log2(e) on the way in (rounded once more to the 16-bit
     // type): the products then are the exponents themselves and the softmax needs no multiply per score.
@@ -725,8 +736,8 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
         return i < nblk_needed ? A.table[i] : -1;             // entries past the chunk's last block are never read
     };
     auto pages_of = [&](int win) -> unsigned long long { return __builtin_amdgcn_ballot_w64(win >= 0 && win < A.NB); };
-    int win_lb0 = 0;
-    int win_a = load_window(0), win_b = load_window(64);
+    int win_lb0 = (((t_begin * kPfBN) >> sh) >> 6) << 6;
+    int win_a = load_window(win_lb0), win_b = load_window(win_lb0 + 64);
     unsigned long long present_a = pages_of(win_a);           // bit i: block win_lb0 + i has a page
     // the wave's page in `tile` (-1: a hole, or past the end) and the tile's four page flags, one per 16-token run
     auto lookup = [&](int tile, int &blk, int &flags) {
@@ -742,7 +753,7 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
         const int tg = tile * kPfBN + tgw;
         const int li = (tg >> sh) - win_lb0;
         const int b = __builtin_amdgcn_readlane(win_a, li);
-        blk = (((present_a >> li) & 1ull) != 0 && tg < lim_wg) ? b : -1;
+        blk = (((present_a >> li) & 1ull) != 0 && tg < lim_part) ? b : -1;
     };
 
     pf_f32x16 o[NDT];
@@ -786,7 +797,7 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
                 sc[j] = 0;
             }
         }
-        lim = blk >= 0 ? lim_wg - tg : 0;
+        lim = blk >= 0 ? lim_part - tg : 0;
     };
     auto stage_k = [&](int tile) {
         if constexpr (Q8) pf_store_group_q8<kPitchK, KV, RB, ROWS>(&k_lds2[tile & 1][0], kreg, w, lane, ksc, klim);
@@ -916,15 +927,15 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
         fl2 = f;
     };
 
-    // ---- prologue: K(0) in LDS; K(1) and V(0) in registers ----
+    // ---- prologue: K(0) in LDS; K(1) and V(0) in registers (tiles counted from the part's first) ----
     {
         int blk0;
-        lookup(0, blk0, fl1);
-        fetch(kreg, ksc, klim, false, 0, blk0);
-        stage_k(0);
-        lookup(1, blk_next, fl2);
-        fetch(kreg, ksc, klim, false, 1, blk_next);
-        fetch(vreg, vsc, vlim, true, 0, blk0);
+        lookup(t_begin, blk0, fl1);
+        fetch(kreg, ksc, klim, false, t_begin, blk0);
+        stage_k(t_begin);
+        lookup(t_begin + 1, blk_next, fl2);
+        fetch(kreg, ksc, klim, false, t_begin + 1, blk_next);
+        fetch(vreg, vsc, vlim, true, t_begin, blk0);
     }
     __syncthreads();
     // Both halves pass the same number of barriers, 2 ntiles + 1.  The loop bodies are straight-line code
@@ -933,9 +944,9 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     // A buffer is rewritten only between its last reader's barrier and its next reader's: K(x) in phases
     // 2x-3 or 2x-2, V(x) in phases 2x-1 or 2x (phase 2t: softmax of A / products of B for tile t).
     if (grpA) {
-        qk(0);
+        qk(t_begin);
 #pragma unroll 1
-        for (int t = 0; t < ntiles; t++) {
+        for (int t = t_begin; t < ntiles; t++) {
             stage(t);                                        // phase 2t: K(t+1), V(t)
             softmax(t, fl0);
             __syncthreads();
@@ -945,11 +956,11 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
         }
         __syncthreads();
     } else {
-        stage(0);                                            // phase 0: K(1), V(0)
-        qk(0);
+        stage(t_begin);                                      // phase 0: K(1), V(0)
+        qk(t_begin);
         __syncthreads();
 #pragma unroll 1
-        for (int t = 0; t < ntiles; t++) {
+        for (int t = t_begin; t < ntiles; t++) {
             softmax(t, fl0);
             stage(t + 1);                                    // phase 2t+1: K(t+2), V(t+1)
             __syncthreads();
@@ -960,6 +971,22 @@ __global__ __launch_bounds__(512, 1) void prefill_pp_kernel(PrefillArgs A)
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (kp > 1) {                                            // a piece: the sums as they are, relative to m_ref (log2 units)
+        if (row_live) {
+            const size_t slot = ((size_t)tq * A.QH + head) * kp + part;
+            if (g == 0) {
+                A.part_m[slot] = m_ref;
+                A.part_l[slot] = l_tot;
+            }
+            float *po = A.part_o + slot * D;
+#pragma unroll
+            for (int dt = 0; dt < NDT; dt++)
+#pragma unroll
+                for (int b4 = 0; b4 < 4; b4++)
+                    *(float4 *)(po + dt * 32 + 8 * b4 + 4 * g) = make_float4(o[dt][4 * b4], o[dt][4 * b4 + 1], o[dt][4 * b4 + 2], o[dt][4 * b4 + 3]);
+        }
+        return;
+    }
     if (A.lse_rows && row_live && g == 0)      // m_ref is the reference the weights were taken against, in log2 units
         A.lse_rows[(size_t)tq * A.QH + head] = l_tot > 0.0f ? m_ref + __builtin_log2f(l_tot) : INFINITY;
     if (row_live && (l_tot > 0.0f || A.gate)) {
@@ -3465,8 +3492,8 @@ static void prefill_split_shape(const Lay &a, int pos_start, int M, int *chunk_t
 // keeps every CU busy.  Rows behind 2k / 32k / 128k tokens, chunk kernel -> split:
 //   16: 59 -> 18, 878 -> 42, 3 992 -> 115 us;  256: 66 -> 37, 868 -> 211, 3 857 -> 799 us;
 //   1 024: 92 -> 98, 928 -> 715, 3 896 -> 2 566 us.
-// (with the two-phase kernel walking its context in parts, prefill_split_ppd_parts, behind 32k tokens: 64 rows 70 -> 55,
-// 256 rows 211 -> 141, 1 024 rows 715 -> 487 us)
+// (with the two-phase kernels walking their context in parts, prefill_split_ppd_parts, behind 32k tokens: 64 rows 70 -> 55,
+// 256 rows 211 -> 141, 1 024 rows 715 -> 487 us; int8 pages 64 rows 81 -> 60, 256 rows 242 -> 168 us)
 static bool d256_direct(const Lay &a);
 static int prefill_split_ppd_parts(const Lay &a, int pos_start, int M);
 static bool prefill_split_applies(const Lay &a, int pos_start, int M)
@@ -3503,13 +3530,13 @@ static bool chunk_kernel_scales_q(const Lay &a, int pos_start, int M)
     return false;
 }
 
-// A chunk of 16-bit pages at head_dim 128 with at least 256 rows per kv head takes the two-phase kernel on that path
+// A chunk at head_dim 128 with at least 256 rows per kv head takes the two-phase kernels on that path
 // too: every walk in parts, one workgroup per CU, the same (o, m, l) pieces and the same merge.  Returns the number of
 // parts per walk (never more than the pieces the workspace was sized for), or 0 for the four-wave kernel.
 static int prefill_split_ppd_parts(const Lay &a, int pos_start, int M)
 {
-    if (!(a.D == 128 && (a.dtype == DRK_BF16 || a.dtype == DRK_F16) && a.bs >= 16 && ilog2_exact((unsigned)a.bs) >= 4)) return 0;
-    if (g_prefill_two_phase == 0 || g_prefill_two_phase == 3) return 0;
+    if (!(a.D == 128 && a.bs >= 16 && ilog2_exact((unsigned)a.bs) >= 4)) return 0;
+    if (g_prefill_two_phase == 0) return 0;
     const int G = a.QH / a.KVH;
     if (G > 256 || (long)M * G < 256) return 0;
     const int tpw2 = 256 / G;
@@ -3825,6 +3852,11 @@ static int prefill_impl(const drk_kv_layout *g, const void *q, const void *pool,
             else DRK_PP_LAUNCH(DRK_F16, DRK_FP8_E4M3, DRK_F16);
 #undef DRK_PP_LAUNCH
             DRK_LAUNCH_CHECK("prefill_pp_kernel");
+            if (split_parts > 0) {
+                hipLaunchKernelGGL(prefill_merge_kernel<128>, dim3((unsigned)((size_t)M * a.QH)), dim3(64), 0, st, A.part_o, A.part_m,
+                                   A.part_l, (uint16_t *)out, split_parts, io_dtype, (const uint16_t *)gate, gate_stride, lse_rows);
+                DRK_LAUNCH_CHECK("prefill_merge_kernel");
+            }
             return DRK_OK;
         }
     }
