@@ -57,6 +57,7 @@ struct GroupedArgs {
     int b_slot[64];                            // first workspace slot of the tail's pieces
     uint8_t *plan;                             // the descriptors of every workgroup in global memory, see DecodePlan
     int plan_mode;                             // 0: build and use; 1: build, store, leave (build_units returns 0); 2: read
+    int max_units;                             // the descriptor table of the kernel that takes the call: no workgroup's run is longer
     // or NULL: one new token per branch, [B][KVH][D] of the pages' 16-bit type, written by the workgroup that owns the
     // last tile of the branch's tail before it reads that tile (decode_group16_kernel only)
     const uint8_t *new_k, *new_v;
@@ -125,18 +126,25 @@ __device__ __forceinline__ uint32_t pack16(float a, float b)
 constexpr float kLazy = 5.0f;
 
 // The grid is dealt to the two kinds of units by what they cost: a tile of a shared range (its waves meet at two
-// barriers) takes about 13 parts of time where a tile of a private tail takes 12.  Workgroups [0, Gs) take runs of
-// Us units of the shared ranges, the others runs of Ut units of the tails.  Kernel and merge compute it alike.
+// barriers) takes about 13 parts of time where a tile of a private tail takes 12 -- and every tail (one kv head of one
+// branch: its own query rows, its first tile's latency, its own partial results) 16 more, which is what counts right
+// after a fork, when 128 tails of one tile each wait behind a long prefix (dealt by tiles alone they went to 7 of 512
+// workgroups, 19 each, and the launch took 77 us instead of 50; with 4 / 8 / 16 / 24 more per tail a step of 36 such
+// layers takes 2.79 / 2.63 / 2.50 / 2.51 ms).  Workgroups [0, Gs) take runs of Us units of the
+// shared ranges, the others runs of Ut units of the tails; neither run is longer than the kernel's descriptor table
+// (`cap`).  Kernel and merge compute it alike.
 struct RegionSplit { int Gs, Us, Ut; };
-__host__ __device__ inline RegionSplit region_split(int group_units, int tail_units, int grid)
+__host__ __device__ inline RegionSplit region_split(int group_units, int tail_units, int tail_runs, int grid, int cap)
 {
     RegionSplit r;
-    const long long cs = 13LL * group_units, ct = 12LL * tail_units;
+    const long long cs = 13LL * group_units, ct = 12LL * tail_units + 16LL * tail_runs;
     if (group_units <= 0) r.Gs = 0;
     else if (tail_units <= 0 || grid < 2) r.Gs = grid;
     else {
         long long gs = (cs * grid + (cs + ct) / 2) / (cs + ct);
         r.Gs = (int)(gs < 1 ? 1 : (gs > grid - 1 ? grid - 1 : gs));
+        const int lo = (group_units + cap - 1) / cap, hi = grid - (tail_units + cap - 1) / cap;
+        if (lo <= hi) r.Gs = r.Gs < lo ? lo : (r.Gs > hi ? hi : r.Gs);
     }
     r.Us = r.Gs > 0 ? (group_units + r.Gs - 1) / r.Gs : 1;
     r.Ut = grid - r.Gs > 0 ? (tail_units + (grid - r.Gs) - 1) / (grid - r.Gs) : 1;
@@ -165,7 +173,8 @@ __device__ __forceinline__ int build_units(const GroupedArgs &A, GUnit *udesc, u
         if (lane >= off) incl += t;
     }
     const int tail_units = __builtin_amdgcn_readlane(incl, 63) * A.KVH;
-    const RegionSplit rs = region_split(A.group_units, tail_units, (int)gridDim.x);
+    const int tail_runs = __popcll(__builtin_amdgcn_ballot_w64(nt_i > 0)) * A.KVH;
+    const RegionSplit rs = region_split(A.group_units, tail_units, tail_runs, (int)gridDim.x, A.max_units);
     const bool tail_wg = (int)blockIdx.x >= rs.Gs;
     const int U = tail_wg ? rs.Ut : rs.Us;
     const int wg_rel = tail_wg ? (int)blockIdx.x - rs.Gs : (int)blockIdx.x;      // the workgroup's place among those of its kind
@@ -930,7 +939,8 @@ __global__ __launch_bounds__(256) void group_merge_kernel(GroupedArgs A, uint16_
         const int nt_b = __shfl(nt, b), excl = __shfl(incl, b) - nt_b;
         int cnt = 0, slot0 = 0;
         if (A.group_units + total * A.KVH > 0) {
-            const RegionSplit rs = region_split(A.group_units, total * A.KVH, grid_wgs);
+            const RegionSplit rs = region_split(A.group_units, total * A.KVH, __popcll(__builtin_amdgcn_ballot_w64(nt > 0)) * A.KVH,
+                                                grid_wgs, A.max_units);
             const int kvh = h / (A.QH / A.KVH);
             if (lane < A.ngroups) {
                 const GSeg sg = A.seg[lane];
@@ -1194,6 +1204,7 @@ int launch_decode_grouped(const drk_kv_layout *g, const void *q, const void *poo
     // 16-bit pages: the tile in LDS, rows dealt to the waves; 8-bit pages (and, as a cross-check, 16-bit pages in
     // diagnostic mode 2): tokens dealt to the waves, K and V through registers
     const bool tile16 = a.E == 2 && g_grouped_mode != 2;
+    A.max_units = tile16 ? kG16MaxUnits : kGMaxUnits;
     const bool fused_append = plan.new_k && plan.new_v && plan.mode != 1;
     if (fused_append && !tile16) return fail(DRK_ERR_INVALID, "decode_grouped: only the 16-bit tile kernel writes the new rows itself");
     A.new_k = fused_append ? plan.new_k : nullptr;
