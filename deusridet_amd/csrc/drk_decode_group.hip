@@ -348,7 +348,11 @@ __global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
         else { lo = f16_bits_to_f((uint16_t)(v & 0xffffu)); hi = f16_bits_to_f((uint16_t)(v >> 16)); }
         return pack16<DOT>(lo * A.scale_log2e, hi * A.scale_log2e);
     };
-    auto load_q = [&](const GUnit &d) {
+    // The next segment's rows are fetched while the last unit of this one is computed and folded (a tail of one tile
+    // is a segment of its own: waiting for its rows at its head was half of what such a unit took) and scaled when
+    // the segment begins.
+    uint4 qraw[4];
+    auto fetch_q = [&](const GUnit &d) {
         const int nrows = (d.flags >> 8) & 0xff;
         const int R = nrows > 16 ? 16 * w + c : c;           // row split: the wave's row group; token split: the one group
 #pragma unroll
@@ -357,10 +361,14 @@ __global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
             if (R < nrows) {
                 const int bl = R / GQ, hd = R - bl * GQ;
                 v = *(const uint4 *)(A.q + (size_t)(d.row0 + bl * A.QH + hd) * (D * 2) + kk * 64 + g * 16);
-                v.x = scaled16(v.x); v.y = scaled16(v.y); v.z = scaled16(v.z); v.w = scaled16(v.w);
             }
-            qop[kk] = v;
+            qraw[kk] = v;
         }
+    };
+    auto take_q = [&]() {                                    // (a row that does not exist was fetched as zeros and stays zero)
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+            qop[kk] = make_uint4(scaled16(qraw[kk].x), scaled16(qraw[kk].y), scaled16(qraw[kk].z), scaled16(qraw[kk].w));
     };
 
     // where this lane finds its operands in a slice
@@ -395,7 +403,8 @@ __global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
     };
 
     request(0);
-    load_q(udesc[0]);
+    fetch_q(udesc[0]);
+    take_q();
     for (int it = 0; it < nunits; it++) {
         const GUnit ud = udesc[it];
         const int flags = __builtin_amdgcn_readfirstlane(ud.flags);
@@ -425,6 +434,7 @@ __global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
         // at all times.  They overwrite the buffer the unit before was read from -- by every wave, if it was split
         // by rows: such a unit ends with a barrier (below).  Row split: every wave reads every slice.
         if (has_next) request(it + 1);
+        if (has_next && (flags & 2)) fetch_q(udesc[it + 1]);
         if (split_rows) __syncthreads();
 
         if (split_rows) {
@@ -563,7 +573,7 @@ __global__ __launch_bounds__(256, 2) void decode_group16_kernel(GroupedArgs A)
 #pragma unroll
             for (int e = 0; e < 8; e++) o[e] = w_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             negm = 0.0f; thr = -INFINITY; l_lane = 0.0f;
-            if (has_next) load_q(udesc[it + 1]);
+            if (has_next) take_q();
         }
     }
 }
