@@ -144,6 +144,8 @@ SIGNATURES = {
     "drk_kv_append_decode_planned": (_i32, [_LP, _vp, _vp, _i32, _vp, _i32, _i32, _GP, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _i32,
                                             _f32, _i32, _vp, _sz, _vp, _sz, _vp]),
     "drk_debug_set_grouped_decode": (None, [_i32]),
+    "drk_debug_grouped_grid": (_i32, [_i32, _i32, _i32, _i32]),
+    "drk_debug_grouped_region_split": (None, [_i32, _i32, _i32, _i32, _i32, C.POINTER(C.c_int)]),
     "drk_prefill_workspace_bytes": (_sz, [_LP, _i32, _i32]),
     "drk_paged_prefill_attention": (_i32, [_LP, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _f32, _i32, _vp, _sz, _vp]),
     "drk_rope_table_fill": (_i32, [_vp, _i32, _i32, _f32, _vp]),

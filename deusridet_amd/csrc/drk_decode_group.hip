@@ -1066,6 +1066,14 @@ struct GroupPlan {
 // loses at its end, the range or tail behind it reads.
 // units one workgroup may own: the descriptor table of the kernel that takes the call
 // (times 12 / 13: the workgroups of the tails take runs up to 13 / 12 of the even share, see region_split)
+// workgroups for t_upper units at most: all that fit on the chip, or as many as keep a workgroup's run within max_units
+static long grouped_grid(long t_upper, int max_units)
+{
+    long G = t_upper < kGWgs ? t_upper : kGWgs;
+    if (G < 1) G = 1;
+    if ((t_upper + G - 1) / G > max_units) G = (t_upper + max_units - 1) / max_units;   // descriptor table size
+    return G;
+}
 static int group_max_units(const Lay &a) { return (a.E == 2 && g_grouped_mode != 2 ? kG16MaxUnits : kGMaxUnits) * 12 / 13; }
 
 static int plan_groups(const Lay &a, int B, int max_seq_len, const drk_prefix_group *groups, int n_in, GroupPlan *P)
@@ -1112,9 +1120,7 @@ static int plan_groups(const Lay &a, int B, int max_seq_len, const drk_prefix_gr
         t_upper += (long)a.KVH * (max_tiles > start ? max_tiles - start : 0);
     }
     for (int b = B; b < 64; b++) P->b_start[b] = P->b_slot[b] = 0;
-    long G = t_upper < kGWgs ? t_upper : kGWgs;
-    if (G < 1) G = 1;
-    if ((t_upper + G - 1) / G > max_units) G = (t_upper + max_units - 1) / max_units;   // descriptor table size
+    const long G = grouped_grid(t_upper, max_units);
     P->grid = (int)G;
     // a run of n tiles of one kv head meets at most min(n, G / KVH + 2) workgroups
     const int cap = (int)(G / a.KVH) + 2;
@@ -1253,6 +1259,18 @@ using namespace drk;
 extern "C" {
 
 void drk_debug_set_grouped_decode(int mode) { g_grouped_mode = (mode == 1 || mode == 2) ? mode : 0; }
+
+int drk_debug_grouped_grid(int kvh, int group_units, int tail_units_upper, int descriptor_table)
+{
+    (void)kvh;
+    return (int)grouped_grid((long)group_units + tail_units_upper, descriptor_table * 12 / 13);
+}
+
+void drk_debug_grouped_region_split(int group_units, int tail_units, int tail_runs, int grid, int descriptor_table, int out[3])
+{
+    const RegionSplit r = region_split(group_units, tail_units, tail_runs, grid, descriptor_table);
+    out[0] = r.Gs; out[1] = r.Us; out[2] = r.Ut;
+}
 
 size_t drk_decode_grouped_workspace_bytes(const drk_kv_layout *g, int B, int max_seq_len, const drk_prefix_group *groups,
                                           int n_groups)

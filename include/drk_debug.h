@@ -38,6 +38,13 @@ void drk_debug_set_prefix_stream(int on);
 /* Diagnostic: 1 = drk_paged_decode_attention_shared never takes the grouped kernel (one launch over
  * shared and private tiles) but always the prefix pass + tail kernel pair; 0 = the library's choice. */
 void drk_debug_set_grouped_decode(int mode);
+/* The arithmetic that deals the fork-tree kernel's grid to its units, for tests on the CPU (no device call).
+ * drk_debug_grouped_grid: the workgroups launched for group_units tiles of shared ranges and an upper bound of
+ * tail_units_upper tail tiles (all kv heads counted), for a kernel whose descriptor table holds descriptor_table units.
+ * drk_debug_grouped_region_split: out = {Gs, Us, Ut} -- workgroups [0, Gs) take runs of Us units of the shared ranges,
+ * the others runs of Ut units of the tails (tail_runs = tails with at least one tile, all kv heads counted). */
+int drk_debug_grouped_grid(int kvh, int group_units, int tail_units_upper, int descriptor_table);
+void drk_debug_grouped_region_split(int group_units, int tail_units, int tail_runs, int grid, int descriptor_table, int out[3]);
 /* Measurement aid for benchmarks: while on, the decode entry points launch the kernels that read the
  * pages and leave their partial results unmerged (no merge kernel: out is not written), so that an event
  * pair the caller records around a call brackets the dominant kernel(s) alone.  Process-wide. */

@@ -117,3 +117,38 @@ def test_random_fork_trees_against_the_tables(seed):
                     k += 1
                 depth = sum(1 for g in groups if g[0] <= i < g[0] + g[1])
                 assert min(covered[i], covered[i + 1]) >= k * bs - (depth + 2) * max(mt, bs), (i, k * bs, covered, groups)
+
+
+def test_the_grid_is_dealt_so_that_every_unit_has_a_workgroup_and_no_run_outgrows_the_table():
+    """The fork-tree kernel's grid goes to runs of units of the shared ranges and runs of units of the tails
+    (region_split in drk_decode_group.hip, the same arithmetic in kernel and merge).  Whatever the shape -- no
+    shared range, no tail, thousands of one-tile tails behind a short range, the host's upper bound above the
+    lengths on the device -- every unit must belong to a workgroup's run and no run may be longer than the
+    kernel's descriptor table.  CPU only: the library's own arithmetic through its debug entry points."""
+    import ctypes as C
+    from deusridet_amd import cabi
+    lib = cabi.lib()
+    rng = np.random.default_rng(20)
+    out = (C.c_int * 3)()
+    for table in (64, 128):                                    # the 16-bit tile kernel's table and the general kernel's
+        for _ in range(20000):
+            kvh = int(rng.choice([1, 2, 4, 8]))
+            B = int(rng.integers(1, 65))
+            gu = kvh * int(rng.choice([0, rng.integers(0, 50), rng.integers(0, 5000)]))
+            tails = [int(rng.choice([0, 1, rng.integers(0, 9), rng.integers(0, 3000)])) for _ in range(B)]
+            upper = [t + int(rng.integers(0, 4)) for t in tails]
+            tu, tr = kvh * sum(tails), kvh * sum(1 for t in tails if t > 0)
+            if gu + kvh * sum(upper) == 0:
+                continue
+            grid = lib.drk_debug_grouped_grid(kvh, gu, kvh * sum(upper), table)
+            assert grid >= 1
+            lib.drk_debug_grouped_region_split(gu, tu, tr, grid, table, out)
+            gs, us, ut = out[0], out[1], out[2]
+            assert 0 <= gs <= grid and 1 <= us <= table and 1 <= ut <= table, (kvh, gu, tu, tr, grid, gs, us, ut)
+            if gu > 0:
+                assert gs >= 1 and gs * us >= gu, (kvh, gu, tu, tr, grid, gs, us, ut)
+            if tu > 0:
+                assert grid - gs >= 1 and (grid - gs) * ut >= tu, (kvh, gu, tu, tr, grid, gs, us, ut)
+    # right after a fork: 128 one-tile tails behind 8 192 shared tiles get enough workgroups not to be the last to finish
+    lib.drk_debug_grouped_region_split(8192, 128, 128, 512, 64, out)
+    assert 512 - out[0] >= 16 and out[2] <= 8
